@@ -1,0 +1,174 @@
+// C entry points of libhf2q_hip.so: argument validation and routing.  Every
+// check that the reference performs on the host before it dispatches (shape
+// alignment, supported types, cache bounds) happens here and turns into an
+// error code; kernels are only launched with shapes they were written for.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "hq_internal.h"
+
+namespace hq {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return HQ_OK;
+    return fail(HQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+static bool known_type(hq_ggml_type t) { return t == HQ_Q8_0 || t == HQ_Q4_K || t == HQ_Q6_K; }
+
+// Largest activation-row count the GEMV kernels take; above it the MFMA GEMM
+// runs (MM_ROUTING_THRESHOLD = 8, src/serve/forward_mlx.rs:9791).
+constexpr uint32_t kGemvMaxRows = 8;
+// mul_mat_id keeps the GEMV form while the routed rows are few enough that
+// experts are rarely shared between rows.
+constexpr uint32_t kGemvIdMaxPairs = 128;
+
+static int check_weight_alignment(const void* w, hq_ggml_type t) {
+    const size_t need = t == HQ_Q4_K ? 16 : 2;
+    if (!is_aligned(w, need))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "weight pointer must be %zu-byte aligned for ggml type %d",
+                    need, (int)t);
+    return HQ_OK;
+}
+
+}  // namespace hq
+
+using namespace hq;
+
+extern "C" {
+
+const char* hq_last_error(void) { return g_err; }
+
+int hq_version(void) { return 100; }
+
+uint32_t hq_block_elems(hq_ggml_type t) {
+    return t == HQ_Q8_0 ? 32u : (t == HQ_Q4_K || t == HQ_Q6_K) ? 256u : 0u;
+}
+
+uint32_t hq_block_bytes(hq_ggml_type t) {
+    return t == HQ_Q8_0 ? Q8_0_BYTES : t == HQ_Q4_K ? Q4K_BYTES : t == HQ_Q6_K ? Q6K_BYTES : 0u;
+}
+
+int hq_dequant_ggml(void* stream, const void* w_blocks, void* out, hq_act_dtype out_dtype,
+                    uint64_t n_elems, hq_ggml_type t) {
+    if (!known_type(t)) return fail(HQ_ERR_UNSUPPORTED, "hq_dequant_ggml: unsupported ggml type %d", (int)t);
+    if (out_dtype != HQ_F32 && out_dtype != HQ_BF16)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dequant_ggml: out_dtype %d", (int)out_dtype);
+    if (n_elems % hq_block_elems(t))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dequant_ggml: n_elems %llu is not a multiple of the block size %u",
+                    (unsigned long long)n_elems, hq_block_elems(t));
+    if (n_elems == 0) return HQ_OK;
+    if (!w_blocks || !out) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dequant_ggml: null buffer");
+    if (int rc = check_weight_alignment(w_blocks, t)) return rc;
+    if (!is_aligned(out, 16)) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dequant_ggml: out must be 16-byte aligned");
+    return launch_dequant((hipStream_t)stream, w_blocks, out, out_dtype, n_elems, t);
+}
+
+int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row,
+                     hq_ggml_type t, void* out_blocks) {
+    if (!known_type(t)) return fail(HQ_ERR_UNSUPPORTED, "hq_quantize_ggml: unsupported ggml type %d", (int)t);
+    const uint32_t be = hq_block_elems(t);
+    // Same two shape rules as GgmlQuantizer::quantize (quantizer.rs:57-71).
+    if (n_per_row == 0 || n_per_row % be)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_quantize_ggml: n_per_row %llu not a multiple of block size %u",
+                    (unsigned long long)n_per_row, be);
+    if (n_elems % n_per_row)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_quantize_ggml: n_elems %llu not a multiple of n_per_row %llu",
+                    (unsigned long long)n_elems, (unsigned long long)n_per_row);
+    if (n_elems == 0) return HQ_OK;
+    if (!src || !out_blocks) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_quantize_ggml: null buffer");
+    if (!is_aligned(src, 16)) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_quantize_ggml: src must be 16-byte aligned");
+    if (int rc = check_weight_alignment(out_blocks, t)) return rc;
+    return launch_quantize((hipStream_t)stream, src, n_elems, n_per_row, t, out_blocks);
+}
+
+static int check_matmul_common(const char* fn, const void* x, hq_act_dtype xdt, const void* w,
+                               const float* y, uint32_t n, uint32_t k, hq_ggml_type t) {
+    if (!known_type(t)) return fail(HQ_ERR_UNSUPPORTED, "%s: unsupported ggml type %d", fn, (int)t);
+    if (xdt != HQ_F32 && xdt != HQ_BF16) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: activation dtype %d", fn, (int)xdt);
+    if (k == 0 || k % hq_block_elems(t))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: k %u is not a multiple of the block size %u", fn, k,
+                    hq_block_elems(t));
+    if (n == 0) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: n is 0", fn);
+    if (!x || !w || !y) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (!is_aligned(x, 16)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: x must be 16-byte aligned", fn);
+    if (!is_aligned(y, 4)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: y must be 4-byte aligned", fn);
+    return check_weight_alignment(w, t);
+}
+
+int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y,
+                    uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
+    if (int rc = check_matmul_common("hq_qmatmul_ggml", x, xdt, w_blocks, y, n, k, t)) return rc;
+    if (m == 0) return HQ_OK;
+    if (m <= kGemvMaxRows) {
+        GemvArgs a{};
+        a.x = x;
+        a.w = static_cast<const uint8_t*>(w_blocks);
+        a.ids = nullptr;
+        a.y = y;
+        a.pairs = m;
+        a.top_k = 1;
+        a.n = n;
+        a.k = k;
+        a.n_experts = 1;
+        a.expert_stride = 0;
+        return launch_gemv((hipStream_t)stream, a, xdt, t);
+    }
+    return fail(HQ_ERR_UNSUPPORTED, "hq_qmatmul_ggml: m = %u (> %u) needs the GEMM path", m, kGemvMaxRows);
+}
+
+size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows) {
+    (void)n_experts;
+    (void)max_rows;
+    return 0;
+}
+
+int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_stack,
+                       const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes,
+                       uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
+                       uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t) {
+    (void)scratch;
+    (void)scratch_bytes;
+    if (int rc = check_matmul_common("hq_qmatmul_id_ggml", x, xdt, w_stack, y, n, k, t)) return rc;
+    if (!ids) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: null ids");
+    if (n_experts == 0 || top_k == 0)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: n_experts %u, top_k %u", n_experts, top_k);
+    const uint64_t expert_bytes = (uint64_t)n * (k / hq_block_elems(t)) * hq_block_bytes(t);
+    if (expert_stride < expert_bytes)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: expert_stride %llu < one expert's %llu bytes",
+                    (unsigned long long)expert_stride, (unsigned long long)expert_bytes);
+    if (expert_stride % (t == HQ_Q4_K ? 16 : 2))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: expert_stride %llu breaks block alignment",
+                    (unsigned long long)expert_stride);
+    const uint64_t pairs = (uint64_t)n_tokens * top_k;
+    if (pairs == 0) return HQ_OK;
+    if (pairs > 0xffffu * 16u) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: too many routed rows");
+    if (pairs <= kGemvIdMaxPairs) {
+        GemvArgs a{};
+        a.x = x;
+        a.w = static_cast<const uint8_t*>(w_stack);
+        a.ids = ids;
+        a.y = y;
+        a.pairs = (uint32_t)pairs;
+        a.top_k = top_k;
+        a.n = n;
+        a.k = k;
+        a.n_experts = n_experts;
+        a.expert_stride = expert_stride;
+        return launch_gemv((hipStream_t)stream, a, xdt, t);
+    }
+    return fail(HQ_ERR_UNSUPPORTED, "hq_qmatmul_id_ggml: %llu routed rows need the grouped GEMM path",
+                (unsigned long long)pairs);
+}
+
+}  // extern "C"

@@ -1,0 +1,118 @@
+// Internal declarations shared by the translation units of libhf2q_hip.so.
+// gfx950 (MI355X) only: 64-lane wavefronts are assumed throughout.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/hf2q_hip.h"
+
+namespace hq {
+
+// Records the message for hq_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+// HQ_OK, or HQ_ERR_HIP with the HIP error string recorded.
+int check_hip(hipError_t e, const char* what);
+// Checks the launch that was just enqueued.
+inline int check_launch(const char* what) { return check_hip(hipGetLastError(), what); }
+
+inline bool is_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+constexpr int kWave = 64;
+constexpr uint32_t Q4K_BYTES = 144, Q6K_BYTES = 210, Q8_0_BYTES = 34;
+
+// ---- launchers (one per .hip file); all validate nothing: the C entry points do ----
+int launch_dequant(hipStream_t s, const void* w, void* out, hq_act_dtype odt, uint64_t n_elems,
+                   hq_ggml_type t);
+int launch_quantize(hipStream_t s, const float* src, uint64_t n_elems, uint64_t n_per_row,
+                    hq_ggml_type t, void* out);
+
+struct GemvArgs {
+    const void* x;        // [x_rows, k] activations
+    const uint8_t* w;     // weight blocks, or the expert stack when ids != nullptr
+    const uint32_t* ids;  // [pairs] expert ids, or nullptr for the dense form
+    float* y;             // [pairs, n]
+    uint32_t pairs;       // dense: m; id form: n_tokens*top_k
+    uint32_t top_k;       // id form: x row of pair p is p / top_k; dense: 1
+    uint32_t n, k;
+    uint32_t n_experts;
+    uint64_t expert_stride;  // bytes
+};
+int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t);
+
+}  // namespace hq
+
+// ---------------------------------------------------------------------------
+// Device helpers
+// ---------------------------------------------------------------------------
+#if defined(__HIPCC__)
+namespace hq {
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+
+// IEEE binary16 bits -> f32, exact (v_cvt_f32_f16; subnormals preserved).
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+// f32 -> bf16 bits, round to nearest even (NaN kept quiet).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// Loads that tolerate 2-byte alignment (Q6_K / Q8_0 blocks are 210 / 34 bytes).
+// gfx950 under HSA runs with unaligned access enabled, so these compile to one
+// global_load_dwordx4 / dwordx2 each.
+__device__ __forceinline__ uint4 ld16_unaligned(const uint8_t* p) {
+    uint4 v;
+    __builtin_memcpy(&v, p, 16);
+    return v;
+}
+__device__ __forceinline__ uint2 ld8_unaligned(const uint8_t* p) {
+    uint2 v;
+    __builtin_memcpy(&v, p, 8);
+    return v;
+}
+__device__ __forceinline__ uint32_t ld2(const uint8_t* p) {
+    return *reinterpret_cast<const uint16_t*>(p);
+}
+
+// a.x*b.x + a.y*b.y + c on two packed bf16 pairs, f32 accumulate (v_dot2c_f32_bf16).
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
+                                           __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+
+// Q4_K: 6-bit scale / min of sub-blocks (2c, 2c+1) for chunk c in [0,4) from the
+// 12 packed bytes held as three little-endian words (y = bytes 0..3, z = 4..7,
+// w = 8..11).  Same bit fields as get_scale_min_k4
+// (src/quantize/ggml_quants/q4_k.rs:329-337), evaluated branch-free.
+__device__ __forceinline__ void q4k_scales(uint32_t y, uint32_t z, uint32_t w, int c, uint32_t& sc0,
+                                           uint32_t& sc1, uint32_t& m0, uint32_t& m1) {
+    const int sh = (c & 1) * 16;
+    const uint32_t ys = y >> sh, zs = z >> sh, ws = w >> sh;
+    if (c < 2) {
+        sc0 = ys & 63u;
+        sc1 = (ys >> 8) & 63u;
+        m0 = zs & 63u;
+        m1 = (zs >> 8) & 63u;
+    } else {
+        sc0 = (ws & 0xFu) | ((ys >> 2) & 0x30u);
+        sc1 = ((ws >> 8) & 0xFu) | ((ys >> 10) & 0x30u);
+        m0 = ((ws >> 4) & 0xFu) | ((zs >> 2) & 0x30u);
+        m1 = ((ws >> 12) & 0xFu) | ((zs >> 10) & 0x30u);
+    }
+}
+
+__device__ __forceinline__ float ubyte0(uint32_t v) { return static_cast<float>(v & 0xffu); }
+__device__ __forceinline__ float ubyte1(uint32_t v) { return static_cast<float>((v >> 8) & 0xffu); }
+__device__ __forceinline__ float ubyte2(uint32_t v) { return static_cast<float>((v >> 16) & 0xffu); }
+__device__ __forceinline__ float ubyte3(uint32_t v) { return static_cast<float>(v >> 24); }
+__device__ __forceinline__ float sbyte(uint32_t v, int i) {
+    return static_cast<float>(static_cast<int>(static_cast<int8_t>((v >> (8 * i)) & 0xffu)));
+}
+
+}  // namespace hq
+#endif

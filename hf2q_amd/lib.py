@@ -1,0 +1,69 @@
+"""ctypes binding of libhf2q_hip.so — the C ABI declared in include/hf2q_hip.h.
+
+There is no fallback: if the shared library is missing the import of the first
+symbol raises, and every non-zero status becomes an ``HqError`` carrying the
+library's own message.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libhf2q_hip.so")
+
+HQ_OK, HQ_ERR_INVALID_ARGUMENT, HQ_ERR_UNSUPPORTED, HQ_ERR_HIP = 0, 1, 2, 3
+HQ_Q8_0, HQ_Q4_K, HQ_Q6_K = 8, 12, 14
+HQ_F32, HQ_BF16 = 0, 1
+
+
+class HqError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"hq status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+_c = ctypes
+_vp, _u32, _u64, _i32, _sz, _f32 = _c.c_void_p, _c.c_uint32, _c.c_uint64, _c.c_int, _c.c_size_t, _c.c_float
+
+# name -> (restype, argtypes); the single source for the symbol-export test.
+SIGNATURES = {
+    "hq_last_error": (_c.c_char_p, []),
+    "hq_version": (_i32, []),
+    "hq_block_elems": (_u32, [_i32]),
+    "hq_block_bytes": (_u32, [_i32]),
+    "hq_dequant_ggml": (_i32, [_vp, _vp, _vp, _i32, _u64, _i32]),
+    "hq_quantize_ggml": (_i32, [_vp, _vp, _u64, _u64, _i32, _vp]),
+    "hq_qmatmul_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32]),
+    "hq_qmatmul_id_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _u32, _u32, _u32, _u32, _u32, _u64, _i32]),
+    "hq_qmatmul_id_scratch_bytes": (_sz, [_u32, _u32]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load libhf2q_hip.so (built by ``python -m hf2q_amd.build``); raises if absent."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                f"{LIB_PATH} is missing: build it with `python -m hf2q_amd.build` "
+                "(there is no CPU fallback for this path)")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def last_error() -> str:
+    return load().hq_last_error().decode()
+
+
+def check(status: int) -> None:
+    if status != HQ_OK:
+        raise HqError(status, last_error())

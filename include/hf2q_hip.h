@@ -1,0 +1,115 @@
+/*
+ * hf2q_hip.h -- C ABI of libhf2q_hip.so: the MI355X (gfx950) implementation of
+ * hf2q's quantized-matmul hot path.
+ *
+ * Conventions (they mirror the contract hf2q's call sites have with their GPU
+ * backend today):
+ *   - every buffer pointer is a DEVICE pointer owned by the caller; nothing is
+ *     allocated, freed or retained by the library (hf2q passes caller-owned
+ *     MlxBuffers and scratch the same way, gpu_ffn.rs:194-204, 644-648);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     Work is enqueued in order on it and the call returns at once, like an
+ *     encoder dispatch without commit; the caller synchronises.  An in-order
+ *     stream provides every read-after-write barrier hf2q declares by hand
+ *     (gpu_ffn.rs:2538-2544);
+ *   - shapes are explicit arguments, never inferred from buffer sizes;
+ *   - every function returns HQ_OK (0) or an hq_status error code and never
+ *     aborts; the message is available from hq_last_error() on the same thread
+ *     ("fail loud", kv_cache.rs:152-153);
+ *   - functions are re-entrant per stream; the only library state is the
+ *     thread-local error string.
+ *
+ * Paths cited below are relative to the hf2q source tree.
+ */
+#ifndef HF2Q_HIP_H
+#define HF2Q_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Exported from the shared library (it is built with hidden visibility). */
+#define HQ_API __attribute__((visibility("default")))
+
+typedef enum {
+    HQ_OK = 0,
+    HQ_ERR_INVALID_ARGUMENT = 1, /* shape / alignment / enum the path rejects */
+    HQ_ERR_UNSUPPORTED = 2,      /* ggml type or mode not on this path */
+    HQ_ERR_HIP = 3               /* a HIP runtime call failed */
+} hq_status;
+
+/* Numeric ids are GGML's (src/quantize/ggml_quants/ggml_type.rs:18-53). */
+typedef enum { HQ_Q8_0 = 8, HQ_Q4_K = 12, HQ_Q6_K = 14 } hq_ggml_type;
+
+/* Activation element type.  hf2q's call sites pass F32 (gpu_full_attn.rs:835);
+ * BF16 is the serving configuration this library is benchmarked on. */
+typedef enum { HQ_F32 = 0, HQ_BF16 = 1 } hq_act_dtype;
+
+/* Thread-local message of the last failing call on this thread ("" if none). */
+HQ_API const char* hq_last_error(void);
+
+/* Library ABI version (major*100 + minor). */
+HQ_API int hq_version(void);
+
+/* Block geometry: GgmlType::block_size / type_size (ggml_type.rs:60-135).
+ * Return 0 for a type this path does not handle. */
+HQ_API uint32_t hq_block_elems(hq_ggml_type t);
+HQ_API uint32_t hq_block_bytes(hq_ggml_type t);
+
+/* Dequantise `n_elems` (a whole number of blocks) of packed GGML blocks to
+ * f32 (out_dtype HQ_F32, bit-exact: one correctly rounded value per element)
+ * or bf16 (HQ_BF16, the f32 value rounded to nearest-even).  Replaces the
+ * load-time `materialize_f16_shadow` pre-dequantisation
+ * (src/serve/forward_mlx.rs:9426-9440) and doubles as the bit-exactness probe
+ * for the in-kernel dequantisers. */
+HQ_API int hq_dequant_ggml(void* stream, const void* w_blocks, void* out, hq_act_dtype out_dtype,
+                    uint64_t n_elems, hq_ggml_type t);
+
+/* Quantise f32 rows to packed GGML blocks on the device, byte-identical to
+ * hf2q's CPU quantizers without an importance matrix
+ * (src/quantize/ggml_quants/quantizer.rs:51-102 -> q4_k.rs:50-217,
+ * q6_k.rs:40-221, q8_0.rs:31-72; load-time use:
+ * src/inference/models/qwen35/in_memory_loader.rs:70-139).
+ * `n_elems` must be a multiple of `n_per_row`, `n_per_row` of the block size. */
+HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row,
+                     hq_ggml_type t, void* out_blocks);
+
+/* dst[m,n] = x[m,k] . W[n,k]^T with W stored as GGML blocks, row-major
+ * [n][k/QK]; fp32 accumulate, f32 output.  Replaces
+ * mlx_native quantized_matmul_ggml(encoder, registry, device, input, weight,
+ * &mut dst, &GgmlQuantizedMatmulParams{m,n,k,ggml_type})
+ * (src/inference/models/qwen35/gpu_ffn.rs:1236-1245; dispatch_qmatmul,
+ * src/serve/forward_mlx.rs:9655-9969).  m <= 8 takes the bandwidth-bound GEMV
+ * kernels, m > 8 the MFMA GEMM (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791).
+ * Requires k % block_elems == 0; Q4_K needs a 16-byte aligned `w_blocks`,
+ * Q6_K / Q8_0 a 2-byte aligned one. */
+HQ_API int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y,
+                    uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t);
+
+/* out[t, s, :] = W[ids[t*top_k + s]] . x[t, :] over an expert stack
+ * [n_experts][n][k/QK] whose experts are `expert_stride` BYTES apart;
+ * ids [n_tokens*top_k] u32 on the device (no host sync); out
+ * [n_tokens*top_k, n] f32.  Replaces quantized_matmul_id_ggml[_pooled]
+ * (gpu_ffn.rs:194-204; forward_mlx.rs:5285-5292, 5367-5374) with
+ * GgmlQuantizedMatmulIdParams{n_tokens, top_k, n, k, n_experts,
+ * expert_stride, ggml_type}.  The "down" projection is the same call with
+ * n_tokens = T*K, top_k = 1 (forward_mlx.rs:650-651).  An id >= n_experts
+ * makes the affected output rows NaN instead of reading out of bounds.
+ * `scratch` (device, hq_qmatmul_id_scratch_bytes) is only needed once
+ * n_tokens*top_k exceeds the GEMV limit; it may be NULL below that. */
+HQ_API int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_stack,
+                       const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes,
+                       uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
+                       uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
+
+/* Bytes of `scratch` hq_qmatmul_id_ggml needs for up to `max_rows` =
+ * n_tokens*top_k routed rows (the IdMmScratch analogue, decode_pool.rs:56-60). */
+HQ_API size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HF2Q_HIP_H */

@@ -1,0 +1,38 @@
+"""Shared helpers for the parity tests (seeded inputs, tolerances)."""
+import numpy as np
+
+GOLDEN = __import__("os").path.join(__import__("os").path.dirname(__file__), "golden")
+
+# north_star tolerance for matmul outputs: 1e-3 relative to the f64 result
+# (fp32 accumulate).  The small absolute floor (1e-5 of the output RMS) only
+# matters for outputs that cancel to ~0.
+REL_TOL = 1e-3
+ABS_FLOOR = 1e-5
+
+
+def assert_matmul_close(got, ref64, what=""):
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref64, dtype=np.float64).reshape(-1)
+    assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    rms = float(np.sqrt(np.mean(ref * ref))) if ref.size else 0.0
+    err = np.abs(got - ref)
+    bound = REL_TOL * np.abs(ref) + ABS_FLOOR * rms
+    bad = err > bound
+    if bad.any():
+        i = int(np.argmax(err - bound))
+        raise AssertionError(f"{what}: {int(bad.sum())}/{ref.size} outside 1e-3 rel; worst idx {i}: "
+                             f"got {got[i]!r} ref {ref[i]!r} (rms {rms:.4g})")
+    if rms > 0:
+        cos = float(got @ ref / (np.linalg.norm(got) * np.linalg.norm(ref)))
+        assert cos >= 0.9999, f"{what}: cosine {cos}"
+    return float(err.max() / rms) if rms > 0 else 0.0
+
+
+def weights(seed, n, k, sigma=0.02):
+    """Seeded N(0, sigma) f32 weight [n, k] (the benchmark's weight distribution)."""
+    return (np.random.default_rng(seed).standard_normal((n, k), dtype=np.float32) * np.float32(sigma))
+
+
+def acts(seed, m, k):
+    return np.random.default_rng(seed).standard_normal((m, k), dtype=np.float32)

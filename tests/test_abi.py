@@ -1,0 +1,65 @@
+"""CPU-only checks of the C ABI: the library loads, exports every symbol the
+header declares, and rejects bad arguments before touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from hf2q_amd import lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hf2q_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 9
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/hf2q_hip.h but not exported"
+        assert n in lib.SIGNATURES, f"{n} has no ctypes signature in hf2q_amd/lib.py"
+    assert sorted(lib.SIGNATURES) == names
+
+
+def test_block_geometry():
+    # ggml_type.rs:60-135
+    L = lib.load()
+    assert (L.hq_block_elems(lib.HQ_Q4_K), L.hq_block_bytes(lib.HQ_Q4_K)) == (256, 144)
+    assert (L.hq_block_elems(lib.HQ_Q6_K), L.hq_block_bytes(lib.HQ_Q6_K)) == (256, 210)
+    assert (L.hq_block_elems(lib.HQ_Q8_0), L.hq_block_bytes(lib.HQ_Q8_0)) == (32, 34)
+    assert L.hq_block_elems(2) == 0 and L.hq_block_bytes(13) == 0
+
+
+def test_argument_errors_are_reported_not_fatal():
+    L = lib.load()
+    fake = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
+    # k not a multiple of the block size (quantizer.rs:57-71)
+    assert L.hq_qmatmul_ggml(None, fake, lib.HQ_F32, fake, fake, 1, 8, 300, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert "multiple of the block size" in lib.last_error()
+    # unsupported ggml type (forward_mlx.rs:9884-9886)
+    assert L.hq_qmatmul_ggml(None, fake, lib.HQ_F32, fake, fake, 1, 8, 256, 13) == lib.HQ_ERR_UNSUPPORTED
+    assert L.hq_dequant_ggml(None, fake, fake, lib.HQ_F32, 100, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    # misaligned Q4_K weights
+    assert L.hq_qmatmul_ggml(None, fake, lib.HQ_F32, ctypes.c_void_p(0x1002), fake, 1, 8, 256, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert "aligned" in lib.last_error()
+    # null buffers
+    assert L.hq_qmatmul_ggml(None, None, lib.HQ_F32, fake, fake, 1, 8, 256, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    # id form: expert stride smaller than an expert
+    assert L.hq_qmatmul_id_ggml(None, fake, lib.HQ_F32, fake, fake, fake, None, 0, 1, 2, 8, 256, 4, 100, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_quantize_ggml(None, fake, 512, 300, lib.HQ_Q4_K, fake) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_quantize_ggml(None, fake, 768, 512, lib.HQ_Q4_K, fake) == lib.HQ_ERR_INVALID_ARGUMENT
+    with pytest.raises(lib.HqError):
+        lib.check(lib.HQ_ERR_INVALID_ARGUMENT)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(FileNotFoundError):
+        lib.load()

@@ -1,0 +1,168 @@
+"""GPU parity of the dequantiser and the dequant-fused GEMV / mul_mat_id kernels
+against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from _util import acts, assert_matmul_close, weights
+from hf2q_amd import ops
+from hf2q_amd.ops import (HQ_Q4_K, HQ_Q6_K, HQ_Q8_0, GgmlQuantizedMatmulIdParams, GgmlQuantizedMatmulParams)
+
+pytestmark = pytest.mark.gpu
+TYPES = [HQ_Q4_K, HQ_Q6_K, HQ_Q8_0]
+
+
+def _adversarial_blocks(oracle, t, nblocks, seed):
+    """Raw random bytes (every nibble / 6-bit scale / sign pattern) with finite f16 scales."""
+    bb = oracle.BLOCK_BYTES[t]
+    raw = np.random.default_rng(seed).integers(0, 256, size=nblocks * bb, dtype=np.uint8)
+    for off in ([1, 3] if t == HQ_Q4_K else [209] if t == HQ_Q6_K else [1]):
+        raw[off::bb] &= 0x3F
+    return raw
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_dequant_bit_exact(oracle, dev, t):
+    be = oracle.BLOCK_ELEMS[t]
+    w = weights(100 + t, 64, 1024)
+    blocks = np.concatenate([oracle.quantize(w, 1024, t), _adversarial_blocks(oracle, t, 4096 // be * 8, t)])
+    n = blocks.size // oracle.BLOCK_BYTES[t] * be
+    want = oracle.dequantize(blocks, t)
+    wd = torch.from_numpy(blocks).to(dev)
+    got = ops.dequantize_ggml(wd, n, t).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    got16 = ops.dequantize_ggml(wd, n, t, torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got16, oracle.f32_to_bf16_bits(want))
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_dequant_golden_blocks(oracle, dev, t):
+    import os
+    from _util import GOLDEN
+    name = {HQ_Q4_K: "q4_k_512", HQ_Q6_K: "q6_k_512", HQ_Q8_0: "q8_0_64"}[t]
+    blocks = np.fromfile(os.path.join(GOLDEN, "ggml_quants", f"{name}_noim_expected.bin"), dtype=np.uint8)
+    n = blocks.size // oracle.BLOCK_BYTES[t] * oracle.BLOCK_ELEMS[t]
+    # Q6_K / Q8_0 blocks need only 2-byte alignment: also run from an odd-word offset
+    pad = torch.zeros(blocks.size + 16, dtype=torch.uint8, device=dev)
+    for off in ([0] if t == HQ_Q4_K else [0, 2, 6]):
+        pad[off:off + blocks.size] = torch.from_numpy(blocks).to(dev)
+        got = ops.dequantize_ggml(pad[off:], n, t).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), oracle.dequantize(blocks, t).view(np.uint32))
+
+
+SHAPES = [  # (m, n, k)
+    (1, 512, 4096), (1, 1000, 2048), (1, 64, 256), (1, 37, 512), (1, 130, 768), (1, 96, 1024),
+    (1, 257, 12288), (3, 200, 4096), (8, 128, 2048), (1, 4, 8192),
+]
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_gemv_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
+    w = weights(7 * n + k + t, n, k)
+    blocks = oracle.quantize(w, k, t, threads=8)
+    x = acts(n + k, m, k)
+    if xdt == "bf16":
+        xb = oracle.f32_to_bf16_bits(x)
+        xd = torch.from_numpy(xb.view(np.int16)).to(dev).view(torch.bfloat16).reshape(m, k)
+        ref = oracle.qmatmul_f64(xb, blocks, m, n, k, t)
+    else:
+        xd = torch.from_numpy(x).to(dev)
+        ref = oracle.qmatmul_f64(x, blocks, m, n, k, t)
+    y = torch.full((m, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd, torch.from_numpy(blocks).to(dev), y, GgmlQuantizedMatmulParams(m, n, k, t))
+    assert_matmul_close(y.cpu().numpy(), ref, f"gemv t={t} {xdt} {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_gemv_adversarial_blocks(oracle, dev, t):
+    """Every scale / min / sign bit pattern, not just what the quantizer emits."""
+    n, k = 96, 1024
+    blocks = _adversarial_blocks(oracle, t, n * k // oracle.BLOCK_ELEMS[t], 5)
+    x = acts(1, 1, k)
+    for xv, xd in ((x, torch.from_numpy(x).to(dev)),
+                   (oracle.f32_to_bf16_bits(x), torch.from_numpy(x).to(dev).to(torch.bfloat16))):
+        ref = oracle.qmatmul_f64(xv, blocks, 1, n, k, t)
+        y = torch.empty((1, n), device=dev)
+        ops.quantized_matmul_ggml(xd, torch.from_numpy(blocks).to(dev), y, GgmlQuantizedMatmulParams(1, n, k, t))
+        assert_matmul_close(y.cpu().numpy(), ref, f"adversarial t={t}")
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_gemv_zero_weights_give_zero(oracle, dev, t):
+    # gpu_ffn.rs:3323-3351
+    n, k = 64, 512
+    blocks = oracle.quantize(np.zeros((n, k), np.float32), k, t)
+    y = torch.full((1, n), 7.0, device=dev)
+    ops.quantized_matmul_ggml(torch.randn(1, k, device=dev), torch.from_numpy(blocks).to(dev), y,
+                              GgmlQuantizedMatmulParams(1, n, k, t))
+    assert not y.cpu().numpy().any()
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_gemv_unaligned_weight_base(oracle, dev, t):
+    if t == HQ_Q4_K:
+        pytest.skip("Q4_K requires 16-byte aligned blocks (144 = 9*16)")
+    n, k = 48, 512
+    blocks = oracle.quantize(weights(3, n, k), k, t)
+    x = acts(4, 1, k)
+    ref = oracle.qmatmul_f64(x, blocks, 1, n, k, t)
+    buf = torch.zeros(blocks.size + 16, dtype=torch.uint8, device=dev)
+    buf[2:2 + blocks.size] = torch.from_numpy(blocks).to(dev)
+    y = torch.empty((1, n), device=dev)
+    ops.quantized_matmul_ggml(torch.from_numpy(x).to(dev), buf[2:], y, GgmlQuantizedMatmulParams(1, n, k, t))
+    assert_matmul_close(y.cpu().numpy(), ref, "unaligned base")
+
+
+ID_CASES = [  # (E, n, k, T, K)
+    (8, 64, 512, 1, 2), (16, 512, 2048, 1, 8), (16, 2048, 512, 8, 1), (256, 128, 256, 8, 8), (4, 33, 768, 5, 3),
+]
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("E,n,k,T,K", ID_CASES)
+def test_mul_mat_id_matches_oracle(oracle, dev, t, xdt, E, n, k, T, K):
+    rng = np.random.default_rng(E * n + k)
+    # quantise a few distinct experts and tile them: cheap to build, ids still select real data
+    base = min(E, 4)
+    blocks = oracle.quantize(weights(E + n, base * n, k), k, t, threads=8)
+    stride = n * ops.ggml_row_bytes(t, k)
+    stack = np.concatenate([blocks[(e % base) * stride:(e % base + 1) * stride] for e in range(E)])
+    ids = rng.integers(0, E, size=T * K).astype(np.uint32)
+    x = acts(k, T, k)
+    xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
+    xd = torch.from_numpy(x).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    ref = oracle.qmatmul_id_f64(xv, stack, ids, T, K, n, k, E, stride, t)
+    y = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(xd, torch.from_numpy(stack).to(dev), torch.from_numpy(ids.view(np.int32)).to(dev), y,
+                                 GgmlQuantizedMatmulIdParams(T, K, n, k, E, stride, t))
+    assert_matmul_close(y.cpu().numpy(), ref, f"mul_mat_id t={t} {xdt}")
+
+
+def test_mul_mat_id_invariants(oracle, dev):
+    """Permuting ids permutes output rows; the down-projection calling form equals the grouped form;
+    an out-of-range id poisons only its own rows."""
+    t, E, n, k, T, K = HQ_Q4_K, 8, 64, 512, 4, 2
+    stride = n * ops.ggml_row_bytes(t, k)
+    stack = torch.from_numpy(oracle.quantize(weights(1, E * n, k), k, t)).to(dev)
+    x = torch.from_numpy(acts(2, T, k)).to(dev)
+    ids = torch.tensor([3, 1, 0, 7, 2, 2, 5, 4], dtype=torch.int32, device=dev)
+    p = GgmlQuantizedMatmulIdParams(T, K, n, k, E, stride, t)
+    y = torch.empty((T * K, n), device=dev)
+    ops.quantized_matmul_id_ggml(x, stack, ids, y, p)
+    swap = ids.view(T, K).flip(1).contiguous().view(-1)
+    y2 = torch.empty_like(y)
+    ops.quantized_matmul_id_ggml(x, stack, swap, y2, p)
+    assert torch.equal(y.view(T, K, n).flip(1), y2.view(T, K, n))
+    y3 = torch.empty_like(y)
+    ops.quantized_matmul_id_ggml(x.repeat_interleave(K, 0).contiguous(), stack, ids, y3,
+                                 GgmlQuantizedMatmulIdParams(T * K, 1, n, k, E, stride, t))
+    assert torch.equal(y, y3)
+    bad = ids.clone()
+    bad[3] = E
+    y4 = torch.empty_like(y)
+    ops.quantized_matmul_id_ggml(x, stack, bad, y4, p)
+    assert torch.isnan(y4[3]).all() and torch.equal(y4[[0, 1, 2, 4, 5, 6, 7]], y[[0, 1, 2, 4, 5, 6, 7]])
