@@ -11,11 +11,13 @@
 //     64-element chunk = 32 bytes of nibbles; Q6_K: 16 bytes of ql, 16 of
 //     ql+32, 16 of qh = four 16-element runs) or one 32-weight Q8_0 block, and
 //     fetches it with 16-byte loads;
-//   * L = min(64, pow2(k / weights-per-lane)) lanes share a row, so a wave
-//     covers 64/L rows per step and strides over the row when it is longer;
-//   * each lane keeps R rows in flight (R*3..5 independent 16-byte loads) to
-//     cover HBM latency, re-using the LDS-fetched activations R times;
-//   * partial sums are reduced across the L lanes with DPP/swizzle shuffles.
+//   * L = the largest power of two <= 64 dividing the pieces of a row; L lanes
+//     share a row, so a wave covers 64/L rows (a "slot") per step and takes
+//     pieces/L steps over the row;
+//   * a wave owns NR slots and keeps D weight fetches in flight while it walks
+//     its (step, slot) tasks; the activations of a step are read from LDS once
+//     and re-used for all NR slots;
+//   * partial sums are reduced across the L lanes with DPP row operations.
 //
 // bf16 activations with K-quants use v_dot2c_f32_bf16: nibbles / 6-bit values
 // are turned into bf16 pairs with one and-or against the magic 0x4300 (=128.0,
@@ -84,15 +86,16 @@ __device__ __forceinline__ uint32_t word(const uint4& v, int i) {
 }
 
 // ---- paired-bf16 activations (xp: 32 words = 64 activations of this lane, sx: 4 run sums) ----
-__device__ __forceinline__ float dot_pair(const Piece<HQ_Q4_K>& p, int c, const uint32_t* xp, const float* sx) {
+__device__ __forceinline__ float dot_pair(const Piece<HQ_Q4_K>& p, int c, const uint32_t* xp, const float* sx,
+                                          uint32_t m4, uint32_t, uint32_t magic) {
     float lo = 0.f, hi = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const uint32_t w = j < 4 ? word(p.q0, j) : word(p.q1, j - 4);
-        lo = dot2_bf16((w & M4) | MAGIC, xp[2 * j], lo);
-        lo = dot2_bf16(((w >> 8) & M4) | MAGIC, xp[2 * j + 1], lo);
-        hi = dot2_bf16(((w >> 4) & M4) | MAGIC, xp[16 + 2 * j], hi);
-        hi = dot2_bf16(((w >> 12) & M4) | MAGIC, xp[16 + 2 * j + 1], hi);
+        lo = dot2_bf16((w & m4) | magic, xp[2 * j], lo);
+        lo = dot2_bf16(((w >> 8) & m4) | magic, xp[2 * j + 1], lo);
+        hi = dot2_bf16(((w >> 4) & m4) | magic, xp[16 + 2 * j], hi);
+        hi = dot2_bf16(((w >> 12) & m4) | magic, xp[16 + 2 * j + 1], hi);
     }
     uint32_t sc0, sc1, m0, m1;
     q4k_scales(p.hdr.y, p.hdr.z, p.hdr.w, c, sc0, sc1, m0, m1);
@@ -104,19 +107,20 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q4_K>& p, int c, const 
     return acc;
 }
 
-__device__ __forceinline__ float dot_pair(const Piece<HQ_Q6_K>& p, int c, const uint32_t* xp, const float* sx) {
+__device__ __forceinline__ float dot_pair(const Piece<HQ_Q6_K>& p, int c, const uint32_t* xp, const float* sx,
+                                          uint32_t m4, uint32_t m2, uint32_t magic) {
     float r0 = 0.f, r1 = 0.f, r2 = 0.f, r3 = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t a = word(p.qa, j), b = word(p.qb, j), v = word(p.qh, j);
-        r0 = dot2_bf16((a & M4) | ((v << 4) & M2) | MAGIC, xp[2 * j], r0);
-        r0 = dot2_bf16(((a >> 8) & M4) | ((v >> 4) & M2) | MAGIC, xp[2 * j + 1], r0);
-        r1 = dot2_bf16((b & M4) | ((v << 2) & M2) | MAGIC, xp[8 + 2 * j], r1);
-        r1 = dot2_bf16(((b >> 8) & M4) | ((v >> 6) & M2) | MAGIC, xp[8 + 2 * j + 1], r1);
-        r2 = dot2_bf16(((a >> 4) & M4) | (v & M2) | MAGIC, xp[16 + 2 * j], r2);
-        r2 = dot2_bf16(((a >> 12) & M4) | ((v >> 8) & M2) | MAGIC, xp[16 + 2 * j + 1], r2);
-        r3 = dot2_bf16(((b >> 4) & M4) | ((v >> 2) & M2) | MAGIC, xp[24 + 2 * j], r3);
-        r3 = dot2_bf16(((b >> 12) & M4) | ((v >> 10) & M2) | MAGIC, xp[24 + 2 * j + 1], r3);
+        r0 = dot2_bf16(and_or((v << 4), m2, (a & m4) | magic), xp[2 * j], r0);
+        r0 = dot2_bf16(and_or((v >> 4), m2, ((a >> 8) & m4) | magic), xp[2 * j + 1], r0);
+        r1 = dot2_bf16(and_or((v << 2), m2, (b & m4) | magic), xp[8 + 2 * j], r1);
+        r1 = dot2_bf16(and_or((v >> 6), m2, ((b >> 8) & m4) | magic), xp[8 + 2 * j + 1], r1);
+        r2 = dot2_bf16(and_or(v, m2, ((a >> 4) & m4) | magic), xp[16 + 2 * j], r2);
+        r2 = dot2_bf16(and_or((v >> 8), m2, ((a >> 12) & m4) | magic), xp[16 + 2 * j + 1], r2);
+        r3 = dot2_bf16(and_or((v >> 2), m2, ((b >> 4) & m4) | magic), xp[24 + 2 * j], r3);
+        r3 = dot2_bf16(and_or((v >> 10), m2, ((b >> 12) & m4) | magic), xp[24 + 2 * j + 1], r3);
     }
     // scale bytes lr, lr+2, lr+4, lr+6 of this half's eight; values hold 128 + q with q in 0..63
     // and the format's own -32, hence the 160.
@@ -246,10 +250,82 @@ struct KArgs {
     uint32_t top_k, n, k, n_experts;
     uint64_t expert_stride;
     uint32_t log_l;  // log2 of the lanes that share one row
+    // Bit masks of the nibble -> bf16 conversion.  They are passed as arguments and
+    // not written as literals so that the compiler keeps them in registers and
+    // forms the three-operand v_and_or_b32 (gfx9 VOP3 takes no literals; with
+    // literals it emits v_and + v_or instead).
+    uint32_t m4, m2, magic;
 };
 
-template <int TYPE, bool X_BF16, bool PAIR, int R>
+// v + (v from the lane selected by a DPP control), one VALU op.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return v + __int_as_float(t);
+}
+
+// Sum over aligned groups of L = 2^log_l lanes; every lane of a group ends up with
+// the group's sum.  Quad permutes and row mirrors cover 16 lanes, the last two
+// levels cross 16-lane rows and go through ds_bpermute.
+__device__ __forceinline__ float group_sum(float v, uint32_t log_l) {
+    if (log_l >= 1) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    if (log_l >= 2) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    if (log_l >= 3) v = dpp_add<0x141>(v);  // row_half_mirror
+    if (log_l >= 4) v = dpp_add<0x140>(v);  // row_mirror
+    if (log_l >= 5) v += __shfl_xor(v, 16);
+    if (log_l >= 6) v += __shfl_xor(v, 32);
+    return v;
+}
+
+// Loads the activations of one piece from LDS into registers.
+template <int TYPE, bool PAIR, int XW>
+__device__ __forceinline__ void load_x_piece(const uint32_t* lds_x, const float* lds_s, uint32_t pc, int c,
+                                             uint32_t* xr, float* sx) {
+    constexpr int EPL = Lane<TYPE>::kElems;
+    if constexpr (TYPE == HQ_Q6_K) {
+        // four runs of 16 at stride 32 inside one 128-element half
+        const uint32_t e0 = (pc >> 2) * 256u + (uint32_t)(c >> 1) * 128u + (uint32_t)(c & 1) * 16u;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t e = e0 + 32u * r;
+            const uint4* src = reinterpret_cast<const uint4*>(lds_x + (PAIR ? e / 2 : e));
+#pragma unroll
+            for (int j = 0; j < XW / 16; ++j) {
+                const uint4 t = src[j];
+                xr[(XW / 4) * r + 4 * j] = t.x;
+                xr[(XW / 4) * r + 4 * j + 1] = t.y;
+                xr[(XW / 4) * r + 4 * j + 2] = t.z;
+                xr[(XW / 4) * r + 4 * j + 3] = t.w;
+            }
+            sx[r] = lds_s[e / 16];
+        }
+    } else {
+        // Q4_K: 64 consecutive activations; Q8_0: 32
+        const uint32_t e0 = pc * EPL;
+        const uint4* src = reinterpret_cast<const uint4*>(lds_x + (PAIR ? e0 / 2 : e0));
+#pragma unroll
+        for (int j = 0; j < XW / 4; ++j) {
+            const uint4 t = src[j];
+            xr[4 * j] = t.x;
+            xr[4 * j + 1] = t.y;
+            xr[4 * j + 2] = t.z;
+            xr[4 * j + 3] = t.w;
+        }
+#pragma unroll
+        for (int r = 0; r < EPL / 16; ++r) sx[r] = lds_s[e0 / 16 + r];
+    }
+}
+
+// One workgroup = 4 waves sharing the staged activation row.  A wave owns NR
+// "row slots" (a slot = the 64/L rows its lanes cover at once) and walks the
+// (step, slot) tasks in step-major order with D weight fetches in flight:
+// the fetch for task t+D is issued right after task t has consumed its
+// registers, so HBM latency is covered by D-1 tasks of arithmetic per wave
+// (times the waves resident on the SIMD).  The activations of a step stay in
+// registers for all NR slots.  NR % D == 0 keeps every buffer index static.
+template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
 __global__ __launch_bounds__(256) void gemv_kernel(KArgs a) {
+    static_assert(NR % D == 0, "buffer rotation must repeat per step");
     extern __shared__ uint4 smem[];
     constexpr int EPL = Lane<TYPE>::kElems;
     constexpr uint32_t BYTES = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES : Q8_0_BYTES;
@@ -259,10 +335,6 @@ __global__ __launch_bounds__(256) void gemv_kernel(KArgs a) {
     float* lds_s = reinterpret_cast<float*>(lds_x + (PAIR ? a.k / 2 : a.k));
 
     const uint32_t p = blockIdx.y;
-    const uint32_t xrow = p / a.top_k;
-    const size_t xbytes = X_BF16 ? 2 : 4;
-    stage_x<X_BF16, PAIR>(static_cast<const uint8_t*>(a.x) + (size_t)xrow * a.k * xbytes, a.k, lds_x, lds_s);
-
     const uint8_t* w = a.w;
     bool valid = true;
     if (a.ids) {
@@ -270,104 +342,97 @@ __global__ __launch_bounds__(256) void gemv_kernel(KArgs a) {
         valid = e < a.n_experts;
         w += (size_t)(valid ? e : 0u) * a.expert_stride;
     }
-    __syncthreads();
 
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t L = 1u << a.log_l;
-    const uint32_t rpw = 64u >> a.log_l;  // rows a wave covers per step
+    const uint32_t rpw = 64u >> a.log_l;  // rows per slot
     const uint32_t li = lane & (L - 1u);
-    const uint32_t pieces = a.k / EPL;    // pieces per row
-    const uint32_t row0 = (blockIdx.x * 4u + wave) * rpw * R + (lane >> a.log_l);
-    const size_t row_bytes = (size_t)(a.k / (TYPE == HQ_Q8_0 ? 32 : 256)) * BYTES;
+    const uint32_t steps = (a.k / EPL) >> a.log_l;  // pieces per row / L (host guarantees divisibility)
+    const uint32_t row0 = (blockIdx.x * 4u + wave) * rpw * NR + (lane >> a.log_l);
+    const uint32_t row_bytes = (a.k / (TYPE == HQ_Q8_0 ? 32 : 256)) * BYTES;
+    // L >= 4 for the K-quants (k >= 256), so a lane keeps the same sub-piece index c
+    // on every step.
+    const int c = TYPE == HQ_Q8_0 ? 0 : (int)(li & 3u);
+    // byte offset of this lane's piece inside a row at step 0, and its advance per step
+    const uint32_t boff0 = (TYPE == HQ_Q8_0 ? li : li >> 2) * BYTES;
+    const uint32_t bstep = (TYPE == HQ_Q8_0 ? L : L >> 2) * BYTES;
 
-    const uint8_t* rowp[R];
-#pragma unroll
-    for (int u = 0; u < R; ++u) {
-        uint32_t r = row0 + u * rpw;
+    // Address of slot u's row (clamped to the last row: always a valid read).
+    const uint8_t* wl = w + boff0;
+    auto row_ptr = [&](int u) -> const uint8_t* {
+        uint32_t r = row0 + (uint32_t)u * rpw;
         r = r < a.n ? r : a.n - 1u;
-        rowp[u] = w + (size_t)r * row_bytes;
-    }
+        return wl + (size_t)r * row_bytes;
+    };
 
-    float acc[R];
+    // First D fetches go out before the activations are staged, so their latency
+    // overlaps the staging and its barrier.
+    Piece<TYPE> buf[D];
 #pragma unroll
-    for (int u = 0; u < R; ++u) acc[u] = 0.f;
+    for (int u = 0; u < D; ++u) buf[u].load(row_ptr(u), c);
 
-    for (uint32_t pc = li; pc < pieces; pc += L) {
-        // piece -> (block, sub-piece) and its byte offset in the row
-        const int c = TYPE == HQ_Q8_0 ? 0 : (int)(pc & 3u);
-        const size_t boff = (size_t)(TYPE == HQ_Q8_0 ? pc : pc >> 2) * BYTES;
-        Piece<TYPE> pr[R];
+    const size_t xbytes = X_BF16 ? 2 : 4;
+    stage_x<X_BF16, PAIR>(static_cast<const uint8_t*>(a.x) + (size_t)(p / a.top_k) * a.k * xbytes, a.k, lds_x,
+                          lds_s);
+
+    // The conversion masks must sit in VGPRs for v_and_or_b32 (one scalar operand
+    // at most per VALU op on gfx9); the copy is opaque so they stay there.
+    uint32_t m4, m2, magic;
+    asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
+                 : "=v"(m4), "=v"(m2), "=v"(magic)
+                 : "s"(a.m4), "s"(a.m2), "s"(a.magic));
+
+    float acc[NR];
 #pragma unroll
-        for (int u = 0; u < R; ++u) pr[u].load(rowp[u] + boff, c);
+    for (int u = 0; u < NR; ++u) acc[u] = 0.f;
 
-        // Activations of this piece.  Q4_K: 64 consecutive; Q6_K: four runs of 16 at
-        // stride 32 inside one 128-element half; Q8_0: 32 consecutive.
+    __syncthreads();
+
+    for (uint32_t s = 0; s < steps; ++s) {
         uint32_t xr[XW];
         float sx[4];
-        if constexpr (TYPE == HQ_Q6_K) {
-            const uint32_t e0 = (pc >> 2) * 256u + (uint32_t)(c >> 1) * 128u + (uint32_t)(c & 1) * 16u;
+        load_x_piece<TYPE, PAIR, XW>(lds_x, lds_s, li + s * L, c, xr, sx);
+        const bool more = s + 1 < steps;  // uniform
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const uint32_t e = e0 + 32u * r;
-                const uint4* src = reinterpret_cast<const uint4*>(lds_x + (PAIR ? e / 2 : e));
-#pragma unroll
-                for (int j = 0; j < XW / 16; ++j) {
-                    const uint4 t = src[j];
-                    xr[(XW / 4) * r + 4 * j] = t.x;
-                    xr[(XW / 4) * r + 4 * j + 1] = t.y;
-                    xr[(XW / 4) * r + 4 * j + 2] = t.z;
-                    xr[(XW / 4) * r + 4 * j + 3] = t.w;
-                }
-                sx[r] = lds_s[e / 16];
-            }
-        } else {
-            const uint32_t e0 = pc * EPL;
-            const uint4* src = reinterpret_cast<const uint4*>(lds_x + (PAIR ? e0 / 2 : e0));
-#pragma unroll
-            for (int j = 0; j < XW / 4; ++j) {
-                const uint4 t = src[j];
-                xr[4 * j] = t.x;
-                xr[4 * j + 1] = t.y;
-                xr[4 * j + 2] = t.z;
-                xr[4 * j + 3] = t.w;
-            }
-#pragma unroll
-            for (int r = 0; r < EPL / 16; ++r) sx[r] = lds_s[e0 / 16 + r];
-        }
-
-#pragma unroll
-        for (int u = 0; u < R; ++u) {
+        for (int u = 0; u < NR; ++u) {
+            Piece<TYPE>& b = buf[u % D];
             if constexpr (PAIR)
-                acc[u] += dot_pair(pr[u], c, xr, sx);
+                acc[u] += dot_pair(b, c, xr, sx, m4, m2, magic);
             else
-                acc[u] += dot_f32(pr[u], c, reinterpret_cast<const float*>(xr), sx);
+                acc[u] += dot_f32(b, c, reinterpret_cast<const float*>(xr), sx);
+            // refill this buffer with the task D ahead: same step while slots remain,
+            // else the first slots of the next step
+            if (u + D < NR || more) {
+                const uint8_t* nxt = u + D < NR ? row_ptr(u + D) + (size_t)s * bstep
+                                                : row_ptr(u + D - NR) + (size_t)(s + 1) * bstep;
+                // Tie the refill to this task's result: without the (empty) asm the
+                // compiler hoists every refill above the arithmetic into fresh
+                // registers, which doubles the buffers and halves occupancy.
+                asm volatile("" : "+v"(nxt) : "v"(acc[u]));
+                b.load(nxt, c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
-    // Reduce over the L lanes of a row (xor butterflies with constant masks).
 #pragma unroll
-    for (int u = 0; u < R; ++u) {
-        float v = acc[u];
-        if (L > 32u) v += __shfl_xor(v, 32);
-        if (L > 16u) v += __shfl_xor(v, 16);
-        if (L > 8u) v += __shfl_xor(v, 8);
-        if (L > 4u) v += __shfl_xor(v, 4);
-        if (L > 2u) v += __shfl_xor(v, 2);
-        if (L > 1u) v += __shfl_xor(v, 1);
-        const uint32_t r = row0 + u * rpw;
+    for (int u = 0; u < NR; ++u) {
+        const float v = group_sum(acc[u], a.log_l);
+        const uint32_t r = row0 + (uint32_t)u * rpw;
         if (li == 0 && r < a.n) a.y[(size_t)p * a.n + r] = valid ? v : __builtin_nanf("");
     }
 }
 
-template <int TYPE, bool X_BF16, bool PAIR, int R>
-int launch_r(hipStream_t s, const KArgs& ka, uint32_t pairs, uint32_t rows_per_wg, size_t lds) {
-    auto kern = gemv_kernel<TYPE, X_BF16, PAIR, R>;
+template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
+int launch_r(hipStream_t s, const KArgs& ka, uint32_t pairs, uint32_t rpw, size_t lds) {
+    auto kern = gemv_kernel<TYPE, X_BF16, PAIR, NR, D>;
     if (lds > 64 * 1024) {
         if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                                "hipFuncSetAttribute(gemv LDS)"))
             return rc;
     }
+    const uint32_t rows_per_wg = 4 * rpw * NR;
     const dim3 grid((ka.n + rows_per_wg - 1) / rows_per_wg, pairs);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, ka);
     return check_launch("gemv kernel launch");
@@ -377,21 +442,25 @@ template <int TYPE, bool X_BF16>
 int launch_t(hipStream_t s, const GemvArgs& a) {
     constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
     constexpr int EPL = Lane<TYPE>::kElems;
-    KArgs ka{a.x, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0};
+    KArgs ka{a.x, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, M4, M2, MAGIC};
     const uint32_t pieces = a.k / EPL;
+    // L = largest power of two <= 64 that divides the pieces of a row
     uint32_t log_l = 0;
-    while (log_l < 6 && (2u << log_l) <= pieces) ++log_l;
+    while (log_l < 6 && pieces % (2u << log_l) == 0) ++log_l;
     ka.log_l = log_l;
     const uint32_t rpw = 64u >> log_l;
     const size_t lds = (size_t)(PAIR ? a.k * 2 : a.k * 4) + (size_t)(a.k / 16) * 4;
     if (lds > 160 * 1024 - 512)
         return fail(HQ_ERR_UNSUPPORTED, "gemv: k = %u needs %zu bytes of LDS (limit 160 KiB)", a.k, lds);
-    // Rows kept in flight per lane: as many as still leave >= 2 workgroups per CU.
-    const uint64_t want_wgs = 512;
-    auto wgs = [&](uint32_t r) { return (uint64_t)((a.n + 4 * rpw * r - 1) / (4 * rpw * r)) * a.pairs; };
-    if (wgs(4) >= want_wgs) return launch_r<TYPE, X_BF16, PAIR, 4>(s, ka, a.pairs, 4 * rpw * 4, lds);
-    if (wgs(2) >= want_wgs) return launch_r<TYPE, X_BF16, PAIR, 2>(s, ka, a.pairs, 4 * rpw * 2, lds);
-    return launch_r<TYPE, X_BF16, PAIR, 1>(s, ka, a.pairs, 4 * rpw, lds);
+    // Tasks (row slot x step) one SIMD would get if the work were spread evenly over
+    // 256 CUs x 4 SIMDs; more slots per wave amortise the per-wave set-up, fewer keep
+    // every SIMD busy on small problems.
+    const uint64_t slots = (uint64_t)((a.n + rpw - 1) / rpw) * a.pairs;
+    const uint64_t per_simd = slots / 1024;
+    if (per_simd >= 32) return launch_r<TYPE, X_BF16, PAIR, 8, 4>(s, ka, a.pairs, rpw, lds);
+    if (per_simd >= 8) return launch_r<TYPE, X_BF16, PAIR, 4, 2>(s, ka, a.pairs, rpw, lds);
+    if (per_simd >= 2) return launch_r<TYPE, X_BF16, PAIR, 2, 2>(s, ka, a.pairs, rpw, lds);
+    return launch_r<TYPE, X_BF16, PAIR, 1, 1>(s, ka, a.pairs, rpw, lds);
 }
 
 }  // namespace

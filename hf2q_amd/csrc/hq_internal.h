@@ -85,25 +85,35 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
                                            __builtin_bit_cast(bf16x2_t, b), c, false);
 }
 
+// (a & b) | c in one VALU op.  The compiler splits this into v_and + v_or when b
+// and c are literals (gfx9 VOP3 takes no literal operands), so the constants are
+// passed in registers and the instruction is written out.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t b, uint32_t c) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // Q4_K: 6-bit scale / min of sub-blocks (2c, 2c+1) for chunk c in [0,4) from the
 // 12 packed bytes held as three little-endian words (y = bytes 0..3, z = 4..7,
 // w = 8..11).  Same bit fields as get_scale_min_k4
 // (src/quantize/ggml_quants/q4_k.rs:329-337), evaluated branch-free.
 __device__ __forceinline__ void q4k_scales(uint32_t y, uint32_t z, uint32_t w, int c, uint32_t& sc0,
                                            uint32_t& sc1, uint32_t& m0, uint32_t& m1) {
+    // c < 2: sc = y.byte & 63, m = z.byte & 63.
+    // c >= 2: sc = (w.byte & 15) | ((y.byte >> 6) << 4), m = (w.byte >> 4) | ((z.byte >> 6) << 4).
+    // Selected with masks that depend on c only, so no divergent branch is formed.
     const int sh = (c & 1) * 16;
+    const uint32_t sel = c < 2 ? 0xffffffffu : 0u;  // take y/z bytes directly
+    const uint32_t lo = c < 2 ? 63u : 15u;
+    const uint32_t hb = c < 2 ? 0u : 0x30u;
     const uint32_t ys = y >> sh, zs = z >> sh, ws = w >> sh;
-    if (c < 2) {
-        sc0 = ys & 63u;
-        sc1 = (ys >> 8) & 63u;
-        m0 = zs & 63u;
-        m1 = (zs >> 8) & 63u;
-    } else {
-        sc0 = (ws & 0xFu) | ((ys >> 2) & 0x30u);
-        sc1 = ((ws >> 8) & 0xFu) | ((ys >> 10) & 0x30u);
-        m0 = ((ws >> 4) & 0xFu) | ((zs >> 2) & 0x30u);
-        m1 = ((ws >> 12) & 0xFu) | ((zs >> 10) & 0x30u);
-    }
+    const uint32_t a = (ys & sel) | (ws & ~sel);
+    const uint32_t b = (zs & sel) | ((ws >> 4) & ~sel);
+    sc0 = (a & lo) | ((ys >> 2) & hb);
+    sc1 = ((a >> 8) & lo) | ((ys >> 10) & hb);
+    m0 = (b & lo) | ((zs >> 2) & hb);
+    m1 = ((b >> 8) & lo) | ((zs >> 10) & hb);
 }
 
 __device__ __forceinline__ float ubyte0(uint32_t v) { return static_cast<float>(v & 0xffu); }
