@@ -1,6 +1,432 @@
+// Device-side GGML quantizers for Q4_K / Q6_K / Q8_0, byte-identical to hf2q's
+// CPU quantizers without an importance matrix
+// (src/quantize/ggml_quants/q4_k.rs:89-217, q6_k.rs:40-151, q8_0.rs:31-72 and the
+// search helpers common.rs:61-167, 174-286).  hf2q quantizes on the host at
+// conversion / load time (in_memory_loader.rs:70-139); here the same bytes are
+// produced on the GPU so that weights never have to cross PCIe as f32.
+//
+// Byte equality needs the same sequence of f32 roundings, so this file is built
+// with -ffp-contract=off and uses fmaf exactly where the reference writes
+// mul_add; divisions and sqrt are the correctly rounded ones (the HIP default).
+// The scale search over a sub-block is an inherently sequential f32
+// accumulation, so the parallelism is across sub-blocks: one thread per
+// 32-element (Q4_K) or 16-element (Q6_K) sub-block, the super-block level
+// decisions (max scale, 6-bit / int8 scale codes, f16 d) are combined through
+// LDS, and the threads of a super-block then pack its bytes cooperatively.
+#include <math.h>
+
 #include "hq_internal.h"
+
 namespace hq {
-int launch_quantize(hipStream_t, const float*, uint64_t, uint64_t, hq_ggml_type, void*) {
-    return fail(HQ_ERR_UNSUPPORTED, "quantize: not built yet");
+namespace {
+
+constexpr float kGroupMaxEps = 1e-15f;  // common.rs:15
+
+// common.rs:23-28: round-half-even through the 1.5*2^23 magic add.
+__device__ __forceinline__ int nearest_int(float f) {
+    const float v = f + 12582912.f;
+    return (__float_as_int(v) & 0x007fffff) - 0x00400000;
 }
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));  // v_cvt_f16_f32, RNE
 }
+
+// ------------------------------------------------------------------ Q8_0
+// q8_0.rs:31-72.  One thread per 32-element block.
+__global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restrict__ src, uint8_t* __restrict__ out,
+                                                            uint64_t n_blocks) {
+    const uint64_t b = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= n_blocks) return;
+    float x[32];
+    const float4* s4 = reinterpret_cast<const float4*>(src + b * 32);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float4 t = s4[i];
+        x[4 * i] = t.x;
+        x[4 * i + 1] = t.y;
+        x[4 * i + 2] = t.z;
+        x[4 * i + 3] = t.w;
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const float a = fabsf(x[i]);
+        if (a > amax) amax = a;
+    }
+    const float d = amax / 127.f;
+    const float id = d != 0.f ? 1.f / d : 0.f;
+    uint8_t* o = out + b * Q8_0_BYTES;
+    *reinterpret_cast<uint16_t*>(o) = (uint16_t)f32_to_f16_bits(d);
+#pragma unroll
+    for (int i = 0; i < 32; i += 2) {
+        // Rust's f32::round is half-away-from-zero == roundf; `as i8` saturates.
+        float r0 = roundf(x[i] * id), r1 = roundf(x[i + 1] * id);
+        r0 = fminf(fmaxf(r0, -128.f), 127.f);
+        r1 = fminf(fmaxf(r1, -128.f), 127.f);
+        const uint32_t q0 = (uint32_t)(int)r0 & 0xffu, q1 = (uint32_t)(int)r1 & 0xffu;
+        *reinterpret_cast<uint16_t*>(o + 2 + i) = (uint16_t)(q0 | (q1 << 8));
+    }
+}
+
+// ------------------------------------------------------------------ Q4_K
+// common.rs:174-286 make_qkx2_quants with n = 32, nmax = 15, rmin = -1,
+// rdelta = 0.1, nstep = 20, use_mad = false (the arguments of q4_k.rs:120-132).
+// L comes back packed four codes per word.
+__device__ float qkx2_search_32(const float (&x)[32], const float (&wt)[32], uint32_t (&Lp)[8], float& the_min) {
+    constexpr int nmax = 15;
+    float mn = x[0], mx = x[0];
+    float sum_w = wt[0];
+    float sum_x = sum_w * x[0];
+#pragma unroll
+    for (int i = 1; i < 32; ++i) {
+        if (x[i] < mn) mn = x[i];
+        if (x[i] > mx) mx = x[i];
+        sum_w += wt[i];
+        sum_x = fmaf(wt[i], x[i], sum_x);
+    }
+    if (mn > 0.f) mn = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) Lp[i] = 0;
+    if (mx == mn) {
+        the_min = -mn;
+        return 0.f;
+    }
+    float iscale = (float)nmax / (mx - mn);
+    float scale = 1.f / iscale;
+    float best_error = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        int l = nearest_int(iscale * (x[i] - mn));
+        l = max(0, min(nmax, l));
+        Lp[i >> 2] |= (uint32_t)l << (8 * (i & 3));
+        float diff = fmaf(scale, (float)l, mn) - x[i];
+        diff = diff * diff;
+        best_error = fmaf(wt[i], diff, best_error);
+    }
+    for (int is = 0; is <= 20; ++is) {
+        iscale = (-1.f + 0.1f * (float)is + (float)nmax) / (mx - mn);
+        float sum_l = 0.f, sum_l2 = 0.f, sum_xl = 0.f;
+        uint32_t La[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) La[i] = 0;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            int l = nearest_int(iscale * (x[i] - mn));
+            l = max(0, min(nmax, l));
+            La[i >> 2] |= (uint32_t)l << (8 * (i & 3));
+            const float lf = (float)l, w = wt[i];
+            sum_l = fmaf(w, lf, sum_l);
+            sum_l2 = fmaf(w * lf, lf, sum_l2);
+            sum_xl = fmaf(w * lf, x[i], sum_xl);
+        }
+        const float D = fmaf(sum_w, sum_l2, -sum_l * sum_l);
+        if (D > 0.f) {
+            float this_scale = fmaf(sum_w, sum_xl, -sum_x * sum_l) / D;
+            float this_min = fmaf(sum_l2, sum_x, -sum_l * sum_xl) / D;
+            if (this_min > 0.f) {
+                this_min = 0.f;
+                this_scale = sum_xl / sum_l2;
+            }
+            float cur_error = 0.f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const float lf = (float)((La[i >> 2] >> (8 * (i & 3))) & 0xffu);
+                float diff = fmaf(this_scale, lf, this_min) - x[i];
+                diff = diff * diff;
+                cur_error = fmaf(wt[i], diff, cur_error);
+            }
+            if (cur_error < best_error) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) Lp[i] = La[i];
+                best_error = cur_error;
+                scale = this_scale;
+                mn = this_min;
+            }
+        }
+    }
+    the_min = -mn;
+    return scale;
+}
+
+// q4_k.rs:89-217.  256 threads = 32 super-blocks x 8 sub-block threads.
+__global__ __launch_bounds__(256) void quantize_q4_k_kernel(const float* __restrict__ src, uint8_t* __restrict__ out,
+                                                            uint64_t n_blocks) {
+    __shared__ float s_scale[256], s_min[256];
+    __shared__ uint32_t s_code[256];   // ls | lm << 8 per sub-block
+    __shared__ uint32_t s_L[256 * 8];  // packed codes of every sub-block (32 bytes each)
+
+    const uint32_t tid = threadIdx.x, j = tid & 7u, lb = tid >> 3;
+    uint64_t blk = (uint64_t)blockIdx.x * 32 + lb;
+    const bool live = blk < n_blocks;
+    if (!live) blk = n_blocks - 1;  // keep every thread in the barriers; its result is discarded
+
+    float x[32], wt[32];
+    const float4* s4 = reinterpret_cast<const float4*>(src + blk * 256 + 32 * j);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float4 t = s4[i];
+        x[4 * i] = t.x;
+        x[4 * i + 1] = t.y;
+        x[4 * i + 2] = t.z;
+        x[4 * i + 3] = t.w;
+    }
+    float sum_x2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) sum_x2 = fmaf(x[i], x[i], sum_x2);
+    const float av_x = sqrtf(sum_x2 / 32.f);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) wt[i] = av_x + fabsf(x[i]);
+
+    uint32_t Lp[8];
+    float the_min;
+    const float scale = qkx2_search_32(x, wt, Lp, the_min);
+    s_scale[tid] = scale;
+    s_min[tid] = the_min;
+    __syncthreads();
+
+    // Super-block maxima in sub-block order (strict > like the reference's scan).
+    float max_scale = 0.f, max_min = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const float sc = s_scale[lb * 8 + t], mi = s_min[lb * 8 + t];
+        if (sc > max_scale) max_scale = sc;
+        if (mi > max_min) max_min = mi;
+    }
+    const float inv_scale = max_scale > 0.f ? 63.f / max_scale : 0.f;
+    const float inv_min = max_min > 0.f ? 63.f / max_min : 0.f;
+    uint32_t ls = (uint32_t)nearest_int(inv_scale * scale) & 0xffu;  // `as u8` truncation
+    uint32_t lm = (uint32_t)nearest_int(inv_min * the_min) & 0xffu;
+    ls = ls > 63u ? 63u : ls;
+    lm = lm > 63u ? 63u : lm;
+    s_code[tid] = ls | (lm << 8);
+
+    // Second stage with the f16-rounded d / dmin (q4_k.rs:181-197).
+    const uint32_t d16 = f32_to_f16_bits(max_scale / 63.f), dmin16 = f32_to_f16_bits(max_min / 63.f);
+    const float d = f16_bits_to_f32(d16) * (float)ls;
+    if (d != 0.f) {
+        const float dm = f16_bits_to_f32(dmin16) * (float)lm;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) Lp[i] = 0;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            int l = nearest_int((x[i] + dm) / d);
+            l = max(0, min(15, l));
+            Lp[i >> 2] |= (uint32_t)l << (8 * (i & 3));
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s_L[tid * 8 + i] = Lp[i];
+    __syncthreads();
+    if (!live) return;
+
+    // Pack: thread j writes the header (j == 0) and 16 bytes of qs.  Chunk c = j/2,
+    // half h = j%2: bytes 16h..16h+15 of the chunk combine code l of sub-block 2c
+    // (low nibble) with code l of sub-block 2c+1 (high nibble), l = 16h + i.
+    uint8_t* o = out + blk * Q4K_BYTES;
+    if (j == 0) {
+        uint32_t sc[8], mi[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            sc[t] = s_code[lb * 8 + t] & 0xffu;
+            mi[t] = s_code[lb * 8 + t] >> 8;
+        }
+        uint32_t q[12];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            q[t] = sc[t] | ((sc[t + 4] >> 4) << 6);
+            q[t + 4] = mi[t] | ((mi[t + 4] >> 4) << 6);
+            q[t + 8] = (sc[t + 4] & 0xFu) | ((mi[t + 4] & 0xFu) << 4);
+        }
+        uint4 hdr;
+        hdr.x = d16 | (dmin16 << 16);
+        hdr.y = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
+        hdr.z = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
+        hdr.w = q[8] | (q[9] << 8) | (q[10] << 16) | (q[11] << 24);
+        *reinterpret_cast<uint4*>(o) = hdr;
+    }
+    const uint32_t c = j >> 1, h = j & 1u;
+    const uint32_t* lo = &s_L[(lb * 8 + 2 * c) * 8 + 4 * h];
+    const uint32_t* hi = &s_L[(lb * 8 + 2 * c + 1) * 8 + 4 * h];
+    uint4 qs;
+    qs.x = lo[0] | (hi[0] << 4);
+    qs.y = lo[1] | (hi[1] << 4);
+    qs.z = lo[2] | (hi[2] << 4);
+    qs.w = lo[3] | (hi[3] << 4);
+    *reinterpret_cast<uint4*>(o + 16 + 32 * c + 16 * h) = qs;
+}
+
+// ------------------------------------------------------------------ Q6_K
+// common.rs:61-167 make_qx_quants with n = 16, nmax = 32, rmse_type = 1, no
+// weights (q6_k.rs:58).  Codes come back as L = l + 32, one per byte.
+__device__ float qx_search_16(const float (&x)[16], uint32_t (&Lp)[4]) {
+    constexpr int nmax = 32;
+    float mx = 0.f, amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const float ax = fabsf(x[i]);
+        if (ax > amax) {
+            amax = ax;
+            mx = x[i];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) Lp[i] = 0;
+    if (amax < kGroupMaxEps) return 0.f;
+    float iscale = -(float)nmax / mx;
+    float sumlx = 0.f, suml2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        int l = nearest_int(iscale * x[i]);
+        l = max(-nmax, min(nmax - 1, l));
+        Lp[i >> 2] |= (uint32_t)(l + nmax) << (8 * (i & 3));
+        const float w = x[i] * x[i];
+        sumlx = fmaf(w * x[i], (float)l, sumlx);
+        suml2 = fmaf(w * (float)l, (float)l, suml2);
+    }
+    float scale = suml2 != 0.f ? sumlx / suml2 : 0.f;
+    float best = scale * sumlx;
+    for (int is = -9; is <= 9; ++is) {
+        if (is == 0) continue;
+        iscale = -((float)nmax + 0.1f * (float)is) / mx;
+        sumlx = 0.f;
+        suml2 = 0.f;
+        uint32_t La[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            int l = nearest_int(iscale * x[i]);
+            l = max(-nmax, min(nmax - 1, l));
+            La[i >> 2] |= (uint32_t)(l + nmax) << (8 * (i & 3));
+            const float w = x[i] * x[i];
+            sumlx = fmaf(w * x[i], (float)l, sumlx);
+            suml2 = fmaf(w * (float)l, (float)l, suml2);
+        }
+        if (suml2 > 0.f && sumlx * sumlx > best * suml2) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) Lp[i] = La[i];
+            scale = sumlx / suml2;
+            best = scale * sumlx;
+        }
+    }
+    return scale;
+}
+
+// q6_k.rs:40-151.  256 threads = 16 super-blocks x 16 sub-block threads.
+__global__ __launch_bounds__(256) void quantize_q6_k_kernel(const float* __restrict__ src, uint8_t* __restrict__ out,
+                                                            uint64_t n_blocks) {
+    __shared__ float s_scale[256];
+    __shared__ uint32_t s_L[256 * 4];  // 16 code bytes per sub-block = the 256 codes of a super-block in order
+    __shared__ int s_sc[256];
+
+    const uint32_t tid = threadIdx.x, ib = tid & 15u, lb = tid >> 4;
+    uint64_t blk = (uint64_t)blockIdx.x * 16 + lb;
+    const bool live = blk < n_blocks;
+    if (!live) blk = n_blocks - 1;
+
+    float x[16];
+    const float4* s4 = reinterpret_cast<const float4*>(src + blk * 256 + 16 * ib);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float4 t = s4[i];
+        x[4 * i] = t.x;
+        x[4 * i + 1] = t.y;
+        x[4 * i + 2] = t.z;
+        x[4 * i + 3] = t.w;
+    }
+    uint32_t Lp[4];
+    const float scale = qx_search_16(x, Lp);
+    s_scale[tid] = scale;
+    __syncthreads();
+
+    // First sub-block with the largest |scale| (strict > in sub-block order).
+    float max_scale = 0.f, max_abs = 0.f;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        const float sc = s_scale[lb * 16 + t];
+        if (fabsf(sc) > max_abs) {
+            max_abs = fabsf(sc);
+            max_scale = sc;
+        }
+    }
+    const bool zero_block = max_abs < kGroupMaxEps;
+    uint32_t d16 = 0;
+    int sc8 = 0;
+    if (!zero_block) {
+        const float iscale = -128.f / max_scale;
+        d16 = f32_to_f16_bits(1.f / iscale);
+        sc8 = min(127, nearest_int(iscale * scale));
+        sc8 = (int)(int8_t)sc8;  // stored as int8
+        const float d = f16_bits_to_f32(d16) * (float)sc8;
+        if (d != 0.f) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) Lp[i] = 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                int l = nearest_int(x[i] / d);
+                l = max(-32, min(31, l));
+                Lp[i >> 2] |= (uint32_t)(l + 32) << (8 * (i & 3));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) Lp[i] = 0;  // memset block (q6_k.rs:67-74)
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_L[tid * 4 + i] = Lp[i];
+    s_sc[tid] = sc8;
+    __syncthreads();
+    if (!live) return;
+
+    // Pack (q6_k.rs:112-150): thread ib covers half h = ib/8 and the four columns
+    // l = 4*(ib%8) .. +3 of that half: 4 bytes of ql[l], 4 of ql[l+32], 4 of qh[l].
+    uint8_t* o = out + blk * Q6K_BYTES;
+    const uint32_t h = ib >> 3, l0 = 4 * (ib & 7u);
+    const uint8_t* Lb = reinterpret_cast<const uint8_t*>(&s_L[lb * 64]) + 128 * h + l0;
+    uint32_t ql_a = 0, ql_b = 0, qh = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t a = Lb[i], b = Lb[i + 32], c = Lb[i + 64], e = Lb[i + 96];
+        ql_a |= ((a & 0xFu) | ((c & 0xFu) << 4)) << (8 * i);
+        ql_b |= ((b & 0xFu) | ((e & 0xFu) << 4)) << (8 * i);
+        qh |= ((a >> 4) | ((b >> 4) << 2) | ((c >> 4) << 4) | ((e >> 4) << 6)) << (8 * i);
+    }
+    // 210-byte blocks are only 2-byte aligned: store as 16-bit halves.
+    uint16_t* p;
+    p = reinterpret_cast<uint16_t*>(o + 64 * h + l0);
+    p[0] = (uint16_t)ql_a;
+    p[1] = (uint16_t)(ql_a >> 16);
+    p = reinterpret_cast<uint16_t*>(o + 64 * h + 32 + l0);
+    p[0] = (uint16_t)ql_b;
+    p[1] = (uint16_t)(ql_b >> 16);
+    p = reinterpret_cast<uint16_t*>(o + 128 + 32 * h + l0);
+    p[0] = (uint16_t)qh;
+    p[1] = (uint16_t)(qh >> 16);
+    o[192 + ib] = zero_block ? 0 : (uint8_t)s_sc[lb * 16 + ib];
+    if (ib == 0) *reinterpret_cast<uint16_t*>(o + 208) = (uint16_t)d16;
+}
+
+}  // namespace
+
+int launch_quantize(hipStream_t s, const float* src, uint64_t n_elems, uint64_t n_per_row, hq_ggml_type t,
+                    void* out) {
+    (void)n_per_row;  // rows are contiguous runs of whole blocks; no imatrix, so no per-row state
+    uint8_t* o = static_cast<uint8_t*>(out);
+    if (t == HQ_Q8_0) {
+        const uint64_t nb = n_elems / 32;
+        if ((nb + 255) / 256 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
+        hipLaunchKernelGGL(quantize_q8_0_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, src, o, nb);
+    } else if (t == HQ_Q4_K) {
+        const uint64_t nb = n_elems / 256;
+        if ((nb + 31) / 32 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
+        hipLaunchKernelGGL(quantize_q4_k_kernel, dim3((unsigned)((nb + 31) / 32)), dim3(256), 0, s, src, o, nb);
+    } else if (t == HQ_Q6_K) {
+        const uint64_t nb = n_elems / 256;
+        if ((nb + 15) / 16 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
+        hipLaunchKernelGGL(quantize_q6_k_kernel, dim3((unsigned)((nb + 15) / 16)), dim3(256), 0, s, src, o, nb);
+    } else {
+        return fail(HQ_ERR_UNSUPPORTED, "quantize: ggml type %d", (int)t);
+    }
+    return check_launch("quantize kernel launch");
+}
+
+}  // namespace hq

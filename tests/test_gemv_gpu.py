@@ -166,3 +166,48 @@ def test_mul_mat_id_invariants(oracle, dev):
     y4 = torch.empty_like(y)
     ops.quantized_matmul_id_ggml(x, stack, bad, y4, p)
     assert torch.isnan(y4[3]).all() and torch.equal(y4[[0, 1, 2, 4, 5, 6, 7]], y[[0, 1, 2, 4, 5, 6, 7]])
+
+
+# ---- device-side quantizer ------------------------------------------------------------
+
+@pytest.mark.parametrize("t", TYPES)
+def test_quantizer_matches_reference_golden_bytes(oracle, dev, t):
+    """The reference's own byte-equality fixtures (q4_k.rs:386-393, q6_k.rs:272-279, q8_0.rs:106-113)."""
+    import os
+    from _util import GOLDEN
+    name, npr = {HQ_Q4_K: ("q4_k_512", 512), HQ_Q6_K: ("q6_k_512", 512), HQ_Q8_0: ("q8_0_64", 64)}[t]
+    x = np.fromfile(os.path.join(GOLDEN, "ggml_quants", f"{name}_noim_input.bin"), dtype=np.float32)
+    want = np.fromfile(os.path.join(GOLDEN, "ggml_quants", f"{name}_noim_expected.bin"), dtype=np.uint8)
+    got = ops.quantize_ggml(torch.from_numpy(x).to(dev), npr, t).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_quantizer_byte_equal_to_oracle(oracle, dev, t):
+    rng = np.random.default_rng(40 + t)
+    parts = [
+        (rng.standard_normal(300 * 256) * 0.02).astype(np.float32),          # the benchmark's weight distribution
+        rng.uniform(-1, 1, 40 * 256).astype(np.float32),
+        (rng.standard_normal(40 * 256) ** 3).astype(np.float32),              # heavy tails
+        np.zeros(2 * 256, np.float32),                                       # zero blocks
+        np.full(256, 0.37, np.float32), np.full(256, -1e-3, np.float32),     # constant blocks
+        (rng.standard_normal(8 * 256) * 1e-18).astype(np.float32),           # below GROUP_MAX_EPS
+        (rng.standard_normal(8 * 256) * 3e4).astype(np.float32),             # near the f16 range of d
+        np.abs(rng.standard_normal(8 * 256)).astype(np.float32),             # all positive (min clamps to 0)
+        np.where(rng.random(8 * 256) < 0.9, 0, rng.standard_normal(8 * 256)).astype(np.float32),  # sparse
+    ]
+    x = np.concatenate(parts)
+    want = oracle.quantize(x, 256, t, threads=8)
+    got = ops.quantize_ggml(torch.from_numpy(x).to(dev), 256, t).cpu().numpy()
+    bb = oracle.BLOCK_BYTES[t]
+    bad = np.nonzero((got.reshape(-1, bb) != want.reshape(-1, bb)).any(axis=1))[0]
+    assert bad.size == 0, f"{bad.size} blocks differ, first {bad[:5]}"
+
+
+def test_quantizer_rejects_bad_shapes(dev):
+    # quantizer.rs:217-235
+    x = torch.zeros(768, device=dev)
+    with pytest.raises(ops.HqError):
+        ops.quantize_ggml(x, 300, HQ_Q4_K)
+    with pytest.raises(ops.HqError):
+        ops.quantize_ggml(x, 512, HQ_Q4_K)
