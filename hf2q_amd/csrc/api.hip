@@ -110,21 +110,26 @@ int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w
                     uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
     if (int rc = check_matmul_common("hq_qmatmul_ggml", x, xdt, w_blocks, y, n, k, t)) return rc;
     if (m == 0) return HQ_OK;
-    if (m <= kGemvMaxRows) {
+    if (m > kGemvMaxRows && gemm_supported(t, k))
+        return launch_gemm((hipStream_t)stream, x, xdt, w_blocks, y, m, n, k, t);
+    // GEMV form, kGemvMaxRows activation rows per launch (also the route of shapes the
+    // tile kernel does not cover).
+    const size_t xrow_bytes = (size_t)k * (xdt == HQ_BF16 ? 2 : 4);
+    for (uint32_t r0 = 0; r0 < m; r0 += kGemvMaxRows) {
         GemvArgs a{};
-        a.x = x;
+        a.x = static_cast<const uint8_t*>(x) + (size_t)r0 * xrow_bytes;
         a.w = static_cast<const uint8_t*>(w_blocks);
         a.ids = nullptr;
-        a.y = y;
-        a.pairs = m;
+        a.y = y + (size_t)r0 * n;
+        a.pairs = m - r0 < kGemvMaxRows ? m - r0 : kGemvMaxRows;
         a.top_k = 1;
         a.n = n;
         a.k = k;
         a.n_experts = 1;
         a.expert_stride = 0;
-        return launch_gemv((hipStream_t)stream, a, xdt, t);
+        if (int rc = launch_gemv((hipStream_t)stream, a, xdt, t)) return rc;
     }
-    return fail(HQ_ERR_UNSUPPORTED, "hq_qmatmul_ggml: m = %u (> %u) needs the GEMM path", m, kGemvMaxRows);
+    return HQ_OK;
 }
 
 size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows) {

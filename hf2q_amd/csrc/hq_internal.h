@@ -40,6 +40,11 @@ struct GemvArgs {
 };
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t);
 
+// MFMA GEMM for m > 8 (prefill).  gemm_supported() says whether (type, k) has a tile kernel.
+bool gemm_supported(hq_ggml_type t, uint32_t k);
+int launch_gemm(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
+                uint32_t k, hq_ggml_type t);
+
 }  // namespace hq
 
 // ---------------------------------------------------------------------------

@@ -4,10 +4,11 @@ import numpy as np
 GOLDEN = __import__("os").path.join(__import__("os").path.dirname(__file__), "golden")
 
 # north_star tolerance for matmul outputs: 1e-3 relative to the f64 result
-# (fp32 accumulate).  The small absolute floor (1e-5 of the output RMS) only
-# matters for outputs that cancel to ~0.
+# (fp32 accumulate), element by element.  A dot product can cancel to ~0, where a
+# relative bound means nothing, so an absolute floor of 1e-4 of the output RMS is
+# added (observed errors are ~3e-6 of the RMS: fp32 accumulation noise).
 REL_TOL = 1e-3
-ABS_FLOOR = 1e-5
+ABS_FLOOR = 1e-4
 
 
 def assert_matmul_close(got, ref64, what=""):
