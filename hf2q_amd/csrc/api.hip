@@ -176,4 +176,71 @@ int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void
                 (unsigned long long)pairs);
 }
 
+static int check_fwht(const char* fn, const float* buf, uint32_t n_heads, uint32_t head_dim) {
+    if (head_dim != 256 && head_dim != 512) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: head_dim %u (256 or 512)", fn, head_dim);
+    if (n_heads && !buf) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (!is_aligned(buf, 16)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: buffer must be 16-byte aligned", fn);
+    return HQ_OK;
+}
+
+int hq_fwht_sign_premult_f32(void* stream, float* buf, uint32_t n_heads, uint32_t head_dim) {
+    if (int rc = check_fwht("hq_fwht_sign_premult_f32", buf, n_heads, head_dim)) return rc;
+    if (n_heads == 0) return HQ_OK;
+    return launch_fwht_sign((hipStream_t)stream, buf, n_heads, head_dim, false);
+}
+
+int hq_fwht_sign_undo_f32(void* stream, float* buf, uint32_t n_heads, uint32_t head_dim) {
+    if (int rc = check_fwht("hq_fwht_sign_undo_f32", buf, n_heads, head_dim)) return rc;
+    if (n_heads == 0) return HQ_OK;
+    return launch_fwht_sign((hipStream_t)stream, buf, n_heads, head_dim, true);
+}
+
+int hq_tq_encode_kv(void* stream, const float* src, uint8_t* codes, float* norms, uint32_t n_tokens,
+                    uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t write_pos) {
+    if (head_dim != 256 && head_dim != 512)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_tq_encode_kv: head_dim %u (256 or 512)", head_dim);
+    if (capacity == 0 || n_tokens > capacity)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_tq_encode_kv: %u tokens into a cache of capacity %u", n_tokens, capacity);
+    if (n_tokens == 0 || n_kv_heads == 0) return HQ_OK;
+    if (!src || !codes || !norms) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_tq_encode_kv: null buffer");
+    if (!is_aligned(src, 16) || !is_aligned(codes, 4) || !is_aligned(norms, 4))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_tq_encode_kv: src needs 16-byte, codes / norms 4-byte alignment");
+    return launch_tq_encode((hipStream_t)stream, src, codes, norms, n_tokens, n_kv_heads, head_dim, capacity,
+                            write_pos % capacity);
+}
+
+size_t hq_flash_attn_vec_tq_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len) {
+    return tq_attn_tmp_bytes(num_heads, head_dim, kv_seq_len);
+}
+
+int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
+                         const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
+                         void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p) {
+    const char* fn = "hq_flash_attn_vec_tq";
+    if (!p) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null params", fn);
+    if (p->head_dim != 256 && p->head_dim != 512)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: head_dim %u (256 or 512)", fn, p->head_dim);
+    if (p->kv_seq_len == 0) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: kv_seq_len is 0", fn);
+    if (p->kv_capacity < p->kv_seq_len)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: kv_capacity %u < kv_seq_len %u", fn, p->kv_capacity, p->kv_seq_len);
+    if (p->codebook_bits != 5 && p->codebook_bits != 6 && p->codebook_bits != 8)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: codebook_bits %u (5, 6 or 8)", fn, p->codebook_bits);
+    if (p->num_kv_heads == 0 || p->num_heads == 0 || p->num_heads % p->num_kv_heads)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: %u heads over %u kv heads", fn, p->num_heads, p->num_kv_heads);
+    if (p->mask_type > 2) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: mask_type %u", fn, p->mask_type);
+    if (p->ring_start >= p->kv_capacity) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: ring_start %u >= capacity", fn, p->ring_start);
+    if (!q || !k_codes || !k_norms || !v_codes || !v_norms || !out || !tmp)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (!is_aligned(q, 16) || !is_aligned(out, 16) || !is_aligned(k_codes, 16) || !is_aligned(v_codes, 16) ||
+        !is_aligned(tmp, 4))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: q / out / codes need 16-byte alignment", fn);
+    if (p->head_dim == 512) return fail(HQ_ERR_UNSUPPORTED, "%s: head_dim 512 is not built", fn);
+    if (p->codebook_bits != 8) return fail(HQ_ERR_UNSUPPORTED, "%s: only the 8-bit cache is built", fn);
+    if (tmp_bytes < tq_attn_tmp_bytes(p->num_heads, p->head_dim, p->kv_seq_len))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: tmp holds %zu bytes, %zu needed", fn, tmp_bytes,
+                    tq_attn_tmp_bytes(p->num_heads, p->head_dim, p->kv_seq_len));
+    return launch_tq_attention((hipStream_t)stream, q, k_codes, k_norms, v_codes, v_norms, lut256, out,
+                               static_cast<float*>(tmp), *p);
+}
+
 }  // extern "C"

@@ -45,6 +45,15 @@ bool gemm_supported(hq_ggml_type t, uint32_t k);
 int launch_gemm(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                 uint32_t k, hq_ggml_type t);
 
+// TurboQuant KV (tq.hip)
+int launch_fwht_sign(hipStream_t s, float* buf, uint32_t n_heads, uint32_t head_dim, bool undo);
+int launch_tq_encode(hipStream_t s, const float* src, uint8_t* codes, float* norms, uint32_t n_tokens,
+                     uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t write_pos);
+size_t tq_attn_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len);
+int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, const float* k_norms,
+                        const uint8_t* v_codes, const float* v_norms, const float* lut, float* out, float* tmp,
+                        const hq_tq_attn_params& p);
+
 }  // namespace hq
 
 // ---------------------------------------------------------------------------

@@ -38,7 +38,20 @@ SIGNATURES = {
     "hq_qmatmul_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32]),
     "hq_qmatmul_id_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _u32, _u32, _u32, _u32, _u32, _u64, _i32]),
     "hq_qmatmul_id_scratch_bytes": (_sz, [_u32, _u32]),
+    "hq_fwht_sign_premult_f32": (_i32, [_vp, _vp, _u32, _u32]),
+    "hq_fwht_sign_undo_f32": (_i32, [_vp, _vp, _u32, _u32]),
+    "hq_tq_encode_kv": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
+    "hq_flash_attn_vec_tq": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "hq_flash_attn_vec_tq_tmp_bytes": (_sz, [_u32, _u32, _u32]),
 }
+
+
+class TqAttnParams(ctypes.Structure):
+    """hq_tq_attn_params (include/hf2q_hip.h)."""
+    _fields_ = [("num_heads", _u32), ("num_kv_heads", _u32), ("head_dim", _u32), ("kv_seq_len", _u32),
+                ("kv_capacity", _u32), ("scale", _f32), ("mask_type", _u32), ("sliding_window", _u32),
+                ("softcap", _f32), ("ring_start", _u32), ("scale_factor_d512", _f32), ("codebook_bits", _u32),
+                ("fuse_fwht_pre", _u32), ("nsg", _u32)]
 
 _lib = None
 

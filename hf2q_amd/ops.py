@@ -117,3 +117,76 @@ def quantize_ggml(src: torch.Tensor, n_per_row: int, ggml_type: int) -> torch.Te
     L = _l.load()
     _l.check(L.hq_quantize_ggml(_stream(), _dev(src, "src"), n, n_per_row, ggml_type, _dev(out, "out")))
     return out
+
+
+# ---- TurboQuant-style 8-bit KV cache ------------------------------------------------------------
+
+@dataclass(frozen=True)
+class FlashAttnVecTqHbParams:
+    """forward_mlx.rs:4687-4705 / kv_cache.rs:589-614 (Qwen35TqSdpaParams)."""
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    kv_seq_len: int
+    kv_capacity: int
+    scale: float
+    mask_type: int = 0
+    sliding_window: int = 0
+    softcap: float = 0.0
+    ring_start: int = 0
+    scale_factor_d512: float = 1.0
+    codebook_bits: int = 8
+    fuse_fwht_pre: int = 0
+    nsg: int = 1
+
+
+def dispatch_fwht_sign_premult_f32(buf: torch.Tensor, num_heads: int, head_dim: int) -> None:
+    """forward_mlx.rs:4662-4666: in-place sign x FWHT of buf[num_heads, head_dim] (f32)."""
+    if buf.dtype != torch.float32:
+        raise TypeError("buf must be float32")
+    _l.check(_l.load().hq_fwht_sign_premult_f32(_stream(), _dev(buf, "buf"), num_heads, head_dim))
+
+
+def dispatch_fwht_sign_undo_f32(buf: torch.Tensor, num_heads: int, head_dim: int) -> None:
+    """forward_mlx.rs:4750: in-place FWHT x sign."""
+    if buf.dtype != torch.float32:
+        raise TypeError("buf must be float32")
+    _l.check(_l.load().hq_fwht_sign_undo_f32(_stream(), _dev(buf, "buf"), num_heads, head_dim))
+
+
+def alloc_tq_kv(n_kv_heads: int, capacity: int, head_dim: int, device) -> tuple[torch.Tensor, torch.Tensor]:
+    """kv_cache.rs:2026-2113: codes [n_kv_heads, capacity, head_dim] u8 + norms [.., head_dim/256] f32."""
+    codes = torch.zeros((n_kv_heads, capacity, head_dim), dtype=torch.uint8, device=device)
+    norms = torch.zeros((n_kv_heads, capacity, max(1, head_dim // 256)), dtype=torch.float32, device=device)
+    return codes, norms
+
+
+def hadamard_quantize_kv(src: torch.Tensor, codes: torch.Tensor, norms: torch.Tensor, write_pos: int) -> None:
+    """kv_cache.rs:180-213: encode src [n_tokens, n_kv_heads, head_dim] f32 at slots write_pos.. of the cache."""
+    if src.dtype != torch.float32 or codes.dtype != torch.uint8 or norms.dtype != torch.float32:
+        raise TypeError("src f32, codes u8, norms f32 expected")
+    n_tokens, n_kv_heads, head_dim = src.shape
+    capacity = codes.shape[1]
+    _l.check(_l.load().hq_tq_encode_kv(_stream(), _dev(src, "src"), _dev(codes, "codes"), _dev(norms, "norms"),
+                                       n_tokens, n_kv_heads, head_dim, capacity, write_pos))
+
+
+def tq_tmp_buffer_bytes(num_heads: int, head_dim: int, kv_seq_len: int) -> int:
+    return _l.load().hq_flash_attn_vec_tq_tmp_bytes(num_heads, head_dim, kv_seq_len)
+
+
+def flash_attn_vec_tq_hb(q: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor, v_packed: torch.Tensor,
+                         v_norms: torch.Tensor, out: torch.Tensor, tmp: torch.Tensor, params: FlashAttnVecTqHbParams,
+                         lut256: torch.Tensor | None = None) -> None:
+    """forward_mlx.rs:4732-4742: single-query attention over the 8-bit cache (rotated domain in and out)."""
+    if q.dtype != torch.float32 or out.dtype != torch.float32:
+        raise TypeError("q and out must be float32")
+    p = _l.TqAttnParams(params.num_heads, params.num_kv_heads, params.head_dim, params.kv_seq_len,
+                        params.kv_capacity, params.scale, params.mask_type, params.sliding_window, params.softcap,
+                        params.ring_start, params.scale_factor_d512, params.codebook_bits, params.fuse_fwht_pre,
+                        params.nsg)
+    import ctypes as _ct
+    _l.check(_l.load().hq_flash_attn_vec_tq(
+        _stream(), _dev(q, "q"), _dev(k_packed, "k_packed"), _dev(k_norms, "k_norms"), _dev(v_packed, "v_packed"),
+        _dev(v_norms, "v_norms"), _dev(lut256, "lut256") if lut256 is not None else None, _dev(out, "out"),
+        _dev(tmp, "tmp"), tmp.numel() * tmp.element_size(), _ct.byref(p)))

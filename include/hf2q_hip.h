@@ -109,6 +109,58 @@ HQ_API int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, con
  * n_tokens*top_k routed rows (the IdMmScratch analogue, decode_pool.rs:56-60). */
 HQ_API size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows);
 
+/* ---- TurboQuant-style 8-bit KV cache -------------------------------------------------------
+ * Cache layout (src/inference/models/qwen35/kv_cache.rs:1982-2113): codes
+ * [n_kv_heads, capacity, head_dim] u8 (1 byte per element) and norms
+ * [n_kv_heads, capacity, max(1, head_dim/256)] f32.  K and V are stored in the rotated
+ * domain  H.(s (.) x)  (normalised Hadamard, sign table kv_cache.rs:3871-3876). */
+
+/* In-place  buf <- H.(s (.) buf)  per 256-element block of buf[n_heads][head_dim] (query
+ * pre-rotation) and its inverse  buf <- s (.) (H.buf)  (output post-rotation).  Replace
+ * dispatch_fwht_sign_premult_f32 / dispatch_fwht_sign_undo_f32(enc, reg, dev, buf, num_heads,
+ * head_dim) (src/serve/forward_mlx.rs:4662-4666, 4750; gpu_full_attn.rs:219, 253).
+ * head_dim must be 256 or 512. */
+HQ_API int hq_fwht_sign_premult_f32(void* stream, float* buf, uint32_t n_heads, uint32_t head_dim);
+HQ_API int hq_fwht_sign_undo_f32(void* stream, float* buf, uint32_t n_heads, uint32_t head_dim);
+
+/* Write-side encode of n_tokens K (or V) vectors, src [n_tokens, n_kv_heads, head_dim] f32, into
+ * cache slots (write_pos + t) % capacity: rotate, then per 256-block norm = amax/127 and
+ * code = round(x/norm) as int8 (two's complement byte).  Stands where
+ * dispatch_hadamard_quantize_kv_hb[_seq] stands in the reference (kv_cache.rs:180-213, 278-294);
+ * the code->value map is the linear int8 one of the benchmark configuration, not the
+ * reference's Lloyd-Max table. */
+HQ_API int hq_tq_encode_kv(void* stream, const float* src, uint8_t* codes, float* norms, uint32_t n_tokens,
+                    uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t write_pos);
+
+/* Field for field FlashAttnVecTqHbParams / Qwen35TqSdpaParams (kv_cache.rs:589-614;
+ * forward_mlx.rs:4687-4705). */
+typedef struct {
+    uint32_t num_heads, num_kv_heads, head_dim;
+    uint32_t kv_seq_len, kv_capacity;
+    float scale;
+    uint32_t mask_type;      /* 0 none, 1 causal, 2 sliding window (single query at the end of the sequence) */
+    uint32_t sliding_window; /* mask_type 2: only the last sliding_window positions are visible */
+    float softcap;           /* 0 = off, else s <- softcap * tanh(s / softcap) */
+    uint32_t ring_start;     /* logical position i lives in slot (ring_start + i) % kv_capacity */
+    float scale_factor_d512;
+    uint32_t codebook_bits;  /* 5, 6 or 8 are valid values; this build implements 8 */
+    uint32_t fuse_fwht_pre;  /* 1: q arrives un-rotated and is rotated inside the kernel */
+    uint32_t nsg;            /* accepted for layout compatibility; the split count is chosen here */
+} hq_tq_attn_params;
+
+/* out[h] = softmax(scale * q[h] . K[kv(h)]^T) . V[kv(h)], kv(h) = h / (num_heads/num_kv_heads), one
+ * query position, K/V dequantised in-kernel, fp32 softmax; q and out are [num_heads, head_dim] f32
+ * in the rotated domain.  lut256 == NULL: cached value = norm * int8(code); otherwise
+ * lut256[code] * norm / 16 / scale_factor.  Replaces flash_attn_vec_tq_hb(enc, reg, dev, q, k_packed,
+ * k_norms, v_packed, v_norms, out, tmp, &params) (forward_mlx.rs:4732-4742; kv_cache.rs:373-386).
+ * `tmp` is device scratch of hq_flash_attn_vec_tq_tmp_bytes() bytes.  Rejects kv_seq_len == 0,
+ * kv_capacity < kv_seq_len (kv_cache.rs:331-333), head_dim not in {256, 512}, codebook_bits not in
+ * {5, 6, 8}; head_dim 512 and codebook_bits 5 / 6 are reported as unsupported. */
+HQ_API int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
+                         const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
+                         void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p);
+HQ_API size_t hq_flash_attn_vec_tq_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,184 @@
+"""GPU parity of the TurboQuant-style KV path: rotation, write-side encode, decode attention."""
+import numpy as np
+import pytest
+import torch
+
+from hf2q_amd import ops
+from hf2q_amd.ops import FlashAttnVecTqHbParams
+
+pytestmark = pytest.mark.gpu
+
+
+def _nrmse(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(np.sqrt(((a - b) ** 2).sum() / (b ** 2).sum()))
+
+
+@pytest.mark.parametrize("hd", [256, 512])
+def test_fwht_sign_bit_exact_and_self_inverse(oracle, dev, hd):
+    x = np.random.default_rng(hd).standard_normal((5, hd)).astype(np.float32)
+    b = torch.from_numpy(x).to(dev)
+    ops.dispatch_fwht_sign_premult_f32(b, 5, hd)
+    want = oracle.fwht_sign_premult(x, 5, hd)
+    assert np.array_equal(b.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    ops.dispatch_fwht_sign_undo_f32(b, 5, hd)
+    assert np.array_equal(b.cpu().numpy().view(np.uint32), oracle.fwht_sign_undo(want, 5, hd).view(np.uint32))
+    assert np.allclose(b.cpu().numpy(), x, atol=1e-5)  # undo(premult(x)) = x
+
+
+def _oracle_cache(oracle, kv, n_kv, hd, cap, start=0):
+    codes = np.zeros((n_kv, cap, hd), np.uint8)
+    norms = np.zeros((n_kv, cap, max(1, hd // 256)), np.float32)
+    for t in range(kv.shape[0]):
+        oracle.tq_encode_int8(kv[t], n_kv, hd, cap, (start + t) % cap, codes, norms)
+    return codes, norms
+
+
+@pytest.mark.parametrize("hd", [256, 512])
+def test_encode_byte_equal_to_oracle(oracle, dev, hd):
+    rng = np.random.default_rng(3)
+    n_kv, cap, n_tok, start = 2, 40, 37, 6   # wraps around the ring: slots 6..39, 0..2
+    kv = rng.standard_normal((n_tok, n_kv, hd)).astype(np.float32)
+    kv[5] = 0.0                               # an all-zero token: scale 0, codes 0
+    want_c, want_n = _oracle_cache(oracle, kv, n_kv, hd, cap, start)
+    codes, norms = ops.alloc_tq_kv(n_kv, cap, hd, dev)
+    ops.hadamard_quantize_kv(torch.from_numpy(kv).to(dev), codes, norms, start)
+    assert np.array_equal(codes.cpu().numpy(), want_c)
+    assert np.array_equal(norms.cpu().numpy().view(np.uint32), want_n.view(np.uint32))
+    # kv_cache.rs:4205: encoding a sequence equals encoding token by token
+    c2, n2 = ops.alloc_tq_kv(n_kv, cap, hd, dev)
+    for t in range(n_tok):
+        ops.hadamard_quantize_kv(torch.from_numpy(kv[t:t + 1]).to(dev), c2, n2, start + t)
+    assert torch.equal(c2, codes) and torch.equal(n2, norms)
+    # kv_cache.rs:3383: only the written slots change
+    assert not codes[:, 3:6].any() and not norms[:, 3:6].any()
+
+
+def _attend(dev, q, kc, kn, vc, vn, p, lut=None):
+    tmp = torch.empty(ops.tq_tmp_buffer_bytes(p.num_heads, p.head_dim, p.kv_seq_len) // 4, device=dev)
+    out = torch.full((p.num_heads, p.head_dim), float("nan"), device=dev)
+    ops.flash_attn_vec_tq_hb(torch.from_numpy(q).to(dev), torch.from_numpy(kc).to(dev), torch.from_numpy(kn).to(dev),
+                             torch.from_numpy(vc).to(dev), torch.from_numpy(vn).to(dev), out, tmp, p,
+                             None if lut is None else torch.from_numpy(lut).to(dev))
+    return out.cpu().numpy()
+
+
+def _assert_attn_close(got, ref, what):
+    assert np.isfinite(got).all(), what
+    scale = np.abs(ref).max(axis=1, keepdims=True)
+    # softmax in fp32 over exact dequantised values: 1e-3 of each head's output magnitude
+    assert (np.abs(got - ref) <= 1e-3 * scale).all(), f"{what}: max err {np.abs(got - ref).max()} vs scale {scale.min()}"
+    assert _nrmse(got, ref) < 1e-4, f"{what}: nrmse {_nrmse(got, ref)}"
+
+
+CASES = [  # nh, nkv, n, cap, kwargs
+    (16, 2, 1, 8, {}),
+    (16, 2, 33, 40, {}),
+    (16, 2, 700, 1024, {}),
+    (8, 4, 257, 300, {}),                                    # group of 2
+    (4, 4, 100, 128, {}),                                    # no grouping
+    (32, 2, 130, 256, {}),                                   # group of 16 = two chunks of 8
+    (16, 2, 500, 512, {"mask_type": 1}),
+    (16, 2, 500, 512, {"mask_type": 2, "sliding_window": 100}),
+    (16, 2, 512, 512, {"mask_type": 2, "sliding_window": 300, "ring_start": 77}),
+    (16, 2, 300, 512, {"softcap": 5.0}),
+    (16, 2, 9000, 9000, {}),                                 # several tiles per wave
+]
+
+
+@pytest.mark.parametrize("nh,nkv,n,cap,kw", CASES)
+def test_attention_matches_f64_oracle(oracle, dev, nh, nkv, n, cap, kw):
+    hd = 256
+    rng = np.random.default_rng(nh * n + cap)
+    k = rng.standard_normal((min(n, cap), nkv, hd)).astype(np.float32)
+    v = rng.standard_normal((min(n, cap), nkv, hd)).astype(np.float32)
+    kc, kn = _oracle_cache(oracle, k, nkv, hd, cap)
+    vc, vn = _oracle_cache(oracle, v, nkv, hd, cap)
+    q = oracle.fwht_sign_premult(rng.standard_normal((nh, hd)).astype(np.float32), nh, hd)
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 1.0 / 16.0, **kw)
+    ref = oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, hd, n, cap, p.scale, p.mask_type, p.sliding_window,
+                              p.softcap, p.ring_start)
+    _assert_attn_close(_attend(dev, q, kc, kn, vc, vn, p), ref, f"attn {nh}/{nkv} n={n} {kw}")
+
+
+def test_attention_lut_form(oracle, dev):
+    hd, nh, nkv, n, cap = 256, 16, 2, 200, 256
+    rng = np.random.default_rng(8)
+    kc = rng.integers(0, 256, (nkv, cap, hd), dtype=np.uint8)
+    vc = rng.integers(0, 256, (nkv, cap, hd), dtype=np.uint8)
+    kn = rng.uniform(5, 20, (nkv, cap, 1)).astype(np.float32)
+    vn = rng.uniform(5, 20, (nkv, cap, 1)).astype(np.float32)
+    lut = np.sort(rng.standard_normal(256)).astype(np.float32) * 2  # an arbitrary (non-linear) 256-entry codebook
+    q = rng.standard_normal((nh, hd)).astype(np.float32)
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 1.0 / 16.0)
+    ref = oracle.tq_attention(q, kc, kn, vc, vn, lut, nh, nkv, hd, n, cap, p.scale)
+    _assert_attn_close(_attend(dev, q, kc, kn, vc, vn, p, lut), ref, "lut form")
+
+
+def test_fused_pre_rotation_equals_separate_dispatch(oracle, dev):
+    hd, nh, nkv, n, cap = 256, 16, 2, 300, 512
+    rng = np.random.default_rng(12)
+    kc, kn = _oracle_cache(oracle, rng.standard_normal((n, nkv, hd)).astype(np.float32), nkv, hd, cap)
+    vc, vn = _oracle_cache(oracle, rng.standard_normal((n, nkv, hd)).astype(np.float32), nkv, hd, cap)
+    q = rng.standard_normal((nh, hd)).astype(np.float32)
+    sep = _attend(dev, oracle.fwht_sign_premult(q, nh, hd), kc, kn, vc, vn, FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 0.0625))
+    fused = _attend(dev, q, kc, kn, vc, vn, FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 0.0625, fuse_fwht_pre=1))
+    assert np.array_equal(sep, fused)  # forward_mlx.rs:4646-4652: the fused path is bit-identical
+
+
+def test_end_to_end_against_unquantised_attention(oracle, dev):
+    """The reference's litmus (kv_cache.rs:3959-4117): rotate q, attend over the 8-bit cache, rotate back, compare
+    with plain f32 attention.  kv_seq_len = 1 must return V[h / heads_per_kv]; gate NRMSE < 0.15."""
+    hd, nh, nkv, cap = 256, 16, 2, 64
+    rng = np.random.default_rng(21)
+    for n in (1, 48):
+        k = rng.standard_normal((n, nkv, hd)).astype(np.float32)
+        v = rng.standard_normal((n, nkv, hd)).astype(np.float32)
+        q = rng.standard_normal((nh, hd)).astype(np.float32)
+        kcod, knrm = ops.alloc_tq_kv(nkv, cap, hd, dev)
+        vcod, vnrm = ops.alloc_tq_kv(nkv, cap, hd, dev)
+        ops.hadamard_quantize_kv(torch.from_numpy(k).to(dev), kcod, knrm, 0)
+        ops.hadamard_quantize_kv(torch.from_numpy(v).to(dev), vcod, vnrm, 0)
+        qd = torch.from_numpy(q).to(dev)
+        ops.dispatch_fwht_sign_premult_f32(qd, nh, hd)
+        out = torch.empty(nh, hd, device=dev)
+        tmp = torch.empty(ops.tq_tmp_buffer_bytes(nh, hd, n) // 4, device=dev)
+        ops.flash_attn_vec_tq_hb(qd, kcod, knrm, vcod, vnrm, out, tmp, FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 0.0625))
+        ops.dispatch_fwht_sign_undo_f32(out, nh, hd)
+        exact = np.zeros((nh, hd))
+        for h in range(nh):
+            s = (k[:, h // 8].astype(np.float64) @ q[h].astype(np.float64)) * 0.0625
+            pr = np.exp(s - s.max())
+            pr /= pr.sum()
+            exact[h] = pr @ v[:, h // 8].astype(np.float64)
+        e = _nrmse(out.cpu().numpy(), exact)
+        assert e < 0.15 and e < 0.02, f"n={n}: nrmse {e}"
+
+
+def test_argument_errors(dev):
+    nh, nkv, hd, cap = 16, 2, 256, 32
+    kc, kn = ops.alloc_tq_kv(nkv, cap, hd, dev)
+    q = torch.zeros(nh, hd, device=dev)
+    out = torch.zeros(nh, hd, device=dev)
+    tmp = torch.zeros(1 << 16, device=dev)
+
+    def call(**kw):
+        base = dict(num_heads=nh, num_kv_heads=nkv, head_dim=hd, kv_seq_len=4, kv_capacity=cap, scale=1.0)
+        base.update(kw)
+        ops.flash_attn_vec_tq_hb(q, kc, kn, kc, kn, out, tmp, FlashAttnVecTqHbParams(**base))
+
+    call()
+    for bad in (dict(kv_seq_len=0),                 # kv_cache.rs:3816 rejects_kv_seq_len_zero
+                dict(kv_seq_len=cap + 1),           # kv_cache.rs:331-333
+                dict(head_dim=128), dict(codebook_bits=7), dict(num_kv_heads=3), dict(mask_type=3)):
+        with pytest.raises(ops.HqError) as e:
+            call(**bad)
+        assert e.value.status == 1
+    for unsupported in (dict(head_dim=512), dict(codebook_bits=5)):
+        with pytest.raises(ops.HqError) as e:
+            call(**unsupported)
+        assert e.value.status == 2
+    with pytest.raises(ops.HqError):                # scratch too small
+        ops.flash_attn_vec_tq_hb(q, kc, kn, kc, kn, out, tmp[:8], FlashAttnVecTqHbParams(nh, nkv, hd, 4, cap, 1.0))
+    with pytest.raises(ops.HqError):
+        ops.dispatch_fwht_sign_premult_f32(q, nh, 128)
