@@ -362,21 +362,52 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     }
 }
 
-// out[h][d] = sum_s e^{m_s - m} O_s[d] / sum_s e^{m_s - m} l_s.  One workgroup of 256 per head.
+// out[h][d] = sum_s e^{m_s - m} O_s[d] / sum_s e^{m_s - m} l_s.  Grid (num_heads, 4): a workgroup
+// owns 64 output coordinates of one head; its 4 waves take a quarter of the splits each, with
+// the loads of 8 splits in flight at a time.
 __global__ __launch_bounds__(256) void tq_attn_reduce_kernel(const float* __restrict__ tmp, float* __restrict__ out,
                                                              uint32_t n_splits) {
-    const uint32_t h = blockIdx.x, d = threadIdx.x;
+    __shared__ float s_w[128];  // e^{m_s - m}
+    __shared__ float s_part[4][64];
+    __shared__ float s_red[4];
+    const uint32_t h = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t d = blockIdx.y * 64u + lane;
     const float* base = tmp + (size_t)h * n_splits * TMP_STRIDE;
-    float m = -INFINITY;
-    for (uint32_t s = 0; s < n_splits; ++s) m = fmaxf(m, base[(size_t)s * TMP_STRIDE + HD]);
-    float o = 0.f, l = 0.f;
-    for (uint32_t s = 0; s < n_splits; ++s) {
-        const float ms = base[(size_t)s * TMP_STRIDE + HD];
-        const float f = ms == -INFINITY ? 0.f : __expf(ms - m);
-        o += f * base[(size_t)s * TMP_STRIDE + d];
-        l += f * base[(size_t)s * TMP_STRIDE + HD + 1];
+    // n_splits <= 128: threads 0..127 fetch the running maxima and sums
+    float ms = -INFINITY, ls = 0.f;
+    if (tid < n_splits) {
+        ms = base[(size_t)tid * TMP_STRIDE + HD];
+        ls = base[(size_t)tid * TMP_STRIDE + HD + 1];
     }
-    out[(size_t)h * HD + d] = l > 0.f ? o / l : 0.f;
+    float m = ms;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if (lane == 0) s_red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    const float w = ms == -INFINITY ? 0.f : __expf(ms - m);
+    if (tid < 128) s_w[tid] = w;
+    float lw = w * ls;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
+    __syncthreads();  // s_red read by everyone before it is reused; s_w visible
+    if (lane == 0) s_red[wave] = lw;
+    float o = 0.f;
+    const uint32_t per = (n_splits + 3u) / 4u, s0 = wave * per, s1 = min(n_splits, s0 + per);
+    for (uint32_t s = s0; s < s1; s += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = s + i < s1 ? base[(size_t)(s + i) * TMP_STRIDE + d] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o = fmaf(s + i < s1 ? s_w[s + i] : 0.f, v[i], o);
+    }
+    s_part[wave][lane] = o;
+    __syncthreads();
+    if (wave == 0) {
+        const float l = s_red[0] + s_red[1] + s_red[2] + s_red[3];
+        const float t = s_part[0][lane] + s_part[1][lane] + s_part[2][lane] + s_part[3][lane];
+        out[(size_t)h * HD + d] = l > 0.f ? t / l : 0.f;
+    }
 }
 
 }  // namespace
@@ -448,7 +479,7 @@ int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, c
     else
         hipLaunchKernelGGL(tq_attn_split_kernel<false>, grid, dim3(256), 0, s, a);
     if (int rc = check_launch("tq attention kernel launch")) return rc;
-    hipLaunchKernelGGL(tq_attn_reduce_kernel, dim3(p.num_heads), dim3(256), 0, s, tmp, out, a.n_splits);
+    hipLaunchKernelGGL(tq_attn_reduce_kernel, dim3(p.num_heads, HD / 64), dim3(256), 0, s, tmp, out, a.n_splits);
     return check_launch("tq attention reduce launch");
 }
 
