@@ -29,9 +29,6 @@ static bool known_type(hq_ggml_type t) { return t == HQ_Q8_0 || t == HQ_Q4_K || 
 // Largest activation-row count the GEMV kernels take; above it the MFMA GEMM
 // runs (MM_ROUTING_THRESHOLD = 8, src/serve/forward_mlx.rs:9791).
 constexpr uint32_t kGemvMaxRows = 8;
-// mul_mat_id keeps the GEMV form while the routed rows are few enough that
-// experts are rarely shared between rows.
-constexpr uint32_t kGemvIdMaxPairs = 128;
 
 static int check_weight_alignment(const void* w, hq_ggml_type t) {
     const size_t need = t == HQ_Q4_K ? 16 : 2;
@@ -157,23 +154,30 @@ int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void
                     (unsigned long long)expert_stride);
     const uint64_t pairs = (uint64_t)n_tokens * top_k;
     if (pairs == 0) return HQ_OK;
-    if (pairs > 0xffffu * 16u) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: too many routed rows");
-    if (pairs <= kGemvIdMaxPairs) {
+    // One GEMV per routed row, up to 65535 rows per launch (grid.y).  Rows that share an expert read
+    // its weights through L2; a grouped MFMA GEMM for long prefills is the next step on this path.
+    const size_t xrow_bytes = (size_t)k * (xdt == HQ_BF16 ? 2 : 4);
+    constexpr uint64_t kMaxPerLaunch = 65535u / 1u;
+    for (uint64_t p0 = 0; p0 < pairs;) {
+        // keep launches aligned to whole tokens so that the x row of pair p is (p0 + p) / top_k
+        uint64_t cnt = pairs - p0 < kMaxPerLaunch ? pairs - p0 : kMaxPerLaunch;
+        if (cnt < pairs - p0) cnt -= cnt % top_k;
+        if (cnt == 0) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: top_k %u too large", top_k);
         GemvArgs a{};
-        a.x = x;
+        a.x = static_cast<const uint8_t*>(x) + (size_t)(p0 / top_k) * xrow_bytes;
         a.w = static_cast<const uint8_t*>(w_stack);
-        a.ids = ids;
-        a.y = y;
-        a.pairs = (uint32_t)pairs;
+        a.ids = ids + p0;
+        a.y = y + (size_t)p0 * n;
+        a.pairs = (uint32_t)cnt;
         a.top_k = top_k;
         a.n = n;
         a.k = k;
         a.n_experts = n_experts;
         a.expert_stride = expert_stride;
-        return launch_gemv((hipStream_t)stream, a, xdt, t);
+        if (int rc = launch_gemv((hipStream_t)stream, a, xdt, t)) return rc;
+        p0 += cnt;
     }
-    return fail(HQ_ERR_UNSUPPORTED, "hq_qmatmul_id_ggml: %llu routed rows need the grouped GEMM path",
-                (unsigned long long)pairs);
+    return HQ_OK;
 }
 
 static int check_fwht(const char* fn, const float* buf, uint32_t n_heads, uint32_t head_dim) {
@@ -241,6 +245,50 @@ int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, c
                     tq_attn_tmp_bytes(p->num_heads, p->head_dim, p->kv_seq_len));
     return launch_tq_attention((hipStream_t)stream, q, k_codes, k_norms, v_codes, v_norms, lut256, out,
                                static_cast<float*>(tmp), *p);
+}
+
+int hq_dense_gemv_bf16(void* stream, const void* x, hq_act_dtype xdt, const void* w_bf16, float* y, uint32_t m,
+                       uint32_t n, uint32_t k) {
+    if (xdt != HQ_F32 && xdt != HQ_BF16) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dense_gemv_bf16: activation dtype %d", (int)xdt);
+    if (k == 0 || k % 8) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dense_gemv_bf16: k %u is not a multiple of 8", k);
+    if (m == 0 || n == 0) return HQ_OK;
+    if (!x || !w_bf16 || !y) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dense_gemv_bf16: null buffer");
+    if (!is_aligned(x, 16) || !is_aligned(w_bf16, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dense_gemv_bf16: x and w must be 16-byte aligned");
+    if (m > 65535) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dense_gemv_bf16: m %u too large", m);
+    return launch_dense_gemv_bf16((hipStream_t)stream, x, xdt, w_bf16, y, m, n, k);
+}
+
+int hq_moe_softmax_topk(void* stream, const float* logits, uint32_t* ids, float* weights, uint32_t n_tokens,
+                        uint32_t n_experts, uint32_t top_k) {
+    if (n_experts == 0 || n_experts > 1024) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_moe_softmax_topk: n_experts %u (1..1024)", n_experts);
+    // ffn.rs:203-204: top-k must be positive and cannot exceed num_experts
+    if (top_k == 0 || top_k > n_experts || top_k > 64)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_moe_softmax_topk: top_k %u with %u experts (1..min(64, n_experts))", top_k, n_experts);
+    if (n_tokens == 0) return HQ_OK;
+    if (!logits || !ids || !weights) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_moe_softmax_topk: null buffer");
+    return launch_moe_softmax_topk((hipStream_t)stream, logits, ids, weights, n_tokens, n_experts, top_k);
+}
+
+int hq_silu_mul(void* stream, const float* gate, const float* up, float* out, uint64_t n) {
+    if (n % 4) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_silu_mul: n %llu is not a multiple of 4", (unsigned long long)n);
+    if (n == 0) return HQ_OK;
+    if (!gate || !up || !out) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_silu_mul: null buffer");
+    if (!is_aligned(gate, 16) || !is_aligned(up, 16) || !is_aligned(out, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_silu_mul: buffers must be 16-byte aligned");
+    return launch_silu_mul((hipStream_t)stream, gate, up, out, n);
+}
+
+int hq_moe_weighted_reduce(void* stream, const float* y, const float* w, const float* shared, const float* shared_logit,
+                           const float* residual, float* out, uint32_t n_tokens, uint32_t top_k, uint32_t hidden) {
+    if (hidden == 0 || hidden % 4) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_moe_weighted_reduce: hidden %u is not a multiple of 4", hidden);
+    if (n_tokens == 0) return HQ_OK;
+    if (n_tokens > 65535) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_moe_weighted_reduce: n_tokens %u too large", n_tokens);
+    if ((top_k && (!y || !w)) || !out) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_moe_weighted_reduce: null buffer");
+    if (shared_logit && !shared) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_moe_weighted_reduce: shared_logit without shared");
+    if (!is_aligned(y, 16) || !is_aligned(shared, 16) || !is_aligned(residual, 16) || !is_aligned(out, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_moe_weighted_reduce: buffers must be 16-byte aligned");
+    return launch_moe_weighted_reduce((hipStream_t)stream, y, w, shared, shared_logit, residual, out, n_tokens, top_k, hidden);
 }
 
 }  // extern "C"

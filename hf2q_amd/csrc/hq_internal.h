@@ -45,6 +45,15 @@ bool gemm_supported(hq_ggml_type t, uint32_t k);
 int launch_gemm(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                 uint32_t k, hq_ggml_type t);
 
+// MoE glue (moe.hip)
+int launch_dense_gemv_bf16(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
+                           uint32_t n, uint32_t k);
+int launch_moe_softmax_topk(hipStream_t s, const float* logits, uint32_t* ids, float* weights, uint32_t n_tokens,
+                            uint32_t n_experts, uint32_t top_k);
+int launch_silu_mul(hipStream_t s, const float* gate, const float* up, float* out, uint64_t n);
+int launch_moe_weighted_reduce(hipStream_t s, const float* y, const float* w, const float* shared, const float* shared_logit,
+                               const float* residual, float* out, uint32_t n_tokens, uint32_t top_k, uint32_t hidden);
+
 // TurboQuant KV (tq.hip)
 int launch_fwht_sign(hipStream_t s, float* buf, uint32_t n_heads, uint32_t head_dim, bool undo);
 int launch_tq_encode(hipStream_t s, const float* src, uint8_t* codes, float* norms, uint32_t n_tokens,

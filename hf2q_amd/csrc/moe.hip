@@ -1,0 +1,212 @@
+// Glue kernels around mul_mat_id for the MoE FFN block: router projection over
+// bf16 weights, softmax + top-k + renormalise, SwiGLU gating, and the weighted
+// reduction of expert outputs with the sigmoid-gated shared expert.  Semantics
+// follow hf2q's CPU specification moe_ffn_cpu_ref
+// (src/inference/models/qwen35/ffn.rs:179-336) and softmax_topk_renorm_cpu
+// (src/inference/models/qwen35/gpu_ffn.rs:1879-1924).  All are small
+// bandwidth-bound kernels; they exist so that a decode token's MoE layer runs
+// without a host round trip between the router and the expert GEMVs.
+#include <math.h>
+
+#include "hq_internal.h"
+
+namespace hq {
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+// y[m, n] = x[m, k] . W[n, k]^T, W bf16 row-major, x f32 or bf16, fp32 accumulate.
+// One wave per output row; grid (ceil(n/4), m).
+template <bool X_BF16>
+__global__ __launch_bounds__(256) void dense_gemv_bf16_kernel(const void* __restrict__ x, const uint16_t* __restrict__ w,
+                                                              float* __restrict__ y, uint32_t n, uint32_t k) {
+    const uint32_t lane = threadIdx.x & 63u, row = blockIdx.x * 4 + (threadIdx.x >> 6), m = blockIdx.y;
+    if (row >= n) return;
+    const uint4* wr = reinterpret_cast<const uint4*>(w + (size_t)row * k);
+    float acc = 0.f;
+    for (uint32_t c = lane; c < k / 8; c += 64) {  // 8 weights per step
+        const uint4 wv = wr[c];
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+        float xv[8];
+        if constexpr (X_BF16) {
+            const uint4 t = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + (size_t)m * k)[c];
+            const uint32_t tw[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                xv[2 * i] = bf16_bits_to_f32(tw[i] & 0xffffu);
+                xv[2 * i + 1] = bf16_bits_to_f32(tw[i] >> 16);
+            }
+        } else {
+            const float4* xp = reinterpret_cast<const float4*>(static_cast<const float*>(x) + (size_t)m * k) + 2 * c;
+            const float4 t0 = xp[0], t1 = xp[1];
+            xv[0] = t0.x, xv[1] = t0.y, xv[2] = t0.z, xv[3] = t0.w, xv[4] = t1.x, xv[5] = t1.y, xv[6] = t1.z, xv[7] = t1.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc = fmaf(bf16_bits_to_f32(ww[i] & 0xffffu), xv[2 * i], acc);
+            acc = fmaf(bf16_bits_to_f32(ww[i] >> 16), xv[2 * i + 1], acc);
+        }
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) y[(size_t)m * n + row] = acc;
+}
+
+// One wave per token: probabilities over all experts, the top_k largest (ties -> lower expert id,
+// as a stable descending sort gives), renormalised over the selection (uniform if it sums to ~0).
+constexpr int kMaxExpertsPerLane = 16;  // n_experts <= 1024
+__global__ __launch_bounds__(64) void moe_softmax_topk_kernel(const float* __restrict__ logits, uint32_t* __restrict__ ids,
+                                                              float* __restrict__ weights, uint32_t n_experts,
+                                                              uint32_t top_k) {
+    const uint32_t t = blockIdx.x, lane = threadIdx.x;
+    const float* row = logits + (size_t)t * n_experts;
+    float p[kMaxExpertsPerLane];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kMaxExpertsPerLane; ++i) {
+        const uint32_t e = lane + 64u * i;
+        p[i] = e < n_experts ? row[e] : -INFINITY;
+        mx = fmaxf(mx, p[i]);
+    }
+    mx = wave_max(mx);
+    float denom = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxExpertsPerLane; ++i) {
+        const uint32_t e = lane + 64u * i;
+        p[i] = e < n_experts ? expf(p[i] - mx) : 0.f;
+        denom += p[i];
+    }
+    denom = wave_sum(denom);
+    const float inv_d = denom > 1e-20f ? 1.f / denom : 1.f;
+#pragma unroll
+    for (int i = 0; i < kMaxExpertsPerLane; ++i) p[i] = lane + 64u * i < n_experts ? p[i] * inv_d : -1.f;  // -1: never chosen
+
+    float sum_sel = 0.f, my_w = 0.f;
+    uint32_t my_id = 0;
+    for (uint32_t s = 0; s < top_k; ++s) {
+        // lane-local best (lowest expert id wins ties: i ascending, strict >)
+        float bv = -1.f;
+        uint32_t be = 0xffffffffu;
+#pragma unroll
+        for (int i = 0; i < kMaxExpertsPerLane; ++i)
+            if (p[i] > bv) {
+                bv = p[i];
+                be = lane + 64u * i;
+            }
+        // wave-wide best: larger value, then smaller id
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o);
+            const uint32_t oe = __shfl_xor(be, o);
+            if (ov > bv || (ov == bv && oe < be)) {
+                bv = ov;
+                be = oe;
+            }
+        }
+        if ((be & 63u) == lane) {  // remove it from the owner's candidates
+#pragma unroll
+            for (int i = 0; i < kMaxExpertsPerLane; ++i)
+                if ((be >> 6) == (uint32_t)i) p[i] = -1.f;
+        }
+        sum_sel += bv;
+        if (lane == s) {  // lane s keeps slot s (top_k <= 64)
+            my_w = bv;
+            my_id = be;
+        }
+    }
+    const float inv_sum = sum_sel > 1e-20f ? 1.f / sum_sel : 1.f / (float)top_k;
+    if (lane < top_k) {
+        ids[(size_t)t * top_k + lane] = my_id;
+        weights[(size_t)t * top_k + lane] = my_w * inv_sum;
+    }
+}
+
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                       float* __restrict__ out, uint64_t n4) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const float4 g = reinterpret_cast<const float4*>(gate)[i], u = reinterpret_cast<const float4*>(up)[i];
+    float4 o;
+    o.x = g.x / (1.f + expf(-g.x)) * u.x;  // ffn.rs:24-26 silu(x) = x / (1 + exp(-x))
+    o.y = g.y / (1.f + expf(-g.y)) * u.y;
+    o.z = g.z / (1.f + expf(-g.z)) * u.z;
+    o.w = g.w / (1.f + expf(-g.w)) * u.w;
+    reinterpret_cast<float4*>(out)[i] = o;
+}
+
+// out[t, :] = sum_s w[t, s] * y[t, s, :]  (+ sigmoid(shared_logit[t]) * shared[t, :])  (+ residual[t, :])
+__global__ __launch_bounds__(256) void moe_weighted_reduce_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                                                  const float* __restrict__ shared,
+                                                                  const float* __restrict__ shared_logit,
+                                                                  const float* __restrict__ residual, float* __restrict__ out,
+                                                                  uint32_t top_k, uint32_t hidden) {
+    const uint32_t t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;  // i indexes float4 columns
+    if (i >= hidden / 4) return;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t s = 0; s < top_k; ++s) {
+        const float ws = w[(size_t)t * top_k + s];
+        const float4 v = reinterpret_cast<const float4*>(y + ((size_t)t * top_k + s) * hidden)[i];
+        acc.x = fmaf(ws, v.x, acc.x);
+        acc.y = fmaf(ws, v.y, acc.y);
+        acc.z = fmaf(ws, v.z, acc.z);
+        acc.w = fmaf(ws, v.w, acc.w);
+    }
+    if (shared) {
+        const float g = shared_logit ? 1.f / (1.f + expf(-shared_logit[t])) : 1.f;  // ffn.rs:28-30 sigmoid
+        const float4 v = reinterpret_cast<const float4*>(shared + (size_t)t * hidden)[i];
+        acc.x = fmaf(g, v.x, acc.x);
+        acc.y = fmaf(g, v.y, acc.y);
+        acc.z = fmaf(g, v.z, acc.z);
+        acc.w = fmaf(g, v.w, acc.w);
+    }
+    if (residual) {
+        const float4 v = reinterpret_cast<const float4*>(residual + (size_t)t * hidden)[i];
+        acc.x += v.x;
+        acc.y += v.y;
+        acc.z += v.z;
+        acc.w += v.w;
+    }
+    reinterpret_cast<float4*>(out + (size_t)t * hidden)[i] = acc;
+}
+
+}  // namespace
+
+int launch_dense_gemv_bf16(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
+                           uint32_t n, uint32_t k) {
+    const dim3 grid((n + 3) / 4, m);
+    if (xdt == HQ_BF16)
+        hipLaunchKernelGGL(dense_gemv_bf16_kernel<true>, grid, dim3(256), 0, s, x, static_cast<const uint16_t*>(w), y, n, k);
+    else
+        hipLaunchKernelGGL(dense_gemv_bf16_kernel<false>, grid, dim3(256), 0, s, x, static_cast<const uint16_t*>(w), y, n, k);
+    return check_launch("dense bf16 gemv launch");
+}
+
+int launch_moe_softmax_topk(hipStream_t s, const float* logits, uint32_t* ids, float* weights, uint32_t n_tokens,
+                            uint32_t n_experts, uint32_t top_k) {
+    hipLaunchKernelGGL(moe_softmax_topk_kernel, dim3(n_tokens), dim3(64), 0, s, logits, ids, weights, n_experts, top_k);
+    return check_launch("moe softmax_topk launch");
+}
+
+int launch_silu_mul(hipStream_t s, const float* gate, const float* up, float* out, uint64_t n) {
+    const uint64_t n4 = n / 4;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, gate, up, out, n4);
+    return check_launch("silu_mul launch");
+}
+
+int launch_moe_weighted_reduce(hipStream_t s, const float* y, const float* w, const float* shared, const float* shared_logit,
+                               const float* residual, float* out, uint32_t n_tokens, uint32_t top_k, uint32_t hidden) {
+    const dim3 grid((hidden / 4 + 255) / 256, n_tokens);
+    hipLaunchKernelGGL(moe_weighted_reduce_kernel, grid, dim3(256), 0, s, y, w, shared, shared_logit, residual, out, top_k,
+                       hidden);
+    return check_launch("moe weighted_reduce launch");
+}
+
+}  // namespace hq

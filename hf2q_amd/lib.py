@@ -38,6 +38,10 @@ SIGNATURES = {
     "hq_qmatmul_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32]),
     "hq_qmatmul_id_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _u32, _u32, _u32, _u32, _u32, _u64, _i32]),
     "hq_qmatmul_id_scratch_bytes": (_sz, [_u32, _u32]),
+    "hq_dense_gemv_bf16": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32]),
+    "hq_moe_softmax_topk": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "hq_silu_mul": (_i32, [_vp, _vp, _vp, _vp, _u64]),
+    "hq_moe_weighted_reduce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "hq_fwht_sign_premult_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_fwht_sign_undo_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_tq_encode_kv": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),

@@ -190,3 +190,96 @@ def flash_attn_vec_tq_hb(q: torch.Tensor, k_packed: torch.Tensor, k_norms: torch
         _stream(), _dev(q, "q"), _dev(k_packed, "k_packed"), _dev(k_norms, "k_norms"), _dev(v_packed, "v_packed"),
         _dev(v_norms, "v_norms"), _dev(lut256, "lut256") if lut256 is not None else None, _dev(out, "out"),
         _dev(tmp, "tmp"), tmp.numel() * tmp.element_size(), _ct.byref(p)))
+
+
+# ---- MoE FFN block ------------------------------------------------------------------------------
+
+def dense_gemv_bf16_f32(x: torch.Tensor, w_bf16: torch.Tensor, y: torch.Tensor, m: int, n: int, k: int) -> None:
+    """gpu_ffn.rs:597-617: y[m,n] = x[m,k] . W[n,k]^T with bf16 weights."""
+    _l.check(_l.load().hq_dense_gemv_bf16(_stream(), _dev(x, "x"), _act_dtype(x), _dev(w_bf16, "w"), _dev(y, "y"), m, n, k))
+
+
+def dispatch_moe_softmax_topk(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, n_tokens: int,
+                              n_experts: int, top_k: int) -> None:
+    _l.check(_l.load().hq_moe_softmax_topk(_stream(), _dev(logits, "logits"), _dev(ids, "ids"), _dev(weights, "weights"),
+                                           n_tokens, n_experts, top_k))
+
+
+def dispatch_silu_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor) -> None:
+    _l.check(_l.load().hq_silu_mul(_stream(), _dev(gate, "gate"), _dev(up, "up"), _dev(out, "out"), gate.numel()))
+
+
+def dispatch_moe_weighted_reduce(y: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_tokens: int, top_k: int,
+                                 hidden: int, shared: torch.Tensor | None = None,
+                                 shared_logit: torch.Tensor | None = None, residual: torch.Tensor | None = None) -> None:
+    o = lambda t, nm: _dev(t, nm) if t is not None else None  # noqa: E731
+    _l.check(_l.load().hq_moe_weighted_reduce(_stream(), _dev(y, "y"), _dev(w, "w"), o(shared, "shared"),
+                                              o(shared_logit, "shared_logit"), o(residual, "residual"), _dev(out, "out"),
+                                              n_tokens, top_k, hidden))
+
+
+@dataclass
+class MoeFfnWeightsGpuQ:
+    """Device weights of one quantized MoE FFN layer (gpu_ffn.rs:214-358): router and shared-gate logit in
+    bf16, expert stacks and the shared expert as raw GGML blocks."""
+    router: torch.Tensor             # [n_experts, hidden] bf16
+    expert_gate: torch.Tensor        # stack [n_experts][inter][hidden/QK] blocks
+    expert_up: torch.Tensor
+    expert_down: torch.Tensor        # stack [n_experts][hidden][inter/QK] blocks
+    shared_gate_logit: torch.Tensor  # [1, hidden] bf16
+    shared_gate: torch.Tensor        # [shared_inter][hidden/QK] blocks
+    shared_up: torch.Tensor
+    shared_down: torch.Tensor        # [hidden][shared_inter/QK] blocks
+    ggml_type: int
+    hidden: int
+    n_experts: int
+    top_k: int
+    inter: int
+    shared_inter: int
+
+
+class MoeFfnScratch:
+    """Caller-owned activations of the block for up to `max_tokens` tokens (the decode pool of
+    decode_pool.rs, allocated once)."""
+
+    def __init__(self, w: MoeFfnWeightsGpuQ, max_tokens: int, device):
+        f = lambda *s: torch.empty(*s, dtype=torch.float32, device=device)  # noqa: E731
+        T, K = max_tokens, w.top_k
+        self.logits, self.sh_logit = f(T, w.n_experts), f(T, 1)
+        self.ids = torch.empty(T * K, dtype=torch.int32, device=device)
+        self.topk_w = f(T * K)
+        self.gate, self.up, self.act = f(T * K, w.inter), f(T * K, w.inter), f(T * K, w.inter)
+        self.down = f(T * K, w.hidden)
+        self.sh_gate, self.sh_up, self.sh_act = f(T, w.shared_inter), f(T, w.shared_inter), f(T, w.shared_inter)
+        self.sh_down = f(T, w.hidden)
+
+
+def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch, out: torch.Tensor,
+                                   residual: torch.Tensor | None = None) -> None:
+    """gpu_ffn.rs:2313-2802, phases A-F, enqueued on the current stream with no host round trip:
+    router / shared projections -> softmax top-k + shared SwiGLU -> gate, up mul_mat_id + shared down ->
+    SwiGLU -> down mul_mat_id (n_tokens = T*K, top_k = 1) -> weighted reduce (+ sigmoid-gated shared, + residual)."""
+    T = x.shape[0]
+    K, H, E, I, SI, t = w.top_k, w.hidden, w.n_experts, w.inter, w.shared_inter, w.ggml_type
+    rb = ggml_row_bytes(t, H)
+    # A
+    dense_gemv_bf16_f32(x, w.router, s.logits, T, E, H)
+    dense_gemv_bf16_f32(x, w.shared_gate_logit, s.sh_logit, T, 1, H)
+    quantized_matmul_ggml(x, w.shared_gate, s.sh_gate, GgmlQuantizedMatmulParams(T, SI, H, t))
+    quantized_matmul_ggml(x, w.shared_up, s.sh_up, GgmlQuantizedMatmulParams(T, SI, H, t))
+    # B
+    dispatch_moe_softmax_topk(s.logits, s.ids, s.topk_w, T, E, K)
+    dispatch_silu_mul(s.sh_gate[:T], s.sh_up[:T], s.sh_act[:T])
+    # C
+    pid = GgmlQuantizedMatmulIdParams(T, K, I, H, E, I * rb, t)
+    quantized_matmul_id_ggml(x, w.expert_gate, s.ids, s.gate, pid)
+    quantized_matmul_id_ggml(x, w.expert_up, s.ids, s.up, pid)
+    quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, GgmlQuantizedMatmulParams(T, H, SI, t))
+    # D
+    dispatch_silu_mul(s.gate[:T * K], s.up[:T * K], s.act[:T * K])
+    # E
+    quantized_matmul_id_ggml(s.act, w.expert_down, s.ids, s.down,
+                             GgmlQuantizedMatmulIdParams(T * K, 1, H, I, E, H * ggml_row_bytes(t, I), t))
+    # F
+    dispatch_moe_weighted_reduce(s.down, s.topk_w, out, T, K, H, shared=s.sh_down, shared_logit=s.sh_logit,
+                                 residual=residual)

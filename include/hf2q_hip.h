@@ -109,6 +109,29 @@ HQ_API int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, con
  * n_tokens*top_k routed rows (the IdMmScratch analogue, decode_pool.rs:56-60). */
 HQ_API size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows);
 
+/* ---- MoE block glue (run between the mul_mat_id calls; ffn.rs:179-336 is the specification) ---- */
+
+/* y[m,n] = x[m,k] . W[n,k]^T with W in bf16 (router / shared-expert gate projections).  Replaces
+ * dense_gemv_bf16_f32 (src/inference/models/qwen35/gpu_ffn.rs:597-617).  k % 8 == 0. */
+HQ_API int hq_dense_gemv_bf16(void* stream, const void* x, hq_act_dtype xdt, const void* w_bf16, float* y,
+                       uint32_t m, uint32_t n, uint32_t k);
+
+/* Per token: softmax over n_experts logits, the top_k most probable experts (ties: lower id), weights
+ * renormalised over the selection.  Replaces dispatch_moe_softmax_topk (gpu_ffn.rs:2551-2573); same
+ * results as softmax_topk_renorm_cpu (gpu_ffn.rs:1879-1924).  n_experts <= 1024, top_k <= 64. */
+HQ_API int hq_moe_softmax_topk(void* stream, const float* logits, uint32_t* ids, float* weights, uint32_t n_tokens,
+                        uint32_t n_experts, uint32_t top_k);
+
+/* out[i] = silu(gate[i]) * up[i]; n % 4 == 0.  Replaces dispatch_silu_mul (gpu_ffn.rs:2701). */
+HQ_API int hq_silu_mul(void* stream, const float* gate, const float* up, float* out, uint64_t n);
+
+/* out[t,:] = sum_s w[t,s] * y[t,s,:] + sigmoid(shared_logit[t]) * shared[t,:] + residual[t,:]; shared,
+ * shared_logit and residual may each be NULL (term omitted; shared without a logit enters with weight 1).
+ * Replaces dispatch_moe_weighted_reduce (gpu_ffn.rs:2777-2792).  hidden % 4 == 0. */
+HQ_API int hq_moe_weighted_reduce(void* stream, const float* y, const float* w, const float* shared,
+                           const float* shared_logit, const float* residual, float* out, uint32_t n_tokens,
+                           uint32_t top_k, uint32_t hidden);
+
 /* ---- TurboQuant-style 8-bit KV cache -------------------------------------------------------
  * Cache layout (src/inference/models/qwen35/kv_cache.rs:1982-2113): codes
  * [n_kv_heads, capacity, head_dim] u8 (1 byte per element) and norms

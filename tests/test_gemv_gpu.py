@@ -211,3 +211,18 @@ def test_quantizer_rejects_bad_shapes(dev):
         ops.quantize_ggml(x, 300, HQ_Q4_K)
     with pytest.raises(ops.HqError):
         ops.quantize_ggml(x, 512, HQ_Q4_K)
+
+
+def test_mul_mat_id_many_rows(oracle, dev):
+    """Prefill-sized routing (n_tokens * top_k in the hundreds) goes through the same per-row kernel."""
+    t, E, n, k, T, K = HQ_Q4_K, 8, 64, 256, 96, 4
+    stride = n * ops.ggml_row_bytes(t, k)
+    stack = oracle.quantize(weights(11, E * n, k), k, t, threads=8)
+    ids = np.random.default_rng(1).integers(0, E, size=T * K).astype(np.uint32)
+    x = acts(12, T, k)
+    ref = oracle.qmatmul_id_f64(x, stack, ids, T, K, n, k, E, stride, t)
+    y = torch.empty(T * K, n, device=dev)
+    ops.quantized_matmul_id_ggml(torch.from_numpy(x).to(dev), torch.from_numpy(stack).to(dev),
+                                 torch.from_numpy(ids.view(np.int32)).to(dev), y,
+                                 GgmlQuantizedMatmulIdParams(T, K, n, k, E, stride, t))
+    assert_matmul_close(y.cpu().numpy(), ref, "mul_mat_id 384 rows")

@@ -1,0 +1,108 @@
+"""GPU parity of the MoE glue kernels and of the whole quantized MoE FFN block against the CPU specification."""
+import numpy as np
+import pytest
+import torch
+
+from _util import acts, weights
+from hf2q_amd import ops
+from hf2q_amd.ops import HQ_Q4_K, HQ_Q8_0
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("T,E,K", [(1, 256, 8), (8, 256, 8), (3, 4, 2), (5, 60, 4), (2, 1000, 64)])
+def test_softmax_topk_matches_cpu_spec(oracle, dev, T, E, K):
+    logits = (np.random.default_rng(E + K).standard_normal((T, E)) * 3).astype(np.float32)
+    want_i, want_w = oracle.softmax_topk_renorm(logits, T, E, K)
+    ids = torch.empty(T * K, dtype=torch.int32, device=dev)
+    w = torch.empty(T * K, device=dev)
+    ops.dispatch_moe_softmax_topk(torch.from_numpy(logits).to(dev), ids, w, T, E, K)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), want_i)
+    assert np.allclose(w.cpu().numpy(), want_w, rtol=1e-5, atol=1e-7)
+    assert np.allclose(w.cpu().numpy().reshape(T, K).sum(1), 1.0, atol=1e-5)
+
+
+def test_softmax_topk_known_answers_and_ties(dev):
+    # gpu_ffn.rs:3577-3593 style: logits [1,2,3,4], top-2 -> experts 3, 2
+    ids = torch.empty(2, dtype=torch.int32, device=dev)
+    w = torch.empty(2, device=dev)
+    ops.dispatch_moe_softmax_topk(torch.tensor([[1., 2., 3., 4.]], device=dev), ids, w, 1, 4, 2)
+    assert ids.tolist() == [3, 2]
+    e = np.exp(np.float64([4, 3]) - 4)
+    assert np.allclose(w.cpu().numpy(), e / e.sum(), rtol=1e-6)
+    # equal probabilities keep ascending expert order, like a stable sort
+    ops.dispatch_moe_softmax_topk(torch.tensor([[0., 5., 5., 5., 1.]], device=dev), ids, w, 1, 5, 2)
+    assert ids.tolist() == [1, 2] and np.allclose(w.cpu().numpy(), [0.5, 0.5])
+    with pytest.raises(ops.HqError):   # ffn.rs:203: top-k cannot exceed num_experts
+        ops.dispatch_moe_softmax_topk(torch.zeros(1, 4, device=dev), ids, w, 1, 4, 5)
+
+
+def test_silu_mul_known_values(dev):
+    # gpu_ffn.rs:3558-3574
+    g = torch.tensor([0.0, 1.0, -1.0, 2.0], device=dev)
+    u = torch.tensor([5.0, 2.0, 2.0, 0.5], device=dev)
+    out = torch.empty(4, device=dev)
+    ops.dispatch_silu_mul(g, u, out)
+    want = [0.0, 0.7310586 * 2, -0.26894143 * 2, 2 / (1 + np.exp(-2.0)) * 0.5]
+    assert np.allclose(out.cpu().numpy(), want, rtol=1e-6, atol=1e-7)
+
+
+def test_weighted_reduce_and_shared_gate_linearity(dev):
+    T, K, H = 3, 4, 64
+    g = torch.Generator(device="cpu").manual_seed(1)
+    y, w = torch.randn(T * K, H, generator=g), torch.rand(T * K, generator=g)
+    sh, lg, res = torch.randn(T, H, generator=g), torch.randn(T, generator=g), torch.randn(T, H, generator=g)
+    out = torch.empty(T, H, device=dev)
+    ops.dispatch_moe_weighted_reduce(y.to(dev), w.to(dev), out, T, K, H, sh.to(dev), lg.to(dev), res.to(dev))
+    want = (y.view(T, K, H) * w.view(T, K, 1)).sum(1) + torch.sigmoid(lg)[:, None] * sh + res
+    assert torch.allclose(out.cpu(), want, rtol=1e-5, atol=1e-6)
+    # gpu_ffn.rs:3493-3551: with a zero logit the shared expert enters with weight exactly 1/2
+    ops.dispatch_moe_weighted_reduce(y.to(dev), w.to(dev), out, T, K, H, sh.to(dev), torch.zeros(T, device=dev))
+    assert torch.allclose(out.cpu(), (y.view(T, K, H) * w.view(T, K, 1)).sum(1) + 0.5 * sh, rtol=1e-5, atol=1e-6)
+    ops.dispatch_moe_weighted_reduce(y.to(dev), w.to(dev), out, T, K, H)
+    assert torch.allclose(out.cpu(), (y.view(T, K, H) * w.view(T, K, 1)).sum(1), rtol=1e-5, atol=1e-6)
+
+
+def test_dense_gemv_bf16(oracle, dev):
+    m, n, k = 3, 70, 2048
+    w = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(weights(1, n, k, 0.05)))
+    x = acts(2, m, k)
+    wd = torch.from_numpy(w).to(dev).to(torch.bfloat16)
+    for xd, xr in ((torch.from_numpy(x).to(dev), x),
+                   (torch.from_numpy(x).to(dev).to(torch.bfloat16), oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(x)))):
+        y = torch.empty(m, n, device=dev)
+        ops.dense_gemv_bf16_f32(xd, wd, y, m, n, k)
+        ref = xr.astype(np.float64) @ w.astype(np.float64).T
+        assert np.abs(y.cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("T", [1, 8])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0])
+def test_moe_block_matches_cpu_spec(oracle, dev, T, t):
+    """moe_ffn_cpu_ref (ffn.rs:179-336) over the dequantised weights vs the device block."""
+    H, E, K, I, SI = 512, 16, 4, 256, 256
+    rng = np.random.default_rng(100 + T)
+    bf = lambda a: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(a))  # noqa: E731
+    router = bf((rng.standard_normal((E, H)) * 0.1).astype(np.float32))
+    sgl = bf((rng.standard_normal((1, H)) * 0.05).astype(np.float32))
+    raw = {nm: weights(seed, n, k, 0.05) for nm, seed, n, k in
+           (("eg", 1, E * I, H), ("eu", 2, E * I, H), ("ed", 3, E * H, I), ("sg", 4, SI, H), ("su", 5, SI, H), ("sd", 6, H, SI))}
+    q = {nm: oracle.quantize(a, a.shape[1], t, threads=8) for nm, a in raw.items()}
+    dq = {nm: oracle.dequantize(q[nm], t).reshape(raw[nm].shape) for nm in raw}
+    x = acts(7, T, H)
+    want = oracle.moe_ffn(x, H, E, K, I, SI, router, dq["eg"], dq["eu"], dq["ed"], sgl[0], dq["sg"], dq["su"], dq["sd"])
+
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    w = ops.MoeFfnWeightsGpuQ(dv(router).to(torch.bfloat16), dv(q["eg"]), dv(q["eu"]), dv(q["ed"]),
+                              dv(sgl).to(torch.bfloat16), dv(q["sg"]), dv(q["su"]), dv(q["sd"]), t, H, E, K, I, SI)
+    s = ops.MoeFfnScratch(w, T, dev)
+    out = torch.full((T, H), float("nan"), device=dev)
+    ops.build_moe_ffn_layer_gpu_q_into(dv(x), w, s, out)
+    got = out.cpu().numpy()
+    scale = np.abs(want).max()
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= 2e-4 * scale, np.abs(got - want).max() / scale
+    # with a residual
+    res = acts(9, T, H)
+    ops.build_moe_ffn_layer_gpu_q_into(dv(x), w, s, out, residual=dv(res))
+    assert np.abs(out.cpu().numpy() - (want + res)).max() <= 2e-4 * np.abs(want + res).max()
