@@ -35,8 +35,16 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="decode_gemv", choices=["decode_gemv"])
+    ap.add_argument("--workload", default="decode_gemv",
+                    choices=["decode_gemv", "moe_decode", "prefill_gemm", "tq_attention"],
+                    help="decode_gemv = BASELINE config 2 (the default and the headline metric); the others are "
+                         "configs 3, 4 and 5, each printing its own JSON line")
+    ap.add_argument("--tokens", type=int, default=1, help="moe_decode: tokens per step (1 or 8)")
+    ap.add_argument("--wtype", default="q4_k", choices=["q4_k", "q8_0"], help="prefill_gemm: weight type")
     ap.add_argument("--weight-sets", type=int, default=4, help="distinct FFN weight sets rotated per step")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="moe_decode / tq_attention: launch every kernel from the host instead of replaying a HIP "
+                         "graph of the step (the steps are 4-12 launches of a few microseconds each)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -90,6 +98,206 @@ def cpu_baseline() -> dict:
     }
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
+
+
+def _events(n):
+    import torch
+    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+
+
+def _graphed(a, step, n_variants):
+    """Capture step(i) for i < n_variants into HIP graphs (one each) and return a replay function; the
+    capture replays exactly the launches step() makes.  No memset nodes are involved: the library only
+    launches kernels."""
+    import torch
+
+    if a.no_graph:
+        return step
+    side = torch.cuda.Stream()
+    graphs = []
+    with torch.cuda.stream(side):
+        for i in range(n_variants):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                step(i)
+            graphs.append(g)
+    torch.cuda.synchronize()
+    return lambda i: graphs[i % n_variants].replay()
+
+
+def _finish(a, out):
+    out.setdefault("n_gpus", 1)
+    out.update({"steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak",
+                "vs_baseline": None, "data": "synthetic"})
+    out["cpu_baseline"] = None if a.no_cpu_baseline else cpu_baseline()
+    print(json.dumps(out))
+
+
+def bench_moe_decode(a):
+    """BASELINE config 3: Qwen3.6-35B-A3B-style MoE FFN layer, hidden 2048, 256 experts (inter 512, Q4_K), one
+    shared expert, top-8 from seeded router logits, batch 1 or 8, bf16 activations.  A step is one layer."""
+    import torch
+
+    from hf2q_amd import ops
+    from hf2q_amd.ops import HQ_Q4_K
+
+    dev = torch.device("cuda:0")
+    H, E, K, I, SI, T = 2048, 256, 8, 512, 512, a.tokens
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    rnd = lambda *s: torch.randn(*s, generator=gen, device=dev, dtype=torch.float32)  # noqa: E731
+    qz = lambda n, k: ops.quantize_ggml(rnd(n * k).mul_(0.02), k, HQ_Q4_K)  # noqa: E731
+    n_layers = max(1, a.weight_sets)  # distinct layers rotated so that experts are not cache-resident
+    layers = []
+    for _ in range(n_layers):
+        layers.append(ops.MoeFfnWeightsGpuQ(
+            rnd(E, H).mul_(0.02).to(torch.bfloat16), qz(E * I, H), qz(E * I, H), qz(E * H, I),
+            rnd(1, H).mul_(0.02).to(torch.bfloat16), qz(SI, H), qz(SI, H), qz(H, SI), HQ_Q4_K, H, E, K, I, SI))
+    gx = torch.Generator(device=dev)
+    gx.manual_seed(5678)
+    x = torch.randn(T, H, generator=gx, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    scratch = ops.MoeFfnScratch(layers[0], T, dev)
+    out = torch.empty(T, H, device=dev)
+    expert_bytes = I * ops.ggml_row_bytes(HQ_Q4_K, H)
+
+    def step(i):
+        ops.build_moe_ffn_layer_gpu_q_into(x, layers[i % n_layers], scratch, out)
+
+    eager_step = step
+    for i in range(max(a.warmup, 1)):
+        step(i)
+    torch.cuda.synchronize()
+    step = _graphed(a, eager_step, n_layers)
+    uniq = []
+    ev = _events(a.steps)
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        ev[i][0].record()
+        step(a.warmup + i)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    for i in range(min(a.steps, n_layers)):  # distinct experts actually routed (after the timed region)
+        eager_step(i)
+        uniq.append(int(torch.unique(scratch.ids[:T * K]).numel()))
+    u = sum(uniq) / len(uniq)
+    layer_us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
+    step_bytes = (u * 3 + 3) * expert_bytes + (E + 1) * H * 2  # routed + shared experts + router (bf16)
+    gbs = step_bytes / layer_us / 1e3
+    _finish(a, {
+        "metric": "MoE decode tok/s (FFN-only, 40 MoE layers)", "value": round(T / (40 * elapsed / a.steps), 1),
+        "unit": "tok/s", "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "bf16",
+        "config": {"workload": f"moe_decode: hidden 2048, 256 experts x inter 512 Q4_K, shared expert, top-8, "
+                               f"batch {T}, bf16 activations (BASELINE config 3); one step = one MoE FFN layer "
+                               f"(router, top-k, 3 mul_mat_id, shared expert, reduce = 12 launches), "
+                               f"{'launched from the host' if a.no_graph else 'replayed as a HIP graph'}",
+                   "distinct_experts_per_layer": round(u, 1), "bytes_per_layer": int(step_bytes),
+                   "layers_rotated": n_layers},
+        "roofline": {"bound": "hbm", "kernel": "MoE FFN layer (all launches)", "achieved": round(gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "us_per_launch": round(layer_us, 3), "bytes_per_launch": int(step_bytes)}})
+
+
+def bench_prefill_gemm(a):
+    """BASELINE config 4: 2048 tokens x K=4096 x N=12288, Q4_K (or Q8_0) weights, bf16 activations, f32 out."""
+    import torch
+
+    from hf2q_amd import ops
+    from hf2q_amd.ops import HQ_Q4_K, HQ_Q8_0, GgmlQuantizedMatmulParams
+
+    dev = torch.device("cuda:0")
+    M, K, N = 2048, 4096, 12288
+    t = HQ_Q4_K if a.wtype == "q4_k" else HQ_Q8_0
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    w = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, t)
+    gx = torch.Generator(device=dev)
+    gx.manual_seed(5678)
+    x = torch.randn(M, K, generator=gx, device=dev).to(torch.bfloat16)
+    y = torch.empty(M, N, device=dev)
+    p = GgmlQuantizedMatmulParams(M, N, K, t)
+    for _ in range(a.warmup):
+        ops.quantized_matmul_ggml(x, w, y, p)
+    torch.cuda.synchronize()
+    ev = _events(a.steps)
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        ev[i][0].record()
+        ops.quantized_matmul_ggml(x, w, y, p)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
+    flops = 2.0 * M * N * K
+    tf = flops / us / 1e6
+    _finish(a, {
+        "metric": "prefill TFLOP/s", "value": round(flops * a.steps / elapsed / 1e12, 1), "unit": "TFLOP/s",
+        "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "bf16",
+        "config": {"workload": f"prefill_gemm: 2048 tokens x K=4096 x N=12288, {a.wtype.upper()} weights, bf16 "
+                               f"activations, fp32 accumulate (BASELINE config 4)", "flop_per_step": flops,
+                   "weight_bytes": w.numel()},
+        "roofline": {"bound": "mfma", "kernel": f"gemm {a.wtype}", "achieved": round(tf, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": None, "us_per_launch": round(us, 2), "flop_per_launch": flops}})
+
+
+def bench_tq_attention(a):
+    """BASELINE config 5: decode attention over the 8-bit KV cache, 32K context, 16 q / 2 kv heads, d=256."""
+    import torch
+
+    from hf2q_amd import ops
+    from hf2q_amd.ops import FlashAttnVecTqHbParams
+
+    dev = torch.device("cuda:0")
+    nh, nkv, hd, n = 16, 2, 256, 32768
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    n_caches = max(8, a.weight_sets)  # 34 MB each: rotate past the 256 MB Infinity Cache
+    caches = []
+    for _ in range(n_caches):
+        kc, kn = ops.alloc_tq_kv(nkv, n, hd, dev)
+        vc, vn = ops.alloc_tq_kv(nkv, n, hd, dev)
+        ops.hadamard_quantize_kv(torch.randn(n, nkv, hd, generator=gen, device=dev), kc, kn, 0)
+        ops.hadamard_quantize_kv(torch.randn(n, nkv, hd, generator=gen, device=dev), vc, vn, 0)
+        caches.append((kc, kn, vc, vn))
+    q = torch.randn(nh, hd, generator=gen, device=dev)
+    out = torch.empty(nh, hd, device=dev)
+    tmp = torch.empty(ops.tq_tmp_buffer_bytes(nh, hd, n) // 4, device=dev)
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, n, 1.0 / 16.0)
+    nbytes = sum(t.numel() * t.element_size() for t in caches[0])
+
+    def step(i):  # the reference's decode chain: rotate q, attend, rotate the output back
+        ops.dispatch_fwht_sign_premult_f32(q, nh, hd)
+        ops.flash_attn_vec_tq_hb(q, *caches[i % n_caches], out, tmp, p)
+        ops.dispatch_fwht_sign_undo_f32(out, nh, hd)
+
+    for i in range(max(a.warmup, 1)):
+        step(i)
+    torch.cuda.synchronize()
+    step = _graphed(a, step, n_caches)
+    ev = _events(a.steps)
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        ev[i][0].record()
+        step(a.warmup + i)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
+    gbs = nbytes / us / 1e3
+    _finish(a, {
+        "metric": "TQ-KV decode attention eff. GB/s", "value": round(nbytes * a.steps / elapsed / 1e9, 1),
+        "unit": "GB/s", "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f32",
+        "config": {"workload": "tq_attention: 32768 context, 16 q heads / 2 kv heads, head_dim 256, int8 codes + f32 "
+                               "norm per (token, head), batch 1 (BASELINE config 5); one step = rotate q + attention "
+                               "(split + merge) + rotate output = 4 launches", "bytes_per_step": nbytes,
+                   "caches_rotated": n_caches},
+        "roofline": {"bound": "hbm", "kernel": "rotate + tq attention split + merge + rotate", "achieved": round(gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "us_per_launch": round(us, 3), "bytes_per_launch": nbytes}})
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -107,6 +315,9 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.workload != "decode_gemv":
+        return {"moe_decode": bench_moe_decode, "prefill_gemm": bench_prefill_gemm,
+                "tq_attention": bench_tq_attention}[a.workload](a)
 
     H, F, V = 4096, 12288, 151936
     shapes = {  # name -> (n, k, type)
