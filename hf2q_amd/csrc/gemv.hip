@@ -29,6 +29,7 @@
 // order in which one masked shift of a little-endian weight word yields values.
 // f32 activations (the reference's dtype) and Q8_0 use exact v_cvt + v_fma.
 #include <math.h>
+#include <mutex>
 
 #include "hq_internal.h"
 
@@ -37,6 +38,8 @@ namespace hq {
 namespace {
 
 constexpr uint32_t M4 = 0x000f000fu, M2 = 0x00300030u, MAGIC = 0x43004300u;
+// Tasks (row slot x step) per CU from which the queue kernel takes over.
+constexpr uint32_t QUEUE_MIN_TASKS_PER_CU = 96;
 
 template <int TYPE>
 struct Lane {  // weights per lane and step
@@ -190,56 +193,65 @@ __device__ __forceinline__ float dot_f32(const Piece<HQ_Q8_0>& p, int, const flo
     return f16_bits_to_f32(p.d) * acc;
 }
 
-// Stage one activation row in LDS: PAIR -> pre-paired bf16 words + per-16 sums,
-// otherwise f32 values + per-16 sums.  Each thread handles 16 activations.
-template <bool X_BF16, bool PAIR>
-__device__ __forceinline__ void stage_x(const void* __restrict__ xrow, uint32_t k, uint32_t* lds_x, float* lds_s) {
-    for (uint32_t i = threadIdx.x; i < k / 16; i += blockDim.x) {
-        float v[16];
-        if constexpr (X_BF16) {
-            const uint4* src = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xrow) + 16 * i);
-            const uint4 a = src[0], b = src[1];
-            const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+// Staging of one activation row in LDS, 16 activations per thread and pass:
+// PAIR -> pre-paired bf16 words + per-16 sums, otherwise f32 values + per-16 sums.
+// The fetch and the conversion are separate so that the first pass can be fetched
+// ahead of the first weight loads (vector loads return in order: activations
+// issued behind a deep queue of weight fetches would hold the whole workgroup at
+// its barrier until those have come back).
+template <bool X_BF16>
+struct XRaw {
+    uint4 r[X_BF16 ? 2 : 4];
+    __device__ __forceinline__ void fetch(const void* __restrict__ xrow, uint32_t i) {
+        const uint4* src = reinterpret_cast<const uint4*>(static_cast<const uint8_t*>(xrow) +
+                                                          (size_t)i * (X_BF16 ? 32 : 64));
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                v[2 * j] = bf16_bits_to_f32(w[j] & 0xffffu);
-                v[2 * j + 1] = bf16_bits_to_f32(w[j] >> 16);
-            }
-            if constexpr (PAIR) {
-                uint4 o0, o1;
-                o0.x = (w[0] & 0xffffu) | (w[1] << 16);
-                o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
-                o0.z = (w[2] & 0xffffu) | (w[3] << 16);
-                o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
-                o1.x = (w[4] & 0xffffu) | (w[5] << 16);
-                o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
-                o1.z = (w[6] & 0xffffu) | (w[7] << 16);
-                o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
-                reinterpret_cast<uint4*>(lds_x)[2 * i] = o0;
-                reinterpret_cast<uint4*>(lds_x)[2 * i + 1] = o1;
-            }
-        } else {
-            const float4* src = reinterpret_cast<const float4*>(static_cast<const float*>(xrow) + 16 * i);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float4 t = src[j];
-                v[4 * j] = t.x;
-                v[4 * j + 1] = t.y;
-                v[4 * j + 2] = t.z;
-                v[4 * j + 3] = t.w;
-            }
-        }
-        if constexpr (!PAIR) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                reinterpret_cast<float4*>(lds_x)[4 * i + j] =
-                    make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
-        }
-        float s = 0.f;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) s += v[j];
-        lds_s[i] = s;
+        for (int j = 0; j < (X_BF16 ? 2 : 4); ++j) r[j] = src[j];
     }
+};
+
+template <bool X_BF16, bool PAIR>
+__device__ __forceinline__ void stage_store(const XRaw<X_BF16>& raw, uint32_t i, uint32_t* lds_x, float* lds_s) {
+    float v[16];
+    if constexpr (X_BF16) {
+        const uint4 a = raw.r[0], b = raw.r[1];
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            v[2 * j] = bf16_bits_to_f32(w[j] & 0xffffu);
+            v[2 * j + 1] = bf16_bits_to_f32(w[j] >> 16);
+        }
+        if constexpr (PAIR) {
+            uint4 o0, o1;
+            o0.x = (w[0] & 0xffffu) | (w[1] << 16);
+            o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
+            o0.z = (w[2] & 0xffffu) | (w[3] << 16);
+            o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
+            o1.x = (w[4] & 0xffffu) | (w[5] << 16);
+            o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
+            o1.z = (w[6] & 0xffffu) | (w[7] << 16);
+            o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
+            reinterpret_cast<uint4*>(lds_x)[2 * i] = o0;
+            reinterpret_cast<uint4*>(lds_x)[2 * i + 1] = o1;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[4 * j] = __uint_as_float(raw.r[j].x);
+            v[4 * j + 1] = __uint_as_float(raw.r[j].y);
+            v[4 * j + 2] = __uint_as_float(raw.r[j].z);
+            v[4 * j + 3] = __uint_as_float(raw.r[j].w);
+        }
+    }
+    if constexpr (!PAIR) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            reinterpret_cast<float4*>(lds_x)[4 * i + j] = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += v[j];
+    lds_s[i] = s;
 }
 
 struct KArgs {
@@ -249,7 +261,8 @@ struct KArgs {
     float* y;
     uint32_t top_k, n, k, n_experts;
     uint64_t expert_stride;
-    uint32_t log_l;  // log2 of the lanes that share one row
+    uint32_t log_l;   // log2 of the lanes that share one row
+    uint32_t groups;  // row groups (one group = the rows a workgroup covers in one pass)
     // Bit masks of the nibble -> bf16 conversion.  They are passed as arguments and
     // not written as literals so that the compiler keeps them in registers and
     // forms the three-operand v_and_or_b32 (gfx9 VOP3 takes no literals; with
@@ -316,25 +329,131 @@ __device__ __forceinline__ void load_x_piece(const uint32_t* lds_x, const float*
     }
 }
 
-// One workgroup = 4 waves sharing the staged activation row.  A wave owns NR
-// "row slots" (a slot = the 64/L rows its lanes cover at once) and walks the
-// (step, slot) tasks in step-major order with D weight fetches in flight:
-// the fetch for task t+D is issued right after task t has consumed its
-// registers, so HBM latency is covered by D-1 tasks of arithmetic per wave
-// (times the waves resident on the SIMD).  The activations of a step stay in
-// registers for all NR slots.  NR % D == 0 keeps every buffer index static.
+// ---- the per-wave walk ------------------------------------------------------
+// A wave owns NR "row slots" (a slot = the 64/L rows its lanes cover at once) of a
+// wave group and walks the (step, slot) tasks in step-major order with D weight
+// fetches in flight: the fetch for task t+D is issued right after task t has
+// consumed its registers, and the ring runs on into the wave's next wave group,
+// so the stream of fetches does not drain between groups.  The activations of a
+// step stay in registers for all NR slots.  NR % D == 0 keeps every buffer index
+// static.  Rows past the end are clamped to the last row (always a valid read;
+// its result is not stored).
+template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
+struct Walk {
+    static_assert(NR % D == 0, "buffer rotation must repeat per step");
+    static constexpr int EPL = Lane<TYPE>::kElems;
+    static constexpr uint32_t BYTES = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES : Q8_0_BYTES;
+    static constexpr int XW = PAIR ? EPL / 2 : EPL;  // LDS words per piece
+
+    const uint8_t* w;  // weight base + this lane's piece offset at step 0
+    const uint32_t* lds_x;
+    const float* lds_s;
+    uint32_t n, log_l, rpw, lane, li, steps, row_bytes, bstep, lane_row;
+    int c;
+    uint32_t m4, m2, magic;
+    Piece<TYPE> buf[D];
+
+    __device__ __forceinline__ void init(const KArgs& a, const uint8_t* wbase, const uint32_t* lx, const float* ls) {
+        lane = threadIdx.x & 63u;
+        n = a.n;
+        log_l = a.log_l;
+        const uint32_t L = 1u << log_l;
+        rpw = 64u >> log_l;
+        li = lane & (L - 1u);
+        lane_row = lane >> log_l;
+        steps = (a.k / EPL) >> log_l;  // pieces per row / L (host guarantees divisibility)
+        row_bytes = (a.k / (TYPE == HQ_Q8_0 ? 32 : 256)) * BYTES;
+        // L >= 4 for the K-quants (k >= 256), so a lane keeps the same sub-piece index c on every step
+        c = TYPE == HQ_Q8_0 ? 0 : (int)(li & 3u);
+        bstep = (TYPE == HQ_Q8_0 ? L : L >> 2) * BYTES;  // bytes of a row one step covers
+        w = wbase + (TYPE == HQ_Q8_0 ? li : li >> 2) * BYTES;
+        lds_x = lx;
+        lds_s = ls;
+    }
+
+    // The conversion masks must sit in VGPRs for v_and_or_b32 (one scalar operand
+    // at most per VALU op on gfx9); the copy is opaque so they stay there.
+    __device__ __forceinline__ void load_masks(const KArgs& a) {
+        asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
+                     : "=v"(m4), "=v"(m2), "=v"(magic)
+                     : "s"(a.m4), "s"(a.m2), "s"(a.magic));
+    }
+
+    // Issues the fetch of task (rowbase, slot u, step s) into f, ordered after the
+    // value `tie` names.
+    __device__ __forceinline__ void fetch(Piece<TYPE>& f, uint32_t rowbase, int u, uint32_t s, float tie) {
+        uint32_t r = rowbase + (uint32_t)u * rpw + lane_row;
+        r = r < n ? r : n - 1u;
+        const uint8_t* ptr = w + (size_t)r * row_bytes + (size_t)s * bstep;
+        asm volatile("" : "+v"(ptr) : "v"(tie));
+        f.load(ptr, c);
+    }
+
+    __device__ __forceinline__ void prime(uint32_t rowbase) {
+#pragma unroll
+        for (int u = 0; u < D; ++u) fetch(buf[u], rowbase, u, 0, 0.f);
+    }
+
+    // All tasks of one wave group; stores its NR slots of results.  next_rowbase /
+    // has_next: where the fetch ring continues after this group.
+    __device__ __forceinline__ void group(uint32_t rowbase, uint32_t next_rowbase, bool has_next, float* yrow,
+                                          bool valid) {
+        float acc[NR];
+#pragma unroll
+        for (int u = 0; u < NR; ++u) acc[u] = 0.f;
+
+        for (uint32_t s = 0; s < steps; ++s) {
+            uint32_t xr[XW];
+            float sx[4];
+            load_x_piece<TYPE, PAIR, XW>(lds_x, lds_s, li + s * (1u << log_l), c, xr, sx);
+            const bool more = s + 1 < steps;  // uniform
+#pragma unroll
+            for (int u = 0; u < NR; ++u) {
+                Piece<TYPE>& b = buf[u % D];
+                if constexpr (PAIR)
+                    acc[u] += dot_pair(b, c, xr, sx, m4, m2, magic);
+                else
+                    acc[u] += dot_f32(b, c, reinterpret_cast<const float*>(xr), sx);
+                // refill with the task D ahead: same step while slots remain, else the
+                // first slots of the next step, else of the next wave group.  The fetch is
+                // tied to this task's result: otherwise the compiler hoists every refill
+                // above the arithmetic into fresh registers, which doubles the buffers
+                // and halves occupancy.
+                if (u + D < NR || more || has_next)
+                    fetch(b, u + D < NR || more ? rowbase : next_rowbase, u + D < NR ? u + D : u + D - NR,
+                          u + D < NR ? s : more ? s + 1 : 0u, acc[u]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+
+#pragma unroll
+        for (int u = 0; u < NR; ++u) {
+            const float v = group_sum(acc[u], log_l);
+            const uint32_t r = rowbase + (uint32_t)u * rpw + lane_row;
+            if (li == 0 && r < n) yrow[r] = valid ? v : __builtin_nanf("");
+        }
+    }
+};
+
+// LDS layout of both kernels: activations | per-16 sums | queue counter (16 bytes).
+//
+// Small and medium problems, and every mul_mat_id launch: one workgroup of four
+// waves per four wave groups, blockIdx.y = the (token, slot) pair.  The
+// activations are requested first (vector loads return in order: behind a queue
+// of weight fetches they would hold the workgroup at its barrier), then the
+// first weight fetches go out so that their latency overlaps the staging.
 template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
 __global__ __launch_bounds__(256) void gemv_kernel(KArgs a) {
-    static_assert(NR % D == 0, "buffer rotation must repeat per step");
     extern __shared__ uint4 smem[];
-    constexpr int EPL = Lane<TYPE>::kElems;
-    constexpr uint32_t BYTES = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES : Q8_0_BYTES;
-    constexpr int XW = PAIR ? EPL / 2 : EPL;  // LDS words per piece
-
     uint32_t* lds_x = reinterpret_cast<uint32_t*>(smem);
     float* lds_s = reinterpret_cast<float*>(lds_x + (PAIR ? a.k / 2 : a.k));
 
     const uint32_t p = blockIdx.y;
+    const uint8_t* xrow = static_cast<const uint8_t*>(a.x) + (size_t)(p / a.top_k) * a.k * (X_BF16 ? 2 : 4);
+    const uint32_t xchunks = a.k / 16;
+    XRaw<X_BF16> xraw;
+    if (threadIdx.x < xchunks) xraw.fetch(xrow, threadIdx.x);
+
     const uint8_t* w = a.w;
     bool valid = true;
     if (a.ids) {
@@ -343,122 +462,155 @@ __global__ __launch_bounds__(256) void gemv_kernel(KArgs a) {
         w += (size_t)(valid ? e : 0u) * a.expert_stride;
     }
 
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t L = 1u << a.log_l;
-    const uint32_t rpw = 64u >> a.log_l;  // rows per slot
-    const uint32_t li = lane & (L - 1u);
-    const uint32_t steps = (a.k / EPL) >> a.log_l;  // pieces per row / L (host guarantees divisibility)
-    const uint32_t row0 = (blockIdx.x * 4u + wave) * rpw * NR + (lane >> a.log_l);
-    const uint32_t row_bytes = (a.k / (TYPE == HQ_Q8_0 ? 32 : 256)) * BYTES;
-    // L >= 4 for the K-quants (k >= 256), so a lane keeps the same sub-piece index c
-    // on every step.
-    const int c = TYPE == HQ_Q8_0 ? 0 : (int)(li & 3u);
-    // byte offset of this lane's piece inside a row at step 0, and its advance per step
-    const uint32_t boff0 = (TYPE == HQ_Q8_0 ? li : li >> 2) * BYTES;
-    const uint32_t bstep = (TYPE == HQ_Q8_0 ? L : L >> 2) * BYTES;
+    Walk<TYPE, X_BF16, PAIR, NR, D> wk;
+    wk.init(a, w, lds_x, lds_s);
+    const uint32_t rowbase = (blockIdx.x * 4u + (threadIdx.x >> 6)) * wk.rpw * NR;
+    wk.prime(rowbase);
 
-    // Address of slot u's row (clamped to the last row: always a valid read).
-    const uint8_t* wl = w + boff0;
-    auto row_ptr = [&](int u) -> const uint8_t* {
-        uint32_t r = row0 + (uint32_t)u * rpw;
-        r = r < a.n ? r : a.n - 1u;
-        return wl + (size_t)r * row_bytes;
-    };
-
-    // First D fetches go out before the activations are staged, so their latency
-    // overlaps the staging and its barrier.
-    Piece<TYPE> buf[D];
-#pragma unroll
-    for (int u = 0; u < D; ++u) buf[u].load(row_ptr(u), c);
-
-    const size_t xbytes = X_BF16 ? 2 : 4;
-    stage_x<X_BF16, PAIR>(static_cast<const uint8_t*>(a.x) + (size_t)(p / a.top_k) * a.k * xbytes, a.k, lds_x,
-                          lds_s);
-
-    // The conversion masks must sit in VGPRs for v_and_or_b32 (one scalar operand
-    // at most per VALU op on gfx9); the copy is opaque so they stay there.
-    uint32_t m4, m2, magic;
-    asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
-                 : "=v"(m4), "=v"(m2), "=v"(magic)
-                 : "s"(a.m4), "s"(a.m2), "s"(a.magic));
-
-    float acc[NR];
-#pragma unroll
-    for (int u = 0; u < NR; ++u) acc[u] = 0.f;
-
+    if (threadIdx.x < xchunks) stage_store<X_BF16, PAIR>(xraw, threadIdx.x, lds_x, lds_s);
+    for (uint32_t i = threadIdx.x + 256u; i < xchunks; i += 256u) {
+        xraw.fetch(xrow, i);
+        stage_store<X_BF16, PAIR>(xraw, i, lds_x, lds_s);
+    }
+    wk.load_masks(a);
     __syncthreads();
 
-    for (uint32_t s = 0; s < steps; ++s) {
-        uint32_t xr[XW];
-        float sx[4];
-        load_x_piece<TYPE, PAIR, XW>(lds_x, lds_s, li + s * L, c, xr, sx);
-        const bool more = s + 1 < steps;  // uniform
-#pragma unroll
-        for (int u = 0; u < NR; ++u) {
-            Piece<TYPE>& b = buf[u % D];
-            if constexpr (PAIR)
-                acc[u] += dot_pair(b, c, xr, sx, m4, m2, magic);
-            else
-                acc[u] += dot_f32(b, c, reinterpret_cast<const float*>(xr), sx);
-            // refill this buffer with the task D ahead: same step while slots remain,
-            // else the first slots of the next step
-            if (u + D < NR || more) {
-                const uint8_t* nxt = u + D < NR ? row_ptr(u + D) + (size_t)s * bstep
-                                                : row_ptr(u + D - NR) + (size_t)(s + 1) * bstep;
-                // Tie the refill to this task's result: without the (empty) asm the
-                // compiler hoists every refill above the arithmetic into fresh
-                // registers, which doubles the buffers and halves occupancy.
-                asm volatile("" : "+v"(nxt) : "v"(acc[u]));
-                b.load(nxt, c);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
+    wk.group(rowbase, 0u, false, a.y + (size_t)p * a.n, valid);
+}
 
-#pragma unroll
-    for (int u = 0; u < NR; ++u) {
-        const float v = group_sum(acc[u], a.log_l);
-        const uint32_t r = row0 + (uint32_t)u * rpw;
-        if (li == 0 && r < a.n) a.y[(size_t)p * a.n + r] = valid ? v : __builtin_nanf("");
+// Dense GEMV for matrices with many wave groups per CU: one workgroup of WAVES
+// waves per CU (the launch asks for more than half of the CU's LDS, so two never
+// share a CU), each CU owning an equal contiguous share of the wave groups.
+// Inside the CU the waves take wave groups from a counter in LDS instead of a
+// fixed split: the SIMD's issue arbitration favours its oldest wave, so with a
+// fixed split the youngest wave of every SIMD finishes long after the others and
+// the CU idles meanwhile.  A wave knows its next wave group one group ahead, so
+// the fetch ring runs across group boundaries.
+template <int TYPE, bool X_BF16, bool PAIR, int NR, int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemv_queue_kernel(KArgs a) {
+    constexpr uint32_t THREADS = 64 * WAVES;
+    extern __shared__ uint4 smem[];
+    uint32_t* lds_x = reinterpret_cast<uint32_t*>(smem);
+    float* lds_s = reinterpret_cast<float*>(lds_x + (PAIR ? a.k / 2 : a.k));
+    uint32_t* lds_q = reinterpret_cast<uint32_t*>(lds_s + a.k / 16);
+
+    const uint8_t* xrow = static_cast<const uint8_t*>(a.x);
+    const uint32_t xchunks = a.k / 16;
+    XRaw<X_BF16> xraw;
+    if (threadIdx.x < xchunks) xraw.fetch(xrow, threadIdx.x);
+
+    Walk<TYPE, X_BF16, PAIR, NR, D> wk;
+    wk.init(a, a.w, lds_x, lds_s);
+
+    // this CU's share of the wave groups: [begin, begin + count)
+    const uint32_t per = a.groups / gridDim.x, rem = a.groups % gridDim.x;
+    const uint32_t begin = blockIdx.x * per + (blockIdx.x < rem ? blockIdx.x : rem);
+    const uint32_t count = per + (blockIdx.x < rem ? 1u : 0u);
+    const uint32_t rows_per_group = wk.rpw * NR;
+
+    // the first WAVES wave groups are claimed by wave index, the rest from the counter
+    uint32_t cur = threadIdx.x >> 6;
+    if (cur < count) wk.prime((begin + cur) * rows_per_group);
+
+    if (threadIdx.x == 0) *lds_q = WAVES;
+    if (threadIdx.x < xchunks) stage_store<X_BF16, PAIR>(xraw, threadIdx.x, lds_x, lds_s);
+    for (uint32_t i = threadIdx.x + THREADS; i < xchunks; i += THREADS) {
+        xraw.fetch(xrow, i);
+        stage_store<X_BF16, PAIR>(xraw, i, lds_x, lds_s);
     }
+    wk.load_masks(a);
+    __syncthreads();
+
+    auto grab = [&]() -> uint32_t {
+        uint32_t v = 0;
+        if (wk.lane == 0) v = __hip_atomic_fetch_add(lds_q, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return v;
+    };
+    uint32_t nxt = __builtin_amdgcn_readfirstlane(grab());
+    while (cur < count) {
+        const uint32_t after = grab();  // claimed now, read when this group is done
+        wk.group((begin + cur) * rows_per_group, (begin + nxt) * rows_per_group, nxt < count, a.y, true);
+        cur = nxt;
+        nxt = __builtin_amdgcn_readfirstlane(after);
+    }
+}
+
+// The device's CU count, cached per device.
+int cu_count(uint32_t* out) {
+    static std::mutex mu;
+    static int cached[64] = {};
+    int dev = 0;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    std::lock_guard<std::mutex> lock(mu);
+    if (dev < 0 || dev >= 64 || cached[dev] == 0) {
+        int cus = 0;
+        if (int rc = check_hip(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev),
+                               "hipDeviceGetAttribute(CU count)"))
+            return rc;
+        if (cus <= 0) cus = 256;
+        if (dev < 0 || dev >= 64) {
+            *out = (uint32_t)cus;
+            return HQ_OK;
+        }
+        cached[dev] = cus;
+    }
+    *out = (uint32_t)cached[dev];
+    return HQ_OK;
+}
+
+template <typename K>
+int set_lds_limit(K kern, size_t lds, const char* what) {
+    if (lds <= 64 * 1024) return HQ_OK;
+    return check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                     what);
 }
 
 template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
 int launch_r(hipStream_t s, const KArgs& ka, uint32_t pairs, uint32_t rpw, size_t lds) {
     auto kern = gemv_kernel<TYPE, X_BF16, PAIR, NR, D>;
-    if (lds > 64 * 1024) {
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
-                               "hipFuncSetAttribute(gemv LDS)"))
-            return rc;
-    }
+    if (int rc = set_lds_limit(kern, lds, "hipFuncSetAttribute(gemv LDS)")) return rc;
     const uint32_t rows_per_wg = 4 * rpw * NR;
-    const dim3 grid((ka.n + rows_per_wg - 1) / rows_per_wg, pairs);
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, ka);
+    hipLaunchKernelGGL(kern, dim3((ka.n + rows_per_wg - 1) / rows_per_wg, pairs), dim3(256), lds, s, ka);
     return check_launch("gemv kernel launch");
+}
+
+template <int TYPE, bool X_BF16, bool PAIR, int NR, int D, int WAVES>
+int launch_q(hipStream_t s, KArgs ka, uint32_t cus, uint32_t rpw, size_t lds) {
+    auto kern = gemv_queue_kernel<TYPE, X_BF16, PAIR, NR, D, WAVES>;
+    if (lds < 81 * 1024) lds = 81 * 1024;  // more than half a CU's LDS: one workgroup per CU
+    if (int rc = set_lds_limit(kern, lds, "hipFuncSetAttribute(gemv queue LDS)")) return rc;
+    const uint32_t rows_per_group = rpw * NR;
+    ka.groups = (ka.n + rows_per_group - 1) / rows_per_group;
+    hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * WAVES), lds, s, ka);
+    return check_launch("gemv queue kernel launch");
 }
 
 template <int TYPE, bool X_BF16>
 int launch_t(hipStream_t s, const GemvArgs& a) {
     constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
     constexpr int EPL = Lane<TYPE>::kElems;
-    KArgs ka{a.x, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, M4, M2, MAGIC};
+    KArgs ka{a.x, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, M4, M2, MAGIC};
     const uint32_t pieces = a.k / EPL;
     // L = largest power of two <= 64 that divides the pieces of a row
     uint32_t log_l = 0;
     while (log_l < 6 && pieces % (2u << log_l) == 0) ++log_l;
     ka.log_l = log_l;
     const uint32_t rpw = 64u >> log_l;
-    const size_t lds = (size_t)(PAIR ? a.k * 2 : a.k * 4) + (size_t)(a.k / 16) * 4;
+    // activations, their per-16 sums, the queue counter
+    const size_t lds = (size_t)(PAIR ? a.k * 2 : a.k * 4) + (size_t)(a.k / 16) * 4 + 16;
     if (lds > 160 * 1024 - 512)
         return fail(HQ_ERR_UNSUPPORTED, "gemv: k = %u needs %zu bytes of LDS (limit 160 KiB)", a.k, lds);
-    // Tasks (row slot x step) one SIMD would get if the work were spread evenly over
-    // 256 CUs x 4 SIMDs; more slots per wave amortise the per-wave set-up, fewer keep
-    // every SIMD busy on small problems.
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
     const uint64_t slots = (uint64_t)((a.n + rpw - 1) / rpw) * a.pairs;
-    const uint64_t per_simd = slots / 1024;
-    if (per_simd >= 32) return launch_r<TYPE, X_BF16, PAIR, 8, 4>(s, ka, a.pairs, rpw, lds);
-    if (per_simd >= 8) return launch_r<TYPE, X_BF16, PAIR, 4, 2>(s, ka, a.pairs, rpw, lds);
+    // Dense matrices with many tasks per wave: the queue kernel.
+    if (a.pairs == 1 && slots * ((a.k / EPL) >> log_l) >= (uint64_t)cus * QUEUE_MIN_TASKS_PER_CU)
+        return launch_q<TYPE, X_BF16, PAIR, 2, 2, 12>(s, ka, cus, rpw, lds);
+    // Slots one SIMD would get if the work were spread evenly; more slots per wave
+    // amortise the per-wave set-up, fewer keep every SIMD busy on small problems.
+    const uint64_t per_simd = slots / (4ull * cus);
+    if (per_simd >= 8) return launch_r<TYPE, X_BF16, PAIR, 4, 4>(s, ka, a.pairs, rpw, lds);
     if (per_simd >= 2) return launch_r<TYPE, X_BF16, PAIR, 2, 2>(s, ka, a.pairs, rpw, lds);
     return launch_r<TYPE, X_BF16, PAIR, 1, 1>(s, ka, a.pairs, rpw, lds);
 }
