@@ -29,6 +29,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 
+# HBM bytes per launch of the dominant kernel of each workload, from rocprofv3 --pmc runs of this
+# file (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
+# for a device copy of known size (--calibration-copy): FETCH_SIZE reads half the bytes (factor
+# 2.0), WRITE_SIZE all of them (1.0).  The runs and their figures are in profiles/*_pmc_traffic.md.
+PMC_TRAFFIC_BYTES = {
+    "gemv_head_q6_k_151936x4096": int(249387.5 * 2.0 * 1024 + 755.3 * 1.0 * 1024),
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -46,6 +54,9 @@ def parse():
                     help="moe_decode / tq_attention: launch every kernel from the host instead of replaying a HIP "
                          "graph of the step (the steps are 4-12 launches of a few microseconds each)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run three 256 MiB device-to-device copies first: the known-size kernel that scales "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this file")
     return ap.parse_args()
 
 
@@ -315,6 +326,13 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.calibration_copy:
+        src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if a.workload != "decode_gemv":
         return {"moe_decode": bench_moe_decode, "prefill_gemm": bench_prefill_gemm,
                 "tq_attention": bench_tq_attention}[a.workload](a)
@@ -374,6 +392,24 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
+    # The same K steps once more as HIP-graph replays (one graph per weight-set / head rotation):
+    # what a caller that records its decode step gets, without the host's per-launch cost.  Reported
+    # beside `value`, which stays the host-launched figure the per-kernel events belong to.
+    graph = None
+    if not a.no_graph:
+        n_var = n_sets * n_heads
+        replay = _graphed(a, step, n_var)
+        for i in range(min(a.warmup, n_var)):
+            replay(i)
+        torch.cuda.synchronize()
+        t0g = time.perf_counter()
+        for i in range(a.steps):
+            replay(a.warmup + i)
+        torch.cuda.synchronize()
+        el_g = time.perf_counter() - t0g
+        graph = {"ms_per_step": round(el_g / a.steps * 1e3, 4), "GBps": round(step_bytes * a.steps / el_g / 1e9, 1),
+                 "frac_hbm_peak": round(step_bytes * a.steps / el_g / 1e9 / HBM_PEAK_GBS, 4)}
+
     names = ("gate", "up", "down", "head")
     kern_us = {nm: sum(evs[i][j][0].elapsed_time(evs[i][j][1]) for i in range(a.steps)) * 1e3 / a.steps
                for j, nm in enumerate(names)}
@@ -404,8 +440,10 @@ def main():
                    "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": "gemv Q6_K head 151936x4096", "achieved": round(head_gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": None, "us_per_launch": round(kern_us["head"], 3), "bytes_per_launch": nbytes["head"]},
+                     "traffic": PMC_TRAFFIC_BYTES["gemv_head_q6_k_151936x4096"],
+                     "us_per_launch": round(kern_us["head"], 3), "bytes_per_launch": nbytes["head"]},
         "kernels": kernels,
+        "graph_replay": graph,
         "q4_k_gemv": {"GBps": round(q4_bytes / q4_us / 1e3, 1), "frac_hbm_peak": round(q4_bytes / q4_us / 1e3 / HBM_PEAK_GBS, 4)},
     }
     out["cpu_baseline"] = None if a.no_cpu_baseline else cpu_baseline()

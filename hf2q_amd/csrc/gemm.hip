@@ -315,49 +315,54 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {
         // ---------------- Q4_K: offset and min terms once per super-block ----------------
         if constexpr (Q4) {
             const uint4 zero4 = make_uint4(0, 0, 0, 0);
+            bf16x8_t scf[2], sc0f[2], mnf[2];
+            float d128[2], dmn[2];
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt) {
                 const uint32_t brow = wn * 64 + nt * 32 + l32;
-                const bf16x8_t scf = as_frag(*reinterpret_cast<const uint4*>(smem + L::kSC + brow * 32 + 16 * lg));
+                scf[nt] = as_frag(*reinterpret_cast<const uint4*>(smem + L::kSC + brow * 32 + 16 * lg));
                 // (sc[8], 0[8]): the upper lane group contributes nothing
-                const bf16x8_t sc0f = as_frag(lg ? zero4 : *reinterpret_cast<const uint4*>(smem + L::kSC + brow * 32));
-                const bf16x8_t mnf = as_frag(*reinterpret_cast<const uint4*>(smem + L::kMN + brow * 32 + 16 * lg));
-                const float d128 = reinterpret_cast<const float*>(smem + L::kDD)[brow * 2];
-                const float dmn = reinterpret_cast<const float*>(smem + L::kDD)[brow * 2 + 1];
+                sc0f[nt] = as_frag(lg ? zero4 : *reinterpret_cast<const uint4*>(smem + L::kSC + brow * 32));
+                mnf[nt] = as_frag(*reinterpret_cast<const uint4*>(smem + L::kMN + brow * 32 + 16 * lg));
+                d128[nt] = reinterpret_cast<const float*>(smem + L::kDD)[brow * 2];
+                dmn[nt] = reinterpret_cast<const float*>(smem + L::kDD)[brow * 2 + 1];
+            }
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    const uint32_t arow = wm * (BM / 2) + mt * 32 + l32;
-                    // S = hi + mid + lo exactly (3 x 8 significant bits).  Lane group 0 feeds k slots 0..7
-                    // = S_hi (first operand) / S_lo (second), lane group 1 feeds slots 8..15 = S_mid / 0.
-                    const float4* Sp = reinterpret_cast<const float4*>(smem + L::kS + arow * 32);
-                    const float4 s0 = Sp[0], s1 = Sp[1];
-                    const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-                    uint32_t fa[8], fb[8];
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint32_t arow = wm * (BM / 2) + mt * 32 + l32;
+                // S = hi + mid + lo exactly (3 x 8 significant bits).  Lane group 0 feeds k slots 0..7
+                // = S_hi (first operand) / S_lo (second), lane group 1 feeds slots 8..15 = S_mid / 0.
+                const float4* Sp = reinterpret_cast<const float4*>(smem + L::kS + arow * 32);
+                const float4 s0 = Sp[0], s1 = Sp[1];
+                const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+                uint32_t fa[8], fb[8];
 #pragma unroll
-                    for (int q = 0; q < 8; ++q) {
-                        const uint32_t sh = bf16_rne(sv[q]);
-                        const float r1 = sv[q] - bf16_bits_to_f32(sh);
-                        const uint32_t sm = bf16_rne(r1);
-                        const uint32_t sl = bf16_rne(r1 - bf16_bits_to_f32(sm));
-                        fa[q] = lg ? sm : sh;
-                        fb[q] = lg ? 0u : sl;
-                    }
-                    const bf16x8_t sa = as_frag(make_uint4(fa[0] | (fa[1] << 16), fa[2] | (fa[3] << 16),
-                                                           fa[4] | (fa[5] << 16), fa[6] | (fa[7] << 16)));
-                    const bf16x8_t sb = as_frag(make_uint4(fb[0] | (fb[1] << 16), fb[2] | (fb[3] << 16),
-                                                           fb[4] | (fb[5] << 16), fb[6] | (fb[7] << 16)));
+                for (int q = 0; q < 8; ++q) {
+                    const uint32_t sh = bf16_rne(sv[q]);
+                    const float r1 = sv[q] - bf16_bits_to_f32(sh);
+                    const uint32_t sm = bf16_rne(r1);
+                    const uint32_t sl = bf16_rne(r1 - bf16_bits_to_f32(sm));
+                    fa[q] = lg ? sm : sh;
+                    fb[q] = lg ? 0u : sl;
+                }
+                const bf16x8_t sa = as_frag(make_uint4(fa[0] | (fa[1] << 16), fa[2] | (fa[3] << 16),
+                                                       fa[4] | (fa[5] << 16), fa[6] | (fa[7] << 16)));
+                const bf16x8_t sb = as_frag(make_uint4(fb[0] | (fb[1] << 16), fb[2] | (fb[3] << 16),
+                                                       fb[4] | (fb[5] << 16), fb[6] | (fb[7] << 16)));
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) {
                     f32x16_t t;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) t[v] = 0.f;
-                    t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sa, scf, t, 0, 0, 0);   // sc*(S_hi+S_mid)
-                    t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sb, sc0f, t, 0, 0, 0);  // sc*S_lo
+                    t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sa, scf[nt], t, 0, 0, 0);   // sc*(S_hi+S_mid)
+                    t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sb, sc0f[nt], t, 0, 0, 0);  // sc*S_lo
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[mt][nt][v] = fmaf(t[v], d128, acc[mt][nt][v]);
+                    for (int v = 0; v < 16; ++v) acc[mt][nt][v] = fmaf(t[v], d128[nt], acc[mt][nt][v]);
 #pragma unroll
                     for (int v = 0; v < 16; ++v) t[v] = 0.f;
-                    t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sa, mnf, t, 0, 0, 0);   // mn*(S_hi+S_mid)
+                    t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sa, mnf[nt], t, 0, 0, 0);   // mn*(S_hi+S_mid)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[mt][nt][v] = fmaf(t[v], dmn, acc[mt][nt][v]);
+                    for (int v = 0; v < 16; ++v) acc[mt][nt][v] = fmaf(t[v], dmn[nt], acc[mt][nt][v]);
                 }
             }
             __syncthreads();  // the next super-block's staging rewrites the S / code arrays
