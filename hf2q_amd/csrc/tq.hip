@@ -150,13 +150,22 @@ __device__ __forceinline__ uint32_t bf16_rne(float f) {
     return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
 }
 
+// Orders a wave's own LDS accesses for the compiler; the hardware serves one wave's LDS
+// instructions in issue order, so data a lane wrote is there when another lane of the same wave
+// reads it afterwards.
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // One workgroup: one kv head, one chunk of <= 8 query heads of its group, one split of the sequence.
 template <bool LUT>
 __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     __shared__ float s_q[8][HD];          // the chunk's queries (rotated here when fuse_fwht_pre)
+    __shared__ uint4 s_qh[8][33], s_ql[8][33];  // their bf16 hi / lo halves, 8 values per entry
     __shared__ float s_p[4][16][8];       // per wave: p * norm_v of the current tile, [position][head]
     __shared__ float s_alpha[4][8];       // per wave: rescale factor of the running output
-    __shared__ uint32_t s_slot[4][16];    // per wave: physical slot of each tile position
     __shared__ float s_o[4][8][HD];       // per wave outputs for the final merge
     __shared__ float s_m[4][8], s_l[4][8];
     __shared__ float s_lut[LUT ? 256 : 1];
@@ -167,6 +176,49 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     const uint32_t h0 = kvh * a.group + hc * 8u;
     const uint32_t nh = min(8u, a.group - hc * 8u);
     const uint32_t split = blockIdx.x;
+
+    const uint32_t j = lane & 15u, g = lane >> 4;
+    const uint32_t half = lane >> 5, dg = lane & 31u;
+    const size_t head_base = (size_t)kvh * a.kv_capacity;
+    const uint32_t split_first = a.first + split * (a.tiles_per_wave * 64u);
+
+    // Operands of one 16-position tile of this wave.  K: lane (position j, quarter g) holds 64
+    // contiguous code bytes; V: lane (half, dg) holds coordinates 8*dg..+7 of positions 2t + half.
+    struct Tile {
+        uint4 k0, k1, k2, k3;
+        uint2 v[8];
+        float kn, vn;
+        bool ok;
+    };
+    // physical slot of logical position idx (ring buffer); ring_start, idx < kv_capacity
+    auto slot_of = [&](uint32_t idx) -> uint32_t {
+        const uint32_t s = a.ring_start + idx;
+        return s >= a.kv_capacity ? s - a.kv_capacity : s;
+    };
+    auto load_tile = [&](uint32_t it, Tile& t) {
+        const uint32_t tile0 = split_first + (it * 4u + wave) * 16u;  // first logical position of this wave's tile
+        const uint32_t idx = tile0 + j;
+        t.ok = idx < a.last;
+        const uint32_t slot = slot_of(t.ok ? idx : a.first);  // positions past the end read a valid slot, weight 0
+        const uint4* kp = reinterpret_cast<const uint4*>(a.k_codes + (head_base + slot) * HD + 64 * g);
+        t.k0 = kp[0], t.k1 = kp[1], t.k2 = kp[2], t.k3 = kp[3];
+        t.kn = a.k_norms[head_base + slot];
+        t.vn = t.ok ? a.v_norms[head_base + slot] : 0.f;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const uint32_t vi = tile0 + 2 * q + half;
+            const uint32_t vs = slot_of(vi < a.last ? vi : a.first);
+            t.v[q] = *reinterpret_cast<const uint2*>(a.v_codes + (head_base + vs) * HD + 8 * dg);
+        }
+    };
+
+    // s_p / s_alpha are private to the wave and LDS serves a wave's accesses in order, so the tile
+    // loop needs no workgroup barrier.
+    // The first tile is requested before anything else so that its trip from HBM overlaps the
+    // staging of the queries; inside the loop the next tile is requested before the current one is
+    // worked on.  With one or two waves per SIMD nothing else hides the latency.
+    Tile cur, nxt;
+    load_tile(0, cur);
 
     // ---- queries -> LDS (zero rows for absent heads), optional sign x FWHT ----
     for (uint32_t i = tid; i < 8 * HD / 4; i += 256) {
@@ -189,20 +241,27 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
         __syncthreads();
     }
 
-    // ---- query fragments: lane (j = lane%16: head, g = lane/16) holds q[j][64g + 8kk + e] ----
-    const uint32_t j = lane & 15u, g = lane >> 4;
-    uint4 qhi[8], qlo[8];
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
+    // ---- query fragments: lane (j = lane%16: head, g = lane/16) holds q[j][64g + 8kk + e] as an exact
+    // bf16 hi + lo pair.  The split is done once per workgroup (thread = head tid/32, chunk tid%32 of 8
+    // values) and every wave reads its fragments back; rows are padded to 33 chunks against bank conflicts.
+    {
+        const uint32_t h = tid >> 5, ch = tid & 31u;
         uint32_t hi[8], lo[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float x = j < 8 ? s_q[j][64 * g + 8 * kk + e] : 0.f;
+            const float x = s_q[h][8 * ch + e];
             hi[e] = bf16_rne(x);
             lo[e] = bf16_rne(x - bf16_bits_to_f32(hi[e]));
         }
-        qhi[kk] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16));
-        qlo[kk] = make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16));
+        s_qh[h][ch] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16));
+        s_ql[h][ch] = make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16));
+    }
+    __syncthreads();
+    uint4 qhi[8], qlo[8];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+        qhi[kk] = j < 8 ? s_qh[j][8 * g + kk] : make_uint4(0, 0, 0, 0);
+        qlo[kk] = j < 8 ? s_ql[j][8 * g + kk] : make_uint4(0, 0, 0, 0);
     }
 
     // ---- running state ----
@@ -212,30 +271,16 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     for (int h = 0; h < 8; ++h)
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
-    const uint32_t half = lane >> 5, dg = lane & 31u;
 
-    const size_t head_base = (size_t)kvh * a.kv_capacity;
-    const uint32_t split_first = a.first + split * (a.tiles_per_wave * 64u);
 
     for (uint32_t it = 0; it < a.tiles_per_wave; ++it) {
-        const uint32_t tile0 = split_first + (it * 4u + wave) * 16u;  // first logical position of this wave's tile
-        // -------- K tile: lane (position i = lane%16, quarter g) loads 64 contiguous code bytes --------
-        const uint32_t idx = tile0 + j;
-        const bool ok = idx < a.last;
-        const uint32_t slot = (uint32_t)(((uint64_t)a.ring_start + (ok ? idx : a.first)) % a.kv_capacity);
-        const uint4* kp = reinterpret_cast<const uint4*>(a.k_codes + (head_base + slot) * HD + 64 * g);
-        const uint4 k0 = kp[0], k1 = kp[1], k2 = kp[2], k3 = kp[3];
-        const float kn = a.k_norms[head_base + slot];
-        const float vn = ok ? a.v_norms[head_base + slot] : 0.f;
-        if (g == 0) s_slot[wave][j] = slot;
-        __syncthreads();  // s_slot visible; also fences the previous tile's reads of s_p / s_alpha
-        // -------- V codes of this tile: lane (half, dg) takes positions 2t + half --------
+        if (it + 1 < a.tiles_per_wave) load_tile(it + 1, nxt);
+        const uint4 k0 = cur.k0, k1 = cur.k1, k2 = cur.k2, k3 = cur.k3;
+        const float kn = cur.kn, vn = cur.vn;
+        const bool ok = cur.ok;
         uint2 vraw[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const uint32_t vs = s_slot[wave][2 * t + half];
-            vraw[t] = *reinterpret_cast<const uint2*>(a.v_codes + (head_base + vs) * HD + 8 * dg);
-        }
+        for (int q = 0; q < 8; ++q) vraw[q] = cur.v[q];
         // -------- scores on the matrix cores --------
         f32x4_t c = {0.f, 0.f, 0.f, 0.f};
         const uint32_t kw[16] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w,
@@ -291,7 +336,7 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
         l_run = l_run * alpha + psum;
         m_run = m_new;
         if (g == 0 && j < 8) s_alpha[wave][j] = alpha;
-        __syncthreads();
+        wave_lds_fence();  // the wave's own writes of s_p / s_alpha before its reads below
         // -------- P.V on the VALU --------
         {
             const float4 a0 = *reinterpret_cast<const float4*>(&s_alpha[wave][0]);
@@ -321,6 +366,8 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) acc[h][e] = fmaf(pp[h], vv[e], acc[h][e]);
         }
+        wave_lds_fence();  // reads of s_p / s_alpha before the next tile overwrites them
+        cur = nxt;
     }
 
     // ---- merge the two position-halves of the wave, then the four waves, and emit the split's partial ----
@@ -367,13 +414,13 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
 // the loads of 8 splits in flight at a time.
 __global__ __launch_bounds__(256) void tq_attn_reduce_kernel(const float* __restrict__ tmp, float* __restrict__ out,
                                                              uint32_t n_splits) {
-    __shared__ float s_w[128];  // e^{m_s - m}
+    __shared__ float s_w[256];  // e^{m_s - m}
     __shared__ float s_part[4][64];
     __shared__ float s_red[4];
     const uint32_t h = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t d = blockIdx.y * 64u + lane;
     const float* base = tmp + (size_t)h * n_splits * TMP_STRIDE;
-    // n_splits <= 128: threads 0..127 fetch the running maxima and sums
+    // n_splits <= 256 = the workgroup size: one thread per split fetches its running maximum and sum
     float ms = -INFINITY, ls = 0.f;
     if (tid < n_splits) {
         ms = base[(size_t)tid * TMP_STRIDE + HD];
@@ -386,7 +433,7 @@ __global__ __launch_bounds__(256) void tq_attn_reduce_kernel(const float* __rest
     __syncthreads();
     m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
     const float w = ms == -INFINITY ? 0.f : __expf(ms - m);
-    if (tid < 128) s_w[tid] = w;
+    s_w[tid] = w;
     float lw = w * ls;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
@@ -437,7 +484,8 @@ static void visible_range(const hq_tq_attn_params& p, uint32_t& first, uint32_t&
 }
 
 uint32_t tq_attn_splits(uint32_t n_positions) {
-    // 64 positions (one 16-position tile per wave) is the least a workgroup takes; at most 128 splits.
+    // 64 positions (one 16-position tile per wave) is the least a workgroup takes; at most 256 splits
+    // (two workgroups per CU at two kv heads).
     const uint32_t groups = (n_positions + 63u) / 64u;
     return groups < 128u ? (groups ? groups : 1u) : 128u;
 }
