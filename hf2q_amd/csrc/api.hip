@@ -103,14 +103,17 @@ static int check_matmul_common(const char* fn, const void* x, hq_act_dtype xdt, 
     return check_weight_alignment(w, t);
 }
 
-int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y,
-                    uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
-    if (int rc = check_matmul_common("hq_qmatmul_ggml", x, xdt, w_blocks, y, n, k, t)) return rc;
-    if (m == 0) return HQ_OK;
-    if (m > kGemvMaxRows && gemm_supported(t, k))
-        return launch_gemm((hipStream_t)stream, x, xdt, w_blocks, y, m, n, k, t);
+namespace {
+
+bool q4k_tile_route(uint32_t m, uint32_t k, hq_ggml_type t) { return t == HQ_Q4_K && m > kGemvMaxRows && k % 256 == 0; }
+
+// All routes of the dense product; `workspace` is only read on the Q4_K tile route.
+int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
+                   uint32_t n, uint32_t k, hq_ggml_type t, void* workspace) {
+    if (q4k_tile_route(m, k, t)) return launch_gemm_q4k(stream, x, xdt, w_blocks, y, m, n, k, workspace);
+    if (m > kGemvMaxRows && gemm_supported(t, k)) return launch_gemm(stream, x, xdt, w_blocks, y, m, n, k, t);
     // GEMV form, kGemvMaxRows activation rows per launch (also the route of shapes the
-    // tile kernel does not cover).
+    // tile kernels do not cover).
     const size_t xrow_bytes = (size_t)k * (xdt == HQ_BF16 ? 2 : 4);
     for (uint32_t r0 = 0; r0 < m; r0 += kGemvMaxRows) {
         GemvArgs a{};
@@ -124,9 +127,46 @@ int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w
         a.k = k;
         a.n_experts = 1;
         a.expert_stride = 0;
-        if (int rc = launch_gemv((hipStream_t)stream, a, xdt, t)) return rc;
+        if (int rc = launch_gemv(stream, a, xdt, t)) return rc;
     }
     return HQ_OK;
+}
+
+}  // namespace
+
+size_t hq_qmatmul_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
+    (void)n;
+    (void)xdt;
+    return q4k_tile_route(m, k, t) ? gemm_q4k_workspace_bytes(m, k) : 0;
+}
+
+int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
+                       uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes) {
+    if (int rc = check_matmul_common("hq_qmatmul_ggml_ws", x, xdt, w_blocks, y, n, k, t)) return rc;
+    if (m == 0) return HQ_OK;
+    const size_t need = hq_qmatmul_ggml_workspace_bytes(m, n, k, xdt, t);
+    if (need) {
+        if (!workspace || workspace_bytes < need)
+            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_ggml_ws: workspace of %zu bytes, %zu needed",
+                        workspace ? workspace_bytes : (size_t)0, need);
+        if (reinterpret_cast<uintptr_t>(workspace) % 256)
+            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_ggml_ws: workspace must be 256-byte aligned");
+    }
+    return qmatmul_routes((hipStream_t)stream, x, xdt, w_blocks, y, m, n, k, t, workspace);
+}
+
+int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y,
+                    uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
+    if (int rc = check_matmul_common("hq_qmatmul_ggml", x, xdt, w_blocks, y, n, k, t)) return rc;
+    if (m == 0) return HQ_OK;
+    const size_t need = hq_qmatmul_ggml_workspace_bytes(m, n, k, xdt, t);
+    if (!need) return qmatmul_routes((hipStream_t)stream, x, xdt, w_blocks, y, m, n, k, t, nullptr);
+    void* ws = nullptr;
+    if (int rc = check_hip(hipMallocAsync(&ws, need, (hipStream_t)stream), "hipMallocAsync(qmatmul workspace)"))
+        return rc;
+    const int rc = qmatmul_routes((hipStream_t)stream, x, xdt, w_blocks, y, m, n, k, t, ws);
+    const int rc_free = check_hip(hipFreeAsync(ws, (hipStream_t)stream), "hipFreeAsync(qmatmul workspace)");
+    return rc ? rc : rc_free;
 }
 
 size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows) {

@@ -1,0 +1,428 @@
+// Batched-prefill GEMM for Q4_K weights (m > 8): y[m,n] = x[m,k] . W[n,k]^T on the
+// f16 matrix cores (v_mfma_f32_32x32x16_f16) with fp32 accumulation.
+//
+// Numerics.  The weight tile holds the dequantised weights rounded to f16, which
+// is what the reference's mul_mm kernels multiply as well (their weight tile is
+// simdgroup_half8x8): w = d*sc*q - dmin*mn is formed in fp32 (exact up to one
+// rounding) and rounded once to f16, a relative error of at most 2^-12 per
+// weight.  The activations are f16 too.  f16 has a narrow exponent range, so a
+// pre-pass rescales every activation row by a power of two that brings its
+// largest magnitude into [512, 1024) and the epilogue scales back: bf16
+// activations are represented exactly (8-bit significands; values more than
+// 2^-34 below the row maximum lose bits, far under fp32 resolution of the
+// result), f32 activations are rounded to 11 bits.  Products are exact in the
+// MFMA and accumulate in fp32.  Weight rows get a power-of-two scale of their own
+// (from the row's largest super-block scale) for the same reason.  The result
+// agrees with an f64 product over the
+// exact weights to about 1.5e-4 of the output's scale (rms), where the kernels
+// that keep every product exact reach 1e-6.
+//
+// Structure.  Workgroup = 256 threads = 2x2 waves, tile 256 (tokens) x 128
+// (weight rows) x 64 (k) per stage; a wave owns 128x64 = 4x2 MFMA tiles (128
+// accumulator registers).
+//   * Activations: the pre-pass output goes global -> LDS directly
+//     (global_load_lds_dwordx4, no registers, no VALU), double buffered, one
+//     barrier per stage.  A wave instruction fills 1 KB of LDS with lane i at
+//     byte 16*i, so tile rows are 128 bytes without padding and the 16-byte
+//     chunks of a row are XOR-swizzled with the row number: lane i fetches the
+//     global chunk (i%8) ^ (i/8) of its row, and the 16-byte fragment reads are
+//     conflict free.
+//   * Weights never touch LDS: a lane fetches the 16 nibble bytes it needs for
+//     its own fragments (row lane%32, bytes 16*(lane/32).. of the 64-element
+//     chunk) straight from global memory, a stage ahead, and dequantises them
+//     in registers.  LDS bandwidth is the scarce resource of this tile shape (a
+//     32x32x16 MFMA consumes 2 KB of fragments per 32 cycles); keeping one
+//     operand out of it is what lets the matrix cores run.  The two waves that
+//     share weight rows dequantise them twice.
+//   * k order.  Inside a stage the MFMA contraction index is a permutation of k
+//     chosen so that a lane's fragments come from its own 16 nibble bytes: lane
+//     group g of k-step s covers k = 16g + 8s + j (s < 2, low nibbles) or
+//     32 + 16g + 8(s-2) + j (high nibbles); for the activations that is only
+//     the address of the fragment.
+#include "hq_internal.h"
+
+namespace hq {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+constexpr int BK = 64;
+constexpr int ROW = BK;  // f16 elements per LDS tile row (128 bytes, chunks XOR-swizzled)
+
+// workspace: [xh m*k f16][rs m f32]
+struct Workspace {
+    size_t xh, rs, total;
+};
+__host__ __device__ inline Workspace workspace_layout(uint32_t m, uint32_t k) {
+    Workspace w;
+    w.xh = 0;
+    w.rs = ((size_t)m * k * 2 + 255) & ~(size_t)255;
+    w.total = w.rs + (((size_t)m * 4 + 255) & ~(size_t)255);
+    return w;
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return fmaxf(v, __int_as_float(t));
+}
+
+__device__ __forceinline__ uint32_t f16_bits(float v) {
+    return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)v);
+}
+
+// Pre-pass, one workgroup per activation row: row scale and f16 conversion.
+template <bool X_BF16>
+__global__ __launch_bounds__(256) void q4k_prep_kernel(const void* __restrict__ x, uint8_t* __restrict__ ws,
+                                                       uint32_t m, uint32_t k) {
+    __shared__ float red[4];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    const Workspace L = workspace_layout(m, k);
+    const uint32_t chunks = k / 8;
+
+    auto load8 = [&](uint32_t i, float* v) {
+        if constexpr (X_BF16) {
+            const uint4 u = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + (size_t)row * k + 8 * i);
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] = bf16_bits_to_f32(w[j] & 0xffffu);
+                v[2 * j + 1] = bf16_bits_to_f32(w[j] >> 16);
+            }
+        } else {
+            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(x) + (size_t)row * k + 8 * i);
+            const float4 a = p[0], b = p[1];
+            v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+        }
+    };
+
+    // largest finite magnitude of the row
+    float amax = 0.f;
+    for (uint32_t i = tid; i < chunks; i += 256) {
+        float v[8];
+        load8(i, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float a = fabsf(v[j]);
+            amax = a <= 3.0e38f ? fmaxf(amax, a) : amax;  // inf / nan do not set the scale
+        }
+    }
+    amax = dpp_max<0xB1>(amax);
+    amax = dpp_max<0x4E>(amax);
+    amax = dpp_max<0x141>(amax);
+    amax = dpp_max<0x140>(amax);
+    amax = fmaxf(amax, __shfl_xor(amax, 16));
+    amax = fmaxf(amax, __shfl_xor(amax, 32));
+    if ((tid & 63u) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+
+    int ex = 0;
+    if (amax > 0.f) (void)frexpf(amax, &ex);  // amax = f * 2^ex, f in [0.5, 1)
+    int sh = 10 - ex;                          // amax * 2^sh in [512, 1024)
+    sh = sh < -100 ? -100 : sh > 100 ? 100 : sh;
+    if (amax == 0.f) sh = 0;
+    const float scale = ldexpf(1.f, sh);
+    if (tid == 0) reinterpret_cast<float*>(ws + L.rs)[row] = ldexpf(1.f, -sh);
+
+    for (uint32_t i = tid; i < chunks; i += 256) {
+        float v[8];
+        load8(i, v);
+        uint32_t h[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) h[j] = f16_bits(v[j] * scale);
+        *reinterpret_cast<uint4*>(ws + L.xh + ((size_t)row * k + 8 * i) * 2) =
+            make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+    }
+}
+
+struct GemmArgs {
+    const uint8_t* ws;  // workspace filled by the pre-pass
+    const uint8_t* w;
+    float* y;
+    uint32_t m, n, k;
+};
+
+__device__ __forceinline__ f16x8_t as_frag(uint4 v) { return __builtin_bit_cast(f16x8_t, v); }
+
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+
+__device__ __forceinline__ uint4 ld16(const uint8_t* p) { return *reinterpret_cast<const uint4*>(p); }
+
+// Four nibbles, one per byte of `nib4`, -> four f16 weights (two words): d*sc*q - dmin*mn in fp32
+// (dsc = d*sc and ndm = -dmin*mn are exact), one rounding to f16.  The masked word is made opaque
+// so that the four conversions stay v_cvt_f32_ubyte0..3 of one register instead of a bit-field
+// extract plus conversion each.
+__device__ __forceinline__ void weights4(uint32_t nib4, float dsc, float ndm, uint32_t& lo, uint32_t& hi) {
+    asm volatile("" : "+v"(nib4));
+    const f32x2_t a = {fmaf(ubyte0(nib4), dsc, ndm), fmaf(ubyte1(nib4), dsc, ndm)};
+    const f32x2_t b = {fmaf(ubyte2(nib4), dsc, ndm), fmaf(ubyte3(nib4), dsc, ndm)};
+    lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(a, f16x2_t));
+    hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(b, f16x2_t));
+}
+
+constexpr int WN = 2;              // waves along the weight rows (and 2 along the tokens)
+constexpr int MT = 4;              // 32-row MFMA tiles per wave along the tokens
+constexpr int BM = 64 * MT;        // token rows per workgroup
+constexpr int BN = 64 * WN;        // weight rows per workgroup
+constexpr int DMA_PER_WAVE = (BM / 8) / (2 * WN);  // BM / 8 one-KB fetches fill the activation tile
+
+__global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
+    extern __shared__ uint4 smem4[];
+    uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
+    constexpr int kTile = BM * ROW * 2;  // one activation tile, padded; two of them in LDS
+    const Workspace W = workspace_layout(a.m, a.k);
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const uint32_t l32 = lane & 31u, lg = lane >> 5;
+
+    // Tile order: workgroups go to the 8 XCDs round-robin and every XCD has its own L2, so workgroup
+    // i runs on XCD i % 8.  Each XCD gets whole rows of tiles (one activation tile, which then stays
+    // in that XCD's L2) and sweeps the weight tiles.
+    const uint32_t tiles_n = (a.n + BN - 1) / BN, tiles_m = (a.m + BM - 1) / BM;
+    uint32_t m0, n0;
+    {
+        const uint32_t xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3;
+        const uint32_t rows_here = (tiles_m + 7u - xcd) / 8u;
+        if (idx >= rows_here * tiles_n) return;  // the grid is padded to 8 * ceil(tiles_m / 8) * tiles_n
+        m0 = (xcd + 8u * (idx / tiles_n)) * BM;
+        n0 = (idx % tiles_n) * BN;
+    }
+    const uint32_t nsb = a.k / 256, nstages = a.k / BK;
+    const uint32_t row_bytes = nsb * Q4K_BYTES;
+
+    // ---- activation staging: wave w, instruction i (< DMA_PER_WAVE) fills 8 LDS rows of the tile,
+    // (w * DMA_PER_WAVE + i) * 8 .. +8; lane L owns row L/8 of them and LDS chunk L%8, which holds
+    // global chunk (L%8) ^ (L/8) ----
+    // byte offset of this lane's source chunk from the tile's first row, stage 0: the wave's first row + L/8
+    // for i = 0, 8 rows further per instruction; rows past the end of x read the last row instead (their
+    // results are never stored)
+    const uint32_t a_swz = ((lane & 7u) ^ (lane >> 3)) << 4;
+    const uint32_t a_row0 = wave * (8u * DMA_PER_WAVE) + (lane >> 3);
+    const uint32_t a_rows_left = a.m - m0;  // >= 1
+    const uint32_t a_last = (a_rows_left - 1u) * (a.k * 2u) + a_swz;
+    const uint8_t* xtile = a.ws + W.xh + (size_t)m0 * a.k * 2;
+    const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);  // the same value, known to be uniform
+    // LDS byte address of the tile buffers (wave-uniform, goes to M0)
+    const uint32_t lds_base =
+        __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem);
+    // Issued as inline assembly: the compiler would otherwise wait for every outstanding
+    // global_load_lds before any later LDS read (it cannot tell the two tile buffers apart), which
+    // exposes the whole fetch latency in every stage.  The waits are placed by hand below.
+    auto load_a = [&](uint32_t st, uint32_t buf) {
+#pragma unroll
+        for (int i = 0; i < DMA_PER_WAVE; ++i) {
+            const uint32_t r = a_row0 + 8u * i;
+            const uint8_t* src = xtile + (r < a_rows_left ? r * (a.k * 2u) + a_swz : a_last) + (size_t)st * (BK * 2);
+            const uint32_t dst = lds_base + buf * kTile + (wave_u * DMA_PER_WAVE + i) * 1024u;
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+            __builtin_amdgcn_sched_barrier(0);  // one address at a time: keeps eight 64-bit pointers out of the registers
+        }
+    };
+
+    // ---- weights: this lane's two rows (one per 32-row tile of the wave), bytes 16*lg.. of each chunk ----
+    const uint8_t* wrow[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+        uint32_t gn = n0 + wn * 64 + nt * 32 + l32;
+        gn = gn < a.n ? gn : a.n - 1u;
+        wrow[nt] = a.w + (size_t)gn * row_bytes;
+    }
+    // Per weight row, a power of two that brings the row's largest possible |w| = |d|*63*15 + |dmin|*63
+    // to about 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
+    // subnormals; the weights are multiplied by it before they are rounded (exact) and the epilogue
+    // divides it out.  Both waves that share a row compute the same value.
+    float wdown[2];  // 2^-e of this lane's two rows
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+        float bound = 0.f;
+        for (uint32_t sb = 0; sb < nsb; ++sb) {
+            const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow[nt] + (size_t)sb * Q4K_BYTES);
+            const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * 945.f + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
+            bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;  // inf / nan scales do not set the exponent
+        }
+        int ex = 0;
+        if (bound > 0.f) (void)frexpf(bound, &ex);  // bound = f * 2^ex, f in [0.5, 1)
+        const int e = bound > 0.f ? ex - 14 : 0;
+        wdown[nt] = ldexpf(1.f, -e);  // |e| <= 40: a normal number
+    }
+    uint4 braw[2][2];       // [stage parity][nt]
+    uint4 hdr[2], hdrn[2];  // super-block headers: current, next
+    auto load_b = [&](uint32_t sblk, int c, int slot) {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+            braw[slot][nt] = ld16(wrow[nt] + (size_t)sblk * Q4K_BYTES + 16 + 32 * c + 16 * lg);
+    };
+    auto load_hdr = [&](uint32_t sblk, uint4* h) {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) h[nt] = ld16(wrow[nt] + (size_t)sblk * Q4K_BYTES);
+    };
+
+    f32x16_t acc[MT][2];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // prologue: activations of stage 0 on their way to LDS, weights of stage 0 requested
+    load_hdr(0, hdr);
+    load_b(0, 0, 0);
+    load_a(0, 0);
+    if (nsb > 1) load_hdr(1, hdrn);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    for (uint32_t sblk = 0; sblk < nsb; ++sblk) {
+        const bool next_sb = sblk + 1 < nsb;  // uniform
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t st = 4 * sblk + c;
+            const uint32_t buf = c & 1;
+            // This stage's nibbles, requested a stage ago.  They are claimed here, before the activation
+            // fetch below is issued: the compiler does not know about that fetch, and the wait it puts
+            // in front of the first use of these registers would otherwise cover it too.
+            uint4 b0 = braw[c & 1][0], b1 = braw[c & 1][1];
+            asm volatile("" : "+v"(b0.x), "+v"(b0.y), "+v"(b0.z), "+v"(b0.w), "+v"(b1.x), "+v"(b1.y), "+v"(b1.z), "+v"(b1.w));
+            if (c == 0 && sblk > 0) {  // this super-block's header; request the next one (before the
+                hdr[0] = hdrn[0];      // activation fetch, so that it is older than it)
+                hdr[1] = hdrn[1];
+                if (next_sb) load_hdr(sblk + 1, hdrn);
+            }
+            // next stage's activations into the other buffer (free since the barrier that ended the
+            // previous stage)
+            if (st + 1 < nstages) load_a(st + 1, buf ^ 1u);
+
+            // this stage's weight scales: sub-blocks 2c (low nibbles) and 2c+1 (high nibbles)
+            float dsc[2][2], ndm[2][2];  // [nt][low / high]
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                uint32_t sc0, sc1, mn0, mn1;
+                q4k_scales(hdr[nt].y, hdr[nt].z, hdr[nt].w, c, sc0, sc1, mn0, mn1);
+                const float d = f16_bits_to_f32(hdr[nt].x & 0xffffu) * wdown[nt];
+                const float dmin = f16_bits_to_f32(hdr[nt].x >> 16) * wdown[nt];
+                dsc[nt][0] = d * (float)sc0;
+                dsc[nt][1] = d * (float)sc1;
+                ndm[nt][0] = -dmin * (float)mn0;
+                ndm[nt][1] = -dmin * (float)mn1;
+            }
+            // request the next stage's nibbles into the other pair of registers (the header fetch of a
+            // super-block, issued a super-block ahead, has already pulled most of its lines into cache)
+            if (c < 3) {
+                load_b(sblk, c + 1, (c & 1) ^ 1);
+            } else if (next_sb) {
+                load_b(sblk + 1, 0, (c & 1) ^ 1);
+            }
+
+            // ---- the stage's 4*MT steps (k-step ks = t/MT, row tile mt = t%MT), software pipelined:
+            // the activation fragment of step t+1 is requested, and a share of the next k-step's
+            // weight fragments is dequantised, between the two MFMAs of step t ----
+            auto a_frag = [&](int t) -> uint4 {
+                const int ks = t / MT, mt = t % MT;
+                // chunk index of this lane group's 8 activations inside the row's 64
+                const uint32_t kchunk = ks < 2 ? 2u * lg + ks : 4u + 2u * lg + (ks - 2);
+                const uint32_t row = wm * (32 * MT) + mt * 32 + l32;
+                return *reinterpret_cast<const uint4*>(smem + buf * kTile + row * (ROW * 2) + ((kchunk ^ (row & 7u)) << 4));
+            };
+            // quarter q (nt = q/2, word pair half = q%2) of k-step ks: four weights -> words 2*(q%2), +1
+            auto b_quarter = [&](int ks, int q, uint4* bfw) {
+                const int nt = q >> 1, half = q & 1;
+                const uint4 b = nt == 0 ? b0 : b1;
+                const uint32_t w = (ks & 1) ? (half ? b.w : b.z) : (half ? b.y : b.x);
+                const int hi = ks >> 1;  // 0: low nibbles, 1: high nibbles
+                uint32_t lo2, hi2;
+                weights4((hi ? w >> 4 : w) & 0x0f0f0f0fu, dsc[nt][hi], ndm[nt][hi], lo2, hi2);
+                if (half == 0)
+                    bfw[nt].x = lo2, bfw[nt].y = hi2;
+                else
+                    bfw[nt].z = lo2, bfw[nt].w = hi2;
+            };
+            uint4 bfc[2], bfn[2];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) b_quarter(0, q, bfc);
+            uint4 af0 = a_frag(0), af1;
+#pragma unroll
+            for (int t = 0; t < 4 * MT; ++t) {
+                const int ks = t / MT, mt = t % MT;
+                if (t + 1 < 4 * MT) af1 = a_frag(t + 1);
+                acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(af0), as_frag(bfc[0]), acc[mt][0], 0, 0, 0);
+                if (ks + 1 < 4) {
+#pragma unroll
+                    for (int q = 0; q < 4 / MT; ++q) b_quarter(ks + 1, mt * (4 / MT) + q, bfn);
+                }
+                acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(af0), as_frag(bfc[1]), acc[mt][1], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                af0 = af1;
+                if (mt == MT - 1) {
+                    bfc[0] = bfn[0];
+                    bfc[1] = bfn[1];
+                }
+            }
+
+            // The next stage's activations must have landed before anyone reads them.  Vector memory
+            // operations complete in order: the only ones issued after them in this stage are the two
+            // weight fetches above, which may stay in flight.
+            if (c < 3 || next_sb)
+                asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+    }
+
+    // ---- store: value v of a lane is row 8*(v/4) + 4*(lane/32) + v%4, column lane%32 (the weight row this
+    // lane dequantised); undo the activation-row and weight-row scales ----
+    const float* rs = reinterpret_cast<const float*>(a.ws + W.rs);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const uint32_t gmb = m0 + wm * (32 * MT) + mt * 32 + 4 * lg;
+        float rsv[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            uint32_t gm = gmb + 8 * (v >> 2) + (v & 3);
+            gm = gm < a.m ? gm : a.m - 1u;
+            rsv[v] = rs[gm];
+        }
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            const uint32_t gcol = n0 + wn * 64 + nt * 32 + l32;
+            const float wup = __uint_as_float(0x7f000000u - __float_as_uint(wdown[nt]));  // 2^e from 2^-e
+            if (gcol < a.n) {
+                float* yp = a.y + (size_t)gmb * a.n + gcol;
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (gmb + 8 * (v >> 2) + (v & 3) < a.m)
+                        yp[(size_t)(8 * (v >> 2) + (v & 3)) * a.n] = acc[mt][nt][v] * (rsv[v] * wup);
+            }
+        }
+    }
+}
+
+}  // namespace
+
+size_t gemm_q4k_workspace_bytes(uint32_t m, uint32_t k) { return workspace_layout(m, k).total; }
+
+int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
+                    uint32_t k, void* workspace) {
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    if (xdt == HQ_BF16)
+        hipLaunchKernelGGL(q4k_prep_kernel<true>, dim3(m), dim3(256), 0, s, x, ws, m, k);
+    else
+        hipLaunchKernelGGL(q4k_prep_kernel<false>, dim3(m), dim3(256), 0, s, x, ws, m, k);
+    if (int rc = check_launch("q4k gemm pre-pass launch")) return rc;
+    GemmArgs a{ws, static_cast<const uint8_t*>(w), y, m, n, k};
+    constexpr int lds = 2 * BM * ROW * 2;
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_gemm_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(q4k gemm LDS)"))
+        return rc;
+    const uint32_t tiles_n = (n + BN - 1) / BN, tiles_m = (m + BM - 1) / BM;
+    hipLaunchKernelGGL(q4k_gemm_kernel, dim3(8u * ((tiles_m + 7u) / 8u) * tiles_n), dim3(128 * WN), lds, s, a);
+    return check_launch("q4k gemm kernel launch");
+}
+
+}  // namespace hq

@@ -44,6 +44,11 @@ int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type
 bool gemm_supported(hq_ggml_type t, uint32_t k);
 int launch_gemm(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                 uint32_t k, hq_ggml_type t);
+// Q4_K GEMM on the f16 matrix cores with an activation pre-pass; needs k % 256 == 0 and a device
+// workspace of gemm_q4k_workspace_bytes().
+size_t gemm_q4k_workspace_bytes(uint32_t m, uint32_t k);
+int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
+                    uint32_t k, void* workspace);
 
 // MoE glue (moe.hip)
 int launch_dense_gemv_bf16(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,

@@ -68,13 +68,26 @@ class GgmlQuantizedMatmulIdParams:
 
 
 def quantized_matmul_ggml(input: torch.Tensor, weight: torch.Tensor, dst: torch.Tensor,
-                          params: GgmlQuantizedMatmulParams) -> None:
-    """dst[m,n] = input[m,k] . W[n,k]^T, W = raw GGML blocks (uint8 tensor)."""
+                          params: GgmlQuantizedMatmulParams, workspace: torch.Tensor | None = None) -> None:
+    """dst[m,n] = input[m,k] . W[n,k]^T, W = raw GGML blocks (uint8 tensor).  With `workspace`
+    (a uint8 device tensor of quantized_matmul_workspace_bytes()) the call allocates nothing."""
     if dst.dtype != torch.float32:
         raise TypeError("dst must be float32")
     L = _l.load()
+    if workspace is not None:
+        _l.check(L.hq_qmatmul_ggml_ws(_stream(), _dev(input, "input"), _act_dtype(input), _dev(weight, "weight"),
+                                      _dev(dst, "dst"), params.m, params.n, params.k, params.ggml_type,
+                                      _dev(workspace, "workspace"), workspace.numel() * workspace.element_size()))
+        return
     _l.check(L.hq_qmatmul_ggml(_stream(), _dev(input, "input"), _act_dtype(input), _dev(weight, "weight"),
                                _dev(dst, "dst"), params.m, params.n, params.k, params.ggml_type))
+
+
+def quantized_matmul_workspace_bytes(params: GgmlQuantizedMatmulParams, act_dtype: torch.dtype) -> int:
+    """Device scratch quantized_matmul_ggml(..., workspace=) needs for this shape (0 for most)."""
+    L = _l.load()
+    xdt = _l.HQ_BF16 if act_dtype == torch.bfloat16 else _l.HQ_F32
+    return int(L.hq_qmatmul_ggml_workspace_bytes(params.m, params.n, params.k, xdt, params.ggml_type))
 
 
 def quantized_matmul_id_ggml(input: torch.Tensor, weight_stack: torch.Tensor, ids: torch.Tensor,

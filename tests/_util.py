@@ -30,6 +30,37 @@ def assert_matmul_close(got, ref64, what=""):
     return float(err.max() / rms) if rms > 0 else 0.0
 
 
+# The Q4_K tile GEMM (m > 8) rounds every dequantised weight once to f16 (2^-12 relative), as the
+# reference's mul_mm kernels do with their half-precision weight tile; bf16 activations stay exact,
+# f32 activations are rounded to f16 as well.  Its gate is the one the scope table states for matmul
+# outputs, max|err| / max|ref| <= 1e-3 with cosine >= 0.9999, plus an element-wise bound of
+# 1e-3 |ref| + 3e-3 rms (observed: rms error 2-3e-4 of the output rms, worst element 1.5e-3 rms).
+F16_TILE_ABS = 3e-3
+
+
+def assert_matmul_close_f16_tile(got, ref64, what=""):
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref64, dtype=np.float64).reshape(-1)
+    assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    if not ref.size:
+        return 0.0
+    rms = float(np.sqrt(np.mean(ref * ref)))
+    err = np.abs(got - ref)
+    peak = float(np.abs(ref).max())
+    if peak == 0.0:
+        assert not got.any(), f"{what}: reference is zero, output is not"
+        return 0.0
+    assert err.max() <= REL_TOL * peak, f"{what}: max|err| {err.max():.4g} > 1e-3 max|ref| {peak:.4g}"
+    bound = REL_TOL * np.abs(ref) + F16_TILE_ABS * rms
+    bad = err > bound
+    assert not bad.any(), f"{what}: {int(bad.sum())}/{ref.size} outside 1e-3 |ref| + 3e-3 rms (rms {rms:.4g})"
+    assert float(np.sqrt(np.mean(err * err))) <= 5e-4 * rms, f"{what}: rms error above 5e-4 of the output rms"
+    cos = float(got @ ref / (np.linalg.norm(got) * np.linalg.norm(ref)))
+    assert cos >= 0.9999, f"{what}: cosine {cos}"
+    return float(err.max() / rms)
+
+
 def weights(seed, n, k, sigma=0.02):
     """Seeded N(0, sigma) f32 weight [n, k] (the benchmark's weight distribution)."""
     return (np.random.default_rng(seed).standard_normal((n, k), dtype=np.float32) * np.float32(sigma))
