@@ -279,7 +279,10 @@ int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, c
         !is_aligned(tmp, 4))
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: q / out / codes need 16-byte alignment", fn);
     if (p->head_dim == 512) return fail(HQ_ERR_UNSUPPORTED, "%s: head_dim 512 is not built", fn);
-    if (p->codebook_bits != 8) return fail(HQ_ERR_UNSUPPORTED, "%s: only the 8-bit cache is built", fn);
+    // 5- and 6-bit caches store one code per byte like the 8-bit one and differ only in the centroid
+    // table, which the caller supplies (its first 2^bits entries); the linear int8 map is 8-bit only.
+    if (p->codebook_bits != 8 && !lut256)
+        return fail(HQ_ERR_UNSUPPORTED, "%s: a %u-bit cache needs its centroid table (lut256)", fn, p->codebook_bits);
     if (tmp_bytes < tq_attn_tmp_bytes(p->num_heads, p->head_dim, p->kv_seq_len))
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: tmp holds %zu bytes, %zu needed", fn, tmp_bytes,
                     tq_attn_tmp_bytes(p->num_heads, p->head_dim, p->kv_seq_len));

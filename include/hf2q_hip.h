@@ -183,7 +183,7 @@ typedef struct {
     float softcap;           /* 0 = off, else s <- softcap * tanh(s / softcap) */
     uint32_t ring_start;     /* logical position i lives in slot (ring_start + i) % kv_capacity */
     float scale_factor_d512;
-    uint32_t codebook_bits;  /* 5, 6 or 8 are valid values; this build implements 8 */
+    uint32_t codebook_bits;  /* 5, 6 or 8; 5 and 6 need the centroid table (lut256) */
     uint32_t fuse_fwht_pre;  /* 1: q arrives un-rotated and is rotated inside the kernel */
     uint32_t nsg;            /* accepted for layout compatibility; the split count is chosen here */
 } hq_tq_attn_params;
@@ -195,7 +195,8 @@ typedef struct {
  * k_norms, v_packed, v_norms, out, tmp, &params) (forward_mlx.rs:4732-4742; kv_cache.rs:373-386).
  * `tmp` is device scratch of hq_flash_attn_vec_tq_tmp_bytes() bytes.  Rejects kv_seq_len == 0,
  * kv_capacity < kv_seq_len (kv_cache.rs:331-333), head_dim not in {256, 512}, codebook_bits not in
- * {5, 6, 8}; head_dim 512 and codebook_bits 5 / 6 are reported as unsupported. */
+ * {5, 6, 8}; head_dim 512, and codebook_bits 5 / 6 without a centroid table, are reported as
+ * unsupported. */
 HQ_API int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
                          const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
                          void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p);

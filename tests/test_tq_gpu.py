@@ -115,6 +115,23 @@ def test_attention_lut_form(oracle, dev):
     _assert_attn_close(_attend(dev, q, kc, kn, vc, vn, p, lut), ref, "lut form")
 
 
+@pytest.mark.parametrize("bits", [5, 6])
+def test_attention_small_codebooks(oracle, dev, bits):
+    """5- and 6-bit caches: one code per byte below 2^bits, values from the caller's centroid table."""
+    hd, nh, nkv, n, cap = 256, 8, 2, 150, 160
+    rng = np.random.default_rng(80 + bits)
+    kc = rng.integers(0, 1 << bits, (nkv, cap, hd), dtype=np.uint8)
+    vc = rng.integers(0, 1 << bits, (nkv, cap, hd), dtype=np.uint8)
+    kn = rng.uniform(5, 20, (nkv, cap, 1)).astype(np.float32)
+    vn = rng.uniform(5, 20, (nkv, cap, 1)).astype(np.float32)
+    lut = np.zeros(256, np.float32)
+    lut[: 1 << bits] = np.sort(rng.standard_normal(1 << bits)).astype(np.float32) * 2
+    q = rng.standard_normal((nh, hd)).astype(np.float32)
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 1.0 / 16.0, codebook_bits=bits)
+    ref = oracle.tq_attention(q, kc, kn, vc, vn, lut, nh, nkv, hd, n, cap, p.scale)
+    _assert_attn_close(_attend(dev, q, kc, kn, vc, vn, p, lut), ref, f"{bits}-bit codebook")
+
+
 def test_fused_pre_rotation_equals_separate_dispatch(oracle, dev):
     hd, nh, nkv, n, cap = 256, 16, 2, 300, 512
     rng = np.random.default_rng(12)
