@@ -201,7 +201,8 @@ def bench_moe_decode(a):
         "unit": "tok/s", "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "bf16",
         "config": {"workload": f"moe_decode: hidden 2048, 256 experts x inter 512 Q4_K, shared expert, top-8, "
                                f"batch {T}, bf16 activations (BASELINE config 3); one step = one MoE FFN layer "
-                               f"(router, top-k, 3 mul_mat_id, shared expert, reduce = 12 launches), "
+                               f"(router + shared logit, top-k, gate/up of routed and shared experts, both SwiGLU-fused "
+                               f"down projections, reduce = 5 launches), "
                                f"{'launched from the host' if a.no_graph else 'replayed as a HIP graph'}",
                    "distinct_experts_per_layer": round(u, 1), "bytes_per_layer": int(step_bytes),
                    "layers_rotated": n_layers},

@@ -220,6 +220,57 @@ int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void
     return HQ_OK;
 }
 
+int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_jobs, hq_act_dtype xdt,
+                          hq_ggml_type t) {
+    const char* fn = "hq_qmatmul_batch_ggml";
+    if (n_jobs == 0) return HQ_OK;
+    if (!jobs) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null jobs", fn);
+    if (n_jobs > HQ_QMATMUL_BATCH_MAX_JOBS)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: %u jobs (limit %d)", fn, n_jobs, HQ_QMATMUL_BATCH_MAX_JOBS);
+    GemvArgs ga[HQ_QMATMUL_BATCH_MAX_JOBS];
+    uint32_t live = 0;
+    for (uint32_t i = 0; i < n_jobs; ++i) {
+        const hq_qmatmul_job& j = jobs[i];
+        if (int rc = check_matmul_common(fn, j.x, xdt, j.w, j.y, j.n, j.k, t)) return rc;
+        if (j.x_up) {
+            if (xdt != HQ_F32) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: x_up needs f32 activations", fn, i);
+            if (!is_aligned(j.x_up, 16)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: x_up must be 16-byte aligned", fn, i);
+        }
+        GemvArgs a{};
+        a.x = j.x;
+        a.x2 = j.x_up;
+        a.w = static_cast<const uint8_t*>(j.w);
+        a.y = j.y;
+        a.n = j.n;
+        a.k = j.k;
+        if (j.ids) {
+            if (j.n_experts == 0 || j.top_k == 0)
+                return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: n_experts %u, top_k %u", fn, i, j.n_experts, j.top_k);
+            const uint64_t expert_bytes = (uint64_t)j.n * (j.k / hq_block_elems(t)) * hq_block_bytes(t);
+            if (j.expert_stride < expert_bytes || j.expert_stride % (t == HQ_Q4_K ? 16 : 2))
+                return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: expert_stride %llu (one expert is %llu bytes)", fn, i,
+                            (unsigned long long)j.expert_stride, (unsigned long long)expert_bytes);
+            const uint64_t pairs = (uint64_t)j.rows * j.top_k;
+            if (pairs > 65535) return fail(HQ_ERR_UNSUPPORTED, "%s: job %u: %llu routed rows (limit 65535)", fn, i, (unsigned long long)pairs);
+            a.ids = j.ids;
+            a.pairs = (uint32_t)pairs;
+            a.top_k = j.top_k;
+            a.n_experts = j.n_experts;
+            a.expert_stride = j.expert_stride;
+        } else {
+            // the dense form is the decode route only: more rows belong to the tile kernels
+            if (j.rows > kGemvMaxRows)
+                return fail(HQ_ERR_UNSUPPORTED, "%s: job %u: %u dense rows (limit %u; use hq_qmatmul_ggml)", fn, i, j.rows, kGemvMaxRows);
+            a.pairs = j.rows;
+            a.top_k = 1;
+            a.n_experts = 1;
+        }
+        if (a.pairs == 0) continue;
+        ga[live++] = a;
+    }
+    return launch_gemv_jobs((hipStream_t)stream, ga, live, xdt, t);
+}
+
 static int check_fwht(const char* fn, const float* buf, uint32_t n_heads, uint32_t head_dim) {
     if (head_dim != 256 && head_dim != 512) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: head_dim %u (256 or 512)", fn, head_dim);
     if (n_heads && !buf) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
@@ -300,6 +351,19 @@ int hq_dense_gemv_bf16(void* stream, const void* x, hq_act_dtype xdt, const void
         return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dense_gemv_bf16: x and w must be 16-byte aligned");
     if (m > 65535) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dense_gemv_bf16: m %u too large", m);
     return launch_dense_gemv_bf16((hipStream_t)stream, x, xdt, w_bf16, y, m, n, k);
+}
+
+int hq_dense_gemv_bf16_pair(void* stream, const void* x, hq_act_dtype xdt, const void* w_a, float* y_a, uint32_t n_a,
+                            const void* w_b, float* y_b, uint32_t n_b, uint32_t m, uint32_t k) {
+    const char* fn = "hq_dense_gemv_bf16_pair";
+    if (xdt != HQ_F32 && xdt != HQ_BF16) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: activation dtype %d", fn, (int)xdt);
+    if (k == 0 || k % 8) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: k %u is not a multiple of 8", fn, k);
+    if (m == 0 || (n_a == 0 && n_b == 0)) return HQ_OK;
+    if (!x || (n_a && (!w_a || !y_a)) || (n_b && (!w_b || !y_b))) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (!is_aligned(x, 16) || !is_aligned(w_a, 16) || !is_aligned(w_b, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: x and both weight matrices must be 16-byte aligned", fn);
+    if (m > 65535) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: m %u too large", fn, m);
+    return launch_dense_gemv_bf16_pair((hipStream_t)stream, x, xdt, w_a, y_a, n_a, w_b, y_b, n_b, m, k);
 }
 
 int hq_moe_softmax_topk(void* stream, const float* logits, uint32_t* ids, float* weights, uint32_t n_tokens,

@@ -254,8 +254,47 @@ __device__ __forceinline__ void stage_store(const XRaw<X_BF16>& raw, uint32_t i,
     lds_s[i] = s;
 }
 
+// SwiGLU staging: activations silu(gate) * up (silu_mul_f32, the arithmetic of the
+// stand-alone SwiGLU kernel) written to LDS as f32 with their per-16 sums.  The
+// exponentials are the expensive part, so every thread takes four activations, not
+// sixteen, and the sum of a run of sixteen is chained through the four lanes of a
+// quad in the order a single thread would add them.
+struct SwigluRaw {
+    uint4 g, u;
+    __device__ __forceinline__ void fetch(const uint8_t* grow, const uint8_t* urow, uint32_t i) {
+        g = reinterpret_cast<const uint4*>(grow)[i];
+        u = reinterpret_cast<const uint4*>(urow)[i];
+    }
+};
+
+__device__ __forceinline__ float swiglu1(uint32_t g, uint32_t u) {
+    return silu_mul_f32(__uint_as_float(g), __uint_as_float(u));
+}
+
+// Value of `v` in the previous lane of the quad (lane 0 of a quad receives its own).
+__device__ __forceinline__ float quad_prev(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x90 /* quad_perm [0,0,1,2] */, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ void stage_swiglu(const SwigluRaw& raw, uint32_t i, uint32_t* lds_x, float* lds_s) {
+#pragma clang fp contract(off)  // the sums add the rounded products, as a kernel reading them from memory would
+    const float v0 = swiglu1(raw.g.x, raw.u.x), v1 = swiglu1(raw.g.y, raw.u.y);
+    const float v2 = swiglu1(raw.g.z, raw.u.z), v3 = swiglu1(raw.g.w, raw.u.w);
+    reinterpret_cast<float4*>(lds_x)[i] = make_float4(v0, v1, v2, v3);
+    const uint32_t q = threadIdx.x & 3u;
+    // lane q of the quad continues the running sum of lanes 0..q-1
+    float s = 0.f;
+#pragma unroll
+    for (uint32_t step = 0; step < 4; ++step) {
+        const float carry = quad_prev(s);
+        if (q == step) s = (((step ? carry : 0.f) + v0) + v1) + v2 + v3;
+    }
+    if (q == 3) lds_s[i >> 2] = s;
+}
+
 struct KArgs {
     const void* x;
+    const void* x2;  // f32 only, may be null: the activations are silu(x) * x2
     const uint8_t* w;
     const uint32_t* ids;
     float* y;
@@ -263,6 +302,7 @@ struct KArgs {
     uint64_t expert_stride;
     uint32_t log_l;   // log2 of the lanes that share one row
     uint32_t groups;  // row groups (one group = the rows a workgroup covers in one pass)
+    uint32_t pairs;   // activation-row / output-row pairs (grid.y of the job)
     // Bit masks of the nibble -> bf16 conversion.  They are passed as arguments and
     // not written as literals so that the compiler keeps them in registers and
     // forms the three-operand v_and_or_b32 (gfx9 VOP3 takes no literals; with
@@ -443,16 +483,25 @@ struct Walk {
 // of weight fetches they would hold the workgroup at its barrier), then the
 // first weight fetches go out so that their latency overlaps the staging.
 template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
-__global__ __launch_bounds__(256) void gemv_kernel(KArgs a) {
+__device__ __forceinline__ void gemv_body(const KArgs& a, uint32_t bx, uint32_t p) {
     extern __shared__ uint4 smem[];
     uint32_t* lds_x = reinterpret_cast<uint32_t*>(smem);
     float* lds_s = reinterpret_cast<float*>(lds_x + (PAIR ? a.k / 2 : a.k));
 
-    const uint32_t p = blockIdx.y;
-    const uint8_t* xrow = static_cast<const uint8_t*>(a.x) + (size_t)(p / a.top_k) * a.k * (X_BF16 ? 2 : 4);
+    const size_t xoff = (size_t)(p / a.top_k) * a.k * (X_BF16 ? 2 : 4);
+    const uint8_t* xrow = static_cast<const uint8_t*>(a.x) + xoff;
     const uint32_t xchunks = a.k / 16;
+    bool swiglu = false;
+    if constexpr (!X_BF16) swiglu = a.x2 != nullptr;
+    [[maybe_unused]] const uint8_t* urow = nullptr;
     XRaw<X_BF16> xraw;
-    if (threadIdx.x < xchunks) xraw.fetch(xrow, threadIdx.x);
+    [[maybe_unused]] SwigluRaw sraw;
+    if (!swiglu) {
+        if (threadIdx.x < xchunks) xraw.fetch(xrow, threadIdx.x);
+    } else if constexpr (!X_BF16) {
+        urow = static_cast<const uint8_t*>(a.x2) + xoff;
+        if (threadIdx.x < a.k / 4) sraw.fetch(xrow, urow, threadIdx.x);
+    }
 
     const uint8_t* w = a.w;
     bool valid = true;
@@ -464,18 +513,47 @@ __global__ __launch_bounds__(256) void gemv_kernel(KArgs a) {
 
     Walk<TYPE, X_BF16, PAIR, NR, D> wk;
     wk.init(a, w, lds_x, lds_s);
-    const uint32_t rowbase = (blockIdx.x * 4u + (threadIdx.x >> 6)) * wk.rpw * NR;
+    const uint32_t rowbase = (bx * 4u + (threadIdx.x >> 6)) * wk.rpw * NR;
     wk.prime(rowbase);
 
-    if (threadIdx.x < xchunks) stage_store<X_BF16, PAIR>(xraw, threadIdx.x, lds_x, lds_s);
-    for (uint32_t i = threadIdx.x + 256u; i < xchunks; i += 256u) {
-        xraw.fetch(xrow, i);
-        stage_store<X_BF16, PAIR>(xraw, i, lds_x, lds_s);
+    if (!swiglu) {
+        if (threadIdx.x < xchunks) stage_store<X_BF16, PAIR>(xraw, threadIdx.x, lds_x, lds_s);
+        for (uint32_t i = threadIdx.x + 256u; i < xchunks; i += 256u) {
+            xraw.fetch(xrow, i);
+            stage_store<X_BF16, PAIR>(xraw, i, lds_x, lds_s);
+        }
+    } else if constexpr (!X_BF16) {
+        // k is a multiple of 16, so the four lanes of a quad enter and leave together
+        if (threadIdx.x < a.k / 4) stage_swiglu(sraw, threadIdx.x, lds_x, lds_s);
+        for (uint32_t i = threadIdx.x + 256u; i < a.k / 4; i += 256u) {
+            sraw.fetch(xrow, urow, i);
+            stage_swiglu(sraw, i, lds_x, lds_s);
+        }
     }
     wk.load_masks(a);
     __syncthreads();
 
     wk.group(rowbase, 0u, false, a.y + (size_t)p * a.n, valid);
+}
+
+template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
+__global__ __launch_bounds__(256) void gemv_kernel(KArgs a) {
+    gemv_body<TYPE, X_BF16, PAIR, NR, D>(a, blockIdx.x, blockIdx.y);
+}
+
+// Several independent GEMVs in one launch: blockIdx.z selects the job, the grid
+// spans the largest job and the workgroups outside a smaller one leave at once.
+constexpr uint32_t MAX_JOBS = 4;
+struct KJobs {
+    KArgs j[MAX_JOBS];
+};
+
+template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
+__global__ __launch_bounds__(256) void gemv_jobs_kernel(KJobs js) {
+    const KArgs& a = js.j[blockIdx.z];
+    const uint32_t rows_per_wg = 4u * (64u >> a.log_l) * NR;
+    if (blockIdx.y >= a.pairs || blockIdx.x * rows_per_wg >= a.n) return;
+    gemv_body<TYPE, X_BF16, PAIR, NR, D>(a, blockIdx.x, blockIdx.y);
 }
 
 // Dense GEMV for matrices with many wave groups per CU: one workgroup of WAVES
@@ -586,26 +664,40 @@ int launch_q(hipStream_t s, KArgs ka, uint32_t cus, uint32_t rpw, size_t lds) {
     return check_launch("gemv queue kernel launch");
 }
 
+// Lanes per row, LDS bytes and slot count of one job.
 template <int TYPE, bool X_BF16>
-int launch_t(hipStream_t s, const GemvArgs& a) {
+int plan_job(const GemvArgs& a, KArgs* ka, size_t* lds, uint64_t* slots) {
     constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
     constexpr int EPL = Lane<TYPE>::kElems;
-    KArgs ka{a.x, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, M4, M2, MAGIC};
+    if (a.x2 && X_BF16) return fail(HQ_ERR_UNSUPPORTED, "gemv: the fused SwiGLU form takes f32 activations");
+    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, M4, M2, MAGIC};
     const uint32_t pieces = a.k / EPL;
     // L = largest power of two <= 64 that divides the pieces of a row
     uint32_t log_l = 0;
     while (log_l < 6 && pieces % (2u << log_l) == 0) ++log_l;
-    ka.log_l = log_l;
+    ka->log_l = log_l;
     const uint32_t rpw = 64u >> log_l;
     // activations, their per-16 sums, the queue counter
-    const size_t lds = (size_t)(PAIR ? a.k * 2 : a.k * 4) + (size_t)(a.k / 16) * 4 + 16;
-    if (lds > 160 * 1024 - 512)
-        return fail(HQ_ERR_UNSUPPORTED, "gemv: k = %u needs %zu bytes of LDS (limit 160 KiB)", a.k, lds);
+    *lds = (size_t)(PAIR ? a.k * 2 : a.k * 4) + (size_t)(a.k / 16) * 4 + 16;
+    if (*lds > 160 * 1024 - 512)
+        return fail(HQ_ERR_UNSUPPORTED, "gemv: k = %u needs %zu bytes of LDS (limit 160 KiB)", a.k, *lds);
+    *slots = (uint64_t)((a.n + rpw - 1) / rpw) * a.pairs;
+    return HQ_OK;
+}
+
+template <int TYPE, bool X_BF16>
+int launch_t(hipStream_t s, const GemvArgs& a) {
+    constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
+    constexpr int EPL = Lane<TYPE>::kElems;
+    KArgs ka;
+    size_t lds;
+    uint64_t slots;
+    if (int rc = plan_job<TYPE, X_BF16>(a, &ka, &lds, &slots)) return rc;
+    const uint32_t log_l = ka.log_l, rpw = 64u >> log_l;
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
-    const uint64_t slots = (uint64_t)((a.n + rpw - 1) / rpw) * a.pairs;
     // Dense matrices with many tasks per wave: the queue kernel.
-    if (a.pairs == 1 && slots * ((a.k / EPL) >> log_l) >= (uint64_t)cus * QUEUE_MIN_TASKS_PER_CU)
+    if (a.pairs == 1 && !a.x2 && slots * ((a.k / EPL) >> log_l) >= (uint64_t)cus * QUEUE_MIN_TASKS_PER_CU)
         return launch_q<TYPE, X_BF16, PAIR, 2, 2, 12>(s, ka, cus, rpw, lds);
     // Slots one SIMD would get if the work were spread evenly; more slots per wave
     // amortise the per-wave set-up, fewer keep every SIMD busy on small problems.
@@ -613,6 +705,42 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     if (per_simd >= 8) return launch_r<TYPE, X_BF16, PAIR, 4, 4>(s, ka, a.pairs, rpw, lds);
     if (per_simd >= 2) return launch_r<TYPE, X_BF16, PAIR, 2, 2>(s, ka, a.pairs, rpw, lds);
     return launch_r<TYPE, X_BF16, PAIR, 1, 1>(s, ka, a.pairs, rpw, lds);
+}
+
+template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
+int launch_j(hipStream_t s, const KJobs& js, uint32_t n_jobs, size_t lds) {
+    auto kern = gemv_jobs_kernel<TYPE, X_BF16, PAIR, NR, D>;
+    if (int rc = set_lds_limit(kern, lds, "hipFuncSetAttribute(gemv jobs LDS)")) return rc;
+    uint32_t gx = 0, gy = 0;
+    for (uint32_t i = 0; i < n_jobs; ++i) {
+        const uint32_t rows_per_wg = 4u * (64u >> js.j[i].log_l) * NR;
+        const uint32_t bx = (js.j[i].n + rows_per_wg - 1) / rows_per_wg;
+        gx = bx > gx ? bx : gx;
+        gy = js.j[i].pairs > gy ? js.j[i].pairs : gy;
+    }
+    hipLaunchKernelGGL(kern, dim3(gx, gy, n_jobs), dim3(256), lds, s, js);
+    return check_launch("gemv jobs kernel launch");
+}
+
+template <int TYPE, bool X_BF16>
+int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
+    constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
+    KJobs js{};
+    size_t lds = 0;
+    uint64_t slots = 0;
+    for (uint32_t i = 0; i < n_jobs; ++i) {
+        size_t l;
+        uint64_t sl;
+        if (int rc = plan_job<TYPE, X_BF16>(jobs[i], &js.j[i], &l, &sl)) return rc;
+        lds = l > lds ? l : lds;
+        slots += sl;
+    }
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
+    const uint64_t per_simd = slots / (4ull * cus);
+    if (per_simd >= 8) return launch_j<TYPE, X_BF16, PAIR, 4, 4>(s, js, n_jobs, lds);
+    if (per_simd >= 2) return launch_j<TYPE, X_BF16, PAIR, 2, 2>(s, js, n_jobs, lds);
+    return launch_j<TYPE, X_BF16, PAIR, 1, 1>(s, js, n_jobs, lds);
 }
 
 }  // namespace
@@ -623,6 +751,19 @@ int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type
         case HQ_Q4_K: return bf ? launch_t<HQ_Q4_K, true>(s, a) : launch_t<HQ_Q4_K, false>(s, a);
         case HQ_Q6_K: return bf ? launch_t<HQ_Q6_K, true>(s, a) : launch_t<HQ_Q6_K, false>(s, a);
         case HQ_Q8_0: return bf ? launch_t<HQ_Q8_0, true>(s, a) : launch_t<HQ_Q8_0, false>(s, a);
+    }
+    return fail(HQ_ERR_UNSUPPORTED, "gemv: ggml type %d", (int)t);
+}
+
+int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_act_dtype xdt, hq_ggml_type t) {
+    if (n_jobs == 0) return HQ_OK;
+    if (n_jobs == 1) return launch_gemv(s, jobs[0], xdt, t);
+    if (n_jobs > MAX_JOBS) return fail(HQ_ERR_INVALID_ARGUMENT, "gemv: %u jobs in one launch (limit %u)", n_jobs, MAX_JOBS);
+    const bool bf = xdt == HQ_BF16;
+    switch (t) {
+        case HQ_Q4_K: return bf ? launch_jobs_t<HQ_Q4_K, true>(s, jobs, n_jobs) : launch_jobs_t<HQ_Q4_K, false>(s, jobs, n_jobs);
+        case HQ_Q6_K: return bf ? launch_jobs_t<HQ_Q6_K, true>(s, jobs, n_jobs) : launch_jobs_t<HQ_Q6_K, false>(s, jobs, n_jobs);
+        case HQ_Q8_0: return bf ? launch_jobs_t<HQ_Q8_0, true>(s, jobs, n_jobs) : launch_jobs_t<HQ_Q8_0, false>(s, jobs, n_jobs);
     }
     return fail(HQ_ERR_UNSUPPORTED, "gemv: ggml type %d", (int)t);
 }

@@ -29,6 +29,7 @@ int launch_quantize(hipStream_t s, const float* src, uint64_t n_elems, uint64_t 
 
 struct GemvArgs {
     const void* x;        // [x_rows, k] activations
+    const void* x2;       // nullptr, or f32 [x_rows, k]: the activations are silu(x) * x2
     const uint8_t* w;     // weight blocks, or the expert stack when ids != nullptr
     const uint32_t* ids;  // [pairs] expert ids, or nullptr for the dense form
     float* y;             // [pairs, n]
@@ -39,6 +40,8 @@ struct GemvArgs {
     uint64_t expert_stride;  // bytes
 };
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t);
+// Up to four independent GEMVs of one weight type and activation dtype in a single launch.
+int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_act_dtype xdt, hq_ggml_type t);
 
 // MFMA GEMM for m > 8 (prefill).  gemm_supported() says whether (type, k) has a tile kernel.
 bool gemm_supported(hq_ggml_type t, uint32_t k);
@@ -53,6 +56,8 @@ int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* 
 // MoE glue (moe.hip)
 int launch_dense_gemv_bf16(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
                            uint32_t n, uint32_t k);
+int launch_dense_gemv_bf16_pair(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_a, float* y_a, uint32_t n_a,
+                                const void* w_b, float* y_b, uint32_t n_b, uint32_t m, uint32_t k);
 int launch_moe_softmax_topk(hipStream_t s, const float* logits, uint32_t* ids, float* weights, uint32_t n_tokens,
                             uint32_t n_experts, uint32_t top_k);
 int launch_silu_mul(hipStream_t s, const float* gate, const float* up, float* out, uint64_t n);
@@ -83,6 +88,16 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
 }
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// silu(g) * u = g / (1 + exp(-g)) * u (ffn.rs:24-26).  Every step is a rounded operation of its own
+// (no contraction into an fma), so that the stand-alone SwiGLU kernel and the down projection that
+// forms its activations on the fly produce the same bits.
+__device__ __forceinline__ float silu_mul_f32(float g, float u) {
+#pragma clang fp contract(off)
+    const float e = expf(-g);
+    const float d = 1.f + e;
+    return g / d * u;
+}
 // f32 -> bf16 bits, round to nearest even (NaN kept quiet).
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     uint32_t u = __float_as_uint(f);

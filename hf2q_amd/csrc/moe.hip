@@ -25,12 +25,21 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // y[m, n] = x[m, k] . W[n, k]^T, W bf16 row-major, x f32 or bf16, fp32 accumulate.
-// One wave per output row; grid (ceil(n/4), m).
+// One wave per output row; grid (ceil((n_a + n_b)/4), m).  Two matrices over the same
+// activations share the launch: rows below n_a belong to the first, the rest to the second.
 template <bool X_BF16>
-__global__ __launch_bounds__(256) void dense_gemv_bf16_kernel(const void* __restrict__ x, const uint16_t* __restrict__ w,
-                                                              float* __restrict__ y, uint32_t n, uint32_t k) {
-    const uint32_t lane = threadIdx.x & 63u, row = blockIdx.x * 4 + (threadIdx.x >> 6), m = blockIdx.y;
-    if (row >= n) return;
+__global__ __launch_bounds__(256) void dense_gemv_bf16_kernel(const void* __restrict__ x, const uint16_t* __restrict__ w_a,
+                                                              float* __restrict__ y_a, uint32_t n_a,
+                                                              const uint16_t* __restrict__ w_b, float* __restrict__ y_b,
+                                                              uint32_t n_b, uint32_t k) {
+    const uint32_t lane = threadIdx.x & 63u, m = blockIdx.y;
+    uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_a + n_b) return;
+    const bool second = row >= n_a;
+    if (second) row -= n_a;
+    const uint16_t* w = second ? w_b : w_a;
+    float* y = second ? y_b : y_a;
+    const uint32_t n = second ? n_b : n_a;
     const uint4* wr = reinterpret_cast<const uint4*>(w + (size_t)row * k);
     float acc = 0.f;
     for (uint32_t c = lane; c < k / 8; c += 64) {  // 8 weights per step
@@ -149,10 +158,10 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
     if (i >= n4) return;
     const float4 g = reinterpret_cast<const float4*>(gate)[i], u = reinterpret_cast<const float4*>(up)[i];
     float4 o;
-    o.x = g.x / (1.f + expf(-g.x)) * u.x;  // ffn.rs:24-26 silu(x) = x / (1 + exp(-x))
-    o.y = g.y / (1.f + expf(-g.y)) * u.y;
-    o.z = g.z / (1.f + expf(-g.z)) * u.z;
-    o.w = g.w / (1.f + expf(-g.w)) * u.w;
+    o.x = silu_mul_f32(g.x, u.x);
+    o.y = silu_mul_f32(g.y, u.y);
+    o.z = silu_mul_f32(g.z, u.z);
+    o.w = silu_mul_f32(g.w, u.w);
     reinterpret_cast<float4*>(out)[i] = o;
 }
 
@@ -193,14 +202,21 @@ __global__ __launch_bounds__(256) void moe_weighted_reduce_kernel(const float* _
 
 }  // namespace
 
+int launch_dense_gemv_bf16_pair(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_a, float* y_a, uint32_t n_a,
+                                const void* w_b, float* y_b, uint32_t n_b, uint32_t m, uint32_t k) {
+    const dim3 grid((n_a + n_b + 3) / 4, m);
+    const uint16_t* wa = static_cast<const uint16_t*>(w_a);
+    const uint16_t* wb = static_cast<const uint16_t*>(w_b);
+    if (xdt == HQ_BF16)
+        hipLaunchKernelGGL(dense_gemv_bf16_kernel<true>, grid, dim3(256), 0, s, x, wa, y_a, n_a, wb, y_b, n_b, k);
+    else
+        hipLaunchKernelGGL(dense_gemv_bf16_kernel<false>, grid, dim3(256), 0, s, x, wa, y_a, n_a, wb, y_b, n_b, k);
+    return check_launch("dense bf16 gemv launch");
+}
+
 int launch_dense_gemv_bf16(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
                            uint32_t n, uint32_t k) {
-    const dim3 grid((n + 3) / 4, m);
-    if (xdt == HQ_BF16)
-        hipLaunchKernelGGL(dense_gemv_bf16_kernel<true>, grid, dim3(256), 0, s, x, static_cast<const uint16_t*>(w), y, n, k);
-    else
-        hipLaunchKernelGGL(dense_gemv_bf16_kernel<false>, grid, dim3(256), 0, s, x, static_cast<const uint16_t*>(w), y, n, k);
-    return check_launch("dense bf16 gemv launch");
+    return launch_dense_gemv_bf16_pair(s, x, xdt, w, y, n, nullptr, nullptr, 0, m, k);
 }
 
 int launch_moe_softmax_topk(hipStream_t s, const float* logits, uint32_t* ids, float* weights, uint32_t n_tokens,

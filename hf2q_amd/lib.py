@@ -27,6 +27,16 @@ class HqError(RuntimeError):
 _c = ctypes
 _vp, _u32, _u64, _i32, _sz, _f32 = _c.c_void_p, _c.c_uint32, _c.c_uint64, _c.c_int, _c.c_size_t, _c.c_float
 
+HQ_QMATMUL_BATCH_MAX_JOBS = 4
+
+
+class QmatmulJob(_c.Structure):
+    """hq_qmatmul_job of include/hf2q_hip.h, field for field."""
+    _fields_ = [("x", _c.c_void_p), ("x_up", _c.c_void_p), ("w", _c.c_void_p), ("ids", _c.c_void_p),
+                ("y", _c.c_void_p), ("rows", _c.c_uint32), ("top_k", _c.c_uint32), ("n", _c.c_uint32),
+                ("k", _c.c_uint32), ("n_experts", _c.c_uint32), ("expert_stride", _c.c_uint64)]
+
+
 # name -> (restype, argtypes); the single source for the symbol-export test.
 SIGNATURES = {
     "hq_last_error": (_c.c_char_p, []),
@@ -40,7 +50,9 @@ SIGNATURES = {
     "hq_qmatmul_ggml_ws": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32, _vp, _sz]),
     "hq_qmatmul_id_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _u32, _u32, _u32, _u32, _u32, _u64, _i32]),
     "hq_qmatmul_id_scratch_bytes": (_sz, [_u32, _u32]),
+    "hq_qmatmul_batch_ggml": (_i32, [_vp, _vp, _u32, _i32, _i32]),
     "hq_dense_gemv_bf16": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32]),
+    "hq_dense_gemv_bf16_pair": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _vp, _vp, _u32, _u32, _u32]),
     "hq_moe_softmax_topk": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "hq_silu_mul": (_i32, [_vp, _vp, _vp, _vp, _u64]),
     "hq_moe_weighted_reduce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),

@@ -107,6 +107,46 @@ def quantized_matmul_id_ggml(input: torch.Tensor, weight_stack: torch.Tensor, id
                                   params.expert_stride, params.ggml_type))
 
 
+@dataclass
+class QmatmulJob:
+    """One product of a batched launch: the arguments of quantized_matmul_id_ggml (ids set) or of
+    quantized_matmul_ggml (ids None, m <= 8).  With `input_up` the activations are
+    silu(input) * input_up, formed while they are staged."""
+    input: torch.Tensor
+    weight: torch.Tensor
+    output: torch.Tensor
+    rows: int
+    n: int
+    k: int
+    ids: torch.Tensor | None = None
+    top_k: int = 1
+    n_experts: int = 1
+    expert_stride: int = 0
+    input_up: torch.Tensor | None = None
+
+
+def quantized_matmul_batch_ggml(jobs: list[QmatmulJob], ggml_type: int) -> None:
+    """The dispatches of one phase of the MoE block, which the reference encodes without a barrier
+    between them (gpu_ffn.rs:2485, 2546), as a single launch."""
+    if not jobs:
+        return
+    arr = (_l.QmatmulJob * len(jobs))()
+    for c, j in zip(arr, jobs):
+        if j.output.dtype != torch.float32:
+            raise TypeError("output must be float32")
+        if _act_dtype(j.input) != _act_dtype(jobs[0].input):
+            raise TypeError("all jobs of a batch share one activation dtype")
+        if j.ids is not None and j.ids.dtype not in (torch.int32, torch.uint32):
+            raise TypeError("ids must be 32-bit")
+        if j.input_up is not None and j.input_up.dtype != torch.float32:
+            raise TypeError("input_up must be float32")
+        c.x, c.w, c.y = _dev(j.input, "input"), _dev(j.weight, "weight"), _dev(j.output, "output")
+        c.x_up = _dev(j.input_up, "input_up") if j.input_up is not None else None
+        c.ids = _dev(j.ids, "ids") if j.ids is not None else None
+        c.rows, c.top_k, c.n, c.k, c.n_experts, c.expert_stride = j.rows, j.top_k, j.n, j.k, j.n_experts, j.expert_stride
+    _l.check(_l.load().hq_qmatmul_batch_ggml(_stream(), arr, len(jobs), _act_dtype(jobs[0].input), ggml_type))
+
+
 def id_scratch_bytes(n_experts: int, max_rows: int) -> int:
     return _l.load().hq_qmatmul_id_scratch_bytes(n_experts, max_rows)
 
@@ -212,6 +252,14 @@ def dense_gemv_bf16_f32(x: torch.Tensor, w_bf16: torch.Tensor, y: torch.Tensor, 
     _l.check(_l.load().hq_dense_gemv_bf16(_stream(), _dev(x, "x"), _act_dtype(x), _dev(w_bf16, "w"), _dev(y, "y"), m, n, k))
 
 
+def dense_gemv_bf16_f32_pair(x: torch.Tensor, w_a: torch.Tensor, y_a: torch.Tensor, n_a: int, w_b: torch.Tensor,
+                             y_b: torch.Tensor, n_b: int, m: int, k: int) -> None:
+    """Two dense_gemv_bf16_f32 dispatches over the same activations (router + shared gate logit,
+    gpu_ffn.rs:2485) in one launch."""
+    _l.check(_l.load().hq_dense_gemv_bf16_pair(_stream(), _dev(x, "x"), _act_dtype(x), _dev(w_a, "w_a"), _dev(y_a, "y_a"),
+                                               n_a, _dev(w_b, "w_b"), _dev(y_b, "y_b"), n_b, m, k))
+
+
 def dispatch_moe_softmax_topk(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, n_tokens: int,
                               n_experts: int, top_k: int) -> None:
     _l.check(_l.load().hq_moe_softmax_topk(_stream(), _dev(logits, "logits"), _dev(ids, "ids"), _dev(weights, "weights"),
@@ -267,14 +315,43 @@ class MoeFfnScratch:
         self.sh_down = f(T, w.hidden)
 
 
+# Dense products above this many rows take the tile (GEMM) route, which the batched launch does not cover.
+_BATCH_MAX_DENSE_ROWS = 8
+
+
 def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch, out: torch.Tensor,
-                                   residual: torch.Tensor | None = None) -> None:
+                                   residual: torch.Tensor | None = None, batched: bool | None = None) -> None:
     """gpu_ffn.rs:2313-2802, phases A-F, enqueued on the current stream with no host round trip:
     router / shared projections -> softmax top-k + shared SwiGLU -> gate, up mul_mat_id + shared down ->
-    SwiGLU -> down mul_mat_id (n_tokens = T*K, top_k = 1) -> weighted reduce (+ sigmoid-gated shared, + residual)."""
+    SwiGLU -> down mul_mat_id (n_tokens = T*K, top_k = 1) -> weighted reduce (+ sigmoid-gated shared, + residual).
+
+    `batched` (default: whenever the token count allows) hands the dispatches that the reference encodes
+    without a barrier between them to the library as one launch each and folds both SwiGLU passes into the
+    staging of the down projections: five launches instead of twelve, same arithmetic, same results."""
     T = x.shape[0]
     K, H, E, I, SI, t = w.top_k, w.hidden, w.n_experts, w.inter, w.shared_inter, w.ggml_type
     rb = ggml_row_bytes(t, H)
+    if batched is None:
+        batched = T <= _BATCH_MAX_DENSE_ROWS
+    if batched:
+        if T > _BATCH_MAX_DENSE_ROWS:
+            raise ValueError(f"batched MoE block: {T} tokens (limit {_BATCH_MAX_DENSE_ROWS})")
+        dense_gemv_bf16_f32_pair(x, w.router, s.logits, E, w.shared_gate_logit, s.sh_logit, 1, T, H)
+        dispatch_moe_softmax_topk(s.logits, s.ids, s.topk_w, T, E, K)
+        quantized_matmul_batch_ggml([
+            QmatmulJob(x, w.expert_gate, s.gate, T, I, H, ids=s.ids, top_k=K, n_experts=E, expert_stride=I * rb),
+            QmatmulJob(x, w.expert_up, s.up, T, I, H, ids=s.ids, top_k=K, n_experts=E, expert_stride=I * rb),
+            QmatmulJob(x, w.shared_gate, s.sh_gate, T, SI, H),
+            QmatmulJob(x, w.shared_up, s.sh_up, T, SI, H),
+        ], t)
+        quantized_matmul_batch_ggml([
+            QmatmulJob(s.gate, w.expert_down, s.down, T * K, H, I, ids=s.ids, top_k=1, n_experts=E,
+                       expert_stride=H * ggml_row_bytes(t, I), input_up=s.up),
+            QmatmulJob(s.sh_gate, w.shared_down, s.sh_down, T, H, SI, input_up=s.sh_up),
+        ], t)
+        dispatch_moe_weighted_reduce(s.down, s.topk_w, out, T, K, H, shared=s.sh_down, shared_logit=s.sh_logit,
+                                     residual=residual)
+        return
     # A
     dense_gemv_bf16_f32(x, w.router, s.logits, T, E, H)
     dense_gemv_bf16_f32(x, w.shared_gate_logit, s.sh_logit, T, 1, H)

@@ -126,12 +126,44 @@ HQ_API int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, con
  * n_tokens*top_k routed rows (the IdMmScratch analogue, decode_pool.rs:56-60). */
 HQ_API size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows);
 
+/* Up to HQ_QMATMUL_BATCH_MAX_JOBS independent decode-sized products of one weight
+ * type and activation dtype in ONE launch.  The reference encodes the dispatches
+ * of a phase of the MoE block without a barrier between them, so the GPU runs
+ * them side by side (gpu_ffn.rs:2546 "Phase B ... (concurrent)", phases A and C
+ * likewise); an in-order HIP stream would serialise separate launches, so the
+ * phase is handed over as one batch instead.  A job is hq_qmatmul_id_ggml's
+ * argument list when `ids` is set (rows = n_tokens, rows*top_k <= 65535) and
+ * hq_qmatmul_ggml's when it is NULL (rows = m <= 8, the decode route).  With
+ * `x_up` set (f32 activations only) the job's activations are
+ * silu(x[i]) * x_up[i], computed while they are staged: the SwiGLU of phase D
+ * folded into the down projection (the quantized_matmul_id_swiglu_q4_0 variant
+ * that gpu_ffn.rs:2685-2697 describes), bit-identical to hq_silu_mul followed by
+ * the plain product. */
+#define HQ_QMATMUL_BATCH_MAX_JOBS 4
+typedef struct hq_qmatmul_job {
+    const void* x;        /* [rows, k] activations */
+    const void* x_up;     /* NULL, or f32 [rows, k] */
+    const void* w;        /* [n][k/QK] blocks, or the expert stack when ids != NULL */
+    const uint32_t* ids;  /* NULL (dense) or [rows*top_k] expert ids on the device */
+    float* y;             /* [rows, n] (dense) or [rows*top_k, n] */
+    uint32_t rows, top_k, n, k, n_experts;
+    uint64_t expert_stride; /* bytes between experts of the stack */
+} hq_qmatmul_job;
+HQ_API int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_jobs, hq_act_dtype xdt,
+                          hq_ggml_type t);
+
 /* ---- MoE block glue (run between the mul_mat_id calls; ffn.rs:179-336 is the specification) ---- */
 
 /* y[m,n] = x[m,k] . W[n,k]^T with W in bf16 (router / shared-expert gate projections).  Replaces
  * dense_gemv_bf16_f32 (src/inference/models/qwen35/gpu_ffn.rs:597-617).  k % 8 == 0. */
 HQ_API int hq_dense_gemv_bf16(void* stream, const void* x, hq_act_dtype xdt, const void* w_bf16, float* y,
                        uint32_t m, uint32_t n, uint32_t k);
+
+/* Two such products over the same activations in one launch: the router logits and the
+ * shared-expert gate logit of phase A (gpu_ffn.rs:2485, "all read from x, concurrent"), which the reference encodes
+ * back to back without a barrier.  y_a [m, n_a], y_b [m, n_b]. */
+HQ_API int hq_dense_gemv_bf16_pair(void* stream, const void* x, hq_act_dtype xdt, const void* w_a, float* y_a,
+                            uint32_t n_a, const void* w_b, float* y_b, uint32_t n_b, uint32_t m, uint32_t k);
 
 /* Per token: softmax over n_experts logits, the top_k most probable experts (ties: lower id), weights
  * renormalised over the selection.  Replaces dispatch_moe_softmax_topk (gpu_ffn.rs:2551-2573); same

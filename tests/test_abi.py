@@ -52,6 +52,19 @@ def test_argument_errors_are_reported_not_fatal():
     assert L.hq_qmatmul_ggml(None, None, lib.HQ_F32, fake, fake, 1, 8, 256, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
     # id form: expert stride smaller than an expert
     assert L.hq_qmatmul_id_ggml(None, fake, lib.HQ_F32, fake, fake, fake, None, 0, 1, 2, 8, 256, 4, 100, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    # batched form: too many jobs, a prefill-sized dense job, SwiGLU over bf16 activations
+    jobs = (lib.QmatmulJob * 5)()
+    for j in jobs:
+        j.x, j.w, j.y, j.rows, j.top_k, j.n, j.k, j.n_experts = 0x1000, 0x1000, 0x1000, 1, 1, 8, 256, 1
+    assert L.hq_qmatmul_batch_ggml(None, jobs, 5, lib.HQ_F32, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_qmatmul_batch_ggml(None, None, 2, lib.HQ_F32, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    jobs[1].rows = 9
+    assert L.hq_qmatmul_batch_ggml(None, jobs, 2, lib.HQ_F32, lib.HQ_Q4_K) == lib.HQ_ERR_UNSUPPORTED
+    jobs[1].rows, jobs[1].x_up = 1, 0x1000
+    assert L.hq_qmatmul_batch_ggml(None, jobs, 2, lib.HQ_BF16, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert "x_up" in lib.last_error()
+    assert L.hq_qmatmul_batch_ggml(None, jobs, 0, lib.HQ_F32, lib.HQ_Q4_K) == lib.HQ_OK
+    assert L.hq_dense_gemv_bf16_pair(None, fake, lib.HQ_F32, fake, fake, 4, fake, fake, 1, 1, 12) == lib.HQ_ERR_INVALID_ARGUMENT
     assert L.hq_quantize_ggml(None, fake, 512, 300, lib.HQ_Q4_K, fake) == lib.HQ_ERR_INVALID_ARGUMENT
     assert L.hq_quantize_ggml(None, fake, 768, 512, lib.HQ_Q4_K, fake) == lib.HQ_ERR_INVALID_ARGUMENT
     with pytest.raises(lib.HqError):

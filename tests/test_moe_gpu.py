@@ -3,9 +3,9 @@ import numpy as np
 import pytest
 import torch
 
-from _util import acts, weights
+from _util import acts, assert_matmul_close, weights
 from hf2q_amd import ops
-from hf2q_amd.ops import HQ_Q4_K, HQ_Q8_0
+from hf2q_amd.ops import HQ_Q4_K, HQ_Q6_K, HQ_Q8_0
 
 pytestmark = pytest.mark.gpu
 
@@ -106,3 +106,93 @@ def test_moe_block_matches_cpu_spec(oracle, dev, T, t):
     res = acts(9, T, H)
     ops.build_moe_ffn_layer_gpu_q_into(dv(x), w, s, out, residual=dv(res))
     assert np.abs(out.cpu().numpy() - (want + res)).max() <= 2e-4 * np.abs(want + res).max()
+
+
+def _moe_weights(oracle, dev, t, H, E, K, I, SI, seed=0):
+    rng = np.random.default_rng(300 + seed)
+    bf = lambda a: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(a))  # noqa: E731
+    router = bf((rng.standard_normal((E, H)) * 0.1).astype(np.float32))
+    sgl = bf((rng.standard_normal((1, H)) * 0.05).astype(np.float32))
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    q = {nm: dv(oracle.quantize(weights(sd + seed, n, k, 0.05), k, t, threads=8)) for nm, sd, n, k in
+         (("eg", 1, E * I, H), ("eu", 2, E * I, H), ("ed", 3, E * H, I), ("sg", 4, SI, H), ("su", 5, SI, H), ("sd", 6, H, SI))}
+    return ops.MoeFfnWeightsGpuQ(dv(router).to(torch.bfloat16), q["eg"], q["eu"], q["ed"], dv(sgl).to(torch.bfloat16),
+                                 q["sg"], q["su"], q["sd"], t, H, E, K, I, SI)
+
+
+@pytest.mark.parametrize("T", [1, 3, 8])
+@pytest.mark.parametrize("t,xdt", [(HQ_Q4_K, torch.float32), (HQ_Q4_K, torch.bfloat16), (HQ_Q6_K, torch.float32),
+                                   (HQ_Q8_0, torch.float32)])
+def test_moe_block_batched_launches_equal_separate_dispatches(oracle, dev, T, t, xdt):
+    """Five launches (batched phases, SwiGLU folded into the down projections) against the twelve
+    separate dispatches: the same kernels' arithmetic in the same order, so every bit must agree.
+    The routed and shared experts differ in width (inter 256 / shared 512), so the jobs of one
+    launch differ in n and in k."""
+    H, E, K, I, SI = 512, 16, 4, 256, 512
+    w = _moe_weights(oracle, dev, t, H, E, K, I, SI, seed=T)
+    x = torch.from_numpy(acts(11 + T, T, H)).to(dev).to(xdt)
+    res = torch.from_numpy(acts(12, T, H)).to(dev)
+    outs = []
+    for batched in (False, True):
+        s = ops.MoeFfnScratch(w, T, dev)
+        out = torch.full((T, H), float("nan"), device=dev)
+        ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out, residual=res, batched=batched)
+        outs.append((out.cpu(), s.gate.cpu(), s.up.cpu(), s.sh_gate.cpu(), s.sh_up.cpu(), s.down.cpu(), s.sh_down.cpu(),
+                     s.logits.cpu(), s.sh_logit.cpu(), s.ids.cpu()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert torch.isfinite(outs[1][0]).all()
+
+
+def test_batched_block_refuses_prefill_sized_token_counts(oracle, dev):
+    H, E, K, I, SI = 256, 4, 2, 256, 256
+    w = _moe_weights(oracle, dev, HQ_Q4_K, H, E, K, I, SI)
+    s = ops.MoeFfnScratch(w, 9, dev)
+    x, out = torch.zeros(9, H, device=dev), torch.empty(9, H, device=dev)
+    with pytest.raises(ValueError):
+        ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out, batched=True)
+    ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out)  # default falls back to separate dispatches
+    assert torch.equal(out.cpu(), torch.zeros(9, H))
+
+
+def test_qmatmul_batch_swiglu_against_cpu_spec(oracle, dev):
+    """down(silu(gate) * up) of one launch against the float64 product over the dequantised weights."""
+    rows, n, k, t = 5, 96, 768, HQ_Q4_K
+    wq = oracle.quantize(weights(21, n, k, 0.05), k, t, threads=8)
+    wd = oracle.dequantize(wq, t).reshape(n, k).astype(np.float64)
+    g, u = acts(22, rows, k), acts(23, rows, k)
+    act = (g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64)))) * u
+    y = torch.full((rows, n), float("nan"), device=dev)
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    ops.quantized_matmul_batch_ggml([ops.QmatmulJob(dv(g), dv(wq), y, rows, n, k, input_up=dv(u))], t)
+    assert_matmul_close(y.cpu().numpy(), act @ wd.T, "swiglu-fused dense job")
+
+
+def test_qmatmul_batch_argument_errors(dev):
+    z = lambda *s, dt=torch.float32: torch.zeros(*s, dtype=dt, device=dev)  # noqa: E731
+    w = z(144 * 8, dt=torch.uint8)
+    job = ops.QmatmulJob(z(1, 256), w, z(1, 8), 1, 8, 256)
+    with pytest.raises(ops.HqError):  # more jobs than one launch takes
+        ops.quantized_matmul_batch_ggml([job] * 5, HQ_Q4_K)
+    with pytest.raises(ops.HqError):  # dense jobs are decode-sized
+        ops.quantized_matmul_batch_ggml([ops.QmatmulJob(z(9, 256), w, z(9, 8), 9, 8, 256), job], HQ_Q4_K)
+    with pytest.raises(ops.HqError):  # the folded SwiGLU reads f32 activations
+        ops.quantized_matmul_batch_ggml([ops.QmatmulJob(z(1, 256, dt=torch.bfloat16), w, z(1, 8), 1, 8, 256,
+                                                        input_up=z(1, 256))], HQ_Q4_K)
+    with pytest.raises(ops.HqError):  # expert stride smaller than one expert
+        ops.quantized_matmul_batch_ggml([ops.QmatmulJob(z(1, 256), w, z(2, 8), 1, 8, 256, ids=z(2, dt=torch.int32),
+                                                        top_k=2, n_experts=1, expert_stride=100), job], HQ_Q4_K)
+    ops.quantized_matmul_batch_ggml([], HQ_Q4_K)
+
+
+def test_dense_gemv_bf16_pair_equals_two_calls(dev):
+    m, na, nb, k = 3, 37, 1, 1024
+    g = torch.Generator(device="cpu").manual_seed(5)
+    x = torch.randn(m, k, generator=g).to(dev)
+    wa = (torch.randn(na, k, generator=g) * 0.05).to(dev).to(torch.bfloat16)
+    wb = (torch.randn(nb, k, generator=g) * 0.05).to(dev).to(torch.bfloat16)
+    ya, yb, ya2, yb2 = (torch.empty(m, n, device=dev) for n in (na, nb, na, nb))
+    ops.dense_gemv_bf16_f32(x, wa, ya, m, na, k)
+    ops.dense_gemv_bf16_f32(x, wb, yb, m, nb, k)
+    ops.dense_gemv_bf16_f32_pair(x, wa, ya2, na, wb, yb2, nb, m, k)
+    assert torch.equal(ya.cpu(), ya2.cpu()) and torch.equal(yb.cpu(), yb2.cpu())
