@@ -5,6 +5,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "hq_internal.h"
 
 namespace hq {
@@ -35,6 +37,29 @@ static int check_weight_alignment(const void* w, hq_ggml_type t) {
     if (!is_aligned(w, need))
         return fail(HQ_ERR_INVALID_ARGUMENT, "weight pointer must be %zu-byte aligned for ggml type %d",
                     need, (int)t);
+    return HQ_OK;
+}
+
+// The device's CU count, cached per device.
+int cu_count(uint32_t* out) {
+    static std::mutex mu;
+    static int cached[64] = {};
+    int dev = 0;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    std::lock_guard<std::mutex> lock(mu);
+    if (dev < 0 || dev >= 64 || cached[dev] == 0) {
+        int cus = 0;
+        if (int rc = check_hip(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev),
+                               "hipDeviceGetAttribute(CU count)"))
+            return rc;
+        if (cus <= 0) cus = 256;
+        if (dev < 0 || dev >= 64) {
+            *out = (uint32_t)cus;
+            return HQ_OK;
+        }
+        cached[dev] = cus;
+    }
+    *out = (uint32_t)cached[dev];
     return HQ_OK;
 }
 
@@ -137,7 +162,7 @@ int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const vo
 size_t hq_qmatmul_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
     (void)n;
     (void)xdt;
-    return q4k_tile_route(m, k, t) ? gemm_q4k_workspace_bytes(m, k) : 0;
+    return q4k_tile_route(m, k, t) ? gemm_q4k_workspace_bytes(m, n, k) : 0;
 }
 
 int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,

@@ -17,23 +17,31 @@
 // exact weights to about 1.5e-4 of the output's scale (rms), where the kernels
 // that keep every product exact reach 1e-6.
 //
-// Structure.  Workgroup = 256 threads = 2x2 waves, tile 256 (tokens) x 128
-// (weight rows) x 64 (k) per stage; a wave owns 128x64 = 4x2 MFMA tiles (128
-// accumulator registers).
+// Structure.  Workgroup = 256 threads = 4 waves side by side along the weight
+// rows, tile 256 (tokens) x 128 (weight rows) x 64 (k) per stage; a wave owns
+// all 256 tokens x 32 weight rows = 8x1 MFMA tiles (128 accumulator
+// registers).  Two workgroups fit a CU.  The SIMD issues MFMA and VALU
+// instructions through one port and an MFMA hides only about four VALU
+// instructions behind it, so the kernel is bound by instructions per MFMA, not
+// by latency: with tall wave tiles every weight is dequantised by exactly one
+// wave of the workgroup (a 2x2 wave grid does it twice, 7.4 instead of 3.7
+// VALU instructions per MFMA) at the price of twice the LDS reads, which the
+// LDS (64 banks, 256 bytes per clock) has room for.  Problems of less than half
+// a round of workgroups use tiles of 64 weight rows (2x2 waves of 128x32) to
+// spread over more CUs.
 //   * Activations: the pre-pass output goes global -> LDS directly
 //     (global_load_lds_dwordx4, no registers, no VALU), double buffered, one
 //     barrier per stage.  A wave instruction fills 1 KB of LDS with lane i at
 //     byte 16*i, so tile rows are 128 bytes without padding and the 16-byte
-//     chunks of a row are XOR-swizzled with the row number: lane i fetches the
-//     global chunk (i%8) ^ (i/8) of its row, and the 16-byte fragment reads are
-//     conflict free.
+//     chunks of a row are XOR-swizzled with the row number.  LDS has 64 banks
+//     and serves a 16-byte read of 16 lanes per cycle, so the 16 rows that 16
+//     consecutive lanes read must land in 16 different 16-byte slots of 256
+//     bytes: the key is (row / 2) % 8 (rows of equal parity share a half).
 //   * Weights never touch LDS: a lane fetches the 16 nibble bytes it needs for
 //     its own fragments (row lane%32, bytes 16*(lane/32).. of the 64-element
 //     chunk) straight from global memory, a stage ahead, and dequantises them
-//     in registers.  LDS bandwidth is the scarce resource of this tile shape (a
-//     32x32x16 MFMA consumes 2 KB of fragments per 32 cycles); keeping one
-//     operand out of it is what lets the matrix cores run.  The two waves that
-//     share weight rows dequantise them twice.
+//     in registers: no LDS traffic, no extra barrier, and each wave produces
+//     exactly the fragments it consumes.
 //   * k order.  Inside a stage the MFMA contraction index is a permutation of k
 //     chosen so that a lane's fragments come from its own 16 nibble bytes: lane
 //     group g of k-step s covers k = 16g + 8s + j (s < 2, low nibbles) or
@@ -51,15 +59,16 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 constexpr int BK = 64;
 constexpr int ROW = BK;  // f16 elements per LDS tile row (128 bytes, chunks XOR-swizzled)
 
-// workspace: [xh m*k f16][rs m f32]
+// workspace: [xh m*k f16][rs m f32][wdown n f32]
 struct Workspace {
-    size_t xh, rs, total;
+    size_t xh, rs, wdown, total;
 };
-__host__ __device__ inline Workspace workspace_layout(uint32_t m, uint32_t k) {
+__host__ __device__ inline Workspace workspace_layout(uint32_t m, uint32_t n, uint32_t k) {
     Workspace w;
     w.xh = 0;
     w.rs = ((size_t)m * k * 2 + 255) & ~(size_t)255;
-    w.total = w.rs + (((size_t)m * 4 + 255) & ~(size_t)255);
+    w.wdown = w.rs + (((size_t)m * 4 + 255) & ~(size_t)255);
+    w.total = w.wdown + (((size_t)n * 4 + 255) & ~(size_t)255);
     return w;
 }
 
@@ -73,13 +82,38 @@ __device__ __forceinline__ uint32_t f16_bits(float v) {
     return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)v);
 }
 
-// Pre-pass, one workgroup per activation row: row scale and f16 conversion.
+// Pre-pass.  Workgroups [0, m): one per activation row, row scale and f16 conversion.  Workgroups
+// from m on: 16 weight rows each, 16 lanes per row over the row's super-block headers.  Per weight
+// row, a power of two that brings the row's largest possible |w| = |d|*63*15 + |dmin|*63 to about
+// 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
+// subnormals; the main kernel multiplies the weights by it before they are rounded (exact) and its
+// epilogue divides it out.
 template <bool X_BF16>
-__global__ __launch_bounds__(256) void q4k_prep_kernel(const void* __restrict__ x, uint8_t* __restrict__ ws,
-                                                       uint32_t m, uint32_t k) {
+__global__ __launch_bounds__(256) void q4k_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
+                                                       uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k) {
     __shared__ float red[4];
-    const uint32_t row = blockIdx.x, tid = threadIdx.x;
-    const Workspace L = workspace_layout(m, k);
+    const uint32_t tid = threadIdx.x;
+    const Workspace L = workspace_layout(m, n, k);
+    if (blockIdx.x >= m) {
+        const uint32_t wr = (blockIdx.x - m) * 16u + (tid >> 4), nsb = k / 256;
+        const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nsb * Q4K_BYTES;
+        float bound = 0.f;
+        for (uint32_t sb = tid & 15u; sb < nsb; sb += 16u) {
+            const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow + (size_t)sb * Q4K_BYTES);
+            const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * 945.f + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
+            bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;  // inf / nan scales do not set the exponent
+        }
+        bound = dpp_max<0xB1>(bound);  // the four steps cover a row of 16 lanes
+        bound = dpp_max<0x4E>(bound);
+        bound = dpp_max<0x141>(bound);
+        bound = dpp_max<0x140>(bound);
+        int ex = 0;
+        if (bound > 0.f) (void)frexpf(bound, &ex);  // bound = f * 2^ex, f in [0.5, 1)
+        const int e = bound > 0.f ? ex - 14 : 0;
+        if ((tid & 15u) == 0 && wr < n) reinterpret_cast<float*>(ws + L.wdown)[wr] = ldexpf(1.f, -e);  // |e| <= 40: normal
+        return;
+    }
+    const uint32_t row = blockIdx.x;
     const uint32_t chunks = k / 8;
 
     auto load8 = [&](uint32_t i, float* v) {
@@ -163,44 +197,35 @@ __device__ __forceinline__ void weights4(uint32_t nib4, float dsc, float ndm, ui
     hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(b, f16x2_t));
 }
 
-constexpr int WN = 2;              // waves along the weight rows (and 2 along the tokens)
-constexpr int MT = 4;              // 32-row MFMA tiles per wave along the tokens
-constexpr int BM = 64 * MT;        // token rows per workgroup
-constexpr int BN = 64 * WN;        // weight rows per workgroup
-constexpr int DMA_PER_WAVE = (BM / 8) / (2 * WN);  // BM / 8 one-KB fetches fill the activation tile
+constexpr int WAVES = 4;           // one per SIMD; two workgroups share a CU
+constexpr int BM = 256;            // token rows per workgroup
+constexpr int DMA_PER_WAVE = (BM / 8) / WAVES;  // BM / 8 one-KB fetches fill the activation tile
+constexpr int BN_WIDE = 128, BN_NARROW = 64;    // weight rows per workgroup
 
-__global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
+// One workgroup tile: rows m0.. of the activations, weight rows n0...  The four waves form a
+// (4 / WN) x WN grid; a wave owns MT x NT MFMA tiles of 32 x 32.
+template <int MT, int NT, int WN>
+__device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
+    static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
     extern __shared__ uint4 smem4[];
     uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
     constexpr int kTile = BM * ROW * 2;  // one activation tile, padded; two of them in LDS
-    const Workspace W = workspace_layout(a.m, a.k);
+    const Workspace W = workspace_layout(a.m, a.n, a.k);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
 
-    // Tile order: workgroups go to the 8 XCDs round-robin and every XCD has its own L2, so workgroup
-    // i runs on XCD i % 8.  Each XCD gets whole rows of tiles (one activation tile, which then stays
-    // in that XCD's L2) and sweeps the weight tiles.
-    const uint32_t tiles_n = (a.n + BN - 1) / BN, tiles_m = (a.m + BM - 1) / BM;
-    uint32_t m0, n0;
-    {
-        const uint32_t xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3;
-        const uint32_t rows_here = (tiles_m + 7u - xcd) / 8u;
-        if (idx >= rows_here * tiles_n) return;  // the grid is padded to 8 * ceil(tiles_m / 8) * tiles_n
-        m0 = (xcd + 8u * (idx / tiles_n)) * BM;
-        n0 = (idx % tiles_n) * BN;
-    }
     const uint32_t nsb = a.k / 256, nstages = a.k / BK;
     const uint32_t row_bytes = nsb * Q4K_BYTES;
 
     // ---- activation staging: wave w, instruction i (< DMA_PER_WAVE) fills 8 LDS rows of the tile,
     // (w * DMA_PER_WAVE + i) * 8 .. +8; lane L owns row L/8 of them and LDS chunk L%8, which holds
-    // global chunk (L%8) ^ (L/8) ----
+    // global chunk (L%8) ^ ((row/2)%8), and (row/2)%8 = L/16 + 4*(i%2) ----
     // byte offset of this lane's source chunk from the tile's first row, stage 0: the wave's first row + L/8
     // for i = 0, 8 rows further per instruction; rows past the end of x read the last row instead (their
     // results are never stored)
-    const uint32_t a_swz = ((lane & 7u) ^ (lane >> 3)) << 4;
+    const uint32_t a_swz = ((lane & 7u) ^ (lane >> 4)) << 4;
     const uint32_t a_row0 = wave * (8u * DMA_PER_WAVE) + (lane >> 3);
     const uint32_t a_rows_left = a.m - m0;  // >= 1
     const uint32_t a_last = (a_rows_left - 1u) * (a.k * 2u) + a_swz;
@@ -216,7 +241,7 @@ __global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
 #pragma unroll
         for (int i = 0; i < DMA_PER_WAVE; ++i) {
             const uint32_t r = a_row0 + 8u * i;
-            const uint8_t* src = xtile + (r < a_rows_left ? r * (a.k * 2u) + a_swz : a_last) + (size_t)st * (BK * 2);
+            const uint8_t* src = xtile + (r < a_rows_left ? r * (a.k * 2u) + (a_swz ^ ((i & 1u) << 6)) : a_last ^ ((i & 1u) << 6)) + (size_t)st * (BK * 2);
             const uint32_t dst = lds_base + buf * kTile + (wave_u * DMA_PER_WAVE + i) * 1024u;
             asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
             __builtin_amdgcn_sched_barrier(0);  // one address at a time: keeps eight 64-bit pointers out of the registers
@@ -224,48 +249,32 @@ __global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
     };
 
     // ---- weights: this lane's two rows (one per 32-row tile of the wave), bytes 16*lg.. of each chunk ----
-    const uint8_t* wrow[2];
+    const uint8_t* wrow[NT];
+    float wdown[NT];  // power-of-two scale 2^-e of the lane's rows, from the pre-pass
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-        uint32_t gn = n0 + wn * 64 + nt * 32 + l32;
+    for (int nt = 0; nt < NT; ++nt) {
+        uint32_t gn = n0 + wn * (32 * NT) + nt * 32 + l32;
         gn = gn < a.n ? gn : a.n - 1u;
         wrow[nt] = a.w + (size_t)gn * row_bytes;
+        wdown[nt] = reinterpret_cast<const float*>(a.ws + W.wdown)[gn];
     }
-    // Per weight row, a power of two that brings the row's largest possible |w| = |d|*63*15 + |dmin|*63
-    // to about 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
-    // subnormals; the weights are multiplied by it before they are rounded (exact) and the epilogue
-    // divides it out.  Both waves that share a row compute the same value.
-    float wdown[2];  // 2^-e of this lane's two rows
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-        float bound = 0.f;
-        for (uint32_t sb = 0; sb < nsb; ++sb) {
-            const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow[nt] + (size_t)sb * Q4K_BYTES);
-            const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * 945.f + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
-            bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;  // inf / nan scales do not set the exponent
-        }
-        int ex = 0;
-        if (bound > 0.f) (void)frexpf(bound, &ex);  // bound = f * 2^ex, f in [0.5, 1)
-        const int e = bound > 0.f ? ex - 14 : 0;
-        wdown[nt] = ldexpf(1.f, -e);  // |e| <= 40: a normal number
-    }
-    uint4 braw[2][2];       // [stage parity][nt]
-    uint4 hdr[2], hdrn[2];  // super-block headers: current, next
+    uint4 braw[2][NT];        // [stage parity][nt]
+    uint4 hdr[NT], hdrn[NT];  // super-block headers: current, next
     auto load_b = [&](uint32_t sblk, int c, int slot) {
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < NT; ++nt)
             braw[slot][nt] = ld16(wrow[nt] + (size_t)sblk * Q4K_BYTES + 16 + 32 * c + 16 * lg);
     };
     auto load_hdr = [&](uint32_t sblk, uint4* h) {
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) h[nt] = ld16(wrow[nt] + (size_t)sblk * Q4K_BYTES);
+        for (int nt = 0; nt < NT; ++nt) h[nt] = ld16(wrow[nt] + (size_t)sblk * Q4K_BYTES);
     };
 
-    f32x16_t acc[MT][2];
+    f32x16_t acc[MT][NT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NT; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
@@ -286,11 +295,15 @@ __global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
             // This stage's nibbles, requested a stage ago.  They are claimed here, before the activation
             // fetch below is issued: the compiler does not know about that fetch, and the wait it puts
             // in front of the first use of these registers would otherwise cover it too.
-            uint4 b0 = braw[c & 1][0], b1 = braw[c & 1][1];
-            asm volatile("" : "+v"(b0.x), "+v"(b0.y), "+v"(b0.z), "+v"(b0.w), "+v"(b1.x), "+v"(b1.y), "+v"(b1.z), "+v"(b1.w));
+            uint4 bcur[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                bcur[nt] = braw[c & 1][nt];
+                asm volatile("" : "+v"(bcur[nt].x), "+v"(bcur[nt].y), "+v"(bcur[nt].z), "+v"(bcur[nt].w));
+            }
             if (c == 0 && sblk > 0) {  // this super-block's header; request the next one (before the
-                hdr[0] = hdrn[0];      // activation fetch, so that it is older than it)
-                hdr[1] = hdrn[1];
+#pragma unroll                         // activation fetch, so that it is older than it)
+                for (int nt = 0; nt < NT; ++nt) hdr[nt] = hdrn[nt];
                 if (next_sb) load_hdr(sblk + 1, hdrn);
             }
             // next stage's activations into the other buffer (free since the barrier that ended the
@@ -298,9 +311,9 @@ __global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
             if (st + 1 < nstages) load_a(st + 1, buf ^ 1u);
 
             // this stage's weight scales: sub-blocks 2c (low nibbles) and 2c+1 (high nibbles)
-            float dsc[2][2], ndm[2][2];  // [nt][low / high]
+            float dsc[NT][2], ndm[NT][2];  // [nt][low / high]
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) {
+            for (int nt = 0; nt < NT; ++nt) {
                 uint32_t sc0, sc1, mn0, mn1;
                 q4k_scales(hdr[nt].y, hdr[nt].z, hdr[nt].w, c, sc0, sc1, mn0, mn1);
                 const float d = f16_bits_to_f32(hdr[nt].x & 0xffffu) * wdown[nt];
@@ -326,12 +339,12 @@ __global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
                 // chunk index of this lane group's 8 activations inside the row's 64
                 const uint32_t kchunk = ks < 2 ? 2u * lg + ks : 4u + 2u * lg + (ks - 2);
                 const uint32_t row = wm * (32 * MT) + mt * 32 + l32;
-                return *reinterpret_cast<const uint4*>(smem + buf * kTile + row * (ROW * 2) + ((kchunk ^ (row & 7u)) << 4));
+                return *reinterpret_cast<const uint4*>(smem + buf * kTile + row * (ROW * 2) + ((kchunk ^ ((row >> 1) & 7u)) << 4));
             };
             // quarter q (nt = q/2, word pair half = q%2) of k-step ks: four weights -> words 2*(q%2), +1
             auto b_quarter = [&](int ks, int q, uint4* bfw) {
                 const int nt = q >> 1, half = q & 1;
-                const uint4 b = nt == 0 ? b0 : b1;
+                const uint4 b = bcur[nt];
                 const uint32_t w = (ks & 1) ? (half ? b.w : b.z) : (half ? b.y : b.x);
                 const int hi = ks >> 1;  // 0: low nibbles, 1: high nibbles
                 uint32_t lo2, hi2;
@@ -341,33 +354,31 @@ __global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
                 else
                     bfw[nt].z = lo2, bfw[nt].w = hi2;
             };
-            uint4 bfc[2], bfn[2];
+            uint4 bfc[NT], bfn[NT];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) b_quarter(0, q, bfc);
+            for (int q = 0; q < 2 * NT; ++q) b_quarter(0, q, bfc);
             uint4 af0 = a_frag(0), af1;
 #pragma unroll
             for (int t = 0; t < 4 * MT; ++t) {
                 const int ks = t / MT, mt = t % MT;
                 if (t + 1 < 4 * MT) af1 = a_frag(t + 1);
                 acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(af0), as_frag(bfc[0]), acc[mt][0], 0, 0, 0);
-                if (ks + 1 < 4) {
-#pragma unroll
-                    for (int q = 0; q < 4 / MT; ++q) b_quarter(ks + 1, mt * (4 / MT) + q, bfn);
-                }
-                acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(af0), as_frag(bfc[1]), acc[mt][1], 0, 0, 0);
+                if (ks + 1 < 4 && mt < 2 * NT) b_quarter(ks + 1, mt, bfn);  // 2*NT quarters over the first of the MT steps
+                if constexpr (NT == 2)
+                    acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(af0), as_frag(bfc[1]), acc[mt][1], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 af0 = af1;
                 if (mt == MT - 1) {
-                    bfc[0] = bfn[0];
-                    bfc[1] = bfn[1];
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) bfc[nt] = bfn[nt];
                 }
             }
 
             // The next stage's activations must have landed before anyone reads them.  Vector memory
-            // operations complete in order: the only ones issued after them in this stage are the two
+            // operations complete in order: the only ones issued after them in this stage are the NT
             // weight fetches above, which may stay in flight.
             if (c < 3 || next_sb)
-                asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+                asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NT) : "memory");
             else
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
@@ -388,8 +399,8 @@ __global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
             rsv[v] = rs[gm];
         }
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-            const uint32_t gcol = n0 + wn * 64 + nt * 32 + l32;
+        for (int nt = 0; nt < NT; ++nt) {
+            const uint32_t gcol = n0 + wn * (32 * NT) + nt * 32 + l32;
             const float wup = __uint_as_float(0x7f000000u - __float_as_uint(wdown[nt]));  // 2^e from 2^-e
             if (gcol < a.n) {
                 float* yp = a.y + (size_t)gmb * a.n + gcol;
@@ -402,17 +413,44 @@ __global__ __launch_bounds__(128 * WN, 2) void q4k_gemm_kernel(GemmArgs a) {
     }
 }
 
+// Tile order: workgroups go to the 8 XCDs round-robin and every XCD has its own L2, so workgroup i
+// runs on XCD i % 8.  Each XCD gets whole rows of tiles (one activation tile, which then stays in
+// that XCD's L2) and sweeps the weight tiles.  The grid is padded to 8 * ceil(tiles_m / 8) * tiles_n.
+__device__ __forceinline__ bool tile_of(uint32_t b, uint32_t tiles_m, uint32_t tiles_n, uint32_t bn, uint32_t& m0, uint32_t& n0) {
+    const uint32_t xcd = b & 7u, idx = b >> 3;
+    const uint32_t rows_here = (tiles_m + 7u - xcd) / 8u;
+    if (idx >= rows_here * tiles_n) return false;
+    m0 = (xcd + 8u * (idx / tiles_n)) * BM;
+    n0 = (idx % tiles_n) * bn;
+    return true;
+}
+
+// Weight rows [0, n_wide) in tiles of 128 (the first grid_wide workgroups), the rest in tiles of 64.
+__global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_kernel(GemmArgs a, uint32_t n_wide, uint32_t grid_wide) {
+    const uint32_t tiles_m = (a.m + BM - 1) / BM;
+    uint32_t m0, n0;
+    if (blockIdx.x < grid_wide) {
+        if (!tile_of(blockIdx.x, tiles_m, n_wide / BN_WIDE, BN_WIDE, m0, n0)) return;
+        q4k_gemm_tile<8, 1, 4>(a, m0, n0);
+    } else {
+        if (!tile_of(blockIdx.x - grid_wide, tiles_m, (a.n - n_wide + BN_NARROW - 1) / BN_NARROW, BN_NARROW, m0, n0)) return;
+        q4k_gemm_tile<4, 1, 2>(a, m0, n_wide + n0);
+    }
+}
+
 }  // namespace
 
-size_t gemm_q4k_workspace_bytes(uint32_t m, uint32_t k) { return workspace_layout(m, k).total; }
+size_t gemm_q4k_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) { return workspace_layout(m, n, k).total; }
 
 int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                     uint32_t k, void* workspace) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const uint8_t* wb = static_cast<const uint8_t*>(w);
+    const dim3 prep_grid(m + (n + 15u) / 16u);
     if (xdt == HQ_BF16)
-        hipLaunchKernelGGL(q4k_prep_kernel<true>, dim3(m), dim3(256), 0, s, x, ws, m, k);
+        hipLaunchKernelGGL(q4k_prep_kernel<true>, prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k);
     else
-        hipLaunchKernelGGL(q4k_prep_kernel<false>, dim3(m), dim3(256), 0, s, x, ws, m, k);
+        hipLaunchKernelGGL(q4k_prep_kernel<false>, prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k);
     if (int rc = check_launch("q4k gemm pre-pass launch")) return rc;
     GemmArgs a{ws, static_cast<const uint8_t*>(w), y, m, n, k};
     constexpr int lds = 2 * BM * ROW * 2;
@@ -420,8 +458,18 @@ int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* 
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                            "hipFuncSetAttribute(q4k gemm LDS)"))
         return rc;
-    const uint32_t tiles_n = (n + BN - 1) / BN, tiles_m = (m + BM - 1) / BM;
-    hipLaunchKernelGGL(q4k_gemm_kernel, dim3(8u * ((tiles_m + 7u) / 8u) * tiles_n), dim3(128 * WN), lds, s, a);
+    // Tiles of 128 weight rows; tiles of 64 when the wide ones would occupy at most half of the CUs.
+    // (Cutting only the last, partly filled round of a large problem into narrow tiles was measured:
+    // no gain, the narrow tiles pay the double dequantisation.)
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
+    const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
+    const uint32_t cols_narrowed = (uint64_t)tiles_m * cols_wide <= cus / 2 ? cols_wide : 0;  // columns cut in two
+    const uint32_t n_wide = (cols_wide - cols_narrowed) * BN_WIDE;  // < n whenever cols_narrowed > 0
+    const uint32_t cols_narrow = n_wide < n ? (n - n_wide + BN_NARROW - 1) / BN_NARROW : 0;
+    const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
+    const uint32_t grid_wide = pad_m * (cols_wide - cols_narrowed), grid_narrow = pad_m * cols_narrow;
+    hipLaunchKernelGGL(q4k_gemm_kernel, dim3(grid_wide + grid_narrow), dim3(64 * WAVES), lds, s, a, n_wide, grid_wide);
     return check_launch("q4k gemm kernel launch");
 }
 

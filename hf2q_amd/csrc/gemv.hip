@@ -613,29 +613,6 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_queue_kernel(KArgs a) {
     }
 }
 
-// The device's CU count, cached per device.
-int cu_count(uint32_t* out) {
-    static std::mutex mu;
-    static int cached[64] = {};
-    int dev = 0;
-    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
-    std::lock_guard<std::mutex> lock(mu);
-    if (dev < 0 || dev >= 64 || cached[dev] == 0) {
-        int cus = 0;
-        if (int rc = check_hip(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev),
-                               "hipDeviceGetAttribute(CU count)"))
-            return rc;
-        if (cus <= 0) cus = 256;
-        if (dev < 0 || dev >= 64) {
-            *out = (uint32_t)cus;
-            return HQ_OK;
-        }
-        cached[dev] = cus;
-    }
-    *out = (uint32_t)cached[dev];
-    return HQ_OK;
-}
-
 template <typename K>
 int set_lds_limit(K kern, size_t lds, const char* what) {
     if (lds <= 64 * 1024) return HQ_OK;

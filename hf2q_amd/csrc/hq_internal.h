@@ -39,6 +39,8 @@ struct GemvArgs {
     uint32_t n_experts;
     uint64_t expert_stride;  // bytes
 };
+// The current device's CU count (cached).
+int cu_count(uint32_t* out);
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t);
 // Up to four independent GEMVs of one weight type and activation dtype in a single launch.
 int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_act_dtype xdt, hq_ggml_type t);
@@ -49,7 +51,7 @@ int launch_gemm(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, f
                 uint32_t k, hq_ggml_type t);
 // Q4_K GEMM on the f16 matrix cores with an activation pre-pass; needs k % 256 == 0 and a device
 // workspace of gemm_q4k_workspace_bytes().
-size_t gemm_q4k_workspace_bytes(uint32_t m, uint32_t k);
+size_t gemm_q4k_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
 int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                     uint32_t k, void* workspace);
 
