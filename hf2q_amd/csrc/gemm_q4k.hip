@@ -185,18 +185,6 @@ typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 
 __device__ __forceinline__ uint4 ld16(const uint8_t* p) { return *reinterpret_cast<const uint4*>(p); }
 
-// Four nibbles, one per byte of `nib4`, -> four f16 weights (two words): d*sc*q - dmin*mn in fp32
-// (dsc = d*sc and ndm = -dmin*mn are exact), one rounding to f16.  The masked word is made opaque
-// so that the four conversions stay v_cvt_f32_ubyte0..3 of one register instead of a bit-field
-// extract plus conversion each.
-__device__ __forceinline__ void weights4(uint32_t nib4, float dsc, float ndm, uint32_t& lo, uint32_t& hi) {
-    asm volatile("" : "+v"(nib4));
-    const f32x2_t a = {fmaf(ubyte0(nib4), dsc, ndm), fmaf(ubyte1(nib4), dsc, ndm)};
-    const f32x2_t b = {fmaf(ubyte2(nib4), dsc, ndm), fmaf(ubyte3(nib4), dsc, ndm)};
-    lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(a, f16x2_t));
-    hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(b, f16x2_t));
-}
-
 constexpr int WAVES = 4;           // one per SIMD; two workgroups share a CU
 constexpr int BM = 256;            // token rows per workgroup
 constexpr int DMA_PER_WAVE = (BM / 8) / WAVES;  // BM / 8 one-KB fetches fill the activation tile
@@ -237,15 +225,16 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     // Issued as inline assembly: the compiler would otherwise wait for every outstanding
     // global_load_lds before any later LDS read (it cannot tell the two tile buffers apart), which
     // exposes the whole fetch latency in every stage.  The waits are placed by hand below.
+    auto load_a1 = [&](uint32_t st, uint32_t buf, int i) {
+        const uint32_t r = a_row0 + 8u * i;
+        const uint8_t* src = xtile + (r < a_rows_left ? r * (a.k * 2u) + (a_swz ^ ((i & 1u) << 6)) : a_last ^ ((i & 1u) << 6)) + (size_t)st * (BK * 2);
+        const uint32_t dst = lds_base + buf * kTile + (wave_u * DMA_PER_WAVE + i) * 1024u;
+        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+        __builtin_amdgcn_sched_barrier(0);  // one address at a time: keeps eight 64-bit pointers out of the registers
+    };
     auto load_a = [&](uint32_t st, uint32_t buf) {
 #pragma unroll
-        for (int i = 0; i < DMA_PER_WAVE; ++i) {
-            const uint32_t r = a_row0 + 8u * i;
-            const uint8_t* src = xtile + (r < a_rows_left ? r * (a.k * 2u) + (a_swz ^ ((i & 1u) << 6)) : a_last ^ ((i & 1u) << 6)) + (size_t)st * (BK * 2);
-            const uint32_t dst = lds_base + buf * kTile + (wave_u * DMA_PER_WAVE + i) * 1024u;
-            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
-            __builtin_amdgcn_sched_barrier(0);  // one address at a time: keeps eight 64-bit pointers out of the registers
-        }
+        for (int i = 0; i < DMA_PER_WAVE; ++i) load_a1(st, buf, i);
     };
 
     // ---- weights: this lane's two rows (one per 32-row tile of the wave), bytes 16*lg.. of each chunk ----
@@ -258,7 +247,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
         wrow[nt] = a.w + (size_t)gn * row_bytes;
         wdown[nt] = reinterpret_cast<const float*>(a.ws + W.wdown)[gn];
     }
-    uint4 braw[2][NT];        // [stage parity][nt]
+    uint4 braw[4][NT];        // nibbles of stages s, s+1, s+2 in slots s%4 (a stage is a chunk of its super-block: slot = c)
     uint4 hdr[NT], hdrn[NT];  // super-block headers: current, next
     auto load_b = [&](uint32_t sblk, int c, int slot) {
 #pragma unroll
@@ -278,62 +267,98 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // prologue: activations of stage 0 on their way to LDS, weights of stage 0 requested
+    // This lane's weight scales of a stage, chunk c of the super-block whose header is h: sub-blocks
+    // 2c (low nibbles) and 2c+1 (high nibbles).
+    auto scales_of = [&](const uint4* h, int c, float (*dsc)[2], float (*ndm)[2]) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            uint32_t sc0, sc1, mn0, mn1;
+            q4k_scales(h[nt].y, h[nt].z, h[nt].w, c, sc0, sc1, mn0, mn1);
+            const float d = f16_bits_to_f32(h[nt].x & 0xffffu) * wdown[nt];
+            const float dmin = f16_bits_to_f32(h[nt].x >> 16) * wdown[nt];
+            dsc[nt][0] = d * (float)sc0;
+            dsc[nt][1] = d * (float)sc1;
+            ndm[nt][0] = -dmin * (float)mn0;
+            ndm[nt][1] = -dmin * (float)mn1;
+        }
+    };
+    // Eighth e of k-step ks of a stage with nibbles b and scales dsc / ndm: two weights -> one
+    // fragment word.  Quarter q = e/2 is one nibble word (nt = q/2, word pair half = q%2), masked
+    // once and kept in mw for its second eighth.
+    uint32_t mw[2 * NT];
+    auto b_eighth = [&](const uint4* b, const float (*dsc)[2], const float (*ndm)[2], int ks, int e, uint4* bfw) {
+        const int q = e >> 1, part = e & 1, nt = q >> 1, half = q & 1;
+        const int hi = ks >> 1;  // 0: low nibbles, 1: high nibbles
+        if (part == 0) {
+            const uint32_t w = (ks & 1) ? (half ? b[nt].w : b[nt].z) : (half ? b[nt].y : b[nt].x);
+            uint32_t m = (hi ? w >> 4 : w) & 0x0f0f0f0fu;
+            // opaque, so that the conversions stay v_cvt_f32_ubyte0..3 of this one register instead of
+            // a bit-field extract plus conversion each
+            asm volatile("" : "+v"(m));
+            mw[q] = m;
+        }
+        const uint32_t m = mw[q];
+        // d*sc*q - dmin*mn in fp32 (dsc and ndm are exact), one rounding to f16
+        const f32x2_t v = {fmaf(part ? ubyte2(m) : ubyte0(m), dsc[nt][hi], ndm[nt][hi]),
+                           fmaf(part ? ubyte3(m) : ubyte1(m), dsc[nt][hi], ndm[nt][hi])};
+        const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+        if (half == 0)
+            (part == 0 ? bfw[nt].x : bfw[nt].y) = r;
+        else
+            (part == 0 ? bfw[nt].z : bfw[nt].w) = r;
+    };
+    constexpr int E = 4 * NT;            // eighths per k-step
+    constexpr int kSteps = 4 * MT;       // MFMA steps per stage: k-step t / MT, row tile t % MT
+    constexpr int PD = NT == 1 ? 3 : 1;  // steps an activation fragment is requested ahead (a step is NT MFMAs)
+    static_assert(kSteps >= DMA_PER_WAVE && (E >= MT ? E % MT == 0 : MT % E == 0 && MT / E >= 2), "the spreading below assumes it");
+
+    // ---- prologue: everything the first stage needs, and the second stage's nibbles ----
     load_hdr(0, hdr);
     load_b(0, 0, 0);
+    if (nstages > 1) load_b(0, 1, 1);  // k >= 256: a super-block has four stages
     load_a(0, 0);
     if (nsb > 1) load_hdr(1, hdrn);
+    float dsc[NT][2], ndm[NT][2];      // scales of the stage being multiplied
+    uint4 bfc[NT], bfn[NT];            // weight fragments: current k-step, next
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    scales_of(hdr, 0, dsc, ndm);
+#pragma unroll
+    for (int e = 0; e < E; ++e) b_eighth(braw[0], dsc, ndm, 0, e, bfc);
     __syncthreads();
 
+    // The loop is software pipelined over stages as well: while the last k-step of stage s is
+    // multiplied, the scales of stage s+1 and the fragments of its first k-step are formed, so a
+    // stage begins with an MFMA and not with sixty VALU instructions that nothing overlaps.
     for (uint32_t sblk = 0; sblk < nsb; ++sblk) {
         const bool next_sb = sblk + 1 < nsb;  // uniform
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t st = 4 * sblk + c;
             const uint32_t buf = c & 1;
-            // This stage's nibbles, requested a stage ago.  They are claimed here, before the activation
-            // fetch below is issued: the compiler does not know about that fetch, and the wait it puts
-            // in front of the first use of these registers would otherwise cover it too.
-            uint4 bcur[NT];
+            const bool has_next = c < 3 || next_sb;  // uniform: stage st + 1 exists
+            // The next stage's nibbles, requested a stage ago.  They are claimed here, before this
+            // stage's activation fetches are issued: the compiler does not know about those, and the
+            // wait it puts in front of the first use of these registers would otherwise cover them too.
+            uint4 bnext[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                bcur[nt] = braw[c & 1][nt];
-                asm volatile("" : "+v"(bcur[nt].x), "+v"(bcur[nt].y), "+v"(bcur[nt].z), "+v"(bcur[nt].w));
+                bnext[nt] = braw[(c + 1) & 3][nt];
+                asm volatile("" : "+v"(bnext[nt].x), "+v"(bnext[nt].y), "+v"(bnext[nt].z), "+v"(bnext[nt].w));
             }
-            if (c == 0 && sblk > 0) {  // this super-block's header; request the next one (before the
-#pragma unroll                         // activation fetch, so that it is older than it)
+            if (c == 0 && sblk > 0) {  // this super-block's header; request the next one
+#pragma unroll
                 for (int nt = 0; nt < NT; ++nt) hdr[nt] = hdrn[nt];
                 if (next_sb) load_hdr(sblk + 1, hdrn);
             }
-            // next stage's activations into the other buffer (free since the barrier that ended the
-            // previous stage)
-            if (st + 1 < nstages) load_a(st + 1, buf ^ 1u);
-
-            // this stage's weight scales: sub-blocks 2c (low nibbles) and 2c+1 (high nibbles)
-            float dsc[NT][2], ndm[NT][2];  // [nt][low / high]
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                uint32_t sc0, sc1, mn0, mn1;
-                q4k_scales(hdr[nt].y, hdr[nt].z, hdr[nt].w, c, sc0, sc1, mn0, mn1);
-                const float d = f16_bits_to_f32(hdr[nt].x & 0xffffu) * wdown[nt];
-                const float dmin = f16_bits_to_f32(hdr[nt].x >> 16) * wdown[nt];
-                dsc[nt][0] = d * (float)sc0;
-                dsc[nt][1] = d * (float)sc1;
-                ndm[nt][0] = -dmin * (float)mn0;
-                ndm[nt][1] = -dmin * (float)mn1;
-            }
-            // request the next stage's nibbles into the other pair of registers (the header fetch of a
-            // super-block, issued a super-block ahead, has already pulled most of its lines into cache)
-            if (c < 3) {
-                load_b(sblk, c + 1, (c & 1) ^ 1);
+            // nibbles of stage st + 2 (the header fetch of a super-block, issued a super-block ahead, has
+            // already pulled most of its lines into cache)
+            if (c < 2) {
+                load_b(sblk, c + 2, (c + 2) & 3);
             } else if (next_sb) {
-                load_b(sblk + 1, 0, (c & 1) ^ 1);
+                load_b(sblk + 1, c - 2, (c + 2) & 3);
             }
+            const bool fetch_a = st + 1 < nstages;  // uniform
 
-            // ---- the stage's 4*MT steps (k-step ks = t/MT, row tile mt = t%MT), software pipelined:
-            // the activation fragment of step t+1 is requested, and a share of the next k-step's
-            // weight fragments is dequantised, between the two MFMAs of step t ----
             auto a_frag = [&](int t) -> uint4 {
                 const int ks = t / MT, mt = t % MT;
                 // chunk index of this lane group's 8 activations inside the row's 64
@@ -341,73 +366,102 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                 const uint32_t row = wm * (32 * MT) + mt * 32 + l32;
                 return *reinterpret_cast<const uint4*>(smem + buf * kTile + row * (ROW * 2) + ((kchunk ^ ((row >> 1) & 7u)) << 4));
             };
-            // quarter q (nt = q/2, word pair half = q%2) of k-step ks: four weights -> words 2*(q%2), +1
-            auto b_quarter = [&](int ks, int q, uint4* bfw) {
-                const int nt = q >> 1, half = q & 1;
-                const uint4 b = bcur[nt];
-                const uint32_t w = (ks & 1) ? (half ? b.w : b.z) : (half ? b.y : b.x);
-                const int hi = ks >> 1;  // 0: low nibbles, 1: high nibbles
-                uint32_t lo2, hi2;
-                weights4((hi ? w >> 4 : w) & 0x0f0f0f0fu, dsc[nt][hi], ndm[nt][hi], lo2, hi2);
-                if (half == 0)
-                    bfw[nt].x = lo2, bfw[nt].y = hi2;
-                else
-                    bfw[nt].z = lo2, bfw[nt].w = hi2;
-            };
-            uint4 bfc[NT], bfn[NT];
+            float dscn[NT][2], ndmn[NT][2];  // scales of stage st + 1
+            uint4 af[PD + 1];
 #pragma unroll
-            for (int q = 0; q < 2 * NT; ++q) b_quarter(0, q, bfc);
-            uint4 af0 = a_frag(0), af1;
+            for (int t = 0; t < PD; ++t) af[t] = a_frag(t);
 #pragma unroll
-            for (int t = 0; t < 4 * MT; ++t) {
+            for (int t = 0; t < kSteps; ++t) {
                 const int ks = t / MT, mt = t % MT;
-                if (t + 1 < 4 * MT) af1 = a_frag(t + 1);
-                acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(af0), as_frag(bfc[0]), acc[mt][0], 0, 0, 0);
-                if (ks + 1 < 4 && mt < 2 * NT) b_quarter(ks + 1, mt, bfn);  // 2*NT quarters over the first of the MT steps
+                if (t + PD < kSteps) af[(t + PD) % (PD + 1)] = a_frag(t + PD);
+                // The next stage's activations go into the other buffer (free since the barrier that ended
+                // the previous stage), one fetch per step at the start of the stage rather than all at once.
+                if (t < DMA_PER_WAVE && fetch_a) load_a1(st + 1, buf ^ 1u, t);
+                const uint4 afc = af[t % (PD + 1)];
+                acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(bfc[0]), as_frag(afc), acc[mt][0], 0, 0, 0);
+                // The next k-step's weights, spread evenly over this k-step's MFMAs (an MFMA hides about
+                // four VALU instructions; what exceeds that delays the next MFMA).  In the last k-step
+                // they are the next stage's first, preceded by that stage's scales.
+                if (ks < 3) {
+                    if constexpr (E >= MT) {
+#pragma unroll
+                        for (int e = 0; e < E / MT; ++e) b_eighth(braw[c], dsc, ndm, ks + 1, mt * (E / MT) + e, bfn);
+                    } else if (mt % (MT / E) == 0) {
+                        b_eighth(braw[c], dsc, ndm, ks + 1, mt / (MT / E), bfn);
+                    }
+                } else if (has_next) {
+                    if (mt == 0) scales_of(c < 3 ? hdr : hdrn, (c + 1) & 3, dscn, ndmn);
+                    if constexpr (E >= MT) {
+                        // the scales come first, so the eighths of row tile 0 move to the last one's slot
+                        if (mt > 0) {
+#pragma unroll
+                            for (int e = 0; e < E / MT; ++e) b_eighth(bnext, dscn, ndmn, 0, (mt - 1) * (E / MT) + e, bfn);
+                        }
+                        if (mt == MT - 1) {
+#pragma unroll
+                            for (int e = 0; e < E / MT; ++e) b_eighth(bnext, dscn, ndmn, 0, (MT - 1) * (E / MT) + e, bfn);
+                        }
+                    } else if (mt % (MT / E) == 1) {
+                        b_eighth(bnext, dscn, ndmn, 0, mt / (MT / E), bfn);
+                    }
+                }
                 if constexpr (NT == 2)
-                    acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(af0), as_frag(bfc[1]), acc[mt][1], 0, 0, 0);
+                    acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(bfc[1]), as_frag(afc), acc[mt][1], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                af0 = af1;
                 if (mt == MT - 1) {
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) bfc[nt] = bfn[nt];
                 }
             }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                dsc[nt][0] = dscn[nt][0], dsc[nt][1] = dscn[nt][1];
+                ndm[nt][0] = ndmn[nt][0], ndm[nt][1] = ndmn[nt][1];
+            }
 
-            // The next stage's activations must have landed before anyone reads them.  Vector memory
-            // operations complete in order: the only ones issued after them in this stage are the NT
-            // weight fetches above, which may stay in flight.
-            if (c < 3 || next_sb)
-                asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NT) : "memory");
-            else
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            // The next stage's activations must have landed before anyone reads them.  They are the
+            // youngest vector memory operations of this wave and such operations complete in order.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
         }
     }
 
-    // ---- store: value v of a lane is row 8*(v/4) + 4*(lane/32) + v%4, column lane%32 (the weight row this
-    // lane dequantised); undo the activation-row and weight-row scales ----
+    // ---- store.  The weights are the MFMA's first operand, so an accumulator tile is indexed
+    // [weight row][token]: value v of a lane belongs to token lane%32 and weight row
+    // 8*(v/4) + 4*(lane/32) + v%4 of the tile, four consecutive outputs of one token per v/4, one
+    // 16-byte store.  Undo the activation-row and weight-row scales. ----
     const float* rs = reinterpret_cast<const float*>(a.ws + W.rs);
+    const float* wd = reinterpret_cast<const float*>(a.ws + W.wdown);
+    const bool vec_ok = a.n % 4 == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;  // uniform
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const uint32_t gmb = m0 + wm * (32 * MT) + mt * 32 + 4 * lg;
-        float rsv[16];
+    for (int nt = 0; nt < NT; ++nt) {
+        const uint32_t gnb = n0 + wn * (32 * NT) + nt * 32 + 4 * lg;
+        float wup[16];  // 2^e of the 16 weight rows, from their 2^-e
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            uint32_t gm = gmb + 8 * (v >> 2) + (v & 3);
-            gm = gm < a.m ? gm : a.m - 1u;
-            rsv[v] = rs[gm];
+            uint32_t gn = gnb + 8 * (v >> 2) + (v & 3);
+            gn = gn < a.n ? gn : a.n - 1u;
+            wup[v] = __uint_as_float(0x7f000000u - __float_as_uint(wd[gn]));
         }
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const uint32_t gcol = n0 + wn * (32 * NT) + nt * 32 + l32;
-            const float wup = __uint_as_float(0x7f000000u - __float_as_uint(wdown[nt]));  // 2^e from 2^-e
-            if (gcol < a.n) {
-                float* yp = a.y + (size_t)gmb * a.n + gcol;
+        for (int mt = 0; mt < MT; ++mt) {
+            const uint32_t gm = m0 + wm * (32 * MT) + mt * 32 + l32;
+            if (gm >= a.m) continue;
+            const float rsv = rs[gm];
+            float* yp = a.y + (size_t)gm * a.n + gnb;
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (gmb + 8 * (v >> 2) + (v & 3) < a.m)
-                        yp[(size_t)(8 * (v >> 2) + (v & 3)) * a.n] = acc[mt][nt][v] * (rsv[v] * wup);
+            for (int g = 0; g < 4; ++g) {
+                const float o0 = acc[mt][nt][4 * g] * (rsv * wup[4 * g]), o1 = acc[mt][nt][4 * g + 1] * (rsv * wup[4 * g + 1]);
+                const float o2 = acc[mt][nt][4 * g + 2] * (rsv * wup[4 * g + 2]), o3 = acc[mt][nt][4 * g + 3] * (rsv * wup[4 * g + 3]);
+                const uint32_t gn = gnb + 8 * g;
+                if (vec_ok) {
+                    if (gn < a.n) *reinterpret_cast<float4*>(yp + 8 * g) = make_float4(o0, o1, o2, o3);
+                } else {
+                    if (gn < a.n) yp[8 * g] = o0;
+                    if (gn + 1 < a.n) yp[8 * g + 1] = o1;
+                    if (gn + 2 < a.n) yp[8 * g + 2] = o2;
+                    if (gn + 3 < a.n) yp[8 * g + 3] = o3;
+                }
             }
         }
     }
