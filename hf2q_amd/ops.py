@@ -280,6 +280,40 @@ def dispatch_moe_weighted_reduce(y: torch.Tensor, w: torch.Tensor, out: torch.Te
 
 
 @dataclass
+class DenseFfnWeightsGpuQ:
+    """gpu_ffn.rs:260-280: gate / up `[inter, hidden]` and down `[hidden, inter]` as raw GGML blocks."""
+    gate_q: torch.Tensor
+    up_q: torch.Tensor
+    down_q: torch.Tensor
+    ggml_type: int
+    hidden: int
+    inter: int
+
+
+def build_dense_ffn_layer_gpu_q_into(x: torch.Tensor, w: DenseFfnWeightsGpuQ, gate_buf: torch.Tensor,
+                                     up_buf: torch.Tensor, act_buf: torch.Tensor | None, out: torch.Tensor,
+                                     batched: bool | None = None) -> None:
+    """gpu_ffn.rs:1086-1330: out = down(silu(gate x) * (up x)) for seq_len rows of x.  The reference encodes gate
+    and up back to back (one barrier after both), then silu_mul, then down.  `batched` (default: whenever the
+    row count is decode-sized) hands gate + up to the library as one launch and folds the SwiGLU into the
+    staging of the down projection: two launches instead of four, identical results (act_buf is then unused)."""
+    m = x.shape[0]
+    H, I, t = w.hidden, w.inter, w.ggml_type
+    if batched is None:
+        batched = m <= _BATCH_MAX_DENSE_ROWS
+    if batched:
+        if m > _BATCH_MAX_DENSE_ROWS:
+            raise ValueError(f"batched dense FFN: {m} rows (limit {_BATCH_MAX_DENSE_ROWS})")
+        quantized_matmul_batch_ggml([QmatmulJob(x, w.gate_q, gate_buf, m, I, H), QmatmulJob(x, w.up_q, up_buf, m, I, H)], t)
+        quantized_matmul_batch_ggml([QmatmulJob(gate_buf, w.down_q, out, m, H, I, input_up=up_buf)], t)
+        return
+    quantized_matmul_ggml(x, w.gate_q, gate_buf, GgmlQuantizedMatmulParams(m, I, H, t))
+    quantized_matmul_ggml(x, w.up_q, up_buf, GgmlQuantizedMatmulParams(m, I, H, t))
+    dispatch_silu_mul(gate_buf[:m], up_buf[:m], act_buf[:m])
+    quantized_matmul_ggml(act_buf, w.down_q, out, GgmlQuantizedMatmulParams(m, H, I, t))
+
+
+@dataclass
 class MoeFfnWeightsGpuQ:
     """Device weights of one quantized MoE FFN layer (gpu_ffn.rs:214-358): router and shared-gate logit in
     bf16, expert stacks and the shared expert as raw GGML blocks."""

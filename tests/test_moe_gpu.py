@@ -196,3 +196,28 @@ def test_dense_gemv_bf16_pair_equals_two_calls(dev):
     ops.dense_gemv_bf16_f32(x, wb, yb, m, nb, k)
     ops.dense_gemv_bf16_f32_pair(x, wa, ya2, na, wb, yb2, nb, m, k)
     assert torch.equal(ya.cpu(), ya2.cpu()) and torch.equal(yb.cpu(), yb2.cpu())
+
+
+@pytest.mark.parametrize("m", [1, 4])
+@pytest.mark.parametrize("t,xdt", [(HQ_Q4_K, torch.bfloat16), (HQ_Q4_K, torch.float32), (HQ_Q6_K, torch.bfloat16)])
+def test_dense_ffn_batched_equals_separate_dispatches_and_cpu_spec(oracle, dev, m, t, xdt):
+    """dense_swiglu (ffn.rs:91-112) over the dequantised weights; two launches against four, bit for bit."""
+    H, I = 512, 1280
+    raw = {"g": weights(31, I, H, 0.05), "u": weights(32, I, H, 0.05), "d": weights(33, H, I, 0.05)}
+    q = {k_: oracle.quantize(v, v.shape[1], t, threads=8) for k_, v in raw.items()}
+    dq = {k_: oracle.dequantize(q[k_], t).reshape(raw[k_].shape).astype(np.float64) for k_ in raw}
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    w = ops.DenseFfnWeightsGpuQ(dv(q["g"]), dv(q["u"]), dv(q["d"]), t, H, I)
+    x = dv(acts(34 + m, m, H)).to(xdt)
+    outs = []
+    for batched in (False, True):
+        g, u, a = (torch.full((m, I), float("nan"), device=dev) for _ in range(3))
+        out = torch.full((m, H), float("nan"), device=dev)
+        ops.build_dense_ffn_layer_gpu_q_into(x, w, g, u, a, out, batched=batched)
+        outs.append((out.cpu(), g.cpu(), u.cpu()))
+    for a_, b_ in zip(*outs):
+        assert torch.equal(a_, b_)
+    xr = x.float().cpu().numpy().astype(np.float64)
+    gate, up = xr @ dq["g"].T, xr @ dq["u"].T
+    want = (gate / (1 + np.exp(-gate)) * up) @ dq["d"].T
+    assert_matmul_close(outs[1][0].numpy(), want, "dense FFN")
