@@ -296,7 +296,7 @@ def build_dense_ffn_layer_gpu_q_into(x: torch.Tensor, w: DenseFfnWeightsGpuQ, ga
     """gpu_ffn.rs:1086-1330: out = down(silu(gate x) * (up x)) for seq_len rows of x.  The reference encodes gate
     and up back to back (one barrier after both), then silu_mul, then down.  `batched` (default: whenever the
     row count is decode-sized) hands gate + up to the library as one launch and folds the SwiGLU into the
-    staging of the down projection: two launches instead of four, identical results (act_buf is then unused)."""
+    staging of the down projection (for inter <= 8192): two launches instead of four, identical results."""
     m = x.shape[0]
     H, I, t = w.hidden, w.inter, w.ggml_type
     if batched is None:
@@ -305,7 +305,13 @@ def build_dense_ffn_layer_gpu_q_into(x: torch.Tensor, w: DenseFfnWeightsGpuQ, ga
         if m > _BATCH_MAX_DENSE_ROWS:
             raise ValueError(f"batched dense FFN: {m} rows (limit {_BATCH_MAX_DENSE_ROWS})")
         quantized_matmul_batch_ggml([QmatmulJob(x, w.gate_q, gate_buf, m, I, H), QmatmulJob(x, w.up_q, up_buf, m, I, H)], t)
-        quantized_matmul_batch_ggml([QmatmulJob(gate_buf, w.down_q, out, m, H, I, input_up=up_buf)], t)
+        # Every workgroup of the fused down projection forms the whole activation vector itself; past a few
+        # thousand activations a separate SwiGLU pass is as fast (measured equal at 12288).
+        if I <= _FUSED_SWIGLU_MAX_K or act_buf is None:
+            quantized_matmul_batch_ggml([QmatmulJob(gate_buf, w.down_q, out, m, H, I, input_up=up_buf)], t)
+        else:
+            dispatch_silu_mul(gate_buf[:m], up_buf[:m], act_buf[:m])
+            quantized_matmul_ggml(act_buf, w.down_q, out, GgmlQuantizedMatmulParams(m, H, I, t))
         return
     quantized_matmul_ggml(x, w.gate_q, gate_buf, GgmlQuantizedMatmulParams(m, I, H, t))
     quantized_matmul_ggml(x, w.up_q, up_buf, GgmlQuantizedMatmulParams(m, I, H, t))
@@ -351,6 +357,7 @@ class MoeFfnScratch:
 
 # Dense products above this many rows take the tile (GEMM) route, which the batched launch does not cover.
 _BATCH_MAX_DENSE_ROWS = 8
+_FUSED_SWIGLU_MAX_K = 8192
 
 
 def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch, out: torch.Tensor,
