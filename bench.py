@@ -229,7 +229,7 @@ def bench_prefill_gemm(a):
     x = torch.randn(M, K, generator=gx, device=dev).to(torch.bfloat16)
     y = torch.empty(M, N, device=dev)
     p = GgmlQuantizedMatmulParams(M, N, K, t)
-    # caller-owned scratch for the Q4_K kernel's activation pre-pass (none for Q8_0): allocated once
+    # caller-owned scratch for the tile kernels' pre-pass (f16 activations, row scales): allocated once
     need = ops.quantized_matmul_workspace_bytes(p, torch.bfloat16)
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     for _ in range(a.warmup):
@@ -248,12 +248,12 @@ def bench_prefill_gemm(a):
     tf = flops / us / 1e6
     _finish(a, {
         "metric": "prefill TFLOP/s", "value": round(flops * a.steps / elapsed / 1e12, 1), "unit": "TFLOP/s",
-        "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f16" if t == HQ_Q4_K else "bf16",
+        "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f16" if need else "bf16",
         "config": {"workload": f"prefill_gemm: 2048 tokens x K=4096 x N=12288, {a.wtype.upper()} weights, bf16 "
                                f"activations, fp32 accumulate (BASELINE config 4)", "flop_per_step": flops,
                    "weight_bytes": w.numel(), "workspace_bytes": need,
                    "launches_per_step": 2 if need else 1},
-        "roofline": {"bound": "mfma", "kernel": ("activation pre-pass + f16 MFMA gemm q4_k" if need else
+        "roofline": {"bound": "mfma", "kernel": (f"activation pre-pass + f16 MFMA gemm {a.wtype}" if need else
                                                  f"bf16 MFMA gemm {a.wtype}"), "achieved": round(tf, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": None, "us_per_launch": round(us, 2), "flop_per_launch": flops}})

@@ -130,12 +130,12 @@ static int check_matmul_common(const char* fn, const void* x, hq_act_dtype xdt, 
 
 namespace {
 
-bool q4k_tile_route(uint32_t m, uint32_t k, hq_ggml_type t) { return t == HQ_Q4_K && m > kGemvMaxRows && k % 256 == 0; }
+bool f16_tile_route(uint32_t m, uint32_t k, hq_ggml_type t) { return m > kGemvMaxRows && gemm_f16_tile_supported(t, k); }
 
-// All routes of the dense product; `workspace` is only read on the Q4_K tile route.
+// All routes of the dense product; `workspace` is only read on the f16 tile route.
 int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
                    uint32_t n, uint32_t k, hq_ggml_type t, void* workspace) {
-    if (q4k_tile_route(m, k, t)) return launch_gemm_q4k(stream, x, xdt, w_blocks, y, m, n, k, workspace);
+    if (f16_tile_route(m, k, t)) return launch_gemm_f16_tile(stream, x, xdt, w_blocks, y, m, n, k, t, workspace);
     if (m > kGemvMaxRows && gemm_supported(t, k)) return launch_gemm(stream, x, xdt, w_blocks, y, m, n, k, t);
     // GEMV form, kGemvMaxRows activation rows per launch (also the route of shapes the
     // tile kernels do not cover).
@@ -162,7 +162,7 @@ int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const vo
 size_t hq_qmatmul_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
     (void)n;
     (void)xdt;
-    return q4k_tile_route(m, k, t) ? gemm_q4k_workspace_bytes(m, n, k) : 0;
+    return f16_tile_route(m, k, t) ? gemm_f16_tile_workspace_bytes(m, n, k) : 0;
 }
 
 int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,

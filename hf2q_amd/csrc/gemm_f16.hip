@@ -1,4 +1,4 @@
-// Batched-prefill GEMM for Q4_K weights (m > 8): y[m,n] = x[m,k] . W[n,k]^T on the
+// Batched-prefill GEMM for Q4_K and Q8_0 weights (m > 8): y[m,n] = x[m,k] . W[n,k]^T on the
 // f16 matrix cores (v_mfma_f32_32x32x16_f16) with fp32 accumulation.
 //
 // Numerics.  The weight tile holds the dequantised weights rounded to f16, which
@@ -83,25 +83,35 @@ __device__ __forceinline__ uint32_t f16_bits(float v) {
 }
 
 // Pre-pass.  Workgroups [0, m): one per activation row, row scale and f16 conversion.  Workgroups
-// from m on: 16 weight rows each, 16 lanes per row over the row's super-block headers.  Per weight
-// row, a power of two that brings the row's largest possible |w| = |d|*63*15 + |dmin|*63 to about
-// 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
+// from m on: 16 weight rows each, 16 lanes per row over the row's block headers.  Per weight row, a
+// power of two that brings the row's largest possible |w| (Q4_K: |d|*63*15 + |dmin|*63, Q8_0:
+// |d|*128) to about 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
 // subnormals; the main kernel multiplies the weights by it before they are rounded (exact) and its
 // epilogue divides it out.
-template <bool X_BF16>
-__global__ __launch_bounds__(256) void q4k_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
-                                                       uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k) {
+template <bool X_BF16, int TYPE>
+__global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
+                                                        uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k) {
     __shared__ float red[4];
     const uint32_t tid = threadIdx.x;
     const Workspace L = workspace_layout(m, n, k);
     if (blockIdx.x >= m) {
-        const uint32_t wr = (blockIdx.x - m) * 16u + (tid >> 4), nsb = k / 256;
-        const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nsb * Q4K_BYTES;
+        const uint32_t wr = (blockIdx.x - m) * 16u + (tid >> 4);
         float bound = 0.f;
-        for (uint32_t sb = tid & 15u; sb < nsb; sb += 16u) {
-            const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow + (size_t)sb * Q4K_BYTES);
-            const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * 945.f + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
-            bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;  // inf / nan scales do not set the exponent
+        if constexpr (TYPE == HQ_Q4_K) {
+            const uint32_t nsb = k / 256;
+            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nsb * Q4K_BYTES;
+            for (uint32_t sb = tid & 15u; sb < nsb; sb += 16u) {
+                const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow + (size_t)sb * Q4K_BYTES);
+                const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * 945.f + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
+                bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;  // inf / nan scales do not set the exponent
+            }
+        } else {  // Q8_0: |w| <= |d| * 128
+            const uint32_t nb = k / 32;
+            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nb * Q8_0_BYTES;
+            for (uint32_t b = tid & 15u; b < nb; b += 16u) {
+                const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)b * Q8_0_BYTES))) * 128.f;
+                bound = v <= 3.0e38f ? fmaxf(bound, v) : bound;
+            }
         }
         bound = dpp_max<0xB1>(bound);  // the four steps cover a row of 16 lanes
         bound = dpp_max<0x4E>(bound);
@@ -190,14 +200,100 @@ constexpr int BM = 256;            // token rows per workgroup
 constexpr int DMA_PER_WAVE = (BM / 8) / WAVES;  // BM / 8 one-KB fetches fill the activation tile
 constexpr int BN_WIDE = 128, BN_NARROW = 64;    // weight rows per workgroup
 
-// One workgroup tile: rows m0.. of the activations, weight rows n0...  The four waves form a
-// (4 / WN) x WN grid; a wave owns MT x NT MFMA tiles of 32 x 32.
+// Activation side of a workgroup tile, the same for every weight type: the pre-pass output goes
+// global -> LDS in 1 KB wave instructions; wave w, instruction i (< DMA_PER_WAVE) fills 8 LDS rows of
+// the tile, (w * DMA_PER_WAVE + i) * 8 .. +8; lane L owns row L/8 of them and LDS chunk L%8, which
+// holds global chunk (L%8) ^ ((row/2)%8), and (row/2)%8 = L/16 + 4*(i%2).  Rows past the end of x read
+// the last row instead (their results are never stored).
+struct ActTile {
+    static constexpr int kTile = BM * ROW * 2;  // bytes of one activation buffer; two of them in LDS
+    uint8_t* smem;
+    const uint8_t* xtile;
+    uint32_t a_swz, a_row0, a_rows_left, a_last, row_pitch, wave_u, lds_base;
+
+    __device__ __forceinline__ void init(const GemmArgs& a, const Workspace& W, uint32_t m0, uint32_t lane, uint32_t wave) {
+        extern __shared__ uint4 smem4[];
+        smem = reinterpret_cast<uint8_t*>(smem4);
+        row_pitch = a.k * 2u;
+        a_swz = ((lane & 7u) ^ (lane >> 4)) << 4;
+        a_row0 = wave * (8u * DMA_PER_WAVE) + (lane >> 3);
+        a_rows_left = a.m - m0;  // >= 1
+        a_last = (a_rows_left - 1u) * row_pitch + a_swz;
+        xtile = a.ws + W.xh + (size_t)m0 * row_pitch;
+        wave_u = __builtin_amdgcn_readfirstlane(wave);  // the same value, known to be uniform
+        // LDS byte address of the tile buffers (wave-uniform, goes to M0)
+        lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem);
+    }
+    // Fetch i of stage st into buffer buf.  Issued as inline assembly: the compiler would otherwise
+    // wait for every outstanding global_load_lds before any later LDS read (it cannot tell the two
+    // buffers apart), which exposes the whole fetch latency in every stage.  The waits are placed by
+    // hand by the callers.
+    __device__ __forceinline__ void fetch(uint32_t st, uint32_t buf, int i) const {
+        const uint32_t r = a_row0 + 8u * i;
+        const uint8_t* src = xtile + (r < a_rows_left ? r * row_pitch + (a_swz ^ ((i & 1u) << 6)) : a_last ^ ((i & 1u) << 6)) + (size_t)st * (BK * 2);
+        const uint32_t dst = lds_base + buf * kTile + (wave_u * DMA_PER_WAVE + i) * 1024u;
+        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+        __builtin_amdgcn_sched_barrier(0);  // one address at a time: keeps eight 64-bit pointers out of the registers
+    }
+    __device__ __forceinline__ void fetch_all(uint32_t st, uint32_t buf) const {
+#pragma unroll
+        for (int i = 0; i < DMA_PER_WAVE; ++i) fetch(st, buf, i);
+    }
+    // The 8 activations of 16-byte chunk kchunk (of the row's 64 per stage) of tile row `row`.
+    __device__ __forceinline__ uint4 frag(uint32_t buf, uint32_t row, uint32_t kchunk) const {
+        return *reinterpret_cast<const uint4*>(smem + buf * kTile + row * (ROW * 2) + ((kchunk ^ ((row >> 1) & 7u)) << 4));
+    }
+};
+
+// Stores a wave's accumulators.  The weights are the MFMA's first operand, so an accumulator tile
+// is indexed [weight row][token]: value v of a lane belongs to token lane%32 and weight row
+// 8*(v/4) + 4*(lane/32) + v%4 of the tile, four consecutive outputs of one token per v/4, one
+// 16-byte store.  Undoes the activation-row and weight-row scales.
+template <int MT, int NT>
+__device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W, const f32x16_t (&acc)[MT][NT],
+                                           uint32_t mbase, uint32_t nbase, uint32_t l32, uint32_t lg) {
+    const float* rs = reinterpret_cast<const float*>(a.ws + W.rs);
+    const float* wd = reinterpret_cast<const float*>(a.ws + W.wdown);
+    const bool vec_ok = a.n % 4 == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;  // uniform
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const uint32_t gnb = nbase + nt * 32 + 4 * lg;
+        float wup[16];  // 2^e of the 16 weight rows, from their 2^-e
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            uint32_t gn = gnb + 8 * (v >> 2) + (v & 3);
+            gn = gn < a.n ? gn : a.n - 1u;
+            wup[v] = __uint_as_float(0x7f000000u - __float_as_uint(wd[gn]));
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const uint32_t gm = mbase + mt * 32 + l32;
+            if (gm >= a.m) continue;
+            const float rsv = rs[gm];
+            float* yp = a.y + (size_t)gm * a.n + gnb;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float o0 = acc[mt][nt][4 * g] * (rsv * wup[4 * g]), o1 = acc[mt][nt][4 * g + 1] * (rsv * wup[4 * g + 1]);
+                const float o2 = acc[mt][nt][4 * g + 2] * (rsv * wup[4 * g + 2]), o3 = acc[mt][nt][4 * g + 3] * (rsv * wup[4 * g + 3]);
+                const uint32_t gn = gnb + 8 * g;
+                if (vec_ok) {
+                    if (gn < a.n) *reinterpret_cast<float4*>(yp + 8 * g) = make_float4(o0, o1, o2, o3);
+                } else {
+                    if (gn < a.n) yp[8 * g] = o0;
+                    if (gn + 1 < a.n) yp[8 * g + 1] = o1;
+                    if (gn + 2 < a.n) yp[8 * g + 2] = o2;
+                    if (gn + 3 < a.n) yp[8 * g + 3] = o3;
+                }
+            }
+        }
+    }
+}
+
+// One workgroup tile of Q4_K weights: rows m0.. of the activations, weight rows n0...  The four
+// waves form a (4 / WN) x WN grid; a wave owns MT x NT MFMA tiles of 32 x 32.
 template <int MT, int NT, int WN>
 __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
-    extern __shared__ uint4 smem4[];
-    uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
-    constexpr int kTile = BM * ROW * 2;  // one activation tile, padded; two of them in LDS
     const Workspace W = workspace_layout(a.m, a.n, a.k);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -206,36 +302,8 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 
     const uint32_t nsb = a.k / 256, nstages = a.k / BK;
     const uint32_t row_bytes = nsb * Q4K_BYTES;
-
-    // ---- activation staging: wave w, instruction i (< DMA_PER_WAVE) fills 8 LDS rows of the tile,
-    // (w * DMA_PER_WAVE + i) * 8 .. +8; lane L owns row L/8 of them and LDS chunk L%8, which holds
-    // global chunk (L%8) ^ ((row/2)%8), and (row/2)%8 = L/16 + 4*(i%2) ----
-    // byte offset of this lane's source chunk from the tile's first row, stage 0: the wave's first row + L/8
-    // for i = 0, 8 rows further per instruction; rows past the end of x read the last row instead (their
-    // results are never stored)
-    const uint32_t a_swz = ((lane & 7u) ^ (lane >> 4)) << 4;
-    const uint32_t a_row0 = wave * (8u * DMA_PER_WAVE) + (lane >> 3);
-    const uint32_t a_rows_left = a.m - m0;  // >= 1
-    const uint32_t a_last = (a_rows_left - 1u) * (a.k * 2u) + a_swz;
-    const uint8_t* xtile = a.ws + W.xh + (size_t)m0 * a.k * 2;
-    const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);  // the same value, known to be uniform
-    // LDS byte address of the tile buffers (wave-uniform, goes to M0)
-    const uint32_t lds_base =
-        __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem);
-    // Issued as inline assembly: the compiler would otherwise wait for every outstanding
-    // global_load_lds before any later LDS read (it cannot tell the two tile buffers apart), which
-    // exposes the whole fetch latency in every stage.  The waits are placed by hand below.
-    auto load_a1 = [&](uint32_t st, uint32_t buf, int i) {
-        const uint32_t r = a_row0 + 8u * i;
-        const uint8_t* src = xtile + (r < a_rows_left ? r * (a.k * 2u) + (a_swz ^ ((i & 1u) << 6)) : a_last ^ ((i & 1u) << 6)) + (size_t)st * (BK * 2);
-        const uint32_t dst = lds_base + buf * kTile + (wave_u * DMA_PER_WAVE + i) * 1024u;
-        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
-        __builtin_amdgcn_sched_barrier(0);  // one address at a time: keeps eight 64-bit pointers out of the registers
-    };
-    auto load_a = [&](uint32_t st, uint32_t buf) {
-#pragma unroll
-        for (int i = 0; i < DMA_PER_WAVE; ++i) load_a1(st, buf, i);
-    };
+    ActTile at;
+    at.init(a, W, m0, lane, wave);
 
     // ---- weights: this lane's two rows (one per 32-row tile of the wave), bytes 16*lg.. of each chunk ----
     const uint8_t* wrow[NT];
@@ -316,7 +384,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     load_hdr(0, hdr);
     load_b(0, 0, 0);
     if (nstages > 1) load_b(0, 1, 1);  // k >= 256: a super-block has four stages
-    load_a(0, 0);
+    at.fetch_all(0, 0);
     if (nsb > 1) load_hdr(1, hdrn);
     float dsc[NT][2], ndm[NT][2];      // scales of the stage being multiplied
     uint4 bfc[NT], bfn[NT];            // weight fragments: current k-step, next
@@ -362,9 +430,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
             auto a_frag = [&](int t) -> uint4 {
                 const int ks = t / MT, mt = t % MT;
                 // chunk index of this lane group's 8 activations inside the row's 64
-                const uint32_t kchunk = ks < 2 ? 2u * lg + ks : 4u + 2u * lg + (ks - 2);
-                const uint32_t row = wm * (32 * MT) + mt * 32 + l32;
-                return *reinterpret_cast<const uint4*>(smem + buf * kTile + row * (ROW * 2) + ((kchunk ^ ((row >> 1) & 7u)) << 4));
+                return at.frag(buf, wm * (32 * MT) + mt * 32 + l32, ks < 2 ? 2u * lg + ks : 4u + 2u * lg + (ks - 2));
             };
             float dscn[NT][2], ndmn[NT][2];  // scales of stage st + 1
             uint4 af[PD + 1];
@@ -376,7 +442,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                 if (t + PD < kSteps) af[(t + PD) % (PD + 1)] = a_frag(t + PD);
                 // The next stage's activations go into the other buffer (free since the barrier that ended
                 // the previous stage), one fetch per step at the start of the stage rather than all at once.
-                if (t < DMA_PER_WAVE && fetch_a) load_a1(st + 1, buf ^ 1u, t);
+                if (t < DMA_PER_WAVE && fetch_a) at.fetch(st + 1, buf ^ 1u, t);
                 const uint4 afc = af[t % (PD + 1)];
                 acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(bfc[0]), as_frag(afc), acc[mt][0], 0, 0, 0);
                 // The next k-step's weights, spread evenly over this k-step's MFMAs (an MFMA hides about
@@ -426,45 +492,122 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
         }
     }
 
-    // ---- store.  The weights are the MFMA's first operand, so an accumulator tile is indexed
-    // [weight row][token]: value v of a lane belongs to token lane%32 and weight row
-    // 8*(v/4) + 4*(lane/32) + v%4 of the tile, four consecutive outputs of one token per v/4, one
-    // 16-byte store.  Undo the activation-row and weight-row scales. ----
-    const float* rs = reinterpret_cast<const float*>(a.ws + W.rs);
-    const float* wd = reinterpret_cast<const float*>(a.ws + W.wdown);
-    const bool vec_ok = a.n % 4 == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;  // uniform
+    store_tile<MT, NT>(a, W, acc, m0 + wm * (32 * MT), n0 + wn * (32 * NT), l32, lg);
+}
+
+// One workgroup tile of Q8_0 weights (34-byte blocks: f16 d, 32 int8), four waves side by side, each
+// 256 tokens x 32 weight rows.  A stage is 64 k = two blocks of a row; lane group lg = lane/32 takes
+// block 2*st + lg whole, so its fragments of k-step ks are bytes 8*ks.. of the block and the
+// activation chunk is 4*lg + ks.  The blocks are only 2-byte aligned: a lane whose blocks start at
+// 4n reads the eight words of int8 from 4n (two bytes early) plus the two bytes that follow them,
+// and shifts by two bytes when it forms a word (v_alignbyte); a lane whose blocks start at 4n + 2
+// reads them from 4n + 4, aligned, and shifts by zero.  Since a stage advances every lane by 68
+// bytes, a lane keeps its case.  w = d * q = d * ((q ^ 0x80) - 128) in fp32 (exact), one rounding
+// to f16.
+template <int MT, int WN>
+__device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
+    static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
+    const Workspace W = workspace_layout(a.m, a.n, a.k);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const uint32_t l32 = lane & 31u, lg = lane >> 5;
+    const uint32_t nstages = a.k / BK;  // even (k % 128 == 0)
+    ActTile at;
+    at.init(a, W, m0, lane, wave);
+
+    uint32_t gn = n0 + wn * 32 + l32;
+    gn = gn < a.n ? gn : a.n - 1u;
+    const uint8_t* blk0 = a.w + (size_t)gn * (a.k / 32) * Q8_0_BYTES + lg * Q8_0_BYTES;  // this lane's block of stage 0
+    const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[gn];
+    const bool early = (reinterpret_cast<uintptr_t>(blk0) & 2u) == 0;  // blocks at 4n: the int8 start two bytes into a word
+    const uint32_t shift = early ? 2u : 0u;
+    const uint8_t* win0 = early ? blk0 : blk0 + 2;                     // first of the eight aligned words
+    // raw registers of a stage's block: d, eight words, and (early lanes) the two bytes behind them
+    struct Raw { uint32_t d; uint4 lo, hi; uint32_t tail; };
+    Raw braw[2];
+    auto load_b = [&](uint32_t st, int slot) {
+        const size_t off = (size_t)st * (2 * Q8_0_BYTES);
+        braw[slot].d = *reinterpret_cast<const uint16_t*>(blk0 + off);
+        braw[slot].lo = ld16_unaligned(win0 + off);  // 4-byte aligned
+        braw[slot].hi = ld16_unaligned(win0 + off + 16);
+        // late lanes do not use it: they re-read their d, which is always inside the buffer
+        braw[slot].tail = *reinterpret_cast<const uint16_t*>(early ? win0 + off + 32 : blk0 + off);
+    };
+
+    f32x16_t acc[MT][1];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const uint32_t gnb = n0 + wn * (32 * NT) + nt * 32 + 4 * lg;
-        float wup[16];  // 2^e of the 16 weight rows, from their 2^-e
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            uint32_t gn = gnb + 8 * (v >> 2) + (v & 3);
-            gn = gn < a.n ? gn : a.n - 1u;
-            wup[v] = __uint_as_float(0x7f000000u - __float_as_uint(wd[gn]));
-        }
+        for (int v = 0; v < 16; ++v) acc[i][0][v] = 0.f;
+
+    constexpr int kSteps = 4 * MT;  // MFMA steps per stage: k-step t / MT, row tile t % MT
+    constexpr int PD = 3;           // steps an activation fragment is requested ahead
+    static_assert(MT % 4 == 0 && kSteps >= DMA_PER_WAVE, "four eighths per k-step, spread over the MT steps");
+
+    load_b(0, 0);
+    at.fetch_all(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    for (uint32_t st2 = 0; st2 < nstages; st2 += 2) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const uint32_t gm = m0 + wm * (32 * MT) + mt * 32 + l32;
-            if (gm >= a.m) continue;
-            const float rsv = rs[gm];
-            float* yp = a.y + (size_t)gm * a.n + gnb;
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const float o0 = acc[mt][nt][4 * g] * (rsv * wup[4 * g]), o1 = acc[mt][nt][4 * g + 1] * (rsv * wup[4 * g + 1]);
-                const float o2 = acc[mt][nt][4 * g + 2] * (rsv * wup[4 * g + 2]), o3 = acc[mt][nt][4 * g + 3] * (rsv * wup[4 * g + 3]);
-                const uint32_t gn = gnb + 8 * g;
-                if (vec_ok) {
-                    if (gn < a.n) *reinterpret_cast<float4*>(yp + 8 * g) = make_float4(o0, o1, o2, o3);
-                } else {
-                    if (gn < a.n) yp[8 * g] = o0;
-                    if (gn + 1 < a.n) yp[8 * g + 1] = o1;
-                    if (gn + 2 < a.n) yp[8 * g + 2] = o2;
-                    if (gn + 3 < a.n) yp[8 * g + 3] = o3;
+        for (int c = 0; c < 2; ++c) {
+            const uint32_t st = st2 + c;
+            const uint32_t buf = c;
+            // This stage's block, requested a stage ago.  It is claimed here, before this stage's
+            // activation fetches are issued: the compiler does not know about those, and the wait it
+            // puts in front of the first use of these registers would otherwise cover them too.
+            Raw cur = braw[c];
+            asm volatile("" : "+v"(cur.d), "+v"(cur.tail), "+v"(cur.lo.x), "+v"(cur.lo.y), "+v"(cur.lo.z), "+v"(cur.lo.w),
+                         "+v"(cur.hi.x), "+v"(cur.hi.y), "+v"(cur.hi.z), "+v"(cur.hi.w));
+            const bool has_next = st + 1 < nstages;  // uniform
+            if (has_next) load_b(st + 1, c ^ 1);
+            const float dsc = f16_bits_to_f32(cur.d & 0xffffu) * wdown, ndm = -128.f * dsc;
+            const uint32_t dw[9] = {cur.lo.x, cur.lo.y, cur.lo.z, cur.lo.w, cur.hi.x, cur.hi.y, cur.hi.z, cur.hi.w, cur.tail};
+            // Eighth e of k-step ks: two weights -> fragment word e.  Word 2*ks + e/2 of the block's int8
+            // is formed (and its sign bits flipped) once and kept for its second eighth.
+            uint32_t uw[2];
+            auto b_eighth = [&](int ks, int e, uint4& bfw) {
+                const int q = e >> 1, part = e & 1, i = 2 * ks + q;
+                if (part == 0) {
+                    uint32_t u = __builtin_amdgcn_alignbyte(dw[i + 1], dw[i], shift) ^ 0x80808080u;
+                    // opaque, so that the conversions stay v_cvt_f32_ubyte0..3 of this one register
+                    asm volatile("" : "+v"(u));
+                    uw[q] = u;
                 }
+                const uint32_t u = uw[q];
+                const f32x2_t v = {fmaf(part ? ubyte2(u) : ubyte0(u), dsc, ndm), fmaf(part ? ubyte3(u) : ubyte1(u), dsc, ndm)};
+                const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+                (e == 0 ? bfw.x : e == 1 ? bfw.y : e == 2 ? bfw.z : bfw.w) = r;
+            };
+            auto a_frag = [&](int t) -> uint4 {
+                return at.frag(buf, wm * (32 * MT) + (t % MT) * 32 + l32, 4u * lg + (t / MT));
+            };
+            uint4 bfc, bfn;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b_eighth(0, e, bfc);
+            uint4 af[PD + 1];
+#pragma unroll
+            for (int t = 0; t < PD; ++t) af[t] = a_frag(t);
+#pragma unroll
+            for (int t = 0; t < kSteps; ++t) {
+                const int ks = t / MT, mt = t % MT;
+                if (t + PD < kSteps) af[(t + PD) % (PD + 1)] = a_frag(t + PD);
+                // next stage's activations into the other buffer (free since the barrier that ended the
+                // previous stage), one fetch per step
+                if (t < DMA_PER_WAVE && has_next) at.fetch(st + 1, buf ^ 1u, t);
+                acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(bfc), as_frag(af[t % (PD + 1)]), acc[mt][0], 0, 0, 0);
+                if (ks < 3 && mt % (MT / 4) == 0) b_eighth(ks + 1, mt / (MT / 4), bfn);
+                __builtin_amdgcn_sched_barrier(0);
+                if (mt == MT - 1) bfc = bfn;
             }
+            // The next stage's activations must have landed before anyone reads them; they are the
+            // youngest vector memory operations of this wave and such operations complete in order.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
         }
     }
+    store_tile<MT, 1>(a, W, acc, m0 + wm * (32 * MT), n0 + wn * 32, l32, lg);
 }
 
 // Tile order: workgroups go to the 8 XCDs round-robin and every XCD has its own L2, so workgroup i
@@ -492,22 +635,50 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_kernel(GemmArgs a, uin
     }
 }
 
+__global__ __launch_bounds__(64 * WAVES, 2) void q80_gemm_kernel(GemmArgs a) {
+    const uint32_t tiles_m = (a.m + BM - 1) / BM;
+    uint32_t m0, n0;
+    if (!tile_of(blockIdx.x, tiles_m, (a.n + BN_WIDE - 1) / BN_WIDE, BN_WIDE, m0, n0)) return;
+    q80_gemm_tile<8, 4>(a, m0, n0);
+}
+
 }  // namespace
 
-size_t gemm_q4k_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) { return workspace_layout(m, n, k).total; }
+size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) { return workspace_layout(m, n, k).total; }
 
-int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
-                    uint32_t k, void* workspace) {
-    uint8_t* ws = static_cast<uint8_t*>(workspace);
-    const uint8_t* wb = static_cast<const uint8_t*>(w);
+template <int TYPE>
+static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, uint8_t* ws, uint32_t m,
+                       uint32_t n, uint32_t k) {
     const dim3 prep_grid(m + (n + 15u) / 16u);
     if (xdt == HQ_BF16)
-        hipLaunchKernelGGL(q4k_prep_kernel<true>, prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k);
+        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k);
     else
-        hipLaunchKernelGGL(q4k_prep_kernel<false>, prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k);
-    if (int rc = check_launch("q4k gemm pre-pass launch")) return rc;
-    GemmArgs a{ws, static_cast<const uint8_t*>(w), y, m, n, k};
-    constexpr int lds = 2 * BM * ROW * 2;
+        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k);
+    return check_launch("tile gemm pre-pass launch");
+}
+
+bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {
+    return (t == HQ_Q4_K && k % 256 == 0) || (t == HQ_Q8_0 && k % 128 == 0);
+}
+
+int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
+                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace) {
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const uint8_t* wb = static_cast<const uint8_t*>(w);
+    GemmArgs a{ws, wb, y, m, n, k};
+    constexpr int lds = 2 * ActTile::kTile;
+    const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
+    const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
+    if (t == HQ_Q8_0) {
+        if (int rc = launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k)) return rc;
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q80_gemm_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                               "hipFuncSetAttribute(q8_0 gemm LDS)"))
+            return rc;
+        hipLaunchKernelGGL(q80_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
+        return check_launch("q8_0 gemm kernel launch");
+    }
+    if (int rc = launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k)) return rc;
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_gemm_kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                            "hipFuncSetAttribute(q4k gemm LDS)"))
@@ -517,11 +688,9 @@ int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* 
     // no gain, the narrow tiles pay the double dequantisation.)
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
-    const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     const uint32_t cols_narrowed = (uint64_t)tiles_m * cols_wide <= cus / 2 ? cols_wide : 0;  // columns cut in two
     const uint32_t n_wide = (cols_wide - cols_narrowed) * BN_WIDE;  // < n whenever cols_narrowed > 0
     const uint32_t cols_narrow = n_wide < n ? (n - n_wide + BN_NARROW - 1) / BN_NARROW : 0;
-    const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
     const uint32_t grid_wide = pad_m * (cols_wide - cols_narrowed), grid_narrow = pad_m * cols_narrow;
     hipLaunchKernelGGL(q4k_gemm_kernel, dim3(grid_wide + grid_narrow), dim3(64 * WAVES), lds, s, a, n_wide, grid_wide);
     return check_launch("q4k gemm kernel launch");

@@ -49,11 +49,12 @@ int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_ac
 bool gemm_supported(hq_ggml_type t, uint32_t k);
 int launch_gemm(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                 uint32_t k, hq_ggml_type t);
-// Q4_K GEMM on the f16 matrix cores with an activation pre-pass; needs k % 256 == 0 and a device
-// workspace of gemm_q4k_workspace_bytes().
-size_t gemm_q4k_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
-int launch_gemm_q4k(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
-                    uint32_t k, void* workspace);
+// GEMM on the f16 matrix cores with an activation pre-pass (Q4_K with k % 256 == 0, Q8_0 with
+// k % 128 == 0); needs a device workspace of gemm_f16_tile_workspace_bytes().
+bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k);
+size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
+                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace);
 
 // MoE glue (moe.hip)
 int launch_dense_gemv_bf16(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,

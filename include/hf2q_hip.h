@@ -84,16 +84,17 @@ HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, ui
  * (src/inference/models/qwen35/gpu_ffn.rs:1236-1245; dispatch_qmatmul,
  * src/serve/forward_mlx.rs:9655-9969).  m <= 8 takes the bandwidth-bound GEMV
  * kernels, m > 8 the MFMA GEMM (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791);
- * the Q4_K GEMM multiplies f16-rounded weights and activations like the
- * reference's mul_mm, the other kernels keep every product exact.
+ * the Q4_K (k % 256 == 0) and Q8_0 (k % 128 == 0) GEMMs multiply f16-rounded
+ * weights and activations like the reference's mul_mm, the other kernels keep
+ * every product exact.
  * Requires k % block_elems == 0; Q4_K needs a 16-byte aligned `w_blocks`,
  * Q6_K / Q8_0 a 2-byte aligned one. */
 HQ_API int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y,
                     uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t);
 
-/* The same product with caller-owned device scratch.  The Q4_K tile kernel
- * (m > 8, k % 256 == 0) converts the activations to row-scaled f16 in a
- * pre-pass and needs hq_qmatmul_ggml_workspace_bytes() bytes (256-byte
+/* The same product with caller-owned device scratch.  The f16 tile kernels
+ * (m > 8; Q4_K with k % 256 == 0, Q8_0 with k % 128 == 0) convert the
+ * activations to row-scaled f16 in a pre-pass and needs hq_qmatmul_ggml_workspace_bytes() bytes (256-byte
  * aligned) for them; every other shape needs none (the function returns 0 and
  * `workspace` may be null).  hq_qmatmul_ggml itself takes that scratch from the
  * stream-ordered allocator (hipMallocAsync / hipFreeAsync on `stream`).  The
