@@ -48,7 +48,7 @@ def parse():
                     help="decode_gemv = BASELINE config 2 (the default and the headline metric); the others are "
                          "configs 3, 4 and 5, each printing its own JSON line")
     ap.add_argument("--tokens", type=int, default=1, help="moe_decode: tokens per step (1 or 8)")
-    ap.add_argument("--wtype", default="q4_k", choices=["q4_k", "q8_0"], help="prefill_gemm: weight type")
+    ap.add_argument("--wtype", default="q4_k", choices=["q4_k", "q8_0", "q6_k"], help="prefill_gemm: weight type")
     ap.add_argument("--weight-sets", type=int, default=4, help="distinct FFN weight sets rotated per step")
     ap.add_argument("--no-graph", action="store_true",
                     help="moe_decode / tq_attention: launch every kernel from the host instead of replaying a HIP "
@@ -220,7 +220,7 @@ def bench_prefill_gemm(a):
 
     dev = torch.device("cuda:0")
     M, K, N = 2048, 4096, 12288
-    t = HQ_Q4_K if a.wtype == "q4_k" else HQ_Q8_0
+    t = {"q4_k": HQ_Q4_K, "q8_0": HQ_Q8_0, "q6_k": ops.HQ_Q6_K}[a.wtype]
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     w = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, t)

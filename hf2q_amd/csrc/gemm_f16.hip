@@ -1,4 +1,4 @@
-// Batched-prefill GEMM for Q4_K and Q8_0 weights (m > 8): y[m,n] = x[m,k] . W[n,k]^T on the
+// Batched-prefill GEMM for Q4_K, Q6_K and Q8_0 weights (m > 8): y[m,n] = x[m,k] . W[n,k]^T on the
 // f16 matrix cores (v_mfma_f32_32x32x16_f16) with fp32 accumulation.
 //
 // Numerics.  The weight tile holds the dequantised weights rounded to f16, which
@@ -84,8 +84,8 @@ __device__ __forceinline__ uint32_t f16_bits(float v) {
 
 // Pre-pass.  Workgroups [0, m): one per activation row, row scale and f16 conversion.  Workgroups
 // from m on: 16 weight rows each, 16 lanes per row over the row's block headers.  Per weight row, a
-// power of two that brings the row's largest possible |w| (Q4_K: |d|*63*15 + |dmin|*63, Q8_0:
-// |d|*128) to about 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
+// power of two that brings the row's largest possible |w| (Q4_K: |d|*63*15 + |dmin|*63, Q6_K:
+// |d|*128*32, Q8_0: |d|*128) to about 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
 // subnormals; the main kernel multiplies the weights by it before they are rounded (exact) and its
 // epilogue divides it out.
 template <bool X_BF16, int TYPE>
@@ -104,6 +104,13 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
                 const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow + (size_t)sb * Q4K_BYTES);
                 const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * 945.f + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
                 bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;  // inf / nan scales do not set the exponent
+            }
+        } else if constexpr (TYPE == HQ_Q6_K) {  // |w| <= |d| * 128 * 32
+            const uint32_t nsb = k / 256;
+            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nsb * Q6K_BYTES;
+            for (uint32_t sb = tid & 15u; sb < nsb; sb += 16u) {
+                const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)sb * Q6K_BYTES + 208))) * 4096.f;
+                bound = v <= 3.0e38f ? fmaxf(bound, v) : bound;
             }
         } else {  // Q8_0: |w| <= |d| * 128
             const uint32_t nb = k / 32;
@@ -610,6 +617,134 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     store_tile<MT, 1>(a, W, acc, m0 + wm * (32 * MT), n0 + wn * 32, l32, lg);
 }
 
+// One workgroup tile of Q6_K weights (210-byte super-blocks: ql[128], qh[64], int8 scales[16], f16
+// d), four waves side by side, each 256 tokens x 32 weight rows.  A 128-element half h of a
+// super-block is two stages that read the same bytes: elements 128h + 32*g + l (g = 0..3, l < 32)
+// are nibble g/2 of ql[64h + 32*(g%2) + l] with bits 2g, 2g+1 of qh[32h + l] on top, scale
+// 8h + 2g + l/16.  Stage s' = g/2 (low nibbles, then high), lane group lg = g%2: a lane fetches its 32
+// ql bytes, the half's 32 qh bytes, eight scale bytes and d once per half, a half ahead.
+// w = d*sc*(q - 32) in fp32 (d*sc exact), one rounding to f16.  The blocks are 2-byte aligned; the
+// hardware takes the unaligned 16-byte loads.
+template <int MT, int WN>
+__device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
+    static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
+    const Workspace W = workspace_layout(a.m, a.n, a.k);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const uint32_t l32 = lane & 31u, lg = lane >> 5;
+    const uint32_t nsb = a.k / 256, nstages = a.k / BK;
+    ActTile at;
+    at.init(a, W, m0, lane, wave);
+
+    uint32_t gn = n0 + wn * 32 + l32;
+    gn = gn < a.n ? gn : a.n - 1u;
+    const uint8_t* wrow = a.w + (size_t)gn * nsb * Q6K_BYTES;
+    const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[gn];
+    struct Raw { uint4 l0, l1, h0, h1; uint2 sc; uint32_t d; };  // one half of a super-block, this lane's share
+    Raw braw[2];
+    auto load_half = [&](uint32_t sb, int h, int slot) {
+        const uint8_t* blk = wrow + (size_t)sb * Q6K_BYTES;
+        braw[slot].l0 = ld16_unaligned(blk + 64 * h + 32 * lg);
+        braw[slot].l1 = ld16_unaligned(blk + 64 * h + 32 * lg + 16);
+        braw[slot].h0 = ld16_unaligned(blk + 128 + 32 * h);
+        braw[slot].h1 = ld16_unaligned(blk + 128 + 32 * h + 16);
+        braw[slot].sc = ld8_unaligned(blk + 192 + 8 * h);
+        braw[slot].d = ld2(blk + 208);
+    };
+
+    f32x16_t acc[MT][1];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][0][v] = 0.f;
+
+    constexpr int kSteps = 4 * MT;  // MFMA steps per stage: k-step t / MT, row tile t % MT
+    constexpr int PD = 3;           // steps an activation fragment is requested ahead
+    static_assert(MT % 4 == 0 && kSteps >= DMA_PER_WAVE, "four eighths per k-step, spread over the MT steps");
+
+    load_half(0, 0, 0);
+    at.fetch_all(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    for (uint32_t sb = 0; sb < nsb; ++sb) {
+        const bool next_sb = sb + 1 < nsb;  // uniform
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int h = c >> 1, hi = c & 1;  // half of the super-block; low / high nibbles
+            const uint32_t st = 4 * sb + c;
+            const uint32_t buf = c & 1;
+            // This half's bytes, requested a half ago.  They are claimed at the start of the half, before
+            // its activation fetches are issued: the compiler does not know about those, and the wait it
+            // puts in front of the first use of these registers would otherwise cover them too.
+            Raw& cur = braw[h];
+            if (hi == 0) {
+                asm volatile("" : "+v"(cur.l0.x), "+v"(cur.l0.y), "+v"(cur.l0.z), "+v"(cur.l0.w), "+v"(cur.l1.x), "+v"(cur.l1.y),
+                             "+v"(cur.l1.z), "+v"(cur.l1.w), "+v"(cur.h0.x), "+v"(cur.h0.y), "+v"(cur.h0.z), "+v"(cur.h0.w),
+                             "+v"(cur.h1.x), "+v"(cur.h1.y), "+v"(cur.h1.z), "+v"(cur.h1.w), "+v"(cur.sc.x), "+v"(cur.sc.y),
+                             "+v"(cur.d));
+                if (h == 0) {
+                    load_half(sb, 1, 1);
+                } else if (next_sb) {
+                    load_half(sb + 1, 0, 0);
+                }
+            }
+            const bool has_next = st + 1 < nstages;  // uniform
+            // the lane's two scales of this stage: bytes 4*hi + 2*lg, +1 of the half's eight
+            const uint32_t scw = (hi ? cur.sc.y : cur.sc.x) >> (16 * lg);
+            const float dw = f16_bits_to_f32(cur.d & 0xffffu) * wdown;
+            const float dsc0 = dw * (float)(int)(int8_t)(scw & 0xffu), dsc1 = dw * (float)(int)(int8_t)((scw >> 8) & 0xffu);
+            const uint32_t lw[8] = {cur.l0.x, cur.l0.y, cur.l0.z, cur.l0.w, cur.l1.x, cur.l1.y, cur.l1.z, cur.l1.w};
+            const uint32_t hw[8] = {cur.h0.x, cur.h0.y, cur.h0.z, cur.h0.w, cur.h1.x, cur.h1.y, cur.h1.z, cur.h1.w};
+            const uint32_t hshift = 4 * hi + 2 * lg;
+            // Eighth e of k-step ks: two weights -> fragment word e.  Word 2*ks + e/2 of the lane's 6-bit
+            // values is assembled once and kept for its second eighth.
+            uint32_t uw[2];
+            auto b_eighth = [&](int ks, int e, uint4& bfw) {
+                const int q = e >> 1, part = e & 1, i = 2 * ks + q;
+                if (part == 0) {
+                    const uint32_t nib = (hi ? lw[i] >> 4 : lw[i]) & 0x0f0f0f0fu;
+                    uint32_t u = (((hw[i] >> hshift) & 0x03030303u) << 4) | nib;
+                    // opaque, so that the conversions stay v_cvt_f32_ubyte0..3 of this one register
+                    asm volatile("" : "+v"(u));
+                    uw[q] = u;
+                }
+                const uint32_t u = uw[q];
+                const float dsc = ks < 2 ? dsc0 : dsc1, ndm = -32.f * dsc;  // elements 8*ks.. of 32: scale ks / 2
+                const f32x2_t v = {fmaf(part ? ubyte2(u) : ubyte0(u), dsc, ndm), fmaf(part ? ubyte3(u) : ubyte1(u), dsc, ndm)};
+                const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+                (e == 0 ? bfw.x : e == 1 ? bfw.y : e == 2 ? bfw.z : bfw.w) = r;
+            };
+            auto a_frag = [&](int t) -> uint4 {
+                return at.frag(buf, wm * (32 * MT) + (t % MT) * 32 + l32, 4u * lg + (t / MT));
+            };
+            uint4 bfc, bfn;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b_eighth(0, e, bfc);
+            uint4 af[PD + 1];
+#pragma unroll
+            for (int t = 0; t < PD; ++t) af[t] = a_frag(t);
+#pragma unroll
+            for (int t = 0; t < kSteps; ++t) {
+                const int ks = t / MT, mt = t % MT;
+                if (t + PD < kSteps) af[(t + PD) % (PD + 1)] = a_frag(t + PD);
+                // next stage's activations into the other buffer (free since the barrier that ended the
+                // previous stage), one fetch per step
+                if (t < DMA_PER_WAVE && has_next) at.fetch(st + 1, buf ^ 1u, t);
+                acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_frag(bfc), as_frag(af[t % (PD + 1)]), acc[mt][0], 0, 0, 0);
+                if (ks < 3 && mt % (MT / 4) == 0) b_eighth(ks + 1, mt / (MT / 4), bfn);
+                __builtin_amdgcn_sched_barrier(0);
+                if (mt == MT - 1) bfc = bfn;
+            }
+            // The next stage's activations must have landed before anyone reads them; they are the
+            // youngest vector memory operations of this wave and such operations complete in order.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+    }
+    store_tile<MT, 1>(a, W, acc, m0 + wm * (32 * MT), n0 + wn * 32, l32, lg);
+}
+
 // Tile order: workgroups go to the 8 XCDs round-robin and every XCD has its own L2, so workgroup i
 // runs on XCD i % 8.  Each XCD gets whole rows of tiles (one activation tile, which then stays in
 // that XCD's L2) and sweeps the weight tiles.  The grid is padded to 8 * ceil(tiles_m / 8) * tiles_n.
@@ -635,6 +770,13 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_kernel(GemmArgs a, uin
     }
 }
 
+__global__ __launch_bounds__(64 * WAVES, 2) void q6k_gemm_kernel(GemmArgs a) {
+    const uint32_t tiles_m = (a.m + BM - 1) / BM;
+    uint32_t m0, n0;
+    if (!tile_of(blockIdx.x, tiles_m, (a.n + BN_WIDE - 1) / BN_WIDE, BN_WIDE, m0, n0)) return;
+    q6k_gemm_tile<8, 4>(a, m0, n0);
+}
+
 __global__ __launch_bounds__(64 * WAVES, 2) void q80_gemm_kernel(GemmArgs a) {
     const uint32_t tiles_m = (a.m + BM - 1) / BM;
     uint32_t m0, n0;
@@ -658,7 +800,7 @@ static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uin
 }
 
 bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {
-    return (t == HQ_Q4_K && k % 256 == 0) || (t == HQ_Q8_0 && k % 128 == 0);
+    return ((t == HQ_Q4_K || t == HQ_Q6_K) && k % 256 == 0) || (t == HQ_Q8_0 && k % 128 == 0);
 }
 
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
@@ -669,6 +811,15 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     constexpr int lds = 2 * ActTile::kTile;
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
+    if (t == HQ_Q6_K) {
+        if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k)) return rc;
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q6k_gemm_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                               "hipFuncSetAttribute(q6_k gemm LDS)"))
+            return rc;
+        hipLaunchKernelGGL(q6k_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
+        return check_launch("q6_k gemm kernel launch");
+    }
     if (t == HQ_Q8_0) {
         if (int rc = launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k)) return rc;
         if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q80_gemm_kernel),

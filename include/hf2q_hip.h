@@ -84,7 +84,7 @@ HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, ui
  * (src/inference/models/qwen35/gpu_ffn.rs:1236-1245; dispatch_qmatmul,
  * src/serve/forward_mlx.rs:9655-9969).  m <= 8 takes the bandwidth-bound GEMV
  * kernels, m > 8 the MFMA GEMM (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791);
- * the Q4_K (k % 256 == 0) and Q8_0 (k % 128 == 0) GEMMs multiply f16-rounded
+ * the Q4_K / Q6_K (k % 256 == 0) and Q8_0 (k % 128 == 0) GEMMs multiply f16-rounded
  * weights and activations like the reference's mul_mm, the other kernels keep
  * every product exact.
  * Requires k % block_elems == 0; Q4_K needs a 16-byte aligned `w_blocks`,
@@ -93,7 +93,7 @@ HQ_API int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const 
                     uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t);
 
 /* The same product with caller-owned device scratch.  The f16 tile kernels
- * (m > 8; Q4_K with k % 256 == 0, Q8_0 with k % 128 == 0) convert the
+ * (m > 8; Q4_K / Q6_K with k % 256 == 0, Q8_0 with k % 128 == 0) convert the
  * activations to row-scaled f16 in a pre-pass and needs hq_qmatmul_ggml_workspace_bytes() bytes (256-byte
  * aligned) for them; every other shape needs none (the function returns 0 and
  * `workspace` may be null).  hq_qmatmul_ggml itself takes that scratch from the

@@ -10,11 +10,11 @@ from hf2q_amd.ops import HQ_Q4_K, HQ_Q6_K, HQ_Q8_0, GgmlQuantizedMatmulParams
 pytestmark = pytest.mark.gpu
 
 def _f16_tile(t, k):
-    return (t == HQ_Q4_K and k % 256 == 0) or (t == HQ_Q8_0 and k % 128 == 0)
+    return (t in (HQ_Q4_K, HQ_Q6_K) and k % 256 == 0) or (t == HQ_Q8_0 and k % 128 == 0)
 
 
 def _check(t, k):
-    """Q4_K with k % 256 == 0 and Q8_0 with k % 128 == 0 take the f16 tile kernels; everything else
+    """Q4_K / Q6_K (k % 256 == 0) and Q8_0 with k % 128 == 0 take the f16 tile kernels; everything else
     keeps every product exact."""
     return assert_matmul_close_f16_tile if _f16_tile(t, k) else assert_matmul_close
 
@@ -50,20 +50,20 @@ def test_gemm_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
     _check(t, k)(y, ref, f"gemm t={t} {xdt} {m}x{n}x{k}")
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K])
 def test_gemm_adversarial_blocks(oracle, dev, t):
     """Every scale / min / nibble bit pattern (raw random bytes with finite f16 fields)."""
     m, n, k = 40, 128, 512
     bb = oracle.BLOCK_BYTES[t]
     raw = np.random.default_rng(9).integers(0, 256, size=n * k // oracle.BLOCK_ELEMS[t] * bb, dtype=np.uint8)
-    for off in ([1, 3] if t == HQ_Q4_K else [1]):
+    for off in ([1, 3] if t == HQ_Q4_K else [209] if t == HQ_Q6_K else [1]):
         raw[off::bb] &= 0x3F
     for xdt in ("bf16", "f32"):
         y, ref = _run(oracle, dev, t, xdt, m, n, k, blocks=raw)
         _check(t, k)(y, ref, f"gemm adversarial t={t} {xdt}")
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K])
 def test_gemm_rows_equal_gemv_rows(oracle, dev, t):
     """Row i of the m>8 result agrees with the m=1 GEMV of activation row i; the tile kernels round
     their weights to f16, so the agreement is to 1e-3 of the row's largest output."""
@@ -104,7 +104,7 @@ def test_q4k_tile_gemm_workspace_variant(oracle, dev):
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(1, n, k, HQ_Q4_K), torch.bfloat16) == 0
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q8_0), torch.bfloat16) >= m * k * 2
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, 320, HQ_Q8_0), torch.bfloat16) == 0
-    assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q6_K), torch.bfloat16) == 0
+    assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q6_K), torch.bfloat16) >= m * k * 2
     y0 = torch.empty(m, n, device=dev)
     y1 = torch.empty(m, n, device=dev)
     ops.quantized_matmul_ggml(x, wd, y0, p)
@@ -115,7 +115,7 @@ def test_q4k_tile_gemm_workspace_variant(oracle, dev):
         ops.quantized_matmul_ggml(x, wd, y1, p, workspace=ws[: need - 256])
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 def test_tile_gemm_scale_equivariance(oracle, dev, xdt, t):
     """Activation rows and weight rows are rescaled by powers of two inside the kernel (f16 has a narrow
