@@ -37,6 +37,12 @@ class QmatmulJob(_c.Structure):
                 ("k", _c.c_uint32), ("n_experts", _c.c_uint32), ("expert_stride", _c.c_uint64)]
 
 
+class GgufTensorInfo(_c.Structure):
+    """hq_gguf_tensor_info of include/hf2q_hip.h, field for field."""
+    _fields_ = [("ggml_type", _c.c_uint32), ("n_dims", _c.c_uint32), ("dims", _c.c_uint64 * 4),
+                ("data_offset", _c.c_uint64), ("byte_len", _c.c_uint64)]
+
+
 # name -> (restype, argtypes); the single source for the symbol-export test.
 SIGNATURES = {
     "hq_last_error": (_c.c_char_p, []),
@@ -61,6 +67,19 @@ SIGNATURES = {
     "hq_tq_encode_kv": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
     "hq_flash_attn_vec_tq": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "hq_flash_attn_vec_tq_tmp_bytes": (_sz, [_u32, _u32, _u32]),
+    "hq_gguf_open": (_i32, [_c.c_char_p, _c.POINTER(_vp)]),
+    "hq_gguf_close": (None, [_vp]),
+    "hq_gguf_tensor_count": (_u64, [_vp]),
+    "hq_gguf_metadata_count": (_u64, [_vp]),
+    "hq_gguf_alignment": (_u64, [_vp]),
+    "hq_gguf_tensor_name": (_c.c_char_p, [_vp, _u64]),
+    "hq_gguf_metadata_key": (_c.c_char_p, [_vp, _u64]),
+    "hq_gguf_tensor_info_by_name": (_i32, [_vp, _c.c_char_p, _c.POINTER(GgufTensorInfo)]),
+    "hq_gguf_metadata_u64": (_i32, [_vp, _c.c_char_p, _c.POINTER(_u64)]),
+    "hq_gguf_metadata_f64": (_i32, [_vp, _c.c_char_p, _c.POINTER(_c.c_double)]),
+    "hq_gguf_metadata_string": (_i32, [_vp, _c.c_char_p, _c.POINTER(_vp), _c.POINTER(_u64)]),
+    "hq_gguf_tensor_data": (_vp, [_vp, _c.c_char_p, _c.POINTER(_u64)]),
+    "hq_gguf_load_tensor": (_i32, [_vp, _c.c_char_p, _vp, _vp, _sz]),
 }
 
 

@@ -10,6 +10,8 @@ all arithmetic happens in libhf2q_hip.so through its C ABI.
 """
 from __future__ import annotations
 
+import ctypes
+import os
 from dataclasses import dataclass
 
 import torch
@@ -170,6 +172,107 @@ def quantize_ggml(src: torch.Tensor, n_per_row: int, ggml_type: int) -> torch.Te
     L = _l.load()
     _l.check(L.hq_quantize_ggml(_stream(), _dev(src, "src"), n, n_per_row, ggml_type, _dev(out, "out")))
     return out
+
+
+# ---- GGUF files ------------------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class QuantWeightInfo:
+    """forward_mlx.rs:395-415 (MlxQWeight.info): what the matmul call sites need to know about a loaded
+    tensor.  `shape` is in GGUF order (innermost first)."""
+    ggml_dtype: int
+    rows: int
+    cols: int
+    shape: tuple
+    byte_len: int
+
+
+class GgufFile:
+    """The reader hf2q opens its model files with (mlx_native::gguf::GgufFile as used in
+    serve/gpu.rs:157-167 and qwen35/weight_loader.rs:52-118): tensor directory, metadata, and the raw
+    GGML blocks of a tensor uploaded to the device."""
+
+    def __init__(self, path: str):
+        h = ctypes.c_void_p()
+        _l.check(_l.load().hq_gguf_open(os.fsencode(path), ctypes.byref(h)))
+        self._h = h
+
+    @classmethod
+    def open(cls, path: str) -> "GgufFile":
+        return cls(path)
+
+    def close(self) -> None:
+        if self._h:
+            _l.load().hq_gguf_close(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def tensor_count(self) -> int:
+        return _l.load().hq_gguf_tensor_count(self._h)
+
+    def metadata_count(self) -> int:
+        return _l.load().hq_gguf_metadata_count(self._h)
+
+    def tensor_names(self) -> list:
+        L = _l.load()
+        return [L.hq_gguf_tensor_name(self._h, i).decode() for i in range(self.tensor_count())]
+
+    def metadata_keys(self) -> list:
+        L = _l.load()
+        return [L.hq_gguf_metadata_key(self._h, i).decode() for i in range(self.metadata_count())]
+
+    def tensor_info(self, name: str) -> QuantWeightInfo:
+        ti = _l.GgufTensorInfo()
+        _l.check(_l.load().hq_gguf_tensor_info_by_name(self._h, name.encode(), ctypes.byref(ti)))
+        shape = tuple(ti.dims[i] for i in range(ti.n_dims))
+        cols = shape[0] if shape else 1
+        rows = 1
+        for d in shape[1:]:
+            rows *= d
+        return QuantWeightInfo(ti.ggml_type, rows, cols, shape, ti.byte_len)
+
+    def metadata_u64(self, key: str) -> int:
+        v = ctypes.c_uint64()
+        _l.check(_l.load().hq_gguf_metadata_u64(self._h, key.encode(), ctypes.byref(v)))
+        return v.value
+
+    def metadata_f64(self, key: str) -> float:
+        v = ctypes.c_double()
+        _l.check(_l.load().hq_gguf_metadata_f64(self._h, key.encode(), ctypes.byref(v)))
+        return v.value
+
+    def metadata_string(self, key: str) -> str:
+        p, n = ctypes.c_void_p(), ctypes.c_uint64()
+        _l.check(_l.load().hq_gguf_metadata_string(self._h, key.encode(), ctypes.byref(p), ctypes.byref(n)))
+        return ctypes.string_at(p.value, n.value).decode()
+
+    def tensor_bytes(self, name: str) -> bytes:
+        """The tensor's raw bytes from the host mapping (tests, CPU-side consumers)."""
+        n = ctypes.c_uint64()
+        p = _l.load().hq_gguf_tensor_data(self._h, name.encode(), ctypes.byref(n))
+        if not p:
+            raise _l.HqError(_l.HQ_ERR_INVALID_ARGUMENT, _l.last_error())
+        return ctypes.string_at(p, n.value)
+
+    def load_tensor(self, name: str, device) -> torch.Tensor:
+        """Raw GGML blocks of `name` as a uint8 device tensor (weight_loader.rs:52-118); the matmul entry
+        points take it as is.  For an expert stack, expert_stride = byte_len // shape[2]."""
+        info = self.tensor_info(name)
+        buf = torch.empty(info.byte_len, dtype=torch.uint8, device=device)
+        with torch.cuda.device(buf.device):
+            _l.check(_l.load().hq_gguf_load_tensor(self._h, name.encode(), _stream(), _dev(buf, name), info.byte_len))
+        return buf
 
 
 # ---- TurboQuant-style 8-bit KV cache ------------------------------------------------------------

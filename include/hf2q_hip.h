@@ -235,6 +235,40 @@ HQ_API int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_c
                          void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p);
 HQ_API size_t hq_flash_attn_vec_tq_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len);
 
+/* ---- GGUF reader (weights as hf2q loads them) ---- */
+
+/* Replaces mlx_native::gguf::GgufFile as hf2q uses it at load time
+ * (src/serve/gpu.rs:157-167, src/inference/models/qwen35/weight_loader.rs:52-118):
+ * open, tensor_info(name) -> {ggml_type, shape, byte_len}, load_tensor(name, device) -> the
+ * tensor's raw GGML blocks in a device buffer, metadata lookups.  The byte format is the one
+ * hf2q's own writer emits (src/backends/gguf/types.rs:20-32, 96-188; writer.rs:171-258).
+ * dims are in GGUF order (innermost first: dims[0] = k, dims[1] = n, dims[2] = experts); an expert
+ * stack is one contiguous tensor and expert_stride = byte_len / dims[2]
+ * (src/serve/forward_mlx.rs:2438-2460).  data_offset is absolute in the file. */
+typedef struct hq_gguf hq_gguf;
+typedef struct hq_gguf_tensor_info {
+    uint32_t ggml_type, n_dims;
+    uint64_t dims[4];
+    uint64_t data_offset, byte_len;
+} hq_gguf_tensor_info;
+HQ_API int hq_gguf_open(const char* path, hq_gguf** out);
+HQ_API void hq_gguf_close(hq_gguf* g);
+HQ_API uint64_t hq_gguf_tensor_count(const hq_gguf* g);
+HQ_API uint64_t hq_gguf_metadata_count(const hq_gguf* g);
+HQ_API uint64_t hq_gguf_alignment(const hq_gguf* g);
+HQ_API const char* hq_gguf_tensor_name(const hq_gguf* g, uint64_t index);   /* NULL past the end */
+HQ_API const char* hq_gguf_metadata_key(const hq_gguf* g, uint64_t index);  /* NULL past the end */
+HQ_API int hq_gguf_tensor_info_by_name(const hq_gguf* g, const char* name, hq_gguf_tensor_info* out);
+/* Integer and bool values widened to u64 (negative: error); f32 / f64 widened to double; strings
+ * are returned as pointer + length into the mapping (not NUL-terminated). */
+HQ_API int hq_gguf_metadata_u64(const hq_gguf* g, const char* key, uint64_t* out);
+HQ_API int hq_gguf_metadata_f64(const hq_gguf* g, const char* key, double* out);
+HQ_API int hq_gguf_metadata_string(const hq_gguf* g, const char* key, const char** out, uint64_t* len);
+/* The tensor's bytes in the host mapping (valid until hq_gguf_close), NULL if there is no such tensor. */
+HQ_API const void* hq_gguf_tensor_data(const hq_gguf* g, const char* name, uint64_t* byte_len);
+/* Copies the tensor's raw bytes to `dev_dst` (at least byte_len bytes) on `stream` and waits for it. */
+HQ_API int hq_gguf_load_tensor(const hq_gguf* g, const char* name, void* stream, void* dev_dst, size_t dst_bytes);
+
 #ifdef __cplusplus
 }
 #endif
