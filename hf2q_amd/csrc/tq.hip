@@ -409,6 +409,369 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     }
 }
 
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+
+// x of the lane eight places round its row of 16 (lanes j and j ^ 8 exchange).
+__device__ __forceinline__ float row_xor8(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+}
+
+// The same split for linear int8 codes with BOTH products on the f16 matrix cores.
+//
+// A code byte c becomes the f16 number 1152 + c without arithmetic: the byte with its sign bit flipped
+// (c + 128, unsigned) placed under the f16 bit pattern of 1024 (0x6400 | u = 1024 + u, exact for
+// u < 1024) by one v_perm_b32 against a register that holds the 0x64.  Odd elements of the reduction
+// dimension take the opposite sign instead: the byte xor 0x7f is 127 - c, and under 0xe4 that is
+// -(1024 + 127 - c) = c - 1151.  The constants are taken out again as a correction,
+// q . (k + off) - sum(off_i q_i) for the scores and sum p (v + off) - sum(off_t p_t) for the output
+// with off = +1152, -1151, +1152, ...; because the signs alternate, the constant part of the running
+// sums stays near zero for smooth operands (a query with a large mean, evenly spread attention)
+// instead of eating accumulator bits.
+//
+// Queries and weights enter as f16 hi + lo pairs (22 bits); products are exact in the MFMA and
+// accumulate in fp32.  A chunk has at most 8 heads and the MFMA has 16 rows / columns, so the hi
+// parts take rows / columns 0..7 and the lo parts 8..15 of the SAME instruction: lane j < 8 stands
+// for the hi part of head j, lane j >= 8 for the lo part of head j - 8.
+//
+// f16 has a narrow exponent range, so both are normalised first: a head's query by the power of two
+// that brings its largest magnitude into [512, 1024); the weights p * norm_v by their own running
+// maximum, i.e. the kernel keeps two running maxima per head, m of the scores s (for the denominator
+// l = sum e^(s - m)) and mv of s + ln norm_v (for the numerator, whose weights e^(s + ln norm_v - mv)
+// * 2^14 then lie in [0, 2^14]).
+//
+// Tiles are 32 positions per wave.  Scores: two 16-position halves, MFMA 16x16x32 with the K codes
+// as rows (lane (j, g): position j, 16 code bytes at 64i + 16g for i = 0..3) and the queries as
+// columns, so lane (j, g) receives, after adding its partner j ^ 8, the scores of head j % 8 for
+// positions 4g..4g+3 of each half: eight positions, which are exactly one k-group of the second
+// product.  P.V: the weights of those eight positions are the lane's A fragment as they stand; the B
+// fragment of output coordinate 16n + 4i + e is byte 4i + e of the eight V rows that lane (n, g)
+// fetched for the same eight positions (16 bytes each), gathered two at a time by v_perm_b32.  16
+// accumulators (i, e) of 4 registers hold row 4g + v (head (4g + v) % 8, hi or lo part), coordinate
+// 16n + 4i + e.
+//
+// Cache offsets are 32-bit here: the launcher takes this kernel only below 4 GiB per code tensor.
+template <bool RING>
+__global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
+    // s_o: per wave and row, the 256 coordinates in the order [i][j][e] (coordinate 16j + 4i + e), so
+    // that a wave's stores are contiguous.  The fused rotation stages the queries in the same memory.
+    __shared__ __align__(16) float s_o[4][16][HD];
+    __shared__ uint4 s_qf[16][33];             // scaled queries as f16, 8 values per entry; rows 0..7 hi, 8..15 lo
+    __shared__ float s_corr[16], s_unscale[8];  // sum(off_i q_i) of a row; 2^e that undoes a head's scaling
+    __shared__ float s_m[4][8], s_l[4][8];
+    float(*s_q)[HD] = reinterpret_cast<float(*)[HD]>(&s_o[0][0][0]);
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t n_chunks = (a.group + 7u) / 8u;
+    const uint32_t kvh = blockIdx.y / n_chunks, hc = blockIdx.y % n_chunks;
+    const uint32_t h0 = kvh * a.group + hc * 8u;
+    const uint32_t nh = min(8u, a.group - hc * 8u);
+    const uint32_t split = blockIdx.x;
+    const uint32_t j = lane & 15u, g = lane >> 4;
+    const uint32_t head_base = kvh * a.kv_capacity;
+    const uint32_t split_first = a.first + split * (a.tiles_per_wave * 64u);
+    const uint32_t split_end = min(a.last, split_first + a.tiles_per_wave * 64u);
+    const uint32_t n_iter = (a.tiles_per_wave + 1u) / 2u;  // 128 positions per workgroup and iteration
+
+    struct Tile {
+        uint4 k[2][4];  // half, i: code bytes 64i + 16g .. +15 of position j
+        uint4 v[8];     // positions 4g..4g+3 of half 0, then of half 1; coordinates 16j..
+        float kn[2];    // norm_k of position j, -1 where the position is past the end
+        float vn[2];    // norm_v, 0 where the position is past the end
+    };
+    // Cache row of logical position idx; positions past the end of the split read a valid row and get
+    // weight 0.  RING: rows start at ring_start and wrap (ring_start, idx < kv_capacity); otherwise
+    // row = position.
+    const uint32_t last_row = max(split_end, a.first + 1u) - 1u;
+    auto row_of = [&](uint32_t idx) -> uint32_t {
+        const uint32_t i = min(idx, last_row);
+        if constexpr (!RING) return i;
+        const uint32_t sl = a.ring_start + i;
+        return sl >= a.kv_capacity ? sl - a.kv_capacity : sl;
+    };
+    const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto load_tile = [&](uint32_t it, Tile& t) {
+        const uint32_t tile0 = split_first + (it * 4u + wave_u) * 32u;  // wave-uniform
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const uint32_t idx = tile0 + 16u * hf + j;
+            const bool ok = idx < split_end;
+            const uint32_t row = head_base + row_of(idx);
+            const uint4* kp = reinterpret_cast<const uint4*>(a.k_codes + (row * (uint32_t)HD + 16u * g));
+            t.k[hf][0] = kp[0], t.k[hf][1] = kp[4], t.k[hf][2] = kp[8], t.k[hf][3] = kp[12];
+            t.kn[hf] = ok ? a.k_norms[row] : -1.f;
+            t.vn[hf] = ok ? a.v_norms[row] : 0.f;
+        }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const uint32_t vi = tile0 + (q < 4 ? 4u * g + q : 16u + 4u * g + (q - 4));
+            const uint32_t row = head_base + row_of(vi);
+            t.v[q] = *reinterpret_cast<const uint4*>(a.v_codes + (row * (uint32_t)HD + 16u * j));
+        }
+    };
+
+    // Everything the first two iterations need is requested before anything else: at the usual context
+    // lengths that is all of the wave's share, and its trip from HBM overlaps the staging of the queries.
+    Tile tile_a, tile_b;
+    load_tile(0, tile_a);
+    if (n_iter > 1) load_tile(1, tile_b);
+
+    // ---- queries: scaled per head, split into f16 hi + lo; thread = head tid/32, chunk tid%32 of 8
+    // values; rows are padded to 33 chunks against bank conflicts ----
+    {
+        const uint32_t h = tid >> 5, ch = tid & 31u;
+        float x[8];
+        if (a.fuse_fwht_pre) {  // sign x FWHT in LDS first
+            for (uint32_t i = tid; i < 8 * HD / 4; i += 256) {
+                const uint32_t hh = i / (HD / 4), c = i % (HD / 4);
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (hh < nh) v = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + hh) * HD)[c];
+                reinterpret_cast<float4*>(&s_q[hh][0])[c] = v;
+            }
+            __syncthreads();
+            for (uint32_t hh = wave; hh < 8; hh += 4) {
+                float4* p = reinterpret_cast<float4*>(&s_q[hh][0]) + lane;
+                const float4 t = *p;
+                float v[4] = {t.x, t.y, t.z, t.w};
+                apply_signs(v, lane);
+                fwht256(v, lane);
+                *p = make_float4(v[0], v[1], v[2], v[3]);
+            }
+            __syncthreads();
+            const float4 v0 = *reinterpret_cast<const float4*>(&s_q[h][8 * ch]), v1 = *reinterpret_cast<const float4*>(&s_q[h][8 * ch + 4]);
+            x[0] = v0.x, x[1] = v0.y, x[2] = v0.z, x[3] = v0.w, x[4] = v1.x, x[5] = v1.y, x[6] = v1.z, x[7] = v1.w;
+        } else {
+            float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
+            if (h < nh) {
+                const float4* qp = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + h) * HD + 8 * ch);
+                v0 = qp[0], v1 = qp[1];
+            }
+            x[0] = v0.x, x[1] = v0.y, x[2] = v0.z, x[3] = v0.w, x[4] = v1.x, x[5] = v1.y, x[6] = v1.z, x[7] = v1.w;
+        }
+        float amax = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float ax = fabsf(x[e]);
+            amax = ax <= 3.0e38f ? fmaxf(amax, ax) : amax;
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));  // the 32 threads of a head
+        // amax = f * 2^ex with f in [0.5, 1): scaling by 2^(10 - ex) brings it into [512, 1024)
+        int sh = amax > 0.f ? 10 - __builtin_amdgcn_frexp_expf(amax) : 0;
+        sh = sh < -100 ? -100 : sh > 100 ? 100 : sh;
+        const float scl = __builtin_amdgcn_ldexpf(1.f, sh);
+        uint32_t hi[8], lo[8];
+        float sum_hi = 0.f, sum_lo = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float xs = x[e] * scl;
+            const _Float16 fh = (_Float16)xs;
+            const _Float16 fl = (_Float16)(xs - (float)fh);
+            hi[e] = __builtin_bit_cast(unsigned short, fh);
+            lo[e] = __builtin_bit_cast(unsigned short, fl);
+            sum_hi += ((e & 1) ? -1151.f : 1152.f) * (float)fh;
+            sum_lo += ((e & 1) ? -1151.f : 1152.f) * (float)fl;
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) {
+            sum_hi += __shfl_xor(sum_hi, o);
+            sum_lo += __shfl_xor(sum_lo, o);
+        }
+        if (a.fuse_fwht_pre) __syncthreads();  // s_q is read, its memory may be written again
+        s_qf[h][ch] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16));
+        s_qf[8 + h][ch] = make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16));
+        if (ch == 0) {
+            s_corr[h] = sum_hi;
+            s_corr[8 + h] = sum_lo;
+            s_unscale[h] = __builtin_amdgcn_ldexpf(1.f, -sh);
+        }
+    }
+    __syncthreads();
+    // MFMA step kk = 2i + w takes words 2w, 2w + 1 of K load i: coordinates 64i + 16g + 8w .. +7
+    uint4 qf[8];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) qf[kk] = s_qf[j][8u * (kk >> 1) + 2u * g + (kk & 1)];
+    const float corr = s_corr[j];
+    const float sscale = s_unscale[j & 7u] * a.scale;
+    const bool lo_lane = j >= 8u;
+
+    const uint32_t magic = 0x0000e464u;
+    // two bytes of one word -> two f16 (1024 + byte, -(1024 + byte)): bytes 0, 1 with sel 0x05010400; 2, 3 with 0x05030402
+    auto pair_of = [&](uint32_t w, uint32_t sel) -> uint32_t { return __builtin_amdgcn_perm(magic, w, sel); };
+    // byte e of two words -> two f16 (1024 + byte of wa, -(1024 + byte of wb))
+    auto gather2 = [&](uint32_t wa, uint32_t wb, int e) -> uint32_t {
+        return __builtin_amdgcn_perm(wb, wa, 0x0c000c00u | (uint32_t)e | ((uint32_t)(4 + e) << 16)) | 0xe4006400u;
+    };
+
+    // of head j % 8: m, mv running maxima; l partial over this lane's positions; of row j: lp = sum(off_t p_t)
+    // over the row's weights (hi or lo parts), partial likewise
+    float m_run = -INFINITY, mv_run = -INFINITY, l_run = 0.f, lp_run = 0.f;
+    f32x4_t acc[4][4];  // [i][e][v]: row 4g + v, coordinate 16j + 4i + e
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[i][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    constexpr float LOG2E = 1.4426950408889634f;
+
+    auto attend = [&](const Tile& cur) {
+        // -------- scores: two independent accumulation chains per half --------
+        float s[8], lv[8];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            f32x4_t c0 = {0.f, 0.f, 0.f, 0.f}, c1 = c0;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const uint4 kq = cur.k[hf][kk >> 1];
+                const uint32_t u0 = ((kk & 1) ? kq.z : kq.x) ^ 0x7f807f80u, u1 = ((kk & 1) ? kq.w : kq.y) ^ 0x7f807f80u;
+                const uint4 fr = make_uint4(pair_of(u0, 0x05010400u), pair_of(u0, 0x05030402u), pair_of(u1, 0x05010400u),
+                                            pair_of(u1, 0x05030402u));
+                const f16x8_t af = __builtin_bit_cast(f16x8_t, fr);
+                if (kk & 1)
+                    c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8_t, qf[kk]), c1, 0, 0, 0);
+                else
+                    c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8_t, qf[kk]), c0, 0, 0, 0);
+            }
+            // c0 + c1 = (hi or lo part of q[head j % 8]) . (K[position 4g + v] + off); the norms of those
+            // positions sit in lanes 4g + v
+            const float lvn_own = __log2f(cur.vn[hf]);  // log 0 = -inf: no weight in the numerator
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int src = 4 * g + v;
+                const float nk = __shfl(cur.kn[hf], src);
+                lv[4 * hf + v] = __shfl(lvn_own, src);
+                const float part = (c0[v] + c1[v]) - corr;
+                const float x = (part + row_xor8(part)) * (sscale * nk);
+                s[4 * hf + v] = nk >= 0.f ? x : -INFINITY;
+            }
+        }
+        if (a.softcap != 0.f) {
+            // cap * tanh(x / cap), tanh y = 1 - 2 / (e^2y + 1)
+            const float inv = 2.f * LOG2E / a.softcap;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const float e2 = __builtin_amdgcn_exp2f(fminf(s[v] * inv, 80.f));
+                s[v] = s[v] == -INFINITY ? -INFINITY : a.softcap * (1.f - __fdividef(2.f, e2 + 1.f));
+            }
+        }
+        // the exponent domain is base 2 from here: s2 = s log2 e, t2 = s2 + log2 norm_v
+        float t[8], smax = -INFINITY, tmax = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            s[v] *= LOG2E;
+            t[v] = s[v] + lv[v];
+            smax = fmaxf(smax, s[v]);
+            tmax = fmaxf(tmax, t[v]);
+        }
+        smax = wave_max4(smax);
+        tmax = wave_max4(tmax);
+        const float m_new = fmaxf(m_run, smax), mv_new = fmaxf(mv_run, tmax);
+        // nothing accumulated yet (running maximum -inf): any factor will do, 1 spares the rescaling below
+        const float alpha = m_run == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
+        const float alpha_v = mv_run == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(mv_run - mv_new);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;           // -inf - (-inf) would be NaN
+        const float mv_use = (mv_new == -INFINITY ? 0.f : mv_new) - 14.f;  // weights scaled by 2^14
+        float psum = 0.f, ppsum = 0.f;
+        uint32_t pb[8];
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            psum += __builtin_amdgcn_exp2f(s[v] - m_use);
+            const float pp = __builtin_amdgcn_exp2f(t[v] - mv_use);
+            const _Float16 fh = (_Float16)pp;
+            const _Float16 mine = (_Float16)(lo_lane ? pp - (float)fh : pp);
+            pb[v] = __builtin_bit_cast(unsigned short, mine);
+            ppsum += ((v & 1) ? -1151.f : 1152.f) * (float)mine;
+        }
+        l_run = l_run * alpha + psum;
+        lp_run = lp_run * alpha_v + ppsum;
+        m_run = m_new;
+        mv_run = mv_new;
+        const f16x8_t pf = __builtin_bit_cast(f16x8_t, make_uint4(pb[0] | (pb[1] << 16), pb[2] | (pb[3] << 16), pb[4] | (pb[5] << 16), pb[6] | (pb[7] << 16)));
+        // -------- P.V --------
+        if (__builtin_amdgcn_ballot_w64(alpha_v != 1.f) != 0) {  // rare once the maximum has settled
+            float al[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) al[v] = __shfl(alpha_v, 4 * g + v);  // lane 4g + v stands for row 4g + v
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[i][e][v] *= al[v];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t vw[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const uint4 vq = cur.v[q];
+                vw[q] = (i == 0 ? vq.x : i == 1 ? vq.y : i == 2 ? vq.z : vq.w) ^ ((q & 1) ? 0x7f7f7f7fu : 0x80808080u);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint4 fr = make_uint4(gather2(vw[0], vw[1], e), gather2(vw[2], vw[3], e), gather2(vw[4], vw[5], e),
+                                            gather2(vw[6], vw[7], e));
+                acc[i][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pf, __builtin_bit_cast(f16x8_t, fr), acc[i][e], 0, 0, 0);
+            }
+        }
+    };
+    for (uint32_t it = 0; it < n_iter; ++it) {
+        attend(tile_a);
+        if (it + 1 < n_iter) tile_a = tile_b;
+        if (it + 2 < n_iter) load_tile(it + 2, tile_b);
+    }
+
+    // ---- merge of the four waves.  First the maxima, so that every wave can bring its own numbers to
+    // the workgroup's scale before they meet: O_row = (acc - lp) * 2^(mv - m_wg) / 2^14, l * 2^(m - m_wg).
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    lp_run += __shfl_xor(lp_run, 16);
+    lp_run += __shfl_xor(lp_run, 32);
+    if (lane < 8u) s_m[wave][lane] = m_run;
+    __syncthreads();
+    const uint32_t hj = j & 7u;
+    const float m_wg = fmaxf(fmaxf(s_m[0][hj], s_m[1][hj]), fmaxf(s_m[2][hj], s_m[3][hj]));
+    const float fo_own = mv_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mv_run - m_wg - 14.f);
+    if (lane < 8u) s_l[wave][lane] = m_run == -INFINITY ? 0.f : l_run * __builtin_amdgcn_exp2f(m_run - m_wg);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const float lpv = __shfl(lp_run, 4 * g + v), fo = __shfl(fo_own, 4 * g + v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 o = make_float4((acc[i][0][v] - lpv) * fo, (acc[i][1][v] - lpv) * fo, (acc[i][2][v] - lpv) * fo,
+                                         (acc[i][3][v] - lpv) * fo);
+            *reinterpret_cast<float4*>(&s_o[wave][4 * g + v][64 * i + 4 * j]) = o;
+        }
+    }
+    __syncthreads();
+    {
+        // thread = head tid / 32, eight consecutive stored values: i = c8 / 8, j = 2 (c8 % 8) and the next, e = 0..3
+        const uint32_t h = tid >> 5, c8 = tid & 31u;
+        if (h < nh) {
+            float4 o0 = make_float4(0.f, 0.f, 0.f, 0.f), o1 = o0;
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+#pragma unroll
+                for (int part = 0; part < 2; ++part) {
+                    const float4 x0 = *reinterpret_cast<const float4*>(&s_o[w][h + 8 * part][8 * c8]);
+                    const float4 x1 = *reinterpret_cast<const float4*>(&s_o[w][h + 8 * part][8 * c8 + 4]);
+                    o0.x += x0.x, o0.y += x0.y, o0.z += x0.z, o0.w += x0.w;
+                    o1.x += x1.x, o1.y += x1.y, o1.z += x1.z, o1.w += x1.w;
+                }
+            float* out = a.tmp + ((size_t)(h0 + h) * a.n_splits + split) * TMP_STRIDE;
+            const uint32_t ci = c8 >> 3, cj = 2u * (c8 & 7u);
+            float* o_at = out + 16u * cj + 4u * ci;  // TMP_STRIDE is even, not a multiple of 4: 8-byte stores
+            reinterpret_cast<float2*>(o_at)[0] = make_float2(o0.x, o0.y);
+            reinterpret_cast<float2*>(o_at)[1] = make_float2(o0.z, o0.w);
+            reinterpret_cast<float2*>(o_at + 16)[0] = make_float2(o1.x, o1.y);
+            reinterpret_cast<float2*>(o_at + 16)[1] = make_float2(o1.z, o1.w);
+            if (c8 == 0) {
+                const float m = fmaxf(fmaxf(s_m[0][h], s_m[1][h]), fmaxf(s_m[2][h], s_m[3][h]));
+                out[HD] = m * (1.f / LOG2E);  // the merge kernel works with natural exponents
+                out[HD + 1] = (s_l[0][h] + s_l[1][h]) + (s_l[2][h] + s_l[3][h]);
+            }
+        }
+    }
+}
+
 // out[h][d] = sum_s e^{m_s - m} O_s[d] / sum_s e^{m_s - m} l_s.  Grid (num_heads, 4): a workgroup
 // owns 64 output coordinates of one head; its 4 waves take a quarter of the splits each, with
 // the loads of 8 splits in flight at a time.
@@ -522,8 +885,14 @@ int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, c
     a.lut_mul = 1.f / (16.f * (p.head_dim == 512 ? p.scale_factor_d512 : 1.f));
     a.fuse_fwht_pre = p.fuse_fwht_pre;
     const dim3 grid(a.n_splits, p.num_kv_heads * ((a.group + 7u) / 8u));
+    // the f16 kernel indexes the code tensors with 32-bit byte offsets
+    const bool small = (uint64_t)p.num_kv_heads * p.kv_capacity * HD <= 0xffffffffull;
     if (lut)
         hipLaunchKernelGGL(tq_attn_split_kernel<true>, grid, dim3(256), 0, s, a);
+    else if (small && p.ring_start == 0)
+        hipLaunchKernelGGL(tq_attn_split_f16_kernel<false>, grid, dim3(256), 0, s, a);
+    else if (small)
+        hipLaunchKernelGGL(tq_attn_split_f16_kernel<true>, grid, dim3(256), 0, s, a);
     else
         hipLaunchKernelGGL(tq_attn_split_kernel<false>, grid, dim3(256), 0, s, a);
     if (int rc = check_launch("tq attention kernel launch")) return rc;

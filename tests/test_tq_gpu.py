@@ -101,6 +101,53 @@ def test_attention_matches_f64_oracle(oracle, dev, nh, nkv, n, cap, kw):
     _assert_attn_close(_attend(dev, q, kc, kn, vc, vn, p), ref, f"attn {nh}/{nkv} n={n} {kw}")
 
 
+def _raw_cache(rng, nkv, cap, hd, norm_lo, norm_hi, log_uniform=False):
+    codes = rng.integers(-127, 128, (nkv, cap, hd)).astype(np.int8).view(np.uint8)
+    if log_uniform:
+        norms = np.exp(rng.uniform(np.log(norm_lo), np.log(norm_hi), (nkv, cap, 1)))
+    else:
+        norms = rng.uniform(norm_lo, norm_hi, (nkv, cap, 1))
+    return codes, norms.astype(np.float32)
+
+
+@pytest.mark.parametrize("case", ["q_large_mean", "q_tiny", "q_huge", "v_norm_range", "v_norm_zeros", "even_attention",
+                                  "peaked", "extreme_codes"])
+def test_attention_adversarial_operands(oracle, dev, case):
+    """Operands that stress the kernel's internal number formats (scaled half-precision operands with a
+    constant offset on the codes): a query far from zero mean, queries of very small and very large magnitude, value
+    norms over many orders of magnitude or zero, evenly spread and sharply peaked attention, codes at
+    the ends of their range.  Same bar as the random cases."""
+    hd, nh, nkv, n, cap = 256, 16, 2, 1500, 1536
+    rng = np.random.default_rng(sum(case.encode()))
+    kc, kn = _raw_cache(rng, nkv, cap, hd, 0.005, 0.02)
+    vc, vn = _raw_cache(rng, nkv, cap, hd, 0.005, 0.02)
+    q = rng.standard_normal((nh, hd)).astype(np.float32)
+    if case == "q_large_mean":
+        q = (3.0 + 0.1 * q).astype(np.float32)
+    elif case == "q_tiny":
+        q = (q * np.logspace(-30, -3, nh)[:, None]).astype(np.float32)
+    elif case == "q_huge":
+        q = (q * np.float32(1e20)).astype(np.float32)
+        kn = (kn * np.float32(1e-20)).astype(np.float32)
+    elif case == "v_norm_range":
+        vc, vn = _raw_cache(rng, nkv, cap, hd, 1e-12, 1e6, log_uniform=True)
+    elif case == "v_norm_zeros":
+        vn[:, ::3] = 0.0
+        vn[:, 700:900] = 0.0
+    elif case == "even_attention":
+        q = (q * np.float32(1e-4)).astype(np.float32)
+    elif case == "peaked":
+        kn[:, 611] = 0.3
+        q[:8] = kc[0, 611].view(np.int8).astype(np.float32) / 40
+        q[8:] = kc[1, 611].view(np.int8).astype(np.float32) / 40
+    elif case == "extreme_codes":
+        kc = rng.choice(np.array([-128, -127, 127], np.int8), (nkv, cap, hd)).view(np.uint8)
+        vc = rng.choice(np.array([-128, 127], np.int8), (nkv, cap, hd)).view(np.uint8)
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 1.0 / 16.0)
+    ref = oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, hd, n, cap, p.scale)
+    _assert_attn_close(_attend(dev, q, kc, kn, vc, vn, p), ref, case)
+
+
 def test_attention_lut_form(oracle, dev):
     hd, nh, nkv, n, cap = 256, 16, 2, 200, 256
     rng = np.random.default_rng(8)
