@@ -117,24 +117,47 @@ def _events(n):
     return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
 
 
-def _graphed(a, step, n_variants):
-    """Capture step(i) for i < n_variants into HIP graphs (one each) and return a replay function; the
-    capture replays exactly the launches step() makes.  No memset nodes are involved: the library only
-    launches kernels."""
+def _timed_steps(a, step, n_variants):
+    """Exactly a.steps calls of step(i) between two synchronisations; returns (wall seconds, device
+    microseconds per step from one HIP event pair around the whole region).  Unless --no-graph, the steps
+    are replayed from HIP graphs the way a decode loop that records its token step runs them: one graph
+    holds a run of consecutive steps (every rotated variant in turn, at least 32 steps), replayed
+    steps // run times, and single-step graphs cover the remainder."""
     import torch
 
+    run = n_variants * max(1, -(-32 // n_variants))
+    q, r = (0, a.steps) if a.no_graph else divmod(a.steps, run)
     if a.no_graph:
-        return step
-    side = torch.cuda.Stream()
-    graphs = []
-    with torch.cuda.stream(side):
-        for i in range(n_variants):
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=side):
-                step(i)
-            graphs.append(g)
+        calls = [lambda i=i: step(a.warmup + i) for i in range(a.steps)]
+    else:
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            big = None
+            if q:
+                big = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(big, stream=side):
+                    for i in range(run):
+                        step(i)
+            singles = []
+            for i in range(min(r, n_variants)):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    step(i)
+                singles.append(g)
+        torch.cuda.synchronize()
+        calls = [big.replay] * q + [singles[i % n_variants].replay for i in range(r)]
+        for c in ([big.replay] if q else []) + [g.replay for g in singles]:  # untimed: first replay of each graph
+            c()
+    e0, e1 = _events(1)[0]
     torch.cuda.synchronize()
-    return lambda i: graphs[i % n_variants].replay()
+    t0 = time.perf_counter()
+    e0.record()
+    for c in calls:
+        c()
+    e1.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    return elapsed, e0.elapsed_time(e1) * 1e3 / a.steps
 
 
 def _finish(a, out):
@@ -179,21 +202,12 @@ def bench_moe_decode(a):
     for i in range(max(a.warmup, 1)):
         step(i)
     torch.cuda.synchronize()
-    step = _graphed(a, eager_step, n_layers)
+    elapsed, layer_us = _timed_steps(a, eager_step, n_layers)
     uniq = []
-    ev = _events(a.steps)
-    t0 = time.perf_counter()
-    for i in range(a.steps):
-        ev[i][0].record()
-        step(a.warmup + i)
-        ev[i][1].record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
     for i in range(min(a.steps, n_layers)):  # distinct experts actually routed (after the timed region)
         eager_step(i)
         uniq.append(int(torch.unique(scratch.ids[:T * K]).numel()))
     u = sum(uniq) / len(uniq)
-    layer_us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
     step_bytes = (u * 3 + 3) * expert_bytes + (E + 1) * H * 2  # routed + shared experts + router (bf16)
     gbs = step_bytes / layer_us / 1e3
     _finish(a, {
@@ -284,35 +298,37 @@ def bench_tq_attention(a):
     p = FlashAttnVecTqHbParams(nh, nkv, hd, n, n, 1.0 / 16.0)
     nbytes = sum(t.numel() * t.element_size() for t in caches[0])
 
-    def step(i):  # the reference's decode chain: rotate q, attend, rotate the output back
+    pf = FlashAttnVecTqHbParams(nh, nkv, hd, n, n, 1.0 / 16.0, fuse_fwht_pre=1)
+
+    def separate(i):  # the reference's decode chain as three dispatches: rotate q, attend, rotate the output back
         ops.dispatch_fwht_sign_premult_f32(q, nh, hd)
         ops.flash_attn_vec_tq_hb(q, *caches[i % n_caches], out, tmp, p)
         ops.dispatch_fwht_sign_undo_f32(out, nh, hd)
 
-    for i in range(max(a.warmup, 1)):
-        step(i)
-    torch.cuda.synchronize()
-    step = _graphed(a, step, n_caches)
-    ev = _events(a.steps)
-    t0 = time.perf_counter()
-    for i in range(a.steps):
-        ev[i][0].record()
-        step(a.warmup + i)
-        ev[i][1].record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
+    def fused(i):  # the same chain with both rotations inside the attention call (bit-identical result)
+        ops.flash_attn_vec_tq_hb(q, *caches[i % n_caches], out, tmp, pf, undo_rotation=True)
+
+    def timed(step):
+        for i in range(max(a.warmup, 1)):
+            step(i)
+        torch.cuda.synchronize()
+        return _timed_steps(a, step, n_caches)
+
+    _, us_sep = timed(separate)
+    elapsed, us = timed(fused)
     gbs = nbytes / us / 1e3
     _finish(a, {
         "metric": "TQ-KV decode attention eff. GB/s", "value": round(nbytes * a.steps / elapsed / 1e9, 1),
         "unit": "GB/s", "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f32",
         "config": {"workload": "tq_attention: 32768 context, 16 q heads / 2 kv heads, head_dim 256, int8 codes + f32 "
-                               "norm per (token, head), batch 1 (BASELINE config 5); one step = rotate q + attention "
-                               "(split + merge) + rotate output = 4 launches", "bytes_per_step": nbytes,
-                   "caches_rotated": n_caches},
-        "roofline": {"bound": "hbm", "kernel": "rotate + tq attention split + merge + rotate", "achieved": round(gbs, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "us_per_launch": round(us, 3), "bytes_per_launch": nbytes}})
+                               "norm per (token, head), batch 1 (BASELINE config 5); one step = rotate q, attend, rotate "
+                               "the output back, as one call = 2 launches (split with the q rotation, merge with the "
+                               "output rotation)", "bytes_per_step": nbytes, "caches_rotated": n_caches,
+                   "separate_dispatch": {"launches": 4, "us_per_step": round(us_sep, 3),
+                                         "GB/s": round(nbytes / us_sep / 1e3, 1)}},
+        "roofline": {"bound": "hbm", "kernel": "tq attention split (+ q rotation) + merge (+ output rotation)",
+                     "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "us_per_launch": round(us, 3), "bytes_per_launch": nbytes}})
 
 
 def main():
@@ -411,21 +427,13 @@ def main():
     host = {"ms_per_step": round(el_host / a.steps * 1e3, 4), "GBps": round(step_bytes * a.steps / el_host / 1e9, 1),
             "frac_hbm_peak": round(step_bytes * a.steps / el_host / 1e9 / HBM_PEAK_GBS, 4)}
 
-    # The timed region behind `value`: exactly K steps, each replayed from a HIP graph of its four
-    # launches (one graph per weight-set / head rotation), as a decode loop that records its step does;
-    # the host's per-launch cost (Python, ctypes) is then out of the way, like in the other workloads.
+    # The timed region behind `value`: exactly K steps replayed from HIP graphs of their three launches
+    # (runs of consecutive steps over the rotated weight sets and heads), as a decode loop that records
+    # its token step does; the host's per-launch cost (Python, ctypes) is then out of the way, like in
+    # the other workloads.
     elapsed = el_host
     if not a.no_graph:
-        n_var = n_sets * n_heads
-        replay = _graphed(a, fused_step, n_var)
-        for i in range(min(a.warmup, n_var)):
-            replay(i)
-        torch.cuda.synchronize()
-        t0g = time.perf_counter()
-        for i in range(a.steps):
-            replay(a.warmup + i)
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0g
+        elapsed, _ = _timed_steps(a, fused_step, n_sets * n_heads)
 
     names = ("gate", "up", "down", "head")
     kern_us = {nm: sum(evs[i][j][0].elapsed_time(evs[i][j][1]) for i in range(a.steps)) * 1e3 / a.steps

@@ -333,10 +333,9 @@ size_t hq_flash_attn_vec_tq_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uin
     return tq_attn_tmp_bytes(num_heads, head_dim, kv_seq_len);
 }
 
-int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
-                         const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
-                         void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p) {
-    const char* fn = "hq_flash_attn_vec_tq";
+static int flash_attn_vec_tq(const char* fn, bool undo_rotation, void* stream, const float* q, const uint8_t* k_codes,
+                             const float* k_norms, const uint8_t* v_codes, const float* v_norms, const float* lut256,
+                             float* out, void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p) {
     if (!p) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null params", fn);
     if (p->head_dim != 256 && p->head_dim != 512)
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: head_dim %u (256 or 512)", fn, p->head_dim);
@@ -363,7 +362,21 @@ int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, c
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: tmp holds %zu bytes, %zu needed", fn, tmp_bytes,
                     tq_attn_tmp_bytes(p->num_heads, p->head_dim, p->kv_seq_len));
     return launch_tq_attention((hipStream_t)stream, q, k_codes, k_norms, v_codes, v_norms, lut256, out,
-                               static_cast<float*>(tmp), *p);
+                               static_cast<float*>(tmp), *p, undo_rotation);
+}
+
+int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
+                         const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
+                         void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p) {
+    return flash_attn_vec_tq("hq_flash_attn_vec_tq", false, stream, q, k_codes, k_norms, v_codes, v_norms, lut256, out, tmp,
+                             tmp_bytes, p);
+}
+
+int hq_flash_attn_vec_tq_undo(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
+                              const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
+                              void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p) {
+    return flash_attn_vec_tq("hq_flash_attn_vec_tq_undo", true, stream, q, k_codes, k_norms, v_codes, v_norms, lut256, out,
+                             tmp, tmp_bytes, p);
 }
 
 int hq_dense_gemv_bf16(void* stream, const void* x, hq_act_dtype xdt, const void* w_bf16, float* y, uint32_t m,

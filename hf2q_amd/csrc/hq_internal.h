@@ -74,7 +74,7 @@ int launch_tq_encode(hipStream_t s, const float* src, uint8_t* codes, float* nor
 size_t tq_attn_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len);
 int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, const float* k_norms,
                         const uint8_t* v_codes, const float* v_norms, const float* lut, float* out, float* tmp,
-                        const hq_tq_attn_params& p);
+                        const hq_tq_attn_params& p, bool undo_rotation);
 
 }  // namespace hq
 

@@ -772,18 +772,34 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
     }
 }
 
-// out[h][d] = sum_s e^{m_s - m} O_s[d] / sum_s e^{m_s - m} l_s.  Grid (num_heads, 4): a workgroup
-// owns 64 output coordinates of one head; its 4 waves take a quarter of the splits each, with
-// the loads of 8 splits in flight at a time.
-__global__ __launch_bounds__(256) void tq_attn_reduce_kernel(const float* __restrict__ tmp, float* __restrict__ out,
-                                                             uint32_t n_splits) {
+// out[h][d] = sum_s e^{m_s - m} O_s[d] / sum_s e^{m_s - m} l_s, optionally followed by the inverse
+// rotation (FWHT, then signs) of the head's 256 coordinates.  One workgroup of 16 waves per head: a
+// wave takes a sixteenth of the splits, a lane four consecutive coordinates, so that at up to 128
+// splits every load of the kernel is in flight at once; wave 0 adds the partial sums, divides and
+// rotates.
+constexpr int MERGE_WAVES = 16;
+template <bool UNDO>
+__global__ __launch_bounds__(64 * MERGE_WAVES) void tq_attn_merge_kernel(const float* __restrict__ tmp, float* __restrict__ out,
+                                                                         uint32_t n_splits) {
     __shared__ float s_w[256];  // e^{m_s - m}
-    __shared__ float s_part[4][64];
-    __shared__ float s_red[4];
+    __shared__ __align__(16) float s_part[MERGE_WAVES][HD];
+    __shared__ float s_red[MERGE_WAVES];
     const uint32_t h = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t d = blockIdx.y * 64u + lane;
     const float* base = tmp + (size_t)h * n_splits * TMP_STRIDE;
-    // n_splits <= 256 = the workgroup size: one thread per split fetches its running maximum and sum
+    const uint32_t per = (n_splits + MERGE_WAVES - 1u) / MERGE_WAVES, s0 = min(n_splits, wave * per), s1 = min(n_splits, s0 + per);
+    constexpr int CH = 8;
+    // rows of tmp are 8-byte aligned (TMP_STRIDE is even): two float2 per lane and split
+    auto fetch = [&](uint32_t s, float2 (&v)[CH][2]) {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            const float2* row = reinterpret_cast<const float2*>(base + (size_t)min(s + i, n_splits - 1u) * TMP_STRIDE) + 2u * lane;
+            v[i][0] = row[0];
+            v[i][1] = row[1];
+        }
+    };
+    float2 v[CH][2];
+    fetch(s0, v);  // on their way while the weights are worked out
+    // n_splits <= 256: one thread per split fetches its running maximum and sum
     float ms = -INFINITY, ls = 0.f;
     if (tid < n_splits) {
         ms = base[(size_t)tid * TMP_STRIDE + HD];
@@ -794,29 +810,43 @@ __global__ __launch_bounds__(256) void tq_attn_reduce_kernel(const float* __rest
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
     if (lane == 0) s_red[wave] = m;
     __syncthreads();
-    m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));  // splits live in the first 256 threads
     const float w = ms == -INFINITY ? 0.f : __expf(ms - m);
-    s_w[tid] = w;
+    if (tid < 256u) s_w[tid] = w;
     float lw = w * ls;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
     __syncthreads();  // s_red read by everyone before it is reused; s_w visible
     if (lane == 0) s_red[wave] = lw;
-    float o = 0.f;
-    const uint32_t per = (n_splits + 3u) / 4u, s0 = wave * per, s1 = min(n_splits, s0 + per);
-    for (uint32_t s = s0; s < s1; s += 8) {
-        float v[8];
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t s = s0; s < s1; s += CH) {
+        if (s != s0) fetch(s, v);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = s + i < s1 ? base[(size_t)(s + i) * TMP_STRIDE + d] : 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o = fmaf(s + i < s1 ? s_w[s + i] : 0.f, v[i], o);
+        for (int i = 0; i < CH; ++i) {
+            const float ws = s + i < s1 ? s_w[s + i] : 0.f;
+            o[0] = fmaf(ws, v[i][0].x, o[0]);
+            o[1] = fmaf(ws, v[i][0].y, o[1]);
+            o[2] = fmaf(ws, v[i][1].x, o[2]);
+            o[3] = fmaf(ws, v[i][1].y, o[3]);
+        }
     }
-    s_part[wave][lane] = o;
+    *reinterpret_cast<float4*>(&s_part[wave][4 * lane]) = make_float4(o[0], o[1], o[2], o[3]);
     __syncthreads();
     if (wave == 0) {
-        const float l = s_red[0] + s_red[1] + s_red[2] + s_red[3];
-        const float t = s_part[0][lane] + s_part[1][lane] + s_part[2][lane] + s_part[3][lane];
-        out[(size_t)h * HD + d] = l > 0.f ? t / l : 0.f;
+        const float l = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+        float r[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w2 = 0; w2 < MERGE_WAVES; ++w2) {
+            const float4 t = *reinterpret_cast<const float4*>(&s_part[w2][4 * lane]);
+            r[0] += t.x, r[1] += t.y, r[2] += t.z, r[3] += t.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = l > 0.f ? r[e] / l : 0.f;
+        if constexpr (UNDO) {
+            fwht256(r, lane);
+            apply_signs(r, lane);
+        }
+        reinterpret_cast<float4*>(out + (size_t)h * HD)[lane] = make_float4(r[0], r[1], r[2], r[3]);
     }
 }
 
@@ -860,7 +890,7 @@ size_t tq_attn_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_
 
 int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, const float* k_norms,
                         const uint8_t* v_codes, const float* v_norms, const float* lut, float* out, float* tmp,
-                        const hq_tq_attn_params& p) {
+                        const hq_tq_attn_params& p, bool undo_rotation) {
     AttnArgs a{};
     a.q = q;
     a.k_codes = k_codes;
@@ -896,8 +926,11 @@ int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, c
     else
         hipLaunchKernelGGL(tq_attn_split_kernel<false>, grid, dim3(256), 0, s, a);
     if (int rc = check_launch("tq attention kernel launch")) return rc;
-    hipLaunchKernelGGL(tq_attn_reduce_kernel, dim3(p.num_heads, HD / 64), dim3(256), 0, s, tmp, out, a.n_splits);
-    return check_launch("tq attention reduce launch");
+    if (undo_rotation)
+        hipLaunchKernelGGL(tq_attn_merge_kernel<true>, dim3(p.num_heads), dim3(64 * MERGE_WAVES), 0, s, tmp, out, a.n_splits);
+    else
+        hipLaunchKernelGGL(tq_attn_merge_kernel<false>, dim3(p.num_heads), dim3(64 * MERGE_WAVES), 0, s, tmp, out, a.n_splits);
+    return check_launch("tq attention merge launch");
 }
 
 }  // namespace hq

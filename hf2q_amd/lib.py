@@ -66,6 +66,7 @@ SIGNATURES = {
     "hq_fwht_sign_undo_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_tq_encode_kv": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
     "hq_flash_attn_vec_tq": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "hq_flash_attn_vec_tq_undo": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "hq_flash_attn_vec_tq_tmp_bytes": (_sz, [_u32, _u32, _u32]),
     "hq_gguf_open": (_i32, [_c.c_char_p, _c.POINTER(_vp)]),
     "hq_gguf_close": (None, [_vp]),

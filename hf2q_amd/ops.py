@@ -333,8 +333,9 @@ def tq_tmp_buffer_bytes(num_heads: int, head_dim: int, kv_seq_len: int) -> int:
 
 def flash_attn_vec_tq_hb(q: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor, v_packed: torch.Tensor,
                          v_norms: torch.Tensor, out: torch.Tensor, tmp: torch.Tensor, params: FlashAttnVecTqHbParams,
-                         lut256: torch.Tensor | None = None) -> None:
-    """forward_mlx.rs:4732-4742: single-query attention over the 8-bit cache (rotated domain in and out)."""
+                         lut256: torch.Tensor | None = None, undo_rotation: bool = False) -> None:
+    """forward_mlx.rs:4732-4742: single-query attention over the 8-bit cache (rotated domain in and out).
+    undo_rotation: the merge pass also applies dispatch_fwht_sign_undo_f32 to `out` (forward_mlx.rs:4744-4760)."""
     if q.dtype != torch.float32 or out.dtype != torch.float32:
         raise TypeError("q and out must be float32")
     p = _l.TqAttnParams(params.num_heads, params.num_kv_heads, params.head_dim, params.kv_seq_len,
@@ -342,7 +343,8 @@ def flash_attn_vec_tq_hb(q: torch.Tensor, k_packed: torch.Tensor, k_norms: torch
                         params.ring_start, params.scale_factor_d512, params.codebook_bits, params.fuse_fwht_pre,
                         params.nsg)
     import ctypes as _ct
-    _l.check(_l.load().hq_flash_attn_vec_tq(
+    fn = _l.load().hq_flash_attn_vec_tq_undo if undo_rotation else _l.load().hq_flash_attn_vec_tq
+    _l.check(fn(
         _stream(), _dev(q, "q"), _dev(k_packed, "k_packed"), _dev(k_norms, "k_norms"), _dev(v_packed, "v_packed"),
         _dev(v_norms, "v_norms"), _dev(lut256, "lut256") if lut256 is not None else None, _dev(out, "out"),
         _dev(tmp, "tmp"), tmp.numel() * tmp.element_size(), _ct.byref(p)))

@@ -233,6 +233,13 @@ typedef struct {
 HQ_API int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
                          const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
                          void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p);
+/* The same attention with the inverse rotation applied to `out` by the merge pass: stands for the
+ * pair flash_attn_vec_tq_hb + dispatch_fwht_sign_undo_f32 that the decode path encodes back to back
+ * (forward_mlx.rs:4732-4760; gpu_full_attn.rs:186-294) and gives the bits that pair gives.  With
+ * fuse_fwht_pre = 1 the whole rotate - attend - rotate chain is this one call (two launches). */
+HQ_API int hq_flash_attn_vec_tq_undo(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
+                              const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
+                              void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p);
 HQ_API size_t hq_flash_attn_vec_tq_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len);
 
 /* ---- GGUF reader (weights as hf2q loads them) ---- */

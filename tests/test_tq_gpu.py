@@ -190,6 +190,34 @@ def test_fused_pre_rotation_equals_separate_dispatch(oracle, dev):
     assert np.array_equal(sep, fused)  # forward_mlx.rs:4646-4652: the fused path is bit-identical
 
 
+@pytest.mark.parametrize("n,cap,kw", [(300, 512, {}), (5000, 5000, {}), (512, 512, {"mask_type": 2, "sliding_window": 200, "ring_start": 31})])
+def test_fused_post_rotation_equals_separate_dispatch(oracle, dev, n, cap, kw):
+    """Attention whose merge pass applies the inverse rotation gives the bits of attention followed by
+    dispatch_fwht_sign_undo_f32; with the fused pre-rotation as well, the bits of the three-dispatch chain."""
+    hd, nh, nkv = 256, 16, 2
+    rng = np.random.default_rng(n)
+    m = min(n, cap)
+    kc, kn = _oracle_cache(oracle, rng.standard_normal((m, nkv, hd)).astype(np.float32), nkv, hd, cap)
+    vc, vn = _oracle_cache(oracle, rng.standard_normal((m, nkv, hd)).astype(np.float32), nkv, hd, cap)
+    q = rng.standard_normal((nh, hd)).astype(np.float32)
+    args = [torch.from_numpy(x).to(dev) for x in (kc, kn, vc, vn)]
+    tmp = torch.empty(ops.tq_tmp_buffer_bytes(nh, hd, n) // 4, device=dev)
+
+    qd = torch.from_numpy(q).to(dev)
+    ops.dispatch_fwht_sign_premult_f32(qd, nh, hd)
+    sep = torch.empty(nh, hd, device=dev)
+    ops.flash_attn_vec_tq_hb(qd, *args, sep, tmp, FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 0.0625, **kw))
+    ops.dispatch_fwht_sign_undo_f32(sep, nh, hd)
+
+    post = torch.full((nh, hd), float("nan"), device=dev)
+    ops.flash_attn_vec_tq_hb(qd, *args, post, tmp, FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 0.0625, **kw), undo_rotation=True)
+    assert torch.equal(sep, post)
+    both = torch.full((nh, hd), float("nan"), device=dev)
+    ops.flash_attn_vec_tq_hb(torch.from_numpy(q).to(dev), *args, both, tmp,
+                             FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 0.0625, fuse_fwht_pre=1, **kw), undo_rotation=True)
+    assert torch.equal(sep, both)
+
+
 def test_end_to_end_against_unquantised_attention(oracle, dev):
     """The reference's litmus (kv_cache.rs:3959-4117): rotate q, attend over the 8-bit cache, rotate back, compare
     with plain f32 attention.  kv_seq_len = 1 must return V[h / heads_per_kv]; gate NRMSE < 0.15."""
