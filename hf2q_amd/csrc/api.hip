@@ -353,7 +353,6 @@ static int flash_attn_vec_tq(const char* fn, bool undo_rotation, void* stream, c
     if (!is_aligned(q, 16) || !is_aligned(out, 16) || !is_aligned(k_codes, 16) || !is_aligned(v_codes, 16) ||
         !is_aligned(tmp, 4))
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: q / out / codes need 16-byte alignment", fn);
-    if (p->head_dim == 512) return fail(HQ_ERR_UNSUPPORTED, "%s: head_dim 512 is not built", fn);
     // 5- and 6-bit caches store one code per byte like the 8-bit one and differ only in the centroid
     // table, which the caller supplies (its first 2^bits entries); the linear int8 map is 8-bit only.
     if (p->codebook_bits != 8 && !lut256)

@@ -159,11 +159,14 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// One workgroup: one kv head, one chunk of <= 8 query heads of its group, one split of the sequence.
-template <bool LUT>
+// One workgroup: one kv head, one chunk of <= 8 query heads of its group, one split of the sequence
+// and, for head_dim = NB * 256, one 256-block of the output (blockIdx.z): the scores run over all NB
+// blocks of K, each with its own norm, the P.V product over the workgroup's block of V.
+template <bool LUT, int NB>
 __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
-    __shared__ float s_q[8][HD];          // the chunk's queries (rotated here when fuse_fwht_pre)
-    __shared__ uint4 s_qh[8][33], s_ql[8][33];  // their bf16 hi / lo halves, 8 values per entry
+    constexpr uint32_t ROW = NB * HD;        // bytes of a cache row, floats of a query
+    __shared__ float s_q[8][ROW];         // the chunk's queries (rotated here when fuse_fwht_pre)
+    __shared__ uint4 s_qh[NB][8][33], s_ql[NB][8][33];  // their bf16 hi / lo halves, 8 values per entry
     __shared__ float s_p[4][16][8];       // per wave: p * norm_v of the current tile, [position][head]
     __shared__ float s_alpha[4][8];       // per wave: rescale factor of the running output
     __shared__ float s_o[4][8][HD];       // per wave outputs for the final merge
@@ -176,6 +179,7 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     const uint32_t h0 = kvh * a.group + hc * 8u;
     const uint32_t nh = min(8u, a.group - hc * 8u);
     const uint32_t split = blockIdx.x;
+    const uint32_t ob = NB > 1 ? blockIdx.z : 0u;
 
     const uint32_t j = lane & 15u, g = lane >> 4;
     const uint32_t half = lane >> 5, dg = lane & 31u;
@@ -185,9 +189,9 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     // Operands of one 16-position tile of this wave.  K: lane (position j, quarter g) holds 64
     // contiguous code bytes; V: lane (half, dg) holds coordinates 8*dg..+7 of positions 2t + half.
     struct Tile {
-        uint4 k0, k1, k2, k3;
+        uint4 k[NB][4];
         uint2 v[8];
-        float kn, vn;
+        float kn[NB], vn;
         bool ok;
     };
     // physical slot of logical position idx (ring buffer); ring_start, idx < kv_capacity
@@ -200,15 +204,18 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
         const uint32_t idx = tile0 + j;
         t.ok = idx < a.last;
         const uint32_t slot = slot_of(t.ok ? idx : a.first);  // positions past the end read a valid slot, weight 0
-        const uint4* kp = reinterpret_cast<const uint4*>(a.k_codes + (head_base + slot) * HD + 64 * g);
-        t.k0 = kp[0], t.k1 = kp[1], t.k2 = kp[2], t.k3 = kp[3];
-        t.kn = a.k_norms[head_base + slot];
-        t.vn = t.ok ? a.v_norms[head_base + slot] : 0.f;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const uint4* kp = reinterpret_cast<const uint4*>(a.k_codes + (head_base + slot) * ROW + HD * b + 64 * g);
+            t.k[b][0] = kp[0], t.k[b][1] = kp[1], t.k[b][2] = kp[2], t.k[b][3] = kp[3];
+            t.kn[b] = a.k_norms[(head_base + slot) * NB + b];
+        }
+        t.vn = t.ok ? a.v_norms[(head_base + slot) * NB + ob] : 0.f;
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
             const uint32_t vi = tile0 + 2 * q + half;
             const uint32_t vs = slot_of(vi < a.last ? vi : a.first);
-            t.v[q] = *reinterpret_cast<const uint2*>(a.v_codes + (head_base + vs) * HD + 8 * dg);
+            t.v[q] = *reinterpret_cast<const uint2*>(a.v_codes + (head_base + vs) * ROW + HD * ob + 8 * dg);
         }
     };
 
@@ -221,17 +228,17 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     load_tile(0, cur);
 
     // ---- queries -> LDS (zero rows for absent heads), optional sign x FWHT ----
-    for (uint32_t i = tid; i < 8 * HD / 4; i += 256) {
-        const uint32_t h = i / (HD / 4), c = i % (HD / 4);
+    for (uint32_t i = tid; i < 8 * ROW / 4; i += 256) {
+        const uint32_t h = i / (ROW / 4), c = i % (ROW / 4);
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (h < nh) v = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + h) * HD)[c];
+        if (h < nh) v = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + h) * ROW)[c];
         reinterpret_cast<float4*>(&s_q[h][0])[c] = v;
     }
     if constexpr (LUT) s_lut[tid] = a.lut[tid] * a.lut_mul;
     __syncthreads();
     if (a.fuse_fwht_pre) {
-        for (uint32_t h = wave; h < 8; h += 4) {
-            float4* p = reinterpret_cast<float4*>(&s_q[h][0]) + lane;
+        for (uint32_t hb = wave; hb < 8 * NB; hb += 4) {  // every 256-block is rotated on its own
+            float4* p = reinterpret_cast<float4*>(&s_q[hb / NB][HD * (hb % NB)]) + lane;
             const float4 t = *p;
             float v[4] = {t.x, t.y, t.z, t.w};
             apply_signs(v, lane);
@@ -244,25 +251,28 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
     // ---- query fragments: lane (j = lane%16: head, g = lane/16) holds q[j][64g + 8kk + e] as an exact
     // bf16 hi + lo pair.  The split is done once per workgroup (thread = head tid/32, chunk tid%32 of 8
     // values) and every wave reads its fragments back; rows are padded to 33 chunks against bank conflicts.
-    {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
         const uint32_t h = tid >> 5, ch = tid & 31u;
         uint32_t hi[8], lo[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float x = s_q[h][8 * ch + e];
+            const float x = s_q[h][HD * b + 8 * ch + e];
             hi[e] = bf16_rne(x);
             lo[e] = bf16_rne(x - bf16_bits_to_f32(hi[e]));
         }
-        s_qh[h][ch] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16));
-        s_ql[h][ch] = make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16));
+        s_qh[b][h][ch] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16));
+        s_ql[b][h][ch] = make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16));
     }
     __syncthreads();
-    uint4 qhi[8], qlo[8];
+    uint4 qhi[NB][8], qlo[NB][8];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-        qhi[kk] = j < 8 ? s_qh[j][8 * g + kk] : make_uint4(0, 0, 0, 0);
-        qlo[kk] = j < 8 ? s_ql[j][8 * g + kk] : make_uint4(0, 0, 0, 0);
-    }
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            qhi[b][kk] = j < 8 ? s_qh[b][j][8 * g + kk] : make_uint4(0, 0, 0, 0);
+            qlo[b][kk] = j < 8 ? s_ql[b][j][8 * g + kk] : make_uint4(0, 0, 0, 0);
+        }
 
     // ---- running state ----
     float m_run = -INFINITY, l_run = 0.f;  // for head j (identical in the 4 lane groups for m; partial for l)
@@ -275,50 +285,55 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
 
     for (uint32_t it = 0; it < a.tiles_per_wave; ++it) {
         if (it + 1 < a.tiles_per_wave) load_tile(it + 1, nxt);
-        const uint4 k0 = cur.k0, k1 = cur.k1, k2 = cur.k2, k3 = cur.k3;
-        const float kn = cur.kn, vn = cur.vn;
+        const float vn = cur.vn;
         const bool ok = cur.ok;
         uint2 vraw[8];
 #pragma unroll
         for (int q = 0; q < 8; ++q) vraw[q] = cur.v[q];
-        // -------- scores on the matrix cores --------
-        f32x4_t c = {0.f, 0.f, 0.f, 0.f};
-        const uint32_t kw[16] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w,
-                                 k2.x, k2.y, k2.z, k2.w, k3.x, k3.y, k3.z, k3.w};
+        // -------- scores on the matrix cores, one accumulator per 256-block (each has its own norm) --------
+        f32x4_t c[NB];
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-            if constexpr (!LUT) {
-                const bf16x8_t af = codes_to_frag(kw[2 * kk], kw[2 * kk + 1]);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8_t, qhi[kk]), c, 0, 0, 0);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8_t, qlo[kk]), c, 0, 0, 0);
-            } else {
-                // table values are arbitrary f32: hi+lo split of K as well, three products
-                uint32_t hi[8], lo[8];
+        for (int b = 0; b < NB; ++b) {
+            c[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            const uint32_t kw[16] = {cur.k[b][0].x, cur.k[b][0].y, cur.k[b][0].z, cur.k[b][0].w, cur.k[b][1].x, cur.k[b][1].y,
+                                     cur.k[b][1].z, cur.k[b][1].w, cur.k[b][2].x, cur.k[b][2].y, cur.k[b][2].z, cur.k[b][2].w,
+                                     cur.k[b][3].x, cur.k[b][3].y, cur.k[b][3].z, cur.k[b][3].w};
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float x = s_lut[(kw[2 * kk + (e >> 2)] >> (8 * (e & 3))) & 0xffu];
-                    hi[e] = bf16_rne(x);
-                    lo[e] = bf16_rne(x - bf16_bits_to_f32(hi[e]));
+            for (int kk = 0; kk < 8; ++kk) {
+                if constexpr (!LUT) {
+                    const bf16x8_t af = codes_to_frag(kw[2 * kk], kw[2 * kk + 1]);
+                    c[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8_t, qhi[b][kk]), c[b], 0, 0, 0);
+                    c[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8_t, qlo[b][kk]), c[b], 0, 0, 0);
+                } else {
+                    // table values are arbitrary f32: hi+lo split of K as well, three products
+                    uint32_t hi[8], lo[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float x = s_lut[(kw[2 * kk + (e >> 2)] >> (8 * (e & 3))) & 0xffu];
+                        hi[e] = bf16_rne(x);
+                        lo[e] = bf16_rne(x - bf16_bits_to_f32(hi[e]));
+                    }
+                    const bf16x8_t ah = __builtin_bit_cast(bf16x8_t, make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16),
+                                                                                hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)));
+                    const bf16x8_t al = __builtin_bit_cast(bf16x8_t, make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16),
+                                                                                lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)));
+                    c[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, __builtin_bit_cast(bf16x8_t, qhi[b][kk]), c[b], 0, 0, 0);
+                    c[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, __builtin_bit_cast(bf16x8_t, qlo[b][kk]), c[b], 0, 0, 0);
+                    c[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, __builtin_bit_cast(bf16x8_t, qhi[b][kk]), c[b], 0, 0, 0);
                 }
-                const bf16x8_t ah = __builtin_bit_cast(bf16x8_t, make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16),
-                                                                            hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)));
-                const bf16x8_t al = __builtin_bit_cast(bf16x8_t, make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16),
-                                                                            lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)));
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, __builtin_bit_cast(bf16x8_t, qhi[kk]), c, 0, 0, 0);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, __builtin_bit_cast(bf16x8_t, qlo[kk]), c, 0, 0, 0);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, __builtin_bit_cast(bf16x8_t, qhi[kk]), c, 0, 0, 0);
             }
         }
-        // c[v] = dot(q[head j], K[position 4g+v]); norms / validity of those positions sit in lanes 4g+v
+        // c[b][v] = dot(q[head j], K[position 4g+v]) over block b; norms / validity of those positions sit in lanes 4g+v
         float s[4], pv_norm[4];
         float tmax = -INFINITY;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int src = 4 * g + v;
-            const float nk = __shfl(kn, src);
             pv_norm[v] = __shfl(vn, src);
             const bool okv = __shfl((int)ok, src) != 0;
-            float x = c[v] * (a.scale * nk);
+            float x = 0.f;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) x += c[b][v] * (a.scale * __shfl(cur.kn[b], src));
             if (a.softcap != 0.f) x = a.softcap * tanhf(x / a.softcap);
             s[v] = okv ? x : -INFINITY;
             tmax = fmaxf(tmax, s[v]);
@@ -400,7 +415,7 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
             o += f * s_o[w][h][tid];
             l += f * s_l[w][h];
         }
-        float* out = a.tmp + ((size_t)(h0 + h) * a.n_splits + split) * TMP_STRIDE;
+        float* out = a.tmp + (((size_t)(h0 + h) * NB + ob) * a.n_splits + split) * TMP_STRIDE;
         out[tid] = o;
         if (tid == 0) {
             out[HD] = m;
@@ -449,16 +464,21 @@ __device__ __forceinline__ float row_xor8(float x) {
 // accumulators (i, e) of 4 registers hold row 4g + v (head (4g + v) % 8, hi or lo part), coordinate
 // 16n + 4i + e.
 //
+// head_dim = NB * 256: blockIdx.z is the 256-block of the output this workgroup produces; the scores
+// run over all NB blocks of K (each block has its own norm and its own query scaling), the P.V
+// product over the workgroup's block of V.
+//
 // Cache offsets are 32-bit here: the launcher takes this kernel only below 4 GiB per code tensor.
-template <bool RING>
+template <bool RING, int NB>
 __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
+    constexpr uint32_t ROW = NB * HD;  // bytes of a cache row, floats of a query
     // s_o: per wave and row, the 256 coordinates in the order [i][j][e] (coordinate 16j + 4i + e), so
     // that a wave's stores are contiguous.  The fused rotation stages the queries in the same memory.
     __shared__ __align__(16) float s_o[4][16][HD];
-    __shared__ uint4 s_qf[16][33];             // scaled queries as f16, 8 values per entry; rows 0..7 hi, 8..15 lo
-    __shared__ float s_corr[16], s_unscale[8];  // sum(off_i q_i) of a row; 2^e that undoes a head's scaling
+    __shared__ uint4 s_qf[NB][16][33];             // scaled queries as f16, 8 values per entry; rows 0..7 hi, 8..15 lo
+    __shared__ float s_corr[NB][16], s_unscale[NB][8];  // sum(off_i q_i) of a row; 2^e that undoes a head's scaling
     __shared__ float s_m[4][8], s_l[4][8];
-    float(*s_q)[HD] = reinterpret_cast<float(*)[HD]>(&s_o[0][0][0]);
+    float(*s_q)[ROW] = reinterpret_cast<float(*)[ROW]>(&s_o[0][0][0]);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t n_chunks = (a.group + 7u) / 8u;
@@ -466,6 +486,7 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
     const uint32_t h0 = kvh * a.group + hc * 8u;
     const uint32_t nh = min(8u, a.group - hc * 8u);
     const uint32_t split = blockIdx.x;
+    const uint32_t ob = NB > 1 ? blockIdx.z : 0u;
     const uint32_t j = lane & 15u, g = lane >> 4;
     const uint32_t head_base = kvh * a.kv_capacity;
     const uint32_t split_first = a.first + split * (a.tiles_per_wave * 64u);
@@ -473,10 +494,10 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
     const uint32_t n_iter = (a.tiles_per_wave + 1u) / 2u;  // 128 positions per workgroup and iteration
 
     struct Tile {
-        uint4 k[2][4];  // half, i: code bytes 64i + 16g .. +15 of position j
-        uint4 v[8];     // positions 4g..4g+3 of half 0, then of half 1; coordinates 16j..
-        float kn[2];    // norm_k of position j, -1 where the position is past the end
-        float vn[2];    // norm_v, 0 where the position is past the end
+        uint4 k[NB][2][4];  // block, half, i: code bytes 64i + 16g .. +15 of position j
+        uint4 v[8];         // positions 4g..4g+3 of half 0, then of half 1; coordinates 16j.. of block ob
+        float kn[NB][2];    // norm_k of position j, -1 where the position is past the end
+        float vn[2];        // norm_v of block ob, 0 where the position is past the end
     };
     // Cache row of logical position idx; positions past the end of the split read a valid row and get
     // weight 0.  RING: rows start at ring_start and wrap (ring_start, idx < kv_capacity); otherwise
@@ -496,16 +517,19 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
             const uint32_t idx = tile0 + 16u * hf + j;
             const bool ok = idx < split_end;
             const uint32_t row = head_base + row_of(idx);
-            const uint4* kp = reinterpret_cast<const uint4*>(a.k_codes + (row * (uint32_t)HD + 16u * g));
-            t.k[hf][0] = kp[0], t.k[hf][1] = kp[4], t.k[hf][2] = kp[8], t.k[hf][3] = kp[12];
-            t.kn[hf] = ok ? a.k_norms[row] : -1.f;
-            t.vn[hf] = ok ? a.v_norms[row] : 0.f;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const uint4* kp = reinterpret_cast<const uint4*>(a.k_codes + (row * ROW + (uint32_t)(HD * b) + 16u * g));
+                t.k[b][hf][0] = kp[0], t.k[b][hf][1] = kp[4], t.k[b][hf][2] = kp[8], t.k[b][hf][3] = kp[12];
+                t.kn[b][hf] = ok ? a.k_norms[row * NB + b] : -1.f;
+            }
+            t.vn[hf] = ok ? a.v_norms[row * NB + ob] : 0.f;
         }
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
             const uint32_t vi = tile0 + (q < 4 ? 4u * g + q : 16u + 4u * g + (q - 4));
             const uint32_t row = head_base + row_of(vi);
-            t.v[q] = *reinterpret_cast<const uint4*>(a.v_codes + (row * (uint32_t)HD + 16u * j));
+            t.v[q] = *reinterpret_cast<const uint4*>(a.v_codes + (row * ROW + HD * ob + 16u * j));
         }
     };
 
@@ -515,38 +539,37 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
     load_tile(0, tile_a);
     if (n_iter > 1) load_tile(1, tile_b);
 
-    // ---- queries: scaled per head, split into f16 hi + lo; thread = head tid/32, chunk tid%32 of 8
-    // values; rows are padded to 33 chunks against bank conflicts ----
-    {
-        const uint32_t h = tid >> 5, ch = tid & 31u;
-        float x[8];
-        if (a.fuse_fwht_pre) {  // sign x FWHT in LDS first
-            for (uint32_t i = tid; i < 8 * HD / 4; i += 256) {
-                const uint32_t hh = i / (HD / 4), c = i % (HD / 4);
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (hh < nh) v = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + hh) * HD)[c];
-                reinterpret_cast<float4*>(&s_q[hh][0])[c] = v;
-            }
-            __syncthreads();
-            for (uint32_t hh = wave; hh < 8; hh += 4) {
-                float4* p = reinterpret_cast<float4*>(&s_q[hh][0]) + lane;
-                const float4 t = *p;
-                float v[4] = {t.x, t.y, t.z, t.w};
-                apply_signs(v, lane);
-                fwht256(v, lane);
-                *p = make_float4(v[0], v[1], v[2], v[3]);
-            }
-            __syncthreads();
-            const float4 v0 = *reinterpret_cast<const float4*>(&s_q[h][8 * ch]), v1 = *reinterpret_cast<const float4*>(&s_q[h][8 * ch + 4]);
-            x[0] = v0.x, x[1] = v0.y, x[2] = v0.z, x[3] = v0.w, x[4] = v1.x, x[5] = v1.y, x[6] = v1.z, x[7] = v1.w;
-        } else {
-            float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
-            if (h < nh) {
-                const float4* qp = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + h) * HD + 8 * ch);
-                v0 = qp[0], v1 = qp[1];
-            }
-            x[0] = v0.x, x[1] = v0.y, x[2] = v0.z, x[3] = v0.w, x[4] = v1.x, x[5] = v1.y, x[6] = v1.z, x[7] = v1.w;
+    // ---- queries: every 256-block of a head scaled on its own and split into f16 hi + lo; thread =
+    // head tid/32, chunk tid%32 of 8 values; rows are padded to 33 chunks against bank conflicts ----
+    if (a.fuse_fwht_pre) {  // sign x FWHT of every block in LDS first
+        for (uint32_t i = tid; i < 8 * ROW / 4; i += 256) {
+            const uint32_t hh = i / (ROW / 4), c = i % (ROW / 4);
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (hh < nh) v = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + hh) * ROW)[c];
+            reinterpret_cast<float4*>(&s_q[hh][0])[c] = v;
         }
+        __syncthreads();
+        for (uint32_t hb = wave; hb < 8 * NB; hb += 4) {
+            float4* p = reinterpret_cast<float4*>(&s_q[hb / NB][HD * (hb % NB)]) + lane;
+            const float4 t = *p;
+            float v[4] = {t.x, t.y, t.z, t.w};
+            apply_signs(v, lane);
+            fwht256(v, lane);
+            *p = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const uint32_t h = tid >> 5, ch = tid & 31u;
+        float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
+        if (a.fuse_fwht_pre) {
+            v0 = *reinterpret_cast<const float4*>(&s_q[h][HD * b + 8 * ch]), v1 = *reinterpret_cast<const float4*>(&s_q[h][HD * b + 8 * ch + 4]);
+        } else if (h < nh) {
+            const float4* qp = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + h) * ROW + HD * b + 8 * ch);
+            v0 = qp[0], v1 = qp[1];
+        }
+        const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
         float amax = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -576,22 +599,25 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
             sum_hi += __shfl_xor(sum_hi, o);
             sum_lo += __shfl_xor(sum_lo, o);
         }
-        if (a.fuse_fwht_pre) __syncthreads();  // s_q is read, its memory may be written again
-        s_qf[h][ch] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16));
-        s_qf[8 + h][ch] = make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16));
+        s_qf[b][h][ch] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16));
+        s_qf[b][8 + h][ch] = make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16));
         if (ch == 0) {
-            s_corr[h] = sum_hi;
-            s_corr[8 + h] = sum_lo;
-            s_unscale[h] = __builtin_amdgcn_ldexpf(1.f, -sh);
+            s_corr[b][h] = sum_hi;
+            s_corr[b][8 + h] = sum_lo;
+            s_unscale[b][h] = __builtin_amdgcn_ldexpf(1.f, -sh);
         }
     }
-    __syncthreads();
+    __syncthreads();  // also: s_q has been read, its memory (s_o) may be written again
     // MFMA step kk = 2i + w takes words 2w, 2w + 1 of K load i: coordinates 64i + 16g + 8w .. +7
-    uint4 qf[8];
+    uint4 qf[NB][8];
+    float corr[NB], sscale[NB];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) qf[kk] = s_qf[j][8u * (kk >> 1) + 2u * g + (kk & 1)];
-    const float corr = s_corr[j];
-    const float sscale = s_unscale[j & 7u] * a.scale;
+    for (int b = 0; b < NB; ++b) {
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) qf[b][kk] = s_qf[b][j][8u * (kk >> 1) + 2u * g + (kk & 1)];
+        corr[b] = s_corr[b][j];
+        sscale[b] = s_unscale[b][j & 7u] * a.scale;
+    }
     const bool lo_lane = j >= 8u;
 
     const uint32_t magic = 0x0000e464u;
@@ -617,30 +643,36 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
         float s[8], lv[8];
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            f32x4_t c0 = {0.f, 0.f, 0.f, 0.f}, c1 = c0;
+            float dot[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) {
-                const uint4 kq = cur.k[hf][kk >> 1];
-                const uint32_t u0 = ((kk & 1) ? kq.z : kq.x) ^ 0x7f807f80u, u1 = ((kk & 1) ? kq.w : kq.y) ^ 0x7f807f80u;
-                const uint4 fr = make_uint4(pair_of(u0, 0x05010400u), pair_of(u0, 0x05030402u), pair_of(u1, 0x05010400u),
-                                            pair_of(u1, 0x05030402u));
-                const f16x8_t af = __builtin_bit_cast(f16x8_t, fr);
-                if (kk & 1)
-                    c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8_t, qf[kk]), c1, 0, 0, 0);
-                else
-                    c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8_t, qf[kk]), c0, 0, 0, 0);
+            for (int b = 0; b < NB; ++b) {
+                f32x4_t c0 = {0.f, 0.f, 0.f, 0.f}, c1 = c0;
+#pragma unroll
+                for (int kk = 0; kk < 8; ++kk) {
+                    const uint4 kq = cur.k[b][hf][kk >> 1];
+                    const uint32_t u0 = ((kk & 1) ? kq.z : kq.x) ^ 0x7f807f80u, u1 = ((kk & 1) ? kq.w : kq.y) ^ 0x7f807f80u;
+                    const uint4 fr = make_uint4(pair_of(u0, 0x05010400u), pair_of(u0, 0x05030402u), pair_of(u1, 0x05010400u),
+                                                pair_of(u1, 0x05030402u));
+                    const f16x8_t af = __builtin_bit_cast(f16x8_t, fr);
+                    if (kk & 1)
+                        c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8_t, qf[b][kk]), c1, 0, 0, 0);
+                    else
+                        c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8_t, qf[b][kk]), c0, 0, 0, 0);
+                }
+                // c0 + c1 = (hi or lo part of q[head j % 8]) . (K[position 4g + v] + off) over block b; the
+                // norms of those positions sit in lanes 4g + v
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float part = (c0[v] + c1[v]) - corr[b];
+                    dot[v] += (part + row_xor8(part)) * (sscale[b] * __shfl(cur.kn[b][hf], 4 * g + v));
+                }
             }
-            // c0 + c1 = (hi or lo part of q[head j % 8]) . (K[position 4g + v] + off); the norms of those
-            // positions sit in lanes 4g + v
             const float lvn_own = __log2f(cur.vn[hf]);  // log 0 = -inf: no weight in the numerator
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int src = 4 * g + v;
-                const float nk = __shfl(cur.kn[hf], src);
                 lv[4 * hf + v] = __shfl(lvn_own, src);
-                const float part = (c0[v] + c1[v]) - corr;
-                const float x = (part + row_xor8(part)) * (sscale * nk);
-                s[4 * hf + v] = nk >= 0.f ? x : -INFINITY;
+                s[4 * hf + v] = __shfl(cur.kn[0][hf], src) >= 0.f ? dot[v] : -INFINITY;
             }
         }
         if (a.softcap != 0.f) {
@@ -756,7 +788,7 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
                     o0.x += x0.x, o0.y += x0.y, o0.z += x0.z, o0.w += x0.w;
                     o1.x += x1.x, o1.y += x1.y, o1.z += x1.z, o1.w += x1.w;
                 }
-            float* out = a.tmp + ((size_t)(h0 + h) * a.n_splits + split) * TMP_STRIDE;
+            float* out = a.tmp + (((size_t)(h0 + h) * NB + ob) * a.n_splits + split) * TMP_STRIDE;
             const uint32_t ci = c8 >> 3, cj = 2u * (c8 & 7u);
             float* o_at = out + 16u * cj + 4u * ci;  // TMP_STRIDE is even, not a multiple of 4: 8-byte stores
             reinterpret_cast<float2*>(o_at)[0] = make_float2(o0.x, o0.y);
@@ -884,8 +916,7 @@ uint32_t tq_attn_splits(uint32_t n_positions) {
 }
 
 size_t tq_attn_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len) {
-    (void)head_dim;
-    return (size_t)num_heads * tq_attn_splits(kv_seq_len) * TMP_STRIDE * sizeof(float);
+    return (size_t)num_heads * (head_dim / HD) * tq_attn_splits(kv_seq_len) * TMP_STRIDE * sizeof(float);
 }
 
 int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, const float* k_norms,
@@ -914,22 +945,27 @@ int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, c
     a.softcap = p.softcap;
     a.lut_mul = 1.f / (16.f * (p.head_dim == 512 ? p.scale_factor_d512 : 1.f));
     a.fuse_fwht_pre = p.fuse_fwht_pre;
-    const dim3 grid(a.n_splits, p.num_kv_heads * ((a.group + 7u) / 8u));
+    const uint32_t nb = p.head_dim / HD;
+    const dim3 grid(a.n_splits, p.num_kv_heads * ((a.group + 7u) / 8u), nb);
     // the f16 kernel indexes the code tensors with 32-bit byte offsets
-    const bool small = (uint64_t)p.num_kv_heads * p.kv_capacity * HD <= 0xffffffffull;
-    if (lut)
-        hipLaunchKernelGGL(tq_attn_split_kernel<true>, grid, dim3(256), 0, s, a);
-    else if (small && p.ring_start == 0)
-        hipLaunchKernelGGL(tq_attn_split_f16_kernel<false>, grid, dim3(256), 0, s, a);
-    else if (small)
-        hipLaunchKernelGGL(tq_attn_split_f16_kernel<true>, grid, dim3(256), 0, s, a);
+    const bool small = (uint64_t)p.num_kv_heads * p.kv_capacity * p.head_dim <= 0xffffffffull;
+    const bool ring = p.ring_start != 0;
+    void (*kern)(AttnArgs);
+    if (nb == 1)
+        kern = lut ? tq_attn_split_kernel<true, 1>
+               : !small ? tq_attn_split_kernel<false, 1>
+               : ring ? tq_attn_split_f16_kernel<true, 1> : tq_attn_split_f16_kernel<false, 1>;
     else
-        hipLaunchKernelGGL(tq_attn_split_kernel<false>, grid, dim3(256), 0, s, a);
+        kern = lut ? tq_attn_split_kernel<true, 2>
+               : !small ? tq_attn_split_kernel<false, 2>
+               : ring ? tq_attn_split_f16_kernel<true, 2> : tq_attn_split_f16_kernel<false, 2>;
+    hipLaunchKernelGGL(kern, grid, dim3(256), 0, s, a);
     if (int rc = check_launch("tq attention kernel launch")) return rc;
+    // every 256-block of a head is a row of its own in tmp and in out
     if (undo_rotation)
-        hipLaunchKernelGGL(tq_attn_merge_kernel<true>, dim3(p.num_heads), dim3(64 * MERGE_WAVES), 0, s, tmp, out, a.n_splits);
+        hipLaunchKernelGGL(tq_attn_merge_kernel<true>, dim3(p.num_heads * nb), dim3(64 * MERGE_WAVES), 0, s, tmp, out, a.n_splits);
     else
-        hipLaunchKernelGGL(tq_attn_merge_kernel<false>, dim3(p.num_heads), dim3(64 * MERGE_WAVES), 0, s, tmp, out, a.n_splits);
+        hipLaunchKernelGGL(tq_attn_merge_kernel<false>, dim3(p.num_heads * nb), dim3(64 * MERGE_WAVES), 0, s, tmp, out, a.n_splits);
     return check_launch("tq attention merge launch");
 }
 

@@ -226,10 +226,12 @@ typedef struct {
  * in the rotated domain.  lut256 == NULL: cached value = norm * int8(code); otherwise
  * lut256[code] * norm / 16 / scale_factor.  Replaces flash_attn_vec_tq_hb(enc, reg, dev, q, k_packed,
  * k_norms, v_packed, v_norms, out, tmp, &params) (forward_mlx.rs:4732-4742; kv_cache.rs:373-386).
+ * head_dim 512: codes are [n_kv_heads, capacity, 512], norms [n_kv_heads, capacity, 2] (one per
+ * 256-block, kv_cache.rs:2010-2012), table values are also divided by scale_factor_d512, and every
+ * 256-block of q / out is rotated on its own.
  * `tmp` is device scratch of hq_flash_attn_vec_tq_tmp_bytes() bytes.  Rejects kv_seq_len == 0,
  * kv_capacity < kv_seq_len (kv_cache.rs:331-333), head_dim not in {256, 512}, codebook_bits not in
- * {5, 6, 8}; head_dim 512, and codebook_bits 5 / 6 without a centroid table, are reported as
- * unsupported. */
+ * {5, 6, 8}; codebook_bits 5 / 6 without a centroid table are reported as unsupported. */
 HQ_API int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
                          const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
                          void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p);

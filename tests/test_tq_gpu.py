@@ -104,10 +104,68 @@ def test_attention_matches_f64_oracle(oracle, dev, nh, nkv, n, cap, kw):
 def _raw_cache(rng, nkv, cap, hd, norm_lo, norm_hi, log_uniform=False):
     codes = rng.integers(-127, 128, (nkv, cap, hd)).astype(np.int8).view(np.uint8)
     if log_uniform:
-        norms = np.exp(rng.uniform(np.log(norm_lo), np.log(norm_hi), (nkv, cap, 1)))
+        norms = np.exp(rng.uniform(np.log(norm_lo), np.log(norm_hi), (nkv, cap, hd // 256)))
     else:
-        norms = rng.uniform(norm_lo, norm_hi, (nkv, cap, 1))
+        norms = rng.uniform(norm_lo, norm_hi, (nkv, cap, hd // 256))
     return codes, norms.astype(np.float32)
+
+
+CASES_512 = [  # nh, nkv, n, cap, kwargs
+    (16, 2, 1, 8, {}),
+    (16, 2, 700, 1024, {}),
+    (8, 4, 257, 300, {"softcap": 4.0}),
+    (32, 2, 130, 256, {"mask_type": 1}),
+    (16, 2, 512, 512, {"mask_type": 2, "sliding_window": 300, "ring_start": 77}),
+    (16, 2, 5000, 5000, {}),
+]
+
+
+@pytest.mark.parametrize("nh,nkv,n,cap,kw", CASES_512)
+def test_attention_head_dim_512(oracle, dev, nh, nkv, n, cap, kw):
+    """head_dim 512 (kv_cache.rs:2010-2012): two 256-blocks per row, each with its own norm and its own rotation."""
+    hd = 512
+    rng = np.random.default_rng(nh * n + cap + 1)
+    k = rng.standard_normal((min(n, cap), nkv, hd)).astype(np.float32)
+    v = rng.standard_normal((min(n, cap), nkv, hd)).astype(np.float32)
+    v[:, :, 256:] *= 7.0  # the two blocks of a row get clearly different norms
+    kc, kn = _oracle_cache(oracle, k, nkv, hd, cap)
+    vc, vn = _oracle_cache(oracle, v, nkv, hd, cap)
+    q = oracle.fwht_sign_premult(rng.standard_normal((nh, hd)).astype(np.float32), nh, hd)
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 1.0 / 22.6, **kw)
+    ref = oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, hd, n, cap, p.scale, p.mask_type, p.sliding_window,
+                              p.softcap, p.ring_start)
+    got = _attend(dev, q, kc, kn, vc, vn, p)
+    _assert_attn_close(got, ref, f"attn d512 {nh}/{nkv} n={n} {kw}")
+    # the fused rotations give the bits of the three-dispatch chain here too
+    qraw = rng.standard_normal((nh, hd)).astype(np.float32)
+    args = [torch.from_numpy(x).to(dev) for x in (kc, kn, vc, vn)]
+    tmp = torch.empty(ops.tq_tmp_buffer_bytes(nh, hd, n) // 4, device=dev)
+    qd = torch.from_numpy(qraw).to(dev)
+    ops.dispatch_fwht_sign_premult_f32(qd, nh, hd)
+    sep = torch.empty(nh, hd, device=dev)
+    ops.flash_attn_vec_tq_hb(qd, *args, sep, tmp, p)
+    ops.dispatch_fwht_sign_undo_f32(sep, nh, hd)
+    both = torch.full((nh, hd), float("nan"), device=dev)
+    pf = FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 1.0 / 22.6, fuse_fwht_pre=1, **kw)
+    ops.flash_attn_vec_tq_hb(torch.from_numpy(qraw).to(dev), *args, both, tmp, pf, undo_rotation=True)
+    assert torch.equal(sep, both)
+
+
+def test_attention_head_dim_512_table_form(oracle, dev):
+    """The reference's D = 512 convention (table value * norm / 16 / scale_factor_d512) with 8- and 5-bit tables."""
+    hd, nh, nkv, n, cap = 512, 16, 2, 200, 256
+    for bits, sf in ((8, 1.0), (5, 1.4142135)):
+        rng = np.random.default_rng(90 + bits)
+        kc = rng.integers(0, 1 << bits, (nkv, cap, hd), dtype=np.uint8)
+        vc = rng.integers(0, 1 << bits, (nkv, cap, hd), dtype=np.uint8)
+        kn = rng.uniform(5, 20, (nkv, cap, 2)).astype(np.float32)
+        vn = rng.uniform(5, 20, (nkv, cap, 2)).astype(np.float32)
+        lut = np.zeros(256, np.float32)
+        lut[: 1 << bits] = np.sort(rng.standard_normal(1 << bits)).astype(np.float32) * 2
+        q = rng.standard_normal((nh, hd)).astype(np.float32)
+        p = FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 1.0 / 22.6, scale_factor_d512=sf, codebook_bits=bits)
+        ref = oracle.tq_attention(q, kc, kn, vc, vn, lut, nh, nkv, hd, n, cap, p.scale, scale_factor_d512=sf)
+        _assert_attn_close(_attend(dev, q, kc, kn, vc, vn, p, lut), ref, f"d512 {bits}-bit table")
 
 
 @pytest.mark.parametrize("case", ["q_large_mean", "q_tiny", "q_huge", "v_norm_range", "v_norm_zeros", "even_attention",
@@ -266,7 +324,7 @@ def test_argument_errors(dev):
         with pytest.raises(ops.HqError) as e:
             call(**bad)
         assert e.value.status == 1
-    for unsupported in (dict(head_dim=512), dict(codebook_bits=5)):
+    for unsupported in (dict(codebook_bits=5),):
         with pytest.raises(ops.HqError) as e:
             call(**unsupported)
         assert e.value.status == 2
