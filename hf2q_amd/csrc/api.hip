@@ -329,6 +329,28 @@ int hq_tq_encode_kv(void* stream, const float* src, uint8_t* codes, float* norms
                             write_pos % capacity);
 }
 
+int hq_tq_dequantize_kv_seq(void* stream, const uint8_t* codes, const float* norms, const float* lut256, float* dst,
+                            uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t start_pos,
+                            uint32_t n_tokens, float scale_factor_d512, uint32_t codebook_bits, int unrotate) {
+    const char* fn = "hq_tq_dequantize_kv_seq";
+    if (head_dim != 256 && head_dim != 512) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: head_dim %u (256 or 512)", fn, head_dim);
+    if (codebook_bits != 5 && codebook_bits != 6 && codebook_bits != 8)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: codebook_bits %u (5, 6 or 8)", fn, codebook_bits);
+    if ((uint64_t)start_pos + n_tokens > capacity)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: positions %u..%llu past the capacity %u", fn, start_pos,
+                    (unsigned long long)start_pos + n_tokens, capacity);
+    if (codebook_bits != 8 && !lut256)
+        return fail(HQ_ERR_UNSUPPORTED, "%s: a %u-bit cache needs its centroid table (lut256)", fn, codebook_bits);
+    if (n_kv_heads == 0 || n_tokens == 0) return HQ_OK;
+    if ((uint64_t)n_kv_heads * n_tokens * (head_dim / 256) > 0x7fffffffull)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: %u heads x %u tokens is too large for one call", fn, n_kv_heads, n_tokens);
+    if (!codes || !norms || !dst) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (!is_aligned(codes, 4) || !is_aligned(norms, 4) || !is_aligned(dst, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: codes / norms need 4-byte, dst 16-byte alignment", fn);
+    return launch_tq_dequantize((hipStream_t)stream, codes, norms, lut256, dst, n_kv_heads, head_dim, capacity, start_pos,
+                                n_tokens, scale_factor_d512, unrotate != 0);
+}
+
 size_t hq_flash_attn_vec_tq_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len) {
     return tq_attn_tmp_bytes(num_heads, head_dim, kv_seq_len);
 }

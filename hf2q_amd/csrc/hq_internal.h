@@ -71,6 +71,9 @@ int launch_moe_weighted_reduce(hipStream_t s, const float* y, const float* w, co
 int launch_fwht_sign(hipStream_t s, float* buf, uint32_t n_heads, uint32_t head_dim, bool undo);
 int launch_tq_encode(hipStream_t s, const float* src, uint8_t* codes, float* norms, uint32_t n_tokens,
                      uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t write_pos);
+int launch_tq_dequantize(hipStream_t s, const uint8_t* codes, const float* norms, const float* lut, float* dst,
+                         uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t start_pos, uint32_t n_tokens,
+                         float scale_factor_d512, bool unrotate);
 size_t tq_attn_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len);
 int launch_tq_attention(hipStream_t s, const float* q, const uint8_t* k_codes, const float* k_norms,
                         const uint8_t* v_codes, const float* v_norms, const float* lut, float* out, float* tmp,

@@ -112,6 +112,39 @@ __global__ __launch_bounds__(64) void tq_encode_kernel(const float* __restrict__
     if (lane == 0) norms[row * npp + blk] = d;
 }
 
+// Bulk dequantisation of positions start .. start + n_tokens - 1 of every kv head into
+// dst[n_kv_heads][n_tokens][head_dim] f32; one wave per 256-block.  Linear codes: norm * int8(code);
+// table codes: lut[code] * norm * lut_mul.  UNROT adds the inverse rotation of the block.
+template <bool LUT, bool UNROT>
+__global__ __launch_bounds__(64) void tq_dequant_kernel(const uint8_t* __restrict__ codes, const float* __restrict__ norms,
+                                                        const float* __restrict__ lut, float lut_mul, float* __restrict__ dst,
+                                                        uint32_t n_tokens, uint32_t head_dim, uint32_t capacity,
+                                                        uint32_t start) {
+    const uint32_t npp = head_dim / 256;
+    const uint32_t blk = blockIdx.x % npp, t = (blockIdx.x / npp) % n_tokens, h = blockIdx.x / (npp * n_tokens);
+    const uint32_t lane = threadIdx.x;
+    const size_t row = (size_t)h * capacity + start + t;
+    const uint32_t w = reinterpret_cast<const uint32_t*>(codes + row * head_dim + 256 * blk)[lane];
+    const float norm = norms[row * npp + blk];
+    float v[4];
+    {
+        // every product is rounded on its own: no fusion with the first additions of the rotation
+#pragma clang fp contract(off)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (LUT)
+                v[e] = lut[(w >> (8 * e)) & 0xffu] * norm * lut_mul;
+            else
+                v[e] = norm * sbyte(w, e);
+        }
+    }
+    if constexpr (UNROT) {
+        fwht256(v, lane);
+        apply_signs(v, lane);
+    }
+    reinterpret_cast<float4*>(dst + ((size_t)h * n_tokens + t) * head_dim + 256 * blk)[lane] = make_float4(v[0], v[1], v[2], v[3]);
+}
+
 struct AttnArgs {
     const float* q;
     const uint8_t* k_codes;
@@ -899,6 +932,19 @@ int launch_tq_encode(hipStream_t s, const float* src, uint8_t* codes, float* nor
     hipLaunchKernelGGL(tq_encode_kernel, dim3(blocks), dim3(64), 0, s, src, codes, norms, n_kv_heads, head_dim, capacity,
                        write_pos);
     return check_launch("tq encode kernel launch");
+}
+
+int launch_tq_dequantize(hipStream_t s, const uint8_t* codes, const float* norms, const float* lut, float* dst,
+                         uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t start_pos, uint32_t n_tokens,
+                         float scale_factor_d512, bool unrotate) {
+    const unsigned blocks = n_kv_heads * n_tokens * (head_dim / 256);
+    const float lut_mul = 1.f / (16.f * (head_dim == 512 ? scale_factor_d512 : 1.f));
+    void (*kern)(const uint8_t*, const float*, const float*, float, float*, uint32_t, uint32_t, uint32_t, uint32_t) =
+        lut ? (unrotate ? tq_dequant_kernel<true, true> : tq_dequant_kernel<true, false>)
+            : (unrotate ? tq_dequant_kernel<false, true> : tq_dequant_kernel<false, false>);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(64), 0, s, codes, norms, lut, lut_mul, dst, n_tokens, head_dim, capacity,
+                       start_pos);
+    return check_launch("tq dequantize kernel launch");
 }
 
 // Visible logical range of a single query at the end of the sequence.

@@ -65,9 +65,18 @@ SIGNATURES = {
     "hq_fwht_sign_premult_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_fwht_sign_undo_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_tq_encode_kv": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
+    "hq_tq_dequantize_kv_seq": (_i32, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _f32, _u32, _i32]),
     "hq_flash_attn_vec_tq": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "hq_flash_attn_vec_tq_undo": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "hq_flash_attn_vec_tq_tmp_bytes": (_sz, [_u32, _u32, _u32]),
+    "hq_tqp_indices_bytes": (_sz, [_vp]),
+    "hq_tqp_norms_bytes": (_sz, [_vp]),
+    "hq_tqp_total_bytes": (_sz, [_vp]),
+    "hq_tqp_pack": (_i32, [_vp, _vp, _sz, _vp, _sz, _vp, _sz]),
+    "hq_tqp_unpack": (_i32, [_vp, _sz, _vp, _c.POINTER(_sz), _c.POINTER(_sz)]),
+    "hq_tq_kv_capture_bytes": (_sz, [_u32, _u32, _u32]),
+    "hq_tq_kv_capture": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _vp, _sz]),
+    "hq_tq_kv_restore": (_i32, [_vp, _vp, _sz, _vp, _vp, _u32, _u32, _u32, _u32]),
     "hq_gguf_open": (_i32, [_c.c_char_p, _c.POINTER(_vp)]),
     "hq_gguf_close": (None, [_vp]),
     "hq_gguf_tensor_count": (_u64, [_vp]),
@@ -82,6 +91,12 @@ SIGNATURES = {
     "hq_gguf_tensor_data": (_vp, [_vp, _c.c_char_p, _c.POINTER(_u64)]),
     "hq_gguf_load_tensor": (_i32, [_vp, _c.c_char_p, _vp, _vp, _sz]),
 }
+
+
+class TqpHeader(ctypes.Structure):
+    """hq_tqp_header (include/hf2q_hip.h)."""
+    _fields_ = [("codec_version", _u32), ("bits_per_coord", _u32), ("head_dim", _u32), ("n_kv_heads", _u32),
+                ("n_tokens", _u32), ("flags", _u32), ("scale", ctypes.c_double)]
 
 
 class TqAttnParams(ctypes.Structure):

@@ -350,6 +350,84 @@ def flash_attn_vec_tq_hb(q: torch.Tensor, k_packed: torch.Tensor, k_norms: torch
         _dev(tmp, "tmp"), tmp.numel() * tmp.element_size(), _ct.byref(p)))
 
 
+def tq_dequantize_hb_kv_seq(packed: torch.Tensor, norms: torch.Tensor, dst: torch.Tensor, n_kv_heads: int, head_dim: int,
+                            cache_capacity: int, start_pos: int, n_tokens: int, scale_factor_d512: float = 1.0,
+                            codebook_bits: int = 8, lut256: torch.Tensor | None = None, unrotate: bool = False) -> None:
+    """kv_cache.rs:431-495 (dequant_seq_to_temp_f32) / :497-583 (…_unrotated): cache positions
+    start_pos .. start_pos + n_tokens - 1 as f32 [n_kv_heads, n_tokens, head_dim]."""
+    if dst.dtype != torch.float32 or dst.numel() < n_kv_heads * n_tokens * head_dim:
+        raise TypeError("dst must be float32 [n_kv_heads, n_tokens, head_dim]")
+    _l.check(_l.load().hq_tq_dequantize_kv_seq(
+        _stream(), _dev(packed, "packed"), _dev(norms, "norms"), _dev(lut256, "lut256") if lut256 is not None else None,
+        _dev(dst, "dst"), n_kv_heads, head_dim, cache_capacity, start_pos, n_tokens, scale_factor_d512, codebook_bits,
+        1 if unrotate else 0))
+
+
+@dataclass
+class TqPackedHeader:
+    """TqPackedV1Header / TqPackedV2Header (kv_persist/families/tq_packed.rs:129-153, 376-396)."""
+    codec_version: int
+    bits_per_coord: int
+    head_dim: int
+    n_kv_heads: int
+    n_tokens: int
+    flags: int = 0
+    scale: float = 1.0
+
+    def _c(self):
+        return _l.TqpHeader(self.codec_version, self.bits_per_coord, self.head_dim, self.n_kv_heads, self.n_tokens,
+                            self.flags, self.scale)
+
+    def indices_bytes_len(self) -> int:
+        import ctypes as _ct
+        return _l.load().hq_tqp_indices_bytes(_ct.byref(self._c()))
+
+    def norms_bytes_len(self) -> int:
+        import ctypes as _ct
+        return _l.load().hq_tqp_norms_bytes(_ct.byref(self._c()))
+
+    def total_bytes(self) -> int:
+        import ctypes as _ct
+        return _l.load().hq_tqp_total_bytes(_ct.byref(self._c()))
+
+
+def pack_tq_payload(header: TqPackedHeader, indices: bytes, norms_le: bytes = b"") -> bytes:
+    """pack_tq_v1_payload / pack_tq_v2_payload (tq_packed.rs:199-226, 459-489)."""
+    import ctypes as _ct
+    out = _ct.create_string_buffer(max(1, header.total_bytes()))
+    _l.check(_l.load().hq_tqp_pack(_ct.byref(header._c()), bytes(indices), len(indices), bytes(norms_le), len(norms_le),
+                                   out, header.total_bytes()))
+    return out.raw[:header.total_bytes()]
+
+
+def unpack_tq_payload(payload: bytes):
+    """unpack_tq_v1_payload / unpack_tq_v2_payload (tq_packed.rs:243-311, 491-566): (header, indices, norms)."""
+    import ctypes as _ct
+    h = _l.TqpHeader()
+    io, no = _ct.c_size_t(), _ct.c_size_t()
+    _l.check(_l.load().hq_tqp_unpack(bytes(payload), len(payload), _ct.byref(h), _ct.byref(io), _ct.byref(no)))
+    hdr = TqPackedHeader(h.codec_version, h.bits_per_coord, h.head_dim, h.n_kv_heads, h.n_tokens, h.flags, h.scale)
+    return hdr, payload[io.value:no.value], payload[no.value:]
+
+
+def capture_tq_kv(packed: torch.Tensor, norms: torch.Tensor, n_kv_heads: int, head_dim: int, capacity: int,
+                  start_pos: int, n_tokens: int) -> bytes:
+    """A version-2 envelope of cache positions start_pos .. start_pos + n_tokens - 1 (tq_packed.rs:568-590)."""
+    import ctypes as _ct
+    need = _l.load().hq_tq_kv_capture_bytes(n_kv_heads, head_dim, n_tokens)
+    out = _ct.create_string_buffer(need)
+    _l.check(_l.load().hq_tq_kv_capture(_stream(), _dev(packed, "packed"), _dev(norms, "norms"), n_kv_heads, head_dim,
+                                        capacity, start_pos, n_tokens, out, need))
+    return out.raw[:need]
+
+
+def restore_tq_kv(payload: bytes, packed: torch.Tensor, norms: torch.Tensor, n_kv_heads: int, head_dim: int,
+                  capacity: int, start_pos: int) -> None:
+    """Writes an envelope's indices and norms back into the cache at start_pos."""
+    _l.check(_l.load().hq_tq_kv_restore(_stream(), bytes(payload), len(payload), _dev(packed, "packed"),
+                                        _dev(norms, "norms"), n_kv_heads, head_dim, capacity, start_pos))
+
+
 # ---- MoE FFN block ------------------------------------------------------------------------------
 
 def dense_gemv_bf16_f32(x: torch.Tensor, w_bf16: torch.Tensor, y: torch.Tensor, m: int, n: int, k: int) -> None:

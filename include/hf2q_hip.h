@@ -205,6 +205,18 @@ HQ_API int hq_fwht_sign_undo_f32(void* stream, float* buf, uint32_t n_heads, uin
 HQ_API int hq_tq_encode_kv(void* stream, const float* src, uint8_t* codes, float* norms, uint32_t n_tokens,
                     uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t write_pos);
 
+/* Bulk dequantisation of cache positions start_pos .. start_pos + n_tokens - 1 of every kv head into
+ * dst [n_kv_heads, n_tokens, head_dim] f32 (head-major), for prefill resume over a TQ-only cache.
+ * Replaces dispatch_tq_dequantize_hb_kv_seq(enc, reg, dev, packed, norms, dst, n_kv_heads, head_dim,
+ * cache_capacity, start_pos, n_tokens, scale_factor_d512, codebook_bits) as dequant_seq_to_temp_f32
+ * calls it (kv_cache.rs:431-495); unrotate != 0 also applies dispatch_fwht_sign_undo_f32 to every
+ * (head, token) chunk, i.e. dequant_seq_to_temp_f32_unrotated (kv_cache.rs:497-583) in one launch
+ * with the bits of the two.  Values as in hq_flash_attn_vec_tq (lut256 == NULL: norm * int8(code)).
+ * Rejects start_pos + n_tokens > capacity (kv_cache.rs:427-428). */
+HQ_API int hq_tq_dequantize_kv_seq(void* stream, const uint8_t* codes, const float* norms, const float* lut256, float* dst,
+                            uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t start_pos,
+                            uint32_t n_tokens, float scale_factor_d512, uint32_t codebook_bits, int unrotate);
+
 /* Field for field FlashAttnVecTqHbParams / Qwen35TqSdpaParams (kv_cache.rs:589-614;
  * forward_mlx.rs:4687-4705). */
 typedef struct {
@@ -243,6 +255,47 @@ HQ_API int hq_flash_attn_vec_tq_undo(void* stream, const float* q, const uint8_t
                               const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
                               void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p);
 HQ_API size_t hq_flash_attn_vec_tq_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len);
+
+/* ---- TQ block envelope (spilled K / V blocks) ---- */
+
+/* TqPackedV1Header / TqPackedV2Header (kv_persist/families/tq_packed.rs:129-153, 376-396): the two
+ * share one 40-byte wire header; codec_version selects the magic ("TQP1" / "TQP2") and whether a
+ * stream of f32 norms follows the indices. */
+typedef struct {
+    uint32_t codec_version;  /* 1 or 2 */
+    uint32_t bits_per_coord; /* 1..8 */
+    uint32_t head_dim, n_kv_heads, n_tokens;
+    uint32_t flags;          /* HQ_TQP_FLAG_* */
+    double scale;
+} hq_tqp_header;
+#define HQ_TQP_HEADER_BYTES 40
+#define HQ_TQP_FLAG_HADAMARD_ROTATED 1u
+#define HQ_TQP_FLAG_SPLIT_CHANNEL_25BIT 2u
+
+/* indices_bytes_len / norms_bytes_len / total_bytes (tq_packed.rs:167-184, 399-440): ceil(heads *
+ * tokens * head_dim * bits / 8); 4 * heads * tokens * max(1, head_dim / 256) at version 2, else 0. */
+HQ_API size_t hq_tqp_indices_bytes(const hq_tqp_header* h);
+HQ_API size_t hq_tqp_norms_bytes(const hq_tqp_header* h);
+HQ_API size_t hq_tqp_total_bytes(const hq_tqp_header* h);
+/* pack_tq_v1_payload / pack_tq_v2_payload (tq_packed.rs:199-226, 459-489): header + indices
+ * (+ norms) into out; the stream lengths must be exactly the ones above (PayloadSizeMismatch). */
+HQ_API int hq_tqp_pack(const hq_tqp_header* h, const void* indices, size_t indices_len, const void* norms_le,
+                size_t norms_len, void* out, size_t out_capacity);
+/* unpack_tq_v1_payload / unpack_tq_v2_payload (tq_packed.rs:243-311, 491-566): parses and checks
+ * (Truncated, BadMagic, UnsupportedCodecVersion, InvalidBitsPerCoord, ReservedNonZero,
+ * PayloadSizeMismatch are all HQ_ERR_INVALID_ARGUMENT, told apart by hq_last_error()); returns the
+ * byte offsets of the two streams inside payload. */
+HQ_API int hq_tqp_unpack(const void* payload, size_t len, hq_tqp_header* h, size_t* indices_offset,
+                  size_t* norms_offset);
+/* capture / restore of a token range between the device cache and a version-2 envelope in host
+ * memory (the raw-bytes helpers of tq_packed.rs:568-590 with the device copy folded in): codes
+ * [n_kv_heads, capacity, head_dim] and norms [n_kv_heads, capacity, head_dim / 256], positions
+ * start_pos .. start_pos + n_tokens - 1.  Both wait for their copies on `stream`. */
+HQ_API size_t hq_tq_kv_capture_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint32_t n_tokens);
+HQ_API int hq_tq_kv_capture(void* stream, const uint8_t* codes, const float* norms, uint32_t n_kv_heads, uint32_t head_dim,
+                     uint32_t capacity, uint32_t start_pos, uint32_t n_tokens, void* payload, size_t payload_capacity);
+HQ_API int hq_tq_kv_restore(void* stream, const void* payload, size_t len, uint8_t* codes, float* norms,
+                     uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t start_pos);
 
 /* ---- GGUF reader (weights as hf2q loads them) ---- */
 

@@ -66,6 +66,8 @@ def lib() -> ctypes.CDLL:
         L.hq_oracle_tq_attention.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32,
                                              i32, i32, f32, i32, f32, vp]
         L.hq_oracle_tq_attention.restype = i32
+        L.hq_oracle_tq_dequantize.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, f32, vp]
+        L.hq_oracle_tq_dequantize.restype = i32
         L.hq_oracle_nearest_int.argtypes = [f32]
         L.hq_oracle_nearest_int.restype = i32
         L.hq_oracle_f32_to_f16.argtypes = [f32]
@@ -198,6 +200,21 @@ def tq_encode_int8(kv, n_kv_heads, head_dim, capacity, pos, codes, norms) -> Non
     kv = _c(kv, np.float32)
     assert codes.dtype == np.uint8 and norms.dtype == np.float32
     lib().hq_oracle_tq_encode_int8(_p(kv), n_kv_heads, head_dim, capacity, pos, _p(codes), _p(norms))
+
+
+def tq_dequantize(codes, norms, lut, n_kv_heads, head_dim, capacity, start_pos, n_tokens,
+                  scale_factor_d512=1.0, unrotate=False) -> np.ndarray:
+    """kv_cache.rs:431-495 (rotated domain) and :497-583 (followed by fwht_sign_undo over every
+    (head, token) chunk): f32 [n_kv_heads, n_tokens, head_dim]."""
+    lutc = None if lut is None else _c(lut, np.float32)
+    out = np.empty((n_kv_heads, n_tokens, head_dim), dtype=np.float32)
+    rc = lib().hq_oracle_tq_dequantize(_p(codes), _p(norms), _p(lutc), n_kv_heads, head_dim, capacity, start_pos,
+                                       n_tokens, scale_factor_d512, _p(out))
+    if rc:
+        raise ValueError(f"hq_oracle_tq_dequantize rc={rc}")
+    if unrotate:
+        out = fwht_sign_undo(out.reshape(-1, head_dim), n_kv_heads * n_tokens, head_dim).reshape(out.shape)
+    return out
 
 
 def tq_attention(q, k_codes, k_norms, v_codes, v_norms, lut, num_heads, num_kv_heads, head_dim,

@@ -870,6 +870,27 @@ static double tq_value(uint8_t code, float norm, const float *lut, float sf) {
     return (double)lut[code] * (double)norm / 16.0 / (double)sf;
 }
 
+/* Bulk dequantisation of cache positions start_pos .. start_pos + n_tokens - 1 (no wrap:
+ * kv_cache.rs:427-428 rejects start_pos + n_tokens > capacity) into out[n_kv_heads][n_tokens][head_dim]
+ * f32, rotated domain (dequant_seq_to_temp_f32, kv_cache.rs:431-495): each element is tq_value()
+ * rounded once to f32. */
+int hq_oracle_tq_dequantize(const uint8_t *codes, const float *norms, const float *lut, int n_kv_heads,
+                            int head_dim, int capacity, int start_pos, int n_tokens,
+                            float scale_factor_d512, float *out) {
+    if (head_dim != 256 && head_dim != 512) return -1;
+    if (start_pos < 0 || n_tokens < 0 || (int64_t)start_pos + n_tokens > capacity) return -2;
+    int npp = head_dim / 256;
+    float sf = head_dim == 512 ? scale_factor_d512 : 1.0f;
+    for (int h = 0; h < n_kv_heads; h++)
+        for (int t = 0; t < n_tokens; t++) {
+            int64_t row = (int64_t)h * capacity + start_pos + t;
+            for (int d = 0; d < head_dim; d++)
+                out[((int64_t)h * n_tokens + t) * head_dim + d] =
+                    (float)tq_value(codes[row * head_dim + d], norms[row * npp + d / 256], lut, sf);
+        }
+    return 0;
+}
+
 /* Single-query attention over the 8-bit cache in float64 (the parity gate for
  * flash_attn_vec_tq_hb, forward_mlx.rs:4687-4742, kv_cache.rs:335-388):
  * out[h] = softmax(scale * q[h] . K[kv(h)]^T [softcapped, masked]) . V[kv(h)],

@@ -305,6 +305,80 @@ def test_end_to_end_against_unquantised_attention(oracle, dev):
         assert e < 0.15 and e < 0.02, f"n={n}: nrmse {e}"
 
 
+@pytest.mark.parametrize("hd", [256, 512])
+@pytest.mark.parametrize("unrotate", [False, True])
+def test_bulk_dequantize_bit_exact(oracle, dev, hd, unrotate):
+    """dequant_seq_to_temp_f32[_unrotated] (kv_cache.rs:431-583): a range of cache positions back to f32,
+    head-major; every element is one rounding of norm * code, the rotation is the bit-exact FWHT."""
+    rng = np.random.default_rng(hd + unrotate)
+    nkv, cap, start, n = 3, 50, 7, 41
+    codes = rng.integers(0, 256, (nkv, cap, hd), dtype=np.uint8)
+    norms = rng.uniform(1e-3, 3.0, (nkv, cap, hd // 256)).astype(np.float32)
+    want = oracle.tq_dequantize(codes, norms, None, nkv, hd, cap, start, n, unrotate=unrotate)
+    dst = torch.full((nkv, n, hd), float("nan"), device=dev)
+    ops.tq_dequantize_hb_kv_seq(torch.from_numpy(codes).to(dev), torch.from_numpy(norms).to(dev), dst, nkv, hd, cap, start, n,
+                                unrotate=unrotate)
+    assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    # table form: lut[code] * norm / 16 (/ scale_factor_d512 at 512)
+    lut = (np.sort(rng.standard_normal(256)) * 2).astype(np.float32)
+    want = oracle.tq_dequantize(codes, norms, lut, nkv, hd, cap, start, n, unrotate=unrotate)
+    ops.tq_dequantize_hb_kv_seq(torch.from_numpy(codes).to(dev), torch.from_numpy(norms).to(dev), dst, nkv, hd, cap, start, n,
+                                lut256=torch.from_numpy(lut).to(dev), unrotate=unrotate)
+    assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    if hd == 512 and not unrotate:  # a scale factor that is no power of two: two roundings instead of one
+        want = oracle.tq_dequantize(codes, norms, lut, nkv, hd, cap, start, n, scale_factor_d512=1.3)
+        ops.tq_dequantize_hb_kv_seq(torch.from_numpy(codes).to(dev), torch.from_numpy(norms).to(dev), dst, nkv, hd, cap,
+                                    start, n, scale_factor_d512=1.3, lut256=torch.from_numpy(lut).to(dev))
+        assert np.allclose(dst.cpu().numpy(), want, rtol=3e-7, atol=0)
+
+
+def test_encode_then_bulk_dequantize_recovers_the_input(dev):
+    """The reference's round-trip gate (kv_cache.rs:497-520, NRMSE threshold 0.15 at production cache shape):
+    encode a sequence, dequantise it un-rotated, compare with the f32 input."""
+    nkv, hd, cap, n, start = 2, 256, 4096, 1000, 100
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4)
+    kv = torch.randn(n, nkv, hd, generator=gen, device=dev)
+    codes, norms = ops.alloc_tq_kv(nkv, cap, hd, dev)
+    ops.hadamard_quantize_kv(kv, codes, norms, start)
+    dst = torch.empty(nkv, n, hd, device=dev)
+    ops.tq_dequantize_hb_kv_seq(codes, norms, dst, nkv, hd, cap, start, n, unrotate=True)
+    e = _nrmse(dst.permute(1, 0, 2).cpu().numpy(), kv.cpu().numpy())
+    assert e < 0.15 and e < 0.01, e
+    with pytest.raises(ops.HqError) as err:  # kv_cache.rs:427-428
+        ops.tq_dequantize_hb_kv_seq(codes, norms, dst, nkv, hd, cap, cap - 10, 11)
+    assert err.value.status == 1
+
+
+@pytest.mark.parametrize("hd", [256, 512])
+def test_capture_and_restore_of_a_token_range(dev, hd):
+    """Cache positions -> version-2 envelope in host memory -> another cache: indices and norms byte-equal, the
+    envelope parses with the oracle's parser, positions outside the range are untouched."""
+    from oracle import tqp
+    nkv, cap, start, n = 3, 64, 9, 40
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(hd)
+    codes, norms = ops.alloc_tq_kv(nkv, cap, hd, dev)
+    ops.hadamard_quantize_kv(torch.randn(cap, nkv, hd, generator=gen, device=dev), codes, norms, 0)
+    payload = ops.capture_tq_kv(codes, norms, nkv, hd, cap, start, n)
+    h, idx, nrm = tqp.unpack(payload)
+    assert (h.codec_version, h.bits_per_coord, h.head_dim, h.n_kv_heads, h.n_tokens, h.flags, h.scale) == (2, 8, hd, nkv, n, 1, 1.0)
+    assert idx == codes[:, start:start + n].contiguous().cpu().numpy().tobytes()
+    assert nrm == norms.view(nkv, cap, -1)[:, start:start + n].contiguous().cpu().numpy().tobytes()
+    codes2, norms2 = ops.alloc_tq_kv(nkv, cap, hd, dev)
+    codes2.fill_(0x55)
+    norms2.fill_(7.0)
+    ops.restore_tq_kv(payload, codes2, norms2, nkv, hd, cap, start + 3)
+    assert torch.equal(codes2[:, start + 3:start + 3 + n], codes[:, start:start + n])
+    assert torch.equal(norms2.view(nkv, cap, -1)[:, start + 3:start + 3 + n], norms.view(nkv, cap, -1)[:, start:start + n])
+    assert (codes2[:, :start + 3] == 0x55).all() and (codes2[:, start + 3 + n:] == 0x55).all()
+    assert (norms2.view(nkv, cap, -1)[:, :start + 3] == 7.0).all() and (norms2.view(nkv, cap, -1)[:, start + 3 + n:] == 7.0).all()
+    with pytest.raises(ops.HqError):  # would run past the capacity
+        ops.restore_tq_kv(payload, codes2, norms2, nkv, hd, cap, cap - n + 1)
+    with pytest.raises(ops.HqError):  # another cache shape
+        ops.restore_tq_kv(payload, codes2, norms2, nkv + 1, hd, cap, 0)
+
+
 def test_argument_errors(dev):
     nh, nkv, hd, cap = 16, 2, 256, 32
     kc, kn = ops.alloc_tq_kv(nkv, cap, hd, dev)
