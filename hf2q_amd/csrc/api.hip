@@ -200,12 +200,29 @@ size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows) {
     return 0;
 }
 
+namespace {
+// Routed rows per expert from which the grouped tile GEMM takes over from one GEMV per row.
+constexpr uint64_t kGroupedRowsPerExpert = 8;
+bool grouped_route(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts, uint64_t expert_stride,
+                   hq_ggml_type t) {
+    const uint64_t pairs = (uint64_t)n_tokens * top_k;
+    return pairs >= 256 && pairs >= kGroupedRowsPerExpert * n_experts &&
+           gemm_f16_grouped_supported(t, n, k, n_experts, expert_stride, pairs);
+}
+}  // namespace
+
+size_t hq_qmatmul_id_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
+                                          uint64_t expert_stride, hq_ggml_type t) {
+    if (t != HQ_Q4_K && t != HQ_Q6_K && t != HQ_Q8_0) return 0;
+    if (n == 0 || k == 0 || k % hq_block_elems(t)) return 0;
+    return grouped_route(n_tokens, top_k, n, k, n_experts, expert_stride, t)
+               ? gemm_f16_grouped_workspace_bytes(n_tokens * top_k, n_experts, n, k) : 0;
+}
+
 int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_stack,
                        const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes,
                        uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
                        uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t) {
-    (void)scratch;
-    (void)scratch_bytes;
     if (int rc = check_matmul_common("hq_qmatmul_id_ggml", x, xdt, w_stack, y, n, k, t)) return rc;
     if (!ids) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: null ids");
     if (n_experts == 0 || top_k == 0)
@@ -219,8 +236,18 @@ int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void
                     (unsigned long long)expert_stride);
     const uint64_t pairs = (uint64_t)n_tokens * top_k;
     if (pairs == 0) return HQ_OK;
+    // Many rows per expert and a workspace from the caller: rows sorted by expert, tile GEMM per expert.
+    if (scratch && grouped_route(n_tokens, top_k, n, k, n_experts, expert_stride, t)) {
+        const size_t need = gemm_f16_grouped_workspace_bytes((uint32_t)pairs, n_experts, n, k);
+        if (scratch_bytes < need)
+            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: scratch of %zu bytes, %zu needed", scratch_bytes, need);
+        if (reinterpret_cast<uintptr_t>(scratch) % 256)
+            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: scratch must be 256-byte aligned");
+        return launch_gemm_f16_grouped((hipStream_t)stream, x, xdt, w_stack, ids, y, scratch, n_tokens, top_k, n, k, n_experts,
+                                       expert_stride, t);
+    }
     // One GEMV per routed row, up to 65535 rows per launch (grid.y).  Rows that share an expert read
-    // its weights through L2; a grouped MFMA GEMM for long prefills is the next step on this path.
+    // its weights through L2.
     const size_t xrow_bytes = (size_t)k * (xdt == HQ_BF16 ? 2 : 4);
     constexpr uint64_t kMaxPerLaunch = 65535u / 1u;
     for (uint64_t p0 = 0; p0 < pairs;) {

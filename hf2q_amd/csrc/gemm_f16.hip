@@ -90,7 +90,8 @@ __device__ __forceinline__ uint32_t f16_bits(float v) {
 // epilogue divides it out.
 template <bool X_BF16, int TYPE>
 __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
-                                                        uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k) {
+                                                        uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k,
+                                                        const uint32_t* __restrict__ row_map, uint32_t top_k) {
     __shared__ float red[4];
     const uint32_t tid = threadIdx.x;
     const Workspace L = workspace_layout(m, n, k);
@@ -130,7 +131,9 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
         if ((tid & 15u) == 0 && wr < n) reinterpret_cast<float*>(ws + L.wdown)[wr] = ldexpf(1.f, -e);  // |e| <= 40: normal
         return;
     }
-    const uint32_t row = blockIdx.x;
+    // grouped form: workspace row r holds the activations of routed row row_map[r], i.e. x row row_map[r] / top_k
+    const uint32_t out_row = blockIdx.x;
+    const uint32_t row = row_map ? row_map[out_row] / top_k : out_row;
     const uint32_t chunks = k / 8;
 
     auto load8 = [&](uint32_t i, float* v) {
@@ -176,7 +179,7 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
     sh = sh < -100 ? -100 : sh > 100 ? 100 : sh;
     if (amax == 0.f) sh = 0;
     const float scale = ldexpf(1.f, sh);
-    if (tid == 0) reinterpret_cast<float*>(ws + L.rs)[row] = ldexpf(1.f, -sh);
+    if (tid == 0) reinterpret_cast<float*>(ws + L.rs)[out_row] = ldexpf(1.f, -sh);
 
     for (uint32_t i = tid; i < chunks; i += 256) {
         float v[8];
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
         uint32_t h[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) h[j] = f16_bits(v[j] * scale);
-        *reinterpret_cast<uint4*>(ws + L.xh + ((size_t)row * k + 8 * i) * 2) =
+        *reinterpret_cast<uint4*>(ws + L.xh + ((size_t)out_row * k + 8 * i) * 2) =
             make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
     }
 }
@@ -194,6 +197,12 @@ struct GemmArgs {
     const uint8_t* w;
     float* y;
     uint32_t m, n, k;
+    // The grouped (expert) form looks at a slice of a larger problem: the workspace is laid out for
+    // lay_m activation rows and lay_n weight rows, the slice's weight rows start at wd_off in the
+    // table of weight-row scales, activation row r of the workspace is output row row_map[r].  The
+    // dense form has lay_m = m, lay_n = n, wd_off = 0, row_map = nullptr.
+    uint32_t lay_m, lay_n, wd_off;
+    const uint32_t* row_map;
 };
 
 __device__ __forceinline__ f16x8_t as_frag(uint4 v) { return __builtin_bit_cast(f16x8_t, v); }
@@ -270,14 +279,14 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W
         for (int v = 0; v < 16; ++v) {
             uint32_t gn = gnb + 8 * (v >> 2) + (v & 3);
             gn = gn < a.n ? gn : a.n - 1u;
-            wup[v] = __uint_as_float(0x7f000000u - __float_as_uint(wd[gn]));
+            wup[v] = __uint_as_float(0x7f000000u - __float_as_uint(wd[a.wd_off + gn]));
         }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const uint32_t gm = mbase + mt * 32 + l32;
             if (gm >= a.m) continue;
             const float rsv = rs[gm];
-            float* yp = a.y + (size_t)gm * a.n + gnb;
+            float* yp = a.y + (size_t)(a.row_map ? a.row_map[gm] : gm) * a.n + gnb;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const float o0 = acc[mt][nt][4 * g] * (rsv * wup[4 * g]), o1 = acc[mt][nt][4 * g + 1] * (rsv * wup[4 * g + 1]);
@@ -301,7 +310,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W
 template <int MT, int NT, int WN>
 __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
-    const Workspace W = workspace_layout(a.m, a.n, a.k);
+    const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t wm = wave / WN, wn = wave % WN;
@@ -320,7 +329,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
         uint32_t gn = n0 + wn * (32 * NT) + nt * 32 + l32;
         gn = gn < a.n ? gn : a.n - 1u;
         wrow[nt] = a.w + (size_t)gn * row_bytes;
-        wdown[nt] = reinterpret_cast<const float*>(a.ws + W.wdown)[gn];
+        wdown[nt] = reinterpret_cast<const float*>(a.ws + W.wdown)[a.wd_off + gn];
     }
     uint4 braw[4][NT];        // nibbles of stages s, s+1, s+2 in slots s%4 (a stage is a chunk of its super-block: slot = c)
     uint4 hdr[NT], hdrn[NT];  // super-block headers: current, next
@@ -514,7 +523,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 template <int MT, int WN>
 __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
-    const Workspace W = workspace_layout(a.m, a.n, a.k);
+    const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
@@ -525,7 +534,7 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     uint32_t gn = n0 + wn * 32 + l32;
     gn = gn < a.n ? gn : a.n - 1u;
     const uint8_t* blk0 = a.w + (size_t)gn * (a.k / 32) * Q8_0_BYTES + lg * Q8_0_BYTES;  // this lane's block of stage 0
-    const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[gn];
+    const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[a.wd_off + gn];
     const bool early = (reinterpret_cast<uintptr_t>(blk0) & 2u) == 0;  // blocks at 4n: the int8 start two bytes into a word
     const uint32_t shift = early ? 2u : 0u;
     const uint8_t* win0 = early ? blk0 : blk0 + 2;                     // first of the eight aligned words
@@ -628,7 +637,7 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 template <int MT, int WN>
 __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
-    const Workspace W = workspace_layout(a.m, a.n, a.k);
+    const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
@@ -639,7 +648,7 @@ __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     uint32_t gn = n0 + wn * 32 + l32;
     gn = gn < a.n ? gn : a.n - 1u;
     const uint8_t* wrow = a.w + (size_t)gn * nsb * Q6K_BYTES;
-    const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[gn];
+    const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[a.wd_off + gn];
     struct Raw { uint4 l0, l1, h0, h1; uint2 sc; uint32_t d; };  // one half of a super-block, this lane's share
     Raw braw[2];
     auto load_half = [&](uint32_t sb, int h, int slot) {
@@ -784,19 +793,148 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80_gemm_kernel(GemmArgs a) {
     q80_gemm_tile<8, 4>(a, m0, n0);
 }
 
+// ---- grouped (expert) form -------------------------------------------------------------------
+// Routed rows are sorted by expert; every expert's run of rows is cut into tiles of BM rows, and a
+// workgroup multiplies one such tile with BN_WIDE weight rows of that expert.  Workspace beyond the
+// dense layout (for P routed rows and n_experts * n weight rows): row_map[P], the tile table (one
+// uint4 per tile: expert, first row, end of the expert's rows) and the tile count.
+struct GroupedLayout {
+    Workspace base;
+    size_t row_map, tiles, count, total;
+    uint32_t max_tiles;
+};
+__host__ __device__ inline GroupedLayout grouped_layout(uint32_t pairs, uint32_t n_experts, uint32_t n, uint32_t k) {
+    GroupedLayout g;
+    g.base = workspace_layout(pairs, n_experts * n, k);
+    g.max_tiles = pairs / BM + n_experts;
+    g.row_map = g.base.total;
+    g.tiles = g.row_map + (((size_t)pairs * 4 + 255) & ~(size_t)255);
+    g.count = g.tiles + (((size_t)g.max_tiles * 16 + 255) & ~(size_t)255);
+    g.total = g.count + 256;
+    return g;
+}
+
+constexpr uint32_t BUCKET_MAX_EXPERTS = 4096;
+
+// One workgroup: counting sort of the routed rows by expert.  Rows whose id is not an expert get NaN
+// outputs here and take no part in the product.  The order of the rows inside an expert's run depends
+// on the order in which the atomics land; every output row is computed on its own, so the results do not.
+__global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __restrict__ ids, uint32_t pairs, uint32_t n_experts,
+                                                          uint32_t* __restrict__ row_map, uint4* __restrict__ tiles,
+                                                          uint32_t* __restrict__ n_tiles, float* __restrict__ y, uint32_t n) {
+    __shared__ uint32_t cnt[BUCKET_MAX_EXPERTS], cur[BUCKET_MAX_EXPERTS];
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t e = tid; e < n_experts; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (uint32_t p = tid; p < pairs; p += 1024) {
+        const uint32_t e = ids[p];
+        if (e < n_experts) atomicAdd(&cnt[e], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t off = 0, nt = 0;
+        for (uint32_t e = 0; e < n_experts; ++e) {
+            const uint32_t c = cnt[e];
+            cur[e] = off;
+            for (uint32_t r = 0; r < c; r += BM) tiles[nt++] = make_uint4(e, off + r, off + c, 0u);
+            off += c;
+        }
+        *n_tiles = nt;
+    }
+    __syncthreads();
+    for (uint32_t p = tid; p < pairs; p += 1024) {
+        const uint32_t e = ids[p];
+        if (e < n_experts) {
+            row_map[atomicAdd(&cur[e], 1u)] = p;
+        } else {
+            for (uint32_t c = 0; c < n; ++c) y[(size_t)p * n + c] = __uint_as_float(0x7fc00000u);
+        }
+    }
+    // rows of the workspace past the sorted ones (invalid ids leave a gap at the end) point at row 0
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t valid = 0;
+        for (uint32_t e = 0; e < n_experts; ++e) valid += cnt[e];
+        for (uint32_t r = valid; r < pairs; ++r) row_map[r] = 0;
+    }
+}
+
+template <int TYPE>
+__global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a, const uint4* __restrict__ tiles,
+                                                                      const uint32_t* __restrict__ n_tiles, uint32_t tiles_n,
+                                                                      uint64_t expert_stride) {
+    const uint32_t t = blockIdx.x / tiles_n, n0 = (blockIdx.x % tiles_n) * BN_WIDE;
+    if (t >= *n_tiles) return;
+    const uint4 tt = tiles[t];
+    a.w += (size_t)tt.x * expert_stride;
+    a.wd_off = tt.x * a.n;
+    a.m = tt.z;  // rows past the expert's run repeat its last row and are not stored
+    if constexpr (TYPE == HQ_Q4_K)
+        q4k_gemm_tile<8, 1, 4>(a, tt.y, n0);
+    else if constexpr (TYPE == HQ_Q6_K)
+        q6k_gemm_tile<8, 4>(a, tt.y, n0);
+    else
+        q80_gemm_tile<8, 4>(a, tt.y, n0);
+}
+
 }  // namespace
 
 size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) { return workspace_layout(m, n, k).total; }
 
+bool gemm_f16_grouped_supported(hq_ggml_type t, uint32_t n, uint32_t k, uint32_t n_experts, uint64_t expert_stride, uint64_t pairs) {
+    if (!gemm_f16_tile_supported(t, k) || n_experts > BUCKET_MAX_EXPERTS || pairs > 0x7fffffffull / 4) return false;
+    const uint64_t row_bytes = t == HQ_Q4_K ? (uint64_t)(k / 256) * Q4K_BYTES : t == HQ_Q6_K ? (uint64_t)(k / 256) * Q6K_BYTES
+                                                                                              : (uint64_t)(k / 32) * Q8_0_BYTES;
+    // the pre-pass walks the stack as one matrix of n_experts * n rows
+    return expert_stride == (uint64_t)n * row_bytes && (uint64_t)n_experts * n <= 0x7fffffffull;
+}
+
+size_t gemm_f16_grouped_workspace_bytes(uint32_t pairs, uint32_t n_experts, uint32_t n, uint32_t k) {
+    return grouped_layout(pairs, n_experts, n, k).total;
+}
+
 template <int TYPE>
 static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, uint8_t* ws, uint32_t m,
-                       uint32_t n, uint32_t k) {
+                       uint32_t n, uint32_t k, const uint32_t* row_map = nullptr, uint32_t top_k = 1) {
     const dim3 prep_grid(m + (n + 15u) / 16u);
     if (xdt == HQ_BF16)
-        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k);
+        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, row_map, top_k);
     else
-        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k);
+        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, row_map, top_k);
     return check_launch("tile gemm pre-pass launch");
+}
+
+template <int TYPE>
+static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, const uint32_t* ids, float* y,
+                            uint8_t* ws, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
+                            uint64_t expert_stride) {
+    const uint32_t pairs = n_tokens * top_k;
+    const GroupedLayout G = grouped_layout(pairs, n_experts, n, k);
+    uint32_t* row_map = reinterpret_cast<uint32_t*>(ws + G.row_map);
+    uint4* tiles = reinterpret_cast<uint4*>(ws + G.tiles);
+    uint32_t* n_tiles = reinterpret_cast<uint32_t*>(ws + G.count);
+    hipLaunchKernelGGL(moe_bucket_kernel, dim3(1), dim3(1024), 0, s, ids, pairs, n_experts, row_map, tiles, n_tiles, y, n);
+    if (int rc = check_launch("expert bucket kernel launch")) return rc;
+    if (int rc = launch_prep<TYPE>(s, x, xdt, wb, ws, pairs, n_experts * n, k, row_map, top_k)) return rc;
+    constexpr int lds = 2 * ActTile::kTile;
+    auto kern = grouped_gemm_kernel<TYPE>;
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(grouped gemm LDS)"))
+        return rc;
+    GemmArgs a{ws, wb, y, pairs, n, k, pairs, n_experts * n, 0u, row_map};
+    const uint32_t tiles_n = (n + BN_WIDE - 1) / BN_WIDE;
+    hipLaunchKernelGGL(kern, dim3(G.max_tiles * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
+    return check_launch("grouped gemm kernel launch");
+}
+
+int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_stack, const uint32_t* ids, float* y,
+                            void* workspace, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
+                            uint64_t expert_stride, hq_ggml_type t) {
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const uint8_t* wb = static_cast<const uint8_t*>(w_stack);
+    if (t == HQ_Q4_K) return launch_grouped_t<HQ_Q4_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+    if (t == HQ_Q6_K) return launch_grouped_t<HQ_Q6_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+    return launch_grouped_t<HQ_Q8_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
 }
 
 bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {
@@ -807,7 +945,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
                          uint32_t n, uint32_t k, hq_ggml_type t, void* workspace) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const uint8_t* wb = static_cast<const uint8_t*>(w);
-    GemmArgs a{ws, wb, y, m, n, k};
+    GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr};
     constexpr int lds = 2 * ActTile::kTile;
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);

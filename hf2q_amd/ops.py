@@ -153,6 +153,12 @@ def id_scratch_bytes(n_experts: int, max_rows: int) -> int:
     return _l.load().hq_qmatmul_id_scratch_bytes(n_experts, max_rows)
 
 
+def quantized_matmul_id_workspace_bytes(params) -> int:
+    """Device scratch quantized_matmul_id_ggml(..., scratch=) can use for this shape (0: per-row GEMVs)."""
+    return _l.load().hq_qmatmul_id_ggml_workspace_bytes(params.n_tokens, params.top_k, params.n, params.k,
+                                                        params.n_experts, params.expert_stride, params.ggml_type)
+
+
 def dequantize_ggml(weight: torch.Tensor, n_elems: int, ggml_type: int,
                     dtype: torch.dtype = torch.float32) -> torch.Tensor:
     out = torch.empty(n_elems, dtype=dtype, device=weight.device)
@@ -536,6 +542,15 @@ class MoeFfnScratch:
         self.down = f(T * K, w.hidden)
         self.sh_gate, self.sh_up, self.sh_act = f(T, w.shared_inter), f(T, w.shared_inter), f(T, w.shared_inter)
         self.sh_down = f(T, w.hidden)
+        # workspace of the grouped (expert-sorted) form that prefill-sized mul_mat_id calls take (IdMmScratch, decode_pool.rs:56-60)
+        rb_h, rb_i = ggml_row_bytes(w.ggml_type, w.hidden), ggml_row_bytes(w.ggml_type, w.inter)
+        need = max(
+            quantized_matmul_id_workspace_bytes(GgmlQuantizedMatmulIdParams(T, K, w.inter, w.hidden, w.n_experts,
+                                                                            w.inter * rb_h, w.ggml_type)),
+            quantized_matmul_id_workspace_bytes(GgmlQuantizedMatmulIdParams(T * K, 1, w.hidden, w.inter, w.n_experts,
+                                                                            w.hidden * rb_i, w.ggml_type)))
+        self.id_mm = torch.empty(need, dtype=torch.uint8, device=device) if need else None
+        self.max_tokens = T
 
 
 # Dense products above this many rows take the tile (GEMM) route, which the batched launch does not cover.
@@ -586,14 +601,15 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
     dispatch_silu_mul(s.sh_gate[:T], s.sh_up[:T], s.sh_act[:T])
     # C
     pid = GgmlQuantizedMatmulIdParams(T, K, I, H, E, I * rb, t)
-    quantized_matmul_id_ggml(x, w.expert_gate, s.ids, s.gate, pid)
-    quantized_matmul_id_ggml(x, w.expert_up, s.ids, s.up, pid)
+    ws = s.id_mm  # sized for max_tokens; fewer tokens need less (or none: decode-sized calls take the GEMV form)
+    quantized_matmul_id_ggml(x, w.expert_gate, s.ids, s.gate, pid, scratch=ws)
+    quantized_matmul_id_ggml(x, w.expert_up, s.ids, s.up, pid, scratch=ws)
     quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, GgmlQuantizedMatmulParams(T, H, SI, t))
     # D
     dispatch_silu_mul(s.gate[:T * K], s.up[:T * K], s.act[:T * K])
     # E
     quantized_matmul_id_ggml(s.act, w.expert_down, s.ids, s.down,
-                             GgmlQuantizedMatmulIdParams(T * K, 1, H, I, E, H * ggml_row_bytes(t, I), t))
+                             GgmlQuantizedMatmulIdParams(T * K, 1, H, I, E, H * ggml_row_bytes(t, I), t), scratch=ws)
     # F
     dispatch_moe_weighted_reduce(s.down, s.topk_w, out, T, K, H, shared=s.sh_down, shared_logit=s.sh_logit,
                                  residual=residual)

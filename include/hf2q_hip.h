@@ -116,16 +116,26 @@ HQ_API int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, con
  * expert_stride, ggml_type}.  The "down" projection is the same call with
  * n_tokens = T*K, top_k = 1 (forward_mlx.rs:650-651).  An id >= n_experts
  * makes the affected output rows NaN instead of reading out of bounds.
- * `scratch` (device, hq_qmatmul_id_scratch_bytes) is only needed once
- * n_tokens*top_k exceeds the GEMV limit; it may be NULL below that. */
+ * Decode-sized calls run one dequant-fused GEMV per routed row and use no
+ * scratch.  With at least 8 routed rows per expert (prefill) and a `scratch`
+ * of hq_qmatmul_id_ggml_workspace_bytes() bytes (device, 256-byte aligned),
+ * the rows are sorted by expert and every expert's rows go through the tile
+ * GEMM of the m > 8 route (the reference's mul_mm_id, forward_mlx.rs:5237-5245);
+ * that form needs a contiguous stack (expert_stride = one expert's bytes).
+ * With scratch == NULL every size takes the GEMV form. */
 HQ_API int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_stack,
                        const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes,
                        uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
                        uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
 
-/* Bytes of `scratch` hq_qmatmul_id_ggml needs for up to `max_rows` =
- * n_tokens*top_k routed rows (the IdMmScratch analogue, decode_pool.rs:56-60). */
+/* Bytes of `scratch` the GEMV form needs for up to `max_rows` = n_tokens*top_k
+ * routed rows (the IdMmScratch analogue, decode_pool.rs:56-60): none. */
 HQ_API size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows);
+/* Bytes of `scratch` for this call's shape: 0 where the GEMV form is used, else
+ * the grouped form's workspace (sorted f16 activations, row and weight-row
+ * scales, the row permutation and the tile table). */
+HQ_API size_t hq_qmatmul_id_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
+                                          uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
 
 /* Up to HQ_QMATMUL_BATCH_MAX_JOBS independent decode-sized products of one weight
  * type and activation dtype in ONE launch.  The reference encodes the dispatches

@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from _util import acts, assert_matmul_close, weights
+from _util import assert_matmul_close_f16_tile
 from hf2q_amd import ops
 from hf2q_amd.ops import (HQ_Q4_K, HQ_Q6_K, HQ_Q8_0, GgmlQuantizedMatmulIdParams, GgmlQuantizedMatmulParams)
 
@@ -226,3 +227,82 @@ def test_mul_mat_id_many_rows(oracle, dev):
                                  torch.from_numpy(ids.view(np.int32)).to(dev), y,
                                  GgmlQuantizedMatmulIdParams(T, K, n, k, E, stride, t))
     assert_matmul_close(y.cpu().numpy(), ref, "mul_mat_id 384 rows")
+
+
+# ---- grouped (expert-sorted) tile GEMM for prefill-sized mul_mat_id -------------------
+
+GROUPED_CASES = [  # (E, n, k, T, K): at least 8 routed rows per expert and 256 rows
+    (8, 128, 512, 64, 4),      # 32 rows per expert: one partly filled tile each
+    (4, 160, 256, 400, 3),     # 300 rows per expert: two tiles each, n not a multiple of the tile
+    (16, 64, 1024, 300, 1),    # the down-projection calling form
+    (3, 256, 512, 700, 2),     # several full tiles
+]
+
+
+def _grouped_setup(oracle, dev, t, E, n, k, T, K, xdt, seed=0, skew=False):
+    rng = np.random.default_rng(seed + E * n + k + T)
+    base = min(E, 4)
+    blocks = oracle.quantize(weights(E + n + seed, base * n, k), k, t, threads=8)
+    stride = n * ops.ggml_row_bytes(t, k)
+    stack = np.concatenate([blocks[(e % base) * stride:(e % base + 1) * stride] for e in range(E)])
+    if skew:  # most rows to one expert, some experts unused
+        ids = np.where(rng.random(T * K) < 0.7, 1, rng.integers(0, max(1, E // 2), size=T * K)).astype(np.uint32)
+    else:
+        ids = rng.integers(0, E, size=T * K).astype(np.uint32)
+    x = acts(k + seed, T, k)
+    xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
+    xd = torch.from_numpy(x).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    p = GgmlQuantizedMatmulIdParams(T, K, n, k, E, stride, t)
+    return stack, ids, xv, xd, p
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("E,n,k,T,K", GROUPED_CASES)
+def test_mul_mat_id_grouped_matches_oracle(oracle, dev, t, xdt, E, n, k, T, K):
+    if t == HQ_Q8_0 and k % 128:
+        pytest.skip("Q8_0 tile kernel needs k % 128 == 0")
+    stack, ids, xv, xd, p = _grouped_setup(oracle, dev, t, E, n, k, T, K, xdt)
+    need = ops.quantized_matmul_id_workspace_bytes(p)
+    assert need > 0, "this shape must take the grouped route"
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    ref = oracle.qmatmul_id_f64(xv, stack, ids, T, K, n, k, E, p.expert_stride, t)
+    y = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(xd, torch.from_numpy(stack).to(dev), torch.from_numpy(ids.view(np.int32)).to(dev), y, p,
+                                 scratch=scratch)
+    # the tile GEMM rounds every dequantised weight (and f32 activations) once to f16: its own gate
+    assert_matmul_close_f16_tile(y.cpu().numpy(), ref, f"grouped mul_mat_id t={t} {xdt}")
+
+
+def test_mul_mat_id_grouped_routing_properties(oracle, dev):
+    """Skewed routing with unused experts, an id that is no expert (NaN rows, the others untouched), agreement with
+    the per-row GEMV form, a scratch that is too small, and a strided stack (which keeps the GEMV form)."""
+    t, E, n, k, T, K = HQ_Q4_K, 8, 128, 512, 200, 2
+    stack, ids, xv, xd, p = _grouped_setup(oracle, dev, t, E, n, k, T, K, "bf16", seed=5, skew=True)
+    need = ops.quantized_matmul_id_workspace_bytes(p)
+    assert need > 0
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    sd = torch.from_numpy(stack).to(dev)
+    idd = torch.from_numpy(ids.view(np.int32)).to(dev)
+    ref = oracle.qmatmul_id_f64(xv, stack, ids, T, K, n, k, E, p.expert_stride, t)
+    y = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(xd, sd, idd, y, p, scratch=scratch)
+    assert_matmul_close_f16_tile(y.cpu().numpy(), ref, "grouped, skewed routing")
+    y_gemv = torch.empty_like(y)
+    ops.quantized_matmul_id_ggml(xd, sd, idd, y_gemv, p)  # no scratch: one GEMV per row
+    assert_matmul_close(y_gemv.cpu().numpy(), ref, "gemv form")
+    assert np.abs(y.cpu().numpy() - y_gemv.cpu().numpy()).max() <= 1e-3 * np.abs(ref).max()
+    bad = idd.clone()
+    bad[[7, 150]] = E + 3
+    y_bad = torch.zeros_like(y)
+    ops.quantized_matmul_id_ggml(xd, sd, bad, y_bad, p, scratch=scratch)
+    keep = np.setdiff1d(np.arange(T * K), [7, 150])
+    assert torch.isnan(y_bad[[7, 150]]).all() and torch.equal(y_bad[keep], y[keep])
+    with pytest.raises(ops.HqError) as e:
+        ops.quantized_matmul_id_ggml(xd, sd, idd, y, p, scratch=scratch[:need - 256])
+    assert e.value.status == 1
+    padded = GgmlQuantizedMatmulIdParams(T, K, n, k, E, p.expert_stride + 16, t)
+    assert ops.quantized_matmul_id_workspace_bytes(padded) == 0
+    small = GgmlQuantizedMatmulIdParams(8, 2, n, k, E, p.expert_stride, t)
+    assert ops.quantized_matmul_id_workspace_bytes(small) == 0

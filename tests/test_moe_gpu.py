@@ -108,6 +108,41 @@ def test_moe_block_matches_cpu_spec(oracle, dev, T, t):
     assert np.abs(out.cpu().numpy() - (want + res)).max() <= 2e-4 * np.abs(want + res).max()
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0])
+def test_moe_block_prefill_sized_matches_cpu_spec(oracle, dev, t):
+    """A prefill-sized block (48 rows per expert): the three mul_mat_id products take the expert-sorted tile GEMM
+    and the dense ones the m > 8 route, both of which round the weights once to f16; a smaller call through the
+    same scratch falls back to the per-row form."""
+    H, E, K, I, SI, T = 512, 8, 4, 256, 256, 96
+    rng = np.random.default_rng(171)
+    bf = lambda a: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(a))  # noqa: E731
+    router = bf((rng.standard_normal((E, H)) * 0.1).astype(np.float32))
+    sgl = bf((rng.standard_normal((1, H)) * 0.05).astype(np.float32))
+    raw = {nm: weights(seed, n, k, 0.05) for nm, seed, n, k in
+           (("eg", 1, E * I, H), ("eu", 2, E * I, H), ("ed", 3, E * H, I), ("sg", 4, SI, H), ("su", 5, SI, H), ("sd", 6, H, SI))}
+    q = {nm: oracle.quantize(a, a.shape[1], t, threads=8) for nm, a in raw.items()}
+    dq = {nm: oracle.dequantize(q[nm], t).reshape(raw[nm].shape) for nm in raw}
+    x = acts(7, T, H)
+    want = oracle.moe_ffn(x, H, E, K, I, SI, router, dq["eg"], dq["eu"], dq["ed"], sgl[0], dq["sg"], dq["su"], dq["sd"])
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    w = ops.MoeFfnWeightsGpuQ(dv(router).to(torch.bfloat16), dv(q["eg"]), dv(q["eu"]), dv(q["ed"]),
+                              dv(sgl).to(torch.bfloat16), dv(q["sg"]), dv(q["su"]), dv(q["sd"]), t, H, E, K, I, SI)
+    s = ops.MoeFfnScratch(w, T, dev)
+    assert s.id_mm is not None and s.id_mm.numel() > 0
+    out = torch.full((T, H), float("nan"), device=dev)
+    ops.build_moe_ffn_layer_gpu_q_into(dv(x), w, s, out)
+    got = out.cpu().numpy()
+    scale = np.abs(want).max()
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= 2e-3 * scale, np.abs(got - want).max() / scale
+    rms = np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    # two f16-rounded products in sequence (gate / up, then down): a few 1e-4 of the rms each
+    assert np.sqrt(np.mean((got - want).astype(np.float64) ** 2)) <= 2e-3 * rms
+    out12 = torch.full((12, H), float("nan"), device=dev)
+    ops.build_moe_ffn_layer_gpu_q_into(dv(x[:12]), w, s, out12)
+    assert np.abs(out12.cpu().numpy() - want[:12]).max() <= 2e-3 * scale
+
+
 def _moe_weights(oracle, dev, t, H, E, K, I, SI, seed=0):
     rng = np.random.default_rng(300 + seed)
     bf = lambda a: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(a))  # noqa: E731
