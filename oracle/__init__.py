@@ -17,9 +17,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libhf2q_oracle.so")
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256}
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210}
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14  # ggml_type.rs:18-53
+BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256}
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210}
 
 # kv_cache.rs:3871-3876 (same 32 bytes as in hf2q_oracle.c; kept here so tests
 # can build the explicit sign vector independently of the C code).

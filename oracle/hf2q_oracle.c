@@ -14,9 +14,10 @@
  * the hf2q source tree).
  *
  * How each function is pinned (what a wrong sign / index / dropped term trips):
- *   quantize_q4_k / q6_k / q8_0 .... byte equality with the reference's twelve
- *       committed golden files tests/fixtures/ggml_quants/{q4_k_512,q6_k_512,
- *       q8_0_64}_{noim,im}_{input,expected}.bin (tests/test_oracle_golden.py).
+ *   quantize_q4_k / q6_k / q8_0 / q5_k / q4_0 .... byte equality with the
+ *       reference's committed golden files tests/fixtures/ggml_quants/{q4_k_512,
+ *       q6_k_512,q8_0_64,q5_k_512,q4_0_64}_{noim,im}_{input,expected}.bin
+ *       (tests/test_oracle_golden.py).
  *   nearest_int ..................... the RNE table of common.rs:525-539.
  *   dequantize_* .................... exact-rational evaluation of the block
  *       formula rounded once to f32 (Python fractions), RMSE of the golden
@@ -44,6 +45,9 @@
 #define Q6K_BYTES 210
 #define QK8_0 32
 #define Q8_0_BYTES 34
+#define Q5K_BYTES 176
+#define QK4_0 32
+#define Q4_0_BYTES 18
 #define GROUP_MAX_EPS 1e-15f /* common.rs:15 */
 
 /* ------------------------------------------------------------------ */
@@ -440,6 +444,144 @@ static void q4k_quantize_block(const float *xb, const float *qw, uint8_t *out) {
         for (int l = 0; l < 32; l++) *q++ = (uint8_t)(L[j + l] | (L[j + l + 32] << 4));
 }
 
+/* q5_k.rs:160-243 (quantize_row_q5_k_ref) and :246-311 (quantize_row_q5_k_impl) with the common
+ * tail finalize_block (q5_k.rs:88-157), one super-block.  `qw` is the imatrix slice or NULL. */
+static void q5k_quantize_block(const float *xb, const float *qw, uint8_t *out) {
+    uint8_t L[QK_K], Laux[32], ls_arr[8], lm_arr[8];
+    float weights[32], mins[8], scales[8], sw[8];
+    uint8_t packed[K_SCALE_SIZE];
+    memset(packed, 0, sizeof packed);
+    memset(L, 0, sizeof L);
+    float d_blk, dmin_blk;
+    if (!qw) {
+        float max_scale = 0.0f, max_min = 0.0f;
+        for (int j = 0; j < 8; j++) {
+            const float *sub = xb + 32 * j;
+            float sum_x2 = 0.0f;
+            for (int l = 0; l < 32; l++) sum_x2 = fmaf(sub[l], sub[l], sum_x2); /* q5_k.rs:183 */
+            float av_x = sqrtf(sum_x2 / 32.0f);
+            for (int l = 0; l < 32; l++) weights[l] = av_x + fabsf(sub[l]);
+            scales[j] = make_qkx_quants(0, 32, 31, sub, weights, L + 32 * j, &mins[j], Laux, -0.5f,
+                                        0.1f, 15, 0);
+            if (scales[j] > max_scale) max_scale = scales[j];
+            if (mins[j] > max_min) max_min = mins[j];
+        }
+        float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+        float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+        for (int j = 0; j < 8; j++) {
+            uint8_t ls = (uint8_t)nearest_int(inv_scale * scales[j]);
+            uint8_t lm = (uint8_t)nearest_int(inv_min * mins[j]);
+            ls_arr[j] = ls > 63 ? 63 : ls;
+            lm_arr[j] = lm > 63 ? 63 : lm;
+        }
+        d_blk = max_scale / 63.0f;
+        dmin_blk = max_min / 63.0f;
+    } else {
+        float sum_x2 = 0.0f;
+        for (int l = 0; l < QK_K; l++) sum_x2 = fmaf(xb[l], xb[l], sum_x2); /* q5_k.rs:261 */
+        float sigma2 = 2.0f * sum_x2 / (float)QK_K;
+        for (int j = 0; j < 8; j++) {
+            const float *sub = xb + 32 * j;
+            for (int l = 0; l < 32; l++) weights[l] = qw[32 * j + l] * sqrtf(sigma2 + sub[l] * sub[l]);
+            float sumw = 0.0f;
+            for (int l = 0; l < 32; l++) sumw += weights[l];
+            sw[j] = sumw;
+            scales[j] = make_qkx_quants(1, 32, 31, sub, weights, L + 32 * j, &mins[j], Laux, -0.9f,
+                                        0.05f, 36, 0);
+        }
+        d_blk = make_qp_quants(8, 63, scales, ls_arr, sw);
+        dmin_blk = make_qp_quants(8, 63, mins, lm_arr, sw);
+        for (int j = 0; j < 8; j++) {
+            if (ls_arr[j] > 63) ls_arr[j] = 63;
+            if (lm_arr[j] > 63) lm_arr[j] = 63;
+        }
+    }
+    for (int j = 0; j < 8; j++) { /* q5_k.rs:72-82 pack_scale_min_k4 */
+        uint8_t ls = ls_arr[j], lm = lm_arr[j];
+        if (j < 4) {
+            packed[j] = ls;
+            packed[j + 4] = lm;
+        } else {
+            packed[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+            packed[j - 4] |= (uint8_t)((ls >> 4) << 6);
+            packed[j] |= (uint8_t)((lm >> 4) << 6);
+        }
+    }
+    uint16_t d16 = f32_to_f16_bits(d_blk), dmin16 = f32_to_f16_bits(dmin_blk);
+    float d_dq = f16_bits_to_f32(d16), dmin_dq = f16_bits_to_f32(dmin16);
+    for (int j = 0; j < 8; j++) { /* q5_k.rs:108-120: sub-blocks with d == 0 keep the search's L */
+        uint8_t sc, m;
+        get_scale_min_k4(j, packed, &sc, &m);
+        float d = d_dq * (float)sc;
+        if (d == 0.0f) continue;
+        float dm = dmin_dq * (float)m;
+        for (int ii = 0; ii < 32; ii++) {
+            int l = nearest_int((xb[32 * j + ii] + dm) / d);
+            L[32 * j + ii] = (uint8_t)imax(0, imin(31, l));
+        }
+    }
+    out[0] = (uint8_t)(d16 & 0xFF);
+    out[1] = (uint8_t)(d16 >> 8);
+    out[2] = (uint8_t)(dmin16 & 0xFF);
+    out[3] = (uint8_t)(dmin16 >> 8);
+    memcpy(out + 4, packed, K_SCALE_SIZE);
+    uint8_t *qh = out + 16, *ql = out + 48;
+    memset(qh, 0, 32);
+    uint8_t m1 = 1, m2 = 2;
+    for (int n = 0; n < QK_K; n += 64) { /* q5_k.rs:138-157 */
+        for (int j = 0; j < 32; j++) {
+            int l1 = L[n + j], l2 = L[n + j + 32];
+            if (l1 > 15) {
+                l1 -= 16;
+                qh[j] |= m1;
+            }
+            if (l2 > 15) {
+                l2 -= 16;
+                qh[j] |= m2;
+            }
+            ql[j] = (uint8_t)(l1 | (l2 << 4));
+        }
+        ql += 32;
+        m1 = (uint8_t)(m1 << 2);
+        m2 = (uint8_t)(m2 << 2);
+    }
+}
+
+/* q4_0.rs:13-50 quantize_row_ref, one block of 32. */
+static void q4_0_quantize_block(const float *xb, uint8_t *out) {
+    float amax = 0.0f, max = 0.0f;
+    for (int j = 0; j < QK4_0; j++) {
+        float v = xb[j];
+        if (amax < fabsf(v)) {
+            amax = fabsf(v);
+            max = v;
+        }
+    }
+    float d = max / -8.0f;
+    float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint16_t d16 = f32_to_f16_bits(d);
+    out[0] = (uint8_t)(d16 & 0xFF);
+    out[1] = (uint8_t)(d16 >> 8);
+    for (int j = 0; j < QK4_0 / 2; j++) {
+        float x0 = xb[j] * id, x1 = xb[QK4_0 / 2 + j] * id;
+        int8_t a = (int8_t)(x0 + 8.5f), b = (int8_t)(x1 + 8.5f); /* truncating casts */
+        uint8_t xi0 = (uint8_t)(a < 15 ? a : 15), xi1 = (uint8_t)(b < 15 ? b : 15);
+        out[2 + j] = (uint8_t)(xi0 | (xi1 << 4));
+    }
+}
+
+/* q4_0.rs:52-87 quantize_row_impl, one block of a row whose sigma2 = sum(x^2) / n_per_row. */
+static void q4_0_quantize_block_im(const float *xb, const float *qw, float sigma2, uint8_t *out) {
+    float weight[QK4_0];
+    int8_t L[QK4_0];
+    for (int j = 0; j < QK4_0; j++) weight[j] = qw[j] * sqrtf(sigma2 + xb[j] * xb[j]);
+    float d = make_qx_quants(QK4_0, 8, xb, L, 1, weight);
+    uint16_t d16 = f32_to_f16_bits(d);
+    out[0] = (uint8_t)(d16 & 0xFF);
+    out[1] = (uint8_t)(d16 >> 8);
+    for (int j = 0; j < 16; j++) out[2 + j] = (uint8_t)((uint8_t)L[j] | ((uint8_t)L[j + 16] << 4));
+}
+
 /* q6_k.rs:40-151 quantize_one_block. */
 static void q6k_quantize_block(const float *xb, const float *qw, uint8_t *out) {
     int8_t L[QK_K];
@@ -507,11 +649,14 @@ static void q8_0_quantize_block(const float *xb, uint8_t *out) {
     }
 }
 
-enum { T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14 }; /* ggml_type.rs:18-53 */
+enum { T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14 }; /* ggml_type.rs:18-53 */
 
-static int block_elems(int t) { return t == T_Q8_0 ? 32 : (t == T_Q4_K || t == T_Q6_K) ? 256 : 0; }
+static int block_elems(int t) {
+    return (t == T_Q8_0 || t == T_Q4_0) ? 32 : (t == T_Q4_K || t == T_Q5_K || t == T_Q6_K) ? 256 : 0;
+}
 static int block_bytes(int t) {
-    return t == T_Q8_0 ? Q8_0_BYTES : t == T_Q4_K ? Q4K_BYTES : t == T_Q6_K ? Q6K_BYTES : 0;
+    return t == T_Q8_0 ? Q8_0_BYTES : t == T_Q4_K ? Q4K_BYTES : t == T_Q6_K ? Q6K_BYTES
+           : t == T_Q5_K ? Q5K_BYTES : t == T_Q4_0 ? Q4_0_BYTES : 0;
 }
 
 /* quantizer.rs:51-102 dispatch + q4_k.rs:50-86 / q6_k.rs:181-221 / q8_0.rs:31-72.
@@ -532,9 +677,20 @@ int hq_oracle_quantize(const float *src, int64_t n_elems, int64_t n_per_row, int
         const float *qw = imatrix ? imatrix + in_row * be : NULL;
         if (ggml_type == T_Q4_K)
             q4k_quantize_block(xb, qw, ob);
+        else if (ggml_type == T_Q5_K)
+            q5k_quantize_block(xb, qw, ob);
         else if (ggml_type == T_Q6_K)
             q6k_quantize_block(xb, qw, ob);
-        else
+        else if (ggml_type == T_Q4_0) {
+            if (qw) { /* q4_0.rs:61-65: the row's mean square enters every block's weights */
+                const float *row = src + (b / blocks_per_row) * n_per_row;
+                float sum_x2 = 0.0f;
+                for (int64_t j = 0; j < n_per_row; j++) sum_x2 += row[j] * row[j];
+                q4_0_quantize_block_im(xb, qw, sum_x2 / (float)n_per_row, ob);
+            } else {
+                q4_0_quantize_block(xb, ob);
+            }
+        } else
             q8_0_quantize_block(xb, ob);
     }
     return 0;
@@ -588,6 +744,38 @@ static void q6k_dequant_block(const uint8_t *b, float *y) {
     }
 }
 
+/* Inverse of q5_k.rs:108-157: y = d*sc*(ql + 16*hbit) - dmin*m; d*sc*q (11 + 6 + 5 bits) and
+ * dmin*m are exact in f32, so y is one rounding of an exact difference. */
+static void q5k_dequant_block(const uint8_t *b, float *y) {
+    float d = f16_bits_to_f32((uint16_t)(b[0] | (b[1] << 8)));
+    float dmin = f16_bits_to_f32((uint16_t)(b[2] | (b[3] << 8)));
+    const uint8_t *qh = b + 16, *ql = b + 48;
+    int is = 0;
+    uint8_t u1 = 1, u2 = 2;
+    for (int j = 0; j < QK_K; j += 64) {
+        uint8_t sc, m;
+        get_scale_min_k4(is, b + 4, &sc, &m);
+        float d1 = d * (float)sc, m1 = dmin * (float)m;
+        get_scale_min_k4(is + 1, b + 4, &sc, &m);
+        float d2 = d * (float)sc, m2 = dmin * (float)m;
+        for (int l = 0; l < 32; l++) y[j + l] = d1 * (float)((ql[l] & 0xF) + ((qh[l] & u1) ? 16 : 0)) - m1;
+        for (int l = 0; l < 32; l++) y[j + 32 + l] = d2 * (float)((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - m2;
+        ql += 32;
+        is += 2;
+        u1 = (uint8_t)(u1 << 2);
+        u2 = (uint8_t)(u2 << 2);
+    }
+}
+
+/* Inverse of q4_0.rs:36-46: y = d * (q - 8), low nibbles are elements 0..15, high 16..31. */
+static void q4_0_dequant_block(const uint8_t *b, float *y) {
+    float d = f16_bits_to_f32((uint16_t)(b[0] | (b[1] << 8)));
+    for (int j = 0; j < 16; j++) {
+        y[j] = d * (float)((int)(b[2 + j] & 0xF) - 8);
+        y[j + 16] = d * (float)((int)(b[2 + j] >> 4) - 8);
+    }
+}
+
 static void q8_0_dequant_block(const uint8_t *b, float *y) {
     float d = f16_bits_to_f32((uint16_t)(b[0] | (b[1] << 8)));
     for (int i = 0; i < QK8_0; i++) y[i] = d * (float)(int8_t)b[2 + i];
@@ -603,8 +791,12 @@ int hq_oracle_dequantize(const uint8_t *blocks, int64_t n_elems, int ggml_type, 
     for (int64_t b = 0; b < nblocks; b++) {
         if (ggml_type == T_Q4_K)
             q4k_dequant_block(blocks + b * bb, out + b * be);
+        else if (ggml_type == T_Q5_K)
+            q5k_dequant_block(blocks + b * bb, out + b * be);
         else if (ggml_type == T_Q6_K)
             q6k_dequant_block(blocks + b * bb, out + b * be);
+        else if (ggml_type == T_Q4_0)
+            q4_0_dequant_block(blocks + b * bb, out + b * be);
         else
             q8_0_dequant_block(blocks + b * bb, out + b * be);
     }

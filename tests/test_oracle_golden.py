@@ -8,8 +8,9 @@ import pytest
 
 from _util import GOLDEN
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-CASES = [("q4_k_512", Q4_K, 512), ("q6_k_512", Q6_K, 512), ("q8_0_64", Q8_0, 64)]
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
+CASES = [("q4_k_512", Q4_K, 512), ("q6_k_512", Q6_K, 512), ("q8_0_64", Q8_0, 64), ("q5_k_512", Q5_K, 512),
+         ("q4_0_64", Q4_0, 64)]
 
 
 def _load(name):
@@ -19,7 +20,7 @@ def _load(name):
 @pytest.mark.parametrize("name,t,npr", CASES)
 @pytest.mark.parametrize("variant", ["noim", "im"])
 def test_quantizer_byte_equal_to_reference_fixture(oracle, name, t, npr, variant):
-    # q4_k.rs:386-403, q6_k.rs:272-289, q8_0.rs:106-125: assert byte equality.
+    # q4_k.rs:386-403, q6_k.rs:272-289, q8_0.rs:106-125, q5_k.rs:395-428, q4_0.rs:196-217: assert byte equality.
     x = _load(f"{name}_{variant}_input.bin").view(np.float32)
     expected = _load(f"{name}_{variant}_expected.bin")
     im = None
@@ -35,6 +36,8 @@ def test_fixture_shapes():
     assert _load("q4_k_512_noim_expected.bin").size == 4 * 144
     assert _load("q6_k_512_noim_expected.bin").size == 4 * 210
     assert _load("q8_0_64_noim_expected.bin").size == 4 * 34
+    assert _load("q5_k_512_noim_expected.bin").size == 4 * 176
+    assert _load("q4_0_64_noim_expected.bin").size == 4 * 18
     assert np.array_equal(_load("q4_k_512_noim_input.bin"), _load("q4_k_512_im_input.bin"))
 
 
@@ -114,6 +117,31 @@ def _ref_dequant_q6k(block):
     return np.array(out, dtype=np.float32)
 
 
+def _ref_dequant_q5k(block):
+    d, dmin = _f16(block[0], block[1]), _f16(block[2], block[3])
+    q = block[4:16]
+    qh, ql = block[16:48], block[48:176]
+    out = []
+    for j in range(8):
+        if j < 4:
+            sc, m = int(q[j]) & 63, int(q[j + 4]) & 63
+        else:
+            sc = (int(q[j + 4]) & 0xF) | ((int(q[j - 4]) >> 6) << 4)
+            m = (int(q[j + 4]) >> 4) | ((int(q[j]) >> 6) << 4)
+        for l in range(32):
+            nib = (int(ql[32 * (j // 2) + l]) >> (4 * (j & 1))) & 0xF
+            hi = (int(qh[l]) >> j) & 1  # bit j of qh[l] belongs to sub-block j
+            out.append(_round_f32(d * int(sc) * (nib + 16 * hi) - dmin * int(m)))
+    return np.array(out, dtype=np.float32)
+
+
+def _ref_dequant_q4_0(block):
+    d = _f16(block[0], block[1])
+    lo = [_round_f32(d * ((int(v) & 0xF) - 8)) for v in block[2:18]]
+    hi = [_round_f32(d * ((int(v) >> 4) - 8)) for v in block[2:18]]
+    return np.array(lo + hi, dtype=np.float32)
+
+
 def _ref_dequant_q8_0(block):
     d = _f16(block[0], block[1])
     return np.array([_round_f32(d * int(v)) for v in block[2:34].view(np.int8)], dtype=np.float32)
@@ -129,12 +157,13 @@ def test_dequant_equals_exact_rational_formula(oracle, name, t, npr):
     bb = oracle.BLOCK_BYTES[t]
     raw = rng.integers(0, 256, size=6 * bb, dtype=np.uint8)
     for i in range(6):  # keep the f16 scale fields finite
-        for off in ([1, 3] if t == Q4_K else [209] if t == Q6_K else [1]):
+        for off in ([1, 3] if t in (Q4_K, Q5_K) else [209] if t == Q6_K else [1]):
             raw[i * bb + off] &= 0x3F
     blocks.append(raw)
     data = np.concatenate(blocks)
     got = oracle.dequantize(data, t)
-    fn = {Q4_K: _ref_dequant_q4k, Q6_K: _ref_dequant_q6k, Q8_0: _ref_dequant_q8_0}[t]
+    fn = {Q4_K: _ref_dequant_q4k, Q6_K: _ref_dequant_q6k, Q8_0: _ref_dequant_q8_0, Q5_K: _ref_dequant_q5k,
+          Q4_0: _ref_dequant_q4_0}[t]
     want = np.concatenate([fn(data[i * bb:(i + 1) * bb]) for i in range(data.size // bb)])
     # exact rationals carry no sign of zero: compare zeros by value, everything else by bits
     nz = want != 0
@@ -144,7 +173,7 @@ def test_dequant_equals_exact_rational_formula(oracle, name, t, npr):
 
 def test_dequant_rmse_known_answers(oracle):
     # RMSE of the reference's golden blocks against their own inputs (uniform[-1,1]).
-    for (name, t, _), want in zip(CASES, (0.03162, 0.00790, 0.00223)):
+    for (name, t, _), want in zip(CASES[:3], (0.03162, 0.00790, 0.00223)):
         x = _load(f"{name}_noim_input.bin").view(np.float32)
         y = oracle.dequantize(_load(f"{name}_noim_expected.bin"), t)
         assert abs(float(np.sqrt(np.mean((x - y) ** 2))) - want) < 2e-5
@@ -158,6 +187,17 @@ def test_q8_0_roundtrip_error_bound(oracle):
     y = oracle.dequantize(b, Q8_0)
     d = b.reshape(-1, 34)[:, :2].copy().view(np.float16).astype(np.float32).repeat(32)
     assert np.all(np.abs(x - y) <= d * 0.5 + np.abs(x) * 2e-3)
+
+
+def test_dequant_rmse_of_the_added_types(oracle):
+    """Round-trip error of the golden blocks against their uniform[-1, 1] inputs: Q5_K has twice the levels of
+    Q4_K (half its error), Q4_0 one scale per 32 with 16 levels: step d = amax / 8, error about d / sqrt(12)."""
+    rm = {}
+    for name, t, _ in CASES:
+        x = _load(f"{name}_noim_input.bin").view(np.float32)
+        rm[t] = float(np.sqrt(np.mean((x - oracle.dequantize(_load(f"{name}_noim_expected.bin"), t)) ** 2)))
+    assert 0.45 < rm[Q5_K] / rm[Q4_K] < 0.55
+    assert 0.030 < rm[Q4_0] < 0.042  # amax ~ 0.97: d ~ 0.121, d / sqrt(12) ~ 0.035
 
 
 @pytest.mark.parametrize("t", [Q4_K, Q6_K, Q8_0])
