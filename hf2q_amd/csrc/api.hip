@@ -26,14 +26,16 @@ int check_hip(hipError_t e, const char* what) {
     return fail(HQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-static bool known_type(hq_ggml_type t) { return t == HQ_Q8_0 || t == HQ_Q4_K || t == HQ_Q6_K; }
+static bool known_type(hq_ggml_type t) {
+    return t == HQ_Q8_0 || t == HQ_Q4_K || t == HQ_Q6_K || t == HQ_Q5_K || t == HQ_Q4_0;
+}
 
 // Largest activation-row count the GEMV kernels take; above it the MFMA GEMM
 // runs (MM_ROUTING_THRESHOLD = 8, src/serve/forward_mlx.rs:9791).
 constexpr uint32_t kGemvMaxRows = 8;
 
 static int check_weight_alignment(const void* w, hq_ggml_type t) {
-    const size_t need = t == HQ_Q4_K ? 16 : 2;
+    const size_t need = (t == HQ_Q4_K || t == HQ_Q5_K) ? 16 : 2;
     if (!is_aligned(w, need))
         return fail(HQ_ERR_INVALID_ARGUMENT, "weight pointer must be %zu-byte aligned for ggml type %d",
                     need, (int)t);
@@ -74,11 +76,12 @@ const char* hq_last_error(void) { return g_err; }
 int hq_version(void) { return 100; }
 
 uint32_t hq_block_elems(hq_ggml_type t) {
-    return t == HQ_Q8_0 ? 32u : (t == HQ_Q4_K || t == HQ_Q6_K) ? 256u : 0u;
+    return (t == HQ_Q8_0 || t == HQ_Q4_0) ? 32u : (t == HQ_Q4_K || t == HQ_Q5_K || t == HQ_Q6_K) ? 256u : 0u;
 }
 
 uint32_t hq_block_bytes(hq_ggml_type t) {
-    return t == HQ_Q8_0 ? Q8_0_BYTES : t == HQ_Q4_K ? Q4K_BYTES : t == HQ_Q6_K ? Q6K_BYTES : 0u;
+    return t == HQ_Q8_0 ? Q8_0_BYTES : t == HQ_Q4_K ? Q4K_BYTES : t == HQ_Q6_K ? Q6K_BYTES : t == HQ_Q5_K ? Q5K_BYTES
+           : t == HQ_Q4_0 ? Q4_0_BYTES : 0u;
 }
 
 int hq_dequant_ggml(void* stream, const void* w_blocks, void* out, hq_act_dtype out_dtype,
@@ -231,7 +234,7 @@ int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void
     if (expert_stride < expert_bytes)
         return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: expert_stride %llu < one expert's %llu bytes",
                     (unsigned long long)expert_stride, (unsigned long long)expert_bytes);
-    if (expert_stride % (t == HQ_Q4_K ? 16 : 2))
+    if (expert_stride % ((t == HQ_Q4_K || t == HQ_Q5_K) ? 16 : 2))
         return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: expert_stride %llu breaks block alignment",
                     (unsigned long long)expert_stride);
     const uint64_t pairs = (uint64_t)n_tokens * top_k;
@@ -299,7 +302,7 @@ int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_j
             if (j.n_experts == 0 || j.top_k == 0)
                 return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: n_experts %u, top_k %u", fn, i, j.n_experts, j.top_k);
             const uint64_t expert_bytes = (uint64_t)j.n * (j.k / hq_block_elems(t)) * hq_block_bytes(t);
-            if (j.expert_stride < expert_bytes || j.expert_stride % (t == HQ_Q4_K ? 16 : 2))
+            if (j.expert_stride < expert_bytes || j.expert_stride % ((t == HQ_Q4_K || t == HQ_Q5_K) ? 16 : 2))
                 return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: expert_stride %llu (one expert is %llu bytes)", fn, i,
                             (unsigned long long)j.expert_stride, (unsigned long long)expert_bytes);
             const uint64_t pairs = (uint64_t)j.rows * j.top_k;

@@ -4,6 +4,7 @@
 // by the second-stage loops of its quantizers (q4_k.rs:185-197:
 // L = (x + dmin*m)/(d*sc); q6_k.rs:97-110: L = x/(d*sc) + 32; q8_0.rs:59-67):
 //   Q4_K  y = (d*sc)*q - dmin*m      Q6_K  y = (d*sc)*(q-32)      Q8_0  y = d*q
+//   Q5_K  as Q4_K with q in 0..31 (q5_k.rs:108-157)              Q4_0  y = d*(q-8) (q4_0.rs:36-46)
 // d*sc, dmin*m and (d*sc)*q (Q4_K) are exact in f32, so each y below is a
 // single rounding of the exact value and does not depend on FMA contraction.
 //
@@ -51,6 +52,34 @@ __device__ __forceinline__ void dequant4(const uint8_t* __restrict__ w, uint64_t
         out[1] = ds * (ubyte1(q) - 32.0f);
         out[2] = ds * (ubyte2(q) - 32.0f);
         out[3] = ds * (ubyte3(q) - 32.0f);
+    } else if constexpr (TYPE == HQ_Q5_K) {  // as Q4_K with a fifth bit: bit (sub-block) of high-bit byte l
+        const uint8_t* blk = w + (e >> 8) * Q5K_BYTES;
+        const uint32_t ib = (uint32_t)e & 255u;
+        const uint32_t c = ib >> 6, hi = (ib >> 5) & 1u, l = ib & 31u;
+        const uint4 hdr = *reinterpret_cast<const uint4*>(blk);
+        const float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
+        uint32_t sc0, sc1, m0, m1;
+        q4k_scales(hdr.y, hdr.z, hdr.w, (int)c, sc0, sc1, m0, m1);
+        const float ds = d * (float)(hi ? sc1 : sc0);
+        const float dm = dmin * (float)(hi ? m1 : m0);
+        uint32_t q = *reinterpret_cast<const uint32_t*>(blk + 48 + 32 * c + l);
+        const uint32_t h = *reinterpret_cast<const uint32_t*>(blk + 16 + l) >> (2 * c + hi);
+        q = ((q >> (4 * hi)) & 0x0f0f0f0fu) | ((h << 4) & 0x10101010u);
+        out[0] = ds * ubyte0(q) - dm;
+        out[1] = ds * ubyte1(q) - dm;
+        out[2] = ds * ubyte2(q) - dm;
+        out[3] = ds * ubyte3(q) - dm;
+    } else if constexpr (TYPE == HQ_Q4_0) {  // y = d * (q - 8); low nibbles elements 0..15, high nibbles 16..31
+        const uint8_t* blk = w + (e >> 5) * Q4_0_BYTES;
+        const uint32_t l = (uint32_t)e & 31u;
+        const float d = f16_bits_to_f32(ld2(blk));
+        uint32_t q;
+        __builtin_memcpy(&q, blk + 2 + (l & 15u), 4);
+        q = (q >> (l & 16u ? 4 : 0)) & 0x0f0f0f0fu;
+        out[0] = d * (ubyte0(q) - 8.0f);
+        out[1] = d * (ubyte1(q) - 8.0f);
+        out[2] = d * (ubyte2(q) - 8.0f);
+        out[3] = d * (ubyte3(q) - 8.0f);
     } else {
         const uint8_t* blk = w + (e >> 5) * Q8_0_BYTES;
         const uint32_t l = (uint32_t)e & 31u;
@@ -100,6 +129,8 @@ int launch_dequant(hipStream_t s, const void* w, void* out, hq_act_dtype odt, ui
         case HQ_Q4_K: return launch_t<HQ_Q4_K>(s, w, out, odt, n_elems);
         case HQ_Q6_K: return launch_t<HQ_Q6_K>(s, w, out, odt, n_elems);
         case HQ_Q8_0: return launch_t<HQ_Q8_0>(s, w, out, odt, n_elems);
+        case HQ_Q5_K: return launch_t<HQ_Q5_K>(s, w, out, odt, n_elems);
+        case HQ_Q4_0: return launch_t<HQ_Q4_0>(s, w, out, odt, n_elems);
     }
     return fail(HQ_ERR_UNSUPPORTED, "dequant: ggml type %d", (int)t);
 }

@@ -37,13 +37,19 @@ namespace hq {
 
 namespace {
 
-constexpr uint32_t M4 = 0x000f000fu, M2 = 0x00300030u, MAGIC = 0x43004300u;
+constexpr uint32_t M4 = 0x000f000fu, M2 = 0x00300030u, M1 = 0x00100010u, MAGIC = 0x43004300u;
+// Types whose block is one lane's piece of 32 weights (the K-quants give a lane 64 of a super-block's 256).
+template <int TYPE>
+constexpr bool kBlock32 = TYPE == HQ_Q8_0 || TYPE == HQ_Q4_0;
+template <int TYPE>
+constexpr uint32_t kBlockBytes = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q5_K ? Q5K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES
+                                 : TYPE == HQ_Q4_0 ? Q4_0_BYTES : Q8_0_BYTES;
 // Tasks (row slot x step) per CU from which the queue kernel takes over.
 constexpr uint32_t QUEUE_MIN_TASKS_PER_CU = 96;
 
 template <int TYPE>
 struct Lane {  // weights per lane and step
-    static constexpr int kElems = TYPE == HQ_Q8_0 ? 32 : 64;
+    static constexpr int kElems = kBlock32<TYPE> ? 32 : 64;
 };
 
 // Per-lane fetch of one piece of row data.
@@ -71,6 +77,26 @@ struct Piece<HQ_Q6_K> {
         qh = ld16_unaligned(blk + 128 + 32 * h + 16 * lr);
         sc = ld8_unaligned(blk + 192 + 8 * h);
         d = ld2(blk + 208);
+    }
+};
+template <>
+struct Piece<HQ_Q5_K> {  // header, the chunk's 32 nibble bytes, all 32 high-bit bytes (bits 2c, 2c+1 are this chunk's)
+    uint4 hdr, q0, q1, h0, h1;
+    __device__ __forceinline__ void load(const uint8_t* blk, int c) {
+        hdr = *reinterpret_cast<const uint4*>(blk);
+        h0 = *reinterpret_cast<const uint4*>(blk + 16);
+        h1 = *reinterpret_cast<const uint4*>(blk + 32);
+        q0 = *reinterpret_cast<const uint4*>(blk + 48 + 32 * c);
+        q1 = *reinterpret_cast<const uint4*>(blk + 64 + 32 * c);
+    }
+};
+template <>
+struct Piece<HQ_Q4_0> {
+    uint4 q;
+    uint32_t d;
+    __device__ __forceinline__ void load(const uint8_t* blk, int) {
+        d = ld2(blk);
+        q = ld16_unaligned(blk + 2);
     }
 };
 template <>
@@ -107,6 +133,30 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q4_K>& p, int c, const 
     const float sl = sx[0] + sx[1], sh = sx[2] + sx[3];
     float acc = d0 * lo - (128.f * d0 + dmin * (float)m0) * sl;
     acc += d1 * hi - (128.f * d1 + dmin * (float)m1) * sh;
+    return acc;
+}
+
+// Q5_K: the fifth bit of element j of sub-blocks 2c / 2c+1 is bit 2c / 2c+1 of high-bit byte j; m1 = 0x00100010
+// arrives in the second mask register.  Values hold 128 + q with q in 0..31.
+__device__ __forceinline__ float dot_pair(const Piece<HQ_Q5_K>& p, int c, const uint32_t* xp, const float* sx,
+                                          uint32_t m4, uint32_t m1, uint32_t magic) {
+    float lo = 0.f, hi = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t w = j < 4 ? word(p.q0, j) : word(p.q1, j - 4);
+        const uint32_t hs = (j < 4 ? word(p.h0, j) : word(p.h1, j - 4)) >> (2 * c);
+        lo = dot2_bf16(and_or(hs << 4, m1, (w & m4) | magic), xp[2 * j], lo);
+        lo = dot2_bf16(and_or(hs >> 4, m1, ((w >> 8) & m4) | magic), xp[2 * j + 1], lo);
+        hi = dot2_bf16(and_or(hs << 3, m1, ((w >> 4) & m4) | magic), xp[16 + 2 * j], hi);
+        hi = dot2_bf16(and_or(hs >> 5, m1, ((w >> 12) & m4) | magic), xp[16 + 2 * j + 1], hi);
+    }
+    uint32_t sc0, sc1, m0, mn1;
+    q4k_scales(p.hdr.y, p.hdr.z, p.hdr.w, c, sc0, sc1, m0, mn1);
+    const float d = f16_bits_to_f32(p.hdr.x & 0xffffu), dmin = f16_bits_to_f32(p.hdr.x >> 16);
+    const float d0 = d * (float)sc0, d1 = d * (float)sc1;
+    const float sl = sx[0] + sx[1], sh = sx[2] + sx[3];
+    float acc = d0 * lo - (128.f * d0 + dmin * (float)m0) * sl;
+    acc += d1 * hi - (128.f * d1 + dmin * (float)mn1) * sh;
     return acc;
 }
 
@@ -180,6 +230,36 @@ __device__ __forceinline__ float dot_f32(const Piece<HQ_Q6_K>& p, int c, const f
     acc += (float)(int)(int8_t)(s23 & 0xff) * (r2 - 32.f * sx[2]);
     acc += (float)(int)(int8_t)((s23 >> 16) & 0xff) * (r3 - 32.f * sx[3]);
     return d * acc;
+}
+
+__device__ __forceinline__ float dot_f32(const Piece<HQ_Q5_K>& p, int c, const float* xf, const float* sx) {
+    float lo = 0.f, hi = 0.f;
+    constexpr uint32_t N4 = 0x0f0f0f0fu, N1 = 0x10101010u;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t w = j < 4 ? word(p.q0, j) : word(p.q1, j - 4);
+        const uint32_t hs = (j < 4 ? word(p.h0, j) : word(p.h1, j - 4)) >> (2 * c);
+        lo = dot4((w & N4) | ((hs << 4) & N1), xf + 4 * j, lo);
+        hi = dot4(((w >> 4) & N4) | ((hs << 3) & N1), xf + 32 + 4 * j, hi);
+    }
+    uint32_t sc0, sc1, m0, m1;
+    q4k_scales(p.hdr.y, p.hdr.z, p.hdr.w, c, sc0, sc1, m0, m1);
+    const float d = f16_bits_to_f32(p.hdr.x & 0xffffu), dmin = f16_bits_to_f32(p.hdr.x >> 16);
+    float acc = d * (float)sc0 * lo - dmin * (float)m0 * (sx[0] + sx[1]);
+    acc += d * (float)sc1 * hi - dmin * (float)m1 * (sx[2] + sx[3]);
+    return acc;
+}
+
+// Q4_0: y = d * (q - 8); low nibbles are elements 0..15 of the block, high nibbles 16..31.
+__device__ __forceinline__ float dot_f32(const Piece<HQ_Q4_0>& p, int, const float* xf, const float* sx) {
+    float lo = 0.f, hi = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t w = word(p.q, j);
+        lo = dot4(w & 0x0f0f0f0fu, xf + 4 * j, lo);
+        hi = dot4((w >> 4) & 0x0f0f0f0fu, xf + 16 + 4 * j, hi);
+    }
+    return f16_bits_to_f32(p.d) * ((lo + hi) - 8.f * (sx[0] + sx[1]));
 }
 
 __device__ __forceinline__ float dot_f32(const Piece<HQ_Q8_0>& p, int, const float* xf, const float*) {
@@ -382,7 +462,7 @@ template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
 struct Walk {
     static_assert(NR % D == 0, "buffer rotation must repeat per step");
     static constexpr int EPL = Lane<TYPE>::kElems;
-    static constexpr uint32_t BYTES = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES : Q8_0_BYTES;
+    static constexpr uint32_t BYTES = kBlockBytes<TYPE>;
     static constexpr int XW = PAIR ? EPL / 2 : EPL;  // LDS words per piece
 
     const uint8_t* w;  // weight base + this lane's piece offset at step 0
@@ -402,11 +482,11 @@ struct Walk {
         li = lane & (L - 1u);
         lane_row = lane >> log_l;
         steps = (a.k / EPL) >> log_l;  // pieces per row / L (host guarantees divisibility)
-        row_bytes = (a.k / (TYPE == HQ_Q8_0 ? 32 : 256)) * BYTES;
+        row_bytes = (a.k / (kBlock32<TYPE> ? 32 : 256)) * BYTES;
         // L >= 4 for the K-quants (k >= 256), so a lane keeps the same sub-piece index c on every step
-        c = TYPE == HQ_Q8_0 ? 0 : (int)(li & 3u);
-        bstep = (TYPE == HQ_Q8_0 ? L : L >> 2) * BYTES;  // bytes of a row one step covers
-        w = wbase + (TYPE == HQ_Q8_0 ? li : li >> 2) * BYTES;
+        c = kBlock32<TYPE> ? 0 : (int)(li & 3u);
+        bstep = (kBlock32<TYPE> ? L : L >> 2) * BYTES;  // bytes of a row one step covers
+        w = wbase + (kBlock32<TYPE> ? li : li >> 2) * BYTES;
         lds_x = lx;
         lds_s = ls;
     }
@@ -644,10 +724,10 @@ int launch_q(hipStream_t s, KArgs ka, uint32_t cus, uint32_t rpw, size_t lds) {
 // Lanes per row, LDS bytes and slot count of one job.
 template <int TYPE, bool X_BF16>
 int plan_job(const GemvArgs& a, KArgs* ka, size_t* lds, uint64_t* slots) {
-    constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
+    constexpr bool PAIR = X_BF16 && !kBlock32<TYPE>;
     constexpr int EPL = Lane<TYPE>::kElems;
     if (a.x2 && X_BF16) return fail(HQ_ERR_UNSUPPORTED, "gemv: the fused SwiGLU form takes f32 activations");
-    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, M4, M2, MAGIC};
+    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, M4, TYPE == HQ_Q5_K ? M1 : M2, MAGIC};
     const uint32_t pieces = a.k / EPL;
     // L = largest power of two <= 64 that divides the pieces of a row
     uint32_t log_l = 0;
@@ -664,7 +744,7 @@ int plan_job(const GemvArgs& a, KArgs* ka, size_t* lds, uint64_t* slots) {
 
 template <int TYPE, bool X_BF16>
 int launch_t(hipStream_t s, const GemvArgs& a) {
-    constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
+    constexpr bool PAIR = X_BF16 && !kBlock32<TYPE>;
     constexpr int EPL = Lane<TYPE>::kElems;
     KArgs ka;
     size_t lds;
@@ -701,7 +781,7 @@ int launch_j(hipStream_t s, const KJobs& js, uint32_t n_jobs, size_t lds) {
 
 template <int TYPE, bool X_BF16>
 int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
-    constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
+    constexpr bool PAIR = X_BF16 && !kBlock32<TYPE>;
     KJobs js{};
     size_t lds = 0;
     uint64_t slots = 0;
@@ -728,6 +808,8 @@ int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type
         case HQ_Q4_K: return bf ? launch_t<HQ_Q4_K, true>(s, a) : launch_t<HQ_Q4_K, false>(s, a);
         case HQ_Q6_K: return bf ? launch_t<HQ_Q6_K, true>(s, a) : launch_t<HQ_Q6_K, false>(s, a);
         case HQ_Q8_0: return bf ? launch_t<HQ_Q8_0, true>(s, a) : launch_t<HQ_Q8_0, false>(s, a);
+        case HQ_Q5_K: return bf ? launch_t<HQ_Q5_K, true>(s, a) : launch_t<HQ_Q5_K, false>(s, a);
+        case HQ_Q4_0: return bf ? launch_t<HQ_Q4_0, true>(s, a) : launch_t<HQ_Q4_0, false>(s, a);
     }
     return fail(HQ_ERR_UNSUPPORTED, "gemv: ggml type %d", (int)t);
 }
@@ -741,6 +823,8 @@ int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_ac
         case HQ_Q4_K: return bf ? launch_jobs_t<HQ_Q4_K, true>(s, jobs, n_jobs) : launch_jobs_t<HQ_Q4_K, false>(s, jobs, n_jobs);
         case HQ_Q6_K: return bf ? launch_jobs_t<HQ_Q6_K, true>(s, jobs, n_jobs) : launch_jobs_t<HQ_Q6_K, false>(s, jobs, n_jobs);
         case HQ_Q8_0: return bf ? launch_jobs_t<HQ_Q8_0, true>(s, jobs, n_jobs) : launch_jobs_t<HQ_Q8_0, false>(s, jobs, n_jobs);
+        case HQ_Q5_K: return bf ? launch_jobs_t<HQ_Q5_K, true>(s, jobs, n_jobs) : launch_jobs_t<HQ_Q5_K, false>(s, jobs, n_jobs);
+        case HQ_Q4_0: return bf ? launch_jobs_t<HQ_Q4_0, true>(s, jobs, n_jobs) : launch_jobs_t<HQ_Q4_0, false>(s, jobs, n_jobs);
     }
     return fail(HQ_ERR_UNSUPPORTED, "gemv: ggml type %d", (int)t);
 }

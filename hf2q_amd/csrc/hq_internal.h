@@ -19,7 +19,7 @@ inline int check_launch(const char* what) { return check_hip(hipGetLastError(), 
 inline bool is_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 constexpr int kWave = 64;
-constexpr uint32_t Q4K_BYTES = 144, Q6K_BYTES = 210, Q8_0_BYTES = 34;
+constexpr uint32_t Q4K_BYTES = 144, Q5K_BYTES = 176, Q6K_BYTES = 210, Q8_0_BYTES = 34, Q4_0_BYTES = 18;
 
 // ---- launchers (one per .hip file); all validate nothing: the C entry points do ----
 int launch_dequant(hipStream_t s, const void* w, void* out, hq_act_dtype odt, uint64_t n_elems,

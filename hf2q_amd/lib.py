@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libhf2q_hip.so")
 
 HQ_OK, HQ_ERR_INVALID_ARGUMENT, HQ_ERR_UNSUPPORTED, HQ_ERR_HIP = 0, 1, 2, 3
-HQ_Q8_0, HQ_Q4_K, HQ_Q6_K = 8, 12, 14
+HQ_Q4_0, HQ_Q8_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K = 2, 8, 12, 13, 14
 HQ_F32, HQ_BF16 = 0, 1
 
 

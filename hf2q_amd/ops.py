@@ -17,10 +17,10 @@ from dataclasses import dataclass
 import torch
 
 from . import lib as _l
-from .lib import HQ_BF16, HQ_F32, HQ_Q4_K, HQ_Q6_K, HQ_Q8_0, HqError  # noqa: F401
+from .lib import HQ_BF16, HQ_F32, HQ_Q4_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HqError  # noqa: F401
 
-BLOCK_ELEMS = {HQ_Q8_0: 32, HQ_Q4_K: 256, HQ_Q6_K: 256}
-BLOCK_BYTES = {HQ_Q8_0: 34, HQ_Q4_K: 144, HQ_Q6_K: 210}
+BLOCK_ELEMS = {HQ_Q4_0: 32, HQ_Q8_0: 32, HQ_Q4_K: 256, HQ_Q5_K: 256, HQ_Q6_K: 256}
+BLOCK_BYTES = {HQ_Q4_0: 18, HQ_Q8_0: 34, HQ_Q4_K: 144, HQ_Q5_K: 176, HQ_Q6_K: 210}
 
 
 def _stream() -> int:

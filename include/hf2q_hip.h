@@ -41,8 +41,11 @@ typedef enum {
     HQ_ERR_HIP = 3               /* a HIP runtime call failed */
 } hq_status;
 
-/* Numeric ids are GGML's (src/quantize/ggml_quants/ggml_type.rs:18-53). */
-typedef enum { HQ_Q8_0 = 8, HQ_Q4_K = 12, HQ_Q6_K = 14 } hq_ggml_type;
+/* Numeric ids are GGML's (src/quantize/ggml_quants/ggml_type.rs:18-53).  Q4_K, Q6_K and Q8_0 are
+ * served by every entry point; Q5_K (block layout q5_k.rs:9-18) and Q4_0 (q4_0.rs:6-12) by the
+ * dequantiser and the matmul entry points (GEMV form at any m), not by hq_quantize_ggml.  Q4_K and
+ * Q5_K blocks must be 16-byte aligned, the others 2-byte. */
+typedef enum { HQ_Q4_0 = 2, HQ_Q8_0 = 8, HQ_Q4_K = 12, HQ_Q5_K = 13, HQ_Q6_K = 14 } hq_ggml_type;
 
 /* Activation element type.  hf2q's call sites pass F32 (gpu_full_attn.rs:835);
  * BF16 is the serving configuration this library is benchmarked on. */

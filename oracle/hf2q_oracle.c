@@ -781,6 +781,19 @@ static void q8_0_dequant_block(const uint8_t *b, float *y) {
     for (int i = 0; i < QK8_0; i++) y[i] = d * (float)(int8_t)b[2 + i];
 }
 
+static void dequant_block(int ggml_type, const uint8_t *b, float *y) {
+    if (ggml_type == T_Q4_K)
+        q4k_dequant_block(b, y);
+    else if (ggml_type == T_Q5_K)
+        q5k_dequant_block(b, y);
+    else if (ggml_type == T_Q6_K)
+        q6k_dequant_block(b, y);
+    else if (ggml_type == T_Q4_0)
+        q4_0_dequant_block(b, y);
+    else
+        q8_0_dequant_block(b, y);
+}
+
 int hq_oracle_dequantize(const uint8_t *blocks, int64_t n_elems, int ggml_type, float *out,
                          int n_threads) {
     int be = block_elems(ggml_type), bb = block_bytes(ggml_type);
@@ -789,16 +802,7 @@ int hq_oracle_dequantize(const uint8_t *blocks, int64_t n_elems, int ggml_type, 
     if (n_threads < 1) n_threads = 1;
 #pragma omp parallel for schedule(static) num_threads(n_threads)
     for (int64_t b = 0; b < nblocks; b++) {
-        if (ggml_type == T_Q4_K)
-            q4k_dequant_block(blocks + b * bb, out + b * be);
-        else if (ggml_type == T_Q5_K)
-            q5k_dequant_block(blocks + b * bb, out + b * be);
-        else if (ggml_type == T_Q6_K)
-            q6k_dequant_block(blocks + b * bb, out + b * be);
-        else if (ggml_type == T_Q4_0)
-            q4_0_dequant_block(blocks + b * bb, out + b * be);
-        else
-            q8_0_dequant_block(blocks + b * bb, out + b * be);
+        dequant_block(ggml_type, blocks + b * bb, out + b * be);
     }
     return 0;
 }
@@ -838,14 +842,7 @@ int hq_oracle_qmatmul_f64(const void *x, int xdt, const uint8_t *w_blocks, int64
 #pragma omp for schedule(static)
         for (int64_t j = 0; j < n; j++) {
             const uint8_t *rb = w_blocks + j * row_bytes;
-            for (int64_t b = 0; b < k / be; b++) {
-                if (ggml_type == T_Q4_K)
-                    q4k_dequant_block(rb + b * bb, wrow + b * be);
-                else if (ggml_type == T_Q6_K)
-                    q6k_dequant_block(rb + b * bb, wrow + b * be);
-                else
-                    q8_0_dequant_block(rb + b * bb, wrow + b * be);
-            }
+            for (int64_t b = 0; b < k / be; b++) dequant_block(ggml_type, rb + b * bb, wrow + b * be);
             for (int64_t i = 0; i < m; i++) {
                 const double *xi = xd + i * k;
                 double acc = 0.0;

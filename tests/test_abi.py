@@ -33,7 +33,9 @@ def test_block_geometry():
     assert (L.hq_block_elems(lib.HQ_Q4_K), L.hq_block_bytes(lib.HQ_Q4_K)) == (256, 144)
     assert (L.hq_block_elems(lib.HQ_Q6_K), L.hq_block_bytes(lib.HQ_Q6_K)) == (256, 210)
     assert (L.hq_block_elems(lib.HQ_Q8_0), L.hq_block_bytes(lib.HQ_Q8_0)) == (32, 34)
-    assert L.hq_block_elems(2) == 0 and L.hq_block_bytes(13) == 0
+    assert (L.hq_block_elems(lib.HQ_Q5_K), L.hq_block_bytes(lib.HQ_Q5_K)) == (256, 176)  # q5_k.rs:57-59
+    assert (L.hq_block_elems(lib.HQ_Q4_0), L.hq_block_bytes(lib.HQ_Q4_0)) == (32, 18)    # q4_0.rs:24-25
+    assert L.hq_block_elems(3) == 0 and L.hq_block_bytes(10) == 0  # Q4_1, Q2_K: not built
 
 
 def test_argument_errors_are_reported_not_fatal():
@@ -43,7 +45,7 @@ def test_argument_errors_are_reported_not_fatal():
     assert L.hq_qmatmul_ggml(None, fake, lib.HQ_F32, fake, fake, 1, 8, 300, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
     assert "multiple of the block size" in lib.last_error()
     # unsupported ggml type (forward_mlx.rs:9884-9886)
-    assert L.hq_qmatmul_ggml(None, fake, lib.HQ_F32, fake, fake, 1, 8, 256, 13) == lib.HQ_ERR_UNSUPPORTED
+    assert L.hq_qmatmul_ggml(None, fake, lib.HQ_F32, fake, fake, 1, 8, 256, 10) == lib.HQ_ERR_UNSUPPORTED  # Q2_K
     assert L.hq_dequant_ggml(None, fake, fake, lib.HQ_F32, 100, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
     # misaligned Q4_K weights
     assert L.hq_qmatmul_ggml(None, fake, lib.HQ_F32, ctypes.c_void_p(0x1002), fake, 1, 8, 256, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT

@@ -140,3 +140,18 @@ def test_tile_gemm_scale_equivariance(oracle, dev, xdt, t):
         xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
         assert_matmul_close_f16_tile(y.cpu().numpy(), oracle.qmatmul_f64(xv, blocks, m, n, k, t),
                                      f"tile gemm t={t} sigma={sigma} {xdt}")
+
+
+@pytest.mark.parametrize("t", [ops.HQ_Q5_K, ops.HQ_Q4_0])
+def test_types_without_a_tile_kernel_run_as_gemv_chunks(oracle, dev, t):
+    """Q5_K / Q4_0 at m > 8: the GEMV form, eight activation rows per launch (exact f32 accumulation of bf16 x weight)."""
+    m, n, k = 21, 96, 1024
+    blocks = oracle.quantize(weights(t, n, k), k, t, threads=8)
+    x = acts(5, m, k)
+    xb = oracle.f32_to_bf16_bits(x)
+    ref = oracle.qmatmul_f64(xb, blocks, m, n, k, t)
+    y = torch.full((m, n), float("nan"), device=dev)
+    p = GgmlQuantizedMatmulParams(m, n, k, t)
+    assert ops.quantized_matmul_workspace_bytes(p, torch.bfloat16) == 0
+    ops.quantized_matmul_ggml(torch.from_numpy(x).to(dev).to(torch.bfloat16), torch.from_numpy(blocks).to(dev), y, p)
+    assert_matmul_close(y.cpu().numpy(), ref, f"m=21 t={t}")

@@ -7,22 +7,26 @@ import torch
 from _util import acts, assert_matmul_close, weights
 from _util import assert_matmul_close_f16_tile
 from hf2q_amd import ops
-from hf2q_amd.ops import (HQ_Q4_K, HQ_Q6_K, HQ_Q8_0, GgmlQuantizedMatmulIdParams, GgmlQuantizedMatmulParams)
+from hf2q_amd.ops import (HQ_Q4_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, GgmlQuantizedMatmulIdParams,
+                          GgmlQuantizedMatmulParams)
 
 pytestmark = pytest.mark.gpu
 TYPES = [HQ_Q4_K, HQ_Q6_K, HQ_Q8_0]
+# dequantiser and GEMV / mul_mat_id also take the next two types of the reference's production models
+# (quantised on the host; the device quantizer and the tile GEMMs cover TYPES)
+ALL_TYPES = TYPES + [HQ_Q5_K, HQ_Q4_0]
 
 
 def _adversarial_blocks(oracle, t, nblocks, seed):
     """Raw random bytes (every nibble / 6-bit scale / sign pattern) with finite f16 scales."""
     bb = oracle.BLOCK_BYTES[t]
     raw = np.random.default_rng(seed).integers(0, 256, size=nblocks * bb, dtype=np.uint8)
-    for off in ([1, 3] if t == HQ_Q4_K else [209] if t == HQ_Q6_K else [1]):
+    for off in ([1, 3] if t in (HQ_Q4_K, HQ_Q5_K) else [209] if t == HQ_Q6_K else [1]):
         raw[off::bb] &= 0x3F
     return raw
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 def test_dequant_bit_exact(oracle, dev, t):
     be = oracle.BLOCK_ELEMS[t]
     w = weights(100 + t, 64, 1024)
@@ -36,16 +40,16 @@ def test_dequant_bit_exact(oracle, dev, t):
     assert np.array_equal(got16, oracle.f32_to_bf16_bits(want))
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 def test_dequant_golden_blocks(oracle, dev, t):
     import os
     from _util import GOLDEN
-    name = {HQ_Q4_K: "q4_k_512", HQ_Q6_K: "q6_k_512", HQ_Q8_0: "q8_0_64"}[t]
+    name = {HQ_Q4_K: "q4_k_512", HQ_Q6_K: "q6_k_512", HQ_Q8_0: "q8_0_64", HQ_Q5_K: "q5_k_512", HQ_Q4_0: "q4_0_64"}[t]
     blocks = np.fromfile(os.path.join(GOLDEN, "ggml_quants", f"{name}_noim_expected.bin"), dtype=np.uint8)
     n = blocks.size // oracle.BLOCK_BYTES[t] * oracle.BLOCK_ELEMS[t]
     # Q6_K / Q8_0 blocks need only 2-byte alignment: also run from an odd-word offset
     pad = torch.zeros(blocks.size + 16, dtype=torch.uint8, device=dev)
-    for off in ([0] if t == HQ_Q4_K else [0, 2, 6]):
+    for off in ([0] if t in (HQ_Q4_K, HQ_Q5_K) else [0, 2, 6]):
         pad[off:off + blocks.size] = torch.from_numpy(blocks).to(dev)
         got = ops.dequantize_ggml(pad[off:], n, t).cpu().numpy()
         assert np.array_equal(got.view(np.uint32), oracle.dequantize(blocks, t).view(np.uint32))
@@ -57,7 +61,7 @@ SHAPES = [  # (m, n, k)
 ]
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,n,k", SHAPES)
 def test_gemv_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
@@ -76,7 +80,7 @@ def test_gemv_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
     assert_matmul_close(y.cpu().numpy(), ref, f"gemv t={t} {xdt} {m}x{n}x{k}")
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 def test_gemv_adversarial_blocks(oracle, dev, t):
     """Every scale / min / sign bit pattern, not just what the quantizer emits."""
     n, k = 96, 1024
@@ -90,7 +94,7 @@ def test_gemv_adversarial_blocks(oracle, dev, t):
         assert_matmul_close(y.cpu().numpy(), ref, f"adversarial t={t}")
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 def test_gemv_zero_weights_give_zero(oracle, dev, t):
     # gpu_ffn.rs:3323-3351
     n, k = 64, 512
@@ -101,10 +105,10 @@ def test_gemv_zero_weights_give_zero(oracle, dev, t):
     assert not y.cpu().numpy().any()
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 def test_gemv_unaligned_weight_base(oracle, dev, t):
-    if t == HQ_Q4_K:
-        pytest.skip("Q4_K requires 16-byte aligned blocks (144 = 9*16)")
+    if t in (HQ_Q4_K, HQ_Q5_K):
+        pytest.skip("Q4_K / Q5_K require 16-byte aligned blocks (144 = 9*16, 176 = 11*16)")
     n, k = 48, 512
     blocks = oracle.quantize(weights(3, n, k), k, t)
     x = acts(4, 1, k)
@@ -121,7 +125,7 @@ ID_CASES = [  # (E, n, k, T, K)
 ]
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("E,n,k,T,K", ID_CASES)
 def test_mul_mat_id_matches_oracle(oracle, dev, t, xdt, E, n, k, T, K):
