@@ -140,6 +140,7 @@ int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const vo
                    uint32_t n, uint32_t k, hq_ggml_type t, void* workspace) {
     if (f16_tile_route(m, k, t)) return launch_gemm_f16_tile(stream, x, xdt, w_blocks, y, m, n, k, t, workspace);
     if (m > kGemvMaxRows && gemm_supported(t, k)) return launch_gemm(stream, x, xdt, w_blocks, y, m, n, k, t);
+    if (gemv_rows_supported(t, m, k)) return launch_gemv_rows(stream, x, xdt, w_blocks, y, m, n, k, t);
     // GEMV form, kGemvMaxRows activation rows per launch (also the route of shapes the
     // tile kernels do not cover).
     const size_t xrow_bytes = (size_t)k * (xdt == HQ_BF16 ? 2 : 4);

@@ -1,0 +1,284 @@
+// Dequant-fused product for 2..8 activation rows (small-batch decode) on the matrix cores:
+// y[m, n] = sum_k x[m, k] * W[n, k] with every weight fetched once for all rows, where the GEMV
+// kernel would fetch it once per row.  Q4_K weights, k a multiple of 1024.
+//
+// Bandwidth-bound like the GEMV (0.5625 bytes per weight); the arithmetic that depends on the row
+// count moves to v_mfma_f32_16x16x32_bf16, what is left on the VALU (nibbles -> bf16, scales) does
+// not depend on it.
+//
+// Mapping.  A workgroup owns 16 weight rows, its four waves a quarter of k each (super-block
+// 4*chunk + wave of every 1024-element chunk), summed through LDS at the end.  The MFMA takes the
+// activations as its first operand and the weights as its second: lane (j, g) (j = lane % 16,
+// g = lane / 16) supplies weights 8g..8g+7 of one 32-weight sub-block of row j -- the nibbles of
+// eight bytes it fetched itself -- and receives the products of row j with activation rows
+// 4g..4g+3.  So the lane that holds a row's outputs also holds that row's block header, and
+// applies the sub-block scale to the four sums without any cross-lane traffic:
+//   acc += d*sc * C - (128 * d*sc + dmin*m) * S,   S = sum of the activations of the sub-block,
+// where C is the MFMA result over the values 128 + q (the nibble under the bit pattern of bf16
+// 128.0, one v_and_or_b32 per pair, exact).  The second term is itself a small product over the
+// sub-blocks, (activation row x sub-block) . (sub-block x weight row), and goes through
+// v_mfma_f32_16x16x4_f32 in full f32, two instructions per super-block.
+//
+// Activations are staged per 1024-element chunk, double-buffered: bf16 rows as they are (rows
+// 0..7 of the MFMA, 8..15 repeat them and are ignored), f32 rows as an exact bf16 hi + lo pair in
+// rows m and m + 8 whose results are added at the end (16 bits of mantissa; the GEMV kernel works
+// in full f32).  Words are stored pre-paired, (x0, x2), (x1, x3), the order in which a masked
+// shift of a little-endian nibble word yields values.  The per-sub-block sums S sit beside them.
+#include "hq_internal.h"
+
+namespace hq {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+struct RowsArgs {
+    const void* x;
+    const uint8_t* w;
+    float* y;
+    uint32_t m, n, k;
+};
+
+constexpr uint32_t KC = 1024;            // activations staged per pass
+constexpr uint32_t XROW = KC * 2 + 16;   // bytes of a staged row; the pad spreads the rows over the banks
+constexpr uint32_t SBUF = 32 * 16 * 4;   // sums [32 sub-blocks][16 rows]
+// One of the two staging buffers: 8 (bf16) or 16 (f32 as hi + lo) staged rows, then the sums.
+template <bool X_BF16>
+constexpr uint32_t kXBuf = (X_BF16 ? 8 : 16) * XROW;
+template <bool X_BF16>
+constexpr uint32_t kStage = kXBuf<X_BF16> + SBUF;
+constexpr uint32_t M4 = 0x000f000fu, MAGIC = 0x43004300u;
+
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2v_t;
+
+// (x0, x1), (x2, x3) -> (x0, x2), (x1, x3): one byte permute each
+__device__ __forceinline__ void pair_words(uint32_t a, uint32_t b, uint32_t& o0, uint32_t& o1) {
+    o0 = __builtin_amdgcn_perm(b, a, 0x05040100u);
+    o1 = __builtin_amdgcn_perm(b, a, 0x07060302u);
+}
+// Two floats -> one word of two bf16 (round to nearest even), low half first.
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2v_t));
+}
+constexpr uint32_t ONES = 0x3f803f80u;  // (1.0, 1.0) in bf16: a dot2 with it adds the two halves of a word
+
+// A thread's share of a chunk: input row tid / 32 (of at most 8), sub-block tid % 32 = 32 activations.
+template <bool X_BF16>
+struct Staged {
+    uint4 r[X_BF16 ? 4 : 8];
+    __device__ __forceinline__ void fetch(const RowsArgs& a, uint32_t chunk, uint32_t tid) {
+        // No branch around the loads: with conditional loads in flight the compiler can no longer count how
+        // many newer loads stand behind an older one and waits for all of them.  Threads of absent rows read
+        // the last row and zero what they got (in store()).
+        const uint32_t row = tid >> 5, sb = tid & 31u;
+        constexpr int N = X_BF16 ? 4 : 8;
+        const uint32_t src_row = row < a.m ? row : a.m - 1u;
+        const uint4* src = reinterpret_cast<const uint4*>(static_cast<const uint8_t*>(a.x) +
+                                                          ((size_t)src_row * a.k + (size_t)chunk * KC + 32u * sb) * (X_BF16 ? 2 : 4));
+#pragma unroll
+        for (int i = 0; i < N; ++i) r[i] = src[i];
+    }
+    __device__ __forceinline__ uint4 masked(int i, bool present) const {
+        return present ? r[i] : make_uint4(0, 0, 0, 0);
+    }
+    __device__ __forceinline__ void store(uint8_t* buf, uint32_t tid, uint32_t m) const {
+        const uint32_t row = tid >> 5, sb = tid & 31u;
+        const bool present = row < m;
+        float* sums = reinterpret_cast<float*>(buf + kXBuf<X_BF16>);
+        if constexpr (X_BF16) {
+            float s = 0.f;
+            uint4 o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint4 t = masked(i, present);
+                pair_words(t.x, t.y, o[i].x, o[i].y);
+                pair_words(t.z, t.w, o[i].z, o[i].w);
+                s = dot2_bf16(t.x, ONES, s);
+                s = dot2_bf16(t.y, ONES, s);
+                s = dot2_bf16(t.z, ONES, s);
+                s = dot2_bf16(t.w, ONES, s);
+            }
+            uint4* dst = reinterpret_cast<uint4*>(buf + row * XROW + sb * 64u);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dst[i] = o[i];
+            sums[sb * 16u + row] = s;
+        } else {
+            // x = hi + lo with hi = bf16(x) and lo = bf16(x - hi); the packing instruction pairs (x0, x2), (x1, x3) for free
+            float sh = 0.f, sl = 0.f;
+            uint4 oh[4], ol[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {  // eight floats -> four hi words and four lo words
+                const uint4 ta = masked(2 * i, present), tb = masked(2 * i + 1, present);
+                const float v[8] = {__uint_as_float(ta.x), __uint_as_float(ta.y), __uint_as_float(ta.z), __uint_as_float(ta.w),
+                                    __uint_as_float(tb.x), __uint_as_float(tb.y), __uint_as_float(tb.z), __uint_as_float(tb.w)};
+                uint32_t hw[4], lw[4];
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {  // elements 4q .. 4q+3
+                    const float* e = v + 4 * q;
+                    const uint32_t ha = pack_bf16(e[0], e[2]), hb = pack_bf16(e[1], e[3]);
+                    const float l0 = e[0] - __uint_as_float(ha << 16), l2 = e[2] - __uint_as_float(ha & 0xffff0000u);
+                    const float l1 = e[1] - __uint_as_float(hb << 16), l3 = e[3] - __uint_as_float(hb & 0xffff0000u);
+                    hw[2 * q] = ha, hw[2 * q + 1] = hb;
+                    lw[2 * q] = pack_bf16(l0, l2), lw[2 * q + 1] = pack_bf16(l1, l3);
+                    sh = dot2_bf16(ha, ONES, sh);
+                    sh = dot2_bf16(hb, ONES, sh);
+                    sl = dot2_bf16(lw[2 * q], ONES, sl);
+                    sl = dot2_bf16(lw[2 * q + 1], ONES, sl);
+                }
+                oh[i] = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+                ol[i] = make_uint4(lw[0], lw[1], lw[2], lw[3]);
+            }
+            uint4* dh = reinterpret_cast<uint4*>(buf + row * XROW + sb * 64u);
+            uint4* dl = reinterpret_cast<uint4*>(buf + (row + 8u) * XROW + sb * 64u);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                dh[i] = oh[i];
+                dl[i] = ol[i];
+            }
+            sums[sb * 16u + row] = sh;
+            sums[sb * 16u + row + 8u] = sl;
+        }
+    }
+};
+
+template <bool X_BF16>
+__global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
+    extern __shared__ uint4 smem4[];
+    uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t j = lane & 15u, g = lane >> 4;
+    const uint32_t row0 = blockIdx.x * 16u;
+    const uint32_t r = row0 + j < a.n ? row0 + j : a.n - 1u;  // rows past the end repeat the last one, not stored
+    const uint32_t nsb = a.k / 256u, nch = a.k / KC;
+    const uint8_t* wrow = a.w + (size_t)r * nsb * Q4K_BYTES + 16u + 8u * g;  // this lane's eight bytes of chunk 0
+    const uint32_t arow = (X_BF16 ? (j & 7u) : j) * XROW + 16u * g;          // this lane's row and k-group in a staged buffer
+
+    struct WBlock {
+        uint4 hdr;
+        uint2 q[4];
+    };
+    auto load_w = [&](uint32_t ch, WBlock& b) {
+        const uint8_t* p = wrow + (size_t)(ch * 4u + wave) * Q4K_BYTES;
+        b.hdr = *reinterpret_cast<const uint4*>(p - 16u - 8u * g);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) b.q[c] = *reinterpret_cast<const uint2*>(p + 32 * c);
+    };
+
+    constexpr uint32_t XBUF = kXBuf<X_BF16>, STAGE = kStage<X_BF16>;
+    // The next chunk's weights and activations are requested before the current chunk's arithmetic.  The two
+    // weight buffers swap roles from chunk to chunk (the loop is unrolled by two): copying one into the other
+    // would make the compiler wait for the newest loads at once.
+    // the conversion masks sit in VGPRs so that (w & m4) | magic is one v_and_or_b32 (one scalar operand
+    // at most per VALU op); the copy is opaque so that they stay there
+    uint32_t m4, magic;
+    asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "=v"(m4), "=v"(magic) : "s"(M4), "s"(MAGIC));
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    Staged<X_BF16> st;
+    auto chunk = [&](uint32_t ch, const WBlock& wb, WBlock& wnext, const uint8_t* bufc, uint8_t* bufn) {
+        // the last chunk requests itself again rather than nothing: see Staged::fetch
+        const bool more = ch + 1 < nch;
+        const uint32_t ahead = more ? ch + 1 : ch;
+        st.fetch(a, ahead, tid);
+        load_w(ahead, wnext);
+        const uint8_t* xb = bufc + arow + wave * 512u;  // the wave's super-block: 256 activations
+        // sums of the wave's eight sub-blocks as the first operand of a 16x16x4 f32 MFMA: lane (j, g) holds
+        // S[activation row j][sub-block 4t + g]
+        const float* sums = reinterpret_cast<const float*>(bufc + XBUF) + wave * 128u + 16u * g + j;
+        const float d = f16_bits_to_f32(wb.hdr.x & 0xffffu), dmin = f16_bits_to_f32(wb.hdr.x >> 16);
+        float ds[8], off[8];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint32_t sc0, sc1, m0, m1;
+            q4k_scales(wb.hdr.y, wb.hdr.z, wb.hdr.w, c, sc0, sc1, m0, m1);
+            ds[2 * c] = d * (float)sc0, ds[2 * c + 1] = d * (float)sc1;
+            off[2 * c] = fmaf(128.f, ds[2 * c], dmin * (float)m0), off[2 * c + 1] = fmaf(128.f, ds[2 * c + 1], dmin * (float)m1);
+        }
+        // -sum_b off_b * S_b for all sixteen activation rows at once: the weights' side of that small product is
+        // off of sub-block 4t + g of this lane's row
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const float o01 = (g & 1u) ? off[4 * t + 1] : off[4 * t], o23 = (g & 1u) ? off[4 * t + 3] : off[4 * t + 2];
+            const float mine = (g & 2u) ? o23 : o01;
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[64 * t], -mine, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t w0 = wb.q[c].x, w1 = wb.q[c].y;
+            const uint4 blo = make_uint4(and_or(w0, m4, magic), and_or(w0 >> 8, m4, magic), and_or(w1, m4, magic),
+                                         and_or(w1 >> 8, m4, magic));
+            const uint4 bhi = make_uint4(and_or(w0 >> 4, m4, magic), and_or(w0 >> 12, m4, magic), and_or(w1 >> 4, m4, magic),
+                                         and_or(w1 >> 12, m4, magic));
+            const uint4 alo = *reinterpret_cast<const uint4*>(xb + 128 * c);       // sub-block 2c: 64 bytes per sub-block
+            const uint4 ahi = *reinterpret_cast<const uint4*>(xb + 128 * c + 64);  // sub-block 2c + 1
+            const f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+            const f32x4_t clo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, alo), __builtin_bit_cast(bf16x8_t, blo), z, 0, 0, 0);
+            const f32x4_t chi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ahi), __builtin_bit_cast(bf16x8_t, bhi), z, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[v] = fmaf(ds[2 * c + 1], chi[v], fmaf(ds[2 * c], clo[v], acc[v]));
+        }
+        st.store(bufn, tid, a.m);
+        __syncthreads();  // the other buffer is complete; this one may be overwritten by the next pass
+    };
+    WBlock wa, wb2;
+    st.fetch(a, 0, tid);
+    load_w(0, wa);
+    st.store(smem, tid, a.m);
+    __syncthreads();
+    for (uint32_t ch = 0; ch < nch; ch += 2) {
+        chunk(ch, wa, wb2, smem, smem + STAGE);
+        if (ch + 1 < nch) chunk(ch + 1, wb2, wa, smem + STAGE, smem);
+    }
+
+    // ---- sum of the four waves (and of the hi and lo rows), store ----
+    float4* red = reinterpret_cast<float4*>(smem);
+    red[wave * 64u + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    __syncthreads();
+    if (wave == 0 && g < 2u && row0 + j < a.n) {
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float4 t = red[w * 64 + lane];
+            o[0] += t.x, o[1] += t.y, o[2] += t.z, o[3] += t.w;
+            if constexpr (!X_BF16) {
+                const float4 u = red[w * 64 + lane + 32];  // the lo rows: activation rows 8 + 4g + v
+                o[0] += u.x, o[1] += u.y, o[2] += u.z, o[3] += u.w;
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            if (4u * g + v < a.m) a.y[(size_t)(4u * g + v) * a.n + row0 + j] = o[v];
+    }
+}
+
+}  // namespace
+
+// From four rows on: below that, one GEMV per row is as fast (measured at 12288 x 4096: 10 / 15 / 19 / 24 us for
+// 1..4 GEMVs against 17..19 us here whatever the row count).
+bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k) { return t == HQ_Q4_K && m >= 4 && m <= 8 && k % KC == 0; }
+
+int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
+                     uint32_t k, hq_ggml_type t) {
+    (void)t;
+    RowsArgs a{x, static_cast<const uint8_t*>(w), y, m, n, k};
+    const int lds = 2 * (xdt == HQ_BF16 ? kStage<true> : kStage<false>);
+    const dim3 grid((n + 15u) / 16u);
+    if (xdt == HQ_BF16) {
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_rows_kernel<true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                               "hipFuncSetAttribute(rows kernel LDS)"))
+            return rc;
+        hipLaunchKernelGGL(q4k_rows_kernel<true>, grid, dim3(256), lds, s, a);
+    } else {
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_rows_kernel<false>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                               "hipFuncSetAttribute(rows kernel LDS)"))
+            return rc;
+        hipLaunchKernelGGL(q4k_rows_kernel<false>, grid, dim3(256), lds, s, a);
+    }
+    return check_launch("rows kernel launch");
+}
+
+}  // namespace hq

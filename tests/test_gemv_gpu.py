@@ -310,3 +310,47 @@ def test_mul_mat_id_grouped_routing_properties(oracle, dev):
     assert ops.quantized_matmul_id_workspace_bytes(padded) == 0
     small = GgmlQuantizedMatmulIdParams(8, 2, n, k, E, p.expert_stride, t)
     assert ops.quantized_matmul_id_workspace_bytes(small) == 0
+
+
+# ---- 4..8 activation rows sharing one pass over the weights (small-batch decode) ------
+
+ROWS_SHAPES = [(4, 64, 1024), (4, 200, 4096), (4, 16, 2048), (5, 33, 1024), (6, 130, 3072), (7, 250, 2048), (8, 96, 12288)]
+
+
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("m,n,k", ROWS_SHAPES)
+def test_small_batch_rows_match_f64_oracle(oracle, dev, xdt, m, n, k):
+    """Q4_K with k % 1024 == 0 and 4 <= m <= 8 takes the kernel that fetches every weight once for all rows."""
+    t = HQ_Q4_K
+    blocks = oracle.quantize(weights(3 * n + k + m, n, k), k, t, threads=8)
+    x = acts(n + k + m, m, k)
+    xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
+    xd = torch.from_numpy(x).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    ref = oracle.qmatmul_f64(xv, blocks, m, n, k, t)
+    y = torch.full((m, n), float("nan"), device=dev)
+    wd = torch.from_numpy(blocks).to(dev)
+    ops.quantized_matmul_ggml(xd, wd, y, GgmlQuantizedMatmulParams(m, n, k, t))
+    assert_matmul_close(y.cpu().numpy(), ref, f"rows {xdt} {m}x{n}x{k}")
+    # every row equals the one-row product of the same activations (the GEMV kernel) to accumulation noise
+    y1 = torch.empty((1, n), device=dev)
+    for r in range(m):
+        ops.quantized_matmul_ggml(xd[r:r + 1].contiguous(), wd, y1, GgmlQuantizedMatmulParams(1, n, k, t))
+        assert np.abs(y1.cpu().numpy()[0] - y.cpu().numpy()[r]).max() <= 1e-4 * np.abs(ref).max()
+
+
+def test_small_batch_rows_adversarial_blocks_and_scaling(oracle, dev):
+    """Every scale / min / nibble pattern; and scaling the activations by a power of two scales the result exactly."""
+    t, m, n, k = HQ_Q4_K, 8, 48, 2048
+    blocks = _adversarial_blocks(oracle, t, n * k // 256, 9)
+    x = acts(2, m, k)
+    wd = torch.from_numpy(blocks).to(dev)
+    for xv, xd in ((x, torch.from_numpy(x).to(dev)),
+                   (oracle.f32_to_bf16_bits(x), torch.from_numpy(x).to(dev).to(torch.bfloat16))):
+        ref = oracle.qmatmul_f64(xv, blocks, m, n, k, t)
+        y = torch.empty((m, n), device=dev)
+        ops.quantized_matmul_ggml(xd, wd, y, GgmlQuantizedMatmulParams(m, n, k, t))
+        assert_matmul_close(y.cpu().numpy(), ref, "rows, adversarial blocks")
+        y2 = torch.empty_like(y)
+        ops.quantized_matmul_ggml(xd * 1024, wd, y2, GgmlQuantizedMatmulParams(m, n, k, t))
+        assert torch.equal(y2, y * 1024)
