@@ -198,6 +198,30 @@ int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w
     return rc ? rc : rc_free;
 }
 
+size_t hq_qmatmul_perm021_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
+    // the tile GEMM gathers while it converts; every other route first copies the activations into row-major order
+    if (f16_tile_route(m, k, t)) return gemm_f16_tile_workspace_bytes(m, n, k);
+    return (((size_t)m * k * (xdt == HQ_BF16 ? 2 : 4)) + 255) & ~(size_t)255;
+}
+
+int hq_qmatmul_perm021_ggml_ws(void* stream, const void* x_perm, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
+                               uint32_t n, uint32_t k, uint32_t head_dim, hq_ggml_type t, void* workspace,
+                               size_t workspace_bytes) {
+    const char* fn = "hq_qmatmul_perm021_ggml_ws";
+    if (int rc = check_matmul_common(fn, x_perm, xdt, w_blocks, y, n, k, t)) return rc;
+    if (head_dim == 0 || head_dim % 8 || k % head_dim)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: head_dim %u must be a multiple of 8 that divides k = %u", fn, head_dim, k);
+    if (m == 0) return HQ_OK;
+    const size_t need = hq_qmatmul_perm021_ggml_workspace_bytes(m, n, k, xdt, t);
+    if (!workspace || workspace_bytes < need)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes, %zu needed", fn, workspace ? workspace_bytes : (size_t)0, need);
+    if (reinterpret_cast<uintptr_t>(workspace) % 256) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace must be 256-byte aligned", fn);
+    if (f16_tile_route(m, k, t))
+        return launch_gemm_f16_tile((hipStream_t)stream, x_perm, xdt, w_blocks, y, m, n, k, t, workspace, head_dim);
+    if (int rc = launch_unpermute021((hipStream_t)stream, x_perm, workspace, m, k, head_dim, xdt == HQ_BF16 ? 2 : 4)) return rc;
+    return qmatmul_routes((hipStream_t)stream, workspace, xdt, w_blocks, y, m, n, k, t, nullptr);
+}
+
 size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows) {
     (void)n_experts;
     (void)max_rows;

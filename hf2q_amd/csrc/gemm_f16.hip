@@ -91,7 +91,7 @@ __device__ __forceinline__ uint32_t f16_bits(float v) {
 template <bool X_BF16, int TYPE>
 __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
                                                         uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k,
-                                                        const uint32_t* __restrict__ row_map, uint32_t top_k) {
+                                                        const uint32_t* __restrict__ row_map, uint32_t top_k, uint32_t perm_hd) {
     __shared__ float red[4];
     const uint32_t tid = threadIdx.x;
     const Workspace L = workspace_layout(m, n, k);
@@ -136,9 +136,15 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
     const uint32_t row = row_map ? row_map[out_row] / top_k : out_row;
     const uint32_t chunks = k / 8;
 
+    // perm_hd != 0: x is stored [k / perm_hd][m][perm_hd] (heads outermost), element (row, kk) at
+    // ((kk / perm_hd) * m + row) * perm_hd + kk % perm_hd; perm_hd is a multiple of 8, so a chunk stays inside a head
+    auto elem0 = [&](uint32_t i) -> size_t {
+        const uint32_t kk = 8u * i;
+        return perm_hd ? ((size_t)(kk / perm_hd) * m + row) * perm_hd + kk % perm_hd : (size_t)row * k + kk;
+    };
     auto load8 = [&](uint32_t i, float* v) {
         if constexpr (X_BF16) {
-            const uint4 u = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + (size_t)row * k + 8 * i);
+            const uint4 u = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + elem0(i));
             const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -146,7 +152,7 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
                 v[2 * j + 1] = bf16_bits_to_f32(w[j] >> 16);
             }
         } else {
-            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(x) + (size_t)row * k + 8 * i);
+            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(x) + elem0(i));
             const float4 a = p[0], b = p[1];
             v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
         }
@@ -895,12 +901,12 @@ size_t gemm_f16_grouped_workspace_bytes(uint32_t pairs, uint32_t n_experts, uint
 
 template <int TYPE>
 static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, uint8_t* ws, uint32_t m,
-                       uint32_t n, uint32_t k, const uint32_t* row_map = nullptr, uint32_t top_k = 1) {
+                       uint32_t n, uint32_t k, const uint32_t* row_map = nullptr, uint32_t top_k = 1, uint32_t perm_hd = 0) {
     const dim3 prep_grid(m + (n + 15u) / 16u);
     if (xdt == HQ_BF16)
-        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, row_map, top_k);
+        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, row_map, top_k, perm_hd);
     else
-        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, row_map, top_k);
+        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, row_map, top_k, perm_hd);
     return check_launch("tile gemm pre-pass launch");
 }
 
@@ -942,7 +948,7 @@ bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {
 }
 
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
-                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace) {
+                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const uint8_t* wb = static_cast<const uint8_t*>(w);
     GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr};
@@ -950,7 +956,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
     if (t == HQ_Q6_K) {
-        if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k)) return rc;
+        if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
         if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q6k_gemm_kernel),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                                "hipFuncSetAttribute(q6_k gemm LDS)"))
@@ -959,7 +965,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         return check_launch("q6_k gemm kernel launch");
     }
     if (t == HQ_Q8_0) {
-        if (int rc = launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k)) return rc;
+        if (int rc = launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
         if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q80_gemm_kernel),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                                "hipFuncSetAttribute(q8_0 gemm LDS)"))
@@ -967,7 +973,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         hipLaunchKernelGGL(q80_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
         return check_launch("q8_0 gemm kernel launch");
     }
-    if (int rc = launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k)) return rc;
+    if (int rc = launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_gemm_kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                            "hipFuncSetAttribute(q4k gemm LDS)"))

@@ -59,8 +59,10 @@ int launch_gemm(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, f
 // k % 128 == 0); needs a device workspace of gemm_f16_tile_workspace_bytes().
 bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k);
 size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+// perm_hd != 0: the activations are stored [k / perm_hd][m][perm_hd] (attention output, heads outermost) and are
+// gathered by the pre-pass.
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
-                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace);
+                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd = 0);
 
 // Grouped form of the tile GEMM for mul_mat_id with many routed rows: rows sorted by expert, one
 // tile = up to 256 rows of one expert; needs a contiguous stack (expert_stride = n rows) and a device
@@ -78,6 +80,8 @@ int launch_dense_gemv_bf16_pair(hipStream_t s, const void* x, hq_act_dtype xdt, 
                                 const void* w_b, float* y_b, uint32_t n_b, uint32_t m, uint32_t k);
 int launch_moe_softmax_topk(hipStream_t s, const float* logits, uint32_t* ids, float* weights, uint32_t n_tokens,
                             uint32_t n_experts, uint32_t top_k);
+// dst[m][k] <- src stored [k / head_dim][m][head_dim]; elem_bytes 2 or 4
+int launch_unpermute021(hipStream_t s, const void* src, void* dst, uint32_t m, uint32_t k, uint32_t head_dim, uint32_t elem_bytes);
 int launch_silu_mul(hipStream_t s, const float* gate, const float* up, float* out, uint64_t n);
 int launch_moe_weighted_reduce(hipStream_t s, const float* y, const float* w, const float* shared, const float* shared_logit,
                                const float* residual, float* out, uint32_t n_tokens, uint32_t top_k, uint32_t hidden);

@@ -231,6 +231,23 @@ int launch_moe_softmax_topk(hipStream_t s, const float* logits, uint32_t* ids, f
     return check_launch("moe softmax_topk launch");
 }
 
+// One 16-byte piece per thread: dst row r, bytes [16 p, 16 p + 16) <- head (16 p) / head_bytes of the head-major source.
+__global__ __launch_bounds__(256) void unpermute021_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, uint32_t m,
+                                                           uint32_t row_pieces, uint32_t head_pieces) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (uint64_t)m * row_pieces) return;
+    const uint32_t r = (uint32_t)(idx / row_pieces), p = (uint32_t)(idx % row_pieces);
+    dst[idx] = src[((uint64_t)(p / head_pieces) * m + r) * head_pieces + p % head_pieces];
+}
+
+int launch_unpermute021(hipStream_t s, const void* src, void* dst, uint32_t m, uint32_t k, uint32_t head_dim, uint32_t elem_bytes) {
+    const uint32_t row_pieces = k * elem_bytes / 16u, head_pieces = head_dim * elem_bytes / 16u;
+    const uint64_t total = (uint64_t)m * row_pieces;
+    hipLaunchKernelGGL(unpermute021_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, static_cast<const uint4*>(src),
+                       static_cast<uint4*>(dst), m, row_pieces, head_pieces);
+    return check_launch("unpermute kernel launch");
+}
+
 int launch_silu_mul(hipStream_t s, const float* gate, const float* up, float* out, uint64_t n) {
     const uint64_t n4 = n / 4;
     hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, gate, up, out, n4);

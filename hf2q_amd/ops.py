@@ -92,6 +92,31 @@ def quantized_matmul_workspace_bytes(params: GgmlQuantizedMatmulParams, act_dtyp
     return int(L.hq_qmatmul_ggml_workspace_bytes(params.m, params.n, params.k, xdt, params.ggml_type))
 
 
+@dataclass
+class GgmlQuantizedMatmulPerm021Params:
+    """forward_prefill_batched.rs:2219-2226."""
+    m: int
+    n: int
+    k: int
+    head_dim: int
+    ggml_type: int
+
+
+def quantized_matmul_mm_tensor_perm021(input_perm: torch.Tensor, weight: torch.Tensor, output: torch.Tensor,
+                                       params: GgmlQuantizedMatmulPerm021Params, workspace: torch.Tensor | None = None) -> None:
+    """forward_prefill_batched.rs:2246-2253: output[m, n] = x[m, k] . W[n, k]^T with x stored [k / head_dim, m, head_dim]."""
+    if output.dtype != torch.float32:
+        raise TypeError("output must be float32")
+    L = _l.load()
+    xdt = _act_dtype(input_perm)
+    need = int(L.hq_qmatmul_perm021_ggml_workspace_bytes(params.m, params.n, params.k, xdt, params.ggml_type))
+    if workspace is None:
+        workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=input_perm.device)
+    _l.check(L.hq_qmatmul_perm021_ggml_ws(_stream(), _dev(input_perm, "input"), xdt, _dev(weight, "weight"), _dev(output, "output"),
+                                          params.m, params.n, params.k, params.head_dim, params.ggml_type,
+                                          _dev(workspace, "workspace"), workspace.numel() * workspace.element_size()))
+
+
 def quantized_matmul_id_ggml(input: torch.Tensor, weight_stack: torch.Tensor, ids: torch.Tensor,
                              output: torch.Tensor, params: GgmlQuantizedMatmulIdParams,
                              scratch: torch.Tensor | None = None) -> None:

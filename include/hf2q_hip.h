@@ -110,6 +110,18 @@ HQ_API int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, con
                        uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, void* workspace,
                        size_t workspace_bytes);
 
+/* y[m, n] = sum_k x[m, k] * W[n, k] with the activations stored heads-outermost, [k / head_dim][m][head_dim]
+ * (the attention output of a batched prefill): element (row, kk) sits at ((kk / head_dim) * m + row) * head_dim +
+ * kk % head_dim.  Replaces quantized_matmul_mm_tensor_perm021(enc, reg, dev, input, weight, dst,
+ * GgmlQuantizedMatmulPerm021Params{m, n, k, head_dim, ggml_type}) (forward_prefill_batched.rs:2219-2257), which
+ * saves the transpose between attention and the output projection.  The tile GEMM (m > 8) gathers in its
+ * activation pre-pass at no extra cost; other shapes copy the activations into row-major order in `workspace`
+ * first.  head_dim: a multiple of 8 that divides k. */
+HQ_API size_t hq_qmatmul_perm021_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t);
+HQ_API int hq_qmatmul_perm021_ggml_ws(void* stream, const void* x_perm, hq_act_dtype xdt, const void* w_blocks, float* y,
+                               uint32_t m, uint32_t n, uint32_t k, uint32_t head_dim, hq_ggml_type t, void* workspace,
+                               size_t workspace_bytes);
+
 /* out[t, s, :] = W[ids[t*top_k + s]] . x[t, :] over an expert stack
  * [n_experts][n][k/QK] whose experts are `expert_stride` BYTES apart;
  * ids [n_tokens*top_k] u32 on the device (no host sync); out

@@ -155,3 +155,27 @@ def test_types_without_a_tile_kernel_run_as_gemv_chunks(oracle, dev, t):
     assert ops.quantized_matmul_workspace_bytes(p, torch.bfloat16) == 0
     ops.quantized_matmul_ggml(torch.from_numpy(x).to(dev).to(torch.bfloat16), torch.from_numpy(blocks).to(dev), y, p)
     assert_matmul_close(y.cpu().numpy(), ref, f"m=21 t={t}")
+
+
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q8_0])
+@pytest.mark.parametrize("m,heads,hd,n", [(64, 4, 256, 96), (300, 8, 128, 160), (5, 2, 256, 64)])
+def test_perm021_matches_oracle_and_the_plain_product(oracle, dev, t, m, heads, hd, n):
+    """quantized_matmul_mm_tensor_perm021 (forward_prefill_batched.rs:2219-2257): activations stored
+    [heads, m, head_dim]; the result is the plain product over the transposed activations, bit for bit."""
+    k = heads * hd
+    blocks = oracle.quantize(weights(t + m, n, k), k, t, threads=8)
+    x = acts(m + hd, m, k)                                   # logical [m, k]
+    xb = oracle.f32_to_bf16_bits(x)
+    ref = oracle.qmatmul_f64(xb, blocks, m, n, k, t)
+    xd = torch.from_numpy(x).to(dev).to(torch.bfloat16)
+    x_perm = xd.view(m, heads, hd).permute(1, 0, 2).contiguous()  # [heads, m, head_dim]
+    wd = torch.from_numpy(blocks).to(dev)
+    y = torch.full((m, n), float("nan"), device=dev)
+    ops.quantized_matmul_mm_tensor_perm021(x_perm, wd, y, ops.GgmlQuantizedMatmulPerm021Params(m, n, k, hd, t))
+    check = assert_matmul_close_f16_tile if (m > 8 and _f16_tile(t, k)) else assert_matmul_close
+    check(y.cpu().numpy(), ref, f"perm021 t={t} m={m}")
+    y2 = torch.empty_like(y)
+    ops.quantized_matmul_ggml(xd, wd, y2, GgmlQuantizedMatmulParams(m, n, k, t))
+    assert torch.equal(y, y2)
+    with pytest.raises(ops.HqError):  # head_dim must divide k
+        ops.quantized_matmul_mm_tensor_perm021(x_perm, wd, y, ops.GgmlQuantizedMatmulPerm021Params(m, n, k, hd + 8, t))
