@@ -1,6 +1,6 @@
 // Dequant-fused product for 2..8 activation rows (small-batch decode) on the matrix cores:
 // y[m, n] = sum_k x[m, k] * W[n, k] with every weight fetched once for all rows, where the GEMV
-// kernel would fetch it once per row.  Q4_K weights, k a multiple of 1024.
+// kernel would fetch it once per row.  Q4_K and Q6_K weights, k a multiple of 1024.
 //
 // Bandwidth-bound like the GEMV (0.5625 bytes per weight); the arithmetic that depends on the row
 // count moves to v_mfma_f32_16x16x32_bf16, what is left on the VALU (nibbles -> bf16, scales) does
@@ -42,7 +42,7 @@ struct RowsArgs {
 
 constexpr uint32_t KC = 1024;            // activations staged per pass
 constexpr uint32_t XROW = KC * 2 + 16;   // bytes of a staged row; the pad spreads the rows over the banks
-constexpr uint32_t SBUF = 32 * 16 * 4;   // sums [32 sub-blocks][16 rows]
+constexpr uint32_t SBUF = 64 * 16 * 4;   // sums [32 sub-blocks of 32, or 64 groups of 16][16 rows]
 // One of the two staging buffers: 8 (bf16) or 16 (f32 as hi + lo) staged rows, then the sums.
 template <bool X_BF16>
 constexpr uint32_t kXBuf = (X_BF16 ? 8 : 16) * XROW;
@@ -66,7 +66,8 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 constexpr uint32_t ONES = 0x3f803f80u;  // (1.0, 1.0) in bf16: a dot2 with it adds the two halves of a word
 
 // A thread's share of a chunk: input row tid / 32 (of at most 8), sub-block tid % 32 = 32 activations.
-template <bool X_BF16>
+// SUM16: the sums are kept per 16 activations (Q6_K's scale groups), two per thread, else per 32.
+template <bool X_BF16, bool SUM16>
 struct Staged {
     uint4 r[X_BF16 ? 4 : 8];
     __device__ __forceinline__ void fetch(const RowsArgs& a, uint32_t chunk, uint32_t tid) {
@@ -81,33 +82,40 @@ struct Staged {
 #pragma unroll
         for (int i = 0; i < N; ++i) r[i] = src[i];
     }
-    __device__ __forceinline__ uint4 masked(int i, bool present) const {
-        return present ? r[i] : make_uint4(0, 0, 0, 0);
+    // Zeroed by an AND, not by a select: a select lets the compiler move the load itself under the condition.
+    __device__ __forceinline__ uint4 masked(int i, uint32_t keep) const {
+        return make_uint4(r[i].x & keep, r[i].y & keep, r[i].z & keep, r[i].w & keep);
     }
     __device__ __forceinline__ void store(uint8_t* buf, uint32_t tid, uint32_t m) const {
         const uint32_t row = tid >> 5, sb = tid & 31u;
-        const bool present = row < m;
+        const uint32_t present = row < m ? 0xffffffffu : 0u;
         float* sums = reinterpret_cast<float*>(buf + kXBuf<X_BF16>);
         if constexpr (X_BF16) {
-            float s = 0.f;
+            float s[2] = {0.f, 0.f};
             uint4 o[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const uint4 t = masked(i, present);
                 pair_words(t.x, t.y, o[i].x, o[i].y);
                 pair_words(t.z, t.w, o[i].z, o[i].w);
-                s = dot2_bf16(t.x, ONES, s);
-                s = dot2_bf16(t.y, ONES, s);
-                s = dot2_bf16(t.z, ONES, s);
-                s = dot2_bf16(t.w, ONES, s);
+                float& si = s[SUM16 ? i / 2 : 0];
+                si = dot2_bf16(t.x, ONES, si);
+                si = dot2_bf16(t.y, ONES, si);
+                si = dot2_bf16(t.z, ONES, si);
+                si = dot2_bf16(t.w, ONES, si);
             }
             uint4* dst = reinterpret_cast<uint4*>(buf + row * XROW + sb * 64u);
 #pragma unroll
             for (int i = 0; i < 4; ++i) dst[i] = o[i];
-            sums[sb * 16u + row] = s;
+            if constexpr (SUM16) {
+                sums[(2u * sb) * 16u + row] = s[0];
+                sums[(2u * sb + 1u) * 16u + row] = s[1];
+            } else {
+                sums[sb * 16u + row] = s[0];
+            }
         } else {
             // x = hi + lo with hi = bf16(x) and lo = bf16(x - hi); the packing instruction pairs (x0, x2), (x1, x3) for free
-            float sh = 0.f, sl = 0.f;
+            float sh2[2] = {0.f, 0.f}, sl2[2] = {0.f, 0.f};
             uint4 oh[4], ol[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {  // eight floats -> four hi words and four lo words
@@ -115,6 +123,7 @@ struct Staged {
                 const float v[8] = {__uint_as_float(ta.x), __uint_as_float(ta.y), __uint_as_float(ta.z), __uint_as_float(ta.w),
                                     __uint_as_float(tb.x), __uint_as_float(tb.y), __uint_as_float(tb.z), __uint_as_float(tb.w)};
                 uint32_t hw[4], lw[4];
+                float &sh = sh2[SUM16 ? i / 2 : 0], &sl = sl2[SUM16 ? i / 2 : 0];
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {  // elements 4q .. 4q+3
                     const float* e = v + 4 * q;
@@ -138,8 +147,15 @@ struct Staged {
                 dh[i] = oh[i];
                 dl[i] = ol[i];
             }
-            sums[sb * 16u + row] = sh;
-            sums[sb * 16u + row + 8u] = sl;
+            if constexpr (SUM16) {
+                sums[(2u * sb) * 16u + row] = sh2[0];
+                sums[(2u * sb) * 16u + row + 8u] = sl2[0];
+                sums[(2u * sb + 1u) * 16u + row] = sh2[1];
+                sums[(2u * sb + 1u) * 16u + row + 8u] = sl2[1];
+            } else {
+                sums[sb * 16u + row] = sh2[0];
+                sums[sb * 16u + row + 8u] = sl2[0];
+            }
         }
     }
 };
@@ -176,7 +192,7 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
     uint32_t m4, magic;
     asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "=v"(m4), "=v"(magic) : "s"(M4), "s"(MAGIC));
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    Staged<X_BF16> st;
+    Staged<X_BF16, false> st;
     auto chunk = [&](uint32_t ch, const WBlock& wb, WBlock& wnext, const uint8_t* bufc, uint8_t* bufn) {
         // the last chunk requests itself again rather than nothing: see Staged::fetch
         const bool more = ch + 1 < nch;
@@ -253,31 +269,146 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
     }
 }
 
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+
+// A word at a 2-byte aligned address (Q6_K blocks are 210 bytes); one global_load_dword.
+__device__ __forceinline__ uint32_t ld4_unaligned(const uint8_t* p) {
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
+
+// The same for Q6_K.  Its scales cover 16 weights, so the product runs on v_mfma_f32_16x16x16_bf16, one
+// instruction per scale group: lane (j, g) supplies weights 4g..4g+3 of the group -- one word of low or high
+// nibbles and the matching two-bit fields of one word of qh, merged into bf16 (128 + q, q < 64) by two
+// v_and_or_b32 per pair -- and receives row j's sums with activation rows 4g..4g+3:
+//   acc += d*sc * C - 160 * d*sc * S16,   S16 = sum of the group's activations (128 + the format's 32),
+// the second term again through the f32 MFMA, four instructions per super-block.
+template <bool X_BF16>
+__global__ __launch_bounds__(256) void q6k_rows_kernel(RowsArgs a) {
+    extern __shared__ uint4 smem4[];
+    uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t j = lane & 15u, g = lane >> 4;
+    const uint32_t row0 = blockIdx.x * 16u;
+    const uint32_t r = row0 + j < a.n ? row0 + j : a.n - 1u;
+    const uint32_t nsb = a.k / 256u, nch = a.k / KC;
+    const uint8_t* wrow = a.w + (size_t)r * nsb * Q6K_BYTES;
+    const uint32_t arow = (X_BF16 ? (j & 7u) : j) * XROW + 8u * g;  // four activations (8 bytes) per lane and group
+
+    struct WBlock {
+        uint32_t ql[8];  // [h][u][s]: bytes 64h + 32u + 16s + 4g .. +3 of ql
+        uint32_t qh[4];  // [h][s]: bytes 32h + 16s + 4g .. +3 of qh
+        uint4 sc;        // the sixteen int8 scales
+        uint32_t d;
+    };
+    auto load_w = [&](uint32_t ch, WBlock& b) {
+        const uint8_t* p = wrow + (size_t)(ch * 4u + wave) * Q6K_BYTES;
+        // (values, not addresses of the struct's fields: taking those would put the block into scratch memory)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b.ql[i] = ld4_unaligned(p + 64 * (i >> 2) + 32 * ((i >> 1) & 1) + 16 * (i & 1) + 4u * g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b.qh[i] = ld4_unaligned(p + 128 + 32 * (i >> 1) + 16 * (i & 1) + 4u * g);
+        b.sc = ld16_unaligned(p + 192);
+        b.d = ld2(p + 208);
+    };
+
+    constexpr uint32_t XBUF = kXBuf<X_BF16>, STAGE = kStage<X_BF16>;
+    uint32_t m4, m2, magic;
+    asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5" : "=v"(m4), "=v"(m2), "=v"(magic) : "s"(M4), "s"(0x00300030u), "s"(MAGIC));
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    Staged<X_BF16, true> st;
+    auto chunk = [&](uint32_t ch, const WBlock& wb, WBlock& wnext, const uint8_t* bufc, uint8_t* bufn) {
+        const bool more = ch + 1 < nch;
+        const uint32_t ahead = more ? ch + 1 : ch;
+        st.fetch(a, ahead, tid);
+        load_w(ahead, wnext);
+        const uint8_t* xb = bufc + arow + wave * 512u;  // the wave's super-block: 256 activations
+        // lane (j, g) of the f32 MFMA: S16[activation row j][group 4t + g] of the wave's sixteen groups
+        const float* sums = reinterpret_cast<const float*>(bufc + XBUF) + wave * 256u + 16u * g + j;
+        const float d = f16_bits_to_f32(wb.d);
+        const uint32_t scw[4] = {wb.sc.x, wb.sc.y, wb.sc.z, wb.sc.w};
+        float ds[16];
+#pragma unroll
+        for (int G = 0; G < 16; ++G) ds[G] = d * (float)(int)(int8_t)((scw[G >> 2] >> (8 * (G & 3))) & 0xffu);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {  // the -160 d sc S16 term: this lane's side is the scale of group 4t + g of its row
+            const float mine = d * (float)(int)(int8_t)((scw[t] >> (8u * g)) & 0xffu);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[64 * t], -160.f * mine, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const uint32_t hq = wb.qh[2 * h + s];
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {  // run rr of half h: group G = 8h + 2rr + s
+                    const uint32_t w = wb.ql[4 * h + 2 * (rr & 1) + s] >> (rr >= 2 ? 4 : 0);
+                    const uint32_t hs = hq >> (2 * rr);
+                    const uint32_t b0 = and_or(hs << 4, m2, and_or(w, m4, magic));        // weights 4g, 4g + 2
+                    const uint32_t b1 = and_or(hs >> 4, m2, and_or(w >> 8, m4, magic));   // weights 4g + 1, 4g + 3
+                    const int G = 8 * h + 2 * rr + s;
+                    const uint2 av = *reinterpret_cast<const uint2*>(xb + 32 * G);  // 16 activations = 32 bytes per group
+                    const f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+                    const f32x4_t c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf16x4_t, av),
+                                                                                __builtin_bit_cast(bf16x4_t, make_uint2(b0, b1)), z, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[v] = fmaf(ds[G], c[v], acc[v]);
+                }
+            }
+        st.store(bufn, tid, a.m);
+        __syncthreads();
+    };
+    WBlock wa, wb2;
+    st.fetch(a, 0, tid);
+    load_w(0, wa);
+    st.store(smem, tid, a.m);
+    __syncthreads();
+    for (uint32_t ch = 0; ch < nch; ch += 2) {
+        chunk(ch, wa, wb2, smem, smem + STAGE);
+        if (ch + 1 < nch) chunk(ch + 1, wb2, wa, smem + STAGE, smem);
+    }
+
+    float4* red = reinterpret_cast<float4*>(smem);
+    red[wave * 64u + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    __syncthreads();
+    if (wave == 0 && g < 2u && row0 + j < a.n) {
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float4 t = red[w * 64 + lane];
+            o[0] += t.x, o[1] += t.y, o[2] += t.z, o[3] += t.w;
+            if constexpr (!X_BF16) {
+                const float4 u = red[w * 64 + lane + 32];
+                o[0] += u.x, o[1] += u.y, o[2] += u.z, o[3] += u.w;
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            if (4u * g + v < a.m) a.y[(size_t)(4u * g + v) * a.n + row0 + j] = o[v];
+    }
+}
+
 }  // namespace
 
-// From four rows on: below that, one GEMV per row is as fast (measured at 12288 x 4096: 10 / 15 / 19 / 24 us for
-// 1..4 GEMVs against 17..19 us here whatever the row count).
-bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k) { return t == HQ_Q4_K && m >= 4 && m <= 8 && k % KC == 0; }
+// From four rows on: below that, one GEMV per row is as fast (measured at 12288 x 4096, Q4_K: 10 / 15 / 19 / 24 us
+// for 1..4 GEMVs against 17..19 us here whatever the row count; Q6_K at 151936 x 4096: 96 us per GEMV row against
+// 343 us here).
+bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k) {
+    return (t == HQ_Q4_K || t == HQ_Q6_K) && m >= 4 && m <= 8 && k % KC == 0;
+}
 
 int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                      uint32_t k, hq_ggml_type t) {
-    (void)t;
     RowsArgs a{x, static_cast<const uint8_t*>(w), y, m, n, k};
-    const int lds = 2 * (xdt == HQ_BF16 ? kStage<true> : kStage<false>);
-    const dim3 grid((n + 15u) / 16u);
-    if (xdt == HQ_BF16) {
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_rows_kernel<true>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                               "hipFuncSetAttribute(rows kernel LDS)"))
-            return rc;
-        hipLaunchKernelGGL(q4k_rows_kernel<true>, grid, dim3(256), lds, s, a);
-    } else {
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_rows_kernel<false>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                               "hipFuncSetAttribute(rows kernel LDS)"))
-            return rc;
-        hipLaunchKernelGGL(q4k_rows_kernel<false>, grid, dim3(256), lds, s, a);
-    }
+    const bool bf = xdt == HQ_BF16;
+    const int lds = 2 * (bf ? kStage<true> : kStage<false>);
+    void (*kern)(RowsArgs) = t == HQ_Q4_K ? (bf ? q4k_rows_kernel<true> : q4k_rows_kernel<false>)
+                                          : (bf ? q6k_rows_kernel<true> : q6k_rows_kernel<false>);
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(rows kernel LDS)"))
+        return rc;
+    hipLaunchKernelGGL(kern, dim3((n + 15u) / 16u), dim3(256), lds, s, a);
     return check_launch("rows kernel launch");
 }
 

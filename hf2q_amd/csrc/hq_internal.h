@@ -157,9 +157,10 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
 // and c are literals (gfx9 VOP3 takes no literal operands), so the constants are
 // passed in registers and the instruction is written out.
 __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t b, uint32_t c) {
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
+    // Plain C on purpose: the compiler fuses it into one v_and_or_b32 when b and c sit in VGPRs, and, unlike an
+    // inline-asm instruction, counts it as a VALU write when it spaces a dependent MFMA (a matrix instruction that
+    // reads a register less than two wait states after an asm-hidden write gets the old contents).
+    return (a & b) | c;
 }
 
 // Q4_K: 6-bit scale / min of sub-blocks (2c, 2c+1) for chunk c in [0,4) from the

@@ -317,11 +317,11 @@ def test_mul_mat_id_grouped_routing_properties(oracle, dev):
 ROWS_SHAPES = [(4, 64, 1024), (4, 200, 4096), (4, 16, 2048), (5, 33, 1024), (6, 130, 3072), (7, 250, 2048), (8, 96, 12288)]
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,n,k", ROWS_SHAPES)
-def test_small_batch_rows_match_f64_oracle(oracle, dev, xdt, m, n, k):
-    """Q4_K with k % 1024 == 0 and 4 <= m <= 8 takes the kernel that fetches every weight once for all rows."""
-    t = HQ_Q4_K
+def test_small_batch_rows_match_f64_oracle(oracle, dev, t, xdt, m, n, k):
+    """Q4_K / Q6_K with k % 1024 == 0 and 4 <= m <= 8 take the kernel that fetches every weight once for all rows."""
     blocks = oracle.quantize(weights(3 * n + k + m, n, k), k, t, threads=8)
     x = acts(n + k + m, m, k)
     xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
@@ -331,7 +331,7 @@ def test_small_batch_rows_match_f64_oracle(oracle, dev, xdt, m, n, k):
     y = torch.full((m, n), float("nan"), device=dev)
     wd = torch.from_numpy(blocks).to(dev)
     ops.quantized_matmul_ggml(xd, wd, y, GgmlQuantizedMatmulParams(m, n, k, t))
-    assert_matmul_close(y.cpu().numpy(), ref, f"rows {xdt} {m}x{n}x{k}")
+    assert_matmul_close(y.cpu().numpy(), ref, f"rows t={t} {xdt} {m}x{n}x{k}")
     # every row equals the one-row product of the same activations (the GEMV kernel) to accumulation noise
     y1 = torch.empty((1, n), device=dev)
     for r in range(m):
@@ -339,9 +339,10 @@ def test_small_batch_rows_match_f64_oracle(oracle, dev, xdt, m, n, k):
         assert np.abs(y1.cpu().numpy()[0] - y.cpu().numpy()[r]).max() <= 1e-4 * np.abs(ref).max()
 
 
-def test_small_batch_rows_adversarial_blocks_and_scaling(oracle, dev):
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
+def test_small_batch_rows_adversarial_blocks_and_scaling(oracle, dev, t):
     """Every scale / min / nibble pattern; and scaling the activations by a power of two scales the result exactly."""
-    t, m, n, k = HQ_Q4_K, 8, 48, 2048
+    m, n, k = 8, 48, 2048
     blocks = _adversarial_blocks(oracle, t, n * k // 256, 9)
     x = acts(2, m, k)
     wd = torch.from_numpy(blocks).to(dev)
