@@ -145,7 +145,7 @@ def _timed_steps(a, step, n_variants):
                     step(i)
                 singles.append(g)
         torch.cuda.synchronize()
-        calls = [big.replay] * q + [singles[i % n_variants].replay for i in range(r)]
+        calls = ([big.replay] * q if q else []) + [singles[i % n_variants].replay for i in range(r)]
         for c in ([big.replay] if q else []) + [g.replay for g in singles]:  # untimed: first replay of each graph
             c()
     e0, e1 = _events(1)[0]
