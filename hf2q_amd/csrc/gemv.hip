@@ -638,7 +638,7 @@ __global__ __launch_bounds__(256) void gemv_jobs_kernel(KJobs js) {
 
 // Dense GEMV for matrices with many wave groups per CU: one workgroup of WAVES
 // waves per CU (the launch asks for more than half of the CU's LDS, so two never
-// share a CU), each CU owning an equal contiguous share of the wave groups.
+// share a CU), each CU owning an equal share of the wave groups.
 // Inside the CU the waves take wave groups from a counter in LDS instead of a
 // fixed split: the SIMD's issue arbitration favours its oldest wave, so with a
 // fixed split the youngest wave of every SIMD finishes long after the others and
@@ -660,15 +660,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_queue_kernel(KArgs a) {
     Walk<TYPE, X_BF16, PAIR, NR, D> wk;
     wk.init(a, a.w, lds_x, lds_s);
 
-    // this CU's share of the wave groups: [begin, begin + count)
-    const uint32_t per = a.groups / gridDim.x, rem = a.groups % gridDim.x;
-    const uint32_t begin = blockIdx.x * per + (blockIdx.x < rem ? blockIdx.x : rem);
-    const uint32_t count = per + (blockIdx.x < rem ? 1u : 0u);
+    // this CU's share of the wave groups: blockIdx.x, blockIdx.x + gridDim.x, ... (its i-th group is group_of(i)).
+    // All CUs so walk the matrix front to back together and the fetches in flight at any moment cover one
+    // dense window of it; with a contiguous share per CU they would come from gridDim.x distant places
+    // (measured 3 % slower).
+    const uint32_t count = (a.groups + gridDim.x - 1u - blockIdx.x) / gridDim.x;
     const uint32_t rows_per_group = wk.rpw * NR;
+    auto group_of = [&](uint32_t i) -> uint32_t { return i * gridDim.x + blockIdx.x; };
 
     // the first WAVES wave groups are claimed by wave index, the rest from the counter
     uint32_t cur = threadIdx.x >> 6;
-    if (cur < count) wk.prime((begin + cur) * rows_per_group);
+    if (cur < count) wk.prime(group_of(cur) * rows_per_group);
 
     if (threadIdx.x == 0) *lds_q = WAVES;
     if (threadIdx.x < xchunks) stage_store<X_BF16, PAIR>(xraw, threadIdx.x, lds_x, lds_s);
@@ -687,7 +689,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_queue_kernel(KArgs a) {
     uint32_t nxt = __builtin_amdgcn_readfirstlane(grab());
     while (cur < count) {
         const uint32_t after = grab();  // claimed now, read when this group is done
-        wk.group((begin + cur) * rows_per_group, (begin + nxt) * rows_per_group, nxt < count, a.y, true);
+        wk.group(group_of(cur) * rows_per_group, group_of(nxt) * rows_per_group, nxt < count, a.y, true);
         cur = nxt;
         nxt = __builtin_amdgcn_readfirstlane(after);
     }

@@ -204,22 +204,23 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
         // S[activation row j][sub-block 4t + g]
         const float* sums = reinterpret_cast<const float*>(bufc + XBUF) + wave * 128u + 16u * g + j;
         const float d = f16_bits_to_f32(wb.hdr.x & 0xffffu), dmin = f16_bits_to_f32(wb.hdr.x >> 16);
-        float ds[8], off[8];
+        // -sum_b off_b * S_b, off_b = 128 d sc_b + dmin m_b, for all sixteen activation rows at once: the weights'
+        // side of that small product is off of sub-block 4t + g of this lane's row.  It is picked while the scales
+        // are unpacked, from plain values: a select between elements of a local array makes the compiler index
+        // the array in scratch memory.
+        float ds[8], mine0 = 0.f, mine1 = 0.f;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             uint32_t sc0, sc1, m0, m1;
             q4k_scales(wb.hdr.y, wb.hdr.z, wb.hdr.w, c, sc0, sc1, m0, m1);
             ds[2 * c] = d * (float)sc0, ds[2 * c + 1] = d * (float)sc1;
-            off[2 * c] = fmaf(128.f, ds[2 * c], dmin * (float)m0), off[2 * c + 1] = fmaf(128.f, ds[2 * c + 1], dmin * (float)m1);
+            const float oe = fmaf(128.f, ds[2 * c], dmin * (float)m0), oo = fmaf(128.f, ds[2 * c + 1], dmin * (float)m1);
+            const float o = (g & 1u) ? oo : oe;  // sub-blocks 2c and 2c + 1 are g = 2 (c & 1) and 2 (c & 1) + 1 of t = c / 2
+            float& mine = c < 2 ? mine0 : mine1;
+            mine = (g >> 1) == (uint32_t)(c & 1) ? o : mine;
         }
-        // -sum_b off_b * S_b for all sixteen activation rows at once: the weights' side of that small product is
-        // off of sub-block 4t + g of this lane's row
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const float o01 = (g & 1u) ? off[4 * t + 1] : off[4 * t], o23 = (g & 1u) ? off[4 * t + 3] : off[4 * t + 2];
-            const float mine = (g & 2u) ? o23 : o01;
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[64 * t], -mine, acc, 0, 0, 0);
-        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[0], -mine0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[64], -mine1, acc, 0, 0, 0);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t w0 = wb.q[c].x, w1 = wb.q[c].y;
