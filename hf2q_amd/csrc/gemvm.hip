@@ -49,6 +49,7 @@ constexpr uint32_t kXBuf = (X_BF16 ? 8 : 16) * XROW;
 template <bool X_BF16>
 constexpr uint32_t kStage = kXBuf<X_BF16> + SBUF;
 constexpr uint32_t M4 = 0x000f000fu, MAGIC = 0x43004300u;
+constexpr uint32_t WIDE_MIN_ROWS = 49152;  // 768 workgroups of 64 rows
 
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2v_t;
@@ -160,13 +161,46 @@ struct Staged {
     }
 };
 
-template <bool X_BF16>
+// Epilogue of both kernels: the sum of the parts of the waves that share rows and of the hi and lo rows (f32
+// activations), through LDS; lanes g < 2 of the first wave of a group store activation rows 4g..4g+3 of weight row
+// row0 + j.
+template <bool X_BF16, int NSB>
+__device__ __forceinline__ void store_rows(const RowsArgs& a, uint8_t* smem, const f32x4_t& acc, uint32_t row0) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t j = lane & 15u, g = lane >> 4;
+    float4* red = reinterpret_cast<float4*>(smem);
+    red[wave * 64u + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    __syncthreads();
+    constexpr uint32_t SHARE = 4u / NSB;  // waves that hold parts of the same rows
+    if (wave % SHARE == 0 && g < 2u && row0 + j < a.n) {
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t w = wave; w < wave + SHARE; ++w) {
+            const float4 t = red[w * 64u + lane];
+            o[0] += t.x, o[1] += t.y, o[2] += t.z, o[3] += t.w;
+            if constexpr (!X_BF16) {
+                const float4 u = red[w * 64u + lane + 32u];  // the lo rows: activation rows 8 + 4g + v
+                o[0] += u.x, o[1] += u.y, o[2] += u.z, o[3] += u.w;
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            if (4u * g + v < a.m) a.y[(size_t)(4u * g + v) * a.n + row0 + j] = o[v];
+    }
+}
+
+// NSB = super-blocks of a 1024-element chunk a wave works through.  1: the workgroup owns 16 weight rows and its
+// waves a quarter of k each (many workgroups for small matrices).  4: it owns 64 rows, each wave 16 of them over
+// all of k, so a staged chunk of activations and its barrier serve four times the weights.  2: 32 rows, two waves
+// per 16 rows (half the registers of 4 for the fetches in flight).
+template <bool X_BF16, int NSB>
 __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
     extern __shared__ uint4 smem4[];
     uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t j = lane & 15u, g = lane >> 4;
-    const uint32_t row0 = blockIdx.x * 16u;
+    constexpr uint32_t SHARE = 4u / NSB;  // waves per 16 rows
+    const uint32_t row0 = (blockIdx.x * (uint32_t)NSB + wave / SHARE) * 16u, sb0 = (wave % SHARE) * NSB;
     const uint32_t r = row0 + j < a.n ? row0 + j : a.n - 1u;  // rows past the end repeat the last one, not stored
     const uint32_t nsb = a.k / 256u, nch = a.k / KC;
     const uint8_t* wrow = a.w + (size_t)r * nsb * Q4K_BYTES + 16u + 8u * g;  // this lane's eight bytes of chunk 0
@@ -176,11 +210,17 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
         uint4 hdr;
         uint2 q[4];
     };
-    auto load_w = [&](uint32_t ch, WBlock& b) {
-        const uint8_t* p = wrow + (size_t)(ch * 4u + wave) * Q4K_BYTES;
-        b.hdr = *reinterpret_cast<const uint4*>(p - 16u - 8u * g);
+    struct WSet {
+        WBlock b[NSB];
+    };
+    auto load_w = [&](uint32_t ch, WSet& set) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) b.q[c] = *reinterpret_cast<const uint2*>(p + 32 * c);
+        for (int s = 0; s < NSB; ++s) {
+            const uint8_t* p = wrow + (size_t)(ch * 4u + sb0 + s) * Q4K_BYTES;
+            set.b[s].hdr = *reinterpret_cast<const uint4*>(p - 16u - 8u * g);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) set.b[s].q[c] = *reinterpret_cast<const uint2*>(p + 32 * c);
+        }
     };
 
     constexpr uint32_t XBUF = kXBuf<X_BF16>, STAGE = kStage<X_BF16>;
@@ -193,16 +233,11 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
     asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "=v"(m4), "=v"(magic) : "s"(M4), "s"(MAGIC));
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     Staged<X_BF16, false> st;
-    auto chunk = [&](uint32_t ch, const WBlock& wb, WBlock& wnext, const uint8_t* bufc, uint8_t* bufn) {
-        // the last chunk requests itself again rather than nothing: see Staged::fetch
-        const bool more = ch + 1 < nch;
-        const uint32_t ahead = more ? ch + 1 : ch;
-        st.fetch(a, ahead, tid);
-        load_w(ahead, wnext);
-        const uint8_t* xb = bufc + arow + wave * 512u;  // the wave's super-block: 256 activations
-        // sums of the wave's eight sub-blocks as the first operand of a 16x16x4 f32 MFMA: lane (j, g) holds
+    auto super_block = [&](const WBlock& wb, uint32_t sbi, const uint8_t* bufc) {
+        const uint8_t* xb = bufc + arow + sbi * 512u;  // super-block sbi of the chunk: 256 activations
+        // sums of its eight sub-blocks as the first operand of a 16x16x4 f32 MFMA: lane (j, g) holds
         // S[activation row j][sub-block 4t + g]
-        const float* sums = reinterpret_cast<const float*>(bufc + XBUF) + wave * 128u + 16u * g + j;
+        const float* sums = reinterpret_cast<const float*>(bufc + XBUF) + sbi * 128u + 16u * g + j;
         const float d = f16_bits_to_f32(wb.hdr.x & 0xffffu), dmin = f16_bits_to_f32(wb.hdr.x >> 16);
         // -sum_b off_b * S_b, off_b = 128 d sc_b + dmin m_b, for all sixteen activation rows at once: the weights'
         // side of that small product is off of sub-block 4t + g of this lane's row.  It is picked while the scales
@@ -236,10 +271,19 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) acc[v] = fmaf(ds[2 * c + 1], chi[v], fmaf(ds[2 * c], clo[v], acc[v]));
         }
+    };
+    auto chunk = [&](uint32_t ch, const WSet& wb, WSet& wnext, const uint8_t* bufc, uint8_t* bufn) {
+        // the last chunk requests itself again rather than nothing: see Staged::fetch
+        const bool more = ch + 1 < nch;
+        const uint32_t ahead = more ? ch + 1 : ch;
+        st.fetch(a, ahead, tid);
+        load_w(ahead, wnext);
+#pragma unroll
+        for (int s = 0; s < NSB; ++s) super_block(wb.b[s], sb0 + s, bufc);
         st.store(bufn, tid, a.m);
         __syncthreads();  // the other buffer is complete; this one may be overwritten by the next pass
     };
-    WBlock wa, wb2;
+    WSet wa, wb2;
     st.fetch(a, 0, tid);
     load_w(0, wa);
     st.store(smem, tid, a.m);
@@ -249,25 +293,7 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
         if (ch + 1 < nch) chunk(ch + 1, wb2, wa, smem + STAGE, smem);
     }
 
-    // ---- sum of the four waves (and of the hi and lo rows), store ----
-    float4* red = reinterpret_cast<float4*>(smem);
-    red[wave * 64u + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    __syncthreads();
-    if (wave == 0 && g < 2u && row0 + j < a.n) {
-        float o[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float4 t = red[w * 64 + lane];
-            o[0] += t.x, o[1] += t.y, o[2] += t.z, o[3] += t.w;
-            if constexpr (!X_BF16) {
-                const float4 u = red[w * 64 + lane + 32];  // the lo rows: activation rows 8 + 4g + v
-                o[0] += u.x, o[1] += u.y, o[2] += u.z, o[3] += u.w;
-            }
-        }
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-            if (4u * g + v < a.m) a.y[(size_t)(4u * g + v) * a.n + row0 + j] = o[v];
-    }
+    store_rows<X_BF16, NSB>(a, smem, acc, row0);
 }
 
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
@@ -285,13 +311,14 @@ __device__ __forceinline__ uint32_t ld4_unaligned(const uint8_t* p) {
 // v_and_or_b32 per pair -- and receives row j's sums with activation rows 4g..4g+3:
 //   acc += d*sc * C - 160 * d*sc * S16,   S16 = sum of the group's activations (128 + the format's 32),
 // the second term again through the f32 MFMA, four instructions per super-block.
-template <bool X_BF16>
+template <bool X_BF16, int NSB>
 __global__ __launch_bounds__(256) void q6k_rows_kernel(RowsArgs a) {
     extern __shared__ uint4 smem4[];
     uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t j = lane & 15u, g = lane >> 4;
-    const uint32_t row0 = blockIdx.x * 16u;
+    constexpr uint32_t SHARE = 4u / NSB;
+    const uint32_t row0 = (blockIdx.x * (uint32_t)NSB + wave / SHARE) * 16u, sb0 = (wave % SHARE) * NSB;
     const uint32_t r = row0 + j < a.n ? row0 + j : a.n - 1u;
     const uint32_t nsb = a.k / 256u, nch = a.k / KC;
     const uint8_t* wrow = a.w + (size_t)r * nsb * Q6K_BYTES;
@@ -303,15 +330,22 @@ __global__ __launch_bounds__(256) void q6k_rows_kernel(RowsArgs a) {
         uint4 sc;        // the sixteen int8 scales
         uint32_t d;
     };
-    auto load_w = [&](uint32_t ch, WBlock& b) {
-        const uint8_t* p = wrow + (size_t)(ch * 4u + wave) * Q6K_BYTES;
-        // (values, not addresses of the struct's fields: taking those would put the block into scratch memory)
+    struct WSet {
+        WBlock b[NSB];
+    };
+    auto load_w = [&](uint32_t ch, WSet& set) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) b.ql[i] = ld4_unaligned(p + 64 * (i >> 2) + 32 * ((i >> 1) & 1) + 16 * (i & 1) + 4u * g);
+        for (int s = 0; s < NSB; ++s) {
+            WBlock& b = set.b[s];
+            const uint8_t* p = wrow + (size_t)(ch * 4u + sb0 + s) * Q6K_BYTES;
+            // (values, not addresses of the struct's fields: taking those would put the block into scratch memory)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) b.qh[i] = ld4_unaligned(p + 128 + 32 * (i >> 1) + 16 * (i & 1) + 4u * g);
-        b.sc = ld16_unaligned(p + 192);
-        b.d = ld2(p + 208);
+            for (int i = 0; i < 8; ++i) b.ql[i] = ld4_unaligned(p + 64 * (i >> 2) + 32 * ((i >> 1) & 1) + 16 * (i & 1) + 4u * g);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b.qh[i] = ld4_unaligned(p + 128 + 32 * (i >> 1) + 16 * (i & 1) + 4u * g);
+            b.sc = ld16_unaligned(p + 192);
+            b.d = ld2(p + 208);
+        }
     };
 
     constexpr uint32_t XBUF = kXBuf<X_BF16>, STAGE = kStage<X_BF16>;
@@ -319,14 +353,10 @@ __global__ __launch_bounds__(256) void q6k_rows_kernel(RowsArgs a) {
     asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5" : "=v"(m4), "=v"(m2), "=v"(magic) : "s"(M4), "s"(0x00300030u), "s"(MAGIC));
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     Staged<X_BF16, true> st;
-    auto chunk = [&](uint32_t ch, const WBlock& wb, WBlock& wnext, const uint8_t* bufc, uint8_t* bufn) {
-        const bool more = ch + 1 < nch;
-        const uint32_t ahead = more ? ch + 1 : ch;
-        st.fetch(a, ahead, tid);
-        load_w(ahead, wnext);
-        const uint8_t* xb = bufc + arow + wave * 512u;  // the wave's super-block: 256 activations
-        // lane (j, g) of the f32 MFMA: S16[activation row j][group 4t + g] of the wave's sixteen groups
-        const float* sums = reinterpret_cast<const float*>(bufc + XBUF) + wave * 256u + 16u * g + j;
+    auto super_block = [&](const WBlock& wb, uint32_t sbi, const uint8_t* bufc) {
+        const uint8_t* xb = bufc + arow + sbi * 512u;  // super-block sbi of the chunk: 256 activations
+        // lane (j, g) of the f32 MFMA: S16[activation row j][group 4t + g] of the super-block's sixteen groups
+        const float* sums = reinterpret_cast<const float*>(bufc + XBUF) + sbi * 256u + 16u * g + j;
         const float d = f16_bits_to_f32(wb.d);
         const uint32_t scw[4] = {wb.sc.x, wb.sc.y, wb.sc.z, wb.sc.w};
         float ds[16];
@@ -357,10 +387,18 @@ __global__ __launch_bounds__(256) void q6k_rows_kernel(RowsArgs a) {
                     for (int v = 0; v < 4; ++v) acc[v] = fmaf(ds[G], c[v], acc[v]);
                 }
             }
+    };
+    auto chunk = [&](uint32_t ch, const WSet& wb, WSet& wnext, const uint8_t* bufc, uint8_t* bufn) {
+        const bool more = ch + 1 < nch;
+        const uint32_t ahead = more ? ch + 1 : ch;
+        st.fetch(a, ahead, tid);
+        load_w(ahead, wnext);
+#pragma unroll
+        for (int s = 0; s < NSB; ++s) super_block(wb.b[s], sb0 + s, bufc);
         st.store(bufn, tid, a.m);
         __syncthreads();
     };
-    WBlock wa, wb2;
+    WSet wa, wb2;
     st.fetch(a, 0, tid);
     load_w(0, wa);
     st.store(smem, tid, a.m);
@@ -370,24 +408,7 @@ __global__ __launch_bounds__(256) void q6k_rows_kernel(RowsArgs a) {
         if (ch + 1 < nch) chunk(ch + 1, wb2, wa, smem + STAGE, smem);
     }
 
-    float4* red = reinterpret_cast<float4*>(smem);
-    red[wave * 64u + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    __syncthreads();
-    if (wave == 0 && g < 2u && row0 + j < a.n) {
-        float o[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float4 t = red[w * 64 + lane];
-            o[0] += t.x, o[1] += t.y, o[2] += t.z, o[3] += t.w;
-            if constexpr (!X_BF16) {
-                const float4 u = red[w * 64 + lane + 32];
-                o[0] += u.x, o[1] += u.y, o[2] += u.z, o[3] += u.w;
-            }
-        }
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-            if (4u * g + v < a.m) a.y[(size_t)(4u * g + v) * a.n + row0 + j] = o[v];
-    }
+    store_rows<X_BF16, NSB>(a, smem, acc, row0);
 }
 
 }  // namespace
@@ -404,12 +425,23 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
     RowsArgs a{x, static_cast<const uint8_t*>(w), y, m, n, k};
     const bool bf = xdt == HQ_BF16;
     const int lds = 2 * (bf ? kStage<true> : kStage<false>);
-    void (*kern)(RowsArgs) = t == HQ_Q4_K ? (bf ? q4k_rows_kernel<true> : q4k_rows_kernel<false>)
-                                          : (bf ? q6k_rows_kernel<true> : q6k_rows_kernel<false>);
+    // more rows per workgroup once that still gives every CU three workgroups of the first round; Q6_K stops at
+    // two super-blocks per wave (at four, the fetches in flight leave one wave per SIMD) except with f32
+    // activations, whose LDS footprint limits the CU to two workgroups anyway
+    const uint32_t nsb = n < WIDE_MIN_ROWS ? 1u : t == HQ_Q4_K || !bf ? 4u : 2u;
+    void (*kern)(RowsArgs);
+    if (t == HQ_Q4_K)
+        kern = nsb == 4 ? (bf ? q4k_rows_kernel<true, 4> : q4k_rows_kernel<false, 4>)
+                        : (bf ? q4k_rows_kernel<true, 1> : q4k_rows_kernel<false, 1>);
+    else
+        kern = nsb == 4 ? q6k_rows_kernel<false, 4>
+               : nsb == 2 ? q6k_rows_kernel<true, 2>
+                          : (bf ? q6k_rows_kernel<true, 1> : q6k_rows_kernel<false, 1>);
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                            "hipFuncSetAttribute(rows kernel LDS)"))
         return rc;
-    hipLaunchKernelGGL(kern, dim3((n + 15u) / 16u), dim3(256), lds, s, a);
+    const uint32_t rows_per_wg = 16u * nsb;
+    hipLaunchKernelGGL(kern, dim3((n + rows_per_wg - 1u) / rows_per_wg), dim3(256), lds, s, a);
     return check_launch("rows kernel launch");
 }
 

@@ -340,6 +340,25 @@ def test_small_batch_rows_match_f64_oracle(oracle, dev, t, xdt, m, n, k):
 
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
+@pytest.mark.parametrize("xdt,m", [("bf16", 8), ("f32", 5)])
+def test_small_batch_rows_tall_matrix(oracle, dev, t, xdt, m):
+    """From 49152 weight rows on a workgroup takes 64 rows instead of 16; the last workgroup here is ragged (n % 64 = 40,
+    so one of its waves has 8 rows and one none).  Weights: a quantized 1024-row tile repeated, rotated per repeat."""
+    n, k, tile = 49152 + 40, 2048, 1024
+    tile_blocks = oracle.quantize(weights(77, tile, k), k, t, threads=8).reshape(tile, -1)
+    reps = -(-n // tile)
+    blocks = np.concatenate([np.roll(tile_blocks, 37 * i, axis=0) for i in range(reps)])[:n].copy().reshape(-1)
+    x = acts(78, m, k)
+    xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
+    xd = torch.from_numpy(x).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    ref = oracle.qmatmul_f64(xv, blocks, m, n, k, t)
+    y = torch.full((m, n + 64), float("nan"), device=dev)[:, :n].contiguous()
+    ops.quantized_matmul_ggml(xd, torch.from_numpy(blocks).to(dev), y, GgmlQuantizedMatmulParams(m, n, k, t))
+    assert_matmul_close(y.cpu().numpy(), ref, f"rows, tall matrix t={t} {xdt} m={m}")
+
+
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
 def test_small_batch_rows_adversarial_blocks_and_scaling(oracle, dev, t):
     """Every scale / min / nibble pattern; and scaling the activations by a power of two scales the result exactly."""
     m, n, k = 8, 48, 2048
