@@ -1,4 +1,4 @@
-// Dequant-fused product for 2..8 activation rows (small-batch decode) on the matrix cores:
+// Dequant-fused product for 3..8 activation rows (small-batch decode) on the matrix cores:
 // y[m, n] = sum_k x[m, k] * W[n, k] with every weight fetched once for all rows, where the GEMV
 // kernel would fetch it once per row.  Q4_K and Q6_K weights, k a multiple of 1024.
 //
@@ -413,11 +413,12 @@ __global__ __launch_bounds__(256) void q6k_rows_kernel(RowsArgs a) {
 
 }  // namespace
 
-// From four rows on: below that, one GEMV per row is as fast (measured at 12288 x 4096, Q4_K: 10 / 15 / 19 / 24 us
-// for 1..4 GEMVs against 17..19 us here whatever the row count; Q6_K at 151936 x 4096: 96 us per GEMV row against
-// 343 us here).
+// Q4_K from three rows on, Q6_K from four: below that, one GEMV per row is as fast.  Measured, bf16 activations:
+// Q4_K 12288 x 4096: 10 / 15 / 19 / 24 us for 1..4 GEMVs against 15..16 us here whatever the row count; Q6_K
+// 151936 x 4096: 96 us per GEMV row against 310 us here.
 bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k) {
-    return (t == HQ_Q4_K || t == HQ_Q6_K) && m >= 4 && m <= 8 && k % KC == 0;
+    const uint32_t from = t == HQ_Q4_K ? 3u : 4u;
+    return (t == HQ_Q4_K || t == HQ_Q6_K) && m >= from && m <= 8 && k % KC == 0;
 }
 
 int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,

@@ -45,7 +45,7 @@ int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type
 // Up to four independent GEMVs of one weight type and activation dtype in a single launch.
 int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_act_dtype xdt, hq_ggml_type t);
 
-// 2..8 activation rows sharing one pass over the weights (gemvm.hip); gemv_rows_supported() says
+// 3..8 activation rows sharing one pass over the weights (gemvm.hip); gemv_rows_supported() says
 // whether (type, m, k) has such a kernel, otherwise the GEMV runs once per row.
 bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k);
 int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,

@@ -314,14 +314,14 @@ def test_mul_mat_id_grouped_routing_properties(oracle, dev):
 
 # ---- 4..8 activation rows sharing one pass over the weights (small-batch decode) ------
 
-ROWS_SHAPES = [(4, 64, 1024), (4, 200, 4096), (4, 16, 2048), (5, 33, 1024), (6, 130, 3072), (7, 250, 2048), (8, 96, 12288)]
+ROWS_SHAPES = [(3, 80, 2048), (4, 64, 1024), (4, 200, 4096), (4, 16, 2048), (5, 33, 1024), (6, 130, 3072), (7, 250, 2048), (8, 96, 12288)]
 
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,n,k", ROWS_SHAPES)
 def test_small_batch_rows_match_f64_oracle(oracle, dev, t, xdt, m, n, k):
-    """Q4_K / Q6_K with k % 1024 == 0 and 4 <= m <= 8 take the kernel that fetches every weight once for all rows."""
+    """Q4_K (3 <= m <= 8) and Q6_K (4 <= m <= 8) with k % 1024 == 0 take the kernel that fetches every weight once for all rows."""
     blocks = oracle.quantize(weights(3 * n + k + m, n, k), k, t, threads=8)
     x = acts(n + k + m, m, k)
     xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
