@@ -98,12 +98,14 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
     if (blockIdx.x >= m) {
         const uint32_t wr = (blockIdx.x - m) * 16u + (tid >> 4);
         float bound = 0.f;
-        if constexpr (TYPE == HQ_Q4_K) {
+        if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K) {  // |w| <= |d| * 63 * qmax + |dmin| * 63
+            constexpr uint32_t BYTES = TYPE == HQ_Q5_K ? Q5K_BYTES : Q4K_BYTES;
+            constexpr float DQ = TYPE == HQ_Q5_K ? 1953.f : 945.f;
             const uint32_t nsb = k / 256;
-            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nsb * Q4K_BYTES;
+            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nsb * BYTES;
             for (uint32_t sb = tid & 15u; sb < nsb; sb += 16u) {
-                const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow + (size_t)sb * Q4K_BYTES);
-                const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * 945.f + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
+                const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow + (size_t)sb * BYTES);
+                const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * DQ + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
                 bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;  // inf / nan scales do not set the exponent
             }
         } else if constexpr (TYPE == HQ_Q6_K) {  // |w| <= |d| * 128 * 32
@@ -313,9 +315,14 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W
 
 // One workgroup tile of Q4_K weights: rows m0.. of the activations, weight rows n0...  The four
 // waves form a (4 / WN) x WN grid; a wave owns MT x NT MFMA tiles of 32 x 32.
-template <int MT, int NT, int WN>
+// TYPE = HQ_Q5_K: the same tile over 176-byte super-blocks; a lane also keeps the sixteen qh bytes that go with
+// its nibble bytes (they serve all four chunks of the super-block, bit 2c + hi for sub-block 2c + hi) and ORs the
+// fifth bit into the masked nibbles, three more VALU instructions per four weights.
+template <int MT, int NT, int WN, int TYPE = HQ_Q4_K>
 __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
+    constexpr bool Q5 = TYPE == HQ_Q5_K;
+    constexpr uint32_t BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES, QS = Q5 ? 48u : 16u;  // super-block size, offset of the nibbles
     const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -323,7 +330,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
 
     const uint32_t nsb = a.k / 256, nstages = a.k / BK;
-    const uint32_t row_bytes = nsb * Q4K_BYTES;
+    const uint32_t row_bytes = nsb * BYTES;
     ActTile at;
     at.init(a, W, m0, lane, wave);
 
@@ -339,14 +346,18 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     }
     uint4 braw[4][NT];        // nibbles of stages s, s+1, s+2 in slots s%4 (a stage is a chunk of its super-block: slot = c)
     uint4 hdr[NT], hdrn[NT];  // super-block headers: current, next
+    [[maybe_unused]] uint4 hq[NT], hqn[NT];  // Q5_K: qh bytes 16*lg.. of the current and the next super-block
     auto load_b = [&](uint32_t sblk, int c, int slot) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-            braw[slot][nt] = ld16(wrow[nt] + (size_t)sblk * Q4K_BYTES + 16 + 32 * c + 16 * lg);
+            braw[slot][nt] = ld16(wrow[nt] + (size_t)sblk * BYTES + QS + 32 * c + 16 * lg);
     };
-    auto load_hdr = [&](uint32_t sblk, uint4* h) {
+    auto load_hdr = [&](uint32_t sblk, uint4* h, [[maybe_unused]] uint4* q) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) h[nt] = ld16(wrow[nt] + (size_t)sblk * Q4K_BYTES);
+        for (int nt = 0; nt < NT; ++nt) {
+            h[nt] = ld16(wrow[nt] + (size_t)sblk * BYTES);
+            if constexpr (Q5) q[nt] = ld16(wrow[nt] + (size_t)sblk * BYTES + 16 + 16 * lg);
+        }
     };
 
     f32x16_t acc[MT][NT];
@@ -376,12 +387,18 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     // fragment word.  Quarter q = e/2 is one nibble word (nt = q/2, word pair half = q%2), masked
     // once and kept in mw for its second eighth.
     uint32_t mw[2 * NT];
-    auto b_eighth = [&](const uint4* b, const float (*dsc)[2], const float (*ndm)[2], int ks, int e, uint4* bfw) {
+    // (qv, cc: Q5_K only -- the qh bytes of the stage's super-block and the stage's chunk index in it)
+    auto b_eighth = [&](const uint4* b, const float (*dsc)[2], const float (*ndm)[2], int ks, int e, uint4* bfw,
+                        [[maybe_unused]] const uint4* qv, [[maybe_unused]] int cc) {
         const int q = e >> 1, part = e & 1, nt = q >> 1, half = q & 1;
         const int hi = ks >> 1;  // 0: low nibbles, 1: high nibbles
         if (part == 0) {
             const uint32_t w = (ks & 1) ? (half ? b[nt].w : b[nt].z) : (half ? b[nt].y : b[nt].x);
             uint32_t m = (hi ? w >> 4 : w) & 0x0f0f0f0fu;
+            if constexpr (Q5) {
+                const uint32_t h = (ks & 1) ? (half ? qv[nt].w : qv[nt].z) : (half ? qv[nt].y : qv[nt].x);
+                m |= ((h >> (2 * cc + hi)) & 0x01010101u) << 4;
+            }
             // opaque, so that the conversions stay v_cvt_f32_ubyte0..3 of this one register instead of
             // a bit-field extract plus conversion each
             asm volatile("" : "+v"(m));
@@ -403,17 +420,17 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     static_assert(kSteps >= DMA_PER_WAVE && (E >= MT ? E % MT == 0 : MT % E == 0 && MT / E >= 2), "the spreading below assumes it");
 
     // ---- prologue: everything the first stage needs, and the second stage's nibbles ----
-    load_hdr(0, hdr);
+    load_hdr(0, hdr, hq);
     load_b(0, 0, 0);
     if (nstages > 1) load_b(0, 1, 1);  // k >= 256: a super-block has four stages
     at.fetch_all(0, 0);
-    if (nsb > 1) load_hdr(1, hdrn);
+    if (nsb > 1) load_hdr(1, hdrn, hqn);
     float dsc[NT][2], ndm[NT][2];      // scales of the stage being multiplied
     uint4 bfc[NT], bfn[NT];            // weight fragments: current k-step, next
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     scales_of(hdr, 0, dsc, ndm);
 #pragma unroll
-    for (int e = 0; e < E; ++e) b_eighth(braw[0], dsc, ndm, 0, e, bfc);
+    for (int e = 0; e < E; ++e) b_eighth(braw[0], dsc, ndm, 0, e, bfc, hq, 0);
     __syncthreads();
 
     // The loop is software pipelined over stages as well: while the last k-step of stage s is
@@ -437,8 +454,11 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
             }
             if (c == 0 && sblk > 0) {  // this super-block's header; request the next one
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) hdr[nt] = hdrn[nt];
-                if (next_sb) load_hdr(sblk + 1, hdrn);
+                for (int nt = 0; nt < NT; ++nt) {
+                    hdr[nt] = hdrn[nt];
+                    if constexpr (Q5) hq[nt] = hqn[nt];
+                }
+                if (next_sb) load_hdr(sblk + 1, hdrn, hqn);
             }
             // nibbles of stage st + 2 (the header fetch of a super-block, issued a super-block ahead, has
             // already pulled most of its lines into cache)
@@ -473,9 +493,9 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                 if (ks < 3) {
                     if constexpr (E >= MT) {
 #pragma unroll
-                        for (int e = 0; e < E / MT; ++e) b_eighth(braw[c], dsc, ndm, ks + 1, mt * (E / MT) + e, bfn);
+                        for (int e = 0; e < E / MT; ++e) b_eighth(braw[c], dsc, ndm, ks + 1, mt * (E / MT) + e, bfn, hq, c);
                     } else if (mt % (MT / E) == 0) {
-                        b_eighth(braw[c], dsc, ndm, ks + 1, mt / (MT / E), bfn);
+                        b_eighth(braw[c], dsc, ndm, ks + 1, mt / (MT / E), bfn, hq, c);
                     }
                 } else if (has_next) {
                     if (mt == 0) scales_of(c < 3 ? hdr : hdrn, (c + 1) & 3, dscn, ndmn);
@@ -483,14 +503,16 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                         // the scales come first, so the eighths of row tile 0 move to the last one's slot
                         if (mt > 0) {
 #pragma unroll
-                            for (int e = 0; e < E / MT; ++e) b_eighth(bnext, dscn, ndmn, 0, (mt - 1) * (E / MT) + e, bfn);
+                            for (int e = 0; e < E / MT; ++e)
+                                b_eighth(bnext, dscn, ndmn, 0, (mt - 1) * (E / MT) + e, bfn, c < 3 ? hq : hqn, (c + 1) & 3);
                         }
                         if (mt == MT - 1) {
 #pragma unroll
-                            for (int e = 0; e < E / MT; ++e) b_eighth(bnext, dscn, ndmn, 0, (MT - 1) * (E / MT) + e, bfn);
+                            for (int e = 0; e < E / MT; ++e)
+                                b_eighth(bnext, dscn, ndmn, 0, (MT - 1) * (E / MT) + e, bfn, c < 3 ? hq : hqn, (c + 1) & 3);
                         }
                     } else if (mt % (MT / E) == 1) {
-                        b_eighth(bnext, dscn, ndmn, 0, mt / (MT / E), bfn);
+                        b_eighth(bnext, dscn, ndmn, 0, mt / (MT / E), bfn, c < 3 ? hq : hqn, (c + 1) & 3);
                     }
                 }
                 if constexpr (NT == 2)
@@ -773,15 +795,16 @@ __device__ __forceinline__ bool tile_of(uint32_t b, uint32_t tiles_m, uint32_t t
 }
 
 // Weight rows [0, n_wide) in tiles of 128 (the first grid_wide workgroups), the rest in tiles of 64.
+template <int TYPE>
 __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_kernel(GemmArgs a, uint32_t n_wide, uint32_t grid_wide) {
     const uint32_t tiles_m = (a.m + BM - 1) / BM;
     uint32_t m0, n0;
     if (blockIdx.x < grid_wide) {
         if (!tile_of(blockIdx.x, tiles_m, n_wide / BN_WIDE, BN_WIDE, m0, n0)) return;
-        q4k_gemm_tile<8, 1, 4>(a, m0, n0);
+        q4k_gemm_tile<8, 1, 4, TYPE>(a, m0, n0);
     } else {
         if (!tile_of(blockIdx.x - grid_wide, tiles_m, (a.n - n_wide + BN_NARROW - 1) / BN_NARROW, BN_NARROW, m0, n0)) return;
-        q4k_gemm_tile<4, 1, 2>(a, m0, n_wide + n0);
+        q4k_gemm_tile<4, 1, 2, TYPE>(a, m0, n_wide + n0);
     }
 }
 
@@ -944,7 +967,7 @@ int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, cons
 }
 
 bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {
-    return ((t == HQ_Q4_K || t == HQ_Q6_K) && k % 256 == 0) || (t == HQ_Q8_0 && k % 128 == 0);
+    return ((t == HQ_Q4_K || t == HQ_Q5_K || t == HQ_Q6_K) && k % 256 == 0) || (t == HQ_Q8_0 && k % 128 == 0);
 }
 
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
@@ -973,9 +996,11 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         hipLaunchKernelGGL(q80_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
         return check_launch("q8_0 gemm kernel launch");
     }
-    if (int rc = launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
-    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_gemm_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+    void (*kern)(GemmArgs, uint32_t, uint32_t) = t == HQ_Q5_K ? q4k_gemm_kernel<HQ_Q5_K> : q4k_gemm_kernel<HQ_Q4_K>;
+    if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
+                              : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
+        return rc;
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                            "hipFuncSetAttribute(q4k gemm LDS)"))
         return rc;
     // Tiles of 128 weight rows; tiles of 64 when the wide ones would occupy at most half of the CUs.
@@ -987,7 +1012,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     const uint32_t n_wide = (cols_wide - cols_narrowed) * BN_WIDE;  // < n whenever cols_narrowed > 0
     const uint32_t cols_narrow = n_wide < n ? (n - n_wide + BN_NARROW - 1) / BN_NARROW : 0;
     const uint32_t grid_wide = pad_m * (cols_wide - cols_narrowed), grid_narrow = pad_m * cols_narrow;
-    hipLaunchKernelGGL(q4k_gemm_kernel, dim3(grid_wide + grid_narrow), dim3(64 * WAVES), lds, s, a, n_wide, grid_wide);
+    hipLaunchKernelGGL(kern, dim3(grid_wide + grid_narrow), dim3(64 * WAVES), lds, s, a, n_wide, grid_wide);
     return check_launch("q4k gemm kernel launch");
 }
 
