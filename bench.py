@@ -48,7 +48,7 @@ def parse():
                     help="decode_gemv = BASELINE config 2 (the default and the headline metric); the others are "
                          "configs 3, 4 and 5, each printing its own JSON line")
     ap.add_argument("--tokens", type=int, default=1, help="moe_decode: tokens per step (1 or 8)")
-    ap.add_argument("--wtype", default="q4_k", choices=["q4_k", "q8_0", "q6_k", "q5_k"], help="prefill_gemm: weight type")
+    ap.add_argument("--wtype", default="q4_k", choices=["q4_k", "q8_0", "q6_k", "q5_k", "q4_0"], help="prefill_gemm: weight type")
     ap.add_argument("--weight-sets", type=int, default=4, help="distinct FFN weight sets rotated per step")
     ap.add_argument("--no-graph", action="store_true",
                     help="moe_decode / tq_attention: launch every kernel from the host instead of replaying a HIP "
@@ -234,7 +234,7 @@ def bench_prefill_gemm(a):
 
     dev = torch.device("cuda:0")
     M, K, N = 2048, 4096, 12288
-    t = {"q4_k": HQ_Q4_K, "q8_0": HQ_Q8_0, "q6_k": ops.HQ_Q6_K, "q5_k": ops.HQ_Q5_K}[a.wtype]
+    t = {"q4_k": HQ_Q4_K, "q8_0": HQ_Q8_0, "q6_k": ops.HQ_Q6_K, "q5_k": ops.HQ_Q5_K, "q4_0": ops.HQ_Q4_0}[a.wtype]
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     if t == ops.HQ_Q5_K:
@@ -243,6 +243,13 @@ def bench_prefill_gemm(a):
         q4 = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, HQ_Q4_K).view(-1, 144)
         qh = torch.randint(0, 256, (q4.shape[0], 32), dtype=torch.uint8, device=dev, generator=gen)
         w = torch.cat([q4[:, :16], qh, q4[:, 16:]], dim=1).contiguous().view(-1)
+    elif t == ops.HQ_Q4_0:
+        # no device quantizer for this type either: the f16 scales of Q8_0 blocks of the same weights (x 16, the
+        # ratio of the two formats' ranges) over random nibbles
+        q8 = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, HQ_Q8_0).view(-1, 34)
+        d = (q8[:, :2].contiguous().view(torch.float16).float() * 16.0).to(torch.float16).view(torch.uint8).view(-1, 2)
+        nib = torch.randint(0, 256, (q8.shape[0], 16), dtype=torch.uint8, device=dev, generator=gen)
+        w = torch.cat([d, nib], dim=1).contiguous().view(-1)
     else:
         w = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, t)
     gx = torch.Generator(device=dev)

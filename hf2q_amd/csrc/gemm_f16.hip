@@ -115,11 +115,13 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
                 const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)sb * Q6K_BYTES + 208))) * 4096.f;
                 bound = v <= 3.0e38f ? fmaxf(bound, v) : bound;
             }
-        } else {  // Q8_0: |w| <= |d| * 128
+        } else {  // Q8_0: |w| <= |d| * 128; Q4_0: |w| <= |d| * 8
+            constexpr uint32_t BYTES = TYPE == HQ_Q4_0 ? Q4_0_BYTES : Q8_0_BYTES;
+            constexpr float QMAX = TYPE == HQ_Q4_0 ? 8.f : 128.f;
             const uint32_t nb = k / 32;
-            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nb * Q8_0_BYTES;
+            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nb * BYTES;
             for (uint32_t b = tid & 15u; b < nb; b += 16u) {
-                const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)b * Q8_0_BYTES))) * 128.f;
+                const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)b * BYTES))) * QMAX;
                 bound = v <= 3.0e38f ? fmaxf(bound, v) : bound;
             }
         }
@@ -548,9 +550,16 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 // reads them from 4n + 4, aligned, and shifts by zero.  Since a stage advances every lane by 68
 // bytes, a lane keeps its case.  w = d * q = d * ((q ^ 0x80) - 128) in fp32 (exact), one rounding
 // to f16.
-template <int MT, int WN>
+//
+// TYPE = HQ_Q4_0 (18-byte blocks: f16 d, 16 bytes of nibbles; elements 0..15 are the low nibbles, 16..31 the
+// high ones): the same frame with four words per block instead of eight; k-steps 0 and 1 take the low nibbles of
+// words 0..1 and 2..3, k-steps 2 and 3 the high nibbles of the same words.  A stage advances a lane by 36 bytes,
+// so it keeps its alignment case here too.  w = d * (q - 8).
+template <int MT, int WN, int TYPE = HQ_Q8_0>
 __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
+    constexpr bool Q4 = TYPE == HQ_Q4_0;
+    constexpr uint32_t BYTES = Q4 ? Q4_0_BYTES : Q8_0_BYTES;
     const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t wm = wave / WN, wn = wave % WN;
@@ -561,7 +570,7 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 
     uint32_t gn = n0 + wn * 32 + l32;
     gn = gn < a.n ? gn : a.n - 1u;
-    const uint8_t* blk0 = a.w + (size_t)gn * (a.k / 32) * Q8_0_BYTES + lg * Q8_0_BYTES;  // this lane's block of stage 0
+    const uint8_t* blk0 = a.w + (size_t)gn * (a.k / 32) * BYTES + lg * BYTES;  // this lane's block of stage 0
     const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[a.wd_off + gn];
     const bool early = (reinterpret_cast<uintptr_t>(blk0) & 2u) == 0;  // blocks at 4n: the int8 start two bytes into a word
     const uint32_t shift = early ? 2u : 0u;
@@ -570,12 +579,12 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     struct Raw { uint32_t d; uint4 lo, hi; uint32_t tail; };
     Raw braw[2];
     auto load_b = [&](uint32_t st, int slot) {
-        const size_t off = (size_t)st * (2 * Q8_0_BYTES);
+        const size_t off = (size_t)st * (2 * BYTES);
         braw[slot].d = *reinterpret_cast<const uint16_t*>(blk0 + off);
         braw[slot].lo = ld16_unaligned(win0 + off);  // 4-byte aligned
-        braw[slot].hi = ld16_unaligned(win0 + off + 16);
+        if constexpr (!Q4) braw[slot].hi = ld16_unaligned(win0 + off + 16);
         // late lanes do not use it: they re-read their d, which is always inside the buffer
-        braw[slot].tail = *reinterpret_cast<const uint16_t*>(early ? win0 + off + 32 : blk0 + off);
+        braw[slot].tail = *reinterpret_cast<const uint16_t*>(early ? win0 + off + (Q4 ? 16 : 32) : blk0 + off);
     };
 
     f32x16_t acc[MT][1];
@@ -602,19 +611,32 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
             // activation fetches are issued: the compiler does not know about those, and the wait it
             // puts in front of the first use of these registers would otherwise cover them too.
             Raw cur = braw[c];
-            asm volatile("" : "+v"(cur.d), "+v"(cur.tail), "+v"(cur.lo.x), "+v"(cur.lo.y), "+v"(cur.lo.z), "+v"(cur.lo.w),
-                         "+v"(cur.hi.x), "+v"(cur.hi.y), "+v"(cur.hi.z), "+v"(cur.hi.w));
+            if constexpr (Q4)
+                asm volatile("" : "+v"(cur.d), "+v"(cur.tail), "+v"(cur.lo.x), "+v"(cur.lo.y), "+v"(cur.lo.z), "+v"(cur.lo.w));
+            else
+                asm volatile("" : "+v"(cur.d), "+v"(cur.tail), "+v"(cur.lo.x), "+v"(cur.lo.y), "+v"(cur.lo.z), "+v"(cur.lo.w),
+                             "+v"(cur.hi.x), "+v"(cur.hi.y), "+v"(cur.hi.z), "+v"(cur.hi.w));
             const bool has_next = st + 1 < nstages;  // uniform
             if (has_next) load_b(st + 1, c ^ 1);
-            const float dsc = f16_bits_to_f32(cur.d & 0xffffu) * wdown, ndm = -128.f * dsc;
-            const uint32_t dw[9] = {cur.lo.x, cur.lo.y, cur.lo.z, cur.lo.w, cur.hi.x, cur.hi.y, cur.hi.z, cur.hi.w, cur.tail};
+            const float dsc = f16_bits_to_f32(cur.d & 0xffffu) * wdown, ndm = (Q4 ? -8.f : -128.f) * dsc;
+            uint32_t dw[9];
+            dw[0] = cur.lo.x, dw[1] = cur.lo.y, dw[2] = cur.lo.z, dw[3] = cur.lo.w;
+            if constexpr (Q4) {
+                dw[4] = cur.tail;
+            } else {
+                dw[4] = cur.hi.x, dw[5] = cur.hi.y, dw[6] = cur.hi.z, dw[7] = cur.hi.w, dw[8] = cur.tail;
+            }
             // Eighth e of k-step ks: two weights -> fragment word e.  Word 2*ks + e/2 of the block's int8
             // is formed (and its sign bits flipped) once and kept for its second eighth.
             uint32_t uw[2];
             auto b_eighth = [&](int ks, int e, uint4& bfw) {
-                const int q = e >> 1, part = e & 1, i = 2 * ks + q;
+                const int q = e >> 1, part = e & 1, i = 2 * (Q4 ? ks & 1 : ks) + q;
                 if (part == 0) {
-                    uint32_t u = __builtin_amdgcn_alignbyte(dw[i + 1], dw[i], shift) ^ 0x80808080u;
+                    uint32_t u = __builtin_amdgcn_alignbyte(dw[i + 1], dw[i], shift);
+                    if constexpr (Q4)
+                        u = (ks >= 2 ? u >> 4 : u) & 0x0f0f0f0fu;
+                    else
+                        u ^= 0x80808080u;
                     // opaque, so that the conversions stay v_cvt_f32_ubyte0..3 of this one register
                     asm volatile("" : "+v"(u));
                     uw[q] = u;
@@ -815,11 +837,12 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q6k_gemm_kernel(GemmArgs a) {
     q6k_gemm_tile<8, 4>(a, m0, n0);
 }
 
+template <int TYPE>
 __global__ __launch_bounds__(64 * WAVES, 2) void q80_gemm_kernel(GemmArgs a) {
     const uint32_t tiles_m = (a.m + BM - 1) / BM;
     uint32_t m0, n0;
     if (!tile_of(blockIdx.x, tiles_m, (a.n + BN_WIDE - 1) / BN_WIDE, BN_WIDE, m0, n0)) return;
-    q80_gemm_tile<8, 4>(a, m0, n0);
+    q80_gemm_tile<8, 4, TYPE>(a, m0, n0);
 }
 
 // ---- grouped (expert) form -------------------------------------------------------------------
@@ -903,7 +926,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
     else if constexpr (TYPE == HQ_Q6_K)
         q6k_gemm_tile<8, 4>(a, tt.y, n0);
     else
-        q80_gemm_tile<8, 4>(a, tt.y, n0);
+        q80_gemm_tile<8, 4, HQ_Q8_0>(a, tt.y, n0);
 }
 
 }  // namespace
@@ -967,7 +990,7 @@ int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, cons
 }
 
 bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {
-    return ((t == HQ_Q4_K || t == HQ_Q5_K || t == HQ_Q6_K) && k % 256 == 0) || (t == HQ_Q8_0 && k % 128 == 0);
+    return ((t == HQ_Q4_K || t == HQ_Q5_K || t == HQ_Q6_K) && k % 256 == 0) || ((t == HQ_Q8_0 || t == HQ_Q4_0) && k % 128 == 0);
 }
 
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
@@ -987,13 +1010,15 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         hipLaunchKernelGGL(q6k_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
         return check_launch("q6_k gemm kernel launch");
     }
-    if (t == HQ_Q8_0) {
-        if (int rc = launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q80_gemm_kernel),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+    if (t == HQ_Q8_0 || t == HQ_Q4_0) {
+        void (*kern)(GemmArgs) = t == HQ_Q4_0 ? q80_gemm_kernel<HQ_Q4_0> : q80_gemm_kernel<HQ_Q8_0>;
+        if (int rc = t == HQ_Q4_0 ? launch_prep<HQ_Q4_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
+                                  : launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
+            return rc;
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                                "hipFuncSetAttribute(q8_0 gemm LDS)"))
             return rc;
-        hipLaunchKernelGGL(q80_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
+        hipLaunchKernelGGL(kern, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
         return check_launch("q8_0 gemm kernel launch");
     }
     void (*kern)(GemmArgs, uint32_t, uint32_t) = t == HQ_Q5_K ? q4k_gemm_kernel<HQ_Q5_K> : q4k_gemm_kernel<HQ_Q4_K>;

@@ -5,16 +5,16 @@ import torch
 
 from _util import acts, assert_matmul_close, assert_matmul_close_f16_tile, weights
 from hf2q_amd import ops
-from hf2q_amd.ops import HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, GgmlQuantizedMatmulParams
+from hf2q_amd.ops import HQ_Q4_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, GgmlQuantizedMatmulParams
 
 pytestmark = pytest.mark.gpu
 
 def _f16_tile(t, k):
-    return (t in (HQ_Q4_K, HQ_Q5_K, HQ_Q6_K) and k % 256 == 0) or (t == HQ_Q8_0 and k % 128 == 0)
+    return (t in (HQ_Q4_K, HQ_Q5_K, HQ_Q6_K) and k % 256 == 0) or (t in (HQ_Q8_0, HQ_Q4_0) and k % 128 == 0)
 
 
 def _check(t, k):
-    """Q4_K / Q5_K / Q6_K (k % 256 == 0) and Q8_0 with k % 128 == 0 take the f16 tile kernels; everything else
+    """Q4_K / Q5_K / Q6_K (k % 256 == 0) and Q8_0 / Q4_0 with k % 128 == 0 take the f16 tile kernels; everything else
     keeps every product exact."""
     return assert_matmul_close_f16_tile if _f16_tile(t, k) else assert_matmul_close
 
@@ -40,7 +40,7 @@ def _run(oracle, dev, t, xdt, m, n, k, blocks=None, seed=0):
     return y.cpu().numpy(), ref
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,n,k", SHAPES)
 def test_gemm_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
@@ -50,7 +50,7 @@ def test_gemm_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
     _check(t, k)(y, ref, f"gemm t={t} {xdt} {m}x{n}x{k}")
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
 def test_gemm_adversarial_blocks(oracle, dev, t):
     """Every scale / min / nibble bit pattern (raw random bytes with finite f16 fields)."""
     m, n, k = 40, 128, 512
@@ -63,7 +63,7 @@ def test_gemm_adversarial_blocks(oracle, dev, t):
         _check(t, k)(y, ref, f"gemm adversarial t={t} {xdt}")
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
 def test_gemm_rows_equal_gemv_rows(oracle, dev, t):
     """Row i of the m>8 result agrees with the m=1 GEMV of activation row i; the tile kernels round
     their weights to f16, so the agreement is to 1e-3 of the row's largest output."""
@@ -115,7 +115,7 @@ def test_q4k_tile_gemm_workspace_variant(oracle, dev):
         ops.quantized_matmul_ggml(x, wd, y1, p, workspace=ws[: need - 256])
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 def test_tile_gemm_scale_equivariance(oracle, dev, xdt, t):
     """Activation rows and weight rows are rescaled by powers of two inside the kernel (f16 has a narrow
@@ -142,10 +142,13 @@ def test_tile_gemm_scale_equivariance(oracle, dev, xdt, t):
                                      f"tile gemm t={t} sigma={sigma} {xdt}")
 
 
-@pytest.mark.parametrize("t", [ops.HQ_Q4_0])
-def test_types_without_a_tile_kernel_run_as_gemv_chunks(oracle, dev, t):
-    """Q4_0 at m > 8: the GEMV form, eight activation rows per launch (exact f32 accumulation of bf16 x weight)."""
-    m, n, k = 21, 96, 1024
+@pytest.mark.parametrize("t", [HQ_Q4_0, HQ_Q5_K])
+def test_shapes_without_a_tile_kernel_run_as_gemv_chunks(oracle, dev, t):
+    """m > 8 with a k no tile kernel takes (Q4_0: k % 128 != 0; Q5_K: k % 256 != 0 cannot occur, so it is not
+    run): the GEMV form, eight activation rows per launch (exact f32 accumulation of bf16 x weight)."""
+    if t == HQ_Q5_K:
+        pytest.skip("every valid Q5_K k is a multiple of 256 and has a tile kernel")
+    m, n, k = 21, 96, 1056
     blocks = oracle.quantize(weights(t, n, k), k, t, threads=8)
     x = acts(5, m, k)
     xb = oracle.f32_to_bf16_bits(x)
@@ -157,7 +160,7 @@ def test_types_without_a_tile_kernel_run_as_gemv_chunks(oracle, dev, t):
     assert_matmul_close(y.cpu().numpy(), ref, f"m=21 t={t}")
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0])
 @pytest.mark.parametrize("m,heads,hd,n", [(64, 4, 256, 96), (300, 8, 128, 160), (5, 2, 256, 64)])
 def test_perm021_matches_oracle_and_the_plain_product(oracle, dev, t, m, heads, hd, n):
     """quantized_matmul_mm_tensor_perm021 (forward_prefill_batched.rs:2219-2257): activations stored
