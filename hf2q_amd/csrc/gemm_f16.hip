@@ -921,12 +921,12 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
     a.w += (size_t)tt.x * expert_stride;
     a.wd_off = tt.x * a.n;
     a.m = tt.z;  // rows past the expert's run repeat its last row and are not stored
-    if constexpr (TYPE == HQ_Q4_K)
-        q4k_gemm_tile<8, 1, 4>(a, tt.y, n0);
+    if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
+        q4k_gemm_tile<8, 1, 4, TYPE>(a, tt.y, n0);
     else if constexpr (TYPE == HQ_Q6_K)
         q6k_gemm_tile<8, 4>(a, tt.y, n0);
     else
-        q80_gemm_tile<8, 4, HQ_Q8_0>(a, tt.y, n0);
+        q80_gemm_tile<8, 4, TYPE>(a, tt.y, n0);
 }
 
 }  // namespace
@@ -935,8 +935,11 @@ size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) { retur
 
 bool gemm_f16_grouped_supported(hq_ggml_type t, uint32_t n, uint32_t k, uint32_t n_experts, uint64_t expert_stride, uint64_t pairs) {
     if (!gemm_f16_tile_supported(t, k) || n_experts > BUCKET_MAX_EXPERTS || pairs > 0x7fffffffull / 4) return false;
-    const uint64_t row_bytes = t == HQ_Q4_K ? (uint64_t)(k / 256) * Q4K_BYTES : t == HQ_Q6_K ? (uint64_t)(k / 256) * Q6K_BYTES
-                                                                                              : (uint64_t)(k / 32) * Q8_0_BYTES;
+    const uint64_t row_bytes = t == HQ_Q4_K   ? (uint64_t)(k / 256) * Q4K_BYTES
+                               : t == HQ_Q5_K ? (uint64_t)(k / 256) * Q5K_BYTES
+                               : t == HQ_Q6_K ? (uint64_t)(k / 256) * Q6K_BYTES
+                               : t == HQ_Q4_0 ? (uint64_t)(k / 32) * Q4_0_BYTES
+                                              : (uint64_t)(k / 32) * Q8_0_BYTES;
     // the pre-pass walks the stack as one matrix of n_experts * n rows
     return expert_stride == (uint64_t)n * row_bytes && (uint64_t)n_experts * n <= 0x7fffffffull;
 }
@@ -984,9 +987,14 @@ int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, cons
                             uint64_t expert_stride, hq_ggml_type t) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const uint8_t* wb = static_cast<const uint8_t*>(w_stack);
-    if (t == HQ_Q4_K) return launch_grouped_t<HQ_Q4_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
-    if (t == HQ_Q6_K) return launch_grouped_t<HQ_Q6_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
-    return launch_grouped_t<HQ_Q8_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+    switch (t) {
+        case HQ_Q4_K: return launch_grouped_t<HQ_Q4_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+        case HQ_Q5_K: return launch_grouped_t<HQ_Q5_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+        case HQ_Q6_K: return launch_grouped_t<HQ_Q6_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+        case HQ_Q8_0: return launch_grouped_t<HQ_Q8_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+        case HQ_Q4_0: return launch_grouped_t<HQ_Q4_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+    }
+    return fail(HQ_ERR_UNSUPPORTED, "grouped gemm: ggml type %d", (int)t);
 }
 
 bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {

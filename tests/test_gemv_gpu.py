@@ -261,12 +261,12 @@ def _grouped_setup(oracle, dev, t, E, n, k, T, K, xdt, seed=0, skew=False):
     return stack, ids, xv, xd, p
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("E,n,k,T,K", GROUPED_CASES)
 def test_mul_mat_id_grouped_matches_oracle(oracle, dev, t, xdt, E, n, k, T, K):
-    if t == HQ_Q8_0 and k % 128:
-        pytest.skip("Q8_0 tile kernel needs k % 128 == 0")
+    if t in (HQ_Q8_0, HQ_Q4_0) and k % 128:
+        pytest.skip("Q8_0 / Q4_0 tile kernel needs k % 128 == 0")
     stack, ids, xv, xd, p = _grouped_setup(oracle, dev, t, E, n, k, T, K, xdt)
     need = ops.quantized_matmul_id_workspace_bytes(p)
     assert need > 0, "this shape must take the grouped route"
