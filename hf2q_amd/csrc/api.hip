@@ -241,7 +241,7 @@ bool grouped_route(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, ui
 
 size_t hq_qmatmul_id_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
                                           uint64_t expert_stride, hq_ggml_type t) {
-    if (t != HQ_Q4_K && t != HQ_Q6_K && t != HQ_Q8_0) return 0;
+    if (hq_block_elems(t) == 0) return 0;  // not a type of this library
     if (n == 0 || k == 0 || k % hq_block_elems(t)) return 0;
     return grouped_route(n_tokens, top_k, n, k, n_experts, expert_stride, t)
                ? gemm_f16_grouped_workspace_bytes(n_tokens * top_k, n_experts, n, k) : 0;
