@@ -237,21 +237,7 @@ def bench_prefill_gemm(a):
     t = {"q4_k": HQ_Q4_K, "q8_0": HQ_Q8_0, "q6_k": ops.HQ_Q6_K, "q5_k": ops.HQ_Q5_K, "q4_0": ops.HQ_Q4_0}[a.wtype]
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
-    if t == ops.HQ_Q5_K:
-        # no device quantizer for this type: Q4_K blocks of the same weights with 32 random qh bytes spliced in
-        # after the 16-byte header (d, dmin, scales are laid out alike)
-        q4 = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, HQ_Q4_K).view(-1, 144)
-        qh = torch.randint(0, 256, (q4.shape[0], 32), dtype=torch.uint8, device=dev, generator=gen)
-        w = torch.cat([q4[:, :16], qh, q4[:, 16:]], dim=1).contiguous().view(-1)
-    elif t == ops.HQ_Q4_0:
-        # no device quantizer for this type either: the f16 scales of Q8_0 blocks of the same weights (x 16, the
-        # ratio of the two formats' ranges) over random nibbles
-        q8 = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, HQ_Q8_0).view(-1, 34)
-        d = (q8[:, :2].contiguous().view(torch.float16).float() * 16.0).to(torch.float16).view(torch.uint8).view(-1, 2)
-        nib = torch.randint(0, 256, (q8.shape[0], 16), dtype=torch.uint8, device=dev, generator=gen)
-        w = torch.cat([d, nib], dim=1).contiguous().view(-1)
-    else:
-        w = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, t)
+    w = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, t)
     gx = torch.Generator(device=dev)
     gx.manual_seed(5678)
     x = torch.randn(M, K, generator=gx, device=dev).to(torch.bfloat16)

@@ -69,12 +69,15 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restr
     }
 }
 
-// ------------------------------------------------------------------ Q4_K
-// common.rs:174-286 make_qkx2_quants with n = 32, nmax = 15, rmin = -1,
-// rdelta = 0.1, nstep = 20, use_mad = false (the arguments of q4_k.rs:120-132).
+// ------------------------------------------------------------------ Q4_K, Q5_K
+// common.rs:174-286 make_qkx2_quants with n = 32, use_mad = false and
+// nmax = 15, rmin = -1, rdelta = 0.1, nstep = 20 (Q4_K, the arguments of q4_k.rs:120-132) or
+// nmax = 31, rmin = -0.5, rdelta = 0.1, nstep = 15 (Q5_K, q5_k.rs).
 // L comes back packed four codes per word.
+template <int nmax>
 __device__ float qkx2_search_32(const float (&x)[32], const float (&wt)[32], uint32_t (&Lp)[8], float& the_min) {
-    constexpr int nmax = 15;
+    constexpr int nstep = nmax == 15 ? 20 : 15;
+    constexpr float rmin = nmax == 15 ? -1.f : -0.5f;
     float mn = x[0], mx = x[0];
     float sum_w = wt[0];
     float sum_x = sum_w * x[0];
@@ -104,8 +107,8 @@ __device__ float qkx2_search_32(const float (&x)[32], const float (&wt)[32], uin
         diff = diff * diff;
         best_error = fmaf(wt[i], diff, best_error);
     }
-    for (int is = 0; is <= 20; ++is) {
-        iscale = (-1.f + 0.1f * (float)is + (float)nmax) / (mx - mn);
+    for (int is = 0; is <= nstep; ++is) {
+        iscale = (rmin + 0.1f * (float)is + (float)nmax) / (mx - mn);
         float sum_l = 0.f, sum_l2 = 0.f, sum_xl = 0.f;
         uint32_t La[8];
 #pragma unroll
@@ -149,9 +152,13 @@ __device__ float qkx2_search_32(const float (&x)[32], const float (&wt)[32], uin
     return scale;
 }
 
-// q4_k.rs:89-217.  256 threads = 32 super-blocks x 8 sub-block threads.
+// q4_k.rs:89-217 (Q5 = false) and its five-bit twin q5_k.rs (Q5 = true: codes 0..31, the fifth bit of every code
+// in qh, bit 2c for sub-block 2c and 2c + 1 for sub-block 2c + 1).  256 threads = 32 super-blocks x 8 sub-block
+// threads.
+template <bool Q5>
 __global__ __launch_bounds__(256) void quantize_q4_k_kernel(const float* __restrict__ src, uint8_t* __restrict__ out,
                                                             uint64_t n_blocks) {
+    constexpr int NMAX = Q5 ? 31 : 15;
     __shared__ float s_scale[256], s_min[256];
     __shared__ uint32_t s_code[256];   // ls | lm << 8 per sub-block
     __shared__ uint32_t s_L[256 * 8];  // packed codes of every sub-block (32 bytes each)
@@ -180,7 +187,7 @@ __global__ __launch_bounds__(256) void quantize_q4_k_kernel(const float* __restr
 
     uint32_t Lp[8];
     float the_min;
-    const float scale = qkx2_search_32(x, wt, Lp, the_min);
+    const float scale = qkx2_search_32<NMAX>(x, wt, Lp, the_min);
     s_scale[tid] = scale;
     s_min[tid] = the_min;
     __syncthreads();
@@ -211,7 +218,7 @@ __global__ __launch_bounds__(256) void quantize_q4_k_kernel(const float* __restr
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
             int l = nearest_int((x[i] + dm) / d);
-            l = max(0, min(15, l));
+            l = max(0, min(NMAX, l));
             Lp[i >> 2] |= (uint32_t)l << (8 * (i & 3));
         }
     }
@@ -223,7 +230,7 @@ __global__ __launch_bounds__(256) void quantize_q4_k_kernel(const float* __restr
     // Pack: thread j writes the header (j == 0) and 16 bytes of qs.  Chunk c = j/2,
     // half h = j%2: bytes 16h..16h+15 of the chunk combine code l of sub-block 2c
     // (low nibble) with code l of sub-block 2c+1 (high nibble), l = 16h + i.
-    uint8_t* o = out + blk * Q4K_BYTES;
+    uint8_t* o = out + blk * (Q5 ? Q5K_BYTES : Q4K_BYTES);
     if (j == 0) {
         uint32_t sc[8], mi[8];
 #pragma unroll
@@ -248,12 +255,70 @@ __global__ __launch_bounds__(256) void quantize_q4_k_kernel(const float* __restr
     const uint32_t c = j >> 1, h = j & 1u;
     const uint32_t* lo = &s_L[(lb * 8 + 2 * c) * 8 + 4 * h];
     const uint32_t* hi = &s_L[(lb * 8 + 2 * c + 1) * 8 + 4 * h];
+    constexpr uint32_t N4 = 0x0f0f0f0fu;  // (a no-op for Q4_K, whose codes have four bits)
     uint4 qs;
-    qs.x = lo[0] | (hi[0] << 4);
-    qs.y = lo[1] | (hi[1] << 4);
-    qs.z = lo[2] | (hi[2] << 4);
-    qs.w = lo[3] | (hi[3] << 4);
-    *reinterpret_cast<uint4*>(o + 16 + 32 * c + 16 * h) = qs;
+    qs.x = (lo[0] & N4) | ((hi[0] & N4) << 4);
+    qs.y = (lo[1] & N4) | ((hi[1] & N4) << 4);
+    qs.z = (lo[2] & N4) | ((hi[2] & N4) << 4);
+    qs.w = (lo[3] & N4) | ((hi[3] & N4) << 4);
+    *reinterpret_cast<uint4*>(o + (Q5 ? 48 : 16) + 32 * c + 16 * h) = qs;
+    if constexpr (Q5) {
+        // threads 0 and 1 of the super-block: qh bytes 16 j .. 16 j + 15, bit sb = the fifth bit of sub-block sb's code
+        if (j < 2) {
+            uint32_t qh[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) qh[w] |= ((s_L[(lb * 8 + sb) * 8 + 4 * j + w] >> 4) & 0x01010101u) << sb;
+            *reinterpret_cast<uint4*>(o + 16 + 16 * j) = make_uint4(qh[0], qh[1], qh[2], qh[3]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ Q4_0
+// q4_0.rs quantize_row (no imatrix): d = (the element of largest magnitude) / -8, codes trunc(x / d + 8.5) capped at
+// 15; elements 0..15 in the low nibbles, 16..31 in the high ones.  One thread per block.
+__global__ __launch_bounds__(256) void quantize_q4_0_kernel(const float* __restrict__ src, uint8_t* __restrict__ out,
+                                                            uint64_t n_blocks) {
+    const uint64_t b = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= n_blocks) return;
+    float x[32];
+    const float4* s4 = reinterpret_cast<const float4*>(src + b * 32);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float4 t = s4[i];
+        x[4 * i] = t.x;
+        x[4 * i + 1] = t.y;
+        x[4 * i + 2] = t.z;
+        x[4 * i + 3] = t.w;
+    }
+    float amax = 0.f, mx = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const float a = fabsf(x[i]);
+        if (amax < a) {
+            amax = a;
+            mx = x[i];
+        }
+    }
+    float d = mx / -8.f;
+    // Opaque: otherwise the division and the conversion below become one v_fma_mixlo_f16 (mx * -0.125 + 0), and
+    // the + 0 turns the -0.0 of an all-zero block into +0.0 (the reference stores 0x8000 there).
+    asm volatile("" : "+v"(d));
+    const float id = d != 0.f ? 1.f / d : 0.f;
+    uint8_t* o = out + b * Q4_0_BYTES;
+    *reinterpret_cast<uint16_t*>(o) = (uint16_t)f32_to_f16_bits(d);
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            // the reference casts to i8 (truncation towards zero; the values lie in [0.5, 16.5]) and caps at 15
+            const int a = (int)(x[i + e] * id + 8.5f), c = (int)(x[16 + i + e] * id + 8.5f);
+            v |= (uint32_t)((a < 15 ? a : 15) | ((c < 15 ? c : 15) << 4)) << (8 * e);
+        }
+        *reinterpret_cast<uint16_t*>(o + 2 + i) = (uint16_t)v;
+    }
 }
 
 // ------------------------------------------------------------------ Q6_K
@@ -418,7 +483,15 @@ int launch_quantize(hipStream_t s, const float* src, uint64_t n_elems, uint64_t 
     } else if (t == HQ_Q4_K) {
         const uint64_t nb = n_elems / 256;
         if ((nb + 31) / 32 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
-        hipLaunchKernelGGL(quantize_q4_k_kernel, dim3((unsigned)((nb + 31) / 32)), dim3(256), 0, s, src, o, nb);
+        hipLaunchKernelGGL(quantize_q4_k_kernel<false>, dim3((unsigned)((nb + 31) / 32)), dim3(256), 0, s, src, o, nb);
+    } else if (t == HQ_Q5_K) {
+        const uint64_t nb = n_elems / 256;
+        if ((nb + 31) / 32 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
+        hipLaunchKernelGGL(quantize_q4_k_kernel<true>, dim3((unsigned)((nb + 31) / 32)), dim3(256), 0, s, src, o, nb);
+    } else if (t == HQ_Q4_0) {
+        const uint64_t nb = n_elems / 32;
+        if ((nb + 255) / 256 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
+        hipLaunchKernelGGL(quantize_q4_0_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, src, o, nb);
     } else if (t == HQ_Q6_K) {
         const uint64_t nb = n_elems / 256;
         if ((nb + 15) / 16 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");

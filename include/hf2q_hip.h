@@ -41,9 +41,8 @@ typedef enum {
     HQ_ERR_HIP = 3               /* a HIP runtime call failed */
 } hq_status;
 
-/* Numeric ids are GGML's (src/quantize/ggml_quants/ggml_type.rs:18-53).  Q4_K, Q6_K and Q8_0 are
- * served by every entry point; Q5_K (block layout q5_k.rs:9-18) and Q4_0 (q4_0.rs:6-12) by the
- * dequantiser and the matmul entry points (GEMV form at any m), not by hq_quantize_ggml.  Q4_K and
+/* Numeric ids are GGML's (src/quantize/ggml_quants/ggml_type.rs:18-53).  Every entry point that takes
+ * a type serves all five (block layouts: q4_0.rs:6-12, q8_0.rs, q4_k.rs, q5_k.rs:9-18, q6_k.rs).  Q4_K and
  * Q5_K blocks must be 16-byte aligned, the others 2-byte. */
 typedef enum { HQ_Q4_0 = 2, HQ_Q8_0 = 8, HQ_Q4_K = 12, HQ_Q5_K = 13, HQ_Q6_K = 14 } hq_ggml_type;
 
@@ -74,7 +73,7 @@ HQ_API int hq_dequant_ggml(void* stream, const void* w_blocks, void* out, hq_act
 /* Quantise f32 rows to packed GGML blocks on the device, byte-identical to
  * hf2q's CPU quantizers without an importance matrix
  * (src/quantize/ggml_quants/quantizer.rs:51-102 -> q4_k.rs:50-217,
- * q6_k.rs:40-221, q8_0.rs:31-72; load-time use:
+ * q6_k.rs:40-221, q8_0.rs:31-72, q5_k.rs, q4_0.rs; load-time use:
  * src/inference/models/qwen35/in_memory_loader.rs:70-139).
  * `n_elems` must be a multiple of `n_per_row`, `n_per_row` of the block size. */
 HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row,

@@ -175,19 +175,21 @@ def test_mul_mat_id_invariants(oracle, dev):
 
 # ---- device-side quantizer ------------------------------------------------------------
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 def test_quantizer_matches_reference_golden_bytes(oracle, dev, t):
-    """The reference's own byte-equality fixtures (q4_k.rs:386-393, q6_k.rs:272-279, q8_0.rs:106-113)."""
+    """The reference's own byte-equality fixtures (q4_k.rs:386-393, q6_k.rs:272-279, q8_0.rs:106-113, and the
+    q5_k / q4_0 files beside them)."""
     import os
     from _util import GOLDEN
-    name, npr = {HQ_Q4_K: ("q4_k_512", 512), HQ_Q6_K: ("q6_k_512", 512), HQ_Q8_0: ("q8_0_64", 64)}[t]
+    name, npr = {HQ_Q4_K: ("q4_k_512", 512), HQ_Q6_K: ("q6_k_512", 512), HQ_Q8_0: ("q8_0_64", 64),
+                 HQ_Q5_K: ("q5_k_512", 512), HQ_Q4_0: ("q4_0_64", 64)}[t]
     x = np.fromfile(os.path.join(GOLDEN, "ggml_quants", f"{name}_noim_input.bin"), dtype=np.float32)
     want = np.fromfile(os.path.join(GOLDEN, "ggml_quants", f"{name}_noim_expected.bin"), dtype=np.uint8)
     got = ops.quantize_ggml(torch.from_numpy(x).to(dev), npr, t).cpu().numpy()
     assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("t", ALL_TYPES)
 def test_quantizer_byte_equal_to_oracle(oracle, dev, t):
     rng = np.random.default_rng(40 + t)
     parts = [
