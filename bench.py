@@ -35,6 +35,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 # 2.0), WRITE_SIZE all of them (1.0).  The runs and their figures are in profiles/*_pmc_traffic.md.
 PMC_TRAFFIC_BYTES = {
     "gemv_head_q6_k_151936x4096": int(249387.5 * 2.0 * 1024 + 755.3 * 1.0 * 1024),
+    # activation pre-pass + tile GEMM, Q4_K, 2048 x 12288 x 4096 (the GEMM re-fetches the weights once per 256-token tile)
+    "prefill_gemm_q4_k_2048x12288x4096": int((23122.3 + 132689.9) * 2.0 * 1024 + (16496.3 + 98314.0) * 1.0 * 1024),
+    # split (with the q rotation) + merge (with the output rotation), 32K context, 2 kv heads, head_dim 256
+    "tq_attention_32k_fused_chain": int((16834.8 + 1072.5) * 2.0 * 1024 + (2112.0 + 16.0) * 1.0 * 1024),
 }
 
 
@@ -270,7 +274,8 @@ def bench_prefill_gemm(a):
         "roofline": {"bound": "mfma", "kernel": (f"activation pre-pass + f16 MFMA gemm {a.wtype}" if need else
                                                  f"bf16 MFMA gemm {a.wtype}"), "achieved": round(tf, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": None, "us_per_launch": round(us, 2), "flop_per_launch": flops}})
+                     "traffic": PMC_TRAFFIC_BYTES["prefill_gemm_q4_k_2048x12288x4096"] if a.wtype == "q4_k" else None,
+                     "us_per_launch": round(us, 2), "flop_per_launch": flops}})
 
 
 def bench_tq_attention(a):
@@ -328,7 +333,8 @@ def bench_tq_attention(a):
                                          "GB/s": round(nbytes / us_sep / 1e3, 1)}},
         "roofline": {"bound": "hbm", "kernel": "tq attention split (+ q rotation) + merge (+ output rotation)",
                      "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": None, "us_per_launch": round(us, 3), "bytes_per_launch": nbytes}})
+                     "traffic": PMC_TRAFFIC_BYTES["tq_attention_32k_fused_chain"], "us_per_launch": round(us, 3),
+                     "bytes_per_launch": nbytes}})
 
 
 def main():
