@@ -1,6 +1,6 @@
 // Dequant-fused product for 3..8 activation rows (small-batch decode) on the matrix cores:
 // y[m, n] = sum_k x[m, k] * W[n, k] with every weight fetched once for all rows, where the GEMV
-// kernel would fetch it once per row.  Q4_K and Q6_K weights, k a multiple of 1024.
+// kernel would fetch it once per row.  Q4_K, Q5_K and Q6_K weights, k a multiple of 1024.
 //
 // Bandwidth-bound like the GEMV (0.5625 bytes per weight); the arithmetic that depends on the row
 // count moves to v_mfma_f32_16x16x32_bf16, what is left on the VALU (nibbles -> bf16, scales) does
@@ -193,8 +193,13 @@ __device__ __forceinline__ void store_rows(const RowsArgs& a, uint8_t* smem, con
 // waves a quarter of k each (many workgroups for small matrices).  4: it owns 64 rows, each wave 16 of them over
 // all of k, so a staged chunk of activations and its barrier serve four times the weights.  2: 32 rows, two waves
 // per 16 rows (half the registers of 4 for the fetches in flight).
-template <bool X_BF16, int NSB>
+//
+// Q5 = true: Q5_K weights (176-byte super-blocks: the same header, 32 bytes of fifth bits, then the nibbles).  A
+// lane also fetches the eight qh bytes that sit over its nibble bytes and ORs bit 2c (2c + 1) of each into the
+// values of sub-block 2c (2c + 1): 128 + q with q < 32 is still exact in bf16.
+template <bool X_BF16, int NSB, bool Q5 = false>
 __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
+    constexpr uint32_t BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES, QS = Q5 ? 48u : 16u;  // super-block size, offset of the nibbles
     extern __shared__ uint4 smem4[];
     uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -203,12 +208,13 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
     const uint32_t row0 = (blockIdx.x * (uint32_t)NSB + wave / SHARE) * 16u, sb0 = (wave % SHARE) * NSB;
     const uint32_t r = row0 + j < a.n ? row0 + j : a.n - 1u;  // rows past the end repeat the last one, not stored
     const uint32_t nsb = a.k / 256u, nch = a.k / KC;
-    const uint8_t* wrow = a.w + (size_t)r * nsb * Q4K_BYTES + 16u + 8u * g;  // this lane's eight bytes of chunk 0
+    const uint8_t* wrow = a.w + (size_t)r * nsb * BYTES + QS + 8u * g;  // this lane's eight bytes of chunk 0
     const uint32_t arow = (X_BF16 ? (j & 7u) : j) * XROW + 16u * g;          // this lane's row and k-group in a staged buffer
 
     struct WBlock {
         uint4 hdr;
         uint2 q[4];
+        uint2 qh;  // Q5_K only
     };
     struct WSet {
         WBlock b[NSB];
@@ -216,8 +222,9 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
     auto load_w = [&](uint32_t ch, WSet& set) {
 #pragma unroll
         for (int s = 0; s < NSB; ++s) {
-            const uint8_t* p = wrow + (size_t)(ch * 4u + sb0 + s) * Q4K_BYTES;
-            set.b[s].hdr = *reinterpret_cast<const uint4*>(p - 16u - 8u * g);
+            const uint8_t* p = wrow + (size_t)(ch * 4u + sb0 + s) * BYTES;
+            set.b[s].hdr = *reinterpret_cast<const uint4*>(p - QS - 8u * g);
+            if constexpr (Q5) set.b[s].qh = *reinterpret_cast<const uint2*>(p - 32u);  // qh bytes 8g..8g+7
 #pragma unroll
             for (int c = 0; c < 4; ++c) set.b[s].q[c] = *reinterpret_cast<const uint2*>(p + 32 * c);
         }
@@ -259,10 +266,18 @@ __global__ __launch_bounds__(256) void q4k_rows_kernel(RowsArgs a) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t w0 = wb.q[c].x, w1 = wb.q[c].y;
-            const uint4 blo = make_uint4(and_or(w0, m4, magic), and_or(w0 >> 8, m4, magic), and_or(w1, m4, magic),
-                                         and_or(w1 >> 8, m4, magic));
-            const uint4 bhi = make_uint4(and_or(w0 >> 4, m4, magic), and_or(w0 >> 12, m4, magic), and_or(w1 >> 4, m4, magic),
-                                         and_or(w1 >> 12, m4, magic));
+            uint4 blo = make_uint4(and_or(w0, m4, magic), and_or(w0 >> 8, m4, magic), and_or(w1, m4, magic),
+                                   and_or(w1 >> 8, m4, magic));
+            uint4 bhi = make_uint4(and_or(w0 >> 4, m4, magic), and_or(w0 >> 12, m4, magic), and_or(w1 >> 4, m4, magic),
+                                   and_or(w1 >> 12, m4, magic));
+            if constexpr (Q5) {
+                // fifth bits of bytes (0, 2) / (1, 3) of a word, for sub-block 2c (low nibbles) and 2c + 1 (high)
+                constexpr uint32_t M1 = 0x00010001u;
+                const uint32_t h0 = wb.qh.x >> (2 * c), h1 = wb.qh.y >> (2 * c);
+                blo.x |= (h0 & M1) << 4, blo.y |= ((h0 >> 8) & M1) << 4, blo.z |= (h1 & M1) << 4, blo.w |= ((h1 >> 8) & M1) << 4;
+                bhi.x |= ((h0 >> 1) & M1) << 4, bhi.y |= ((h0 >> 9) & M1) << 4, bhi.z |= ((h1 >> 1) & M1) << 4,
+                    bhi.w |= ((h1 >> 9) & M1) << 4;
+            }
             const uint4 alo = *reinterpret_cast<const uint4*>(xb + 128 * c);       // sub-block 2c: 64 bytes per sub-block
             const uint4 ahi = *reinterpret_cast<const uint4*>(xb + 128 * c + 64);  // sub-block 2c + 1
             const f32x4_t z = {0.f, 0.f, 0.f, 0.f};
@@ -413,12 +428,12 @@ __global__ __launch_bounds__(256) void q6k_rows_kernel(RowsArgs a) {
 
 }  // namespace
 
-// Q4_K from three rows on, Q6_K from four: below that, one GEMV per row is as fast.  Measured, bf16 activations:
+// Q4_K and Q5_K from three rows on, Q6_K from four: below that, one GEMV per row is as fast.  Measured, bf16 activations:
 // Q4_K 12288 x 4096: 10 / 15 / 19 / 24 us for 1..4 GEMVs against 15..16 us here whatever the row count; Q6_K
 // 151936 x 4096: 96 us per GEMV row against 310 us here.
 bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k) {
-    const uint32_t from = t == HQ_Q4_K ? 3u : 4u;
-    return (t == HQ_Q4_K || t == HQ_Q6_K) && m >= from && m <= 8 && k % KC == 0;
+    const uint32_t from = t == HQ_Q6_K ? 4u : 3u;
+    return (t == HQ_Q4_K || t == HQ_Q5_K || t == HQ_Q6_K) && m >= from && m <= 8 && k % KC == 0;
 }
 
 int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
@@ -429,11 +444,14 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
     // more rows per workgroup once that still gives every CU three workgroups of the first round; Q6_K stops at
     // two super-blocks per wave (at four, the fetches in flight leave one wave per SIMD) except with f32
     // activations, whose LDS footprint limits the CU to two workgroups anyway
-    const uint32_t nsb = n < WIDE_MIN_ROWS ? 1u : t == HQ_Q4_K || !bf ? 4u : 2u;
+    const uint32_t nsb = n < WIDE_MIN_ROWS ? 1u : t != HQ_Q6_K || !bf ? 4u : 2u;
     void (*kern)(RowsArgs);
     if (t == HQ_Q4_K)
         kern = nsb == 4 ? (bf ? q4k_rows_kernel<true, 4> : q4k_rows_kernel<false, 4>)
                         : (bf ? q4k_rows_kernel<true, 1> : q4k_rows_kernel<false, 1>);
+    else if (t == HQ_Q5_K)
+        kern = nsb == 4 ? (bf ? q4k_rows_kernel<true, 4, true> : q4k_rows_kernel<false, 4, true>)
+                        : (bf ? q4k_rows_kernel<true, 1, true> : q4k_rows_kernel<false, 1, true>);
     else
         kern = nsb == 4 ? q6k_rows_kernel<false, 4>
                : nsb == 2 ? q6k_rows_kernel<true, 2>

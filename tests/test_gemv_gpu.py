@@ -319,11 +319,11 @@ def test_mul_mat_id_grouped_routing_properties(oracle, dev):
 ROWS_SHAPES = [(3, 80, 2048), (4, 64, 1024), (4, 200, 4096), (4, 16, 2048), (5, 33, 1024), (6, 130, 3072), (7, 250, 2048), (8, 96, 12288)]
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q5_K])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,n,k", ROWS_SHAPES)
 def test_small_batch_rows_match_f64_oracle(oracle, dev, t, xdt, m, n, k):
-    """Q4_K (3 <= m <= 8) and Q6_K (4 <= m <= 8) with k % 1024 == 0 take the kernel that fetches every weight once for all rows."""
+    """Q4_K / Q5_K (3 <= m <= 8) and Q6_K (4 <= m <= 8) with k % 1024 == 0 take the kernel that fetches every weight once for all rows."""
     blocks = oracle.quantize(weights(3 * n + k + m, n, k), k, t, threads=8)
     x = acts(n + k + m, m, k)
     xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
@@ -341,7 +341,7 @@ def test_small_batch_rows_match_f64_oracle(oracle, dev, t, xdt, m, n, k):
         assert np.abs(y1.cpu().numpy()[0] - y.cpu().numpy()[r]).max() <= 1e-4 * np.abs(ref).max()
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q5_K])
 @pytest.mark.parametrize("xdt,m", [("bf16", 8), ("f32", 5)])
 def test_small_batch_rows_tall_matrix(oracle, dev, t, xdt, m):
     """From 49152 weight rows on a workgroup takes 64 rows instead of 16; the last workgroup here is ragged (n % 64 = 40,
@@ -360,7 +360,7 @@ def test_small_batch_rows_tall_matrix(oracle, dev, t, xdt, m):
     assert_matmul_close(y.cpu().numpy(), ref, f"rows, tall matrix t={t} {xdt} m={m}")
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q5_K])
 def test_small_batch_rows_adversarial_blocks_and_scaling(oracle, dev, t):
     """Every scale / min / nibble pattern; and scaling the activations by a power of two scales the result exactly."""
     m, n, k = 8, 48, 2048
