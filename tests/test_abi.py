@@ -38,6 +38,26 @@ def test_block_geometry():
     assert L.hq_block_elems(3) == 0 and L.hq_block_bytes(10) == 0  # Q4_1, Q2_K: not built
 
 
+def test_workspace_queries_follow_the_routing():
+    """Pure host arithmetic (no GPU call): which shapes take a tile kernel and how much scratch that needs."""
+    L = lib.load()
+    for t, kq in ((lib.HQ_Q4_K, 256), (lib.HQ_Q5_K, 256), (lib.HQ_Q6_K, 256), (lib.HQ_Q8_0, 128), (lib.HQ_Q4_0, 128)):
+        bb, be = L.hq_block_bytes(t), L.hq_block_elems(t)
+        # dense: m <= 8 never needs scratch, m > 8 needs the f16 activations (+ row scales) when k suits the tile kernel
+        assert L.hq_qmatmul_ggml_workspace_bytes(8, 512, 4 * kq, lib.HQ_BF16, t) == 0
+        need = L.hq_qmatmul_ggml_workspace_bytes(64, 512, 4 * kq, lib.HQ_BF16, t)
+        assert need >= 64 * 4 * kq * 2 and need % 256 == 0
+        if be == 32:
+            assert L.hq_qmatmul_ggml_workspace_bytes(64, 512, 96, lib.HQ_BF16, t) == 0  # k % 128 != 0: no tile kernel
+        # mul_mat_id: the grouped route wants >= 256 routed rows, >= 8 per expert and a contiguous stack
+        n, k, E = 128, 2 * kq, 8
+        stride = n * (k // be) * bb
+        assert L.hq_qmatmul_id_ggml_workspace_bytes(64, 4, n, k, E, stride, t) > 0
+        assert L.hq_qmatmul_id_ggml_workspace_bytes(64, 4, n, k, E, stride + 32, t) == 0  # padded stack
+        assert L.hq_qmatmul_id_ggml_workspace_bytes(8, 4, n, k, E, stride, t) == 0        # decode-sized
+    assert L.hq_qmatmul_id_ggml_workspace_bytes(64, 4, 128, 512, 8, 128 * 2 * 144, 10) == 0  # not a type of the library
+
+
 def test_argument_errors_are_reported_not_fatal():
     L = lib.load()
     fake = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
