@@ -1,0 +1,182 @@
+"""The benchmark configurations at their full sizes.
+
+The other GPU tests compare whole outputs with the oracle at sizes it finishes in seconds.  Here every
+configuration runs at the shape its throughput is quoted on, and is checked (a) against the oracle on a sample
+of output rows that the oracle can afford (its inputs are slices of the same device-quantized weights, and the
+device quantizer is byte-equal to the oracle's by test_gemv_gpu.py), and (b) through properties that hold at
+any size: linearity in the activations, exact scaling by powers of two, a known closed form."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_matmul_close, assert_matmul_close_f16_tile
+from hf2q_amd import ops
+from hf2q_amd.ops import HQ_Q4_K, HQ_Q6_K, FlashAttnVecTqHbParams, GgmlQuantizedMatmulParams
+
+pytestmark = pytest.mark.gpu
+
+
+def _quantized(dev, n, k, t, seed):
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    return ops.quantize_ggml(torch.randn(n * k, generator=g, device=dev).mul_(0.02), k, t)
+
+
+def _rows_of(blocks, rows, k, t, oracle):
+    """The packed rows `rows` of a device weight matrix, as one small host matrix."""
+    rb = k // oracle.BLOCK_ELEMS[t] * oracle.BLOCK_BYTES[t]
+    m = blocks.view(-1, rb)
+    return m[torch.as_tensor(rows, device=blocks.device)].contiguous().view(-1).cpu().numpy()
+
+
+# decode GEMV: gate / up 12288 x 4096 and down 4096 x 12288 in Q4_K, the output head 151936 x 4096 in Q6_K
+DECODE_SHAPES = [(12288, 4096, HQ_Q4_K), (4096, 12288, HQ_Q4_K), (151936, 4096, HQ_Q6_K)]
+
+
+@pytest.mark.parametrize("n,k,t", DECODE_SHAPES)
+@pytest.mark.parametrize("m", [1, 8])
+def test_decode_gemv_full_size(oracle, dev, n, k, t, m):
+    """m = 1: the GEMV kernels of the decode step; m = 8: the small-batch kernels on the same matrices."""
+    w = _quantized(dev, n, k, t, 7 + n)
+    rng = np.random.default_rng(n + m)
+    # multiples of 1/8 below 4 in magnitude: exact in bf16, and so are the sums of two of them
+    xa = (rng.integers(-12, 13, (m, k)) / 8.0).astype(np.float32)
+    xb = (rng.integers(-12, 13, (m, k)) / 8.0).astype(np.float32)
+    p = GgmlQuantizedMatmulParams(m, n, k, t)
+
+    def run(x):
+        y = torch.full((m, n), float("nan"), device=dev)
+        ops.quantized_matmul_ggml(torch.from_numpy(x).to(dev).to(torch.bfloat16), w, y, p)
+        return y
+
+    ya, yb, yab = run(xa), run(xb), run(xa + xb)
+    assert torch.isfinite(yab).all()
+    # (a) sampled rows against the f64 oracle
+    rows = np.unique(np.concatenate([[0, 1, n - 2, n - 1], rng.integers(0, n, 60)]))
+    ref = oracle.qmatmul_f64(oracle.f32_to_bf16_bits(xa), _rows_of(w, rows, k, t, oracle), m, rows.size, k, t)
+    assert_matmul_close(ya[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, f"gemv {n}x{k} m={m}, sampled rows")
+    # (b) linearity over every output, to f32 accumulation noise of the output's scale
+    scale = yab.abs().max().item()
+    assert (yab - (ya + yb)).abs().max().item() <= 2e-5 * scale
+    # (c) exact scaling by a power of two
+    assert torch.equal(run(xa * 4.0), ya * 4.0)
+
+
+def test_prefill_gemm_full_size(oracle, dev):
+    """2048 tokens x K = 4096 x N = 12288, Q4_K, bf16 activations: a sample of (token, weight row) pairs against the
+    oracle, scaling of a token row by a power of two, and agreement of token rows with the m = 1 GEMV."""
+    m, k, n, t = 2048, 4096, 12288, HQ_Q4_K
+    w = _quantized(dev, n, k, t, 1234)
+    g = torch.Generator(device=dev)
+    g.manual_seed(5678)
+    x = torch.randn(m, k, generator=g, device=dev).to(torch.bfloat16)
+    p = GgmlQuantizedMatmulParams(m, n, k, t)
+    ws = torch.empty(ops.quantized_matmul_workspace_bytes(p, torch.bfloat16), dtype=torch.uint8, device=dev)
+    y = torch.full((m, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(x, w, y, p, workspace=ws)
+    assert torch.isfinite(y).all()
+    rng = np.random.default_rng(3)
+    toks = np.unique(np.concatenate([[0, 255, 256, m - 1], rng.integers(0, m, 12)]))
+    rows = np.unique(np.concatenate([[0, 127, 128, n - 1], rng.integers(0, n, 44)]))
+    xs = x[torch.as_tensor(toks, device=dev)].float().cpu().numpy()
+    ref = oracle.qmatmul_f64(oracle.f32_to_bf16_bits(xs), _rows_of(w, rows, k, t, oracle), toks.size, rows.size, k, t)
+    got = y[torch.as_tensor(toks, device=dev)][:, torch.as_tensor(rows, device=dev)].cpu().numpy()
+    assert_matmul_close_f16_tile(got, ref, "prefill gemm, sampled tokens x rows")
+    # a token row scaled by 2^5 gives that output row scaled by 2^5, bit for bit; the others do not move
+    x2 = x.clone()
+    x2[777] *= 32.0
+    y2 = torch.empty_like(y)
+    ops.quantized_matmul_ggml(x2, w, y2, p, workspace=ws)
+    assert torch.equal(y2[777], y[777] * 32.0)
+    assert torch.equal(y2[:777], y[:777]) and torch.equal(y2[778:], y[778:])
+    # token rows agree with the GEMV of the same row (exact products there, f16-rounded weights here)
+    y1 = torch.empty(1, n, device=dev)
+    for i in (0, 1029, m - 1):
+        ops.quantized_matmul_ggml(x[i:i + 1].contiguous(), w, y1, GgmlQuantizedMatmulParams(1, n, k, t))
+        assert (y[i] - y1[0]).abs().max().item() <= 1e-3 * y1.abs().max().item()
+
+
+def test_moe_layer_full_size(oracle, dev):
+    """hidden 2048, 256 experts x inter 512 (Q4_K), one shared expert, top-8, one token and eight: the block against
+    a float64 evaluation over the device-dequantised weights of the experts the router picked."""
+    H, E, I, K, t = 2048, 256, 512, 8, HQ_Q4_K
+    g = torch.Generator(device=dev)
+    g.manual_seed(99)
+    rnd = lambda *s: torch.randn(*s, generator=g, device=dev)  # noqa: E731
+    w = ops.MoeFfnWeightsGpuQ(
+        router=(rnd(E, H) * 0.1).to(torch.bfloat16), expert_gate=_quantized(dev, E * I, H, t, 1),
+        expert_up=_quantized(dev, E * I, H, t, 2), expert_down=_quantized(dev, E * H, I, t, 3),
+        shared_gate_logit=(rnd(1, H) * 0.1).to(torch.bfloat16), shared_gate=_quantized(dev, I, H, t, 4),
+        shared_up=_quantized(dev, I, H, t, 5), shared_down=_quantized(dev, H, I, t, 6),
+        n_experts=E, top_k=K, hidden=H, inter=I, shared_inter=I, ggml_type=t)
+    deq = lambda b, r, c: ops.dequantize_ggml(b, r * c, t).view(r, c).double()  # noqa: E731
+    sg, su, sd = deq(w.shared_gate, I, H), deq(w.shared_up, I, H), deq(w.shared_down, H, I)
+    rb_h, rb_i = ops.ggml_row_bytes(t, H), ops.ggml_row_bytes(t, I)
+    for T in (1, 8):
+        x = rnd(T, H).to(torch.bfloat16)
+        s = ops.MoeFfnScratch(w, T, dev)
+        out = torch.full((T, H), float("nan"), device=dev)
+        ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out)
+        xd = x.double()
+        ids, tw = s.ids.view(T, K).long(), s.topk_w.view(T, K).double()
+        # the routing itself: softmax / top-k of the router logits, against the CPU specification
+        want_i, want_w = oracle.softmax_topk_renorm(s.logits.cpu().numpy(), T, E, K)
+        assert np.array_equal(ids.cpu().numpy().reshape(-1).astype(np.uint32), want_i)
+        assert np.allclose(tw.cpu().numpy().reshape(-1), want_w, rtol=1e-5, atol=1e-7)
+        assert torch.allclose(s.logits.double(), xd @ w.router.double().T, rtol=1e-4, atol=1e-4)
+        ref = torch.zeros(T, H, dtype=torch.float64, device=dev)
+        for ti in range(T):
+            for kk in range(K):
+                e = int(ids[ti, kk])
+                eg = deq(w.expert_gate.view(E, -1)[e], I, H)
+                eu = deq(w.expert_up.view(E, -1)[e], I, H)
+                ed = deq(w.expert_down.view(E, -1)[e], H, I)
+                a = torch.nn.functional.silu(eg @ xd[ti]) * (eu @ xd[ti])
+                ref[ti] += tw[ti, kk] * (ed @ a)
+            gate = torch.sigmoid((w.shared_gate_logit.double() @ xd[ti])[0])
+            ref[ti] += gate * (sd @ (torch.nn.functional.silu(sg @ xd[ti]) * (su @ xd[ti])))
+        assert rb_h * I * E == w.expert_gate.numel() and rb_i * H * E == w.expert_down.numel()
+        err = (out.double() - ref).abs().max().item()
+        rms = ref.pow(2).mean().sqrt().item()
+        assert err <= 2e-3 * rms, f"T={T}: max err {err} vs rms {rms}"
+
+
+def test_tq_attention_full_size(oracle, dev):
+    """32768 cached tokens, 16 query heads over 2 KV heads, head_dim 256, int8 codes: the whole output against the
+    f64 oracle, the fused rotate-attend-rotate call against the three separate calls, and the closed form of a
+    cache whose values are all one vector."""
+    nh, nkv, hd, n = 16, 2, 256, 32768
+    rng = np.random.default_rng(5)
+    kc = rng.integers(-127, 128, (nkv, n, hd)).astype(np.int8).view(np.uint8)
+    vc = rng.integers(-127, 128, (nkv, n, hd)).astype(np.int8).view(np.uint8)
+    kn = rng.uniform(0.5, 2.0, (nkv, n, 1)).astype(np.float32)
+    vn = rng.uniform(0.5, 2.0, (nkv, n, 1)).astype(np.float32)
+    q = rng.standard_normal((nh, hd)).astype(np.float32)
+    qr = oracle.fwht_sign_premult(q.copy(), nh, hd)
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, n, 1.0 / 16.0)
+    ref = oracle.tq_attention(qr, kc, kn, vc, vn, None, nh, nkv, hd, n, n, p.scale)
+    d = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    kcd, knd, vcd, vnd = d(kc), d(kn), d(vc), d(vn)
+    tmp = torch.empty(ops.tq_tmp_buffer_bytes(nh, hd, n) // 4, device=dev)
+    out = torch.full((nh, hd), float("nan"), device=dev)
+    ops.flash_attn_vec_tq_hb(d(qr), kcd, knd, vcd, vnd, out, tmp, p)
+    got = out.cpu().numpy()
+    scale = np.abs(ref).max(axis=1, keepdims=True)
+    assert np.isfinite(got).all() and (np.abs(got - ref) <= 1e-3 * scale).all()
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) < 1e-4
+    # one call with both rotations inside = rotate, attend, rotate back
+    sep = out.clone()
+    ops.dispatch_fwht_sign_undo_f32(sep, nh, hd)
+    fused = torch.full((nh, hd), float("nan"), device=dev)
+    pf = FlashAttnVecTqHbParams(nh, nkv, hd, n, n, 1.0 / 16.0, fuse_fwht_pre=1)
+    ops.flash_attn_vec_tq_hb(d(q), kcd, knd, vcd, vnd, fused, tmp, pf, undo_rotation=True)
+    assert torch.equal(fused, sep)
+    # every cached value the same vector (per KV head): the output is that vector whatever the scores
+    v1 = rng.integers(-127, 128, (nkv, 1, hd)).astype(np.int8)
+    vcc = np.broadcast_to(v1, (nkv, n, hd)).copy().view(np.uint8)
+    vnc = np.full((nkv, n, 1), 1.25, np.float32)
+    ops.flash_attn_vec_tq_hb(d(qr), kcd, knd, d(vcc), d(vnc), out, tmp, p)
+    want = np.repeat(oracle.tq_dequantize(vcc, vnc, None, nkv, hd, n, 0, 1)[:, 0, :], nh // nkv, axis=0)
+    # (the softmax weights are 22-bit numbers summed over 32768 positions: 2e-5 of the magnitude observed)
+    err, mag = float(np.abs(out.cpu().numpy() - want).max()), float(np.abs(want).max())
+    assert err <= 1e-4 * mag, f"constant-value cache: {err} vs {mag}"
