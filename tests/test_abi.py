@@ -58,6 +58,26 @@ def test_workspace_queries_follow_the_routing():
     assert L.hq_qmatmul_id_ggml_workspace_bytes(64, 4, 128, 512, 8, 128 * 2 * 144, 10) == 0  # not a type of the library
 
 
+def test_empty_inputs_are_accepted_without_work():
+    """Zero rows / tokens / elements: HQ_OK before any launch (the pointers here are never dereferenced); an empty
+    attention cache is an error, as there is nothing to attend to."""
+    L = lib.load()
+    fake = ctypes.c_void_p(0x1000)
+    assert L.hq_qmatmul_ggml(None, fake, lib.HQ_BF16, fake, fake, 0, 8, 256, lib.HQ_Q4_K) == lib.HQ_OK
+    assert L.hq_qmatmul_ggml_ws(None, fake, lib.HQ_BF16, fake, fake, 0, 8, 256, lib.HQ_Q6_K, None, 0) == lib.HQ_OK
+    assert L.hq_qmatmul_id_ggml(None, fake, lib.HQ_F32, fake, fake, fake, None, 0, 0, 2, 8, 256, 4, 8 * 144, lib.HQ_Q4_K) == lib.HQ_OK
+    assert L.hq_dequant_ggml(None, fake, fake, lib.HQ_F32, 0, lib.HQ_Q8_0) == lib.HQ_OK
+    assert L.hq_quantize_ggml(None, fake, 0, 256, lib.HQ_Q5_K, fake) == lib.HQ_OK
+    assert L.hq_moe_softmax_topk(None, fake, fake, fake, 0, 256, 8) == lib.HQ_OK
+    assert L.hq_moe_weighted_reduce(None, fake, fake, None, None, None, fake, 0, 8, 2048) == lib.HQ_OK
+    assert L.hq_silu_mul(None, fake, fake, fake, 0) == lib.HQ_OK
+    assert L.hq_dense_gemv_bf16(None, fake, lib.HQ_F32, fake, fake, 0, 4, 16) == lib.HQ_OK
+    assert L.hq_fwht_sign_premult_f32(None, fake, 0, 256) == lib.HQ_OK
+    p = lib.TqAttnParams(16, 2, 256, 0, 64, 0.0625, 0, 0, 0.0, 0, 1.0, 8, 0, 1)
+    assert L.hq_flash_attn_vec_tq(None, fake, fake, fake, fake, fake, None, fake, fake, 1 << 20, ctypes.byref(p)) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert "kv_seq_len" in lib.last_error()
+
+
 def test_argument_errors_are_reported_not_fatal():
     L = lib.load()
     fake = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
