@@ -133,18 +133,35 @@ static int check_matmul_common(const char* fn, const void* x, hq_act_dtype xdt, 
 
 namespace {
 
-bool f16_tile_route(uint32_t m, uint32_t k, hq_ggml_type t) { return m > kGemvMaxRows && gemm_f16_tile_supported(t, k); }
+// A few rows past the GEMV limit still run in chunks of kGemvMaxRows rows: a tile kernel multiplies 256 token rows
+// whatever m is, so it costs what a dozen passes of the small-batch kernel cost (measured, 12288 x 4096 Q4_K: 211 us
+// for any m <= 256 against 17.5 us per eight rows; 151936 x 4096 Q6_K: 2650 against 339 us), or what two to four
+// rounds of per-row GEMVs cost where there is no small-batch kernel.
+uint32_t chunked_rows_limit(uint32_t k, hq_ggml_type t) {
+    if (!gemv_rows_supported(t, kGemvMaxRows, k)) return 2 * kGemvMaxRows;
+    return t == HQ_Q6_K ? 6 * kGemvMaxRows : 8 * kGemvMaxRows;
+}
+
+bool f16_tile_route(uint32_t m, uint32_t k, hq_ggml_type t) {
+    return m > chunked_rows_limit(k, t) && gemm_f16_tile_supported(t, k);
+}
 
 // All routes of the dense product; `workspace` is only read on the f16 tile route.
 int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
                    uint32_t n, uint32_t k, hq_ggml_type t, void* workspace) {
     if (f16_tile_route(m, k, t)) return launch_gemm_f16_tile(stream, x, xdt, w_blocks, y, m, n, k, t, workspace);
-    if (m > kGemvMaxRows && gemm_supported(t, k)) return launch_gemm(stream, x, xdt, w_blocks, y, m, n, k, t);
-    if (gemv_rows_supported(t, m, k)) return launch_gemv_rows(stream, x, xdt, w_blocks, y, m, n, k, t);
-    // GEMV form, kGemvMaxRows activation rows per launch (also the route of shapes the
-    // tile kernels do not cover).
+    if (m > chunked_rows_limit(k, t) && gemm_supported(t, k)) return launch_gemm(stream, x, xdt, w_blocks, y, m, n, k, t);
+    // kGemvMaxRows activation rows per launch: the small-batch kernel where it exists for the chunk, else one GEMV
+    // per row (also the route of shapes the tile kernels do not cover).
     const size_t xrow_bytes = (size_t)k * (xdt == HQ_BF16 ? 2 : 4);
     for (uint32_t r0 = 0; r0 < m; r0 += kGemvMaxRows) {
+        const uint32_t rows = m - r0 < kGemvMaxRows ? m - r0 : kGemvMaxRows;
+        if (gemv_rows_supported(t, rows, k)) {
+            if (int rc = launch_gemv_rows(stream, static_cast<const uint8_t*>(x) + (size_t)r0 * xrow_bytes, xdt, w_blocks,
+                                          y + (size_t)r0 * n, rows, n, k, t))
+                return rc;
+            continue;
+        }
         GemvArgs a{};
         a.x = static_cast<const uint8_t*>(x) + (size_t)r0 * xrow_bytes;
         a.w = static_cast<const uint8_t*>(w_blocks);

@@ -43,12 +43,14 @@ def test_workspace_queries_follow_the_routing():
     L = lib.load()
     for t, kq in ((lib.HQ_Q4_K, 256), (lib.HQ_Q5_K, 256), (lib.HQ_Q6_K, 256), (lib.HQ_Q8_0, 128), (lib.HQ_Q4_0, 128)):
         bb, be = L.hq_block_bytes(t), L.hq_block_elems(t)
-        # dense: m <= 8 never needs scratch, m > 8 needs the f16 activations (+ row scales) when k suits the tile kernel
+        # dense: up to 8 rows (and a few chunks of 8 beyond: 16 rows at least) never need scratch; prefill-sized m
+        # needs the f16 activations (+ row scales) when k suits the tile kernel
         assert L.hq_qmatmul_ggml_workspace_bytes(8, 512, 4 * kq, lib.HQ_BF16, t) == 0
-        need = L.hq_qmatmul_ggml_workspace_bytes(64, 512, 4 * kq, lib.HQ_BF16, t)
-        assert need >= 64 * 4 * kq * 2 and need % 256 == 0
+        assert L.hq_qmatmul_ggml_workspace_bytes(16, 512, 4 * kq, lib.HQ_BF16, t) == 0
+        need = L.hq_qmatmul_ggml_workspace_bytes(512, 512, 4 * kq, lib.HQ_BF16, t)
+        assert need >= 512 * 4 * kq * 2 and need % 256 == 0
         if be == 32:
-            assert L.hq_qmatmul_ggml_workspace_bytes(64, 512, 96, lib.HQ_BF16, t) == 0  # k % 128 != 0: no tile kernel
+            assert L.hq_qmatmul_ggml_workspace_bytes(512, 512, 96, lib.HQ_BF16, t) == 0  # k % 128 != 0: no tile kernel
         # mul_mat_id: the grouped route wants >= 256 routed rows, >= 8 per expert and a contiguous stack
         n, k, E = 128, 2 * kq, 8
         stride = n * (k // be) * bb
