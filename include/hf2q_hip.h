@@ -85,17 +85,18 @@ HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, ui
  * &mut dst, &GgmlQuantizedMatmulParams{m,n,k,ggml_type})
  * (src/inference/models/qwen35/gpu_ffn.rs:1236-1245; dispatch_qmatmul,
  * src/serve/forward_mlx.rs:9655-9969).  m <= 8 takes the bandwidth-bound GEMV
- * kernels, m > 8 the MFMA GEMM (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791);
- * the Q4_K / Q6_K (k % 256 == 0) and Q8_0 (k % 128 == 0) GEMMs multiply f16-rounded
+ * kernels (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791) and so do a few more rows, eight at a
+ * time (up to 16 .. 64, by type: a tile kernel multiplies 256 token rows whatever m is); larger m the
+ * MFMA GEMM.  The K-quant (k % 256 == 0) and Q8_0 / Q4_0 (k % 128 == 0) GEMMs multiply f16-rounded
  * weights and activations like the reference's mul_mm, the other kernels keep
  * every product exact.
- * Requires k % block_elems == 0; Q4_K needs a 16-byte aligned `w_blocks`,
- * Q6_K / Q8_0 a 2-byte aligned one. */
+ * Requires k % block_elems == 0; Q4_K / Q5_K need a 16-byte aligned `w_blocks`,
+ * the other types a 2-byte aligned one. */
 HQ_API int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y,
                     uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t);
 
 /* The same product with caller-owned device scratch.  The f16 tile kernels
- * (m > 8; Q4_K / Q6_K with k % 256 == 0, Q8_0 with k % 128 == 0) convert the
+ * (prefill-sized m; K-quants with k % 256 == 0, Q8_0 / Q4_0 with k % 128 == 0) convert the
  * activations to row-scaled f16 in a pre-pass and needs hq_qmatmul_ggml_workspace_bytes() bytes (256-byte
  * aligned) for them; every other shape needs none (the function returns 0 and
  * `workspace` may be null).  hq_qmatmul_ggml itself takes that scratch from the
