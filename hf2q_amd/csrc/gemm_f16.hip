@@ -866,7 +866,7 @@ __host__ __device__ inline GroupedLayout grouped_layout(uint32_t pairs, uint32_t
     return g;
 }
 
-constexpr uint32_t BUCKET_MAX_EXPERTS = 4096;
+constexpr uint32_t BUCKET_MAX_EXPERTS = 1024;  // one expert per thread of the sort kernel (hq_moe_softmax_topk's limit too)
 
 // One workgroup: counting sort of the routed rows by expert.  Rows whose id is not an expert get NaN
 // outputs here and take no part in the product.  The order of the rows inside an expert's run depends
@@ -883,16 +883,29 @@ __global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __rest
         if (e < n_experts) atomicAdd(&cnt[e], 1u);
     }
     __syncthreads();
-    if (tid == 0) {
-        uint32_t off = 0, nt = 0;
-        for (uint32_t e = 0; e < n_experts; ++e) {
-            const uint32_t c = cnt[e];
-            cur[e] = off;
-            for (uint32_t r = 0; r < c; r += BM) tiles[nt++] = make_uint4(e, off + r, off + c, 0u);
-            off += c;
-        }
-        *n_tiles = nt;
+    // Exclusive prefix sums over the experts of (rows, tiles), one expert per thread (n_experts <= 1024 = the
+    // workgroup): inside a wave by shuffles, across the sixteen waves through LDS.  Expert e then writes its own tiles.
+    __shared__ uint32_t wave_rows[16], wave_tiles[16];
+    const uint32_t my_rows = tid < n_experts ? cnt[tid] : 0u, my_tiles = (my_rows + BM - 1) / BM;
+    uint32_t inc_rows = my_rows, inc_tiles = my_tiles;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t r = __shfl_up(inc_rows, d), t = __shfl_up(inc_tiles, d);
+        if ((tid & 63u) >= (uint32_t)d) inc_rows += r, inc_tiles += t;
     }
+    if ((tid & 63u) == 63u) wave_rows[tid >> 6] = inc_rows, wave_tiles[tid >> 6] = inc_tiles;
+    __syncthreads();
+    uint32_t off = inc_rows - my_rows, first_tile = inc_tiles - my_tiles, total_rows = 0, total_tiles = 0;
+#pragma unroll
+    for (uint32_t w = 0; w < 16; ++w) {
+        if (w < (tid >> 6)) off += wave_rows[w], first_tile += wave_tiles[w];
+        total_rows += wave_rows[w], total_tiles += wave_tiles[w];
+    }
+    if (tid < n_experts) {
+        cur[tid] = off;
+        for (uint32_t r = 0; r < my_rows; r += BM) tiles[first_tile + r / BM] = make_uint4(tid, off + r, off + my_rows, 0u);
+    }
+    if (tid == 0) *n_tiles = total_tiles;
     __syncthreads();
     for (uint32_t p = tid; p < pairs; p += 1024) {
         const uint32_t e = ids[p];
@@ -903,12 +916,7 @@ __global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __rest
         }
     }
     // rows of the workspace past the sorted ones (invalid ids leave a gap at the end) point at row 0
-    __syncthreads();
-    if (tid == 0) {
-        uint32_t valid = 0;
-        for (uint32_t e = 0; e < n_experts; ++e) valid += cnt[e];
-        for (uint32_t r = valid; r < pairs; ++r) row_map[r] = 0;
-    }
+    for (uint32_t r = total_rows + tid; r < pairs; r += 1024) row_map[r] = 0;
 }
 
 template <int TYPE>
