@@ -142,12 +142,10 @@ def test_tile_gemm_scale_equivariance(oracle, dev, xdt, t):
                                      f"tile gemm t={t} sigma={sigma} {xdt}")
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_0, HQ_Q5_K])
-def test_shapes_without_a_tile_kernel_run_as_gemv_chunks(oracle, dev, t):
-    """m > 8 with a k no tile kernel takes (Q4_0: k % 128 != 0; Q5_K: k % 256 != 0 cannot occur, so it is not
-    run): the GEMV form, eight activation rows per launch (exact f32 accumulation of bf16 x weight)."""
-    if t == HQ_Q5_K:
-        pytest.skip("every valid Q5_K k is a multiple of 256 and has a tile kernel")
+def test_shapes_without_a_tile_kernel_run_as_gemv_chunks(oracle, dev):
+    """Prefill-sized m with a k no tile kernel takes (Q4_0, k % 128 != 0): the GEMV form, eight activation rows per
+    launch (exact f32 accumulation of bf16 x weight)."""
+    t = HQ_Q4_0
     m, n, k = 21, 96, 1056
     blocks = oracle.quantize(weights(t, n, k), k, t, threads=8)
     x = acts(5, m, k)

@@ -360,6 +360,23 @@ def test_small_batch_rows_tall_matrix(oracle, dev, t, xdt, m):
     assert_matmul_close(y.cpu().numpy(), ref, f"rows, tall matrix t={t} {xdt} m={m}")
 
 
+@pytest.mark.parametrize("t,m,k", [(HQ_Q4_K, 9, 2048), (HQ_Q4_K, 41, 1024), (HQ_Q5_K, 64, 1024), (HQ_Q6_K, 18, 2048),
+                                   (HQ_Q6_K, 48, 1024), (HQ_Q8_0, 13, 1024), (HQ_Q4_K, 15, 768)])
+def test_a_few_rows_past_eight_run_in_chunks_of_eight(oracle, dev, t, m, k):
+    """Up to 64 (Q4_K / Q5_K), 48 (Q6_K) or 16 rows (no small-batch kernel for the type or k) do not take a 256-row
+    tile: chunks of eight through the small-batch kernel, the remainder through it or the GEMV.  Every product is
+    exact on this route, so the GEMV's tolerance holds, and no scratch is asked for."""
+    n = 136
+    blocks = oracle.quantize(weights(m + k + t, n, k), k, t, threads=8)
+    x = acts(m + t, m, k)
+    ref = oracle.qmatmul_f64(oracle.f32_to_bf16_bits(x), blocks, m, n, k, t)
+    y = torch.full((m, n), float("nan"), device=dev)
+    p = GgmlQuantizedMatmulParams(m, n, k, t)
+    assert ops.quantized_matmul_workspace_bytes(p, torch.bfloat16) == 0
+    ops.quantized_matmul_ggml(torch.from_numpy(x).to(dev).to(torch.bfloat16), torch.from_numpy(blocks).to(dev), y, p)
+    assert_matmul_close(y.cpu().numpy(), ref, f"chunked rows t={t} m={m} k={k}")
+
+
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q5_K])
 def test_small_batch_rows_adversarial_blocks_and_scaling(oracle, dev, t):
     """Every scale / min / nibble pattern; and scaling the activations by a power of two scales the result exactly."""
