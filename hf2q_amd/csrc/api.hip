@@ -340,7 +340,14 @@ int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_j
         a.y = j.y;
         a.n = j.n;
         a.k = j.k;
-        if (j.ids) {
+        if (j.route_logits) {
+            if (j.ids) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: ids and route_logits are both set", fn, i);
+            if (j.n_experts > 256 || j.top_k > 64 || j.top_k > j.n_experts)
+                return fail(HQ_ERR_UNSUPPORTED, "%s: job %u: in-launch routing takes n_experts <= 256 and top_k <= min(64, n_experts)", fn, i);
+            if (!j.route_ids != !j.route_weights)
+                return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: route_ids and route_weights go together", fn, i);
+        }
+        if (j.ids || j.route_logits) {
             if (j.n_experts == 0 || j.top_k == 0)
                 return fail(HQ_ERR_INVALID_ARGUMENT, "%s: job %u: n_experts %u, top_k %u", fn, i, j.n_experts, j.top_k);
             const uint64_t expert_bytes = (uint64_t)j.n * (j.k / hq_block_elems(t)) * hq_block_bytes(t);
@@ -350,6 +357,9 @@ int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_j
             const uint64_t pairs = (uint64_t)j.rows * j.top_k;
             if (pairs > 65535) return fail(HQ_ERR_UNSUPPORTED, "%s: job %u: %llu routed rows (limit 65535)", fn, i, (unsigned long long)pairs);
             a.ids = j.ids;
+            a.route_logits = j.route_logits;
+            a.route_ids = j.route_ids;
+            a.route_w = j.route_weights;
             a.pairs = (uint32_t)pairs;
             a.top_k = j.top_k;
             a.n_experts = j.n_experts;

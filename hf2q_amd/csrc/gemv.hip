@@ -32,6 +32,7 @@
 #include <mutex>
 
 #include "hq_internal.h"
+#include "moe_topk.h"
 
 namespace hq {
 
@@ -377,6 +378,9 @@ struct KArgs {
     const void* x2;  // f32 only, may be null: the activations are silu(x) * x2
     const uint8_t* w;
     const uint32_t* ids;
+    const float* route_logits;  // see GemvArgs
+    uint32_t* route_ids;
+    float* route_w;
     float* y;
     uint32_t top_k, n, k, n_experts;
     uint64_t expert_stride;
@@ -589,6 +593,18 @@ __device__ __forceinline__ void gemv_body(const KArgs& a, uint32_t bx, uint32_t 
         const uint32_t e = a.ids[p];
         valid = e < a.n_experts;
         w += (size_t)(valid ? e : 0u) * a.expert_stride;
+    } else if (a.route_logits) {
+        // every wave works the token's routing out for itself (no barrier before the first weight fetch); one
+        // wave of the launch per token also writes it down
+        const uint32_t tok = p / a.top_k, slot = p % a.top_k, lane = threadIdx.x & 63u;
+        uint32_t id;
+        float wt;
+        softmax_topk_lane<4>(a.route_logits + (size_t)tok * a.n_experts, a.n_experts, a.top_k, lane, id, wt);
+        if (a.route_ids && bx == 0 && slot == 0 && threadIdx.x < a.top_k) {
+            a.route_ids[(size_t)tok * a.top_k + lane] = id;
+            a.route_w[(size_t)tok * a.top_k + lane] = wt;
+        }
+        w += (size_t)__shfl(id, slot) * a.expert_stride;
     }
 
     Walk<TYPE, X_BF16, PAIR, NR, D> wk;
@@ -729,7 +745,7 @@ int plan_job(const GemvArgs& a, KArgs* ka, size_t* lds, uint64_t* slots) {
     constexpr bool PAIR = X_BF16 && !kBlock32<TYPE>;
     constexpr int EPL = Lane<TYPE>::kElems;
     if (a.x2 && X_BF16) return fail(HQ_ERR_UNSUPPORTED, "gemv: the fused SwiGLU form takes f32 activations");
-    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, M4, TYPE == HQ_Q5_K ? M1 : M2, MAGIC};
+    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.route_logits, a.route_ids, a.route_w, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, M4, TYPE == HQ_Q5_K ? M1 : M2, MAGIC};
     const uint32_t pieces = a.k / EPL;
     // L = largest power of two <= 64 that divides the pieces of a row
     uint32_t log_l = 0;
@@ -756,7 +772,8 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
     // Dense matrices with many tasks per wave: the queue kernel.
-    if (a.pairs == 1 && !a.x2 && slots * ((a.k / EPL) >> log_l) >= (uint64_t)cus * QUEUE_MIN_TASKS_PER_CU)
+    if (a.pairs == 1 && !a.x2 && !a.ids && !a.route_logits &&
+        slots * ((a.k / EPL) >> log_l) >= (uint64_t)cus * QUEUE_MIN_TASKS_PER_CU)
         return launch_q<TYPE, X_BF16, PAIR, 2, 2, 12>(s, ka, cus, rpw, lds);
     // Slots one SIMD would get if the work were spread evenly; more slots per wave
     // amortise the per-wave set-up, fewer keep every SIMD busy on small problems.

@@ -38,6 +38,12 @@ struct GemvArgs {
     uint32_t n, k;
     uint32_t n_experts;
     uint64_t expert_stride;  // bytes
+    // Routing computed by the launch itself (ids == nullptr, n_experts <= 256): router logits [pairs / top_k, n_experts];
+    // the expert of pair p is slot p % top_k of its token's softmax / top-k.  route_ids / route_w: nullptr, or where the
+    // selection is also written ([pairs] each) for the launches that follow.
+    const float* route_logits;
+    uint32_t* route_ids;
+    float* route_w;
 };
 // The current device's CU count (cached).
 int cu_count(uint32_t* out);

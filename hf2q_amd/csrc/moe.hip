@@ -9,20 +9,10 @@
 #include <math.h>
 
 #include "hq_internal.h"
+#include "moe_topk.h"
 
 namespace hq {
 namespace {
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-    return v;
-}
 
 // y[m, n] = x[m, k] . W[n, k]^T, W bf16 row-major, x f32 or bf16, fp32 accumulate.
 // One wave per output row; grid (ceil((n_a + n_b)/4), m).  Two matrices over the same
@@ -69,86 +59,17 @@ __global__ __launch_bounds__(256) void dense_gemv_bf16_kernel(const void* __rest
     if (lane == 0) y[(size_t)m * n + row] = acc;
 }
 
-// Wave-wide maximum of a 64-bit key with DPP moves only (no LDS traffic); every lane gets the
-// result.  Quad permutes and row mirrors cover a row of 16 lanes, row_bcast 15 / 31 carry the row
-// maxima upwards, lane 63 then holds the maximum and is read back as a scalar.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint64_t dpp_max_u64(uint64_t v) {
-    const uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
-    const uint32_t olo = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)lo, CTRL, ROW_MASK, 0xf, false);
-    const uint32_t ohi = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)hi, CTRL, ROW_MASK, 0xf, false);
-    const uint64_t o = ((uint64_t)ohi << 32) | olo;
-    return o > v ? o : v;
-}
-__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-    v = dpp_max_u64<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
-    v = dpp_max_u64<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
-    v = dpp_max_u64<0x141, 0xf>(v);  // row_half_mirror
-    v = dpp_max_u64<0x140, 0xf>(v);  // row_mirror
-    v = dpp_max_u64<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-    v = dpp_max_u64<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 63);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 63);
-    return ((uint64_t)hi << 32) | lo;
-}
-
-// One wave per token: probabilities over all experts, the top_k largest (ties -> lower expert id,
-// as a stable descending sort gives), renormalised over the selection (uniform if it sums to ~0).
-// PL = experts per lane (n_experts <= 64 * PL).  A candidate is the key (probability bits,
-// ~expert id): probabilities are >= 0, so their bit patterns order like the values, and the
-// complemented id makes the lower expert win a tie; 0 marks a taken or absent candidate.
 template <int PL>
 __global__ __launch_bounds__(64) void moe_softmax_topk_kernel(const float* __restrict__ logits, uint32_t* __restrict__ ids,
                                                               float* __restrict__ weights, uint32_t n_experts,
                                                               uint32_t top_k) {
     const uint32_t t = blockIdx.x, lane = threadIdx.x;
-    const float* row = logits + (size_t)t * n_experts;
-    float p[PL];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < PL; ++i) {
-        const uint32_t e = lane + 64u * i;
-        p[i] = e < n_experts ? row[e] : -INFINITY;
-        mx = fmaxf(mx, p[i]);
-    }
-    mx = wave_max(mx);
-    float denom = 0.f;
-#pragma unroll
-    for (int i = 0; i < PL; ++i) {
-        const uint32_t e = lane + 64u * i;
-        p[i] = e < n_experts ? expf(p[i] - mx) : 0.f;
-        denom += p[i];
-    }
-    denom = wave_sum(denom);
-    const float inv_d = denom > 1e-20f ? 1.f / denom : 1.f;
-    uint64_t key[PL];
-#pragma unroll
-    for (int i = 0; i < PL; ++i) {
-        const uint32_t e = lane + 64u * i;
-        key[i] = e < n_experts ? ((uint64_t)__float_as_uint(p[i] * inv_d) << 32) | (0xffffffffu - e) : 0ull;
-    }
-
-    float sum_sel = 0.f, my_w = 0.f;
-    uint32_t my_id = 0;
-    for (uint32_t s = 0; s < top_k; ++s) {
-        uint64_t best = 0ull;
-#pragma unroll
-        for (int i = 0; i < PL; ++i) best = key[i] > best ? key[i] : best;
-        best = wave_max_u64(best);  // uniform
-#pragma unroll
-        for (int i = 0; i < PL; ++i) key[i] = key[i] == best ? 0ull : key[i];  // keys are unique: only the owner matches
-        const float bv = __uint_as_float((uint32_t)(best >> 32));
-        const uint32_t be = 0xffffffffu - (uint32_t)best;
-        sum_sel += bv;
-        if (lane == s) {  // lane s keeps slot s (top_k <= 64)
-            my_w = bv;
-            my_id = be;
-        }
-    }
-    const float inv_sum = sum_sel > 1e-20f ? 1.f / sum_sel : 1.f / (float)top_k;
+    uint32_t id;
+    float w;
+    softmax_topk_lane<PL>(logits + (size_t)t * n_experts, n_experts, top_k, lane, id, w);
     if (lane < top_k) {
-        ids[(size_t)t * top_k + lane] = my_id;
-        weights[(size_t)t * top_k + lane] = my_w * inv_sum;
+        ids[(size_t)t * top_k + lane] = id;
+        weights[(size_t)t * top_k + lane] = w;
     }
 }
 

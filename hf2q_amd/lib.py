@@ -34,7 +34,8 @@ class QmatmulJob(_c.Structure):
     """hq_qmatmul_job of include/hf2q_hip.h, field for field."""
     _fields_ = [("x", _c.c_void_p), ("x_up", _c.c_void_p), ("w", _c.c_void_p), ("ids", _c.c_void_p),
                 ("y", _c.c_void_p), ("rows", _c.c_uint32), ("top_k", _c.c_uint32), ("n", _c.c_uint32),
-                ("k", _c.c_uint32), ("n_experts", _c.c_uint32), ("expert_stride", _c.c_uint64)]
+                ("k", _c.c_uint32), ("n_experts", _c.c_uint32), ("expert_stride", _c.c_uint64),
+                ("route_logits", _c.c_void_p), ("route_ids", _c.c_void_p), ("route_weights", _c.c_void_p)]
 
 
 class GgufTensorInfo(_c.Structure):

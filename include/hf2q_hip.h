@@ -164,7 +164,12 @@ HQ_API size_t hq_qmatmul_id_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top
  * silu(x[i]) * x_up[i], computed while they are staged: the SwiGLU of phase D
  * folded into the down projection (the quantized_matmul_id_swiglu_q4_0 variant
  * that gpu_ffn.rs:2685-2697 describes), bit-identical to hq_silu_mul followed by
- * the plain product. */
+ * the plain product.
+ * With `route_logits` set (and `ids` NULL) the job is routed by the launch itself: every workgroup works out
+ * hq_moe_softmax_topk of its token's logits (the same arithmetic, the same bits) and takes the expert of its
+ * slot, so the dispatch_moe_softmax_topk of phase B (gpu_ffn.rs:2551-2573) needs no launch of its own;
+ * `route_ids` / `route_weights`, if not NULL, also receive the selection ([rows*top_k] each) for the
+ * launches that follow.  n_experts <= 256, top_k <= 64. */
 #define HQ_QMATMUL_BATCH_MAX_JOBS 4
 typedef struct hq_qmatmul_job {
     const void* x;        /* [rows, k] activations */
@@ -174,6 +179,9 @@ typedef struct hq_qmatmul_job {
     float* y;             /* [rows, n] (dense) or [rows*top_k, n] */
     uint32_t rows, top_k, n, k, n_experts;
     uint64_t expert_stride; /* bytes between experts of the stack */
+    const float* route_logits; /* NULL, or [rows, n_experts] router logits (ids must be NULL) */
+    uint32_t* route_ids;       /* NULL, or out [rows*top_k] */
+    float* route_weights;      /* NULL, or out [rows*top_k] */
 } hq_qmatmul_job;
 HQ_API int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_jobs, hq_act_dtype xdt,
                           hq_ggml_type t);

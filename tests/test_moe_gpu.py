@@ -168,15 +168,20 @@ def test_moe_block_batched_launches_equal_separate_dispatches(oracle, dev, T, t,
     x = torch.from_numpy(acts(11 + T, T, H)).to(dev).to(xdt)
     res = torch.from_numpy(acts(12, T, H)).to(dev)
     outs = []
-    for batched in (False, True):
+    # separate dispatches; batched with the softmax / top-k as its own launch; batched with the routing worked out
+    # inside the gate / up launch (four launches)
+    for batched, route_in_launch in ((False, False), (True, False), (True, True)):
         s = ops.MoeFfnScratch(w, T, dev)
+        s.ids.fill_(-1)
+        s.topk_w.fill_(float("nan"))
         out = torch.full((T, H), float("nan"), device=dev)
-        ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out, residual=res, batched=batched)
+        ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out, residual=res, batched=batched, route_in_launch=route_in_launch)
         outs.append((out.cpu(), s.gate.cpu(), s.up.cpu(), s.sh_gate.cpu(), s.sh_up.cpu(), s.down.cpu(), s.sh_down.cpu(),
-                     s.logits.cpu(), s.sh_logit.cpu(), s.ids.cpu()))
-    for a, b in zip(*outs):
-        assert torch.equal(a, b)
-    assert torch.isfinite(outs[1][0]).all()
+                     s.logits.cpu(), s.sh_logit.cpu(), s.ids.cpu(), s.topk_w.cpu()))
+    for other in outs[1:]:
+        for a, b in zip(outs[0], other):
+            assert torch.equal(a, b)
+    assert torch.isfinite(outs[2][0]).all()
 
 
 def test_batched_block_refuses_prefill_sized_token_counts(oracle, dev):
