@@ -711,6 +711,175 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_queue_kernel(KArgs a) {
     }
 }
 
+
+// Dense single-row GEMV over K-quants with bf16 activations and k % 4096 == 0 (64 lanes per row step): one
+// workgroup of W waves per CU.  Requests that join an HBM queue already holding the whole matrix wait microseconds
+// (a 28 MB matrix asked for at once: the activations of late waves arrive after 2-3 us, and nothing can be
+// computed before), so this form keeps little in flight: the workgroup stages the activations first, then every
+// wave walks its rows with ONE fetch outstanding (16 waves x 2.3 KB per CU is what 8 TB/s x 1 us needs); the
+// other waves of the SIMD compute meanwhile.  Row of (iteration i, wave wv, workgroup b) = (i*W + wv)*G + b, so all
+// CUs walk the matrix front to back together.  Rows >= n0 belong to a second matrix of the same shape (the gate /
+// up pair of a decode step in one launch).  Per-row arithmetic (order of the partial sums, per-16 activation sums)
+// is that of gemv_kernel: the results are bit-identical.
+struct SArgs {
+    const void* x;
+    const uint8_t* w0;
+    const uint8_t* w1;
+    float* y0;
+    float* y1;
+    uint32_t n0, n, k;
+    uint32_t m4, m2, magic;
+};
+
+// LDS slot of 16-byte chunk ch (8 activations as 4 paired words): lanes that read together differ in the piece
+// index (Q4_K / Q5_K: ch / 8) or in bits 1, 4, 5.. of ch (Q6_K: run half, block half, block), which the swizzle
+// spreads over the sixteen 16-byte bank groups.
+template <int TYPE>
+__device__ __forceinline__ uint32_t stream_swz(uint32_t ch) {
+    if constexpr (TYPE == HQ_Q6_K) return ch ^ (((ch >> 4) & 1u) | (((ch >> 5) & 3u) << 2));
+    return ch ^ ((ch >> 4) & 7u);
+}
+
+template <int TYPE>
+__device__ __forceinline__ void stream_load_x(const uint4* lds_x, const float* lds_s, uint32_t st, uint32_t lane, int c,
+                                              uint32_t* xp, float* sx) {
+    if constexpr (TYPE == HQ_Q6_K) {
+        const uint32_t ch0 = st * 512u + (lane >> 2) * 32u + (uint32_t)(c >> 1) * 16u + (uint32_t)(c & 1) * 2u;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const uint4 v = lds_x[stream_swz<TYPE>(ch0 + 4 * r + u)];
+                xp[8 * r + 4 * u] = v.x;
+                xp[8 * r + 4 * u + 1] = v.y;
+                xp[8 * r + 4 * u + 2] = v.z;
+                xp[8 * r + 4 * u + 3] = v.w;
+            }
+            sx[r] = lds_s[(ch0 + 4 * r) / 2];
+        }
+    } else {
+        const uint32_t ch0 = (st * 64u + lane) * 8u;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint4 v = lds_x[stream_swz<TYPE>(ch0 + j)];
+            xp[4 * j] = v.x;
+            xp[4 * j + 1] = v.y;
+            xp[4 * j + 2] = v.z;
+            xp[4 * j + 3] = v.w;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sx[r] = lds_s[ch0 / 2 + r];
+    }
+}
+
+template <int TYPE, int W, bool XREG>
+__global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
+    constexpr uint32_t NT = 64 * W, BB = kBlockBytes<TYPE>;
+    extern __shared__ uint4 smem[];
+    uint4* lds_x = smem;
+    float* lds_s = reinterpret_cast<float*>(lds_x + a.k / 8);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
+    const int c = (int)(lane & 3u);
+    const uint32_t S = a.k / 4096u, rowb = a.k / 256u * BB;
+    const uint32_t stride = W * gridDim.x;
+    const uint32_t row_first = wv * gridDim.x + blockIdx.x;
+    const uint32_t rows_mine = row_first < a.n ? (a.n - row_first + stride - 1u) / stride : 0u;
+    const uint32_t ntask = rows_mine * S;
+
+    // the activations first, nothing else of this workgroup in front of them
+    for (uint32_t i = tid; i < a.k / 16u; i += NT) {
+        XRaw<true> raw;
+        raw.fetch(a.x, i);
+        const uint4 p = raw.r[0], q = raw.r[1];
+        const uint32_t w[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
+        uint4 o0, o1;
+        o0.x = (w[0] & 0xffffu) | (w[1] << 16);
+        o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
+        o0.z = (w[2] & 0xffffu) | (w[3] << 16);
+        o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
+        o1.x = (w[4] & 0xffffu) | (w[5] << 16);
+        o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
+        o1.z = (w[6] & 0xffffu) | (w[7] << 16);
+        o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
+        lds_x[stream_swz<TYPE>(2 * i)] = o0;
+        lds_x[stream_swz<TYPE>(2 * i + 1)] = o1;
+        float s = 0.f;  // the same order of additions as stage_store
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            s += bf16_bits_to_f32(w[j] & 0xffffu);
+            s += bf16_bits_to_f32(w[j] >> 16);
+        }
+        lds_s[i] = s;
+    }
+
+    Piece<TYPE> pc;
+    auto fetch = [&](uint32_t row, uint32_t st) {
+        const uint8_t* base = row < a.n0 ? a.w0 + (size_t)row * rowb : a.w1 + (size_t)(row - a.n0) * rowb;
+        pc.load(base + (st * 16u + (lane >> 2)) * BB, c);
+    };
+    uint32_t f_row = row_first, f_st = 0;
+    if (ntask) fetch(f_row, f_st);
+    __syncthreads();
+
+    uint32_t m4, m2, magic;
+    asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
+                 : "=v"(m4), "=v"(m2), "=v"(magic)
+                 : "s"(a.m4), "s"(a.m2), "s"(a.magic));
+    uint32_t xp[32];
+    float sx[4];
+    if constexpr (XREG) stream_load_x<TYPE>(lds_x, lds_s, 0, lane, c, xp, sx);  // k == 4096: one piece per lane for every row
+
+    uint32_t row = row_first, st = 0;
+    float acc = 0.f;
+    for (uint32_t t = 0; t < ntask; ++t) {
+        if constexpr (!XREG) stream_load_x<TYPE>(lds_x, lds_s, st, lane, c, xp, sx);
+        acc += dot_pair(pc, c, xp, sx, m4, m2, magic);
+        if (t + 1 < ntask) {
+            if (++f_st == S) {
+                f_st = 0;
+                f_row += stride;
+            }
+            asm volatile("" : "+v"(acc));  // the refill follows the arithmetic that frees its registers
+            fetch(f_row, f_st);
+        }
+        if (++st == S) {
+            const float v = group_sum(acc, 6);
+            if (lane == 0) {
+                if (row < a.n0) a.y0[row] = v;
+                else a.y1[row - a.n0] = v;
+            }
+            acc = 0.f;
+            st = 0;
+            row += stride;
+        }
+    }
+}
+
+// Whether the streaming form takes (type, k, rows): K-quants, whole 4096-element steps, enough rows to occupy the waves.
+template <int TYPE>
+constexpr bool kStreamType = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K;
+constexpr uint32_t STREAM_MIN_ROWS_PER_WAVE = 2;
+
+template <int TYPE>
+int launch_stream(hipStream_t s, const SArgs& sa, uint32_t cus) {
+    constexpr int W = TYPE == HQ_Q6_K ? 12 : 16;
+    const size_t lds = (size_t)sa.k * 2 + (size_t)(sa.k / 16) * 4;
+    if (sa.k == 4096) {
+        auto kern = gemv_stream_kernel<TYPE, W, true>;
+        hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
+    } else {
+        auto kern = gemv_stream_kernel<TYPE, W, false>;
+        hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
+    }
+    return check_launch("gemv stream kernel launch");
+}
+
+template <int TYPE>
+bool stream_takes(uint32_t n_total, uint32_t k, uint32_t cus) {
+    constexpr uint32_t W = TYPE == HQ_Q6_K ? 12 : 16;
+    return k % 4096 == 0 && k <= 24576 && (uint64_t)n_total * (k / 4096) >= (uint64_t)cus * W * STREAM_MIN_ROWS_PER_WAVE;
+}
+
 template <typename K>
 int set_lds_limit(K kern, size_t lds, const char* what) {
     if (lds <= 64 * 1024) return HQ_OK;
@@ -771,6 +940,10 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     const uint32_t log_l = ka.log_l, rpw = 64u >> log_l;
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
+    if constexpr (X_BF16 && kStreamType<TYPE>) {
+        if (a.pairs == 1 && !a.x2 && !a.ids && !a.route_logits && stream_takes<TYPE>(a.n, a.k, cus))
+            return launch_stream<TYPE>(s, SArgs{a.x, a.w, a.w, a.y, a.y, a.n, a.n, a.k, M4, TYPE == HQ_Q5_K ? M1 : M2, MAGIC}, cus);
+    }
     // Dense matrices with many tasks per wave: the queue kernel.
     if (a.pairs == 1 && !a.x2 && !a.ids && !a.route_logits &&
         slots * ((a.k / EPL) >> log_l) >= (uint64_t)cus * QUEUE_MIN_TASKS_PER_CU)
@@ -813,6 +986,12 @@ int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
     }
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
+    if constexpr (X_BF16 && kStreamType<TYPE>) {
+        const GemvArgs &j0 = jobs[0], &j1 = jobs[1];
+        auto plain = [](const GemvArgs& j) { return j.pairs == 1 && !j.x2 && !j.ids && !j.route_logits; };
+        if (n_jobs == 2 && plain(j0) && plain(j1) && j0.x == j1.x && j0.k == j1.k && stream_takes<TYPE>(j0.n + j1.n, j0.k, cus))
+            return launch_stream<TYPE>(s, SArgs{j0.x, j0.w, j1.w, j0.y, j1.y, j0.n, j0.n + j1.n, j0.k, M4, TYPE == HQ_Q5_K ? M1 : M2, MAGIC}, cus);
+    }
     const uint64_t per_simd = slots / (4ull * cus);
     if (per_simd >= 8) return launch_j<TYPE, X_BF16, PAIR, 4, 4>(s, js, n_jobs, lds);
     if (per_simd >= 2) return launch_j<TYPE, X_BF16, PAIR, 2, 2>(s, js, n_jobs, lds);
