@@ -12,9 +12,12 @@ that no step finds its weights in the 256 MB Infinity Cache.
 
 Prints ONE JSON line: metric = effective GB/s of packed weight bytes, with a
 `roofline` object for the dominant kernel (the Q6_K head GEMV) from HIP-event
-timings taken inside the timed region, a `kernels` table for the others, and a
-`cpu_baseline` object (the scalar CPU port of hf2q's quantize -> dequantize ->
-scalar matmul, timed on this host).
+timings taken inside the timed region, a `kernels` table for the others, a
+`workloads` object with the other BASELINE configurations (MoE decode at 1 and 8
+tokens, the Q4_K and Q8_0 prefill GEMM, the TQ attention), each with its own
+roofline, and a `cpu_baseline` object (the scalar CPU port of hf2q's
+quantize -> dequantize -> scalar matmul, timed on this host).
+`--workload <name>` runs one of them alone and prints its own line.
 """
 from __future__ import annotations
 
@@ -47,13 +50,14 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="decode_gemv",
-                    choices=["decode_gemv", "moe_decode", "prefill_gemm", "tq_attention"],
-                    help="decode_gemv = BASELINE config 2 (the default and the headline metric); the others are "
-                         "configs 3, 4 and 5, each printing its own JSON line")
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "decode_gemv", "moe_decode", "prefill_gemm", "tq_attention"],
+                    help="all (default) = the BASELINE config 2 headline plus configs 3, 4 and 5 under `workloads` in the "
+                         "same JSON line; a single name runs that workload alone and prints its own line")
     ap.add_argument("--tokens", type=int, default=1, help="moe_decode: tokens per step (1 or 8)")
     ap.add_argument("--wtype", default="q4_k", choices=["q4_k", "q8_0", "q6_k", "q5_k", "q4_0"], help="prefill_gemm: weight type")
-    ap.add_argument("--weight-sets", type=int, default=4, help="distinct FFN weight sets rotated per step")
+    ap.add_argument("--weight-sets", type=int, default=6, help="distinct FFN weight sets rotated per step")
+    ap.add_argument("--moe-layers", type=int, default=20, help="moe_decode: distinct MoE layers rotated per step")
     ap.add_argument("--no-graph", action="store_true",
                     help="moe_decode / tq_attention: launch every kernel from the host instead of replaying a HIP "
                          "graph of the step (the steps are 4-12 launches of a few microseconds each)")
@@ -125,33 +129,30 @@ def _timed_steps(a, step, n_variants):
     """Exactly a.steps calls of step(i) between two synchronisations; returns (wall seconds, device
     microseconds per step from one HIP event pair around the whole region).  Unless --no-graph, the steps
     are replayed from HIP graphs the way a decode loop that records its token step runs them: one graph
-    holds a run of consecutive steps (every rotated variant in turn, at least 32 steps), replayed
-    steps // run times, and single-step graphs cover the remainder."""
+    holds a run of min(32, steps) consecutive steps (the rotated variants in turn), replayed steps // run
+    times, and a second graph holds the remaining steps."""
     import torch
 
-    run = n_variants * max(1, -(-32 // n_variants))
+    run = min(32, a.steps)
     q, r = (0, a.steps) if a.no_graph else divmod(a.steps, run)
     if a.no_graph:
         calls = [lambda i=i: step(a.warmup + i) for i in range(a.steps)]
     else:
         side = torch.cuda.Stream()
+        graphs = []
         with torch.cuda.stream(side):
-            big = None
-            if q:
-                big = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(big, stream=side):
-                    for i in range(run):
-                        step(i)
-            singles = []
-            for i in range(min(r, n_variants)):
+            for count in (run, r):
+                if not count:
+                    continue
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g, stream=side):
-                    step(i)
-                singles.append(g)
+                    for i in range(count):
+                        step(i)
+                graphs.append(g)
         torch.cuda.synchronize()
-        calls = ([big.replay] * q if q else []) + [singles[i % n_variants].replay for i in range(r)]
-        for c in ([big.replay] if q else []) + [g.replay for g in singles]:  # untimed: first replay of each graph
-            c()
+        calls = [graphs[0].replay] * q + ([graphs[1].replay] if r else [])
+        for g in graphs:  # untimed: first replay of each graph
+            g.replay()
     e0, e1 = _events(1)[0]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -164,15 +165,47 @@ def _timed_steps(a, step, n_variants):
     return elapsed, e0.elapsed_time(e1) * 1e3 / a.steps
 
 
+def _launch_us(launches, reps=3):
+    """Average device time of one launch: the callables (each enqueues ONE kernel, over weights no other of them
+    touches) are recorded into a HIP graph back to back and the graph is replayed `reps` times between one HIP
+    event pair on the replay stream; elapsed / (reps * len(launches)).  A kernel of a few microseconds cannot be
+    timed by an event pair of its own: the pair adds ~2.5 us."""
+    import torch
+
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            for f in launches:
+                f()
+    torch.cuda.synchronize()
+    g.replay()
+    e0, e1 = _events(1)[0]
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * len(launches))
+
+
 def _finish(a, out):
+    """A workload run alone prints its own line; as part of the default run its dict goes under `workloads`."""
+    if a.workload == "all":
+        return out
     out.setdefault("n_gpus", 1)
     out.update({"steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak",
                 "vs_baseline": None, "data": "synthetic"})
     out["cpu_baseline"] = None if a.no_cpu_baseline else cpu_baseline()
     print(json.dumps(out))
+    return out
 
 
-def bench_moe_decode(a):
+_MOE_LAYERS = {}  # the layers of bench_moe_decode, shared by its T = 1 and T = 8 runs
+
+
+def bench_moe_decode(a, tokens=None):
     """BASELINE config 3: Qwen3.6-35B-A3B-style MoE FFN layer, hidden 2048, 256 experts (inter 512, Q4_K), one
     shared expert, top-8 from seeded router logits, batch 1 or 8, bf16 activations.  A step is one layer."""
     import torch
@@ -181,17 +214,20 @@ def bench_moe_decode(a):
     from hf2q_amd.ops import HQ_Q4_K
 
     dev = torch.device("cuda:0")
-    H, E, K, I, SI, T = 2048, 256, 8, 512, 512, a.tokens
+    H, E, K, I, SI, T = 2048, 256, 8, 512, 512, tokens or a.tokens
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     rnd = lambda *s: torch.randn(*s, generator=gen, device=dev, dtype=torch.float32)  # noqa: E731
     qz = lambda n, k: ops.quantize_ggml(rnd(n * k).mul_(0.02), k, HQ_Q4_K)  # noqa: E731
-    n_layers = max(1, a.weight_sets)  # distinct layers rotated so that experts are not cache-resident
-    layers = []
-    for _ in range(n_layers):
-        layers.append(ops.MoeFfnWeightsGpuQ(
+    n_layers = max(1, a.moe_layers)  # distinct layers rotated: a token touches 17 MB (T=1) of a layer, and the
+    # 256 MB Infinity Cache must not hold the experts a layer routes to from its previous turn
+    if n_layers not in _MOE_LAYERS:
+        _MOE_LAYERS.clear()
+        _MOE_LAYERS[n_layers] = [ops.MoeFfnWeightsGpuQ(
             rnd(E, H).mul_(0.02).to(torch.bfloat16), qz(E * I, H), qz(E * I, H), qz(E * H, I),
-            rnd(1, H).mul_(0.02).to(torch.bfloat16), qz(SI, H), qz(SI, H), qz(H, SI), HQ_Q4_K, H, E, K, I, SI))
+            rnd(1, H).mul_(0.02).to(torch.bfloat16), qz(SI, H), qz(SI, H), qz(H, SI), HQ_Q4_K, H, E, K, I, SI)
+            for _ in range(n_layers)]
+    layers = _MOE_LAYERS[n_layers]
     gx = torch.Generator(device=dev)
     gx.manual_seed(5678)
     x = torch.randn(T, H, generator=gx, device=dev, dtype=torch.float32).to(torch.bfloat16)
@@ -214,7 +250,7 @@ def bench_moe_decode(a):
     u = sum(uniq) / len(uniq)
     step_bytes = (u * 3 + 3) * expert_bytes + (E + 1) * H * 2  # routed + shared experts + router (bf16)
     gbs = step_bytes / layer_us / 1e3
-    _finish(a, {
+    return _finish(a, {
         "metric": "MoE decode tok/s (FFN-only, 40 MoE layers)", "value": round(T / (40 * elapsed / a.steps), 1),
         "unit": "tok/s", "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "bf16",
         "config": {"workload": f"moe_decode: hidden 2048, 256 experts x inter 512 Q4_K, shared expert, top-8, "
@@ -230,7 +266,7 @@ def bench_moe_decode(a):
                      "us_per_launch": round(layer_us, 3), "bytes_per_launch": int(step_bytes)}})
 
 
-def bench_prefill_gemm(a):
+def bench_prefill_gemm(a, wtype=None):
     """BASELINE config 4: 2048 tokens x K=4096 x N=12288, Q4_K (or Q8_0) weights, bf16 activations, f32 out."""
     import torch
 
@@ -239,7 +275,8 @@ def bench_prefill_gemm(a):
 
     dev = torch.device("cuda:0")
     M, K, N = 2048, 4096, 12288
-    t = {"q4_k": HQ_Q4_K, "q8_0": HQ_Q8_0, "q6_k": ops.HQ_Q6_K, "q5_k": ops.HQ_Q5_K, "q4_0": ops.HQ_Q4_0}[a.wtype]
+    wtype = wtype or a.wtype
+    t = {"q4_k": HQ_Q4_K, "q8_0": HQ_Q8_0, "q6_k": ops.HQ_Q6_K, "q5_k": ops.HQ_Q5_K, "q4_0": ops.HQ_Q4_0}[wtype]
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     w = ops.quantize_ggml(torch.randn(N * K, generator=gen, device=dev).mul_(0.02), K, t)
@@ -265,17 +302,17 @@ def bench_prefill_gemm(a):
     us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
     flops = 2.0 * M * N * K
     tf = flops / us / 1e6
-    _finish(a, {
+    return _finish(a, {
         "metric": "prefill TFLOP/s", "value": round(flops * a.steps / elapsed / 1e12, 1), "unit": "TFLOP/s",
         "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f16" if need else "bf16",
-        "config": {"workload": f"prefill_gemm: 2048 tokens x K=4096 x N=12288, {a.wtype.upper()} weights, bf16 "
+        "config": {"workload": f"prefill_gemm: 2048 tokens x K=4096 x N=12288, {wtype.upper()} weights, bf16 "
                                f"activations, fp32 accumulate (BASELINE config 4)", "flop_per_step": flops,
                    "weight_bytes": w.numel(), "workspace_bytes": need,
                    "launches_per_step": 2 if need else 1},
-        "roofline": {"bound": "mfma", "kernel": (f"activation pre-pass + f16 MFMA gemm {a.wtype}" if need else
-                                                 f"bf16 MFMA gemm {a.wtype}"), "achieved": round(tf, 1),
+        "roofline": {"bound": "mfma", "kernel": (f"activation pre-pass + f16 MFMA gemm {wtype}" if need else
+                                                 f"bf16 MFMA gemm {wtype}"), "achieved": round(tf, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": PMC_TRAFFIC_BYTES["prefill_gemm_q4_k_2048x12288x4096"] if a.wtype == "q4_k" else None,
+                     "traffic": PMC_TRAFFIC_BYTES["prefill_gemm_q4_k_2048x12288x4096"] if wtype == "q4_k" else None,
                      "us_per_launch": round(us, 2), "flop_per_launch": flops}})
 
 
@@ -290,7 +327,7 @@ def bench_tq_attention(a):
     nh, nkv, hd, n = 16, 2, 256, 32768
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
-    n_caches = max(8, a.weight_sets)  # 34 MB each: rotate past the 256 MB Infinity Cache
+    n_caches = 12  # 34 MB each: rotate past the 256 MB Infinity Cache
     caches = []
     for _ in range(n_caches):
         kc, kn = ops.alloc_tq_kv(nkv, n, hd, dev)
@@ -323,7 +360,7 @@ def bench_tq_attention(a):
     _, us_sep = timed(separate)
     elapsed, us = timed(fused)
     gbs = nbytes / us / 1e3
-    _finish(a, {
+    return _finish(a, {
         "metric": "TQ-KV decode attention eff. GB/s", "value": round(nbytes * a.steps / elapsed / 1e9, 1),
         "unit": "GB/s", "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f32",
         "config": {"workload": "tq_attention: 32768 context, 16 q heads / 2 kv heads, head_dim 256, int8 codes + f32 "
@@ -362,10 +399,38 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    if a.workload != "decode_gemv":
+    if a.workload not in ("all", "decode_gemv"):
         return {"moe_decode": bench_moe_decode, "prefill_gemm": bench_prefill_gemm,
                 "tq_attention": bench_tq_attention}[a.workload](a)
+    out = bench_decode_gemv(a)
+    if a.workload == "all":
+        def brief(d):
+            keep = ("metric", "value", "unit", "ms_per_step", "dtype", "config", "roofline")
+            return {k: d[k] for k in keep if k in d}
+        import gc
+        wl = {}
+        for name, fn in (("moe_decode_t1", lambda: bench_moe_decode(a, 1)), ("moe_decode_t8", lambda: bench_moe_decode(a, 8)),
+                         ("prefill_gemm_q4_k", lambda: bench_prefill_gemm(a, "q4_k")),
+                         ("prefill_gemm_q8_0", lambda: bench_prefill_gemm(a, "q8_0")),
+                         ("tq_attention_32k", lambda: bench_tq_attention(a))):
+            gc.collect()
+            torch.cuda.empty_cache()
+            wl[name] = brief(fn())
+            if name == "moe_decode_t8":
+                _MOE_LAYERS.clear()
+        out["workloads"] = wl
+    out["cpu_baseline"] = None if a.no_cpu_baseline else cpu_baseline()
+    print(json.dumps(out))
 
+
+def bench_decode_gemv(a):
+    """BASELINE config 2 (the headline): the four dense decode GEMVs of one token."""
+    import torch
+
+    from hf2q_amd import ops
+    from hf2q_amd.ops import HQ_Q4_K, HQ_Q6_K, GgmlQuantizedMatmulParams
+
+    dev = torch.device("cuda:0")
     H, F, V = 4096, 12288, 151936
     shapes = {  # name -> (n, k, type)
         "gate": (F, H, HQ_Q4_K), "up": (F, H, HQ_Q4_K), "down": (H, F, HQ_Q4_K), "head": (V, H, HQ_Q6_K),
@@ -396,16 +461,13 @@ def main():
     nbytes = {nm: sets[0][nm].numel() if nm != "head" else heads[0].numel() for nm in shapes}
     step_bytes = sum(nbytes.values())
 
-    def step(i, ev=None):
+    def one(nm, w):
+        return lambda: ops.quantized_matmul_ggml(x_f if nm == "down" else x_h, w, y[nm], params[nm])
+
+    def step(i):
         ws = sets[i % n_sets]
-        for j, nm in enumerate(("gate", "up", "down", "head")):
-            w = heads[i % n_heads] if nm == "head" else ws[nm]
-            xin = x_f if nm == "down" else x_h
-            if ev is not None:
-                ev[j][0].record()
-            ops.quantized_matmul_ggml(xin, w, y[nm], params[nm])
-            if ev is not None:
-                ev[j][1].record()
+        for nm in ("gate", "up", "down", "head"):
+            one(nm, heads[i % n_heads] if nm == "head" else ws[nm])()
 
     # The same four products as a decode step dispatches them: gate and up read the same activations and
     # the reference encodes them without a barrier in between (gpu_ffn.rs:1236-1258), so they go to the
@@ -417,18 +479,16 @@ def main():
         ops.quantized_matmul_ggml(x_f, ws["down"], y["down"], params["down"])
         ops.quantized_matmul_ggml(x_h, heads[i % n_heads], y["head"], params["head"])
 
-    for i in range(a.warmup):
+    for i in range(max(a.warmup, 1)):
         step(i)
+        fused_step(i)
     torch.cuda.synchronize()
 
-    # K steps launched from the host, with a HIP event pair around every kernel (same stream): the
-    # per-kernel durations behind `roofline` and `kernels`.
-    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(4)]
-           for _ in range(a.steps)]
+    # K steps launched one kernel at a time from the host (Python + ctypes per launch).
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(a.steps):
-        step(a.warmup + i, evs[i])
+        step(a.warmup + i)
     torch.cuda.synchronize()
     el_host = time.perf_counter() - t0
     host = {"ms_per_step": round(el_host / a.steps * 1e3, 4), "GBps": round(step_bytes * a.steps / el_host / 1e9, 1),
@@ -438,22 +498,33 @@ def main():
     # (runs of consecutive steps over the rotated weight sets and heads), as a decode loop that records
     # its token step does; the host's per-launch cost (Python, ctypes) is then out of the way, like in
     # the other workloads.
-    elapsed = el_host
+    elapsed, step_us_events = el_host, None
     if not a.no_graph:
-        elapsed, _ = _timed_steps(a, fused_step, n_sets * n_heads)
+        elapsed, step_us_events = _timed_steps(a, fused_step, n_sets * n_heads)
 
-    names = ("gate", "up", "down", "head")
-    kern_us = {nm: sum(evs[i][j][0].elapsed_time(evs[i][j][1]) for i in range(a.steps)) * 1e3 / a.steps
-               for j, nm in enumerate(names)}
-    kernels = {nm: {"us": round(kern_us[nm], 3), "bytes": nbytes[nm],
-                    "GBps": round(nbytes[nm] / kern_us[nm] / 1e3, 1),
-                    "frac_hbm_peak": round(nbytes[nm] / kern_us[nm] / 1e3 / HBM_PEAK_GBS, 4)} for nm in names}
-    q4_bytes = nbytes["gate"] + nbytes["up"] + nbytes["down"]
-    q4_us = kern_us["gate"] + kern_us["up"] + kern_us["down"]
+    # Per-kernel durations behind `roofline` and `kernels`: HIP events around back-to-back launches of ONE kernel
+    # over distinct matrices (every set's gate and up for the 12288 x 4096 shape: 2 * n_sets * 28 MB, the sets'
+    # down matrices, the two heads twice), see _launch_us.
+    kern_us = {
+        "gate_up_12288x4096": _launch_us([one(nm, ws[nm]) for ws in sets for nm in ("gate", "up")] * 4),
+        "down_4096x12288": _launch_us([one("down", ws["down"]) for ws in sets] * 8),
+        "head_151936x4096": _launch_us([one("head", h) for h in heads] * 8),
+        "gate_and_up_one_launch": _launch_us([
+            (lambda ws=ws: ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x_h, ws["gate"], y["gate"], 1, F, H),
+                                                            ops.QmatmulJob(x_h, ws["up"], y["up"], 1, F, H)], HQ_Q4_K))
+            for ws in sets] * 8),
+    }
+    kbytes = {"gate_up_12288x4096": nbytes["gate"], "down_4096x12288": nbytes["down"], "head_151936x4096": nbytes["head"],
+              "gate_and_up_one_launch": nbytes["gate"] + nbytes["up"]}
+    kernels = {nm: {"us": round(kern_us[nm], 3), "bytes": kbytes[nm], "GBps": round(kbytes[nm] / kern_us[nm] / 1e3, 1),
+                    "frac_hbm_peak": round(kbytes[nm] / kern_us[nm] / 1e3 / HBM_PEAK_GBS, 4)} for nm in kern_us}
+    q4_bytes = 2 * nbytes["gate"] + nbytes["down"]
+    q4_us = 2 * kern_us["gate_up_12288x4096"] + kern_us["down_4096x12288"]
 
     value = step_bytes * a.steps / elapsed / 1e9
-    head_gbs = nbytes["head"] / kern_us["head"] / 1e3
-    out = {
+    head_us = kern_us["head_151936x4096"]
+    head_gbs = nbytes["head"] / head_us / 1e3
+    return {
         "metric": "Q4_K/Q6_K GEMV eff. GB/s (% HBM peak)",
         "value": round(value, 1),
         "unit": "GB/s",
@@ -471,17 +542,17 @@ def main():
                                + ("the four GEMVs launched one by one from the host" if a.no_graph else
                                   "gate + up in one batched launch, down, head = 3 launches replayed as a HIP graph"),
                    "bytes_per_step": step_bytes, "weight_sets": n_sets, "head_copies": n_heads,
-                   "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+                   "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                   "step_us_by_hip_events": None if step_us_events is None else round(step_us_events, 2)},
         "roofline": {"bound": "hbm", "kernel": "gemv Q6_K head 151936x4096", "achieved": round(head_gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head_gbs / HBM_PEAK_GBS, 4),
                      "traffic": PMC_TRAFFIC_BYTES["gemv_head_q6_k_151936x4096"],
-                     "us_per_launch": round(kern_us["head"], 3), "bytes_per_launch": nbytes["head"]},
+                     "traffic_source": "recorded: rocprofv3 --pmc runs of this file, profiles/gemv_decode_config2_pmc_traffic.md",
+                     "us_per_launch": round(head_us, 3), "bytes_per_launch": nbytes["head"]},
         "kernels": kernels,
         "host_launched": host,
         "q4_k_gemv": {"GBps": round(q4_bytes / q4_us / 1e3, 1), "frac_hbm_peak": round(q4_bytes / q4_us / 1e3 / HBM_PEAK_GBS, 4)},
     }
-    out["cpu_baseline"] = None if a.no_cpu_baseline else cpu_baseline()
-    print(json.dumps(out))
 
 
 if __name__ == "__main__":

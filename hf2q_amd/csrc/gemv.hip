@@ -39,6 +39,7 @@ namespace hq {
 namespace {
 
 constexpr uint32_t M4 = 0x000f000fu, M2 = 0x00300030u, M1 = 0x00100010u, MAGIC = 0x43004300u;
+constexpr uint32_t N4 = 0x0f0f0f0fu, N2 = 0x30303030u;  // the Q6_K kernels work on four bytes at a time
 // Types whose block is one lane's piece of 32 weights (the K-quants give a lane 64 of a super-block's 256).
 template <int TYPE>
 constexpr bool kBlock32 = TYPE == HQ_Q8_0 || TYPE == HQ_Q4_0;
@@ -161,20 +162,28 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q5_K>& p, int c, const 
     return acc;
 }
 
+// Q6_K: four 6-bit values at a time as the bytes of one word (nibbles of ql, two-bit fields of qh; n4 = 0x0f0f0f0f and
+// n2 = 0x30303030 arrive in the mask registers), then two byte permutes put bytes (0, 2) and (1, 3) under the high
+// byte 0x43 of `magic`: bf16 128 + q, the pair order of the staged activations.
 __device__ __forceinline__ float dot_pair(const Piece<HQ_Q6_K>& p, int c, const uint32_t* xp, const float* sx,
-                                          uint32_t m4, uint32_t m2, uint32_t magic) {
+                                          uint32_t n4, uint32_t n2, uint32_t magic) {
     float r0 = 0.f, r1 = 0.f, r2 = 0.f, r3 = 0.f;
+    constexpr uint32_t SEL02 = 0x07020500u, SEL13 = 0x07030501u;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t a = word(p.qa, j), b = word(p.qb, j), v = word(p.qh, j);
-        r0 = dot2_bf16(and_or((v << 4), m2, (a & m4) | magic), xp[2 * j], r0);
-        r0 = dot2_bf16(and_or((v >> 4), m2, ((a >> 8) & m4) | magic), xp[2 * j + 1], r0);
-        r1 = dot2_bf16(and_or((v << 2), m2, (b & m4) | magic), xp[8 + 2 * j], r1);
-        r1 = dot2_bf16(and_or((v >> 6), m2, ((b >> 8) & m4) | magic), xp[8 + 2 * j + 1], r1);
-        r2 = dot2_bf16(and_or(v, m2, ((a >> 4) & m4) | magic), xp[16 + 2 * j], r2);
-        r2 = dot2_bf16(and_or((v >> 8), m2, ((a >> 12) & m4) | magic), xp[16 + 2 * j + 1], r2);
-        r3 = dot2_bf16(and_or((v >> 2), m2, ((b >> 4) & m4) | magic), xp[24 + 2 * j], r3);
-        r3 = dot2_bf16(and_or((v >> 10), m2, ((b >> 12) & m4) | magic), xp[24 + 2 * j + 1], r3);
+        const uint32_t q0 = and_or(v << 4, n2, a & n4);
+        const uint32_t q1 = and_or(v << 2, n2, b & n4);
+        const uint32_t q2 = and_or(v, n2, (a >> 4) & n4);
+        const uint32_t q3 = and_or(v >> 2, n2, (b >> 4) & n4);
+        r0 = dot2_bf16(__builtin_amdgcn_perm(magic, q0, SEL02), xp[2 * j], r0);
+        r0 = dot2_bf16(__builtin_amdgcn_perm(magic, q0, SEL13), xp[2 * j + 1], r0);
+        r1 = dot2_bf16(__builtin_amdgcn_perm(magic, q1, SEL02), xp[8 + 2 * j], r1);
+        r1 = dot2_bf16(__builtin_amdgcn_perm(magic, q1, SEL13), xp[8 + 2 * j + 1], r1);
+        r2 = dot2_bf16(__builtin_amdgcn_perm(magic, q2, SEL02), xp[16 + 2 * j], r2);
+        r2 = dot2_bf16(__builtin_amdgcn_perm(magic, q2, SEL13), xp[16 + 2 * j + 1], r2);
+        r3 = dot2_bf16(__builtin_amdgcn_perm(magic, q3, SEL02), xp[24 + 2 * j], r3);
+        r3 = dot2_bf16(__builtin_amdgcn_perm(magic, q3, SEL13), xp[24 + 2 * j + 1], r3);
     }
     // scale bytes lr, lr+2, lr+4, lr+6 of this half's eight; values hold 128 + q with q in 0..63
     // and the format's own -32, hence the 160.
@@ -855,6 +864,7 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     }
 }
 
+
 // Whether the streaming form takes (type, k, rows): K-quants, whole 4096-element steps, enough rows to occupy the waves.
 template <int TYPE>
 constexpr bool kStreamType = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K;
@@ -914,7 +924,7 @@ int plan_job(const GemvArgs& a, KArgs* ka, size_t* lds, uint64_t* slots) {
     constexpr bool PAIR = X_BF16 && !kBlock32<TYPE>;
     constexpr int EPL = Lane<TYPE>::kElems;
     if (a.x2 && X_BF16) return fail(HQ_ERR_UNSUPPORTED, "gemv: the fused SwiGLU form takes f32 activations");
-    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.route_logits, a.route_ids, a.route_w, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, M4, TYPE == HQ_Q5_K ? M1 : M2, MAGIC};
+    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.route_logits, a.route_ids, a.route_w, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
     const uint32_t pieces = a.k / EPL;
     // L = largest power of two <= 64 that divides the pieces of a row
     uint32_t log_l = 0;
@@ -942,7 +952,7 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     if (int rc = cu_count(&cus)) return rc;
     if constexpr (X_BF16 && kStreamType<TYPE>) {
         if (a.pairs == 1 && !a.x2 && !a.ids && !a.route_logits && stream_takes<TYPE>(a.n, a.k, cus))
-            return launch_stream<TYPE>(s, SArgs{a.x, a.w, a.w, a.y, a.y, a.n, a.n, a.k, M4, TYPE == HQ_Q5_K ? M1 : M2, MAGIC}, cus);
+            return launch_stream<TYPE>(s, SArgs{a.x, a.w, a.w, a.y, a.y, a.n, a.n, a.k, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC}, cus);
     }
     // Dense matrices with many tasks per wave: the queue kernel.
     if (a.pairs == 1 && !a.x2 && !a.ids && !a.route_logits &&
@@ -990,7 +1000,7 @@ int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
         const GemvArgs &j0 = jobs[0], &j1 = jobs[1];
         auto plain = [](const GemvArgs& j) { return j.pairs == 1 && !j.x2 && !j.ids && !j.route_logits; };
         if (n_jobs == 2 && plain(j0) && plain(j1) && j0.x == j1.x && j0.k == j1.k && stream_takes<TYPE>(j0.n + j1.n, j0.k, cus))
-            return launch_stream<TYPE>(s, SArgs{j0.x, j0.w, j1.w, j0.y, j1.y, j0.n, j0.n + j1.n, j0.k, M4, TYPE == HQ_Q5_K ? M1 : M2, MAGIC}, cus);
+            return launch_stream<TYPE>(s, SArgs{j0.x, j0.w, j1.w, j0.y, j1.y, j0.n, j0.n + j1.n, j0.k, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC}, cus);
     }
     const uint64_t per_simd = slots / (4ull * cus);
     if (per_simd >= 8) return launch_j<TYPE, X_BF16, PAIR, 4, 4>(s, js, n_jobs, lds);
