@@ -455,8 +455,8 @@ static int flash_attn_vec_tq(const char* fn, bool undo_rotation, void* stream, c
     if (!q || !k_codes || !k_norms || !v_codes || !v_norms || !out || !tmp)
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
     if (!is_aligned(q, 16) || !is_aligned(out, 16) || !is_aligned(k_codes, 16) || !is_aligned(v_codes, 16) ||
-        !is_aligned(tmp, 4))
-        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: q / out / codes need 16-byte alignment", fn);
+        !is_aligned(tmp, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: q / out / codes / tmp need 16-byte alignment", fn);
     // 5- and 6-bit caches store one code per byte like the 8-bit one and differ only in the centroid
     // table, which the caller supplies (its first 2^bits entries); the linear int8 map is 8-bit only.
     if (p->codebook_bits != 8 && !lut256)
@@ -480,6 +480,48 @@ int hq_flash_attn_vec_tq_undo(void* stream, const float* q, const uint8_t* k_cod
                               void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p) {
     return flash_attn_vec_tq("hq_flash_attn_vec_tq_undo", true, stream, q, k_codes, k_norms, v_codes, v_norms, lut256, out,
                              tmp, tmp_bytes, p);
+}
+
+// Scratch of hq_flash_attn_vec_tq_static: one copy per GPU, held until the process ends.  In host code the array's
+// name is only a handle for hipGetSymbolAddress; the address the kernels get is looked up once per device.
+static __device__ __align__(256) unsigned char scratch[HQ_TQ_STATIC_TMP_BYTES];
+
+static int static_scratch(void** out) {
+    static std::mutex mu;
+    static void* ptr[64] = {};
+    int dev = 0;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (dev < 0 || dev >= 64) return fail(HQ_ERR_UNSUPPORTED, "hq_flash_attn_vec_tq_static: device ordinal %d (0..63)", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void* p = nullptr;
+        if (int rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(static attention scratch)"))
+            return rc;
+        if (!p) return fail(HQ_ERR_HIP, "hq_flash_attn_vec_tq_static: no address for the static scratch");
+        ptr[dev] = p;
+    }
+    *out = ptr[dev];
+    return HQ_OK;
+}
+
+int hq_flash_attn_vec_tq_static(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
+                                const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
+                                const hq_tq_attn_params* p, int undo_rotation) {
+    const char* fn = "hq_flash_attn_vec_tq_static";
+    if (!p) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null params", fn);
+    // sizes first: the scratch is fixed, so the shape check does not depend on the other arguments being sane
+    if ((p->head_dim == 256 || p->head_dim == 512) && p->kv_seq_len != 0) {
+        const size_t need = tq_attn_tmp_bytes(p->num_heads, p->head_dim, p->kv_seq_len);
+        if (need > HQ_TQ_STATIC_TMP_BYTES)
+            return fail(HQ_ERR_INVALID_ARGUMENT,
+                        "%s: %u heads x head_dim %u over %u positions need %zu bytes of scratch, the static buffer holds %zu; "
+                        "use hq_flash_attn_vec_tq with caller scratch",
+                        fn, p->num_heads, p->head_dim, p->kv_seq_len, need, (size_t)HQ_TQ_STATIC_TMP_BYTES);
+    }
+    void* tmp = nullptr;
+    if (int rc = static_scratch(&tmp)) return rc;
+    return flash_attn_vec_tq(fn, undo_rotation != 0, stream, q, k_codes, k_norms, v_codes, v_norms, lut256, out, tmp,
+                             HQ_TQ_STATIC_TMP_BYTES, p);
 }
 
 int hq_dense_gemv_bf16(void* stream, const void* x, hq_act_dtype xdt, const void* w_bf16, float* y, uint32_t m,

@@ -73,6 +73,7 @@ SIGNATURES = {
     "hq_flash_attn_vec_tq": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "hq_flash_attn_vec_tq_undo": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "hq_flash_attn_vec_tq_tmp_bytes": (_sz, [_u32, _u32, _u32]),
+    "hq_flash_attn_vec_tq_static": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32]),
     "hq_tqp_indices_bytes": (_sz, [_vp]),
     "hq_tqp_norms_bytes": (_sz, [_vp]),
     "hq_tqp_total_bytes": (_sz, [_vp]),

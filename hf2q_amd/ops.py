@@ -391,6 +391,24 @@ def flash_attn_vec_tq_hb(q: torch.Tensor, k_packed: torch.Tensor, k_norms: torch
         _dev(tmp, "tmp"), tmp.numel() * tmp.element_size(), _ct.byref(p)))
 
 
+def flash_attn_vec_tq_hb_static(q: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor, v_packed: torch.Tensor,
+                                v_norms: torch.Tensor, out: torch.Tensor, params: FlashAttnVecTqHbParams,
+                                lut256: torch.Tensor | None = None, undo_rotation: bool = False) -> None:
+    """flash_attn_vec_tq_hb without the tmp argument: the partial results go to the library's static device buffer
+    (hq_flash_attn_vec_tq_static; nothing is allocated, shapes beyond the buffer are rejected)."""
+    if q.dtype != torch.float32 or out.dtype != torch.float32:
+        raise TypeError("q and out must be float32")
+    p = _l.TqAttnParams(params.num_heads, params.num_kv_heads, params.head_dim, params.kv_seq_len,
+                        params.kv_capacity, params.scale, params.mask_type, params.sliding_window, params.softcap,
+                        params.ring_start, params.scale_factor_d512, params.codebook_bits, params.fuse_fwht_pre,
+                        params.nsg)
+    import ctypes as _ct
+    _l.check(_l.load().hq_flash_attn_vec_tq_static(
+        _stream(), _dev(q, "q"), _dev(k_packed, "k_packed"), _dev(k_norms, "k_norms"), _dev(v_packed, "v_packed"),
+        _dev(v_norms, "v_norms"), _dev(lut256, "lut256") if lut256 is not None else None, _dev(out, "out"),
+        _ct.byref(p), 1 if undo_rotation else 0))
+
+
 def tq_dequantize_hb_kv_seq(packed: torch.Tensor, norms: torch.Tensor, dst: torch.Tensor, n_kv_heads: int, head_dim: int,
                             cache_capacity: int, start_pos: int, n_tokens: int, scale_factor_d512: float = 1.0,
                             codebook_bits: int = 8, lut256: torch.Tensor | None = None, unrotate: bool = False) -> None:

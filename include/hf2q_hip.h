@@ -274,7 +274,7 @@ typedef struct {
  * head_dim 512: codes are [n_kv_heads, capacity, 512], norms [n_kv_heads, capacity, 2] (one per
  * 256-block, kv_cache.rs:2010-2012), table values are also divided by scale_factor_d512, and every
  * 256-block of q / out is rotated on its own.
- * `tmp` is device scratch of hq_flash_attn_vec_tq_tmp_bytes() bytes.  Rejects kv_seq_len == 0,
+ * `tmp` is device scratch of hq_flash_attn_vec_tq_tmp_bytes() bytes, 16-byte aligned.  Rejects kv_seq_len == 0,
  * kv_capacity < kv_seq_len (kv_cache.rs:331-333), head_dim not in {256, 512}, codebook_bits not in
  * {5, 6, 8}; codebook_bits 5 / 6 without a centroid table are reported as unsupported. */
 HQ_API int hq_flash_attn_vec_tq(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
@@ -288,6 +288,19 @@ HQ_API int hq_flash_attn_vec_tq_undo(void* stream, const float* q, const uint8_t
                               const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
                               void* tmp, size_t tmp_bytes, const hq_tq_attn_params* p);
 HQ_API size_t hq_flash_attn_vec_tq_tmp_bytes(uint32_t num_heads, uint32_t head_dim, uint32_t kv_seq_len);
+/* The same attention (undo_rotation != 0: hq_flash_attn_vec_tq_undo) without a scratch argument: the partial
+ * results live in a buffer of HQ_TQ_STATIC_TMP_BYTES that is part of the library's device image (one copy per GPU,
+ * held until the process ends).  It has no counterpart in the reference.  It is for callers that cannot allocate:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc; nothing is allocated or freed
+ * here.  Shapes whose hq_flash_attn_vec_tq_tmp_bytes() exceeds the buffer are rejected with
+ * HQ_ERR_INVALID_ARGUMENT (16 heads x head_dim 256 at any context fit).  Every call on a GPU uses that GPU's one
+ * buffer: calls that overlap on one GPU (two streams) race, and nothing of it needs to be cleared between calls.  The
+ * first call on a device looks the buffer's address up (hipGetSymbolAddress); make that call outside stream
+ * capture. */
+#define HQ_TQ_STATIC_TMP_BYTES (4u << 20)
+HQ_API int hq_flash_attn_vec_tq_static(void* stream, const float* q, const uint8_t* k_codes, const float* k_norms,
+                                const uint8_t* v_codes, const float* v_norms, const float* lut256, float* out,
+                                const hq_tq_attn_params* p, int undo_rotation);
 
 /* ---- TQ block envelope (spilled K / V blocks) ---- */
 
