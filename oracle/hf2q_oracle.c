@@ -1084,7 +1084,8 @@ int hq_oracle_tq_dequantize(const uint8_t *codes, const float *norms, const floa
  * flash_attn_vec_tq_hb, forward_mlx.rs:4687-4742, kv_cache.rs:335-388):
  * out[h] = softmax(scale * q[h] . K[kv(h)]^T [softcapped, masked]) . V[kv(h)],
  * kv(h) = h / (num_heads/num_kv_heads) (kv_cache.rs:4091-4096).  Logical
- * position i lives in physical slot (ring_start + i) % kv_capacity; mask 2
+ * position i lives in physical slot (ring_start + i) % kv_capacity (the inverse of
+ * forward_mlx.rs:7299, logical = (k_pos - ring_start + cap) % cap); mask 2
  * keeps only the last `sliding_window` logical positions; masks 0 and 1 keep
  * all kv_seq_len positions for a single query at the end of the sequence. */
 int hq_oracle_tq_attention(const float *q, const uint8_t *k_codes, const float *k_norms,

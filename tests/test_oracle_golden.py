@@ -440,6 +440,105 @@ def test_tq_attention_matches_numpy_softmax(oracle):
     assert np.sqrt(((o - exact) ** 2).sum() / (exact ** 2).sum()) < 0.02
 
 
+def _np_attention(q, K, V, scale, group):
+    """Textbook softmax attention in float64 over explicit K, V [n_kv, n, d]."""
+    out = np.zeros((q.shape[0], q.shape[1]))
+    for h in range(q.shape[0]):
+        s = (K[h // group] @ q[h].astype(np.float64)) * scale
+        p = np.exp(s - s.max())
+        p /= p.sum()
+        out[h] = p @ V[h // group]
+    return out
+
+
+def test_tq_dequantize_is_code_times_norm(oracle):
+    """hq_oracle_tq_dequantize against codes.view(int8) * norms in numpy: a window that does not start at 0, and
+    head_dim 512 with a norm of its own per 256-block (kv_cache.rs:2010-2012)."""
+    rng = np.random.default_rng(41)
+    for d in (256, 512):
+        nkv, cap, start, n = 3, 50, 17, 21
+        codes = rng.integers(0, 256, (nkv, cap, d), dtype=np.uint8)
+        norms = rng.uniform(0.01, 2.0, (nkv, cap, d // 256)).astype(np.float32)
+        got = oracle.tq_dequantize(codes, norms, None, nkv, d, cap, start, n)
+        want = (codes.view(np.int8).astype(np.float64).reshape(nkv, cap, d // 256, 256)
+                * norms.astype(np.float64)[..., None]).reshape(nkv, cap, d)[:, start:start + n]
+        assert got.shape == (nkv, n, d)
+        assert np.array_equal(got, want.astype(np.float32))  # int8 * f32 has at most 31 significant bits: one rounding
+        assert not np.array_equal(got[:, 0], want[:, 1].astype(np.float32))  # the window really starts at `start`
+        # table form: lut[code] * norm / 16 / scale_factor (scale_factor only at head_dim 512)
+        lut = rng.standard_normal(256).astype(np.float32)
+        sf = 1.7
+        got = oracle.tq_dequantize(codes, norms, lut, nkv, d, cap, start, n, scale_factor_d512=sf)
+        div = 16.0 * (np.float64(np.float32(sf)) if d == 512 else 1.0)
+        want = (lut.astype(np.float64)[codes].reshape(nkv, cap, d // 256, 256) * norms.astype(np.float64)[..., None]
+                / div).reshape(nkv, cap, d)[:, start:start + n]
+        assert np.allclose(got, want, rtol=1e-6, atol=0)
+    with pytest.raises(ValueError):   # kv_cache.rs:427-428: the window may not run past the capacity
+        oracle.tq_dequantize(codes, norms, None, 3, 512, 50, 40, 11)
+
+
+def test_tq_attention_ring_buffer_matches_rolled_cache(oracle):
+    """ring_start != 0: logical position i sits in slot (ring_start + i) % capacity, the inverse of
+    forward_mlx.rs:7299 (logical = (k_pos - ring_start + cap) % cap).  Checked against numpy attention over the
+    cache rolled back explicitly, for a wrapped window, with and without a sliding window."""
+    rng = np.random.default_rng(43)
+    nh, nkv, d, cap, n, ring = 4, 2, 256, 24, 20, 9   # slots 9..23, 0..4
+    kc = rng.integers(0, 256, (nkv, cap, d), dtype=np.uint8)
+    vc = rng.integers(0, 256, (nkv, cap, d), dtype=np.uint8)
+    kn = rng.uniform(0.001, 0.02, (nkv, cap, 1)).astype(np.float32)
+    vn = rng.uniform(0.001, 0.02, (nkv, cap, 1)).astype(np.float32)
+    q = rng.standard_normal((nh, d)).astype(np.float32)
+    order = [(ring + i) % cap for i in range(n)]      # physical slot of logical position i
+    K = (kc.view(np.int8).astype(np.float64) * kn.astype(np.float64))[:, order]
+    V = (vc.view(np.int8).astype(np.float64) * vn.astype(np.float64))[:, order]
+    got = oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, d, n, cap, 0.0625, ring_start=ring)
+    assert np.allclose(got, _np_attention(q, K, V, 0.0625, 2), rtol=1e-10, atol=1e-13)
+    # the unrolled reading (ring_start ignored) is a different answer, so the check above can fail
+    assert not np.allclose(got, oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, d, n, cap, 0.0625), rtol=1e-3)
+    got = oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, d, n, cap, 0.0625, mask_type=2, sliding_window=7,
+                              ring_start=ring)
+    assert np.allclose(got, _np_attention(q, K[:, n - 7:], V[:, n - 7:], 0.0625, 2), rtol=1e-10, atol=1e-13)
+    # mask types 0 and 1 see the same positions for the single query at the end of the sequence
+    a = oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, d, n, cap, 0.0625, mask_type=1, ring_start=ring)
+    b = oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, d, n, cap, 0.0625, mask_type=0, ring_start=ring)
+    assert np.array_equal(a, b)
+
+
+def test_tq_attention_head_dim_512_two_norms_and_table_scale(oracle):
+    """head_dim 512: every row carries two norms, one per 256-block (kv_cache.rs:2010-2012), and the table form
+    divides by scale_factor_d512.  Against numpy over the explicitly dequantised cache; rows whose two norms differ
+    by orders of magnitude make a swapped or shared norm visible."""
+    rng = np.random.default_rng(47)
+    nh, nkv, d, cap, n = 4, 2, 512, 16, 13
+    kc = rng.integers(0, 256, (nkv, cap, d), dtype=np.uint8)
+    vc = rng.integers(0, 256, (nkv, cap, d), dtype=np.uint8)
+    kn = (rng.uniform(0.5, 1.5, (nkv, cap, 2)) * np.array([1e-3, 3e-2])).astype(np.float32)
+    vn = (rng.uniform(0.5, 1.5, (nkv, cap, 2)) * np.array([4e-2, 2e-3])).astype(np.float32)
+    q = rng.standard_normal((nh, d)).astype(np.float32)
+
+    def deq(c, nrm, lut=None, sf=1.0):
+        vals = c.view(np.int8).astype(np.float64) if lut is None else lut.astype(np.float64)[c] / 16.0 / sf
+        return (vals.reshape(nkv, cap, 2, 256) * nrm.astype(np.float64)[..., None]).reshape(nkv, cap, d)[:, :n]
+
+    got = oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, d, n, cap, 0.046875)
+    assert np.allclose(got, _np_attention(q, deq(kc, kn), deq(vc, vn), 0.046875, 2), rtol=1e-10, atol=1e-13)
+    swapped = _np_attention(q, deq(kc, kn[..., ::-1]), deq(vc, vn), 0.046875, 2)
+    assert not np.allclose(got, swapped, rtol=1e-3)
+    lut = (rng.standard_normal(256) * 40).astype(np.float32)
+    for sf in (1.0, 2.5):
+        got = oracle.tq_attention(q, kc, kn, vc, vn, lut, nh, nkv, d, n, cap, 0.046875, scale_factor_d512=sf)
+        want = _np_attention(q, deq(kc, kn, lut, np.float64(np.float32(sf))), deq(vc, vn, lut, np.float64(np.float32(sf))),
+                             0.046875, 2)
+        assert np.allclose(got, want, rtol=1e-9, atol=1e-13)
+    # at head_dim 256 the scale factor is not applied
+    q256 = q[:, :256].copy()
+    a = oracle.tq_attention(q256, kc[..., :256].copy(), kn[..., :1].copy(), vc[..., :256].copy(), vn[..., :1].copy(), lut,
+                            nh, nkv, 256, n, cap, 0.046875, scale_factor_d512=2.5)
+    b = oracle.tq_attention(q256, kc[..., :256].copy(), kn[..., :1].copy(), vc[..., :256].copy(), vn[..., :1].copy(), lut,
+                            nh, nkv, 256, n, cap, 0.046875, scale_factor_d512=1.0)
+    assert np.array_equal(a, b)
+
+
 def test_tq_attention_rejects_bad_shapes(oracle):
     z8, zf = np.zeros((1, 4, 256), np.uint8), np.zeros((1, 4, 1), np.float32)
     q = np.zeros((2, 256), np.float32)
