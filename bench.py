@@ -254,10 +254,9 @@ def bench_moe_decode(a, tokens=None):
         "metric": "MoE decode tok/s (FFN-only, 40 MoE layers)", "value": round(T / (40 * elapsed / a.steps), 1),
         "unit": "tok/s", "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "bf16",
         "config": {"workload": f"moe_decode: hidden 2048, 256 experts x inter 512 Q4_K, shared expert, top-8, "
-                               f"batch {T}, bf16 activations (BASELINE config 3); one step = one MoE FFN layer "
-                               f"(router + shared logit, top-k, gate/up of routed and shared experts, both SwiGLU-fused "
-                               f"down projections, reduce = {4 if T <= 4 else 5} launches"
-                               f"{': the gate / up launch works the top-k out itself' if T <= 4 else ''}), "
+                               f"batch {T}, bf16 activations (BASELINE config 3); one step = one MoE FFN layer = ONE launch "
+                               f"(hq_moe_ffn_decode: router + shared logit, top-k, gate / up with SwiGLU, down, weighted "
+                               f"sum, handed between workgroups inside the launch), "
                                f"{'launched from the host' if a.no_graph else 'replayed as a HIP graph'}",
                    "distinct_experts_per_layer": round(u, 1), "bytes_per_layer": int(step_bytes),
                    "layers_rotated": n_layers},

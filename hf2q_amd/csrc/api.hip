@@ -378,6 +378,64 @@ int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_j
     return launch_gemv_jobs((hipStream_t)stream, ga, live, xdt, t);
 }
 
+size_t hq_moe_ffn_decode_scratch_bytes(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k, uint32_t inter,
+                                       uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt) {
+    if (!moe_fused_supported(n_tokens, hidden, n_experts, top_k, inter, shared_inter, t, xdt)) return 0;
+    return moe_fused_scratch_bytes(n_tokens, n_experts, top_k);
+}
+
+int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* l, const void* x, hq_act_dtype xdt, const float* residual,
+                      float* out, uint32_t n_tokens, void* scratch, size_t scratch_bytes, uint32_t* route_ids,
+                      float* route_weights) {
+    const char* fn = "hq_moe_ffn_decode";
+    if (!l) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null layer", fn);
+    if (n_tokens == 0) return HQ_OK;
+    if (!moe_fused_supported(n_tokens, l->hidden, l->n_experts, l->top_k, l->inter, l->shared_inter, l->ggml_type, xdt))
+        return fail(HQ_ERR_UNSUPPORTED,
+                    "%s: takes 1..8 tokens of bf16 activations, Q4_K experts, hidden 2048, expert and shared FFN width 512, "
+                    "<= 256 experts (got %u tokens, dtype %d, type %d, hidden %u, inter %u / %u, %u experts, top-%u); "
+                    "run the block as separate dispatches",
+                    fn, n_tokens, (int)xdt, (int)l->ggml_type, l->hidden, l->inter, l->shared_inter, l->n_experts, l->top_k);
+    if (!x || !out || !scratch || !l->router || !l->expert_gate || !l->expert_up || !l->expert_down || !l->shared_gate ||
+        !l->shared_up || !l->shared_down)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (!route_ids != !route_weights) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: route_ids and route_weights go together", fn);
+    const void* al16[] = {x, out, l->router, l->shared_gate_logit, l->expert_gate, l->expert_up, l->expert_down,
+                          l->shared_gate, l->shared_up, l->shared_down, residual};
+    for (const void* p : al16)
+        if (!is_aligned(p, 16)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: every buffer must be 16-byte aligned", fn);
+    if (!is_aligned(scratch, 256)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch must be 256-byte aligned", fn);
+    const size_t need = moe_fused_scratch_bytes(n_tokens, l->n_experts, l->top_k);
+    if (scratch_bytes < need) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch of %zu bytes, %zu needed", fn, scratch_bytes, need);
+    const uint64_t gu_bytes = (uint64_t)l->inter * (l->hidden / 256) * Q4K_BYTES, d_bytes = (uint64_t)l->hidden * (l->inter / 256) * Q4K_BYTES;
+    if (l->expert_stride_gate_up < gu_bytes || l->expert_stride_gate_up % 16 || l->expert_stride_down < d_bytes || l->expert_stride_down % 16)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: expert strides %llu / %llu (one expert is %llu / %llu bytes)", fn,
+                    (unsigned long long)l->expert_stride_gate_up, (unsigned long long)l->expert_stride_down,
+                    (unsigned long long)gu_bytes, (unsigned long long)d_bytes);
+    MoeFusedArgs a{};
+    a.x = x;
+    a.router = l->router;
+    a.shared_gate_logit = l->shared_gate_logit;
+    a.expert_gate = l->expert_gate;
+    a.expert_up = l->expert_up;
+    a.expert_down = l->expert_down;
+    a.shared_gate = l->shared_gate;
+    a.shared_up = l->shared_up;
+    a.shared_down = l->shared_down;
+    a.residual = residual;
+    a.out = out;
+    a.route_ids = route_ids;
+    a.route_weights = route_weights;
+    a.scratch = scratch;
+    a.n_tokens = n_tokens;
+    a.n_experts = l->n_experts;
+    a.top_k = l->top_k;
+    a.stride_gate_up = l->expert_stride_gate_up;
+    a.stride_down = l->expert_stride_down;
+    a.spin_limit = 0;
+    return launch_moe_fused((hipStream_t)stream, a);
+}
+
 static int check_fwht(const char* fn, const float* buf, uint32_t n_heads, uint32_t head_dim) {
     if (head_dim != 256 && head_dim != 512) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: head_dim %u (256 or 512)", fn, head_dim);
     if (n_heads && !buf) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);

@@ -92,6 +92,26 @@ int launch_silu_mul(hipStream_t s, const float* gate, const float* up, float* ou
 int launch_moe_weighted_reduce(hipStream_t s, const float* y, const float* w, const float* shared, const float* shared_logit,
                                const float* residual, float* out, uint32_t n_tokens, uint32_t top_k, uint32_t hidden);
 
+// The whole MoE FFN block of a decode step in one launch (moe_fused.hip).
+struct MoeFusedArgs {
+    const void* x;                  // [n_tokens, hidden] bf16
+    const void* router;             // [n_experts, hidden] bf16
+    const void* shared_gate_logit;  // [hidden] bf16 or nullptr
+    const void *expert_gate, *expert_up, *expert_down, *shared_gate, *shared_up, *shared_down;
+    const float* residual;          // nullptr or [n_tokens, hidden]
+    float* out;                     // [n_tokens, hidden]
+    uint32_t* route_ids;            // nullptr or out [n_tokens * top_k]
+    float* route_weights;
+    void* scratch;
+    uint32_t n_tokens, n_experts, top_k;
+    uint64_t stride_gate_up, stride_down;
+    uint32_t spin_limit;            // 0: default
+};
+bool moe_fused_supported(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k, uint32_t inter,
+                         uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt);
+size_t moe_fused_scratch_bytes(uint32_t n_tokens, uint32_t n_experts, uint32_t top_k);
+int launch_moe_fused(hipStream_t s, const MoeFusedArgs& a);
+
 // TurboQuant KV (tq.hip)
 int launch_fwht_sign(hipStream_t s, float* buf, uint32_t n_heads, uint32_t head_dim, bool undo);
 int launch_tq_encode(hipStream_t s, const float* src, uint8_t* codes, float* norms, uint32_t n_tokens,

@@ -1,0 +1,435 @@
+// The MoE FFN block of a decode step (1..8 tokens) as ONE launch: router and shared-gate logits, softmax / top-k,
+// gate and up projections of the routed and the shared expert with their SwiGLU, the down projections, and the
+// weighted reduction (+ sigmoid-gated shared expert, + residual).  build_moe_ffn_layer_gpu_q_into
+// (src/inference/models/qwen35/gpu_ffn.rs:2313-2802) encodes these as phases A-F of one command buffer;
+// moe_ffn_cpu_ref (src/inference/models/qwen35/ffn.rs:179-336) is the specification.
+//
+// As separate launches the block costs four to five launch latencies in series (each small kernel spends 3-4 us
+// before its first result whatever it computes).  Here one workgroup per CU walks the phases and hands results
+// to the other workgroups through memory:
+//   * every hand-over is a relaxed device-scope atomic store / load (write-through, cache-bypassing accesses) and no
+//     fence is ever executed: a device-scope release fence writes a whole L2 back on this multi-XCD part;
+//   * a consumer recognises fresh data by a TAG = (calls so far on this scratch) + 1: router logits and SwiGLU
+//     activations travel as 64-bit (tag, value) words, so a value and its freshness arrive in one store, no store has
+//     to be ordered behind another, and nothing has to be cleared between calls; workgroup 0 stores the new call count
+//     when it leaves (every workgroup has read the old one by then: workgroup 0 cannot get past the routing before
+//     all of them have delivered their logits);
+//   * the down projections are cut by output columns, not by expert: a workgroup computes its 8 .. 64 columns for every
+//     slot of a token and sums them itself, so the outputs never cross workgroups.
+// No workgroup ever waits for a later phase of another one, so the grid drains whatever the residency; the waits are
+// bounded all the same (spin_limit polls, then the error word of the scratch is set and the wave goes on).
+//
+// Row arithmetic is that of the separate dispatches — the same piece dot products, the same reduction order, the
+// same SwiGLU rounding, the same order of the weighted sum — so the block's output has the bits of
+// hq_dense_gemv_bf16_pair + hq_qmatmul_batch_ggml x 2 + hq_moe_weighted_reduce.
+//
+// Shapes: K-quant Q4_K experts, hidden = 2048 (32 lanes per gate / up row: a wave step is one gate row and the up row
+// of the same index), expert FFN = shared FFN = 512 (8 lanes per down row), <= 256 experts, bf16 activations.
+#include <math.h>
+
+#include "hq_internal.h"
+#include "moe_topk.h"
+#include "gemv_pieces.h"
+
+namespace hq {
+namespace {
+
+constexpr uint32_t FH = 2048, FI = 512;               // hidden, expert FFN width
+constexpr uint32_t ROWB_H = FH / 256 * Q4K_BYTES;     // bytes of a gate / up row
+constexpr uint32_t ROWB_I = FI / 256 * Q4K_BYTES;     // bytes of a down row
+constexpr uint32_t WAVES = 8, THREADS = 64 * WAVES;
+constexpr uint32_t MAX_T = 8;                         // tokens per call
+constexpr int RING = 4;                               // weight fetches a wave keeps in flight
+
+struct FusedArgs {
+    const uint16_t* x;       // [T][H] bf16
+    const uint16_t* router;  // [E][H] bf16
+    const uint16_t* sh_lw;   // [H] bf16 or null: shared-expert gate logit
+    const uint8_t *eg, *eu, *ed, *sg, *su, *sd;
+    const float* residual;
+    float* out;
+    uint32_t* route_ids;
+    float* route_w;
+    uint8_t* scratch;
+    uint32_t T, E, K;
+    uint64_t stride_gu, stride_d;
+    uint32_t m4, m2, magic, spin_limit;
+};
+
+// Scratch layout (byte offsets), the same on host and device: call counter and error word, then the two hand-over
+// areas, both of (tag << 32 | value bits) words.
+struct Layout {
+    uint32_t T, E, K;
+    __host__ __device__ uint32_t slots() const { return K + 1; }  // routed slots + the shared expert
+    __host__ __device__ size_t logits() const { return 64; }     // u64 [T][E + 1]
+    __host__ __device__ size_t act() const { return logits() + (size_t)T * (E + 1) * 8; }  // u64 [T][K + 1][I]
+    __host__ __device__ size_t total() const { return act() + (size_t)T * slots() * FI * 8; }
+};
+
+template <typename V>
+__device__ __forceinline__ void st_dev(V* p, V v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename V>
+__device__ __forceinline__ V ld_dev(const V* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The value of a (tag, value) word once its tag is `tag`; polls at most `limit` times, then reports through *err.
+__device__ __forceinline__ uint32_t wait_tagged(const uint64_t* p, uint32_t tag, uint32_t limit, uint32_t* err) {
+    uint64_t got = ld_dev(p);
+    for (uint32_t n = 0; (uint32_t)(got >> 32) != tag; ++n) {
+        if (n >= limit) {
+            st_dev(err, 1u);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+        got = ld_dev(p);
+    }
+    return (uint32_t)got;
+}
+
+__device__ __forceinline__ uint32_t swz8(uint32_t ch) { return ch ^ ((ch >> 4) & 7u); }
+
+__global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
+    extern __shared__ uint4 smem[];
+    const Layout L{a.T, a.E, a.K};
+    const uint32_t T = a.T, E = a.E, K = a.K, S = K + 1;
+    // LDS: [staged activations of all tokens | later: one token's SwiGLU activations of all slots] | logits | ids | weights | partials
+    uint4* lds_x = smem;                                                       // T * H/8 chunks (paired bf16 words)
+    float* lds_sx = reinterpret_cast<float*>(lds_x + (size_t)T * (FH / 8));    // T * H/16 per-16 sums
+    const uint32_t area = T * (FH / 8) * 16 + T * (FH / 16) * 4, act_bytes = S * (FI * 4 + FI / 16 * 4);
+    uint8_t* after = reinterpret_cast<uint8_t*>(smem) + (area > act_bytes ? area : act_bytes);
+    float4* lds_act = reinterpret_cast<float4*>(smem);                         // S * I floats (over the activations, after phase 2)
+    float* lds_as = reinterpret_cast<float*>(lds_act + (size_t)S * (FI / 4));  // S * I/16 sums
+    float* lds_lg = reinterpret_cast<float*>(after);                           // T * (E + 1)
+    uint32_t* lds_id = reinterpret_cast<uint32_t*>(lds_lg + (size_t)T * (E + 1));  // T * K
+    float* lds_w = reinterpret_cast<float*>(lds_id + (size_t)T * K);           // T * (K + 1): slot K = shared gate
+    float* lds_part = lds_w + (size_t)T * S;                                   // S * 64 down partials of one unit
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6, b = blockIdx.x, G = gridDim.x;
+    const uint32_t gw = b * WAVES + wv, NW = G * WAVES;  // this wave among all waves of the launch
+    uint32_t* s_epoch = reinterpret_cast<uint32_t*>(a.scratch);
+    uint32_t* s_err = s_epoch + 1;
+    uint64_t* s_lg = reinterpret_cast<uint64_t*>(a.scratch + L.logits());
+    uint64_t* s_act = reinterpret_cast<uint64_t*>(a.scratch + L.act());
+
+    const uint32_t tag = ld_dev(s_epoch) + 1u;
+    const uint64_t tag_hi = (uint64_t)tag << 32;
+
+    // the activations of all tokens, requested first and staged while the logits travel (the layout and sums of
+    // stage_store); 16 activations per thread and pass
+    constexpr uint32_t XPASS = (MAX_T * (FH / 16) + THREADS - 1) / THREADS;
+    XRaw<true> xraw[XPASS];
+#pragma unroll
+    for (uint32_t ps = 0; ps < XPASS; ++ps) {
+        const uint32_t i = tid + ps * THREADS;
+        if (i < T * (FH / 16)) xraw[ps].fetch(a.x + (size_t)(i / (FH / 16)) * FH, i % (FH / 16));
+    }
+
+    // ---- phase 1: router logits and the shared-gate logit, one (row, token) per wave and turn, with the arithmetic of
+    // dense_gemv_bf16_kernel.  Every workgroup has a task here, which is what lets workgroup 0 bump the call counter at
+    // its end (see the header comment). ----
+    const uint32_t n_rows = E + (a.sh_lw ? 1u : 0u);
+    for (uint32_t q = b + G * wv; q < n_rows * T; q += NW) {  // task q belongs to workgroup q % G (G <= n_rows: every workgroup has one)
+        const uint32_t r = q / T, t = q % T;
+        const uint4* wr = reinterpret_cast<const uint4*>(r < E ? a.router + (size_t)r * FH : a.sh_lw);
+        const uint4* xr = reinterpret_cast<const uint4*>(a.x + (size_t)t * FH);
+        uint4 wq[FH / 8 / 64], xq[FH / 8 / 64];
+#pragma unroll
+        for (uint32_t c = 0; c < FH / 8 / 64; ++c) {
+            wq[c] = wr[lane + 64 * c];
+            xq[c] = xr[lane + 64 * c];
+        }
+        float acc = 0.f;
+#pragma unroll
+        for (uint32_t c = 0; c < FH / 8 / 64; ++c) {
+            const uint32_t ww[4] = {wq[c].x, wq[c].y, wq[c].z, wq[c].w}, tw[4] = {xq[c].x, xq[c].y, xq[c].z, xq[c].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc = fmaf(bf16_bits_to_f32(ww[i] & 0xffffu), bf16_bits_to_f32(tw[i] & 0xffffu), acc);
+                acc = fmaf(bf16_bits_to_f32(ww[i] >> 16), bf16_bits_to_f32(tw[i] >> 16), acc);
+            }
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) st_dev(&s_lg[(size_t)t * (E + 1) + r], tag_hi | __float_as_uint(acc));
+    }
+
+    // ---- while the logits travel: the staged activations go to LDS ----
+#pragma unroll
+    for (uint32_t ps = 0; ps < XPASS; ++ps) {
+        const uint32_t i = tid + ps * THREADS;
+        if (i < T * (FH / 16)) {
+            const uint32_t t = i / (FH / 16), j = i % (FH / 16);
+            const uint4 p = xraw[ps].r[0], q = xraw[ps].r[1];
+            const uint32_t w[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
+            uint4 o0, o1;
+            o0.x = (w[0] & 0xffffu) | (w[1] << 16);
+            o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
+            o0.z = (w[2] & 0xffffu) | (w[3] << 16);
+            o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
+            o1.x = (w[4] & 0xffffu) | (w[5] << 16);
+            o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
+            o1.z = (w[6] & 0xffffu) | (w[7] << 16);
+            o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
+            lds_x[t * (FH / 8) + swz8(2 * j)] = o0;
+            lds_x[t * (FH / 8) + swz8(2 * j + 1)] = o1;
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                sum += bf16_bits_to_f32(w[e] & 0xffffu);
+                sum += bf16_bits_to_f32(w[e] >> 16);
+            }
+            lds_sx[i] = sum;
+        }
+    }
+
+    // ---- every logit of every token, then the routing (each workgroup for itself, a wave per token) ----
+    for (uint32_t i = tid; i < T * (E + 1); i += THREADS)
+        lds_lg[i] = i % (E + 1) < n_rows ? __uint_as_float(wait_tagged(&s_lg[i], tag, a.spin_limit, s_err)) : 0.f;
+    __syncthreads();
+    for (uint32_t t = wv; t < T; t += WAVES) {
+        uint32_t id;
+        float wt;
+        softmax_topk_lane<4>(lds_lg + (size_t)t * (E + 1), E, K, lane, id, wt);
+        if (lane < K) {
+            lds_id[t * K + lane] = id;
+            lds_w[t * S + lane] = wt;
+            if (b == 0 && a.route_ids) {
+                a.route_ids[t * K + lane] = id;
+                a.route_w[t * K + lane] = wt;
+            }
+        }
+        if (lane == 0) lds_w[t * S + K] = a.sh_lw ? 1.f / (1.f + expf(-lds_lg[(size_t)t * (E + 1) + E])) : 1.f;  // ffn.rs:28-30
+    }
+    __syncthreads();
+
+    uint32_t m4, m2, magic;
+    asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
+                 : "=v"(m4), "=v"(m2), "=v"(magic)
+                 : "s"(a.m4), "s"(a.m2), "s"(a.magic));
+
+    // ---- phase 2: gate and up row p % I of slot (p / I) % S of token p / (I * S), lanes 0-31 the gate row and 32-63
+    // the up row, then the SwiGLU; the waves of the launch take the rows in turn, RING fetches ahead ----
+    {
+        const uint32_t li = lane & 31u, hf = lane >> 5;
+        const int c4 = (int)(li & 3u);
+        const uint32_t P = T * S * FI;
+        const uint32_t mine = gw < P ? (P - gw + NW - 1u) / NW : 0u;
+        const uint32_t lane_off = (li >> 2) * Q4K_BYTES;
+        auto fetch = [&](Piece<HQ_Q4_K>& pc, uint32_t p) {
+            const uint32_t r = p % FI, ts = p / FI, s = ts % S, t = ts / S;
+            const uint8_t* base = s < K ? (hf ? a.eu : a.eg) + (size_t)lds_id[t * K + s] * a.stride_gu : (hf ? a.su : a.sg);
+            pc.load(base + (size_t)r * ROWB_H + lane_off, c4);
+        };
+        Piece<HQ_Q4_K> ring[RING];
+#pragma unroll
+        for (int i = 0; i < RING; ++i)
+            if ((uint32_t)i < mine) fetch(ring[i], gw + (uint32_t)i * NW);
+        uint32_t xp[32];
+        float sx[4];
+        uint32_t cur_t = ~0u;
+        for (uint32_t i0 = 0; i0 < mine; i0 += RING) {
+#pragma unroll
+            for (int i = 0; i < RING; ++i) {
+                const uint32_t n = i0 + (uint32_t)i;
+                if (n < mine) {
+                    const uint32_t p = gw + n * NW, t = p / (FI * S);
+                    if (t != cur_t) {  // uniform
+                        cur_t = t;
+                        const uint32_t ch0 = li * 8u;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const uint4 v = lds_x[t * (FH / 8) + swz8(ch0 + j)];
+                            xp[4 * j] = v.x;
+                            xp[4 * j + 1] = v.y;
+                            xp[4 * j + 2] = v.z;
+                            xp[4 * j + 3] = v.w;
+                        }
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) sx[r] = lds_sx[t * (FH / 16) + ch0 / 2 + r];
+                    }
+                    const float v = group_sum(dot_pair(ring[i], c4, xp, sx, m4, m2, magic), 5);
+                    const float up = __shfl(v, 32);
+                    if (n + RING < mine) {
+                        float tie = v;
+                        asm volatile("" : "+v"(tie));
+                        fetch(ring[i], p + RING * NW);
+                    }
+                    if (lane == 0) st_dev(&s_act[p], tag_hi | __float_as_uint(silu_mul_f32(v, up)));
+                }
+            }
+        }
+    }
+    __syncthreads();  // the staged activations are dead from here on: their LDS holds the SwiGLU activations next
+
+    // ---- phases 3 + 4: unit (token t, column slice c): the down rows of the slice for every slot of the token, then
+    // the weighted sum over the slots in slot order, the shared expert last (the order of moe_weighted_reduce_kernel) ----
+    {
+        const uint32_t li = lane & 7u, sub = lane >> 3;
+        const int c4 = (int)(li & 3u);
+        const uint32_t groups = T <= 1 ? 1u : T <= 2 ? 2u : T <= 4 ? 4u : 8u, cols = 8u * groups;  // columns per unit: about one unit per workgroup
+        const uint32_t units_per_t = FH / cols, U = T * units_per_t;
+        for (uint32_t u = b; u < U; u += G) {
+            const uint32_t t = u / units_per_t, c = u % units_per_t;
+            // steps of this wave: (slot s, row group g) = step index wv, wv + WAVES, ... of S * groups
+            const uint32_t n_steps = S * groups, mine = wv < n_steps ? (n_steps - wv + WAVES - 1u) / WAVES : 0u;
+            auto fetch = [&](Piece<HQ_Q4_K>& pc, uint32_t n) {
+                const uint32_t st = wv + n * WAVES, s = st / groups, g = st % groups;
+                const uint8_t* base = s < K ? a.ed + (size_t)lds_id[t * K + s] * a.stride_d : a.sd;
+                pc.load(base + (size_t)(cols * c + 8 * g + sub) * ROWB_I + (li >> 2) * Q4K_BYTES, c4);
+            };
+            Piece<HQ_Q4_K> ring[RING];
+#pragma unroll
+            for (int i = 0; i < RING; ++i)
+                if ((uint32_t)i < mine) fetch(ring[i], (uint32_t)i);
+            // the token's SwiGLU activations of every slot: (tag, value) words, two per 16-byte load, all of a thread's
+            // loads in flight at once and the whole batch asked for again until every word of it is fresh
+            {
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                const uint64_t* src = s_act + (size_t)(t * S) * FI;
+                const uint32_t n2 = S * FI / 2;
+                for (uint32_t base = 0; base < n2; base += 8 * THREADS) {
+                    u32x4 got[8];
+                    bool fresh = false;
+                    for (uint32_t tries = 0; !fresh; ++tries) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) {
+                            const uint32_t e2 = base + tid + (uint32_t)i * THREADS;
+                            const uint64_t* p = src + 2 * (e2 < n2 ? e2 : 0u);
+                            asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(got[i]) : "v"(p) : "memory");
+                        }
+                        // the results exist once the counter has drained; naming them keeps their uses below the wait
+                        asm volatile("s_waitcnt vmcnt(0)"
+                                     : "+v"(got[0]), "+v"(got[1]), "+v"(got[2]), "+v"(got[3]), "+v"(got[4]), "+v"(got[5]), "+v"(got[6]), "+v"(got[7])
+                                     :
+                                     : "memory");
+                        fresh = true;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) fresh = fresh && got[i].y == tag && got[i].w == tag;
+                        if (!fresh && tries >= a.spin_limit) {
+                            st_dev(s_err, 2u);
+                            break;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const uint32_t e2 = base + tid + (uint32_t)i * THREADS;
+                        if (e2 < n2) {
+                            const uint32_t e = 2 * e2, sl = e / FI, k = e % FI, q = k >> 2;  // piece p = q / 16 reads float4 slot q ^ p
+                            float* dst = reinterpret_cast<float*>(lds_act) + sl * FI + (((q ^ (q >> 4)) << 2) | (k & 3u));
+                            dst[0] = __uint_as_float(got[i].x);
+                            dst[1] = __uint_as_float(got[i].z);
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+            for (uint32_t e = tid; e < S * (FI / 16); e += THREADS) {  // per-16 sums in the order one thread adds them (stage_swiglu)
+                const uint32_t s = e / (FI / 16), j = e % (FI / 16);
+                float sum = 0.f;
+#pragma unroll
+                for (uint32_t k = 0; k < 16; ++k) {
+                    const uint32_t q = (j * 16 + k) >> 2;
+                    sum += reinterpret_cast<float*>(lds_act)[s * FI + (((q ^ (q >> 4)) << 2) | (k & 3u))];
+                }
+                lds_as[e] = sum;
+            }
+            __syncthreads();
+            float xf[64], sx[4];
+            uint32_t cur_s = ~0u;
+            for (uint32_t i0 = 0; i0 < mine; i0 += RING) {
+#pragma unroll
+                for (int i = 0; i < RING; ++i) {
+                    const uint32_t n = i0 + (uint32_t)i;
+                    if (n < mine) {
+                        const uint32_t st = wv + n * WAVES, s = st / groups, g = st % groups;
+                        if (s != cur_s) {  // uniform
+                            cur_s = s;
+#pragma unroll
+                            for (int q = 0; q < 16; ++q) {
+                                const float4 v = lds_act[s * (FI / 4) + ((li * 16 + q) ^ li)];
+                                xf[4 * q] = v.x;
+                                xf[4 * q + 1] = v.y;
+                                xf[4 * q + 2] = v.z;
+                                xf[4 * q + 3] = v.w;
+                            }
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) sx[r] = lds_as[s * (FI / 16) + li * 4 + r];
+                        }
+                        const float v = group_sum(dot_f32(ring[i], c4, xf, sx), 3);
+                        if (n + RING < mine) {
+                            float tie = v;
+                            asm volatile("" : "+v"(tie));
+                            fetch(ring[i], n + RING);
+                        }
+                        if (li == 0) lds_part[s * cols + 8 * g + sub] = v;
+                    }
+                }
+            }
+            __syncthreads();
+            if (tid < cols) {
+                const uint32_t col = cols * c + tid;
+                float acc = 0.f;
+                for (uint32_t s = 0; s < S; ++s) acc = fmaf(lds_w[t * S + s], lds_part[s * cols + tid], acc);
+                if (a.residual) acc += a.residual[(size_t)t * FH + col];
+                a.out[(size_t)t * FH + col] = acc;
+            }
+            __syncthreads();  // lds_act / lds_part are rewritten by the next unit
+        }
+    }
+    if (b == 0 && tid == 0) st_dev(s_epoch, tag);
+}
+
+}  // namespace
+
+size_t moe_fused_scratch_bytes(uint32_t n_tokens, uint32_t n_experts, uint32_t top_k) {
+    return (Layout{n_tokens, n_experts, top_k}.total() + 255) & ~(size_t)255;
+}
+
+bool moe_fused_supported(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k, uint32_t inter,
+                         uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt) {
+    return t == HQ_Q4_K && xdt == HQ_BF16 && hidden == FH && inter == FI && shared_inter == FI && n_tokens >= 1 &&
+           n_tokens <= 8 && n_experts >= 1 && n_experts <= 256 && top_k >= 1 && top_k <= 64 && top_k <= n_experts;
+}
+
+int launch_moe_fused(hipStream_t s, const MoeFusedArgs& m) {
+    FusedArgs a{};
+    a.x = static_cast<const uint16_t*>(m.x);
+    a.router = static_cast<const uint16_t*>(m.router);
+    a.sh_lw = static_cast<const uint16_t*>(m.shared_gate_logit);
+    a.eg = static_cast<const uint8_t*>(m.expert_gate);
+    a.eu = static_cast<const uint8_t*>(m.expert_up);
+    a.ed = static_cast<const uint8_t*>(m.expert_down);
+    a.sg = static_cast<const uint8_t*>(m.shared_gate);
+    a.su = static_cast<const uint8_t*>(m.shared_up);
+    a.sd = static_cast<const uint8_t*>(m.shared_down);
+    a.residual = m.residual;
+    a.out = m.out;
+    a.route_ids = m.route_ids;
+    a.route_w = m.route_weights;
+    a.scratch = static_cast<uint8_t*>(m.scratch);
+    a.T = m.n_tokens;
+    a.E = m.n_experts;
+    a.K = m.top_k;
+    a.stride_gu = m.stride_gate_up;
+    a.stride_d = m.stride_down;
+    a.m4 = M4;
+    a.m2 = M2;
+    a.magic = MAGIC;
+    a.spin_limit = m.spin_limit ? m.spin_limit : (1u << 20);
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
+    // every workgroup must deliver at least one logit row (see the header comment), and one workgroup per CU
+    const uint32_t rows = m.n_experts + (m.shared_gate_logit ? 1u : 0u);
+    const uint32_t grid = cus < rows ? cus : rows;
+    const uint32_t T = m.n_tokens, S = m.top_k + 1;
+    const size_t area = (size_t)T * (FH / 8) * 16 + (size_t)T * (FH / 16) * 4, act_bytes = (size_t)S * (FI * 4 + FI / 16 * 4);
+    const size_t lds = (area > act_bytes ? area : act_bytes) + (size_t)T * (m.n_experts + 1) * 4 + (size_t)T * m.top_k * 4 +
+                       (size_t)T * S * 4 + (size_t)S * 64 * 4;
+    if (lds > 64 * 1024) return fail(HQ_ERR_UNSUPPORTED, "fused MoE block: %zu bytes of LDS", lds);
+    hipLaunchKernelGGL(moe_fused_kernel, dim3(grid), dim3(THREADS), lds, s, a);
+    return check_launch("fused MoE block launch");
+}
+
+}  // namespace hq

@@ -19,26 +19,28 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// Wave-wide maximum of a 64-bit key with DPP moves only (no LDS traffic); every lane gets the
-// result.  Quad permutes and row mirrors cover a row of 16 lanes, row_bcast 15 / 31 carry the row
-// maxima upwards, lane 63 then holds the maximum and is read back as a scalar.
+// Wave-wide maximum of a 64-bit key with DPP moves only (no LDS traffic); every lane gets the result.  Two passes over
+// 32-bit halves: the largest high word, then the largest low word among the lanes that hold it (a key's low word is
+// never 0 unless the key is absent), which is the 64-bit maximum with half the moves of a 64-bit exchange.  Quad
+// permutes and row mirrors cover a row of 16 lanes, row_bcast 15 / 31 carry the row maxima upwards, lane 63 then holds
+// the maximum and is read back as a scalar.
 template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint64_t dpp_max_u64(uint64_t v) {
-    const uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
-    const uint32_t olo = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)lo, CTRL, ROW_MASK, 0xf, false);
-    const uint32_t ohi = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)hi, CTRL, ROW_MASK, 0xf, false);
-    const uint64_t o = ((uint64_t)ohi << 32) | olo;
+__device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xf, false);
     return o > v ? o : v;
 }
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    v = dpp_max_u32<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+    v = dpp_max_u32<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+    v = dpp_max_u32<0x141, 0xf>(v);  // row_half_mirror
+    v = dpp_max_u32<0x140, 0xf>(v);  // row_mirror
+    v = dpp_max_u32<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_max_u32<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-    v = dpp_max_u64<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
-    v = dpp_max_u64<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
-    v = dpp_max_u64<0x141, 0xf>(v);  // row_half_mirror
-    v = dpp_max_u64<0x140, 0xf>(v);  // row_mirror
-    v = dpp_max_u64<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-    v = dpp_max_u64<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 63);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 63);
+    const uint32_t hi = wave_max_u32((uint32_t)(v >> 32));
+    const uint32_t lo = wave_max_u32((uint32_t)(v >> 32) == hi ? (uint32_t)v : 0u);
     return ((uint64_t)hi << 32) | lo;
 }
 

@@ -66,6 +66,8 @@ SIGNATURES = {
     "hq_moe_softmax_topk": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "hq_silu_mul": (_i32, [_vp, _vp, _vp, _vp, _u64]),
     "hq_moe_weighted_reduce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "hq_moe_ffn_decode_scratch_bytes": (_sz, [_u32, _u32, _u32, _u32, _u32, _u32, _i32, _i32]),
+    "hq_moe_ffn_decode": (_i32, [_vp, _vp, _vp, _i32, _vp, _vp, _u32, _vp, _sz, _vp, _vp]),
     "hq_fwht_sign_premult_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_fwht_sign_undo_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_tq_encode_kv": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
@@ -102,6 +104,14 @@ class TqpHeader(ctypes.Structure):
     """hq_tqp_header (include/hf2q_hip.h)."""
     _fields_ = [("codec_version", _u32), ("bits_per_coord", _u32), ("head_dim", _u32), ("n_kv_heads", _u32),
                 ("n_tokens", _u32), ("flags", _u32), ("scale", ctypes.c_double)]
+
+
+class MoeFfnLayer(ctypes.Structure):
+    """hq_moe_ffn_layer (include/hf2q_hip.h), field for field."""
+    _fields_ = [("router", _vp), ("shared_gate_logit", _vp), ("expert_gate", _vp), ("expert_up", _vp), ("expert_down", _vp),
+                ("shared_gate", _vp), ("shared_up", _vp), ("shared_down", _vp), ("hidden", _u32), ("n_experts", _u32),
+                ("top_k", _u32), ("inter", _u32), ("shared_inter", _u32), ("ggml_type", _i32),
+                ("expert_stride_gate_up", _u64), ("expert_stride_down", _u64)]
 
 
 class TqAttnParams(ctypes.Structure):

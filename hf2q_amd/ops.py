@@ -604,6 +604,10 @@ class MoeFfnScratch:
                                                                             w.hidden * rb_i, w.ggml_type)))
         self.id_mm = torch.empty(need, dtype=torch.uint8, device=device) if need else None
         self.max_tokens = T
+        # scratch of the one-launch decode block (hq_moe_ffn_decode): zeroed once, then the library's
+        fb = _l.load().hq_moe_ffn_decode_scratch_bytes(min(T, 8), w.hidden, w.n_experts, K, w.inter, w.shared_inter, w.ggml_type,
+                                                       _l.HQ_BF16)
+        self.fused = torch.zeros(fb, dtype=torch.uint8, device=device) if fb else None
 
 
 # Dense products above this many rows take the tile (GEMM) route, which the batched launch does not cover.
@@ -613,9 +617,31 @@ _ROUTE_IN_LAUNCH_MAX_TOKENS = 4
 _FUSED_SWIGLU_MAX_K = 8192
 
 
+def moe_ffn_decode_fused(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch, out: torch.Tensor,
+                         residual: torch.Tensor | None = None) -> None:
+    """The whole block as one launch (hq_moe_ffn_decode); raises HqError(HQ_ERR_UNSUPPORTED) for shapes it does not take."""
+    import ctypes as _ct
+    T = x.shape[0]
+    rb_h, rb_i = ggml_row_bytes(w.ggml_type, w.hidden), ggml_row_bytes(w.ggml_type, w.inter)
+    layer = _l.MoeFfnLayer(_dev(w.router, "router"), _dev(w.shared_gate_logit, "shared_gate_logit"),
+                           _dev(w.expert_gate, "expert_gate"), _dev(w.expert_up, "expert_up"), _dev(w.expert_down, "expert_down"),
+                           _dev(w.shared_gate, "shared_gate"), _dev(w.shared_up, "shared_up"), _dev(w.shared_down, "shared_down"),
+                           w.hidden, w.n_experts, w.top_k, w.inter, w.shared_inter, w.ggml_type, w.inter * rb_h, w.hidden * rb_i)
+    if s.fused is None:
+        raise _l.HqError(_l.HQ_ERR_UNSUPPORTED, "no scratch for the one-launch MoE block (shape not supported)")
+    _l.check(_l.load().hq_moe_ffn_decode(
+        _stream(), _ct.byref(layer), _dev(x, "x"), _act_dtype(x), _dev(residual, "residual") if residual is not None else None,
+        _dev(out, "out"), T, _dev(s.fused, "scratch"), s.fused.numel(), _dev(s.ids, "ids"), _dev(s.topk_w, "topk_w")))
+
+
+def moe_ffn_decode_fused_supported(x: torch.Tensor, w: MoeFfnWeightsGpuQ) -> bool:
+    return bool(_l.load().hq_moe_ffn_decode_scratch_bytes(x.shape[0], w.hidden, w.n_experts, w.top_k, w.inter, w.shared_inter,
+                                                          w.ggml_type, _act_dtype(x)))
+
+
 def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch, out: torch.Tensor,
                                    residual: torch.Tensor | None = None, batched: bool | None = None,
-                                   route_in_launch: bool | None = None) -> None:
+                                   route_in_launch: bool | None = None, fused: bool | None = None) -> None:
     """gpu_ffn.rs:2313-2802, phases A-F, enqueued on the current stream with no host round trip:
     router / shared projections -> softmax top-k + shared SwiGLU -> gate, up mul_mat_id + shared down ->
     SwiGLU -> down mul_mat_id (n_tokens = T*K, top_k = 1) -> weighted reduce (+ sigmoid-gated shared, + residual).
@@ -629,6 +655,11 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
     T = x.shape[0]
     K, H, E, I, SI, t = w.top_k, w.hidden, w.n_experts, w.inter, w.shared_inter, w.ggml_type
     rb = ggml_row_bytes(t, H)
+    if fused is None:
+        fused = batched is None and route_in_launch is None and s.fused is not None and moe_ffn_decode_fused_supported(x, w)
+    if fused:
+        # one launch for the whole block, the bits of the batched dispatches below
+        return moe_ffn_decode_fused(x, w, s, out, residual)
     if batched is None:
         batched = T <= _BATCH_MAX_DENSE_ROWS
     if batched:

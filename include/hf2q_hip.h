@@ -221,6 +221,41 @@ HQ_API int hq_moe_weighted_reduce(void* stream, const float* y, const float* w, 
  * [n_kv_heads, capacity, max(1, head_dim/256)] f32.  K and V are stored in the rotated
  * domain  H.(s (.) x)  (normalised Hadamard, sign table kv_cache.rs:3871-3876). */
 
+/* The whole MoE FFN block of a decode step as ONE launch: router + shared-gate logits, softmax / top-k / renormalise,
+ * gate and up of the routed and the shared expert with their SwiGLU, the down projections, and
+ * out[t] = sum_s w[t,s] * down[t,s] + sigmoid(shared logit[t]) * shared_down[t] (+ residual[t]).  Replaces
+ * build_moe_ffn_layer_gpu_q_into (src/inference/models/qwen35/gpu_ffn.rs:2313-2802: phases A-F of one command
+ * buffer); moe_ffn_cpu_ref (ffn.rs:179-336) is the specification.  The result has the bits of the separate dispatches
+ * (hq_dense_gemv_bf16_pair, hq_qmatmul_batch_ggml twice with the routing and the SwiGLU folded in,
+ * hq_moe_weighted_reduce).  Takes 1..8 tokens of bf16 activations, Q4_K experts, hidden 2048, expert and shared FFN
+ * width 512, <= 256 experts, top_k <= 64; anything else is HQ_ERR_UNSUPPORTED (hq_moe_ffn_decode_scratch_bytes
+ * returns 0 for it) and runs as the separate dispatches.
+ * `scratch`: hq_moe_ffn_decode_scratch_bytes() bytes of device memory, 256-byte aligned, ZEROED ONCE before its first
+ * use and then left to the library (it carries a call counter; calls that share a scratch must not overlap, and a
+ * scratch serves one (n_experts, top_k) shape).  The workgroups of the launch hand results to each other through it
+ * and wait for each other with bounded polling; if a wait ever runs out (it cannot, unless the device is shared with a
+ * kernel that starves the launch for seconds) the second 32-bit word of the scratch becomes non-zero and the output is
+ * undefined.  route_ids / route_weights: NULL, or where the routing is also written ([n_tokens * top_k] each). */
+typedef struct hq_moe_ffn_layer {
+    const void* router;            /* [n_experts, hidden] bf16 */
+    const void* shared_gate_logit; /* [hidden] bf16, or NULL: the shared expert enters with weight 1 */
+    const void* expert_gate;       /* [n_experts][inter][hidden / 256] blocks */
+    const void* expert_up;
+    const void* expert_down;       /* [n_experts][hidden][inter / 256] blocks */
+    const void* shared_gate;       /* [shared_inter][hidden / 256] blocks */
+    const void* shared_up;
+    const void* shared_down;       /* [hidden][shared_inter / 256] blocks */
+    uint32_t hidden, n_experts, top_k, inter, shared_inter;
+    hq_ggml_type ggml_type;
+    uint64_t expert_stride_gate_up; /* bytes between experts of expert_gate / expert_up */
+    uint64_t expert_stride_down;
+} hq_moe_ffn_layer;
+HQ_API size_t hq_moe_ffn_decode_scratch_bytes(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k,
+                                       uint32_t inter, uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt);
+HQ_API int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* layer, const void* x, hq_act_dtype xdt,
+                      const float* residual, float* out, uint32_t n_tokens, void* scratch, size_t scratch_bytes,
+                      uint32_t* route_ids, float* route_weights);
+
 /* In-place  buf <- H.(s (.) buf)  per 256-element block of buf[n_heads][head_dim] (query
  * pre-rotation) and its inverse  buf <- s (.) (H.buf)  (output post-rotation).  Replace
  * dispatch_fwht_sign_premult_f32 / dispatch_fwht_sign_undo_f32(enc, reg, dev, buf, num_heads,

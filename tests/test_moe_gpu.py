@@ -261,3 +261,57 @@ def test_dense_ffn_batched_equals_separate_dispatches_and_cpu_spec(oracle, dev, 
     gate, up = xr @ dq["g"].T, xr @ dq["u"].T
     want = (gate / (1 + np.exp(-gate)) * up) @ dq["d"].T
     assert_matmul_close(outs[1][0].numpy(), want, "dense FFN")
+
+
+@pytest.mark.parametrize("T", [1, 2, 5, 8])
+def test_moe_block_one_launch_equals_batched_dispatches_and_cpu_spec(oracle, dev, T):
+    """hq_moe_ffn_decode (the whole block in one launch, workgroups handing results to each other through the
+    scratch) at the Qwen3.6-35B-A3B expert shape, fewer experts: the bits of the batched dispatches, the CPU
+    specification within the block's tolerance, and the same answer on repeated calls over one scratch (the call
+    counter in the scratch tells fresh hand-overs from the previous call's)."""
+    H, E, K, I, SI = 2048, 24, 8, 512, 512
+    rng = np.random.default_rng(500 + T)
+    bf = lambda a: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(a))  # noqa: E731
+    router = bf((rng.standard_normal((E, H)) * 0.1).astype(np.float32))
+    sgl = bf((rng.standard_normal((1, H)) * 0.05).astype(np.float32))
+    raw = {nm: weights(seed + T, n, k, 0.05) for nm, seed, n, k in
+           (("eg", 31, E * I, H), ("eu", 32, E * I, H), ("ed", 33, E * H, I), ("sg", 34, SI, H), ("su", 35, SI, H), ("sd", 36, H, SI))}
+    q = {nm: oracle.quantize(a, a.shape[1], HQ_Q4_K, threads=8) for nm, a in raw.items()}
+    dq = {nm: oracle.dequantize(q[nm], HQ_Q4_K, threads=8).reshape(raw[nm].shape) for nm in raw}
+    xb = bf(acts(37 + T, T, H))
+    res = acts(38, T, H)
+    want = oracle.moe_ffn(xb, H, E, K, I, SI, router, dq["eg"], dq["eu"], dq["ed"], sgl[0], dq["sg"], dq["su"], dq["sd"]) + res
+
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    w = ops.MoeFfnWeightsGpuQ(dv(router).to(torch.bfloat16), dv(q["eg"]), dv(q["eu"]), dv(q["ed"]),
+                              dv(sgl).to(torch.bfloat16), dv(q["sg"]), dv(q["su"]), dv(q["sd"]), HQ_Q4_K, H, E, K, I, SI)
+    x = dv(xb).to(torch.bfloat16)
+    assert ops.moe_ffn_decode_fused_supported(x, w)
+    s = ops.MoeFfnScratch(w, T, dev)
+    ref = torch.full((T, H), float("nan"), device=dev)
+    ops.build_moe_ffn_layer_gpu_q_into(x, w, s, ref, residual=dv(res), batched=True)
+    ids_ref, w_ref = s.ids.clone(), s.topk_w.clone()
+    for call in range(3):
+        s.ids.fill_(-1)
+        s.topk_w.fill_(float("nan"))
+        out = torch.full((T, H), float("nan"), device=dev)
+        ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out, residual=dv(res))  # default: the one-launch form
+        torch.cuda.synchronize()
+        assert int(s.fused[4:8].view(torch.int32).item()) == 0, "a wait inside the launch ran out"
+        assert int(s.fused[0:4].view(torch.int32).item()) == call + 1
+        assert torch.equal(s.ids, ids_ref) and torch.equal(s.topk_w, w_ref)
+        assert torch.equal(out, ref), f"call {call}: max diff {(out - ref).abs().max().item()}"
+    got = out.cpu().numpy()
+    assert np.abs(got - want).max() <= 2e-4 * np.abs(want).max(), np.abs(got - want).max() / np.abs(want).max()
+
+
+def test_moe_block_one_launch_rejects_other_shapes(oracle, dev):
+    H, E, K, I, SI = 512, 16, 4, 256, 512
+    w = _moe_weights(oracle, dev, HQ_Q4_K, H, E, K, I, SI)
+    s = ops.MoeFfnScratch(w, 2, dev)
+    assert s.fused is None
+    x = torch.zeros(2, H, device=dev, dtype=torch.bfloat16)
+    assert not ops.moe_ffn_decode_fused_supported(x, w)
+    with pytest.raises(ops.HqError) as e:
+        ops.moe_ffn_decode_fused(x, w, s, torch.empty(2, H, device=dev))
+    assert e.value.status == 2
