@@ -43,6 +43,29 @@ static int check_weight_alignment(const void* w, hq_ggml_type t) {
 }
 
 // The device's CU count, cached per device.
+int ensure_lds_limit(const void* kernel, size_t bytes, const char* what) {
+    if (bytes < 64 * 1024) return HQ_OK;  // below the default limit
+    struct Entry {
+        const void* fn;
+        int dev;
+        size_t bytes;
+    };
+    static std::mutex mu;
+    static Entry table[256];
+    static int used = 0;
+    int dev = 0;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    std::lock_guard<std::mutex> lock(mu);
+    Entry* e = nullptr;
+    for (int i = 0; i < used; ++i)
+        if (table[i].fn == kernel && table[i].dev == dev) e = &table[i];
+    if (e && e->bytes >= bytes) return HQ_OK;
+    if (int rc = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes), what)) return rc;
+    if (!e && used < 256) e = &table[used++];
+    if (e) *e = Entry{kernel, dev, bytes};  // a full table only means the attribute is set again next time
+    return HQ_OK;
+}
+
 int cu_count(uint32_t* out) {
     static std::mutex mu;
     static int cached[64] = {};
@@ -87,7 +110,7 @@ uint32_t hq_block_bytes(hq_ggml_type t) {
 int hq_dequant_ggml(void* stream, const void* w_blocks, void* out, hq_act_dtype out_dtype,
                     uint64_t n_elems, hq_ggml_type t) {
     if (!known_type(t)) return fail(HQ_ERR_UNSUPPORTED, "hq_dequant_ggml: unsupported ggml type %d", (int)t);
-    if (out_dtype != HQ_F32 && out_dtype != HQ_BF16)
+    if (out_dtype != HQ_F32 && out_dtype != HQ_BF16 && out_dtype != HQ_F16)
         return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dequant_ggml: out_dtype %d", (int)out_dtype);
     if (n_elems % hq_block_elems(t))
         return fail(HQ_ERR_INVALID_ARGUMENT, "hq_dequant_ggml: n_elems %llu is not a multiple of the block size %u",

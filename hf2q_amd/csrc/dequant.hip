@@ -93,16 +93,27 @@ __device__ __forceinline__ void dequant4(const uint8_t* __restrict__ w, uint64_t
     }
 }
 
-template <int TYPE, bool BF16_OUT>
+template <int TYPE, int OUT>  // OUT: hq_act_dtype of the output
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w, void* __restrict__ out,
                                                       uint64_t n_quads) {
     for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n_quads; i += (uint64_t)gridDim.x * 256) {
         float v[4];
         dequant4<TYPE>(w, i * 4, v);
-        if constexpr (BF16_OUT) {
+        if constexpr (OUT == HQ_BF16) {
             uint2 o;
             o.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
             o.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+            reinterpret_cast<uint2*>(out)[i] = o;
+        } else if constexpr (OUT == HQ_F16) {  // v_cvt_f16_f32: round to nearest even, overflow to infinity
+            // (the f32 value is made opaque first: the compiler otherwise folds its last multiplication into the
+            // conversion as v_fma_mixlo_f16 x, y, +0, which turns a product of -0.0 into +0.0)
+            const auto h = [](float f) {
+                asm volatile("" : "+v"(f));
+                return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)f);
+            };
+            uint2 o;
+            o.x = h(v[0]) | (h(v[1]) << 16);
+            o.y = h(v[2]) | (h(v[3]) << 16);
             reinterpret_cast<uint2*>(out)[i] = o;
         } else {
             reinterpret_cast<float4*>(out)[i] = make_float4(v[0], v[1], v[2], v[3]);
@@ -117,9 +128,11 @@ static int launch_t(hipStream_t s, const void* w, void* out, hq_act_dtype odt, u
     const unsigned grid = (unsigned)(want < 65536 ? want : 65536);
     const uint8_t* wb = static_cast<const uint8_t*>(w);
     if (odt == HQ_BF16)
-        hipLaunchKernelGGL((dequant_kernel<TYPE, true>), dim3(grid), dim3(256), 0, s, wb, out, quads);
+        hipLaunchKernelGGL((dequant_kernel<TYPE, HQ_BF16>), dim3(grid), dim3(256), 0, s, wb, out, quads);
+    else if (odt == HQ_F16)
+        hipLaunchKernelGGL((dequant_kernel<TYPE, HQ_F16>), dim3(grid), dim3(256), 0, s, wb, out, quads);
     else
-        hipLaunchKernelGGL((dequant_kernel<TYPE, false>), dim3(grid), dim3(256), 0, s, wb, out, quads);
+        hipLaunchKernelGGL((dequant_kernel<TYPE, HQ_F32>), dim3(grid), dim3(256), 0, s, wb, out, quads);
     return check_launch("dequant kernel launch");
 }
 

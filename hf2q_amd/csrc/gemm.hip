@@ -394,9 +394,7 @@ template <int TYPE, bool X_BF16, int BM>
 int launch_t(hipStream_t s, const GemmArgs& a) {
     auto kern = gemm_kernel<TYPE, X_BF16, BM>;
     constexpr int lds = Lds<X_BF16, BM>::kTotal;
-    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                           "hipFuncSetAttribute(gemm LDS)"))
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(gemm LDS)"))
         return rc;
     const uint32_t tiles_n = (a.n + BN - 1) / BN, tiles_m = (a.m + BM - 1) / BM;
     const dim3 grid(8u * ((tiles_m + 7u) / 8u) * tiles_n);  // see the tile order in the kernel

@@ -981,8 +981,7 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     if (int rc = launch_prep<TYPE>(s, x, xdt, wb, ws, pairs, n_experts * n, k, row_map, top_k)) return rc;
     constexpr int lds = 2 * ActTile::kTile;
     auto kern = grouped_gemm_kernel<TYPE>;
-    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                           "hipFuncSetAttribute(grouped gemm LDS)"))
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;
     GemmArgs a{ws, wb, y, pairs, n, k, pairs, n_experts * n, 0u, row_map};
     const uint32_t tiles_n = (n + BN_WIDE - 1) / BN_WIDE;
@@ -1019,9 +1018,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
     if (t == HQ_Q6_K) {
         if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(q6k_gemm_kernel),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                               "hipFuncSetAttribute(q6_k gemm LDS)"))
+        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(q6k_gemm_kernel), (size_t)lds, "hipFuncSetAttribute(q6_k gemm LDS)"))
             return rc;
         hipLaunchKernelGGL(q6k_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
         return check_launch("q6_k gemm kernel launch");
@@ -1031,8 +1028,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         if (int rc = t == HQ_Q4_0 ? launch_prep<HQ_Q4_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
                                   : launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
             return rc;
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                               "hipFuncSetAttribute(q8_0 gemm LDS)"))
+        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(q8_0 gemm LDS)"))
             return rc;
         hipLaunchKernelGGL(kern, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
         return check_launch("q8_0 gemm kernel launch");
@@ -1041,8 +1037,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
                               : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
         return rc;
-    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                           "hipFuncSetAttribute(q4k gemm LDS)"))
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(q4k gemm LDS)"))
         return rc;
     // Tiles of 128 weight rows; tiles of 64 when the wide ones would occupy at most half of the CUs.
     // (Cutting only the last, partly filled round of a large problem into narrow tiles was measured:

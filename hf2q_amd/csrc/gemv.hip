@@ -532,10 +532,7 @@ bool stream_takes(uint32_t n_total, uint32_t k, uint32_t cus) {
 
 template <typename K>
 int set_lds_limit(K kern, size_t lds, const char* what) {
-    if (lds <= 64 * 1024) return HQ_OK;
-    return check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
-                     what);
+    return ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, what);
 }
 
 template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>

@@ -456,8 +456,7 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
         kern = nsb == 4 ? q6k_rows_kernel<false, 4>
                : nsb == 2 ? q6k_rows_kernel<true, 2>
                           : (bf ? q6k_rows_kernel<true, 1> : q6k_rows_kernel<false, 1>);
-    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                           "hipFuncSetAttribute(rows kernel LDS)"))
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(rows kernel LDS)"))
         return rc;
     const uint32_t rows_per_wg = 16u * nsb;
     hipLaunchKernelGGL(kern, dim3((n + rows_per_wg - 1u) / rows_per_wg), dim3(256), lds, s, a);

@@ -185,6 +185,9 @@ int parse(hq_gguf* g, const char* path) {
         if (ti.n_dims && ti.dims[0] % tg->block_elems)
             return fail(HQ_ERR_INVALID_ARGUMENT, "hq_gguf_open: %s: tensor %s: row length %llu is not a multiple of the block size %u",
                         path, name.c_str(), (unsigned long long)ti.dims[0], tg->block_elems);
+        if (elems / tg->block_elems > UINT64_MAX / tg->block_bytes)
+            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_gguf_open: %s: tensor %s: %llu elements do not fit a 64-bit byte count", path,
+                        name.c_str(), (unsigned long long)elems);
         ti.byte_len = elems / tg->block_elems * tg->block_bytes;
         g->by_name.emplace(name, g->infos.size());
         g->names.push_back(std::move(name));

@@ -16,6 +16,10 @@ int check_hip(hipError_t e, const char* what);
 // Checks the launch that was just enqueued.
 inline int check_launch(const char* what) { return check_hip(hipGetLastError(), what); }
 
+// Raises a kernel's dynamic-LDS limit to `bytes` (hipFuncAttributeMaxDynamicSharedMemorySize) unless an earlier call
+// on this device already set it at least that high: the attribute call costs microseconds of host time per launch.
+int ensure_lds_limit(const void* kernel, size_t bytes, const char* what);
+
 inline bool is_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 constexpr int kWave = 64;

@@ -32,17 +32,24 @@ extern "C" {
 
 size_t hq_tqp_indices_bytes(const hq_tqp_header* h) {
     if (!h) return 0;
+    // four 32-bit factors: at most 2^128 - 2^98, which the 128-bit product holds; a count beyond size_t saturates (no
+    // buffer has that length, so hq_tqp_pack / hq_tqp_unpack reject the header)
     const unsigned __int128 bits = (unsigned __int128)h->n_kv_heads * h->n_tokens * h->head_dim * h->bits_per_coord;
-    return (size_t)((bits + 7) / 8);
+    const unsigned __int128 bytes = (bits + 7) / 8;
+    return bytes > (unsigned __int128)SIZE_MAX ? SIZE_MAX : (size_t)bytes;
 }
 
 size_t hq_tqp_norms_bytes(const hq_tqp_header* h) {
     if (!h || h->codec_version != 2) return 0;
-    return (size_t)h->n_kv_heads * h->n_tokens * norms_per_pos(h->head_dim) * 4;
+    const unsigned __int128 bytes = (unsigned __int128)h->n_kv_heads * h->n_tokens * norms_per_pos(h->head_dim) * 4;
+    return bytes > (unsigned __int128)SIZE_MAX ? SIZE_MAX : (size_t)bytes;
 }
 
 size_t hq_tqp_total_bytes(const hq_tqp_header* h) {
-    return h ? HQ_TQP_HEADER_BYTES + hq_tqp_indices_bytes(h) + hq_tqp_norms_bytes(h) : 0;
+    if (!h) return 0;
+    const size_t a = hq_tqp_indices_bytes(h), b = hq_tqp_norms_bytes(h);
+    if (a > SIZE_MAX - HQ_TQP_HEADER_BYTES || b > SIZE_MAX - HQ_TQP_HEADER_BYTES - a) return SIZE_MAX;
+    return HQ_TQP_HEADER_BYTES + a + b;
 }
 
 int hq_tqp_pack(const hq_tqp_header* h, const void* indices, size_t indices_len, const void* norms_le, size_t norms_len,

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(HERE, "libhf2q_hip.so")
 
 HQ_OK, HQ_ERR_INVALID_ARGUMENT, HQ_ERR_UNSUPPORTED, HQ_ERR_HIP = 0, 1, 2, 3
 HQ_Q4_0, HQ_Q8_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K = 2, 8, 12, 13, 14
-HQ_F32, HQ_BF16 = 0, 1
+HQ_F32, HQ_BF16, HQ_F16 = 0, 1, 2
 
 
 class HqError(RuntimeError):

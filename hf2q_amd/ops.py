@@ -198,8 +198,8 @@ def dequantize_ggml(weight: torch.Tensor, n_elems: int, ggml_type: int,
                     dtype: torch.dtype = torch.float32) -> torch.Tensor:
     out = torch.empty(n_elems, dtype=dtype, device=weight.device)
     L = _l.load()
-    _l.check(L.hq_dequant_ggml(_stream(), _dev(weight, "weight"), _dev(out, "out"), _act_dtype(out), n_elems,
-                               ggml_type))
+    odt = _l.HQ_F16 if dtype == torch.float16 else _act_dtype(out)  # f16: the output dtype of the F16 shadow only
+    _l.check(L.hq_dequant_ggml(_stream(), _dev(weight, "weight"), _dev(out, "out"), odt, n_elems, ggml_type))
     return out
 
 

@@ -48,7 +48,7 @@ typedef enum { HQ_Q4_0 = 2, HQ_Q8_0 = 8, HQ_Q4_K = 12, HQ_Q5_K = 13, HQ_Q6_K = 1
 
 /* Activation element type.  hf2q's call sites pass F32 (gpu_full_attn.rs:835);
  * BF16 is the serving configuration this library is benchmarked on. */
-typedef enum { HQ_F32 = 0, HQ_BF16 = 1 } hq_act_dtype;
+typedef enum { HQ_F32 = 0, HQ_BF16 = 1, HQ_F16 = 2 /* output of hq_dequant_ggml only */ } hq_act_dtype;
 
 /* Thread-local message of the last failing call on this thread ("" if none). */
 HQ_API const char* hq_last_error(void);
@@ -63,7 +63,8 @@ HQ_API uint32_t hq_block_bytes(hq_ggml_type t);
 
 /* Dequantise `n_elems` (a whole number of blocks) of packed GGML blocks to
  * f32 (out_dtype HQ_F32, bit-exact: one correctly rounded value per element)
- * or bf16 (HQ_BF16, the f32 value rounded to nearest-even).  Replaces the
+ * or bf16 / f16 (HQ_BF16 / HQ_F16, the f32 value rounded to nearest-even; f16 is
+ * the reference's shadow dtype).  Replaces the
  * load-time `materialize_f16_shadow` pre-dequantisation
  * (src/serve/forward_mlx.rs:9426-9440) and doubles as the bit-exactness probe
  * for the in-kernel dequantisers. */

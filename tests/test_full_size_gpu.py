@@ -11,7 +11,7 @@ import torch
 
 from _util import assert_matmul_close, assert_matmul_close_f16_tile
 from hf2q_amd import ops
-from hf2q_amd.ops import HQ_Q4_K, HQ_Q6_K, FlashAttnVecTqHbParams, GgmlQuantizedMatmulParams
+from hf2q_amd.ops import HQ_Q4_K, HQ_Q6_K, HQ_Q8_0, FlashAttnVecTqHbParams, GgmlQuantizedMatmulParams
 
 pytestmark = pytest.mark.gpu
 
@@ -62,10 +62,12 @@ def test_decode_gemv_full_size(oracle, dev, n, k, t, m):
     assert torch.equal(run(xa * 4.0), ya * 4.0)
 
 
-def test_prefill_gemm_full_size(oracle, dev):
-    """2048 tokens x K = 4096 x N = 12288, Q4_K, bf16 activations: a sample of (token, weight row) pairs against the
-    oracle, scaling of a token row by a power of two, and agreement of token rows with the m = 1 GEMV."""
-    m, k, n, t = 2048, 4096, 12288, HQ_Q4_K
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0])
+def test_prefill_gemm_full_size(oracle, dev, t):
+    """2048 tokens x K = 4096 x N = 12288, Q4_K and Q8_0 (both variants of BASELINE config 4), bf16 activations: a
+    sample of (token, weight row) pairs against the oracle, scaling of a token row by a power of two, and agreement
+    of token rows with the m = 1 GEMV."""
+    m, k, n = 2048, 4096, 12288
     w = _quantized(dev, n, k, t, 1234)
     g = torch.Generator(device=dev)
     g.manual_seed(5678)

@@ -180,3 +180,36 @@ def test_perm021_matches_oracle_and_the_plain_product(oracle, dev, t, m, heads, 
     assert torch.equal(y, y2)
     with pytest.raises(ops.HqError):  # head_dim must divide k
         ops.quantized_matmul_mm_tensor_perm021(x_perm, wd, y, ops.GgmlQuantizedMatmulPerm021Params(m, n, k, hd + 8, t))
+
+
+def test_tile_gemm_with_caller_workspace_replays_from_a_hip_graph(oracle, dev):
+    """hq_qmatmul_ggml_ws on the f16 tile route (m > 64) allocates nothing, so a prefill step can record it into a
+    HIP graph: three replays with the activations rewritten in between, each checked against the eager call."""
+    m, n, k, t = 96, 384, 1024, HQ_Q4_K
+    w = torch.from_numpy(oracle.quantize(weights(71, n, k), k, t, threads=8)).to(dev)
+    p = GgmlQuantizedMatmulParams(m, n, k, t)
+    need = ops.quantized_matmul_workspace_bytes(p, torch.bfloat16)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    x = torch.zeros(m, k, device=dev, dtype=torch.bfloat16)
+    y = torch.empty(m, n, device=dev)
+    ops.quantized_matmul_ggml(x, w, y, p, workspace=ws)  # warm-up outside the capture (kernel attributes are set here)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            ops.quantized_matmul_ggml(x, w, y, p, workspace=ws)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        x.copy_(torch.from_numpy(acts(80 + rep, m, k)).to(dev).to(torch.bfloat16))
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        eager = torch.empty_like(y)
+        ops.quantized_matmul_ggml(x, w, eager, p, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay {rep}"
+        assert torch.isfinite(got).all()

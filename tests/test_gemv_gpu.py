@@ -38,6 +38,13 @@ def test_dequant_bit_exact(oracle, dev, t):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     got16 = ops.dequantize_ggml(wd, n, t, torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16)
     assert np.array_equal(got16, oracle.f32_to_bf16_bits(want))
+    # the f16 shadow of materialize_f16_shadow (forward_mlx.rs:9426-9440): the f32 value rounded to nearest even
+    goth = ops.dequantize_ggml(wd, n, t, torch.float16).view(torch.int16).cpu().numpy().view(np.uint16)
+    with np.errstate(over="ignore", invalid="ignore"):
+        wanth = want.astype(np.float16)
+    nan = np.isnan(wanth)  # (adversarial raw blocks hold NaN scales: any NaN payload will do)
+    assert np.array_equal(np.isnan(goth.view(np.float16)), nan)
+    assert np.array_equal(goth[~nan], wanth.view(np.uint16)[~nan])
 
 
 @pytest.mark.parametrize("t", ALL_TYPES)

@@ -108,6 +108,11 @@ def test_reader_rejects_malformed_files(tmp_path, tiny):
     # unknown ggml type
     data, _ = W.build([], [("t", [32], 99, bytes(32))])
     assert not opens(data)
+    # an element count whose byte length does not fit 64 bits (F32 = type 0: 2^62 + 8 elements would wrap to 32 bytes)
+    data, _ = W.build([], [("t", [(1 << 62) + 8], 0, bytes(32))])
+    assert not opens(data)
+    data, _ = W.build([], [("t", [1 << 62], 0, bytes(32))])
+    assert not opens(data)
     # general.alignment is honoured
     data, offs = W.build([("general.alignment", W.U32, 64)], [("a", [32], 8, bytes(34)), ("b", [32], 8, bytes(range(34)))], 64)
     p = tmp_path / "a64.gguf"

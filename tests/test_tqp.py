@@ -1,12 +1,13 @@
 """TurboQuant block envelope ("TQP1" / "TQP2"): the library's packer / parser against the oracle
 restatement and against the reference's own known answers (kv_persist/families/tq_packed.rs tests
 :1625-1852 and :2139-2200).  Host code only: runs without a GPU."""
+import ctypes
 import struct
 
 import numpy as np
 import pytest
 
-from hf2q_amd import ops
+from hf2q_amd import lib, ops
 from oracle import tqp
 
 
@@ -81,3 +82,16 @@ def test_rejections():
     h2, _ = _hdr(2, 8, 2, 16, 256)
     with pytest.raises(ops.HqError):                                                       # version 2 needs its norms
         ops.pack_tq_payload(h2, bytes(h2.indices_bytes_len()), b"")
+
+
+def test_stream_lengths_do_not_wrap():
+    """Header fields are 32 bits each: the largest products exceed size_t and must not come back truncated."""
+    L = lib.load()
+    h = lib.TqpHeader()
+    h.codec_version, h.bits_per_coord, h.head_dim, h.n_kv_heads, h.n_tokens = 2, 8, 0xFFFFFF00, 0xFFFFFFFF, 0xFFFFFFFF
+    size_max = ctypes.c_size_t(-1).value
+    assert L.hq_tqp_indices_bytes(ctypes.byref(h)) == size_max
+    assert L.hq_tqp_norms_bytes(ctypes.byref(h)) == size_max
+    assert L.hq_tqp_total_bytes(ctypes.byref(h)) == size_max
+    h.head_dim, h.n_kv_heads, h.n_tokens = 256, 2, 5
+    assert L.hq_tqp_indices_bytes(ctypes.byref(h)) == 2 * 5 * 256 and L.hq_tqp_norms_bytes(ctypes.byref(h)) == 2 * 5 * 4
