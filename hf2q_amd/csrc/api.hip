@@ -154,14 +154,18 @@ static int check_matmul_common(const char* fn, const void* x, hq_act_dtype xdt, 
     return check_weight_alignment(w, t);
 }
 
+#ifndef HQ_CHUNK_LIMIT_Q4K
+#define HQ_CHUNK_LIMIT_Q4K 2
+#endif
 namespace {
 
-// A few rows past the GEMV limit still run in chunks of kGemvMaxRows rows: a tile kernel multiplies 256 token rows
-// whatever m is, so it costs what a dozen passes of the small-batch kernel cost (measured, 12288 x 4096 Q4_K: 211 us
-// for any m <= 256 against 17.5 us per eight rows; 151936 x 4096 Q6_K: 2650 against 339 us), or what two to four
-// rounds of per-row GEMVs cost where there is no small-batch kernel.
+// A few rows past the GEMV limit still run in chunks of kGemvMaxRows rows.  Q4_K / Q5_K have tiles of 64 token rows
+// (one launch for any m <= 128 costs about what two to three chunks cost), the other types only tiles of 256 rows,
+// which cost what a dozen passes of the small-batch kernel cost (151936 x 4096 Q6_K: 2650 us against 339 us per
+// eight rows), or what two to four rounds of per-row GEMVs cost where there is no small-batch kernel.
 uint32_t chunked_rows_limit(uint32_t k, hq_ggml_type t) {
     if (!gemv_rows_supported(t, kGemvMaxRows, k)) return 2 * kGemvMaxRows;
+    if (t == HQ_Q4_K || t == HQ_Q5_K) return HQ_CHUNK_LIMIT_Q4K * kGemvMaxRows;
     return t == HQ_Q6_K ? 6 * kGemvMaxRows : 8 * kGemvMaxRows;
 }
 
@@ -206,7 +210,7 @@ int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const vo
 size_t hq_qmatmul_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
     (void)n;
     (void)xdt;
-    return f16_tile_route(m, k, t) ? gemm_f16_tile_workspace_bytes(m, n, k) : 0;
+    return f16_tile_route(m, k, t) ? gemm_f16_tile_workspace_bytes(m, n, k, t) : 0;
 }
 
 int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
@@ -240,7 +244,7 @@ int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w
 
 size_t hq_qmatmul_perm021_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
     // the tile GEMM gathers while it converts; every other route first copies the activations into row-major order
-    if (f16_tile_route(m, k, t)) return gemm_f16_tile_workspace_bytes(m, n, k);
+    if (f16_tile_route(m, k, t)) return gemm_f16_tile_workspace_bytes(m, n, k, t);
     return (((size_t)m * k * (xdt == HQ_BF16 ? 2 : 4)) + 255) & ~(size_t)255;
 }
 

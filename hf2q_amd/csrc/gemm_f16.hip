@@ -213,6 +213,9 @@ struct GemmArgs {
     // dense form has lay_m = m, lay_n = n, wd_off = 0, row_map = nullptr.
     uint32_t lay_m, lay_n, wd_off;
     const uint32_t* row_map;
+    // Q4_K / Q5_K tiles: the super-blocks [sb0, sb1) of every row that the workgroup multiplies (all of them except
+    // in the split form of the small tiles, whose workgroups each write the partial sums of a slice of k)
+    uint32_t sb0, sb1;
 };
 
 __device__ __forceinline__ f16x8_t as_frag(uint4 v) { return __builtin_bit_cast(f16x8_t, v); }
@@ -222,17 +225,20 @@ typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 __device__ __forceinline__ uint4 ld16(const uint8_t* p) { return *reinterpret_cast<const uint4*>(p); }
 
 constexpr int WAVES = 4;           // one per SIMD; two workgroups share a CU
-constexpr int BM = 256;            // token rows per workgroup
-constexpr int DMA_PER_WAVE = (BM / 8) / WAVES;  // BM / 8 one-KB fetches fill the activation tile
+constexpr int BM = 256;            // token rows per workgroup of the prefill-sized tiles
+constexpr int BM_SMALL = 64;       // ... of the tiles for a few token rows (up to 128)
+constexpr int BM_MID = 128;        // ... of the tiles for sparsely filled experts
 constexpr int BN_WIDE = 128, BN_NARROW = 64;    // weight rows per workgroup
 
 // Activation side of a workgroup tile, the same for every weight type: the pre-pass output goes
-// global -> LDS in 1 KB wave instructions; wave w, instruction i (< DMA_PER_WAVE) fills 8 LDS rows of
-// the tile, (w * DMA_PER_WAVE + i) * 8 .. +8; lane L owns row L/8 of them and LDS chunk L%8, which
+// global -> LDS in 1 KB wave instructions; wave w, instruction i (< kDma) fills 8 LDS rows of
+// the tile, (w * kDma + i) * 8 .. +8; lane L owns row L/8 of them and LDS chunk L%8, which
 // holds global chunk (L%8) ^ ((row/2)%8), and (row/2)%8 = L/16 + 4*(i%2).  Rows past the end of x read
-// the last row instead (their results are never stored).
-struct ActTile {
-    static constexpr int kTile = BM * ROW * 2;  // bytes of one activation buffer; two of them in LDS
+// the last row instead (their results are never stored).  BMT = token rows of the tile.
+template <int BMT>
+struct ActTileT {
+    static constexpr int kDma = (BMT / 8) / WAVES;  // BMT / 8 one-KB fetches fill the activation tile
+    static constexpr int kTile = BMT * ROW * 2;     // bytes of one activation buffer; two of them in LDS
     uint8_t* smem;
     const uint8_t* xtile;
     uint32_t a_swz, a_row0, a_rows_left, a_last, row_pitch, wave_u, lds_base;
@@ -242,7 +248,7 @@ struct ActTile {
         smem = reinterpret_cast<uint8_t*>(smem4);
         row_pitch = a.k * 2u;
         a_swz = ((lane & 7u) ^ (lane >> 4)) << 4;
-        a_row0 = wave * (8u * DMA_PER_WAVE) + (lane >> 3);
+        a_row0 = wave * (8u * kDma) + (lane >> 3);
         a_rows_left = a.m - m0;  // >= 1
         a_last = (a_rows_left - 1u) * row_pitch + a_swz;
         xtile = a.ws + W.xh + (size_t)m0 * row_pitch;
@@ -257,19 +263,21 @@ struct ActTile {
     __device__ __forceinline__ void fetch(uint32_t st, uint32_t buf, int i) const {
         const uint32_t r = a_row0 + 8u * i;
         const uint8_t* src = xtile + (r < a_rows_left ? r * row_pitch + (a_swz ^ ((i & 1u) << 6)) : a_last ^ ((i & 1u) << 6)) + (size_t)st * (BK * 2);
-        const uint32_t dst = lds_base + buf * kTile + (wave_u * DMA_PER_WAVE + i) * 1024u;
+        const uint32_t dst = lds_base + buf * kTile + (wave_u * kDma + i) * 1024u;
         asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
         __builtin_amdgcn_sched_barrier(0);  // one address at a time: keeps eight 64-bit pointers out of the registers
     }
     __device__ __forceinline__ void fetch_all(uint32_t st, uint32_t buf) const {
 #pragma unroll
-        for (int i = 0; i < DMA_PER_WAVE; ++i) fetch(st, buf, i);
+        for (int i = 0; i < kDma; ++i) fetch(st, buf, i);
     }
     // The 8 activations of 16-byte chunk kchunk (of the row's 64 per stage) of tile row `row`.
     __device__ __forceinline__ uint4 frag(uint32_t buf, uint32_t row, uint32_t kchunk) const {
         return *reinterpret_cast<const uint4*>(smem + buf * kTile + row * (ROW * 2) + ((kchunk ^ ((row >> 1) & 7u)) << 4));
     }
 };
+using ActTile = ActTileT<BM>;
+
 
 // Stores a wave's accumulators.  The weights are the MFMA's first operand, so an accumulator tile
 // is indexed [weight row][token]: value v of a lane belongs to token lane%32 and weight row
@@ -322,7 +330,8 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W
 // fifth bit into the masked nibbles, three more VALU instructions per four weights.
 template <int MT, int NT, int WN, int TYPE = HQ_Q4_K>
 __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
-    static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
+    constexpr int BMT = 32 * MT * (WAVES / WN);  // token rows of the workgroup tile: 256, or 64 for the small tiles
+    constexpr int DMA_PER_WAVE = ActTileT<BMT>::kDma;
     constexpr bool Q5 = TYPE == HQ_Q5_K;
     constexpr uint32_t BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES, QS = Q5 ? 48u : 16u;  // super-block size, offset of the nibbles
     const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
@@ -331,9 +340,9 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
 
-    const uint32_t nsb = a.k / 256, nstages = a.k / BK;
-    const uint32_t row_bytes = nsb * BYTES;
-    ActTile at;
+    const uint32_t row_bytes = (a.k / 256) * BYTES;
+    const uint32_t sb0 = a.sb0, sb1 = a.sb1;  // sb0 < sb1
+    ActTileT<BMT> at;
     at.init(a, W, m0, lane, wave);
 
     // ---- weights: this lane's two rows (one per 32-row tile of the wave), bytes 16*lg.. of each chunk ----
@@ -422,11 +431,11 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     static_assert(kSteps >= DMA_PER_WAVE && (E >= MT ? E % MT == 0 : MT % E == 0 && MT / E >= 2), "the spreading below assumes it");
 
     // ---- prologue: everything the first stage needs, and the second stage's nibbles ----
-    load_hdr(0, hdr, hq);
-    load_b(0, 0, 0);
-    if (nstages > 1) load_b(0, 1, 1);  // k >= 256: a super-block has four stages
-    at.fetch_all(0, 0);
-    if (nsb > 1) load_hdr(1, hdrn, hqn);
+    load_hdr(sb0, hdr, hq);
+    load_b(sb0, 0, 0);
+    load_b(sb0, 1, 1);  // a super-block has four stages
+    at.fetch_all(4 * sb0, 0);
+    if (sb0 + 1 < sb1) load_hdr(sb0 + 1, hdrn, hqn);
     float dsc[NT][2], ndm[NT][2];      // scales of the stage being multiplied
     uint4 bfc[NT], bfn[NT];            // weight fragments: current k-step, next
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -438,13 +447,13 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     // The loop is software pipelined over stages as well: while the last k-step of stage s is
     // multiplied, the scales of stage s+1 and the fragments of its first k-step are formed, so a
     // stage begins with an MFMA and not with sixty VALU instructions that nothing overlaps.
-    for (uint32_t sblk = 0; sblk < nsb; ++sblk) {
-        const bool next_sb = sblk + 1 < nsb;  // uniform
+    for (uint32_t sblk = sb0; sblk < sb1; ++sblk) {
+        const bool next_sb = sblk + 1 < sb1;  // uniform
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t st = 4 * sblk + c;
             const uint32_t buf = c & 1;
-            const bool has_next = c < 3 || next_sb;  // uniform: stage st + 1 exists
+            const bool has_next = c < 3 || next_sb;  // uniform: stage st + 1 belongs to this workgroup
             // The next stage's nibbles, requested a stage ago.  They are claimed here, before this
             // stage's activation fetches are issued: the compiler does not know about those, and the
             // wait it puts in front of the first use of these registers would otherwise cover them too.
@@ -454,7 +463,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                 bnext[nt] = braw[(c + 1) & 3][nt];
                 asm volatile("" : "+v"(bnext[nt].x), "+v"(bnext[nt].y), "+v"(bnext[nt].z), "+v"(bnext[nt].w));
             }
-            if (c == 0 && sblk > 0) {  // this super-block's header; request the next one
+            if (c == 0 && sblk > sb0) {  // this super-block's header; request the next one
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     hdr[nt] = hdrn[nt];
@@ -469,7 +478,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
             } else if (next_sb) {
                 load_b(sblk + 1, c - 2, (c + 2) & 3);
             }
-            const bool fetch_a = st + 1 < nstages;  // uniform
+            const bool fetch_a = has_next;
 
             auto a_frag = [&](int t) -> uint4 {
                 const int ks = t / MT, mt = t % MT;
@@ -557,6 +566,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 // so it keeps its alignment case here too.  w = d * (q - 8).
 template <int MT, int WN, int TYPE = HQ_Q8_0>
 __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
+    constexpr int DMA_PER_WAVE = ActTile::kDma;
     static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
     constexpr bool Q4 = TYPE == HQ_Q4_0;
     constexpr uint32_t BYTES = Q4 ? Q4_0_BYTES : Q8_0_BYTES;
@@ -686,6 +696,7 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 // hardware takes the unaligned 16-byte loads.
 template <int MT, int WN>
 __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
+    constexpr int DMA_PER_WAVE = ActTile::kDma;
     static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
     const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -830,6 +841,45 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_kernel(GemmArgs a, uin
     }
 }
 
+// 9 .. 128 token rows: tiles of 64 token rows x 64 weight rows (2 x 2 waves of 32 x 32), so that a few rows do not
+// pay for 256 and the weight rows spread over the CUs (12288 rows: 192 workgroups per token tile).  Where that is
+// still less than a workgroup per CU, k is cut into `splits` slices of sb_per super-blocks, each with workgroups of
+// its own that store their products into slice `s` of `partial` ([splits][m][n] floats, same scaling as y);
+// split_sum_kernel then adds the slices in order.
+template <int TYPE>
+__global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_small_kernel(GemmArgs a, uint32_t splits, uint32_t sb_per,
+                                                                       float* __restrict__ partial) {
+    // consecutive workgroups (which the hardware deals to the XCDs in turn) take consecutive weight-row tiles
+    const uint32_t tiles_n = (a.n + BN_NARROW - 1) / BN_NARROW, tiles_m = (a.m + BM_SMALL - 1) / BM_SMALL;
+    const uint32_t s = blockIdx.x / (tiles_n * tiles_m), t = blockIdx.x % (tiles_n * tiles_m);
+    if (splits > 1) {
+        a.sb0 = s * sb_per;
+        a.sb1 = a.sb0 + sb_per < a.sb1 ? a.sb0 + sb_per : a.sb1;
+        a.y = partial + (size_t)s * a.m * a.n;
+    }
+    q4k_gemm_tile<1, 1, 2, TYPE>(a, (t / tiles_n) * BM_SMALL, (t % tiles_n) * BN_NARROW);
+}
+
+// y[i] = partial[0][i] + partial[1][i] + ... in this order, whatever order the slices were written in.
+__global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict__ partial, float* __restrict__ y, uint32_t count,
+                                                        uint32_t splits) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= count) return;
+    float v = partial[i];
+    for (uint32_t s = 1; s < splits; ++s) v += partial[(size_t)s * count + i];
+    y[i] = v;
+}
+
+// Slices of k for the small tiles: doubled while the grid has fewer workgroups than the device has CUs (256) and a slice
+// keeps at least four super-blocks (sixteen stages, so that its prologue and epilogue stay a fraction of its work).
+inline uint32_t small_tile_splits(uint32_t m, uint32_t n, uint32_t k) {
+    const uint64_t tiles = (uint64_t)((m + BM_SMALL - 1) / BM_SMALL) * ((n + BN_NARROW - 1) / BN_NARROW);
+    const uint32_t nsb = k / 256;
+    uint32_t s = 1;
+    while (s < 4 && tiles * s < 256 && nsb / (2 * s) >= 4) s *= 2;
+    return s;
+}
+
 __global__ __launch_bounds__(64 * WAVES, 2) void q6k_gemm_kernel(GemmArgs a) {
     const uint32_t tiles_m = (a.m + BM - 1) / BM;
     uint32_t m0, n0;
@@ -858,7 +908,7 @@ struct GroupedLayout {
 __host__ __device__ inline GroupedLayout grouped_layout(uint32_t pairs, uint32_t n_experts, uint32_t n, uint32_t k) {
     GroupedLayout g;
     g.base = workspace_layout(pairs, n_experts * n, k);
-    g.max_tiles = pairs / BM + n_experts;
+    g.max_tiles = pairs / BM_SMALL + n_experts;  // enough for tiles of 64 rows or more
     g.row_map = g.base.total;
     g.tiles = g.row_map + (((size_t)pairs * 4 + 255) & ~(size_t)255);
     g.count = g.tiles + (((size_t)g.max_tiles * 16 + 255) & ~(size_t)255);
@@ -873,7 +923,8 @@ constexpr uint32_t BUCKET_MAX_EXPERTS = 1024;  // one expert per thread of the s
 // on the order in which the atomics land; every output row is computed on its own, so the results do not.
 __global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __restrict__ ids, uint32_t pairs, uint32_t n_experts,
                                                           uint32_t* __restrict__ row_map, uint4* __restrict__ tiles,
-                                                          uint32_t* __restrict__ n_tiles, float* __restrict__ y, uint32_t n) {
+                                                          uint32_t* __restrict__ n_tiles, float* __restrict__ y, uint32_t n,
+                                                          uint32_t bm) {
     __shared__ uint32_t cnt[BUCKET_MAX_EXPERTS], cur[BUCKET_MAX_EXPERTS];
     const uint32_t tid = threadIdx.x;
     for (uint32_t e = tid; e < n_experts; e += 1024) cnt[e] = 0;
@@ -886,7 +937,7 @@ __global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __rest
     // Exclusive prefix sums over the experts of (rows, tiles), one expert per thread (n_experts <= 1024 = the
     // workgroup): inside a wave by shuffles, across the sixteen waves through LDS.  Expert e then writes its own tiles.
     __shared__ uint32_t wave_rows[16], wave_tiles[16];
-    const uint32_t my_rows = tid < n_experts ? cnt[tid] : 0u, my_tiles = (my_rows + BM - 1) / BM;
+    const uint32_t my_rows = tid < n_experts ? cnt[tid] : 0u, my_tiles = (my_rows + bm - 1) / bm;
     uint32_t inc_rows = my_rows, inc_tiles = my_tiles;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -903,7 +954,7 @@ __global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __rest
     }
     if (tid < n_experts) {
         cur[tid] = off;
-        for (uint32_t r = 0; r < my_rows; r += BM) tiles[first_tile + r / BM] = make_uint4(tid, off + r, off + my_rows, 0u);
+        for (uint32_t r = 0; r < my_rows; r += bm) tiles[first_tile + r / bm] = make_uint4(tid, off + r, off + my_rows, 0u);
     }
     if (tid == 0) *n_tiles = total_tiles;
     __syncthreads();
@@ -919,7 +970,7 @@ __global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __rest
     for (uint32_t r = total_rows + tid; r < pairs; r += 1024) row_map[r] = 0;
 }
 
-template <int TYPE>
+template <int TYPE, bool SMALL>
 __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a, const uint4* __restrict__ tiles,
                                                                       const uint32_t* __restrict__ n_tiles, uint32_t tiles_n,
                                                                       uint64_t expert_stride) {
@@ -929,7 +980,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
     a.w += (size_t)tt.x * expert_stride;
     a.wd_off = tt.x * a.n;
     a.m = tt.z;  // rows past the expert's run repeat its last row and are not stored
-    if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
+    if constexpr (SMALL)
+        q4k_gemm_tile<4, 1, 4, TYPE>(a, tt.y, n0);  // 128 routed rows x 128 weight rows (Q4_K / Q5_K), a wave 128 x 32
+    else if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
         q4k_gemm_tile<8, 1, 4, TYPE>(a, tt.y, n0);
     else if constexpr (TYPE == HQ_Q6_K)
         q6k_gemm_tile<8, 4>(a, tt.y, n0);
@@ -939,7 +992,16 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
 
 }  // namespace
 
-size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) { return workspace_layout(m, n, k).total; }
+bool gemm_f16_small_tiles(hq_ggml_type t, uint32_t m) { return (t == HQ_Q4_K || t == HQ_Q5_K) && m <= 2 * BM_SMALL; }
+
+size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
+    size_t total = workspace_layout(m, n, k).total;
+    if (gemm_f16_small_tiles(t, m)) {  // partial sums of the slices of k
+        const uint32_t splits = small_tile_splits(m, n, k);
+        if (splits > 1) total += (size_t)splits * m * n * 4;
+    }
+    return total;
+}
 
 bool gemm_f16_grouped_supported(hq_ggml_type t, uint32_t n, uint32_t k, uint32_t n_experts, uint64_t expert_stride, uint64_t pairs) {
     if (!gemm_f16_tile_supported(t, k) || n_experts > BUCKET_MAX_EXPERTS || pairs > 0x7fffffffull / 4) return false;
@@ -976,16 +1038,24 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     uint32_t* row_map = reinterpret_cast<uint32_t*>(ws + G.row_map);
     uint4* tiles = reinterpret_cast<uint4*>(ws + G.tiles);
     uint32_t* n_tiles = reinterpret_cast<uint32_t*>(ws + G.count);
-    hipLaunchKernelGGL(moe_bucket_kernel, dim3(1), dim3(1024), 0, s, ids, pairs, n_experts, row_map, tiles, n_tiles, y, n);
+    // Experts with few rows each (Qwen3.6-35B-A3B: 2048 tokens x top-8 over 256 experts = 64 rows per expert) take tiles
+    // of 64 routed rows; the 256-row tiles would run a quarter full.
+    constexpr bool HAS_SMALL = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K;
+    const bool small = HAS_SMALL && (uint64_t)pairs < (uint64_t)n_experts * 160u;
+    const uint32_t bm = small ? BM_MID : BM, bn = BN_WIDE;
+    hipLaunchKernelGGL(moe_bucket_kernel, dim3(1), dim3(1024), 0, s, ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm);
     if (int rc = check_launch("expert bucket kernel launch")) return rc;
     if (int rc = launch_prep<TYPE>(s, x, xdt, wb, ws, pairs, n_experts * n, k, row_map, top_k)) return rc;
-    constexpr int lds = 2 * ActTile::kTile;
-    auto kern = grouped_gemm_kernel<TYPE>;
+    const int lds = 2 * (small ? ActTileT<BM_MID>::kTile : ActTile::kTile);
+    void (*kern)(GemmArgs, const uint4*, const uint32_t*, uint32_t, uint64_t) = grouped_gemm_kernel<TYPE, false>;
+    if constexpr (HAS_SMALL)
+        if (small) kern = grouped_gemm_kernel<TYPE, true>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;
-    GemmArgs a{ws, wb, y, pairs, n, k, pairs, n_experts * n, 0u, row_map};
-    const uint32_t tiles_n = (n + BN_WIDE - 1) / BN_WIDE;
-    hipLaunchKernelGGL(kern, dim3(G.max_tiles * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
+    GemmArgs a{ws, wb, y, pairs, n, k, pairs, n_experts * n, 0u, row_map, 0u, k / 256};
+    const uint32_t tiles_n = (n + bn - 1) / bn;
+    const uint32_t max_tiles = pairs / bm + n_experts;
+    hipLaunchKernelGGL(kern, dim3(max_tiles * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
     return check_launch("grouped gemm kernel launch");
 }
 
@@ -1012,7 +1082,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
                          uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const uint8_t* wb = static_cast<const uint8_t*>(w);
-    GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr};
+    GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr, 0u, k / 256};
     constexpr int lds = 2 * ActTile::kTile;
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
@@ -1033,10 +1103,22 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         hipLaunchKernelGGL(kern, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
         return check_launch("q8_0 gemm kernel launch");
     }
-    void (*kern)(GemmArgs, uint32_t, uint32_t) = t == HQ_Q5_K ? q4k_gemm_kernel<HQ_Q5_K> : q4k_gemm_kernel<HQ_Q4_K>;
     if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
                               : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
         return rc;
+    if (gemm_f16_small_tiles(t, m)) {  // up to two token tiles of 64 rows
+        void (*ksmall)(GemmArgs, uint32_t, uint32_t, float*) = t == HQ_Q5_K ? q4k_gemm_small_kernel<HQ_Q5_K> : q4k_gemm_small_kernel<HQ_Q4_K>;
+        const uint32_t tm = (m + BM_SMALL - 1) / BM_SMALL, tn = (n + BN_NARROW - 1) / BN_NARROW;
+        const uint32_t splits = small_tile_splits(m, n, k), nsb = k / 256, sb_per = (nsb + splits - 1) / splits;
+        float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
+        hipLaunchKernelGGL(ksmall, dim3(tm * tn * splits), dim3(64 * WAVES), 2 * ActTileT<BM_SMALL>::kTile, s, a, splits, sb_per, partial);
+        if (int rc = check_launch("q4k small gemm kernel launch")) return rc;
+        if (splits == 1) return HQ_OK;
+        const uint32_t count = m * n;  // m <= 128
+        hipLaunchKernelGGL(split_sum_kernel, dim3((count + 255u) / 256u), dim3(256), 0, s, partial, y, count, splits);
+        return check_launch("split sum kernel launch");
+    }
+    void (*kern)(GemmArgs, uint32_t, uint32_t) = t == HQ_Q5_K ? q4k_gemm_kernel<HQ_Q5_K> : q4k_gemm_kernel<HQ_Q4_K>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(q4k gemm LDS)"))
         return rc;
     // Tiles of 128 weight rows; tiles of 64 when the wide ones would occupy at most half of the CUs.

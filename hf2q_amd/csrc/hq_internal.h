@@ -68,7 +68,7 @@ int launch_gemm(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, f
 // GEMM on the f16 matrix cores with an activation pre-pass (Q4_K with k % 256 == 0, Q8_0 with
 // k % 128 == 0); needs a device workspace of gemm_f16_tile_workspace_bytes().
 bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k);
-size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t);
 // perm_hd != 0: the activations are stored [k / perm_hd][m][perm_hd] (attention output, heads outermost) and are
 // gathered by the pre-pass.
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,

@@ -50,6 +50,23 @@ def test_gemm_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
     _check(t, k)(y, ref, f"gemm t={t} {xdt} {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K])
+@pytest.mark.parametrize("m,n,k", [
+    (17, 64, 2048),     # one tile of 64 x 64, k in two slices
+    (65, 130, 2304),    # two token tiles, ragged weight rows, nine super-blocks in slices of five and four
+    (128, 70, 4352),    # seventeen super-blocks in four slices (5, 5, 5, 2)
+    (100, 320, 256),    # a single super-block: no slices
+    (64, 12288, 512),   # more tiles than CUs' worth: no slices
+])
+def test_small_tiles_and_k_slices_match_f64_oracle(oracle, dev, t, m, n, k):
+    """17 .. 128 activation rows of Q4_K / Q5_K: tiles of 64 token rows, with k cut into slices (summed in a fixed
+    order by a second launch) where the tiles alone would leave most CUs idle; the same result on every call."""
+    y, ref = _run(oracle, dev, t, "bf16", m, n, k)
+    assert_matmul_close_f16_tile(y, ref, f"small tiles t={t} {m}x{n}x{k}")
+    y2, _ = _run(oracle, dev, t, "bf16", m, n, k)
+    assert np.array_equal(y, y2)
+
+
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
 def test_gemm_adversarial_blocks(oracle, dev, t):
     """Every scale / min / nibble bit pattern (raw random bytes with finite f16 fields)."""

@@ -249,6 +249,7 @@ GROUPED_CASES = [  # (E, n, k, T, K): at least 8 routed rows per expert and 256 
     (4, 160, 256, 400, 3),     # 300 rows per expert: two tiles each, n not a multiple of the tile
     (16, 64, 1024, 300, 1),    # the down-projection calling form
     (3, 256, 512, 700, 2),     # several full tiles
+    (6, 200, 768, 150, 5),     # about 125 rows per expert: tiles of 128 rows, two for the experts above that
 ]
 
 
@@ -367,12 +368,13 @@ def test_small_batch_rows_tall_matrix(oracle, dev, t, xdt, m):
     assert_matmul_close(y.cpu().numpy(), ref, f"rows, tall matrix t={t} {xdt} m={m}")
 
 
-@pytest.mark.parametrize("t,m,k", [(HQ_Q4_K, 9, 2048), (HQ_Q4_K, 41, 1024), (HQ_Q5_K, 64, 1024), (HQ_Q6_K, 18, 2048),
+@pytest.mark.parametrize("t,m,k", [(HQ_Q4_K, 9, 2048), (HQ_Q4_K, 16, 1024), (HQ_Q5_K, 16, 1024), (HQ_Q6_K, 18, 2048),
                                    (HQ_Q6_K, 48, 1024), (HQ_Q8_0, 13, 1024), (HQ_Q4_K, 15, 768)])
 def test_a_few_rows_past_eight_run_in_chunks_of_eight(oracle, dev, t, m, k):
-    """Up to 64 (Q4_K / Q5_K), 48 (Q6_K) or 16 rows (no small-batch kernel for the type or k) do not take a 256-row
-    tile: chunks of eight through the small-batch kernel, the remainder through it or the GEMV.  Every product is
-    exact on this route, so the GEMV's tolerance holds, and no scratch is asked for."""
+    """Up to 16 (Q4_K / Q5_K, which have tiles of 64 token rows beyond that), 48 (Q6_K) or 16 rows (no small-batch
+    kernel for the type or k) do not take a tile kernel: chunks of eight through the small-batch kernel, the remainder
+    through it or the GEMV.  Every product is exact on this route, so the GEMV's tolerance holds, and no scratch is
+    asked for."""
     n = 136
     blocks = oracle.quantize(weights(m + k + t, n, k), k, t, threads=8)
     x = acts(m + t, m, k)
