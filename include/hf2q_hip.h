@@ -5,8 +5,11 @@
  * Conventions (they mirror the contract hf2q's call sites have with their GPU
  * backend today):
  *   - every buffer pointer is a DEVICE pointer owned by the caller; nothing is
- *     allocated, freed or retained by the library (hf2q passes caller-owned
- *     MlxBuffers and scratch the same way, gpu_ffn.rs:194-204, 644-648);
+ *     retained by the library (hf2q passes caller-owned MlxBuffers and scratch
+ *     the same way, gpu_ffn.rs:194-204, 644-648).  Two entry points allocate
+ *     stream-ordered scratch of their own for prefill-sized inputs and say so
+ *     (hq_qmatmul_ggml, hq_qmatmul_id_ggml without scratch never does); their
+ *     _ws forms take the scratch from the caller and allocate nothing;
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
  *     Work is enqueued in order on it and the call returns at once, like an
  *     encoder dispatch without commit; the caller synchronises.  An in-order
@@ -16,8 +19,14 @@
  *   - every function returns HQ_OK (0) or an hq_status error code and never
  *     aborts; the message is available from hq_last_error() on the same thread
  *     ("fail loud", kv_cache.rs:152-153);
- *   - functions are re-entrant per stream; the only library state is the
- *     thread-local error string.
+ *   - functions are re-entrant per stream; the library's state is the
+ *     thread-local error string, a per-device note of which kernels had their
+ *     LDS limit raised, and the static device scratch of
+ *     hq_flash_attn_vec_tq_static (shared by every call on a GPU);
+ *   - data-dependent conditions are not errors: an expert id >= n_experts
+ *     gives NaN output rows for that (token, slot), never an out-of-bounds read
+ *     and never a status code (the ids live on the device and are not read by
+ *     the host); hq_tq_attn_params.nsg is accepted and ignored.
  *
  * Paths cited below are relative to the hf2q source tree.
  */
@@ -87,7 +96,8 @@ HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, ui
  * (src/inference/models/qwen35/gpu_ffn.rs:1236-1245; dispatch_qmatmul,
  * src/serve/forward_mlx.rs:9655-9969).  m <= 8 takes the bandwidth-bound GEMV
  * kernels (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791) and so do a few more rows, eight at a
- * time (up to 16 .. 64, by type: a tile kernel multiplies 256 token rows whatever m is); larger m the
+ * time (up to 16 for Q4_K / Q5_K, whose MFMA GEMM has tiles of 64 token rows for 17 .. 128 rows; up to
+ * 48 for Q6_K and 64 for Q8_0 / Q4_0, whose tiles multiply 256 token rows whatever m is); larger m the
  * MFMA GEMM.  The K-quant (k % 256 == 0) and Q8_0 / Q4_0 (k % 128 == 0) GEMMs multiply f16-rounded
  * weights and activations like the reference's mul_mm, the other kernels keep
  * every product exact.
@@ -98,8 +108,9 @@ HQ_API int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const 
 
 /* The same product with caller-owned device scratch.  The f16 tile kernels
  * (prefill-sized m; K-quants with k % 256 == 0, Q8_0 / Q4_0 with k % 128 == 0) convert the
- * activations to row-scaled f16 in a pre-pass and needs hq_qmatmul_ggml_workspace_bytes() bytes (256-byte
- * aligned) for them; every other shape needs none (the function returns 0 and
+ * activations to row-scaled f16 in a pre-pass and need hq_qmatmul_ggml_workspace_bytes() bytes (256-byte
+ * aligned) for them -- plus, for 17 .. 128 rows of Q4_K / Q5_K over few weight rows, the partial sums of
+ * the slices k is cut into, which a second launch adds in a fixed order; every other shape needs none (the function returns 0 and
  * `workspace` may be null).  hq_qmatmul_ggml itself takes that scratch from the
  * stream-ordered allocator (hipMallocAsync / hipFreeAsync on `stream`).  The
  * reference has no such buffer: its mul_mm kernel (quantized_matmul_ggml's
@@ -145,7 +156,10 @@ HQ_API int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, con
                        uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
 
 /* Bytes of `scratch` the GEMV form needs for up to `max_rows` = n_tokens*top_k
- * routed rows (the IdMmScratch analogue, decode_pool.rs:56-60): none. */
+ * routed rows (the IdMmScratch analogue, decode_pool.rs:56-60): always 0.  Kept
+ * so that a port of the reference's scratch sizing call has something to call;
+ * new code asks hq_qmatmul_id_ggml_workspace_bytes(), which returns what the
+ * grouped (prefill) form needs and 0 where the GEMV form runs. */
 HQ_API size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows);
 /* Bytes of `scratch` for this call's shape: 0 where the GEMV form is used, else
  * the grouped form's workspace (sorted f16 activations, row and weight-row
