@@ -42,6 +42,18 @@ __device__ __forceinline__ void apply_signs(float (&v)[4], uint32_t lane) {
         if ((bits >> e) & 1u) v[e] = -v[e];
 }
 
+// The same from literals instead of a table in memory, for kernels that have many loads in flight when they reach the
+// rotation (a wave's loads return in order: a table fetch would wait for all of them).  Word w holds bytes 4w..4w+3.
+__device__ __forceinline__ void apply_signs_inline(float (&v)[4], uint32_t lane) {
+    const uint32_t w = lane >> 3;
+    const uint32_t lo = w & 2u ? (w & 1u ? 0x1cea4589u : 0xd6247fb3u) : (w & 1u ? 0x0e58c26du : 0xf4913ba7u);
+    const uint32_t hi = w & 2u ? (w & 1u ? 0xdb2c854au : 0xfe19c476u) : (w & 1u ? 0x3de10b97u : 0x52d8af63u);
+    const uint32_t bits = (w & 4u ? hi : lo) >> (4u * (lane & 7u));  // elements 4l..4l+3
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        if ((bits >> e) & 1u) v[e] = -v[e];
+}
+
 // Normalised Walsh-Hadamard transform of 256 elements held 4 per lane.  Stages
 // run in the order h = 1, 2, 4, ... 128 with (a, b) -> (a+b, a-b) on the pair
 // (j, j+h), the same operations in the same order as the plain iterative form,
@@ -529,8 +541,9 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
     struct Tile {
         uint4 k[NB][2][4];  // block, half, i: code bytes 64i + 16g .. +15 of position j
         uint4 v[8];         // positions 4g..4g+3 of half 0, then of half 1; coordinates 16j.. of block ob
-        float kn[NB][2];    // norm_k of position j, -1 where the position is past the end
-        float vn[2];        // norm_v of block ob, 0 where the position is past the end
+        float kn[NB][2];    // norm_k of position j
+        float vn[2];        // norm_v of block ob
+        uint32_t keep[2];   // all ones, or 0 where the position is past the end (the norms then read as -1 and 0)
     };
     // Cache row of logical position idx; positions past the end of the split read a valid row and get
     // weight 0.  RING: rows start at ring_start and wrap (ring_start, idx < kv_capacity); otherwise
@@ -548,15 +561,18 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
             const uint32_t idx = tile0 + 16u * hf + j;
-            const bool ok = idx < split_end;
+            const uint32_t keep = idx < split_end ? 0xffffffffu : 0u;
             const uint32_t row = head_base + row_of(idx);
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const uint4* kp = reinterpret_cast<const uint4*>(a.k_codes + (row * ROW + (uint32_t)(HD * b) + 16u * g));
                 t.k[b][hf][0] = kp[0], t.k[b][hf][1] = kp[4], t.k[b][hf][2] = kp[8], t.k[b][hf][3] = kp[12];
-                t.kn[b][hf] = ok ? a.k_norms[row * NB + b] : -1.f;
+                // (no select here: it lets the compiler put the load under a branch, and it then waits for every
+                // load in flight where the branch ends; the row is a valid one either way, attend() masks it)
+                t.kn[b][hf] = a.k_norms[row * NB + b];
             }
-            t.vn[hf] = ok ? a.v_norms[row * NB + ob] : 0.f;
+            t.vn[hf] = a.v_norms[row * NB + ob];
+            t.keep[hf] = keep;
         }
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
@@ -566,27 +582,45 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
         }
     };
 
-    // Everything the first two iterations need is requested before anything else: at the usual context
-    // lengths that is all of the wave's share, and its trip from HBM overlaps the staging of the queries.
+    // The queries are requested first and the cache rows of the first iteration right after them: a wave's loads
+    // return in the order they were issued, so the queries arrive ahead of the rows and their staging overlaps the
+    // rows' trip from HBM.
+    // Fused rotation: thread tid takes float4 chunks tid, tid + 256, ... of the 8 x ROW staged values; otherwise
+    // head tid / 32, values 8 (tid % 32) .. +7 of every block.
+    constexpr int QV = 2 * NB;
+    float4 qv[QV];
+#pragma unroll
+    for (int r = 0; r < QV; ++r) {
+        // No branch around the loads (the compiler would wait for them where the branches join, before the cache
+        // rows are requested): heads past the chunk's last read that one and are zeroed by an AND.
+        const uint32_t i = tid + 256u * r;
+        const uint32_t hh = a.fuse_fwht_pre ? i / (ROW / 4) : tid >> 5;
+        const uint32_t off = a.fuse_fwht_pre ? 4u * (i % (ROW / 4)) : (uint32_t)HD * (r >> 1) + 8u * (tid & 31u) + 4u * (r & 1);
+        const uint4 raw = *reinterpret_cast<const uint4*>(a.q + (size_t)(h0 + min(hh, nh - 1u)) * ROW + off);
+        const uint32_t keep = hh < nh ? 0xffffffffu : 0u;
+        qv[r] = make_float4(__uint_as_float(raw.x & keep), __uint_as_float(raw.y & keep), __uint_as_float(raw.z & keep),
+                            __uint_as_float(raw.w & keep));
+    }
+    // The second iteration's rows are requested after the queries have been staged: a wave stalls in the issue of a
+    // load while the memory pipeline is full, and the first iteration's rows of the four waves fill it on their own
+    // (80 KB per CU), so asking for more up front only delays the staging.
     Tile tile_a, tile_b;
     load_tile(0, tile_a);
-    if (n_iter > 1) load_tile(1, tile_b);
 
     // ---- queries: every 256-block of a head scaled on its own and split into f16 hi + lo; thread =
     // head tid/32, chunk tid%32 of 8 values; rows are padded to 33 chunks against bank conflicts ----
     if (a.fuse_fwht_pre) {  // sign x FWHT of every block in LDS first
-        for (uint32_t i = tid; i < 8 * ROW / 4; i += 256) {
-            const uint32_t hh = i / (ROW / 4), c = i % (ROW / 4);
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (hh < nh) v = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + hh) * ROW)[c];
-            reinterpret_cast<float4*>(&s_q[hh][0])[c] = v;
+#pragma unroll
+        for (int r = 0; r < QV; ++r) {
+            const uint32_t i = tid + 256u * r;
+            reinterpret_cast<float4*>(&s_q[i / (ROW / 4)][0])[i % (ROW / 4)] = qv[r];
         }
         __syncthreads();
         for (uint32_t hb = wave; hb < 8 * NB; hb += 4) {
             float4* p = reinterpret_cast<float4*>(&s_q[hb / NB][HD * (hb % NB)]) + lane;
             const float4 t = *p;
             float v[4] = {t.x, t.y, t.z, t.w};
-            apply_signs(v, lane);
+            apply_signs_inline(v, lane);
             fwht256(v, lane);
             *p = make_float4(v[0], v[1], v[2], v[3]);
         }
@@ -598,9 +632,8 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
         if (a.fuse_fwht_pre) {
             v0 = *reinterpret_cast<const float4*>(&s_q[h][HD * b + 8 * ch]), v1 = *reinterpret_cast<const float4*>(&s_q[h][HD * b + 8 * ch + 4]);
-        } else if (h < nh) {
-            const float4* qp = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + h) * ROW + HD * b + 8 * ch);
-            v0 = qp[0], v1 = qp[1];
+        } else {
+            v0 = qv[2 * b], v1 = qv[2 * b + 1];
         }
         const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
         float amax = 0.f;
@@ -652,6 +685,7 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
         sscale[b] = s_unscale[b][j & 7u] * a.scale;
     }
     const bool lo_lane = j >= 8u;
+    if (n_iter > 1) load_tile(1, tile_b);
 
     const uint32_t magic = 0x0000e464u;
     // two bytes of one word -> two f16 (1024 + byte, -(1024 + byte)): bytes 0, 1 with sel 0x05010400; 2, 3 with 0x05030402
@@ -672,6 +706,15 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
     constexpr float LOG2E = 1.4426950408889634f;
 
     auto attend = [&](const Tile& cur) {
+        // positions past the end: norm_k = -1 (score -inf), norm_v = 0 (no weight)
+        float kn[NB][2], vn[2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                kn[b][hf] = __uint_as_float((__float_as_uint(cur.kn[b][hf]) & cur.keep[hf]) | (0xbf800000u & ~cur.keep[hf]));
+            vn[hf] = __uint_as_float(__float_as_uint(cur.vn[hf]) & cur.keep[hf]);
+        }
         // -------- scores: two independent accumulation chains per half --------
         float s[8], lv[8];
 #pragma unroll
@@ -697,15 +740,15 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const float part = (c0[v] + c1[v]) - corr[b];
-                    dot[v] += (part + row_xor8(part)) * (sscale[b] * __shfl(cur.kn[b][hf], 4 * g + v));
+                    dot[v] += (part + row_xor8(part)) * (sscale[b] * __shfl(kn[b][hf], 4 * g + v));
                 }
             }
-            const float lvn_own = __log2f(cur.vn[hf]);  // log 0 = -inf: no weight in the numerator
+            const float lvn_own = __log2f(vn[hf]);  // log 0 = -inf: no weight in the numerator
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int src = 4 * g + v;
                 lv[4 * hf + v] = __shfl(lvn_own, src);
-                s[4 * hf + v] = __shfl(cur.kn[0][hf], src) >= 0.f ? dot[v] : -INFINITY;
+                s[4 * hf + v] = __shfl(kn[0][hf], src) >= 0.f ? dot[v] : -INFINITY;
             }
         }
         if (a.softcap != 0.f) {
@@ -778,10 +821,14 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
             }
         }
     };
-    for (uint32_t it = 0; it < n_iter; ++it) {
+    // the two tiles swap roles from iteration to iteration (copying one into the other costs a move per register)
+    for (uint32_t it = 0; it < n_iter; it += 2) {
         attend(tile_a);
-        if (it + 1 < n_iter) tile_a = tile_b;
-        if (it + 2 < n_iter) load_tile(it + 2, tile_b);
+        if (it + 2 < n_iter) load_tile(it + 2, tile_a);
+        if (it + 1 < n_iter) {
+            attend(tile_b);
+            if (it + 3 < n_iter) load_tile(it + 3, tile_b);
+        }
     }
 
     // ---- merge of the four waves.  First the maxima, so that every wave can bring its own numbers to
