@@ -37,11 +37,15 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 # for a device copy of known size (--calibration-copy): FETCH_SIZE reads half the bytes (factor
 # 2.0), WRITE_SIZE all of them (1.0).  The runs and their figures are in profiles/*_pmc_traffic.md.
 PMC_TRAFFIC_BYTES = {
-    "gemv_head_q6_k_151936x4096": int(249387.5 * 2.0 * 1024 + 755.3 * 1.0 * 1024),
+    # (FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0) x 1024 per dispatch
+    "gemv_head_q6_k_151936x4096": int(256455.0 * 2.0 * 1024 + 5151.7 * 1.0 * 1024),
     # activation pre-pass + tile GEMM, Q4_K, 2048 x 12288 x 4096 (the GEMM re-fetches the weights once per 256-token tile)
-    "prefill_gemm_q4_k_2048x12288x4096": int((23122.3 + 132689.9) * 2.0 * 1024 + (16496.3 + 98314.0) * 1.0 * 1024),
+    "prefill_gemm_q4_k_2048x12288x4096": int((23301.6 + 132573.1) * 2.0 * 1024 + (16496.5 + 98311.8) * 1.0 * 1024),
     # split (with the q rotation) + merge (with the output rotation), 32K context, 2 kv heads, head_dim 256
-    "tq_attention_32k_fused_chain": int((16834.8 + 1072.5) * 2.0 * 1024 + (2112.0 + 16.0) * 1.0 * 1024),
+    "tq_attention_32k_fused_chain": int((16897.5 + 1072.5) * 2.0 * 1024 + (2112.0 + 16.0) * 1.0 * 1024),
+    # the one-launch MoE FFN block, hidden 2048, 256 experts x 512, top-8, 1 and 8 tokens
+    "moe_ffn_decode_t1": int(8711.3 * 2.0 * 1024 + 160.1 * 1.0 * 1024),
+    "moe_ffn_decode_t8": int(56290.7 * 2.0 * 1024 + 1280.8 * 1.0 * 1024),
 }
 
 
@@ -260,8 +264,9 @@ def bench_moe_decode(a, tokens=None):
                                f"{'launched from the host' if a.no_graph else 'replayed as a HIP graph'}",
                    "distinct_experts_per_layer": round(u, 1), "bytes_per_layer": int(step_bytes),
                    "layers_rotated": n_layers},
-        "roofline": {"bound": "hbm", "kernel": "MoE FFN layer (all launches)", "achieved": round(gbs, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+        "roofline": {"bound": "hbm", "kernel": "MoE FFN layer (hq_moe_ffn_decode, one launch)", "achieved": round(gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": PMC_TRAFFIC_BYTES.get(f"moe_ffn_decode_t{T}"),
                      "us_per_launch": round(layer_us, 3), "bytes_per_launch": int(step_bytes)}})
 
 
