@@ -84,6 +84,18 @@ def test_prefill_gemm_full_size(oracle, dev, t):
     ref = oracle.qmatmul_f64(oracle.f32_to_bf16_bits(xs), _rows_of(w, rows, k, t, oracle), toks.size, rows.size, k, t)
     got = y[torch.as_tensor(toks, device=dev)][:, torch.as_tensor(rows, device=dev)].cpu().numpy()
     assert_matmul_close_f16_tile(got, ref, "prefill gemm, sampled tokens x rows")
+    # The distribution of the error, tighter than the gate above (the tile kernels round every dequantised weight once
+    # to f16, so they are not held to the GEMV's bound element by element).  Observed at this shape, Q4_K / Q8_0 /
+    # Q6_K alike: |err| / rms(ref) median 1.4e-4, 99th percentile 5.3e-4, maximum 7.6e-4 .. 8.4e-4; rms error 2.1e-4
+    # of the output rms; 93 % of the elements inside the GEMV's own bound 1e-3 |ref| + 1e-4 rms; every output of at
+    # least rms magnitude within 7.5e-4 of its own value.
+    e = np.abs(got.astype(np.float64) - ref).reshape(-1)
+    r = np.abs(ref).reshape(-1)
+    rms = float(np.sqrt(np.mean(r * r)))
+    assert np.quantile(e, 0.5) <= 2.5e-4 * rms and np.quantile(e, 0.99) <= 8e-4 * rms and e.max() <= 1.5e-3 * rms
+    assert np.mean(e <= 1e-3 * r + 1e-4 * rms) >= 0.9
+    big = r >= rms
+    assert (e[big] <= 1e-3 * r[big]).all(), "an output of at least rms magnitude is off by more than 1e-3 of its value"
     # a token row scaled by 2^5 gives that output row scaled by 2^5, bit for bit; the others do not move
     x2 = x.clone()
     x2[777] *= 32.0
