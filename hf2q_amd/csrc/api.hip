@@ -164,7 +164,7 @@ namespace {
 // which cost what a dozen passes of the small-batch kernel cost (151936 x 4096 Q6_K: 2650 us against 339 us per
 // eight rows), or what two to four rounds of per-row GEMVs cost where there is no small-batch kernel.
 uint32_t chunked_rows_limit(uint32_t k, hq_ggml_type t) {
-    if (!gemv_rows_supported(t, kGemvMaxRows, k)) return 2 * kGemvMaxRows;
+    if (!gemv_rows_supported(t, kGemvMaxRows, k) && !gemv_rows32_supported(t, kGemvMaxRows, k)) return 2 * kGemvMaxRows;
     if (t == HQ_Q4_K || t == HQ_Q5_K) return HQ_CHUNK_LIMIT_Q4K * kGemvMaxRows;
     return t == HQ_Q6_K ? 6 * kGemvMaxRows : 8 * kGemvMaxRows;
 }
@@ -186,6 +186,12 @@ int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const vo
         if (gemv_rows_supported(t, rows, k)) {
             if (int rc = launch_gemv_rows(stream, static_cast<const uint8_t*>(x) + (size_t)r0 * xrow_bytes, xdt, w_blocks,
                                           y + (size_t)r0 * n, rows, n, k, t))
+                return rc;
+            continue;
+        }
+        if (gemv_rows32_supported(t, rows, k)) {
+            if (int rc = launch_gemv_rows32(stream, static_cast<const uint8_t*>(x) + (size_t)r0 * xrow_bytes, xdt, w_blocks,
+                                            y + (size_t)r0 * n, rows, n, k, t))
                 return rc;
             continue;
         }

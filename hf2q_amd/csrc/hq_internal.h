@@ -60,6 +60,11 @@ int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_ac
 bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k);
 int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                      uint32_t k, hq_ggml_type t);
+// The same for the 32-weight-block types (Q8_0, Q4_0), 2 <= m <= 8: exact products on the VALU, every weight fetched
+// once for all rows.
+bool gemv_rows32_supported(hq_ggml_type t, uint32_t m, uint32_t k);
+int launch_gemv_rows32(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
+                       uint32_t k, hq_ggml_type t);
 
 // MFMA GEMM for m > 8 (prefill).  gemm_supported() says whether (type, k) has a tile kernel.
 bool gemm_supported(hq_ggml_type t, uint32_t k);

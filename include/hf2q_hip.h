@@ -95,7 +95,8 @@ HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, ui
  * &mut dst, &GgmlQuantizedMatmulParams{m,n,k,ggml_type})
  * (src/inference/models/qwen35/gpu_ffn.rs:1236-1245; dispatch_qmatmul,
  * src/serve/forward_mlx.rs:9655-9969).  m <= 8 takes the bandwidth-bound GEMV
- * kernels (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791) and so do a few more rows, eight at a
+ * kernels (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791; from two to four rows on, by type, a form that fetches every
+ * weight once for all rows) and so do a few more rows, eight at a
  * time (up to 16 for Q4_K / Q5_K, whose MFMA GEMM has tiles of 64 token rows for 17 .. 128 rows; up to
  * 48 for Q6_K and 64 for Q8_0 / Q4_0, whose tiles multiply 256 token rows whatever m is); larger m the
  * MFMA GEMM.  The K-quant (k % 256 == 0) and Q8_0 / Q4_0 (k % 128 == 0) GEMMs multiply f16-rounded

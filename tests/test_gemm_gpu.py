@@ -70,7 +70,7 @@ def test_small_tiles_and_k_slices_match_f64_oracle(oracle, dev, t, m, n, k):
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
 def test_gemm_adversarial_blocks(oracle, dev, t):
     """Every scale / min / nibble bit pattern (raw random bytes with finite f16 fields)."""
-    m, n, k = 40, 128, 512
+    m, n, k = 72, 128, 512  # past every type's chunked range: the tile kernels
     bb = oracle.BLOCK_BYTES[t]
     raw = np.random.default_rng(9).integers(0, 256, size=n * k // oracle.BLOCK_ELEMS[t] * bb, dtype=np.uint8)
     for off in ([1, 3] if t in (HQ_Q4_K, HQ_Q5_K) else [209] if t == HQ_Q6_K else [1]):
@@ -84,14 +84,14 @@ def test_gemm_adversarial_blocks(oracle, dev, t):
 def test_gemm_rows_equal_gemv_rows(oracle, dev, t):
     """Row i of the m>8 result agrees with the m=1 GEMV of activation row i; the tile kernels round
     their weights to f16, so the agreement is to 1e-3 of the row's largest output."""
-    m, n, k = 24, 256, 1024
+    m, n, k = 72, 256, 1024
     blocks = oracle.quantize(weights(5, n, k), k, t, threads=8)
     wd = torch.from_numpy(blocks).to(dev)
     x = torch.from_numpy(acts(6, m, k)).to(dev).to(torch.bfloat16)
     y = torch.empty(m, n, device=dev)
     ops.quantized_matmul_ggml(x, wd, y, GgmlQuantizedMatmulParams(m, n, k, t))
     y1 = torch.empty(1, n, device=dev)
-    for i in (0, 7, 23):
+    for i in (0, 7, 71):
         ops.quantized_matmul_ggml(x[i:i + 1].contiguous(), wd, y1, GgmlQuantizedMatmulParams(1, n, k, t))
         scale = y1.abs().max().item()
         assert (y[i] - y1[0]).abs().max().item() <= 1e-3 * scale
@@ -119,7 +119,9 @@ def test_q4k_tile_gemm_workspace_variant(oracle, dev):
     need = ops.quantized_matmul_workspace_bytes(p, torch.bfloat16)
     assert need >= m * k * 2 + m * 4
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(1, n, k, HQ_Q4_K), torch.bfloat16) == 0
-    assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q8_0), torch.bfloat16) >= m * k * 2
+    # Q8_0: up to 64 rows run as chunks of eight through its small-batch kernel (no scratch), the tile kernel beyond
+    assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q8_0), torch.bfloat16) == 0
+    assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(80, n, k, HQ_Q8_0), torch.bfloat16) >= 80 * k * 2
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, 320, HQ_Q8_0), torch.bfloat16) == 0
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q6_K), torch.bfloat16) >= m * k * 2
     y0 = torch.empty(m, n, device=dev)
@@ -138,7 +140,7 @@ def test_tile_gemm_scale_equivariance(oracle, dev, xdt, t):
     """Activation rows and weight rows are rescaled by powers of two inside the kernel (f16 has a narrow
     exponent range): scaling an activation row by 2^a scales its output row by exactly 2^a, across 80
     binades, and weights 10^4 times smaller or larger than usual lose no accuracy."""
-    m, n, k = 40, 128, 512
+    m, n, k = 72, 128, 512  # past every type's chunked range: the tile kernels
     x = acts(21, m, k)
     if xdt == "bf16":
         x = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(x)).reshape(m, k)

@@ -349,6 +349,60 @@ def test_small_batch_rows_match_f64_oracle(oracle, dev, t, xdt, m, n, k):
         assert np.abs(y1.cpu().numpy()[0] - y.cpu().numpy()[r]).max() <= 1e-4 * np.abs(ref).max()
 
 
+ROWS32_SHAPES = [  # (m, n, k): Q8_0 / Q4_0; k is walked in chunks of 2048 (64 blocks, one per lane)
+    (2, 80, 2048), (3, 64, 1024), (4, 200, 4096), (4, 5, 32), (5, 33, 320), (6, 130, 3104), (7, 250, 2048), (8, 96, 12288),
+    (8, 4100, 256),   # more rows than one pass of 16 waves x 256 workgroups covers on a small device share
+]
+
+
+@pytest.mark.parametrize("t", [HQ_Q8_0, HQ_Q4_0])
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("m,n,k", ROWS32_SHAPES)
+def test_small_batch_rows_of_32_weight_blocks_match_f64_oracle(oracle, dev, t, xdt, m, n, k):
+    """Q8_0 / Q4_0 with 2 <= m <= 8 take the kernel that fetches every weight once for all rows: exact products, so the
+    GEMV's tolerance; a short last chunk (k % 2048 != 0), fewer rows than waves, ragged n; the same bits on every call
+    (later chunks are added to y by the row's one writer, in chunk order)."""
+    blocks = oracle.quantize(weights(3 * n + k + m + t, n, k), k, t, threads=8)
+    x = acts(n + k + m, m, k)
+    xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
+    xd = torch.from_numpy(x).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    ref = oracle.qmatmul_f64(xv, blocks, m, n, k, t)
+    y = torch.full((m, n), float("nan"), device=dev)
+    wd = torch.from_numpy(blocks).to(dev)
+    ops.quantized_matmul_ggml(xd, wd, y, GgmlQuantizedMatmulParams(m, n, k, t))
+    assert_matmul_close(y.cpu().numpy(), ref, f"rows32 t={t} {xdt} {m}x{n}x{k}")
+    y2 = torch.full((m, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd, wd, y2, GgmlQuantizedMatmulParams(m, n, k, t))
+    assert torch.equal(y, y2)
+    y1 = torch.empty((1, n), device=dev)
+    for r in range(m):
+        ops.quantized_matmul_ggml(xd[r:r + 1].contiguous(), wd, y1, GgmlQuantizedMatmulParams(1, n, k, t))
+        assert np.abs(y1.cpu().numpy()[0] - y.cpu().numpy()[r]).max() <= 1e-4 * max(np.abs(ref).max(), 1e-30)
+
+
+@pytest.mark.parametrize("t", [HQ_Q8_0, HQ_Q4_0])
+def test_small_batch_rows_of_32_weight_blocks_adversarial_and_scaling(oracle, dev, t):
+    """Every byte pattern of the blocks (finite scales); scaling the activations by a power of two scales the result
+    exactly; rows past m of the staged activations do not leak into the output (m = 3 runs the 4-row instantiation)."""
+    m, n, k = 3, 48, 2048 + 64
+    bb = oracle.BLOCK_BYTES[t]
+    raw = np.random.default_rng(11).integers(0, 256, size=n * k // 32 * bb, dtype=np.uint8)
+    raw[1::bb] &= 0x3F  # f16 scale: finite, modest magnitude
+    x = acts(4, m, k)
+    wd = torch.from_numpy(raw).to(dev)
+    for xv, xd in ((x, torch.from_numpy(x).to(dev)),
+                   (oracle.f32_to_bf16_bits(x), torch.from_numpy(x).to(dev).to(torch.bfloat16))):
+        ref = oracle.qmatmul_f64(xv, raw, m, n, k, t)
+        y = torch.full((m + 1, n), 7.0, device=dev)
+        ops.quantized_matmul_ggml(xd, wd, y[:m], GgmlQuantizedMatmulParams(m, n, k, t))
+        assert_matmul_close(y[:m].cpu().numpy(), ref, "rows32, adversarial blocks")
+        assert (y[m] == 7.0).all()
+        y4 = torch.empty((m, n), device=dev)
+        ops.quantized_matmul_ggml(xd * 4.0, wd, y4, GgmlQuantizedMatmulParams(m, n, k, t))
+        assert torch.equal(y4, y[:m] * 4.0)
+
+
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q5_K])
 @pytest.mark.parametrize("xdt,m", [("bf16", 8), ("f32", 5)])
 def test_small_batch_rows_tall_matrix(oracle, dev, t, xdt, m):
