@@ -157,16 +157,23 @@ static int check_matmul_common(const char* fn, const void* x, hq_act_dtype xdt, 
 #ifndef HQ_CHUNK_LIMIT_Q4K
 #define HQ_CHUNK_LIMIT_Q4K 2
 #endif
+#ifndef HQ_CHUNK_LIMIT_Q6K
+#define HQ_CHUNK_LIMIT_Q6K 1
+#endif
+#ifndef HQ_CHUNK_LIMIT_Q80
+#define HQ_CHUNK_LIMIT_Q80 1
+#endif
 namespace {
 
-// A few rows past the GEMV limit still run in chunks of kGemvMaxRows rows.  Q4_K / Q5_K have tiles of 64 token rows
-// (one launch for any m <= 128 costs about what two to three chunks cost), the other types only tiles of 256 rows,
-// which cost what a dozen passes of the small-batch kernel cost (151936 x 4096 Q6_K: 2650 us against 339 us per
-// eight rows), or what two to four rounds of per-row GEMVs cost where there is no small-batch kernel.
+// Rows past the GEMV limit.  Every type has small tiles (Q4_K / Q5_K: 64 token rows, the others 128) whose one launch
+// for any m <= 128 costs about what one to two chunks of kGemvMaxRows rows through the small-batch kernel cost
+// (measured at 12288 x 4096: Q4_K 34 us against 15.5 us per chunk; Q6_K 44 against 32; Q8_0 43 against 33; Q4_0 33
+// against 30), so Q4_K / Q5_K run two chunks before the tiles take over and the other types one.  Where a type has no
+// small-batch kernel for this k (K-quants with k % 1024 != 0) two rounds of per-row GEMVs run first.
 uint32_t chunked_rows_limit(uint32_t k, hq_ggml_type t) {
     if (!gemv_rows_supported(t, kGemvMaxRows, k) && !gemv_rows32_supported(t, kGemvMaxRows, k)) return 2 * kGemvMaxRows;
     if (t == HQ_Q4_K || t == HQ_Q5_K) return HQ_CHUNK_LIMIT_Q4K * kGemvMaxRows;
-    return t == HQ_Q6_K ? 6 * kGemvMaxRows : 8 * kGemvMaxRows;
+    return t == HQ_Q6_K ? HQ_CHUNK_LIMIT_Q6K * kGemvMaxRows : HQ_CHUNK_LIMIT_Q80 * kGemvMaxRows;
 }
 
 bool f16_tile_route(uint32_t m, uint32_t k, hq_ggml_type t) {

@@ -213,8 +213,9 @@ struct GemmArgs {
     // dense form has lay_m = m, lay_n = n, wd_off = 0, row_map = nullptr.
     uint32_t lay_m, lay_n, wd_off;
     const uint32_t* row_map;
-    // Q4_K / Q5_K tiles: the super-blocks [sb0, sb1) of every row that the workgroup multiplies (all of them except
-    // in the split form of the small tiles, whose workgroups each write the partial sums of a slice of k)
+    // The 256-element runs [sb0, sb1) of every row that the workgroup multiplies (K-quants: super-blocks; Q8_0 / Q4_0:
+    // eight blocks, the last run may be half a one): all of them except in the split form of the small tiles, whose
+    // workgroups each write the partial sums of a slice of k
     uint32_t sb0, sb1;
 };
 
@@ -566,16 +567,17 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 // so it keeps its alignment case here too.  w = d * (q - 8).
 template <int MT, int WN, int TYPE = HQ_Q8_0>
 __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
-    constexpr int DMA_PER_WAVE = ActTile::kDma;
-    static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
+    constexpr int BMT = 32 * MT * (WAVES / WN);  // token rows of the workgroup tile: 256, or 128 for the small tiles
+    constexpr int DMA_PER_WAVE = ActTileT<BMT>::kDma;
     constexpr bool Q4 = TYPE == HQ_Q4_0;
     constexpr uint32_t BYTES = Q4 ? Q4_0_BYTES : Q8_0_BYTES;
     const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
-    const uint32_t nstages = a.k / BK;  // even (k % 128 == 0)
-    ActTile at;
+    // stages [st_first, nstages) of every row, an even number of them (k % 128 == 0; slices of k are whole 256s)
+    const uint32_t st_first = 4u * a.sb0, nstages = a.sb1 * 4u < a.k / BK ? a.sb1 * 4u : a.k / BK;
+    ActTileT<BMT> at;
     at.init(a, W, m0, lane, wave);
 
     uint32_t gn = n0 + wn * 32 + l32;
@@ -607,12 +609,12 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     constexpr int PD = 3;           // steps an activation fragment is requested ahead
     static_assert(MT % 4 == 0 && kSteps >= DMA_PER_WAVE, "four eighths per k-step, spread over the MT steps");
 
-    load_b(0, 0);
-    at.fetch_all(0, 0);
+    load_b(st_first, 0);
+    at.fetch_all(st_first, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    for (uint32_t st2 = 0; st2 < nstages; st2 += 2) {
+    for (uint32_t st2 = st_first; st2 < nstages; st2 += 2) {
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
             const uint32_t st = st2 + c;
@@ -696,19 +698,19 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 // hardware takes the unaligned 16-byte loads.
 template <int MT, int WN>
 __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
-    constexpr int DMA_PER_WAVE = ActTile::kDma;
-    static_assert(32 * MT * (WAVES / WN) == BM, "the waves cover the workgroup's token rows");
+    constexpr int BMT = 32 * MT * (WAVES / WN);  // token rows of the workgroup tile: 256, or 128 for the small tiles
+    constexpr int DMA_PER_WAVE = ActTileT<BMT>::kDma;
     const Workspace W = workspace_layout(a.lay_m, a.lay_n, a.k);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
-    const uint32_t nsb = a.k / 256, nstages = a.k / BK;
-    ActTile at;
+    const uint32_t nsb = a.sb1, nstages = 4u * a.sb1;  // super-blocks [sb0, sb1) of every row
+    ActTileT<BMT> at;
     at.init(a, W, m0, lane, wave);
 
     uint32_t gn = n0 + wn * 32 + l32;
     gn = gn < a.n ? gn : a.n - 1u;
-    const uint8_t* wrow = a.w + (size_t)gn * nsb * Q6K_BYTES;
+    const uint8_t* wrow = a.w + (size_t)gn * (a.k / 256) * Q6K_BYTES;
     const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[a.wd_off + gn];
     struct Raw { uint4 l0, l1, h0, h1; uint2 sc; uint32_t d; };  // one half of a super-block, this lane's share
     Raw braw[2];
@@ -732,12 +734,12 @@ __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     constexpr int PD = 3;           // steps an activation fragment is requested ahead
     static_assert(MT % 4 == 0 && kSteps >= DMA_PER_WAVE, "four eighths per k-step, spread over the MT steps");
 
-    load_half(0, 0, 0);
-    at.fetch_all(0, 0);
+    load_half(a.sb0, 0, 0);
+    at.fetch_all(4u * a.sb0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    for (uint32_t sb = 0; sb < nsb; ++sb) {
+    for (uint32_t sb = a.sb0; sb < nsb; ++sb) {
         const bool next_sb = sb + 1 < nsb;  // uniform
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -870,14 +872,34 @@ __global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict_
     y[i] = v;
 }
 
-// Slices of k for the small tiles: doubled while the grid has fewer workgroups than the device has CUs (256) and a slice
-// keeps at least four super-blocks (sixteen stages, so that its prologue and epilogue stay a fraction of its work).
-inline uint32_t small_tile_splits(uint32_t m, uint32_t n, uint32_t k) {
-    const uint64_t tiles = (uint64_t)((m + BM_SMALL - 1) / BM_SMALL) * ((n + BN_NARROW - 1) / BN_NARROW);
+// Slices of k for the small tiles (bm token rows x bn weight rows): doubled while the grid has fewer workgroups than
+// the device has CUs (256) and a slice keeps at least four 256-element runs (sixteen stages, so that its prologue and
+// epilogue stay a fraction of its work); k must be whole runs for that.
+inline uint32_t small_tile_splits(uint32_t m, uint32_t n, uint32_t k, uint32_t bm, uint32_t bn) {
+    const uint64_t tiles = (uint64_t)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
     const uint32_t nsb = k / 256;
     uint32_t s = 1;
+    if (k % 256) return s;
     while (s < 4 && tiles * s < 256 && nsb / (2 * s) >= 4) s *= 2;
     return s;
+}
+
+// The same for Q6_K and Q8_0 / Q4_0, up to 128 token rows: tiles of 128 token rows x 128 weight rows (four waves side by
+// side, each 128 x 32; these tile bodies spread a k-step's four fragment words over MT >= 4 row tiles).
+template <int TYPE>
+__global__ __launch_bounds__(64 * WAVES, 2) void mid_gemm_small_kernel(GemmArgs a, uint32_t splits, uint32_t sb_per,
+                                                                       float* __restrict__ partial) {
+    const uint32_t tiles_n = (a.n + BN_WIDE - 1) / BN_WIDE, tiles_m = (a.m + BM_MID - 1) / BM_MID;
+    const uint32_t s = blockIdx.x / (tiles_n * tiles_m), t = blockIdx.x % (tiles_n * tiles_m);
+    if (splits > 1) {
+        a.sb0 = s * sb_per;
+        a.sb1 = a.sb0 + sb_per < a.sb1 ? a.sb0 + sb_per : a.sb1;
+        a.y = partial + (size_t)s * a.m * a.n;
+    }
+    if constexpr (TYPE == HQ_Q6_K)
+        q6k_gemm_tile<4, 4>(a, (t / tiles_n) * BM_MID, (t % tiles_n) * BN_WIDE);
+    else
+        q80_gemm_tile<4, 4, TYPE>(a, (t / tiles_n) * BM_MID, (t % tiles_n) * BN_WIDE);
 }
 
 __global__ __launch_bounds__(64 * WAVES, 2) void q6k_gemm_kernel(GemmArgs a) {
@@ -992,12 +1014,17 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
 
 }  // namespace
 
-bool gemm_f16_small_tiles(hq_ggml_type t, uint32_t m) { return (t == HQ_Q4_K || t == HQ_Q5_K) && m <= 2 * BM_SMALL; }
+bool gemm_f16_small_tiles(hq_ggml_type t, uint32_t m) { return m <= (uint32_t)BM_MID; }
+
+// Slices of k the small tiles of type t cut the product into (1: none).
+static uint32_t small_splits_of(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) {
+    return t == HQ_Q4_K || t == HQ_Q5_K ? small_tile_splits(m, n, k, BM_SMALL, BN_NARROW) : small_tile_splits(m, n, k, BM_MID, BN_WIDE);
+}
 
 size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
     size_t total = workspace_layout(m, n, k).total;
     if (gemm_f16_small_tiles(t, m)) {  // partial sums of the slices of k
-        const uint32_t splits = small_tile_splits(m, n, k);
+        const uint32_t splits = small_splits_of(t, m, n, k);
         if (splits > 1) total += (size_t)splits * m * n * 4;
     }
     return total;
@@ -1052,7 +1079,7 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
         if (small) kern = grouped_gemm_kernel<TYPE, true>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;
-    GemmArgs a{ws, wb, y, pairs, n, k, pairs, n_experts * n, 0u, row_map, 0u, k / 256};
+    GemmArgs a{ws, wb, y, pairs, n, k, pairs, n_experts * n, 0u, row_map, 0u, (k + 255u) / 256u};
     const uint32_t tiles_n = (n + bn - 1) / bn;
     const uint32_t max_tiles = pairs / bm + n_experts;
     hipLaunchKernelGGL(kern, dim3(max_tiles * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
@@ -1082,12 +1109,25 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
                          uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const uint8_t* wb = static_cast<const uint8_t*>(w);
-    GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr, 0u, k / 256};
+    GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr, 0u, (k + 255u) / 256u};
     constexpr int lds = 2 * ActTile::kTile;
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
+    // up to 128 token rows of Q6_K / Q8_0 / Q4_0: tiles of 128 x 128, k in slices where that leaves CUs idle
+    auto launch_mid_small = [&](void (*kern)(GemmArgs, uint32_t, uint32_t, float*)) -> int {
+        const uint32_t tm = (m + BM_MID - 1) / BM_MID, tn = (n + BN_WIDE - 1) / BN_WIDE;
+        const uint32_t splits = small_splits_of(t, m, n, k), nsb = (k + 255u) / 256u, sb_per = (nsb + splits - 1) / splits;
+        float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
+        hipLaunchKernelGGL(kern, dim3(tm * tn * splits), dim3(64 * WAVES), 2 * ActTileT<BM_MID>::kTile, s, a, splits, sb_per, partial);
+        if (int rc = check_launch("small gemm kernel launch")) return rc;
+        if (splits == 1) return HQ_OK;
+        const uint32_t count = m * n;  // m <= 128
+        hipLaunchKernelGGL(split_sum_kernel, dim3((count + 255u) / 256u), dim3(256), 0, s, partial, y, count, splits);
+        return check_launch("split sum kernel launch");
+    };
     if (t == HQ_Q6_K) {
         if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
+        if (gemm_f16_small_tiles(t, m)) return launch_mid_small(mid_gemm_small_kernel<HQ_Q6_K>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(q6k_gemm_kernel), (size_t)lds, "hipFuncSetAttribute(q6_k gemm LDS)"))
             return rc;
         hipLaunchKernelGGL(q6k_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
@@ -1098,6 +1138,8 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         if (int rc = t == HQ_Q4_0 ? launch_prep<HQ_Q4_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
                                   : launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
             return rc;
+        if (gemm_f16_small_tiles(t, m))
+            return launch_mid_small(t == HQ_Q4_0 ? mid_gemm_small_kernel<HQ_Q4_0> : mid_gemm_small_kernel<HQ_Q8_0>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(q8_0 gemm LDS)"))
             return rc;
         hipLaunchKernelGGL(kern, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
@@ -1106,10 +1148,10 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
                               : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
         return rc;
-    if (gemm_f16_small_tiles(t, m)) {  // up to two token tiles of 64 rows
+    if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: up to two token tiles of 64 rows
         void (*ksmall)(GemmArgs, uint32_t, uint32_t, float*) = t == HQ_Q5_K ? q4k_gemm_small_kernel<HQ_Q5_K> : q4k_gemm_small_kernel<HQ_Q4_K>;
         const uint32_t tm = (m + BM_SMALL - 1) / BM_SMALL, tn = (n + BN_NARROW - 1) / BN_NARROW;
-        const uint32_t splits = small_tile_splits(m, n, k), nsb = k / 256, sb_per = (nsb + splits - 1) / splits;
+        const uint32_t splits = small_splits_of(t, m, n, k), nsb = k / 256, sb_per = (nsb + splits - 1) / splits;
         float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
         hipLaunchKernelGGL(ksmall, dim3(tm * tn * splits), dim3(64 * WAVES), 2 * ActTileT<BM_SMALL>::kTile, s, a, splits, sb_per, partial);
         if (int rc = check_launch("q4k small gemm kernel launch")) return rc;

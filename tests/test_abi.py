@@ -43,19 +43,17 @@ def test_workspace_queries_follow_the_routing():
     L = lib.load()
     for t, kq in ((lib.HQ_Q4_K, 256), (lib.HQ_Q5_K, 256), (lib.HQ_Q6_K, 256), (lib.HQ_Q8_0, 128), (lib.HQ_Q4_0, 128)):
         bb, be = L.hq_block_bytes(t), L.hq_block_elems(t)
-        # dense: up to 8 rows (and a few chunks of 8 beyond: 16 rows at least) never need scratch; prefill-sized m
-        # needs the f16 activations (+ row scales) when k suits the tile kernel
+        # dense: up to 8 rows never need scratch, nor do 16 rows of Q4_K / Q5_K (two chunks of eight through the
+        # small-batch kernel); beyond that every type has small tiles (64 or 128 token rows) and needs the f16
+        # activations (+ row scales) when k suits the tile kernel -- and the partial sums where k is cut into slices
+        # (64 x 64 x 8192 Q4_K: one tile, four slices)
         assert L.hq_qmatmul_ggml_workspace_bytes(8, 512, 4 * kq, lib.HQ_BF16, t) == 0
-        assert L.hq_qmatmul_ggml_workspace_bytes(16, 512, 4 * kq, lib.HQ_BF16, t) == 0
-        # 17 rows: Q4_K / Q5_K have tiles of 64 token rows (a third chunk of 8 would already cost more); their scratch
-        # also holds the partial sums where k is cut into slices (64 x 64 x 8192: one tile, four slices)
-        small = L.hq_qmatmul_ggml_workspace_bytes(17, 512, 4 * kq, lib.HQ_BF16, t)
         if t in (lib.HQ_Q4_K, lib.HQ_Q5_K):
-            assert small >= 17 * 4 * kq * 2
-        elif t == lib.HQ_Q6_K:
-            assert small == 0  # chunks of 8 rows through the small-batch kernel up to 48 rows
-        if t in (lib.HQ_Q4_K, lib.HQ_Q5_K):
+            assert L.hq_qmatmul_ggml_workspace_bytes(16, 512, 4 * kq, lib.HQ_BF16, t) == 0
             assert L.hq_qmatmul_ggml_workspace_bytes(64, 64, 8192, lib.HQ_BF16, t) >= 64 * 8192 * 2 + 4 * 64 * 64 * 4
+        else:
+            assert L.hq_qmatmul_ggml_workspace_bytes(9, 512, 4 * kq, lib.HQ_BF16, t) >= 9 * 4 * kq * 2
+        assert L.hq_qmatmul_ggml_workspace_bytes(17, 512, 4 * kq, lib.HQ_BF16, t) >= 17 * 4 * kq * 2
         need = L.hq_qmatmul_ggml_workspace_bytes(512, 512, 4 * kq, lib.HQ_BF16, t)
         assert need >= 512 * 4 * kq * 2 and need % 256 == 0
         if be == 32:

@@ -50,17 +50,21 @@ def test_gemm_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
     _check(t, k)(y, ref, f"gemm t={t} {xdt} {m}x{n}x{k}")
 
 
-@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K])
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0])
 @pytest.mark.parametrize("m,n,k", [
-    (17, 64, 2048),     # one tile of 64 x 64, k in two slices
-    (65, 130, 2304),    # two token tiles, ragged weight rows, nine super-blocks in slices of five and four
-    (128, 70, 4352),    # seventeen super-blocks in four slices (5, 5, 5, 2)
-    (100, 320, 256),    # a single super-block: no slices
+    (17, 64, 2048),     # one tile, k in two slices
+    (65, 130, 2304),    # ragged weight rows, nine runs of 256 in slices of five and four
+    (128, 70, 4352),    # seventeen runs in four slices (5, 5, 5, 2)
+    (100, 320, 256),    # a single run: no slices
     (64, 12288, 512),   # more tiles than CUs' worth: no slices
+    (40, 200, 1152),    # Q8_0 / Q4_0 only: k % 256 = 128, the last run is half a one (and k is not cut)
 ])
 def test_small_tiles_and_k_slices_match_f64_oracle(oracle, dev, t, m, n, k):
-    """17 .. 128 activation rows of Q4_K / Q5_K: tiles of 64 token rows, with k cut into slices (summed in a fixed
-    order by a second launch) where the tiles alone would leave most CUs idle; the same result on every call."""
+    """Up to 128 activation rows: tiles of 64 token rows (Q4_K / Q5_K) or 128 (the other types), with k cut into slices
+    (summed in a fixed order by a second launch) where the tiles alone would leave most CUs idle; the same result on
+    every call."""
+    if k % oracle.BLOCK_ELEMS[t]:
+        pytest.skip("k is not a multiple of the block size")
     y, ref = _run(oracle, dev, t, "bf16", m, n, k)
     assert_matmul_close_f16_tile(y, ref, f"small tiles t={t} {m}x{n}x{k}")
     y2, _ = _run(oracle, dev, t, "bf16", m, n, k)
@@ -119,9 +123,7 @@ def test_q4k_tile_gemm_workspace_variant(oracle, dev):
     need = ops.quantized_matmul_workspace_bytes(p, torch.bfloat16)
     assert need >= m * k * 2 + m * 4
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(1, n, k, HQ_Q4_K), torch.bfloat16) == 0
-    # Q8_0: up to 64 rows run as chunks of eight through its small-batch kernel (no scratch), the tile kernel beyond
-    assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q8_0), torch.bfloat16) == 0
-    assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(80, n, k, HQ_Q8_0), torch.bfloat16) >= 80 * k * 2
+    assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q8_0), torch.bfloat16) >= m * k * 2
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, 320, HQ_Q8_0), torch.bfloat16) == 0
     assert ops.quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, n, k, HQ_Q6_K), torch.bfloat16) >= m * k * 2
     y0 = torch.empty(m, n, device=dev)

@@ -422,13 +422,13 @@ def test_small_batch_rows_tall_matrix(oracle, dev, t, xdt, m):
     assert_matmul_close(y.cpu().numpy(), ref, f"rows, tall matrix t={t} {xdt} m={m}")
 
 
-@pytest.mark.parametrize("t,m,k", [(HQ_Q4_K, 9, 2048), (HQ_Q4_K, 16, 1024), (HQ_Q5_K, 16, 1024), (HQ_Q6_K, 18, 2048),
-                                   (HQ_Q6_K, 48, 1024), (HQ_Q8_0, 13, 1024), (HQ_Q4_K, 15, 768)])
+@pytest.mark.parametrize("t,m,k", [(HQ_Q4_K, 9, 2048), (HQ_Q4_K, 16, 1024), (HQ_Q5_K, 16, 1024), (HQ_Q6_K, 12, 768),
+                                   (HQ_Q6_K, 16, 1280), (HQ_Q5_K, 13, 256), (HQ_Q4_K, 15, 768)])
 def test_a_few_rows_past_eight_run_in_chunks_of_eight(oracle, dev, t, m, k):
-    """Up to 16 (Q4_K / Q5_K, which have tiles of 64 token rows beyond that), 48 (Q6_K) or 16 rows (no small-batch
-    kernel for the type or k) do not take a tile kernel: chunks of eight through the small-batch kernel, the remainder
-    through it or the GEMV.  Every product is exact on this route, so the GEMV's tolerance holds, and no scratch is
-    asked for."""
+    """Up to 16 rows of Q4_K / Q5_K (whose tiles of 64 token rows take over beyond that), and up to 16 rows of a K-quant
+    whose k has no small-batch kernel (k % 1024 != 0), do not take a tile kernel: chunks of eight through the
+    small-batch kernel, the remainder through it or the GEMV.  Every product is exact on this route, so the GEMV's
+    tolerance holds, and no scratch is asked for."""
     n = 136
     blocks = oracle.quantize(weights(m + k + t, n, k), k, t, threads=8)
     x = acts(m + t, m, k)
