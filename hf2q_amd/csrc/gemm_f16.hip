@@ -1002,9 +1002,14 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
     a.w += (size_t)tt.x * expert_stride;
     a.wd_off = tt.x * a.n;
     a.m = tt.z;  // rows past the expert's run repeat its last row and are not stored
-    if constexpr (SMALL)
-        q4k_gemm_tile<4, 1, 4, TYPE>(a, tt.y, n0);  // 128 routed rows x 128 weight rows (Q4_K / Q5_K), a wave 128 x 32
-    else if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
+    if constexpr (SMALL) {  // 128 routed rows x 128 weight rows, a wave 128 x 32
+        if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
+            q4k_gemm_tile<4, 1, 4, TYPE>(a, tt.y, n0);
+        else if constexpr (TYPE == HQ_Q6_K)
+            q6k_gemm_tile<4, 4>(a, tt.y, n0);
+        else
+            q80_gemm_tile<4, 4, TYPE>(a, tt.y, n0);
+    } else if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
         q4k_gemm_tile<8, 1, 4, TYPE>(a, tt.y, n0);
     else if constexpr (TYPE == HQ_Q6_K)
         q6k_gemm_tile<8, 4>(a, tt.y, n0);
@@ -1066,17 +1071,15 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     uint4* tiles = reinterpret_cast<uint4*>(ws + G.tiles);
     uint32_t* n_tiles = reinterpret_cast<uint32_t*>(ws + G.count);
     // Experts with few rows each (Qwen3.6-35B-A3B: 2048 tokens x top-8 over 256 experts = 64 rows per expert) take tiles
-    // of 64 routed rows; the 256-row tiles would run a quarter full.
-    constexpr bool HAS_SMALL = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K;
-    const bool small = HAS_SMALL && (uint64_t)pairs < (uint64_t)n_experts * 160u;
+    // of 128 routed rows; the 256-row tiles would run a quarter full.
+    const bool small = (uint64_t)pairs < (uint64_t)n_experts * 160u;
     const uint32_t bm = small ? BM_MID : BM, bn = BN_WIDE;
     hipLaunchKernelGGL(moe_bucket_kernel, dim3(1), dim3(1024), 0, s, ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm);
     if (int rc = check_launch("expert bucket kernel launch")) return rc;
     if (int rc = launch_prep<TYPE>(s, x, xdt, wb, ws, pairs, n_experts * n, k, row_map, top_k)) return rc;
     const int lds = 2 * (small ? ActTileT<BM_MID>::kTile : ActTile::kTile);
-    void (*kern)(GemmArgs, const uint4*, const uint32_t*, uint32_t, uint64_t) = grouped_gemm_kernel<TYPE, false>;
-    if constexpr (HAS_SMALL)
-        if (small) kern = grouped_gemm_kernel<TYPE, true>;
+    void (*kern)(GemmArgs, const uint4*, const uint32_t*, uint32_t, uint64_t) =
+        small ? grouped_gemm_kernel<TYPE, true> : grouped_gemm_kernel<TYPE, false>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;
     GemmArgs a{ws, wb, y, pairs, n, k, pairs, n_experts * n, 0u, row_map, 0u, (k + 255u) / 256u};
