@@ -227,7 +227,7 @@ __device__ __forceinline__ uint4 ld16(const uint8_t* p) { return *reinterpret_ca
 
 constexpr int WAVES = 4;           // one per SIMD; two workgroups share a CU
 constexpr int BM = 256;            // token rows per workgroup of the prefill-sized tiles
-constexpr int BM_SMALL = 64;       // ... of the tiles for a few token rows (up to 128)
+constexpr int BM_SMALL = 64;       // ... of the Q4_K / Q5_K tiles for a few token rows (up to 128)
 constexpr int BM_MID = 128;        // ... of the tiles for sparsely filled experts
 constexpr int BN_WIDE = 128, BN_NARROW = 64;    // weight rows per workgroup
 
@@ -843,23 +843,23 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_kernel(GemmArgs a, uin
     }
 }
 
-// 9 .. 128 token rows: tiles of 64 token rows x 64 weight rows (2 x 2 waves of 32 x 32), so that a few rows do not
-// pay for 256 and the weight rows spread over the CUs (12288 rows: 192 workgroups per token tile).  Where that is
-// still less than a workgroup per CU, k is cut into `splits` slices of sb_per super-blocks, each with workgroups of
+// Up to 128 token rows of Q4_K / Q5_K: tiles of 64 token rows x 128 weight rows (four waves side by side, each 64 x 32,
+// so every weight is dequantised once per tile), so that a few rows do not pay for 256.  Where the tiles alone are
+// fewer workgroups than the device has CUs, k is cut into `splits` slices of sb_per super-blocks, each with workgroups of
 // its own that store their products into slice `s` of `partial` ([splits][m][n] floats, same scaling as y);
 // split_sum_kernel then adds the slices in order.
 template <int TYPE>
 __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_small_kernel(GemmArgs a, uint32_t splits, uint32_t sb_per,
                                                                        float* __restrict__ partial) {
     // consecutive workgroups (which the hardware deals to the XCDs in turn) take consecutive weight-row tiles
-    const uint32_t tiles_n = (a.n + BN_NARROW - 1) / BN_NARROW, tiles_m = (a.m + BM_SMALL - 1) / BM_SMALL;
+    const uint32_t tiles_n = (a.n + BN_WIDE - 1) / BN_WIDE, tiles_m = (a.m + BM_SMALL - 1) / BM_SMALL;
     const uint32_t s = blockIdx.x / (tiles_n * tiles_m), t = blockIdx.x % (tiles_n * tiles_m);
     if (splits > 1) {
         a.sb0 = s * sb_per;
         a.sb1 = a.sb0 + sb_per < a.sb1 ? a.sb0 + sb_per : a.sb1;
         a.y = partial + (size_t)s * a.m * a.n;
     }
-    q4k_gemm_tile<1, 1, 2, TYPE>(a, (t / tiles_n) * BM_SMALL, (t % tiles_n) * BN_NARROW);
+    q4k_gemm_tile<2, 1, 4, TYPE>(a, (t / tiles_n) * BM_SMALL, (t % tiles_n) * BN_WIDE);
 }
 
 // y[i] = partial[0][i] + partial[1][i] + ... in this order, whatever order the slices were written in.
@@ -874,13 +874,13 @@ __global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict_
 
 // Slices of k for the small tiles (bm token rows x bn weight rows): doubled while the grid has fewer workgroups than
 // the device has CUs (256) and a slice keeps at least four 256-element runs (sixteen stages, so that its prologue and
-// epilogue stay a fraction of its work); k must be whole runs for that.
+// epilogue stay a fraction of its work), up to eight slices; k must be whole runs for that.
 inline uint32_t small_tile_splits(uint32_t m, uint32_t n, uint32_t k, uint32_t bm, uint32_t bn) {
     const uint64_t tiles = (uint64_t)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
     const uint32_t nsb = k / 256;
     uint32_t s = 1;
     if (k % 256) return s;
-    while (s < 4 && tiles * s < 256 && nsb / (2 * s) >= 4) s *= 2;
+    while (s < 8 && tiles * s < 256 && nsb / (2 * s) >= 4) s *= 2;
     return s;
 }
 
@@ -1023,7 +1023,7 @@ bool gemm_f16_small_tiles(hq_ggml_type t, uint32_t m) { return m <= (uint32_t)BM
 
 // Slices of k the small tiles of type t cut the product into (1: none).
 static uint32_t small_splits_of(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) {
-    return t == HQ_Q4_K || t == HQ_Q5_K ? small_tile_splits(m, n, k, BM_SMALL, BN_NARROW) : small_tile_splits(m, n, k, BM_MID, BN_WIDE);
+    return t == HQ_Q4_K || t == HQ_Q5_K ? small_tile_splits(m, n, k, BM_SMALL, BN_WIDE) : small_tile_splits(m, n, k, BM_MID, BN_WIDE);
 }
 
 size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
@@ -1151,9 +1151,9 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
                               : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
         return rc;
-    if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: up to two token tiles of 64 rows
+    if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: up to two token tiles of 64 rows x 128 weight rows
         void (*ksmall)(GemmArgs, uint32_t, uint32_t, float*) = t == HQ_Q5_K ? q4k_gemm_small_kernel<HQ_Q5_K> : q4k_gemm_small_kernel<HQ_Q4_K>;
-        const uint32_t tm = (m + BM_SMALL - 1) / BM_SMALL, tn = (n + BN_NARROW - 1) / BN_NARROW;
+        const uint32_t tm = (m + BM_SMALL - 1) / BM_SMALL, tn = (n + BN_WIDE - 1) / BN_WIDE;
         const uint32_t splits = small_splits_of(t, m, n, k), nsb = k / 256, sb_per = (nsb + splits - 1) / splits;
         float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
         hipLaunchKernelGGL(ksmall, dim3(tm * tn * splits), dim3(64 * WAVES), 2 * ActTileT<BM_SMALL>::kTile, s, a, splits, sb_per, partial);
