@@ -843,23 +843,24 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_kernel(GemmArgs a, uin
     }
 }
 
-// Up to 128 token rows of Q4_K / Q5_K: tiles of 64 token rows x 128 weight rows (four waves side by side, each 64 x 32,
-// so every weight is dequantised once per tile), so that a few rows do not pay for 256.  Where the tiles alone are
+// Up to 128 token rows of Q4_K / Q5_K: one token tile of 64 rows (m <= 64) or of 128, x 128 weight rows (four waves side by
+// side, each 64 or 128 x 32, so every weight is dequantised once), so that a few rows do not pay for 256.  Where the tiles alone are
 // fewer workgroups than the device has CUs, k is cut into `splits` slices of sb_per super-blocks, each with workgroups of
 // its own that store their products into slice `s` of `partial` ([splits][m][n] floats, same scaling as y);
 // split_sum_kernel then adds the slices in order.
-template <int TYPE>
+template <int TYPE, int MTS>  // MTS = 2: 64 token rows per tile (m <= 64); 4: 128
 __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_small_kernel(GemmArgs a, uint32_t splits, uint32_t sb_per,
                                                                        float* __restrict__ partial) {
+    constexpr uint32_t BMS = 32 * MTS;
     // consecutive workgroups (which the hardware deals to the XCDs in turn) take consecutive weight-row tiles
-    const uint32_t tiles_n = (a.n + BN_WIDE - 1) / BN_WIDE, tiles_m = (a.m + BM_SMALL - 1) / BM_SMALL;
+    const uint32_t tiles_n = (a.n + BN_WIDE - 1) / BN_WIDE, tiles_m = (a.m + BMS - 1) / BMS;
     const uint32_t s = blockIdx.x / (tiles_n * tiles_m), t = blockIdx.x % (tiles_n * tiles_m);
     if (splits > 1) {
         a.sb0 = s * sb_per;
         a.sb1 = a.sb0 + sb_per < a.sb1 ? a.sb0 + sb_per : a.sb1;
         a.y = partial + (size_t)s * a.m * a.n;
     }
-    q4k_gemm_tile<2, 1, 4, TYPE>(a, (t / tiles_n) * BM_SMALL, (t % tiles_n) * BN_WIDE);
+    q4k_gemm_tile<MTS, 1, 4, TYPE>(a, (t / tiles_n) * BMS, (t % tiles_n) * BN_WIDE);
 }
 
 // y[i] = partial[0][i] + partial[1][i] + ... in this order, whatever order the slices were written in.
@@ -1023,7 +1024,8 @@ bool gemm_f16_small_tiles(hq_ggml_type t, uint32_t m) { return m <= (uint32_t)BM
 
 // Slices of k the small tiles of type t cut the product into (1: none).
 static uint32_t small_splits_of(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) {
-    return t == HQ_Q4_K || t == HQ_Q5_K ? small_tile_splits(m, n, k, BM_SMALL, BN_WIDE) : small_tile_splits(m, n, k, BM_MID, BN_WIDE);
+    return (t == HQ_Q4_K || t == HQ_Q5_K) && m <= (uint32_t)BM_SMALL ? small_tile_splits(m, n, k, BM_SMALL, BN_WIDE)
+                                                                   : small_tile_splits(m, n, k, BM_MID, BN_WIDE);
 }
 
 size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
@@ -1151,12 +1153,16 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
                               : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
         return rc;
-    if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: up to two token tiles of 64 rows x 128 weight rows
-        void (*ksmall)(GemmArgs, uint32_t, uint32_t, float*) = t == HQ_Q5_K ? q4k_gemm_small_kernel<HQ_Q5_K> : q4k_gemm_small_kernel<HQ_Q4_K>;
-        const uint32_t tm = (m + BM_SMALL - 1) / BM_SMALL, tn = (n + BN_WIDE - 1) / BN_WIDE;
+    if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: one token tile of 64 or of 128 rows, tiles of 128 weight rows
+        const bool one64 = m <= (uint32_t)BM_SMALL;
+        void (*ksmall)(GemmArgs, uint32_t, uint32_t, float*) =
+            t == HQ_Q5_K ? (one64 ? q4k_gemm_small_kernel<HQ_Q5_K, 2> : q4k_gemm_small_kernel<HQ_Q5_K, 4>)
+                         : (one64 ? q4k_gemm_small_kernel<HQ_Q4_K, 2> : q4k_gemm_small_kernel<HQ_Q4_K, 4>);
+        const uint32_t tn = (n + BN_WIDE - 1) / BN_WIDE;
         const uint32_t splits = small_splits_of(t, m, n, k), nsb = k / 256, sb_per = (nsb + splits - 1) / splits;
         float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
-        hipLaunchKernelGGL(ksmall, dim3(tm * tn * splits), dim3(64 * WAVES), 2 * ActTileT<BM_SMALL>::kTile, s, a, splits, sb_per, partial);
+        const int lds_small = 2 * (one64 ? ActTileT<BM_SMALL>::kTile : ActTileT<BM_MID>::kTile);
+        hipLaunchKernelGGL(ksmall, dim3(tn * splits), dim3(64 * WAVES), lds_small, s, a, splits, sb_per, partial);
         if (int rc = check_launch("q4k small gemm kernel launch")) return rc;
         if (splits == 1) return HQ_OK;
         const uint32_t count = m * n;  // m <= 128
