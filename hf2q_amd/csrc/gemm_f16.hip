@@ -848,7 +848,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_kernel(GemmArgs a, uin
 // fewer workgroups than the device has CUs, k is cut into `splits` slices of sb_per super-blocks, each with workgroups of
 // its own that store their products into slice `s` of `partial` ([splits][m][n] floats, same scaling as y);
 // split_sum_kernel then adds the slices in order.
-template <int TYPE, int MTS>  // MTS = 2: 64 token rows per tile (m <= 64); 4: 128
+template <int TYPE, int MTS>  // MTS = 2: 64 token rows per tile (m <= 64); 4: 128; 8: 256
 __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_small_kernel(GemmArgs a, uint32_t splits, uint32_t sb_per,
                                                                        float* __restrict__ partial) {
     constexpr uint32_t BMS = 32 * MTS;
@@ -887,10 +887,11 @@ inline uint32_t small_tile_splits(uint32_t m, uint32_t n, uint32_t k, uint32_t b
 
 // The same for Q6_K and Q8_0 / Q4_0, up to 128 token rows: tiles of 128 token rows x 128 weight rows (four waves side by
 // side, each 128 x 32; these tile bodies spread a k-step's four fragment words over MT >= 4 row tiles).
-template <int TYPE>
+template <int TYPE, int MTS>  // MTS = 4: 128 token rows per tile (m <= 128); 8: 256
 __global__ __launch_bounds__(64 * WAVES, 2) void mid_gemm_small_kernel(GemmArgs a, uint32_t splits, uint32_t sb_per,
                                                                        float* __restrict__ partial) {
-    const uint32_t tiles_n = (a.n + BN_WIDE - 1) / BN_WIDE, tiles_m = (a.m + BM_MID - 1) / BM_MID;
+    constexpr uint32_t BMS = 32 * MTS;
+    const uint32_t tiles_n = (a.n + BN_WIDE - 1) / BN_WIDE, tiles_m = (a.m + BMS - 1) / BMS;
     const uint32_t s = blockIdx.x / (tiles_n * tiles_m), t = blockIdx.x % (tiles_n * tiles_m);
     if (splits > 1) {
         a.sb0 = s * sb_per;
@@ -898,9 +899,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void mid_gemm_small_kernel(GemmArgs 
         a.y = partial + (size_t)s * a.m * a.n;
     }
     if constexpr (TYPE == HQ_Q6_K)
-        q6k_gemm_tile<4, 4>(a, (t / tiles_n) * BM_MID, (t % tiles_n) * BN_WIDE);
+        q6k_gemm_tile<MTS, 4>(a, (t / tiles_n) * BMS, (t % tiles_n) * BN_WIDE);
     else
-        q80_gemm_tile<4, 4, TYPE>(a, (t / tiles_n) * BM_MID, (t % tiles_n) * BN_WIDE);
+        q80_gemm_tile<MTS, 4, TYPE>(a, (t / tiles_n) * BMS, (t % tiles_n) * BN_WIDE);
 }
 
 __global__ __launch_bounds__(64 * WAVES, 2) void q6k_gemm_kernel(GemmArgs a) {
@@ -1020,12 +1021,13 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
 
 }  // namespace
 
-bool gemm_f16_small_tiles(hq_ggml_type t, uint32_t m) { return m <= (uint32_t)BM_MID; }
+// One token tile (m <= 256) takes the form whose k may be cut into slices: a single row of tiles seldom fills the device.
+bool gemm_f16_small_tiles(hq_ggml_type t, uint32_t m) { return m <= (uint32_t)BM; }
 
 // Slices of k the small tiles of type t cut the product into (1: none).
 static uint32_t small_splits_of(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) {
-    return (t == HQ_Q4_K || t == HQ_Q5_K) && m <= (uint32_t)BM_SMALL ? small_tile_splits(m, n, k, BM_SMALL, BN_WIDE)
-                                                                   : small_tile_splits(m, n, k, BM_MID, BN_WIDE);
+    const uint32_t bm = (t == HQ_Q4_K || t == HQ_Q5_K) && m <= (uint32_t)BM_SMALL ? BM_SMALL : m <= (uint32_t)BM_MID ? BM_MID : BM;
+    return small_tile_splits(m, n, k, bm, BN_WIDE);
 }
 
 size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
@@ -1118,21 +1120,28 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     constexpr int lds = 2 * ActTile::kTile;
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
-    // up to 128 token rows of Q6_K / Q8_0 / Q4_0: tiles of 128 x 128, k in slices where that leaves CUs idle
-    auto launch_mid_small = [&](void (*kern)(GemmArgs, uint32_t, uint32_t, float*)) -> int {
-        const uint32_t tm = (m + BM_MID - 1) / BM_MID, tn = (n + BN_WIDE - 1) / BN_WIDE;
+    // up to 256 token rows of Q6_K / Q8_0 / Q4_0: one token tile of 128 or 256 rows x 128 weight rows, k in slices where
+    // that leaves CUs idle
+    auto launch_mid_small = [&](void (*k128)(GemmArgs, uint32_t, uint32_t, float*),
+                                void (*k256)(GemmArgs, uint32_t, uint32_t, float*)) -> int {
+        const bool one128 = m <= (uint32_t)BM_MID;
+        void (*kern)(GemmArgs, uint32_t, uint32_t, float*) = one128 ? k128 : k256;
+        const uint32_t tn = (n + BN_WIDE - 1) / BN_WIDE;
         const uint32_t splits = small_splits_of(t, m, n, k), nsb = (k + 255u) / 256u, sb_per = (nsb + splits - 1) / splits;
         float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
-        hipLaunchKernelGGL(kern, dim3(tm * tn * splits), dim3(64 * WAVES), 2 * ActTileT<BM_MID>::kTile, s, a, splits, sb_per, partial);
+        const int lds_small = 2 * (one128 ? ActTileT<BM_MID>::kTile : ActTile::kTile);
+        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds_small, "hipFuncSetAttribute(small gemm LDS)"))
+            return rc;
+        hipLaunchKernelGGL(kern, dim3(tn * splits), dim3(64 * WAVES), lds_small, s, a, splits, sb_per, partial);
         if (int rc = check_launch("small gemm kernel launch")) return rc;
         if (splits == 1) return HQ_OK;
-        const uint32_t count = m * n;  // m <= 128
+        const uint32_t count = m * n;  // m <= 256
         hipLaunchKernelGGL(split_sum_kernel, dim3((count + 255u) / 256u), dim3(256), 0, s, partial, y, count, splits);
         return check_launch("split sum kernel launch");
     };
     if (t == HQ_Q6_K) {
         if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
-        if (gemm_f16_small_tiles(t, m)) return launch_mid_small(mid_gemm_small_kernel<HQ_Q6_K>);
+        if (gemm_f16_small_tiles(t, m)) return launch_mid_small(mid_gemm_small_kernel<HQ_Q6_K, 4>, mid_gemm_small_kernel<HQ_Q6_K, 8>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(q6k_gemm_kernel), (size_t)lds, "hipFuncSetAttribute(q6_k gemm LDS)"))
             return rc;
         hipLaunchKernelGGL(q6k_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
@@ -1144,7 +1153,8 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
                                   : launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
             return rc;
         if (gemm_f16_small_tiles(t, m))
-            return launch_mid_small(t == HQ_Q4_0 ? mid_gemm_small_kernel<HQ_Q4_0> : mid_gemm_small_kernel<HQ_Q8_0>);
+            return t == HQ_Q4_0 ? launch_mid_small(mid_gemm_small_kernel<HQ_Q4_0, 4>, mid_gemm_small_kernel<HQ_Q4_0, 8>)
+                                : launch_mid_small(mid_gemm_small_kernel<HQ_Q8_0, 4>, mid_gemm_small_kernel<HQ_Q8_0, 8>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(q8_0 gemm LDS)"))
             return rc;
         hipLaunchKernelGGL(kern, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
@@ -1153,19 +1163,21 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
                               : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
         return rc;
-    if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: one token tile of 64 or of 128 rows, tiles of 128 weight rows
-        const bool one64 = m <= (uint32_t)BM_SMALL;
+    if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: one token tile of 64, 128 or 256 rows, tiles of 128 weight rows
+        const int mts = m <= (uint32_t)BM_SMALL ? 2 : m <= (uint32_t)BM_MID ? 4 : 8;
         void (*ksmall)(GemmArgs, uint32_t, uint32_t, float*) =
-            t == HQ_Q5_K ? (one64 ? q4k_gemm_small_kernel<HQ_Q5_K, 2> : q4k_gemm_small_kernel<HQ_Q5_K, 4>)
-                         : (one64 ? q4k_gemm_small_kernel<HQ_Q4_K, 2> : q4k_gemm_small_kernel<HQ_Q4_K, 4>);
+            t == HQ_Q5_K ? (mts == 2 ? q4k_gemm_small_kernel<HQ_Q5_K, 2> : mts == 4 ? q4k_gemm_small_kernel<HQ_Q5_K, 4> : q4k_gemm_small_kernel<HQ_Q5_K, 8>)
+                         : (mts == 2 ? q4k_gemm_small_kernel<HQ_Q4_K, 2> : mts == 4 ? q4k_gemm_small_kernel<HQ_Q4_K, 4> : q4k_gemm_small_kernel<HQ_Q4_K, 8>);
         const uint32_t tn = (n + BN_WIDE - 1) / BN_WIDE;
         const uint32_t splits = small_splits_of(t, m, n, k), nsb = k / 256, sb_per = (nsb + splits - 1) / splits;
         float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
-        const int lds_small = 2 * (one64 ? ActTileT<BM_SMALL>::kTile : ActTileT<BM_MID>::kTile);
+        const int lds_small = 2 * (mts == 2 ? ActTileT<BM_SMALL>::kTile : mts == 4 ? ActTileT<BM_MID>::kTile : ActTile::kTile);
+        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(ksmall), (size_t)lds_small, "hipFuncSetAttribute(q4k small gemm LDS)"))
+            return rc;
         hipLaunchKernelGGL(ksmall, dim3(tn * splits), dim3(64 * WAVES), lds_small, s, a, splits, sb_per, partial);
         if (int rc = check_launch("q4k small gemm kernel launch")) return rc;
         if (splits == 1) return HQ_OK;
-        const uint32_t count = m * n;  // m <= 128
+        const uint32_t count = m * n;  // m <= 256
         hipLaunchKernelGGL(split_sum_kernel, dim3((count + 255u) / 256u), dim3(256), 0, s, partial, y, count, splits);
         return check_launch("split sum kernel launch");
     }

@@ -97,7 +97,8 @@ HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, ui
  * src/serve/forward_mlx.rs:9655-9969).  m <= 8 takes the bandwidth-bound GEMV
  * kernels (MM_ROUTING_THRESHOLD, forward_mlx.rs:9791; from two to four rows on, by type, a form that fetches every
  * weight once for all rows), and Q4_K / Q5_K run up to 16 rows as two such passes; larger m takes the MFMA GEMM,
- * whose tiles are 64 token rows (Q4_K / Q5_K, up to 128 rows) or 128 (the other types, up to 128 rows) and 256 beyond.
+ * whose tiles are 64 (Q4_K / Q5_K), 128 or 256 token rows by m; up to 256 rows k is cut into slices where the
+ * weight-row tiles alone would leave CUs idle.
  * Where a K-quant's k has no small-batch kernel (k % 1024 != 0), up to 16 rows run as per-row GEMVs first.
  * MFMA GEMM.  The K-quant (k % 256 == 0) and Q8_0 / Q4_0 (k % 128 == 0) GEMMs multiply f16-rounded
  * weights and activations like the reference's mul_mm, the other kernels keep
@@ -110,8 +111,8 @@ HQ_API int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const 
 /* The same product with caller-owned device scratch.  The f16 tile kernels
  * (prefill-sized m; K-quants with k % 256 == 0, Q8_0 / Q4_0 with k % 128 == 0) convert the
  * activations to row-scaled f16 in a pre-pass and need hq_qmatmul_ggml_workspace_bytes() bytes (256-byte
- * aligned) for them -- plus, for up to 128 rows over few weight rows, the partial sums of
- * the slices k is cut into, which a second launch adds in a fixed order; every other shape needs none (the function returns 0 and
+ * aligned) for them -- plus, for up to 256 rows over few weight rows, the partial sums of
+ * the slices k is cut into (slices x m x n floats, up to eight slices), which a second launch adds in a fixed order; every other shape needs none (the function returns 0 and
  * `workspace` may be null).  hq_qmatmul_ggml itself takes that scratch from the
  * stream-ordered allocator (hipMallocAsync / hipFreeAsync on `stream`).  The
  * reference has no such buffer: its mul_mm kernel (quantized_matmul_ggml's

@@ -58,11 +58,13 @@ def test_gemm_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
     (100, 320, 256),    # a single run: no slices
     (64, 12288, 512),   # more tiles than CUs' worth: no slices
     (40, 200, 1152),    # Q8_0 / Q4_0 only: k % 256 = 128, the last run is half a one (and k is not cut)
+    (200, 130, 2304),   # one token tile of 256 rows, two slices
+    (256, 64, 4352),    # a full one, four slices
 ])
 def test_small_tiles_and_k_slices_match_f64_oracle(oracle, dev, t, m, n, k):
-    """Up to 128 activation rows: tiles of 64 token rows (Q4_K / Q5_K) or 128 (the other types), with k cut into slices
-    (summed in a fixed order by a second launch) where the tiles alone would leave most CUs idle; the same result on
-    every call."""
+    """Up to 256 activation rows are one token tile (64, 128 or 256 rows; Q4_K / Q5_K have the 64-row one), with k cut
+    into slices (summed in a fixed order by a second launch) where the weight-row tiles alone would leave most CUs idle;
+    the same result on every call."""
     if k % oracle.BLOCK_ELEMS[t]:
         pytest.skip("k is not a multiple of the block size")
     y, ref = _run(oracle, dev, t, "bf16", m, n, k)
