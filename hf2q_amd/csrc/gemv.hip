@@ -421,12 +421,14 @@ __device__ __forceinline__ void stream_load_x(const uint4* lds_x, const float* l
     }
 }
 
-template <int TYPE, int W, bool XREG>
+// ROWS = 2: two activation rows (x[0], x[1] -> y[0], y[1] of one matrix) share every weight fetch and the
+// nibble-to-bf16 work; the dot products and sums are per row, in the order of the one-row form.
+template <int TYPE, int W, bool XREG, int ROWS = 1>
 __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     constexpr uint32_t NT = 64 * W, BB = kBlockBytes<TYPE>;
     extern __shared__ uint4 smem[];
-    uint4* lds_x = smem;
-    float* lds_s = reinterpret_cast<float*>(lds_x + a.k / 8);
+    uint4* lds_x = smem;                                                // [ROWS][k / 8]
+    float* lds_s = reinterpret_cast<float*>(lds_x + ROWS * (a.k / 8));  // [ROWS][k / 16]
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
     const int c = (int)(lane & 3u);
     const uint32_t S = a.k / 4096u, rowb = a.k / 256u * BB;
@@ -436,9 +438,10 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     const uint32_t ntask = rows_mine * S;
 
     // the activations first, nothing else of this workgroup in front of them
-    for (uint32_t i = tid; i < a.k / 16u; i += NT) {
+    for (uint32_t ii = tid; ii < ROWS * (a.k / 16u); ii += NT) {
+        const uint32_t xr = ROWS == 1 ? 0u : ii / (a.k / 16u), i = ROWS == 1 ? ii : ii % (a.k / 16u);
         XRaw<true> raw;
-        raw.fetch(a.x, i);
+        raw.fetch(static_cast<const uint8_t*>(a.x) + (size_t)xr * a.k * 2u, i);
         const uint4 p = raw.r[0], q = raw.r[1];
         const uint32_t w[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
         uint4 o0, o1;
@@ -450,15 +453,15 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
         o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
         o1.z = (w[6] & 0xffffu) | (w[7] << 16);
         o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
-        lds_x[stream_swz<TYPE>(2 * i)] = o0;
-        lds_x[stream_swz<TYPE>(2 * i + 1)] = o1;
+        lds_x[xr * (a.k / 8u) + stream_swz<TYPE>(2 * i)] = o0;
+        lds_x[xr * (a.k / 8u) + stream_swz<TYPE>(2 * i + 1)] = o1;
         float s = 0.f;  // the same order of additions as stage_store
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             s += bf16_bits_to_f32(w[j] & 0xffffu);
             s += bf16_bits_to_f32(w[j] >> 16);
         }
-        lds_s[i] = s;
+        lds_s[xr * (a.k / 16u) + i] = s;
     }
 
     Piece<TYPE> pc;
@@ -474,30 +477,42 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
                  : "=v"(m4), "=v"(m2), "=v"(magic)
                  : "s"(a.m4), "s"(a.m2), "s"(a.magic));
-    uint32_t xp[32];
-    float sx[4];
-    if constexpr (XREG) stream_load_x<TYPE>(lds_x, lds_s, 0, lane, c, xp, sx);  // k == 4096: one piece per lane for every row
+    uint32_t xp[ROWS][32];
+    float sx[ROWS][4];
+    if constexpr (XREG) {  // k == 4096: one piece per lane for every row
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) stream_load_x<TYPE>(lds_x + r * (a.k / 8u), lds_s + r * (a.k / 16u), 0, lane, c, xp[r], sx[r]);
+    }
 
     uint32_t row = row_first, st = 0;
-    float acc = 0.f;
+    float acc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) acc[r] = 0.f;
     for (uint32_t t = 0; t < ntask; ++t) {
-        if constexpr (!XREG) stream_load_x<TYPE>(lds_x, lds_s, st, lane, c, xp, sx);
-        acc += dot_pair(pc, c, xp, sx, m4, m2, magic);
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            if constexpr (!XREG) stream_load_x<TYPE>(lds_x + r * (a.k / 8u), lds_s + r * (a.k / 16u), st, lane, c, xp[r], sx[r]);
+            acc[r] += dot_pair(pc, c, xp[r], sx[r], m4, m2, magic);
+        }
         if (t + 1 < ntask) {
             if (++f_st == S) {
                 f_st = 0;
                 f_row += stride;
             }
-            asm volatile("" : "+v"(acc));  // the refill follows the arithmetic that frees its registers
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) asm volatile("" : "+v"(acc[r]));  // the refill follows the arithmetic that frees its registers
             fetch(f_row, f_st);
         }
         if (++st == S) {
-            const float v = group_sum(acc, 6);
-            if (lane == 0) {
-                if (row < a.n0) a.y0[row] = v;
-                else a.y1[row - a.n0] = v;
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const float v = group_sum(acc[r], 6);
+                if (lane == 0) {
+                    if (row < a.n0) a.y0[(size_t)r * a.n + row] = v;  // (ROWS == 2: one matrix, n0 == n)
+                    else a.y1[row - a.n0] = v;
+                }
+                acc[r] = 0.f;
             }
-            acc = 0.f;
             st = 0;
             row += stride;
         }
@@ -510,15 +525,18 @@ template <int TYPE>
 constexpr bool kStreamType = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K;
 constexpr uint32_t STREAM_MIN_ROWS_PER_WAVE = 2;
 
-template <int TYPE>
+template <int TYPE, int ROWS = 1>
 int launch_stream(hipStream_t s, const SArgs& sa, uint32_t cus) {
     constexpr int W = TYPE == HQ_Q6_K ? 12 : 16;
-    const size_t lds = (size_t)sa.k * 2 + (size_t)(sa.k / 16) * 4;
-    if (sa.k == 4096) {
-        auto kern = gemv_stream_kernel<TYPE, W, true>;
+    const size_t lds = ROWS * ((size_t)sa.k * 2 + (size_t)(sa.k / 16) * 4);
+    // (the two-row Q5_K form with its activations in registers would spill: it reads them from LDS per row piece)
+    if (sa.k == 4096 && !(TYPE == HQ_Q5_K && ROWS == 2)) {
+        auto kern = gemv_stream_kernel<TYPE, W, true, ROWS>;
+        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
         hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
     } else {
-        auto kern = gemv_stream_kernel<TYPE, W, false>;
+        auto kern = gemv_stream_kernel<TYPE, W, false, ROWS>;
+        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
         hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
     }
     return check_launch("gemv stream kernel launch");
@@ -588,8 +606,15 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
     if constexpr (X_BF16 && kStreamType<TYPE>) {
-        if (a.pairs == 1 && !a.x2 && !a.ids && !a.route_logits && stream_takes<TYPE>(a.n, a.k, cus))
-            return launch_stream<TYPE>(s, SArgs{a.x, a.w, a.w, a.y, a.y, a.n, a.n, a.k, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC}, cus);
+        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && stream_takes<TYPE>(a.n, a.k, cus)) {
+            // activation rows of a dense product two at a time (one pass over the weights per two rows), a last odd one alone
+            for (uint32_t r = 0; r < a.pairs; r += 2) {
+                const SArgs sa{static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * 2, a.w, a.w, a.y + (size_t)r * a.n, a.y + (size_t)r * a.n,
+                               a.n, a.n, a.k, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
+                if (int rc = a.pairs - r >= 2 ? launch_stream<TYPE, 2>(s, sa, cus) : launch_stream<TYPE, 1>(s, sa, cus)) return rc;
+            }
+            return HQ_OK;
+        }
     }
     // Dense matrices with many tasks per wave: the queue kernel.
     if (a.pairs == 1 && !a.x2 && !a.ids && !a.route_logits &&
@@ -646,6 +671,15 @@ int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
 }
 
 }  // namespace
+
+// Q6_K with bf16 activations on a matrix the streaming kernel takes: passes of two rows cost less than the small-batch
+// kernel up to five rows (151936 x 4096: 105 us per two rows against 310 us for any 4..8; 12288 x 4096: 10 against 32).
+bool gemv_two_row_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
+    if (t != HQ_Q6_K || xdt != HQ_BF16 || m < 3 || m > 5) return false;
+    uint32_t cus = 0;
+    if (cu_count(&cus)) return false;
+    return stream_takes<HQ_Q6_K>(n, k, cus);
+}
 
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t) {
     const bool bf = xdt == HQ_BF16;
