@@ -306,13 +306,34 @@ def bench_prefill_gemm(a, wtype=None):
     us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
     flops = 2.0 * M * N * K
     tf = flops / us / 1e6
+    # For scale only (not part of the path, not in `value`): the vendor library's plain f16 GEMM of the same shape,
+    # no dequantisation, through torch.matmul; the same event timing over the same number of launches.
+    vendor = None
+    try:
+        xa = x.to(torch.float16)
+        wb = [torch.randn(N, K, generator=gen, device=dev).mul_(0.02).to(torch.float16) for _ in range(3)]
+        for i in range(max(3, a.warmup)):
+            torch.matmul(xa, wb[i % 3].t())
+        torch.cuda.synchronize()
+        evv = _events(a.steps)
+        for i in range(a.steps):
+            evv[i][0].record()
+            torch.matmul(xa, wb[i % 3].t())
+            evv[i][1].record()
+        torch.cuda.synchronize()
+        vus = sum(e0.elapsed_time(e1) for e0, e1 in evv) * 1e3 / a.steps
+        vendor = {"what": "torch.matmul f16 2048x4096 @ 4096x12288 (hipBLASLt), plain weights", "us_per_launch": round(vus, 2),
+                  "TFLOP/s": round(flops / vus / 1e6, 1), "frac_mfma_peak": round(flops / vus / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        del wb
+    except Exception as e:  # the reference figure must never take the bench line down
+        vendor = {"error": str(e)[:200]}
     return _finish(a, {
         "metric": "prefill TFLOP/s", "value": round(flops * a.steps / elapsed / 1e12, 1), "unit": "TFLOP/s",
         "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f16" if need else "bf16",
         "config": {"workload": f"prefill_gemm: 2048 tokens x K=4096 x N=12288, {wtype.upper()} weights, bf16 "
                                f"activations, fp32 accumulate (BASELINE config 4)", "flop_per_step": flops,
                    "weight_bytes": w.numel(), "workspace_bytes": need,
-                   "launches_per_step": 2 if need else 1},
+                   "launches_per_step": 2 if need else 1, "vendor_dense_gemm_same_shape": vendor},
         "roofline": {"bound": "mfma", "kernel": (f"activation pre-pass + f16 MFMA gemm {wtype}" if need else
                                                  f"bf16 MFMA gemm {wtype}"), "achieved": round(tf, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
