@@ -818,16 +818,22 @@ __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 }
 
 // Tile order: workgroups go to the 8 XCDs round-robin and every XCD has its own L2, so workgroup i
-// runs on XCD i % 8.  Each XCD gets whole rows of tiles (one activation tile, which then stays in
-// that XCD's L2) and sweeps the weight tiles.  The grid is padded to 8 * ceil(tiles_m / 8) * tiles_n.
+// runs on XCD i % 8.  The tiles, counted along the weight rows first, are cut into eight equal runs and
+// XCD x takes run x: its workgroups share one activation tile (or two, at a seam) that stays in that XCD's L2 while
+// they sweep the weight tiles -- and every XCD has work whatever the number of token tiles is (with whole rows of
+// tiles per XCD, 512 .. 1792 tokens kept two to seven of the eight XCDs busy and took the time of 2048).
+// The grid is padded to 8 * ceil(tiles / 8).
 __device__ __forceinline__ bool tile_of(uint32_t b, uint32_t tiles_m, uint32_t tiles_n, uint32_t bn, uint32_t& m0, uint32_t& n0) {
+    const uint32_t total = tiles_m * tiles_n, run = (total + 7u) / 8u;
     const uint32_t xcd = b & 7u, idx = b >> 3;
-    const uint32_t rows_here = (tiles_m + 7u - xcd) / 8u;
-    if (idx >= rows_here * tiles_n) return false;
-    m0 = (xcd + 8u * (idx / tiles_n)) * BM;
-    n0 = (idx % tiles_n) * bn;
+    const uint32_t flat = xcd * run + idx;
+    if (idx >= run || flat >= total) return false;
+    m0 = (flat / tiles_n) * BM;
+    n0 = (flat % tiles_n) * bn;
     return true;
 }
+// Workgroups of a launch whose tiles tile_of() hands out.
+inline uint32_t tile_grid(uint32_t tiles_m, uint32_t tiles_n) { return 8u * ((tiles_m * tiles_n + 7u) / 8u); }
 
 // Weight rows [0, n_wide) in tiles of 128 (the first grid_wide workgroups), the rest in tiles of 64.
 template <int TYPE>
@@ -1119,7 +1125,6 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr, 0u, (k + 255u) / 256u};
     constexpr int lds = 2 * ActTile::kTile;
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
-    const uint32_t pad_m = 8u * ((tiles_m + 7u) / 8u);
     // up to 256 token rows of Q6_K / Q8_0 / Q4_0: one token tile of 128 or 256 rows x 128 weight rows, k in slices where
     // that leaves CUs idle
     auto launch_mid_small = [&](void (*k128)(GemmArgs, uint32_t, uint32_t, float*),
@@ -1144,7 +1149,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         if (gemm_f16_small_tiles(t, m)) return launch_mid_small(mid_gemm_small_kernel<HQ_Q6_K, 4>, mid_gemm_small_kernel<HQ_Q6_K, 8>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(q6k_gemm_kernel), (size_t)lds, "hipFuncSetAttribute(q6_k gemm LDS)"))
             return rc;
-        hipLaunchKernelGGL(q6k_gemm_kernel, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
+        hipLaunchKernelGGL(q6k_gemm_kernel, dim3(tile_grid(tiles_m, cols_wide)), dim3(64 * WAVES), lds, s, a);
         return check_launch("q6_k gemm kernel launch");
     }
     if (t == HQ_Q8_0 || t == HQ_Q4_0) {
@@ -1157,7 +1162,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
                                 : launch_mid_small(mid_gemm_small_kernel<HQ_Q8_0, 4>, mid_gemm_small_kernel<HQ_Q8_0, 8>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(q8_0 gemm LDS)"))
             return rc;
-        hipLaunchKernelGGL(kern, dim3(pad_m * cols_wide), dim3(64 * WAVES), lds, s, a);
+        hipLaunchKernelGGL(kern, dim3(tile_grid(tiles_m, cols_wide)), dim3(64 * WAVES), lds, s, a);
         return check_launch("q8_0 gemm kernel launch");
     }
     if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
@@ -1192,7 +1197,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     const uint32_t cols_narrowed = (uint64_t)tiles_m * cols_wide <= cus / 2 ? cols_wide : 0;  // columns cut in two
     const uint32_t n_wide = (cols_wide - cols_narrowed) * BN_WIDE;  // < n whenever cols_narrowed > 0
     const uint32_t cols_narrow = n_wide < n ? (n - n_wide + BN_NARROW - 1) / BN_NARROW : 0;
-    const uint32_t grid_wide = pad_m * (cols_wide - cols_narrowed), grid_narrow = pad_m * cols_narrow;
+    const uint32_t grid_wide = tile_grid(tiles_m, cols_wide - cols_narrowed), grid_narrow = tile_grid(tiles_m, cols_narrow);
     hipLaunchKernelGGL(kern, dim3(grid_wide + grid_narrow), dim3(64 * WAVES), lds, s, a, n_wide, grid_wide);
     return check_launch("q4k gemm kernel launch");
 }
