@@ -205,10 +205,12 @@ def test_perm021_matches_oracle_and_the_plain_product(oracle, dev, t, m, heads, 
         ops.quantized_matmul_mm_tensor_perm021(x_perm, wd, y, ops.GgmlQuantizedMatmulPerm021Params(m, n, k, hd + 8, t))
 
 
-def test_tile_gemm_with_caller_workspace_replays_from_a_hip_graph(oracle, dev):
-    """hq_qmatmul_ggml_ws on the f16 tile route (m > 64) allocates nothing, so a prefill step can record it into a
-    HIP graph: three replays with the activations rewritten in between, each checked against the eager call."""
-    m, n, k, t = 96, 384, 1024, HQ_Q4_K
+@pytest.mark.parametrize("k", [1024, 4096])
+def test_tile_gemm_with_caller_workspace_replays_from_a_hip_graph(oracle, dev, k):
+    """hq_qmatmul_ggml_ws on the f16 tile route allocates nothing, so a prefill step can record it into a HIP graph:
+    three replays with the activations rewritten in between, each checked against the eager call.  k = 4096 cuts k
+    into four slices here (pre-pass, tiles, ordered sum: three launches, no memset node)."""
+    m, n, t = 96, 384, HQ_Q4_K
     w = torch.from_numpy(oracle.quantize(weights(71, n, k), k, t, threads=8)).to(dev)
     p = GgmlQuantizedMatmulParams(m, n, k, t)
     need = ops.quantized_matmul_workspace_bytes(p, torch.bfloat16)
