@@ -12,8 +12,10 @@
 //   * a consumer recognises fresh data by a TAG = (calls so far on this scratch) + 1: router logits and SwiGLU
 //     activations travel as 64-bit (tag, value) words, so a value and its freshness arrive in one store, no store has
 //     to be ordered behind another, and nothing has to be cleared between calls; workgroup 0 stores the new call count
-//     when it leaves (every workgroup has read the old one by then: workgroup 0 cannot get past the routing before
-//     all of them have delivered their logits);
+//     when it leaves (every workgroup has read the old one by then: every workgroup delivers logits of every token,
+//     so workgroup 0 cannot get past its token's routing before all of them have started);
+//   * after the logits a workgroup works for one token (token b % T): it polls that token's logits only, routes it,
+//     takes gate / up rows and down columns of that token;
 //   * the down projections are cut by output columns, not by expert: a workgroup computes its 8 .. 64 columns for every
 //     slot of a token and sums them itself, so the outputs never cross workgroups.
 // No workgroup ever waits for a later phase of another one, so the grid drains whatever the residency; the waits are
@@ -95,20 +97,23 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
     extern __shared__ uint4 smem[];
     const Layout L{a.T, a.E, a.K};
     const uint32_t T = a.T, E = a.E, K = a.K, S = K + 1;
-    // LDS: [staged activations of all tokens | later: one token's SwiGLU activations of all slots] | logits | ids | weights | partials
-    uint4* lds_x = smem;                                                       // T * H/8 chunks (paired bf16 words)
-    float* lds_sx = reinterpret_cast<float*>(lds_x + (size_t)T * (FH / 8));    // T * H/16 per-16 sums
-    const uint32_t area = T * (FH / 8) * 16 + T * (FH / 16) * 4, act_bytes = S * (FI * 4 + FI / 16 * 4);
+    // After phase 1 a workgroup works for ONE token, token b % T: it needs that token's logits, activations and routing
+    // only (eight tokens: an eighth of the words to poll for).
+    // LDS: [the token's staged activations | later: its SwiGLU activations of all slots] | logits | ids | weights | partials
+    uint4* lds_x = smem;                                                       // H/8 chunks (paired bf16 words)
+    float* lds_sx = reinterpret_cast<float*>(lds_x + FH / 8);                  // H/16 per-16 sums
+    const uint32_t area = (FH / 8) * 16 + (FH / 16) * 4, act_bytes = S * (FI * 4 + FI / 16 * 4);
     uint8_t* after = reinterpret_cast<uint8_t*>(smem) + (area > act_bytes ? area : act_bytes);
     float4* lds_act = reinterpret_cast<float4*>(smem);                         // S * I floats (over the activations, after phase 2)
     float* lds_as = reinterpret_cast<float*>(lds_act + (size_t)S * (FI / 4));  // S * I/16 sums
-    float* lds_lg = reinterpret_cast<float*>(after);                           // T * (E + 1)
-    uint32_t* lds_id = reinterpret_cast<uint32_t*>(lds_lg + (size_t)T * (E + 1));  // T * K
-    float* lds_w = reinterpret_cast<float*>(lds_id + (size_t)T * K);           // T * (K + 1): slot K = shared gate
-    float* lds_part = lds_w + (size_t)T * S;                                   // S * 64 down partials of one unit
+    float* lds_lg = reinterpret_cast<float*>(after);                           // E + 1
+    uint32_t* lds_id = reinterpret_cast<uint32_t*>(lds_lg + (E + 1));          // K
+    float* lds_w = reinterpret_cast<float*>(lds_id + K);                       // K + 1: slot K = shared gate
+    float* lds_part = lds_w + S;                                               // S * 64 down partials of one unit
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6, b = blockIdx.x, G = gridDim.x;
-    const uint32_t gw = b * WAVES + wv, NW = G * WAVES;  // this wave among all waves of the launch
+    const uint32_t tok = b % T, jb = b / T, nb = (G - tok + T - 1u) / T;  // the token, this workgroup among its nb workgroups
+    const uint32_t tw = jb * WAVES + wv, NTW = nb * WAVES;               // this wave among the token's waves
     uint32_t* s_epoch = reinterpret_cast<uint32_t*>(a.scratch);
     uint32_t* s_err = s_epoch + 1;
     uint64_t* s_lg = reinterpret_cast<uint64_t*>(a.scratch + L.logits());
@@ -119,20 +124,19 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
 
     // the activations of all tokens, requested first and staged while the logits travel (the layout and sums of
     // stage_store); 16 activations per thread and pass
-    constexpr uint32_t XPASS = (MAX_T * (FH / 16) + THREADS - 1) / THREADS;
-    XRaw<true> xraw[XPASS];
-#pragma unroll
-    for (uint32_t ps = 0; ps < XPASS; ++ps) {
-        const uint32_t i = tid + ps * THREADS;
-        if (i < T * (FH / 16)) xraw[ps].fetch(a.x + (size_t)(i / (FH / 16)) * FH, i % (FH / 16));
-    }
+    static_assert(FH / 16 <= THREADS, "one pass stages a token");
+    XRaw<true> xraw;
+    xraw.fetch(a.x + (size_t)tok * FH, tid < FH / 16 ? tid : 0u);  // (no branch around the load)
 
     // ---- phase 1: router logits and the shared-gate logit, one (row, token) per wave and turn, with the arithmetic of
-    // dense_gemv_bf16_kernel.  Every workgroup has a task here, which is what lets workgroup 0 bump the call counter at
-    // its end (see the header comment). ----
+    // dense_gemv_bf16_kernel. ----
     const uint32_t n_rows = E + (a.sh_lw ? 1u : 0u);
-    for (uint32_t q = b + G * wv; q < n_rows * T; q += NW) {  // task q belongs to workgroup q % G (G <= n_rows: every workgroup has one)
-        const uint32_t r = q / T, t = q % T;
+    // Workgroup b takes the rows b, b + G, ... for every token (G <= n_rows: it has at least one row), its waves the
+    // (row, token) pairs in turn.  Every workgroup so delivers logits of EVERY token, which matters for the call
+    // counter: a workgroup cannot get past its token's routing before all workgroups have started and read it.
+    const uint32_t rows_mine = (n_rows - b + G - 1u) / G;
+    for (uint32_t q = wv; q < rows_mine * T; q += WAVES) {
+        const uint32_t r = b + G * (q / T), t = q % T;
         const uint4* wr = reinterpret_cast<const uint4*>(r < E ? a.router + (size_t)r * FH : a.sh_lw);
         const uint4* xr = reinterpret_cast<const uint4*>(a.x + (size_t)t * FH);
         uint4 wq[FH / 8 / 64], xq[FH / 8 / 64];
@@ -156,51 +160,47 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
     }
 
     // ---- while the logits travel: the staged activations go to LDS ----
+    if (tid < FH / 16) {
+        const uint32_t j = tid;
+        const uint4 p = xraw.r[0], q = xraw.r[1];
+        const uint32_t w[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
+        uint4 o0, o1;
+        o0.x = (w[0] & 0xffffu) | (w[1] << 16);
+        o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
+        o0.z = (w[2] & 0xffffu) | (w[3] << 16);
+        o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
+        o1.x = (w[4] & 0xffffu) | (w[5] << 16);
+        o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
+        o1.z = (w[6] & 0xffffu) | (w[7] << 16);
+        o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
+        lds_x[swz8(2 * j)] = o0;
+        lds_x[swz8(2 * j + 1)] = o1;
+        float sum = 0.f;
 #pragma unroll
-    for (uint32_t ps = 0; ps < XPASS; ++ps) {
-        const uint32_t i = tid + ps * THREADS;
-        if (i < T * (FH / 16)) {
-            const uint32_t t = i / (FH / 16), j = i % (FH / 16);
-            const uint4 p = xraw[ps].r[0], q = xraw[ps].r[1];
-            const uint32_t w[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
-            uint4 o0, o1;
-            o0.x = (w[0] & 0xffffu) | (w[1] << 16);
-            o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
-            o0.z = (w[2] & 0xffffu) | (w[3] << 16);
-            o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
-            o1.x = (w[4] & 0xffffu) | (w[5] << 16);
-            o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
-            o1.z = (w[6] & 0xffffu) | (w[7] << 16);
-            o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
-            lds_x[t * (FH / 8) + swz8(2 * j)] = o0;
-            lds_x[t * (FH / 8) + swz8(2 * j + 1)] = o1;
-            float sum = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                sum += bf16_bits_to_f32(w[e] & 0xffffu);
-                sum += bf16_bits_to_f32(w[e] >> 16);
-            }
-            lds_sx[i] = sum;
+        for (int e = 0; e < 8; ++e) {
+            sum += bf16_bits_to_f32(w[e] & 0xffffu);
+            sum += bf16_bits_to_f32(w[e] >> 16);
         }
+        lds_sx[j] = sum;
     }
 
-    // ---- every logit of every token, then the routing (each workgroup for itself, a wave per token) ----
-    for (uint32_t i = tid; i < T * (E + 1); i += THREADS)
-        lds_lg[i] = i % (E + 1) < n_rows ? __uint_as_float(wait_tagged(&s_lg[i], tag, a.spin_limit, s_err)) : 0.f;
+    // ---- the token's logits, then its routing (every workgroup of the token for itself, one wave) ----
+    for (uint32_t i = tid; i < E + 1; i += THREADS)
+        lds_lg[i] = i < n_rows ? __uint_as_float(wait_tagged(&s_lg[(size_t)tok * (E + 1) + i], tag, a.spin_limit, s_err)) : 0.f;
     __syncthreads();
-    for (uint32_t t = wv; t < T; t += WAVES) {
+    if (wv == 0) {
         uint32_t id;
         float wt;
-        softmax_topk_lane<4>(lds_lg + (size_t)t * (E + 1), E, K, lane, id, wt);
+        softmax_topk_lane<4>(lds_lg, E, K, lane, id, wt);
         if (lane < K) {
-            lds_id[t * K + lane] = id;
-            lds_w[t * S + lane] = wt;
-            if (b == 0 && a.route_ids) {
-                a.route_ids[t * K + lane] = id;
-                a.route_w[t * K + lane] = wt;
+            lds_id[lane] = id;
+            lds_w[lane] = wt;
+            if (jb == 0 && a.route_ids) {
+                a.route_ids[tok * K + lane] = id;
+                a.route_w[tok * K + lane] = wt;
             }
         }
-        if (lane == 0) lds_w[t * S + K] = a.sh_lw ? 1.f / (1.f + expf(-lds_lg[(size_t)t * (E + 1) + E])) : 1.f;  // ffn.rs:28-30
+        if (lane == 0) lds_w[K] = a.sh_lw ? 1.f / (1.f + expf(-lds_lg[E])) : 1.f;  // ffn.rs:28-30
     }
     __syncthreads();
 
@@ -209,54 +209,52 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
                  : "=v"(m4), "=v"(m2), "=v"(magic)
                  : "s"(a.m4), "s"(a.m2), "s"(a.magic));
 
-    // ---- phase 2: gate and up row p % I of slot (p / I) % S of token p / (I * S), lanes 0-31 the gate row and 32-63
-    // the up row, then the SwiGLU; the waves of the launch take the rows in turn, RING fetches ahead ----
+    // ---- phase 2: gate and up row p % I of slot p / I of the token, lanes 0-31 the gate row and 32-63 the up row, then
+    // the SwiGLU; the waves of the token's workgroups take the rows in turn, RING fetches ahead ----
     {
         const uint32_t li = lane & 31u, hf = lane >> 5;
         const int c4 = (int)(li & 3u);
-        const uint32_t P = T * S * FI;
-        const uint32_t mine = gw < P ? (P - gw + NW - 1u) / NW : 0u;
+        const uint32_t P = S * FI;
+        const uint32_t mine = tw < P ? (P - tw + NTW - 1u) / NTW : 0u;
         const uint32_t lane_off = (li >> 2) * Q4K_BYTES;
         auto fetch = [&](Piece<HQ_Q4_K>& pc, uint32_t p) {
-            const uint32_t r = p % FI, ts = p / FI, s = ts % S, t = ts / S;
-            const uint8_t* base = s < K ? (hf ? a.eu : a.eg) + (size_t)lds_id[t * K + s] * a.stride_gu : (hf ? a.su : a.sg);
+            const uint32_t r = p % FI, s = p / FI;
+            const uint8_t* base = s < K ? (hf ? a.eu : a.eg) + (size_t)lds_id[s] * a.stride_gu : (hf ? a.su : a.sg);
             pc.load(base + (size_t)r * ROWB_H + lane_off, c4);
         };
         Piece<HQ_Q4_K> ring[RING];
 #pragma unroll
         for (int i = 0; i < RING; ++i)
-            if ((uint32_t)i < mine) fetch(ring[i], gw + (uint32_t)i * NW);
+            if ((uint32_t)i < mine) fetch(ring[i], tw + (uint32_t)i * NTW);
         uint32_t xp[32];
         float sx[4];
-        uint32_t cur_t = ~0u;
+        {
+            const uint32_t ch0 = li * 8u;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint4 v = lds_x[swz8(ch0 + j)];
+                xp[4 * j] = v.x;
+                xp[4 * j + 1] = v.y;
+                xp[4 * j + 2] = v.z;
+                xp[4 * j + 3] = v.w;
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sx[r] = lds_sx[ch0 / 2 + r];
+        }
         for (uint32_t i0 = 0; i0 < mine; i0 += RING) {
 #pragma unroll
             for (int i = 0; i < RING; ++i) {
                 const uint32_t n = i0 + (uint32_t)i;
                 if (n < mine) {
-                    const uint32_t p = gw + n * NW, t = p / (FI * S);
-                    if (t != cur_t) {  // uniform
-                        cur_t = t;
-                        const uint32_t ch0 = li * 8u;
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const uint4 v = lds_x[t * (FH / 8) + swz8(ch0 + j)];
-                            xp[4 * j] = v.x;
-                            xp[4 * j + 1] = v.y;
-                            xp[4 * j + 2] = v.z;
-                            xp[4 * j + 3] = v.w;
-                        }
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) sx[r] = lds_sx[t * (FH / 16) + ch0 / 2 + r];
-                    }
+                    const uint32_t p = tw + n * NTW;
                     const float v = group_sum(dot_pair(ring[i], c4, xp, sx, m4, m2, magic), 5);
                     const float up = __shfl(v, 32);
                     if (n + RING < mine) {
                         float tie = v;
                         asm volatile("" : "+v"(tie));
-                        fetch(ring[i], p + RING * NW);
+                        fetch(ring[i], p + RING * NTW);
                     }
-                    if (lane == 0) st_dev(&s_act[p], tag_hi | __float_as_uint(silu_mul_f32(v, up)));
+                    if (lane == 0) st_dev(&s_act[(size_t)tok * P + p], tag_hi | __float_as_uint(silu_mul_f32(v, up)));
                 }
             }
         }
@@ -269,14 +267,13 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
         const uint32_t li = lane & 7u, sub = lane >> 3;
         const int c4 = (int)(li & 3u);
         const uint32_t groups = T <= 1 ? 1u : T <= 2 ? 2u : T <= 4 ? 4u : 8u, cols = 8u * groups;  // columns per unit: about one unit per workgroup
-        const uint32_t units_per_t = FH / cols, U = T * units_per_t;
-        for (uint32_t u = b; u < U; u += G) {
-            const uint32_t t = u / units_per_t, c = u % units_per_t;
+        const uint32_t units_per_t = FH / cols, t = tok;
+        for (uint32_t c = jb; c < units_per_t; c += nb) {
             // steps of this wave: (slot s, row group g) = step index wv, wv + WAVES, ... of S * groups
             const uint32_t n_steps = S * groups, mine = wv < n_steps ? (n_steps - wv + WAVES - 1u) / WAVES : 0u;
             auto fetch = [&](Piece<HQ_Q4_K>& pc, uint32_t n) {
                 const uint32_t st = wv + n * WAVES, s = st / groups, g = st % groups;
-                const uint8_t* base = s < K ? a.ed + (size_t)lds_id[t * K + s] * a.stride_d : a.sd;
+                const uint8_t* base = s < K ? a.ed + (size_t)lds_id[s] * a.stride_d : a.sd;
                 pc.load(base + (size_t)(cols * c + 8 * g + sub) * ROWB_I + (li >> 2) * Q4K_BYTES, c4);
             };
             Piece<HQ_Q4_K> ring[RING];
@@ -371,7 +368,7 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
             if (tid < cols) {
                 const uint32_t col = cols * c + tid;
                 float acc = 0.f;
-                for (uint32_t s = 0; s < S; ++s) acc = fmaf(lds_w[t * S + s], lds_part[s * cols + tid], acc);
+                for (uint32_t s = 0; s < S; ++s) acc = fmaf(lds_w[s], lds_part[s * cols + tid], acc);
                 if (a.residual) acc += a.residual[(size_t)t * FH + col];
                 a.out[(size_t)t * FH + col] = acc;
             }
@@ -390,7 +387,7 @@ size_t moe_fused_scratch_bytes(uint32_t n_tokens, uint32_t n_experts, uint32_t t
 bool moe_fused_supported(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k, uint32_t inter,
                          uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt) {
     return t == HQ_Q4_K && xdt == HQ_BF16 && hidden == FH && inter == FI && shared_inter == FI && n_tokens >= 1 &&
-           n_tokens <= 8 && n_experts >= 1 && n_experts <= 256 && top_k >= 1 && top_k <= 64 && top_k <= n_experts;
+           n_tokens <= 8 && n_experts >= n_tokens && n_experts <= 256 && top_k >= 1 && top_k <= 64 && top_k <= n_experts;
 }
 
 int launch_moe_fused(hipStream_t s, const MoeFusedArgs& m) {
@@ -423,10 +420,12 @@ int launch_moe_fused(hipStream_t s, const MoeFusedArgs& m) {
     // every workgroup must deliver at least one logit row (see the header comment), and one workgroup per CU
     const uint32_t rows = m.n_experts + (m.shared_gate_logit ? 1u : 0u);
     const uint32_t grid = cus < rows ? cus : rows;
-    const uint32_t T = m.n_tokens, S = m.top_k + 1;
-    const size_t area = (size_t)T * (FH / 8) * 16 + (size_t)T * (FH / 16) * 4, act_bytes = (size_t)S * (FI * 4 + FI / 16 * 4);
-    const size_t lds = (area > act_bytes ? area : act_bytes) + (size_t)T * (m.n_experts + 1) * 4 + (size_t)T * m.top_k * 4 +
-                       (size_t)T * S * 4 + (size_t)S * 64 * 4;
+    if (grid < m.n_tokens)  // after the logits a workgroup works for one token: every token needs a workgroup
+        return fail(HQ_ERR_UNSUPPORTED, "fused MoE block: %u tokens over %u router rows", m.n_tokens, rows);
+    const uint32_t S = m.top_k + 1;
+    const size_t area = (size_t)(FH / 8) * 16 + (size_t)(FH / 16) * 4, act_bytes = (size_t)S * (FI * 4 + FI / 16 * 4);
+    const size_t lds = (area > act_bytes ? area : act_bytes) + (size_t)(m.n_experts + 1) * 4 + (size_t)m.top_k * 4 + (size_t)S * 4 +
+                       (size_t)S * 64 * 4;
     if (lds > 64 * 1024) return fail(HQ_ERR_UNSUPPORTED, "fused MoE block: %zu bytes of LDS", lds);
     hipLaunchKernelGGL(moe_fused_kernel, dim3(grid), dim3(THREADS), lds, s, a);
     return check_launch("fused MoE block launch");

@@ -245,7 +245,7 @@ HQ_API int hq_moe_weighted_reduce(void* stream, const float* y, const float* w, 
  * buffer); moe_ffn_cpu_ref (ffn.rs:179-336) is the specification.  The result has the bits of the separate dispatches
  * (hq_dense_gemv_bf16_pair, hq_qmatmul_batch_ggml twice with the routing and the SwiGLU folded in,
  * hq_moe_weighted_reduce).  Takes 1..8 tokens of bf16 activations, Q4_K experts, hidden 2048, expert and shared FFN
- * width 512, <= 256 experts, top_k <= 64; anything else is HQ_ERR_UNSUPPORTED (hq_moe_ffn_decode_scratch_bytes
+ * width 512, n_tokens <= n_experts <= 256, top_k <= 64; anything else is HQ_ERR_UNSUPPORTED (hq_moe_ffn_decode_scratch_bytes
  * returns 0 for it) and runs as the separate dispatches.
  * `scratch`: hq_moe_ffn_decode_scratch_bytes() bytes of device memory, 256-byte aligned, ZEROED ONCE before its first
  * use and then left to the library (it carries a call counter; calls that share a scratch must not overlap, and a
