@@ -167,6 +167,9 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q6_K>& p, int c, const 
 
 // ---- f32 activations (xf: this lane's 64 (32 for Q8_0) activations, sx: run sums) ----
 __device__ __forceinline__ float dot4(uint32_t q, const float* x, float acc) {
+    // q is a word of four masked bytes; hidden from the optimiser, which would otherwise fold the mask into a bit-field
+    // extract per byte (v_bfe + v_cvt_f32_ubyte0) where v_cvt_f32_ubyte0..3 of the one masked word do
+    asm("" : "+v"(q));
     acc = fmaf(ubyte0(q), x[0], acc);
     acc = fmaf(ubyte1(q), x[1], acc);
     acc = fmaf(ubyte2(q), x[2], acc);
@@ -359,14 +362,14 @@ __device__ __forceinline__ float dpp_add(float v) {
 
 // Sum over aligned groups of L = 2^log_l lanes; every lane of a group ends up with
 // the group's sum.  Quad permutes and row mirrors cover 16 lanes, the last two
-// levels cross 16-lane rows and go through ds_bpermute.
+// levels cross 16-lane rows with permlane swaps.
 __device__ __forceinline__ float group_sum(float v, uint32_t log_l) {
     if (log_l >= 1) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
     if (log_l >= 2) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
     if (log_l >= 3) v = dpp_add<0x141>(v);  // row_half_mirror
     if (log_l >= 4) v = dpp_add<0x140>(v);  // row_mirror
-    if (log_l >= 5) v += __shfl_xor(v, 16);
-    if (log_l >= 6) v += __shfl_xor(v, 32);
+    if (log_l >= 5) v = xor16_add(v);
+    if (log_l >= 6) v = xor32_add(v);
     return v;
 }
 

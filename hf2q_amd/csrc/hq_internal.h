@@ -191,6 +191,31 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
                                            __builtin_bit_cast(bf16x2_t, b), c, false);
 }
 
+// Exchanges across the 16-lane rows of a wave without LDS traffic: v_permlane16_swap / v_permlane32_swap hand every
+// lane its own value and the one of lane ^ 16 (resp. lane ^ 32) as the pair r[0], r[1] — which of the two is the
+// lane's own depends on the row, so they serve commutative operations.  The results have the bits of the
+// __shfl_xor forms they replace.
+__device__ __forceinline__ float xor16_add(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor32_add(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor16_max(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor32_max(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 // (a & b) | c in one VALU op.  The compiler splits this into v_and + v_or when b
 // and c are literals (gfx9 VOP3 takes no literal operands), so the constants are
 // passed in registers and the instruction is written out.

@@ -31,6 +31,7 @@
 
 #include "hq_internal.h"
 #include "moe_topk.h"
+
 #include "gemv_pieces.h"
 
 namespace hq {
@@ -42,6 +43,10 @@ constexpr uint32_t ROWB_I = FI / 256 * Q4K_BYTES;     // bytes of a down row
 constexpr uint32_t WAVES = 8, THREADS = 64 * WAVES;
 constexpr uint32_t MAX_T = 8;                         // tokens per call
 constexpr int RING = 4;                               // weight fetches a wave keeps in flight
+constexpr int POLL = 5;  // activation loads of a thread per polling pass: (8 + 1) slots x 512 / 2 words over 512 threads = 4.5
+// A logit is stored LG_COPIES times and a workgroup polls copy (its index among its token's workgroups) % LG_COPIES: at
+// one token 256 workgroups would otherwise poll the same 2 KB (sixteen cache lines, a few memory channels).
+constexpr uint32_t LG_COPIES = 8;
 
 struct FusedArgs {
     const uint16_t* x;       // [T][H] bf16
@@ -63,8 +68,8 @@ struct FusedArgs {
 struct Layout {
     uint32_t T, E, K;
     __host__ __device__ uint32_t slots() const { return K + 1; }  // routed slots + the shared expert
-    __host__ __device__ size_t logits() const { return 64; }     // u64 [T][E + 1]
-    __host__ __device__ size_t act() const { return logits() + (size_t)T * (E + 1) * 8; }  // u64 [T][K + 1][I]
+    __host__ __device__ size_t logits() const { return 64; }  // u64 [LG_COPIES][T][E + 1]
+    __host__ __device__ size_t act() const { return logits() + (size_t)LG_COPIES * T * (E + 1) * 8; }  // u64 [T][K + 1][I]
     __host__ __device__ size_t total() const { return act() + (size_t)T * slots() * FI * 8; }
 };
 
@@ -156,7 +161,7 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
             }
         }
         acc = wave_sum(acc);
-        if (lane == 0) st_dev(&s_lg[(size_t)t * (E + 1) + r], tag_hi | __float_as_uint(acc));
+        if (lane < LG_COPIES) st_dev(&s_lg[((size_t)lane * T + t) * (E + 1) + r], tag_hi | __float_as_uint(acc));
     }
 
     // ---- while the logits travel: the staged activations go to LDS ----
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
 
     // ---- the token's logits, then its routing (every workgroup of the token for itself, one wave) ----
     for (uint32_t i = tid; i < E + 1; i += THREADS)
-        lds_lg[i] = i < n_rows ? __uint_as_float(wait_tagged(&s_lg[(size_t)tok * (E + 1) + i], tag, a.spin_limit, s_err)) : 0.f;
+        lds_lg[i] = i < n_rows ? __uint_as_float(wait_tagged(&s_lg[((size_t)(jb % LG_COPIES) * T + tok) * (E + 1) + i], tag, a.spin_limit, s_err)) : 0.f;
     __syncthreads();
     if (wv == 0) {
         uint32_t id;
@@ -269,10 +274,15 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
         const uint32_t groups = T <= 1 ? 1u : T <= 2 ? 2u : T <= 4 ? 4u : 8u, cols = 8u * groups;  // columns per unit: about one unit per workgroup
         const uint32_t units_per_t = FH / cols, t = tok;
         for (uint32_t c = jb; c < units_per_t; c += nb) {
-            // steps of this wave: (slot s, row group g) = step index wv, wv + WAVES, ... of S * groups
-            const uint32_t n_steps = S * groups, mine = wv < n_steps ? (n_steps - wv + WAVES - 1u) / WAVES : 0u;
+            // steps (slot s, row group g) = step index s * groups + g.  With several row groups a wave takes a run of
+            // consecutive steps, so that it changes slot (and reloads the slot's activations from LDS) as seldom as
+            // possible; with one row group (one token) every step is another slot and the waves take the steps in turn.
+            const uint32_t n_steps = S * groups;
+            const bool runs = groups > 1;
+            const uint32_t st0 = runs ? wv * n_steps / WAVES : wv, stp = runs ? 1u : WAVES;
+            const uint32_t mine = runs ? (wv + 1u) * n_steps / WAVES - st0 : wv < n_steps ? (n_steps - wv + WAVES - 1u) / WAVES : 0u;
             auto fetch = [&](Piece<HQ_Q4_K>& pc, uint32_t n) {
-                const uint32_t st = wv + n * WAVES, s = st / groups, g = st % groups;
+                const uint32_t st = st0 + n * stp, s = st / groups, g = st % groups;
                 const uint8_t* base = s < K ? a.ed + (size_t)lds_id[s] * a.stride_d : a.sd;
                 pc.load(base + (size_t)(cols * c + 8 * g + sub) * ROWB_I + (li >> 2) * Q4K_BYTES, c4);
             };
@@ -281,36 +291,41 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
             for (int i = 0; i < RING; ++i)
                 if ((uint32_t)i < mine) fetch(ring[i], (uint32_t)i);
             // the token's SwiGLU activations of every slot: (tag, value) words, two per 16-byte load, all of a thread's
-            // loads in flight at once and the whole batch asked for again until every word of it is fresh
+            // loads of a pass in flight at once; a load whose words are not both fresh is asked for again
             {
                 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
                 const uint64_t* src = s_act + (size_t)(t * S) * FI;
                 const uint32_t n2 = S * FI / 2;
-                for (uint32_t base = 0; base < n2; base += 8 * THREADS) {
-                    u32x4 got[8];
-                    bool fresh = false;
-                    for (uint32_t tries = 0; !fresh; ++tries) {
+                for (uint32_t base = 0; base < n2; base += POLL * THREADS) {
+                    u32x4 got[POLL];
+                    uint32_t off[POLL];
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) {
-                            const uint32_t e2 = base + tid + (uint32_t)i * THREADS;
-                            const uint64_t* p = src + 2 * (e2 < n2 ? e2 : 0u);
-                            asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(got[i]) : "v"(p) : "memory");
-                        }
+                    for (int i = 0; i < POLL; ++i) {
+                        const uint32_t e2 = base + tid + (uint32_t)i * THREADS;
+                        off[i] = 16u * (e2 < n2 ? e2 : tid);  // past the end: a word of the thread's own, not used
+                        asm volatile("global_load_dwordx4 %0, %1, %2 sc0 sc1" : "=v"(got[i]) : "v"(off[i]), "s"(src) : "memory");
+                    }
+                    for (uint32_t tries = 0;; ++tries) {
                         // the results exist once the counter has drained; naming them keeps their uses below the wait
-                        asm volatile("s_waitcnt vmcnt(0)"
-                                     : "+v"(got[0]), "+v"(got[1]), "+v"(got[2]), "+v"(got[3]), "+v"(got[4]), "+v"(got[5]), "+v"(got[6]), "+v"(got[7])
-                                     :
-                                     : "memory");
-                        fresh = true;
+                        if constexpr (POLL == 5)
+                            asm volatile("s_waitcnt vmcnt(0)" : "+v"(got[0]), "+v"(got[1]), "+v"(got[2]), "+v"(got[3]), "+v"(got[4]) : : "memory");
+                        bool fresh = true;
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) fresh = fresh && got[i].y == tag && got[i].w == tag;
-                        if (!fresh && tries >= a.spin_limit) {
+                        for (int i = 0; i < POLL; ++i) {
+                            if (got[i].y != tag || got[i].w != tag) {
+                                fresh = false;
+                                asm volatile("global_load_dwordx4 %0, %1, %2 sc0 sc1" : "+v"(got[i]) : "v"(off[i]), "s"(src) : "memory");
+                            }
+                        }
+                        if (fresh) break;
+                        if (tries >= a.spin_limit) {
                             st_dev(s_err, 2u);
+                            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                             break;
                         }
                     }
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) {
+                    for (int i = 0; i < POLL; ++i) {
                         const uint32_t e2 = base + tid + (uint32_t)i * THREADS;
                         if (e2 < n2) {
                             const uint32_t e = 2 * e2, sl = e / FI, k = e % FI, q = k >> 2;  // piece p = q / 16 reads float4 slot q ^ p
@@ -340,7 +355,7 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
                 for (int i = 0; i < RING; ++i) {
                     const uint32_t n = i0 + (uint32_t)i;
                     if (n < mine) {
-                        const uint32_t st = wv + n * WAVES, s = st / groups, g = st % groups;
+                        const uint32_t st = st0 + n * stp, s = st / groups, g = st % groups;
                         if (s != cur_s) {  // uniform
                             cur_s = s;
 #pragma unroll

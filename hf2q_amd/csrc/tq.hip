@@ -176,8 +176,7 @@ constexpr int HD = 256;           // head_dim handled by the attention kernels
 constexpr int TMP_STRIDE = HD + 2;  // per (head, split): unnormalised output, running max, running sum
 
 __device__ __forceinline__ float wave_max4(float v) {  // over the 4 lane groups that share lane%16
-    v = fmaxf(v, __shfl_xor(v, 16));
-    return fmaxf(v, __shfl_xor(v, 32));
+    return xor32_max(xor16_max(v));
 }
 
 // 8 int8 (two words) -> 8 bf16 as an MFMA fragment.
@@ -434,9 +433,8 @@ __global__ __launch_bounds__(256) void tq_attn_split_kernel(AttnArgs a) {
 #pragma unroll
     for (int h = 0; h < 8; ++h)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] += __shfl_xor(acc[h][e], 32);
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
+        for (int e = 0; e < 8; ++e) acc[h][e] = xor32_add(acc[h][e]);
+    l_run = xor32_add(xor16_add(l_run));
     __syncthreads();
     if (half == 0) {
 #pragma unroll
@@ -833,10 +831,8 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
 
     // ---- merge of the four waves.  First the maxima, so that every wave can bring its own numbers to
     // the workgroup's scale before they meet: O_row = (acc - lp) * 2^(mv - m_wg) / 2^14, l * 2^(m - m_wg).
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
-    lp_run += __shfl_xor(lp_run, 16);
-    lp_run += __shfl_xor(lp_run, 32);
+    l_run = xor32_add(xor16_add(l_run));
+    lp_run = xor32_add(xor16_add(lp_run));
     if (lane < 8u) s_m[wave][lane] = m_run;
     __syncthreads();
     const uint32_t hj = j & 7u;
