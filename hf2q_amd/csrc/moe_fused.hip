@@ -96,6 +96,11 @@ __device__ __forceinline__ uint32_t wait_tagged(const uint64_t* p, uint32_t tag,
     return (uint32_t)got;
 }
 
+// A workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for the wave's outstanding global
+// stores, and a write-through store is acknowledged by memory a microsecond or more after it was issued (several under
+// load): time in which the next phase's loads can already be on their way.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 __device__ __forceinline__ uint32_t swz8(uint32_t ch) { return ch ^ ((ch >> 4) & 7u); }
 
 __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
@@ -115,8 +120,10 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
     uint32_t* lds_id = reinterpret_cast<uint32_t*>(lds_lg + (E + 1));          // K
     float* lds_w = reinterpret_cast<float*>(lds_id + K);                       // K + 1: slot K = shared gate
     float* lds_part = lds_w + S;                                               // S * 64 down partials of one unit
+    uint32_t* lds_gath = reinterpret_cast<uint32_t*>(lds_part + S * 64);       // 64 * WAVES: the workgroup's SwiGLU activations
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6, b = blockIdx.x, G = gridDim.x;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, b = blockIdx.x, G = gridDim.x;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));  // known to be the same in a wave: scalar branches
     const uint32_t tok = b % T, jb = b / T, nb = (G - tok + T - 1u) / T;  // the token, this workgroup among its nb workgroups
     const uint32_t tw = jb * WAVES + wv, NTW = nb * WAVES;               // this wave among the token's waves
     uint32_t* s_epoch = reinterpret_cast<uint32_t*>(a.scratch);
@@ -216,11 +223,24 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
 
     // ---- phase 2: gate and up row p % I of slot p / I of the token, lanes 0-31 the gate row and 32-63 the up row, then
     // the SwiGLU; the waves of the token's workgroups take the rows in turn, RING fetches ahead ----
+    // The activations are not stored where they arise.  Loads and stores are counted by one counter and return in order,
+    // and a write-through store is acknowledged by memory a microsecond or more after its issue (several under load): a
+    // store among the fetches holds back every fetch behind it.  Lane n keeps the activation of the wave's row n; after
+    // the phase the waves put theirs together in LDS and ONE wave stores the workgroup's rows (eight consecutive words
+    // per row index: 64-byte pieces instead of 8-byte ones), after the next phase's first weight fetches have been issued.
+    // (A wave with more than 64 rows, which takes a small grid and many slots, stores for itself.)
+    uint32_t keep = 0;
+    const uint32_t P = S * FI;
+    const uint32_t rows2 = tw < P ? (P - tw + NTW - 1u) / NTW : 0u;
+    const uint32_t rows2_wg = jb * WAVES < P ? (P - jb * WAVES + NTW - 1u) / NTW : 0u;  // of the workgroup's first wave: the most
+    const bool gather = rows2_wg <= 64u;
+    auto flush = [&](uint32_t first, uint32_t count) {
+        if (lane < count) st_dev(&s_act[(size_t)tok * P + tw + (first + lane) * NTW], tag_hi | keep);
+    };
     {
         const uint32_t li = lane & 31u, hf = lane >> 5;
         const int c4 = (int)(li & 3u);
-        const uint32_t P = S * FI;
-        const uint32_t mine = tw < P ? (P - tw + NTW - 1u) / NTW : 0u;
+        const uint32_t mine = rows2;
         const uint32_t lane_off = (li >> 2) * Q4K_BYTES;
         auto fetch = [&](Piece<HQ_Q4_K>& pc, uint32_t p) {
             const uint32_t r = p % FI, s = p / FI;
@@ -246,6 +266,7 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) sx[r] = lds_sx[ch0 / 2 + r];
         }
+        float keep_g = 0.f, keep_u = 0.f;
         for (uint32_t i0 = 0; i0 < mine; i0 += RING) {
 #pragma unroll
             for (int i = 0; i < RING; ++i) {
@@ -253,18 +274,50 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
                 if (n < mine) {
                     const uint32_t p = tw + n * NTW;
                     const float v = group_sum(dot_pair(ring[i], c4, xp, sx, m4, m2, magic), 5);
-                    const float up = __shfl(v, 32);
+                    const float gate = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+                    const float up = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
                     if (n + RING < mine) {
                         float tie = v;
                         asm volatile("" : "+v"(tie));
                         fetch(ring[i], p + RING * NTW);
                     }
-                    if (lane == 0) st_dev(&s_act[(size_t)tok * P + p], tag_hi | __float_as_uint(silu_mul_f32(v, up)));
+                    keep_g = lane == (n & 63u) ? gate : keep_g;  // the SwiGLU of up to 64 rows is one pass at the end
+                    keep_u = lane == (n & 63u) ? up : keep_u;
+                    if ((n & 63u) == 63u && n + 1u < mine) {
+                        keep = __float_as_uint(silu_mul_f32(keep_g, keep_u));
+                        flush(n - 63u, 64u);
+                    }
                 }
             }
         }
+        keep = __float_as_uint(silu_mul_f32(keep_g, keep_u));
     }
-    __syncthreads();  // the staged activations are dead from here on: their LDS holds the SwiGLU activations next
+    if (gather && lane < rows2) lds_gath[lane * WAVES + wv] = keep;
+    // The workgroup's activations go out by its last wave (or by every wave for itself), which then waits for the stores'
+    // acknowledgement while the other waves issue the next phase's first weight fetches; nobody polls before that: the
+    // other workgroups' stores were issued at about the same time, so the first poll finds nearly everything, and polls
+    // that start earlier only get in the way of the stores.
+    const bool storing = !gather || wv == WAVES - 1u;
+    auto store_acts = [&]() {
+        if (gather) {
+            if (storing)
+                for (uint32_t idx = lane; idx < rows2_wg * WAVES; idx += 64u) {
+                    const uint32_t p = jb * WAVES + idx % WAVES + idx / WAVES * NTW;
+                    if (p < P) st_dev(&s_act[(size_t)tok * P + p], tag_hi | lds_gath[idx]);
+                }
+        } else if (rows2) {
+            flush((rows2 - 1u) & ~63u, ((rows2 - 1u) & 63u) + 1u);
+        }
+    };
+    auto await_acts_stored = [&]() {
+        if (storing) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (gather) lds_barrier();
+    };
+    // Every fetch of the phase has been consumed: a wait that costs nothing and tells the compiler so (it cannot see it
+    // from the loop's conditions), or it would make the next phase's fetches wait for each other for the sake of the
+    // registers they share with these.
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    lds_barrier();  // the staged activations are dead from here on: their LDS holds the SwiGLU activations next
 
     // ---- phases 3 + 4: unit (token t, column slice c): the down rows of the slice for every slot of the token, then
     // the weighted sum over the slots in slot order, the shared expert last (the order of moe_weighted_reduce_kernel) ----
@@ -273,6 +326,8 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
         const int c4 = (int)(li & 3u);
         const uint32_t groups = T <= 1 ? 1u : T <= 2 ? 2u : T <= 4 ? 4u : 8u, cols = 8u * groups;  // columns per unit: about one unit per workgroup
         const uint32_t units_per_t = FH / cols, t = tok;
+        store_acts();
+        if (jb >= units_per_t) await_acts_stored();  // a workgroup without a unit
         for (uint32_t c = jb; c < units_per_t; c += nb) {
             // steps (slot s, row group g) = step index s * groups + g.  With several row groups a wave takes a run of
             // consecutive steps, so that it changes slot (and reloads the slot's activations from LDS) as seldom as
@@ -287,9 +342,18 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
                 pc.load(base + (size_t)(cols * c + 8 * g + sub) * ROWB_I + (li >> 2) * Q4K_BYTES, c4);
             };
             Piece<HQ_Q4_K> ring[RING];
+            auto prefetch = [&]() {
 #pragma unroll
-            for (int i = 0; i < RING; ++i)
-                if ((uint32_t)i < mine) fetch(ring[i], (uint32_t)i);
+                for (int i = 0; i < RING; ++i)
+                    if ((uint32_t)i < mine) fetch(ring[i], (uint32_t)i);
+            };
+            if (c == jb && storing) {  // (a storing wave's fetches would stand in the queue in front of the acknowledgement's wait)
+                await_acts_stored();
+                prefetch();
+            } else {
+                prefetch();
+                if (c == jb) await_acts_stored();
+            }
             // the token's SwiGLU activations of every slot: (tag, value) words, two per 16-byte load, all of a thread's
             // loads of a pass in flight at once; a load whose words are not both fresh is asked for again
             {
@@ -379,6 +443,9 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
                     }
                 }
             }
+            // (every fetch has been consumed: a free wait that tells the compiler so, or it would make the next unit's first
+            // fetches wait for the output store below)
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
             __syncthreads();
             if (tid < cols) {
                 const uint32_t col = cols * c + tid;
@@ -440,7 +507,7 @@ int launch_moe_fused(hipStream_t s, const MoeFusedArgs& m) {
     const uint32_t S = m.top_k + 1;
     const size_t area = (size_t)(FH / 8) * 16 + (size_t)(FH / 16) * 4, act_bytes = (size_t)S * (FI * 4 + FI / 16 * 4);
     const size_t lds = (area > act_bytes ? area : act_bytes) + (size_t)(m.n_experts + 1) * 4 + (size_t)m.top_k * 4 + (size_t)S * 4 +
-                       (size_t)S * 64 * 4;
+                       (size_t)S * 64 * 4 + (size_t)64 * WAVES * 4;
     if (lds > 64 * 1024) return fail(HQ_ERR_UNSUPPORTED, "fused MoE block: %zu bytes of LDS", lds);
     hipLaunchKernelGGL(moe_fused_kernel, dim3(grid), dim3(THREADS), lds, s, a);
     return check_launch("fused MoE block launch");
