@@ -44,8 +44,8 @@ PMC_TRAFFIC_BYTES = {
     # split (with the q rotation) + merge (with the output rotation), 32K context, 2 kv heads, head_dim 256
     "tq_attention_32k_fused_chain": int((16897.5 + 1072.5) * 2.0 * 1024 + (2112.0 + 16.0) * 1.0 * 1024),
     # the one-launch MoE FFN block, hidden 2048, 256 experts x 512, top-8, 1 and 8 tokens
-    "moe_ffn_decode_t1": int(8711.3 * 2.0 * 1024 + 160.1 * 1.0 * 1024),
-    "moe_ffn_decode_t8": int(56290.7 * 2.0 * 1024 + 1280.8 * 1.0 * 1024),
+    "moe_ffn_decode_t1": int(8675.0 * 2.0 * 1024 + 108.3 * 1.0 * 1024),
+    "moe_ffn_decode_t8": int(63307.0 * 2.0 * 1024 + 866.5 * 1.0 * 1024),
 }
 
 
