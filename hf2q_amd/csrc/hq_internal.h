@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
 #include <stdint.h>
 
 #include "../../include/hf2q_hip.h"
@@ -214,6 +215,51 @@ __device__ __forceinline__ float xor32_max(float v) {
     const uint32_t u = __float_as_uint(v);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// x of lane ^ M without LDS traffic (a __shfl_xor is an LDS permute: a hundred cycles and more in a dependent chain).
+// Inside a row of 16 lanes two DPP moves compose the xor from the mirrors the hardware has (half mirror = l ^ 7, row
+// mirror = l ^ 15, quad reverse = l ^ 3); across rows a permlane swap delivers the pair (own row's value, partner
+// row's value) and the lane picks the partner's: r[0] holds the even rows' (lower half's) values, r[1] the odd rows'.
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int M>
+__device__ __forceinline__ float lane_xor(float x, uint32_t lane) {
+    static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "one bit of the lane index");
+    if constexpr (M == 1) {
+        return dpp_mov<0xB1>(x);  // quad_perm [1,0,3,2]
+    } else if constexpr (M == 2) {
+        return dpp_mov<0x4E>(x);  // quad_perm [2,3,0,1]
+    } else if constexpr (M == 4) {
+        return dpp_mov<0x1B>(dpp_mov<0x141>(x));  // half mirror, then quad_perm [3,2,1,0]
+    } else if constexpr (M == 8) {
+        return dpp_mov<0x141>(dpp_mov<0x140>(x));  // row mirror, then half mirror
+    } else if constexpr (M == 16) {
+        const uint32_t u = __float_as_uint(x);
+        const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+        return __uint_as_float(lane & 16u ? r[0] : r[1]);
+    } else {
+        const uint32_t u = __float_as_uint(x);
+        const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        return __uint_as_float(lane & 32u ? r[0] : r[1]);
+    }
+}
+
+// Butterfly reductions over aligned groups of lanes with the partners taken in the order of the xor distances
+// given (the order fixes the rounding of a sum); every lane of a group gets the result.
+template <int M, int... REST>
+__device__ __forceinline__ float xor_sum(float v, uint32_t lane) {
+    v += lane_xor<M>(v, lane);
+    if constexpr (sizeof...(REST) > 0) v = xor_sum<REST...>(v, lane);
+    return v;
+}
+template <int M, int... REST>
+__device__ __forceinline__ float xor_max(float v, uint32_t lane) {
+    v = fmaxf(v, lane_xor<M>(v, lane));
+    if constexpr (sizeof...(REST) > 0) v = xor_max<REST...>(v, lane);
+    return v;
 }
 
 // (a & b) | c in one VALU op.  The compiler splits this into v_and + v_or when b

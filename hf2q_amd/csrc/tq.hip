@@ -21,6 +21,8 @@
 // merges the splits.
 #include <math.h>
 
+#include <type_traits>
+
 #include "hq_internal.h"
 
 namespace hq {
@@ -69,15 +71,19 @@ __device__ __forceinline__ void fwht256(float (&v)[4], uint32_t lane) {
     v[2] = a - c;
     v[1] = b + d;
     v[3] = b - d;
+    // h = 4m: the partner lane differs in bit m; the upper lane's o - v is formed as (-v) + o, the same number
+    auto stage = [&](auto mm) {
+        constexpr int m = decltype(mm)::value;
+        const uint32_t flip = lane & (uint32_t)m ? 0x80000000u : 0u;
 #pragma unroll
-    for (int m = 1; m < 64; m <<= 1) {  // h = 4m: partner lane differs in bit m
-        const bool upper = lane & m;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const float o = __shfl_xor(v[e], m);
-            v[e] = upper ? o - v[e] : v[e] + o;
-        }
-    }
+        for (int e = 0; e < 4; ++e) v[e] = __uint_as_float(__float_as_uint(v[e]) ^ flip) + lane_xor<m>(v[e], lane);
+    };
+    stage(std::integral_constant<int, 1>{});
+    stage(std::integral_constant<int, 2>{});
+    stage(std::integral_constant<int, 4>{});
+    stage(std::integral_constant<int, 8>{});
+    stage(std::integral_constant<int, 16>{});
+    stage(std::integral_constant<int, 32>{});
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] *= 0.0625f;
 }
@@ -108,8 +114,7 @@ __global__ __launch_bounds__(64) void tq_encode_kernel(const float* __restrict__
     apply_signs(v, lane);
     fwht256(v, lane);
     float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
+    amax = xor_max<1, 2, 4, 8, 16, 32>(amax, lane);
     const float d = amax / 127.f;
     const float id = d != 0.f ? 1.f / d : 0.f;
     uint32_t packed = 0;
@@ -640,8 +645,7 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
             const float ax = fabsf(x[e]);
             amax = ax <= 3.0e38f ? fmaxf(amax, ax) : amax;
         }
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));  // the 32 threads of a head
+        amax = xor_max<16, 8, 4, 2, 1>(amax, lane);  // the 32 threads of a head
         // amax = f * 2^ex with f in [0.5, 1): scaling by 2^(10 - ex) brings it into [512, 1024)
         int sh = amax > 0.f ? 10 - __builtin_amdgcn_frexp_expf(amax) : 0;
         sh = sh < -100 ? -100 : sh > 100 ? 100 : sh;
@@ -658,11 +662,8 @@ __global__ __launch_bounds__(256) void tq_attn_split_f16_kernel(AttnArgs a) {
             sum_hi += ((e & 1) ? -1151.f : 1152.f) * (float)fh;
             sum_lo += ((e & 1) ? -1151.f : 1152.f) * (float)fl;
         }
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) {
-            sum_hi += __shfl_xor(sum_hi, o);
-            sum_lo += __shfl_xor(sum_lo, o);
-        }
+        sum_hi = xor_sum<16, 8, 4, 2, 1>(sum_hi, lane);
+        sum_lo = xor_sum<16, 8, 4, 2, 1>(sum_lo, lane);
         s_qf[b][h][ch] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16));
         s_qf[b][8 + h][ch] = make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16));
         if (ch == 0) {
@@ -914,16 +915,14 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void tq_attn_merge_kernel(const f
         ls = base[(size_t)tid * TMP_STRIDE + HD + 1];
     }
     float m = ms;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    m = xor_max<32, 16, 8, 4, 2, 1>(m, lane);
     if (lane == 0) s_red[wave] = m;
     __syncthreads();
     m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));  // splits live in the first 256 threads
     const float w = ms == -INFINITY ? 0.f : __expf(ms - m);
     if (tid < 256u) s_w[tid] = w;
     float lw = w * ls;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
+    lw = xor_sum<32, 16, 8, 4, 2, 1>(lw, lane);
     __syncthreads();  // s_red read by everyone before it is reused; s_w visible
     if (lane == 0) s_red[wave] = lw;
     float o[4] = {0.f, 0.f, 0.f, 0.f};
