@@ -39,14 +39,16 @@ template <>
 struct Piece<HQ_Q6_K> {
     uint4 qa, qb, qh;
     uint2 sc;
-    uint32_t d;
+    uint32_t d;  // the block's last four bytes: two scale bytes, then d (f16) in the upper half
     __device__ __forceinline__ void load(const uint8_t* blk, int c) {
         const int h = c >> 1, lr = c & 1;
         qa = ld16_unaligned(blk + 64 * h + 16 * lr);
         qb = ld16_unaligned(blk + 64 * h + 32 + 16 * lr);
         qh = ld16_unaligned(blk + 128 + 32 * h + 16 * lr);
         sc = ld8_unaligned(blk + 192 + 8 * h);
-        d = ld2(blk + 208);
+        // (a full word and a shift where d is used, not a half-word load: the masking that the compiler attaches to a
+        // half-word load sits where the load is issued, and in a pipelined loop its wait drains every fetch in flight)
+        d = ld4_unaligned(blk + 206);
     }
 };
 template <>
@@ -157,7 +159,7 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q6_K>& p, int c, const 
     // and the format's own -32, hence the 160.
     const int lr = c & 1;
     const uint32_t s01 = p.sc.x >> (8 * lr), s23 = p.sc.y >> (8 * lr);
-    const float d = f16_bits_to_f32(p.d);
+    const float d = f16_bits_to_f32(p.d >> 16);
     float acc = (float)(int)(int8_t)(s01 & 0xff) * (r0 - 160.f * sx[0]);
     acc += (float)(int)(int8_t)((s01 >> 16) & 0xff) * (r1 - 160.f * sx[1]);
     acc += (float)(int)(int8_t)(s23 & 0xff) * (r2 - 160.f * sx[2]);
@@ -205,7 +207,7 @@ __device__ __forceinline__ float dot_f32(const Piece<HQ_Q6_K>& p, int c, const f
     }
     const int lr = c & 1;
     const uint32_t s01 = p.sc.x >> (8 * lr), s23 = p.sc.y >> (8 * lr);
-    const float d = f16_bits_to_f32(p.d);
+    const float d = f16_bits_to_f32(p.d >> 16);
     float acc = (float)(int)(int8_t)(s01 & 0xff) * (r0 - 32.f * sx[0]);
     acc += (float)(int)(int8_t)((s01 >> 16) & 0xff) * (r1 - 32.f * sx[1]);
     acc += (float)(int)(int8_t)(s23 & 0xff) * (r2 - 32.f * sx[2]);

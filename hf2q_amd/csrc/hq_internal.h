@@ -182,6 +182,11 @@ __device__ __forceinline__ uint2 ld8_unaligned(const uint8_t* p) {
     __builtin_memcpy(&v, p, 8);
     return v;
 }
+__device__ __forceinline__ uint32_t ld4_unaligned(const uint8_t* p) {
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
 __device__ __forceinline__ uint32_t ld2(const uint8_t* p) {
     return *reinterpret_cast<const uint16_t*>(p);
 }
