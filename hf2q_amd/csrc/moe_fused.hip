@@ -96,11 +96,6 @@ __device__ __forceinline__ uint32_t wait_tagged(const uint64_t* p, uint32_t tag,
     return (uint32_t)got;
 }
 
-// A workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for the wave's outstanding global
-// stores, and a write-through store is acknowledged by memory a microsecond or more after it was issued (several under
-// load): time in which the next phase's loads can already be on their way.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
 __device__ __forceinline__ uint32_t swz8(uint32_t ch) { return ch ^ ((ch >> 4) & 7u); }
 
 __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
@@ -311,13 +306,13 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
     };
     auto await_acts_stored = [&]() {
         if (storing) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (gather) lds_barrier();
+        if (gather) __syncthreads();
     };
     // Every fetch of the phase has been consumed: a wait that costs nothing and tells the compiler so (it cannot see it
     // from the loop's conditions), or it would make the next phase's fetches wait for each other for the sake of the
     // registers they share with these.
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-    lds_barrier();  // the staged activations are dead from here on: their LDS holds the SwiGLU activations next
+    __syncthreads();  // the staged activations are dead from here on: their LDS holds the SwiGLU activations next
 
     // ---- phases 3 + 4: unit (token t, column slice c): the down rows of the slice for every slot of the token, then
     // the weighted sum over the slots in slot order, the shared expert last (the order of moe_weighted_reduce_kernel) ----
