@@ -305,6 +305,50 @@ def test_moe_block_one_launch_equals_batched_dispatches_and_cpu_spec(oracle, dev
     assert np.abs(got - want).max() <= 2e-4 * np.abs(want).max(), np.abs(got - want).max() / np.abs(want).max()
 
 
+@pytest.mark.parametrize("T", [1, 8])
+def test_moe_block_one_launch_replays_from_a_hip_graph(oracle, dev, T):
+    """Three consecutive layers' worth of hq_moe_ffn_decode over ONE scratch, recorded into a HIP graph (the call
+    counter in the scratch keeps counting across replays, nothing is cleared in between): four replays with the
+    activations rewritten and eager calls and synchronisations in between, every replay equal to the eager result."""
+    H, E, K, I, SI = 2048, 32, 8, 512, 512
+    layers = [_moe_weights(oracle, dev, HQ_Q4_K, H, E, K, I, SI, seed=40 + i) for i in range(3)]
+    x = torch.zeros(T, H, device=dev, dtype=torch.bfloat16)
+    res = torch.from_numpy(acts(61, T, H)).to(dev)
+    assert ops.moe_ffn_decode_fused_supported(x, layers[0])
+    s = ops.MoeFfnScratch(layers[0], T, dev)
+    outs = [torch.empty(T, H, device=dev) for _ in layers]
+    for w, o in zip(layers, outs):  # warm-up outside the capture
+        ops.build_moe_ffn_layer_gpu_q_into(x, w, s, o, residual=res)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            for w, o in zip(layers, outs):
+                ops.build_moe_ffn_layer_gpu_q_into(x, w, s, o, residual=res)
+    torch.cuda.synchronize()
+    calls = int(s.fused[0:4].view(torch.int32).item())
+    for rep in range(4):
+        x.copy_(torch.from_numpy(acts(70 + rep, T, H)).to(dev).to(torch.bfloat16))
+        for o in outs:
+            o.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        calls += 3
+        assert int(s.fused[0:4].view(torch.int32).item()) == calls
+        assert int(s.fused[4:8].view(torch.int32).item()) == 0, "a wait inside the launch ran out"
+        for i, w in enumerate(layers):  # eager: the batched dispatches (other kernels, the same bits)
+            want = torch.empty(T, H, device=dev)
+            ops.build_moe_ffn_layer_gpu_q_into(x, w, s, want, residual=res, batched=True)
+            torch.cuda.synchronize()
+            assert torch.equal(got[i], want), f"replay {rep}, layer {i}: max diff {(got[i] - want).abs().max().item()}"
+        ops.build_moe_ffn_layer_gpu_q_into(x, layers[0], s, outs[0], residual=res)  # an eager one-launch call in between
+        calls += 1
+        torch.cuda.synchronize()
+
+
 def test_moe_block_one_launch_rejects_other_shapes(oracle, dev):
     H, E, K, I, SI = 512, 16, 4, 256, 512
     w = _moe_weights(oracle, dev, HQ_Q4_K, H, E, K, I, SI)

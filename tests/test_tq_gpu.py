@@ -248,6 +248,42 @@ def test_fused_pre_rotation_equals_separate_dispatch(oracle, dev):
     assert np.array_equal(sep, fused)  # forward_mlx.rs:4646-4652: the fused path is bit-identical
 
 
+def test_one_call_attention_chain_replays_from_a_hip_graph(oracle, dev):
+    """The decode step's attention (split with the query rotation inside, merge with the output rotation inside: two
+    launches, caller-owned tmp, no allocation) recorded into a HIP graph: four replays with the query rewritten and an
+    eager call in between, every replay equal to the eager result."""
+    hd, nh, nkv, n, cap = 256, 16, 2, 3000, 4096
+    rng = np.random.default_rng(77)
+    kc, kn = _oracle_cache(oracle, rng.standard_normal((n, nkv, hd)).astype(np.float32), nkv, hd, cap)
+    vc, vn = _oracle_cache(oracle, rng.standard_normal((n, nkv, hd)).astype(np.float32), nkv, hd, cap)
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    kc, kn, vc, vn = dv(kc), dv(kn), dv(vc), dv(vn)
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, cap, 0.0625, fuse_fwht_pre=1)
+    q = torch.zeros(nh, hd, device=dev)
+    out = torch.empty(nh, hd, device=dev)
+    tmp = torch.empty(ops.tq_tmp_buffer_bytes(nh, hd, n) // 4, device=dev)
+    ops.flash_attn_vec_tq_hb(q, kc, kn, vc, vn, out, tmp, p, undo_rotation=True)  # warm-up outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            ops.flash_attn_vec_tq_hb(q, kc, kn, vc, vn, out, tmp, p, undo_rotation=True)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        q.copy_(dv(rng.standard_normal((nh, hd)).astype(np.float32)))
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = torch.empty_like(out)
+        ops.flash_attn_vec_tq_hb(q, kc, kn, vc, vn, want, tmp, p, undo_rotation=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {rep}"
+        assert torch.isfinite(got).all()
+
+
 @pytest.mark.parametrize("n,cap,kw", [(300, 512, {}), (5000, 5000, {}), (512, 512, {"mask_type": 2, "sliding_window": 200, "ring_start": 31})])
 def test_fused_post_rotation_equals_separate_dispatch(oracle, dev, n, cap, kw):
     """Attention whose merge pass applies the inverse rotation gives the bits of attention followed by
