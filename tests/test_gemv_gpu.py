@@ -456,3 +456,48 @@ def test_small_batch_rows_adversarial_blocks_and_scaling(oracle, dev, t):
         y2 = torch.empty_like(y)
         ops.quantized_matmul_ggml(xd * 1024, wd, y2, GgmlQuantizedMatmulParams(m, n, k, t))
         assert torch.equal(y2, y * 1024)
+
+
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
+def test_decode_gemvs_replay_from_a_hip_graph(oracle, dev, t):
+    """The streaming GEMV form (one workgroup per CU, results kept in lanes and stored 64 rows at a time) as a decode
+    loop runs it: a single matrix and the two-matrix launch recorded into a HIP graph, three replays with the
+    activations rewritten, every replay equal to the eager calls and within the GEMV bound of the f64 product."""
+    n, k = 8192, 4096  # enough rows for two per wave of the device: the streaming route
+    w0 = oracle.quantize(weights(201, n, k), k, t, threads=8)
+    w1 = oracle.quantize(weights(202, n, k), k, t, threads=8)
+    dq0 = oracle.dequantize(w0, t, threads=8).reshape(n, k).astype(np.float64)
+    wd0, wd1 = torch.from_numpy(w0).to(dev), torch.from_numpy(w1).to(dev)
+    x = torch.zeros(1, k, device=dev, dtype=torch.bfloat16)
+    y, ya, yb = (torch.empty(1, n, device=dev) for _ in range(3))
+    p = GgmlQuantizedMatmulParams(1, n, k, t)
+
+    def step(o, oa, ob):
+        ops.quantized_matmul_ggml(x, wd0, o, p)
+        ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x, wd0, oa, 1, n, k), ops.QmatmulJob(x, wd1, ob, 1, n, k)], t)
+
+    step(y, ya, yb)  # warm-up outside the capture (kernel attributes are set here)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            step(y, ya, yb)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        xa = acts(210 + rep, 1, k)
+        x.copy_(torch.from_numpy(xa).to(dev).to(torch.bfloat16))
+        for o in (y, ya, yb):
+            o.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in (y, ya, yb)]
+        want = [torch.empty(1, n, device=dev) for _ in range(3)]
+        step(*want)
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), f"replay {rep}"
+        assert torch.equal(got[0], got[1])  # the same matrix through the one-matrix and the two-matrix launch
+        xb = x.float().cpu().numpy().astype(np.float64)
+        assert_matmul_close(got[0].cpu().numpy(), xb @ dq0.T, f"replay {rep}")
