@@ -82,62 +82,78 @@ __device__ __forceinline__ uint32_t f16_bits(float v) {
     return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)v);
 }
 
-// Pre-pass.  Workgroups [0, m): one per activation row, row scale and f16 conversion.  Workgroups
-// from m on: 16 weight rows each, 16 lanes per row over the row's block headers.  Per weight row, a
-// power of two that brings the row's largest possible |w| (Q4_K: |d|*63*15 + |dmin|*63, Q6_K:
-// |d|*128*32, Q8_0: |d|*128) to about 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
-// subnormals; the main kernel multiplies the weights by it before they are rounded (exact) and its
-// epilogue divides it out.
-template <bool X_BF16, int TYPE>
-__global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
-                                                        uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k,
-                                                        const uint32_t* __restrict__ row_map, uint32_t top_k, uint32_t perm_hd) {
-    __shared__ float red[4];
-    const uint32_t tid = threadIdx.x;
-    const Workspace L = workspace_layout(m, n, k);
-    if (blockIdx.x >= m) {
-        const uint32_t wr = (blockIdx.x - m) * 16u + (tid >> 4);
-        float bound = 0.f;
-        if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K) {  // |w| <= |d| * 63 * qmax + |dmin| * 63
-            constexpr uint32_t BYTES = TYPE == HQ_Q5_K ? Q5K_BYTES : Q4K_BYTES;
-            constexpr float DQ = TYPE == HQ_Q5_K ? 1953.f : 945.f;
-            const uint32_t nsb = k / 256;
-            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nsb * BYTES;
-            for (uint32_t sb = tid & 15u; sb < nsb; sb += 16u) {
-                const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow + (size_t)sb * BYTES);
-                const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * DQ + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
-                bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;  // inf / nan scales do not set the exponent
-            }
-        } else if constexpr (TYPE == HQ_Q6_K) {  // |w| <= |d| * 128 * 32
-            const uint32_t nsb = k / 256;
-            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nsb * Q6K_BYTES;
-            for (uint32_t sb = tid & 15u; sb < nsb; sb += 16u) {
-                const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)sb * Q6K_BYTES + 208))) * 4096.f;
-                bound = v <= 3.0e38f ? fmaxf(bound, v) : bound;
-            }
-        } else {  // Q8_0: |w| <= |d| * 128; Q4_0: |w| <= |d| * 8
-            constexpr uint32_t BYTES = TYPE == HQ_Q4_0 ? Q4_0_BYTES : Q8_0_BYTES;
-            constexpr float QMAX = TYPE == HQ_Q4_0 ? 8.f : 128.f;
-            const uint32_t nb = k / 32;
-            const uint8_t* wrow = w + (size_t)(wr < n ? wr : n - 1u) * nb * BYTES;
-            for (uint32_t b = tid & 15u; b < nb; b += 16u) {
-                const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)b * BYTES))) * QMAX;
-                bound = v <= 3.0e38f ? fmaxf(bound, v) : bound;
-            }
+// Largest possible |w| of the blocks first, first + step, ... (< count) of a weight row, from their scales alone
+// (Q4_K: |d|*63*15 + |dmin|*63, Q5_K: |d|*63*31 + |dmin|*63, Q6_K: |d|*128*32, Q8_0: |d|*128, Q4_0: |d|*8); blocks are
+// the type's own (super-blocks of 256 for the K-quants, blocks of 32 otherwise).  inf / nan scales do not count.
+template <int TYPE>
+__device__ __forceinline__ float weight_row_bound(const uint8_t* wrow, uint32_t k, uint32_t first, uint32_t step) {
+    float bound = 0.f;
+    if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K) {
+        constexpr uint32_t BYTES = TYPE == HQ_Q5_K ? Q5K_BYTES : Q4K_BYTES;
+        constexpr float DQ = TYPE == HQ_Q5_K ? 1953.f : 945.f;
+        for (uint32_t sb = first; sb < k / 256; sb += step) {
+            const uint32_t dd = *reinterpret_cast<const uint32_t*>(wrow + (size_t)sb * BYTES);
+            const float b = fabsf(f16_bits_to_f32(dd & 0xffffu)) * DQ + fabsf(f16_bits_to_f32(dd >> 16)) * 63.f;
+            bound = b <= 3.0e38f ? fmaxf(bound, b) : bound;
         }
-        bound = dpp_max<0xB1>(bound);  // the four steps cover a row of 16 lanes
-        bound = dpp_max<0x4E>(bound);
-        bound = dpp_max<0x141>(bound);
-        bound = dpp_max<0x140>(bound);
-        int ex = 0;
-        if (bound > 0.f) (void)frexpf(bound, &ex);  // bound = f * 2^ex, f in [0.5, 1)
-        const int e = bound > 0.f ? ex - 14 : 0;
-        if ((tid & 15u) == 0 && wr < n) reinterpret_cast<float*>(ws + L.wdown)[wr] = ldexpf(1.f, -e);  // |e| <= 40: normal
-        return;
+    } else if constexpr (TYPE == HQ_Q6_K) {
+        for (uint32_t sb = first; sb < k / 256; sb += step) {
+            const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)sb * Q6K_BYTES + 208))) * 4096.f;
+            bound = v <= 3.0e38f ? fmaxf(bound, v) : bound;
+        }
+    } else {
+        constexpr uint32_t BYTES = TYPE == HQ_Q4_0 ? Q4_0_BYTES : Q8_0_BYTES;
+        constexpr float QMAX = TYPE == HQ_Q4_0 ? 8.f : 128.f;
+        for (uint32_t b = first; b < k / 32; b += step) {
+            const float v = fabsf(f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(wrow + (size_t)b * BYTES))) * QMAX;
+            bound = v <= 3.0e38f ? fmaxf(bound, v) : bound;
+        }
     }
-    // grouped form: workspace row r holds the activations of routed row row_map[r], i.e. x row row_map[r] / top_k
-    const uint32_t out_row = blockIdx.x;
-    const uint32_t row = row_map ? row_map[out_row] / top_k : out_row;
+    return bound;
+}
+// The power of two 2^-e that brings a row whose largest possible |w| is `bound` to about 2^14.
+__device__ __forceinline__ float weight_row_scale(float bound) {
+    int ex = 0;
+    if (bound > 0.f) (void)frexpf(bound, &ex);  // bound = f * 2^ex, f in [0.5, 1)
+    return ldexpf(1.f, -(bound > 0.f ? ex - 14 : 0));  // |e| <= 40: normal
+}
+
+// Lanes that share one weight row in the scan of the block headers: a power of two, at most 16 and no more than the
+// row has blocks (a row of two super-blocks under 16 lanes would leave 14 of them idle).
+template <int TYPE>
+__host__ __device__ __forceinline__ uint32_t weight_scan_lanes(uint32_t k) {
+    const uint32_t blocks = k / ((TYPE == HQ_Q8_0 || TYPE == HQ_Q4_0) ? 32u : 256u);
+    uint32_t lanes = 16u;
+    while (lanes > 1u && lanes / 2u >= blocks) lanes /= 2u;
+    return lanes;
+}
+
+// One group of 256 threads (t = thread within the group): the scales of 256 / lanes weight rows from first_row on,
+// `lanes` = weight_scan_lanes(k) lanes per row over the row's block headers.
+template <int TYPE>
+__device__ __forceinline__ void prep_weight_rows(const uint8_t* __restrict__ w, uint8_t* __restrict__ ws, const Workspace& L,
+                                                 uint32_t n, uint32_t k, uint32_t first_row, uint32_t t, uint32_t lanes) {
+    const uint32_t wr = first_row + t / lanes, sub = t & (lanes - 1u);
+    constexpr uint32_t BLOCK = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q5_K ? Q5K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES
+                               : TYPE == HQ_Q4_0 ? Q4_0_BYTES : Q8_0_BYTES;
+    constexpr uint32_t PER = (TYPE == HQ_Q8_0 || TYPE == HQ_Q4_0) ? 32u : 256u;
+    float bound = weight_row_bound<TYPE>(w + (size_t)(wr < n ? wr : n - 1u) * (k / PER) * BLOCK, k, sub, lanes);
+    if (lanes > 1u) bound = dpp_max<0xB1>(bound);  // as many of the four steps as cover the row's lanes
+    if (lanes > 2u) bound = dpp_max<0x4E>(bound);
+    if (lanes > 4u) bound = dpp_max<0x141>(bound);
+    if (lanes > 8u) bound = dpp_max<0x140>(bound);
+    if (sub == 0 && wr < n) reinterpret_cast<float*>(ws + L.wdown)[wr] = weight_row_scale(bound);
+}
+
+// One group of GROUP threads (256, or 64 = one wave for short rows): row scale and f16 conversion of activation row
+// `row` (rows >= m: the last row is read and nothing is stored).  GROUP 256: every thread of the workgroup calls it (one
+// barrier inside); red: four floats of the group.  GROUP 64: no barrier, red unused.
+template <bool X_BF16, uint32_t GROUP = 256>
+__device__ __forceinline__ void prep_activation_row(const void* __restrict__ x, uint8_t* __restrict__ ws, const Workspace& L,
+                                                    uint32_t m, uint32_t k, uint32_t perm_hd, uint32_t row_in, uint32_t t,
+                                                    float* red) {
+    const bool valid = row_in < m;
+    const uint32_t out_row = valid ? row_in : m - 1u, row = out_row;
     const uint32_t chunks = k / 8;
 
     // perm_hd != 0: x is stored [k / perm_hd][m][perm_hd] (heads outermost), element (row, kk) at
@@ -164,7 +180,7 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
 
     // largest finite magnitude of the row
     float amax = 0.f;
-    for (uint32_t i = tid; i < chunks; i += 256) {
+    for (uint32_t i = t; i < chunks; i += GROUP) {
         float v[8];
         load8(i, v);
 #pragma unroll
@@ -177,11 +193,12 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
     amax = dpp_max<0x4E>(amax);
     amax = dpp_max<0x141>(amax);
     amax = dpp_max<0x140>(amax);
-    amax = fmaxf(amax, __shfl_xor(amax, 16));
-    amax = fmaxf(amax, __shfl_xor(amax, 32));
-    if ((tid & 63u) == 0) red[tid >> 6] = amax;
-    __syncthreads();
-    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    amax = xor32_max(xor16_max(amax));
+    if constexpr (GROUP == 256) {
+        if ((t & 63u) == 0) red[t >> 6] = amax;
+        __syncthreads();
+        amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    }
 
     int ex = 0;
     if (amax > 0.f) (void)frexpf(amax, &ex);  // amax = f * 2^ex, f in [0.5, 1)
@@ -189,9 +206,10 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
     sh = sh < -100 ? -100 : sh > 100 ? 100 : sh;
     if (amax == 0.f) sh = 0;
     const float scale = ldexpf(1.f, sh);
-    if (tid == 0) reinterpret_cast<float*>(ws + L.rs)[out_row] = ldexpf(1.f, -sh);
+    if (!valid) return;
+    if (t == 0) reinterpret_cast<float*>(ws + L.rs)[out_row] = ldexpf(1.f, -sh);
 
-    for (uint32_t i = tid; i < chunks; i += 256) {
+    for (uint32_t i = t; i < chunks; i += GROUP) {
         float v[8];
         load8(i, v);
         uint32_t h[8];
@@ -200,6 +218,25 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
         *reinterpret_cast<uint4*>(ws + L.xh + ((size_t)out_row * k + 8 * i) * 2) =
             make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
     }
+}
+
+// Pre-pass.  Workgroups [0, m): one per activation row, row scale and f16 conversion.  Workgroups
+// from m on: 256 / weight_scan_lanes(k) weight rows each, that many lanes per row over the row's block headers.  Per weight row, a
+// power of two that brings the row's largest possible |w| (Q4_K: |d|*63*15 + |dmin|*63, Q6_K:
+// |d|*128*32, Q8_0: |d|*128) to about 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
+// subnormals; the main kernel multiplies the weights by it before they are rounded (exact) and its
+// epilogue divides it out.
+template <bool X_BF16, int TYPE>
+__global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
+                                                        uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k,
+                                                        uint32_t perm_hd) {
+    __shared__ float red[4];
+    const Workspace L = workspace_layout(m, n, k);
+    if (blockIdx.x >= m) {
+        const uint32_t lanes = weight_scan_lanes<TYPE>(k);
+        prep_weight_rows<TYPE>(w, ws, L, n, k, (blockIdx.x - m) * (256u / lanes), threadIdx.x, lanes);
+    } else
+        prep_activation_row<X_BF16>(x, ws, L, m, k, perm_hd, blockIdx.x, threadIdx.x, red);
 }
 
 struct GemmArgs {
@@ -217,6 +254,9 @@ struct GemmArgs {
     // eight blocks, the last run may be half a one): all of them except in the split form of the small tiles, whose
     // workgroups each write the partial sums of a slice of k
     uint32_t sb0, sb1;
+    // Grouped form: the workspace holds one converted row per TOKEN and tile row r reads token row_map[r] / gather_div
+    // (the routed rows of a token share its activations: top_k of them at gate / up, one at down).
+    uint32_t gather_div;
 };
 
 __device__ __forceinline__ f16x8_t as_frag(uint4 v) { return __builtin_bit_cast(f16x8_t, v); }
@@ -236,13 +276,14 @@ constexpr int BN_WIDE = 128, BN_NARROW = 64;    // weight rows per workgroup
 // the tile, (w * kDma + i) * 8 .. +8; lane L owns row L/8 of them and LDS chunk L%8, which
 // holds global chunk (L%8) ^ ((row/2)%8), and (row/2)%8 = L/16 + 4*(i%2).  Rows past the end of x read
 // the last row instead (their results are never stored).  BMT = token rows of the tile.
-template <int BMT>
+template <int BMT, bool GATHER = false>
 struct ActTileT {
     static constexpr int kDma = (BMT / 8) / WAVES;  // BMT / 8 one-KB fetches fill the activation tile
     static constexpr int kTile = BMT * ROW * 2;     // bytes of one activation buffer; two of them in LDS
     uint8_t* smem;
     const uint8_t* xtile;
     uint32_t a_swz, a_row0, a_rows_left, a_last, row_pitch, wave_u, lds_base;
+    uint32_t g_tok[GATHER ? kDma : 1];  // GATHER: the token row behind this lane's row of fetch i
 
     __device__ __forceinline__ void init(const GemmArgs& a, const Workspace& W, uint32_t m0, uint32_t lane, uint32_t wave) {
         extern __shared__ uint4 smem4[];
@@ -252,7 +293,14 @@ struct ActTileT {
         a_row0 = wave * (8u * kDma) + (lane >> 3);
         a_rows_left = a.m - m0;  // >= 1
         a_last = (a_rows_left - 1u) * row_pitch + a_swz;
-        xtile = a.ws + W.xh + (size_t)m0 * row_pitch;
+        xtile = a.ws + W.xh + (GATHER ? (size_t)0 : (size_t)m0 * row_pitch);
+        if constexpr (GATHER) {
+#pragma unroll
+            for (int i = 0; i < kDma; ++i) {
+                const uint32_t r = a_row0 + 8u * i;
+                g_tok[i] = a.row_map[m0 + (r < a_rows_left ? r : a_rows_left - 1u)] / a.gather_div;
+            }
+        }
         wave_u = __builtin_amdgcn_readfirstlane(wave);  // the same value, known to be uniform
         // LDS byte address of the tile buffers (wave-uniform, goes to M0)
         lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem);
@@ -263,7 +311,11 @@ struct ActTileT {
     // hand by the callers.
     __device__ __forceinline__ void fetch(uint32_t st, uint32_t buf, int i) const {
         const uint32_t r = a_row0 + 8u * i;
-        const uint8_t* src = xtile + (r < a_rows_left ? r * row_pitch + (a_swz ^ ((i & 1u) << 6)) : a_last ^ ((i & 1u) << 6)) + (size_t)st * (BK * 2);
+        const uint8_t* src = xtile + (size_t)st * (BK * 2);
+        if constexpr (GATHER)
+            src += (size_t)g_tok[i] * row_pitch + (a_swz ^ ((i & 1u) << 6));
+        else
+            src += r < a_rows_left ? r * row_pitch + (a_swz ^ ((i & 1u) << 6)) : a_last ^ ((i & 1u) << 6);
         const uint32_t dst = lds_base + buf * kTile + (wave_u * kDma + i) * 1024u;
         asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
         __builtin_amdgcn_sched_barrier(0);  // one address at a time: keeps eight 64-bit pointers out of the registers
@@ -304,8 +356,9 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W
         for (int mt = 0; mt < MT; ++mt) {
             const uint32_t gm = mbase + mt * 32 + l32;
             if (gm >= a.m) continue;
-            const float rsv = rs[gm];
-            float* yp = a.y + (size_t)(a.row_map ? a.row_map[gm] : gm) * a.n + gnb;
+            const uint32_t orow = a.row_map ? a.row_map[gm] : gm;
+            const float rsv = rs[a.gather_div ? orow / a.gather_div : gm];
+            float* yp = a.y + (size_t)orow * a.n + gnb;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const float o0 = acc[mt][nt][4 * g] * (rsv * wup[4 * g]), o1 = acc[mt][nt][4 * g + 1] * (rsv * wup[4 * g + 1]);
@@ -329,7 +382,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W
 // TYPE = HQ_Q5_K: the same tile over 176-byte super-blocks; a lane also keeps the sixteen qh bytes that go with
 // its nibble bytes (they serve all four chunks of the super-block, bit 2c + hi for sub-block 2c + hi) and ORs the
 // fifth bit into the masked nibbles, three more VALU instructions per four weights.
-template <int MT, int NT, int WN, int TYPE = HQ_Q4_K>
+template <int MT, int NT, int WN, int TYPE = HQ_Q4_K, bool GATHER = false>
 __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     constexpr int BMT = 32 * MT * (WAVES / WN);  // token rows of the workgroup tile: 256, or 64 for the small tiles
     constexpr int DMA_PER_WAVE = ActTileT<BMT>::kDma;
@@ -343,7 +396,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 
     const uint32_t row_bytes = (a.k / 256) * BYTES;
     const uint32_t sb0 = a.sb0, sb1 = a.sb1;  // sb0 < sb1
-    ActTileT<BMT> at;
+    ActTileT<BMT, GATHER> at;
     at.init(a, W, m0, lane, wave);
 
     // ---- weights: this lane's two rows (one per 32-row tile of the wave), bytes 16*lg.. of each chunk ----
@@ -565,7 +618,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 // high ones): the same frame with four words per block instead of eight; k-steps 0 and 1 take the low nibbles of
 // words 0..1 and 2..3, k-steps 2 and 3 the high nibbles of the same words.  A stage advances a lane by 36 bytes,
 // so it keeps its alignment case here too.  w = d * (q - 8).
-template <int MT, int WN, int TYPE = HQ_Q8_0>
+template <int MT, int WN, int TYPE = HQ_Q8_0, bool GATHER = false>
 __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     constexpr int BMT = 32 * MT * (WAVES / WN);  // token rows of the workgroup tile: 256, or 128 for the small tiles
     constexpr int DMA_PER_WAVE = ActTileT<BMT>::kDma;
@@ -577,7 +630,7 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
     // stages [st_first, nstages) of every row, an even number of them (k % 128 == 0; slices of k are whole 256s)
     const uint32_t st_first = 4u * a.sb0, nstages = a.sb1 * 4u < a.k / BK ? a.sb1 * 4u : a.k / BK;
-    ActTileT<BMT> at;
+    ActTileT<BMT, GATHER> at;
     at.init(a, W, m0, lane, wave);
 
     uint32_t gn = n0 + wn * 32 + l32;
@@ -696,7 +749,7 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
 // ql bytes, the half's 32 qh bytes, eight scale bytes and d once per half, a half ahead.
 // w = d*sc*(q - 32) in fp32 (d*sc exact), one rounding to f16.  The blocks are 2-byte aligned; the
 // hardware takes the unaligned 16-byte loads.
-template <int MT, int WN>
+template <int MT, int WN, bool GATHER = false>
 __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
     constexpr int BMT = 32 * MT * (WAVES / WN);  // token rows of the workgroup tile: 256, or 128 for the small tiles
     constexpr int DMA_PER_WAVE = ActTileT<BMT>::kDma;
@@ -705,7 +758,7 @@ __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31u, lg = lane >> 5;
     const uint32_t nsb = a.sb1, nstages = 4u * a.sb1;  // super-blocks [sb0, sb1) of every row
-    ActTileT<BMT> at;
+    ActTileT<BMT, GATHER> at;
     at.init(a, W, m0, lane, wave);
 
     uint32_t gn = n0 + wn * 32 + l32;
@@ -951,18 +1004,58 @@ constexpr uint32_t BUCKET_MAX_EXPERTS = 1024;  // one expert per thread of the s
 // One workgroup: counting sort of the routed rows by expert.  Rows whose id is not an expert get NaN
 // outputs here and take no part in the product.  The order of the rows inside an expert's run depends
 // on the order in which the atomics land; every output row is computed on its own, so the results do not.
-__global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __restrict__ ids, uint32_t pairs, uint32_t n_experts,
-                                                          uint32_t* __restrict__ row_map, uint4* __restrict__ tiles,
-                                                          uint32_t* __restrict__ n_tiles, float* __restrict__ y, uint32_t n,
-                                                          uint32_t bm) {
+struct BucketArgs {
+    const uint32_t* ids;
+    uint32_t pairs, n_experts;
+    uint32_t* row_map;
+    uint4* tiles;
+    uint32_t* n_tiles;
+    float* y;
+    uint32_t n, bm;
+};
+__device__ __forceinline__ void moe_bucket_sort(const BucketArgs& b) {
+    const uint32_t* __restrict__ ids = b.ids;
+    uint32_t* __restrict__ row_map = b.row_map;
+    uint4* __restrict__ tiles = b.tiles;
+    uint32_t* __restrict__ n_tiles = b.n_tiles;
+    float* __restrict__ y = b.y;
+    const uint32_t pairs = b.pairs, n_experts = b.n_experts, n = b.n, bm = b.bm;
     __shared__ uint32_t cnt[BUCKET_MAX_EXPERTS], cur[BUCKET_MAX_EXPERTS];
     const uint32_t tid = threadIdx.x;
     for (uint32_t e = tid; e < n_experts; e += 1024) cnt[e] = 0;
     __syncthreads();
-    for (uint32_t p = tid; p < pairs; p += 1024) {
-        const uint32_t e = ids[p];
+    // The ids are walked in batches of 16 per thread, four 16-byte loads in flight at once (one trip to memory per
+    // 16384 ids instead of sixteen); ids that are not 16-byte aligned or not a multiple of four take single loads.
+    const bool vec = pairs % 4u == 0 && (reinterpret_cast<uintptr_t>(ids) & 15u) == 0;
+    auto for_each_id = [&](auto&& f) {  // f(position p, expert id)
+        if (vec) {
+            const uint4* ids4 = reinterpret_cast<const uint4*>(ids);
+            const uint32_t quads = pairs / 4u;
+            for (uint32_t q0 = 0; q0 < quads; q0 += 4096u) {
+                uint4 v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t q = q0 + tid + 1024u * j;
+                    v[j] = ids4[q < quads ? q : quads - 1u];
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t q = q0 + tid + 1024u * j;
+                    if (q < quads) {
+                        f(4u * q, v[j].x);
+                        f(4u * q + 1u, v[j].y);
+                        f(4u * q + 2u, v[j].z);
+                        f(4u * q + 3u, v[j].w);
+                    }
+                }
+            }
+        } else {
+            for (uint32_t p = tid; p < pairs; p += 1024) f(p, ids[p]);
+        }
+    };
+    for_each_id([&](uint32_t, uint32_t e) {
         if (e < n_experts) atomicAdd(&cnt[e], 1u);
-    }
+    });
     __syncthreads();
     // Exclusive prefix sums over the experts of (rows, tiles), one expert per thread (n_experts <= 1024 = the
     // workgroup): inside a wave by shuffles, across the sixteen waves through LDS.  Expert e then writes its own tiles.
@@ -988,19 +1081,48 @@ __global__ __launch_bounds__(1024) void moe_bucket_kernel(const uint32_t* __rest
     }
     if (tid == 0) *n_tiles = total_tiles;
     __syncthreads();
-    for (uint32_t p = tid; p < pairs; p += 1024) {
-        const uint32_t e = ids[p];
+    for_each_id([&](uint32_t p, uint32_t e) {
         if (e < n_experts) {
             row_map[atomicAdd(&cur[e], 1u)] = p;
         } else {
             for (uint32_t c = 0; c < n; ++c) y[(size_t)p * n + c] = __uint_as_float(0x7fc00000u);
         }
-    }
+    });
     // rows of the workspace past the sorted ones (invalid ids leave a gap at the end) point at row 0
     for (uint32_t r = total_rows + tid; r < pairs; r += 1024) row_map[r] = 0;
 }
 
-template <int TYPE, bool SMALL>
+// The grouped form's pre-pass as ONE launch of 1024-thread workgroups: workgroup 0 sorts the routed rows by expert,
+// the next ones convert the activation rows (one per token; four rows per workgroup, or sixteen, a wave each, when a
+// row is at most 1024 values), the rest scan the scales of 1024 / weight_scan_lanes(k) weight rows each.  The sort is
+// a single workgroup's work of about 13 us; beside the other two it costs nothing.
+__host__ __device__ __forceinline__ uint32_t grouped_prep_rows_per_wg(uint32_t k) { return k <= 1024u ? 16u : 4u; }
+
+template <bool X_BF16, int TYPE>
+__global__ __launch_bounds__(1024) void grouped_prep_kernel(BucketArgs b, const void* __restrict__ x, const uint8_t* __restrict__ w,
+                                                            uint8_t* __restrict__ ws, uint32_t m, uint32_t n_rows, uint32_t k) {
+    if (blockIdx.x == 0) {
+        moe_bucket_sort(b);
+        return;
+    }
+    __shared__ float red[16];
+    const Workspace L = workspace_layout(m, n_rows, k);
+    const uint32_t per_wg = grouped_prep_rows_per_wg(k), row_wgs = (m + per_wg - 1u) / per_wg, wg = blockIdx.x - 1u;
+    if (wg < row_wgs) {
+        if (per_wg == 16u)
+            prep_activation_row<X_BF16, 64>(x, ws, L, m, k, 0u, wg * 16u + (threadIdx.x >> 6), threadIdx.x & 63u, red);
+        else
+            prep_activation_row<X_BF16, 256>(x, ws, L, m, k, 0u, wg * 4u + (threadIdx.x >> 8), threadIdx.x & 255u,
+                                             red + 4u * (threadIdx.x >> 8));
+    } else {
+        const uint32_t lanes = weight_scan_lanes<TYPE>(k);
+        prep_weight_rows<TYPE>(w, ws, L, n_rows, k, ((wg - row_wgs) * 4u + (threadIdx.x >> 8)) * (256u / lanes),
+                               threadIdx.x & 255u, lanes);
+    }
+}
+
+// A tile is 32 * MT routed rows (MT 8: 256 rows; 4: 128; 2: 64, Q4_K / Q5_K only) x 128 weight rows, a wave all its rows x 32.
+template <int TYPE, int MT>
 __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a, const uint4* __restrict__ tiles,
                                                                       const uint32_t* __restrict__ n_tiles, uint32_t tiles_n,
                                                                       uint64_t expert_stride) {
@@ -1010,19 +1132,12 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
     a.w += (size_t)tt.x * expert_stride;
     a.wd_off = tt.x * a.n;
     a.m = tt.z;  // rows past the expert's run repeat its last row and are not stored
-    if constexpr (SMALL) {  // 128 routed rows x 128 weight rows, a wave 128 x 32
-        if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
-            q4k_gemm_tile<4, 1, 4, TYPE>(a, tt.y, n0);
-        else if constexpr (TYPE == HQ_Q6_K)
-            q6k_gemm_tile<4, 4>(a, tt.y, n0);
-        else
-            q80_gemm_tile<4, 4, TYPE>(a, tt.y, n0);
-    } else if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
-        q4k_gemm_tile<8, 1, 4, TYPE>(a, tt.y, n0);
+    if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
+        q4k_gemm_tile<MT, 1, 4, TYPE, true>(a, tt.y, n0);
     else if constexpr (TYPE == HQ_Q6_K)
-        q6k_gemm_tile<8, 4>(a, tt.y, n0);
+        q6k_gemm_tile<MT, 4, true>(a, tt.y, n0);
     else
-        q80_gemm_tile<8, 4, TYPE>(a, tt.y, n0);
+        q80_gemm_tile<MT, 4, TYPE, true>(a, tt.y, n0);
 }
 
 }  // namespace
@@ -1062,12 +1177,13 @@ size_t gemm_f16_grouped_workspace_bytes(uint32_t pairs, uint32_t n_experts, uint
 
 template <int TYPE>
 static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, uint8_t* ws, uint32_t m,
-                       uint32_t n, uint32_t k, const uint32_t* row_map = nullptr, uint32_t top_k = 1, uint32_t perm_hd = 0) {
-    const dim3 prep_grid(m + (n + 15u) / 16u);
+                       uint32_t n, uint32_t k, uint32_t perm_hd = 0) {
+    const uint32_t rows_per_wg = 256u / weight_scan_lanes<TYPE>(k);
+    const dim3 prep_grid(m + (n + rows_per_wg - 1u) / rows_per_wg);
     if (xdt == HQ_BF16)
-        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, row_map, top_k, perm_hd);
+        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd);
     else
-        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, row_map, top_k, perm_hd);
+        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd);
     return check_launch("tile gemm pre-pass launch");
 }
 
@@ -1080,19 +1196,31 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     uint32_t* row_map = reinterpret_cast<uint32_t*>(ws + G.row_map);
     uint4* tiles = reinterpret_cast<uint4*>(ws + G.tiles);
     uint32_t* n_tiles = reinterpret_cast<uint32_t*>(ws + G.count);
-    // Experts with few rows each (Qwen3.6-35B-A3B: 2048 tokens x top-8 over 256 experts = 64 rows per expert) take tiles
-    // of 128 routed rows; the 256-row tiles would run a quarter full.
-    const bool small = (uint64_t)pairs < (uint64_t)n_experts * 160u;
-    const uint32_t bm = small ? BM_MID : BM, bn = BN_WIDE;
-    hipLaunchKernelGGL(moe_bucket_kernel, dim3(1), dim3(1024), 0, s, ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm);
-    if (int rc = check_launch("expert bucket kernel launch")) return rc;
-    if (int rc = launch_prep<TYPE>(s, x, xdt, wb, ws, pairs, n_experts * n, k, row_map, top_k)) return rc;
-    const int lds = 2 * (small ? ActTileT<BM_MID>::kTile : ActTile::kTile);
-    void (*kern)(GemmArgs, const uint4*, const uint32_t*, uint32_t, uint64_t) =
-        small ? grouped_gemm_kernel<TYPE, true> : grouped_gemm_kernel<TYPE, false>;
+    // Experts with few rows each take smaller tiles (Qwen3.6-35B-A3B: 2048 tokens x top-8 over 256 experts = 64 rows per
+    // expert on average, tiles of 128 routed rows: the 256-row tiles would run a quarter full, and half of the experts
+    // would need two 64-row tiles); at 40 rows per expert or fewer the Q4_K / Q5_K tiles of 64 rows.
+    constexpr bool HAS_64 = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K;
+    const int mt = HAS_64 && (uint64_t)pairs <= (uint64_t)n_experts * 40u ? 2 : (uint64_t)pairs < (uint64_t)n_experts * 160u ? 4 : 8;
+    const uint32_t bm = 32u * (uint32_t)mt, bn = BN_WIDE;
+    // sort by expert + one converted activation row per token (the tiles gather the rows of their routed rows from
+    // them) + the weight rows' scales, in one launch
+    const BucketArgs b{ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm};
+    const uint32_t n_rows = n_experts * n;
+    const uint32_t act_per_wg = grouped_prep_rows_per_wg(k), w_per_wg = 1024u / weight_scan_lanes<TYPE>(k);
+    const dim3 prep_grid(1u + (n_tokens + act_per_wg - 1u) / act_per_wg + (n_rows + w_per_wg - 1u) / w_per_wg);
+    if (xdt == HQ_BF16)
+        hipLaunchKernelGGL((grouped_prep_kernel<true, TYPE>), prep_grid, dim3(1024), 0, s, b, x, wb, ws, n_tokens, n_rows, k);
+    else
+        hipLaunchKernelGGL((grouped_prep_kernel<false, TYPE>), prep_grid, dim3(1024), 0, s, b, x, wb, ws, n_tokens, n_rows, k);
+    if (int rc = check_launch("grouped gemm pre-pass launch")) return rc;
+    const int lds = 2 * (mt == 2 ? ActTileT<BM_SMALL>::kTile : mt == 4 ? ActTileT<BM_MID>::kTile : ActTile::kTile);
+    void (*kern)(GemmArgs, const uint4*, const uint32_t*, uint32_t, uint64_t) = grouped_gemm_kernel<TYPE, 8>;
+    if (mt == 4) kern = grouped_gemm_kernel<TYPE, 4>;
+    if constexpr (HAS_64)
+        if (mt == 2) kern = grouped_gemm_kernel<TYPE, 2>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;
-    GemmArgs a{ws, wb, y, pairs, n, k, pairs, n_experts * n, 0u, row_map, 0u, (k + 255u) / 256u};
+    GemmArgs a{ws, wb, y, pairs, n, k, n_tokens, n_experts * n, 0u, row_map, 0u, (k + 255u) / 256u, top_k};
     const uint32_t tiles_n = (n + bn - 1) / bn;
     const uint32_t max_tiles = pairs / bm + n_experts;
     hipLaunchKernelGGL(kern, dim3(max_tiles * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
@@ -1145,7 +1273,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         return check_launch("split sum kernel launch");
     };
     if (t == HQ_Q6_K) {
-        if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)) return rc;
+        if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k, perm_hd)) return rc;
         if (gemm_f16_small_tiles(t, m)) return launch_mid_small(mid_gemm_small_kernel<HQ_Q6_K, 4>, mid_gemm_small_kernel<HQ_Q6_K, 8>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(q6k_gemm_kernel), (size_t)lds, "hipFuncSetAttribute(q6_k gemm LDS)"))
             return rc;
@@ -1154,8 +1282,8 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     }
     if (t == HQ_Q8_0 || t == HQ_Q4_0) {
         void (*kern)(GemmArgs) = t == HQ_Q4_0 ? q80_gemm_kernel<HQ_Q4_0> : q80_gemm_kernel<HQ_Q8_0>;
-        if (int rc = t == HQ_Q4_0 ? launch_prep<HQ_Q4_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
-                                  : launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
+        if (int rc = t == HQ_Q4_0 ? launch_prep<HQ_Q4_0>(s, x, xdt, wb, ws, m, n, k, perm_hd)
+                                  : launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, perm_hd))
             return rc;
         if (gemm_f16_small_tiles(t, m))
             return t == HQ_Q4_0 ? launch_mid_small(mid_gemm_small_kernel<HQ_Q4_0, 4>, mid_gemm_small_kernel<HQ_Q4_0, 8>)
@@ -1165,8 +1293,8 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         hipLaunchKernelGGL(kern, dim3(tile_grid(tiles_m, cols_wide)), dim3(64 * WAVES), lds, s, a);
         return check_launch("q8_0 gemm kernel launch");
     }
-    if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd)
-                              : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, nullptr, 1, perm_hd))
+    if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, perm_hd)
+                              : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, perm_hd))
         return rc;
     if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: one token tile of 64, 128 or 256 rows, tiles of 128 weight rows
         const int mts = m <= (uint32_t)BM_SMALL ? 2 : m <= (uint32_t)BM_MID ? 4 : 8;

@@ -289,6 +289,23 @@ def test_mul_mat_id_grouped_matches_oracle(oracle, dev, t, xdt, E, n, k, T, K):
     assert_matmul_close_f16_tile(y.cpu().numpy(), ref, f"grouped mul_mat_id t={t} {xdt}")
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K])
+def test_mul_mat_id_grouped_sparse_experts_skewed(oracle, dev, t):
+    """40 routed rows per expert on average (the smallest tiles: 64 rows for Q4_K / Q5_K) with most rows on one expert,
+    which then takes several of those tiles, and experts without rows."""
+    E, n, k, T, K = 16, 160, 512, 160, 4
+    stack, ids, xv, xd, p = _grouped_setup(oracle, dev, t, E, n, k, T, K, "bf16", seed=9, skew=True)
+    assert np.bincount(ids, minlength=E).max() > 300
+    need = ops.quantized_matmul_id_workspace_bytes(p)
+    assert need > 0
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    ref = oracle.qmatmul_id_f64(xv, stack, ids, T, K, n, k, E, p.expert_stride, t)
+    y = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(xd, torch.from_numpy(stack).to(dev), torch.from_numpy(ids.view(np.int32)).to(dev), y, p,
+                                 scratch=scratch)
+    assert_matmul_close_f16_tile(y.cpu().numpy(), ref, f"grouped, sparse + skewed, t={t}")
+
+
 def test_mul_mat_id_grouped_routing_properties(oracle, dev):
     """Skewed routing with unused experts, an id that is no expert (NaN rows, the others untouched), agreement with
     the per-row GEMV form, a scratch that is too small, and a strided stack (which keeps the GEMV form)."""
