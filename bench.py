@@ -14,7 +14,8 @@ Prints ONE JSON line: metric = effective GB/s of packed weight bytes, with a
 `roofline` object for the dominant kernel (the Q6_K head GEMV) from HIP-event
 timings taken inside the timed region, a `kernels` table for the others, a
 `workloads` object with the other BASELINE configurations (MoE decode at 1 and 8
-tokens, the Q4_K and Q8_0 prefill GEMM, the TQ attention), each with its own
+tokens, its prefill-sized grouped mul_mat_id, the Q4_K and Q8_0 prefill GEMM, the
+TQ attention), each with its own
 roofline, and a `cpu_baseline` object (the scalar CPU port of hf2q's
 quantize -> dequantize -> scalar matmul, timed on this host).
 `--workload <name>` runs one of them alone and prints its own line.
@@ -55,7 +56,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "decode_gemv", "moe_decode", "prefill_gemm", "tq_attention"],
+                    choices=["all", "decode_gemv", "moe_decode", "moe_prefill", "prefill_gemm", "tq_attention"],
                     help="all (default) = the BASELINE config 2 headline plus configs 3, 4 and 5 under `workloads` in the "
                          "same JSON line; a single name runs that workload alone and prints its own line")
     ap.add_argument("--tokens", type=int, default=1, help="moe_decode: tokens per step (1 or 8)")
@@ -63,7 +64,7 @@ def parse():
     ap.add_argument("--weight-sets", type=int, default=6, help="distinct FFN weight sets rotated per step")
     ap.add_argument("--moe-layers", type=int, default=20, help="moe_decode: distinct MoE layers rotated per step")
     ap.add_argument("--no-graph", action="store_true",
-                    help="moe_decode / tq_attention: launch every kernel from the host instead of replaying a HIP "
+                    help="moe_decode / moe_prefill / tq_attention: launch every kernel from the host instead of replaying a HIP "
                          "graph of the step (the steps are 4-12 launches of a few microseconds each)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -306,6 +307,19 @@ def bench_prefill_gemm(a, wtype=None):
     us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
     flops = 2.0 * M * N * K
     tf = flops / us / 1e6
+    us_prepared = None
+    if need:  # the same product with the weight-row scales kept from load time (hq_qmatmul_ggml_ws_prepared; same bits)
+        scales = ops.weight_row_scales_ggml(w, N, K, t)
+        for _ in range(max(a.warmup, 1)):
+            ops.quantized_matmul_ggml(x, w, y, p, workspace=ws, w_row_scales=scales)
+        torch.cuda.synchronize()
+        evp = _events(a.steps)
+        for i in range(a.steps):
+            evp[i][0].record()
+            ops.quantized_matmul_ggml(x, w, y, p, workspace=ws, w_row_scales=scales)
+            evp[i][1].record()
+        torch.cuda.synchronize()
+        us_prepared = round(sum(e0.elapsed_time(e1) for e0, e1 in evp) * 1e3 / a.steps, 2)
     # For scale only (not part of the path, not in `value`): the vendor library's plain f16 GEMM of the same shape,
     # no dequantisation, through torch.matmul; the same event timing over the same number of launches.
     vendor = None
@@ -333,12 +347,79 @@ def bench_prefill_gemm(a, wtype=None):
         "config": {"workload": f"prefill_gemm: 2048 tokens x K=4096 x N=12288, {wtype.upper()} weights, bf16 "
                                f"activations, fp32 accumulate (BASELINE config 4)", "flop_per_step": flops,
                    "weight_bytes": w.numel(), "workspace_bytes": need,
-                   "launches_per_step": 2 if need else 1, "vendor_dense_gemm_same_shape": vendor},
+                   "launches_per_step": 2 if need else 1, "us_per_step_with_weight_row_scales_kept_from_load_time": us_prepared,
+                   "vendor_dense_gemm_same_shape": vendor},
         "roofline": {"bound": "mfma", "kernel": (f"activation pre-pass + f16 MFMA gemm {wtype}" if need else
                                                  f"bf16 MFMA gemm {wtype}"), "achieved": round(tf, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": PMC_TRAFFIC_BYTES["prefill_gemm_q4_k_2048x12288x4096"] if wtype == "q4_k" else None,
                      "us_per_launch": round(us, 2), "flop_per_launch": flops}})
+
+
+def bench_moe_prefill(a):
+    """The prefill side of BASELINE config 3's layer: mul_mat_id over 2048 tokens x top-8 of 256 experts, Q4_K, bf16
+    activations, f32 out -- the gate / up shape (expert 512 x 2048, one activation row per token) and the down shape
+    (expert 2048 x 512, one activation row per routed row).  A step is one gate / up call: the expert sort, the
+    activation conversion and the weight-row scales in one launch, then the grouped tile GEMM."""
+    import torch
+
+    from hf2q_amd import ops
+    from hf2q_amd.ops import HQ_Q4_K, GgmlQuantizedMatmulIdParams
+
+    dev = torch.device("cuda:0")
+    E, K, T, H, I = 256, 8, 2048, 2048, 512
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    n_stacks = 3  # 151 MB each, rotated past the 256 MB Infinity Cache
+
+    def shape(n, k, rows, top_k):
+        stacks = [ops.quantize_ggml(torch.randn(E * n * k, generator=gen, device=dev).mul_(0.02), k, HQ_Q4_K)
+                  for _ in range(n_stacks)]
+        p = GgmlQuantizedMatmulIdParams(rows, top_k, n, k, E, n * ops.ggml_row_bytes(HQ_Q4_K, k), HQ_Q4_K)
+        x = torch.randn(rows, k, generator=gen, device=dev).to(torch.bfloat16)
+        ids = torch.randint(0, E, (T * K,), generator=gen, device=dev, dtype=torch.int32)
+        y = torch.empty(T * K, n, device=dev)
+        need = ops.quantized_matmul_id_workspace_bytes(p)
+        assert need > 0, "this shape must take the grouped route"
+        scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+
+        scales = [ops.weight_row_scales_ggml(w, E * n, k, HQ_Q4_K) for w in stacks]  # once per stack, as at load time
+
+        def step(i):
+            ops.quantized_matmul_id_ggml(x, stacks[i % n_stacks], ids, y, p, scratch=scratch)
+
+        def step_prepared(i):
+            ops.quantized_matmul_id_ggml(x, stacks[i % n_stacks], ids, y, p, scratch=scratch, w_row_scales=scales[i % n_stacks])
+
+        for i in range(max(a.warmup, 1)):
+            step(i)
+            step_prepared(i)
+        torch.cuda.synchronize()
+        _, us_prepared = _timed_steps(a, step_prepared, n_stacks)
+        elapsed, us = _timed_steps(a, step, n_stacks)
+        return elapsed, us, us_prepared, need
+
+    elapsed, us, us_prep, need = shape(I, H, T, K)
+    _, us_down, us_down_prep, _ = shape(H, I, T * K, 1)
+    flops = 2.0 * T * K * I * H
+    tf = flops / us / 1e6
+    return _finish(a, {
+        "metric": "MoE prefill mul_mat_id eff. TFLOP/s", "value": round(flops * a.steps / elapsed / 1e12, 1), "unit": "TFLOP/s",
+        "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f16",
+        "config": {"workload": "moe_prefill: mul_mat_id, 2048 tokens x top-8 over 256 experts, expert 512 x 2048 Q4_K (gate / up "
+                               "shape of BASELINE config 3's layer), bf16 activations, fp32 accumulate; one step = 2 launches "
+                               "(expert sort + activation conversion + weight-row scales; grouped tile GEMM), "
+                               + ("launched from the host" if a.no_graph else "replayed as a HIP graph"),
+                   "flop_per_step": flops, "workspace_bytes": need, "stacks_rotated": n_stacks,
+                   "with_weight_row_scales_kept_from_load_time": {
+                       "what": "hq_qmatmul_id_ggml_prepared: the stack's row scales (a function of the weights alone) computed "
+                               "once, the call's pre-pass skips their scan; same bits", "us_per_step": round(us_prep, 2),
+                       "TFLOP/s": round(flops / us_prep / 1e6, 1)},
+                   "down_shape_2048x512": {"us_per_step": round(us_down, 2), "TFLOP/s": round(flops / us_down / 1e6, 1),
+                                           "us_per_step_with_kept_scales": round(us_down_prep, 2)}},
+        "roofline": {"bound": "mfma", "kernel": "grouped pre-pass + grouped f16 MFMA gemm q4_k", "achieved": round(tf, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": None, "us_per_launch": round(us, 2), "flop_per_launch": flops}})
 
 
 def bench_tq_attention(a):
@@ -425,7 +506,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if a.workload not in ("all", "decode_gemv"):
-        return {"moe_decode": bench_moe_decode, "prefill_gemm": bench_prefill_gemm,
+        return {"moe_decode": bench_moe_decode, "moe_prefill": bench_moe_prefill, "prefill_gemm": bench_prefill_gemm,
                 "tq_attention": bench_tq_attention}[a.workload](a)
     out = bench_decode_gemv(a)
     if a.workload == "all":
@@ -440,6 +521,7 @@ def main():
         a = copy.copy(a)
         a.steps = max(a.steps, 256)
         for name, fn in (("moe_decode_t1", lambda: bench_moe_decode(a, 1)), ("moe_decode_t8", lambda: bench_moe_decode(a, 8)),
+                         ("moe_prefill_2048x8", lambda: bench_moe_prefill(a)),
                          ("prefill_gemm_q4_k", lambda: bench_prefill_gemm(a, "q4_k")),
                          ("prefill_gemm_q8_0", lambda: bench_prefill_gemm(a, "q8_0")),
                          ("tq_attention_32k", lambda: bench_tq_attention(a))):

@@ -182,8 +182,8 @@ bool f16_tile_route(uint32_t m, uint32_t k, hq_ggml_type t) {
 
 // All routes of the dense product; `workspace` is only read on the f16 tile route.
 int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
-                   uint32_t n, uint32_t k, hq_ggml_type t, void* workspace) {
-    if (f16_tile_route(m, k, t)) return launch_gemm_f16_tile(stream, x, xdt, w_blocks, y, m, n, k, t, workspace);
+                   uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, const float* w_scales = nullptr) {
+    if (f16_tile_route(m, k, t)) return launch_gemm_f16_tile(stream, x, xdt, w_blocks, y, m, n, k, t, workspace, 0, w_scales);
     if (m > chunked_rows_limit(k, t) && gemm_supported(t, k)) return launch_gemm(stream, x, xdt, w_blocks, y, m, n, k, t);
     // kGemvMaxRows activation rows per launch: the small-batch kernel where it exists for the chunk, else one GEMV
     // per row (also the route of shapes the tile kernels do not cover).
@@ -226,19 +226,46 @@ size_t hq_qmatmul_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ac
     return f16_tile_route(m, k, t) ? gemm_f16_tile_workspace_bytes(m, n, k, t) : 0;
 }
 
-int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
-                       uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes) {
-    if (int rc = check_matmul_common("hq_qmatmul_ggml_ws", x, xdt, w_blocks, y, n, k, t)) return rc;
+namespace {
+int qmatmul_ws(const char* fn, void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, const float* w_scales,
+               float* y, uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes) {
+    if (int rc = check_matmul_common(fn, x, xdt, w_blocks, y, n, k, t)) return rc;
     if (m == 0) return HQ_OK;
     const size_t need = hq_qmatmul_ggml_workspace_bytes(m, n, k, xdt, t);
     if (need) {
         if (!workspace || workspace_bytes < need)
-            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_ggml_ws: workspace of %zu bytes, %zu needed",
+            return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes, %zu needed", fn,
                         workspace ? workspace_bytes : (size_t)0, need);
         if (reinterpret_cast<uintptr_t>(workspace) % 256)
-            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_ggml_ws: workspace must be 256-byte aligned");
+            return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace must be 256-byte aligned", fn);
     }
-    return qmatmul_routes((hipStream_t)stream, x, xdt, w_blocks, y, m, n, k, t, workspace);
+    return qmatmul_routes((hipStream_t)stream, x, xdt, w_blocks, y, m, n, k, t, workspace, w_scales);
+}
+}  // namespace
+
+int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
+                       uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes) {
+    return qmatmul_ws("hq_qmatmul_ggml_ws", stream, x, xdt, w_blocks, nullptr, y, m, n, k, t, workspace, workspace_bytes);
+}
+
+int hq_qmatmul_ggml_ws_prepared(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, const float* w_row_scales,
+                                float* y, uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, void* workspace,
+                                size_t workspace_bytes) {
+    if (!w_row_scales || !is_aligned(w_row_scales, 4))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_ggml_ws_prepared: w_row_scales is null or not 4-byte aligned");
+    return qmatmul_ws("hq_qmatmul_ggml_ws_prepared", stream, x, xdt, w_blocks, w_row_scales, y, m, n, k, t, workspace,
+                      workspace_bytes);
+}
+
+int hq_weight_row_scales_ggml(void* stream, const void* w_blocks, float* scales, uint64_t n_rows, uint32_t k, hq_ggml_type t) {
+    const char* fn = "hq_weight_row_scales_ggml";
+    if (hq_block_elems(t) == 0) return fail(HQ_ERR_UNSUPPORTED, "%s: ggml type %d", fn, (int)t);
+    if (k == 0 || k % hq_block_elems(t)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: k = %u is not a multiple of the block", fn, k);
+    if (n_rows == 0) return HQ_OK;
+    if (n_rows > 0x7fffffffull) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: %llu rows", fn, (unsigned long long)n_rows);
+    if (!w_blocks || !scales || !is_aligned(scales, 4)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null or misaligned buffer", fn);
+    if (int rc = check_weight_alignment(w_blocks, t)) return rc;
+    return launch_weight_row_scales((hipStream_t)stream, w_blocks, scales, (uint32_t)n_rows, k, t);
 }
 
 int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y,
@@ -304,20 +331,44 @@ size_t hq_qmatmul_id_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uin
                ? gemm_f16_grouped_workspace_bytes(n_tokens * top_k, n_experts, n, k) : 0;
 }
 
+namespace {
+int qmatmul_id(const char* fn, void* stream, const void* x, hq_act_dtype xdt, const void* w_stack, const float* w_scales,
+               const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes, uint32_t n_tokens, uint32_t top_k, uint32_t n,
+               uint32_t k, uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
+}  // namespace
+
 int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_stack,
                        const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes,
                        uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
                        uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t) {
-    if (int rc = check_matmul_common("hq_qmatmul_id_ggml", x, xdt, w_stack, y, n, k, t)) return rc;
-    if (!ids) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: null ids");
+    return qmatmul_id("hq_qmatmul_id_ggml", stream, x, xdt, w_stack, nullptr, ids, y, scratch, scratch_bytes, n_tokens, top_k, n, k,
+                      n_experts, expert_stride, t);
+}
+
+int hq_qmatmul_id_ggml_prepared(void* stream, const void* x, hq_act_dtype xdt, const void* w_stack, const float* w_row_scales,
+                                const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes, uint32_t n_tokens,
+                                uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts, uint64_t expert_stride,
+                                hq_ggml_type t) {
+    if (!w_row_scales || !is_aligned(w_row_scales, 4))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml_prepared: w_row_scales is null or not 4-byte aligned");
+    return qmatmul_id("hq_qmatmul_id_ggml_prepared", stream, x, xdt, w_stack, w_row_scales, ids, y, scratch, scratch_bytes, n_tokens,
+                      top_k, n, k, n_experts, expert_stride, t);
+}
+
+namespace {
+int qmatmul_id(const char* fn, void* stream, const void* x, hq_act_dtype xdt, const void* w_stack, const float* w_scales,
+               const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes, uint32_t n_tokens, uint32_t top_k, uint32_t n,
+               uint32_t k, uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t) {
+    if (int rc = check_matmul_common(fn, x, xdt, w_stack, y, n, k, t)) return rc;
+    if (!ids) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null ids", fn);
     if (n_experts == 0 || top_k == 0)
-        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: n_experts %u, top_k %u", n_experts, top_k);
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: n_experts %u, top_k %u", fn, n_experts, top_k);
     const uint64_t expert_bytes = (uint64_t)n * (k / hq_block_elems(t)) * hq_block_bytes(t);
     if (expert_stride < expert_bytes)
-        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: expert_stride %llu < one expert's %llu bytes",
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: expert_stride %llu < one expert's %llu bytes", fn,
                     (unsigned long long)expert_stride, (unsigned long long)expert_bytes);
     if (expert_stride % ((t == HQ_Q4_K || t == HQ_Q5_K) ? 16 : 2))
-        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: expert_stride %llu breaks block alignment",
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: expert_stride %llu breaks block alignment", fn,
                     (unsigned long long)expert_stride);
     const uint64_t pairs = (uint64_t)n_tokens * top_k;
     if (pairs == 0) return HQ_OK;
@@ -325,11 +376,11 @@ int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void
     if (scratch && grouped_route(n_tokens, top_k, n, k, n_experts, expert_stride, t)) {
         const size_t need = gemm_f16_grouped_workspace_bytes((uint32_t)pairs, n_experts, n, k);
         if (scratch_bytes < need)
-            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: scratch of %zu bytes, %zu needed", scratch_bytes, need);
+            return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch of %zu bytes, %zu needed", fn, scratch_bytes, need);
         if (reinterpret_cast<uintptr_t>(scratch) % 256)
-            return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: scratch must be 256-byte aligned");
+            return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch must be 256-byte aligned", fn);
         return launch_gemm_f16_grouped((hipStream_t)stream, x, xdt, w_stack, ids, y, scratch, n_tokens, top_k, n, k, n_experts,
-                                       expert_stride, t);
+                                       expert_stride, t, w_scales);
     }
     // One GEMV per routed row, up to 65535 rows per launch (grid.y).  Rows that share an expert read
     // its weights through L2.
@@ -339,7 +390,7 @@ int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void
         // keep launches aligned to whole tokens so that the x row of pair p is (p0 + p) / top_k
         uint64_t cnt = pairs - p0 < kMaxPerLaunch ? pairs - p0 : kMaxPerLaunch;
         if (cnt < pairs - p0) cnt -= cnt % top_k;
-        if (cnt == 0) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_id_ggml: top_k %u too large", top_k);
+        if (cnt == 0) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: top_k %u too large", fn, top_k);
         GemvArgs a{};
         a.x = static_cast<const uint8_t*>(x) + (size_t)(p0 / top_k) * xrow_bytes;
         a.w = static_cast<const uint8_t*>(w_stack);
@@ -356,6 +407,7 @@ int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, const void
     }
     return HQ_OK;
 }
+}  // namespace
 
 int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_jobs, hq_act_dtype xdt,
                           hq_ggml_type t) {

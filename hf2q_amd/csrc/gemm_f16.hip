@@ -47,6 +47,8 @@
 //     group g of k-step s covers k = 16g + 8s + j (s < 2, low nibbles) or
 //     32 + 16g + 8(s-2) + j (high nibbles); for the activations that is only
 //     the address of the fragment.
+#include <type_traits>
+
 #include "hq_internal.h"
 
 namespace hq {
@@ -131,8 +133,8 @@ __host__ __device__ __forceinline__ uint32_t weight_scan_lanes(uint32_t k) {
 // One group of 256 threads (t = thread within the group): the scales of 256 / lanes weight rows from first_row on,
 // `lanes` = weight_scan_lanes(k) lanes per row over the row's block headers.
 template <int TYPE>
-__device__ __forceinline__ void prep_weight_rows(const uint8_t* __restrict__ w, uint8_t* __restrict__ ws, const Workspace& L,
-                                                 uint32_t n, uint32_t k, uint32_t first_row, uint32_t t, uint32_t lanes) {
+__device__ __forceinline__ void prep_weight_rows(const uint8_t* __restrict__ w, float* __restrict__ scales, uint32_t n,
+                                                 uint32_t k, uint32_t first_row, uint32_t t, uint32_t lanes) {
     const uint32_t wr = first_row + t / lanes, sub = t & (lanes - 1u);
     constexpr uint32_t BLOCK = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q5_K ? Q5K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES
                                : TYPE == HQ_Q4_0 ? Q4_0_BYTES : Q8_0_BYTES;
@@ -142,7 +144,7 @@ __device__ __forceinline__ void prep_weight_rows(const uint8_t* __restrict__ w, 
     if (lanes > 2u) bound = dpp_max<0x4E>(bound);
     if (lanes > 4u) bound = dpp_max<0x141>(bound);
     if (lanes > 8u) bound = dpp_max<0x140>(bound);
-    if (sub == 0 && wr < n) reinterpret_cast<float*>(ws + L.wdown)[wr] = weight_row_scale(bound);
+    if (sub == 0 && wr < n) scales[wr] = weight_row_scale(bound);
 }
 
 // One group of GROUP threads (256, or 64 = one wave for short rows): row scale and f16 conversion of activation row
@@ -234,9 +236,17 @@ __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__
     const Workspace L = workspace_layout(m, n, k);
     if (blockIdx.x >= m) {
         const uint32_t lanes = weight_scan_lanes<TYPE>(k);
-        prep_weight_rows<TYPE>(w, ws, L, n, k, (blockIdx.x - m) * (256u / lanes), threadIdx.x, lanes);
+        prep_weight_rows<TYPE>(w, reinterpret_cast<float*>(ws + L.wdown), n, k, (blockIdx.x - m) * (256u / lanes), threadIdx.x, lanes);
     } else
         prep_activation_row<X_BF16>(x, ws, L, m, k, perm_hd, blockIdx.x, threadIdx.x, red);
+}
+
+// The weight-row scales alone: what the pre-pass's weight workgroups compute, for a caller that keeps them.
+template <int TYPE>
+__global__ __launch_bounds__(256) void weight_scales_kernel(const uint8_t* __restrict__ w, float* __restrict__ scales,
+                                                            uint32_t n, uint32_t k) {
+    const uint32_t lanes = weight_scan_lanes<TYPE>(k);
+    prep_weight_rows<TYPE>(w, scales, n, k, blockIdx.x * (256u / lanes), threadIdx.x, lanes);
 }
 
 struct GemmArgs {
@@ -257,6 +267,9 @@ struct GemmArgs {
     // Grouped form: the workspace holds one converted row per TOKEN and tile row r reads token row_map[r] / gather_div
     // (the routed rows of a token share its activations: top_k of them at gate / up, one at down).
     uint32_t gather_div;
+    // the weight rows' scales (lay_n floats): the pre-pass's in the workspace, or the caller's, computed once for weights
+    // that do not change (hq_weight_row_scales_ggml)
+    const float* wscale;
 };
 
 __device__ __forceinline__ f16x8_t as_frag(uint4 v) { return __builtin_bit_cast(f16x8_t, v); }
@@ -340,7 +353,7 @@ template <int MT, int NT>
 __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W, const f32x16_t (&acc)[MT][NT],
                                            uint32_t mbase, uint32_t nbase, uint32_t l32, uint32_t lg) {
     const float* rs = reinterpret_cast<const float*>(a.ws + W.rs);
-    const float* wd = reinterpret_cast<const float*>(a.ws + W.wdown);
+    const float* wd = a.wscale;
     const bool vec_ok = a.n % 4 == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;  // uniform
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -407,7 +420,7 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
         uint32_t gn = n0 + wn * (32 * NT) + nt * 32 + l32;
         gn = gn < a.n ? gn : a.n - 1u;
         wrow[nt] = a.w + (size_t)gn * row_bytes;
-        wdown[nt] = reinterpret_cast<const float*>(a.ws + W.wdown)[a.wd_off + gn];
+        wdown[nt] = a.wscale[a.wd_off + gn];
     }
     uint4 braw[4][NT];        // nibbles of stages s, s+1, s+2 in slots s%4 (a stage is a chunk of its super-block: slot = c)
     uint4 hdr[NT], hdrn[NT];  // super-block headers: current, next
@@ -636,7 +649,7 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     uint32_t gn = n0 + wn * 32 + l32;
     gn = gn < a.n ? gn : a.n - 1u;
     const uint8_t* blk0 = a.w + (size_t)gn * (a.k / 32) * BYTES + lg * BYTES;  // this lane's block of stage 0
-    const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[a.wd_off + gn];
+    const float wdown = a.wscale[a.wd_off + gn];
     const bool early = (reinterpret_cast<uintptr_t>(blk0) & 2u) == 0;  // blocks at 4n: the int8 start two bytes into a word
     const uint32_t shift = early ? 2u : 0u;
     const uint8_t* win0 = early ? blk0 : blk0 + 2;                     // first of the eight aligned words
@@ -764,7 +777,7 @@ __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     uint32_t gn = n0 + wn * 32 + l32;
     gn = gn < a.n ? gn : a.n - 1u;
     const uint8_t* wrow = a.w + (size_t)gn * (a.k / 256) * Q6K_BYTES;
-    const float wdown = reinterpret_cast<const float*>(a.ws + W.wdown)[a.wd_off + gn];
+    const float wdown = a.wscale[a.wd_off + gn];
     struct Raw { uint4 l0, l1, h0, h1; uint2 sc; uint32_t d; };  // one half of a super-block, this lane's share
     Raw braw[2];
     auto load_half = [&](uint32_t sb, int h, int slot) {
@@ -1116,8 +1129,8 @@ __global__ __launch_bounds__(1024) void grouped_prep_kernel(BucketArgs b, const 
                                              red + 4u * (threadIdx.x >> 8));
     } else {
         const uint32_t lanes = weight_scan_lanes<TYPE>(k);
-        prep_weight_rows<TYPE>(w, ws, L, n_rows, k, ((wg - row_wgs) * 4u + (threadIdx.x >> 8)) * (256u / lanes),
-                               threadIdx.x & 255u, lanes);
+        prep_weight_rows<TYPE>(w, reinterpret_cast<float*>(ws + L.wdown), n_rows, k,
+                               ((wg - row_wgs) * 4u + (threadIdx.x >> 8)) * (256u / lanes), threadIdx.x & 255u, lanes);
     }
 }
 
@@ -1177,9 +1190,9 @@ size_t gemm_f16_grouped_workspace_bytes(uint32_t pairs, uint32_t n_experts, uint
 
 template <int TYPE>
 static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, uint8_t* ws, uint32_t m,
-                       uint32_t n, uint32_t k, uint32_t perm_hd = 0) {
+                       uint32_t n, uint32_t k, uint32_t perm_hd, bool scan_weights) {
     const uint32_t rows_per_wg = 256u / weight_scan_lanes<TYPE>(k);
-    const dim3 prep_grid(m + (n + rows_per_wg - 1u) / rows_per_wg);
+    const dim3 prep_grid(m + (scan_weights ? (n + rows_per_wg - 1u) / rows_per_wg : 0u));  // the weight workgroups come last
     if (xdt == HQ_BF16)
         hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd);
     else
@@ -1190,7 +1203,7 @@ static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uin
 template <int TYPE>
 static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, const uint32_t* ids, float* y,
                             uint8_t* ws, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
-                            uint64_t expert_stride) {
+                            uint64_t expert_stride, const float* w_scales) {
     const uint32_t pairs = n_tokens * top_k;
     const GroupedLayout G = grouped_layout(pairs, n_experts, n, k);
     uint32_t* row_map = reinterpret_cast<uint32_t*>(ws + G.row_map);
@@ -1207,7 +1220,8 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     const BucketArgs b{ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm};
     const uint32_t n_rows = n_experts * n;
     const uint32_t act_per_wg = grouped_prep_rows_per_wg(k), w_per_wg = 1024u / weight_scan_lanes<TYPE>(k);
-    const dim3 prep_grid(1u + (n_tokens + act_per_wg - 1u) / act_per_wg + (n_rows + w_per_wg - 1u) / w_per_wg);
+    const dim3 prep_grid(1u + (n_tokens + act_per_wg - 1u) / act_per_wg +
+                         (w_scales ? 0u : (n_rows + w_per_wg - 1u) / w_per_wg));  // the weight workgroups come last
     if (xdt == HQ_BF16)
         hipLaunchKernelGGL((grouped_prep_kernel<true, TYPE>), prep_grid, dim3(1024), 0, s, b, x, wb, ws, n_tokens, n_rows, k);
     else
@@ -1220,24 +1234,43 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
         if (mt == 2) kern = grouped_gemm_kernel<TYPE, 2>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;
-    GemmArgs a{ws, wb, y, pairs, n, k, n_tokens, n_experts * n, 0u, row_map, 0u, (k + 255u) / 256u, top_k};
+    GemmArgs a{ws, wb, y, pairs, n, k, n_tokens, n_experts * n, 0u, row_map, 0u, (k + 255u) / 256u, top_k,
+               w_scales ? w_scales : reinterpret_cast<const float*>(ws + workspace_layout(n_tokens, n_rows, k).wdown)};
     const uint32_t tiles_n = (n + bn - 1) / bn;
     const uint32_t max_tiles = pairs / bm + n_experts;
     hipLaunchKernelGGL(kern, dim3(max_tiles * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
     return check_launch("grouped gemm kernel launch");
 }
 
+int launch_weight_row_scales(hipStream_t s, const void* w, float* scales, uint32_t n_rows, uint32_t k, hq_ggml_type t) {
+    const uint8_t* wb = static_cast<const uint8_t*>(w);
+    auto go = [&](auto tag) {
+        constexpr int TYPE = decltype(tag)::value;
+        const uint32_t per_wg = 256u / weight_scan_lanes<TYPE>(k);
+        hipLaunchKernelGGL((weight_scales_kernel<TYPE>), dim3((n_rows + per_wg - 1u) / per_wg), dim3(256), 0, s, wb, scales, n_rows, k);
+        return check_launch("weight row scales launch");
+    };
+    switch (t) {
+        case HQ_Q4_K: return go(std::integral_constant<int, HQ_Q4_K>{});
+        case HQ_Q5_K: return go(std::integral_constant<int, HQ_Q5_K>{});
+        case HQ_Q6_K: return go(std::integral_constant<int, HQ_Q6_K>{});
+        case HQ_Q8_0: return go(std::integral_constant<int, HQ_Q8_0>{});
+        case HQ_Q4_0: return go(std::integral_constant<int, HQ_Q4_0>{});
+    }
+    return fail(HQ_ERR_UNSUPPORTED, "weight row scales: ggml type %d", (int)t);
+}
+
 int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_stack, const uint32_t* ids, float* y,
                             void* workspace, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
-                            uint64_t expert_stride, hq_ggml_type t) {
+                            uint64_t expert_stride, hq_ggml_type t, const float* w_scales) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const uint8_t* wb = static_cast<const uint8_t*>(w_stack);
     switch (t) {
-        case HQ_Q4_K: return launch_grouped_t<HQ_Q4_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
-        case HQ_Q5_K: return launch_grouped_t<HQ_Q5_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
-        case HQ_Q6_K: return launch_grouped_t<HQ_Q6_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
-        case HQ_Q8_0: return launch_grouped_t<HQ_Q8_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
-        case HQ_Q4_0: return launch_grouped_t<HQ_Q4_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride);
+        case HQ_Q4_K: return launch_grouped_t<HQ_Q4_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
+        case HQ_Q5_K: return launch_grouped_t<HQ_Q5_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
+        case HQ_Q6_K: return launch_grouped_t<HQ_Q6_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
+        case HQ_Q8_0: return launch_grouped_t<HQ_Q8_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
+        case HQ_Q4_0: return launch_grouped_t<HQ_Q4_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
     }
     return fail(HQ_ERR_UNSUPPORTED, "grouped gemm: ggml type %d", (int)t);
 }
@@ -1247,10 +1280,11 @@ bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {
 }
 
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
-                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd) {
+                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd, const float* w_scales) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const uint8_t* wb = static_cast<const uint8_t*>(w);
-    GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr, 0u, (k + 255u) / 256u};
+    GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr, 0u, (k + 255u) / 256u, 0u,
+               w_scales ? w_scales : reinterpret_cast<const float*>(ws + workspace_layout(m, n, k).wdown)};
     constexpr int lds = 2 * ActTile::kTile;
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     // up to 256 token rows of Q6_K / Q8_0 / Q4_0: one token tile of 128 or 256 rows x 128 weight rows, k in slices where
@@ -1273,7 +1307,7 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         return check_launch("split sum kernel launch");
     };
     if (t == HQ_Q6_K) {
-        if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k, perm_hd)) return rc;
+        if (int rc = launch_prep<HQ_Q6_K>(s, x, xdt, wb, ws, m, n, k, perm_hd, !w_scales)) return rc;
         if (gemm_f16_small_tiles(t, m)) return launch_mid_small(mid_gemm_small_kernel<HQ_Q6_K, 4>, mid_gemm_small_kernel<HQ_Q6_K, 8>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(q6k_gemm_kernel), (size_t)lds, "hipFuncSetAttribute(q6_k gemm LDS)"))
             return rc;
@@ -1282,8 +1316,8 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
     }
     if (t == HQ_Q8_0 || t == HQ_Q4_0) {
         void (*kern)(GemmArgs) = t == HQ_Q4_0 ? q80_gemm_kernel<HQ_Q4_0> : q80_gemm_kernel<HQ_Q8_0>;
-        if (int rc = t == HQ_Q4_0 ? launch_prep<HQ_Q4_0>(s, x, xdt, wb, ws, m, n, k, perm_hd)
-                                  : launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, perm_hd))
+        if (int rc = t == HQ_Q4_0 ? launch_prep<HQ_Q4_0>(s, x, xdt, wb, ws, m, n, k, perm_hd, !w_scales)
+                                  : launch_prep<HQ_Q8_0>(s, x, xdt, wb, ws, m, n, k, perm_hd, !w_scales))
             return rc;
         if (gemm_f16_small_tiles(t, m))
             return t == HQ_Q4_0 ? launch_mid_small(mid_gemm_small_kernel<HQ_Q4_0, 4>, mid_gemm_small_kernel<HQ_Q4_0, 8>)
@@ -1293,8 +1327,8 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         hipLaunchKernelGGL(kern, dim3(tile_grid(tiles_m, cols_wide)), dim3(64 * WAVES), lds, s, a);
         return check_launch("q8_0 gemm kernel launch");
     }
-    if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, perm_hd)
-                              : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, perm_hd))
+    if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wb, ws, m, n, k, perm_hd, !w_scales)
+                              : launch_prep<HQ_Q4_K>(s, x, xdt, wb, ws, m, n, k, perm_hd, !w_scales))
         return rc;
     if (gemm_f16_small_tiles(t, m)) {  // Q4_K / Q5_K: one token tile of 64, 128 or 256 rows, tiles of 128 weight rows
         const int mts = m <= (uint32_t)BM_SMALL ? 2 : m <= (uint32_t)BM_MID ? 4 : 8;

@@ -81,7 +81,11 @@ size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml
 // perm_hd != 0: the activations are stored [k / perm_hd][m][perm_hd] (attention output, heads outermost) and are
 // gathered by the pre-pass.
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
-                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd = 0);
+                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd = 0,
+                         const float* w_scales = nullptr);
+// The tile kernels' weight-row scales (n_rows floats, a function of the weights alone): what the pre-pass of every tile
+// or grouped call works out when w_scales is null.
+int launch_weight_row_scales(hipStream_t s, const void* w, float* scales, uint32_t n_rows, uint32_t k, hq_ggml_type t);
 
 // Grouped form of the tile GEMM for mul_mat_id with many routed rows: rows sorted by expert, one
 // tile = up to 256 rows of one expert; needs a contiguous stack (expert_stride = n rows) and a device
@@ -90,7 +94,7 @@ bool gemm_f16_grouped_supported(hq_ggml_type t, uint32_t n, uint32_t k, uint32_t
 size_t gemm_f16_grouped_workspace_bytes(uint32_t pairs, uint32_t n_experts, uint32_t n, uint32_t k);
 int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_stack, const uint32_t* ids, float* y,
                             void* workspace, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
-                            uint64_t expert_stride, hq_ggml_type t);
+                            uint64_t expert_stride, hq_ggml_type t, const float* w_scales = nullptr);
 
 // MoE glue (moe.hip)
 int launch_dense_gemv_bf16(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,

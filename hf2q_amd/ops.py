@@ -69,13 +69,38 @@ class GgmlQuantizedMatmulIdParams:
     ggml_type: int
 
 
+def weight_row_scales_ggml(weight: torch.Tensor, n_rows: int, k: int, ggml_type: int) -> torch.Tensor:
+    """The f16 tile kernels' scale of every weight row (n_rows floats; a stack counts its experts' rows in order): a
+    function of the weights alone, computed once when they are loaded and passed as `w_row_scales` to the matmul
+    calls, whose pre-pass then skips the scan of the block headers.  Same results to the bit."""
+    out = torch.empty(n_rows, dtype=torch.float32, device=weight.device)
+    _l.check(_l.load().hq_weight_row_scales_ggml(_stream(), _dev(weight, "weight"), _dev(out, "scales"), n_rows, k, ggml_type))
+    return out
+
+
+def _check_scales(s: torch.Tensor, rows: int) -> None:
+    if s.dtype != torch.float32 or s.numel() < rows or not s.is_contiguous():
+        raise ValueError(f"w_row_scales must be {rows} contiguous float32 values")
+
+
 def quantized_matmul_ggml(input: torch.Tensor, weight: torch.Tensor, dst: torch.Tensor,
-                          params: GgmlQuantizedMatmulParams, workspace: torch.Tensor | None = None) -> None:
+                          params: GgmlQuantizedMatmulParams, workspace: torch.Tensor | None = None,
+                          w_row_scales: torch.Tensor | None = None) -> None:
     """dst[m,n] = input[m,k] . W[n,k]^T, W = raw GGML blocks (uint8 tensor).  With `workspace`
-    (a uint8 device tensor of quantized_matmul_workspace_bytes()) the call allocates nothing."""
+    (a uint8 device tensor of quantized_matmul_workspace_bytes()) the call allocates nothing; `w_row_scales`
+    (weight_row_scales_ggml of this weight; needs `workspace`) saves the pre-pass its scan of the weights."""
     if dst.dtype != torch.float32:
         raise TypeError("dst must be float32")
     L = _l.load()
+    if w_row_scales is not None:
+        if workspace is None:
+            raise ValueError("w_row_scales needs a workspace")
+        _check_scales(w_row_scales, params.n)
+        _l.check(L.hq_qmatmul_ggml_ws_prepared(_stream(), _dev(input, "input"), _act_dtype(input), _dev(weight, "weight"),
+                                               _dev(w_row_scales, "w_row_scales"), _dev(dst, "dst"), params.m, params.n,
+                                               params.k, params.ggml_type, _dev(workspace, "workspace"),
+                                               workspace.numel() * workspace.element_size()))
+        return
     if workspace is not None:
         _l.check(L.hq_qmatmul_ggml_ws(_stream(), _dev(input, "input"), _act_dtype(input), _dev(weight, "weight"),
                                       _dev(dst, "dst"), params.m, params.n, params.k, params.ggml_type,
@@ -119,8 +144,9 @@ def quantized_matmul_mm_tensor_perm021(input_perm: torch.Tensor, weight: torch.T
 
 def quantized_matmul_id_ggml(input: torch.Tensor, weight_stack: torch.Tensor, ids: torch.Tensor,
                              output: torch.Tensor, params: GgmlQuantizedMatmulIdParams,
-                             scratch: torch.Tensor | None = None) -> None:
-    """output[t, s, :] = W[ids[t, s]] . input[t, :]."""
+                             scratch: torch.Tensor | None = None, w_row_scales: torch.Tensor | None = None) -> None:
+    """output[t, s, :] = W[ids[t, s]] . input[t, :].  `w_row_scales`: weight_row_scales_ggml of the whole stack
+    (n_experts * n rows), which the grouped (prefill) form then does not work out again."""
     if output.dtype != torch.float32:
         raise TypeError("output must be float32")
     if ids.dtype not in (torch.int32, torch.uint32):
@@ -128,6 +154,13 @@ def quantized_matmul_id_ggml(input: torch.Tensor, weight_stack: torch.Tensor, id
     L = _l.load()
     sp = _dev(scratch, "scratch") if scratch is not None else None
     sb = scratch.numel() * scratch.element_size() if scratch is not None else 0
+    if w_row_scales is not None:
+        _check_scales(w_row_scales, params.n_experts * params.n)
+        _l.check(L.hq_qmatmul_id_ggml_prepared(_stream(), _dev(input, "input"), _act_dtype(input),
+                                               _dev(weight_stack, "weight_stack"), _dev(w_row_scales, "w_row_scales"),
+                                               _dev(ids, "ids"), _dev(output, "output"), sp, sb, params.n_tokens, params.top_k,
+                                               params.n, params.k, params.n_experts, params.expert_stride, params.ggml_type))
+        return
     _l.check(L.hq_qmatmul_id_ggml(_stream(), _dev(input, "input"), _act_dtype(input),
                                   _dev(weight_stack, "weight_stack"), _dev(ids, "ids"), _dev(output, "output"),
                                   sp, sb, params.n_tokens, params.top_k, params.n, params.k, params.n_experts,

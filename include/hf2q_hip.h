@@ -157,6 +157,28 @@ HQ_API int hq_qmatmul_id_ggml(void* stream, const void* x, hq_act_dtype xdt, con
                        uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
                        uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
 
+/* The weight-row scales of the f16 tile kernels, kept by the caller.  Those kernels (the prefill-sized routes of
+ * hq_qmatmul_ggml[_ws] and the grouped route of hq_qmatmul_id_ggml) multiply every weight row by a power of two taken
+ * from the row's block headers before the weights are rounded to f16, and divide it out in the epilogue; every call
+ * works the scales out again in its pre-pass, which touches each cache line of the weights for four bytes of every
+ * block header (151 MB for a stack of 256 experts of 512 x 2048 Q4_K: 12-17 us of the call at 2048 tokens x top-8).  They
+ * are a function of the weights alone, so a caller whose weights do not change (inference) computes them once when the
+ * weights are loaded -- hq_weight_row_scales_ggml: `scales` receives n_rows floats, row r of the matrix, or row
+ * e * n + r of a contiguous stack -- and passes them to the _prepared forms, which skip that scan and are otherwise the
+ * calls they are named after, with the same results to the bit.  Scales that do not belong to the weights give wrong
+ * products (possibly inf / nan), never a fault.  Routes that do not use the tile kernels ignore the argument.  No
+ * counterpart in the reference, whose mul_mm kernels round the dequantised weights to half without a row scale
+ * (forward_mlx.rs:9791-9830). */
+HQ_API int hq_weight_row_scales_ggml(void* stream, const void* w_blocks, float* scales, uint64_t n_rows, uint32_t k,
+                              hq_ggml_type t);
+HQ_API int hq_qmatmul_ggml_ws_prepared(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks,
+                                const float* w_row_scales, float* y, uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t,
+                                void* workspace, size_t workspace_bytes);
+HQ_API int hq_qmatmul_id_ggml_prepared(void* stream, const void* x, hq_act_dtype xdt, const void* w_stack,
+                                const float* w_row_scales, const uint32_t* ids, float* y, void* scratch,
+                                size_t scratch_bytes, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
+                                uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
+
 /* Bytes of `scratch` the GEMV form needs for up to `max_rows` = n_tokens*top_k
  * routed rows (the IdMmScratch analogue, decode_pool.rs:56-60): always 0.  Kept
  * so that a port of the reference's scratch sizing call has something to call;

@@ -75,6 +75,9 @@ def test_empty_inputs_are_accepted_without_work():
     assert L.hq_qmatmul_ggml(None, fake, lib.HQ_BF16, fake, fake, 0, 8, 256, lib.HQ_Q4_K) == lib.HQ_OK
     assert L.hq_qmatmul_ggml_ws(None, fake, lib.HQ_BF16, fake, fake, 0, 8, 256, lib.HQ_Q6_K, None, 0) == lib.HQ_OK
     assert L.hq_qmatmul_id_ggml(None, fake, lib.HQ_F32, fake, fake, fake, None, 0, 0, 2, 8, 256, 4, 8 * 144, lib.HQ_Q4_K) == lib.HQ_OK
+    assert L.hq_qmatmul_ggml_ws_prepared(None, fake, lib.HQ_BF16, fake, fake, fake, 0, 8, 256, lib.HQ_Q6_K, None, 0) == lib.HQ_OK
+    assert L.hq_qmatmul_id_ggml_prepared(None, fake, lib.HQ_F32, fake, fake, fake, fake, None, 0, 0, 2, 8, 256, 4, 8 * 144, lib.HQ_Q4_K) == lib.HQ_OK
+    assert L.hq_weight_row_scales_ggml(None, fake, fake, 0, 256, lib.HQ_Q4_K) == lib.HQ_OK
     assert L.hq_dequant_ggml(None, fake, fake, lib.HQ_F32, 0, lib.HQ_Q8_0) == lib.HQ_OK
     assert L.hq_quantize_ggml(None, fake, 0, 256, lib.HQ_Q5_K, fake) == lib.HQ_OK
     assert L.hq_moe_softmax_topk(None, fake, fake, fake, 0, 256, 8) == lib.HQ_OK
@@ -103,6 +106,13 @@ def test_argument_errors_are_reported_not_fatal():
     assert L.hq_qmatmul_ggml(None, None, lib.HQ_F32, fake, fake, 1, 8, 256, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
     # id form: expert stride smaller than an expert
     assert L.hq_qmatmul_id_ggml(None, fake, lib.HQ_F32, fake, fake, fake, None, 0, 1, 2, 8, 256, 4, 100, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    # the prepared forms want the scales; the scales call wants whole blocks and a type of the library
+    assert L.hq_qmatmul_ggml_ws_prepared(None, fake, lib.HQ_BF16, fake, None, fake, 64, 8, 256, lib.HQ_Q4_K, fake, 1 << 20) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert "w_row_scales" in lib.last_error()
+    assert L.hq_qmatmul_id_ggml_prepared(None, fake, lib.HQ_F32, fake, None, fake, fake, None, 0, 1, 2, 8, 256, 4, 8 * 144, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_weight_row_scales_ggml(None, fake, fake, 8, 300, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_weight_row_scales_ggml(None, fake, fake, 8, 256, 10) == lib.HQ_ERR_UNSUPPORTED
+    assert L.hq_weight_row_scales_ggml(None, fake, None, 8, 256, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
     # batched form: too many jobs, a prefill-sized dense job, SwiGLU over bf16 activations
     jobs = (lib.QmatmulJob * 5)()
     for j in jobs:

@@ -138,6 +138,57 @@ def test_q4k_tile_gemm_workspace_variant(oracle, dev):
         ops.quantized_matmul_ggml(x, wd, y1, p, workspace=ws[: need - 256])
 
 
+def _row_bounds(blocks, n, k, t):
+    """Largest possible |w| of every weight row from its block headers alone, in f64."""
+    per, nbytes, d_at = {HQ_Q4_K: (256, 144, 0), HQ_Q5_K: (256, 176, 0), HQ_Q6_K: (256, 210, 208), HQ_Q8_0: (32, 34, 0),
+                         HQ_Q4_0: (32, 18, 0)}[t]
+    b = blocks.reshape(n, k // per, nbytes)
+    d = np.abs(b[:, :, d_at:d_at + 2].copy().view(np.float16).astype(np.float64)[:, :, 0])
+    if t in (HQ_Q4_K, HQ_Q5_K):
+        dmin = np.abs(b[:, :, 2:4].copy().view(np.float16).astype(np.float64)[:, :, 0])
+        return (d * (63 * 15 if t == HQ_Q4_K else 63 * 31) + dmin * 63).max(axis=1)
+    return (d * {HQ_Q6_K: 128 * 32, HQ_Q8_0: 128, HQ_Q4_0: 8}[t]).max(axis=1)
+
+
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
+def test_prepared_weight_row_scales(oracle, dev, t):
+    """The weight-row scales computed once (powers of two that bring a row's largest possible weight to [2^13, 2^14])
+    and handed to the call give the bits of the call that works them out itself, for the large and the small tiles;
+    a route without tile kernels ignores them."""
+    for m, n, k in ((300, 257, 768), (48, 160, 512), (64, 200, 256)):
+        blocks = oracle.quantize(weights(17 * n + k + t, n, k), k, t, threads=8)
+        blocks = blocks.copy()
+        per_row = blocks.size // n
+        blocks[3 * per_row:4 * per_row] = 0  # a row of zero scales: scale 1
+        wd = torch.from_numpy(blocks).to(dev)
+        scales = ops.weight_row_scales_ggml(wd, n, k, t)
+        sc = scales.cpu().numpy().astype(np.float64)
+        mant, _ = np.frexp(sc)
+        assert (mant == 0.5).all(), "powers of two"
+        bound = _row_bounds(blocks, n, k, t)
+        live = bound > 0
+        assert live.sum() == n - 1 and sc[~live] == 1.0
+        scaled = bound[live] * sc[live]
+        assert (scaled >= 2.0 ** 13 * (1 - 1e-6)).all() and (scaled <= 2.0 ** 14 * (1 + 1e-6)).all()
+        x = torch.from_numpy(acts(m + n, m, k)).to(dev).to(torch.bfloat16)
+        p = GgmlQuantizedMatmulParams(m, n, k, t)
+        need = ops.quantized_matmul_workspace_bytes(p, torch.bfloat16)
+        assert need > 0
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        y0 = torch.empty(m, n, device=dev)
+        ops.quantized_matmul_ggml(x, wd, y0, p, workspace=ws)
+        ws.fill_(0xFF)  # nothing of the first call's pre-pass is left to lean on
+        y1 = torch.full((m, n), float("nan"), device=dev)
+        ops.quantized_matmul_ggml(x, wd, y1, p, workspace=ws, w_row_scales=scales)
+        assert torch.equal(y0, y1), (m, n, k)
+    # one row: the GEMV route, no workspace needed, the scales are not looked at
+    p1 = GgmlQuantizedMatmulParams(1, n, k, t)
+    ya, yb = torch.empty(1, n, device=dev), torch.empty(1, n, device=dev)
+    ops.quantized_matmul_ggml(x[:1], wd, ya, p1)
+    ops.quantized_matmul_ggml(x[:1], wd, yb, p1, workspace=ws, w_row_scales=scales)
+    assert torch.equal(ya, yb)
+
+
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 def test_tile_gemm_scale_equivariance(oracle, dev, xdt, t):

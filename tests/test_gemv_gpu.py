@@ -306,6 +306,29 @@ def test_mul_mat_id_grouped_sparse_experts_skewed(oracle, dev, t):
     assert_matmul_close_f16_tile(y.cpu().numpy(), ref, f"grouped, sparse + skewed, t={t}")
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q8_0])
+@pytest.mark.parametrize("E,n,k,T,K", [(8, 128, 512, 64, 4), (4, 160, 256, 400, 3), (16, 64, 1024, 300, 1)])
+def test_mul_mat_id_grouped_with_prepared_weight_row_scales(oracle, dev, t, E, n, k, T, K):
+    """The stack's weight-row scales computed once and handed to the call: the bits of the call that works them out."""
+    if t == HQ_Q8_0 and k % 128:
+        pytest.skip("Q8_0 tile kernel needs k % 128 == 0")
+    stack, ids, xv, xd, p = _grouped_setup(oracle, dev, t, E, n, k, T, K, "bf16", seed=3)
+    need = ops.quantized_matmul_id_workspace_bytes(p)
+    assert need > 0
+    sd = torch.from_numpy(stack).to(dev)
+    idd = torch.from_numpy(ids.view(np.int32)).to(dev)
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    y0 = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(xd, sd, idd, y0, p, scratch=scratch)
+    scales = ops.weight_row_scales_ggml(sd, E * n, k, t)
+    scratch.fill_(0xFF)
+    y1 = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(xd, sd, idd, y1, p, scratch=scratch, w_row_scales=scales)
+    assert torch.equal(y0, y1)
+    with pytest.raises(ValueError):
+        ops.quantized_matmul_id_ggml(xd, sd, idd, y1, p, scratch=scratch, w_row_scales=scales[: E * n - 1])
+
+
 def test_mul_mat_id_grouped_routing_properties(oracle, dev):
     """Skewed routing with unused experts, an id that is no expert (NaN rows, the others untouched), agreement with
     the per-row GEMV form, a scratch that is too small, and a strided stack (which keeps the GEMV form)."""
