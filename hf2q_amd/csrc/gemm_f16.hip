@@ -164,32 +164,68 @@ __device__ __forceinline__ void prep_activation_row(const void* __restrict__ x, 
         const uint32_t kk = 8u * i;
         return perm_hd ? ((size_t)(kk / perm_hd) * m + row) * perm_hd + kk % perm_hd : (size_t)row * k + kk;
     };
-    auto load8 = [&](uint32_t i, float* v) {
+    struct Raw {
+        uint4 a, b;  // bf16: a holds the eight values; f32: a and b four each
+    };
+    auto load_raw = [&](uint32_t i) -> Raw {
+        Raw r{};
         if constexpr (X_BF16) {
-            const uint4 u = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + elem0(i));
-            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+            r.a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(x) + elem0(i));
+        } else {
+            const uint4* p = reinterpret_cast<const uint4*>(static_cast<const float*>(x) + elem0(i));
+            r.a = p[0], r.b = p[1];
+        }
+        return r;
+    };
+    auto decode = [&](const Raw& r, float* v) {
+        if constexpr (X_BF16) {
+            const uint32_t w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 v[2 * j] = bf16_bits_to_f32(w[j] & 0xffffu);
                 v[2 * j + 1] = bf16_bits_to_f32(w[j] >> 16);
             }
         } else {
-            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(x) + elem0(i));
-            const float4 a = p[0], b = p[1];
-            v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+            const uint32_t w[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = __uint_as_float(w[j]);
         }
     };
-
-    // largest finite magnitude of the row
-    float amax = 0.f;
-    for (uint32_t i = t; i < chunks; i += GROUP) {
+    auto fold = [&](const Raw& r, float& amax) {
         float v[8];
-        load8(i, v);
+        decode(r, v);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const float a = fabsf(v[j]);
             amax = a <= 3.0e38f ? fmaxf(amax, a) : amax;  // inf / nan do not set the scale
         }
+    };
+    auto convert = [&](const Raw& r, uint32_t i, float scale) {
+        float v[8];
+        decode(r, v);
+        uint32_t h[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) h[j] = f16_bits(v[j] * scale);
+        *reinterpret_cast<uint4*>(ws + L.xh + ((size_t)out_row * k + 8 * i) * 2) =
+            make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+    };
+
+    // largest finite magnitude of the row; a row of up to 2 * GROUP chunks (k <= 4096 for a group of 256) stays in
+    // registers for the conversion, longer ones are read a second time
+    const bool kept = chunks <= 2u * GROUP;
+    Raw held[2];
+    float amax = 0.f;
+    if (kept) {
+#pragma unroll
+        for (uint32_t j = 0; j < 2; ++j) {
+            const uint32_t i = t + j * GROUP;
+            held[j] = load_raw(i < chunks ? i : chunks - 1u);
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 2; ++j)
+            if (t + j * GROUP < chunks) fold(held[j], amax);
+    } else {
+        for (uint32_t i = t; i < chunks; i += GROUP) fold(load_raw(i), amax);
     }
     amax = dpp_max<0xB1>(amax);
     amax = dpp_max<0x4E>(amax);
@@ -211,19 +247,19 @@ __device__ __forceinline__ void prep_activation_row(const void* __restrict__ x, 
     if (!valid) return;
     if (t == 0) reinterpret_cast<float*>(ws + L.rs)[out_row] = ldexpf(1.f, -sh);
 
-    for (uint32_t i = t; i < chunks; i += GROUP) {
-        float v[8];
-        load8(i, v);
-        uint32_t h[8];
+    if (kept) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) h[j] = f16_bits(v[j] * scale);
-        *reinterpret_cast<uint4*>(ws + L.xh + ((size_t)out_row * k + 8 * i) * 2) =
-            make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+        for (uint32_t j = 0; j < 2; ++j)
+            if (t + j * GROUP < chunks) convert(held[j], t + j * GROUP, scale);
+    } else {
+        for (uint32_t i = t; i < chunks; i += GROUP) convert(load_raw(i), i, scale);
     }
 }
 
-// Pre-pass.  Workgroups [0, m): one per activation row, row scale and f16 conversion.  Workgroups
-// from m on: 256 / weight_scan_lanes(k) weight rows each, that many lanes per row over the row's block headers.  Per weight row, a
+// Pre-pass.  The first scan_wgs workgroups (none when the caller brings the scales): 256 / weight_scan_lanes(k) weight
+// rows each, that many lanes per row over the row's block headers; they are one load per lane and go first so that
+// they run beside the activation rows instead of behind them.  The next m workgroups: one per activation row, row
+// scale and f16 conversion.  Per weight row, a
 // power of two that brings the row's largest possible |w| (Q4_K: |d|*63*15 + |dmin|*63, Q6_K:
 // |d|*128*32, Q8_0: |d|*128) to about 2^14, so that neither large super-block scales overflow f16 nor small ones fall into its
 // subnormals; the main kernel multiplies the weights by it before they are rounded (exact) and its
@@ -231,14 +267,14 @@ __device__ __forceinline__ void prep_activation_row(const void* __restrict__ x, 
 template <bool X_BF16, int TYPE>
 __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
                                                         uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k,
-                                                        uint32_t perm_hd) {
+                                                        uint32_t perm_hd, uint32_t scan_wgs) {
     __shared__ float red[4];
     const Workspace L = workspace_layout(m, n, k);
-    if (blockIdx.x >= m) {
+    if (blockIdx.x < scan_wgs) {
         const uint32_t lanes = weight_scan_lanes<TYPE>(k);
-        prep_weight_rows<TYPE>(w, reinterpret_cast<float*>(ws + L.wdown), n, k, (blockIdx.x - m) * (256u / lanes), threadIdx.x, lanes);
+        prep_weight_rows<TYPE>(w, reinterpret_cast<float*>(ws + L.wdown), n, k, blockIdx.x * (256u / lanes), threadIdx.x, lanes);
     } else
-        prep_activation_row<X_BF16>(x, ws, L, m, k, perm_hd, blockIdx.x, threadIdx.x, red);
+        prep_activation_row<X_BF16>(x, ws, L, m, k, perm_hd, blockIdx.x - scan_wgs, threadIdx.x, red);
 }
 
 // The weight-row scales alone: what the pre-pass's weight workgroups compute, for a caller that keeps them.
@@ -1192,11 +1228,12 @@ template <int TYPE>
 static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, uint8_t* ws, uint32_t m,
                        uint32_t n, uint32_t k, uint32_t perm_hd, bool scan_weights) {
     const uint32_t rows_per_wg = 256u / weight_scan_lanes<TYPE>(k);
-    const dim3 prep_grid(m + (scan_weights ? (n + rows_per_wg - 1u) / rows_per_wg : 0u));  // the weight workgroups come last
+    const uint32_t scan_wgs = scan_weights ? (n + rows_per_wg - 1u) / rows_per_wg : 0u;
+    const dim3 prep_grid(scan_wgs + m);
     if (xdt == HQ_BF16)
-        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd);
+        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd, scan_wgs);
     else
-        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd);
+        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd, scan_wgs);
     return check_launch("tile gemm pre-pass launch");
 }
 
