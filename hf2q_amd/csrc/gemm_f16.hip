@@ -1064,6 +1064,7 @@ struct BucketArgs {
     uint32_t* n_tiles;
     float* y;
     uint32_t n, bm;
+    uint32_t half_tiles;  // a tile of at most bm / 2 rows is marked (tiles[].w = 1): the tile kernel runs it at half height
 };
 __device__ __forceinline__ void moe_bucket_sort(const BucketArgs& b, uint32_t* stage) {
     const uint32_t* __restrict__ ids = b.ids;
@@ -1129,7 +1130,8 @@ __device__ __forceinline__ void moe_bucket_sort(const BucketArgs& b, uint32_t* s
     }
     if (tid < n_experts) {
         cur[tid] = off;
-        for (uint32_t r = 0; r < my_rows; r += bm) tiles[first_tile + r / bm] = make_uint4(tid, off + r, off + my_rows, 0u);
+        for (uint32_t r = 0; r < my_rows; r += bm)
+            tiles[first_tile + r / bm] = make_uint4(tid, off + r, off + my_rows, b.half_tiles && my_rows - r <= bm / 2u ? 1u : 0u);
     }
     if (tid == 0) *n_tiles = total_tiles;
     __syncthreads();
@@ -1196,9 +1198,16 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
     a.w += (size_t)tt.x * expert_stride;
     a.wd_off = tt.x * a.n;
     a.m = tt.z;  // rows past the expert's run repeat its last row and are not stored
-    if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)
+    if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K) {
+        // the last tile of an expert, when at most half full, at half height (64 rows of 128: half of the MFMA work)
+        if constexpr (MT == 4) {
+            if (tt.w) {
+                q4k_gemm_tile<2, 1, 4, TYPE, true>(a, tt.y, n0);
+                return;
+            }
+        }
         q4k_gemm_tile<MT, 1, 4, TYPE, true>(a, tt.y, n0);
-    else if constexpr (TYPE == HQ_Q6_K)
+    } else if constexpr (TYPE == HQ_Q6_K)
         q6k_gemm_tile<MT, 4, true>(a, tt.y, n0);
     else
         q80_gemm_tile<MT, 4, TYPE, true>(a, tt.y, n0);
@@ -1269,7 +1278,7 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     const uint32_t bm = 32u * (uint32_t)mt, bn = BN_WIDE;
     // sort by expert + one converted activation row per token (the tiles gather the rows of their routed rows from
     // them) + the weight rows' scales, in one launch
-    const BucketArgs b{ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm};
+    const BucketArgs b{ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm, HAS_64 && mt == 4 ? 1u : 0u};
     const uint32_t n_rows = n_experts * n;
     const uint32_t act_per_wg = grouped_prep_rows_per_wg(k), w_per_wg = 1024u / weight_scan_lanes<TYPE>(k);
     const dim3 prep_grid(1u + (n_tokens + act_per_wg - 1u) / act_per_wg +
