@@ -111,6 +111,55 @@ def test_prefill_gemm_full_size(oracle, dev, t):
         assert (y[i] - y1[0]).abs().max().item() <= 1e-3 * y1.abs().max().item()
 
 
+@pytest.mark.parametrize("shape", ["gate_up", "down"])
+def test_grouped_mul_mat_id_full_size(oracle, dev, shape):
+    """Prefill-sized mul_mat_id of BASELINE config 3's layer: 2048 tokens x top-8 over 256 Q4_K experts, expert
+    512 x 2048 with one activation row per token (gate / up) or 2048 x 512 with one per routed row (down).  The
+    grouped tile form against the oracle on a sample of routed rows, against the per-row GEMV form (exact products,
+    itself checked against the oracle elsewhere) on every output, and with the stack's weight-row scales computed
+    once: the same bits."""
+    E, K, T = 256, 8, 2048
+    n, k = (512, 2048) if shape == "gate_up" else (2048, 512)
+    t = HQ_Q4_K
+    stack = _quantized(dev, E * n, k, t, 4321 + n)
+    stride = n * (k // oracle.BLOCK_ELEMS[t]) * oracle.BLOCK_BYTES[t]
+    g = torch.Generator(device=dev)
+    g.manual_seed(99)
+    rows, top_k = (T, K) if shape == "gate_up" else (T * K, 1)
+    x = torch.randn(rows, k, generator=g, device=dev).to(torch.bfloat16)
+    ids = torch.randint(0, E, (T * K,), generator=g, device=dev, dtype=torch.int32)
+    p = ops.GgmlQuantizedMatmulIdParams(rows, top_k, n, k, E, stride, t)
+    need = ops.quantized_matmul_id_workspace_bytes(p)
+    assert need > 0, "this shape takes the grouped route"
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    y = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(x, stack, ids, y, p, scratch=scratch)
+    assert torch.isfinite(y).all()
+    # (a) sampled routed rows against the f64 oracle
+    rng = np.random.default_rng(5)
+    ids_h = ids.cpu().numpy()
+    for pair in np.unique(np.concatenate([[0, 1, T * K - 1], rng.integers(0, T * K, 13)])):
+        e = int(ids_h[pair])
+        xs = x[pair // top_k:pair // top_k + 1].float().cpu().numpy()
+        wrows = stack[e * stride:(e + 1) * stride].cpu().numpy()
+        ref = oracle.qmatmul_f64(oracle.f32_to_bf16_bits(xs), wrows, 1, n, k, t)
+        assert_matmul_close_f16_tile(y[pair].cpu().numpy(), ref, f"grouped {shape}, routed row {pair} (expert {e})")
+    # (b) every output against the per-row GEMV form
+    y_gemv = torch.empty_like(y)
+    ops.quantized_matmul_id_ggml(x, stack, ids, y_gemv, p)
+    ref = y_gemv.double()
+    rms = ref.pow(2).mean().sqrt().item()
+    err = (y.double() - ref).abs()
+    assert (err <= 1e-3 * ref.abs() + 3e-3 * rms).all()
+    assert err.pow(2).mean().sqrt().item() <= 5e-4 * rms
+    # (c) the weight-row scales kept from an earlier pass over the stack
+    scales = ops.weight_row_scales_ggml(stack, E * n, k, t)
+    scratch.fill_(0xFF)
+    y2 = torch.full_like(y, float("nan"))
+    ops.quantized_matmul_id_ggml(x, stack, ids, y2, p, scratch=scratch, w_row_scales=scales)
+    assert torch.equal(y, y2)
+
+
 def test_moe_layer_full_size(oracle, dev):
     """hidden 2048, 256 experts x inter 512 (Q4_K), one shared expert, top-8, one token and eight: the block against
     a float64 evaluation over the device-dequantised weights of the experts the router picked.  The reference here is
