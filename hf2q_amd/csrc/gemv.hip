@@ -421,8 +421,9 @@ __device__ __forceinline__ void stream_load_x(const uint4* lds_x, const float* l
     }
 }
 
-// ROWS = 2: two activation rows (x[0], x[1] -> y[0], y[1] of one matrix) share every weight fetch and the
-// nibble-to-bf16 work; the dot products and sums are per row, in the order of the one-row form.
+// ROWS = 2 .. 4: that many activation rows (x[r] -> y[r] of one matrix) share every weight fetch and the
+// nibble-to-bf16 work; the dot products and sums are per row, in the order of the one-row form.  Three and four rows
+// read their activations from LDS per piece (in registers they would be 32 each per row).
 template <int TYPE, int W, bool XREG, int ROWS = 1>
 __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     constexpr uint32_t NT = 64 * W, BB = kBlockBytes<TYPE>;
@@ -545,7 +546,7 @@ int launch_stream(hipStream_t s, const SArgs& sa, uint32_t cus) {
     constexpr int W = TYPE == HQ_Q6_K ? 12 : 16;
     const size_t lds = ROWS * ((size_t)sa.k * 2 + (size_t)(sa.k / 16) * 4);
     // (the two-row Q5_K form with its activations in registers would spill: it reads them from LDS per row piece)
-    if (sa.k == 4096 && !(TYPE == HQ_Q5_K && ROWS == 2)) {
+    if (sa.k == 4096 && ROWS <= 2 && !(TYPE == HQ_Q5_K && ROWS == 2)) {
         auto kern = gemv_stream_kernel<TYPE, W, true, ROWS>;
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
         hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
@@ -622,11 +623,17 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     if (int rc = cu_count(&cus)) return rc;
     if constexpr (X_BF16 && kStreamType<TYPE>) {
         if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && stream_takes<TYPE>(a.n, a.k, cus)) {
-            // activation rows of a dense product two at a time (one pass over the weights per two rows), a last odd one alone
-            for (uint32_t r = 0; r < a.pairs; r += 2) {
+            // activation rows of a dense product up to four at a time (one pass over the weights for them)
+            for (uint32_t r = 0; r < a.pairs;) {
                 const SArgs sa{static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * 2, a.w, a.w, a.y + (size_t)r * a.n, a.y + (size_t)r * a.n,
                                a.n, a.n, a.k, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
-                if (int rc = a.pairs - r >= 2 ? launch_stream<TYPE, 2>(s, sa, cus) : launch_stream<TYPE, 1>(s, sa, cus)) return rc;
+                const uint32_t left = a.pairs - r, take = left >= 4 ? 4 : left;
+                if (int rc = take == 4   ? launch_stream<TYPE, 4>(s, sa, cus)
+                             : take == 3 ? launch_stream<TYPE, 3>(s, sa, cus)
+                             : take == 2 ? launch_stream<TYPE, 2>(s, sa, cus)
+                                         : launch_stream<TYPE, 1>(s, sa, cus))
+                    return rc;
+                r += take;
             }
             return HQ_OK;
         }
@@ -687,13 +694,19 @@ int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
 
 }  // namespace
 
-// Q6_K with bf16 activations on a matrix the streaming kernel takes: passes of two rows cost less than the small-batch
-// kernel up to five rows (151936 x 4096: 105 us per two rows against 310 us for any 4..8; 12288 x 4096: 10 against 32).
-bool gemv_two_row_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
-    if (t != HQ_Q6_K || xdt != HQ_BF16 || m < 3 || m > 5) return false;
+// A K-quant with bf16 activations on a matrix the streaming kernel takes: passes of up to four rows (one pass over the
+// weights each, every row's sum in the order of the one-row form) against the small-batch MFMA kernels, which cost the
+// same for any 3 / 4 .. 8 rows.  Q6_K, 151936 x 4096: 163 / 173 us for three / four rows and 252 .. 281 for five .. seven
+// against 307; 12288 x 4096: 13 .. 28 against 29.  Q4_K / Q5_K: three and four rows, 10.8 / 12.9 against 14.2 us at
+// 12288 x 4096 (102 / 132 against 134 at 151936 x 4096); from five rows on their small-batch kernel is ahead.
+bool gemv_stream_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
+    if (xdt != HQ_BF16 || m < 3) return false;
     uint32_t cus = 0;
     if (cu_count(&cus)) return false;
-    return stream_takes<HQ_Q6_K>(n, k, cus);
+    if (t == HQ_Q6_K) return m <= 7 && stream_takes<HQ_Q6_K>(n, k, cus);
+    if (t == HQ_Q4_K) return m <= 4 && stream_takes<HQ_Q4_K>(n, k, cus);
+    if (t == HQ_Q5_K) return m <= 4 && stream_takes<HQ_Q5_K>(n, k, cus);
+    return false;
 }
 
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t) {

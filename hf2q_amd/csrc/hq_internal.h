@@ -53,9 +53,9 @@ struct GemvArgs {
 // The current device's CU count (cached).
 int cu_count(uint32_t* out);
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t);
-// True where a few dense rows are better served by launch_gemv (which takes them two at a time) than by the
-// small-batch kernel.
-bool gemv_two_row_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k);
+// True where a few dense rows are better served by launch_gemv (which takes them up to four at a time, one pass over
+// the weights each) than by the small-batch kernel.
+bool gemv_stream_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k);
 // Up to four independent GEMVs of one weight type and activation dtype in a single launch.
 int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_act_dtype xdt, hq_ggml_type t);
 

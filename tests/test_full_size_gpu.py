@@ -34,10 +34,10 @@ DECODE_SHAPES = [(12288, 4096, HQ_Q4_K), (4096, 12288, HQ_Q4_K), (151936, 4096, 
 
 
 @pytest.mark.parametrize("n,k,t", DECODE_SHAPES)
-@pytest.mark.parametrize("m", [1, 2, 3, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 8])
 def test_decode_gemv_full_size(oracle, dev, n, k, t, m):
-    """m = 1: the GEMV kernels of the decode step; m = 2: their two-row form (one pass over the weights); m = 3: the
-    small-batch kernel (Q4_K) or a two-row and a one-row pass (Q6_K); m = 8: the small-batch kernels."""
+    """m = 1: the GEMV kernels of the decode step; m = 2 .. 4: their multi-row forms (one pass over the weights);
+    m = 7: a four-row and a three-row pass (Q6_K) or the small-batch kernel (Q4_K); m = 8: the small-batch kernels."""
     w = _quantized(dev, n, k, t, 7 + n)
     rng = np.random.default_rng(n + m)
     # multiples of 1/8 below 4 in magnitude: exact in bf16, and so are the sums of two of them
