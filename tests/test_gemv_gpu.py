@@ -329,6 +329,33 @@ def test_mul_mat_id_grouped_with_prepared_weight_row_scales(oracle, dev, t, E, n
         ops.quantized_matmul_id_ggml(xd, sd, idd, y1, p, scratch=scratch, w_row_scales=scales[: E * n - 1])
 
 
+def test_mul_mat_id_grouped_many_rows_and_unaligned_ids(oracle, dev):
+    """More routed rows than the expert sort stages in LDS (its permutation then goes straight to memory, and the ids
+    are walked in several batches), and ids that start 4 bytes past a 16-byte boundary (single loads instead of
+    16-byte ones): the same products."""
+    t, E, n, k, T, K = HQ_Q4_K, 8, 128, 256, 5200, 4
+    stack, ids, xv, xd, p = _grouped_setup(oracle, dev, t, E, n, k, T, K, "bf16", seed=11)
+    assert T * K > 16384
+    need = ops.quantized_matmul_id_workspace_bytes(p)
+    assert need > 0
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    sd = torch.from_numpy(stack).to(dev)
+    ref = oracle.qmatmul_id_f64(xv, stack, ids, T, K, n, k, E, p.expert_stride, t)
+    y = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(xd, sd, torch.from_numpy(ids.view(np.int32)).to(dev), y, p, scratch=scratch)
+    assert_matmul_close_f16_tile(y.cpu().numpy(), ref, "grouped, 20800 routed rows")
+    # a shorter call over ids that are not 16-byte aligned
+    T2 = 300
+    p2 = GgmlQuantizedMatmulIdParams(T2, K, n, k, E, p.expert_stride, t)
+    holder = torch.zeros(T2 * K + 1, dtype=torch.int32, device=dev)
+    holder[1:] = torch.from_numpy(ids[:T2 * K].view(np.int32)).to(dev)
+    off = holder[1:]
+    assert off.data_ptr() % 16 == 4
+    y2 = torch.full((T2 * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_ggml(xd[:T2].contiguous(), sd, off, y2, p2, scratch=scratch)
+    assert torch.equal(y2, y[:T2 * K])
+
+
 def test_mul_mat_id_grouped_routing_properties(oracle, dev):
     """Skewed routing with unused experts, an id that is no expert (NaN rows, the others untouched), agreement with
     the per-row GEMV form, a scratch that is too small, and a strided stack (which keeps the GEMV form)."""
