@@ -293,6 +293,27 @@ def bench_prefill_gemm(a, wtype=None):
     # caller-owned scratch for the tile kernels' pre-pass (f16 activations, row scales): allocated once
     need = ops.quantized_matmul_workspace_bytes(p, torch.bfloat16)
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+    flops = 2.0 * M * N * K
+    # The same product with the weight-row scales kept from load time (hq_qmatmul_ggml_ws_prepared; same bits), for
+    # `config`.  The first tens of calls after an idle gap run slower, and of two forms timed one after the other the
+    # first looked 6-8 us worse: this one is run once before the workload's own timing (not reported) and timed after it.
+    scales = ops.weight_row_scales_ggml(w, N, K, t) if need else None
+
+    def time_prepared():
+        if not need:
+            return None
+        for _ in range(max(a.warmup, 1)):
+            ops.quantized_matmul_ggml(x, w, y, p, workspace=ws, w_row_scales=scales)
+        torch.cuda.synchronize()
+        evp = _events(a.steps)
+        for i in range(a.steps):
+            evp[i][0].record()
+            ops.quantized_matmul_ggml(x, w, y, p, workspace=ws, w_row_scales=scales)
+            evp[i][1].record()
+        torch.cuda.synchronize()
+        return round(sum(e0.elapsed_time(e1) for e0, e1 in evp) * 1e3 / a.steps, 2)
+
+    time_prepared()
     for _ in range(a.warmup):
         ops.quantized_matmul_ggml(x, w, y, p, workspace=ws)
     torch.cuda.synchronize()
@@ -305,21 +326,8 @@ def bench_prefill_gemm(a, wtype=None):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     us = sum(e0.elapsed_time(e1) for e0, e1 in ev) * 1e3 / a.steps
-    flops = 2.0 * M * N * K
     tf = flops / us / 1e6
-    us_prepared = None
-    if need:  # the same product with the weight-row scales kept from load time (hq_qmatmul_ggml_ws_prepared; same bits)
-        scales = ops.weight_row_scales_ggml(w, N, K, t)
-        for _ in range(max(a.warmup, 1)):
-            ops.quantized_matmul_ggml(x, w, y, p, workspace=ws, w_row_scales=scales)
-        torch.cuda.synchronize()
-        evp = _events(a.steps)
-        for i in range(a.steps):
-            evp[i][0].record()
-            ops.quantized_matmul_ggml(x, w, y, p, workspace=ws, w_row_scales=scales)
-            evp[i][1].record()
-        torch.cuda.synchronize()
-        us_prepared = round(sum(e0.elapsed_time(e1) for e0, e1 in evp) * 1e3 / a.steps, 2)
+    us_prepared = time_prepared()
     # For scale only (not part of the path, not in `value`): the vendor library's plain f16 GEMM of the same shape,
     # no dequantisation, through torch.matmul; the same event timing over the same number of launches.
     vendor = None
@@ -395,8 +403,11 @@ def bench_moe_prefill(a):
             step(i)
             step_prepared(i)
         torch.cuda.synchronize()
-        _, us_prepared = _timed_steps(a, step_prepared, n_stacks)
+        # (of two forms timed one after the other the first looks a few microseconds worse: the kept-scales form is
+        # run once before the workload's own timing, not reported, and timed after it)
+        _timed_steps(a, step_prepared, n_stacks)
         elapsed, us = _timed_steps(a, step, n_stacks)
+        _, us_prepared = _timed_steps(a, step_prepared, n_stacks)
         return elapsed, us, us_prepared, need
 
     elapsed, us, us_prep, need = shape(I, H, T, K)
