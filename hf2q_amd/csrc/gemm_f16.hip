@@ -493,8 +493,9 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
             const float dmin = f16_bits_to_f32(h[nt].x >> 16) * wdown[nt];
             dsc[nt][0] = d * (float)sc0;
             dsc[nt][1] = d * (float)sc1;
-            ndm[nt][0] = -dmin * (float)mn0;
-            ndm[nt][1] = -dmin * (float)mn1;
+            // the weights are formed from 1024 + q (see b_eighth): the offset goes into the constant term
+            ndm[nt][0] = fmaf(-1024.f, dsc[nt][0], -dmin * (float)mn0);
+            ndm[nt][1] = fmaf(-1024.f, dsc[nt][1], -dmin * (float)mn1);
         }
     };
     // Eighth e of k-step ks of a stage with nibbles b and scales dsc / ndm: two weights -> one
@@ -513,16 +514,19 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                 const uint32_t h = (ks & 1) ? (half ? qv[nt].w : qv[nt].z) : (half ? qv[nt].y : qv[nt].x);
                 m |= ((h >> (2 * cc + hi)) & 0x01010101u) << 4;
             }
-            // opaque, so that the conversions stay v_cvt_f32_ubyte0..3 of this one register instead of
-            // a bit-field extract plus conversion each
+            // opaque: the masked word is formed once, here, and both byte permutes below read this register
             asm volatile("" : "+v"(m));
             mw[q] = m;
         }
         const uint32_t m = mw[q];
-        // d*sc*q - dmin*mn in fp32 (dsc and ndm are exact), one rounding to f16
-        const f32x2_t v = {fmaf(part ? ubyte2(m) : ubyte0(m), dsc[nt][hi], ndm[nt][hi]),
-                           fmaf(part ? ubyte3(m) : ubyte1(m), dsc[nt][hi], ndm[nt][hi])};
-        const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+        // Two values q < 32 placed under the f16 bit pattern of 1024 by one byte permute (0x6400 | q = 1024 + q), then
+        // d*sc*(1024 + q) + (-1024*d*sc - dmin*mn) per value as a mixed-precision FMA (f16 operand, f32 scale and
+        // constant, f32 arithmetic, f16 result): three instructions for two weights where conversion, FMA and packing
+        // took five.
+        const uint32_t pq = __builtin_amdgcn_perm(0x64646464u, m, part ? 0x04030402u : 0x04010400u);
+        uint32_t r;
+        asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(pq), "v"(dsc[nt][hi]), "v"(ndm[nt][hi]));
+        asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(r) : "v"(pq), "v"(dsc[nt][hi]), "v"(ndm[nt][hi]));
         if (half == 0)
             (part == 0 ? bfw[nt].x : bfw[nt].y) = r;
         else
