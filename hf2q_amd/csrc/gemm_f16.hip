@@ -314,6 +314,18 @@ typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 
 __device__ __forceinline__ uint4 ld16(const uint8_t* p) { return *reinterpret_cast<const uint4*>(p); }
 
+// Two f16 weights from bytes 2*part and 2*part + 1 of u (each below 256): the bytes are placed under the f16 bit
+// pattern of 1024 by one byte permute (0x6400 | b = 1024 + b, exact), then scale * (1024 + b) + c per value as a
+// mixed-precision FMA (f16 operand, f32 scale and constant, f32 arithmetic, f16 result); c carries -1024 * scale and the
+// format's own offset.  Three instructions for two weights where conversion, FMA and packing took five.
+__device__ __forceinline__ uint32_t mix_pair(uint32_t u, int part, float scale, float c) {
+    const uint32_t pq = __builtin_amdgcn_perm(0x64646464u, u, part ? 0x04030402u : 0x04010400u);
+    uint32_t r;
+    asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(pq), "v"(scale), "v"(c));
+    asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(r) : "v"(pq), "v"(scale), "v"(c));
+    return r;
+}
+
 constexpr int WAVES = 4;           // one per SIMD; two workgroups share a CU
 constexpr int BM = 256;            // token rows per workgroup of the prefill-sized tiles
 constexpr int BM_SMALL = 64;       // ... of the Q4_K / Q5_K tiles for a few token rows (up to 128)
@@ -519,14 +531,8 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
             mw[q] = m;
         }
         const uint32_t m = mw[q];
-        // Two values q < 32 placed under the f16 bit pattern of 1024 by one byte permute (0x6400 | q = 1024 + q), then
-        // d*sc*(1024 + q) + (-1024*d*sc - dmin*mn) per value as a mixed-precision FMA (f16 operand, f32 scale and
-        // constant, f32 arithmetic, f16 result): three instructions for two weights where conversion, FMA and packing
-        // took five.
-        const uint32_t pq = __builtin_amdgcn_perm(0x64646464u, m, part ? 0x04030402u : 0x04010400u);
-        uint32_t r;
-        asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(pq), "v"(dsc[nt][hi]), "v"(ndm[nt][hi]));
-        asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(r) : "v"(pq), "v"(dsc[nt][hi]), "v"(ndm[nt][hi]));
+        // d*sc*(1024 + q) + (-1024*d*sc - dmin*mn), see mix_pair
+        const uint32_t r = mix_pair(m, part, dsc[nt][hi], ndm[nt][hi]);
         if (half == 0)
             (part == 0 ? bfw[nt].x : bfw[nt].y) = r;
         else
@@ -736,7 +742,8 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                              "+v"(cur.hi.x), "+v"(cur.hi.y), "+v"(cur.hi.z), "+v"(cur.hi.w));
             const bool has_next = st + 1 < nstages;  // uniform
             if (has_next) load_b(st + 1, c ^ 1);
-            const float dsc = f16_bits_to_f32(cur.d & 0xffffu) * wdown, ndm = (Q4 ? -8.f : -128.f) * dsc;
+            // (the weights are formed from 1024 + q, see mix_pair: the constant term carries the -1024 as well; exact)
+            const float dsc = f16_bits_to_f32(cur.d & 0xffffu) * wdown, ndm = (Q4 ? -1032.f : -1152.f) * dsc;
             uint32_t dw[9];
             dw[0] = cur.lo.x, dw[1] = cur.lo.y, dw[2] = cur.lo.z, dw[3] = cur.lo.w;
             if constexpr (Q4) {
@@ -755,13 +762,11 @@ __device__ __forceinline__ void q80_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                         u = (ks >= 2 ? u >> 4 : u) & 0x0f0f0f0fu;
                     else
                         u ^= 0x80808080u;
-                    // opaque, so that the conversions stay v_cvt_f32_ubyte0..3 of this one register
+                    // opaque: the word is formed once, here, and both byte permutes of mix_pair read this register
                     asm volatile("" : "+v"(u));
                     uw[q] = u;
                 }
-                const uint32_t u = uw[q];
-                const f32x2_t v = {fmaf(part ? ubyte2(u) : ubyte0(u), dsc, ndm), fmaf(part ? ubyte3(u) : ubyte1(u), dsc, ndm)};
-                const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+                const uint32_t r = mix_pair(uw[q], part, dsc, ndm);
                 (e == 0 ? bfw.x : e == 1 ? bfw.y : e == 2 ? bfw.z : bfw.w) = r;
             };
             auto a_frag = [&](int t) -> uint4 {
@@ -872,6 +877,7 @@ __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
             const uint32_t scw = (hi ? cur.sc.y : cur.sc.x) >> (16 * lg);
             const float dw = f16_bits_to_f32(cur.d & 0xffffu) * wdown;
             const float dsc0 = dw * (float)(int)(int8_t)(scw & 0xffu), dsc1 = dw * (float)(int)(int8_t)((scw >> 8) & 0xffu);
+            const float ndm0 = -1056.f * dsc0, ndm1 = -1056.f * dsc1;
             const uint32_t lw[8] = {cur.l0.x, cur.l0.y, cur.l0.z, cur.l0.w, cur.l1.x, cur.l1.y, cur.l1.z, cur.l1.w};
             const uint32_t hw[8] = {cur.h0.x, cur.h0.y, cur.h0.z, cur.h0.w, cur.h1.x, cur.h1.y, cur.h1.z, cur.h1.w};
             const uint32_t hshift = 4 * hi + 2 * lg;
@@ -883,14 +889,12 @@ __device__ __forceinline__ void q6k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
                 if (part == 0) {
                     const uint32_t nib = (hi ? lw[i] >> 4 : lw[i]) & 0x0f0f0f0fu;
                     uint32_t u = (((hw[i] >> hshift) & 0x03030303u) << 4) | nib;
-                    // opaque, so that the conversions stay v_cvt_f32_ubyte0..3 of this one register
+                    // opaque: the word is formed once, here, and both byte permutes of mix_pair read this register
                     asm volatile("" : "+v"(u));
                     uw[q] = u;
                 }
-                const uint32_t u = uw[q];
-                const float dsc = ks < 2 ? dsc0 : dsc1, ndm = -32.f * dsc;  // elements 8*ks.. of 32: scale ks / 2
-                const f32x2_t v = {fmaf(part ? ubyte2(u) : ubyte0(u), dsc, ndm), fmaf(part ? ubyte3(u) : ubyte1(u), dsc, ndm)};
-                const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+                // elements 8*ks.. of 32: scale ks / 2; d*sc*(1024 + q) - 1056*d*sc (the format's 32 and mix_pair's 1024)
+                const uint32_t r = mix_pair(uw[q], part, ks < 2 ? dsc0 : dsc1, ks < 2 ? ndm0 : ndm1);
                 (e == 0 ? bfw.x : e == 1 ? bfw.y : e == 2 ? bfw.z : bfw.w) = r;
             };
             auto a_frag = [&](int t) -> uint4 {
