@@ -239,6 +239,35 @@ pub unsafe fn qmatmul_ggml_ws(stream: *mut c_void, x: *const c_void, xdt: hq_act
     check(hq_qmatmul_ggml_ws(stream, x, xdt, w_blocks, y, m, n, k, t, workspace, workspace_bytes))
 }
 
+/// The weight-row scales of the f16 tile kernels (`n_rows` floats; a contiguous expert stack counts its experts' rows
+/// in order).  They depend on the weights alone: compute them once after a tensor's blocks are uploaded, keep the
+/// buffer beside the weight and pass it to the `_prepared` calls, whose pre-pass then skips the scan of the block
+/// headers (same results to the bit).
+///
+/// # Safety
+/// Device pointers: `w_blocks` holds `n_rows` rows of `k` weights of type `t`, `scales` has room for `n_rows` floats.
+pub unsafe fn weight_row_scales_ggml(stream: *mut c_void, w_blocks: *const c_void, scales: *mut f32, n_rows: u64, k: u32, t: hq_ggml_type) -> Result<(), HqError> {
+    check(hq_weight_row_scales_ggml(stream, w_blocks, scales, n_rows, k, t))
+}
+
+/// `qmatmul_ggml_ws` with the weight's row scales from `weight_row_scales_ggml`.
+///
+/// # Safety
+/// As `qmatmul_ggml_ws`; `w_row_scales` holds the `n` floats computed for exactly these `w_blocks`.
+#[allow(clippy::too_many_arguments)]
+pub unsafe fn qmatmul_ggml_ws_prepared(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, w_row_scales: *const f32, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> Result<(), HqError> {
+    check(hq_qmatmul_ggml_ws_prepared(stream, x, xdt, w_blocks, w_row_scales, y, m, n, k, t, workspace, workspace_bytes))
+}
+
+/// `qmatmul_id_ggml` with the stack's row scales (`n_experts * n` floats) from `weight_row_scales_ggml`.
+///
+/// # Safety
+/// As `qmatmul_id_ggml`; `w_row_scales` holds the floats computed for exactly this `w_stack`.
+#[allow(clippy::too_many_arguments)]
+pub unsafe fn qmatmul_id_ggml_prepared(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_stack: *const c_void, w_row_scales: *const f32, ids: *const u32, y: *mut f32, scratch: *mut c_void, scratch_bytes: usize, n_tokens: u32, top_k: u32, n: u32, k: u32, n_experts: u32, expert_stride: u64, t: hq_ggml_type) -> Result<(), HqError> {
+    check(hq_qmatmul_id_ggml_prepared(stream, x, xdt, w_stack, w_row_scales, ids, y, scratch, scratch_bytes, n_tokens, top_k, n, k, n_experts, expert_stride, t))
+}
+
 /// `quantized_matmul_id_ggml`: one product per (token, slot) with the slot's expert.  `scratch` = null keeps the
 /// per-row GEMV form; with `hq_qmatmul_id_ggml_workspace_bytes(..)` bytes of scratch, prefill-sized inputs are
 /// sorted by expert and multiplied as tiles.
