@@ -412,6 +412,42 @@ def bench_moe_prefill(a):
 
     elapsed, us, us_prep, need = shape(I, H, T, K)
     _, us_down, us_down_prep, _ = shape(H, I, T * K, 1)
+
+    # gate, up and SwiGLU of the block: two calls and hq_silu_mul, against the one grouped call that does all three
+    def block():
+        gates = [ops.quantize_ggml(torch.randn(E * I * H, generator=gen, device=dev).mul_(0.02), H, HQ_Q4_K) for _ in range(2)]
+        ups = [ops.quantize_ggml(torch.randn(E * I * H, generator=gen, device=dev).mul_(0.02), H, HQ_Q4_K) for _ in range(2)]
+        p = GgmlQuantizedMatmulIdParams(T, K, I, H, E, I * ops.ggml_row_bytes(HQ_Q4_K, H), HQ_Q4_K)
+        x = torch.randn(T, H, generator=gen, device=dev).to(torch.bfloat16)
+        ids = torch.randint(0, E, (T * K,), generator=gen, device=dev, dtype=torch.int32)
+        yg, yu, act = (torch.empty(T * K, I, device=dev) for _ in range(3))
+        scratch = torch.empty(ops.quantized_matmul_id_swiglu_workspace_bytes(p), dtype=torch.uint8, device=dev)
+
+        def separate(i):
+            ops.quantized_matmul_id_ggml(x, gates[i % 2], ids, yg, p, scratch=scratch)
+            ops.quantized_matmul_id_ggml(x, ups[i % 2], ids, yu, p, scratch=scratch)
+            ops.dispatch_silu_mul(yg, yu, act)
+
+        def fused(i):
+            ops.quantized_matmul_id_swiglu_ggml(x, gates[i % 2], ups[i % 2], ids, act, p, scratch)
+
+        gs = [ops.weight_row_scales_ggml(w, E * I, H, HQ_Q4_K) for w in gates]
+        us_ = [ops.weight_row_scales_ggml(w, E * I, H, HQ_Q4_K) for w in ups]
+
+        def fused_kept(i):
+            ops.quantized_matmul_id_swiglu_ggml(x, gates[i % 2], ups[i % 2], ids, act, p, scratch, gs[i % 2], us_[i % 2])
+
+        for i in range(max(a.warmup, 1)):
+            separate(i)
+            fused(i)
+        torch.cuda.synchronize()
+        _timed_steps(a, fused, 2)
+        _, us_sep = _timed_steps(a, separate, 2)
+        _, us_fused = _timed_steps(a, fused, 2)
+        _, us_kept = _timed_steps(a, fused_kept, 2)
+        return us_sep, us_fused, us_kept
+
+    us_sep, us_fused, us_fused_kept = block()
     flops = 2.0 * T * K * I * H
     tf = flops / us / 1e6
     return _finish(a, {
@@ -426,6 +462,11 @@ def bench_moe_prefill(a):
                        "what": "hq_qmatmul_id_ggml_prepared: the stack's row scales (a function of the weights alone) computed "
                                "once, the call's pre-pass skips their scan; same bits", "us_per_step": round(us_prep, 2),
                        "TFLOP/s": round(flops / us_prep / 1e6, 1)},
+                   "gate_up_swiglu": {"what": "gate, up and SwiGLU of the block (2 x 34.4 GFLOP): two mul_mat_id calls + hq_silu_mul "
+                                              "(5 launches) against hq_qmatmul_id_swiglu_ggml (2 launches), same bits",
+                                      "separate_us": round(us_sep, 2), "one_call_us": round(us_fused, 2),
+                                      "one_call_with_kept_scales_us": round(us_fused_kept, 2),
+                                      "one_call_TFLOP/s": round(2 * flops / us_fused / 1e6, 1)},
                    "down_shape_2048x512": {"us_per_step": round(us_down, 2), "TFLOP/s": round(flops / us_down / 1e6, 1),
                                            "us_per_step_with_kept_scales": round(us_down_prep, 2)}},
         "roofline": {"bound": "mfma", "kernel": "grouped pre-pass + grouped f16 MFMA gemm q4_k", "achieved": round(tf, 1),

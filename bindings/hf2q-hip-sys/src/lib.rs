@@ -151,6 +151,8 @@ extern "C" {
     pub fn hq_weight_row_scales_ggml(stream: *mut c_void, w_blocks: *const c_void, scales: *mut f32, n_rows: u64, k: u32, t: hq_ggml_type) -> c_int;
     pub fn hq_qmatmul_ggml_ws_prepared(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, w_row_scales: *const f32, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
     pub fn hq_qmatmul_id_ggml_prepared(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_stack: *const c_void, w_row_scales: *const f32, ids: *const u32, y: *mut f32, scratch: *mut c_void, scratch_bytes: usize, n_tokens: u32, top_k: u32, n: u32, k: u32, n_experts: u32, expert_stride: u64, t: hq_ggml_type) -> c_int;
+    pub fn hq_qmatmul_id_swiglu_ggml_workspace_bytes(n_tokens: u32, top_k: u32, n: u32, k: u32, n_experts: u32, expert_stride: u64, t: hq_ggml_type) -> usize;
+    pub fn hq_qmatmul_id_swiglu_ggml(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_gate_stack: *const c_void, w_up_stack: *const c_void, gate_row_scales: *const f32, up_row_scales: *const f32, ids: *const u32, y: *mut f32, scratch: *mut c_void, scratch_bytes: usize, n_tokens: u32, top_k: u32, n: u32, k: u32, n_experts: u32, expert_stride: u64, t: hq_ggml_type) -> c_int;
     pub fn hq_qmatmul_id_scratch_bytes(n_experts: u32, max_rows: u32) -> usize;
     pub fn hq_qmatmul_id_ggml_workspace_bytes(n_tokens: u32, top_k: u32, n: u32, k: u32, n_experts: u32, expert_stride: u64, t: hq_ggml_type) -> usize;
     pub fn hq_qmatmul_batch_ggml(stream: *mut c_void, jobs: *const hq_qmatmul_job, n_jobs: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> c_int;

@@ -328,7 +328,7 @@ size_t hq_qmatmul_id_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uin
     if (hq_block_elems(t) == 0) return 0;  // not a type of this library
     if (n == 0 || k == 0 || k % hq_block_elems(t)) return 0;
     return grouped_route(n_tokens, top_k, n, k, n_experts, expert_stride, t)
-               ? gemm_f16_grouped_workspace_bytes(n_tokens * top_k, n_experts, n, k) : 0;
+               ? gemm_f16_grouped_workspace_bytes(n_tokens, top_k, n_experts, n, k) : 0;
 }
 
 namespace {
@@ -374,7 +374,7 @@ int qmatmul_id(const char* fn, void* stream, const void* x, hq_act_dtype xdt, co
     if (pairs == 0) return HQ_OK;
     // Many rows per expert and a workspace from the caller: rows sorted by expert, tile GEMM per expert.
     if (scratch && grouped_route(n_tokens, top_k, n, k, n_experts, expert_stride, t)) {
-        const size_t need = gemm_f16_grouped_workspace_bytes((uint32_t)pairs, n_experts, n, k);
+        const size_t need = gemm_f16_grouped_workspace_bytes(n_tokens, top_k, n_experts, n, k);
         if (scratch_bytes < need)
             return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch of %zu bytes, %zu needed", fn, scratch_bytes, need);
         if (reinterpret_cast<uintptr_t>(scratch) % 256)
@@ -408,6 +408,40 @@ int qmatmul_id(const char* fn, void* stream, const void* x, hq_act_dtype xdt, co
     return HQ_OK;
 }
 }  // namespace
+
+size_t hq_qmatmul_id_swiglu_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
+                                                 uint64_t expert_stride, hq_ggml_type t) {
+    if (hq_block_elems(t) == 0 || n == 0 || k == 0 || k % hq_block_elems(t)) return 0;
+    return gemm_f16_grouped_swiglu_supported(t) && grouped_route(n_tokens, top_k, n, k, n_experts, expert_stride, t)
+               ? gemm_f16_grouped_workspace_bytes(n_tokens, top_k, n_experts, n, k, 2) : 0;
+}
+
+int hq_qmatmul_id_swiglu_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate_stack, const void* w_up_stack,
+                              const float* gate_row_scales, const float* up_row_scales, const uint32_t* ids, float* y,
+                              void* scratch, size_t scratch_bytes, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
+                              uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t) {
+    const char* fn = "hq_qmatmul_id_swiglu_ggml";
+    if (int rc = check_matmul_common(fn, x, xdt, w_gate_stack, y, n, k, t)) return rc;
+    if (!w_up_stack) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (int rc = check_weight_alignment(w_up_stack, t)) return rc;
+    if (!ids) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null ids", fn);
+    if (n_experts == 0 || top_k == 0) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: n_experts %u, top_k %u", fn, n_experts, top_k);
+    if ((gate_row_scales == nullptr) != (up_row_scales == nullptr))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: the row scales of both stacks, or of neither", fn);
+    if (gate_row_scales && (!is_aligned(gate_row_scales, 4) || !is_aligned(up_row_scales, 4)))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: row scales must be 4-byte aligned", fn);
+    if ((uint64_t)n_tokens * top_k == 0) return HQ_OK;
+    const size_t need = hq_qmatmul_id_swiglu_ggml_workspace_bytes(n_tokens, top_k, n, k, n_experts, expert_stride, t);
+    if (!need)
+        return fail(HQ_ERR_UNSUPPORTED,
+                    "%s: this shape or type has no grouped SwiGLU form (hq_qmatmul_id_swiglu_ggml_workspace_bytes is 0): "
+                    "two hq_qmatmul_id_ggml calls and hq_silu_mul give the same result", fn);
+    if (!scratch || scratch_bytes < need)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch of %zu bytes, %zu needed", fn, scratch ? scratch_bytes : (size_t)0, need);
+    if (reinterpret_cast<uintptr_t>(scratch) % 256) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch must be 256-byte aligned", fn);
+    return launch_gemm_f16_grouped((hipStream_t)stream, x, xdt, w_gate_stack, ids, y, scratch, n_tokens, top_k, n, k, n_experts,
+                                   expert_stride, t, gate_row_scales, w_up_stack, up_row_scales);
+}
 
 int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_jobs, hq_act_dtype xdt,
                           hq_ggml_type t) {

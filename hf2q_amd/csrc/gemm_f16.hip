@@ -306,6 +306,10 @@ struct GemmArgs {
     // the weight rows' scales (lay_n floats): the pre-pass's in the workspace, or the caller's, computed once for weights
     // that do not change (hq_weight_row_scales_ggml)
     const float* wscale;
+    // SwiGLU form of the grouped Q4_K / Q5_K tiles: a second stack (the up projection beside the gate projection in
+    // `w`) and its rows' scales; the tile multiplies both and stores silu(gate) * up.  Null otherwise.
+    const uint8_t* w2;
+    const float* wscale2;
 };
 
 __device__ __forceinline__ f16x8_t as_frag(uint4 v) { return __builtin_bit_cast(f16x8_t, v); }
@@ -438,13 +442,60 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W
     }
 }
 
+// The epilogue of the SwiGLU form: acc[mt][0] holds the gate products and acc[mt][1] the up products of the same
+// output elements; both are scaled as store_tile scales them and silu(gate) * up is stored (silu_mul_f32: the bits
+// of the stand-alone kernel over the two separately stored products).
+template <int MT>
+__device__ __forceinline__ void store_tile_swiglu(const GemmArgs& a, const Workspace& W, const f32x16_t (&acc)[MT][2],
+                                                  uint32_t mbase, uint32_t nbase, uint32_t l32, uint32_t lg) {
+    const float* rs = reinterpret_cast<const float*>(a.ws + W.rs);
+    const bool vec_ok = a.n % 4 == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15u) == 0;  // uniform
+    const uint32_t gnb = nbase + 4 * lg;
+    float wup_g[16], wup_u[16];  // 2^e of the 16 weight rows of either stack, from their 2^-e
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        uint32_t gn = gnb + 8 * (v >> 2) + (v & 3);
+        gn = gn < a.n ? gn : a.n - 1u;
+        wup_g[v] = __uint_as_float(0x7f000000u - __float_as_uint(a.wscale[a.wd_off + gn]));
+        wup_u[v] = __uint_as_float(0x7f000000u - __float_as_uint(a.wscale2[a.wd_off + gn]));
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const uint32_t gm = mbase + mt * 32 + l32;
+        if (gm >= a.m) continue;
+        const uint32_t orow = a.row_map ? a.row_map[gm] : gm;
+        const float rsv = rs[a.gather_div ? orow / a.gather_div : gm];
+        float* yp = a.y + (size_t)orow * a.n + gnb;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float gv = acc[mt][0][4 * g + i] * (rsv * wup_g[4 * g + i]), uv = acc[mt][1][4 * g + i] * (rsv * wup_u[4 * g + i]);
+                o[i] = silu_mul_f32(gv, uv);
+            }
+            const uint32_t gn = gnb + 8 * g;
+            if (vec_ok) {
+                if (gn < a.n) *reinterpret_cast<float4*>(yp + 8 * g) = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (gn + i < a.n) yp[8 * g + i] = o[i];
+            }
+        }
+    }
+}
+
 // One workgroup tile of Q4_K weights: rows m0.. of the activations, weight rows n0...  The four
 // waves form a (4 / WN) x WN grid; a wave owns MT x NT MFMA tiles of 32 x 32.
 // TYPE = HQ_Q5_K: the same tile over 176-byte super-blocks; a lane also keeps the sixteen qh bytes that go with
 // its nibble bytes (they serve all four chunks of the super-block, bit 2c + hi for sub-block 2c + hi) and ORs the
 // fifth bit into the masked nibbles, three more VALU instructions per four weights.
-template <int MT, int NT, int WN, int TYPE = HQ_Q4_K, bool GATHER = false>
+// SWIGLU (NT = 2): the wave's two weight tiles are the same 32 rows of two stacks (a.w: gate, a.w2: up) and the
+// epilogue stores silu(gate) * up.
+template <int MT, int NT, int WN, int TYPE = HQ_Q4_K, bool GATHER = false, bool SWIGLU = false>
 __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, uint32_t n0) {
+    static_assert(!SWIGLU || NT == 2, "gate and up are the wave's two weight tiles");
     constexpr int BMT = 32 * MT * (WAVES / WN);  // token rows of the workgroup tile: 256, or 64 for the small tiles
     constexpr int DMA_PER_WAVE = ActTileT<BMT>::kDma;
     constexpr bool Q5 = TYPE == HQ_Q5_K;
@@ -465,10 +516,10 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
     float wdown[NT];  // power-of-two scale 2^-e of the lane's rows, from the pre-pass
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        uint32_t gn = n0 + wn * (32 * NT) + nt * 32 + l32;
+        uint32_t gn = SWIGLU ? n0 + wn * 32 + l32 : n0 + wn * (32 * NT) + nt * 32 + l32;
         gn = gn < a.n ? gn : a.n - 1u;
-        wrow[nt] = a.w + (size_t)gn * row_bytes;
-        wdown[nt] = a.wscale[a.wd_off + gn];
+        wrow[nt] = (SWIGLU && nt == 1 ? a.w2 : a.w) + (size_t)gn * row_bytes;
+        wdown[nt] = (SWIGLU && nt == 1 ? a.wscale2 : a.wscale)[a.wd_off + gn];
     }
     uint4 braw[4][NT];        // nibbles of stages s, s+1, s+2 in slots s%4 (a stage is a chunk of its super-block: slot = c)
     uint4 hdr[NT], hdrn[NT];  // super-block headers: current, next
@@ -660,7 +711,10 @@ __device__ __forceinline__ void q4k_gemm_tile(const GemmArgs& a, uint32_t m0, ui
         }
     }
 
-    store_tile<MT, NT>(a, W, acc, m0 + wm * (32 * MT), n0 + wn * (32 * NT), l32, lg);
+    if constexpr (SWIGLU)
+        store_tile_swiglu<MT>(a, W, acc, m0 + wm * (32 * MT), n0 + wn * 32, l32, lg);
+    else
+        store_tile<MT, NT>(a, W, acc, m0 + wm * (32 * MT), n0 + wn * (32 * NT), l32, lg);
 }
 
 // One workgroup tile of Q8_0 weights (34-byte blocks: f16 d, 32 int8), four waves side by side, each
@@ -1045,9 +1099,11 @@ struct GroupedLayout {
     size_t row_map, tiles, count, total;
     uint32_t max_tiles;
 };
-__host__ __device__ inline GroupedLayout grouped_layout(uint32_t pairs, uint32_t n_experts, uint32_t n, uint32_t k) {
+// n_tokens converted activation rows (the tiles gather their routed rows' tokens from them), the scales of w_rows
+// weight rows (n_experts * n, twice that for the SwiGLU form's two stacks), the permutation of the routed rows, the tiles.
+__host__ __device__ inline GroupedLayout grouped_layout(uint32_t n_tokens, uint32_t pairs, uint32_t n_experts, uint32_t w_rows, uint32_t k) {
     GroupedLayout g;
-    g.base = workspace_layout(pairs, n_experts * n, k);
+    g.base = workspace_layout(n_tokens, w_rows, k);
     g.max_tiles = pairs / BM_SMALL + n_experts;  // enough for tiles of 64 rows or more
     g.row_map = g.base.total;
     g.tiles = g.row_map + (((size_t)pairs * 4 + 255) & ~(size_t)255);
@@ -1172,15 +1228,16 @@ __host__ __device__ __forceinline__ uint32_t grouped_prep_rows_per_wg(uint32_t k
 
 template <bool X_BF16, int TYPE>
 __global__ __launch_bounds__(1024) void grouped_prep_kernel(BucketArgs b, const void* __restrict__ x, const uint8_t* __restrict__ w,
-                                                            uint8_t* __restrict__ ws, uint32_t m, uint32_t n_rows, uint32_t k,
-                                                            uint32_t stage_words) {
+                                                            const uint8_t* __restrict__ w2, uint8_t* __restrict__ ws, uint32_t m,
+                                                            uint32_t n_rows, uint32_t k, uint32_t stage_words) {
     extern __shared__ __align__(16) uint32_t sort_stage[];  // b.pairs words for workgroup 0 when the launch brings them
     if (blockIdx.x == 0) {
         moe_bucket_sort(b, stage_words ? sort_stage : nullptr);
         return;
     }
     __shared__ float red[16];
-    const Workspace L = workspace_layout(m, n_rows, k);
+    // (w2: a second stack of n_rows rows, scanned by workgroups of its own after the first stack's; its scales follow)
+    const Workspace L = workspace_layout(m, w2 ? 2u * n_rows : n_rows, k);
     const uint32_t per_wg = grouped_prep_rows_per_wg(k), row_wgs = (m + per_wg - 1u) / per_wg, wg = blockIdx.x - 1u;
     if (wg < row_wgs) {
         if (per_wg == 16u)
@@ -1189,14 +1246,16 @@ __global__ __launch_bounds__(1024) void grouped_prep_kernel(BucketArgs b, const 
             prep_activation_row<X_BF16, 256>(x, ws, L, m, k, 0u, wg * 4u + (threadIdx.x >> 8), threadIdx.x & 255u,
                                              red + 4u * (threadIdx.x >> 8));
     } else {
-        const uint32_t lanes = weight_scan_lanes<TYPE>(k);
-        prep_weight_rows<TYPE>(w, reinterpret_cast<float*>(ws + L.wdown), n_rows, k,
-                               ((wg - row_wgs) * 4u + (threadIdx.x >> 8)) * (256u / lanes), threadIdx.x & 255u, lanes);
+        const uint32_t lanes = weight_scan_lanes<TYPE>(k), per_scan_wg = 1024u / lanes;
+        const uint32_t stack_wgs = (n_rows + per_scan_wg - 1u) / per_scan_wg;
+        const uint32_t sw = wg - row_wgs, second = sw >= stack_wgs ? 1u : 0u;
+        prep_weight_rows<TYPE>(second ? w2 : w, reinterpret_cast<float*>(ws + L.wdown) + second * n_rows, n_rows, k,
+                               ((sw - second * stack_wgs) * 4u + (threadIdx.x >> 8)) * (256u / lanes), threadIdx.x & 255u, lanes);
     }
 }
 
 // A tile is 32 * MT routed rows (MT 8: 256 rows; 4: 128; 2: 64, Q4_K / Q5_K only) x 128 weight rows, a wave all its rows x 32.
-template <int TYPE, int MT>
+template <int TYPE, int MT, bool SWIGLU = false>
 __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a, const uint4* __restrict__ tiles,
                                                                       const uint32_t* __restrict__ n_tiles, uint32_t tiles_n,
                                                                       uint64_t expert_stride) {
@@ -1206,7 +1265,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
     a.w += (size_t)tt.x * expert_stride;
     a.wd_off = tt.x * a.n;
     a.m = tt.z;  // rows past the expert's run repeat its last row and are not stored
-    if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K) {
+    if constexpr (SWIGLU) {  // Q4_K / Q5_K: gate and up of the same 32 weight rows per wave, silu(gate) * up stored
+        a.w2 += (size_t)tt.x * expert_stride;
+        q4k_gemm_tile<MT, 2, 4, TYPE, true, true>(a, tt.y, n0);
+    } else if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K) {
         // the last tile of an expert, when at most half full, at half height (64 rows of 128: half of the MFMA work)
         if constexpr (MT == 4) {
             if (tt.w) {
@@ -1252,9 +1314,14 @@ bool gemm_f16_grouped_supported(hq_ggml_type t, uint32_t n, uint32_t k, uint32_t
     return expert_stride == (uint64_t)n * row_bytes && (uint64_t)n_experts * n <= 0x7fffffffull;
 }
 
-size_t gemm_f16_grouped_workspace_bytes(uint32_t pairs, uint32_t n_experts, uint32_t n, uint32_t k) {
-    return grouped_layout(pairs, n_experts, n, k).total;
+size_t gemm_f16_grouped_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n_experts, uint32_t n, uint32_t k,
+                                        uint32_t stacks) {
+    return grouped_layout(n_tokens, n_tokens * top_k, n_experts, stacks * n_experts * n, k).total;
 }
+
+// The SwiGLU form (two stacks, silu(gate) * up stored) exists for the Q4_K / Q5_K tiles, whose waves take two weight
+// tiles side by side.
+bool gemm_f16_grouped_swiglu_supported(hq_ggml_type t) { return t == HQ_Q4_K || t == HQ_Q5_K; }
 
 template <int TYPE>
 static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, uint8_t* ws, uint32_t m,
@@ -1272,9 +1339,10 @@ static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uin
 template <int TYPE>
 static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, const uint32_t* ids, float* y,
                             uint8_t* ws, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
-                            uint64_t expert_stride, const float* w_scales) {
+                            uint64_t expert_stride, const float* w_scales, const uint8_t* wb2, const float* w_scales2) {
+    // wb2: the SwiGLU form, y = silu(W[ids] . x) * (W2[ids] . x); Q4_K / Q5_K only (the caller has checked)
     const uint32_t pairs = n_tokens * top_k;
-    const GroupedLayout G = grouped_layout(pairs, n_experts, n, k);
+    const GroupedLayout G = grouped_layout(n_tokens, pairs, n_experts, (wb2 ? 2u : 1u) * n_experts * n, k);
     uint32_t* row_map = reinterpret_cast<uint32_t*>(ws + G.row_map);
     uint4* tiles = reinterpret_cast<uint4*>(ws + G.tiles);
     uint32_t* n_tiles = reinterpret_cast<uint32_t*>(ws + G.count);
@@ -1286,30 +1354,33 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     const uint32_t bm = 32u * (uint32_t)mt, bn = BN_WIDE;
     // sort by expert + one converted activation row per token (the tiles gather the rows of their routed rows from
     // them) + the weight rows' scales, in one launch
-    const BucketArgs b{ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm, HAS_64 && mt == 4 ? 1u : 0u};
+    const BucketArgs b{ids, pairs, n_experts, row_map, tiles, n_tiles, y, n, bm, HAS_64 && mt == 4 && !wb2 ? 1u : 0u};
     const uint32_t n_rows = n_experts * n;
     const uint32_t act_per_wg = grouped_prep_rows_per_wg(k), w_per_wg = 1024u / weight_scan_lanes<TYPE>(k);
     const dim3 prep_grid(1u + (n_tokens + act_per_wg - 1u) / act_per_wg +
-                         (w_scales ? 0u : (n_rows + w_per_wg - 1u) / w_per_wg));  // the weight workgroups come last
+                         (w_scales ? 0u : (wb2 ? 2u : 1u) * ((n_rows + w_per_wg - 1u) / w_per_wg)));  // the weight workgroups come last
     // up to 16384 routed rows: the sort stages its permutation in LDS (two workgroups of this launch still share a CU)
     const uint32_t stage_words = pairs <= BUCKET_STAGE_MAX_PAIRS ? (pairs + 3u) & ~3u : 0u;
-    void (*prep)(BucketArgs, const void*, const uint8_t*, uint8_t*, uint32_t, uint32_t, uint32_t, uint32_t) =
+    void (*prep)(BucketArgs, const void*, const uint8_t*, const uint8_t*, uint8_t*, uint32_t, uint32_t, uint32_t, uint32_t) =
         xdt == HQ_BF16 ? grouped_prep_kernel<true, TYPE> : grouped_prep_kernel<false, TYPE>;
     // (the kernel's static LDS, under 16 KB, counts towards the 64 KB a launch may use without the attribute)
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(prep), stage_words ? (size_t)stage_words * 4 + 16384 : 0,
                                   "hipFuncSetAttribute(grouped pre-pass LDS)"))
         return rc;
-    hipLaunchKernelGGL(prep, prep_grid, dim3(1024), stage_words * 4, s, b, x, wb, ws, n_tokens, n_rows, k, stage_words);
+    hipLaunchKernelGGL(prep, prep_grid, dim3(1024), stage_words * 4, s, b, x, wb, wb2, ws, n_tokens, n_rows, k, stage_words);
     if (int rc = check_launch("grouped gemm pre-pass launch")) return rc;
     const int lds = 2 * (mt == 2 ? ActTileT<BM_SMALL>::kTile : mt == 4 ? ActTileT<BM_MID>::kTile : ActTile::kTile);
     void (*kern)(GemmArgs, const uint4*, const uint32_t*, uint32_t, uint64_t) = grouped_gemm_kernel<TYPE, 8>;
     if (mt == 4) kern = grouped_gemm_kernel<TYPE, 4>;
-    if constexpr (HAS_64)
+    if constexpr (HAS_64) {
         if (mt == 2) kern = grouped_gemm_kernel<TYPE, 2>;
+        if (wb2) kern = mt == 2 ? grouped_gemm_kernel<TYPE, 2, true> : mt == 4 ? grouped_gemm_kernel<TYPE, 4, true> : grouped_gemm_kernel<TYPE, 8, true>;
+    }
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;
-    GemmArgs a{ws, wb, y, pairs, n, k, n_tokens, n_experts * n, 0u, row_map, 0u, (k + 255u) / 256u, top_k,
-               w_scales ? w_scales : reinterpret_cast<const float*>(ws + workspace_layout(n_tokens, n_rows, k).wdown)};
+    const float* ws_scales = reinterpret_cast<const float*>(ws + G.base.wdown);  // the pre-pass's: first stack, then second
+    GemmArgs a{ws, wb, y, pairs, n, k, n_tokens, (wb2 ? 2u : 1u) * n_rows, 0u, row_map, 0u, (k + 255u) / 256u, top_k,
+               w_scales ? w_scales : ws_scales, wb2, wb2 ? (w_scales ? w_scales2 : ws_scales + n_rows) : nullptr};
     const uint32_t tiles_n = (n + bn - 1) / bn;
     const uint32_t max_tiles = pairs / bm + n_experts;
     hipLaunchKernelGGL(kern, dim3(max_tiles * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
@@ -1336,15 +1407,18 @@ int launch_weight_row_scales(hipStream_t s, const void* w, float* scales, uint32
 
 int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_stack, const uint32_t* ids, float* y,
                             void* workspace, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
-                            uint64_t expert_stride, hq_ggml_type t, const float* w_scales) {
+                            uint64_t expert_stride, hq_ggml_type t, const float* w_scales, const void* w_stack2,
+                            const float* w_scales2) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const uint8_t* wb2 = static_cast<const uint8_t*>(w_stack2);
+    if (wb2 && !gemm_f16_grouped_swiglu_supported(t)) return fail(HQ_ERR_UNSUPPORTED, "grouped gemm, SwiGLU form: ggml type %d", (int)t);
     const uint8_t* wb = static_cast<const uint8_t*>(w_stack);
     switch (t) {
-        case HQ_Q4_K: return launch_grouped_t<HQ_Q4_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
-        case HQ_Q5_K: return launch_grouped_t<HQ_Q5_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
-        case HQ_Q6_K: return launch_grouped_t<HQ_Q6_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
-        case HQ_Q8_0: return launch_grouped_t<HQ_Q8_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
-        case HQ_Q4_0: return launch_grouped_t<HQ_Q4_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales);
+        case HQ_Q4_K: return launch_grouped_t<HQ_Q4_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales, wb2, w_scales2);
+        case HQ_Q5_K: return launch_grouped_t<HQ_Q5_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales, wb2, w_scales2);
+        case HQ_Q6_K: return launch_grouped_t<HQ_Q6_K>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales, nullptr, nullptr);
+        case HQ_Q8_0: return launch_grouped_t<HQ_Q8_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales, nullptr, nullptr);
+        case HQ_Q4_0: return launch_grouped_t<HQ_Q4_0>(s, x, xdt, wb, ids, y, ws, n_tokens, top_k, n, k, n_experts, expert_stride, w_scales, nullptr, nullptr);
     }
     return fail(HQ_ERR_UNSUPPORTED, "grouped gemm: ggml type %d", (int)t);
 }

@@ -91,10 +91,15 @@ int launch_weight_row_scales(hipStream_t s, const void* w, float* scales, uint32
 // tile = up to 256 rows of one expert; needs a contiguous stack (expert_stride = n rows) and a device
 // workspace of gemm_f16_grouped_workspace_bytes().
 bool gemm_f16_grouped_supported(hq_ggml_type t, uint32_t n, uint32_t k, uint32_t n_experts, uint64_t expert_stride, uint64_t pairs);
-size_t gemm_f16_grouped_workspace_bytes(uint32_t pairs, uint32_t n_experts, uint32_t n, uint32_t k);
+size_t gemm_f16_grouped_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n_experts, uint32_t n, uint32_t k,
+                                        uint32_t stacks = 1);
+// w_stack2 (Q4_K / Q5_K, see gemm_f16_grouped_swiglu_supported): y = silu(W[ids] . x) * (W2[ids] . x), the gate and up
+// projections of a MoE block and their SwiGLU as one grouped product; workspace for stacks = 2.
+bool gemm_f16_grouped_swiglu_supported(hq_ggml_type t);
 int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_stack, const uint32_t* ids, float* y,
                             void* workspace, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts,
-                            uint64_t expert_stride, hq_ggml_type t, const float* w_scales = nullptr);
+                            uint64_t expert_stride, hq_ggml_type t, const float* w_scales = nullptr,
+                            const void* w_stack2 = nullptr, const float* w_scales2 = nullptr);
 
 // MoE glue (moe.hip)
 int launch_dense_gemv_bf16(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,

@@ -167,6 +167,35 @@ def quantized_matmul_id_ggml(input: torch.Tensor, weight_stack: torch.Tensor, id
                                   params.expert_stride, params.ggml_type))
 
 
+def quantized_matmul_id_swiglu_workspace_bytes(params) -> int:
+    """Device scratch of quantized_matmul_id_swiglu_ggml for this shape; 0 where that form does not exist (the caller
+    then runs gate, up and silu_mul as separate calls)."""
+    return _l.load().hq_qmatmul_id_swiglu_ggml_workspace_bytes(params.n_tokens, params.top_k, params.n, params.k,
+                                                               params.n_experts, params.expert_stride, params.ggml_type)
+
+
+def quantized_matmul_id_swiglu_ggml(input: torch.Tensor, gate_stack: torch.Tensor, up_stack: torch.Tensor, ids: torch.Tensor,
+                                    output: torch.Tensor, params: GgmlQuantizedMatmulIdParams, scratch: torch.Tensor,
+                                    gate_row_scales: torch.Tensor | None = None,
+                                    up_row_scales: torch.Tensor | None = None) -> None:
+    """output[t, s, :] = silu(W_gate[ids[t, s]] . input[t]) * (W_up[ids[t, s]] . input[t]): phases B and D of the MoE
+    block (gpu_ffn.rs:2546-2697) at prefill as one grouped product."""
+    if output.dtype != torch.float32:
+        raise TypeError("output must be float32")
+    if ids.dtype not in (torch.int32, torch.uint32):
+        raise TypeError("ids must be 32-bit")
+    for s_ in (gate_row_scales, up_row_scales):
+        if s_ is not None:
+            _check_scales(s_, params.n_experts * params.n)
+    L = _l.load()
+    _l.check(L.hq_qmatmul_id_swiglu_ggml(
+        _stream(), _dev(input, "input"), _act_dtype(input), _dev(gate_stack, "gate_stack"), _dev(up_stack, "up_stack"),
+        _dev(gate_row_scales, "gate_row_scales") if gate_row_scales is not None else None,
+        _dev(up_row_scales, "up_row_scales") if up_row_scales is not None else None, _dev(ids, "ids"), _dev(output, "output"),
+        _dev(scratch, "scratch"), scratch.numel() * scratch.element_size(), params.n_tokens, params.top_k, params.n, params.k,
+        params.n_experts, params.expert_stride, params.ggml_type))
+
+
 @dataclass
 class QmatmulJob:
     """One product of a batched launch: the arguments of quantized_matmul_id_ggml (ids set) or of

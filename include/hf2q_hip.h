@@ -179,6 +179,24 @@ HQ_API int hq_qmatmul_id_ggml_prepared(void* stream, const void* x, hq_act_dtype
                                 size_t scratch_bytes, uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
                                 uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
 
+/* Gate, up and SwiGLU of a prefill-sized MoE block as one grouped product:
+ *   y[p, :] = silu(W_gate[ids[p]] . x[p / top_k]) * (W_up[ids[p]] . x[p / top_k])       p < n_tokens * top_k
+ * Replaces the two quantized_matmul_id_ggml dispatches of phase B ("gate || up", gpu_ffn.rs:2546, 2623-2683) and the
+ * silu_mul of phase D (gpu_ffn.rs:2685-2697) at prefill: the routed rows are sorted and the activations converted
+ * once, a tile multiplies the same activation rows with the same weight rows of both stacks, and the two f32
+ * products never go to memory.  The result has the bits of hq_qmatmul_id_ggml (grouped form) twice followed by
+ * hq_silu_mul.  Exists where hq_qmatmul_id_swiglu_ggml_workspace_bytes() is not 0: Q4_K / Q5_K on the grouped
+ * route (at least 8 routed rows per expert and 256 rows, contiguous stacks of equal geometry); other calls return
+ * HQ_ERR_UNSUPPORTED and the caller issues the separate calls.  gate_row_scales / up_row_scales: both null, or both
+ * from hq_weight_row_scales_ggml (n_experts * n floats each), see there. */
+HQ_API size_t hq_qmatmul_id_swiglu_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
+                                                 uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
+HQ_API int hq_qmatmul_id_swiglu_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate_stack,
+                              const void* w_up_stack, const float* gate_row_scales, const float* up_row_scales,
+                              const uint32_t* ids, float* y, void* scratch, size_t scratch_bytes, uint32_t n_tokens,
+                              uint32_t top_k, uint32_t n, uint32_t k, uint32_t n_experts, uint64_t expert_stride,
+                              hq_ggml_type t);
+
 /* Bytes of `scratch` the GEMV form needs for up to `max_rows` = n_tokens*top_k
  * routed rows (the IdMmScratch analogue, decode_pool.rs:56-60): always 0.  Kept
  * so that a port of the reference's scratch sizing call has something to call;

@@ -78,6 +78,7 @@ def test_empty_inputs_are_accepted_without_work():
     assert L.hq_qmatmul_ggml_ws_prepared(None, fake, lib.HQ_BF16, fake, fake, fake, 0, 8, 256, lib.HQ_Q6_K, None, 0) == lib.HQ_OK
     assert L.hq_qmatmul_id_ggml_prepared(None, fake, lib.HQ_F32, fake, fake, fake, fake, None, 0, 0, 2, 8, 256, 4, 8 * 144, lib.HQ_Q4_K) == lib.HQ_OK
     assert L.hq_weight_row_scales_ggml(None, fake, fake, 0, 256, lib.HQ_Q4_K) == lib.HQ_OK
+    assert L.hq_qmatmul_id_swiglu_ggml(None, fake, lib.HQ_BF16, fake, fake, None, None, fake, fake, None, 0, 0, 8, 128, 512, 8, 128 * 2 * 144, lib.HQ_Q4_K) == lib.HQ_OK
     assert L.hq_dequant_ggml(None, fake, fake, lib.HQ_F32, 0, lib.HQ_Q8_0) == lib.HQ_OK
     assert L.hq_quantize_ggml(None, fake, 0, 256, lib.HQ_Q5_K, fake) == lib.HQ_OK
     assert L.hq_moe_softmax_topk(None, fake, fake, fake, 0, 256, 8) == lib.HQ_OK
@@ -113,6 +114,13 @@ def test_argument_errors_are_reported_not_fatal():
     assert L.hq_weight_row_scales_ggml(None, fake, fake, 8, 300, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
     assert L.hq_weight_row_scales_ggml(None, fake, fake, 8, 256, 10) == lib.HQ_ERR_UNSUPPORTED
     assert L.hq_weight_row_scales_ggml(None, fake, None, 8, 256, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    # the SwiGLU form of mul_mat_id: both stacks' scales or neither; no form for this shape / type -> unsupported, said so
+    assert L.hq_qmatmul_id_swiglu_ggml(None, fake, lib.HQ_BF16, fake, fake, fake, None, fake, fake, fake, 1 << 20, 64, 4, 128, 512, 8, 128 * 2 * 144, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_qmatmul_id_swiglu_ggml(None, fake, lib.HQ_BF16, fake, None, None, None, fake, fake, fake, 1 << 20, 64, 4, 128, 512, 8, 128 * 2 * 144, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_qmatmul_id_swiglu_ggml(None, fake, lib.HQ_BF16, fake, fake, None, None, fake, fake, fake, 1 << 20, 64, 4, 128, 512, 8, 128 * 2 * 210, lib.HQ_Q6_K) == lib.HQ_ERR_UNSUPPORTED
+    assert L.hq_qmatmul_id_swiglu_ggml_workspace_bytes(64, 4, 128, 512, 8, 128 * 2 * 144, lib.HQ_Q4_K) > L.hq_qmatmul_id_ggml_workspace_bytes(64, 4, 128, 512, 8, 128 * 2 * 144, lib.HQ_Q4_K) > 0
+    assert L.hq_qmatmul_id_swiglu_ggml(None, fake, lib.HQ_BF16, fake, fake, None, None, fake, fake, None, 0, 64, 4, 128, 512, 8, 128 * 2 * 144, lib.HQ_Q4_K) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert "scratch" in lib.last_error()
     # batched form: too many jobs, a prefill-sized dense job, SwiGLU over bf16 activations
     jobs = (lib.QmatmulJob * 5)()
     for j in jobs:

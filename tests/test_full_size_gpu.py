@@ -160,6 +160,41 @@ def test_grouped_mul_mat_id_full_size(oracle, dev, shape):
     assert torch.equal(y, y2)
 
 
+def test_grouped_swiglu_full_size(oracle, dev):
+    """Gate, up and SwiGLU of BASELINE config 3's layer at prefill size (2048 tokens x top-8 over 256 Q4_K experts of
+    512 x 2048) as one grouped product: the bits of the two grouped calls followed by silu_mul, and a sample of routed
+    rows against silu(gate) * up of the f64 oracle."""
+    E, K, T, n, k, t = 256, 8, 2048, 512, 2048, HQ_Q4_K
+    gate, up = _quantized(dev, E * n, k, t, 777), _quantized(dev, E * n, k, t, 778)
+    stride = n * (k // oracle.BLOCK_ELEMS[t]) * oracle.BLOCK_BYTES[t]
+    g = torch.Generator(device=dev)
+    g.manual_seed(42)
+    x = torch.randn(T, k, generator=g, device=dev).to(torch.bfloat16)
+    ids = torch.randint(0, E, (T * K,), generator=g, device=dev, dtype=torch.int32)
+    p = ops.GgmlQuantizedMatmulIdParams(T, K, n, k, E, stride, t)
+    need = ops.quantized_matmul_id_swiglu_workspace_bytes(p)
+    assert need > 0
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    yg, yu, sep = (torch.empty(T * K, n, device=dev) for _ in range(3))
+    ops.quantized_matmul_id_ggml(x, gate, ids, yg, p, scratch=scratch)
+    ops.quantized_matmul_id_ggml(x, up, ids, yu, p, scratch=scratch)
+    ops.dispatch_silu_mul(yg, yu, sep)
+    y = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_swiglu_ggml(x, gate, up, ids, y, p, scratch)
+    assert torch.equal(y, sep)
+    rng = np.random.default_rng(6)
+    ids_h = ids.cpu().numpy()
+    for pair in np.unique(np.concatenate([[0, T * K - 1], rng.integers(0, T * K, 10)])):
+        e = int(ids_h[pair])
+        xs = oracle.f32_to_bf16_bits(x[pair // K:pair // K + 1].float().cpu().numpy())
+        rg = oracle.qmatmul_f64(xs, gate[e * stride:(e + 1) * stride].cpu().numpy(), 1, n, k, t)
+        ru = oracle.qmatmul_f64(xs, up[e * stride:(e + 1) * stride].cpu().numpy(), 1, n, k, t)
+        ref = (rg / (1.0 + np.exp(-rg)) * ru).reshape(-1)
+        got = y[pair].cpu().numpy().astype(np.float64)
+        assert np.sqrt(np.mean((got - ref) ** 2)) <= 1.5e-3 * np.sqrt(np.mean(ref * ref)), pair
+        assert np.abs(got - ref).max() <= 5e-3 * np.abs(ref).max(), pair
+
+
 def test_moe_layer_full_size(oracle, dev):
     """hidden 2048, 256 experts x inter 512 (Q4_K), one shared expert, top-8, one token and eight: the block against
     a float64 evaluation over the device-dequantised weights of the experts the router picked.  The reference here is

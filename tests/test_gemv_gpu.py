@@ -356,6 +356,59 @@ def test_mul_mat_id_grouped_many_rows_and_unaligned_ids(oracle, dev):
     assert torch.equal(y2, y[:T2 * K])
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K])
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("E,n,k,T,K", [(8, 128, 512, 64, 4), (6, 200, 768, 150, 5), (4, 160, 256, 400, 3)])
+def test_mul_mat_id_swiglu_grouped(oracle, dev, t, xdt, E, n, k, T, K):
+    """Gate, up and SwiGLU of a MoE block as one grouped product: the bits of two grouped calls followed by silu_mul
+    (also with the stacks' row scales computed beforehand), and silu(gate) * up of the f64 oracle's two products."""
+    gate, ids, xv, xd, p = _grouped_setup(oracle, dev, t, E, n, k, T, K, xdt, seed=1)
+    up, _, _, _, _ = _grouped_setup(oracle, dev, t, E, n, k, T, K, xdt, seed=2)
+    assert not np.array_equal(gate, up)
+    need = ops.quantized_matmul_id_swiglu_workspace_bytes(p)
+    assert need >= ops.quantized_matmul_id_workspace_bytes(p) > 0
+    gd, ud = torch.from_numpy(gate).to(dev), torch.from_numpy(up).to(dev)
+    idd = torch.from_numpy(ids.view(np.int32)).to(dev)
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    yg, yu = torch.empty(T * K, n, device=dev), torch.empty(T * K, n, device=dev)
+    ops.quantized_matmul_id_ggml(xd, gd, idd, yg, p, scratch=scratch)
+    ops.quantized_matmul_id_ggml(xd, ud, idd, yu, p, scratch=scratch)
+    sep = torch.empty_like(yg)
+    ops.dispatch_silu_mul(yg, yu, sep)
+    scratch.fill_(0xFF)
+    y = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_swiglu_ggml(xd, gd, ud, idd, y, p, scratch)
+    assert torch.equal(y, sep)
+    scratch.fill_(0xFF)
+    y2 = torch.full((T * K, n), float("nan"), device=dev)
+    ops.quantized_matmul_id_swiglu_ggml(xd, gd, ud, idd, y2, p, scratch, ops.weight_row_scales_ggml(gd, E * n, k, t),
+                                        ops.weight_row_scales_ggml(ud, E * n, k, t))
+    assert torch.equal(y2, sep)
+    rg = oracle.qmatmul_id_f64(xv, gate, ids, T, K, n, k, E, p.expert_stride, t)
+    ru = oracle.qmatmul_id_f64(xv, up, ids, T, K, n, k, E, p.expert_stride, t)
+    ref = rg / (1.0 + np.exp(-rg)) * ru
+    got = y.cpu().numpy().astype(np.float64)
+    # silu(g) * u moves by at most |u| (1.1 dg) + |silu(g)| du for errors dg, du of the two products (|silu'| <= 1.1)
+    tg = 1e-3 * np.abs(rg) + 3e-3 * np.sqrt(np.mean(rg * rg))
+    tu = 1e-3 * np.abs(ru) + 3e-3 * np.sqrt(np.mean(ru * ru))
+    bound = 1.1 * np.abs(ru) * tg + np.abs(rg) * tu + tg * tu + 1e-6 * np.abs(ref)
+    assert (np.abs(got - ref) <= bound).all()
+    assert np.sqrt(np.mean((got - ref) ** 2)) <= 1.5e-3 * np.sqrt(np.mean(ref * ref))
+
+
+def test_mul_mat_id_swiglu_has_no_form_for_other_types_and_small_calls(dev):
+    p = GgmlQuantizedMatmulIdParams(64, 4, 128, 512, 8, 128 * ops.ggml_row_bytes(HQ_Q6_K, 512), HQ_Q6_K)
+    assert ops.quantized_matmul_id_workspace_bytes(p) > 0 and ops.quantized_matmul_id_swiglu_workspace_bytes(p) == 0
+    small = GgmlQuantizedMatmulIdParams(8, 2, 128, 512, 8, 128 * ops.ggml_row_bytes(HQ_Q4_K, 512), HQ_Q4_K)
+    assert ops.quantized_matmul_id_swiglu_workspace_bytes(small) == 0
+    x = torch.zeros(8, 512, device=dev)
+    w = torch.zeros(8 * small.expert_stride, dtype=torch.uint8, device=dev)
+    with pytest.raises(ops.HqError) as e:
+        ops.quantized_matmul_id_swiglu_ggml(x, w, w, torch.zeros(16, dtype=torch.int32, device=dev), torch.empty(16, 128, device=dev),
+                                            small, torch.empty(256, dtype=torch.uint8, device=dev))
+    assert e.value.status == 2 and "hq_silu_mul" in str(e.value)
+
+
 def test_mul_mat_id_grouped_routing_properties(oracle, dev):
     """Skewed routing with unused experts, an id that is no expert (NaN rows, the others untouched), agreement with
     the per-row GEMV form, a scratch that is too small, and a strided stack (which keeps the GEMV form)."""
