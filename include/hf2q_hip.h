@@ -204,7 +204,7 @@ HQ_API int hq_qmatmul_id_swiglu_ggml(void* stream, const void* x, hq_act_dtype x
  * grouped (prefill) form needs and 0 where the GEMV form runs. */
 HQ_API size_t hq_qmatmul_id_scratch_bytes(uint32_t n_experts, uint32_t max_rows);
 /* Bytes of `scratch` for this call's shape: 0 where the GEMV form is used, else
- * the grouped form's workspace (sorted f16 activations, row and weight-row
+ * the grouped form's workspace (one f16 row per token, row and weight-row
  * scales, the row permutation and the tile table). */
 HQ_API size_t hq_qmatmul_id_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,
                                           uint32_t n_experts, uint64_t expert_stride, hq_ggml_type t);
