@@ -660,6 +660,8 @@ class MoeFfnScratch:
         # workspace of the grouped (expert-sorted) form that prefill-sized mul_mat_id calls take (IdMmScratch, decode_pool.rs:56-60)
         rb_h, rb_i = ggml_row_bytes(w.ggml_type, w.hidden), ggml_row_bytes(w.ggml_type, w.inter)
         need = max(
+            quantized_matmul_id_swiglu_workspace_bytes(GgmlQuantizedMatmulIdParams(T, K, w.inter, w.hidden, w.n_experts,
+                                                                                   w.inter * rb_h, w.ggml_type)),
             quantized_matmul_id_workspace_bytes(GgmlQuantizedMatmulIdParams(T, K, w.inter, w.hidden, w.n_experts,
                                                                             w.inter * rb_h, w.ggml_type)),
             quantized_matmul_id_workspace_bytes(GgmlQuantizedMatmulIdParams(T * K, 1, w.hidden, w.inter, w.n_experts,
@@ -759,14 +761,18 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
     # B
     dispatch_moe_softmax_topk(s.logits, s.ids, s.topk_w, T, E, K)
     dispatch_silu_mul(s.sh_gate[:T], s.sh_up[:T], s.sh_act[:T])
-    # C
+    # C, D
     pid = GgmlQuantizedMatmulIdParams(T, K, I, H, E, I * rb, t)
     ws = s.id_mm  # sized for max_tokens; fewer tokens need less (or none: decode-sized calls take the GEMV form)
-    quantized_matmul_id_ggml(x, w.expert_gate, s.ids, s.gate, pid, scratch=ws)
-    quantized_matmul_id_ggml(x, w.expert_up, s.ids, s.up, pid, scratch=ws)
-    quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, GgmlQuantizedMatmulParams(T, H, SI, t))
-    # D
-    dispatch_silu_mul(s.gate[:T * K], s.up[:T * K], s.act[:T * K])
+    if ws is not None and quantized_matmul_id_swiglu_workspace_bytes(pid):
+        # a prefill chunk of Q4_K / Q5_K experts: gate, up and their SwiGLU as one grouped product (the same bits)
+        quantized_matmul_id_swiglu_ggml(x, w.expert_gate, w.expert_up, s.ids, s.act, pid, ws)
+        quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, GgmlQuantizedMatmulParams(T, H, SI, t))
+    else:
+        quantized_matmul_id_ggml(x, w.expert_gate, s.ids, s.gate, pid, scratch=ws)
+        quantized_matmul_id_ggml(x, w.expert_up, s.ids, s.up, pid, scratch=ws)
+        quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, GgmlQuantizedMatmulParams(T, H, SI, t))
+        dispatch_silu_mul(s.gate[:T * K], s.up[:T * K], s.act[:T * K])
     # E
     quantized_matmul_id_ggml(s.act, w.expert_down, s.ids, s.down,
                              GgmlQuantizedMatmulIdParams(T * K, 1, H, I, E, H * ggml_row_bytes(t, I), t), scratch=ws)

@@ -76,6 +76,29 @@ def test_dense_gemv_bf16(oracle, dev):
         assert np.abs(y.cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("m,n,k", [(2048, 256, 2048), (100, 70, 528), (33, 1, 2048), (32, 33, 16)])
+def test_dense_bf16_product_of_many_rows(oracle, dev, m, n, k):
+    """The router of a prefill chunk: many bf16 activation rows take the matrix-core form (exact products, f32 sums),
+    edges in every dimension; the pair form gives the same bits as two calls; f32 activations keep the GEMV form."""
+    w = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(weights(3 + n, n, k, 0.05)))
+    xb = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(acts(4 + m, m, k)))
+    wd = torch.from_numpy(w).to(dev).to(torch.bfloat16)
+    xd = torch.from_numpy(xb).to(dev).to(torch.bfloat16)
+    y = torch.full((m, n), float("nan"), device=dev)
+    ops.dense_gemv_bf16_f32(xd, wd, y, m, n, k)
+    ref = xb.astype(np.float64) @ w.astype(np.float64).T
+    assert np.abs(y.cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
+    yf = torch.empty(m, n, device=dev)
+    ops.dense_gemv_bf16_f32(torch.from_numpy(xb).to(dev), wd, yf, m, n, k)  # the same values as f32: one wave per output
+    assert (y - yf).abs().max().item() <= 2e-5 * np.abs(ref).max()
+    w2 = torch.from_numpy(oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(weights(9, 1, k, 0.05)))).to(dev).to(torch.bfloat16)
+    ya, yb = torch.empty(m, n, device=dev), torch.empty(m, 1, device=dev)
+    ops.dense_gemv_bf16_f32_pair(xd, wd, ya, n, w2, yb, 1, m, k)
+    y1 = torch.empty(m, 1, device=dev)
+    ops.dense_gemv_bf16_f32(xd, w2, y1, m, 1, k)
+    assert torch.equal(ya, y) and torch.equal(yb, y1)
+
+
 @pytest.mark.parametrize("T", [1, 8])
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0])
 def test_moe_block_matches_cpu_spec(oracle, dev, T, t):
