@@ -282,6 +282,35 @@ int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w
     return rc ? rc : rc_free;
 }
 
+size_t hq_qmatmul_swiglu_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
+    (void)xdt;
+    if (hq_block_elems(t) == 0 || n == 0 || k == 0 || k % hq_block_elems(t)) return 0;
+    return (t == HQ_Q4_K || t == HQ_Q5_K) && f16_tile_route(m, k, t) ? gemm_f16_swiglu_workspace_bytes(m, n, k) : 0;
+}
+
+int hq_qmatmul_swiglu_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up,
+                              const float* gate_row_scales, const float* up_row_scales, float* y, uint32_t m, uint32_t n,
+                              uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes) {
+    const char* fn = "hq_qmatmul_swiglu_ggml_ws";
+    if (int rc = check_matmul_common(fn, x, xdt, w_gate, y, n, k, t)) return rc;
+    if (!w_up) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (int rc = check_weight_alignment(w_up, t)) return rc;
+    if ((gate_row_scales == nullptr) != (up_row_scales == nullptr))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: the row scales of both matrices, or of neither", fn);
+    if (gate_row_scales && (!is_aligned(gate_row_scales, 4) || !is_aligned(up_row_scales, 4)))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: row scales must be 4-byte aligned", fn);
+    if (m == 0) return HQ_OK;
+    const size_t need = hq_qmatmul_swiglu_ggml_workspace_bytes(m, n, k, xdt, t);
+    if (!need)
+        return fail(HQ_ERR_UNSUPPORTED,
+                    "%s: this shape or type has no SwiGLU tile form (hq_qmatmul_swiglu_ggml_workspace_bytes is 0): two "
+                    "hq_qmatmul_ggml calls and hq_silu_mul give the same result", fn);
+    if (!workspace || workspace_bytes < need)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes, %zu needed", fn, workspace ? workspace_bytes : (size_t)0, need);
+    if (reinterpret_cast<uintptr_t>(workspace) % 256) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace must be 256-byte aligned", fn);
+    return launch_gemm_f16_swiglu((hipStream_t)stream, x, xdt, w_gate, w_up, y, m, n, k, t, workspace, gate_row_scales, up_row_scales);
+}
+
 size_t hq_qmatmul_perm021_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
     // the tile GEMM gathers while it converts; every other route first copies the activations into row-major order
     if (f16_tile_route(m, k, t)) return gemm_f16_tile_workspace_bytes(m, n, k, t);

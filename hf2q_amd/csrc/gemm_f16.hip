@@ -266,13 +266,17 @@ __device__ __forceinline__ void prep_activation_row(const void* __restrict__ x, 
 // epilogue divides it out.
 template <bool X_BF16, int TYPE>
 __global__ __launch_bounds__(256) void tile_prep_kernel(const void* __restrict__ x, const uint8_t* __restrict__ w,
-                                                        uint8_t* __restrict__ ws, uint32_t m, uint32_t n, uint32_t k,
-                                                        uint32_t perm_hd, uint32_t scan_wgs) {
+                                                        const uint8_t* __restrict__ w2, uint8_t* __restrict__ ws, uint32_t m,
+                                                        uint32_t n, uint32_t k, uint32_t perm_hd, uint32_t scan_wgs) {
     __shared__ float red[4];
-    const Workspace L = workspace_layout(m, n, k);
+    // (w2: a second matrix of n rows -- the SwiGLU form -- scanned by the second half of the scan workgroups; its scales
+    // follow the first matrix's)
+    const Workspace L = workspace_layout(m, w2 ? 2u * n : n, k);
     if (blockIdx.x < scan_wgs) {
         const uint32_t lanes = weight_scan_lanes<TYPE>(k);
-        prep_weight_rows<TYPE>(w, reinterpret_cast<float*>(ws + L.wdown), n, k, blockIdx.x * (256u / lanes), threadIdx.x, lanes);
+        const uint32_t per_matrix = w2 ? scan_wgs / 2u : scan_wgs, second = blockIdx.x >= per_matrix ? 1u : 0u;
+        prep_weight_rows<TYPE>(second ? w2 : w, reinterpret_cast<float*>(ws + L.wdown) + second * n, n, k,
+                               (blockIdx.x - second * per_matrix) * (256u / lanes), threadIdx.x, lanes);
     } else
         prep_activation_row<X_BF16>(x, ws, L, m, k, perm_hd, blockIdx.x - scan_wgs, threadIdx.x, red);
 }
@@ -1033,6 +1037,16 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q4k_gemm_small_kernel(GemmArgs 
     q4k_gemm_tile<MTS, 1, 4, TYPE>(a, (t / tiles_n) * BMS, (t % tiles_n) * BN_WIDE);
 }
 
+// y = silu(x . Wg^T) * (x . Wu^T) for Q4_K / Q5_K: one workgroup per (tile of 32 * MTS token rows, 128 output columns), a
+// wave the same 32 weight rows of both matrices (see q4k_gemm_tile's SWIGLU form).  No slices of k: the result is not
+// linear in the partial products.
+template <int TYPE, int MTS>
+__global__ __launch_bounds__(64 * WAVES, 2) void q4k_swiglu_kernel(GemmArgs a) {
+    constexpr uint32_t BMS = 32 * MTS;
+    const uint32_t tiles_n = (a.n + BN_WIDE - 1) / BN_WIDE;
+    q4k_gemm_tile<MTS, 2, 4, TYPE, false, true>(a, (blockIdx.x / tiles_n) * BMS, (blockIdx.x % tiles_n) * BN_WIDE);
+}
+
 // y[i] = partial[0][i] + partial[1][i] + ... in this order, whatever order the slices were written in.
 __global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict__ partial, float* __restrict__ y, uint32_t count,
                                                         uint32_t splits) {
@@ -1325,14 +1339,14 @@ bool gemm_f16_grouped_swiglu_supported(hq_ggml_type t) { return t == HQ_Q4_K || 
 
 template <int TYPE>
 static int launch_prep(hipStream_t s, const void* x, hq_act_dtype xdt, const uint8_t* wb, uint8_t* ws, uint32_t m,
-                       uint32_t n, uint32_t k, uint32_t perm_hd, bool scan_weights) {
+                       uint32_t n, uint32_t k, uint32_t perm_hd, bool scan_weights, const uint8_t* wb2 = nullptr) {
     const uint32_t rows_per_wg = 256u / weight_scan_lanes<TYPE>(k);
-    const uint32_t scan_wgs = scan_weights ? (n + rows_per_wg - 1u) / rows_per_wg : 0u;
+    const uint32_t scan_wgs = scan_weights ? (wb2 ? 2u : 1u) * ((n + rows_per_wg - 1u) / rows_per_wg) : 0u;
     const dim3 prep_grid(scan_wgs + m);
     if (xdt == HQ_BF16)
-        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd, scan_wgs);
+        hipLaunchKernelGGL((tile_prep_kernel<true, TYPE>), prep_grid, dim3(256), 0, s, x, wb, wb2, ws, m, n, k, perm_hd, scan_wgs);
     else
-        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, ws, m, n, k, perm_hd, scan_wgs);
+        hipLaunchKernelGGL((tile_prep_kernel<false, TYPE>), prep_grid, dim3(256), 0, s, x, wb, wb2, ws, m, n, k, perm_hd, scan_wgs);
     return check_launch("tile gemm pre-pass launch");
 }
 
@@ -1425,6 +1439,35 @@ int launch_gemm_f16_grouped(hipStream_t s, const void* x, hq_act_dtype xdt, cons
 
 bool gemm_f16_tile_supported(hq_ggml_type t, uint32_t k) {
     return ((t == HQ_Q4_K || t == HQ_Q5_K || t == HQ_Q6_K) && k % 256 == 0) || ((t == HQ_Q8_0 || t == HQ_Q4_0) && k % 128 == 0);
+}
+
+size_t gemm_f16_swiglu_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) { return workspace_layout(m, 2u * n, k).total; }
+
+// y[m, n] = silu(x . Wg^T) * (x . Wu^T), Q4_K / Q5_K, k % 256 == 0: the activation pre-pass once (with both matrices'
+// row scales unless the caller brings them) and one launch of tiles that multiply the same activation rows with both
+// matrices.  Tiles of 64 token rows while those leave CUs idle, of 128 beyond.
+int launch_gemm_f16_swiglu(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up, float* y, uint32_t m,
+                           uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, const float* gate_scales, const float* up_scales) {
+    if (t != HQ_Q4_K && t != HQ_Q5_K) return fail(HQ_ERR_UNSUPPORTED, "tile gemm, SwiGLU form: ggml type %d", (int)t);
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const uint8_t *wg = static_cast<const uint8_t*>(w_gate), *wu = static_cast<const uint8_t*>(w_up);
+    if (int rc = t == HQ_Q5_K ? launch_prep<HQ_Q5_K>(s, x, xdt, wg, ws, m, n, k, 0, !gate_scales, wu)
+                              : launch_prep<HQ_Q4_K>(s, x, xdt, wg, ws, m, n, k, 0, !gate_scales, wu))
+        return rc;
+    const float* ws_scales = reinterpret_cast<const float*>(ws + workspace_layout(m, 2u * n, k).wdown);
+    GemmArgs a{ws, wg, y, m, n, k, m, 2u * n, 0u, nullptr, 0u, (k + 255u) / 256u, 0u,
+               gate_scales ? gate_scales : ws_scales, wu, gate_scales ? up_scales : ws_scales + n};
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
+    const uint32_t tiles_n = (n + BN_WIDE - 1) / BN_WIDE;
+    const bool small = (uint64_t)((m + BM_MID - 1) / BM_MID) * tiles_n < cus;
+    void (*kern)(GemmArgs) = t == HQ_Q5_K ? (small ? q4k_swiglu_kernel<HQ_Q5_K, 2> : q4k_swiglu_kernel<HQ_Q5_K, 4>)
+                                          : (small ? q4k_swiglu_kernel<HQ_Q4_K, 2> : q4k_swiglu_kernel<HQ_Q4_K, 4>);
+    const uint32_t bm = small ? BM_SMALL : BM_MID;
+    const int lds = 2 * (small ? ActTileT<BM_SMALL>::kTile : ActTileT<BM_MID>::kTile);
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(swiglu gemm LDS)")) return rc;
+    hipLaunchKernelGGL(kern, dim3(((m + bm - 1) / bm) * tiles_n), dim3(64 * WAVES), lds, s, a);
+    return check_launch("swiglu gemm kernel launch");
 }
 
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,

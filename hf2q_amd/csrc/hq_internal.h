@@ -87,6 +87,12 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
 // or grouped call works out when w_scales is null.
 int launch_weight_row_scales(hipStream_t s, const void* w, float* scales, uint32_t n_rows, uint32_t k, hq_ggml_type t);
 
+// y = silu(x . Wg^T) * (x . Wu^T) on the tile route (Q4_K / Q5_K, k % 256 == 0): both products of a dense SwiGLU
+// layer and the gating as one launch after the pre-pass; gate_scales / up_scales: both null, or both the caller's.
+size_t gemm_f16_swiglu_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+int launch_gemm_f16_swiglu(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up, float* y, uint32_t m,
+                           uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, const float* gate_scales, const float* up_scales);
+
 // Grouped form of the tile GEMM for mul_mat_id with many routed rows: rows sorted by expert, one
 // tile = up to 256 rows of one expert; needs a contiguous stack (expert_stride = n rows) and a device
 // workspace of gemm_f16_grouped_workspace_bytes().

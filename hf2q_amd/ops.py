@@ -117,6 +117,29 @@ def quantized_matmul_workspace_bytes(params: GgmlQuantizedMatmulParams, act_dtyp
     return int(L.hq_qmatmul_ggml_workspace_bytes(params.m, params.n, params.k, xdt, params.ggml_type))
 
 
+def quantized_matmul_swiglu_workspace_bytes(params: GgmlQuantizedMatmulParams, act_dtype: torch.dtype) -> int:
+    """Device scratch of quantized_matmul_swiglu_ggml for this shape; 0 where that form does not exist."""
+    xdt = _l.HQ_BF16 if act_dtype == torch.bfloat16 else _l.HQ_F32
+    return int(_l.load().hq_qmatmul_swiglu_ggml_workspace_bytes(params.m, params.n, params.k, xdt, params.ggml_type))
+
+
+def quantized_matmul_swiglu_ggml(input: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, dst: torch.Tensor,
+                                 params: GgmlQuantizedMatmulParams, workspace: torch.Tensor,
+                                 gate_row_scales: torch.Tensor | None = None, up_row_scales: torch.Tensor | None = None) -> None:
+    """dst[m, n] = silu(input . gate^T) * (input . up^T): the two products of a dense SwiGLU layer (or of the MoE
+    block's shared expert) and the gating at prefill as one call, the bits of the three separate ones."""
+    if dst.dtype != torch.float32:
+        raise TypeError("dst must be float32")
+    for s_ in (gate_row_scales, up_row_scales):
+        if s_ is not None:
+            _check_scales(s_, params.n)
+    _l.check(_l.load().hq_qmatmul_swiglu_ggml_ws(
+        _stream(), _dev(input, "input"), _act_dtype(input), _dev(gate, "gate"), _dev(up, "up"),
+        _dev(gate_row_scales, "gate_row_scales") if gate_row_scales is not None else None,
+        _dev(up_row_scales, "up_row_scales") if up_row_scales is not None else None, _dev(dst, "dst"), params.m, params.n,
+        params.k, params.ggml_type, _dev(workspace, "workspace"), workspace.numel() * workspace.element_size()))
+
+
 @dataclass
 class GgmlQuantizedMatmulPerm021Params:
     """forward_prefill_batched.rs:2219-2226."""
@@ -667,6 +690,12 @@ class MoeFfnScratch:
             quantized_matmul_id_workspace_bytes(GgmlQuantizedMatmulIdParams(T * K, 1, w.hidden, w.inter, w.n_experts,
                                                                             w.hidden * rb_i, w.ggml_type)))
         self.id_mm = torch.empty(need, dtype=torch.uint8, device=device) if need else None
+        # workspace of the shared expert's prefill-sized dense products (the SwiGLU form where it exists, and the down product)
+        pg = GgmlQuantizedMatmulParams(T, w.shared_inter, w.hidden, w.ggml_type)
+        pd = GgmlQuantizedMatmulParams(T, w.hidden, w.shared_inter, w.ggml_type)
+        need = max(quantized_matmul_swiglu_workspace_bytes(pg, torch.bfloat16), quantized_matmul_workspace_bytes(pg, torch.bfloat16),
+                   quantized_matmul_workspace_bytes(pd, torch.float32))
+        self.dense_ws = torch.empty(need, dtype=torch.uint8, device=device) if need else None
         self.max_tokens = T
         # scratch of the one-launch decode block (hq_moe_ffn_decode): zeroed once, then the library's
         fb = _l.load().hq_moe_ffn_decode_scratch_bytes(min(T, 8), w.hidden, w.n_experts, K, w.inter, w.shared_inter, w.ggml_type,
@@ -756,11 +785,19 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
     # A
     dense_gemv_bf16_f32(x, w.router, s.logits, T, E, H)
     dense_gemv_bf16_f32(x, w.shared_gate_logit, s.sh_logit, T, 1, H)
-    quantized_matmul_ggml(x, w.shared_gate, s.sh_gate, GgmlQuantizedMatmulParams(T, SI, H, t))
-    quantized_matmul_ggml(x, w.shared_up, s.sh_up, GgmlQuantizedMatmulParams(T, SI, H, t))
+    psh = GgmlQuantizedMatmulParams(T, SI, H, t)
+    dws = s.dense_ws if T <= s.max_tokens else None  # sized for max_tokens: enough for any fewer
+    shared_one_call = dws is not None and quantized_matmul_swiglu_workspace_bytes(psh, x.dtype) > 0
+    if shared_one_call:
+        # a prefill chunk, Q4_K / Q5_K: the shared expert's gate, up and SwiGLU as one call (the same bits)
+        quantized_matmul_swiglu_ggml(x, w.shared_gate, w.shared_up, s.sh_act, psh, dws)
+    else:
+        quantized_matmul_ggml(x, w.shared_gate, s.sh_gate, psh)
+        quantized_matmul_ggml(x, w.shared_up, s.sh_up, psh)
     # B
     dispatch_moe_softmax_topk(s.logits, s.ids, s.topk_w, T, E, K)
-    dispatch_silu_mul(s.sh_gate[:T], s.sh_up[:T], s.sh_act[:T])
+    if not shared_one_call:
+        dispatch_silu_mul(s.sh_gate[:T], s.sh_up[:T], s.sh_act[:T])
     # C, D
     pid = GgmlQuantizedMatmulIdParams(T, K, I, H, E, I * rb, t)
     ws = s.id_mm  # sized for max_tokens; fewer tokens need less (or none: decode-sized calls take the GEMV form)

@@ -124,6 +124,22 @@ HQ_API int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, con
                        uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, void* workspace,
                        size_t workspace_bytes);
 
+/* The gate and up products of a dense SwiGLU layer and the gating as one call on the prefill route:
+ *   y[m, n] = silu(x . W_gate^T) * (x . W_up^T)
+ * Replaces the two quantized_matmul_ggml dispatches and the silu_mul between them that the dense FFN and the shared
+ * expert of the MoE block encode at prefill (gpu_ffn.rs:1236-1306, 2485-2545): one activation pre-pass, one launch of
+ * tiles of 64 or 128 token rows that multiply the same activation rows with the same weight rows of both matrices;
+ * the two f32 products never go to memory.  Exists where hq_qmatmul_swiglu_ggml_workspace_bytes() is not 0 (Q4_K /
+ * Q5_K on the tile route: more rows than the small-batch kernels take, k % 256 == 0); other calls return
+ * HQ_ERR_UNSUPPORTED and the caller issues the separate calls.  The separate calls run 256-row tiles from 257 rows
+ * on, which use the matrix cores better: this form pays for few weight rows (the shared expert: 512) or few tokens,
+ * not for a 12288-row layer over thousands of tokens.  gate_row_scales / up_row_scales: both null, or both from
+ * hq_weight_row_scales_ggml (n floats each). */
+HQ_API size_t hq_qmatmul_swiglu_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t);
+HQ_API int hq_qmatmul_swiglu_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up,
+                              const float* gate_row_scales, const float* up_row_scales, float* y, uint32_t m, uint32_t n,
+                              uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes);
+
 /* y[m, n] = sum_k x[m, k] * W[n, k] with the activations stored heads-outermost, [k / head_dim][m][head_dim]
  * (the attention output of a batched prefill): element (row, kk) sits at ((kk / head_dim) * m + row) * head_dim +
  * kk % head_dim.  Replaces quantized_matmul_mm_tensor_perm021(enc, reg, dev, input, weight, dst,

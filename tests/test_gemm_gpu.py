@@ -138,6 +138,61 @@ def test_q4k_tile_gemm_workspace_variant(oracle, dev):
         ops.quantized_matmul_ggml(x, wd, y1, p, workspace=ws[: need - 256])
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K])
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("m,n,k", [(48, 160, 512), (300, 257, 768), (2048, 512, 2048), (130, 128, 256)])
+def test_dense_swiglu_tile_form(oracle, dev, t, xdt, m, n, k):
+    """silu(x . Wg^T) * (x . Wu^T) as one call: the bits of the two tile products followed by silu_mul (also with the
+    row scales of both matrices computed beforehand), and silu(gate) * up of the f64 oracle's products."""
+    from hf2q_amd import lib
+    gate = oracle.quantize(weights(41 * n + k + t, n, k), k, t, threads=8)
+    up = oracle.quantize(weights(43 * n + k + t, n, k), k, t, threads=8)
+    x = acts(n + k + m, m, k)
+    if xdt == "bf16":
+        xv = oracle.f32_to_bf16_bits(x)
+        xd = torch.from_numpy(xv.view(np.int16)).to(dev).view(torch.bfloat16).reshape(m, k)
+    else:
+        xv, xd = x, torch.from_numpy(x).to(dev)
+    gd, ud = torch.from_numpy(gate).to(dev), torch.from_numpy(up).to(dev)
+    p = GgmlQuantizedMatmulParams(m, n, k, t)
+    adt = torch.bfloat16 if xdt == "bf16" else torch.float32
+    need = ops.quantized_matmul_swiglu_workspace_bytes(p, adt)
+    assert need >= ops.quantized_matmul_workspace_bytes(p, adt) > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    yg, yu, sep = (torch.empty(m, n, device=dev) for _ in range(3))
+    ops.quantized_matmul_ggml(xd, gd, yg, p, workspace=ws)
+    ops.quantized_matmul_ggml(xd, ud, yu, p, workspace=ws)
+    ops.dispatch_silu_mul(yg.view(-1)[: m * n - (m * n) % 4], yu.view(-1)[: m * n - (m * n) % 4], sep.view(-1)[: m * n - (m * n) % 4])
+    ws.fill_(0xFF)
+    y = torch.full((m, n), float("nan"), device=dev)
+    ops.quantized_matmul_swiglu_ggml(xd, gd, ud, y, p, ws)
+    cut = m * n - (m * n) % 4
+    assert torch.equal(y.view(-1)[:cut], sep.view(-1)[:cut])
+    ws.fill_(0xFF)
+    y2 = torch.full((m, n), float("nan"), device=dev)
+    ops.quantized_matmul_swiglu_ggml(xd, gd, ud, y2, p, ws, ops.weight_row_scales_ggml(gd, n, k, t), ops.weight_row_scales_ggml(ud, n, k, t))
+    assert torch.equal(y2, y)
+    rg, ru = oracle.qmatmul_f64(xv, gate, m, n, k, t), oracle.qmatmul_f64(xv, up, m, n, k, t)
+    ref = rg / (1.0 + np.exp(-rg)) * ru
+    got = y.cpu().numpy().astype(np.float64)
+    assert np.isfinite(got).all()
+    assert np.sqrt(np.mean((got - ref) ** 2)) <= 1.5e-3 * np.sqrt(np.mean(ref * ref))
+    assert np.abs(got - ref).max() <= 5e-3 * np.abs(ref).max()
+    with pytest.raises(lib.HqError):
+        ops.quantized_matmul_swiglu_ggml(xd, gd, ud, y, p, ws[: need - 256])
+
+
+def test_dense_swiglu_has_no_form_for_other_types_and_few_rows(dev):
+    assert ops.quantized_matmul_swiglu_workspace_bytes(GgmlQuantizedMatmulParams(64, 128, 512, HQ_Q6_K), torch.bfloat16) == 0
+    assert ops.quantized_matmul_swiglu_workspace_bytes(GgmlQuantizedMatmulParams(4, 128, 512, HQ_Q4_K), torch.bfloat16) == 0
+    x = torch.zeros(4, 512, device=dev)
+    w = torch.zeros(128 * 2 * 144, dtype=torch.uint8, device=dev)
+    with pytest.raises(ops.HqError) as e:
+        ops.quantized_matmul_swiglu_ggml(x, w, w, torch.empty(4, 128, device=dev), GgmlQuantizedMatmulParams(4, 128, 512, HQ_Q4_K),
+                                         torch.empty(256, dtype=torch.uint8, device=dev))
+    assert e.value.status == 2
+
+
 def _row_bounds(blocks, n, k, t):
     """Largest possible |w| of every weight row from its block headers alone, in f64."""
     per, nbytes, d_at = {HQ_Q4_K: (256, 144, 0), HQ_Q5_K: (256, 176, 0), HQ_Q6_K: (256, 210, 208), HQ_Q8_0: (32, 34, 0),
