@@ -1364,7 +1364,8 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     // expert on average, tiles of 128 routed rows: the 256-row tiles would run a quarter full, and half of the experts
     // would need two 64-row tiles); at 40 rows per expert or fewer the Q4_K / Q5_K tiles of 64 rows.
     constexpr bool HAS_64 = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K;
-    const int mt = HAS_64 && (uint64_t)pairs <= (uint64_t)n_experts * 40u ? 2 : (uint64_t)pairs < (uint64_t)n_experts * 160u ? 4 : 8;
+    // (the SwiGLU form keeps two accumulator tiles per row tile: 128 rows is the most a wave's registers hold)
+    const int mt = HAS_64 && (uint64_t)pairs <= (uint64_t)n_experts * 40u ? 2 : (uint64_t)pairs < (uint64_t)n_experts * 160u || wb2 ? 4 : 8;
     const uint32_t bm = 32u * (uint32_t)mt, bn = BN_WIDE;
     // sort by expert + one converted activation row per token (the tiles gather the rows of their routed rows from
     // them) + the weight rows' scales, in one launch
@@ -1388,7 +1389,7 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     if (mt == 4) kern = grouped_gemm_kernel<TYPE, 4>;
     if constexpr (HAS_64) {
         if (mt == 2) kern = grouped_gemm_kernel<TYPE, 2>;
-        if (wb2) kern = mt == 2 ? grouped_gemm_kernel<TYPE, 2, true> : mt == 4 ? grouped_gemm_kernel<TYPE, 4, true> : grouped_gemm_kernel<TYPE, 8, true>;
+        if (wb2) kern = mt == 2 ? grouped_gemm_kernel<TYPE, 2, true> : grouped_gemm_kernel<TYPE, 4, true>;
     }
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;

@@ -664,6 +664,23 @@ class MoeFfnWeightsGpuQ:
     top_k: int
     inter: int
     shared_inter: int
+    # the tile kernels' weight-row scales of the six quantized matrices, filled by prepare_prefill() (optional)
+    row_scales: dict | None = None
+
+    def prepare_prefill(self) -> None:
+        """Once after the weights are uploaded: the row scales that prefill-sized calls would otherwise work out again in
+        every pre-pass (4 bytes per weight row; they depend on the weights alone, so the results do not change)."""
+        t, H, E, I, SI = self.ggml_type, self.hidden, self.n_experts, self.inter, self.shared_inter
+        if t not in (HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0):
+            return
+        self.row_scales = {
+            "expert_gate": weight_row_scales_ggml(self.expert_gate, E * I, H, t),
+            "expert_up": weight_row_scales_ggml(self.expert_up, E * I, H, t),
+            "expert_down": weight_row_scales_ggml(self.expert_down, E * H, I, t),
+            "shared_gate": weight_row_scales_ggml(self.shared_gate, SI, H, t),
+            "shared_up": weight_row_scales_ggml(self.shared_up, SI, H, t),
+            "shared_down": weight_row_scales_ggml(self.shared_down, H, SI, t),
+        }
 
 
 class MoeFfnScratch:
@@ -788,9 +805,10 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
     psh = GgmlQuantizedMatmulParams(T, SI, H, t)
     dws = s.dense_ws if T <= s.max_tokens else None  # sized for max_tokens: enough for any fewer
     shared_one_call = dws is not None and quantized_matmul_swiglu_workspace_bytes(psh, x.dtype) > 0
+    rsc = w.row_scales or {}  # kept from load time (prepare_prefill), or worked out by every call's pre-pass
     if shared_one_call:
         # a prefill chunk, Q4_K / Q5_K: the shared expert's gate, up and SwiGLU as one call (the same bits)
-        quantized_matmul_swiglu_ggml(x, w.shared_gate, w.shared_up, s.sh_act, psh, dws)
+        quantized_matmul_swiglu_ggml(x, w.shared_gate, w.shared_up, s.sh_act, psh, dws, rsc.get("shared_gate"), rsc.get("shared_up"))
     else:
         quantized_matmul_ggml(x, w.shared_gate, s.sh_gate, psh)
         quantized_matmul_ggml(x, w.shared_up, s.sh_up, psh)
@@ -803,16 +821,21 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
     ws = s.id_mm  # sized for max_tokens; fewer tokens need less (or none: decode-sized calls take the GEMV form)
     if ws is not None and quantized_matmul_id_swiglu_workspace_bytes(pid):
         # a prefill chunk of Q4_K / Q5_K experts: gate, up and their SwiGLU as one grouped product (the same bits)
-        quantized_matmul_id_swiglu_ggml(x, w.expert_gate, w.expert_up, s.ids, s.act, pid, ws)
-        quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, GgmlQuantizedMatmulParams(T, H, SI, t))
+        quantized_matmul_id_swiglu_ggml(x, w.expert_gate, w.expert_up, s.ids, s.act, pid, ws, rsc.get("expert_gate"),
+                                        rsc.get("expert_up"))
     else:
-        quantized_matmul_id_ggml(x, w.expert_gate, s.ids, s.gate, pid, scratch=ws)
-        quantized_matmul_id_ggml(x, w.expert_up, s.ids, s.up, pid, scratch=ws)
-        quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, GgmlQuantizedMatmulParams(T, H, SI, t))
+        quantized_matmul_id_ggml(x, w.expert_gate, s.ids, s.gate, pid, scratch=ws, w_row_scales=rsc.get("expert_gate"))
+        quantized_matmul_id_ggml(x, w.expert_up, s.ids, s.up, pid, scratch=ws, w_row_scales=rsc.get("expert_up"))
         dispatch_silu_mul(s.gate[:T * K], s.up[:T * K], s.act[:T * K])
+    pdn = GgmlQuantizedMatmulParams(T, H, SI, t)
+    if dws is not None and quantized_matmul_workspace_bytes(pdn, torch.float32):
+        quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, pdn, workspace=dws, w_row_scales=rsc.get("shared_down"))
+    else:
+        quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, pdn)
     # E
     quantized_matmul_id_ggml(s.act, w.expert_down, s.ids, s.down,
-                             GgmlQuantizedMatmulIdParams(T * K, 1, H, I, E, H * ggml_row_bytes(t, I), t), scratch=ws)
+                             GgmlQuantizedMatmulIdParams(T * K, 1, H, I, E, H * ggml_row_bytes(t, I), t), scratch=ws,
+                             w_row_scales=rsc.get("expert_down"))
     # F
     dispatch_moe_weighted_reduce(s.down, s.topk_w, out, T, K, H, shared=s.sh_down, shared_logit=s.sh_logit,
                                  residual=residual)

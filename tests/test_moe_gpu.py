@@ -164,6 +164,16 @@ def test_moe_block_prefill_sized_matches_cpu_spec(oracle, dev, t):
     out12 = torch.full((12, H), float("nan"), device=dev)
     ops.build_moe_ffn_layer_gpu_q_into(dv(x[:12]), w, s, out12)
     assert np.abs(out12.cpu().numpy() - want[:12]).max() <= 2e-3 * scale
+    # the weight-row scales kept from load time: the same bits, for bf16 activations too
+    xb = dv(x).to(torch.bfloat16)
+    plain = torch.empty_like(out)
+    ops.build_moe_ffn_layer_gpu_q_into(xb, w, s, plain)
+    w.prepare_prefill()
+    assert w.row_scales is not None and len(w.row_scales) == 6
+    for xin, ref in ((dv(x), out), (xb, plain)):
+        kept = torch.full((T, H), float("nan"), device=dev)
+        ops.build_moe_ffn_layer_gpu_q_into(xin, w, s, kept)
+        assert torch.equal(kept, ref)
 
 
 def _moe_weights(oracle, dev, t, H, E, K, I, SI, seed=0):
