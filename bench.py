@@ -448,6 +448,35 @@ def bench_moe_prefill(a):
         return us_sep, us_fused, us_kept
 
     us_sep, us_fused, us_fused_kept = block()
+
+    # the whole MoE FFN block of a prefill chunk (router, routing, routed and shared experts, weighted sum), as the
+    # host-side mirror of build_moe_ffn_layer_gpu_q_into encodes it above 8 tokens
+    def layer():
+        rnd = lambda *s: torch.randn(*s, generator=gen, device=dev, dtype=torch.float32)  # noqa: E731
+        qz = lambda n, k: ops.quantize_ggml(rnd(n * k).mul_(0.02), k, HQ_Q4_K)  # noqa: E731
+        ls = [ops.MoeFfnWeightsGpuQ(rnd(E, H).mul_(0.02).to(torch.bfloat16), qz(E * I, H), qz(E * I, H), qz(E * H, I),
+                                    rnd(1, H).mul_(0.02).to(torch.bfloat16), qz(I, H), qz(I, H), qz(H, I), HQ_Q4_K, H, E, K, I, I)
+              for _ in range(2)]
+        x = rnd(T, H).to(torch.bfloat16)
+        sc = ops.MoeFfnScratch(ls[0], T, dev)
+        out = torch.empty(T, H, device=dev)
+
+        def step(i):
+            ops.build_moe_ffn_layer_gpu_q_into(x, ls[i % 2], sc, out)
+
+        for i in range(max(a.warmup, 1)):
+            step(i)
+        torch.cuda.synchronize()
+        _, us_plain = _timed_steps(a, step, 2)
+        for l in ls:
+            l.prepare_prefill()
+        for i in range(2):
+            step(i)
+        torch.cuda.synchronize()
+        _, us_kept = _timed_steps(a, step, 2)
+        return us_plain, us_kept
+
+    us_layer, us_layer_kept = layer()
     flops = 2.0 * T * K * I * H
     tf = flops / us / 1e6
     return _finish(a, {
@@ -467,6 +496,11 @@ def bench_moe_prefill(a):
                                       "separate_us": round(us_sep, 2), "one_call_us": round(us_fused, 2),
                                       "one_call_with_kept_scales_us": round(us_fused_kept, 2),
                                       "one_call_TFLOP/s": round(2 * flops / us_fused / 1e6, 1)},
+                   "whole_block_2048_tokens": {"what": "build_moe_ffn_layer_gpu_q_into at 2048 tokens: router, softmax / top-8, gate / up / "
+                                                       "SwiGLU and down of the routed experts (grouped), the shared expert, the weighted "
+                                                       "sum; 12 launches", "us_per_layer": round(us_layer, 1),
+                                               "us_per_layer_with_kept_scales": round(us_layer_kept, 1),
+                                               "tok/s_over_40_layers": round(T / (40 * us_layer * 1e-6), 0)},
                    "down_shape_2048x512": {"us_per_step": round(us_down, 2), "TFLOP/s": round(flops / us_down / 1e6, 1),
                                            "us_per_step_with_kept_scales": round(us_down_prep, 2)}},
         "roofline": {"bound": "mfma", "kernel": "grouped pre-pass + grouped f16 MFMA gemm q4_k", "achieved": round(tf, 1),
