@@ -145,6 +145,8 @@ extern "C" {
     pub fn hq_qmatmul_ggml(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type) -> c_int;
     pub fn hq_qmatmul_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;
     pub fn hq_qmatmul_ggml_ws(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
+    pub fn hq_qmatmul_gated_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;
+    pub fn hq_qmatmul_gated_ggml_ws(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, w_row_scales: *const f32, gate: *const f32, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
     pub fn hq_qmatmul_swiglu_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;
     pub fn hq_qmatmul_swiglu_ggml_ws(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_gate: *const c_void, w_up: *const c_void, gate_row_scales: *const f32, up_row_scales: *const f32, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
     pub fn hq_qmatmul_perm021_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;

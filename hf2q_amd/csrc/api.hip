@@ -282,6 +282,30 @@ int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w
     return rc ? rc : rc_free;
 }
 
+size_t hq_qmatmul_gated_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
+    if (hq_block_elems(t) == 0 || n == 0 || k == 0 || k % hq_block_elems(t)) return 0;
+    return f16_tile_route(m, k, t) && gemm_f16_tile_gated_supported(t, m, n, k) ? hq_qmatmul_ggml_workspace_bytes(m, n, k, xdt, t) : 0;
+}
+
+int hq_qmatmul_gated_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, const float* w_row_scales,
+                             const float* gate, float* y, uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, void* workspace,
+                             size_t workspace_bytes) {
+    const char* fn = "hq_qmatmul_gated_ggml_ws";
+    if (int rc = check_matmul_common(fn, x, xdt, w_blocks, y, n, k, t)) return rc;
+    if (!gate || !is_aligned(gate, 4)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: gate is null or not 4-byte aligned", fn);
+    if (w_row_scales && !is_aligned(w_row_scales, 4)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: w_row_scales must be 4-byte aligned", fn);
+    if (m == 0) return HQ_OK;
+    const size_t need = hq_qmatmul_gated_ggml_workspace_bytes(m, n, k, xdt, t);
+    if (!need)
+        return fail(HQ_ERR_UNSUPPORTED,
+                    "%s: this shape or type has no gated tile form (hq_qmatmul_gated_ggml_workspace_bytes is 0): "
+                    "hq_qmatmul_ggml and hq_silu_mul give the same result", fn);
+    if (!workspace || workspace_bytes < need)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes, %zu needed", fn, workspace ? workspace_bytes : (size_t)0, need);
+    if (reinterpret_cast<uintptr_t>(workspace) % 256) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace must be 256-byte aligned", fn);
+    return launch_gemm_f16_tile((hipStream_t)stream, x, xdt, w_blocks, y, m, n, k, t, workspace, 0, w_row_scales, gate);
+}
+
 size_t hq_qmatmul_swiglu_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
     (void)xdt;
     if (hq_block_elems(t) == 0 || n == 0 || k == 0 || k % hq_block_elems(t)) return 0;

@@ -314,6 +314,9 @@ struct GemmArgs {
     // `w`) and its rows' scales; the tile multiplies both and stores silu(gate) * up.  Null otherwise.
     const uint8_t* w2;
     const float* wscale2;
+    // Dense form only, may be null: a [m][n] f32 matrix g; the epilogue stores silu(g) * (x . W^T) instead of the
+    // product (the up projection of a SwiGLU layer finishing the gating of the gate projection computed before it).
+    const float* gate_in;
 };
 
 __device__ __forceinline__ f16x8_t as_frag(uint4 v) { return __builtin_bit_cast(f16x8_t, v); }
@@ -430,9 +433,23 @@ __device__ __forceinline__ void store_tile(const GemmArgs& a, const Workspace& W
             float* yp = a.y + (size_t)orow * a.n + gnb;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const float o0 = acc[mt][nt][4 * g] * (rsv * wup[4 * g]), o1 = acc[mt][nt][4 * g + 1] * (rsv * wup[4 * g + 1]);
-                const float o2 = acc[mt][nt][4 * g + 2] * (rsv * wup[4 * g + 2]), o3 = acc[mt][nt][4 * g + 3] * (rsv * wup[4 * g + 3]);
+                float o0 = acc[mt][nt][4 * g] * (rsv * wup[4 * g]), o1 = acc[mt][nt][4 * g + 1] * (rsv * wup[4 * g + 1]);
+                float o2 = acc[mt][nt][4 * g + 2] * (rsv * wup[4 * g + 2]), o3 = acc[mt][nt][4 * g + 3] * (rsv * wup[4 * g + 3]);
                 const uint32_t gn = gnb + 8 * g;
+                if (a.gate_in) {  // (uniform) silu(gate) * up, the stand-alone kernel's arithmetic
+                    const float* gp = a.gate_in + (size_t)orow * a.n + gnb + 8 * g;
+                    if (vec_ok && (reinterpret_cast<uintptr_t>(a.gate_in) & 15u) == 0) {
+                        if (gn < a.n) {
+                            const float4 gv = *reinterpret_cast<const float4*>(gp);
+                            o0 = silu_mul_f32(gv.x, o0), o1 = silu_mul_f32(gv.y, o1), o2 = silu_mul_f32(gv.z, o2), o3 = silu_mul_f32(gv.w, o3);
+                        }
+                    } else {
+                        if (gn < a.n) o0 = silu_mul_f32(gp[0], o0);
+                        if (gn + 1 < a.n) o1 = silu_mul_f32(gp[1], o1);
+                        if (gn + 2 < a.n) o2 = silu_mul_f32(gp[2], o2);
+                        if (gn + 3 < a.n) o3 = silu_mul_f32(gp[3], o3);
+                    }
+                }
                 if (vec_ok) {
                     if (gn < a.n) *reinterpret_cast<float4*>(yp + 8 * g) = make_float4(o0, o1, o2, o3);
                 } else {
@@ -1308,6 +1325,10 @@ static uint32_t small_splits_of(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t
     return small_tile_splits(m, n, k, bm, BN_WIDE);
 }
 
+bool gemm_f16_tile_gated_supported(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) {
+    return gemm_f16_tile_supported(t, k) && !(gemm_f16_small_tiles(t, m) && small_splits_of(t, m, n, k) > 1);
+}
+
 size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t) {
     size_t total = workspace_layout(m, n, k).total;
     if (gemm_f16_small_tiles(t, m)) {  // partial sums of the slices of k
@@ -1472,11 +1493,15 @@ int launch_gemm_f16_swiglu(hipStream_t s, const void* x, hq_act_dtype xdt, const
 }
 
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
-                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd, const float* w_scales) {
+                         uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd, const float* w_scales,
+                         const float* gate_in) {
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const uint8_t* wb = static_cast<const uint8_t*>(w);
     GemmArgs a{ws, wb, y, m, n, k, m, n, 0u, nullptr, 0u, (k + 255u) / 256u, 0u,
-               w_scales ? w_scales : reinterpret_cast<const float*>(ws + workspace_layout(m, n, k).wdown)};
+               w_scales ? w_scales : reinterpret_cast<const float*>(ws + workspace_layout(m, n, k).wdown), nullptr, nullptr, gate_in};
+    // (the forms that cut k into slices add partial products: the gating cannot go into their epilogue)
+    if (gate_in && gemm_f16_small_tiles(t, m) && small_splits_of(t, m, n, k) > 1)
+        return fail(HQ_ERR_UNSUPPORTED, "tile gemm with a gated epilogue: this shape is cut into slices of k");
     constexpr int lds = 2 * ActTile::kTile;
     const uint32_t tiles_m = (m + BM - 1) / BM, cols_wide = (n + BN_WIDE - 1) / BN_WIDE;
     // up to 256 token rows of Q6_K / Q8_0 / Q4_0: one token tile of 128 or 256 rows x 128 weight rows, k in slices where

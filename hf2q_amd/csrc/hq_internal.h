@@ -82,7 +82,9 @@ size_t gemm_f16_tile_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_ggml
 // gathered by the pre-pass.
 int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m,
                          uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, uint32_t perm_hd = 0,
-                         const float* w_scales = nullptr);
+                         const float* w_scales = nullptr, const float* gate_in = nullptr);
+// Whether launch_gemm_f16_tile takes gate_in for this shape (not where k is cut into slices).
+bool gemm_f16_tile_gated_supported(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k);
 // The tile kernels' weight-row scales (n_rows floats, a function of the weights alone): what the pre-pass of every tile
 // or grouped call works out when w_scales is null.
 int launch_weight_row_scales(hipStream_t s, const void* w, float* scales, uint32_t n_rows, uint32_t k, hq_ggml_type t);

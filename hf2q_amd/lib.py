@@ -61,6 +61,8 @@ SIGNATURES = {
     "hq_qmatmul_id_ggml_prepared": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _u32, _u32, _u32, _u32, _u32, _u64, _i32]),
     "hq_qmatmul_id_swiglu_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _u32, _u32, _u64, _i32]),
     "hq_qmatmul_id_swiglu_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _u32, _u32, _u32, _u32, _u32, _u64, _i32]),
+    "hq_qmatmul_gated_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),
+    "hq_qmatmul_gated_ggml_ws": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _i32, _vp, _sz]),
     "hq_qmatmul_swiglu_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),
     "hq_qmatmul_swiglu_ggml_ws": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _i32, _vp, _sz]),
     "hq_qmatmul_perm021_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),

@@ -117,6 +117,29 @@ def quantized_matmul_workspace_bytes(params: GgmlQuantizedMatmulParams, act_dtyp
     return int(L.hq_qmatmul_ggml_workspace_bytes(params.m, params.n, params.k, xdt, params.ggml_type))
 
 
+def quantized_matmul_gated_workspace_bytes(params: GgmlQuantizedMatmulParams, act_dtype: torch.dtype) -> int:
+    """Device scratch of quantized_matmul_gated_ggml for this shape; 0 where that form does not exist."""
+    xdt = _l.HQ_BF16 if act_dtype == torch.bfloat16 else _l.HQ_F32
+    return int(_l.load().hq_qmatmul_gated_ggml_workspace_bytes(params.m, params.n, params.k, xdt, params.ggml_type))
+
+
+def quantized_matmul_gated_ggml(input: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, dst: torch.Tensor,
+                                params: GgmlQuantizedMatmulParams, workspace: torch.Tensor,
+                                w_row_scales: torch.Tensor | None = None) -> None:
+    """dst[m, n] = silu(gate[m, n]) * (input . W^T)[m, n]: the up projection of a dense SwiGLU layer at prefill with
+    the gating in its epilogue (gate: the f32 output of the gate projection; dst may be that buffer)."""
+    if dst.dtype != torch.float32 or gate.dtype != torch.float32:
+        raise TypeError("dst and gate must be float32")
+    if gate.numel() < params.m * params.n:
+        raise ValueError("gate must hold m * n values")
+    if w_row_scales is not None:
+        _check_scales(w_row_scales, params.n)
+    _l.check(_l.load().hq_qmatmul_gated_ggml_ws(
+        _stream(), _dev(input, "input"), _act_dtype(input), _dev(weight, "weight"),
+        _dev(w_row_scales, "w_row_scales") if w_row_scales is not None else None, _dev(gate, "gate"), _dev(dst, "dst"),
+        params.m, params.n, params.k, params.ggml_type, _dev(workspace, "workspace"), workspace.numel() * workspace.element_size()))
+
+
 def quantized_matmul_swiglu_workspace_bytes(params: GgmlQuantizedMatmulParams, act_dtype: torch.dtype) -> int:
     """Device scratch of quantized_matmul_swiglu_ggml for this shape; 0 where that form does not exist."""
     xdt = _l.HQ_BF16 if act_dtype == torch.bfloat16 else _l.HQ_F32
@@ -617,9 +640,15 @@ class DenseFfnWeightsGpuQ:
     inter: int
 
 
+def dense_ffn_workspace_bytes(w: "DenseFfnWeightsGpuQ", m: int, act_dtype: torch.dtype) -> int:
+    """Device scratch build_dense_ffn_layer_gpu_q_into(..., workspace=) needs for m rows (0: none needed)."""
+    return max(quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, w.inter, w.hidden, w.ggml_type), act_dtype),
+               quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, w.hidden, w.inter, w.ggml_type), torch.float32))
+
+
 def build_dense_ffn_layer_gpu_q_into(x: torch.Tensor, w: DenseFfnWeightsGpuQ, gate_buf: torch.Tensor,
                                      up_buf: torch.Tensor, act_buf: torch.Tensor | None, out: torch.Tensor,
-                                     batched: bool | None = None) -> None:
+                                     batched: bool | None = None, workspace: torch.Tensor | None = None) -> None:
     """gpu_ffn.rs:1086-1330: out = down(silu(gate x) * (up x)) for seq_len rows of x.  The reference encodes gate
     and up back to back (one barrier after both), then silu_mul, then down.  `batched` (default: whenever the
     row count is decode-sized) hands gate + up to the library as one launch and folds the SwiGLU into the
@@ -640,10 +669,18 @@ def build_dense_ffn_layer_gpu_q_into(x: torch.Tensor, w: DenseFfnWeightsGpuQ, ga
             dispatch_silu_mul(gate_buf[:m], up_buf[:m], act_buf[:m])
             quantized_matmul_ggml(act_buf, w.down_q, out, GgmlQuantizedMatmulParams(m, H, I, t))
         return
-    quantized_matmul_ggml(x, w.gate_q, gate_buf, GgmlQuantizedMatmulParams(m, I, H, t))
-    quantized_matmul_ggml(x, w.up_q, up_buf, GgmlQuantizedMatmulParams(m, I, H, t))
+    pgu, pdn = GgmlQuantizedMatmulParams(m, I, H, t), GgmlQuantizedMatmulParams(m, H, I, t)
+    if workspace is not None and quantized_matmul_gated_workspace_bytes(pgu, x.dtype):
+        # a prefill chunk with caller scratch (dense_ffn_workspace_bytes): nothing is allocated, and the up projection
+        # finishes the gating in its epilogue -- no SwiGLU pass over both products (the same bits)
+        quantized_matmul_ggml(x, w.gate_q, gate_buf, pgu, workspace=workspace)
+        quantized_matmul_gated_ggml(x, w.up_q, gate_buf, act_buf, pgu, workspace)
+        quantized_matmul_ggml(act_buf, w.down_q, out, pdn, workspace=workspace)
+        return
+    quantized_matmul_ggml(x, w.gate_q, gate_buf, pgu, workspace=workspace)
+    quantized_matmul_ggml(x, w.up_q, up_buf, pgu, workspace=workspace)
     dispatch_silu_mul(gate_buf[:m], up_buf[:m], act_buf[:m])
-    quantized_matmul_ggml(act_buf, w.down_q, out, GgmlQuantizedMatmulParams(m, H, I, t))
+    quantized_matmul_ggml(act_buf, w.down_q, out, pdn, workspace=workspace)
 
 
 @dataclass

@@ -124,6 +124,21 @@ HQ_API int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, con
                        uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, void* workspace,
                        size_t workspace_bytes);
 
+/* The up projection of a dense SwiGLU layer finishing the gating in its epilogue, on the prefill route:
+ *   y[m, n] = silu(gate[m, n]) * (x . W^T)[m, n]
+ * with `gate` the f32 output of the gate projection computed before it.  Replaces the second quantized_matmul_ggml
+ * and the silu_mul of the dense FFN at prefill (gpu_ffn.rs:1236-1306): the stand-alone SwiGLU pass reads both
+ * products and writes the activations (300 MB at 2048 x 12288, about 50 us); here the gate values are read while the
+ * tiles are stored and the up product never goes to memory.  The bits of the separate calls.  Every weight type of
+ * the tile route, any token count above the small-batch kernels' -- except where the product is cut into slices of k
+ * (up to 256 rows over few weight rows): hq_qmatmul_gated_ggml_workspace_bytes() is 0 there and the call returns
+ * HQ_ERR_UNSUPPORTED.  y may be the gate buffer itself (every element is read before it is written, by the same lane).
+ * w_row_scales: null, or from hq_weight_row_scales_ggml. */
+HQ_API size_t hq_qmatmul_gated_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t);
+HQ_API int hq_qmatmul_gated_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks,
+                             const float* w_row_scales, const float* gate, float* y, uint32_t m, uint32_t n, uint32_t k,
+                             hq_ggml_type t, void* workspace, size_t workspace_bytes);
+
 /* The gate and up products of a dense SwiGLU layer and the gating as one call on the prefill route:
  *   y[m, n] = silu(x . W_gate^T) * (x . W_up^T)
  * Replaces the two quantized_matmul_ggml dispatches and the silu_mul between them that the dense FFN and the shared

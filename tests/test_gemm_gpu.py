@@ -182,6 +182,41 @@ def test_dense_swiglu_tile_form(oracle, dev, t, xdt, m, n, k):
         ops.quantized_matmul_swiglu_ggml(xd, gd, ud, y, p, ws[: need - 256])
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0, HQ_Q6_K, HQ_Q5_K, HQ_Q4_0])
+@pytest.mark.parametrize("m,n,k", [(300, 257, 768), (2048, 384, 512), (64, 1024, 256)])
+def test_gated_epilogue_equals_product_then_silu_mul(oracle, dev, t, m, n, k):
+    """y = silu(gate) * (x . W^T) from the up projection's epilogue: the bits of the product followed by silu_mul, also in
+    place over the gate buffer and with the weight's row scales brought by the caller."""
+    blocks = oracle.quantize(weights(51 * n + k + t, n, k), k, t, threads=8)
+    wd = torch.from_numpy(blocks).to(dev)
+    x = torch.from_numpy(acts(n + m, m, k)).to(dev).to(torch.bfloat16)
+    gate = torch.from_numpy(acts(n + m + 1, m, n)).to(dev) * 2.0
+    p = GgmlQuantizedMatmulParams(m, n, k, t)
+    need = ops.quantized_matmul_gated_workspace_bytes(p, torch.bfloat16)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    up = torch.empty(m, n, device=dev)
+    ops.quantized_matmul_ggml(x, wd, up, p, workspace=ws)
+    want = gate / (1.0 + torch.exp(-gate)) * up  # torch's silu * up: close; the library's own kernel is the bit reference
+    cut = m * n - (m * n) % 4
+    sep = torch.empty(m, n, device=dev)
+    ops.dispatch_silu_mul(gate.view(-1)[:cut], up.view(-1)[:cut], sep.view(-1)[:cut])
+    y = torch.full((m, n), float("nan"), device=dev)
+    ops.quantized_matmul_gated_ggml(x, wd, gate, y, p, ws)
+    assert torch.equal(y.view(-1)[:cut], sep.view(-1)[:cut])
+    assert torch.allclose(y, want, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
+    g2 = gate.clone()
+    ops.quantized_matmul_gated_ggml(x, wd, g2, g2, p, ws, ops.weight_row_scales_ggml(wd, n, k, t))
+    assert torch.equal(g2, y)
+
+
+def test_gated_epilogue_has_no_form_where_k_is_cut_into_slices(dev):
+    p = GgmlQuantizedMatmulParams(64, 256, 4096, HQ_Q4_K)  # 64 rows over two column tiles: slices of k
+    assert ops.quantized_matmul_workspace_bytes(p, torch.bfloat16) > 0
+    assert ops.quantized_matmul_gated_workspace_bytes(p, torch.bfloat16) == 0
+    assert ops.quantized_matmul_gated_workspace_bytes(GgmlQuantizedMatmulParams(4, 256, 4096, HQ_Q4_K), torch.bfloat16) == 0
+
+
 def test_dense_swiglu_has_no_form_for_other_types_and_few_rows(dev):
     assert ops.quantized_matmul_swiglu_workspace_bytes(GgmlQuantizedMatmulParams(64, 128, 512, HQ_Q6_K), torch.bfloat16) == 0
     assert ops.quantized_matmul_swiglu_workspace_bytes(GgmlQuantizedMatmulParams(4, 128, 512, HQ_Q4_K), torch.bfloat16) == 0

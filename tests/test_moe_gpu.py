@@ -296,6 +296,27 @@ def test_dense_ffn_batched_equals_separate_dispatches_and_cpu_spec(oracle, dev, 
     assert_matmul_close(outs[1][0].numpy(), want, "dense FFN")
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
+def test_dense_ffn_prefill_with_workspace_equals_the_allocating_calls(oracle, dev, t):
+    """A prefill-sized dense FFN with caller scratch (gate, up with the gating in its epilogue, down; nothing
+    allocated) gives the bits of the four separate dispatches."""
+    H, I, m = 512, 1024, 300
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    w = ops.DenseFfnWeightsGpuQ(dv(oracle.quantize(weights(1, I, H, 0.05), H, t, threads=8)),
+                                dv(oracle.quantize(weights(2, I, H, 0.05), H, t, threads=8)),
+                                dv(oracle.quantize(weights(3, H, I, 0.05), I, t, threads=8)), t, H, I)
+    x = dv(acts(4, m, H)).to(torch.bfloat16)
+    bufs = [torch.empty(m, I, device=dev) for _ in range(3)]
+    out0, out1 = torch.empty(m, H, device=dev), torch.full((m, H), float("nan"), device=dev)
+    ops.build_dense_ffn_layer_gpu_q_into(x, w, *bufs, out0)
+    need = ops.dense_ffn_workspace_bytes(w, m, torch.bfloat16)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    bufs2 = [torch.full((m, I), float("nan"), device=dev) for _ in range(3)]
+    ops.build_dense_ffn_layer_gpu_q_into(x, w, *bufs2, out1, workspace=ws)
+    assert torch.equal(out0, out1) and torch.equal(bufs[2], bufs2[2])
+
+
 @pytest.mark.parametrize("T", [1, 2, 5, 8])
 def test_moe_block_one_launch_equals_batched_dispatches_and_cpu_spec(oracle, dev, T):
     """hq_moe_ffn_decode (the whole block in one launch, workgroups handing results to each other through the
