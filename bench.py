@@ -66,6 +66,10 @@ def parse():
     ap.add_argument("--no-graph", action="store_true",
                     help="moe_decode / moe_prefill / tq_attention: launch every kernel from the host instead of replaying a HIP "
                          "graph of the step (the steps are 4-12 launches of a few microseconds each)")
+    ap.add_argument("--block-only", action="store_true",
+                    help="moe_prefill: run only the whole-block part (for a kernel trace of the block's launches alone)")
+    ap.add_argument("--kept-scales", action="store_true",
+                    help="moe_prefill --block-only: the block with its weight-row scales kept from load time")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies first: the known-size kernel that scales "
@@ -409,6 +413,33 @@ def bench_moe_prefill(a):
         elapsed, us = _timed_steps(a, step, n_stacks)
         _, us_prepared = _timed_steps(a, step_prepared, n_stacks)
         return elapsed, us, us_prepared, need
+
+    if getattr(a, "block_only", False):  # the whole block alone, launched as asked (see `layer` below for what it is)
+        rnd = lambda *s: torch.randn(*s, generator=gen, device=dev, dtype=torch.float32)  # noqa: E731
+        qz = lambda n, k: ops.quantize_ggml(rnd(n * k).mul_(0.02), k, HQ_Q4_K)  # noqa: E731
+        ls = [ops.MoeFfnWeightsGpuQ(rnd(E, H).mul_(0.02).to(torch.bfloat16), qz(E * I, H), qz(E * I, H), qz(E * H, I),
+                                    rnd(1, H).mul_(0.02).to(torch.bfloat16), qz(I, H), qz(I, H), qz(H, I), HQ_Q4_K, H, E, K, I, I)
+              for _ in range(2)]
+        if a.kept_scales:
+            for l in ls:
+                l.prepare_prefill()
+        x = rnd(T, H).to(torch.bfloat16)
+        sc = ops.MoeFfnScratch(ls[0], T, dev)
+        out = torch.empty(T, H, device=dev)
+
+        def step(i):
+            ops.build_moe_ffn_layer_gpu_q_into(x, ls[i % 2], sc, out)
+
+        for i in range(max(a.warmup, 1)):
+            step(i)
+        torch.cuda.synchronize()
+        elapsed, us = _timed_steps(a, step, 2)
+        return _finish(a, {
+            "metric": "MoE prefill tok/s (FFN-only, 40 MoE layers)", "value": round(T / (40 * elapsed / a.steps), 0), "unit": "tok/s",
+            "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f16",
+            "config": {"workload": "moe_prefill --block-only: build_moe_ffn_layer_gpu_q_into at 2048 tokens, hidden 2048, 256 experts x "
+                                   "512 Q4_K, top-8, one shared expert" + (", weight-row scales kept from load time" if a.kept_scales else ""),
+                       "us_per_layer": round(us, 1)}})
 
     elapsed, us, us_prep, need = shape(I, H, T, K)
     _, us_down, us_down_prep, _ = shape(H, I, T * K, 1)
