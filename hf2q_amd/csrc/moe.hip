@@ -125,51 +125,69 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
 // The same product for many activation rows (the router of a prefill chunk: 2048 tokens x 256 experts), bf16
-// activations: both operands go from memory straight into the matrix cores, one workgroup per 32 x 32 tile of y, its
-// four waves a quarter of k each (eight k-steps of loads in flight per wave: with a whole row per wave the kernel was
-// one memory round trip after another, 40 us), their partial tiles added in wave order through LDS.  The bf16 products
-// are exact and the sums f32.  The weights are the MFMA's first operand, so a lane ends up with sixteen outputs of ONE
-// token (lane % 32), four runs of four consecutive n.  Rows past m or n repeat the last one and are not stored.
-// k % 16 == 0.
+// activations: both operands go from memory straight into the matrix cores.  One workgroup per tile of 32 token rows x
+// 64 weight rows, its four waves a quarter of k each; a wave reads one activation fragment and two weight fragments per
+// k-step (eight k-steps of loads in flight) for two MFMAs -- the loads are row-strided, a cache line per lane, and their
+// line look-ups are what bounds the kernel, so fewer of them per MFMA is what counts.  The partial tiles are added in
+// wave order through LDS.  The bf16 products are exact and the sums f32.  The weights are the MFMA's first operand, so
+// a lane ends up with sixteen outputs of ONE token (lane % 32) per weight tile, four runs of four consecutive n.  Rows
+// past m or n repeat the last one and are not stored.  k % 16 == 0.
 __global__ __launch_bounds__(256) void dense_gemm_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                               float* __restrict__ y, uint32_t m, uint32_t n, uint32_t k) {
-    __shared__ float part[3][16][64];
+    __shared__ float part[3][2][16][64];
     const uint32_t lane = threadIdx.x & 63u, l32 = lane & 31u, lg = lane >> 5, wave = threadIdx.x >> 6;
-    const uint32_t tiles_n = (n + 31u) / 32u;
-    const uint32_t m0 = (blockIdx.x / tiles_n) * 32u, n0 = (blockIdx.x % tiles_n) * 32u;
-    const uint32_t wr = n0 + l32 < n ? n0 + l32 : n - 1u, xr = m0 + l32 < m ? m0 + l32 : m - 1u;
-    const uint4* wp = reinterpret_cast<const uint4*>(w + (size_t)wr * k) + lg;  // 8 values per uint4, this lane's k-group
-    const uint4* xp = reinterpret_cast<const uint4*>(x + (size_t)xr * k) + lg;
-    f32x16_t acc;
+    const uint32_t tiles_n = (n + 63u) / 64u;
+    const uint32_t m0 = (blockIdx.x / tiles_n) * 32u, n0 = (blockIdx.x % tiles_n) * 64u;
+    const uint32_t xr = m0 + l32 < m ? m0 + l32 : m - 1u;
+    const uint4* xp = reinterpret_cast<const uint4*>(x + (size_t)xr * k) + lg;  // 8 values per uint4, this lane's k-group
+    const uint4* wp[2];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    for (int t = 0; t < 2; ++t) {
+        const uint32_t wr = n0 + 32u * t + l32 < n ? n0 + 32u * t + l32 : n - 1u;
+        wp[t] = reinterpret_cast<const uint4*>(w + (size_t)wr * k) + lg;
+    }
+    f32x16_t acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
     const uint32_t steps = k / 16u, per = (steps + 3u) / 4u;
     uint32_t st = wave * per;
     const uint32_t end = st + per < steps ? st + per : steps;
     for (; st + 8u <= end; st += 8u) {
-        uint4 a[8], b[8];
+        uint4 a0[8], a1[8], b[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) a[u] = wp[2u * (st + u)], b[u] = xp[2u * (st + u)];
+        for (int u = 0; u < 8; ++u) a0[u] = wp[0][2u * (st + u)], a1[u] = wp[1][2u * (st + u)], b[u] = xp[2u * (st + u)];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[u]), __builtin_bit_cast(bf16x8_t, b[u]), acc, 0, 0, 0);
+        for (int u = 0; u < 8; ++u) {
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0[u]), __builtin_bit_cast(bf16x8_t, b[u]), acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1[u]), __builtin_bit_cast(bf16x8_t, b[u]), acc[1], 0, 0, 0);
+        }
     }
-    for (; st < end; ++st)
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wp[2u * st]), __builtin_bit_cast(bf16x8_t, xp[2u * st]), acc, 0, 0, 0);
+    for (; st < end; ++st) {
+        const bf16x8_t b = __builtin_bit_cast(bf16x8_t, xp[2u * st]);
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wp[0][2u * st]), b, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wp[1][2u * st]), b, acc[1], 0, 0, 0);
+    }
     if (wave) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) part[wave - 1][v][lane] = acc[v];
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) part[wave - 1][t][v][lane] = acc[t][v];
     }
     __syncthreads();
     if (wave || m0 + l32 >= m) return;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = ((acc[v] + part[0][v][lane]) + part[1][v][lane]) + part[2][v][lane];
-    float* yp = y + (size_t)(m0 + l32) * n + n0 + 4u * lg;
+    for (int t = 0; t < 2; ++t) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
+        for (int v = 0; v < 16; ++v) acc[t][v] = ((acc[t][v] + part[0][t][v][lane]) + part[1][t][v][lane]) + part[2][t][v][lane];
+        float* yp = y + (size_t)(m0 + l32) * n + n0 + 32u * t + 4u * lg;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (n0 + 4u * lg + 8u * g + i < n) yp[8 * g + i] = acc[4 * g + i];
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n0 + 32u * t + 4u * lg + 8u * g + i < n) yp[8 * g + i] = acc[t][4 * g + i];
+    }
 }
 
 }  // namespace
@@ -182,7 +200,7 @@ int launch_dense_gemv_bf16_pair(hipStream_t s, const void* x, hq_act_dtype xdt, 
     // tokens x 256 experts x 2048: one wave per (token, expert) over the whole row took 175 us); a second matrix of a few
     // rows (the shared expert's gate) keeps the one-wave-per-output form in a launch of its own.
     if (xdt == HQ_BF16 && m >= 32 && n_a >= 32 && k % 16 == 0) {
-        const uint32_t tiles_a = ((m + 31u) / 32u) * ((n_a + 31u) / 32u);
+        const uint32_t tiles_a = ((m + 31u) / 32u) * ((n_a + 63u) / 64u);
         hipLaunchKernelGGL(dense_gemm_bf16_kernel, dim3(tiles_a), dim3(256), 0, s, static_cast<const uint16_t*>(x), wa, y_a, m, n_a, k);
         if (int rc = check_launch("dense bf16 gemm launch")) return rc;
         if (!n_b) return HQ_OK;
