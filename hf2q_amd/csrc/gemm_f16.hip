@@ -1385,8 +1385,11 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     // expert on average, tiles of 128 routed rows: the 256-row tiles would run a quarter full, and half of the experts
     // would need two 64-row tiles); at 40 rows per expert or fewer the Q4_K / Q5_K tiles of 64 rows.
     constexpr bool HAS_64 = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K;
-    // (the SwiGLU form keeps two accumulator tiles per row tile: 128 rows is the most a wave's registers hold)
-    const int mt = HAS_64 && (uint64_t)pairs <= (uint64_t)n_experts * 40u ? 2 : (uint64_t)pairs < (uint64_t)n_experts * 160u || wb2 ? 4 : 8;
+    // (the SwiGLU form keeps two accumulator tiles per row tile: 128 rows is the most a wave's registers hold, and with
+    // Q5_K's high-bit words beside them 64 rows -- its 128-row form spills 42 registers)
+    const int mt = (HAS_64 && (uint64_t)pairs <= (uint64_t)n_experts * 40u) || (wb2 && TYPE == HQ_Q5_K) ? 2
+                   : (uint64_t)pairs < (uint64_t)n_experts * 160u || wb2                              ? 4
+                                                                                                      : 8;
     const uint32_t bm = 32u * (uint32_t)mt, bn = BN_WIDE;
     // sort by expert + one converted activation row per token (the tiles gather the rows of their routed rows from
     // them) + the weight rows' scales, in one launch
@@ -1410,7 +1413,11 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
     if (mt == 4) kern = grouped_gemm_kernel<TYPE, 4>;
     if constexpr (HAS_64) {
         if (mt == 2) kern = grouped_gemm_kernel<TYPE, 2>;
-        if (wb2) kern = mt == 2 ? grouped_gemm_kernel<TYPE, 2, true> : grouped_gemm_kernel<TYPE, 4, true>;
+        if (wb2) {
+            kern = grouped_gemm_kernel<TYPE, 2, true>;
+            if constexpr (TYPE == HQ_Q4_K)
+                if (mt == 4) kern = grouped_gemm_kernel<TYPE, 4, true>;
+        }
     }
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds, "hipFuncSetAttribute(grouped gemm LDS)"))
         return rc;
@@ -1482,8 +1489,8 @@ int launch_gemm_f16_swiglu(hipStream_t s, const void* x, hq_act_dtype xdt, const
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
     const uint32_t tiles_n = (n + BN_WIDE - 1) / BN_WIDE;
-    const bool small = (uint64_t)((m + BM_MID - 1) / BM_MID) * tiles_n < cus;
-    void (*kern)(GemmArgs) = t == HQ_Q5_K ? (small ? q4k_swiglu_kernel<HQ_Q5_K, 2> : q4k_swiglu_kernel<HQ_Q5_K, 4>)
+    const bool small = t == HQ_Q5_K || (uint64_t)((m + BM_MID - 1) / BM_MID) * tiles_n < cus;  // (Q5_K's 128-row form spills)
+    void (*kern)(GemmArgs) = t == HQ_Q5_K ? q4k_swiglu_kernel<HQ_Q5_K, 2>
                                           : (small ? q4k_swiglu_kernel<HQ_Q4_K, 2> : q4k_swiglu_kernel<HQ_Q4_K, 4>);
     const uint32_t bm = small ? BM_SMALL : BM_MID;
     const int lds = 2 * (small ? ActTileT<BM_SMALL>::kTile : ActTileT<BM_MID>::kTile);
