@@ -545,12 +545,18 @@ template <int TYPE, int ROWS = 1>
 int launch_stream(hipStream_t s, const SArgs& sa, uint32_t cus) {
     constexpr int W = TYPE == HQ_Q6_K ? 12 : 16;
     const size_t lds = ROWS * ((size_t)sa.k * 2 + (size_t)(sa.k / 16) * 4);
-    // (the two-row Q5_K form with its activations in registers would spill: it reads them from LDS per row piece)
-    if (sa.k == 4096 && ROWS <= 2 && !(TYPE == HQ_Q5_K && ROWS == 2)) {
-        auto kern = gemv_stream_kernel<TYPE, W, true, ROWS>;
-        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
-        hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
-    } else {
+    // (three and four rows in registers would spill, so would the two-row Q5_K form: not instantiated)
+    constexpr bool XREG_FITS = ROWS <= 2 && !(TYPE == HQ_Q5_K && ROWS == 2);
+    bool launched = false;
+    if constexpr (XREG_FITS) {
+        if (sa.k == 4096) {
+            auto kern = gemv_stream_kernel<TYPE, W, true, ROWS>;
+            if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
+            hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
+            launched = true;
+        }
+    }
+    if (!launched) {
         auto kern = gemv_stream_kernel<TYPE, W, false, ROWS>;
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
         hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
