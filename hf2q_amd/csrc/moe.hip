@@ -132,14 +132,43 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 // wave order through LDS.  The bf16 products are exact and the sums f32.  The weights are the MFMA's first operand, so
 // a lane ends up with sixteen outputs of ONE token (lane % 32) per weight tile, four runs of four consecutive n.  Rows
 // past m or n repeat the last one and are not stored.  k % 16 == 0.
-__global__ __launch_bounds__(256) void dense_gemm_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+// f32 activations are split into three bf16 terms each (truncations of x, of x - hi and of the rest: every step exact, 24
+// significant bits in all), so an activation fragment costs three MFMAs per weight tile and the products stay exact.
+template <bool X_BF16>
+__global__ __launch_bounds__(256) void dense_gemm_bf16_kernel(const void* __restrict__ xv, const uint16_t* __restrict__ w,
                                                               float* __restrict__ y, uint32_t m, uint32_t n, uint32_t k) {
     __shared__ float part[3][2][16][64];
     const uint32_t lane = threadIdx.x & 63u, l32 = lane & 31u, lg = lane >> 5, wave = threadIdx.x >> 6;
     const uint32_t tiles_n = (n + 63u) / 64u;
     const uint32_t m0 = (blockIdx.x / tiles_n) * 32u, n0 = (blockIdx.x % tiles_n) * 64u;
     const uint32_t xr = m0 + l32 < m ? m0 + l32 : m - 1u;
-    const uint4* xp = reinterpret_cast<const uint4*>(x + (size_t)xr * k) + lg;  // 8 values per uint4, this lane's k-group
+    // this lane's k-group of eight values: one uint4 of bf16, or two of f32
+    const uint4* xp = X_BF16 ? reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + (size_t)xr * k) + lg
+                             : reinterpret_cast<const uint4*>(static_cast<const float*>(xv) + (size_t)xr * k) + 2u * lg;
+    // k-step st of the activations: 1 (bf16) or 3 (f32) fragments
+    constexpr int XT = X_BF16 ? 1 : 3;
+    auto x_frags = [&](uint32_t st, bf16x8_t* f) {
+        if constexpr (X_BF16) {
+            f[0] = __builtin_bit_cast(bf16x8_t, xp[2u * st]);
+        } else {
+            const uint4 v0 = xp[4u * st], v1 = xp[4u * st + 1u];
+            const uint32_t u[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+            uint32_t t[3][8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t hi = u[i] & 0xffff0000u;
+                // (inf / nan stay in the first term alone: inf - inf would turn an infinite product into nan)
+                const float r1 = (hi & 0x7f800000u) == 0x7f800000u ? 0.f : __uint_as_float(u[i]) - __uint_as_float(hi);
+                const uint32_t mid = __float_as_uint(r1) & 0xffff0000u;
+                const float r2 = r1 - __uint_as_float(mid);
+                t[0][i] = hi, t[1][i] = mid, t[2][i] = __float_as_uint(r2) & 0xffff0000u;
+            }
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+                f[j] = __builtin_bit_cast(bf16x8_t, make_uint4((t[j][0] >> 16) | t[j][1], (t[j][2] >> 16) | t[j][3],
+                                                               (t[j][4] >> 16) | t[j][5], (t[j][6] >> 16) | t[j][7]));
+        }
+    };
     const uint4* wp[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -154,20 +183,28 @@ __global__ __launch_bounds__(256) void dense_gemm_bf16_kernel(const uint16_t* __
     const uint32_t steps = k / 16u, per = (steps + 3u) / 4u;
     uint32_t st = wave * per;
     const uint32_t end = st + per < steps ? st + per : steps;
-    for (; st + 8u <= end; st += 8u) {
-        uint4 a0[8], a1[8], b[8];
+    constexpr uint32_t UN = X_BF16 ? 8u : 4u;  // k-steps of loads in flight
+    for (; st + UN <= end; st += UN) {
+        uint4 a0[UN], a1[UN];
+        bf16x8_t b[UN][XT];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) a0[u] = wp[0][2u * (st + u)], a1[u] = wp[1][2u * (st + u)], b[u] = xp[2u * (st + u)];
+        for (uint32_t u = 0; u < UN; ++u) a0[u] = wp[0][2u * (st + u)], a1[u] = wp[1][2u * (st + u)], x_frags(st + u, b[u]);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0[u]), __builtin_bit_cast(bf16x8_t, b[u]), acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1[u]), __builtin_bit_cast(bf16x8_t, b[u]), acc[1], 0, 0, 0);
-        }
+        for (uint32_t u = 0; u < UN; ++u)
+#pragma unroll
+            for (int j = XT - 1; j >= 0; --j) {  // the smallest term first
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0[u]), b[u][j], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1[u]), b[u][j], acc[1], 0, 0, 0);
+            }
     }
     for (; st < end; ++st) {
-        const bf16x8_t b = __builtin_bit_cast(bf16x8_t, xp[2u * st]);
-        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wp[0][2u * st]), b, acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wp[1][2u * st]), b, acc[1], 0, 0, 0);
+        bf16x8_t b[XT];
+        x_frags(st, b);
+#pragma unroll
+        for (int j = XT - 1; j >= 0; --j) {
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wp[0][2u * st]), b[j], acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wp[1][2u * st]), b[j], acc[1], 0, 0, 0);
+        }
     }
     if (wave) {
 #pragma unroll
@@ -196,12 +233,15 @@ int launch_dense_gemv_bf16_pair(hipStream_t s, const void* x, hq_act_dtype xdt, 
                                 const void* w_b, float* y_b, uint32_t n_b, uint32_t m, uint32_t k) {
     const uint16_t* wa = static_cast<const uint16_t*>(w_a);
     const uint16_t* wb = static_cast<const uint16_t*>(w_b);
-    // Many rows of bf16 activations (a prefill chunk) and a matrix of at least 32 rows: the matrix-core form for it (2048
+    // Many activation rows (a prefill chunk) and a matrix of at least 32 rows: the matrix-core form for it (2048
     // tokens x 256 experts x 2048: one wave per (token, expert) over the whole row took 175 us); a second matrix of a few
     // rows (the shared expert's gate) keeps the one-wave-per-output form in a launch of its own.
-    if (xdt == HQ_BF16 && m >= 32 && n_a >= 32 && k % 16 == 0) {
+    if (m >= 32 && n_a >= 32 && k % 16 == 0) {
         const uint32_t tiles_a = ((m + 31u) / 32u) * ((n_a + 63u) / 64u);
-        hipLaunchKernelGGL(dense_gemm_bf16_kernel, dim3(tiles_a), dim3(256), 0, s, static_cast<const uint16_t*>(x), wa, y_a, m, n_a, k);
+        if (xdt == HQ_BF16)
+            hipLaunchKernelGGL(dense_gemm_bf16_kernel<true>, dim3(tiles_a), dim3(256), 0, s, x, wa, y_a, m, n_a, k);
+        else
+            hipLaunchKernelGGL(dense_gemm_bf16_kernel<false>, dim3(tiles_a), dim3(256), 0, s, x, wa, y_a, m, n_a, k);
         if (int rc = check_launch("dense bf16 gemm launch")) return rc;
         if (!n_b) return HQ_OK;
         return launch_dense_gemv_bf16_pair(s, x, xdt, w_b, y_b, n_b, nullptr, nullptr, 0, m, k);

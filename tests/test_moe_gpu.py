@@ -89,8 +89,18 @@ def test_dense_bf16_product_of_many_rows(oracle, dev, m, n, k):
     ref = xb.astype(np.float64) @ w.astype(np.float64).T
     assert np.abs(y.cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
     yf = torch.empty(m, n, device=dev)
-    ops.dense_gemv_bf16_f32(torch.from_numpy(xb).to(dev), wd, yf, m, n, k)  # the same values as f32: one wave per output
+    ops.dense_gemv_bf16_f32(torch.from_numpy(xb).to(dev), wd, yf, m, n, k)  # the same values as f32
     assert (y - yf).abs().max().item() <= 2e-5 * np.abs(ref).max()
+    # f32 activations that are no bf16 values: split into three bf16 terms, the products stay exact
+    xf = acts(5 + m, m, k)
+    xf[0, :4] = [np.inf, -3.0e38, 1e-40, 0.0]
+    ops.dense_gemv_bf16_f32(torch.from_numpy(xf).to(dev), wd, yf, m, n, k)
+    with np.errstate(invalid="ignore", over="ignore"):
+        reff = xf.astype(np.float64) @ w.astype(np.float64).T
+    got = yf.cpu().numpy()
+    assert np.abs(got[1:] - reff[1:]).max() <= 1e-5 * np.abs(reff[1:]).max()
+    fin = np.isfinite(reff[0]) & (np.abs(reff[0]) < 3e38)
+    assert np.array_equal(np.isinf(got[0]), np.isinf(reff[0]) | ~fin) or np.isinf(got[0]).all()
     w2 = torch.from_numpy(oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(weights(9, 1, k, 0.05)))).to(dev).to(torch.bfloat16)
     ya, yb = torch.empty(m, n, device=dev), torch.empty(m, 1, device=dev)
     ops.dense_gemv_bf16_f32_pair(xd, wd, ya, n, w2, yb, 1, m, k)
