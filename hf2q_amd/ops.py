@@ -776,13 +776,27 @@ def moe_ffn_decode_fused(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch
                            w.hidden, w.n_experts, w.top_k, w.inter, w.shared_inter, w.ggml_type, w.inter * rb_h, w.hidden * rb_i)
     if s.fused is None:
         raise _l.HqError(_l.HQ_ERR_UNSUPPORTED, "no scratch for the one-launch MoE block (shape not supported)")
-    _l.check(_l.load().hq_moe_ffn_decode(
-        _stream(), _ct.byref(layer), _dev(x, "x"), _act_dtype(x), _dev(residual, "residual") if residual is not None else None,
-        _dev(out, "out"), T, _dev(s.fused, "scratch"), s.fused.numel(), _dev(s.ids, "ids"), _dev(s.topk_w, "topk_w")))
+    L = _l.load()
+    # more than eight tokens (up to _FUSED_CHUNKED_MAX_TOKENS): one launch per eight, one after the other over the same scratch
+    for t0 in range(0, T, 8):
+        t1 = min(T, t0 + 8)
+        _l.check(L.hq_moe_ffn_decode(
+            _stream(), _ct.byref(layer), _dev(x[t0:t1], "x"), _act_dtype(x),
+            _dev(residual[t0:t1], "residual") if residual is not None else None, _dev(out[t0:t1], "out"), t1 - t0,
+            _dev(s.fused, "scratch"), s.fused.numel(), _dev(s.ids[t0 * w.top_k:], "ids"), _dev(s.topk_w[t0 * w.top_k:], "topk_w")))
+
+
+# Up to this many tokens the block runs as launches of the one-launch form over eight tokens each (33 us per eight:
+# 47 / 67 / 133 us at 9 / 16 / 32 tokens) rather than as separate dispatches with one GEMV per routed row (114 us at
+# 9 .. 16 tokens, 178 at 32, 257 at 64, where eight launches would cost the same).
+_FUSED_CHUNKED_MAX_TOKENS = 48
 
 
 def moe_ffn_decode_fused_supported(x: torch.Tensor, w: MoeFfnWeightsGpuQ) -> bool:
-    return bool(_l.load().hq_moe_ffn_decode_scratch_bytes(x.shape[0], w.hidden, w.n_experts, w.top_k, w.inter, w.shared_inter,
+    T = x.shape[0]
+    if T > _FUSED_CHUNKED_MAX_TOKENS:
+        return False
+    return bool(_l.load().hq_moe_ffn_decode_scratch_bytes(min(T, 8), w.hidden, w.n_experts, w.top_k, w.inter, w.shared_inter,
                                                           w.ggml_type, _act_dtype(x)))
 
 

@@ -369,6 +369,39 @@ def test_moe_block_one_launch_equals_batched_dispatches_and_cpu_spec(oracle, dev
     assert np.abs(got - want).max() <= 2e-4 * np.abs(want).max(), np.abs(got - want).max() / np.abs(want).max()
 
 
+@pytest.mark.parametrize("T", [9, 20, 48])
+def test_moe_block_of_up_to_48_tokens_runs_as_one_launch_per_eight(oracle, dev, T):
+    """9 .. 48 tokens: the block is the one-launch form over eight tokens at a time, sharing one scratch -- the bits of
+    separate calls over the chunks, the routing of every token written out, the separate dispatches within tolerance;
+    49 tokens take the separate dispatches."""
+    H, E, K, I, SI = 2048, 24, 8, 512, 512
+    w = _moe_weights(oracle, dev, HQ_Q4_K, H, E, K, I, SI, seed=T)
+    x = torch.from_numpy(acts(3 + T, T, H)).to(dev).to(torch.bfloat16)
+    res = torch.from_numpy(acts(4 + T, T, H)).to(dev)
+    assert ops.moe_ffn_decode_fused_supported(x, w)
+    assert not ops.moe_ffn_decode_fused_supported(torch.zeros(49, H, device=dev, dtype=torch.bfloat16), w)
+    s = ops.MoeFfnScratch(w, T, dev)
+    s.ids.fill_(-1)
+    out = torch.full((T, H), float("nan"), device=dev)
+    ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out, residual=res)
+    torch.cuda.synchronize()
+    assert int(s.fused[0:4].view(torch.int32).item()) == (T + 7) // 8, "one launch per eight tokens"
+    assert int(s.fused[4:8].view(torch.int32).item()) == 0
+    ids_all = s.ids.clone()
+    assert (ids_all >= 0).all() and (ids_all < E).all()
+    s8 = ops.MoeFfnScratch(w, 8, dev)
+    for t0 in range(0, T, 8):
+        t1 = min(T, t0 + 8)
+        part = torch.full((t1 - t0, H), float("nan"), device=dev)
+        ops.build_moe_ffn_layer_gpu_q_into(x[t0:t1].contiguous(), w, s8, part, residual=res[t0:t1].contiguous())
+        assert torch.equal(part, out[t0:t1])
+        assert torch.equal(s8.ids[: (t1 - t0) * K], ids_all[t0 * K:t1 * K])
+    # the separate dispatches (other kernels, other rounding) agree within the block's tolerance
+    sep = torch.empty_like(out)
+    ops.build_moe_ffn_layer_gpu_q_into(x, w, s, sep, residual=res, fused=False)
+    assert (sep - out).abs().max().item() <= 2e-3 * out.abs().max().item()
+
+
 @pytest.mark.parametrize("T", [1, 8])
 def test_moe_block_one_launch_replays_from_a_hip_graph(oracle, dev, T):
     """Three consecutive layers' worth of hq_moe_ffn_decode over ONE scratch, recorded into a HIP graph (the call
