@@ -177,7 +177,7 @@ HQ_API int hq_qmatmul_perm021_ggml_ws(void* stream, const void* x_perm, hq_act_d
  * n_tokens = T*K, top_k = 1 (forward_mlx.rs:650-651).  An id >= n_experts
  * makes the affected output rows NaN instead of reading out of bounds.
  * Decode-sized calls run one dequant-fused GEMV per routed row and use no
- * scratch.  With at least 8 routed rows per expert (prefill) and a `scratch`
+ * scratch.  With at least 3 routed rows per expert (prefill) and a `scratch`
  * of hq_qmatmul_id_ggml_workspace_bytes() bytes (device, 256-byte aligned),
  * the rows are sorted by expert and every expert's rows go through the tile
  * GEMM of the m > 8 route (the reference's mul_mm_id, forward_mlx.rs:5237-5245);
@@ -217,7 +217,7 @@ HQ_API int hq_qmatmul_id_ggml_prepared(void* stream, const void* x, hq_act_dtype
  * once, a tile multiplies the same activation rows with the same weight rows of both stacks, and the two f32
  * products never go to memory.  The result has the bits of hq_qmatmul_id_ggml (grouped form) twice followed by
  * hq_silu_mul.  Exists where hq_qmatmul_id_swiglu_ggml_workspace_bytes() is not 0: Q4_K / Q5_K on the grouped
- * route (at least 8 routed rows per expert and 256 rows, contiguous stacks of equal geometry); other calls return
+ * route (at least 3 routed rows per expert and 256 rows, contiguous stacks of equal geometry); other calls return
  * HQ_ERR_UNSUPPORTED and the caller issues the separate calls.  gate_row_scales / up_row_scales: both null, or both
  * from hq_weight_row_scales_ggml (n_experts * n floats each), see there. */
 HQ_API size_t hq_qmatmul_id_swiglu_ggml_workspace_bytes(uint32_t n_tokens, uint32_t top_k, uint32_t n, uint32_t k,

@@ -58,7 +58,7 @@ def test_workspace_queries_follow_the_routing():
         assert need >= 512 * 4 * kq * 2 and need % 256 == 0
         if be == 32:
             assert L.hq_qmatmul_ggml_workspace_bytes(512, 512, 96, lib.HQ_BF16, t) == 0  # k % 128 != 0: no tile kernel
-        # mul_mat_id: the grouped route wants >= 256 routed rows, >= 8 per expert and a contiguous stack
+        # mul_mat_id: the grouped route wants >= 256 routed rows, >= 3 per expert and a contiguous stack
         n, k, E = 128, 2 * kq, 8
         stride = n * (k // be) * bb
         assert L.hq_qmatmul_id_ggml_workspace_bytes(64, 4, n, k, E, stride, t) > 0

@@ -244,7 +244,7 @@ def test_mul_mat_id_many_rows(oracle, dev):
 
 # ---- grouped (expert-sorted) tile GEMM for prefill-sized mul_mat_id -------------------
 
-GROUPED_CASES = [  # (E, n, k, T, K): at least 8 routed rows per expert and 256 rows
+GROUPED_CASES = [  # (E, n, k, T, K): at least 3 routed rows per expert and 256 rows
     (8, 128, 512, 64, 4),      # 32 rows per expert: one partly filled tile each
     (4, 160, 256, 400, 3),     # 300 rows per expert: two tiles each, n not a multiple of the tile
     (16, 64, 1024, 300, 1),    # the down-projection calling form
