@@ -150,7 +150,9 @@ def quantized_matmul_swiglu_ggml(input: torch.Tensor, gate: torch.Tensor, up: to
                                  params: GgmlQuantizedMatmulParams, workspace: torch.Tensor,
                                  gate_row_scales: torch.Tensor | None = None, up_row_scales: torch.Tensor | None = None) -> None:
     """dst[m, n] = silu(input . gate^T) * (input . up^T): the two products of a dense SwiGLU layer (or of the MoE
-    block's shared expert) and the gating at prefill as one call, the bits of the three separate ones."""
+    block's shared expert) and the gating at prefill as one call: the bits of the three separate ones where the plain
+    product sums all of k in one tile (quantized_matmul_gated_workspace_bytes > 0), a few units in the last place from
+    them where it cuts k into slices."""
     if dst.dtype != torch.float32:
         raise TypeError("dst must be float32")
     for s_ in (gate_row_scales, up_row_scales):

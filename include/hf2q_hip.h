@@ -144,7 +144,11 @@ HQ_API int hq_qmatmul_gated_ggml_ws(void* stream, const void* x, hq_act_dtype xd
  * Replaces the two quantized_matmul_ggml dispatches and the silu_mul between them that the dense FFN and the shared
  * expert of the MoE block encode at prefill (gpu_ffn.rs:1236-1306, 2485-2545): one activation pre-pass, one launch of
  * tiles of 64 or 128 token rows that multiply the same activation rows with the same weight rows of both matrices;
- * the two f32 products never go to memory.  Exists where hq_qmatmul_swiglu_ggml_workspace_bytes() is not 0 (Q4_K /
+ * the two f32 products never go to memory.  The bits of the three separate calls wherever hq_qmatmul_ggml_ws sums
+ * all of k inside one tile (hq_qmatmul_gated_ggml_workspace_bytes() is not 0 for the shape); where that call cuts k
+ * into slices (up to 256 rows over few weight rows) this form still sums k in one tile, so the f32 sums associate
+ * differently and the results agree to a few units in the last place.  Exists where
+ * hq_qmatmul_swiglu_ggml_workspace_bytes() is not 0 (Q4_K /
  * Q5_K on the tile route: more rows than the small-batch kernels take, k % 256 == 0); other calls return
  * HQ_ERR_UNSUPPORTED and the caller issues the separate calls.  The separate calls run 256-row tiles from 257 rows
  * on, which use the matrix cores better: this form pays for few weight rows (the shared expert: 512) or few tokens,
