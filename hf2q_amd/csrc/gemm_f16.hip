@@ -1077,13 +1077,20 @@ __global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict_
 // Slices of k for the small tiles (bm token rows x bn weight rows): doubled while the grid has fewer workgroups than
 // the device has CUs (256) and a slice keeps at least four 256-element runs (sixteen stages, so that its prologue and
 // epilogue stay a fraction of its work), up to eight slices; k must be whole runs for that.
-inline uint32_t small_tile_splits(uint32_t m, uint32_t n, uint32_t k, uint32_t bm, uint32_t bn) {
+// The slices actually cut are ceil(nsb / sb_per) with sb_per = ceil(nsb / s): for nsb that s does not divide this can be
+// fewer than s (33 runs in eight slices of five: seven slices), and every slice then starts inside k, so no tile is
+// handed an empty or negative range of super-blocks.
+struct KSlices {
+    uint32_t splits, sb_per;
+};
+inline KSlices small_tile_splits(uint32_t m, uint32_t n, uint32_t k, uint32_t bm, uint32_t bn) {
     const uint64_t tiles = (uint64_t)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
-    const uint32_t nsb = k / 256;
+    const uint32_t nsb = (k + 255u) / 256u;
     uint32_t s = 1;
-    if (k % 256) return s;
+    if (k % 256) return KSlices{1u, nsb};
     while (s < 8 && tiles * s < 256 && nsb / (2 * s) >= 4) s *= 2;
-    return s;
+    const uint32_t sb_per = (nsb + s - 1) / s;
+    return KSlices{(nsb + sb_per - 1) / sb_per, sb_per};  // (splits - 1) * sb_per < nsb
 }
 
 // The same for Q6_K and Q8_0 / Q4_0, up to 128 token rows: tiles of 128 token rows x 128 weight rows (four waves side by
@@ -1320,9 +1327,16 @@ __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a,
 bool gemm_f16_small_tiles(hq_ggml_type t, uint32_t m) { return m <= (uint32_t)BM; }
 
 // Slices of k the small tiles of type t cut the product into (1: none).
-static uint32_t small_splits_of(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) {
+static KSlices small_slices_of(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) {
     const uint32_t bm = (t == HQ_Q4_K || t == HQ_Q5_K) && m <= (uint32_t)BM_SMALL ? BM_SMALL : m <= (uint32_t)BM_MID ? BM_MID : BM;
     return small_tile_splits(m, n, k, bm, BN_WIDE);
+}
+static uint32_t small_splits_of(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) { return small_slices_of(t, m, n, k).splits; }
+
+void gemm_f16_small_tile_slices(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k, uint32_t* splits, uint32_t* sb_per) {
+    const KSlices ks = small_slices_of(t, m, n, k);
+    *splits = ks.splits;
+    *sb_per = ks.sb_per;
 }
 
 bool gemm_f16_tile_gated_supported(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k) {
@@ -1518,7 +1532,8 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
         const bool one128 = m <= (uint32_t)BM_MID;
         void (*kern)(GemmArgs, uint32_t, uint32_t, float*) = one128 ? k128 : k256;
         const uint32_t tn = (n + BN_WIDE - 1) / BN_WIDE;
-        const uint32_t splits = small_splits_of(t, m, n, k), nsb = (k + 255u) / 256u, sb_per = (nsb + splits - 1) / splits;
+        const KSlices ks = small_slices_of(t, m, n, k);
+        const uint32_t splits = ks.splits, sb_per = ks.sb_per;
         float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
         const int lds_small = 2 * (one128 ? ActTileT<BM_MID>::kTile : ActTile::kTile);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), (size_t)lds_small, "hipFuncSetAttribute(small gemm LDS)"))
@@ -1560,7 +1575,8 @@ int launch_gemm_f16_tile(hipStream_t s, const void* x, hq_act_dtype xdt, const v
             t == HQ_Q5_K ? (mts == 2 ? q4k_gemm_small_kernel<HQ_Q5_K, 2> : mts == 4 ? q4k_gemm_small_kernel<HQ_Q5_K, 4> : q4k_gemm_small_kernel<HQ_Q5_K, 8>)
                          : (mts == 2 ? q4k_gemm_small_kernel<HQ_Q4_K, 2> : mts == 4 ? q4k_gemm_small_kernel<HQ_Q4_K, 4> : q4k_gemm_small_kernel<HQ_Q4_K, 8>);
         const uint32_t tn = (n + BN_WIDE - 1) / BN_WIDE;
-        const uint32_t splits = small_splits_of(t, m, n, k), nsb = k / 256, sb_per = (nsb + splits - 1) / splits;
+        const KSlices ks = small_slices_of(t, m, n, k);
+        const uint32_t splits = ks.splits, sb_per = ks.sb_per;
         float* partial = reinterpret_cast<float*>(ws + workspace_layout(m, n, k).total);
         const int lds_small = 2 * (mts == 2 ? ActTileT<BM_SMALL>::kTile : mts == 4 ? ActTileT<BM_MID>::kTile : ActTile::kTile);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(ksmall), (size_t)lds_small, "hipFuncSetAttribute(q4k small gemm LDS)"))

@@ -34,6 +34,7 @@
 #include "hq_internal.h"
 #include "moe_topk.h"
 #include "gemv_pieces.h"
+#include "gemv_walk.h"
 
 namespace hq {
 
@@ -569,6 +570,91 @@ bool stream_takes(uint32_t n_total, uint32_t k, uint32_t cus) {
     constexpr uint32_t W = TYPE == HQ_Q6_K ? 12 : 16;
     return k % 4096 == 0 && k <= 24576 && (uint64_t)n_total * (k / 4096) >= (uint64_t)cus * W * STREAM_MIN_ROWS_PER_WAVE;
 }
+// Activation rows one pass of the streaming kernel can stage: ROWS * (2k + k / 4) bytes of a CU's 160 KiB of LDS.
+inline uint32_t stream_rows_that_fit(uint32_t k) {
+    const size_t per_row = (size_t)k * 2 + (size_t)(k / 16) * 4;
+    const size_t fit = (160 * 1024 - 512) / per_row;
+    return fit >= 4 ? 4u : (uint32_t)fit;
+}
+
+// Dense single-row GEMV for everything the kernel above does not take: f32 activations (the dtype of the reference's
+// call sites), any k that is whole blocks (k = 2816, 2048, 11264 ...), Q8_0 / Q4_0.  One workgroup of W waves per CU, the
+// activations staged once, one window of 64 lanes per wave in flight, windows laid over the matrix as one contiguous
+// run of blocks whatever the row length (gemv_walk.h).  With two matrices of one shape over the same activations (gate
+// and up of a decode step) a wave walks the same rows of both.
+struct FArgs {
+    const void* x;
+    const uint8_t* w0;
+    const uint8_t* w1;
+    float* y0;
+    float* y1;
+    uint32_t n, k, nm;
+    FlatGeom g;
+    uint32_t m4, m2, magic;
+};
+
+template <int TYPE, bool X_BF16, int W, int D>
+__global__ __launch_bounds__(64 * W) void gemv_flat_kernel(FArgs a) {
+    using X = FlatX<TYPE, X_BF16>;
+    extern __shared__ uint4 smem[];
+    uint4* lds_x = smem;
+    float* lds_s = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(smem) + X::value_bytes(a.k));
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    // the activations first, nothing else of this workgroup in front of them
+    X::stage(a.x, a.k, lds_x, lds_s, tid, 64u * W);
+    FlatWalk<TYPE, X_BF16, D> wk;
+    wk.init(a.w0, a.w1, a.n, a.nm, a.g, wv * gridDim.x + blockIdx.x, W * gridDim.x);
+    wk.prime();
+    __syncthreads();
+    wk.load_masks(a.m4, a.m2, a.magic);
+    wk.run(lds_x, lds_s, [&](uint32_t first, uint32_t cnt, float k0, float k1) {
+        if (lane < cnt) {
+            const uint32_t row = wk.row_of_slot(first + lane);
+            if (row < a.n) {
+                a.y0[row] = k0;
+                if (a.nm == 2u) a.y1[row] = k1;
+            }
+        }
+    });
+}
+
+#ifndef HQ_FLAT_MIN_WINDOWS_PER_CU
+#define HQ_FLAT_MIN_WINDOWS_PER_CU 8
+#endif
+#ifndef HQ_FLAT_D_Q80
+#define HQ_FLAT_D_Q80 1
+#endif
+#ifndef HQ_FLAT_D_Q40
+#define HQ_FLAT_D_Q40 1
+#endif
+// Whether the flat form takes (type, rows, k): about a window per wave of the device or more, block counts that fit 32 bits.
+template <int TYPE>
+bool flat_takes(uint64_t n_total, uint32_t k, uint32_t cus, size_t lds) {
+    constexpr uint32_t UE = kUnitElems<TYPE>, UW = kUnitsPerWindow<TYPE>;
+    if (k % UE || k / UE < 2 || lds > 160 * 1024 - 512) return false;
+    const uint64_t units = n_total * (k / UE);
+    return units < 0x7fff0000ull && units / UW >= (uint64_t)cus * HQ_FLAT_MIN_WINDOWS_PER_CU;
+}
+// Fetches a wave keeps in flight: one (a ring of two or four windows of 32-weight blocks, which are only 1.1 / 2.2 KB,
+// measured slower: Q4_0 12288 x 4096 13.8 against 9.7 us).
+template <int TYPE>
+constexpr int kFlatDepth = TYPE == HQ_Q8_0 ? HQ_FLAT_D_Q80 : TYPE == HQ_Q4_0 ? HQ_FLAT_D_Q40 : 1;
+
+template <int TYPE, bool X_BF16>
+int launch_flat(hipStream_t s, const void* x, const uint8_t* w0, const uint8_t* w1, float* y0, float* y1, uint32_t n, uint32_t k,
+                uint32_t nm, uint32_t cus) {
+    constexpr int W = (TYPE == HQ_Q6_K && X_BF16) ? 12 : 16;
+    using X = FlatX<TYPE, X_BF16>;
+    const FArgs fa{x, w0, w1, y0, y1, n, k, nm, flat_geom(k, kUnitElems<TYPE>, kUnitsPerWindow<TYPE>, n, nm, cus * W),
+                   TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
+    auto kern = gemv_flat_kernel<TYPE, X_BF16, W, kFlatDepth<TYPE>>;
+    size_t lds = X::lds_bytes(k);
+    if (lds < 81 * 1024) lds = 81 * 1024;  // more than half a CU's LDS: one workgroup per CU
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv flat LDS)")) return rc;
+    hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, fa);
+    return check_launch("gemv flat kernel launch");
+}
 
 template <typename K>
 int set_lds_limit(K kern, size_t lds, const char* what) {
@@ -633,7 +719,7 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
             for (uint32_t r = 0; r < a.pairs;) {
                 const SArgs sa{static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * 2, a.w, a.w, a.y + (size_t)r * a.n, a.y + (size_t)r * a.n,
                                a.n, a.n, a.k, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
-                const uint32_t left = a.pairs - r, take = left >= 4 ? 4 : left;
+                const uint32_t fit = stream_rows_that_fit(a.k), left = a.pairs - r, take = left >= fit ? fit : left;
                 if (int rc = take == 4   ? launch_stream<TYPE, 4>(s, sa, cus)
                              : take == 3 ? launch_stream<TYPE, 3>(s, sa, cus)
                              : take == 2 ? launch_stream<TYPE, 2>(s, sa, cus)
@@ -643,6 +729,15 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
             }
             return HQ_OK;
         }
+    }
+    // Other dense matrices with enough rows (any k of whole blocks, f32 activations, Q8_0 / Q4_0): the flat streaming form,
+    // one pass per activation row.
+    if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && flat_takes<TYPE>(a.n, a.k, cus, FlatX<TYPE, X_BF16>::lds_bytes(a.k))) {
+        for (uint32_t r = 0; r < a.pairs; ++r)
+            if (int rc = launch_flat<TYPE, X_BF16>(s, static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * (X_BF16 ? 2 : 4), a.w, a.w,
+                                                   a.y + (size_t)r * a.n, a.y + (size_t)r * a.n, a.n, a.k, 1, cus))
+                return rc;
+        return HQ_OK;
     }
     // Dense matrices with many tasks per wave: the queue kernel.
     if (a.pairs == 1 && !a.x2 && !a.ids && !a.route_logits &&
@@ -691,6 +786,13 @@ int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
         auto plain = [](const GemvArgs& j) { return j.pairs == 1 && !j.x2 && !j.ids && !j.route_logits; };
         if (n_jobs == 2 && plain(j0) && plain(j1) && j0.x == j1.x && j0.k == j1.k && stream_takes<TYPE>(j0.n + j1.n, j0.k, cus))
             return launch_stream<TYPE>(s, SArgs{j0.x, j0.w, j1.w, j0.y, j1.y, j0.n, j0.n + j1.n, j0.k, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC}, cus);
+    }
+    {
+        const GemvArgs &j0 = jobs[0], &j1 = jobs[1];
+        auto plain = [](const GemvArgs& j) { return j.pairs == 1 && !j.x2 && !j.ids && !j.route_logits; };
+        if (n_jobs == 2 && plain(j0) && plain(j1) && j0.x == j1.x && j0.k == j1.k && j0.n == j1.n &&
+            flat_takes<TYPE>((uint64_t)j0.n * 2, j0.k, cus, FlatX<TYPE, X_BF16>::lds_bytes(j0.k)))
+            return launch_flat<TYPE, X_BF16>(s, j0.x, j0.w, j1.w, j0.y, j1.y, j0.n, j0.k, 2, cus);
     }
     const uint64_t per_simd = slots / (4ull * cus);
     if (per_simd >= 8) return launch_j<TYPE, X_BF16, PAIR, 4, 4>(s, js, n_jobs, lds);

@@ -167,6 +167,26 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q6_K>& p, int c, const 
     return d * acc;
 }
 
+// Q4_0: y = d * (q - 8); low nibbles are elements 0..15 of the block, high nibbles 16..31; values hold 128 + q.
+// xp: 16 paired words = the block's 32 activations, sx: the sums of its two runs of sixteen.
+__device__ __forceinline__ float dot_pair(const Piece<HQ_Q4_0>& p, int, const uint32_t* xp, const float* sx, uint32_t m4,
+                                          uint32_t, uint32_t magic) {
+    float lo = 0.f, hi = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t w = word(p.q, j);
+        lo = dot2_bf16((w & m4) | magic, xp[2 * j], lo);
+        lo = dot2_bf16(((w >> 8) & m4) | magic, xp[2 * j + 1], lo);
+        hi = dot2_bf16(((w >> 4) & m4) | magic, xp[8 + 2 * j], hi);
+        hi = dot2_bf16(((w >> 12) & m4) | magic, xp[8 + 2 * j + 1], hi);
+    }
+    return f16_bits_to_f32(p.d) * ((lo + hi) - 136.f * (sx[0] + sx[1]));
+}
+// (Q8_0 has no paired form: 128 + q needs eight mantissa bits beside the leading one, bf16 has seven.)
+__device__ __forceinline__ float dot_pair(const Piece<HQ_Q8_0>&, int, const uint32_t*, const float*, uint32_t, uint32_t, uint32_t) {
+    return 0.f;
+}
+
 // ---- f32 activations (xf: this lane's 64 (32 for Q8_0) activations, sx: run sums) ----
 __device__ __forceinline__ float dot4(uint32_t q, const float* x, float acc) {
     // q is a word of four masked bytes; hidden from the optimiser, which would otherwise fold the mask into a bit-field

@@ -1,0 +1,304 @@
+// The streaming row walk shared by the dense GEMV of any k (gemv.hip) and the one-launch dense FFN block
+// (dense_ffn.hip).
+//
+// A weight matrix [n][k] of GGML blocks is one contiguous run of units (a unit = one 256-weight super-block of a
+// K-quant, four lanes, or one 32-weight block of Q8_0 / Q4_0, one lane).  A wave reads it in WINDOWS of 64 lanes =
+// 16 super-blocks (2304 .. 3360 contiguous bytes) or 64 blocks (1152 / 2176 bytes), whatever the row length is:
+// a window may start and end in the middle of a row.  Windows are grouped into SUPER-TASKS of R whole rows = ST windows
+// (R a power of two; the host picks R and the units per window, flat_geom below); a wave owns super-tasks first,
+// first + stride, ...  After the dot products of a window the
+// lanes' partial sums are added per row (one masked wave reduction for every row the window touches) into the
+// lane that keeps that row's result; 64 finished rows leave through one call of the caller's output functor.
+//
+// One fetch per wave is in flight (D = 1), or a ring of D; every fetch is unconditional (past the wave's last task it
+// repeats the last one) and its address is clamped to the matrix, so the loop has one path and no branch around a load.
+#pragma once
+
+#include "gemv_pieces.h"
+
+namespace hq {
+namespace {
+
+template <int TYPE>
+constexpr uint32_t kLanesPerUnit = kBlock32<TYPE> ? 1u : 4u;
+template <int TYPE>
+constexpr uint32_t kUnitsPerWindow = 64u / kLanesPerUnit<TYPE>;
+template <int TYPE>
+constexpr uint32_t kUnitElems = kBlock32<TYPE> ? 32u : 256u;
+
+struct FlatGeom {
+    uint32_t bu;     // units per row
+    uint32_t magic;  // ceil(2^32 / bu): v / bu == umulhi(v, magic) while v * bu < 2^32
+    uint32_t log_r;  // a super-task is 1 << log_r rows ...
+    uint32_t st;     // ... = st windows ...
+    uint32_t uwe;    // ... of uwe <= UW units each (the lanes past uwe * lanes-per-unit idle)
+};
+
+// The window width and the rows per super-task for a matrix of n rows (nm matrices walked side by side) on `waves` waves.
+// Full windows (uwe = uw) waste no lane but tie R = uw / gcd(bu, uw) rows together, which leaves waves without work when
+// n / R is small (k = 2816: 11 super-blocks per row, R = 16); narrower windows that divide R * bu for a smaller R (11 of 16
+// units: one row per window) spread the rows over more waves at the price of idle lanes.  Chosen: the pair with the fewest
+// windows on the busiest wave, then the fewest windows in all.
+inline FlatGeom flat_geom(uint32_t k, uint32_t unit_elems, uint32_t uw, uint32_t n, uint32_t nm, uint32_t waves) {
+    FlatGeom g{};
+    g.bu = k / unit_elems;
+    g.magic = (uint32_t)((0x100000000ull + g.bu - 1) / g.bu);  // bu >= 2
+    uint64_t best_crit = ~0ull, best_total = ~0ull;
+    for (uint32_t log_r = 0; (1u << log_r) <= uw; ++log_r) {
+        const uint32_t r = 1u << log_r;
+        uint32_t uwe = uw;
+        while ((r * g.bu) % uwe) --uwe;
+        const uint32_t st = r * g.bu / uwe;
+        const uint64_t n_super = (n + r - 1) / r;
+        const uint64_t crit = ((n_super + waves - 1) / waves) * nm * st, total = n_super * nm * st;
+        if (crit < best_crit || (crit == best_crit && total < best_total)) {
+            best_crit = crit;
+            best_total = total;
+            g.log_r = log_r;
+            g.st = st;
+            g.uwe = uwe;
+        }
+    }
+    return g;
+}
+
+// ---- activations of one row in LDS: the values in the order the dot products read them + per-16 sums ----
+// PAIR (bf16 activations; K-quants and Q4_0): pre-paired bf16 words, 16-byte chunks of 8 activations, for
+// v_dot2c_f32_bf16.  Otherwise f32 values (f32 activations; bf16 ones widened for Q8_0), 16-byte chunks of 4.  A lane reads
+// the chunks of its piece one after the other, sixteen lanes of a ds_read_b128 at a time: the pieces are padded apart
+// (one chunk per piece; Q6_K, whose lane reads four runs of a super-block: 36 / 81 chunks per super-block with the
+// halves 17 / 40 apart) so that those sixteen lanes hit sixteen different 16-byte bank groups and every chunk of a
+// piece is an immediate offset from the lane's one base address.
+template <int TYPE, bool X_BF16>
+struct FlatX {
+    static constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
+    static constexpr int XW = PAIR ? (kBlock32<TYPE> ? 16 : 32) : (kBlock32<TYPE> ? 32 : 64);  // registers of one lane's activations
+    static constexpr uint32_t CA = PAIR ? 8u : 4u;                                              // activations per chunk
+    static constexpr uint32_t G = (kBlock32<TYPE> ? 32u : 64u) / CA;                             // chunks per piece
+
+    // LDS slot of chunk ch
+    static __host__ __device__ __forceinline__ uint32_t slot(uint32_t ch) {
+        if constexpr (TYPE == HQ_Q6_K) {
+            if constexpr (PAIR) return (ch >> 5) * 36u + ((ch >> 4) & 1u) * 17u + (ch & 15u);
+            return (ch >> 6) * 81u + ((ch >> 5) & 1u) * 40u + (ch & 31u);
+        } else {
+            return ch + ch / G;
+        }
+    }
+    static __host__ __device__ __forceinline__ size_t value_bytes(uint32_t k) { return (size_t)slot(k / CA) * 16; }
+    static __host__ __device__ __forceinline__ size_t lds_bytes(uint32_t k) { return value_bytes(k) + (size_t)(k / 16) * 4; }
+
+    // 16 activations per thread and pass; the sum of a run of sixteen adds them in index order.
+    static __device__ __forceinline__ void stage(const void* x, uint32_t k, uint4* lds_x, float* lds_s, uint32_t tid,
+                                                 uint32_t nthreads) {
+        for (uint32_t i = tid; i < k / 16u; i += nthreads) {
+            XRaw<X_BF16> raw;
+            raw.fetch(x, i);
+            float v[16];
+            if constexpr (X_BF16) {
+                const uint4 p = raw.r[0], q = raw.r[1];
+                const uint32_t w[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    v[2 * j] = bf16_bits_to_f32(w[j] & 0xffffu);
+                    v[2 * j + 1] = bf16_bits_to_f32(w[j] >> 16);
+                }
+                if constexpr (PAIR) {
+                    uint4 o0, o1;
+                    o0.x = (w[0] & 0xffffu) | (w[1] << 16);
+                    o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
+                    o0.z = (w[2] & 0xffffu) | (w[3] << 16);
+                    o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
+                    o1.x = (w[4] & 0xffffu) | (w[5] << 16);
+                    o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
+                    o1.z = (w[6] & 0xffffu) | (w[7] << 16);
+                    o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
+                    lds_x[slot(2 * i)] = o0;
+                    lds_x[slot(2 * i + 1)] = o1;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    v[4 * j] = __uint_as_float(raw.r[j].x);
+                    v[4 * j + 1] = __uint_as_float(raw.r[j].y);
+                    v[4 * j + 2] = __uint_as_float(raw.r[j].z);
+                    v[4 * j + 3] = __uint_as_float(raw.r[j].w);
+                }
+            }
+            if constexpr (!PAIR) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    reinterpret_cast<float4*>(lds_x)[slot(4 * i + j)] = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
+            }
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s += v[j];
+            lds_s[i] = s;
+        }
+    }
+
+    // The activations of the lane's piece: unit `ur` of the row, sub-piece c (K-quants: the lane's quarter).
+    static __device__ __forceinline__ void load(const uint4* lds_x, const float* lds_s, uint32_t ur, int c, uint32_t* xr,
+                                                float* sx) {
+        auto put = [&](int at, const uint4 v) {
+            xr[at] = v.x;
+            xr[at + 1] = v.y;
+            xr[at + 2] = v.z;
+            xr[at + 3] = v.w;
+        };
+        if constexpr (TYPE == HQ_Q6_K) {
+            // four runs of 16 activations, 32 apart, in the half (c >> 1) of the super-block, starting at 16 * (c & 1)
+            constexpr int CR = 16 / (int)CA;  // chunks per run
+            const uint4* base = lds_x + (PAIR ? ur * 36u + (uint32_t)(c >> 1) * 17u : ur * 81u + (uint32_t)(c >> 1) * 40u) +
+                                (uint32_t)(c & 1) * CR;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+#pragma unroll
+                for (int u = 0; u < CR; ++u) put((CR * r + u) * 4, base[2 * CR * r + u]);
+                sx[r] = lds_s[ur * 16u + (uint32_t)(c >> 1) * 8u + (uint32_t)(c & 1) + 2u * r];
+            }
+        } else {
+            const uint32_t piece = kBlock32<TYPE> ? ur : ur * 4u + (uint32_t)c;
+            const uint4* base = lds_x + piece * (G + 1u);
+#pragma unroll
+            for (int j = 0; j < (int)G; ++j) put(4 * j, base[j]);
+            constexpr int RUNS = kBlock32<TYPE> ? 2 : 4;
+#pragma unroll
+            for (int r = 0; r < RUNS; ++r) sx[r] = lds_s[piece * RUNS + r];
+        }
+    }
+};
+
+template <int TYPE, bool X_BF16, int D = 1>
+struct FlatWalk {
+    using X = FlatX<TYPE, X_BF16>;
+    static constexpr uint32_t LPU = kLanesPerUnit<TYPE>, UW = kUnitsPerWindow<TYPE>, BB = kBlockBytes<TYPE>;
+
+    const uint8_t* w0;
+    const uint8_t* w1;       // second matrix of the same shape (nm == 2), walked super-task by super-task beside the first
+    uint32_t nrows, nm;
+    FlatGeom g;
+    uint32_t first, stride, count;  // this wave's super-tasks: first + i * stride, i < count
+    uint32_t lane, lv;  // lv: the lane's unit inside a window (idle lanes: the last active one's)
+    bool active;
+    int c;
+    uint32_t m4, m2, magic;
+    uint32_t f_i, f_m, f_w, f_left;  // the next task to fetch; tasks not yet fetched
+    Piece<TYPE> buf[D];
+
+    __device__ __forceinline__ void init(const uint8_t* wa, const uint8_t* wb, uint32_t n, uint32_t n_matrices, const FlatGeom& geom,
+                                         uint32_t first_super, uint32_t super_stride) {
+        w0 = wa;
+        w1 = wb;
+        nrows = n;
+        nm = n_matrices;
+        g = geom;
+        lane = threadIdx.x & 63u;
+        c = (int)(lane & 3u);
+        active = lane / LPU < g.uwe;
+        lv = active ? lane / LPU : g.uwe - 1u;
+        const uint32_t n_super = (n + (1u << g.log_r) - 1u) >> g.log_r;
+        first = first_super;
+        stride = super_stride;
+        count = first < n_super ? (n_super - first + stride - 1u) / stride : 0u;
+        f_i = f_m = f_w = 0;
+        f_left = tasks();
+    }
+    __device__ __forceinline__ uint32_t tasks() const { return count * nm * g.st; }
+
+    // The conversion masks of the paired-bf16 dot products must sit in VGPRs (v_and_or_b32 takes one scalar operand at
+    // most); the copy is opaque so they stay there.
+    __device__ __forceinline__ void load_masks(uint32_t a_m4, uint32_t a_m2, uint32_t a_magic) {
+        asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
+                     : "=v"(m4), "=v"(m2), "=v"(magic)
+                     : "s"(a_m4), "s"(a_m2), "s"(a_magic));
+    }
+
+    __device__ __forceinline__ void fetch_next(Piece<TYPE>& p) {
+        const uint32_t sid = first + f_i * stride;
+        uint32_t u = (sid << g.log_r) * g.bu + g.uwe * f_w + lv;
+        const uint32_t last = nrows * g.bu - 1u;
+        u = u < last ? u : last;
+        const uint8_t* base = f_m ? w1 : w0;
+        p.load(base + (size_t)u * BB, c);
+        if (f_left > 1u) {  // (scalar: no memory operation inside)
+            --f_left;
+            if (++f_w == g.st) {
+                f_w = 0;
+                if (++f_m == nm) {
+                    f_m = 0;
+                    ++f_i;
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void prime() {
+        if (tasks()) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) fetch_next(buf[d]);
+        }
+    }
+
+    // Row of the wave's j-th finished row (the order in which results reach the output functor).
+    __device__ __forceinline__ uint32_t row_of_slot(uint32_t j) const {
+        return ((first + (j >> g.log_r) * stride) << g.log_r) + (j & ((1u << g.log_r) - 1u));
+    }
+
+    // out(first_slot, count, keep0, keep1): lane l < count holds the sums of row_of_slot(first_slot + l) over the first
+    // (keep0) and the second matrix (keep1).
+    template <typename OUT>
+    __device__ __forceinline__ void run(const uint4* lds_x, const float* lds_s, OUT&& out) {
+        const uint32_t ntask = tasks();
+        uint32_t c_m = 0, c_w = 0, done = 0;
+        float keep0 = 0.f, keep1 = 0.f;
+        uint32_t xr[X::XW];
+        float sx[4] = {0.f, 0.f, 0.f, 0.f};
+        const bool xinv = g.st == 1u && g.log_r == 0u;  // every window is one whole row: the lane's activations never change
+        if (xinv) X::load(lds_x, lds_s, lv, c, xr, sx);
+        const int last_lane = (int)(g.uwe * LPU - 1u);
+        for (uint32_t t = 0; t < ntask; t += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                Piece<TYPE>& p = buf[d];
+                const uint32_t lu = g.uwe * c_w + lv;
+                uint32_t lrow = __umulhi(lu, g.magic);
+                const uint32_t ur = lu - lrow * g.bu;
+                if (!xinv) X::load(lds_x, lds_s, ur, c, xr, sx);
+                float part;
+                if constexpr (X::PAIR)
+                    part = dot_pair(p, c, xr, sx, m4, m2, magic);
+                else
+                    part = dot_f32(p, c, reinterpret_cast<const float*>(xr), sx);
+                asm volatile("" : "+v"(part));  // the refill follows the arithmetic that frees its registers
+                fetch_next(p);
+                const bool live = D == 1 || t + (uint32_t)d < ntask;  // (a ring's last round may run past the end)
+                const uint32_t r_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)lrow);
+                const uint32_t r_hi = (uint32_t)__builtin_amdgcn_readlane((int)lrow, last_lane);
+                lrow = active ? lrow : 0xffffffffu;  // an idle lane's duplicate belongs to no row
+                for (uint32_t r = r_lo; r <= r_hi; ++r) {
+                    float v = lrow == r ? part : 0.f;
+                    v = group_sum(v, 6);
+                    const bool mine = live && lane == ((done + r) & 63u);
+                    keep0 = mine && c_m == 0u ? keep0 + v : keep0;
+                    keep1 = mine && c_m != 0u ? keep1 + v : keep1;
+                }
+                if (live && ++c_w == g.st) {
+                    c_w = 0;
+                    if (++c_m == nm) {
+                        c_m = 0;
+                        done += 1u << g.log_r;
+                        if ((done & 63u) == 0u) {
+                            out(done - 64u, 64u, keep0, keep1);
+                            keep0 = keep1 = 0.f;
+                        }
+                    }
+                }
+            }
+        }
+        if (done & 63u) out(done & ~63u, done & 63u, keep0, keep1);
+    }
+};
+
+}  // namespace
+}  // namespace hq

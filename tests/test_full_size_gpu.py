@@ -11,7 +11,8 @@ import torch
 
 from _util import assert_matmul_close, assert_matmul_close_f16_tile
 from hf2q_amd import ops
-from hf2q_amd.ops import HQ_Q4_K, HQ_Q6_K, HQ_Q8_0, FlashAttnVecTqHbParams, GgmlQuantizedMatmulParams
+from hf2q_amd.ops import (HQ_Q4_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, FlashAttnVecTqHbParams,
+                          GgmlQuantizedMatmulParams)
 
 pytestmark = pytest.mark.gpu
 
@@ -61,6 +62,65 @@ def test_decode_gemv_full_size(oracle, dev, n, k, t, m):
     assert (yab - (ya + yb)).abs().max().item() <= 2e-5 * scale
     # (c) exact scaling by a power of two
     assert torch.equal(run(xa * 4.0), ya * 4.0)
+
+
+# The reference's own decode shapes and dtype: f32 activations (gpu_full_attn.rs:835), k = 2816 (Gemma-4 projections, 11
+# super-blocks per row: windows of the streaming walk straddle rows) and k = 2048 (Qwen3.6 hidden: two rows per window), and
+# the 32-weight-block types; plus k = 4096 with f32 activations.  All of them take the flat streaming GEMV.
+FLAT_SHAPES = [(12288, 2816), (16384, 2048), (12288, 4096), (4099, 11264), (4096, 2816), (2816, 4096), (1500, 8960)]
+
+
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0])
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("n,k", FLAT_SHAPES)
+def test_decode_gemv_any_k_and_dtype(oracle, dev, t, xdt, n, k):
+    w = _quantized(dev, n, k, t, 11 + n + k)
+    rng = np.random.default_rng(n + k + t)
+    m = 2 if (n, k) == (16384, 2048) else 1
+    xa = (rng.integers(-12, 13, (m, k)) / 8.0).astype(np.float32)  # exact in bf16
+    xb = (rng.integers(-12, 13, (m, k)) / 8.0).astype(np.float32)
+    if xdt == "f32":  # values that need all of f32's 24 bits
+        xa = (xa + rng.standard_normal((m, k)) * 1e-3).astype(np.float32)
+        xb = (xb + rng.standard_normal((m, k)) * 1e-3).astype(np.float32)
+    p = GgmlQuantizedMatmulParams(m, n, k, t)
+
+    def run(x):
+        y = torch.full((m, n), float("nan"), device=dev)
+        xd = torch.from_numpy(x).to(dev)
+        ops.quantized_matmul_ggml(xd.to(torch.bfloat16) if xdt == "bf16" else xd, w, y, p)
+        return y
+
+    ya, yb, yab = run(xa), run(xb), run((xa + xb).astype(np.float32))
+    assert torch.isfinite(yab).all()
+    rows = np.unique(np.concatenate([[0, 1, 2, 15, 16, 17, n - 3, n - 2, n - 1], rng.integers(0, n, 80)]))
+    xin = oracle.f32_to_bf16_bits(xa) if xdt == "bf16" else xa
+    ref = oracle.qmatmul_f64(xin, _rows_of(w, rows, k, t, oracle), m, rows.size, k, t)
+    assert_matmul_close(ya[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, f"gemv {n}x{k} t={t} {xdt}, sampled rows")
+    scale = yab.abs().max().item()
+    assert (yab - (ya + yb)).abs().max().item() <= 2e-5 * scale
+    assert torch.equal(run(xa * 4.0), ya * 4.0)
+
+
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q8_0])
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+def test_gate_and_up_in_one_launch_any_k(oracle, dev, t, xdt):
+    """Two matrices of one shape over the same activations as one batched launch: the bits of the two separate calls."""
+    n, k = 12288, 2816
+    wg, wu = _quantized(dev, n, k, t, 5), _quantized(dev, n, k, t, 6)
+    g = torch.Generator(device=dev)
+    g.manual_seed(9)
+    x = torch.randn(1, k, generator=g, device=dev)
+    x = x.to(torch.bfloat16) if xdt == "bf16" else x
+    p = GgmlQuantizedMatmulParams(1, n, k, t)
+    yg, yu, bg, bu = (torch.full((1, n), float("nan"), device=dev) for _ in range(4))
+    ops.quantized_matmul_ggml(x, wg, yg, p)
+    ops.quantized_matmul_ggml(x, wu, yu, p)
+    ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x, wg, bg, 1, n, k), ops.QmatmulJob(x, wu, bu, 1, n, k)], t)
+    assert torch.equal(yg, bg) and torch.equal(yu, bu)
+    rows = np.arange(0, n, 397)
+    xin = oracle.f32_to_bf16_bits(x.float().cpu().numpy()) if xdt == "bf16" else x.cpu().numpy()
+    ref = oracle.qmatmul_f64(xin, _rows_of(wu, rows, k, t, oracle), 1, rows.size, k, t)
+    assert_matmul_close(bu[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, "up of the pair")
 
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q8_0])
