@@ -143,12 +143,15 @@ extern "C" {
     pub fn hq_dequant_ggml(stream: *mut c_void, w_blocks: *const c_void, out: *mut c_void, out_dtype: hq_act_dtype, n_elems: u64, t: hq_ggml_type) -> c_int;
     pub fn hq_quantize_ggml(stream: *mut c_void, src: *const f32, n_elems: u64, n_per_row: u64, t: hq_ggml_type, out_blocks: *mut c_void) -> c_int;
     pub fn hq_qmatmul_ggml(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type) -> c_int;
+    pub fn hq_qmatmul_ggml_k_slices(m: u32, n: u32, k: u32, t: hq_ggml_type, slices: *mut u32, blocks_per_slice: *mut u32) -> c_int;
     pub fn hq_qmatmul_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;
     pub fn hq_qmatmul_ggml_ws(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
     pub fn hq_qmatmul_gated_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;
     pub fn hq_qmatmul_gated_ggml_ws(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, w_row_scales: *const f32, gate: *const f32, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
     pub fn hq_qmatmul_swiglu_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;
     pub fn hq_qmatmul_swiglu_ggml_ws(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_gate: *const c_void, w_up: *const c_void, gate_row_scales: *const f32, up_row_scales: *const f32, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
+    pub fn hq_qmatmul_swiglu_decode_supported(n: u32, k: u32, t: hq_ggml_type, xdt: hq_act_dtype) -> c_int;
+    pub fn hq_qmatmul_swiglu_decode(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_gate: *const c_void, w_up: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type) -> c_int;
     pub fn hq_qmatmul_perm021_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;
     pub fn hq_qmatmul_perm021_ggml_ws(stream: *mut c_void, x_perm: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, head_dim: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
     pub fn hq_qmatmul_id_ggml(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_stack: *const c_void, ids: *const u32, y: *mut f32, scratch: *mut c_void, scratch_bytes: usize, n_tokens: u32, top_k: u32, n: u32, k: u32, n_experts: u32, expert_stride: u64, t: hq_ggml_type) -> c_int;
@@ -167,6 +170,10 @@ extern "C" {
     pub fn hq_moe_weighted_reduce(stream: *mut c_void, y: *const f32, w: *const f32, shared: *const f32, shared_logit: *const f32, residual: *const f32, out: *mut f32, n_tokens: u32, top_k: u32, hidden: u32) -> c_int;
     pub fn hq_moe_ffn_decode_scratch_bytes(n_tokens: u32, hidden: u32, n_experts: u32, top_k: u32, inter: u32, shared_inter: u32, t: hq_ggml_type, xdt: hq_act_dtype) -> usize;
     pub fn hq_moe_ffn_decode(stream: *mut c_void, layer: *const hq_moe_ffn_layer, x: *const c_void, xdt: hq_act_dtype, residual: *const f32, out: *mut f32, n_tokens: u32, scratch: *mut c_void, scratch_bytes: usize, route_ids: *mut u32, route_weights: *mut f32) -> c_int;
+    pub fn hq_handover_status(stream: *mut c_void, scratch: *const c_void, error: *mut u32) -> c_int;
+    pub fn hq_set_handover_spin_limit(limit: u32);
+    pub fn hq_dense_ffn_decode_scratch_bytes(hidden: u32, inter: u32, t_gate_up: hq_ggml_type, t_down: hq_ggml_type, xdt: hq_act_dtype) -> usize;
+    pub fn hq_dense_ffn_decode(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_gate: *const c_void, w_up: *const c_void, w_down: *const c_void, t_gate_up: hq_ggml_type, t_down: hq_ggml_type, residual: *const f32, out: *mut f32, hidden: u32, inter: u32, scratch: *mut c_void, scratch_bytes: usize) -> c_int;
     pub fn hq_fwht_sign_premult_f32(stream: *mut c_void, buf: *mut f32, n_heads: u32, head_dim: u32) -> c_int;
     pub fn hq_fwht_sign_undo_f32(stream: *mut c_void, buf: *mut f32, n_heads: u32, head_dim: u32) -> c_int;
     pub fn hq_tq_encode_kv(stream: *mut c_void, src: *const f32, codes: *mut u8, norms: *mut f32, n_tokens: u32, n_kv_heads: u32, head_dim: u32, capacity: u32, write_pos: u32) -> c_int;

@@ -5,6 +5,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "hq_internal.h"
@@ -91,6 +92,9 @@ int cu_count(uint32_t* out) {
 }  // namespace hq
 
 using namespace hq;
+
+// Polling limit of the in-launch hand-overs (0: the kernels' default); see hq_set_handover_spin_limit.
+static std::atomic<uint32_t> g_spin_limit{0};
 
 extern "C" {
 
@@ -243,6 +247,16 @@ int qmatmul_ws(const char* fn, void* stream, const void* x, hq_act_dtype xdt, co
 }
 }  // namespace
 
+int hq_qmatmul_ggml_k_slices(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, uint32_t* slices, uint32_t* blocks_per_slice) {
+    if (!slices || !blocks_per_slice) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_ggml_k_slices: null output");
+    if (!known_type(t) || n == 0 || k == 0 || k % hq_block_elems(t))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_qmatmul_ggml_k_slices: type %d, n %u, k %u", (int)t, n, k);
+    *slices = 1;
+    *blocks_per_slice = (k + 255u) / 256u;
+    if (f16_tile_route(m, k, t) && m <= 256) gemm_f16_small_tile_slices(t, m, n, k, slices, blocks_per_slice);
+    return HQ_OK;
+}
+
 int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
                        uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes) {
     return qmatmul_ws("hq_qmatmul_ggml_ws", stream, x, xdt, w_blocks, nullptr, y, m, n, k, t, workspace, workspace_bytes);
@@ -333,6 +347,22 @@ int hq_qmatmul_swiglu_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, con
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes, %zu needed", fn, workspace ? workspace_bytes : (size_t)0, need);
     if (reinterpret_cast<uintptr_t>(workspace) % 256) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace must be 256-byte aligned", fn);
     return launch_gemm_f16_swiglu((hipStream_t)stream, x, xdt, w_gate, w_up, y, m, n, k, t, workspace, gate_row_scales, up_row_scales);
+}
+
+int hq_qmatmul_swiglu_decode_supported(uint32_t n, uint32_t k, hq_ggml_type t, hq_act_dtype xdt) {
+    if (!known_type(t) || (xdt != HQ_F32 && xdt != HQ_BF16) || n == 0 || k == 0 || k % hq_block_elems(t)) return 0;
+    return launch_gemv_swiglu(nullptr, nullptr, xdt, nullptr, nullptr, nullptr, 1, n, k, t, true) == HQ_OK;
+}
+
+int hq_qmatmul_swiglu_decode(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up, float* y, uint32_t m,
+                             uint32_t n, uint32_t k, hq_ggml_type t) {
+    const char* fn = "hq_qmatmul_swiglu_decode";
+    if (int rc = check_matmul_common(fn, x, xdt, w_gate, y, n, k, t)) return rc;
+    if (!w_up) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (int rc = check_weight_alignment(w_up, t)) return rc;
+    if (m > kGemvMaxRows) return fail(HQ_ERR_UNSUPPORTED, "%s: %u rows (limit %u; hq_qmatmul_swiglu_ggml_ws is the prefill form)", fn, m, kGemvMaxRows);
+    if (m == 0) return HQ_OK;
+    return launch_gemv_swiglu((hipStream_t)stream, x, xdt, w_gate, w_up, y, m, n, k, t, false);
 }
 
 size_t hq_qmatmul_perm021_ggml_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_ggml_type t) {
@@ -613,8 +643,57 @@ int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* l, const void* x, hq
     a.top_k = l->top_k;
     a.stride_gate_up = l->expert_stride_gate_up;
     a.stride_down = l->expert_stride_down;
-    a.spin_limit = 0;
+    a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
     return launch_moe_fused((hipStream_t)stream, a);
+}
+
+void hq_set_handover_spin_limit(uint32_t limit) { g_spin_limit.store(limit, std::memory_order_relaxed); }
+
+int hq_handover_status(void* stream, const void* scratch, uint32_t* error) {
+    if (!scratch || !error) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_handover_status: null argument");
+    if (int rc = check_hip(hipMemcpyAsync(error, static_cast<const uint8_t*>(scratch) + 4, 4, hipMemcpyDeviceToHost, (hipStream_t)stream),
+                           "hipMemcpyAsync(hand-over error word)"))
+        return rc;
+    return check_hip(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize(hand-over status)");
+}
+
+static int dense_ffn_args(const char* fn, DenseFfnArgs* a, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up,
+                          const void* w_down, hq_ggml_type t_gate_up, hq_ggml_type t_down, const float* residual, float* out,
+                          uint32_t hidden, uint32_t inter, void* scratch) {
+    if (!known_type(t_gate_up) || !known_type(t_down)) return fail(HQ_ERR_UNSUPPORTED, "%s: ggml types %d / %d", fn, (int)t_gate_up, (int)t_down);
+    if (xdt != HQ_F32 && xdt != HQ_BF16) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: activation dtype %d", fn, (int)xdt);
+    *a = DenseFfnArgs{x, xdt, w_gate, w_up, w_down, t_gate_up, t_down, residual, out, scratch, hidden, inter,
+                      g_spin_limit.load(std::memory_order_relaxed)};
+    return HQ_OK;
+}
+
+size_t hq_dense_ffn_decode_scratch_bytes(uint32_t hidden, uint32_t inter, hq_ggml_type t_gate_up, hq_ggml_type t_down, hq_act_dtype xdt) {
+    DenseFfnArgs a;
+    if (hidden == 0 || inter == 0) return 0;
+    if (dense_ffn_args("hq_dense_ffn_decode_scratch_bytes", &a, nullptr, xdt, nullptr, nullptr, nullptr, t_gate_up, t_down, nullptr,
+                       nullptr, hidden, inter, nullptr))
+        return 0;
+    return launch_dense_ffn(nullptr, a, true) == HQ_OK ? dense_ffn_scratch_bytes(inter) : 0;
+}
+
+int hq_dense_ffn_decode(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up, const void* w_down,
+                        hq_ggml_type t_gate_up, hq_ggml_type t_down, const float* residual, float* out, uint32_t hidden,
+                        uint32_t inter, void* scratch, size_t scratch_bytes) {
+    const char* fn = "hq_dense_ffn_decode";
+    DenseFfnArgs a;
+    if (int rc = dense_ffn_args(fn, &a, x, xdt, w_gate, w_up, w_down, t_gate_up, t_down, residual, out, hidden, inter, scratch)) return rc;
+    if (hidden == 0 || inter == 0) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: hidden %u, inter %u", fn, hidden, inter);
+    if (int rc = launch_dense_ffn(nullptr, a, true)) return rc;  // shape and types
+    if (!x || !w_gate || !w_up || !w_down || !out || !scratch) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (!is_aligned(x, 16) || !is_aligned(out, 4) || !is_aligned(residual, 4))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: x needs 16-byte, out / residual 4-byte alignment", fn);
+    if (int rc = check_weight_alignment(w_gate, t_gate_up)) return rc;
+    if (int rc = check_weight_alignment(w_up, t_gate_up)) return rc;
+    if (int rc = check_weight_alignment(w_down, t_down)) return rc;
+    if (!is_aligned(scratch, 256)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch must be 256-byte aligned", fn);
+    if (scratch_bytes < dense_ffn_scratch_bytes(inter))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch of %zu bytes, %zu needed", fn, scratch_bytes, dense_ffn_scratch_bytes(inter));
+    return launch_dense_ffn((hipStream_t)stream, a, false);
 }
 
 static int check_fwht(const char* fn, const float* buf, uint32_t n_heads, uint32_t head_dim) {

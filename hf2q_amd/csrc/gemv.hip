@@ -589,29 +589,39 @@ struct FArgs {
     float* y0;
     float* y1;
     uint32_t n, k, nm;
+    uint32_t swiglu;  // nm == 2: y0 = silu(W0 . x) * (W1 . x) instead of the two products
     FlatGeom g;
     uint32_t m4, m2, magic;
 };
 
-template <int TYPE, bool X_BF16, int W, int D>
+// DYN: the waves of a workgroup take its super-tasks from a counter (see gemv_walk.h): worth it where a wave has many
+// (the 151936-row head in f32: 101 against 108 us); with a handful per wave the three claimed ahead are all there is.
+template <int TYPE, bool X_BF16, int W, int D, bool DYN>
 __global__ __launch_bounds__(64 * W) void gemv_flat_kernel(FArgs a) {
     using X = FlatX<TYPE, X_BF16>;
     extern __shared__ uint4 smem[];
+    __shared__ uint32_t lds_queue;
     uint4* lds_x = smem;
     float* lds_s = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(smem) + X::value_bytes(a.k));
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    if (tid == 0) lds_queue = W;
     // the activations first, nothing else of this workgroup in front of them
     X::stage(a.x, a.k, lds_x, lds_s, tid, 64u * W);
-    FlatWalk<TYPE, X_BF16, D> wk;
-    wk.init(a.w0, a.w1, a.n, a.nm, a.g, wv * gridDim.x + blockIdx.x, W * gridDim.x);
-    wk.prime();
+    FlatWalk<TYPE, X_BF16, D, false, DYN> wk;
+    if constexpr (DYN)
+        wk.init(a.w0, a.w1, a.n, a.nm, a.g, blockIdx.x, gridDim.x, &lds_queue, wv);
+    else
+        wk.init(a.w0, a.w1, a.n, a.nm, a.g, wv * gridDim.x + blockIdx.x, W * gridDim.x);
+    if constexpr (!DYN) wk.prime();
     __syncthreads();
+    if constexpr (DYN) wk.prime();
     wk.load_masks(a.m4, a.m2, a.magic);
-    wk.run(lds_x, lds_s, [&](uint32_t first, uint32_t cnt, float k0, float k1) {
-        if (lane < cnt) {
-            const uint32_t row = wk.row_of_slot(first + lane);
-            if (row < a.n) {
+    wk.run(lds_x, lds_s, [&](uint32_t cnt, float k0, float k1, uint32_t row) {
+        if (lane < cnt && row < a.n) {
+            if (a.swiglu) {
+                a.y0[row] = silu_mul_f32(k0, k1);
+            } else {
                 a.y0[row] = k0;
                 if (a.nm == 2u) a.y1[row] = k1;
             }
@@ -643,12 +653,14 @@ constexpr int kFlatDepth = TYPE == HQ_Q8_0 ? HQ_FLAT_D_Q80 : TYPE == HQ_Q4_0 ? H
 
 template <int TYPE, bool X_BF16>
 int launch_flat(hipStream_t s, const void* x, const uint8_t* w0, const uint8_t* w1, float* y0, float* y1, uint32_t n, uint32_t k,
-                uint32_t nm, uint32_t cus) {
+                uint32_t nm, uint32_t cus, bool swiglu = false) {
     constexpr int W = (TYPE == HQ_Q6_K && X_BF16) ? 12 : 16;
     using X = FlatX<TYPE, X_BF16>;
-    const FArgs fa{x, w0, w1, y0, y1, n, k, nm, flat_geom(k, kUnitElems<TYPE>, kUnitsPerWindow<TYPE>, n, nm, cus * W),
+    const FArgs fa{x, w0, w1, y0, y1, n, k, nm, swiglu ? 1u : 0u, flat_geom(k, kUnitElems<TYPE>, kUnitsPerWindow<TYPE>, n, nm, cus * W),
                    TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
-    auto kern = gemv_flat_kernel<TYPE, X_BF16, W, kFlatDepth<TYPE>>;
+    const uint64_t supers = ((uint64_t)n + (1u << fa.g.log_r) - 1) >> fa.g.log_r;
+    const bool dyn = kFlatDepth<TYPE> == 1 && supers >= (uint64_t)cus * W * 8u;
+    auto kern = dyn ? gemv_flat_kernel<TYPE, X_BF16, W, 1, true> : gemv_flat_kernel<TYPE, X_BF16, W, kFlatDepth<TYPE>, false>;
     size_t lds = X::lds_bytes(k);
     if (lds < 81 * 1024) lds = 81 * 1024;  // more than half a CU's LDS: one workgroup per CU
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv flat LDS)")) return rc;
@@ -815,6 +827,38 @@ bool gemv_stream_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, 
     if (t == HQ_Q4_K) return m <= 4 && stream_takes<HQ_Q4_K>(n, k, cus);
     if (t == HQ_Q5_K) return m <= 4 && stream_takes<HQ_Q5_K>(n, k, cus);
     return false;
+}
+
+namespace {
+template <int TYPE, bool X_BF16>
+int swiglu_t(hipStream_t s, const void* x, const void* wg, const void* wu, float* y, uint32_t m, uint32_t n, uint32_t k, bool dry) {
+    uint32_t cus = 256;
+    if (!dry)
+        if (int rc = cu_count(&cus)) return rc;
+    if (!flat_takes<TYPE>((uint64_t)n * 2, k, cus, FlatX<TYPE, X_BF16>::lds_bytes(k)))
+        return fail(HQ_ERR_UNSUPPORTED, "gate + up + SwiGLU GEMV: %u x %u is too small for the streaming form (or k = %u does not fit a CU's LDS)", n, k, k);
+    if (dry) return HQ_OK;
+    for (uint32_t r = 0; r < m; ++r)
+        if (int rc = launch_flat<TYPE, X_BF16>(s, static_cast<const uint8_t*>(x) + (size_t)r * k * (X_BF16 ? 2 : 4), static_cast<const uint8_t*>(wg),
+                                               static_cast<const uint8_t*>(wu), y + (size_t)r * n, y + (size_t)r * n, n, k, 2, cus, true))
+            return rc;
+    return HQ_OK;
+}
+}  // namespace
+
+// y[r] = silu(W_gate . x[r]) * (W_up . x[r]) for m activation rows, one pass over both matrices per row; dry: only whether
+// the shape is taken.
+int launch_gemv_swiglu(hipStream_t s, const void* x, hq_act_dtype xdt, const void* wg, const void* wu, float* y, uint32_t m, uint32_t n,
+                       uint32_t k, hq_ggml_type t, bool dry) {
+    const bool bf = xdt == HQ_BF16;
+    switch (t) {
+        case HQ_Q4_K: return bf ? swiglu_t<HQ_Q4_K, true>(s, x, wg, wu, y, m, n, k, dry) : swiglu_t<HQ_Q4_K, false>(s, x, wg, wu, y, m, n, k, dry);
+        case HQ_Q6_K: return bf ? swiglu_t<HQ_Q6_K, true>(s, x, wg, wu, y, m, n, k, dry) : swiglu_t<HQ_Q6_K, false>(s, x, wg, wu, y, m, n, k, dry);
+        case HQ_Q8_0: return bf ? swiglu_t<HQ_Q8_0, true>(s, x, wg, wu, y, m, n, k, dry) : swiglu_t<HQ_Q8_0, false>(s, x, wg, wu, y, m, n, k, dry);
+        case HQ_Q5_K: return bf ? swiglu_t<HQ_Q5_K, true>(s, x, wg, wu, y, m, n, k, dry) : swiglu_t<HQ_Q5_K, false>(s, x, wg, wu, y, m, n, k, dry);
+        case HQ_Q4_0: return bf ? swiglu_t<HQ_Q4_0, true>(s, x, wg, wu, y, m, n, k, dry) : swiglu_t<HQ_Q4_0, false>(s, x, wg, wu, y, m, n, k, dry);
+    }
+    return fail(HQ_ERR_UNSUPPORTED, "gemv: ggml type %d", (int)t);
 }
 
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t) {

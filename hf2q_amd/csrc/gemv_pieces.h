@@ -253,6 +253,74 @@ __device__ __forceinline__ float dot_f32(const Piece<HQ_Q5_K>& p, int c, const f
     return acc;
 }
 
+// The same dot products in two halves of 32 activations each (xh: the half's activations), for callers that cannot
+// afford all 64 in registers: half h leaves its raw sums in out[], dot_f32_finish combines both halves' sums.  The
+// operations and their order are those of dot_f32: the same bits.
+__device__ __forceinline__ void dot_f32_half(const Piece<HQ_Q4_K>& p, int, int h, const float* xh, float* out) {
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t w = j < 4 ? word(p.q0, j) : word(p.q1, j - 4);
+        acc = dot4((h ? w >> 4 : w) & 0x0f0f0f0fu, xh + 4 * j, acc);
+    }
+    out[0] = acc;
+}
+__device__ __forceinline__ float dot_f32_finish(const Piece<HQ_Q4_K>& p, int c, const float* lo, const float* hi, const float* sx) {
+    uint32_t sc0, sc1, m0, m1;
+    q4k_scales(p.hdr.y, p.hdr.z, p.hdr.w, c, sc0, sc1, m0, m1);
+    const float d = f16_bits_to_f32(p.hdr.x & 0xffffu), dmin = f16_bits_to_f32(p.hdr.x >> 16);
+    float acc = d * (float)sc0 * lo[0] - dmin * (float)m0 * (sx[0] + sx[1]);
+    acc += d * (float)sc1 * hi[0] - dmin * (float)m1 * (sx[2] + sx[3]);
+    return acc;
+}
+__device__ __forceinline__ void dot_f32_half(const Piece<HQ_Q5_K>& p, int c, int h, const float* xh, float* out) {
+    float acc = 0.f;
+    constexpr uint32_t N4 = 0x0f0f0f0fu, N1 = 0x10101010u;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t w = j < 4 ? word(p.q0, j) : word(p.q1, j - 4);
+        const uint32_t hs = (j < 4 ? word(p.h0, j) : word(p.h1, j - 4)) >> (2 * c);
+        acc = dot4(h ? ((w >> 4) & N4) | ((hs << 3) & N1) : (w & N4) | ((hs << 4) & N1), xh + 4 * j, acc);
+    }
+    out[0] = acc;
+}
+__device__ __forceinline__ float dot_f32_finish(const Piece<HQ_Q5_K>& p, int c, const float* lo, const float* hi, const float* sx) {
+    uint32_t sc0, sc1, m0, m1;
+    q4k_scales(p.hdr.y, p.hdr.z, p.hdr.w, c, sc0, sc1, m0, m1);
+    const float d = f16_bits_to_f32(p.hdr.x & 0xffffu), dmin = f16_bits_to_f32(p.hdr.x >> 16);
+    float acc = d * (float)sc0 * lo[0] - dmin * (float)m0 * (sx[0] + sx[1]);
+    acc += d * (float)sc1 * hi[0] - dmin * (float)m1 * (sx[2] + sx[3]);
+    return acc;
+}
+// Q6_K: half 0 = the runs of the low nibbles (r0, r1), half 1 = those of the high nibbles (r2, r3).
+__device__ __forceinline__ void dot_f32_half(const Piece<HQ_Q6_K>& p, int, int h, const float* xh, float* out) {
+    float ra = 0.f, rb = 0.f;
+    constexpr uint32_t N4 = 0x0f0f0f0fu, N2 = 0x30303030u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t a = word(p.qa, j), b = word(p.qb, j), v = word(p.qh, j);
+        if (h == 0) {
+            ra = dot4((a & N4) | ((v << 4) & N2), xh + 4 * j, ra);
+            rb = dot4((b & N4) | ((v << 2) & N2), xh + 16 + 4 * j, rb);
+        } else {
+            ra = dot4(((a >> 4) & N4) | (v & N2), xh + 4 * j, ra);
+            rb = dot4(((b >> 4) & N4) | ((v >> 2) & N2), xh + 16 + 4 * j, rb);
+        }
+    }
+    out[0] = ra;
+    out[1] = rb;
+}
+__device__ __forceinline__ float dot_f32_finish(const Piece<HQ_Q6_K>& p, int c, const float* lo, const float* hi, const float* sx) {
+    const int lr = c & 1;
+    const uint32_t s01 = p.sc.x >> (8 * lr), s23 = p.sc.y >> (8 * lr);
+    const float d = f16_bits_to_f32(p.d >> 16);
+    float acc = (float)(int)(int8_t)(s01 & 0xff) * (lo[0] - 32.f * sx[0]);
+    acc += (float)(int)(int8_t)((s01 >> 16) & 0xff) * (lo[1] - 32.f * sx[1]);
+    acc += (float)(int)(int8_t)(s23 & 0xff) * (hi[0] - 32.f * sx[2]);
+    acc += (float)(int)(int8_t)((s23 >> 16) & 0xff) * (hi[1] - 32.f * sx[3]);
+    return d * acc;
+}
+
 // Q4_0: y = d * (q - 8); low nibbles are elements 0..15 of the block, high nibbles 16..31.
 __device__ __forceinline__ float dot_f32(const Piece<HQ_Q4_0>& p, int, const float* xf, const float* sx) {
     float lo = 0.f, hi = 0.f;

@@ -167,10 +167,49 @@ struct FlatX {
             for (int r = 0; r < RUNS; ++r) sx[r] = lds_s[piece * RUNS + r];
         }
     }
+
+    // f32 K-quant pieces in two halves of 32 activations (see dot_f32_half); h = 0 also loads the four run sums.
+    static __device__ __forceinline__ void load_half(const uint4* lds_x, const float* lds_s, uint32_t ur, int c, int h, uint32_t* xh,
+                                                     float* sx) {
+        static_assert(!PAIR && !kBlock32<TYPE>, "f32 activations of a K-quant");
+        auto put = [&](int at, const uint4 v) {
+            xh[at] = v.x;
+            xh[at + 1] = v.y;
+            xh[at + 2] = v.z;
+            xh[at + 3] = v.w;
+        };
+        if constexpr (TYPE == HQ_Q6_K) {
+            const uint4* base = lds_x + ur * 81u + (uint32_t)(c >> 1) * 40u + (uint32_t)(c & 1) * 4u + 16u * (uint32_t)h;
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) put((4 * r + u) * 4, base[8 * r + u]);
+            }
+            if (h == 0) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sx[r] = lds_s[ur * 16u + (uint32_t)(c >> 1) * 8u + (uint32_t)(c & 1) + 2u * r];
+            }
+        } else {
+            const uint32_t piece = ur * 4u + (uint32_t)c;
+            const uint4* base = lds_x + piece * (G + 1u) + 8u * (uint32_t)h;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) put(4 * j, base[j]);
+            if (h == 0) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sx[r] = lds_s[piece * 4u + r];
+            }
+        }
+    }
 };
 
-template <int TYPE, bool X_BF16, int D = 1>
+// XHALF: f32 activations of a K-quant are read from LDS 32 at a time (half the registers; the same sums).
+// DYN (D == 1): the waves of a workgroup take the workgroup's super-tasks from a counter in LDS instead of a fixed split.
+// The SIMD's issue arbitration favours its oldest wave, so with equal shares the youngest wave of every SIMD finishes long
+// after the others; with the counter all waves of a CU end together.  A wave claims its next super-task one ahead, so its
+// fetch runs on across the boundary.
+template <int TYPE, bool X_BF16, int D = 1, bool XHALF = false, bool DYN = false>
 struct FlatWalk {
+    static_assert(!DYN || D == 1, "the dynamic split keeps one fetch in flight");
     using X = FlatX<TYPE, X_BF16>;
     static constexpr uint32_t LPU = kLanesPerUnit<TYPE>, UW = kUnitsPerWindow<TYPE>, BB = kBlockBytes<TYPE>;
 
@@ -178,16 +217,22 @@ struct FlatWalk {
     const uint8_t* w1;       // second matrix of the same shape (nm == 2), walked super-task by super-task beside the first
     uint32_t nrows, nm;
     FlatGeom g;
-    uint32_t first, stride, count;  // this wave's super-tasks: first + i * stride, i < count
+    // Super-task q of the sequence is seq_first + q * seq_stride, q < count.  Fixed split: the sequence is the wave's own and
+    // it takes q = 0, 1, ...; dynamic: the sequence is the workgroup's and q comes from *queue (the first claims are the
+    // wave indices: the kernel sets the counter to the number of waves before its first barrier).
+    uint32_t seq_first, seq_stride, count;
+    uint32_t* queue;
+    uint32_t q_cur, q_nxt, q_nn;  // the super-task being summed, its successor and the one after (dynamic: claimed ahead)
     uint32_t lane, lv;  // lv: the lane's unit inside a window (idle lanes: the last active one's)
     bool active;
     int c;
     uint32_t m4, m2, magic;
-    uint32_t f_i, f_m, f_w, f_left;  // the next task to fetch; tasks not yet fetched
+    uint32_t f_q, f_m, f_w;  // the next task to fetch
     Piece<TYPE> buf[D];
 
     __device__ __forceinline__ void init(const uint8_t* wa, const uint8_t* wb, uint32_t n, uint32_t n_matrices, const FlatGeom& geom,
-                                         uint32_t first_super, uint32_t super_stride) {
+                                         uint32_t first_super, uint32_t super_stride, uint32_t* lds_queue = nullptr,
+                                         uint32_t first_claim = 0) {
         w0 = wa;
         w1 = wb;
         nrows = n;
@@ -198,13 +243,15 @@ struct FlatWalk {
         active = lane / LPU < g.uwe;
         lv = active ? lane / LPU : g.uwe - 1u;
         const uint32_t n_super = (n + (1u << g.log_r) - 1u) >> g.log_r;
-        first = first_super;
-        stride = super_stride;
-        count = first < n_super ? (n_super - first + stride - 1u) / stride : 0u;
-        f_i = f_m = f_w = 0;
-        f_left = tasks();
+        seq_first = first_super;
+        seq_stride = super_stride;
+        count = first_super < n_super ? (n_super - first_super + super_stride - 1u) / super_stride : 0u;
+        queue = lds_queue;
+        q_cur = DYN ? first_claim : 0u;
+        q_nxt = q_nn = q_cur + 1u;  // (dynamic: replaced by the first claims in prime())
+        f_q = q_cur;
+        f_m = f_w = 0;
     }
-    __device__ __forceinline__ uint32_t tasks() const { return count * nm * g.st; }
 
     // The conversion masks of the paired-bf16 dot products must sit in VGPRs (v_and_or_b32 takes one scalar operand at
     // most); the copy is opaque so they stay there.
@@ -215,73 +262,118 @@ struct FlatWalk {
     }
 
     __device__ __forceinline__ void fetch_next(Piece<TYPE>& p) {
-        const uint32_t sid = first + f_i * stride;
+        const uint32_t sid = seq_first + f_q * seq_stride;
         uint32_t u = (sid << g.log_r) * g.bu + g.uwe * f_w + lv;
         const uint32_t last = nrows * g.bu - 1u;
         u = u < last ? u : last;
         const uint8_t* base = f_m ? w1 : w0;
         p.load(base + (size_t)u * BB, c);
-        if (f_left > 1u) {  // (scalar: no memory operation inside)
-            --f_left;
-            if (++f_w == g.st) {
+        // (scalar: no memory operation inside)  Past the sequence's end the last task is fetched again, not used.
+        if (f_w + 1u < g.st) {
+            ++f_w;
+        } else if (f_m + 1u < nm) {
+            f_w = 0;
+            ++f_m;
+        } else {
+            // the fetch is one task ahead of the sums: it is in their super-task or in its successor
+            const uint32_t nq = DYN ? (f_q == q_cur ? q_nxt : q_nn) : f_q + 1u;
+            if (nq < count) {
                 f_w = 0;
-                if (++f_m == nm) {
-                    f_m = 0;
-                    ++f_i;
-                }
+                f_m = 0;
+                f_q = nq;
             }
         }
     }
 
+    // (dynamic: call after the barrier behind which the counter is initialised)
     __device__ __forceinline__ void prime() {
-        if (tasks()) {
+        if constexpr (DYN) {
+            q_nxt = claim_wait(claim());
+            q_nn = claim_wait(claim());
+        }
+        if (q_cur < count) {
 #pragma unroll
             for (int d = 0; d < D; ++d) fetch_next(buf[d]);
         }
     }
 
-    // Row of the wave's j-th finished row (the order in which results reach the output functor).
-    __device__ __forceinline__ uint32_t row_of_slot(uint32_t j) const {
-        return ((first + (j >> g.log_r) * stride) << g.log_r) + (j & ((1u << g.log_r) - 1u));
+    __device__ __forceinline__ uint32_t claim() {
+        uint32_t v = 0;
+        if (lane == 0) v = __hip_atomic_fetch_add(queue, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return v;
     }
+    __device__ __forceinline__ uint32_t claim_wait(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
-    // out(first_slot, count, keep0, keep1): lane l < count holds the sums of row_of_slot(first_slot + l) over the first
+    // out(count, keep0, keep1, row): lane l < count holds the sums of row `row` (its own value of the argument) over the first
     // (keep0) and the second matrix (keep1).
     template <typename OUT>
     __device__ __forceinline__ void run(const uint4* lds_x, const float* lds_s, OUT&& out) {
-        const uint32_t ntask = tasks();
         uint32_t c_m = 0, c_w = 0, done = 0;
         float keep0 = 0.f, keep1 = 0.f;
-        uint32_t xr[X::XW];
+        uint32_t keep_row = 0;
+        constexpr bool HALVES = XHALF && !X::PAIR && !kBlock32<TYPE>;
+        uint32_t xr[HALVES ? 32 : X::XW];
         float sx[4] = {0.f, 0.f, 0.f, 0.f};
-        const bool xinv = g.st == 1u && g.log_r == 0u;  // every window is one whole row: the lane's activations never change
-        if (xinv) X::load(lds_x, lds_s, lv, c, xr, sx);
+        const bool xinv = !HALVES && g.st == 1u && g.log_r == 0u;  // every window is one whole row: the lane's activations never change
+        if constexpr (!HALVES)
+            if (xinv) X::load(lds_x, lds_s, lv, c, xr, sx);
         const int last_lane = (int)(g.uwe * LPU - 1u);
-        for (uint32_t t = 0; t < ntask; t += D) {
+        const bool one_row = g.log_r == 0u;
+        float acc = 0.f;
+        [[maybe_unused]] uint32_t pending = 0;
+        if constexpr (DYN)
+            if (q_cur < count) pending = claim();  // the third super-task from here
+        while (q_cur < count) {
 #pragma unroll
             for (int d = 0; d < D; ++d) {
                 Piece<TYPE>& p = buf[d];
                 const uint32_t lu = g.uwe * c_w + lv;
                 uint32_t lrow = __umulhi(lu, g.magic);
                 const uint32_t ur = lu - lrow * g.bu;
-                if (!xinv) X::load(lds_x, lds_s, ur, c, xr, sx);
                 float part;
-                if constexpr (X::PAIR)
-                    part = dot_pair(p, c, xr, sx, m4, m2, magic);
-                else
-                    part = dot_f32(p, c, reinterpret_cast<const float*>(xr), sx);
+                if constexpr (HALVES) {
+                    float lo[2], hi[2];
+                    X::load_half(lds_x, lds_s, ur, c, 0, xr, sx);
+                    dot_f32_half(p, c, 0, reinterpret_cast<const float*>(xr), lo);
+                    asm volatile("" : "+v"(lo[0]));  // the second half's activations take the first half's registers
+                    X::load_half(lds_x, lds_s, ur, c, 1, xr, sx);
+                    dot_f32_half(p, c, 1, reinterpret_cast<const float*>(xr), hi);
+                    part = dot_f32_finish(p, c, lo, hi, sx);
+                } else {
+                    if (!xinv) X::load(lds_x, lds_s, ur, c, xr, sx);
+                    if constexpr (X::PAIR)
+                        part = dot_pair(p, c, xr, sx, m4, m2, magic);
+                    else
+                        part = dot_f32(p, c, reinterpret_cast<const float*>(xr), sx);
+                }
                 asm volatile("" : "+v"(part));  // the refill follows the arithmetic that frees its registers
                 fetch_next(p);
-                const bool live = D == 1 || t + (uint32_t)d < ntask;  // (a ring's last round may run past the end)
-                const uint32_t r_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)lrow);
-                const uint32_t r_hi = (uint32_t)__builtin_amdgcn_readlane((int)lrow, last_lane);
-                lrow = active ? lrow : 0xffffffffu;  // an idle lane's duplicate belongs to no row
-                for (uint32_t r = r_lo; r <= r_hi; ++r) {
-                    float v = lrow == r ? part : 0.f;
-                    v = group_sum(v, 6);
-                    const bool mine = live && lane == ((done + r) & 63u);
-                    keep0 = mine && c_m == 0u ? keep0 + v : keep0;
-                    keep1 = mine && c_m != 0u ? keep1 + v : keep1;
+                const bool live = D == 1 || q_cur < count;  // (a ring's last round may run past the end)
+                const uint32_t row0 = (seq_first + q_cur * seq_stride) << g.log_r;
+                if (one_row) {
+                    // every window of the super-task belongs to its one row: the lanes add their windows up and meet once
+                    // (the order of sums of the aligned streaming kernel: the same bits)
+                    acc += active && live ? part : 0.f;
+                    if (live && c_w + 1u == g.st) {
+                        const float v = group_sum(acc, 6);
+                        acc = 0.f;
+                        const bool mine = lane == (done & 63u);
+                        keep0 = mine && c_m == 0u ? v : keep0;
+                        keep1 = mine && c_m != 0u ? v : keep1;
+                        keep_row = mine ? row0 : keep_row;
+                    }
+                } else {
+                    const uint32_t r_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)lrow);
+                    const uint32_t r_hi = (uint32_t)__builtin_amdgcn_readlane((int)lrow, last_lane);
+                    lrow = active ? lrow : 0xffffffffu;  // an idle lane's duplicate belongs to no row
+                    for (uint32_t r = r_lo; r <= r_hi; ++r) {
+                        float v = lrow == r ? part : 0.f;
+                        v = group_sum(v, 6);
+                        const bool mine = live && lane == ((done + r) & 63u);
+                        keep0 = mine && c_m == 0u ? keep0 + v : keep0;
+                        keep1 = mine && c_m != 0u ? keep1 + v : keep1;
+                        keep_row = mine ? row0 + r : keep_row;
+                    }
                 }
                 if (live && ++c_w == g.st) {
                     c_w = 0;
@@ -289,14 +381,22 @@ struct FlatWalk {
                         c_m = 0;
                         done += 1u << g.log_r;
                         if ((done & 63u) == 0u) {
-                            out(done - 64u, 64u, keep0, keep1);
+                            out(64u, keep0, keep1, keep_row);
                             keep0 = keep1 = 0.f;
+                        }
+                        if constexpr (DYN) {
+                            q_cur = q_nxt;
+                            q_nxt = q_nn;
+                            q_nn = claim_wait(pending);
+                            if (q_cur < count) pending = claim();
+                        } else {
+                            ++q_cur;
                         }
                     }
                 }
             }
         }
-        if (done & 63u) out(done & ~63u, done & 63u, keep0, keep1);
+        if (done & 63u) out(done & 63u, keep0, keep1, keep_row);
     }
 };
 

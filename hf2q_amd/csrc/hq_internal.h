@@ -59,6 +59,9 @@ bool gemv_stream_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, 
 // Up to four independent GEMVs of one weight type and activation dtype in a single launch.
 int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_act_dtype xdt, hq_ggml_type t);
 
+int launch_gemv_swiglu(hipStream_t s, const void* x, hq_act_dtype xdt, const void* wg, const void* wu, float* y, uint32_t m, uint32_t n,
+                       uint32_t k, hq_ggml_type t, bool dry);
+
 // 3..8 activation rows sharing one pass over the weights (gemvm.hip); gemv_rows_supported() says
 // whether (type, m, k) has such a kernel, otherwise the GEMV runs once per row.
 bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k);
@@ -141,6 +144,22 @@ bool moe_fused_supported(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts,
                          uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt);
 size_t moe_fused_scratch_bytes(uint32_t n_tokens, uint32_t n_experts, uint32_t top_k);
 int launch_moe_fused(hipStream_t s, const MoeFusedArgs& a);
+
+// The dense SwiGLU FFN of one decode token in one launch (dense_ffn.hip).  dry: only say whether the shape is taken.
+struct DenseFfnArgs {
+    const void* x;  // [hidden]
+    hq_act_dtype xdt;
+    const void *w_gate, *w_up, *w_down;
+    hq_ggml_type t_gate_up, t_down;
+    const float* residual;  // nullptr or [hidden]
+    float* out;             // [hidden]
+    void* scratch;
+    uint32_t hidden, inter;
+    uint32_t spin_limit;  // 0: default
+};
+size_t dense_ffn_scratch_bytes(uint32_t inter);
+int launch_dense_ffn(hipStream_t s, const DenseFfnArgs& a, bool dry);
+void gemm_f16_small_tile_slices(hq_ggml_type t, uint32_t m, uint32_t n, uint32_t k, uint32_t* splits, uint32_t* sb_per);
 
 // TurboQuant KV (tq.hip)
 int launch_fwht_sign(hipStream_t s, float* buf, uint32_t n_heads, uint32_t head_dim, bool undo);

@@ -54,6 +54,7 @@ SIGNATURES = {
     "hq_quantize_ggml": (_i32, [_vp, _vp, _u64, _u64, _i32, _vp]),
     "hq_qmatmul_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32]),
     "hq_qmatmul_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),
+    "hq_qmatmul_ggml_k_slices": (_i32, [_u32, _u32, _u32, _i32, _c.POINTER(_u32), _c.POINTER(_u32)]),
     "hq_qmatmul_ggml_ws": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32, _vp, _sz]),
     "hq_qmatmul_id_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _u32, _u32, _u32, _u32, _u32, _u64, _i32]),
     "hq_weight_row_scales_ggml": (_i32, [_vp, _vp, _vp, _u64, _u32, _i32]),
@@ -65,6 +66,8 @@ SIGNATURES = {
     "hq_qmatmul_gated_ggml_ws": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _i32, _vp, _sz]),
     "hq_qmatmul_swiglu_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),
     "hq_qmatmul_swiglu_ggml_ws": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _i32, _vp, _sz]),
+    "hq_qmatmul_swiglu_decode_supported": (_i32, [_u32, _u32, _i32, _i32]),
+    "hq_qmatmul_swiglu_decode": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _u32, _u32, _u32, _i32]),
     "hq_qmatmul_perm021_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),
     "hq_qmatmul_perm021_ggml_ws": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _u32, _i32, _vp, _sz]),
     "hq_qmatmul_id_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _u32, _u32, _u64, _i32]),
@@ -77,6 +80,10 @@ SIGNATURES = {
     "hq_moe_weighted_reduce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "hq_moe_ffn_decode_scratch_bytes": (_sz, [_u32, _u32, _u32, _u32, _u32, _u32, _i32, _i32]),
     "hq_moe_ffn_decode": (_i32, [_vp, _vp, _vp, _i32, _vp, _vp, _u32, _vp, _sz, _vp, _vp]),
+    "hq_handover_status": (_i32, [_vp, _vp, _c.POINTER(_u32)]),
+    "hq_set_handover_spin_limit": (None, [_u32]),
+    "hq_dense_ffn_decode_scratch_bytes": (_sz, [_u32, _u32, _i32, _i32, _i32]),
+    "hq_dense_ffn_decode": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _u32, _u32, _vp, _sz]),
     "hq_fwht_sign_premult_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_fwht_sign_undo_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_tq_encode_kv": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),

@@ -165,6 +165,19 @@ def quantized_matmul_swiglu_ggml(input: torch.Tensor, gate: torch.Tensor, up: to
         params.k, params.ggml_type, _dev(workspace, "workspace"), workspace.numel() * workspace.element_size()))
 
 
+def quantized_matmul_swiglu_decode_supported(params: GgmlQuantizedMatmulParams, act_dtype: torch.dtype) -> bool:
+    xdt = HQ_BF16 if act_dtype == torch.bfloat16 else HQ_F32
+    return bool(_l.load().hq_qmatmul_swiglu_decode_supported(params.n, params.k, params.ggml_type, xdt))
+
+
+def quantized_matmul_swiglu_decode(input: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, dst: torch.Tensor,
+                                   params: GgmlQuantizedMatmulParams) -> None:
+    """dst[m, n] = silu(input . gate^T) * (input . up^T) for m <= 8 rows: the gate / up pair of a decode step
+    (gpu_ffn.rs:1231-1258) and the silu_mul behind it as one launch per row; the bits of the separate dispatches."""
+    _l.check(_l.load().hq_qmatmul_swiglu_decode(_stream(), _dev(input, "input"), _act_dtype(input), _dev(gate, "gate"), _dev(up, "up"),
+                                                _dev(dst, "dst"), params.m, params.n, params.k, params.ggml_type))
+
+
 @dataclass
 class GgmlQuantizedMatmulPerm021Params:
     """forward_prefill_batched.rs:2219-2226."""
@@ -640,12 +653,41 @@ class DenseFfnWeightsGpuQ:
     ggml_type: int
     hidden: int
     inter: int
+    down_type: int | None = None  # the down matrix's type where it differs from gate / up (Q6_K in Q4_K_M / Q5_K_M files)
+
+
+def dense_ffn_decode_scratch_bytes(w: "DenseFfnWeightsGpuQ", act_dtype: torch.dtype) -> int:
+    """Bytes of zeroed device scratch dense_ffn_decode needs for this layer; 0: the one-launch form does not take it."""
+    xdt = HQ_BF16 if act_dtype == torch.bfloat16 else HQ_F32
+    dt = w.down_type if w.down_type is not None else w.ggml_type
+    return int(_l.load().hq_dense_ffn_decode_scratch_bytes(w.hidden, w.inter, w.ggml_type, dt, xdt))
+
+
+def dense_ffn_decode(x: torch.Tensor, w: "DenseFfnWeightsGpuQ", out: torch.Tensor, scratch: torch.Tensor,
+                     residual: torch.Tensor | None = None) -> None:
+    """build_dense_ffn_layer_gpu_q (gpu_ffn.rs:1017-1351) for ONE token as one launch: out = down(silu(gate x) * (up x))
+    (+ residual).  `scratch`: dense_ffn_decode_scratch_bytes() bytes, zeroed once by the caller (torch.zeros), then left
+    to the library; the bits of the separate dispatches."""
+    if x.numel() != w.hidden or out.numel() != w.hidden:
+        raise ValueError("dense_ffn_decode takes one token: x and out of `hidden` values")
+    dt = w.down_type if w.down_type is not None else w.ggml_type
+    _l.check(_l.load().hq_dense_ffn_decode(_stream(), _dev(x, "x"), _act_dtype(x), _dev(w.gate_q, "gate"), _dev(w.up_q, "up"),
+                                           _dev(w.down_q, "down"), w.ggml_type, dt,
+                                           _dev(residual, "residual") if residual is not None else None, _dev(out, "out"),
+                                           w.hidden, w.inter, _dev(scratch, "scratch"), scratch.numel() * scratch.element_size()))
+
+
+def handover_status(scratch: torch.Tensor) -> int:
+    """The error word of a scratch of dense_ffn_decode / moe_ffn_decode_fused (0: fine); synchronises the stream."""
+    err = ctypes.c_uint32(0)
+    _l.check(_l.load().hq_handover_status(_stream(), _dev(scratch, "scratch"), ctypes.byref(err)))
+    return int(err.value)
 
 
 def dense_ffn_workspace_bytes(w: "DenseFfnWeightsGpuQ", m: int, act_dtype: torch.dtype) -> int:
     """Device scratch build_dense_ffn_layer_gpu_q_into(..., workspace=) needs for m rows (0: none needed)."""
     return max(quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, w.inter, w.hidden, w.ggml_type), act_dtype),
-               quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, w.hidden, w.inter, w.ggml_type), torch.float32))
+               quantized_matmul_workspace_bytes(GgmlQuantizedMatmulParams(m, w.hidden, w.inter, w.down_type if w.down_type is not None else w.ggml_type), torch.float32))
 
 
 def build_dense_ffn_layer_gpu_q_into(x: torch.Tensor, w: DenseFfnWeightsGpuQ, gate_buf: torch.Tensor,
@@ -657,21 +699,28 @@ def build_dense_ffn_layer_gpu_q_into(x: torch.Tensor, w: DenseFfnWeightsGpuQ, ga
     staging of the down projection (for inter <= 8192): two launches instead of four, identical results."""
     m = x.shape[0]
     H, I, t = w.hidden, w.inter, w.ggml_type
+    td = w.down_type if w.down_type is not None else t
     if batched is None:
         batched = m <= _BATCH_MAX_DENSE_ROWS
     if batched:
         if m > _BATCH_MAX_DENSE_ROWS:
             raise ValueError(f"batched dense FFN: {m} rows (limit {_BATCH_MAX_DENSE_ROWS})")
+        pgu = GgmlQuantizedMatmulParams(m, I, H, t)
+        if act_buf is not None and quantized_matmul_swiglu_decode_supported(pgu, x.dtype):
+            # gate, up and the SwiGLU as one launch per row, then down over the f32 activations: two launches at batch 1
+            quantized_matmul_swiglu_decode(x, w.gate_q, w.up_q, act_buf, pgu)
+            quantized_matmul_ggml(act_buf, w.down_q, out, GgmlQuantizedMatmulParams(m, H, I, td))
+            return
         quantized_matmul_batch_ggml([QmatmulJob(x, w.gate_q, gate_buf, m, I, H), QmatmulJob(x, w.up_q, up_buf, m, I, H)], t)
         # Every workgroup of the fused down projection forms the whole activation vector itself; past a few
         # thousand activations a separate SwiGLU pass is as fast (measured equal at 12288).
         if I <= _FUSED_SWIGLU_MAX_K or act_buf is None:
-            quantized_matmul_batch_ggml([QmatmulJob(gate_buf, w.down_q, out, m, H, I, input_up=up_buf)], t)
+            quantized_matmul_batch_ggml([QmatmulJob(gate_buf, w.down_q, out, m, H, I, input_up=up_buf)], td)
         else:
             dispatch_silu_mul(gate_buf[:m], up_buf[:m], act_buf[:m])
-            quantized_matmul_ggml(act_buf, w.down_q, out, GgmlQuantizedMatmulParams(m, H, I, t))
+            quantized_matmul_ggml(act_buf, w.down_q, out, GgmlQuantizedMatmulParams(m, H, I, td))
         return
-    pgu, pdn = GgmlQuantizedMatmulParams(m, I, H, t), GgmlQuantizedMatmulParams(m, H, I, t)
+    pgu, pdn = GgmlQuantizedMatmulParams(m, I, H, t), GgmlQuantizedMatmulParams(m, H, I, td)
     if workspace is not None and quantized_matmul_gated_workspace_bytes(pgu, x.dtype):
         # a prefill chunk with caller scratch (dense_ffn_workspace_bytes): nothing is allocated, and the up projection
         # finishes the gating in its epilogue -- no SwiGLU pass over both products (the same bits)

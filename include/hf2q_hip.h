@@ -108,6 +108,13 @@ HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, ui
 HQ_API int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y,
                     uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t);
 
+/* How hq_qmatmul_ggml[_ws] cuts k for up to 256 activation rows on the tile route: `slices` slices of
+ * `blocks_per_slice` 256-element runs each (the last one shorter), every slice a launch-time workgroup set of its own whose
+ * partial products a second launch adds in slice order.  slices = 1: no cut.  (slices - 1) * blocks_per_slice < k / 256
+ * always holds, so no slice starts past the end of a row.  Pure host arithmetic; a query for tests and for sizing. */
+HQ_API int hq_qmatmul_ggml_k_slices(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, uint32_t* slices,
+                             uint32_t* blocks_per_slice);
+
 /* The same product with caller-owned device scratch.  The f16 tile kernels
  * (prefill-sized m; K-quants with k % 256 == 0, Q8_0 / Q4_0 with k % 128 == 0) convert the
  * activations to row-scaled f16 in a pre-pass and need hq_qmatmul_ggml_workspace_bytes() bytes (256-byte
@@ -158,6 +165,15 @@ HQ_API size_t hq_qmatmul_swiglu_ggml_workspace_bytes(uint32_t m, uint32_t n, uin
 HQ_API int hq_qmatmul_swiglu_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up,
                               const float* gate_row_scales, const float* up_row_scales, float* y, uint32_t m, uint32_t n,
                               uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes);
+
+/* The same on the decode route (m <= 8 activation rows): one launch per row walks the same weight rows of both matrices
+ * and stores silu(gate) * up -- the two f32 products never go to memory and the hq_silu_mul dispatch between them and the
+ * down projection disappears (gpu_ffn.rs:1231-1306 at batch 1).  The bits of hq_qmatmul_batch_ggml(gate, up) followed by
+ * hq_silu_mul.  Any type, f32 or bf16 activations, any k of whole blocks; matrices too small for the streaming GEMV
+ * (hq_qmatmul_swiglu_decode_supported() == 0) return HQ_ERR_UNSUPPORTED and take the separate calls. */
+HQ_API int hq_qmatmul_swiglu_decode_supported(uint32_t n, uint32_t k, hq_ggml_type t, hq_act_dtype xdt);
+HQ_API int hq_qmatmul_swiglu_decode(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up, float* y,
+                             uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t);
 
 /* y[m, n] = sum_k x[m, k] * W[n, k] with the activations stored heads-outermost, [k / head_dim][m][head_dim]
  * (the attention output of a batched prefill): element (row, kk) sits at ((kk / head_dim) * m + row) * head_dim +
@@ -347,6 +363,36 @@ HQ_API size_t hq_moe_ffn_decode_scratch_bytes(uint32_t n_tokens, uint32_t hidden
 HQ_API int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* layer, const void* x, hq_act_dtype xdt,
                       const float* residual, float* out, uint32_t n_tokens, void* scratch, size_t scratch_bytes,
                       uint32_t* route_ids, float* route_weights);
+
+/* The hand-over state of a scratch of hq_moe_ffn_decode or hq_dense_ffn_decode: *error receives the scratch's error
+ * word (0: every wait inside the launches so far ended by itself; non-zero: one ran into the polling limit, the output
+ * of that call is undefined and the scratch must be zeroed again before its next use).  Waits for `stream` (a 4-byte
+ * copy to the host): call it where the serving loop
+ * synchronises anyway.  hq_set_handover_spin_limit sets the polling limit of launches made after it (0: the default,
+ * about a million polls, seconds): a tiny limit makes every wait give up at once, which is how the tests exercise the
+ * bail-out path without hanging anything. */
+HQ_API int hq_handover_status(void* stream, const void* scratch, uint32_t* error);
+HQ_API void hq_set_handover_spin_limit(uint32_t limit);
+
+/* The dense SwiGLU FFN of ONE decode token as ONE launch:
+ *   out[hidden] = W_down . (silu(W_gate . x) * (W_up . x)) (+ residual)
+ * Replaces build_dense_ffn_layer_gpu_q (src/inference/models/qwen35/gpu_ffn.rs:1017-1351: gate and up encoded without a
+ * barrier between them, :1231-1255, then silu_mul, then down) at batch 1.  One grid of a workgroup per CU streams the
+ * three matrices (85 MB at hidden 4096 / inter 12288 in Q4_K): gate and up rows with their SwiGLU, the activations handed
+ * to every workgroup through `scratch` as tagged words while the first down-weight fetches are already in flight, then
+ * the down rows.  The result has the bits of hq_qmatmul_batch_ggml(gate, up), hq_silu_mul and hq_qmatmul_ggml(down) over
+ * the f32 activations.  x: [hidden] f32 or bf16.  Types: gate / up and down of one type (any of the five), or Q4_K / Q5_K
+ * gate / up with a Q6_K down; hidden and inter whole blocks (at least two per row) and small enough for the CU's LDS
+ * (2 .. 4 bytes per value of hidden plus 4.25 per value of inter within 160 KiB); anything else: HQ_ERR_UNSUPPORTED,
+ * hq_dense_ffn_decode_scratch_bytes() returns 0, and the separate calls do the work.
+ * `scratch`: hq_dense_ffn_decode_scratch_bytes() bytes of device memory, 256-byte aligned, ZEROED ONCE before its first
+ * use and then left to the library (call counter, error word, hand-over words); calls that share a scratch must not
+ * overlap.  The waits inside the launch are bounded (hq_handover_status). */
+HQ_API size_t hq_dense_ffn_decode_scratch_bytes(uint32_t hidden, uint32_t inter, hq_ggml_type t_gate_up, hq_ggml_type t_down,
+                                         hq_act_dtype xdt);
+HQ_API int hq_dense_ffn_decode(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up,
+                        const void* w_down, hq_ggml_type t_gate_up, hq_ggml_type t_down, const float* residual, float* out,
+                        uint32_t hidden, uint32_t inter, void* scratch, size_t scratch_bytes);
 
 /* In-place  buf <- H.(s (.) buf)  per 256-element block of buf[n_heads][head_dim] (query
  * pre-rotation) and its inverse  buf <- s (.) (H.buf)  (output post-rotation).  Replace

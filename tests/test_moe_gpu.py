@@ -5,7 +5,7 @@ import torch
 
 from _util import acts, assert_matmul_close, weights
 from hf2q_amd import ops
-from hf2q_amd.ops import HQ_Q4_K, HQ_Q6_K, HQ_Q8_0
+from hf2q_amd.ops import HQ_Q4_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, GgmlQuantizedMatmulParams
 
 pytestmark = pytest.mark.gpu
 
@@ -456,3 +456,113 @@ def test_moe_block_one_launch_rejects_other_shapes(oracle, dev):
     with pytest.raises(ops.HqError) as e:
         ops.moe_ffn_decode_fused(x, w, s, torch.empty(2, H, device=dev))
     assert e.value.status == 2
+
+
+DENSE_DECODE_CASES = [  # (hidden, inter, gate / up type, down type)
+    (4096, 12288, HQ_Q4_K, HQ_Q4_K), (2816, 4096, HQ_Q5_K, HQ_Q6_K), (2048, 8192, HQ_Q4_K, HQ_Q6_K), (1536, 8960, HQ_Q4_K, HQ_Q4_K),
+    (4096, 12288, HQ_Q6_K, HQ_Q6_K), (4096, 11008, HQ_Q8_0, HQ_Q8_0), (2048, 5632, HQ_Q4_0, HQ_Q4_0), (1024, 512, HQ_Q5_K, HQ_Q5_K),
+]
+
+
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("H,I,tg,td", DENSE_DECODE_CASES)
+def test_dense_ffn_decode_one_launch_equals_separate_dispatches_and_cpu_spec(oracle, dev, H, I, tg, td, xdt):
+    """hq_dense_ffn_decode against (a) the separate dispatches -- gate + up as one batched launch, hq_silu_mul, the down
+    product over the f32 activations -- bit for bit, (b) dense_swiglu_cpu_ref (ffn.rs:91-112) over the dequantised weights
+    in float64; twice in a row on one scratch (the second call must not see the first call's words as its own), with a
+    residual, and replayed from a HIP graph."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(H + I + tg)
+    qz = lambda n, k, t: ops.quantize_ggml(torch.randn(n * k, generator=g, device=dev).mul_(0.02), k, t)  # noqa: E731
+    w = ops.DenseFfnWeightsGpuQ(qz(I, H, tg), qz(I, H, tg), qz(H, I, td), tg, H, I, down_type=td)
+    x32 = torch.randn(1, H, generator=g, device=dev)
+    x = x32.to(torch.bfloat16) if xdt == "bf16" else x32
+    need = ops.dense_ffn_decode_scratch_bytes(w, x.dtype)
+    assert need > 0
+    scratch = torch.zeros(need, dtype=torch.uint8, device=dev)
+    # (a) the separate dispatches
+    gate, up, act, ref = (torch.full((1, n), float("nan"), device=dev) for n in (I, I, I, H))
+    ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x, w.gate_q, gate, 1, I, H), ops.QmatmulJob(x, w.up_q, up, 1, I, H)], tg)
+    ops.dispatch_silu_mul(gate, up, act)
+    ops.quantized_matmul_ggml(act, w.down_q, ref, GgmlQuantizedMatmulParams(1, H, I, td))
+    out = torch.full((1, H), float("nan"), device=dev)
+    ops.dense_ffn_decode(x, w, out, scratch)
+    assert torch.equal(out, ref)
+    # gate + up + SwiGLU as one launch (the decode route's two-launch form): the same activations bit for bit
+    pgu = GgmlQuantizedMatmulParams(1, I, H, tg)
+    if ops.quantized_matmul_swiglu_decode_supported(pgu, x.dtype):
+        act2 = torch.full((1, I), float("nan"), device=dev)
+        ops.quantized_matmul_swiglu_decode(x, w.gate_q, w.up_q, act2, pgu)
+        assert torch.equal(act2, act)
+    else:
+        assert I * H < 4 * 1024 * 1024  # only small matrices are left to the separate calls
+    # second call on the same scratch, other activations and a residual
+    x2 = (x32 * 0.5 + 0.25).to(x.dtype)
+    res = torch.randn(1, H, generator=g, device=dev)
+    ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x2, w.gate_q, gate, 1, I, H), ops.QmatmulJob(x2, w.up_q, up, 1, I, H)], tg)
+    ops.dispatch_silu_mul(gate, up, act)
+    ops.quantized_matmul_ggml(act, w.down_q, ref, GgmlQuantizedMatmulParams(1, H, I, td))
+    out2 = torch.full((1, H), float("nan"), device=dev)
+    ops.dense_ffn_decode(x2, w, out2, scratch, residual=res)
+    assert torch.equal(out2, ref + res)
+    assert ops.handover_status(scratch) == 0
+    # (b) the CPU specification in float64 over the dequantised weights
+    deq = lambda q, n, k, t: ops.dequantize_ggml(q, n * k, t).double().view(n, k)  # noqa: E731
+    xd = x.double()
+    gd, ud = xd @ deq(w.gate_q, I, H, tg).T, xd @ deq(w.up_q, I, H, tg).T
+    want = ((gd / (1 + torch.exp(-gd))) * ud) @ deq(w.down_q, H, I, td).T
+    from _util import assert_matmul_close
+    assert_matmul_close(out.cpu().numpy(), want.cpu().numpy(), f"dense ffn {H}x{I}")
+    # replayed from a HIP graph, with eager work between the replays
+    side = torch.cuda.Stream()
+    gr = torch.cuda.CUDAGraph()
+    out3 = torch.empty_like(out)
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(gr, stream=side):
+            ops.dense_ffn_decode(x, w, out3, scratch)
+    for _ in range(3):
+        out3.fill_(float("nan"))
+        gr.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out3, out)
+        ops.dense_ffn_decode(x2, w, out2, scratch, residual=res)
+        torch.cuda.synchronize()
+
+
+def test_dense_ffn_decode_rejects_what_it_does_not_take(dev):
+    w = ops.DenseFfnWeightsGpuQ(None, None, None, HQ_Q6_K, 4096, 12288, down_type=HQ_Q4_K)
+    assert ops.dense_ffn_decode_scratch_bytes(w, torch.bfloat16) == 0  # type mix outside the list
+    w = ops.DenseFfnWeightsGpuQ(None, None, None, HQ_Q4_K, 8192, 32768)
+    assert ops.dense_ffn_decode_scratch_bytes(w, torch.float32) == 0   # activations do not fit a CU's LDS
+    w = ops.DenseFfnWeightsGpuQ(None, None, None, HQ_Q4_K, 4096, 12288)
+    assert ops.dense_ffn_decode_scratch_bytes(w, torch.bfloat16) >= 12288 * 8
+
+
+def test_hand_over_waits_give_up_at_the_spin_limit_and_report_it(oracle, dev):
+    """A polling limit of zero makes every wait inside the one-launch blocks give up at once: all kernels still exit, the
+    scratch's error word says so, and the next call with the default limit is right again."""
+    from hf2q_amd import lib
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    H, I, t = 4096, 12288, HQ_Q4_K
+    qz = lambda n, k: ops.quantize_ggml(torch.randn(n * k, generator=g, device=dev).mul_(0.02), k, t)  # noqa: E731
+    w = ops.DenseFfnWeightsGpuQ(qz(I, H), qz(I, H), qz(H, I), t, H, I)
+    x = torch.randn(1, H, generator=g, device=dev).to(torch.bfloat16)
+    scratch = torch.zeros(ops.dense_ffn_decode_scratch_bytes(w, x.dtype), dtype=torch.uint8, device=dev)
+    good, out = torch.empty(1, H, device=dev), torch.empty(1, H, device=dev)
+    ops.dense_ffn_decode(x, w, good, scratch)
+    assert ops.handover_status(scratch) == 0
+    L = lib.load()
+    try:
+        L.hq_set_handover_spin_limit(1)
+        for _ in range(3):
+            ops.dense_ffn_decode(x, w, out, scratch)
+        torch.cuda.synchronize()
+        status = ops.handover_status(scratch)
+    finally:
+        L.hq_set_handover_spin_limit(0)
+    # (with a limit of one poll a wait may still find everything in place; three launches of 256 workgroups never all do)
+    assert status != 0
+    scratch.zero_()  # after a reported time-out the scratch starts over
+    ops.dense_ffn_decode(x, w, out, scratch)
+    assert torch.equal(out, good) and ops.handover_status(scratch) == 0
