@@ -86,6 +86,18 @@ pub struct hq_moe_ffn_layer {
     pub ggml_type: hq_ggml_type,
     pub expert_stride_gate_up: u64,
     pub expert_stride_down: u64,
+    pub down_type: u32,
+}
+
+#[repr(C)]
+#[derive(Clone, Copy, Debug)]
+pub struct hq_moe_ffn_row_scales {
+    pub expert_gate: *const f32,
+    pub expert_up: *const f32,
+    pub expert_down: *const f32,
+    pub shared_gate: *const f32,
+    pub shared_up: *const f32,
+    pub shared_down: *const f32,
 }
 
 #[repr(C)]
@@ -174,6 +186,10 @@ extern "C" {
     pub fn hq_set_handover_spin_limit(limit: u32);
     pub fn hq_dense_ffn_decode_scratch_bytes(hidden: u32, inter: u32, t_gate_up: hq_ggml_type, t_down: hq_ggml_type, xdt: hq_act_dtype) -> usize;
     pub fn hq_dense_ffn_decode(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_gate: *const c_void, w_up: *const c_void, w_down: *const c_void, t_gate_up: hq_ggml_type, t_down: hq_ggml_type, residual: *const f32, out: *mut f32, hidden: u32, inter: u32, scratch: *mut c_void, scratch_bytes: usize) -> c_int;
+    pub fn hq_moe_ffn_prefill_scratch_bytes(layer: *const hq_moe_ffn_layer, n_tokens: u32, xdt: hq_act_dtype) -> usize;
+    pub fn hq_moe_ffn_prefill(stream: *mut c_void, layer: *const hq_moe_ffn_layer, row_scales: *const hq_moe_ffn_row_scales, x: *const c_void, xdt: hq_act_dtype, residual: *const f32, out: *mut f32, n_tokens: u32, scratch: *mut c_void, scratch_bytes: usize, route_ids: *mut u32, route_weights: *mut f32) -> c_int;
+    pub fn hq_dense_ffn_scratch_bytes(m: u32, hidden: u32, inter: u32, t_gate_up: hq_ggml_type, t_down: hq_ggml_type, xdt: hq_act_dtype) -> usize;
+    pub fn hq_dense_ffn(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_gate: *const c_void, w_up: *const c_void, w_down: *const c_void, t_gate_up: hq_ggml_type, t_down: hq_ggml_type, gate_row_scales: *const f32, up_row_scales: *const f32, down_row_scales: *const f32, out: *mut f32, m: u32, hidden: u32, inter: u32, scratch: *mut c_void, scratch_bytes: usize) -> c_int;
     pub fn hq_fwht_sign_premult_f32(stream: *mut c_void, buf: *mut f32, n_heads: u32, head_dim: u32) -> c_int;
     pub fn hq_fwht_sign_undo_f32(stream: *mut c_void, buf: *mut f32, n_heads: u32, head_dim: u32) -> c_int;
     pub fn hq_tq_encode_kv(stream: *mut c_void, src: *const f32, codes: *mut u8, norms: *mut f32, n_tokens: u32, n_kv_heads: u32, head_dim: u32, capacity: u32, write_pos: u32) -> c_int;

@@ -601,7 +601,8 @@ int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* l, const void* x, hq
     const char* fn = "hq_moe_ffn_decode";
     if (!l) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null layer", fn);
     if (n_tokens == 0) return HQ_OK;
-    if (!moe_fused_supported(n_tokens, l->hidden, l->n_experts, l->top_k, l->inter, l->shared_inter, l->ggml_type, xdt))
+    if ((l->down_type && l->down_type != (uint32_t)l->ggml_type) ||
+        !moe_fused_supported(n_tokens, l->hidden, l->n_experts, l->top_k, l->inter, l->shared_inter, l->ggml_type, xdt))
         return fail(HQ_ERR_UNSUPPORTED,
                     "%s: takes 1..8 tokens of bf16 activations, Q4_K experts, hidden 2048, expert and shared FFN width 512, "
                     "<= 256 experts (got %u tokens, dtype %d, type %d, hidden %u, inter %u / %u, %u experts, top-%u); "

@@ -84,6 +84,10 @@ SIGNATURES = {
     "hq_set_handover_spin_limit": (None, [_u32]),
     "hq_dense_ffn_decode_scratch_bytes": (_sz, [_u32, _u32, _i32, _i32, _i32]),
     "hq_dense_ffn_decode": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _u32, _u32, _vp, _sz]),
+    "hq_moe_ffn_prefill_scratch_bytes": (_sz, [_vp, _u32, _i32]),
+    "hq_moe_ffn_prefill": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _vp, _u32, _vp, _sz, _vp, _vp]),
+    "hq_dense_ffn_scratch_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32, _i32]),
+    "hq_dense_ffn": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp, _sz]),
     "hq_fwht_sign_premult_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_fwht_sign_undo_f32": (_i32, [_vp, _vp, _u32, _u32]),
     "hq_tq_encode_kv": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
@@ -127,7 +131,13 @@ class MoeFfnLayer(ctypes.Structure):
     _fields_ = [("router", _vp), ("shared_gate_logit", _vp), ("expert_gate", _vp), ("expert_up", _vp), ("expert_down", _vp),
                 ("shared_gate", _vp), ("shared_up", _vp), ("shared_down", _vp), ("hidden", _u32), ("n_experts", _u32),
                 ("top_k", _u32), ("inter", _u32), ("shared_inter", _u32), ("ggml_type", _i32),
-                ("expert_stride_gate_up", _u64), ("expert_stride_down", _u64)]
+                ("expert_stride_gate_up", _u64), ("expert_stride_down", _u64), ("down_type", _u32)]
+
+
+class MoeFfnRowScales(ctypes.Structure):
+    """hq_moe_ffn_row_scales (include/hf2q_hip.h)."""
+    _fields_ = [("expert_gate", _vp), ("expert_up", _vp), ("expert_down", _vp), ("shared_gate", _vp), ("shared_up", _vp),
+                ("shared_down", _vp)]
 
 
 class TqAttnParams(ctypes.Structure):

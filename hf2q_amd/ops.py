@@ -754,20 +754,35 @@ class MoeFfnWeightsGpuQ:
     shared_inter: int
     # the tile kernels' weight-row scales of the six quantized matrices, filled by prepare_prefill() (optional)
     row_scales: dict | None = None
+    # type of expert_down / shared_down where it differs from ggml_type (Qwen3.6-35B-A3B: gate / up Q5_K, down Q6_K)
+    down_type: int | None = None
+
+    @property
+    def td(self) -> int:
+        return self.down_type if self.down_type is not None else self.ggml_type
+
+    def c_layer(self) -> "_l.MoeFfnLayer":
+        """hq_moe_ffn_layer of these weights (contiguous stacks)."""
+        rb_h, rb_i = ggml_row_bytes(self.ggml_type, self.hidden), ggml_row_bytes(self.td, self.inter)
+        return _l.MoeFfnLayer(_dev(self.router, "router"), _dev(self.shared_gate_logit, "shared_gate_logit"),
+                              _dev(self.expert_gate, "expert_gate"), _dev(self.expert_up, "expert_up"), _dev(self.expert_down, "expert_down"),
+                              _dev(self.shared_gate, "shared_gate"), _dev(self.shared_up, "shared_up"), _dev(self.shared_down, "shared_down"),
+                              self.hidden, self.n_experts, self.top_k, self.inter, self.shared_inter, self.ggml_type, self.inter * rb_h,
+                              self.hidden * rb_i, 0 if self.down_type is None else self.down_type)
 
     def prepare_prefill(self) -> None:
         """Once after the weights are uploaded: the row scales that prefill-sized calls would otherwise work out again in
         every pre-pass (4 bytes per weight row; they depend on the weights alone, so the results do not change)."""
-        t, H, E, I, SI = self.ggml_type, self.hidden, self.n_experts, self.inter, self.shared_inter
+        t, td, H, E, I, SI = self.ggml_type, self.td, self.hidden, self.n_experts, self.inter, self.shared_inter
         if t not in (HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0):
             return
         self.row_scales = {
             "expert_gate": weight_row_scales_ggml(self.expert_gate, E * I, H, t),
             "expert_up": weight_row_scales_ggml(self.expert_up, E * I, H, t),
-            "expert_down": weight_row_scales_ggml(self.expert_down, E * H, I, t),
+            "expert_down": weight_row_scales_ggml(self.expert_down, E * H, I, td),
             "shared_gate": weight_row_scales_ggml(self.shared_gate, SI, H, t),
             "shared_up": weight_row_scales_ggml(self.shared_up, SI, H, t),
-            "shared_down": weight_row_scales_ggml(self.shared_down, H, SI, t),
+            "shared_down": weight_row_scales_ggml(self.shared_down, H, SI, td),
         }
 
 
@@ -786,25 +801,25 @@ class MoeFfnScratch:
         self.sh_gate, self.sh_up, self.sh_act = f(T, w.shared_inter), f(T, w.shared_inter), f(T, w.shared_inter)
         self.sh_down = f(T, w.hidden)
         # workspace of the grouped (expert-sorted) form that prefill-sized mul_mat_id calls take (IdMmScratch, decode_pool.rs:56-60)
-        rb_h, rb_i = ggml_row_bytes(w.ggml_type, w.hidden), ggml_row_bytes(w.ggml_type, w.inter)
+        rb_h, rb_i = ggml_row_bytes(w.ggml_type, w.hidden), ggml_row_bytes(w.td, w.inter)
         need = max(
             quantized_matmul_id_swiglu_workspace_bytes(GgmlQuantizedMatmulIdParams(T, K, w.inter, w.hidden, w.n_experts,
                                                                                    w.inter * rb_h, w.ggml_type)),
             quantized_matmul_id_workspace_bytes(GgmlQuantizedMatmulIdParams(T, K, w.inter, w.hidden, w.n_experts,
                                                                             w.inter * rb_h, w.ggml_type)),
             quantized_matmul_id_workspace_bytes(GgmlQuantizedMatmulIdParams(T * K, 1, w.hidden, w.inter, w.n_experts,
-                                                                            w.hidden * rb_i, w.ggml_type)))
+                                                                            w.hidden * rb_i, w.td)))
         self.id_mm = torch.empty(need, dtype=torch.uint8, device=device) if need else None
         # workspace of the shared expert's prefill-sized dense products (the SwiGLU form where it exists, and the down product)
         pg = GgmlQuantizedMatmulParams(T, w.shared_inter, w.hidden, w.ggml_type)
-        pd = GgmlQuantizedMatmulParams(T, w.hidden, w.shared_inter, w.ggml_type)
+        pd = GgmlQuantizedMatmulParams(T, w.hidden, w.shared_inter, w.td)
         need = max(quantized_matmul_swiglu_workspace_bytes(pg, torch.bfloat16), quantized_matmul_workspace_bytes(pg, torch.bfloat16),
                    quantized_matmul_workspace_bytes(pd, torch.float32))
         self.dense_ws = torch.empty(need, dtype=torch.uint8, device=device) if need else None
         self.max_tokens = T
         # scratch of the one-launch decode block (hq_moe_ffn_decode): zeroed once, then the library's
-        fb = _l.load().hq_moe_ffn_decode_scratch_bytes(min(T, 8), w.hidden, w.n_experts, K, w.inter, w.shared_inter, w.ggml_type,
-                                                       _l.HQ_BF16)
+        fb = 0 if w.td != w.ggml_type else _l.load().hq_moe_ffn_decode_scratch_bytes(
+            min(T, 8), w.hidden, w.n_experts, K, w.inter, w.shared_inter, w.ggml_type, _l.HQ_BF16)
         self.fused = torch.zeros(fb, dtype=torch.uint8, device=device) if fb else None
 
 
@@ -820,11 +835,7 @@ def moe_ffn_decode_fused(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch
     """The whole block as one launch (hq_moe_ffn_decode); raises HqError(HQ_ERR_UNSUPPORTED) for shapes it does not take."""
     import ctypes as _ct
     T = x.shape[0]
-    rb_h, rb_i = ggml_row_bytes(w.ggml_type, w.hidden), ggml_row_bytes(w.ggml_type, w.inter)
-    layer = _l.MoeFfnLayer(_dev(w.router, "router"), _dev(w.shared_gate_logit, "shared_gate_logit"),
-                           _dev(w.expert_gate, "expert_gate"), _dev(w.expert_up, "expert_up"), _dev(w.expert_down, "expert_down"),
-                           _dev(w.shared_gate, "shared_gate"), _dev(w.shared_up, "shared_up"), _dev(w.shared_down, "shared_down"),
-                           w.hidden, w.n_experts, w.top_k, w.inter, w.shared_inter, w.ggml_type, w.inter * rb_h, w.hidden * rb_i)
+    layer = w.c_layer()
     if s.fused is None:
         raise _l.HqError(_l.HQ_ERR_UNSUPPORTED, "no scratch for the one-launch MoE block (shape not supported)")
     L = _l.load()
@@ -845,7 +856,7 @@ _FUSED_CHUNKED_MAX_TOKENS = 48
 
 def moe_ffn_decode_fused_supported(x: torch.Tensor, w: MoeFfnWeightsGpuQ) -> bool:
     T = x.shape[0]
-    if T > _FUSED_CHUNKED_MAX_TOKENS:
+    if T > _FUSED_CHUNKED_MAX_TOKENS or w.td != w.ggml_type:
         return False
     return bool(_l.load().hq_moe_ffn_decode_scratch_bytes(min(T, 8), w.hidden, w.n_experts, w.top_k, w.inter, w.shared_inter,
                                                           w.ggml_type, _act_dtype(x)))
@@ -865,7 +876,7 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
     softmax / top-k, four launches (measured per layer: 23.9 -> 21.7 us at one token, 35.3 -> 33.8 at four, 50.3 ->
     51.6 at eight, where every one of the many workgroups repeating the routing costs more than the launch saved)."""
     T = x.shape[0]
-    K, H, E, I, SI, t = w.top_k, w.hidden, w.n_experts, w.inter, w.shared_inter, w.ggml_type
+    K, H, E, I, SI, t, td = w.top_k, w.hidden, w.n_experts, w.inter, w.shared_inter, w.ggml_type, w.td
     rb = ggml_row_bytes(t, H)
     if fused is None:
         fused = batched is None and route_in_launch is None and s.fused is not None and moe_ffn_decode_fused_supported(x, w)
@@ -895,9 +906,9 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
         ], t)
         quantized_matmul_batch_ggml([
             QmatmulJob(s.gate, w.expert_down, s.down, T * K, H, I, ids=s.ids, top_k=1, n_experts=E,
-                       expert_stride=H * ggml_row_bytes(t, I), input_up=s.up),
+                       expert_stride=H * ggml_row_bytes(td, I), input_up=s.up),
             QmatmulJob(s.sh_gate, w.shared_down, s.sh_down, T, H, SI, input_up=s.sh_up),
-        ], t)
+        ], td)
         dispatch_moe_weighted_reduce(s.down, s.topk_w, out, T, K, H, shared=s.sh_down, shared_logit=s.sh_logit,
                                      residual=residual)
         return
@@ -929,15 +940,58 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
         quantized_matmul_id_ggml(x, w.expert_gate, s.ids, s.gate, pid, scratch=ws, w_row_scales=rsc.get("expert_gate"))
         quantized_matmul_id_ggml(x, w.expert_up, s.ids, s.up, pid, scratch=ws, w_row_scales=rsc.get("expert_up"))
         dispatch_silu_mul(s.gate[:T * K], s.up[:T * K], s.act[:T * K])
-    pdn = GgmlQuantizedMatmulParams(T, H, SI, t)
+    pdn = GgmlQuantizedMatmulParams(T, H, SI, td)
     if dws is not None and quantized_matmul_workspace_bytes(pdn, torch.float32):
         quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, pdn, workspace=dws, w_row_scales=rsc.get("shared_down"))
     else:
         quantized_matmul_ggml(s.sh_act, w.shared_down, s.sh_down, pdn)
     # E
     quantized_matmul_id_ggml(s.act, w.expert_down, s.ids, s.down,
-                             GgmlQuantizedMatmulIdParams(T * K, 1, H, I, E, H * ggml_row_bytes(t, I), t), scratch=ws,
+                             GgmlQuantizedMatmulIdParams(T * K, 1, H, I, E, H * ggml_row_bytes(td, I), td), scratch=ws,
                              w_row_scales=rsc.get("expert_down"))
     # F
     dispatch_moe_weighted_reduce(s.down, s.topk_w, out, T, K, H, shared=s.sh_down, shared_logit=s.sh_logit,
                                  residual=residual)
+
+
+def moe_ffn_prefill_scratch_bytes(w: MoeFfnWeightsGpuQ, n_tokens: int, act_dtype: torch.dtype) -> int:
+    import ctypes as _ct
+    layer = w.c_layer()
+    xdt = HQ_BF16 if act_dtype == torch.bfloat16 else HQ_F32
+    return int(_l.load().hq_moe_ffn_prefill_scratch_bytes(_ct.byref(layer), n_tokens, xdt))
+
+
+def moe_ffn_prefill(x: torch.Tensor, w: MoeFfnWeightsGpuQ, out: torch.Tensor, scratch: torch.Tensor,
+                    residual: torch.Tensor | None = None, route_ids: torch.Tensor | None = None,
+                    route_weights: torch.Tensor | None = None) -> None:
+    """build_moe_ffn_layer_gpu_q_into (gpu_ffn.rs:2313-2802) as ONE library call at any token count, every buffer carved
+    from `scratch` (moe_ffn_prefill_scratch_bytes); the bits of the separate dispatches above.  Row scales kept by
+    prepare_prefill() are passed on."""
+    import ctypes as _ct
+    layer = w.c_layer()
+    rs = None
+    if w.row_scales:
+        g = lambda k: _dev(w.row_scales[k], k) if w.row_scales.get(k) is not None else None  # noqa: E731
+        rs = _l.MoeFfnRowScales(g("expert_gate"), g("expert_up"), g("expert_down"), g("shared_gate"), g("shared_up"), g("shared_down"))
+    _l.check(_l.load().hq_moe_ffn_prefill(
+        _stream(), _ct.byref(layer), _ct.byref(rs) if rs is not None else None, _dev(x, "x"), _act_dtype(x),
+        _dev(residual, "residual") if residual is not None else None, _dev(out, "out"), x.shape[0], _dev(scratch, "scratch"),
+        scratch.numel() * scratch.element_size(), _dev(route_ids, "route_ids") if route_ids is not None else None,
+        _dev(route_weights, "route_weights") if route_weights is not None else None))
+
+
+def dense_ffn_scratch_bytes(w: DenseFfnWeightsGpuQ, m: int, act_dtype: torch.dtype) -> int:
+    xdt = HQ_BF16 if act_dtype == torch.bfloat16 else HQ_F32
+    td = w.down_type if w.down_type is not None else w.ggml_type
+    return int(_l.load().hq_dense_ffn_scratch_bytes(m, w.hidden, w.inter, w.ggml_type, td, xdt))
+
+
+def dense_ffn(x: torch.Tensor, w: DenseFfnWeightsGpuQ, out: torch.Tensor, scratch: torch.Tensor, row_scales: dict | None = None) -> None:
+    """build_dense_ffn_layer_gpu_q (gpu_ffn.rs:1017-1351) as ONE library call at any row count, buffers carved from
+    `scratch` (dense_ffn_scratch_bytes); the bits of build_dense_ffn_layer_gpu_q_into."""
+    td = w.down_type if w.down_type is not None else w.ggml_type
+    rs = row_scales or {}
+    g = lambda k: _dev(rs[k], k) if rs.get(k) is not None else None  # noqa: E731
+    _l.check(_l.load().hq_dense_ffn(_stream(), _dev(x, "x"), _act_dtype(x), _dev(w.gate_q, "gate"), _dev(w.up_q, "up"), _dev(w.down_q, "down"),
+                                    w.ggml_type, td, g("gate"), g("up"), g("down"), _dev(out, "out"), x.shape[0], w.hidden, w.inter,
+                                    _dev(scratch, "scratch"), scratch.numel() * scratch.element_size()))

@@ -357,6 +357,8 @@ typedef struct hq_moe_ffn_layer {
     hq_ggml_type ggml_type;
     uint64_t expert_stride_gate_up; /* bytes between experts of expert_gate / expert_up */
     uint64_t expert_stride_down;
+    uint32_t down_type;             /* hq_ggml_type of expert_down / shared_down where it differs from ggml_type
+                                     * (Qwen3.6-35B-A3B stores gate / up in Q5_K and down in Q6_K); 0: ggml_type */
 } hq_moe_ffn_layer;
 HQ_API size_t hq_moe_ffn_decode_scratch_bytes(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k,
                                        uint32_t inter, uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt);
@@ -393,6 +395,45 @@ HQ_API size_t hq_dense_ffn_decode_scratch_bytes(uint32_t hidden, uint32_t inter,
 HQ_API int hq_dense_ffn_decode(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up,
                         const void* w_down, hq_ggml_type t_gate_up, hq_ggml_type t_down, const float* residual, float* out,
                         uint32_t hidden, uint32_t inter, void* scratch, size_t scratch_bytes);
+
+/* The whole MoE FFN block at ANY token count, as the sequence of this library's calls that a caller encoding the phases
+ * of build_moe_ffn_layer_gpu_q_into (gpu_ffn.rs:2313-2802) one by one would issue, with every intermediate buffer and
+ * workspace carved out of ONE caller scratch (the decode pool and IdMmScratch of decode_pool.rs:56-60 in one piece):
+ *   up to 8 tokens   the decode dispatches, a phase per launch: router + shared-gate logits, [routing inside] gate / up of
+ *                    the routed and the shared expert, both down projections with their SwiGLU folded in, weighted sum;
+ *   more             router and shared logits, the shared expert (gate + up + SwiGLU as one tile call where that exists),
+ *                    softmax / top-k, the routed experts' gate + up + SwiGLU as one grouped product where that exists (else
+ *                    two mul_mat_id calls and hq_silu_mul; the grouped tile form from 3 routed rows per expert, one GEMV
+ *                    per routed row below), the down mul_mat_id over n_tokens * top_k rows, the weighted sum.
+ * The result has the bits of those calls made by hand.  Per-matrix types: gate / up of layer->ggml_type, down of
+ * layer->down_type.  row_scales: NULL, or the weight-row scales of the six matrices kept from load time
+ * (hq_weight_row_scales_ggml; any member may be NULL), which take the header scans out of the prefill-sized calls.
+ * scratch: hq_moe_ffn_prefill_scratch_bytes() bytes for this token count (more tokens need more), 256-byte aligned,
+ * contents irrelevant.  route_ids / route_weights: NULL, or where the routing is also copied ([n_tokens * top_k] each).
+ * (hq_moe_ffn_decode is the one-launch form of the same block for the shapes it takes.) */
+typedef struct hq_moe_ffn_row_scales {
+    const float *expert_gate, *expert_up, *expert_down, *shared_gate, *shared_up, *shared_down;
+} hq_moe_ffn_row_scales;
+HQ_API size_t hq_moe_ffn_prefill_scratch_bytes(const hq_moe_ffn_layer* layer, uint32_t n_tokens, hq_act_dtype xdt);
+HQ_API int hq_moe_ffn_prefill(void* stream, const hq_moe_ffn_layer* layer, const hq_moe_ffn_row_scales* row_scales, const void* x,
+                       hq_act_dtype xdt, const float* residual, float* out, uint32_t n_tokens, void* scratch,
+                       size_t scratch_bytes, uint32_t* route_ids, float* route_weights);
+
+/* The dense SwiGLU FFN at ANY row count: out[m, hidden] = W_down . (silu(W_gate . x) * (W_up . x)), the sequence of calls
+ * that stands for build_dense_ffn_layer_gpu_q (gpu_ffn.rs:1017-1351) with its buffers carved out of one caller scratch:
+ *   up to 8 rows   gate + up + SwiGLU as one streaming launch per row (hq_qmatmul_swiglu_decode) and the down GEMV; for
+ *                  matrices too small for that, gate and up as one batched launch and the down GEMV with the SwiGLU
+ *                  folded into its staging (inter <= 8192) or behind hq_silu_mul;
+ *   more           gate, the up projection finishing the gating in its epilogue (hq_qmatmul_gated_ggml_ws; where the tile
+ *                  route has no such form: up and hq_silu_mul), down.
+ * The bits of those calls made by hand.  *_row_scales: NULL, or from hq_weight_row_scales_ggml.  scratch:
+ * hq_dense_ffn_scratch_bytes() bytes for this m, 256-byte aligned, contents irrelevant. */
+HQ_API size_t hq_dense_ffn_scratch_bytes(uint32_t m, uint32_t hidden, uint32_t inter, hq_ggml_type t_gate_up, hq_ggml_type t_down,
+                                  hq_act_dtype xdt);
+HQ_API int hq_dense_ffn(void* stream, const void* x, hq_act_dtype xdt, const void* w_gate, const void* w_up, const void* w_down,
+                 hq_ggml_type t_gate_up, hq_ggml_type t_down, const float* gate_row_scales, const float* up_row_scales,
+                 const float* down_row_scales, float* out, uint32_t m, uint32_t hidden, uint32_t inter, void* scratch,
+                 size_t scratch_bytes);
 
 /* In-place  buf <- H.(s (.) buf)  per 256-element block of buf[n_heads][head_dim] (query
  * pre-rotation) and its inverse  buf <- s (.) (H.buf)  (output post-rotation).  Replace

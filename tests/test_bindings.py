@@ -70,7 +70,7 @@ def test_extern_block_matches_the_header():
 
 def test_repr_c_structs_match_the_header():
     h, r = _header_structs(), _rust_structs()
-    for name in ("hq_qmatmul_job", "hq_moe_ffn_layer", "hq_tq_attn_params", "hq_tqp_header", "hq_gguf_tensor_info"):
+    for name in ("hq_qmatmul_job", "hq_moe_ffn_layer", "hq_moe_ffn_row_scales", "hq_tq_attn_params", "hq_tqp_header", "hq_gguf_tensor_info"):
         assert name in h and name in r, name
         assert h[name] == r[name], f"{name}: header {h[name]} vs crate {r[name]}"
 

@@ -344,3 +344,50 @@ def test_tq_attention_full_size(oracle, dev):
     # (the softmax weights are 22-bit numbers summed over 32768 positions: 2e-5 of the magnitude observed)
     err, mag = float(np.abs(out.cpu().numpy() - want).max()), float(np.abs(want).max())
     assert err <= 1e-4 * mag, f"constant-value cache: {err} vs {mag}"
+
+
+def test_tq_attention_full_size_over_an_encoded_cache(oracle, dev):
+    """BASELINE config 5 as it is stated: K and V ~ N(0, 1), rotated and quantised per (token, head) by hq_tq_encode_kv
+    (the cache then has the code and scale statistics of real keys, not uniform codes), 32768 positions, 16 / 2 heads,
+    d = 256.  The device encode is byte-equal to the oracle's on sampled positions, the attention over the device-built
+    cache matches the f64 oracle over the same bytes, and against exact f32 attention over the un-quantised K / V the
+    whole chain stays far inside the reference's NRMSE gate (kv_cache.rs:3959: < 0.15)."""
+    nh, nkv, hd, n = 16, 2, 256, 32768
+    g = torch.Generator(device=dev)
+    g.manual_seed(1234)
+    k = torch.randn(n, nkv, hd, generator=g, device=dev)
+    v = torch.randn(n, nkv, hd, generator=g, device=dev)
+    q = torch.randn(nh, hd, generator=g, device=dev)
+    kc, kn = ops.alloc_tq_kv(nkv, n, hd, dev)
+    vc, vn = ops.alloc_tq_kv(nkv, n, hd, dev)
+    ops.hadamard_quantize_kv(k, kc, kn, 0)
+    ops.hadamard_quantize_kv(v, vc, vn, 0)
+    kch, knh, vch, vnh = (t.cpu().numpy() for t in (kc, kn, vc, vn))
+    # the encode, on sampled positions, against the oracle
+    rng = np.random.default_rng(7)
+    for pos in np.unique(np.concatenate([[0, 1, n - 1], rng.integers(0, n, 29)])):
+        codes = np.zeros((nkv, 1, hd), np.uint8)
+        norms = np.zeros((nkv, 1, 1), np.float32)
+        oracle.tq_encode_int8(k[pos].cpu().numpy(), nkv, hd, 1, 0, codes, norms)
+        assert np.array_equal(codes[:, 0], kch[:, pos]) and np.array_equal(norms[:, 0], knh[:, pos]), pos
+    p = FlashAttnVecTqHbParams(nh, nkv, hd, n, n, 1.0 / 16.0, fuse_fwht_pre=1)
+    tmp = torch.empty(ops.tq_tmp_buffer_bytes(nh, hd, n) // 4, device=dev)
+    out = torch.full((nh, hd), float("nan"), device=dev)
+    ops.flash_attn_vec_tq_hb(q, kc, kn, vc, vn, out, tmp, p, undo_rotation=True)
+    got = out.cpu().numpy()
+    qr = oracle.fwht_sign_premult(q.cpu().numpy().copy(), nh, hd)
+    ref = oracle.tq_attention(qr, kch, knh, vch, vnh, None, nh, nkv, hd, n, n, p.scale)
+    ref = oracle.fwht_sign_undo(ref.astype(np.float32), nh, hd)
+    scale = np.abs(ref).max(axis=1, keepdims=True)
+    assert np.isfinite(got).all() and (np.abs(got - ref) <= 1e-3 * scale).all()
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) < 1e-4
+    # against attention over the un-quantised keys and values (float64 on the device)
+    qd, kd, vd = q.double(), k.double(), v.double()
+    exact = torch.empty(nh, hd, dtype=torch.float64, device=dev)
+    for h in range(nh):
+        kv = h // (nh // nkv)
+        w = torch.softmax((kd[:, kv, :] @ qd[h]) * p.scale, dim=0)
+        exact[h] = w @ vd[:, kv, :]
+    ex = exact.cpu().numpy()
+    nrmse = np.sqrt(((got - ex) ** 2).sum() / (ex ** 2).sum())
+    assert nrmse < 0.05, nrmse

@@ -566,3 +566,92 @@ def test_hand_over_waits_give_up_at_the_spin_limit_and_report_it(oracle, dev):
     scratch.zero_()  # after a reported time-out the scratch starts over
     ops.dense_ffn_decode(x, w, out, scratch)
     assert torch.equal(out, good) and ops.handover_status(scratch) == 0
+
+
+def _moe_weights_mixed(oracle, dev, t, td, H, E, K, I, SI, seed=0):
+    w = _moe_weights(oracle, dev, t, H, E, K, I, SI, seed=seed)
+    if td != t:
+        dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+        w.expert_down = dv(oracle.quantize(weights(3 + seed, E * H, I, 0.05), I, td, threads=8))
+        w.shared_down = dv(oracle.quantize(weights(6 + seed, H, SI, 0.05), SI, td, threads=8))
+        w.down_type = td
+    return w
+
+
+@pytest.mark.parametrize("T", [1, 3, 8, 9, 40, 96, 300])
+@pytest.mark.parametrize("t,td,xdt", [(HQ_Q4_K, HQ_Q4_K, torch.bfloat16), (HQ_Q5_K, HQ_Q6_K, torch.float32), (HQ_Q8_0, HQ_Q8_0, torch.bfloat16)])
+def test_moe_block_as_one_library_call_equals_the_dispatches_made_by_hand(oracle, dev, T, t, td, xdt):
+    """hq_moe_ffn_prefill (one C call, one scratch, any token count; also the reference's real type mix: gate / up Q5_K, down
+    Q6_K) against build_moe_ffn_layer_gpu_q_into's own sequence of dispatches: bit for bit, routing included; with row scales
+    kept from load time as well."""
+    H, E, K, I, SI = 512, 8, 4, 256, 256
+    w = _moe_weights_mixed(oracle, dev, t, td, H, E, K, I, SI, seed=T)
+    x = torch.from_numpy(acts(21 + T, T, H)).to(dev).to(xdt)
+    res = torch.from_numpy(acts(22, T, H)).to(dev)
+    s = ops.MoeFfnScratch(w, T, dev)
+    want = torch.full((T, H), float("nan"), device=dev)
+    ops.build_moe_ffn_layer_gpu_q_into(x, w, s, want, residual=res, fused=False)
+    need = ops.moe_ffn_prefill_scratch_bytes(w, T, x.dtype)
+    assert need > 0
+    scratch = torch.full((need,), 0xA5, dtype=torch.uint8, device=dev)  # contents irrelevant
+    got = torch.full((T, H), float("nan"), device=dev)
+    ids = torch.full((T * K,), -1, dtype=torch.int32, device=dev)
+    wts = torch.full((T * K,), float("nan"), device=dev)
+    ops.moe_ffn_prefill(x, w, got, scratch, residual=res, route_ids=ids, route_weights=wts)
+    assert torch.isfinite(got).all() and torch.equal(got, want)
+    assert torch.equal(ids, s.ids[:T * K]) and torch.equal(wts, s.topk_w[:T * K])
+    w.prepare_prefill()
+    got2 = torch.full((T, H), float("nan"), device=dev)
+    ops.moe_ffn_prefill(x, w, got2, scratch, residual=res)
+    assert torch.equal(got2, want)
+    # too small a scratch is refused before anything runs
+    with pytest.raises(ops.HqError):
+        ops.moe_ffn_prefill(x, w, got2, scratch[:need - 256], residual=res)
+
+
+def test_moe_block_mixed_types_match_cpu_spec(oracle, dev):
+    """gate / up Q5_K with down Q6_K (the reference model's mix, docs/ADR-028...:4942-4946) against moe_ffn_cpu_ref over the
+    dequantised weights, at one token (decode dispatches) and at 96 (grouped tiles)."""
+    H, E, K, I, SI = 512, 8, 4, 256, 256
+    t, td = HQ_Q5_K, HQ_Q6_K
+    rng = np.random.default_rng(77)
+    bf = lambda a: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(a))  # noqa: E731
+    router = bf((rng.standard_normal((E, H)) * 0.1).astype(np.float32))
+    sgl = bf((rng.standard_normal((1, H)) * 0.05).astype(np.float32))
+    raw = {nm: (weights(seed, n, k, 0.05), ty) for nm, seed, n, k, ty in
+           (("eg", 1, E * I, H, t), ("eu", 2, E * I, H, t), ("ed", 3, E * H, I, td), ("sg", 4, SI, H, t), ("su", 5, SI, H, t), ("sd", 6, H, SI, td))}
+    q = {nm: oracle.quantize(a, a.shape[1], ty, threads=8) for nm, (a, ty) in raw.items()}
+    dq = {nm: oracle.dequantize(q[nm], raw[nm][1]).reshape(raw[nm][0].shape) for nm in raw}
+    dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    w = ops.MoeFfnWeightsGpuQ(dv(router).to(torch.bfloat16), dv(q["eg"]), dv(q["eu"]), dv(q["ed"]), dv(sgl).to(torch.bfloat16),
+                              dv(q["sg"]), dv(q["su"]), dv(q["sd"]), t, H, E, K, I, SI, down_type=td)
+    for T, tol in ((1, 2e-4), (96, 2e-3)):
+        x = acts(7 + T, T, H)
+        want = oracle.moe_ffn(x, H, E, K, I, SI, router, dq["eg"], dq["eu"], dq["ed"], sgl[0], dq["sg"], dq["su"], dq["sd"])
+        scratch = torch.empty(ops.moe_ffn_prefill_scratch_bytes(w, T, torch.float32), dtype=torch.uint8, device=dev)
+        out = torch.full((T, H), float("nan"), device=dev)
+        ops.moe_ffn_prefill(dv(x), w, out, scratch)
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all() and np.abs(got - want).max() <= tol * np.abs(want).max()
+
+
+@pytest.mark.parametrize("m", [1, 4, 8, 9, 64, 300])
+@pytest.mark.parametrize("H,I,tg,td,xdt", [(4096, 8192, HQ_Q4_K, HQ_Q4_K, torch.bfloat16), (512, 1024, HQ_Q4_K, HQ_Q6_K, torch.float32),
+                                           (1024, 12288, HQ_Q8_0, HQ_Q8_0, torch.bfloat16)])
+def test_dense_ffn_as_one_library_call_equals_the_dispatches_made_by_hand(oracle, dev, m, H, I, tg, td, xdt):
+    """hq_dense_ffn against build_dense_ffn_layer_gpu_q_into (decode: gate + up + SwiGLU launch or batched launches; prefill:
+    gate, gated up, down with a workspace): bit for bit."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(H + I + m)
+    qz = lambda n, k, t: ops.quantize_ggml(torch.randn(n * k, generator=g, device=dev).mul_(0.02), k, t)  # noqa: E731
+    w = ops.DenseFfnWeightsGpuQ(qz(I, H, tg), qz(I, H, tg), qz(H, I, td), tg, H, I, down_type=td)
+    x = torch.randn(m, H, generator=g, device=dev).to(xdt)
+    gate, up, act = (torch.full((m, I), float("nan"), device=dev) for _ in range(3))
+    want = torch.full((m, H), float("nan"), device=dev)
+    nws = ops.dense_ffn_workspace_bytes(w, m, x.dtype)
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev) if nws else None
+    ops.build_dense_ffn_layer_gpu_q_into(x, w, gate, up, act, want, workspace=ws)
+    scratch = torch.full((ops.dense_ffn_scratch_bytes(w, m, x.dtype),), 0x5A, dtype=torch.uint8, device=dev)
+    got = torch.full((m, H), float("nan"), device=dev)
+    ops.dense_ffn(x, w, got, scratch)
+    assert torch.isfinite(got).all() and torch.equal(got, want)

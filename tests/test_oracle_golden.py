@@ -365,6 +365,63 @@ def test_rotation_is_sign_then_sylvester_hadamard(oracle):
     assert np.allclose(g2[0, 256:], (y[0, 256:] * s) @ H.T, atol=1e-5)
 
 
+def test_sign_table_is_the_reference_table_byte_for_byte(oracle):
+    # kv_cache.rs:3871-3876 (TBQ_SIGNS_256); its first eight bytes are ggml's TBQ_SIGNS_64 (docs/ADR-007...:624)
+    want = bytes.fromhex("a73b91f46dc2580e b37f24d68945ea1c 63afd852970be13d 76c419fe4a852cdb".replace(" ", ""))
+    assert bytes(int(b) for b in oracle.TBQ_SIGNS_256) == want and len(want) == 32
+    # and the rotation really uses all of them: flipping the sign of element j alone flips the table's bit j
+    x = np.ones((1, 256), np.float32)
+    H = _hadamard(256)
+    got = oracle.fwht_sign_premult(x, 1, 256)[0]
+    s = np.array([-1.0 if (want[j >> 3] >> (j & 7)) & 1 else 1.0 for j in range(256)])
+    assert np.allclose(got, s @ H.T, atol=1e-5)
+    assert np.allclose(oracle.fwht_sign_undo(got.reshape(1, 256).copy(), 1, 256)[0], 1.0, atol=1e-5)
+
+
+def test_tq_encode_int8_is_amax_over_127_and_round_half_away(oracle):
+    """The linear int8 map of the benchmark configuration, restated in numpy on the ROTATED vector: norm = amax / 127 (an
+    f32 division), code = round-half-away-from-zero(x * (1 / norm)) as int8, an all-zero vector gives norm 0 and codes 0.
+    A truncating cast, round-half-even, a division instead of the reciprocal multiply or amax / 128 each change bytes here."""
+    rng = np.random.default_rng(41)
+    d, cap = 256, 4
+    for trial in range(6):
+        if trial == 0:
+            rot = np.zeros(d, np.float32)
+        elif trial == 1:  # exact ties: amax 127 => norm 1, values k + 0.5 must round away from zero
+            rot = (rng.integers(-126, 126, d) + 0.5).astype(np.float32)
+            rot[0] = 127.0
+        elif trial == 2:  # a scale whose reciprocal is not exact: x * (1 / d) and x / d differ in the last bit for some x
+            rot = (rng.standard_normal(d) * 3.0).astype(np.float32)
+            rot[5] = 7.3
+        else:
+            rot = (rng.standard_normal(d) * 10.0 ** rng.integers(-6, 6)).astype(np.float32)
+        # the oracle encodes un-rotated input: hand it the inverse rotation of `rot` so that its rotation gives `rot` back
+        # bit for bit only where the FWHT is exact; take what its own rotation yields as the vector that was quantised
+        x = oracle.fwht_sign_undo(rot.reshape(1, d).copy(), 1, d).astype(np.float32)
+        r = oracle.fwht_sign_premult(x.copy(), 1, d)[0].astype(np.float32)
+        codes = np.zeros((1, cap, d), np.uint8)
+        norms = np.zeros((1, cap, 1), np.float32)
+        oracle.tq_encode_int8(x, 1, d, cap, 2, codes, norms)
+        amax = np.float32(np.abs(r).max())
+        norm = np.float32(amax / np.float32(127.0))
+        assert norms[0, 2, 0] == norm
+        inv = np.float32(1.0) / norm if norm != 0 else np.float32(0.0)
+        prod = (r * inv).astype(np.float32)
+        want = (np.sign(prod) * np.floor(np.abs(prod) + np.float32(0.5))).astype(np.int32)  # half away from zero
+        assert np.abs(want).max() <= 127
+        assert np.array_equal(codes[0, 2].view(np.int8).astype(np.int32), want), f"trial {trial}"
+        assert not codes[0, [0, 1, 3]].any() and not norms[0, [0, 1, 3]].any()  # only the addressed slot is written
+    # ties really occurred and went away from zero in trial 1
+    rot = np.array([127.0, 0.5, -0.5, 1.5, -2.5] + [0.0] * 251, np.float32)
+    x = oracle.fwht_sign_undo(rot.reshape(1, d).copy(), 1, d).astype(np.float32)
+    r = oracle.fwht_sign_premult(x.copy(), 1, d)[0]
+    if np.array_equal(r[:5], rot[:5]):  # (the rotation reproduces these small dyadic values exactly)
+        codes = np.zeros((1, 1, d), np.uint8)
+        norms = np.zeros((1, 1, 1), np.float32)
+        oracle.tq_encode_int8(x, 1, d, 1, 0, codes, norms)
+        assert codes[0, 0, :5].view(np.int8).tolist() == [127, 1, -1, 2, -3]
+
+
 def _encode_cache(oracle, kv, n_kv, d, cap):
     codes = np.zeros((n_kv, cap, d), np.uint8)
     norms = np.zeros((n_kv, cap, max(1, d // 256)), np.float32)
