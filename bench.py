@@ -126,6 +126,80 @@ def cpu_baseline() -> dict:
     }
 
 
+def cpu_baselines_by_config() -> dict:
+    """hf2q's CPU path (dequantize + scalar f32 matmul, ffn.rs:38-50; the scalar MoE block, ffn.rs:179-336) on bounded samples
+    of BASELINE configs 2-5, one thread, in each config's own unit; a few seconds each.  The oracle is what is timed here."""
+    import numpy as np
+
+    import oracle
+
+    oracle.build()
+    rng = np.random.default_rng(1234)
+    out = {}
+
+    def gemv(n_full, k, t, rows, name):
+        w = rng.standard_normal((rows, k), dtype=np.float32) * np.float32(0.02)
+        x = np.random.default_rng(5678).standard_normal((1, k), dtype=np.float32)
+        blocks = oracle.quantize(w, k, t, threads=min(os.cpu_count() or 1, 16))
+        wd = oracle.dequantize(blocks, t, threads=1)  # (untimed: the first call pays for the pages of its output)
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            wd = oracle.dequantize(blocks, t, threads=1)
+        t_deq = (time.perf_counter() - t0) / reps
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            oracle.matmul_a_by_bt(x, wd, 1, k, rows, threads=1)
+        t_mm = (time.perf_counter() - t0) / reps
+        return {"value": round(blocks.size / (t_deq + t_mm) / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{name}: the first {rows} of {n_full} rows x {k}, dequantize {t_deq * 1e3:.1f} ms + scalar f32 GEMV {t_mm * 1e3:.1f} ms"}
+
+    # config 2: the Q4_K gate / up shape and the Q6_K head, a slice of rows each
+    out["config2_decode_gemv"] = {"q4_k_12288x4096": gemv(12288, 4096, oracle.Q4_K, 2048, "Q4_K 12288 x 4096"),
+                                  "q6_k_head_151936x4096": gemv(151936, 4096, oracle.Q6_K, 2048, "Q6_K 151936 x 4096")}
+    # config 3: the scalar MoE block at one token; 32 of the 256 experts resident (the block touches the 8 routed ones and the
+    # shared one, the router over 32 instead of 256 rows), weights dequantised once as hf2q's CPU path does at load time
+    H, E, K, I = 2048, 32, 8, 512
+    mk = lambda n, k: oracle.dequantize(oracle.quantize(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02), k, oracle.Q4_K,  # noqa: E731
+                                                        threads=min(os.cpu_count() or 1, 16)), oracle.Q4_K, threads=8).reshape(n, k)
+    eg, eu, ed, sg, su, sd = mk(E * I, H), mk(E * I, H), mk(E * H, I), mk(I, H), mk(I, H), mk(H, I)
+    router = rng.standard_normal((E, H), dtype=np.float32) * np.float32(0.1)
+    sgl = rng.standard_normal(H, dtype=np.float32) * np.float32(0.05)
+    x = rng.standard_normal((1, H), dtype=np.float32)
+    reps = 5
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        oracle.moe_ffn(x, H, E, K, I, I, router, eg, eu, ed, sgl, sg, su, sd)
+    t_layer = (time.perf_counter() - t0) / reps
+    out["config3_moe_decode_t1"] = {"value": round(1.0 / (40 * t_layer), 3), "unit": "tok/s", "cores": 1, "kind": "port",
+                                    "sample": f"scalar MoE block (moe_ffn_cpu_ref) at one token, hidden 2048, top-8 of 32 resident experts x 512 + "
+                                              f"shared expert, f32 weights dequantised beforehand: {t_layer * 1e3:.1f} ms per layer, x 40 layers"}
+    # config 4: scalar f32 matmul over the dequantised Q4_K weights, 2 of the 2048 tokens
+    M, Kd, N = 2, 4096, 12288
+    wd = mk(N, Kd)
+    xs = rng.standard_normal((M, Kd), dtype=np.float32)
+    t0 = time.perf_counter()
+    oracle.matmul_a_by_bt(xs, wd, M, Kd, N, threads=1)
+    t_mm = time.perf_counter() - t0
+    out["config4_prefill_gemm"] = {"value": round(2.0 * M * N * Kd / t_mm / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                                   "sample": f"matmul_a_by_bt over dequantised Q4_K weights, {M} of 2048 tokens x 4096 x 12288: {t_mm * 1e3:.0f} ms"}
+    # config 5: scalar attention over the int8 cache, 2048 of the 32768 positions
+    nh, nkv, hd, n = 16, 2, 256, 2048
+    kc = rng.integers(-127, 128, (nkv, n, hd)).astype(np.int8).view(np.uint8)
+    vc = rng.integers(-127, 128, (nkv, n, hd)).astype(np.int8).view(np.uint8)
+    kn = rng.uniform(0.5, 2.0, (nkv, n, 1)).astype(np.float32)
+    vn = rng.uniform(0.5, 2.0, (nkv, n, 1)).astype(np.float32)
+    q = rng.standard_normal((nh, hd)).astype(np.float32)
+    t0 = time.perf_counter()
+    oracle.tq_attention(q, kc, kn, vc, vn, None, nh, nkv, hd, n, n, 1.0 / 16.0)
+    t_at = time.perf_counter() - t0
+    nbytes = 2 * nkv * n * (hd + 4)
+    out["config5_tq_attention"] = {"value": round(nbytes / t_at / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                                   "sample": f"scalar C attention over the int8 cache (dequantise in the loop, f64 accumulate), {n} of 32768 "
+                                             f"positions, 16 / 2 heads, d = 256: {t_at * 1e3:.1f} ms"}
+    return out
+
+
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
 
 
@@ -649,6 +723,8 @@ def main():
                 _MOE_LAYERS.clear()
         out["workloads"] = wl
     out["cpu_baseline"] = None if a.no_cpu_baseline else cpu_baseline()
+    if not a.no_cpu_baseline and a.workload == "all":
+        out["cpu_baseline"]["by_config"] = cpu_baselines_by_config()
     print(json.dumps(out))
 
 
@@ -749,6 +825,57 @@ def bench_decode_gemv(a):
                     "frac_hbm_peak": round(kbytes[nm] / kern_us[nm] / 1e3 / HBM_PEAK_GBS, 4)} for nm in kern_us}
     q4_bytes = 2 * nbytes["gate"] + nbytes["down"]
     q4_us = 2 * kern_us["gate_up_12288x4096"] + kern_us["down_4096x12288"]
+    q4_us_fewer = kern_us["gate_and_up_one_launch"] + kern_us["down_4096x12288"]
+
+    # The dense FFN of the decode step as a chain (x bf16 -> gate, up -> SwiGLU in f32 -> down over the f32 activations,
+    # the reference's dataflow, gpu_ffn.rs:1231-1306): three dispatches + hq_silu_mul, two launches (gate + up + SwiGLU as
+    # one streaming launch, then down), and the whole block as one launch with an in-launch hand-over.
+    gate_b, up_b, act_b = (torch.empty(1, F, device=dev) for _ in range(3))
+    ffn_w = [ops.DenseFfnWeightsGpuQ(ws["gate"], ws["up"], ws["down"], HQ_Q4_K, H, F) for ws in sets]
+    ffn_out = torch.empty(1, H, device=dev)
+    ffn_scratch = torch.zeros(ops.dense_ffn_decode_scratch_bytes(ffn_w[0], torch.bfloat16), dtype=torch.uint8, device=dev)
+    p_gu = GgmlQuantizedMatmulParams(1, F, H, HQ_Q4_K)
+
+    def ffn_separate(w):
+        ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x_h, w.gate_q, gate_b, 1, F, H), ops.QmatmulJob(x_h, w.up_q, up_b, 1, F, H)], HQ_Q4_K)
+        ops.dispatch_silu_mul(gate_b, up_b, act_b)
+        ops.quantized_matmul_ggml(act_b, w.down_q, ffn_out, params["down"])
+
+    def ffn_two(w):
+        ops.quantized_matmul_swiglu_decode(x_h, w.gate_q, w.up_q, act_b, p_gu)
+        ops.quantized_matmul_ggml(act_b, w.down_q, ffn_out, params["down"])
+
+    def ffn_one(w):
+        ops.dense_ffn_decode(x_h, w, ffn_out, ffn_scratch)
+
+    ffn_bytes = q4_bytes
+    ffn_us = {nm: _launch_us([(lambda w=w, f=f: f(w)) for w in ffn_w] * 5) for nm, f in
+              (("separate_dispatches_4_launches", ffn_separate), ("two_launches", ffn_two), ("one_launch", ffn_one))}
+    dense_ffn = {nm: {"us": round(us, 3), "GBps": round(ffn_bytes / us / 1e3, 1), "frac_hbm_peak": round(ffn_bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+                 for nm, us in ffn_us.items()}
+    dense_ffn["bytes"] = ffn_bytes
+    dense_ffn["what"] = ("the FFN of the decode step as a chain, Q4_K 4096 -> 12288 -> 4096, bf16 input, f32 SwiGLU activations into the down "
+                         "projection (gpu_ffn.rs:1231-1306); us per FFN, every form the same bits")
+    del ffn_w, gate_b, up_b
+
+    # The reference's own published decode shapes (docs/ADR-028...:5247, 5248, 4884, 8564), both activation
+    # dtypes (its call sites pass f32, gpu_full_attn.rs:835): lm_head 262144 x 2816 in Q6_K and Q8_0, the 4096 x 2816 and
+    # 2816 x 4096 projections in Q5_K.
+    ref_shapes = {}
+    for nm, (n, k, t) in (("q6_k_lm_head_262144x2816", (262144, 2816, HQ_Q6_K)), ("q8_0_lm_head_262144x2816", (262144, 2816, ops.HQ_Q8_0)),
+                          ("q5_k_4096x2816", (4096, 2816, ops.HQ_Q5_K)), ("q5_k_2816x4096", (2816, 4096, ops.HQ_Q5_K))):
+        copies = 2 if n > 100000 else 8
+        wsr = [make_weight(n, k, t) for _ in range(copies)]
+        yr = torch.empty(1, n, device=dev)
+        pr = GgmlQuantizedMatmulParams(1, n, k, t)
+        entry = {"bytes": wsr[0].numel()}
+        for dt, dn in ((torch.bfloat16, "bf16"), (torch.float32, "f32")):
+            xr = torch.randn(1, k, generator=gx, device=dev, dtype=torch.float32).to(dt)
+            us = _launch_us([(lambda w=w: ops.quantized_matmul_ggml(xr, w, yr, pr)) for w in wsr] * (4 if copies == 2 else 4))
+            entry[dn] = {"us": round(us, 3), "GBps": round(wsr[0].numel() / us / 1e3, 1),
+                         "frac_hbm_peak": round(wsr[0].numel() / us / 1e3 / HBM_PEAK_GBS, 4)}
+        ref_shapes[nm] = entry
+        del wsr
 
     value = step_bytes * a.steps / elapsed / 1e9
     head_us = kern_us["head_151936x4096"]
@@ -780,7 +907,12 @@ def bench_decode_gemv(a):
                      "us_per_launch": round(head_us, 3), "bytes_per_launch": nbytes["head"]},
         "kernels": kernels,
         "host_launched": host,
-        "q4_k_gemv": {"GBps": round(q4_bytes / q4_us / 1e3, 1), "frac_hbm_peak": round(q4_bytes / q4_us / 1e3 / HBM_PEAK_GBS, 4)},
+        "q4_k_gemv": {"GBps": round(q4_bytes / q4_us / 1e3, 1), "frac_hbm_peak": round(q4_bytes / q4_us / 1e3 / HBM_PEAK_GBS, 4),
+                      "what": "gate, up, down as three launches of their own (bf16 activations each)",
+                      "gate_and_up_as_one_launch": {"GBps": round(q4_bytes / q4_us_fewer / 1e3, 1),
+                                                    "frac_hbm_peak": round(q4_bytes / q4_us_fewer / 1e3 / HBM_PEAK_GBS, 4)}},
+        "dense_ffn_decode_chain": dense_ffn,
+        "reference_shapes": ref_shapes,
     }
 
 

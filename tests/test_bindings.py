@@ -89,3 +89,48 @@ def test_crate_files_are_present():
     for f in ("Cargo.toml", "build.rs", os.path.join("src", "lib.rs")):
         assert os.path.isfile(os.path.join(CRATE, f)), f
     assert 'links = "hf2q_hip"' in open(os.path.join(CRATE, "Cargo.toml")).read()
+
+
+def test_build_rs_compiles_the_library_the_way_build_py_does():
+    """build.rs runs hipcc over hf2q_amd/csrc/*.hip: its source list is the directory's, its flags are build.py's."""
+    from hf2q_amd import build as hq_build
+
+    text = open(os.path.join(CRATE, "build.rs")).read()
+    sources = re.search(r"const SOURCES: &\[&str\] = &\[(.*?)\];", text, flags=re.S).group(1)
+    assert re.findall(r'"([^"]+)"', sources) == hq_build.sources()
+    flags = re.search(r"const FLAGS: &\[&str\] = &\[(.*?)\];", text, flags=re.S).group(1)
+    assert re.findall(r'"([^"]+)"', flags) == hq_build.FLAGS
+    strict = re.search(r"const STRICT_FP: &\[\(&str, &str\)\] = &\[(.*?)\];", text, flags=re.S).group(1)
+    assert {f: [fl] for f, fl in re.findall(r'\("([^"]+)", "([^"]+)"\)', strict)} == hq_build.STRICT_FP
+    assert "Command::new(&hipcc)" in text and '"-shared"' in text and "cargo:rustc-link-lib=dylib=hf2q_hip" in text
+
+
+def test_extern_block_types_match_the_header():
+    """Parameter and field TYPES too, not only names: every C type maps to one Rust type."""
+    cmap = {"void*": "*mut c_void", "const void*": "*const c_void", "const float*": "*const f32", "float*": "*mut f32",
+            "const uint32_t*": "*const u32", "uint32_t*": "*mut u32", "const uint8_t*": "*const u8", "uint8_t*": "*mut u8",
+            "uint32_t": "u32", "uint64_t": "u64", "size_t": "usize", "int": "c_int", "float": "f32", "double": "f64",
+            "hq_ggml_type": "hq_ggml_type", "hq_act_dtype": "hq_act_dtype", "const char*": "*const c_char",
+            "size_t*": "*mut usize", "uint64_t*": "*mut u64", "double*": "*mut f64", "const char**": "*mut *const c_char",
+            "const hq_tq_attn_params*": "*const hq_tq_attn_params", "const hq_tqp_header*": "*const hq_tqp_header",
+            "hq_tqp_header*": "*mut hq_tqp_header", "const hq_qmatmul_job*": "*const hq_qmatmul_job",
+            "const hq_moe_ffn_layer*": "*const hq_moe_ffn_layer", "const hq_moe_ffn_row_scales*": "*const hq_moe_ffn_row_scales",
+            "hq_gguf**": "*mut *mut hq_gguf", "hq_gguf*": "*mut hq_gguf", "const hq_gguf*": "*const hq_gguf",
+            "hq_gguf_tensor_info*": "*mut hq_gguf_tensor_info"}
+    text = _strip_comments(open(HEADER).read())
+    rust = _strip_comments(open(os.path.join(CRATE, "src", "lib.rs")).read())
+    block = re.search(r'extern\s+"C"\s*\{(.*?)\n\}', rust, flags=re.S).group(1)
+    rfn = {m.group(1): ([p.split(":", 1)[1].strip() for p in m.group(2).split(",") if p.strip()], (m.group(3) or "").strip())
+           for m in re.finditer(r"pub\s+fn\s+(hq_\w+)\s*\(([^)]*)\)\s*(?:->\s*([^;]+))?;", block, flags=re.S)}
+    checked = 0
+    for m in re.finditer(r"HQ_API\s+([^;(]+?)\b(hq_\w+)\s*\(([^)]*)\)\s*;", text, flags=re.S):
+        ret, name, params = " ".join(m.group(1).split()), m.group(2), [p.strip() for p in m.group(3).split(",")]
+        ctypes_ = [] if params == ["void"] else [" ".join(re.sub(r"\b\w+\s*(\[\d*\])?$", "", p).split()).replace(" *", "*") for p in params]
+        want = [cmap[c] for c in ctypes_]
+        got, rret = rfn[name]
+        assert got == want, f"{name}: header {ctypes_} -> {want}, crate {got}"
+        want_ret = {"void": "", "int": "c_int", "size_t": "usize", "uint32_t": "u32", "uint64_t": "u64", "const char*": "*const c_char",
+                    "const void*": "*const c_void"}[ret.replace(" *", "*")]
+        assert rret == want_ret, f"{name}: returns {ret} vs {rret}"
+        checked += 1
+    assert checked >= 60
