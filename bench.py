@@ -60,6 +60,7 @@ def parse():
                     help="all (default) = the BASELINE config 2 headline plus configs 3, 4 and 5 under `workloads` in the "
                          "same JSON line; a single name runs that workload alone and prints its own line")
     ap.add_argument("--tokens", type=int, default=1, help="moe_decode: tokens per step (1 or 8)")
+    ap.add_argument("--mix", action="store_true", help="moe_decode: gate / up Q5_K and down Q6_K instead of Q4_K")
     ap.add_argument("--wtype", default="q4_k", choices=["q4_k", "q8_0", "q6_k", "q5_k", "q4_0"], help="prefill_gemm: weight type")
     ap.add_argument("--weight-sets", type=int, default=6, help="distinct FFN weight sets rotated per step")
     ap.add_argument("--moe-layers", type=int, default=20, help="moe_decode: distinct MoE layers rotated per step")
@@ -288,9 +289,10 @@ def _finish(a, out):
 _MOE_LAYERS = {}  # the layers of bench_moe_decode, shared by its T = 1 and T = 8 runs
 
 
-def bench_moe_decode(a, tokens=None):
+def bench_moe_decode(a, tokens=None, mix=False):
     """BASELINE config 3: Qwen3.6-35B-A3B-style MoE FFN layer, hidden 2048, 256 experts (inter 512, Q4_K), one
-    shared expert, top-8 from seeded router logits, batch 1 or 8, bf16 activations.  A step is one layer."""
+    shared expert, top-8 from seeded router logits, batch 1 or 8, bf16 activations.  A step is one layer.
+    mix: the types the reference's model file really holds, gate / up Q5_K and down Q6_K (docs/ADR-028...:4942-4946)."""
     import torch
 
     from hf2q_amd import ops
@@ -298,25 +300,27 @@ def bench_moe_decode(a, tokens=None):
 
     dev = torch.device("cuda:0")
     H, E, K, I, SI, T = 2048, 256, 8, 512, 512, tokens or a.tokens
+    tg, td = (ops.HQ_Q5_K, ops.HQ_Q6_K) if mix else (HQ_Q4_K, HQ_Q4_K)
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     rnd = lambda *s: torch.randn(*s, generator=gen, device=dev, dtype=torch.float32)  # noqa: E731
-    qz = lambda n, k: ops.quantize_ggml(rnd(n * k).mul_(0.02), k, HQ_Q4_K)  # noqa: E731
+    qz = lambda n, k, t: ops.quantize_ggml(rnd(n * k).mul_(0.02), k, t)  # noqa: E731
     n_layers = max(1, a.moe_layers)  # distinct layers rotated: a token touches 17 MB (T=1) of a layer, and the
     # 256 MB Infinity Cache must not hold the experts a layer routes to from its previous turn
-    if n_layers not in _MOE_LAYERS:
+    if (n_layers, mix) not in _MOE_LAYERS:
         _MOE_LAYERS.clear()
-        _MOE_LAYERS[n_layers] = [ops.MoeFfnWeightsGpuQ(
-            rnd(E, H).mul_(0.02).to(torch.bfloat16), qz(E * I, H), qz(E * I, H), qz(E * H, I),
-            rnd(1, H).mul_(0.02).to(torch.bfloat16), qz(SI, H), qz(SI, H), qz(H, SI), HQ_Q4_K, H, E, K, I, SI)
+        _MOE_LAYERS[(n_layers, mix)] = [ops.MoeFfnWeightsGpuQ(
+            rnd(E, H).mul_(0.02).to(torch.bfloat16), qz(E * I, H, tg), qz(E * I, H, tg), qz(E * H, I, td),
+            rnd(1, H).mul_(0.02).to(torch.bfloat16), qz(SI, H, tg), qz(SI, H, tg), qz(H, SI, td), tg, H, E, K, I, SI,
+            down_type=None if td == tg else td)
             for _ in range(n_layers)]
-    layers = _MOE_LAYERS[n_layers]
+    layers = _MOE_LAYERS[(n_layers, mix)]
     gx = torch.Generator(device=dev)
     gx.manual_seed(5678)
     x = torch.randn(T, H, generator=gx, device=dev, dtype=torch.float32).to(torch.bfloat16)
     scratch = ops.MoeFfnScratch(layers[0], T, dev)
     out = torch.empty(T, H, device=dev)
-    expert_bytes = I * ops.ggml_row_bytes(HQ_Q4_K, H)
+    gu_bytes, dn_bytes = I * ops.ggml_row_bytes(tg, H), H * ops.ggml_row_bytes(td, I)
 
     def step(i):
         ops.build_moe_ffn_layer_gpu_q_into(x, layers[i % n_layers], scratch, out)
@@ -331,12 +335,12 @@ def bench_moe_decode(a, tokens=None):
         eager_step(i)
         uniq.append(int(torch.unique(scratch.ids[:T * K]).numel()))
     u = sum(uniq) / len(uniq)
-    step_bytes = (u * 3 + 3) * expert_bytes + (E + 1) * H * 2  # routed + shared experts + router (bf16)
+    step_bytes = (u + 1) * (2 * gu_bytes + dn_bytes) + (E + 1) * H * 2  # routed + shared experts + router (bf16)
     gbs = step_bytes / layer_us / 1e3
     return _finish(a, {
         "metric": "MoE decode tok/s (FFN-only, 40 MoE layers)", "value": round(T / (40 * elapsed / a.steps), 1),
         "unit": "tok/s", "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "bf16",
-        "config": {"workload": f"moe_decode: hidden 2048, 256 experts x inter 512 Q4_K, shared expert, top-8, "
+        "config": {"workload": f"moe_decode: hidden 2048, 256 experts x inter 512 {'gate / up Q5_K, down Q6_K' if mix else 'Q4_K'}, shared expert, top-8, "
                                f"batch {T}, bf16 activations (BASELINE config 3); one step = one MoE FFN layer = ONE launch "
                                f"(hq_moe_ffn_decode: router + shared logit, top-k, gate / up with SwiGLU, down, weighted "
                                f"sum, handed between workgroups inside the launch), "
@@ -345,7 +349,7 @@ def bench_moe_decode(a, tokens=None):
                    "layers_rotated": n_layers},
         "roofline": {"bound": "hbm", "kernel": "MoE FFN layer (hq_moe_ffn_decode, one launch)", "achieved": round(gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": PMC_TRAFFIC_BYTES.get(f"moe_ffn_decode_t{T}"),
+                     "traffic": None if mix else PMC_TRAFFIC_BYTES.get(f"moe_ffn_decode_t{T}"),
                      "us_per_launch": round(layer_us, 3), "bytes_per_launch": int(step_bytes)}})
 
 
@@ -697,7 +701,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if a.workload not in ("all", "decode_gemv"):
-        return {"moe_decode": bench_moe_decode, "moe_prefill": bench_moe_prefill, "prefill_gemm": bench_prefill_gemm,
+        if a.workload == "moe_decode":
+            return bench_moe_decode(a, mix=a.mix)
+        return {"moe_prefill": bench_moe_prefill, "prefill_gemm": bench_prefill_gemm,
                 "tq_attention": bench_tq_attention}[a.workload](a)
     out = bench_decode_gemv(a)
     if a.workload == "all":
@@ -712,6 +718,8 @@ def main():
         a = copy.copy(a)
         a.steps = max(a.steps, 256)
         for name, fn in (("moe_decode_t1", lambda: bench_moe_decode(a, 1)), ("moe_decode_t8", lambda: bench_moe_decode(a, 8)),
+                         ("moe_decode_t1_q5k_q6k", lambda: bench_moe_decode(a, 1, mix=True)),
+                         ("moe_decode_t8_q5k_q6k", lambda: bench_moe_decode(a, 8, mix=True)),
                          ("moe_prefill_2048x8", lambda: bench_moe_prefill(a)),
                          ("prefill_gemm_q4_k", lambda: bench_prefill_gemm(a, "q4_k")),
                          ("prefill_gemm_q8_0", lambda: bench_prefill_gemm(a, "q8_0")),
@@ -719,7 +727,7 @@ def main():
             gc.collect()
             torch.cuda.empty_cache()
             wl[name] = brief(fn())
-            if name == "moe_decode_t8":
+            if name == "moe_decode_t8_q5k_q6k":
                 _MOE_LAYERS.clear()
         out["workloads"] = wl
     out["cpu_baseline"] = None if a.no_cpu_baseline else cpu_baseline()

@@ -181,6 +181,7 @@ extern "C" {
     pub fn hq_silu_mul(stream: *mut c_void, gate: *const f32, up: *const f32, out: *mut f32, n: u64) -> c_int;
     pub fn hq_moe_weighted_reduce(stream: *mut c_void, y: *const f32, w: *const f32, shared: *const f32, shared_logit: *const f32, residual: *const f32, out: *mut f32, n_tokens: u32, top_k: u32, hidden: u32) -> c_int;
     pub fn hq_moe_ffn_decode_scratch_bytes(n_tokens: u32, hidden: u32, n_experts: u32, top_k: u32, inter: u32, shared_inter: u32, t: hq_ggml_type, xdt: hq_act_dtype) -> usize;
+    pub fn hq_moe_ffn_decode_layer_scratch_bytes(layer: *const hq_moe_ffn_layer, n_tokens: u32, xdt: hq_act_dtype) -> usize;
     pub fn hq_moe_ffn_decode(stream: *mut c_void, layer: *const hq_moe_ffn_layer, x: *const c_void, xdt: hq_act_dtype, residual: *const f32, out: *mut f32, n_tokens: u32, scratch: *mut c_void, scratch_bytes: usize, route_ids: *mut u32, route_weights: *mut f32) -> c_int;
     pub fn hq_handover_status(stream: *mut c_void, scratch: *const c_void, error: *mut u32) -> c_int;
     pub fn hq_set_handover_spin_limit(limit: u32);

@@ -591,8 +591,15 @@ int hq_qmatmul_batch_ggml(void* stream, const hq_qmatmul_job* jobs, uint32_t n_j
 
 size_t hq_moe_ffn_decode_scratch_bytes(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k, uint32_t inter,
                                        uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt) {
-    if (!moe_fused_supported(n_tokens, hidden, n_experts, top_k, inter, shared_inter, t, xdt)) return 0;
+    if (!moe_fused_supported(n_tokens, hidden, n_experts, top_k, inter, shared_inter, t, t, xdt)) return 0;
     return moe_fused_scratch_bytes(n_tokens, n_experts, top_k);
+}
+
+size_t hq_moe_ffn_decode_layer_scratch_bytes(const hq_moe_ffn_layer* l, uint32_t n_tokens, hq_act_dtype xdt) {
+    if (!l) return 0;
+    const hq_ggml_type td = l->down_type ? (hq_ggml_type)l->down_type : l->ggml_type;
+    if (!moe_fused_supported(n_tokens, l->hidden, l->n_experts, l->top_k, l->inter, l->shared_inter, l->ggml_type, td, xdt)) return 0;
+    return moe_fused_scratch_bytes(n_tokens, l->n_experts, l->top_k);
 }
 
 int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* l, const void* x, hq_act_dtype xdt, const float* residual,
@@ -601,13 +608,13 @@ int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* l, const void* x, hq
     const char* fn = "hq_moe_ffn_decode";
     if (!l) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null layer", fn);
     if (n_tokens == 0) return HQ_OK;
-    if ((l->down_type && l->down_type != (uint32_t)l->ggml_type) ||
-        !moe_fused_supported(n_tokens, l->hidden, l->n_experts, l->top_k, l->inter, l->shared_inter, l->ggml_type, xdt))
+    const hq_ggml_type t_down = l->down_type ? (hq_ggml_type)l->down_type : l->ggml_type;
+    if (!moe_fused_supported(n_tokens, l->hidden, l->n_experts, l->top_k, l->inter, l->shared_inter, l->ggml_type, t_down, xdt))
         return fail(HQ_ERR_UNSUPPORTED,
-                    "%s: takes 1..8 tokens of bf16 activations, Q4_K experts, hidden 2048, expert and shared FFN width 512, "
-                    "<= 256 experts (got %u tokens, dtype %d, type %d, hidden %u, inter %u / %u, %u experts, top-%u); "
-                    "run the block as separate dispatches",
-                    fn, n_tokens, (int)xdt, (int)l->ggml_type, l->hidden, l->inter, l->shared_inter, l->n_experts, l->top_k);
+                    "%s: takes 1..8 tokens of bf16 activations, K-quant experts (one type, or Q4_K / Q5_K gate / up with a Q6_K down), "
+                    "hidden 2048, expert and shared FFN width 512, <= 256 experts (got %u tokens, dtype %d, types %d / %d, hidden %u, "
+                    "inter %u / %u, %u experts, top-%u); run the block as separate dispatches",
+                    fn, n_tokens, (int)xdt, (int)l->ggml_type, (int)t_down, l->hidden, l->inter, l->shared_inter, l->n_experts, l->top_k);
     if (!x || !out || !scratch || !l->router || !l->expert_gate || !l->expert_up || !l->expert_down || !l->shared_gate ||
         !l->shared_up || !l->shared_down)
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
@@ -619,7 +626,8 @@ int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* l, const void* x, hq
     if (!is_aligned(scratch, 256)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch must be 256-byte aligned", fn);
     const size_t need = moe_fused_scratch_bytes(n_tokens, l->n_experts, l->top_k);
     if (scratch_bytes < need) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch of %zu bytes, %zu needed", fn, scratch_bytes, need);
-    const uint64_t gu_bytes = (uint64_t)l->inter * (l->hidden / 256) * Q4K_BYTES, d_bytes = (uint64_t)l->hidden * (l->inter / 256) * Q4K_BYTES;
+    const uint64_t gu_bytes = (uint64_t)l->inter * (l->hidden / 256) * hq_block_bytes(l->ggml_type),
+                   d_bytes = (uint64_t)l->hidden * (l->inter / 256) * hq_block_bytes(t_down);
     if (l->expert_stride_gate_up < gu_bytes || l->expert_stride_gate_up % 16 || l->expert_stride_down < d_bytes || l->expert_stride_down % 16)
         return fail(HQ_ERR_INVALID_ARGUMENT, "%s: expert strides %llu / %llu (one expert is %llu / %llu bytes)", fn,
                     (unsigned long long)l->expert_stride_gate_up, (unsigned long long)l->expert_stride_down,
@@ -645,6 +653,8 @@ int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* l, const void* x, hq
     a.stride_gate_up = l->expert_stride_gate_up;
     a.stride_down = l->expert_stride_down;
     a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+    a.t_gate_up = l->ggml_type;
+    a.t_down = t_down;
     return launch_moe_fused((hipStream_t)stream, a);
 }
 

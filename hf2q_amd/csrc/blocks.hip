@@ -28,7 +28,7 @@ struct Carver {
     void* bytes(size_t n) { return take<uint8_t>(n); }
 };
 
-uint64_t row_bytes(hq_ggml_type t, uint32_t k) { return (uint64_t)(k / hq_block_elems(t)) * hq_block_bytes(t); }
+
 
 // ---- dense SwiGLU FFN ----
 struct DenseBufs {

@@ -132,6 +132,22 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q5_K>& p, int c, const 
     return acc;
 }
 
+// Q6_K: the four runs' sums r[i] (of (q + off) * x) and activation sums sx[i] combined with the runs' scales (bytes lr,
+// lr + 2, lr + 4, lr + 6 of this half's eight) and d.  Every operation is written out and nothing else is fused: the
+// kernels that share this get the same bits whatever surrounds the call.
+__device__ __forceinline__ float q6k_combine(const Piece<HQ_Q6_K>& p, int c, float off, float r0, float r1, float r2, float r3,
+                                             const float* sx) {
+#pragma clang fp contract(off)
+    const int lr = c & 1;
+    const uint32_t s01 = p.sc.x >> (8 * lr), s23 = p.sc.y >> (8 * lr);
+    const float d = f16_bits_to_f32(p.d >> 16);
+    float acc = (float)(int)(int8_t)(s01 & 0xff) * fmaf(-off, sx[0], r0);
+    acc = fmaf((float)(int)(int8_t)((s01 >> 16) & 0xff), fmaf(-off, sx[1], r1), acc);
+    acc = fmaf((float)(int)(int8_t)(s23 & 0xff), fmaf(-off, sx[2], r2), acc);
+    acc = fmaf((float)(int)(int8_t)((s23 >> 16) & 0xff), fmaf(-off, sx[3], r3), acc);
+    return d * acc;
+}
+
 // Q6_K: four 6-bit values at a time as the bytes of one word (nibbles of ql, two-bit fields of qh; n4 = 0x0f0f0f0f and
 // n2 = 0x30303030 arrive in the mask registers), then two byte permutes put bytes (0, 2) and (1, 3) under the high
 // byte 0x43 of `magic`: bf16 128 + q, the pair order of the staged activations.
@@ -155,16 +171,8 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q6_K>& p, int c, const 
         r3 = dot2_bf16(__builtin_amdgcn_perm(magic, q3, SEL02), xp[24 + 2 * j], r3);
         r3 = dot2_bf16(__builtin_amdgcn_perm(magic, q3, SEL13), xp[24 + 2 * j + 1], r3);
     }
-    // scale bytes lr, lr+2, lr+4, lr+6 of this half's eight; values hold 128 + q with q in 0..63
-    // and the format's own -32, hence the 160.
-    const int lr = c & 1;
-    const uint32_t s01 = p.sc.x >> (8 * lr), s23 = p.sc.y >> (8 * lr);
-    const float d = f16_bits_to_f32(p.d >> 16);
-    float acc = (float)(int)(int8_t)(s01 & 0xff) * (r0 - 160.f * sx[0]);
-    acc += (float)(int)(int8_t)((s01 >> 16) & 0xff) * (r1 - 160.f * sx[1]);
-    acc += (float)(int)(int8_t)(s23 & 0xff) * (r2 - 160.f * sx[2]);
-    acc += (float)(int)(int8_t)((s23 >> 16) & 0xff) * (r3 - 160.f * sx[3]);
-    return d * acc;
+    // values hold 128 + q with q in 0..63 and the format's own -32, hence the 160
+    return q6k_combine(p, c, 160.f, r0, r1, r2, r3, sx);
 }
 
 // Q4_0: y = d * (q - 8); low nibbles are elements 0..15 of the block, high nibbles 16..31; values hold 128 + q.
@@ -225,14 +233,7 @@ __device__ __forceinline__ float dot_f32(const Piece<HQ_Q6_K>& p, int c, const f
         r2 = dot4(((a >> 4) & N4) | (v & N2), xf + 32 + 4 * j, r2);
         r3 = dot4(((b >> 4) & N4) | ((v >> 2) & N2), xf + 48 + 4 * j, r3);
     }
-    const int lr = c & 1;
-    const uint32_t s01 = p.sc.x >> (8 * lr), s23 = p.sc.y >> (8 * lr);
-    const float d = f16_bits_to_f32(p.d >> 16);
-    float acc = (float)(int)(int8_t)(s01 & 0xff) * (r0 - 32.f * sx[0]);
-    acc += (float)(int)(int8_t)((s01 >> 16) & 0xff) * (r1 - 32.f * sx[1]);
-    acc += (float)(int)(int8_t)(s23 & 0xff) * (r2 - 32.f * sx[2]);
-    acc += (float)(int)(int8_t)((s23 >> 16) & 0xff) * (r3 - 32.f * sx[3]);
-    return d * acc;
+    return q6k_combine(p, c, 32.f, r0, r1, r2, r3, sx);
 }
 
 __device__ __forceinline__ float dot_f32(const Piece<HQ_Q5_K>& p, int c, const float* xf, const float* sx) {
@@ -311,14 +312,7 @@ __device__ __forceinline__ void dot_f32_half(const Piece<HQ_Q6_K>& p, int, int h
     out[1] = rb;
 }
 __device__ __forceinline__ float dot_f32_finish(const Piece<HQ_Q6_K>& p, int c, const float* lo, const float* hi, const float* sx) {
-    const int lr = c & 1;
-    const uint32_t s01 = p.sc.x >> (8 * lr), s23 = p.sc.y >> (8 * lr);
-    const float d = f16_bits_to_f32(p.d >> 16);
-    float acc = (float)(int)(int8_t)(s01 & 0xff) * (lo[0] - 32.f * sx[0]);
-    acc += (float)(int)(int8_t)((s01 >> 16) & 0xff) * (lo[1] - 32.f * sx[1]);
-    acc += (float)(int)(int8_t)(s23 & 0xff) * (hi[0] - 32.f * sx[2]);
-    acc += (float)(int)(int8_t)((s23 >> 16) & 0xff) * (hi[1] - 32.f * sx[3]);
-    return d * acc;
+    return q6k_combine(p, c, 32.f, lo[0], lo[1], hi[0], hi[1], sx);
 }
 
 // Q4_0: y = d * (q - 8); low nibbles are elements 0..15 of the block, high nibbles 16..31.

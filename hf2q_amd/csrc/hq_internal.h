@@ -139,9 +139,10 @@ struct MoeFusedArgs {
     uint32_t n_tokens, n_experts, top_k;
     uint64_t stride_gate_up, stride_down;
     uint32_t spin_limit;            // 0: default
+    hq_ggml_type t_gate_up, t_down;
 };
 bool moe_fused_supported(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k, uint32_t inter,
-                         uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt);
+                         uint32_t shared_inter, hq_ggml_type t, hq_ggml_type t_down, hq_act_dtype xdt);
 size_t moe_fused_scratch_bytes(uint32_t n_tokens, uint32_t n_experts, uint32_t top_k);
 int launch_moe_fused(hipStream_t s, const MoeFusedArgs& a);
 

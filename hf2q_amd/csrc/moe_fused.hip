@@ -25,8 +25,10 @@
 // same SwiGLU rounding, the same order of the weighted sum — so the block's output has the bits of
 // hq_dense_gemv_bf16_pair + hq_qmatmul_batch_ggml x 2 + hq_moe_weighted_reduce.
 //
-// Shapes: K-quant Q4_K experts, hidden = 2048 (32 lanes per gate / up row: a wave step is one gate row and the up row
-// of the same index), expert FFN = shared FFN = 512 (8 lanes per down row), <= 256 experts, bf16 activations.
+// Shapes: K-quant experts (Q4_K, Q5_K or Q6_K; gate / up of one type, down of the same or -- the mix GGUF files of the
+// reference's model hold, docs/ADR-028...:4942-4946 -- Q4_K / Q5_K gate / up with a Q6_K down), hidden = 2048 (32 lanes
+// per gate / up row: a wave step is one gate row and the up row of the same index), expert FFN = shared FFN = 512 (8
+// lanes per down row), <= 256 experts, bf16 activations.
 #include <math.h>
 
 #include "hq_internal.h"
@@ -38,8 +40,10 @@ namespace hq {
 namespace {
 
 constexpr uint32_t FH = 2048, FI = 512;               // hidden, expert FFN width
-constexpr uint32_t ROWB_H = FH / 256 * Q4K_BYTES;     // bytes of a gate / up row
-constexpr uint32_t ROWB_I = FI / 256 * Q4K_BYTES;     // bytes of a down row
+template <int TYPE>
+constexpr uint32_t kRowBytesH = FH / 256 * kBlockBytes<TYPE>;  // bytes of a gate / up row
+template <int TYPE>
+constexpr uint32_t kRowBytesI = FI / 256 * kBlockBytes<TYPE>;  // bytes of a down row
 constexpr uint32_t WAVES = 8, THREADS = 64 * WAVES;
 constexpr uint32_t MAX_T = 8;                         // tokens per call
 constexpr int RING = 4;                               // weight fetches a wave keeps in flight
@@ -96,9 +100,23 @@ __device__ __forceinline__ uint32_t wait_tagged(const uint64_t* p, uint32_t tag,
     return (uint32_t)got;
 }
 
-__device__ __forceinline__ uint32_t swz8(uint32_t ch) { return ch ^ ((ch >> 4) & 7u); }
+// LDS slot of 16-byte chunk ch of the staged activations.  Lanes that read together differ in the piece index (ch / 8)
+// or, Q6_K, whose lane reads four runs of sixteen at a stride of 32 inside one half of a super-block, in bits 1, 4, 5, 6.
+template <int TYPE>
+__device__ __forceinline__ uint32_t swz8(uint32_t ch) {
+    if constexpr (TYPE == HQ_Q6_K) return ch ^ (((ch >> 4) & 1u) | (((ch >> 5) & 3u) << 2));
+    return ch ^ ((ch >> 4) & 7u);
+}
+// First float4 of run r (sixteen activations) of a lane's 64 activations of a row of FI: lane li = (super-block, quarter).
+template <int TYPE>
+__device__ __forceinline__ uint32_t act_run(uint32_t li, uint32_t r) {
+    if constexpr (TYPE == HQ_Q6_K) return (li >> 2) * 64u + ((li >> 1) & 1u) * 32u + (li & 1u) * 4u + 8u * r;
+    return li * 16u + 4u * r;
+}
 
+template <int TG, int TD>  // types of gate / up and of down
 __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
+    constexpr uint32_t ROWB_H = kRowBytesH<TG>, ROWB_I = kRowBytesI<TD>;
     extern __shared__ uint4 smem[];
     const Layout L{a.T, a.E, a.K};
     const uint32_t T = a.T, E = a.E, K = a.K, S = K + 1;
@@ -180,8 +198,8 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
         o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
         o1.z = (w[6] & 0xffffu) | (w[7] << 16);
         o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
-        lds_x[swz8(2 * j)] = o0;
-        lds_x[swz8(2 * j + 1)] = o1;
+        lds_x[swz8<TG>(2 * j)] = o0;
+        lds_x[swz8<TG>(2 * j + 1)] = o1;
         float sum = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -200,6 +218,7 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
         float wt;
         softmax_topk_lane<4>(lds_lg, E, K, lane, id, wt);
         if (lane < K) {
+            id = id < E ? id : E - 1u;  // (the selection only yields indices below E; a bound the fetch addresses can rely on)
             lds_id[lane] = id;
             lds_w[lane] = wt;
             if (jb == 0 && a.route_ids) {
@@ -236,30 +255,32 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
         const uint32_t li = lane & 31u, hf = lane >> 5;
         const int c4 = (int)(li & 3u);
         const uint32_t mine = rows2;
-        const uint32_t lane_off = (li >> 2) * Q4K_BYTES;
-        auto fetch = [&](Piece<HQ_Q4_K>& pc, uint32_t p) {
+        const uint32_t lane_off = (li >> 2) * kBlockBytes<TG>;
+        auto fetch = [&](Piece<TG>& pc, uint32_t p) {
             const uint32_t r = p % FI, s = p / FI;
             const uint8_t* base = s < K ? (hf ? a.eu : a.eg) + (size_t)lds_id[s] * a.stride_gu : (hf ? a.su : a.sg);
             pc.load(base + (size_t)r * ROWB_H + lane_off, c4);
         };
-        Piece<HQ_Q4_K> ring[RING];
+        Piece<TG> ring[RING];
 #pragma unroll
         for (int i = 0; i < RING; ++i)
             if ((uint32_t)i < mine) fetch(ring[i], tw + (uint32_t)i * NTW);
         uint32_t xp[32];
         float sx[4];
         {
-            const uint32_t ch0 = li * 8u;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint4 v = lds_x[swz8(ch0 + j)];
-                xp[4 * j] = v.x;
-                xp[4 * j + 1] = v.y;
-                xp[4 * j + 2] = v.z;
-                xp[4 * j + 3] = v.w;
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t ch = act_run<TG>(li, (uint32_t)r) / 2u;  // two chunks of eight per run
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint4 v = lds_x[swz8<TG>(ch + u)];
+                    xp[8 * r + 4 * u] = v.x;
+                    xp[8 * r + 4 * u + 1] = v.y;
+                    xp[8 * r + 4 * u + 2] = v.z;
+                    xp[8 * r + 4 * u + 3] = v.w;
+                }
+                sx[r] = lds_sx[ch / 2];
             }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sx[r] = lds_sx[ch0 / 2 + r];
         }
         float keep_g = 0.f, keep_u = 0.f;
         for (uint32_t i0 = 0; i0 < mine; i0 += RING) {
@@ -317,6 +338,7 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
     // ---- phases 3 + 4: unit (token t, column slice c): the down rows of the slice for every slot of the token, then
     // the weighted sum over the slots in slot order, the shared expert last (the order of moe_weighted_reduce_kernel) ----
     {
+        constexpr int RD = TD == HQ_Q5_K ? 3 : RING;  // (a ring of four Q5_K pieces beside the 64 activations spills)
         const uint32_t li = lane & 7u, sub = lane >> 3;
         const int c4 = (int)(li & 3u);
         const uint32_t groups = T <= 1 ? 1u : T <= 2 ? 2u : T <= 4 ? 4u : 8u, cols = 8u * groups;  // columns per unit: about one unit per workgroup
@@ -331,15 +353,15 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
             const bool runs = groups > 1;
             const uint32_t st0 = runs ? wv * n_steps / WAVES : wv, stp = runs ? 1u : WAVES;
             const uint32_t mine = runs ? (wv + 1u) * n_steps / WAVES - st0 : wv < n_steps ? (n_steps - wv + WAVES - 1u) / WAVES : 0u;
-            auto fetch = [&](Piece<HQ_Q4_K>& pc, uint32_t n) {
+            auto fetch = [&](Piece<TD>& pc, uint32_t n) {
                 const uint32_t st = st0 + n * stp, s = st / groups, g = st % groups;
                 const uint8_t* base = s < K ? a.ed + (size_t)lds_id[s] * a.stride_d : a.sd;
-                pc.load(base + (size_t)(cols * c + 8 * g + sub) * ROWB_I + (li >> 2) * Q4K_BYTES, c4);
+                pc.load(base + (size_t)(cols * c + 8 * g + sub) * ROWB_I + (li >> 2) * kBlockBytes<TD>, c4);
             };
-            Piece<HQ_Q4_K> ring[RING];
+            Piece<TD> ring[RD];
             auto prefetch = [&]() {
 #pragma unroll
-                for (int i = 0; i < RING; ++i)
+                for (int i = 0; i < RD; ++i)
                     if ((uint32_t)i < mine) fetch(ring[i], (uint32_t)i);
             };
             if (c == jb && storing) {  // (a storing wave's fetches would stand in the queue in front of the acknowledgement's wait)
@@ -409,30 +431,34 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
             __syncthreads();
             float xf[64], sx[4];
             uint32_t cur_s = ~0u;
-            for (uint32_t i0 = 0; i0 < mine; i0 += RING) {
+            for (uint32_t i0 = 0; i0 < mine; i0 += RD) {
 #pragma unroll
-                for (int i = 0; i < RING; ++i) {
+                for (int i = 0; i < RD; ++i) {
                     const uint32_t n = i0 + (uint32_t)i;
                     if (n < mine) {
                         const uint32_t st = st0 + n * stp, s = st / groups, g = st % groups;
                         if (s != cur_s) {  // uniform
                             cur_s = s;
 #pragma unroll
-                            for (int q = 0; q < 16; ++q) {
-                                const float4 v = lds_act[s * (FI / 4) + ((li * 16 + q) ^ li)];
-                                xf[4 * q] = v.x;
-                                xf[4 * q + 1] = v.y;
-                                xf[4 * q + 2] = v.z;
-                                xf[4 * q + 3] = v.w;
-                            }
+                            for (int r = 0; r < 4; ++r) {
+                                const uint32_t f0 = act_run<TD>(li, (uint32_t)r);
 #pragma unroll
-                            for (int r = 0; r < 4; ++r) sx[r] = lds_as[s * (FI / 16) + li * 4 + r];
+                                for (int j = 0; j < 4; ++j) {
+                                    const uint32_t f = f0 + (uint32_t)j;
+                                    const float4 v = lds_act[s * (FI / 4) + (f ^ (f >> 4))];
+                                    xf[16 * r + 4 * j] = v.x;
+                                    xf[16 * r + 4 * j + 1] = v.y;
+                                    xf[16 * r + 4 * j + 2] = v.z;
+                                    xf[16 * r + 4 * j + 3] = v.w;
+                                }
+                                sx[r] = lds_as[s * (FI / 16) + f0 / 4];
+                            }
                         }
                         const float v = group_sum(dot_f32(ring[i], c4, xf, sx), 3);
-                        if (n + RING < mine) {
+                        if (n + RD < mine) {
                             float tie = v;
                             asm volatile("" : "+v"(tie));
-                            fetch(ring[i], n + RING);
+                            fetch(ring[i], n + RD);
                         }
                         if (li == 0) lds_part[s * cols + 8 * g + sub] = v;
                     }
@@ -461,10 +487,23 @@ size_t moe_fused_scratch_bytes(uint32_t n_tokens, uint32_t n_experts, uint32_t t
     return (Layout{n_tokens, n_experts, top_k}.total() + 255) & ~(size_t)255;
 }
 
+namespace {
+// The kernel instantiated for (gate / up type, down type), or null: one K-quant for all three, or Q4_K / Q5_K gate / up
+// with a Q6_K down.
+void (*fused_kernel_for(hq_ggml_type t, hq_ggml_type td))(FusedArgs) {
+    if (t == HQ_Q4_K && td == HQ_Q4_K) return moe_fused_kernel<HQ_Q4_K, HQ_Q4_K>;
+    if (t == HQ_Q5_K && td == HQ_Q5_K) return moe_fused_kernel<HQ_Q5_K, HQ_Q5_K>;
+    if (t == HQ_Q6_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q6_K, HQ_Q6_K>;
+    if (t == HQ_Q4_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q4_K, HQ_Q6_K>;
+    if (t == HQ_Q5_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q5_K, HQ_Q6_K>;
+    return nullptr;
+}
+}  // namespace
+
 bool moe_fused_supported(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k, uint32_t inter,
-                         uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt) {
-    return t == HQ_Q4_K && xdt == HQ_BF16 && hidden == FH && inter == FI && shared_inter == FI && n_tokens >= 1 &&
-           n_tokens <= 8 && n_experts >= n_tokens && n_experts <= 256 && top_k >= 1 && top_k <= 64 && top_k <= n_experts;
+                         uint32_t shared_inter, hq_ggml_type t, hq_ggml_type t_down, hq_act_dtype xdt) {
+    return fused_kernel_for(t, t_down) != nullptr && xdt == HQ_BF16 && hidden == FH && inter == FI && shared_inter == FI && n_tokens >= 1 &&
+           n_tokens <= MAX_T && n_experts >= n_tokens && n_experts <= 256 && top_k >= 1 && top_k <= 64 && top_k <= n_experts;
 }
 
 int launch_moe_fused(hipStream_t s, const MoeFusedArgs& m) {
@@ -488,10 +527,12 @@ int launch_moe_fused(hipStream_t s, const MoeFusedArgs& m) {
     a.K = m.top_k;
     a.stride_gu = m.stride_gate_up;
     a.stride_d = m.stride_down;
-    a.m4 = M4;
-    a.m2 = M2;
+    a.m4 = m.t_gate_up == HQ_Q6_K ? N4 : M4;
+    a.m2 = m.t_gate_up == HQ_Q5_K ? M1 : m.t_gate_up == HQ_Q6_K ? N2 : M2;
     a.magic = MAGIC;
     a.spin_limit = m.spin_limit ? m.spin_limit : (1u << 20);
+    auto kern = fused_kernel_for(m.t_gate_up, m.t_down);
+    if (!kern) return fail(HQ_ERR_UNSUPPORTED, "fused MoE block: gate / up type %d with down type %d", (int)m.t_gate_up, (int)m.t_down);
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
     // every workgroup must deliver at least one logit row (see the header comment), and one workgroup per CU
@@ -504,7 +545,7 @@ int launch_moe_fused(hipStream_t s, const MoeFusedArgs& m) {
     const size_t lds = (area > act_bytes ? area : act_bytes) + (size_t)(m.n_experts + 1) * 4 + (size_t)m.top_k * 4 + (size_t)S * 4 +
                        (size_t)S * 64 * 4 + (size_t)64 * WAVES * 4;
     if (lds > 64 * 1024) return fail(HQ_ERR_UNSUPPORTED, "fused MoE block: %zu bytes of LDS", lds);
-    hipLaunchKernelGGL(moe_fused_kernel, dim3(grid), dim3(THREADS), lds, s, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), lds, s, a);
     return check_launch("fused MoE block launch");
 }
 

@@ -79,6 +79,7 @@ SIGNATURES = {
     "hq_silu_mul": (_i32, [_vp, _vp, _vp, _vp, _u64]),
     "hq_moe_weighted_reduce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "hq_moe_ffn_decode_scratch_bytes": (_sz, [_u32, _u32, _u32, _u32, _u32, _u32, _i32, _i32]),
+    "hq_moe_ffn_decode_layer_scratch_bytes": (_sz, [_vp, _u32, _i32]),
     "hq_moe_ffn_decode": (_i32, [_vp, _vp, _vp, _i32, _vp, _vp, _u32, _vp, _sz, _vp, _vp]),
     "hq_handover_status": (_i32, [_vp, _vp, _c.POINTER(_u32)]),
     "hq_set_handover_spin_limit": (None, [_u32]),

@@ -818,8 +818,8 @@ class MoeFfnScratch:
         self.dense_ws = torch.empty(need, dtype=torch.uint8, device=device) if need else None
         self.max_tokens = T
         # scratch of the one-launch decode block (hq_moe_ffn_decode): zeroed once, then the library's
-        fb = 0 if w.td != w.ggml_type else _l.load().hq_moe_ffn_decode_scratch_bytes(
-            min(T, 8), w.hidden, w.n_experts, K, w.inter, w.shared_inter, w.ggml_type, _l.HQ_BF16)
+        _layer = w.c_layer()
+        fb = _l.load().hq_moe_ffn_decode_layer_scratch_bytes(ctypes.byref(_layer), min(T, 8), _l.HQ_BF16)
         self.fused = torch.zeros(fb, dtype=torch.uint8, device=device) if fb else None
 
 
@@ -856,10 +856,10 @@ _FUSED_CHUNKED_MAX_TOKENS = 48
 
 def moe_ffn_decode_fused_supported(x: torch.Tensor, w: MoeFfnWeightsGpuQ) -> bool:
     T = x.shape[0]
-    if T > _FUSED_CHUNKED_MAX_TOKENS or w.td != w.ggml_type:
+    if T > _FUSED_CHUNKED_MAX_TOKENS:
         return False
-    return bool(_l.load().hq_moe_ffn_decode_scratch_bytes(min(T, 8), w.hidden, w.n_experts, w.top_k, w.inter, w.shared_inter,
-                                                          w.ggml_type, _act_dtype(x)))
+    layer = w.c_layer()
+    return bool(_l.load().hq_moe_ffn_decode_layer_scratch_bytes(ctypes.byref(layer), min(T, 8), _act_dtype(x)))
 
 
 def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch, out: torch.Tensor,

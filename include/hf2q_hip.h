@@ -335,7 +335,8 @@ HQ_API int hq_moe_weighted_reduce(void* stream, const float* y, const float* w, 
  * build_moe_ffn_layer_gpu_q_into (src/inference/models/qwen35/gpu_ffn.rs:2313-2802: phases A-F of one command
  * buffer); moe_ffn_cpu_ref (ffn.rs:179-336) is the specification.  The result has the bits of the separate dispatches
  * (hq_dense_gemv_bf16_pair, hq_qmatmul_batch_ggml twice with the routing and the SwiGLU folded in,
- * hq_moe_weighted_reduce).  Takes 1..8 tokens of bf16 activations, Q4_K experts, hidden 2048, expert and shared FFN
+ * hq_moe_weighted_reduce).  Takes 1..8 tokens of bf16 activations, K-quant experts (Q4_K, Q5_K or Q6_K for all three
+ * matrices, or Q4_K / Q5_K gate / up with a Q6_K down: layer->down_type), hidden 2048, expert and shared FFN
  * width 512, n_tokens <= n_experts <= 256, top_k <= 64; anything else is HQ_ERR_UNSUPPORTED (hq_moe_ffn_decode_scratch_bytes
  * returns 0 for it) and runs as the separate dispatches.
  * `scratch`: hq_moe_ffn_decode_scratch_bytes() bytes of device memory, 256-byte aligned, ZEROED ONCE before its first
@@ -362,6 +363,8 @@ typedef struct hq_moe_ffn_layer {
 } hq_moe_ffn_layer;
 HQ_API size_t hq_moe_ffn_decode_scratch_bytes(uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t top_k,
                                        uint32_t inter, uint32_t shared_inter, hq_ggml_type t, hq_act_dtype xdt);
+/* The same query from the layer description (its down_type included). */
+HQ_API size_t hq_moe_ffn_decode_layer_scratch_bytes(const hq_moe_ffn_layer* layer, uint32_t n_tokens, hq_act_dtype xdt);
 HQ_API int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* layer, const void* x, hq_act_dtype xdt,
                       const float* residual, float* out, uint32_t n_tokens, void* scratch, size_t scratch_bytes,
                       uint32_t* route_ids, float* route_weights);

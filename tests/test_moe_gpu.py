@@ -328,7 +328,8 @@ def test_dense_ffn_prefill_with_workspace_equals_the_allocating_calls(oracle, de
 
 
 @pytest.mark.parametrize("T", [1, 2, 5, 8])
-def test_moe_block_one_launch_equals_batched_dispatches_and_cpu_spec(oracle, dev, T):
+@pytest.mark.parametrize("t,td", [(HQ_Q4_K, HQ_Q4_K), (HQ_Q5_K, HQ_Q6_K), (HQ_Q6_K, HQ_Q6_K), (HQ_Q5_K, HQ_Q5_K), (HQ_Q4_K, HQ_Q6_K)])
+def test_moe_block_one_launch_equals_batched_dispatches_and_cpu_spec(oracle, dev, T, t, td):
     """hq_moe_ffn_decode (the whole block in one launch, workgroups handing results to each other through the
     scratch) at the Qwen3.6-35B-A3B expert shape, fewer experts: the bits of the batched dispatches, the CPU
     specification within the block's tolerance, and the same answer on repeated calls over one scratch (the call
@@ -340,15 +341,17 @@ def test_moe_block_one_launch_equals_batched_dispatches_and_cpu_spec(oracle, dev
     sgl = bf((rng.standard_normal((1, H)) * 0.05).astype(np.float32))
     raw = {nm: weights(seed + T, n, k, 0.05) for nm, seed, n, k in
            (("eg", 31, E * I, H), ("eu", 32, E * I, H), ("ed", 33, E * H, I), ("sg", 34, SI, H), ("su", 35, SI, H), ("sd", 36, H, SI))}
-    q = {nm: oracle.quantize(a, a.shape[1], HQ_Q4_K, threads=8) for nm, a in raw.items()}
-    dq = {nm: oracle.dequantize(q[nm], HQ_Q4_K, threads=8).reshape(raw[nm].shape) for nm in raw}
+    ty = {nm: (td if nm in ("ed", "sd") else t) for nm in raw}  # Q5_K / Q6_K is the reference model's own mix
+    q = {nm: oracle.quantize(a, a.shape[1], ty[nm], threads=8) for nm, a in raw.items()}
+    dq = {nm: oracle.dequantize(q[nm], ty[nm], threads=8).reshape(raw[nm].shape) for nm in raw}
     xb = bf(acts(37 + T, T, H))
     res = acts(38, T, H)
     want = oracle.moe_ffn(xb, H, E, K, I, SI, router, dq["eg"], dq["eu"], dq["ed"], sgl[0], dq["sg"], dq["su"], dq["sd"]) + res
 
     dv = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
     w = ops.MoeFfnWeightsGpuQ(dv(router).to(torch.bfloat16), dv(q["eg"]), dv(q["eu"]), dv(q["ed"]),
-                              dv(sgl).to(torch.bfloat16), dv(q["sg"]), dv(q["su"]), dv(q["sd"]), HQ_Q4_K, H, E, K, I, SI)
+                              dv(sgl).to(torch.bfloat16), dv(q["sg"]), dv(q["su"]), dv(q["sd"]), t, H, E, K, I, SI,
+                              down_type=None if td == t else td)
     x = dv(xb).to(torch.bfloat16)
     assert ops.moe_ffn_decode_fused_supported(x, w)
     s = ops.MoeFfnScratch(w, T, dev)
