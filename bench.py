@@ -431,6 +431,28 @@ def bench_prefill_gemm(a, wtype=None):
         del wb
     except Exception as e:  # the reference figure must never take the bench line down
         vendor = {"error": str(e)[:200]}
+    # The same product over the F16 shadow of the weight (hq_matmul_f16_shadow: the reference's route for m > 8 when a
+    # weight has one, forward_mlx.rs:9790-9817): 2 bytes per weight kept in memory, no dequantisation in the product.
+    shadow_line = None
+    try:
+        shadow = ops.dequantize_ggml(w, N * K, t, dtype=torch.float16)
+        sws = torch.empty(ops.matmul_f16_shadow_workspace_bytes(M, N, K), dtype=torch.uint8, device=dev)
+        for _ in range(max(3, a.warmup)):
+            ops.matmul_f16_shadow(x, shadow, y, M, N, K, sws)
+        torch.cuda.synchronize()
+        evs = _events(a.steps)
+        for i in range(a.steps):
+            evs[i][0].record()
+            ops.matmul_f16_shadow(x, shadow, y, M, N, K, sws)
+            evs[i][1].record()
+        torch.cuda.synchronize()
+        sus = sum(e0.elapsed_time(e1) for e0, e1 in evs) * 1e3 / a.steps
+        shadow_line = {"what": "hq_matmul_f16_shadow: activations cast to f16 + the vendor library's dense GEMM over the weight's F16 shadow",
+                       "us_per_step": round(sus, 2), "TFLOP/s": round(flops / sus / 1e6, 1),
+                       "frac_mfma_peak": round(flops / sus / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4), "shadow_bytes": shadow.numel() * 2}
+        del shadow, sws
+    except Exception as e:
+        shadow_line = {"error": str(e)[:200]}
     return _finish(a, {
         "metric": "prefill TFLOP/s", "value": round(flops * a.steps / elapsed / 1e12, 1), "unit": "TFLOP/s",
         "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f16" if need else "bf16",
@@ -438,7 +460,7 @@ def bench_prefill_gemm(a, wtype=None):
                                f"activations, fp32 accumulate (BASELINE config 4)", "flop_per_step": flops,
                    "weight_bytes": w.numel(), "workspace_bytes": need,
                    "launches_per_step": 2 if need else 1, "us_per_step_with_weight_row_scales_kept_from_load_time": us_prepared,
-                   "vendor_dense_gemm_same_shape": vendor},
+                   "vendor_dense_gemm_same_shape": vendor, "f16_shadow_route": shadow_line},
         "roofline": {"bound": "mfma", "kernel": (f"activation pre-pass + f16 MFMA gemm {wtype}" if need else
                                                  f"bf16 MFMA gemm {wtype}"), "achieved": round(tf, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
@@ -885,6 +907,18 @@ def bench_decode_gemv(a):
         ref_shapes[nm] = entry
         del wsr
 
+    # What streaming these bytes costs on this device with no arithmetic at all (hq_stream_read_probe: plain 16-byte loads,
+    # the same back-to-back timing over the same rotated buffers): the rate the figures above can be read against beside
+    # the published peak.
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    probe = {}
+    for nm, bufs, reps in (("head_510MB", heads, 8), ("gate_28MB", [ws["gate"] for ws in sets] + [ws["up"] for ws in sets], 4)):
+        us = _launch_us([(lambda b=b: ops.stream_read_probe(b, sink)) for b in bufs] * reps)
+        nb_ = bufs[0].numel()
+        probe[nm] = {"us": round(us, 3), "bytes": nb_, "GBps": round(nb_ / us / 1e3, 1), "frac_hbm_peak": round(nb_ / us / 1e3 / HBM_PEAK_GBS, 4)}
+    probe["what"] = ("one plain read of the same buffers, 16 bytes per lane, no arithmetic (hq_stream_read_probe), timed like `kernels`: the "
+                     "streaming rate this device reaches; kernels[...].us / this us = how far a kernel is from it")
+
     value = step_bytes * a.steps / elapsed / 1e9
     head_us = kern_us["head_151936x4096"]
     head_gbs = nbytes["head"] / head_us / 1e3
@@ -921,6 +955,7 @@ def bench_decode_gemv(a):
                                                     "frac_hbm_peak": round(q4_bytes / q4_us_fewer / 1e3 / HBM_PEAK_GBS, 4)}},
         "dense_ffn_decode_chain": dense_ffn,
         "reference_shapes": ref_shapes,
+        "stream_read_probe": probe,
     }
 
 

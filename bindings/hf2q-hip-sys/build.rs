@@ -24,9 +24,13 @@ const SOURCES: &[&str] = &[
     "moe.hip",
     "moe_fused.hip",
     "quantize.hip",
+    "shadow.hip",
     "tq.hip",
     "tqp.hip",
 ];
+
+// Libraries the shared object is linked against beside the HIP runtime (the vendor GEMM behind hq_matmul_f16_shadow).
+const LINK_LIBS: &[&str] = &["-lhipblaslt"];
 
 // Flags of every compile; -Xclang -target-feature -Xclang -packed-fp32-ops keeps the compiler from forming packed-fp32
 // VALU operations.
@@ -89,7 +93,7 @@ fn main() {
             objects.push(obj);
         }
         let mut link = Command::new(&hipcc);
-        link.args(["--offload-arch=gfx950", "-shared", "-fPIC", "-o"]).arg(out.join("libhf2q_hip.so")).args(&objects);
+        link.args(["--offload-arch=gfx950", "-shared", "-fPIC", "-o"]).arg(out.join("libhf2q_hip.so")).args(&objects).args(LINK_LIBS);
         run(&mut link);
         out
     };

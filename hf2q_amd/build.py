@@ -21,6 +21,8 @@ FLAGS = [
     # keep the compiler from forming packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# Libraries the shared object is linked against beside the HIP runtime: the vendor GEMM behind the F16-shadow product.
+LINK_LIBS = ["-lhipblaslt"]
 # Translation units whose arithmetic must not be re-associated or contracted
 # (byte-exact quantizers): contraction off, fused ops only where fmaf is written.
 STRICT_FP = {"quantize.hip": ["-ffp-contract=off"]}
@@ -60,7 +62,7 @@ def build(force: bool = False, verbose: bool = True) -> str:
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         list(ex.map(run, jobs))
     if force or jobs or not os.path.exists(LIB):
-        run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
+        run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, *LINK_LIBS])
     return LIB
 
 

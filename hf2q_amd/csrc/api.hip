@@ -89,6 +89,21 @@ int cu_count(uint32_t* out) {
     return HQ_OK;
 }
 
+// hq_stream_read_probe: 64 KiB per workgroup, sixteen 16-byte loads per lane, all issued before the first is used.
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ p, uint64_t n16, uint32_t* sink) {
+    const uint64_t base = (uint64_t)blockIdx.x * 4096u + threadIdx.x;
+    uint4 v[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint64_t j = base + 256u * i;
+        v[i] = j < n16 ? p[j] : make_uint4(0, 0, 0, 0);
+    }
+    uint32_t acc = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    if (acc == 0x9e3779b9u && *sink != acc) *sink = acc;  // keeps the loads; practically never taken
+}
+
 }  // namespace hq
 
 using namespace hq;
@@ -656,6 +671,35 @@ int hq_moe_ffn_decode(void* stream, const hq_moe_ffn_layer* l, const void* x, hq
     a.t_gate_up = l->ggml_type;
     a.t_down = t_down;
     return launch_moe_fused((hipStream_t)stream, a);
+}
+
+size_t hq_matmul_f16_shadow_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
+    if (m == 0 || n == 0 || k == 0) return 0;
+    return f16_shadow_workspace_bytes(m, k);
+}
+
+int hq_matmul_f16_shadow(void* stream, const void* x, hq_act_dtype xdt, const void* w_f16, float* y, uint32_t m, uint32_t n, uint32_t k,
+                         void* workspace, size_t workspace_bytes) {
+    const char* fn = "hq_matmul_f16_shadow";
+    if (m == 0 || n == 0) return HQ_OK;
+    if (xdt != HQ_F32 && xdt != HQ_BF16) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: activation dtype %d", fn, (int)xdt);
+    if (k == 0 || k % 8) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: k = %u is not a positive multiple of 8", fn, k);
+    if (!x || !w_f16 || !y || !workspace) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+    if (!is_aligned(x, 16) || !is_aligned(w_f16, 16) || !is_aligned(y, 16) || !is_aligned(workspace, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: x, w_f16, y and workspace must be 16-byte aligned", fn);
+    const size_t need = f16_shadow_workspace_bytes(m, k);
+    if (workspace_bytes < need) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes, %zu needed", fn, workspace_bytes, need);
+    return launch_f16_shadow_matmul((hipStream_t)stream, x, xdt, w_f16, y, m, n, k, workspace, need);
+}
+
+int hq_stream_read_probe(void* stream, const void* buf, size_t bytes, uint32_t* sink) {
+    if (bytes == 0) return HQ_OK;
+    if (!buf || !sink || bytes % 16 || !is_aligned(buf, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_stream_read_probe: buf / sink null, or buf / bytes not multiples of 16");
+    const uint64_t n16 = bytes / 16, blocks = (n16 + 4095) / 4096;
+    if (blocks > 0x7fffffffull) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_stream_read_probe: %zu bytes", bytes);
+    hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, static_cast<const uint4*>(buf), n16, sink);
+    return check_launch("stream read probe launch");
 }
 
 void hq_set_handover_spin_limit(uint32_t limit) { g_spin_limit.store(limit, std::memory_order_relaxed); }

@@ -50,6 +50,10 @@ struct GemvArgs {
     uint32_t* route_ids;
     float* route_w;
 };
+// The F16-shadow product (shadow.hip): activations cast to f16 into `workspace`, then the vendor library's GEMM.
+size_t f16_shadow_workspace_bytes(uint32_t m, uint32_t k);
+int launch_f16_shadow_matmul(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_f16, float* y, uint32_t m, uint32_t n,
+                             uint32_t k, void* workspace, size_t workspace_bytes);
 // The current device's CU count (cached).
 int cu_count(uint32_t* out);
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t);

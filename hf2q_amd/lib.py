@@ -105,6 +105,9 @@ SIGNATURES = {
     "hq_tq_kv_capture_bytes": (_sz, [_u32, _u32, _u32]),
     "hq_tq_kv_capture": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _vp, _sz]),
     "hq_tq_kv_restore": (_i32, [_vp, _vp, _sz, _vp, _vp, _u32, _u32, _u32, _u32]),
+    "hq_matmul_f16_shadow_workspace_bytes": (_sz, [_u32, _u32, _u32]),
+    "hq_matmul_f16_shadow": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _vp, _sz]),
+    "hq_stream_read_probe": (_i32, [_vp, _vp, _sz, _vp]),
     "hq_gguf_open": (_i32, [_c.c_char_p, _c.POINTER(_vp)]),
     "hq_gguf_close": (None, [_vp]),
     "hq_gguf_tensor_count": (_u64, [_vp]),

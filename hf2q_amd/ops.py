@@ -326,6 +326,29 @@ def dequantize_ggml(weight: torch.Tensor, n_elems: int, ggml_type: int,
     return out
 
 
+def matmul_f16_shadow_workspace_bytes(m: int, n: int, k: int) -> int:
+    return int(_l.load().hq_matmul_f16_shadow_workspace_bytes(m, n, k))
+
+
+def matmul_f16_shadow(input: torch.Tensor, weight_f16: torch.Tensor, dst: torch.Tensor, m: int, n: int, k: int,
+                      workspace: torch.Tensor) -> None:
+    """dispatch_mm_v2_f16 (forward_mlx.rs:9790-9817): dst[m, n] = input[m, k] . weight_f16[n, k]^T over the F16 shadow of a
+    weight (dequantize_ggml(..., dtype=torch.float16)); f32 or bf16 activations, f32 output, the vendor library's GEMM."""
+    if weight_f16.dtype != torch.float16 or weight_f16.numel() < n * k:
+        raise ValueError("weight_f16 must hold n * k float16 values")
+    if dst.dtype != torch.float32 or dst.numel() < m * n or input.numel() < m * k:
+        raise ValueError("dst must hold m * n float32 values and input m * k activations")
+    if workspace.dtype != torch.uint8:
+        raise TypeError("workspace must be a uint8 tensor")
+    _l.check(_l.load().hq_matmul_f16_shadow(_stream(), _dev(input, "input"), _act_dtype(input), _dev(weight_f16, "weight_f16"),
+                                            _dev(dst, "dst"), m, n, k, _dev(workspace, "workspace"), workspace.numel()))
+
+
+def stream_read_probe(buf: torch.Tensor, sink: torch.Tensor) -> None:
+    """One plain streaming read of `buf` (hq_stream_read_probe): what moving that many bytes costs on this device."""
+    _l.check(_l.load().hq_stream_read_probe(_stream(), _dev(buf, "buf"), buf.numel() * buf.element_size(), _dev(sink, "sink")))
+
+
 def quantize_ggml(src: torch.Tensor, n_per_row: int, ggml_type: int) -> torch.Tensor:
     """f32 rows -> packed GGML blocks on the device (GgmlQuantizer::quantize without imatrix)."""
     if src.dtype != torch.float32:
@@ -854,12 +877,17 @@ def moe_ffn_decode_fused(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch
 _FUSED_CHUNKED_MAX_TOKENS = 48
 
 
-def moe_ffn_decode_fused_supported(x: torch.Tensor, w: MoeFfnWeightsGpuQ) -> bool:
+def moe_ffn_decode_fused_bytes(x: torch.Tensor, w: MoeFfnWeightsGpuQ) -> int:
+    """Scratch bytes of the one-launch form for these tokens; 0: the shape is not one it takes."""
     T = x.shape[0]
     if T > _FUSED_CHUNKED_MAX_TOKENS:
-        return False
+        return 0
     layer = w.c_layer()
-    return bool(_l.load().hq_moe_ffn_decode_layer_scratch_bytes(ctypes.byref(layer), min(T, 8), _act_dtype(x)))
+    return int(_l.load().hq_moe_ffn_decode_layer_scratch_bytes(ctypes.byref(layer), min(T, 8), _act_dtype(x)))
+
+
+def moe_ffn_decode_fused_supported(x: torch.Tensor, w: MoeFfnWeightsGpuQ) -> bool:
+    return moe_ffn_decode_fused_bytes(x, w) > 0
 
 
 def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: MoeFfnScratch, out: torch.Tensor,
@@ -879,7 +907,9 @@ def build_moe_ffn_layer_gpu_q_into(x: torch.Tensor, w: MoeFfnWeightsGpuQ, s: Moe
     K, H, E, I, SI, t, td = w.top_k, w.hidden, w.n_experts, w.inter, w.shared_inter, w.ggml_type, w.td
     rb = ggml_row_bytes(t, H)
     if fused is None:
-        fused = batched is None and route_in_launch is None and s.fused is not None and moe_ffn_decode_fused_supported(x, w)
+        # (a scratch made for fewer tokens than this call brings is too small for the one-launch form: separate dispatches then)
+        need = moe_ffn_decode_fused_bytes(x, w) if batched is None and route_in_launch is None and s.fused is not None else 0
+        fused = need > 0 and s.fused.numel() >= need
     if fused:
         # one launch for the whole block, the bits of the batched dispatches below
         return moe_ffn_decode_fused(x, w, s, out, residual)

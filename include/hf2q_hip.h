@@ -560,6 +560,30 @@ HQ_API int hq_tq_kv_capture(void* stream, const uint8_t* codes, const float* nor
 HQ_API int hq_tq_kv_restore(void* stream, const void* payload, size_t len, uint8_t* codes, float* norms,
                      uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t start_pos);
 
+/* ---- the F16 shadow of a weight ---- */
+
+/* y[m][n] (f32) = x[m][k] . W[n][k]^T over a weight that was dequantised to f16 once at load time (hq_dequant_ggml with
+ * HQ_F16): the route dispatch_qmatmul takes for m > 8 when a weight has a shadow (src/serve/forward_mlx.rs:9790-9817 ->
+ * dispatch_mm_v2_f16, F16 weight x F32 input -> F32 output; the shadow itself: materialize_f16_shadow, :9426-9440).
+ * Memory for speed: 2 bytes per weight instead of 0.56 - 1.06, no dequantisation inside the product.  x: [m][k] f32 or
+ * bf16, cast to f16 (round to nearest even) by a kernel of this library; the product is the vendor library's dense GEMM
+ * (hipBLASLt) with f32 accumulation.  k % 8 == 0; x, w_f16, y and `workspace` 16-byte aligned; `workspace`:
+ * hq_matmul_f16_shadow_workspace_bytes() bytes of device memory (the f16 activations + what the vendor library may use).
+ * The first call for a shape asks the vendor library for its kernel (host time, not capturable in a HIP graph); later
+ * calls of that shape only launch. */
+HQ_API size_t hq_matmul_f16_shadow_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+HQ_API int hq_matmul_f16_shadow(void* stream, const void* x, hq_act_dtype xdt, const void* w_f16, float* y, uint32_t m, uint32_t n,
+                         uint32_t k, void* workspace, size_t workspace_bytes);
+
+/* ---- measurement aid ---- */
+
+/* Reads `bytes` (a multiple of 16) of device memory at `buf` (16-byte aligned) once with plain 16-byte loads, one
+ * workgroup of 256 lanes per 64 KiB, and nothing else: the time of this launch over a buffer the caches do not hold is
+ * what streaming that many bytes costs on the device, the rate the bandwidth-bound kernels of this library can be read
+ * against beside the published peak.  `sink`: 4 writable bytes (written only if the data xor to a value they do not).
+ * No counterpart in the reference. */
+HQ_API int hq_stream_read_probe(void* stream, const void* buf, size_t bytes, uint32_t* sink);
+
 /* ---- GGUF reader (weights as hf2q loads them) ---- */
 
 /* Replaces mlx_native::gguf::GgufFile as hf2q uses it at load time

@@ -67,6 +67,28 @@ def test_workspace_queries_follow_the_routing():
     assert L.hq_qmatmul_id_ggml_workspace_bytes(64, 4, 128, 512, 8, 128 * 2 * 144, 10) == 0  # not a type of the library
 
 
+def test_k_slices_never_start_past_the_end_of_a_row():
+    """hq_qmatmul_ggml_k_slices for every k / 256 up to 130 and a spread of (m, n): the slices cover k, none is empty, and the
+    last one starts inside the row (k = 8448, 8704, 8960, 10496, 10752, 12544 once gave eight slices of which the last began
+    past it).  Pure host arithmetic: no GPU."""
+    L = lib.load()
+    s, per = ctypes.c_uint32(), ctypes.c_uint32()
+    cut = 0
+    for t in (lib.HQ_Q4_K, lib.HQ_Q5_K, lib.HQ_Q6_K, lib.HQ_Q8_0, lib.HQ_Q4_0):
+        for nsb in range(1, 131):
+            for m, n in ((9, 64), (17, 64), (64, 1536), (100, 130), (128, 4096), (200, 640), (256, 64), (256, 12288), (257, 64), (2048, 64)):
+                lib.check(L.hq_qmatmul_ggml_k_slices(m, n, nsb * 256, t, ctypes.byref(s), ctypes.byref(per)))
+                assert s.value >= 1 and per.value >= 1
+                assert s.value * per.value >= nsb, (t, m, n, nsb, s.value, per.value)
+                assert (s.value - 1) * per.value < nsb, (t, m, n, nsb, s.value, per.value)
+                if m > 256:
+                    assert s.value == 1
+                cut += s.value > 1
+    assert cut > 1000  # the query does describe cut products
+    assert L.hq_qmatmul_ggml_k_slices(17, 64, 100, lib.HQ_Q4_K, ctypes.byref(s), ctypes.byref(per)) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_qmatmul_ggml_k_slices(17, 64, 256, lib.HQ_Q4_K, None, ctypes.byref(per)) == lib.HQ_ERR_INVALID_ARGUMENT
+
+
 def test_empty_inputs_are_accepted_without_work():
     """Zero rows / tokens / elements: HQ_OK before any launch (the pointers here are never dereferenced); an empty
     attention cache is an error, as there is nothing to attend to."""

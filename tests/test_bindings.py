@@ -100,6 +100,8 @@ def test_build_rs_compiles_the_library_the_way_build_py_does():
     assert re.findall(r'"([^"]+)"', sources) == hq_build.sources()
     flags = re.search(r"const FLAGS: &\[&str\] = &\[(.*?)\];", text, flags=re.S).group(1)
     assert re.findall(r'"([^"]+)"', flags) == hq_build.FLAGS
+    libs = re.search(r"const LINK_LIBS: &\[&str\] = &\[(.*?)\];", text, flags=re.S).group(1)
+    assert re.findall(r'"([^"]+)"', libs) == hq_build.LINK_LIBS
     strict = re.search(r"const STRICT_FP: &\[\(&str, &str\)\] = &\[(.*?)\];", text, flags=re.S).group(1)
     assert {f: [fl] for f, fl in re.findall(r'\("([^"]+)", "([^"]+)"\)', strict)} == hq_build.STRICT_FP
     assert "Command::new(&hipcc)" in text and '"-shared"' in text and "cargo:rustc-link-lib=dylib=hf2q_hip" in text

@@ -60,6 +60,8 @@ def test_gemm_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
     (40, 200, 1152),    # Q8_0 / Q4_0 only: k % 256 = 128, the last run is half a one (and k is not cut)
     (200, 130, 2304),   # one token tile of 256 rows, two slices
     (256, 64, 4352),    # a full one, four slices
+    (64, 1536, 8960),   # 35 runs: slices of five, seven of them (eight of ceil(35 / 8) would leave the last one empty)
+    (200, 256, 8448),   # 33 runs
 ])
 def test_small_tiles_and_k_slices_match_f64_oracle(oracle, dev, t, m, n, k):
     """Up to 256 activation rows are one token tile (64, 128 or 256 rows; Q4_K / Q5_K have the 64-row one), with k cut
@@ -390,3 +392,48 @@ def test_tile_gemm_with_caller_workspace_replays_from_a_hip_graph(oracle, dev, k
         torch.cuda.synchronize()
         assert torch.equal(got, eager), f"replay {rep}"
         assert torch.isfinite(got).all()
+
+
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q8_0])
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("m,n,k", [(9, 64, 256), (72, 130, 1024), (300, 256, 2048), (17, 1000, 520)])
+def test_f16_shadow_matmul_matches_f64_oracle(oracle, dev, t, xdt, m, n, k):
+    """dispatch_mm_v2_f16's route (forward_mlx.rs:9790-9817): the weight dequantised to f16 once, then a dense product.
+    Against float64 over exactly those f16 weights and the f16-rounded activations (what the product consumes), to the
+    tile kernels' bound; and against the quantized-weight product of the same call, which differs by the f16 rounding
+    of the weights (2^-11 relative per weight)."""
+    if k % oracle.BLOCK_ELEMS[t]:
+        k = k // 256 * 256
+    blocks = oracle.quantize(weights(11 + m, n, k), k, t, threads=8)
+    x = acts(12 + n, m, k)
+    xd = torch.from_numpy(x).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    wd = torch.from_numpy(blocks).to(dev)
+    shadow = ops.dequantize_ggml(wd, n * k, t, dtype=torch.float16)
+    assert torch.equal(shadow.float(), ops.dequantize_ggml(wd, n * k, t).half().float())
+    ws = torch.empty(ops.matmul_f16_shadow_workspace_bytes(m, n, k), dtype=torch.uint8, device=dev)
+    y = torch.full((m, n), float("nan"), device=dev)
+    for _ in range(2):  # the second call reuses the remembered plan
+        ops.matmul_f16_shadow(xd, shadow, y, m, n, k, ws)
+    torch.cuda.synchronize()
+    x16 = xd.float().half().double().cpu().numpy()
+    ref = x16 @ shadow.double().cpu().numpy().reshape(n, k).T
+    assert_matmul_close_f16_tile(y.cpu().numpy(), ref, f"f16 shadow t={t} {xdt} {m}x{n}x{k}")
+    yq = torch.empty(m, n, device=dev)
+    ops.quantized_matmul_ggml(xd, wd, yq, GgmlQuantizedMatmulParams(m, n, k, t))
+    assert (y - yq).abs().max().item() <= 2e-3 * np.abs(ref).max()
+
+
+def test_f16_shadow_matmul_rejects_bad_arguments(dev):
+    m, n, k = 16, 32, 64
+    x = torch.zeros(m, k, device=dev)
+    w = torch.zeros(n, k, device=dev, dtype=torch.float16)
+    y = torch.empty(m, n, device=dev)
+    ws = torch.empty(ops.matmul_f16_shadow_workspace_bytes(m, n, k), dtype=torch.uint8, device=dev)
+    with pytest.raises(ops.HqError):
+        ops.matmul_f16_shadow(x, w, y, m, n, k, ws[:1024])       # workspace too small
+    with pytest.raises(ops.HqError):
+        ops.matmul_f16_shadow(x, w, y, m, n, 60, ws)             # k % 8
+    with pytest.raises(ValueError):
+        ops.matmul_f16_shadow(x, w.float(), y, m, n, k, ws)      # not an f16 shadow
+    assert ops.matmul_f16_shadow_workspace_bytes(0, n, k) == 0

@@ -469,6 +469,26 @@ def test_small_batch_rows_match_f64_oracle(oracle, dev, t, xdt, m, n, k):
         assert np.abs(y1.cpu().numpy()[0] - y.cpu().numpy()[r]).max() <= 1e-4 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K])
+@pytest.mark.parametrize("m,k", [(3, 24576), (4, 24576), (4, 20480), (7, 24576)])
+def test_small_batch_rows_of_very_wide_matrices(oracle, dev, t, m, k):
+    """bf16 rows over k = 20480 / 24576: three or four staged activation rows would not fit a workgroup's LDS (4 x 24576 x
+    2.25 bytes = 221 KB), so the rows go in passes of as many as do fit; each row equals its one-row product."""
+    n = 2048  # enough rows for the streaming form at 256 CUs x 16 waves
+    blocks = oracle.quantize(weights(k + m + t, n, k), k, t, threads=8)
+    x = acts(k + m, m, k)
+    ref = oracle.qmatmul_f64(oracle.f32_to_bf16_bits(x), blocks, m, n, k, t)
+    xd = torch.from_numpy(x).to(dev).to(torch.bfloat16)
+    wd = torch.from_numpy(blocks).to(dev)
+    y = torch.full((m, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd, wd, y, GgmlQuantizedMatmulParams(m, n, k, t))
+    assert_matmul_close(y.cpu().numpy(), ref, f"wide rows t={t} {m}x{n}x{k}")
+    y1 = torch.empty((1, n), device=dev)
+    for r in range(m):
+        ops.quantized_matmul_ggml(xd[r:r + 1].contiguous(), wd, y1, GgmlQuantizedMatmulParams(1, n, k, t))
+        assert np.abs(y1.cpu().numpy()[0] - y.cpu().numpy()[r]).max() <= 1e-4 * np.abs(ref).max()
+
+
 ROWS32_SHAPES = [  # (m, n, k): Q8_0 / Q4_0; k is walked in chunks of 2048 (64 blocks, one per lane)
     (2, 80, 2048), (3, 64, 1024), (4, 200, 4096), (4, 5, 32), (5, 33, 320), (6, 130, 3104), (7, 250, 2048), (8, 96, 12288),
     (8, 4100, 256),   # more rows than one pass of 16 waves x 256 workgroups covers on a small device share

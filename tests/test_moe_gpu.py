@@ -461,6 +461,25 @@ def test_moe_block_one_launch_rejects_other_shapes(oracle, dev):
     assert e.value.status == 2
 
 
+def test_moe_block_falls_back_when_the_one_launch_scratch_is_too_small(oracle, dev):
+    """The default route takes the one-launch form only with a scratch of the size the library asks for; with a smaller one
+    the block runs as separate dispatches (same bits), it does not raise."""
+    H, E, K, I, SI, T = 2048, 32, 4, 512, 512, 2
+    w = _moe_weights(oracle, dev, HQ_Q4_K, H, E, K, I, SI)
+    x = torch.from_numpy(acts(5, T, H)).to(dev).to(torch.bfloat16)
+    s = ops.MoeFfnScratch(w, T, dev)
+    assert s.fused is not None and s.fused.numel() >= ops.moe_ffn_decode_fused_bytes(x, w) > 0
+    ref = torch.empty(T, H, device=dev)
+    ops.build_moe_ffn_layer_gpu_q_into(x, w, s, ref)
+    s.fused = s.fused[:256]
+    out = torch.full((T, H), float("nan"), device=dev)
+    ops.build_moe_ffn_layer_gpu_q_into(x, w, s, out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+    with pytest.raises(ops.HqError):
+        ops.moe_ffn_decode_fused(x, w, s, out)
+
+
 DENSE_DECODE_CASES = [  # (hidden, inter, gate / up type, down type)
     (4096, 12288, HQ_Q4_K, HQ_Q4_K), (2816, 4096, HQ_Q5_K, HQ_Q6_K), (2048, 8192, HQ_Q4_K, HQ_Q6_K), (1536, 8960, HQ_Q4_K, HQ_Q4_K),
     (4096, 12288, HQ_Q6_K, HQ_Q6_K), (4096, 11008, HQ_Q8_0, HQ_Q8_0), (2048, 5632, HQ_Q4_0, HQ_Q4_0), (1024, 512, HQ_Q5_K, HQ_Q5_K),
