@@ -819,10 +819,14 @@ int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
 // same for any 3 / 4 .. 8 rows.  Q6_K, 151936 x 4096: 163 / 173 us for three / four rows and 252 .. 281 for five .. seven
 // against 307; 12288 x 4096: 13 .. 28 against 29.  Q4_K / Q5_K: three and four rows, 10.8 / 12.9 against 14.2 us at
 // 12288 x 4096 (102 / 132 against 134 at 151936 x 4096); from five rows on their small-batch kernel is ahead.
+// Where the small-batch kernel has its stage-once form (gemv_rows_stream_fast: Q6_K 151936 x 4096 134 us, Q4_K 65536 x 4096
+// 41 us, Q4_K / Q6_K 12288 x 4096 13 / 21 us for any 3 .. 8 rows) it is ahead from five rows on, and from three on
+// matrices of 32768 rows or more (three and four rows in passes: 55 / 62 us on the 65536-row Q4_K matrix).
 bool gemv_stream_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
     if (xdt != HQ_BF16 || m < 3) return false;
     uint32_t cus = 0;
     if (cu_count(&cus)) return false;
+    if (gemv_rows_stream_fast(t, xdt, m, n, k) && (m >= 5 || n >= 32768)) return false;
     if (t == HQ_Q6_K) return m <= 7 && stream_takes<HQ_Q6_K>(n, k, cus);
     if (t == HQ_Q4_K) return m <= 4 && stream_takes<HQ_Q4_K>(n, k, cus);
     if (t == HQ_Q5_K) return m <= 4 && stream_takes<HQ_Q5_K>(n, k, cus);

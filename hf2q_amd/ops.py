@@ -344,6 +344,46 @@ def matmul_f16_shadow(input: torch.Tensor, weight_f16: torch.Tensor, dst: torch.
                                             _dev(dst, "dst"), m, n, k, _dev(workspace, "workspace"), workspace.numel()))
 
 
+# Above this many activation rows dispatch_qmatmul takes the matrix-matrix routes (mlx-native's MM_ROUTING_THRESHOLD,
+# forward_mlx.rs:9791).
+MM_ROUTING_THRESHOLD = 8
+
+
+@dataclass
+class MlxQWeight:
+    """A quantized linear weight as dispatch_qmatmul sees it (forward_mlx.rs:340-402): the raw GGML blocks with their type
+    and shape (QuantWeightInfo: rows = n, cols = k) and, optionally, the weight's F16 shadow."""
+    buffer: torch.Tensor
+    ggml_dtype: int
+    rows: int
+    cols: int
+    f16_shadow: torch.Tensor | None = None
+
+    def matmul_params(self, m: int) -> GgmlQuantizedMatmulParams:
+        """forward_mlx.rs:408-415."""
+        return GgmlQuantizedMatmulParams(m, self.rows, self.cols, self.ggml_dtype)
+
+    def populate_f16_shadow(self) -> None:
+        """populate_f16_shadow_if_enabled / materialize_f16_shadow (forward_mlx.rs:9403-9440): the blocks dequantised once to
+        f16 [rows, cols], kept beside them (2 bytes per weight more)."""
+        self.f16_shadow = dequantize_ggml(self.buffer, self.rows * self.cols, self.ggml_dtype, dtype=torch.float16)
+
+
+def dispatch_qmatmul(input: torch.Tensor, weight: MlxQWeight, output: torch.Tensor, m: int,
+                     workspace: torch.Tensor | None = None) -> None:
+    """dispatch_qmatmul (forward_mlx.rs:9655-9969) for GGML-block weights: more than MM_ROUTING_THRESHOLD rows over a weight
+    with an F16 shadow take the dense f16 product (:9790-9817), everything else the quantized product, whose own routing
+    by m (GEMV, small-batch, tile kernels) is the library's.  `workspace`: device scratch for the route taken
+    (matmul_f16_shadow_workspace_bytes / quantized_matmul_workspace_bytes); allocated here when absent."""
+    n, k = weight.rows, weight.cols
+    if m > MM_ROUTING_THRESHOLD and weight.f16_shadow is not None:
+        need = matmul_f16_shadow_workspace_bytes(m, n, k)
+        if workspace is None or workspace.numel() * workspace.element_size() < need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=input.device)
+        return matmul_f16_shadow(input, weight.f16_shadow, output, m, n, k, workspace)
+    quantized_matmul_ggml(input, weight.buffer, output, weight.matmul_params(m), workspace=workspace)
+
+
 def stream_read_probe(buf: torch.Tensor, sink: torch.Tensor) -> None:
     """One plain streaming read of `buf` (hq_stream_read_probe): what moving that many bytes costs on this device."""
     _l.check(_l.load().hq_stream_read_probe(_stream(), _dev(buf, "buf"), buf.numel() * buf.element_size(), _dev(sink, "sink")))

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import assert_matmul_close, assert_matmul_close_f16_tile
+from _util import acts, assert_matmul_close, assert_matmul_close_f16_tile
 from hf2q_amd import ops
 from hf2q_amd.ops import (HQ_Q4_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, FlashAttnVecTqHbParams,
                           GgmlQuantizedMatmulParams)
@@ -62,6 +62,38 @@ def test_decode_gemv_full_size(oracle, dev, n, k, t, m):
     assert (yab - (ya + yb)).abs().max().item() <= 2e-5 * scale
     # (c) exact scaling by a power of two
     assert torch.equal(run(xa * 4.0), ya * 4.0)
+
+
+@pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K])
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048)])
+def test_small_batch_rows_staged_once(oracle, dev, t, xdt, n, k):
+    """3 .. 8 activation rows over matrices of two groups of 16 rows per CU or more, all of k in LDS: the small-batch form
+    that stages the activations once per CU (bf16: weights fetched as 16-byte pieces through LDS; f32: fetched by the
+    lanes that use them).  Ragged last group (n % 16 = 8 / 3 / 0).  Sampled rows against the f64 oracle, every row
+    against the one-row product of the same activations, and the same result on a second call."""
+    w = _quantized(dev, n, k, t, 11 + n + t)
+    rng = np.random.default_rng(n + k + t)
+    rows = np.unique(np.concatenate([[0, 1, 15, 16, n - 17, n - 16, n - 2, n - 1], rng.integers(0, n, 50)]))
+    wr = _rows_of(w, rows, k, t, oracle)
+    for m in (3, 5, 8):
+        x = acts(m + n, m, k)
+        xd = torch.from_numpy(x).to(dev)
+        xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+        xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
+        y = torch.full((m, n), float("nan"), device=dev)
+        p = GgmlQuantizedMatmulParams(m, n, k, t)
+        ops.quantized_matmul_ggml(xd, w, y, p)
+        assert torch.isfinite(y).all()
+        ref = oracle.qmatmul_f64(xv, wr, m, rows.size, k, t)
+        assert_matmul_close(y[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, f"rows staged once t={t} {xdt} {m}x{n}x{k}")
+        y1 = torch.empty((1, n), device=dev)
+        for r in range(m):
+            ops.quantized_matmul_ggml(xd[r:r + 1].contiguous(), w, y1, GgmlQuantizedMatmulParams(1, n, k, t))
+            assert (y1[0] - y[r]).abs().max().item() <= 1e-4 * np.abs(ref).max()
+        y2 = torch.full((m, n), float("nan"), device=dev)
+        ops.quantized_matmul_ggml(xd, w, y2, p)
+        assert torch.equal(y, y2)
 
 
 # The reference's own decode shapes and dtype: f32 activations (gpu_full_attn.rs:835), k = 2816 (Gemma-4 projections, 11

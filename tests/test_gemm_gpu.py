@@ -437,3 +437,31 @@ def test_f16_shadow_matmul_rejects_bad_arguments(dev):
     with pytest.raises(ValueError):
         ops.matmul_f16_shadow(x, w.float(), y, m, n, k, ws)      # not an f16 shadow
     assert ops.matmul_f16_shadow_workspace_bytes(0, n, k) == 0
+
+
+def test_dispatch_qmatmul_routes_by_rows_and_shadow(oracle, dev):
+    """dispatch_qmatmul (forward_mlx.rs:9655-9969): up to 8 rows, or no shadow -> the quantized product (same bits as
+    calling it); more rows over a weight with a shadow -> the f16 product (same bits as calling that)."""
+    n, k, t = 192, 1024, HQ_Q4_K
+    wq = ops.MlxQWeight(torch.from_numpy(oracle.quantize(weights(3, n, k), k, t, threads=8)).to(dev), t, n, k)
+    assert wq.matmul_params(5) == GgmlQuantizedMatmulParams(5, n, k, t)
+    for m in (1, 8, 40):
+        x = torch.from_numpy(acts(m, m, k)).to(dev)
+        yq = torch.empty(m, n, device=dev)
+        ops.quantized_matmul_ggml(x, wq.buffer, yq, wq.matmul_params(m))
+        y = torch.full((m, n), float("nan"), device=dev)
+        ops.dispatch_qmatmul(x, wq, y, m)
+        assert torch.equal(y, yq)
+    wq.populate_f16_shadow()
+    assert wq.f16_shadow.dtype == torch.float16 and wq.f16_shadow.numel() == n * k
+    for m in (8, 9, 40):
+        x = torch.from_numpy(acts(m, m, k)).to(dev)
+        want = torch.empty(m, n, device=dev)
+        if m > ops.MM_ROUTING_THRESHOLD:
+            ws = torch.empty(ops.matmul_f16_shadow_workspace_bytes(m, n, k), dtype=torch.uint8, device=dev)
+            ops.matmul_f16_shadow(x, wq.f16_shadow, want, m, n, k, ws)
+        else:
+            ops.quantized_matmul_ggml(x, wq.buffer, want, wq.matmul_params(m))
+        y = torch.full((m, n), float("nan"), device=dev)
+        ops.dispatch_qmatmul(x, wq, y, m)
+        assert torch.equal(y, want)
