@@ -907,6 +907,23 @@ def bench_decode_gemv(a):
         ref_shapes[nm] = entry
         del wsr
 
+    # A few activation rows at once (batched decode): one pass over the weights for all of them.  The head and the gate
+    # matrix of the step above, and a 65536 x 4096 Q4_K matrix; us per launch, weight bytes / time.
+    small_batch = {}
+    big = [make_weight(65536, H, HQ_Q4_K) for _ in range(4)]
+    for nm, mats, (n_, k_, t_) in (("head_q6_k_151936x4096", heads, shapes["head"]), ("q4_k_65536x4096", big, (65536, H, HQ_Q4_K)),
+                                   ("gate_q4_k_12288x4096", [ws["gate"] for ws in sets] + [ws["up"] for ws in sets], shapes["gate"])):
+        entry = {"bytes": mats[0].numel()}
+        for m_ in (2, 4, 8):
+            xm = torch.randn(m_, k_, generator=gx, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            ym = torch.empty(m_, n_, device=dev)
+            pm = GgmlQuantizedMatmulParams(m_, n_, k_, t_)
+            us = _launch_us([(lambda w=w: ops.quantized_matmul_ggml(xm, w, ym, pm)) for w in mats] * max(1, 12 // len(mats)))
+            entry[f"rows_{m_}"] = {"us": round(us, 2), "GBps": round(mats[0].numel() / us / 1e3, 1),
+                                   "frac_hbm_peak": round(mats[0].numel() / us / 1e3 / HBM_PEAK_GBS, 4)}
+        small_batch[nm] = entry
+    del big
+
     # What streaming these bytes costs on this device with no arithmetic at all (hq_stream_read_probe: plain 16-byte loads,
     # the same back-to-back timing over the same rotated buffers): the rate the figures above can be read against beside
     # the published peak.
@@ -956,6 +973,7 @@ def bench_decode_gemv(a):
         "dense_ffn_decode_chain": dense_ffn,
         "reference_shapes": ref_shapes,
         "stream_read_probe": probe,
+        "small_batch_rows": small_batch,
     }
 
 

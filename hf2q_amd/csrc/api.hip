@@ -89,18 +89,23 @@ int cu_count(uint32_t* out) {
     return HQ_OK;
 }
 
-// hq_stream_read_probe: 64 KiB per workgroup, sixteen 16-byte loads per lane, all issued before the first is used.
+// hq_stream_read_probe: a fixed grid of waves, each reading runs of 8 KiB (eight 16-byte loads per lane, all issued
+// before the first is used) a grid's width apart, front to back through the buffer.
 __global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ p, uint64_t n16, uint32_t* sink) {
-    const uint64_t base = (uint64_t)blockIdx.x * 4096u + threadIdx.x;
-    uint4 v[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const uint64_t j = base + 256u * i;
-        v[i] = j < n16 ? p[j] : make_uint4(0, 0, 0, 0);
-    }
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint64_t wave = (uint64_t)blockIdx.x * 4u + (threadIdx.x >> 6), waves = (uint64_t)gridDim.x * 4u;
+    const uint64_t chunks = (n16 + 511u) / 512u;
     uint32_t acc = 0;
+    for (uint64_t c = wave; c < chunks; c += waves) {
+        uint4 v[8];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+        for (int i = 0; i < 8; ++i) {
+            const uint64_t j = c * 512u + 64u * i + lane;
+            v[i] = j < n16 ? p[j] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    }
     if (acc == 0x9e3779b9u && *sink != acc) *sink = acc;  // keeps the loads; practically never taken
 }
 
@@ -696,8 +701,10 @@ int hq_stream_read_probe(void* stream, const void* buf, size_t bytes, uint32_t* 
     if (bytes == 0) return HQ_OK;
     if (!buf || !sink || bytes % 16 || !is_aligned(buf, 16))
         return fail(HQ_ERR_INVALID_ARGUMENT, "hq_stream_read_probe: buf / sink null, or buf / bytes not multiples of 16");
-    const uint64_t n16 = bytes / 16, blocks = (n16 + 4095) / 4096;
-    if (blocks > 0x7fffffffull) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_stream_read_probe: %zu bytes", bytes);
+    const uint64_t n16 = bytes / 16, chunks = (n16 + 511) / 512;
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
+    const uint64_t blocks = chunks / 4 + 1 < 8ull * cus ? chunks / 4 + 1 : 8ull * cus;  // eight workgroups of four waves per CU
     hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, static_cast<const uint4*>(buf), n16, sink);
     return check_launch("stream read probe launch");
 }

@@ -641,3 +641,19 @@ def test_decode_gemvs_replay_from_a_hip_graph(oracle, dev, t):
         assert torch.equal(got[0], got[1])  # the same matrix through the one-matrix and the two-matrix launch
         xb = x.float().cpu().numpy().astype(np.float64)
         assert_matmul_close(got[0].cpu().numpy(), xb @ dq0.T, f"replay {rep}")
+
+
+def test_stream_read_probe_reads_and_writes_nothing(dev):
+    """hq_stream_read_probe only reads: any size that is whole 16-byte pieces (ragged against the 8 KiB runs), the buffer and
+    the sink unchanged; odd sizes and alignments are rejected."""
+    buf = torch.arange(0, (3 << 20) + 4, dtype=torch.int32, device=dev)  # 12 MiB + 16 bytes
+    keep = buf.clone()
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    ops.stream_read_probe(buf, sink)
+    ops.stream_read_probe(buf[:4], sink)
+    torch.cuda.synchronize()
+    assert torch.equal(buf, keep) and sink.item() == 0
+    with pytest.raises(ops.HqError):
+        ops.stream_read_probe(buf[:3], sink)   # 12 bytes
+    with pytest.raises(ops.HqError):
+        ops.stream_read_probe(buf[1:5], sink)  # not 16-byte aligned
