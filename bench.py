@@ -39,14 +39,23 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 # 2.0), WRITE_SIZE all of them (1.0).  The runs and their figures are in profiles/*_pmc_traffic.md.
 PMC_TRAFFIC_BYTES = {
     # (FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0) x 1024 per dispatch
-    "gemv_head_q6_k_151936x4096": int(256455.0 * 2.0 * 1024 + 4829.5 * 1.0 * 1024),
+    "gemv_head_q6_k_151936x4096": int(256451.5 * 2.0 * 1024 + 4890.7 * 1.0 * 1024),
     # activation pre-pass + tile GEMM, Q4_K, 2048 x 12288 x 4096 (the GEMM re-fetches the weights once per 256-token tile)
     "prefill_gemm_q4_k_2048x12288x4096": int((23301.6 + 132573.1) * 2.0 * 1024 + (16496.5 + 98311.8) * 1.0 * 1024),
     # split (with the q rotation) + merge (with the output rotation), 32K context, 2 kv heads, head_dim 256
     "tq_attention_32k_fused_chain": int((16897.5 + 1072.5) * 2.0 * 1024 + (2112.0 + 16.0) * 1.0 * 1024),
     # the one-launch MoE FFN block, hidden 2048, 256 experts x 512, top-8, 1 and 8 tokens
-    "moe_ffn_decode_t1": int(8675.0 * 2.0 * 1024 + 108.3 * 1.0 * 1024),
-    "moe_ffn_decode_t8": int(63307.0 * 2.0 * 1024 + 866.5 * 1.0 * 1024),
+    "moe_ffn_decode_t1": int(8698.0 * 2.0 * 1024 + 108.3 * 1.0 * 1024),
+    "moe_ffn_decode_t8": int(63320.4 * 2.0 * 1024 + 866.5 * 1.0 * 1024),
+    # the same block with gate / up in Q5_K and down in Q6_K
+    "moe_ffn_decode_t1_q5k_q6k": int(11157.5 * 2.0 * 1024 + 108.3 * 1.0 * 1024),
+    "moe_ffn_decode_t8_q5k_q6k": int(82141.3 * 2.0 * 1024 + 866.5 * 1.0 * 1024),
+    # Q8_0, 2048 x 12288 x 4096: tile GEMM + the plain call's pre-pass (that one worked out of a run that mixes plain and
+    # kept-scales calls 1 : 2: 68,804 KiB fetched for the activations and every line of the weights, 16,464 written)
+    "prefill_gemm_q8_0_2048x12288x4096": int((232529.5 + 68804.0 / 2.0) * 2.0 * 1024 + (98572.3 + 16464.2) * 1.0 * 1024),
+    # grouped mul_mat_id, 2048 tokens x top-8 over 256 experts of 512 x 2048 Q4_K: pre-pass (sort, conversion, scan of the stack's
+    # headers) + grouped tile GEMM (bench.py --workload moe_prefill --step-only)
+    "moe_prefill_gate_up_2048x8": int((163244.4 + 69718.9) * 2.0 * 1024 + (32887.6 + 8788.0) * 1.0 * 1024),
 }
 
 
@@ -67,6 +76,7 @@ def parse():
     ap.add_argument("--no-graph", action="store_true",
                     help="moe_decode / moe_prefill / tq_attention: launch every kernel from the host instead of replaying a HIP "
                          "graph of the step (the steps are 4-12 launches of a few microseconds each)")
+    ap.add_argument("--step-only", action="store_true", help="moe_prefill: only the workload's own step (the gate / up call)")
     ap.add_argument("--block-only", action="store_true",
                     help="moe_prefill: run only the whole-block part (for a kernel trace of the block's launches alone)")
     ap.add_argument("--kept-scales", action="store_true",
@@ -349,7 +359,7 @@ def bench_moe_decode(a, tokens=None, mix=False):
                    "layers_rotated": n_layers},
         "roofline": {"bound": "hbm", "kernel": "MoE FFN layer (hq_moe_ffn_decode, one launch)", "achieved": round(gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": None if mix else PMC_TRAFFIC_BYTES.get(f"moe_ffn_decode_t{T}"),
+                     "traffic": PMC_TRAFFIC_BYTES.get(f"moe_ffn_decode_t{T}" + ("_q5k_q6k" if mix else "")),
                      "us_per_launch": round(layer_us, 3), "bytes_per_launch": int(step_bytes)}})
 
 
@@ -464,7 +474,7 @@ def bench_prefill_gemm(a, wtype=None):
         "roofline": {"bound": "mfma", "kernel": (f"activation pre-pass + f16 MFMA gemm {wtype}" if need else
                                                  f"bf16 MFMA gemm {wtype}"), "achieved": round(tf, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": PMC_TRAFFIC_BYTES["prefill_gemm_q4_k_2048x12288x4096"] if wtype == "q4_k" else None,
+                     "traffic": PMC_TRAFFIC_BYTES.get(f"prefill_gemm_{wtype}_2048x12288x4096"),
                      "us_per_launch": round(us, 2), "flop_per_launch": flops}})
 
 
@@ -503,6 +513,12 @@ def bench_moe_prefill(a):
         def step_prepared(i):
             ops.quantized_matmul_id_ggml(x, stacks[i % n_stacks], ids, y, p, scratch=scratch, w_row_scales=scales[i % n_stacks])
 
+        if a.step_only:  # the plain call and nothing else
+            for i in range(max(a.warmup, 1)):
+                step(i)
+            torch.cuda.synchronize()
+            elapsed, us = _timed_steps(a, step, n_stacks)
+            return elapsed, us, us, need
         for i in range(max(a.warmup, 1)):
             step(i)
             step_prepared(i)
@@ -542,6 +558,11 @@ def bench_moe_prefill(a):
                        "us_per_layer": round(us, 1)}})
 
     elapsed, us, us_prep, need = shape(I, H, T, K)
+    if a.step_only:  # the workload's own step and nothing else: for counter passes, whose per-kernel averages would mix shapes
+        flops = 2.0 * T * K * I * H
+        return _finish(a, {"metric": "MoE prefill mul_mat_id eff. TFLOP/s", "value": round(flops * a.steps / elapsed / 1e12, 1), "unit": "TFLOP/s",
+                           "ms_per_step": round(elapsed / a.steps * 1e3, 4), "dtype": "f16",
+                           "config": {"workload": "moe_prefill --step-only: the gate / up mul_mat_id call alone", "us_per_step": round(us, 2)}})
     _, us_down, us_down_prep, _ = shape(H, I, T * K, 1)
 
     # gate, up and SwiGLU of the block: two calls and hq_silu_mul, against the one grouped call that does all three
@@ -636,7 +657,7 @@ def bench_moe_prefill(a):
                                            "us_per_step_with_kept_scales": round(us_down_prep, 2)}},
         "roofline": {"bound": "mfma", "kernel": "grouped pre-pass + grouped f16 MFMA gemm q4_k", "achieved": round(tf, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": None, "us_per_launch": round(us, 2), "flop_per_launch": flops}})
+                     "traffic": PMC_TRAFFIC_BYTES["moe_prefill_gate_up_2048x8"], "us_per_launch": round(us, 2), "flop_per_launch": flops}})
 
 
 def bench_tq_attention(a):
