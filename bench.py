@@ -909,7 +909,7 @@ def bench_decode_gemv(a):
                          "projection (gpu_ffn.rs:1231-1306); us per FFN, every form the same bits")
     del ffn_w, gate_b, up_b
 
-    # The reference's own published decode shapes (BASELINE.md: docs/ADR-028...:5247, 5248, 4884, 8564), both activation
+    # The reference's own published decode shapes (docs/ADR-028...:5247, 5248, 4884, 8564), both activation
     # dtypes (its call sites pass f32, gpu_full_attn.rs:835): lm_head 262144 x 2816 in Q6_K and Q8_0, the 4096 x 2816 and
     # 2816 x 4096 projections in Q5_K.
     ref_shapes = {}

@@ -146,22 +146,47 @@ int hq_dequant_ggml(void* stream, const void* w_blocks, void* out, hq_act_dtype 
     return launch_dequant((hipStream_t)stream, w_blocks, out, out_dtype, n_elems, t);
 }
 
-int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row,
-                     hq_ggml_type t, void* out_blocks) {
-    if (!known_type(t)) return fail(HQ_ERR_UNSUPPORTED, "hq_quantize_ggml: unsupported ggml type %d", (int)t);
+static int quantize_common(const char* fn, void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row, hq_ggml_type t,
+                           void* out_blocks, const float* imatrix, bool with_imatrix, void* scratch, size_t scratch_bytes) {
+    if (!known_type(t)) return fail(HQ_ERR_UNSUPPORTED, "%s: unsupported ggml type %d", fn, (int)t);
     const uint32_t be = hq_block_elems(t);
     // Same two shape rules as GgmlQuantizer::quantize (quantizer.rs:57-71).
     if (n_per_row == 0 || n_per_row % be)
-        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_quantize_ggml: n_per_row %llu not a multiple of block size %u",
-                    (unsigned long long)n_per_row, be);
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: n_per_row %llu not a multiple of block size %u", fn, (unsigned long long)n_per_row, be);
     if (n_elems % n_per_row)
-        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_quantize_ggml: n_elems %llu not a multiple of n_per_row %llu",
-                    (unsigned long long)n_elems, (unsigned long long)n_per_row);
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: n_elems %llu not a multiple of n_per_row %llu", fn, (unsigned long long)n_elems,
+                    (unsigned long long)n_per_row);
+    if (n_per_row / be > 0xffffffffull) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: n_per_row %llu", fn, (unsigned long long)n_per_row);
     if (n_elems == 0) return HQ_OK;
-    if (!src || !out_blocks) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_quantize_ggml: null buffer");
-    if (!is_aligned(src, 16)) return fail(HQ_ERR_INVALID_ARGUMENT, "hq_quantize_ggml: src must be 16-byte aligned");
+    if (!src || !out_blocks) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null buffer", fn);
+    if (!is_aligned(src, 16)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: src must be 16-byte aligned", fn);
     if (int rc = check_weight_alignment(out_blocks, t)) return rc;
-    return launch_quantize((hipStream_t)stream, src, n_elems, n_per_row, t, out_blocks);
+    float* rows = nullptr;
+    if (with_imatrix) {
+        if (!imatrix || !is_aligned(imatrix, 4)) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: imatrix is null or not 4-byte aligned", fn);
+        const size_t need = hq_quantize_ggml_imatrix_scratch_bytes(n_elems, n_per_row, t);
+        if (need) {
+            if (!scratch || !is_aligned(scratch, 4) || scratch_bytes < need)
+                return fail(HQ_ERR_INVALID_ARGUMENT, "%s: scratch of %zu bytes, %zu needed (4-byte aligned)", fn, scratch_bytes, need);
+            rows = static_cast<float*>(scratch);
+        }
+    }
+    return launch_quantize((hipStream_t)stream, src, n_elems, n_per_row, t, out_blocks, with_imatrix ? imatrix : nullptr, rows);
+}
+
+int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row,
+                     hq_ggml_type t, void* out_blocks) {
+    return quantize_common("hq_quantize_ggml", stream, src, n_elems, n_per_row, t, out_blocks, nullptr, false, nullptr, 0);
+}
+
+size_t hq_quantize_ggml_imatrix_scratch_bytes(uint64_t n_elems, uint64_t n_per_row, hq_ggml_type t) {
+    if (t != HQ_Q4_0 || n_per_row == 0) return 0;
+    return (size_t)(n_elems / n_per_row) * sizeof(float);  // the mean square of every row
+}
+
+int hq_quantize_ggml_imatrix(void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row, hq_ggml_type t,
+                             const float* imatrix, void* out_blocks, void* scratch, size_t scratch_bytes) {
+    return quantize_common("hq_quantize_ggml_imatrix", stream, src, n_elems, n_per_row, t, out_blocks, imatrix, true, scratch, scratch_bytes);
 }
 
 static int check_matmul_common(const char* fn, const void* x, hq_act_dtype xdt, const void* w,

@@ -29,8 +29,10 @@ constexpr uint32_t Q4K_BYTES = 144, Q5K_BYTES = 176, Q6K_BYTES = 210, Q8_0_BYTES
 // ---- launchers (one per .hip file); all validate nothing: the C entry points do ----
 int launch_dequant(hipStream_t s, const void* w, void* out, hq_act_dtype odt, uint64_t n_elems,
                    hq_ggml_type t);
+// imatrix: nullptr, or n_per_row importance weights shared by every row; row_scratch: one float per row, used by Q4_0
+// with an importance matrix only.
 int launch_quantize(hipStream_t s, const float* src, uint64_t n_elems, uint64_t n_per_row,
-                    hq_ggml_type t, void* out);
+                    hq_ggml_type t, void* out, const float* imatrix = nullptr, float* row_scratch = nullptr);
 
 struct GemvArgs {
     const void* x;        // [x_rows, k] activations

@@ -1,7 +1,9 @@
-// Device-side GGML quantizers for Q4_K / Q6_K / Q8_0, byte-identical to hf2q's
-// CPU quantizers without an importance matrix
+// Device-side GGML quantizers for Q4_K / Q5_K / Q6_K / Q8_0 / Q4_0, byte-identical to hf2q's
+// CPU quantizers, without an importance matrix
 // (src/quantize/ggml_quants/q4_k.rs:89-217, q6_k.rs:40-151, q8_0.rs:31-72 and the
-// search helpers common.rs:61-167, 174-286).  hf2q quantizes on the host at
+// search helpers common.rs:61-167, 174-286) and with one (q4_k.rs:220-324, q5_k.rs:246-311,
+// q6_k.rs:40-151 with weights, q4_0.rs:52-87; helpers common.rs:294-408 make_qkx3_quants and
+// common.rs:415-518 make_qp_quants).  hf2q quantizes on the host at
 // conversion / load time (in_memory_loader.rs:70-139); here the same bytes are
 // produced on the GPU so that weights never have to cross PCIe as f32.
 //
@@ -74,10 +76,13 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restr
 // nmax = 15, rmin = -1, rdelta = 0.1, nstep = 20 (Q4_K, the arguments of q4_k.rs:120-132) or
 // nmax = 31, rmin = -0.5, rdelta = 0.1, nstep = 15 (Q5_K, q5_k.rs).
 // L comes back packed four codes per word.
-template <int nmax>
+// V3 = true is common.rs:294-408 make_qkx3_quants as the importance-matrix paths call it (q4_k.rs:262-274,
+// q5_k.rs:283-295): rmin = -0.9, rdelta = 0.05, nstep = 36, and the early return on max <= min.
+template <int nmax, bool V3 = false>
 __device__ float qkx2_search_32(const float (&x)[32], const float (&wt)[32], uint32_t (&Lp)[8], float& the_min) {
-    constexpr int nstep = nmax == 15 ? 20 : 15;
-    constexpr float rmin = nmax == 15 ? -1.f : -0.5f;
+    constexpr int nstep = V3 ? 36 : nmax == 15 ? 20 : 15;
+    constexpr float rmin = V3 ? -0.9f : nmax == 15 ? -1.f : -0.5f;
+    constexpr float rdelta = V3 ? 0.05f : 0.1f;
     float mn = x[0], mx = x[0];
     float sum_w = wt[0];
     float sum_x = sum_w * x[0];
@@ -91,7 +96,7 @@ __device__ float qkx2_search_32(const float (&x)[32], const float (&wt)[32], uin
     if (mn > 0.f) mn = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) Lp[i] = 0;
-    if (mx == mn) {
+    if (V3 ? (mx <= mn) : (mx == mn)) {
         the_min = -mn;
         return 0.f;
     }
@@ -108,7 +113,7 @@ __device__ float qkx2_search_32(const float (&x)[32], const float (&wt)[32], uin
         best_error = fmaf(wt[i], diff, best_error);
     }
     for (int is = 0; is <= nstep; ++is) {
-        iscale = (rmin + 0.1f * (float)is + (float)nmax) / (mx - mn);
+        iscale = (rmin + rdelta * (float)is + (float)nmax) / (mx - mn);
         float sum_l = 0.f, sum_l2 = 0.f, sum_xl = 0.f;
         uint32_t La[8];
 #pragma unroll
@@ -152,14 +157,90 @@ __device__ float qkx2_search_32(const float (&x)[32], const float (&wt)[32], uin
     return scale;
 }
 
+// common.rs:415-518 make_qp_quants with n = 8, nmax = 63: the eight sub-block scales (or mins) of a super-block against
+// their weights; the codes come back in L, the return value is the super-block's d (or dmin).
+__device__ float qp_quants_8(const float* x, const float* qw, uint32_t* L) {
+    constexpr int n = 8, nmax = 63;
+    float mx = 0.f;
+    for (int i = 0; i < n; ++i)
+        if (x[i] > mx) mx = x[i];
+    if (mx < kGroupMaxEps) {
+        for (int i = 0; i < n; ++i) L[i] = 0;
+        return 0.f;
+    }
+    float iscale = (float)nmax / mx;
+    for (int i = 0; i < n; ++i) L[i] = (uint32_t)nearest_int(iscale * x[i]) & 0xffu;
+    const float scale = 1.f / iscale;
+    float best_mse = 0.f;
+    for (int i = 0; i < n; ++i) {
+        const float diff = fmaf(scale, -(float)L[i], x[i]);
+        best_mse = fmaf(qw[i] * diff, diff, best_mse);
+    }
+    for (int is = -4; is <= 4; ++is) {
+        if (is == 0) continue;
+        const float iscale_is = (0.1f * (float)is + (float)nmax) / mx;
+        const float scale_is = 1.f / iscale_is;
+        float mse = 0.f;
+        for (int i = 0; i < n; ++i) {
+            int l = nearest_int(iscale_is * x[i]);
+            if (l > nmax) l = nmax;
+            const float diff = fmaf(scale_is, -(float)l, x[i]);
+            mse = fmaf(qw[i] * diff, diff, mse);
+        }
+        if (mse < best_mse) {
+            best_mse = mse;
+            iscale = iscale_is;
+        }
+    }
+    float sumlx = 0.f, suml2 = 0.f;
+    for (int i = 0; i < n; ++i) {
+        int l = nearest_int(iscale * x[i]);
+        if (l > nmax) l = nmax;
+        L[i] = (uint32_t)l & 0xffu;
+        const float w = qw[i];
+        sumlx = fmaf(w * x[i], (float)l, sumlx);
+        suml2 = fmaf(w * (float)l, (float)l, suml2);
+    }
+    for (int itry = 0; itry < 5; ++itry) {
+        int n_changed = 0;
+        for (int i = 0; i < n; ++i) {
+            const float w = qw[i];
+            const float cur_l = (float)L[i];
+            float slx = fmaf(w * x[i], -cur_l, sumlx);
+            float sl2 = fmaf(w * cur_l, -cur_l, suml2);
+            if (slx > 0.f && sl2 > 0.f) {
+                int new_l = nearest_int(x[i] * sl2 / slx);
+                if (new_l > nmax) new_l = nmax;
+                if (((uint32_t)new_l & 0xffu) != L[i]) {
+                    slx = fmaf(w * x[i], (float)new_l, slx);
+                    sl2 = fmaf(w * (float)new_l, (float)new_l, sl2);
+                    if (slx * slx * suml2 > sumlx * sumlx * sl2) {
+                        L[i] = (uint32_t)new_l & 0xffu;
+                        sumlx = slx;
+                        suml2 = sl2;
+                        ++n_changed;
+                    }
+                }
+            }
+        }
+        if (!n_changed) break;
+    }
+    return suml2 > 0.f ? sumlx / suml2 : 0.f;
+}
+
 // q4_k.rs:89-217 (Q5 = false) and its five-bit twin q5_k.rs (Q5 = true: codes 0..31, the fifth bit of every code
 // in qh, bit 2c for sub-block 2c and 2c + 1 for sub-block 2c + 1).  256 threads = 32 super-blocks x 8 sub-block
-// threads.
-template <bool Q5>
+// threads.  IM: the importance-matrix paths q4_k.rs:220-324 / q5_k.rs:246-311: `imatrix` holds one weight per column of
+// a row (n_per_row = 256 * blocks_per_row values); a sub-block's search weights are qw * sqrt(sigma2 + x^2) with sigma2
+// from the whole super-block, and the super-block's scale and min codes come from make_qp_quants over the eight
+// sub-blocks (one thread per super-block) instead of from the maxima.
+template <bool Q5, bool IM = false>
 __global__ __launch_bounds__(256) void quantize_q4_k_kernel(const float* __restrict__ src, uint8_t* __restrict__ out,
-                                                            uint64_t n_blocks) {
+                                                            uint64_t n_blocks, const float* __restrict__ imatrix = nullptr,
+                                                            uint32_t blocks_per_row = 1) {
     constexpr int NMAX = Q5 ? 31 : 15;
     __shared__ float s_scale[256], s_min[256];
+    __shared__ float s_sw[IM ? 256 : 1], s_d[IM ? 64 : 1];  // IM: sub-block weight sums; d and dmin per super-block
     __shared__ uint32_t s_code[256];   // ls | lm << 8 per sub-block
     __shared__ uint32_t s_L[256 * 8];  // packed codes of every sub-block (32 bytes each)
 
@@ -178,38 +259,83 @@ __global__ __launch_bounds__(256) void quantize_q4_k_kernel(const float* __restr
         x[4 * i + 2] = t.z;
         x[4 * i + 3] = t.w;
     }
-    float sum_x2 = 0.f;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) sum_x2 = fmaf(x[i], x[i], sum_x2);
-    const float av_x = sqrtf(sum_x2 / 32.f);
-#pragma unroll
-    for (int i = 0; i < 32; ++i) wt[i] = av_x + fabsf(x[i]);
-
     uint32_t Lp[8];
-    float the_min;
-    const float scale = qkx2_search_32<NMAX>(x, wt, Lp, the_min);
-    s_scale[tid] = scale;
-    s_min[tid] = the_min;
-    __syncthreads();
-
-    // Super-block maxima in sub-block order (strict > like the reference's scan).
-    float max_scale = 0.f, max_min = 0.f;
+    float the_min, scale;
+    uint32_t ls, lm, d16, dmin16;
+    if constexpr (IM) {
+        // sigma2 from the sum of squares of the whole super-block, in element order (q4_k.rs:240-241): every thread
+        // adds up all 256 for itself
+        float sum_x2 = 0.f;
+        const float4* b4 = reinterpret_cast<const float4*>(src + blk * 256);
+        for (int i = 0; i < 64; ++i) {
+            const float4 t = b4[i];
+            sum_x2 = fmaf(t.x, t.x, sum_x2);
+            sum_x2 = fmaf(t.y, t.y, sum_x2);
+            sum_x2 = fmaf(t.z, t.z, sum_x2);
+            sum_x2 = fmaf(t.w, t.w, sum_x2);
+        }
+        const float sigma2 = 2.f * sum_x2 / 256.f;
+        const float* qw = imatrix + (size_t)(blk % blocks_per_row) * 256 + 32 * j;
+        float sumw = 0.f;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        const float sc = s_scale[lb * 8 + t], mi = s_min[lb * 8 + t];
-        if (sc > max_scale) max_scale = sc;
-        if (mi > max_min) max_min = mi;
+        for (int i = 0; i < 32; ++i) {
+            wt[i] = qw[i] * sqrtf(sigma2 + x[i] * x[i]);
+            sumw += wt[i];
+        }
+        scale = qkx2_search_32<NMAX, true>(x, wt, Lp, the_min);
+        s_scale[tid] = scale;
+        s_min[tid] = the_min;
+        s_sw[tid] = sumw;
+        __syncthreads();
+        if (j == 0) {  // the super-block's codes and d / dmin: make_qp_quants over its eight sub-blocks (q4_k.rs:277-278)
+            uint32_t Ls[8], Lm[8];
+            const float d_blk = qp_quants_8(&s_scale[lb * 8], &s_sw[lb * 8], Ls);
+            const float dmin_blk = qp_quants_8(&s_min[lb * 8], &s_sw[lb * 8], Lm);
+            for (int t = 0; t < 8; ++t) {
+                const uint32_t a = Ls[t] > 63u ? 63u : Ls[t], b = Lm[t] > 63u ? 63u : Lm[t];
+                s_code[lb * 8 + t] = a | (b << 8);
+            }
+            s_d[lb * 2] = d_blk;
+            s_d[lb * 2 + 1] = dmin_blk;
+        }
+        __syncthreads();
+        ls = s_code[tid] & 0xffu;
+        lm = s_code[tid] >> 8;
+        d16 = f32_to_f16_bits(s_d[lb * 2]);
+        dmin16 = f32_to_f16_bits(s_d[lb * 2 + 1]);
+    } else {
+        float sum_x2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) sum_x2 = fmaf(x[i], x[i], sum_x2);
+        const float av_x = sqrtf(sum_x2 / 32.f);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) wt[i] = av_x + fabsf(x[i]);
+
+        scale = qkx2_search_32<NMAX>(x, wt, Lp, the_min);
+        s_scale[tid] = scale;
+        s_min[tid] = the_min;
+        __syncthreads();
+
+        // Super-block maxima in sub-block order (strict > like the reference's scan).
+        float max_scale = 0.f, max_min = 0.f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const float sc = s_scale[lb * 8 + t], mi = s_min[lb * 8 + t];
+            if (sc > max_scale) max_scale = sc;
+            if (mi > max_min) max_min = mi;
+        }
+        const float inv_scale = max_scale > 0.f ? 63.f / max_scale : 0.f;
+        const float inv_min = max_min > 0.f ? 63.f / max_min : 0.f;
+        ls = (uint32_t)nearest_int(inv_scale * scale) & 0xffu;  // `as u8` truncation
+        lm = (uint32_t)nearest_int(inv_min * the_min) & 0xffu;
+        ls = ls > 63u ? 63u : ls;
+        lm = lm > 63u ? 63u : lm;
+        s_code[tid] = ls | (lm << 8);
+        d16 = f32_to_f16_bits(max_scale / 63.f);
+        dmin16 = f32_to_f16_bits(max_min / 63.f);
     }
-    const float inv_scale = max_scale > 0.f ? 63.f / max_scale : 0.f;
-    const float inv_min = max_min > 0.f ? 63.f / max_min : 0.f;
-    uint32_t ls = (uint32_t)nearest_int(inv_scale * scale) & 0xffu;  // `as u8` truncation
-    uint32_t lm = (uint32_t)nearest_int(inv_min * the_min) & 0xffu;
-    ls = ls > 63u ? 63u : ls;
-    lm = lm > 63u ? 63u : lm;
-    s_code[tid] = ls | (lm << 8);
 
     // Second stage with the f16-rounded d / dmin (q4_k.rs:181-197).
-    const uint32_t d16 = f32_to_f16_bits(max_scale / 63.f), dmin16 = f32_to_f16_bits(max_min / 63.f);
     const float d = f16_bits_to_f32(d16) * (float)ls;
     if (d != 0.f) {
         const float dm = f16_bits_to_f32(dmin16) * (float)lm;
@@ -322,13 +448,14 @@ __global__ __launch_bounds__(256) void quantize_q4_0_kernel(const float* __restr
 }
 
 // ------------------------------------------------------------------ Q6_K
-// common.rs:61-167 make_qx_quants with n = 16, nmax = 32, rmse_type = 1, no
-// weights (q6_k.rs:58).  Codes come back as L = l + 32, one per byte.
-__device__ float qx_search_16(const float (&x)[16], uint32_t (&Lp)[4]) {
-    constexpr int nmax = 32;
+// common.rs:61-167 make_qx_quants with rmse_type = 1: n = 16, nmax = 32 for Q6_K (q6_k.rs:58; W: the sub-block's slice
+// of the importance matrix as the weights, else x^2), n = 32, nmax = 8 with weights for Q4_0's importance-matrix path
+// (q4_0.rs:75).  Codes come back as L = l + nmax, one per byte.
+template <int N, int nmax, bool W>
+__device__ float qx_search(const float (&x)[N], const float* qw, uint32_t (&Lp)[N / 4]) {
     float mx = 0.f, amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < N; ++i) {
         const float ax = fabsf(x[i]);
         if (ax > amax) {
             amax = ax;
@@ -336,16 +463,16 @@ __device__ float qx_search_16(const float (&x)[16], uint32_t (&Lp)[4]) {
         }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) Lp[i] = 0;
+    for (int i = 0; i < N / 4; ++i) Lp[i] = 0;
     if (amax < kGroupMaxEps) return 0.f;
     float iscale = -(float)nmax / mx;
     float sumlx = 0.f, suml2 = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < N; ++i) {
         int l = nearest_int(iscale * x[i]);
         l = max(-nmax, min(nmax - 1, l));
         Lp[i >> 2] |= (uint32_t)(l + nmax) << (8 * (i & 3));
-        const float w = x[i] * x[i];
+        const float w = W ? qw[i] : x[i] * x[i];
         sumlx = fmaf(w * x[i], (float)l, sumlx);
         suml2 = fmaf(w * (float)l, (float)l, suml2);
     }
@@ -356,19 +483,21 @@ __device__ float qx_search_16(const float (&x)[16], uint32_t (&Lp)[4]) {
         iscale = -((float)nmax + 0.1f * (float)is) / mx;
         sumlx = 0.f;
         suml2 = 0.f;
-        uint32_t La[4] = {0, 0, 0, 0};
+        uint32_t La[N / 4];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < N / 4; ++i) La[i] = 0;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
             int l = nearest_int(iscale * x[i]);
             l = max(-nmax, min(nmax - 1, l));
             La[i >> 2] |= (uint32_t)(l + nmax) << (8 * (i & 3));
-            const float w = x[i] * x[i];
+            const float w = W ? qw[i] : x[i] * x[i];
             sumlx = fmaf(w * x[i], (float)l, sumlx);
             suml2 = fmaf(w * (float)l, (float)l, suml2);
         }
         if (suml2 > 0.f && sumlx * sumlx > best * suml2) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) Lp[i] = La[i];
+            for (int i = 0; i < N / 4; ++i) Lp[i] = La[i];
             scale = sumlx / suml2;
             best = scale * sumlx;
         }
@@ -376,9 +505,55 @@ __device__ float qx_search_16(const float (&x)[16], uint32_t (&Lp)[4]) {
     return scale;
 }
 
+// Q4_0 with an importance matrix (q4_0.rs:52-87): sigma2 of a ROW = (sum of its squares, added in element order) / n_per_row,
+// one thread per row; then per block weights qw * sqrt(sigma2 + x^2) and make_qx_quants(32, 8, rmse_type 1).
+__global__ __launch_bounds__(64) void row_mean_square_kernel(const float* __restrict__ src, float* __restrict__ sigma2, uint64_t n_rows,
+                                                             uint64_t n_per_row) {
+    const uint64_t r = (uint64_t)blockIdx.x * 64 + threadIdx.x;
+    if (r >= n_rows) return;
+    const float* row = src + r * n_per_row;
+    float sum = 0.f;
+    for (uint64_t i = 0; i < n_per_row; ++i) sum += row[i] * row[i];
+    sigma2[r] = sum / (float)n_per_row;
+}
+__global__ __launch_bounds__(256) void quantize_q4_0_im_kernel(const float* __restrict__ src, uint8_t* __restrict__ out, uint64_t n_blocks,
+                                                               const float* __restrict__ imatrix, const float* __restrict__ sigma2,
+                                                               uint32_t blocks_per_row) {
+    const uint64_t b = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= n_blocks) return;
+    float x[32], wt[32];
+    const float4* s4 = reinterpret_cast<const float4*>(src + b * 32);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float4 t = s4[i];
+        x[4 * i] = t.x;
+        x[4 * i + 1] = t.y;
+        x[4 * i + 2] = t.z;
+        x[4 * i + 3] = t.w;
+    }
+    const float s2 = sigma2[b / blocks_per_row];
+    const float* qw = imatrix + (size_t)(b % blocks_per_row) * 32;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) wt[i] = qw[i] * sqrtf(s2 + x[i] * x[i]);
+    uint32_t Lp[8];
+    const float d = qx_search<32, 8, true>(x, wt, Lp);
+    uint8_t* o = out + b * Q4_0_BYTES;
+    *reinterpret_cast<uint16_t*>(o) = (uint16_t)f32_to_f16_bits(d);
+    // byte j = code j | code (j + 16) << 4: words 0..3 hold codes 0..15, words 4..7 codes 16..31
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t v = (Lp[w] & 0x0f0f0f0fu) | ((Lp[w + 4] & 0x0f0f0f0fu) << 4);
+        *reinterpret_cast<uint16_t*>(o + 2 + 4 * w) = (uint16_t)v;
+        *reinterpret_cast<uint16_t*>(o + 4 + 4 * w) = (uint16_t)(v >> 16);
+    }
+}
+
 // q6_k.rs:40-151.  256 threads = 16 super-blocks x 16 sub-block threads.
+// IM: the sub-block's sixteen importance-matrix values are the search weights (q6_k.rs:58-64).
+template <bool IM>
 __global__ __launch_bounds__(256) void quantize_q6_k_kernel(const float* __restrict__ src, uint8_t* __restrict__ out,
-                                                            uint64_t n_blocks) {
+                                                            uint64_t n_blocks, const float* __restrict__ imatrix = nullptr,
+                                                            uint32_t blocks_per_row = 1) {
     __shared__ float s_scale[256];
     __shared__ uint32_t s_L[256 * 4];  // 16 code bytes per sub-block = the 256 codes of a super-block in order
     __shared__ int s_sc[256];
@@ -399,7 +574,7 @@ __global__ __launch_bounds__(256) void quantize_q6_k_kernel(const float* __restr
         x[4 * i + 3] = t.w;
     }
     uint32_t Lp[4];
-    const float scale = qx_search_16(x, Lp);
+    const float scale = qx_search<16, 32, IM>(x, IM ? imatrix + (size_t)(blk % blocks_per_row) * 256 + 16 * ib : nullptr, Lp);
     s_scale[tid] = scale;
     __syncthreads();
 
@@ -473,29 +648,42 @@ __global__ __launch_bounds__(256) void quantize_q6_k_kernel(const float* __restr
 }  // namespace
 
 int launch_quantize(hipStream_t s, const float* src, uint64_t n_elems, uint64_t n_per_row, hq_ggml_type t,
-                    void* out) {
-    (void)n_per_row;  // rows are contiguous runs of whole blocks; no imatrix, so no per-row state
+                    void* out, const float* imatrix, float* row_scratch) {
     uint8_t* o = static_cast<uint8_t*>(out);
-    if (t == HQ_Q8_0) {
+    const bool im = imatrix != nullptr;
+    if (t == HQ_Q8_0) {  // (q8_0.rs:31-72 takes the importance matrix and does not use it)
         const uint64_t nb = n_elems / 32;
         if ((nb + 255) / 256 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
         hipLaunchKernelGGL(quantize_q8_0_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, src, o, nb);
-    } else if (t == HQ_Q4_K) {
+    } else if (t == HQ_Q4_K || t == HQ_Q5_K) {
         const uint64_t nb = n_elems / 256;
+        const uint32_t bpr = (uint32_t)(n_per_row / 256);
         if ((nb + 31) / 32 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
-        hipLaunchKernelGGL(quantize_q4_k_kernel<false>, dim3((unsigned)((nb + 31) / 32)), dim3(256), 0, s, src, o, nb);
-    } else if (t == HQ_Q5_K) {
-        const uint64_t nb = n_elems / 256;
-        if ((nb + 31) / 32 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
-        hipLaunchKernelGGL(quantize_q4_k_kernel<true>, dim3((unsigned)((nb + 31) / 32)), dim3(256), 0, s, src, o, nb);
+        const dim3 grid((unsigned)((nb + 31) / 32));
+        if (t == HQ_Q4_K) {
+            if (im) hipLaunchKernelGGL((quantize_q4_k_kernel<false, true>), grid, dim3(256), 0, s, src, o, nb, imatrix, bpr);
+            else hipLaunchKernelGGL((quantize_q4_k_kernel<false, false>), grid, dim3(256), 0, s, src, o, nb, nullptr, 1u);
+        } else {
+            if (im) hipLaunchKernelGGL((quantize_q4_k_kernel<true, true>), grid, dim3(256), 0, s, src, o, nb, imatrix, bpr);
+            else hipLaunchKernelGGL((quantize_q4_k_kernel<true, false>), grid, dim3(256), 0, s, src, o, nb, nullptr, 1u);
+        }
     } else if (t == HQ_Q4_0) {
         const uint64_t nb = n_elems / 32;
         if ((nb + 255) / 256 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
-        hipLaunchKernelGGL(quantize_q4_0_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, src, o, nb);
+        if (im) {
+            const uint64_t n_rows = n_elems / n_per_row;
+            hipLaunchKernelGGL(row_mean_square_kernel, dim3((unsigned)((n_rows + 63) / 64)), dim3(64), 0, s, src, row_scratch, n_rows, n_per_row);
+            if (int rc = check_launch("quantize row sums launch")) return rc;
+            hipLaunchKernelGGL(quantize_q4_0_im_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, src, o, nb, imatrix, row_scratch,
+                               (uint32_t)(n_per_row / 32));
+        } else {
+            hipLaunchKernelGGL(quantize_q4_0_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, src, o, nb);
+        }
     } else if (t == HQ_Q6_K) {
         const uint64_t nb = n_elems / 256;
         if ((nb + 15) / 16 > 0x7fffffffu) return fail(HQ_ERR_INVALID_ARGUMENT, "quantize: too many blocks");
-        hipLaunchKernelGGL(quantize_q6_k_kernel, dim3((unsigned)((nb + 15) / 16)), dim3(256), 0, s, src, o, nb);
+        if (im) hipLaunchKernelGGL(quantize_q6_k_kernel<true>, dim3((unsigned)((nb + 15) / 16)), dim3(256), 0, s, src, o, nb, imatrix, (uint32_t)(n_per_row / 256));
+        else hipLaunchKernelGGL(quantize_q6_k_kernel<false>, dim3((unsigned)((nb + 15) / 16)), dim3(256), 0, s, src, o, nb, nullptr, 1u);
     } else {
         return fail(HQ_ERR_UNSUPPORTED, "quantize: ggml type %d", (int)t);
     }

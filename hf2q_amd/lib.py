@@ -52,6 +52,8 @@ SIGNATURES = {
     "hq_block_bytes": (_u32, [_i32]),
     "hq_dequant_ggml": (_i32, [_vp, _vp, _vp, _i32, _u64, _i32]),
     "hq_quantize_ggml": (_i32, [_vp, _vp, _u64, _u64, _i32, _vp]),
+    "hq_quantize_ggml_imatrix_scratch_bytes": (_sz, [_u64, _u64, _i32]),
+    "hq_quantize_ggml_imatrix": (_i32, [_vp, _vp, _u64, _u64, _i32, _vp, _vp, _vp, _sz]),
     "hq_qmatmul_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32]),
     "hq_qmatmul_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),
     "hq_qmatmul_ggml_k_slices": (_i32, [_u32, _u32, _u32, _i32, _c.POINTER(_u32), _c.POINTER(_u32)]),

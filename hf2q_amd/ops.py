@@ -326,6 +326,24 @@ def dequantize_ggml(weight: torch.Tensor, n_elems: int, ggml_type: int,
     return out
 
 
+def _quantize_ggml_imatrix(src: torch.Tensor, n_per_row: int, ggml_type: int, imatrix: torch.Tensor) -> torch.Tensor:
+    if src.dtype != torch.float32 or imatrix.dtype != torch.float32:
+        raise TypeError("src and imatrix must be float32")
+    if imatrix.numel() != n_per_row:
+        raise ValueError("imatrix length must equal n_per_row")  # QuantizeError::ImatrixLenMismatch
+    n = src.numel()
+    be, bb = BLOCK_ELEMS[ggml_type], BLOCK_BYTES[ggml_type]
+    if n_per_row % be or n % n_per_row:
+        raise ValueError(f"n_per_row {n_per_row} / len {n} not aligned to block {be}")
+    L = _l.load()
+    out = torch.empty(n // be * bb, dtype=torch.uint8, device=src.device)
+    need = int(L.hq_quantize_ggml_imatrix_scratch_bytes(n, n_per_row, ggml_type))
+    scratch = torch.empty(need, dtype=torch.uint8, device=src.device) if need else None
+    _l.check(L.hq_quantize_ggml_imatrix(_stream(), _dev(src, "src"), n, n_per_row, ggml_type, _dev(imatrix, "imatrix"), _dev(out, "out"),
+                                        _dev(scratch, "scratch") if need else None, need))
+    return out
+
+
 def matmul_f16_shadow_workspace_bytes(m: int, n: int, k: int) -> int:
     return int(_l.load().hq_matmul_f16_shadow_workspace_bytes(m, n, k))
 
@@ -389,8 +407,11 @@ def stream_read_probe(buf: torch.Tensor, sink: torch.Tensor) -> None:
     _l.check(_l.load().hq_stream_read_probe(_stream(), _dev(buf, "buf"), buf.numel() * buf.element_size(), _dev(sink, "sink")))
 
 
-def quantize_ggml(src: torch.Tensor, n_per_row: int, ggml_type: int) -> torch.Tensor:
-    """f32 rows -> packed GGML blocks on the device (GgmlQuantizer::quantize without imatrix)."""
+def quantize_ggml(src: torch.Tensor, n_per_row: int, ggml_type: int, imatrix: torch.Tensor | None = None) -> torch.Tensor:
+    """f32 rows -> packed GGML blocks on the device (GgmlQuantizer::quantize, quantizer.rs:51-102); `imatrix`: n_per_row
+    float32 importance weights on the device, or None."""
+    if imatrix is not None:
+        return _quantize_ggml_imatrix(src, n_per_row, ggml_type, imatrix)
     if src.dtype != torch.float32:
         raise TypeError("src must be float32")
     n = src.numel()

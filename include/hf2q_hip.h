@@ -89,6 +89,15 @@ HQ_API int hq_dequant_ggml(void* stream, const void* w_blocks, void* out, hq_act
 HQ_API int hq_quantize_ggml(void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row,
                      hq_ggml_type t, void* out_blocks);
 
+/* The same with an importance matrix: GgmlQuantizer::quantize(src, n_per_row, Some(imatrix))
+ * (quantizer.rs:51-102 -> q4_k.rs:220-324, q5_k.rs:246-311, q6_k.rs:40-151 with weights, q4_0.rs:52-87; Q8_0 takes the
+ * argument and does not use it, q8_0.rs:31-72), byte-identical to the CPU quantizers.  `imatrix`: n_per_row f32 weights
+ * in device memory, one per column, shared by every row.  `scratch`: hq_quantize_ggml_imatrix_scratch_bytes() bytes of
+ * device memory (Q4_0: one float per row for the row's mean square; 0 for the other types, `scratch` may then be null). */
+HQ_API size_t hq_quantize_ggml_imatrix_scratch_bytes(uint64_t n_elems, uint64_t n_per_row, hq_ggml_type t);
+HQ_API int hq_quantize_ggml_imatrix(void* stream, const float* src, uint64_t n_elems, uint64_t n_per_row, hq_ggml_type t,
+                             const float* imatrix, void* out_blocks, void* scratch, size_t scratch_bytes);
+
 /* dst[m,n] = x[m,k] . W[n,k]^T with W stored as GGML blocks, row-major
  * [n][k/QK]; fp32 accumulate, f32 output.  Replaces
  * mlx_native quantized_matmul_ggml(encoder, registry, device, input, weight,

@@ -218,6 +218,66 @@ def test_quantizer_byte_equal_to_oracle(oracle, dev, t):
     assert bad.size == 0, f"{bad.size} blocks differ, first {bad[:5]}"
 
 
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_imatrix_quantizer_matches_reference_golden_bytes(oracle, dev, t):
+    """The reference's importance-matrix fixtures (q4_k.rs:395-403, q6_k.rs:281-289, q8_0.rs:115-125, q5_k.rs, q4_0.rs): the
+    same inputs, the mulberry32 weights of the reference's tests (ones for Q8_0), byte equality with the `_im_` files."""
+    import os
+    from _util import GOLDEN
+    name, npr = {HQ_Q4_K: ("q4_k_512", 512), HQ_Q6_K: ("q6_k_512", 512), HQ_Q8_0: ("q8_0_64", 64),
+                 HQ_Q5_K: ("q5_k_512", 512), HQ_Q4_0: ("q4_0_64", 64)}[t]
+    x = np.fromfile(os.path.join(GOLDEN, "ggml_quants", f"{name}_im_input.bin"), dtype=np.float32)
+    want = np.fromfile(os.path.join(GOLDEN, "ggml_quants", f"{name}_im_expected.bin"), dtype=np.uint8)
+    im = np.ones(npr, np.float32) if t == HQ_Q8_0 else oracle.mulberry32_imatrix(npr, 2)
+    got = ops.quantize_ggml(torch.from_numpy(x).to(dev), npr, t, imatrix=torch.from_numpy(im).to(dev)).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_imatrix_quantizer_byte_equal_to_oracle(oracle, dev, t):
+    """Rows of several blocks (the weights of a column depend on its place in the row), the distributions of the plain
+    quantizer's test, importance weights over four decades with some zeros; Q4_0's weights also depend on the whole row."""
+    rng = np.random.default_rng(140 + t)
+    npr = 1024
+    parts = [
+        (rng.standard_normal(96 * npr) * 0.02).astype(np.float32),
+        rng.uniform(-1, 1, 12 * npr).astype(np.float32),
+        (rng.standard_normal(12 * npr) ** 3).astype(np.float32),
+        np.zeros(npr, np.float32), np.full(npr, 0.37, np.float32), np.full(npr, -1e-3, np.float32),
+        (rng.standard_normal(2 * npr) * 1e-18).astype(np.float32),
+        (rng.standard_normal(2 * npr) * 3e4).astype(np.float32),
+        np.abs(rng.standard_normal(2 * npr)).astype(np.float32),
+        np.where(rng.random(2 * npr) < 0.9, 0, rng.standard_normal(2 * npr)).astype(np.float32),
+    ]
+    x = np.concatenate(parts)
+    for im in (oracle.mulberry32_imatrix(npr, 7),
+               (10.0 ** rng.uniform(-2, 2, npr) * (rng.random(npr) > 0.05)).astype(np.float32)):
+        want = oracle.quantize(x, npr, t, im, threads=8)
+        got = ops.quantize_ggml(torch.from_numpy(x).to(dev), npr, t, imatrix=torch.from_numpy(im).to(dev)).cpu().numpy()
+        bb = oracle.BLOCK_BYTES[t]
+        bad = np.nonzero((got.reshape(-1, bb) != want.reshape(-1, bb)).any(axis=1))[0]
+        assert bad.size == 0, f"{bad.size} blocks differ, first {bad[:5]}"
+    if t != HQ_Q8_0:  # the importance matrix matters: not the bytes of the plain quantizer
+        assert not np.array_equal(got, ops.quantize_ggml(torch.from_numpy(x).to(dev), npr, t).cpu().numpy())
+
+
+def test_imatrix_quantizer_rejects_bad_arguments(dev):
+    x = torch.zeros(1024, device=dev)
+    with pytest.raises(ValueError):
+        ops.quantize_ggml(x, 512, HQ_Q4_K, imatrix=torch.ones(256, device=dev))  # ImatrixLenMismatch (quantizer.rs:72-80)
+    import ctypes
+    from hf2q_amd import lib
+    L = lib.load()
+    out = torch.empty(1024 // 32 * 18, dtype=torch.uint8, device=dev)
+    im = torch.ones(512, device=dev)
+    assert L.hq_quantize_ggml_imatrix_scratch_bytes(1024, 512, HQ_Q4_0) == 8
+    assert L.hq_quantize_ggml_imatrix_scratch_bytes(1024, 512, HQ_Q4_K) == 0
+    rc = L.hq_quantize_ggml_imatrix(None, x.data_ptr(), 1024, 512, HQ_Q4_0, im.data_ptr(), out.data_ptr(), None, 0)
+    assert rc == lib.HQ_ERR_INVALID_ARGUMENT  # Q4_0 needs its row scratch
+    rc = L.hq_quantize_ggml_imatrix(None, x.data_ptr(), 1024, 512, HQ_Q4_K, None, out.data_ptr(), None, 0)
+    assert rc == lib.HQ_ERR_INVALID_ARGUMENT  # no imatrix
+
+
 def test_quantizer_rejects_bad_shapes(dev):
     # quantizer.rs:217-235
     x = torch.zeros(768, device=dev)
