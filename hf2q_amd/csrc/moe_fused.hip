@@ -44,10 +44,11 @@ template <int TYPE>
 constexpr uint32_t kRowBytesH = FH / 256 * kBlockBytes<TYPE>;  // bytes of a gate / up row
 template <int TYPE>
 constexpr uint32_t kRowBytesI = FI / 256 * kBlockBytes<TYPE>;  // bytes of a down row
-constexpr uint32_t WAVES = 8, THREADS = 64 * WAVES;
 constexpr uint32_t MAX_T = 8;                         // tokens per call
-constexpr int RING = 4;                               // weight fetches a wave keeps in flight
-constexpr int POLL = 5;  // activation loads of a thread per polling pass: (8 + 1) slots x 512 / 2 words over 512 threads = 4.5
+// Two shapes of workgroup (template arguments WAVES_, RING_ of the kernel): 8 waves with four weight fetches in flight
+// each -- one token: the phases are round trips, few rows per wave -- and 12 waves with two -- several tokens: the
+// phases are bound by VALU issue, and three waves per SIMD keep it a little busier than two (16 waves leave 128
+// registers per lane and spill 60 .. 200 of them).
 // A logit is stored LG_COPIES times and a workgroup polls copy (its index among its token's workgroups) % LG_COPIES: at
 // one token 256 workgroups would otherwise poll the same 2 KB (sixteen cache lines, a few memory channels).
 constexpr uint32_t LG_COPIES = 8;
@@ -114,8 +115,12 @@ __device__ __forceinline__ uint32_t act_run(uint32_t li, uint32_t r) {
     return li * 16u + 4u * r;
 }
 
-template <int TG, int TD>  // types of gate / up and of down
-__global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
+template <int TG, int TD, int WAVES_, int RING_>  // types of gate / up and of down; waves per workgroup; fetches in flight per wave
+__global__ __launch_bounds__(64 * WAVES_) void moe_fused_kernel(FusedArgs a) {
+    constexpr uint32_t WAVES = WAVES_, THREADS = 64 * WAVES;
+    constexpr int RING = RING_;
+    // activation loads of a thread per polling pass: (8 + 1) slots x 512 / 2 words = 4.5 per thread of 512, 2.25 of 1024
+    constexpr int POLL = WAVES_ == 8 ? 5 : 3;
     constexpr uint32_t ROWB_H = kRowBytesH<TG>, ROWB_I = kRowBytesI<TD>;
     extern __shared__ uint4 smem[];
     const Layout L{a.T, a.E, a.K};
@@ -338,7 +343,7 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
     // ---- phases 3 + 4: unit (token t, column slice c): the down rows of the slice for every slot of the token, then
     // the weighted sum over the slots in slot order, the shared expert last (the order of moe_weighted_reduce_kernel) ----
     {
-        constexpr int RD = TD == HQ_Q5_K ? 3 : RING;  // (a ring of four Q5_K pieces beside the 64 activations spills)
+        constexpr int RD = TD == HQ_Q5_K && RING > 3 ? 3 : RING;  // (a ring of four Q5_K pieces beside the 64 activations spills)
         const uint32_t li = lane & 7u, sub = lane >> 3;
         const int c4 = (int)(li & 3u);
         const uint32_t groups = T <= 1 ? 1u : T <= 2 ? 2u : T <= 4 ? 4u : 8u, cols = 8u * groups;  // columns per unit: about one unit per workgroup
@@ -390,6 +395,8 @@ __global__ __launch_bounds__(THREADS) void moe_fused_kernel(FusedArgs a) {
                         // the results exist once the counter has drained; naming them keeps their uses below the wait
                         if constexpr (POLL == 5)
                             asm volatile("s_waitcnt vmcnt(0)" : "+v"(got[0]), "+v"(got[1]), "+v"(got[2]), "+v"(got[3]), "+v"(got[4]) : : "memory");
+                        else
+                            asm volatile("s_waitcnt vmcnt(0)" : "+v"(got[0]), "+v"(got[1]), "+v"(got[2]) : : "memory");
                         bool fresh = true;
 #pragma unroll
                         for (int i = 0; i < POLL; ++i) {
@@ -490,13 +497,18 @@ size_t moe_fused_scratch_bytes(uint32_t n_tokens, uint32_t n_experts, uint32_t t
 namespace {
 // The kernel instantiated for (gate / up type, down type), or null: one K-quant for all three, or Q4_K / Q5_K gate / up
 // with a Q6_K down.
-void (*fused_kernel_for(hq_ggml_type t, hq_ggml_type td))(FusedArgs) {
-    if (t == HQ_Q4_K && td == HQ_Q4_K) return moe_fused_kernel<HQ_Q4_K, HQ_Q4_K>;
-    if (t == HQ_Q5_K && td == HQ_Q5_K) return moe_fused_kernel<HQ_Q5_K, HQ_Q5_K>;
-    if (t == HQ_Q6_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q6_K, HQ_Q6_K>;
-    if (t == HQ_Q4_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q4_K, HQ_Q6_K>;
-    if (t == HQ_Q5_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q5_K, HQ_Q6_K>;
+template <int W, int R>
+void (*fused_kernel_of(hq_ggml_type t, hq_ggml_type td))(FusedArgs) {
+    if (t == HQ_Q4_K && td == HQ_Q4_K) return moe_fused_kernel<HQ_Q4_K, HQ_Q4_K, W, R>;
+    if (t == HQ_Q5_K && td == HQ_Q5_K) return moe_fused_kernel<HQ_Q5_K, HQ_Q5_K, W, R>;
+    if (t == HQ_Q6_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q6_K, HQ_Q6_K, W, R>;
+    if (t == HQ_Q4_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q4_K, HQ_Q6_K, W, R>;
+    if (t == HQ_Q5_K && td == HQ_Q6_K) return moe_fused_kernel<HQ_Q5_K, HQ_Q6_K, W, R>;
     return nullptr;
+}
+// wide: the 12-wave form
+void (*fused_kernel_for(hq_ggml_type t, hq_ggml_type td, bool wide = false))(FusedArgs) {
+    return wide ? fused_kernel_of<12, 2>(t, td) : fused_kernel_of<8, 4>(t, td);
 }
 }  // namespace
 
@@ -531,7 +543,10 @@ int launch_moe_fused(hipStream_t s, const MoeFusedArgs& m) {
     a.m2 = m.t_gate_up == HQ_Q5_K ? M1 : m.t_gate_up == HQ_Q6_K ? N2 : M2;
     a.magic = MAGIC;
     a.spin_limit = m.spin_limit ? m.spin_limit : (1u << 20);
-    auto kern = fused_kernel_for(m.t_gate_up, m.t_down);
+    // from two tokens on the 12-wave form (17.8 / 22.5 / 34.3 us at 2 / 4 / 8 tokens against 19.0 / 24.2 / 34.8; one token: the same)
+    const bool wide = m.n_tokens >= 2u;
+    const uint32_t WAVES = wide ? 12u : 8u, THREADS = 64u * WAVES;
+    auto kern = fused_kernel_for(m.t_gate_up, m.t_down, wide);
     if (!kern) return fail(HQ_ERR_UNSUPPORTED, "fused MoE block: gate / up type %d with down type %d", (int)m.t_gate_up, (int)m.t_down);
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
