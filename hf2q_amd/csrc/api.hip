@@ -715,8 +715,8 @@ int hq_matmul_f16_shadow(void* stream, const void* x, hq_act_dtype xdt, const vo
     if (xdt != HQ_F32 && xdt != HQ_BF16) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: activation dtype %d", fn, (int)xdt);
     if (k == 0 || k % 8) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: k = %u is not a positive multiple of 8", fn, k);
     if (!x || !w_f16 || !y || !workspace) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
-    if (!is_aligned(x, 16) || !is_aligned(w_f16, 16) || !is_aligned(y, 16) || !is_aligned(workspace, 16))
-        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: x, w_f16, y and workspace must be 16-byte aligned", fn);
+    if (!is_aligned(x, 16) || !is_aligned(w_f16, 16) || !is_aligned(y, 16) || !is_aligned(workspace, 256))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: x, w_f16 and y must be 16-byte aligned, workspace 256-byte aligned", fn);
     const size_t need = f16_shadow_workspace_bytes(m, k);
     if (workspace_bytes < need) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes, %zu needed", fn, workspace_bytes, need);
     return launch_f16_shadow_matmul((hipStream_t)stream, x, xdt, w_f16, y, m, n, k, workspace, need);

@@ -576,7 +576,7 @@ HQ_API int hq_tq_kv_restore(void* stream, const void* payload, size_t len, uint8
  * dispatch_mm_v2_f16, F16 weight x F32 input -> F32 output; the shadow itself: materialize_f16_shadow, :9426-9440).
  * Memory for speed: 2 bytes per weight instead of 0.56 - 1.06, no dequantisation inside the product.  x: [m][k] f32 or
  * bf16, cast to f16 (round to nearest even) by a kernel of this library; the product is the vendor library's dense GEMM
- * (hipBLASLt) with f32 accumulation.  k % 8 == 0; x, w_f16, y and `workspace` 16-byte aligned; `workspace`:
+ * (hipBLASLt) with f32 accumulation.  k % 8 == 0; x, w_f16 and y 16-byte aligned; `workspace` 256-byte aligned:
  * hq_matmul_f16_shadow_workspace_bytes() bytes of device memory (the f16 activations + what the vendor library may use).
  * The first call for a shape asks the vendor library for its kernel (host time, not capturable in a HIP graph); later
  * calls of that shape only launch. */
