@@ -1297,7 +1297,12 @@ template <int TYPE, int MT, bool SWIGLU = false>
 __global__ __launch_bounds__(64 * WAVES, 2) void grouped_gemm_kernel(GemmArgs a, const uint4* __restrict__ tiles,
                                                                       const uint32_t* __restrict__ n_tiles, uint32_t tiles_n,
                                                                       uint64_t expert_stride) {
-    const uint32_t t = blockIdx.x / tiles_n, n0 = (blockIdx.x % tiles_n) * BN_WIDE;
+    // Workgroups go to the XCDs in turn (workgroup b to XCD b % 8), and every XCD has an L2 of its own: the tiles_n
+    // workgroups that multiply the same routed rows with different weight rows are b = 8 (tiles_n q + i) + x for
+    // i = 0 .. tiles_n - 1, all on XCD x and dispatched together, so the gathered activation rows cross the fabric
+    // once instead of once per weight-row tile.
+    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+    const uint32_t t = (slot / tiles_n) * 8u + xcd, n0 = (slot % tiles_n) * BN_WIDE;
     if (t >= *n_tiles) return;
     const uint4 tt = tiles[t];
     a.w += (size_t)tt.x * expert_stride;
@@ -1440,7 +1445,7 @@ static int launch_grouped_t(hipStream_t s, const void* x, hq_act_dtype xdt, cons
                w_scales ? w_scales : ws_scales, wb2, wb2 ? (w_scales ? w_scales2 : ws_scales + n_rows) : nullptr};
     const uint32_t tiles_n = (n + bn - 1) / bn;
     const uint32_t max_tiles = pairs / bm + n_experts;
-    hipLaunchKernelGGL(kern, dim3(max_tiles * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
+    hipLaunchKernelGGL(kern, dim3(((max_tiles + 7u) & ~7u) * tiles_n), dim3(64 * WAVES), lds, s, a, tiles, n_tiles, tiles_n, expert_stride);
     return check_launch("grouped gemm kernel launch");
 }
 
