@@ -55,7 +55,7 @@ PMC_TRAFFIC_BYTES = {
     "prefill_gemm_q8_0_2048x12288x4096": int((232529.5 + 68804.0 / 2.0) * 2.0 * 1024 + (98572.3 + 16464.2) * 1.0 * 1024),
     # grouped mul_mat_id, 2048 tokens x top-8 over 256 experts of 512 x 2048 Q4_K: pre-pass (sort, conversion, scan of the stack's
     # headers) + grouped tile GEMM (bench.py --workload moe_prefill --step-only)
-    "moe_prefill_gate_up_2048x8": int((163244.4 + 69718.9) * 2.0 * 1024 + (32887.6 + 8788.0) * 1.0 * 1024),
+    "moe_prefill_gate_up_2048x8": int((106321.0 + 69719.0) * 2.0 * 1024 + (32940.8 + 8788.0) * 1.0 * 1024),
 }
 
 
