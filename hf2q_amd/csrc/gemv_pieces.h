@@ -9,7 +9,7 @@
 namespace hq {
 namespace {
 
-constexpr uint32_t M4 = 0x000f000fu, M2 = 0x00300030u, M1 = 0x00100010u, MAGIC = 0x43004300u;
+constexpr uint32_t M4 = 0x000f000fu, M2 = 0x00300030u, M1 = 0x10101010u, MAGIC = 0x43004300u;
 constexpr uint32_t N4 = 0x0f0f0f0fu, N2 = 0x30303030u;  // the Q6_K kernels work on four bytes at a time
 // Types whose block is one lane's piece of 32 weights (the K-quants give a lane 64 of a super-block's 256).
 template <int TYPE>
@@ -108,19 +108,24 @@ __device__ __forceinline__ float dot_pair(const Piece<HQ_Q4_K>& p, int c, const 
     return acc;
 }
 
-// Q5_K: the fifth bit of element j of sub-blocks 2c / 2c+1 is bit 2c / 2c+1 of high-bit byte j; m1 = 0x00100010
-// arrives in the second mask register.  Values hold 128 + q with q in 0..31.
+// Q5_K: the fifth bit of element j of sub-blocks 2c / 2c+1 is bit 2c / 2c+1 of high-bit byte j.  Four 5-bit values at a
+// time as the bytes of one word (m1 = 0x10101010 arrives in the second mask register), then two byte permutes put bytes
+// (0, 2) and (1, 3) under the high byte 0x43 of `magic`: bf16 128 + q with q in 0..31, the pair order of the staged
+// activations.
 __device__ __forceinline__ float dot_pair(const Piece<HQ_Q5_K>& p, int c, const uint32_t* xp, const float* sx,
-                                          uint32_t m4, uint32_t m1, uint32_t magic) {
+                                          uint32_t, uint32_t m1, uint32_t magic) {
     float lo = 0.f, hi = 0.f;
+    constexpr uint32_t SEL02 = 0x07020500u, SEL13 = 0x07030501u;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const uint32_t w = j < 4 ? word(p.q0, j) : word(p.q1, j - 4);
         const uint32_t hs = (j < 4 ? word(p.h0, j) : word(p.h1, j - 4)) >> (2 * c);
-        lo = dot2_bf16(and_or(hs << 4, m1, (w & m4) | magic), xp[2 * j], lo);
-        lo = dot2_bf16(and_or(hs >> 4, m1, ((w >> 8) & m4) | magic), xp[2 * j + 1], lo);
-        hi = dot2_bf16(and_or(hs << 3, m1, ((w >> 4) & m4) | magic), xp[16 + 2 * j], hi);
-        hi = dot2_bf16(and_or(hs >> 5, m1, ((w >> 12) & m4) | magic), xp[16 + 2 * j + 1], hi);
+        const uint32_t ql = and_or(hs << 4, m1, w & 0x0f0f0f0fu);
+        const uint32_t qh = and_or(hs << 3, m1, (w >> 4) & 0x0f0f0f0fu);
+        lo = dot2_bf16(__builtin_amdgcn_perm(magic, ql, SEL02), xp[2 * j], lo);
+        lo = dot2_bf16(__builtin_amdgcn_perm(magic, ql, SEL13), xp[2 * j + 1], lo);
+        hi = dot2_bf16(__builtin_amdgcn_perm(magic, qh, SEL02), xp[16 + 2 * j], hi);
+        hi = dot2_bf16(__builtin_amdgcn_perm(magic, qh, SEL13), xp[16 + 2 * j + 1], hi);
     }
     uint32_t sc0, sc1, m0, mn1;
     q4k_scales(p.hdr.y, p.hdr.z, p.hdr.w, c, sc0, sc1, m0, mn1);

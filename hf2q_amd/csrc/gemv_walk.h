@@ -31,32 +31,41 @@ struct FlatGeom {
     uint32_t magic;  // ceil(2^32 / bu): v / bu == umulhi(v, magic) while v * bu < 2^32
     uint32_t log_r;  // a super-task is 1 << log_r rows ...
     uint32_t st;     // ... = st windows ...
-    uint32_t uwe;    // ... of uwe <= UW units each (the lanes past uwe * lanes-per-unit idle)
+    uint32_t uwe;    // ... of uwe <= UW units each (the lanes past uwe * lanes-per-unit idle); the last window of a
+                     // super-task may be ragged (st * uwe > the super-task's units): its lanes past the end idle too
 };
 
 // The window width and the rows per super-task for a matrix of n rows (nm matrices walked side by side) on `waves` waves.
 // Full windows (uwe = uw) waste no lane but tie R = uw / gcd(bu, uw) rows together, which leaves waves without work when
 // n / R is small (k = 2816: 11 super-blocks per row, R = 16); narrower windows that divide R * bu for a smaller R (11 of 16
-// units: one row per window) spread the rows over more waves at the price of idle lanes.  Chosen: the pair with the fewest
-// windows on the busiest wave, then the fewest windows in all.
+// units: one row per window) spread the rows over more waves at the price of idle lanes.  Chosen: the pair with the smallest
+// sum of the windows on the busiest wave and the windows per wave on average.
 inline FlatGeom flat_geom(uint32_t k, uint32_t unit_elems, uint32_t uw, uint32_t n, uint32_t nm, uint32_t waves) {
     FlatGeom g{};
     g.bu = k / unit_elems;
     g.magic = (uint32_t)((0x100000000ull + g.bu - 1) / g.bu);  // bu >= 2
-    uint64_t best_crit = ~0ull, best_total = ~0ull;
+    uint64_t best = ~0ull;
     for (uint32_t log_r = 0; (1u << log_r) <= uw; ++log_r) {
         const uint32_t r = 1u << log_r;
         uint32_t uwe = uw;
         while ((r * g.bu) % uwe) --uwe;
-        const uint32_t st = r * g.bu / uwe;
-        const uint64_t n_super = (n + r - 1) / r;
-        const uint64_t crit = ((n_super + waves - 1) / waves) * nm * st, total = n_super * nm * st;
-        if (crit < best_crit || (crit == best_crit && total < best_total)) {
-            best_crit = crit;
-            best_total = total;
-            g.log_r = log_r;
-            g.st = st;
-            g.uwe = uwe;
+        // the widest window that divides the super-task, and full windows with a ragged last one (68 super-blocks per row:
+        // windows of 16, 16, 16, 16 and 4 where the divisors offer 4 per row or 17 windows of 16 for four rows)
+        for (int ragged = 0; ragged < 2; ++ragged) {
+            if (ragged && uwe == uw) break;
+            const uint32_t w = ragged ? uw : uwe;
+            const uint32_t st = (r * g.bu + w - 1) / w;
+            const uint64_t n_super = (n + r - 1) / r;
+            const uint64_t crit = ((n_super + waves - 1) / waves) * nm * st, total = n_super * nm * st;
+            // windows of the busiest wave + windows per wave on average: the first bounds the time when waves run short
+            // of work, the second when the device is busy throughout (a ragged window's idle lanes cost their arithmetic)
+            const uint64_t score = crit * waves + total;
+            if (score < best) {
+                best = score;
+                g.log_r = log_r;
+                g.st = st;
+                g.uwe = w;
+            }
         }
     }
     return g;
@@ -263,7 +272,9 @@ struct FlatWalk {
 
     __device__ __forceinline__ void fetch_next(Piece<TYPE>& p) {
         const uint32_t sid = seq_first + f_q * seq_stride;
-        uint32_t u = (sid << g.log_r) * g.bu + g.uwe * f_w + lv;
+        // (a ragged last window: the lanes past the super-task's end fetch its last unit again)
+        const uint32_t wu = g.uwe * f_w + lv, su = g.bu << g.log_r;
+        uint32_t u = (sid << g.log_r) * g.bu + (wu < su ? wu : su - 1u);
         const uint32_t last = nrows * g.bu - 1u;
         u = u < last ? u : last;
         const uint8_t* base = f_m ? w1 : w0;
@@ -327,7 +338,9 @@ struct FlatWalk {
 #pragma unroll
             for (int d = 0; d < D; ++d) {
                 Piece<TYPE>& p = buf[d];
-                const uint32_t lu = g.uwe * c_w + lv;
+                const uint32_t lu_raw = g.uwe * c_w + lv, su = g.bu << g.log_r;
+                const bool in_task = lu_raw < su;  // false only in the idle part of a ragged last window
+                const uint32_t lu = in_task ? lu_raw : su - 1u;
                 uint32_t lrow = __umulhi(lu, g.magic);
                 const uint32_t ur = lu - lrow * g.bu;
                 float part;
@@ -353,7 +366,7 @@ struct FlatWalk {
                 if (one_row) {
                     // every window of the super-task belongs to its one row: the lanes add their windows up and meet once
                     // (the order of sums of the aligned streaming kernel: the same bits)
-                    acc += active && live ? part : 0.f;
+                    acc += active && in_task && live ? part : 0.f;
                     if (live && c_w + 1u == g.st) {
                         const float v = group_sum(acc, 6);
                         acc = 0.f;
@@ -365,7 +378,7 @@ struct FlatWalk {
                 } else {
                     const uint32_t r_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)lrow);
                     const uint32_t r_hi = (uint32_t)__builtin_amdgcn_readlane((int)lrow, last_lane);
-                    lrow = active ? lrow : 0xffffffffu;  // an idle lane's duplicate belongs to no row
+                    lrow = active && in_task ? lrow : 0xffffffffu;  // an idle lane's duplicate belongs to no row
                     for (uint32_t r = r_lo; r <= r_hi; ++r) {
                         float v = lrow == r ? part : 0.f;
                         v = group_sum(v, 6);
