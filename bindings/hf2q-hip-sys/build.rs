@@ -13,6 +13,7 @@ use std::process::Command;
 const SOURCES: &[&str] = &[
     "api.hip",
     "blocks.hip",
+    "dense.hip",
     "dense_ffn.hip",
     "dequant.hip",
     "gemm.hip",

@@ -211,6 +211,8 @@ extern "C" {
     pub fn hq_tq_kv_restore(stream: *mut c_void, payload: *const c_void, len: usize, codes: *mut u8, norms: *mut f32, n_kv_heads: u32, head_dim: u32, capacity: u32, start_pos: u32) -> c_int;
     pub fn hq_matmul_f16_shadow_workspace_bytes(m: u32, n: u32, k: u32) -> usize;
     pub fn hq_matmul_f16_shadow(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_f16: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
+    pub fn hq_dense_matmul_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, wdt: hq_act_dtype) -> usize;
+    pub fn hq_dense_matmul(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w: *const c_void, wdt: hq_act_dtype, y: *mut f32, m: u32, n: u32, k: u32, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
     pub fn hq_stream_read_probe(stream: *mut c_void, buf: *const c_void, bytes: usize, sink: *mut u32) -> c_int;
     pub fn hq_gguf_open(path: *const c_char, out: *mut *mut hq_gguf) -> c_int;
     pub fn hq_gguf_close(g: *mut hq_gguf);

@@ -722,6 +722,32 @@ int hq_matmul_f16_shadow(void* stream, const void* x, hq_act_dtype xdt, const vo
     return launch_f16_shadow_matmul((hipStream_t)stream, x, xdt, w_f16, y, m, n, k, workspace, need);
 }
 
+// Rows that take the GEMV of dense.hip (the reference's matvec kernels serve m = 1; a few rows are as many passes).
+static bool dense_rows_as_gemv(uint32_t m, uint32_t k, hq_act_dtype wdt) { return m <= kGemvMaxRows && dense_gemv_takes(k, wdt); }
+
+size_t hq_dense_matmul_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_act_dtype wdt) {
+    if (m == 0 || n == 0 || k == 0 || (wdt != HQ_F16 && wdt != HQ_F32) || dense_rows_as_gemv(m, k, wdt)) return 0;
+    return wdt == HQ_F16 ? f16_shadow_workspace_bytes(m, k) : f32_dense_workspace_bytes(m, k, xdt);
+}
+
+int hq_dense_matmul(void* stream, const void* x, hq_act_dtype xdt, const void* w, hq_act_dtype wdt, float* y, uint32_t m, uint32_t n,
+                    uint32_t k, void* workspace, size_t workspace_bytes) {
+    const char* fn = "hq_dense_matmul";
+    if (m == 0 || n == 0) return HQ_OK;
+    if (xdt != HQ_F32 && xdt != HQ_BF16) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: activation dtype %d", fn, (int)xdt);
+    if (wdt != HQ_F32 && wdt != HQ_F16) return fail(HQ_ERR_UNSUPPORTED, "%s: weight dtype %d (f32 or f16)", fn, (int)wdt);
+    if (k == 0 || k % 8) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: k = %u is not a positive multiple of 8", fn, k);
+    if (!x || !w || !y) return fail(HQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+    if (!is_aligned(x, 16) || !is_aligned(w, 16) || !is_aligned(y, 16))
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: x, w and y must be 16-byte aligned", fn);
+    if (dense_rows_as_gemv(m, k, wdt)) return launch_dense_gemv((hipStream_t)stream, x, xdt, w, wdt, y, m, n, k);
+    const size_t need = hq_dense_matmul_workspace_bytes(m, n, k, xdt, wdt);
+    if (!workspace || !is_aligned(workspace, 256) || workspace_bytes < need)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes (256-byte aligned), %zu needed", fn, workspace ? workspace_bytes : (size_t)0, need);
+    if (wdt == HQ_F16) return launch_f16_shadow_matmul((hipStream_t)stream, x, xdt, w, y, m, n, k, workspace, need);
+    return launch_f32_dense_matmul((hipStream_t)stream, x, xdt, w, y, m, n, k, workspace, need);
+}
+
 int hq_stream_read_probe(void* stream, const void* buf, size_t bytes, uint32_t* sink) {
     if (bytes == 0) return HQ_OK;
     if (!buf || !sink || bytes % 16 || !is_aligned(buf, 16))

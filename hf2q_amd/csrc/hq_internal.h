@@ -56,6 +56,14 @@ struct GemvArgs {
 size_t f16_shadow_workspace_bytes(uint32_t m, uint32_t k);
 int launch_f16_shadow_matmul(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_f16, float* y, uint32_t m, uint32_t n,
                              uint32_t k, void* workspace, size_t workspace_bytes);
+// The same over weights stored as f32 (bf16 activations are widened into the workspace).
+size_t f32_dense_workspace_bytes(uint32_t m, uint32_t k, hq_act_dtype xdt);
+int launch_f32_dense_matmul(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_f32, float* y, uint32_t m, uint32_t n,
+                            uint32_t k, void* workspace, size_t workspace_bytes);
+// One row at a time over f16 or f32 weights (dense.hip): k a multiple of 8 (f16) or 4 (f32) that fits LDS as f32.
+bool dense_gemv_takes(uint32_t k, hq_act_dtype wdt);
+int launch_dense_gemv(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, hq_act_dtype wdt, float* y, uint32_t m, uint32_t n,
+                      uint32_t k);
 // The current device's CU count (cached).
 int cu_count(uint32_t* out);
 int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type t);

@@ -57,14 +57,15 @@ struct Plan {
 };
 struct PerDevice {
     hipblasLtHandle_t handle = nullptr;
-    std::map<std::tuple<uint32_t, uint32_t, uint32_t, size_t>, Plan> plans;
+    std::map<std::tuple<uint32_t, uint32_t, uint32_t, size_t, bool>, Plan> plans;  // (m, n, k, workspace, f32 operands)
 };
 std::mutex g_mu;
 std::map<int, PerDevice> g_dev;
 
 // The plan for (m, n, k) with at most `ws_cap` bytes of library workspace, made on first use.  Column-major reading of
 // the row-major operands: D (n x m, ld n) = op_T(A = W as k x n, ld k) . (B = X as k x m, ld k).
-int plan_for(uint32_t m, uint32_t n, uint32_t k, size_t ws_cap, hipblasLtHandle_t* handle, Plan* out) {
+// f32_operands: both operands f32 (weights that are stored as f32) instead of f16.
+int plan_for(uint32_t m, uint32_t n, uint32_t k, size_t ws_cap, bool f32_operands, hipblasLtHandle_t* handle, Plan* out) {
     int dev = 0;
     if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
     std::lock_guard<std::mutex> lock(g_mu);
@@ -72,7 +73,8 @@ int plan_for(uint32_t m, uint32_t n, uint32_t k, size_t ws_cap, hipblasLtHandle_
     if (!pd.handle)
         if (int rc = check_lt(hipblasLtCreate(&pd.handle), "hipblasLtCreate")) return rc;
     *handle = pd.handle;
-    const auto key = std::make_tuple(m, n, k, ws_cap);
+    const auto key = std::make_tuple(m, n, k, ws_cap, f32_operands);
+    const hipDataType op_type = f32_operands ? HIP_R_32F : HIP_R_16F;
     auto it = pd.plans.find(key);
     if (it != pd.plans.end()) {
         *out = it->second;
@@ -83,8 +85,8 @@ int plan_for(uint32_t m, uint32_t n, uint32_t k, size_t ws_cap, hipblasLtHandle_
     const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
     int rc = check_lt(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)), "hipblasLtMatmulDescSetAttribute(TRANSA)");
     if (!rc) rc = check_lt(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)), "hipblasLtMatmulDescSetAttribute(TRANSB)");
-    if (!rc) rc = check_lt(hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16F, k, n, k), "hipblasLtMatrixLayoutCreate(weights)");
-    if (!rc) rc = check_lt(hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16F, k, m, k), "hipblasLtMatrixLayoutCreate(activations)");
+    if (!rc) rc = check_lt(hipblasLtMatrixLayoutCreate(&p.a, op_type, k, n, k), "hipblasLtMatrixLayoutCreate(weights)");
+    if (!rc) rc = check_lt(hipblasLtMatrixLayoutCreate(&p.b, op_type, k, m, k), "hipblasLtMatrixLayoutCreate(activations)");
     if (!rc) rc = check_lt(hipblasLtMatrixLayoutCreate(&p.c, HIP_R_32F, n, m, n), "hipblasLtMatrixLayoutCreate(output)");
     hipblasLtMatmulPreference_t pref = nullptr;
     if (!rc) rc = check_lt(hipblasLtMatmulPreferenceCreate(&pref), "hipblasLtMatmulPreferenceCreate");
@@ -94,7 +96,7 @@ int plan_for(uint32_t m, uint32_t n, uint32_t k, size_t ws_cap, hipblasLtHandle_
     int found = 0;
     if (!rc) rc = check_lt(hipblasLtMatmulAlgoGetHeuristic(pd.handle, p.desc, p.a, p.b, p.c, p.c, pref, 1, res, &found), "hipblasLtMatmulAlgoGetHeuristic");
     if (pref) hipblasLtMatmulPreferenceDestroy(pref);
-    if (!rc && found < 1) rc = fail(HQ_ERR_UNSUPPORTED, "F16-shadow matmul: the vendor library has no kernel for %u x %u x %u", m, n, k);
+    if (!rc && found < 1) rc = fail(HQ_ERR_UNSUPPORTED, "dense matmul: the vendor library has no %s kernel for %u x %u x %u", f32_operands ? "f32" : "f16", m, n, k);
     if (rc) {
         if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
         if (p.b) hipblasLtMatrixLayoutDestroy(p.b);
@@ -130,11 +132,49 @@ int launch_f16_shadow_matmul(hipStream_t s, const void* x, hq_act_dtype xdt, con
     const size_t ws_cap = workspace_bytes - xb;
     hipblasLtHandle_t handle = nullptr;
     Plan p;
-    if (int rc = plan_for(m, n, k, ws_cap, &handle, &p)) return rc;
+    if (int rc = plan_for(m, n, k, ws_cap, false, &handle, &p)) return rc;
     const float alpha = 1.f, beta = 0.f;
     return check_lt(hipblasLtMatmul(handle, p.desc, &alpha, w_f16, p.a, xh, p.b, &beta, y, p.c, y, p.c, &p.algo,
                                     static_cast<uint8_t*>(workspace) + xb, ws_cap, s),
                     "hipblasLtMatmul");
+}
+
+// The same product over weights stored as f32 (dense_matmul_f32_f32_tensor, src/serve/forward_mlx.rs:9851-9866): f32
+// operands, f32 accumulation.  bf16 activations are widened into the workspace first (exact).
+namespace {
+__global__ __launch_bounds__(256) void widen_bf16_kernel(const uint4* __restrict__ x, float4* __restrict__ out, uint64_t n8) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= n8) return;
+    const uint4 r = x[i];
+    out[2 * i] = make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
+                             __uint_as_float(r.y & 0xffff0000u));
+    out[2 * i + 1] = make_float4(__uint_as_float(r.z << 16), __uint_as_float(r.z & 0xffff0000u), __uint_as_float(r.w << 16),
+                                 __uint_as_float(r.w & 0xffff0000u));
+}
+inline size_t widen_bytes(uint32_t m, uint32_t k, hq_act_dtype xdt) { return xdt == HQ_BF16 ? ((size_t)m * k * 4 + 255) & ~(size_t)255 : 0; }
+}  // namespace
+
+size_t f32_dense_workspace_bytes(uint32_t m, uint32_t k, hq_act_dtype xdt) { return widen_bytes(m, k, xdt) + kLibraryWorkspace; }
+
+int launch_f32_dense_matmul(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w_f32, float* y, uint32_t m, uint32_t n,
+                            uint32_t k, void* workspace, size_t workspace_bytes) {
+    const size_t xb = widen_bytes(m, k, xdt);
+    const void* xf = x;
+    if (xdt == HQ_BF16) {
+        const uint64_t n8 = (uint64_t)m * k / 8;
+        hipLaunchKernelGGL(widen_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, s, static_cast<const uint4*>(x),
+                           static_cast<float4*>(workspace), n8);
+        if (int rc = check_launch("bf16 widening kernel launch")) return rc;
+        xf = workspace;
+    }
+    const size_t ws_cap = workspace_bytes - xb;
+    hipblasLtHandle_t handle = nullptr;
+    Plan p;
+    if (int rc = plan_for(m, n, k, ws_cap, true, &handle, &p)) return rc;
+    const float alpha = 1.f, beta = 0.f;
+    return check_lt(hipblasLtMatmul(handle, p.desc, &alpha, w_f32, p.a, xf, p.b, &beta, y, p.c, y, p.c, &p.algo,
+                                    static_cast<uint8_t*>(workspace) + xb, ws_cap, s),
+                    "hipblasLtMatmul(f32)");
 }
 
 }  // namespace hq

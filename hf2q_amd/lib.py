@@ -109,6 +109,8 @@ SIGNATURES = {
     "hq_tq_kv_restore": (_i32, [_vp, _vp, _sz, _vp, _vp, _u32, _u32, _u32, _u32]),
     "hq_matmul_f16_shadow_workspace_bytes": (_sz, [_u32, _u32, _u32]),
     "hq_matmul_f16_shadow": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _vp, _sz]),
+    "hq_dense_matmul_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),
+    "hq_dense_matmul": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _u32, _u32, _u32, _vp, _sz]),
     "hq_stream_read_probe": (_i32, [_vp, _vp, _sz, _vp]),
     "hq_gguf_open": (_i32, [_c.c_char_p, _c.POINTER(_vp)]),
     "hq_gguf_close": (None, [_vp]),

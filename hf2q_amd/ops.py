@@ -17,7 +17,7 @@ from dataclasses import dataclass
 import torch
 
 from . import lib as _l
-from .lib import HQ_BF16, HQ_F32, HQ_Q4_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HqError  # noqa: F401
+from .lib import HQ_BF16, HQ_F16, HQ_F32, HQ_Q4_0, HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HqError  # noqa: F401
 
 BLOCK_ELEMS = {HQ_Q4_0: 32, HQ_Q8_0: 32, HQ_Q4_K: 256, HQ_Q5_K: 256, HQ_Q6_K: 256}
 BLOCK_BYTES = {HQ_Q4_0: 18, HQ_Q8_0: 34, HQ_Q4_K: 144, HQ_Q5_K: 176, HQ_Q6_K: 210}
@@ -362,6 +362,34 @@ def matmul_f16_shadow(input: torch.Tensor, weight_f16: torch.Tensor, dst: torch.
                                             _dev(dst, "dst"), m, n, k, _dev(workspace, "workspace"), workspace.numel()))
 
 
+# GGML ids of the two plain element types a weight tensor may have (ggml_type.rs:18-53).
+GGML_F32, GGML_F16 = 0, 1
+
+
+def dense_matmul_workspace_bytes(m: int, n: int, k: int, act_dtype: torch.dtype, weight_dtype: torch.dtype) -> int:
+    xdt = HQ_BF16 if act_dtype == torch.bfloat16 else HQ_F32
+    wdt = HQ_F16 if weight_dtype == torch.float16 else HQ_F32
+    return int(_l.load().hq_dense_matmul_workspace_bytes(m, n, k, xdt, wdt))
+
+
+def dense_matmul(input: torch.Tensor, weight: torch.Tensor, dst: torch.Tensor, m: int, n: int, k: int,
+                 workspace: torch.Tensor | None = None) -> None:
+    """The branches of dispatch_qmatmul for weights that are not quantized (forward_mlx.rs:9820-9917): dst[m, n] =
+    input[m, k] . weight[n, k]^T for float32 or float16 weights, f32 or bf16 activations, f32 output.  Up to eight rows are
+    streaming passes over the weights (dispatch_dense_matvec_f32 / dispatch_dense_matvec_f16w_f32io), more rows the vendor
+    library's GEMM (dense_matmul_f32_f32_tensor / dispatch_mm_v2_f16)."""
+    if weight.dtype not in (torch.float32, torch.float16) or weight.numel() < n * k:
+        raise ValueError("weight must hold n * k float32 or float16 values")
+    if dst.dtype != torch.float32 or dst.numel() < m * n or input.numel() < m * k:
+        raise ValueError("dst must hold m * n float32 values and input m * k activations")
+    need = dense_matmul_workspace_bytes(m, n, k, input.dtype, weight.dtype)
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=input.device)
+    wdt = HQ_F16 if weight.dtype == torch.float16 else HQ_F32
+    _l.check(_l.load().hq_dense_matmul(_stream(), _dev(input, "input"), _act_dtype(input), _dev(weight, "weight"), wdt, _dev(dst, "dst"),
+                                       m, n, k, _dev(workspace, "workspace") if need else None, workspace.numel() if need else 0))
+
+
 # Above this many activation rows dispatch_qmatmul takes the matrix-matrix routes (mlx-native's MM_ROUTING_THRESHOLD,
 # forward_mlx.rs:9791).
 MM_ROUTING_THRESHOLD = 8
@@ -369,8 +397,9 @@ MM_ROUTING_THRESHOLD = 8
 
 @dataclass
 class MlxQWeight:
-    """A quantized linear weight as dispatch_qmatmul sees it (forward_mlx.rs:340-402): the raw GGML blocks with their type
-    and shape (QuantWeightInfo: rows = n, cols = k) and, optionally, the weight's F16 shadow."""
+    """A linear weight as dispatch_qmatmul sees it (forward_mlx.rs:340-402): the raw GGML blocks with their type and
+    shape (QuantWeightInfo: rows = n, cols = k) and, optionally, the weight's F16 shadow; or, with ggml_dtype GGML_F32 /
+    GGML_F16, the tensor's plain float32 / float16 values."""
     buffer: torch.Tensor
     ggml_dtype: int
     rows: int
@@ -389,11 +418,16 @@ class MlxQWeight:
 
 def dispatch_qmatmul(input: torch.Tensor, weight: MlxQWeight, output: torch.Tensor, m: int,
                      workspace: torch.Tensor | None = None) -> None:
-    """dispatch_qmatmul (forward_mlx.rs:9655-9969) for GGML-block weights: more than MM_ROUTING_THRESHOLD rows over a weight
-    with an F16 shadow take the dense f16 product (:9790-9817), everything else the quantized product, whose own routing
-    by m (GEMV, small-batch, tile kernels) is the library's.  `workspace`: device scratch for the route taken
+    """dispatch_qmatmul (forward_mlx.rs:9655-9969): float32 / float16 weights take the dense products (:9820-9917); more than
+    MM_ROUTING_THRESHOLD rows over a block weight with an F16 shadow the dense f16 product (:9790-9817); everything else the
+    quantized product, whose own routing by m (GEMV, small-batch, tile kernels) is the library's.  `workspace`: device scratch for the route taken
     (matmul_f16_shadow_workspace_bytes / quantized_matmul_workspace_bytes); allocated here when absent."""
     n, k = weight.rows, weight.cols
+    if weight.ggml_dtype in (GGML_F32, GGML_F16):  # :9820-9917
+        want = torch.float32 if weight.ggml_dtype == GGML_F32 else torch.float16
+        if weight.buffer.dtype != want:
+            raise TypeError(f"a weight of ggml type {weight.ggml_dtype} must be a {want} tensor")
+        return dense_matmul(input, weight.buffer, output, m, n, k, workspace)
     if m > MM_ROUTING_THRESHOLD and weight.f16_shadow is not None:
         need = matmul_f16_shadow_workspace_bytes(m, n, k)
         if workspace is None or workspace.numel() * workspace.element_size() < need:

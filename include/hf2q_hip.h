@@ -584,6 +584,21 @@ HQ_API size_t hq_matmul_f16_shadow_workspace_bytes(uint32_t m, uint32_t n, uint3
 HQ_API int hq_matmul_f16_shadow(void* stream, const void* x, hq_act_dtype xdt, const void* w_f16, float* y, uint32_t m, uint32_t n,
                          uint32_t k, void* workspace, size_t workspace_bytes);
 
+/* ---- weights that are not quantized ---- */
+
+/* y[m][n] (f32) = x[m][k] . W[n][k]^T over a weight stored as f32 or f16 (`wdt`: HQ_F32 or HQ_F16), row-major as in
+ * the file: the branches of dispatch_qmatmul for such tensors (src/serve/forward_mlx.rs:9820-9917) -- f32 weights (a
+ * router projection): dispatch_dense_matvec_f32 at m = 1, dense_matmul_f32_f32_tensor above; native f16 weights (tensors
+ * whose rows are not whole super-blocks, an f16 lm_head): dispatch_dense_matvec_f16w_f32io at m = 1, dispatch_mm_v2_f16
+ * above.  Here up to 8 rows take one streaming pass over the weights each (weights widened exactly, f32 multiply-add);
+ * more rows the vendor library's GEMM with f32 accumulation (f16 weights: the activations are cast to f16 first, as in
+ * hq_matmul_f16_shadow; f32 weights: f32 operands).  x: [m][k] f32 or bf16.  k % 8 == 0; x, w and y 16-byte aligned.
+ * `workspace`: hq_dense_matmul_workspace_bytes() bytes of device memory, 256-byte aligned (0 bytes, and the pointer may
+ * be null, where the row passes run). */
+HQ_API size_t hq_dense_matmul_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, hq_act_dtype xdt, hq_act_dtype wdt);
+HQ_API int hq_dense_matmul(void* stream, const void* x, hq_act_dtype xdt, const void* w, hq_act_dtype wdt, float* y, uint32_t m,
+                    uint32_t n, uint32_t k, void* workspace, size_t workspace_bytes);
+
 /* ---- measurement aid ---- */
 
 /* Reads `bytes` (a multiple of 16) of device memory at `buf` (16-byte aligned) once with plain 16-byte loads, eight

@@ -465,3 +465,61 @@ def test_dispatch_qmatmul_routes_by_rows_and_shadow(oracle, dev):
         y = torch.full((m, n), float("nan"), device=dev)
         ops.dispatch_qmatmul(x, wq, y, m)
         assert torch.equal(y, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("wdt", ["f16", "f32"])
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("m,n,k", [
+    (1, 128, 2816),     # a router projection (Gemma 4: ffn_gate_inp f32 [2816, 128], forward_mlx.rs:9827-9830)
+    (1, 2816, 704),     # an expert down projection kept as f16 (rows of 704 are not whole super-blocks, :9878-9880)
+    (1, 1000, 4096),    # an lm_head slice: 512 pieces of a row, eight per lane
+    (1, 70, 64),        # eight pieces per row: eight rows per wave step, ragged last step
+    (3, 300, 2112),     # a few rows: one pass each
+    (8, 33, 8200),      # a row of more pieces than 64 lanes x 8 in flight
+    (9, 130, 704),      # one row more: the vendor library's GEMM
+    (300, 257, 2112),
+])
+def test_dense_matmul_over_f16_and_f32_weights(dev, wdt, xdt, m, n, k):
+    """dispatch_qmatmul's routes for weights that are not quantized (forward_mlx.rs:9820-9917) against numpy float64 over
+    the same values: the row passes widen the weights exactly and accumulate in f32 (1e-5 of the row's magnitude); the
+    GEMM over f16 weights rounds the activations to f16 first, like hq_matmul_f16_shadow; over f32 weights the vendor
+    library may split f32 operands (1e-3 of the magnitude allowed, 1e-6 observed)."""
+    rng = np.random.default_rng(m * 1000 + n + k)
+    w32 = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    wd = torch.from_numpy(w32).to(dev)
+    wd = wd.half() if wdt == "f16" else wd
+    xd = torch.from_numpy(acts(m + n, m, k)).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    y = torch.full((m, n), float("nan"), device=dev)
+    for _ in range(2):
+        ops.dense_matmul(xd, wd, y, m, n, k)
+    torch.cuda.synchronize()
+    rows = m <= 8
+    assert (ops.dense_matmul_workspace_bytes(m, n, k, xd.dtype, wd.dtype) == 0) == rows
+    xv = xd.float() if rows or wdt == "f32" else xd.float().half()
+    ref = xv.double().cpu().numpy() @ wd.double().cpu().numpy().T
+    got = y.cpu().numpy()
+    assert np.isfinite(got).all()
+    scale = np.sqrt((ref ** 2).mean())
+    tol = 1e-5 if rows else 1e-3
+    assert np.abs(got - ref).max() <= tol * max(scale, np.abs(ref).max()), (np.abs(got - ref).max(), scale)
+    # the same through dispatch_qmatmul
+    wq = ops.MlxQWeight(wd, ops.GGML_F16 if wdt == "f16" else ops.GGML_F32, n, k)
+    y2 = torch.full((m, n), float("nan"), device=dev)
+    ops.dispatch_qmatmul(xd, wq, y2, m)
+    assert torch.equal(y2, y)
+
+
+@pytest.mark.gpu
+def test_dense_matmul_rejects_bad_arguments(dev):
+    x = torch.zeros(2, 64, device=dev)
+    w = torch.zeros(16, 64, device=dev)
+    y = torch.empty(2, 16, device=dev)
+    with pytest.raises(ops.HqError):
+        ops.dense_matmul(x, w, y, 2, 16, 60)                      # k % 8
+    with pytest.raises(ValueError):
+        ops.dense_matmul(x, w.to(torch.bfloat16), y, 2, 16, 64)   # bf16 weights have no route here
+    with pytest.raises(TypeError):
+        ops.dispatch_qmatmul(x, ops.MlxQWeight(w, ops.GGML_F16, 16, 64), y, 2)  # an f32 tensor declared f16
+    assert ops.dense_matmul_workspace_bytes(0, 16, 64, torch.float32, torch.float32) == 0
