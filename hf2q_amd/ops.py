@@ -556,6 +556,17 @@ class GgufFile:
             _l.check(_l.load().hq_gguf_load_tensor(self._h, name.encode(), _stream(), _dev(buf, name), info.byte_len))
         return buf
 
+    def load_weight(self, name: str, device) -> "MlxQWeight":
+        """The tensor as dispatch_qmatmul takes it (MlxQWeight, forward_mlx.rs:340-402): raw blocks for the block types, the
+        values themselves for F32 / F16 tensors (router projections, tensors whose rows are not whole super-blocks)."""
+        info = self.tensor_info(name)
+        buf = self.load_tensor(name, device)
+        if info.ggml_dtype == GGML_F32:
+            buf = buf.view(torch.float32)
+        elif info.ggml_dtype == GGML_F16:
+            buf = buf.view(torch.float16)
+        return MlxQWeight(buf, info.ggml_dtype, info.rows, info.cols)
+
 
 # ---- TurboQuant-style 8-bit KV cache ------------------------------------------------------------
 

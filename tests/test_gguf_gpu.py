@@ -39,3 +39,35 @@ def test_gguf_tensors_drive_gemv_and_mul_mat_id(oracle, dev, tmp_path):
     for p, e in enumerate(ids):
         ref = oracle.qmatmul_f64(x[p // top_k:p // top_k + 1], per[e], 1, n, k, HQ_Q4_K)
         assert_matmul_close(yid[p].cpu().numpy(), ref, f"mul_mat_id row {p} from gguf")
+
+
+def test_gguf_float_tensors_take_the_dense_routes_of_dispatch_qmatmul(oracle, dev, tmp_path):
+    """An f32 router projection and an f16 tensor whose rows are not whole super-blocks (forward_mlx.rs:9820-9917), loaded
+    as MlxQWeight and multiplied through dispatch_qmatmul at one row and at a prompt's worth."""
+    k, n_r, n_d = 704, 128, 96
+    rng = np.random.default_rng(5)
+    router = (rng.standard_normal((n_r, k)) * 0.05).astype(np.float32)
+    down = (rng.standard_normal((n_d, k)) * 0.05).astype(np.float16)
+    blocks = oracle.quantize(weights(4, n_d, 768), 768, HQ_Q4_K, threads=8)
+    path = str(tmp_path / "f.gguf")
+    W.write(path, [("general.architecture", W.STRING, "test")],
+            [("blk.0.ffn_gate_inp.weight", [k, n_r], ops.GGML_F32, router.tobytes()),
+             ("blk.0.ffn_down.weight", [k, n_d], ops.GGML_F16, down.tobytes()), ("blk.0.ffn_up.weight", [768, n_d], HQ_Q4_K, blocks.tobytes())])
+    with ops.GgufFile.open(path) as g:
+        wr, wdn, wq = (g.load_weight(nm, dev) for nm in ("blk.0.ffn_gate_inp.weight", "blk.0.ffn_down.weight", "blk.0.ffn_up.weight"))
+    assert (wr.buffer.dtype, wr.rows, wr.cols) == (torch.float32, n_r, k) and (wdn.buffer.dtype, wdn.rows, wdn.cols) == (torch.float16, n_d, k)
+    assert wq.buffer.dtype == torch.uint8 and wq.ggml_dtype == HQ_Q4_K
+    assert torch.equal(wr.buffer.cpu().view(n_r, k), torch.from_numpy(router)) and torch.equal(wdn.buffer.cpu().view(n_d, k), torch.from_numpy(down))
+    for m in (1, 20):
+        x = acts(m, m, k)
+        xd = torch.from_numpy(x).to(dev)
+        for w, host in ((wr, router), (wdn, down)):
+            y = torch.full((m, w.rows), float("nan"), device=dev)
+            ops.dispatch_qmatmul(xd, w, y, m)
+            xv = x.astype(np.float16) if (m > 8 and host.dtype == np.float16) else x
+            ref = xv.astype(np.float64) @ host.astype(np.float64).T
+            assert np.abs(y.cpu().numpy() - ref).max() <= (1e-5 if m <= 8 else 1e-3) * np.abs(ref).max()
+    x = acts(9, 1, 768)
+    y = torch.empty(1, n_d, device=dev)
+    ops.dispatch_qmatmul(torch.from_numpy(x).to(dev), wq, y, 1)
+    assert_matmul_close(y.cpu().numpy(), oracle.qmatmul_f64(x, blocks, 1, n_d, 768, HQ_Q4_K), "block weight through load_weight")
