@@ -158,6 +158,7 @@ extern "C" {
     pub fn hq_quantize_ggml_imatrix(stream: *mut c_void, src: *const f32, n_elems: u64, n_per_row: u64, t: hq_ggml_type, imatrix: *const f32, out_blocks: *mut c_void, scratch: *mut c_void, scratch_bytes: usize) -> c_int;
     pub fn hq_qmatmul_ggml(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type) -> c_int;
     pub fn hq_qmatmul_ggml_k_slices(m: u32, n: u32, k: u32, t: hq_ggml_type, slices: *mut u32, blocks_per_slice: *mut u32) -> c_int;
+    pub fn hq_gemv_flat_plan(n: u32, k: u32, t: hq_ggml_type, waves: u32, units_per_row: *mut u32, rows_per_task: *mut u32, windows_per_task: *mut u32, units_per_window: *mut u32, window_capacity: *mut u32) -> c_int;
     pub fn hq_qmatmul_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;
     pub fn hq_qmatmul_ggml_ws(stream: *mut c_void, x: *const c_void, xdt: hq_act_dtype, w_blocks: *const c_void, y: *mut f32, m: u32, n: u32, k: u32, t: hq_ggml_type, workspace: *mut c_void, workspace_bytes: usize) -> c_int;
     pub fn hq_qmatmul_gated_ggml_workspace_bytes(m: u32, n: u32, k: u32, xdt: hq_act_dtype, t: hq_ggml_type) -> usize;

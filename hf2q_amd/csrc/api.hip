@@ -302,6 +302,17 @@ int hq_qmatmul_ggml_k_slices(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t,
     return HQ_OK;
 }
 
+int hq_gemv_flat_plan(uint32_t n, uint32_t k, hq_ggml_type t, uint32_t waves, uint32_t* units_per_row, uint32_t* rows_per_task,
+                      uint32_t* windows_per_task, uint32_t* units_per_window, uint32_t* window_capacity) {
+    if (!units_per_row || !rows_per_task || !windows_per_task || !units_per_window || !window_capacity)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_gemv_flat_plan: null output");
+    const uint32_t ue = t == HQ_Q8_0 || t == HQ_Q4_0 ? 32u : 256u;
+    if (!known_type(t) || n == 0 || waves == 0 || k % ue || k / ue < 2)
+        return fail(HQ_ERR_INVALID_ARGUMENT, "hq_gemv_flat_plan: type %d, n %u, k %u, waves %u", (int)t, n, k, waves);
+    gemv_flat_plan(t, n, k, waves, units_per_row, rows_per_task, windows_per_task, units_per_window, window_capacity);
+    return HQ_OK;
+}
+
 int hq_qmatmul_ggml_ws(void* stream, const void* x, hq_act_dtype xdt, const void* w_blocks, float* y, uint32_t m,
                        uint32_t n, uint32_t k, hq_ggml_type t, void* workspace, size_t workspace_bytes) {
     return qmatmul_ws("hq_qmatmul_ggml_ws", stream, x, xdt, w_blocks, nullptr, y, m, n, k, t, workspace, workspace_bytes);

@@ -822,6 +822,19 @@ int launch_jobs_t(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs) {
 // Where the small-batch kernel has its stage-once form (gemv_rows_stream_fast: Q6_K 151936 x 4096 134 us, Q4_K 65536 x 4096
 // 41 us, Q4_K / Q6_K 12288 x 4096 13 / 21 us for any 3 .. 8 rows) it is ahead from five rows on, and from three on
 // matrices of 32768 rows or more (three and four rows in passes: 55 / 62 us on the 65536-row Q4_K matrix).
+// The flat walk's plan for an n x k matrix of type t on `waves` waves (host arithmetic).
+void gemv_flat_plan(hq_ggml_type t, uint32_t n, uint32_t k, uint32_t waves, uint32_t* units_per_row, uint32_t* rows_per_task,
+                    uint32_t* windows_per_task, uint32_t* units_per_window, uint32_t* window_capacity) {
+    const bool b32 = t == HQ_Q8_0 || t == HQ_Q4_0;
+    const uint32_t ue = b32 ? 32u : 256u, uw = b32 ? 64u : 16u;
+    const FlatGeom g = flat_geom(k, ue, uw, n, 1, waves);
+    *units_per_row = g.bu;
+    *rows_per_task = 1u << g.log_r;
+    *windows_per_task = g.st;
+    *units_per_window = g.uwe;
+    *window_capacity = uw;
+}
+
 bool gemv_stream_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
     if (xdt != HQ_BF16 || m < 3) return false;
     uint32_t cus = 0;

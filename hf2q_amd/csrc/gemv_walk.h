@@ -325,7 +325,8 @@ struct FlatWalk {
         constexpr bool HALVES = XHALF && !X::PAIR && !kBlock32<TYPE>;
         uint32_t xr[HALVES ? 32 : X::XW];
         float sx[4] = {0.f, 0.f, 0.f, 0.f};
-        const bool xinv = !HALVES && g.st == 1u && g.log_r == 0u;  // every window is one whole row: the lane's activations never change
+        // every window is one whole row (and not a ragged one): the lane's activations never change
+        const bool xinv = !HALVES && g.st == 1u && g.log_r == 0u && g.uwe == g.bu;
         if constexpr (!HALVES)
             if (xinv) X::load(lds_x, lds_s, lv, c, xr, sx);
         const int last_lane = (int)(g.uwe * LPU - 1u);

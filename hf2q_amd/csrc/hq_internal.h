@@ -70,6 +70,8 @@ int launch_gemv(hipStream_t s, const GemvArgs& a, hq_act_dtype xdt, hq_ggml_type
 // True where a few dense rows are better served by launch_gemv (which takes them up to four at a time, one pass over
 // the weights each) than by the small-batch kernel.
 bool gemv_stream_passes_preferred(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k);
+void gemv_flat_plan(hq_ggml_type t, uint32_t n, uint32_t k, uint32_t waves, uint32_t* units_per_row, uint32_t* rows_per_task,
+                    uint32_t* windows_per_task, uint32_t* units_per_window, uint32_t* window_capacity);
 // Up to four independent GEMVs of one weight type and activation dtype in a single launch.
 int launch_gemv_jobs(hipStream_t s, const GemvArgs* jobs, uint32_t n_jobs, hq_act_dtype xdt, hq_ggml_type t);
 

@@ -57,6 +57,7 @@ SIGNATURES = {
     "hq_qmatmul_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32]),
     "hq_qmatmul_ggml_workspace_bytes": (_sz, [_u32, _u32, _u32, _i32, _i32]),
     "hq_qmatmul_ggml_k_slices": (_i32, [_u32, _u32, _u32, _i32, _c.POINTER(_u32), _c.POINTER(_u32)]),
+    "hq_gemv_flat_plan": (_i32, [_u32, _u32, _i32, _u32] + [_c.POINTER(_u32)] * 5),
     "hq_qmatmul_ggml_ws": (_i32, [_vp, _vp, _i32, _vp, _vp, _u32, _u32, _u32, _i32, _vp, _sz]),
     "hq_qmatmul_id_ggml": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _sz, _u32, _u32, _u32, _u32, _u32, _u64, _i32]),
     "hq_weight_row_scales_ggml": (_i32, [_vp, _vp, _vp, _u64, _u32, _i32]),

@@ -124,6 +124,15 @@ HQ_API int hq_qmatmul_ggml(void* stream, const void* x, hq_act_dtype xdt, const 
 HQ_API int hq_qmatmul_ggml_k_slices(uint32_t m, uint32_t n, uint32_t k, hq_ggml_type t, uint32_t* slices,
                              uint32_t* blocks_per_slice);
 
+/* How the single-row product of any k lays its work out (the walk that serves f32 activations, k that is not a multiple
+ * of 4096, Q8_0 / Q4_0): a row is `units_per_row` units (a 256-weight super-block, or a 32-weight block); a task is
+ * `rows_per_task` (a power of two) whole rows = `windows_per_task` windows of `units_per_window` units, at most
+ * `window_capacity` (16 super-blocks or 64 blocks: one wave's 64 lanes); the last window of a task may be ragged
+ * (windows_per_task * units_per_window >= rows_per_task * units_per_row > (windows_per_task - 1) * units_per_window always
+ * holds: no window is empty).  `waves`: the waves the launch has (CUs x 16).  Pure host arithmetic; a query for tests. */
+HQ_API int hq_gemv_flat_plan(uint32_t n, uint32_t k, hq_ggml_type t, uint32_t waves, uint32_t* units_per_row, uint32_t* rows_per_task,
+                      uint32_t* windows_per_task, uint32_t* units_per_window, uint32_t* window_capacity);
+
 /* The same product with caller-owned device scratch.  The f16 tile kernels
  * (prefill-sized m; K-quants with k % 256 == 0, Q8_0 / Q4_0 with k % 128 == 0) convert the
  * activations to row-scaled f16 in a pre-pass and need hq_qmatmul_ggml_workspace_bytes() bytes (256-byte

@@ -167,3 +167,27 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(FileNotFoundError):
         lib.load()
+
+
+def test_flat_walk_plan_covers_every_row_with_no_empty_window():
+    """hq_gemv_flat_plan for every row length of whole units up to 130 super-blocks / 400 blocks and a spread of row counts:
+    a task is a power-of-two number of rows, its windows are within a wave's capacity, together they cover the task's
+    units, and none of them is empty (only the last may be ragged)."""
+    L = lib.load()
+    outs = [ctypes.c_uint32() for _ in range(5)]
+    refs = [ctypes.byref(o) for o in outs]
+    for t, ue, cap, kmax in ((lib.HQ_Q4_K, 256, 16, 130), (lib.HQ_Q6_K, 256, 16, 130), (lib.HQ_Q8_0, 32, 64, 400)):
+        for units in range(2, kmax + 1):
+            for n in (1, 63, 512, 4096, 5120, 151936):
+                lib.check(L.hq_gemv_flat_plan(n, units * ue, t, 4096, *refs))
+                bu, r, st, uwe, capacity = (o.value for o in outs)
+                assert bu == units and capacity == cap
+                assert r >= 1 and r & (r - 1) == 0 and r <= cap
+                assert 1 <= uwe <= cap and st >= 1
+                assert st * uwe >= r * bu > (st - 1) * uwe, (t, units, n, r, st, uwe)
+    # the shapes behind the ragged windows: 68 super-blocks a row on 4096 waves, 5120 rows -> two rows in nine windows
+    lib.check(L.hq_gemv_flat_plan(5120, 17408, lib.HQ_Q4_K, 4096, *refs))
+    assert [o.value for o in outs] == [68, 2, 9, 16, 16]
+    assert L.hq_gemv_flat_plan(16, 256, lib.HQ_Q4_K, 4096, *refs) == lib.HQ_ERR_INVALID_ARGUMENT   # a single unit per row
+    assert L.hq_gemv_flat_plan(16, 512, lib.HQ_Q4_K, 0, *refs) == lib.HQ_ERR_INVALID_ARGUMENT
+    assert L.hq_gemv_flat_plan(16, 512, lib.HQ_Q4_K, 4096, None, *refs[1:]) == lib.HQ_ERR_INVALID_ARGUMENT
