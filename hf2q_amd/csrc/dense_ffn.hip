@@ -240,7 +240,13 @@ int route(hipStream_t s, const DenseFfnArgs& d, uint32_t cus, bool dry) {
             case HQ_Q4_K: return launch_t<HQ_Q4_K, HQ_Q4_K, X_BF16>(s, d, cus, dry);
             case HQ_Q5_K: return launch_t<HQ_Q5_K, HQ_Q5_K, X_BF16>(s, d, cus, dry);
             case HQ_Q6_K: return launch_t<HQ_Q6_K, HQ_Q6_K, X_BF16>(s, d, cus, dry);
-            case HQ_Q8_0: return launch_t<HQ_Q8_0, HQ_Q8_0, X_BF16>(s, d, cus, dry);
+            case HQ_Q8_0: {  // the walk's own rule for block pairs, per matrix (gate and up are walked side by side)
+                const bool pg = q80_walk_in_pairs(2ull * d.inter, d.hidden), pd = q80_walk_in_pairs(d.hidden, d.inter);
+                if (pg && pd) return launch_t<HQ_Q8_0_X2, HQ_Q8_0_X2, X_BF16>(s, d, cus, dry);
+                if (pg) return launch_t<HQ_Q8_0_X2, HQ_Q8_0, X_BF16>(s, d, cus, dry);
+                if (pd) return launch_t<HQ_Q8_0, HQ_Q8_0_X2, X_BF16>(s, d, cus, dry);
+                return launch_t<HQ_Q8_0, HQ_Q8_0, X_BF16>(s, d, cus, dry);
+            }
             case HQ_Q4_0: return launch_t<HQ_Q4_0, HQ_Q4_0, X_BF16>(s, d, cus, dry);
         }
     }

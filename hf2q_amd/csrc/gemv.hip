@@ -654,6 +654,8 @@ constexpr int kFlatDepth = TYPE == HQ_Q8_0 ? HQ_FLAT_D_Q80 : TYPE == HQ_Q4_0 ? H
 template <int TYPE, bool X_BF16>
 int launch_flat(hipStream_t s, const void* x, const uint8_t* w0, const uint8_t* w1, float* y0, float* y1, uint32_t n, uint32_t k,
                 uint32_t nm, uint32_t cus, bool swiglu = false) {
+    if constexpr (TYPE == HQ_Q8_0)
+        if (q80_walk_in_pairs((uint64_t)n * nm, k)) return launch_flat<HQ_Q8_0_X2, X_BF16>(s, x, w0, w1, y0, y1, n, k, nm, cus, swiglu);
     constexpr int W = (TYPE == HQ_Q6_K && X_BF16) ? 12 : 16;
     using X = FlatX<TYPE, X_BF16>;
     const FArgs fa{x, w0, w1, y0, y1, n, k, nm, swiglu ? 1u : 0u, flat_geom(k, kUnitElems<TYPE>, kUnitsPerWindow<TYPE>, n, nm, cus * W),

@@ -11,12 +11,16 @@ namespace {
 
 constexpr uint32_t M4 = 0x000f000fu, M2 = 0x00300030u, M1 = 0x10101010u, MAGIC = 0x43004300u;
 constexpr uint32_t N4 = 0x0f0f0f0fu, N2 = 0x30303030u;  // the Q6_K kernels work on four bytes at a time
+// A pseudo type of the flat walk (gemv_walk.h), not a GGML id: two consecutive Q8_0 blocks of a row as one lane's piece,
+// 68 bytes and 64 weights, so that a wave has twice the bytes of a window in flight (one 34-byte block per lane is
+// 2.2 KB per wave, less than the memory system needs from sixteen waves per CU).
+constexpr int HQ_Q8_0_X2 = 1008;
 // Types whose block is one lane's piece of 32 weights (the K-quants give a lane 64 of a super-block's 256).
 template <int TYPE>
 constexpr bool kBlock32 = TYPE == HQ_Q8_0 || TYPE == HQ_Q4_0;
 template <int TYPE>
 constexpr uint32_t kBlockBytes = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q5_K ? Q5K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES
-                                 : TYPE == HQ_Q4_0 ? Q4_0_BYTES : Q8_0_BYTES;
+                                 : TYPE == HQ_Q4_0 ? Q4_0_BYTES : TYPE == HQ_Q8_0_X2 ? 2 * Q8_0_BYTES : Q8_0_BYTES;
 template <int TYPE>
 struct Lane {  // weights per lane and step
     static constexpr int kElems = kBlock32<TYPE> ? 32 : 64;
@@ -79,6 +83,19 @@ struct Piece<HQ_Q8_0> {
         d = ld2(blk);
         q0 = ld16_unaligned(blk + 2);
         q1 = ld16_unaligned(blk + 18);
+    }
+};
+
+template <>
+struct Piece<HQ_Q8_0_X2> {  // [d0][32 int8][d1][32 int8] as seventeen words
+    uint4 a, b, c, e;
+    uint32_t t;
+    __device__ __forceinline__ void load(const uint8_t* blk, int) {
+        a = ld16_unaligned(blk);
+        b = ld16_unaligned(blk + 16);
+        c = ld16_unaligned(blk + 32);
+        e = ld16_unaligned(blk + 48);
+        t = ld4_unaligned(blk + 64);
     }
 };
 
@@ -341,6 +358,29 @@ __device__ __forceinline__ float dot_f32(const Piece<HQ_Q8_0>& p, int, const flo
         for (int i = 0; i < 4; ++i) acc = fmaf(sbyte(w, i), xf[4 * j + i], acc);
     }
     return f16_bits_to_f32(p.d) * acc;
+}
+
+// Two blocks: the first one's weights are bytes 2 .. 33 (each word spans two of the fetched ones), its scale the low half
+// of word 0; the second one's scale is the high half of word 8, its weights words 9 .. 16.  Per block the operations of
+// the one-block form; the lane adds the two.
+__device__ __forceinline__ float dot_f32(const Piece<HQ_Q8_0_X2>& p, int, const float* xf, const float*) {
+    const uint32_t w[17] = {p.a.x, p.a.y, p.a.z, p.a.w, p.b.x, p.b.y, p.b.z, p.b.w, p.c.x, p.c.y, p.c.z, p.c.w, p.e.x, p.e.y, p.e.z, p.e.w, p.t};
+    float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t q = __builtin_amdgcn_alignbyte(w[j + 1], w[j], 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc0 = fmaf(sbyte(q, i), xf[4 * j + i], acc0);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc1 = fmaf(sbyte(w[9 + j], i), xf[32 + 4 * j + i], acc1);
+    }
+    return f16_bits_to_f32(w[0] & 0xffffu) * acc0 + f16_bits_to_f32(w[8] >> 16) * acc1;
+}
+__device__ __forceinline__ float dot_pair(const Piece<HQ_Q8_0_X2>&, int, const uint32_t*, const float*, uint32_t, uint32_t, uint32_t) {
+    return 0.f;
 }
 
 // Staging of one activation row in LDS, 16 activations per thread and pass:

@@ -20,11 +20,17 @@ namespace hq {
 namespace {
 
 template <int TYPE>
-constexpr uint32_t kLanesPerUnit = kBlock32<TYPE> ? 1u : 4u;
+constexpr bool kLaneUnit = kBlock32<TYPE> || TYPE == HQ_Q8_0_X2;  // a unit is one lane's piece
+template <int TYPE>
+constexpr uint32_t kLanesPerUnit = kLaneUnit<TYPE> ? 1u : 4u;
 template <int TYPE>
 constexpr uint32_t kUnitsPerWindow = 64u / kLanesPerUnit<TYPE>;
 template <int TYPE>
-constexpr uint32_t kUnitElems = kBlock32<TYPE> ? 32u : 256u;
+constexpr uint32_t kUnitElems = kBlock32<TYPE> ? 32u : TYPE == HQ_Q8_0_X2 ? 64u : 256u;
+
+// Q8_0 rows of whole block pairs are walked as pairs (HQ_Q8_0_X2) from about a window per wave of the device on; the same
+// rule wherever the walk is used, so that every caller gets the same sums.
+inline bool q80_walk_in_pairs(uint64_t n_total, uint32_t k) { return k % 64u == 0 && n_total * (k / 64u) >= 64ull * 4096ull; }
 
 struct FlatGeom {
     uint32_t bu;     // units per row
@@ -80,7 +86,7 @@ inline FlatGeom flat_geom(uint32_t k, uint32_t unit_elems, uint32_t uw, uint32_t
 // piece is an immediate offset from the lane's one base address.
 template <int TYPE, bool X_BF16>
 struct FlatX {
-    static constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0;
+    static constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0 && TYPE != HQ_Q8_0_X2;
     static constexpr int XW = PAIR ? (kBlock32<TYPE> ? 16 : 32) : (kBlock32<TYPE> ? 32 : 64);  // registers of one lane's activations
     static constexpr uint32_t CA = PAIR ? 8u : 4u;                                              // activations per chunk
     static constexpr uint32_t G = (kBlock32<TYPE> ? 32u : 64u) / CA;                             // chunks per piece
@@ -167,7 +173,7 @@ struct FlatX {
                 sx[r] = lds_s[ur * 16u + (uint32_t)(c >> 1) * 8u + (uint32_t)(c & 1) + 2u * r];
             }
         } else {
-            const uint32_t piece = kBlock32<TYPE> ? ur : ur * 4u + (uint32_t)c;
+            const uint32_t piece = kLaneUnit<TYPE> ? ur : ur * 4u + (uint32_t)c;
             const uint4* base = lds_x + piece * (G + 1u);
 #pragma unroll
             for (int j = 0; j < (int)G; ++j) put(4 * j, base[j]);
@@ -322,7 +328,7 @@ struct FlatWalk {
         uint32_t c_m = 0, c_w = 0, done = 0;
         float keep0 = 0.f, keep1 = 0.f;
         uint32_t keep_row = 0;
-        constexpr bool HALVES = XHALF && !X::PAIR && !kBlock32<TYPE>;
+        constexpr bool HALVES = XHALF && !X::PAIR && !kLaneUnit<TYPE>;
         uint32_t xr[HALVES ? 32 : X::XW];
         float sx[4] = {0.f, 0.f, 0.f, 0.f};
         // every window is one whole row (and not a ragged one): the lane's activations never change
