@@ -232,6 +232,16 @@ int launch_t(hipStream_t s, const DenseFfnArgs& d, uint32_t cus, bool dry) {
     return check_launch("dense FFN block launch");
 }
 
+// Q8_0 / Q4_0: the walk's own rule for doubled pieces, per matrix (gate and up are walked side by side).
+template <int T, bool X_BF16>
+int route_blocks(hipStream_t s, const DenseFfnArgs& d, uint32_t cus, bool dry) {
+    const bool pg = walk_doubled<T, X_BF16>(2ull * d.inter, d.hidden), pd = walk_doubled<T, false>(d.hidden, d.inter);
+    if (pg && pd) return launch_t<kX2 + T, kX2 + T, X_BF16>(s, d, cus, dry);
+    if (pg) return launch_t<kX2 + T, T, X_BF16>(s, d, cus, dry);
+    if (pd) return launch_t<T, kX2 + T, X_BF16>(s, d, cus, dry);
+    return launch_t<T, T, X_BF16>(s, d, cus, dry);
+}
+
 template <bool X_BF16>
 int route(hipStream_t s, const DenseFfnArgs& d, uint32_t cus, bool dry) {
     const hq_ggml_type g = d.t_gate_up, n = d.t_down;
@@ -240,14 +250,8 @@ int route(hipStream_t s, const DenseFfnArgs& d, uint32_t cus, bool dry) {
             case HQ_Q4_K: return launch_t<HQ_Q4_K, HQ_Q4_K, X_BF16>(s, d, cus, dry);
             case HQ_Q5_K: return launch_t<HQ_Q5_K, HQ_Q5_K, X_BF16>(s, d, cus, dry);
             case HQ_Q6_K: return launch_t<HQ_Q6_K, HQ_Q6_K, X_BF16>(s, d, cus, dry);
-            case HQ_Q8_0: {  // the walk's own rule for block pairs, per matrix (gate and up are walked side by side)
-                const bool pg = q80_walk_in_pairs(2ull * d.inter, d.hidden), pd = q80_walk_in_pairs(d.hidden, d.inter);
-                if (pg && pd) return launch_t<HQ_Q8_0_X2, HQ_Q8_0_X2, X_BF16>(s, d, cus, dry);
-                if (pg) return launch_t<HQ_Q8_0_X2, HQ_Q8_0, X_BF16>(s, d, cus, dry);
-                if (pd) return launch_t<HQ_Q8_0, HQ_Q8_0_X2, X_BF16>(s, d, cus, dry);
-                return launch_t<HQ_Q8_0, HQ_Q8_0, X_BF16>(s, d, cus, dry);
-            }
-            case HQ_Q4_0: return launch_t<HQ_Q4_0, HQ_Q4_0, X_BF16>(s, d, cus, dry);
+            case HQ_Q8_0: return route_blocks<HQ_Q8_0, X_BF16>(s, d, cus, dry);
+            case HQ_Q4_0: return route_blocks<HQ_Q4_0, X_BF16>(s, d, cus, dry);
         }
     }
     // the mixes GGUF files of the reference's models hold: down in Q6_K over Q4_K or Q5_K gate / up

@@ -649,17 +649,17 @@ bool flat_takes(uint64_t n_total, uint32_t k, uint32_t cus, size_t lds) {
 // Fetches a wave keeps in flight: one (a ring of two or four windows of 32-weight blocks, which are only 1.1 / 2.2 KB,
 // measured slower: Q4_0 12288 x 4096 13.8 against 9.7 us).
 template <int TYPE>
-constexpr int kFlatDepth = TYPE == HQ_Q8_0 ? HQ_FLAT_D_Q80 : TYPE == HQ_Q4_0 ? HQ_FLAT_D_Q40 : 1;
+constexpr int kFlatDepth = kIsX2<TYPE> ? 1 : TYPE == HQ_Q8_0 ? HQ_FLAT_D_Q80 : TYPE == HQ_Q4_0 ? HQ_FLAT_D_Q40 : 1;
 
 template <int TYPE, bool X_BF16>
 int launch_flat(hipStream_t s, const void* x, const uint8_t* w0, const uint8_t* w1, float* y0, float* y1, uint32_t n, uint32_t k,
                 uint32_t nm, uint32_t cus, bool swiglu = false) {
-    if constexpr (TYPE == HQ_Q8_0)
-        if (q80_walk_in_pairs((uint64_t)n * nm, k)) return launch_flat<HQ_Q8_0_X2, X_BF16>(s, x, w0, w1, y0, y1, n, k, nm, cus, swiglu);
-    constexpr int W = (TYPE == HQ_Q6_K && X_BF16) ? 12 : 16;
+    if constexpr (kBlock32<TYPE>)
+        if (walk_doubled<TYPE, X_BF16>((uint64_t)n * nm, k)) return launch_flat<kX2 + TYPE, X_BF16>(s, x, w0, w1, y0, y1, n, k, nm, cus, swiglu);
+    constexpr int W = (kBaseType<TYPE> == HQ_Q6_K && X_BF16) ? 12 : 16;
     using X = FlatX<TYPE, X_BF16>;
     const FArgs fa{x, w0, w1, y0, y1, n, k, nm, swiglu ? 1u : 0u, flat_geom(k, kUnitElems<TYPE>, kUnitsPerWindow<TYPE>, n, nm, cus * W),
-                   TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
+                   kBaseType<TYPE> == HQ_Q6_K ? N4 : M4, kBaseType<TYPE> == HQ_Q5_K ? M1 : kBaseType<TYPE> == HQ_Q6_K ? N2 : M2, MAGIC};
     const uint64_t supers = ((uint64_t)n + (1u << fa.g.log_r) - 1) >> fa.g.log_r;
     const bool dyn = kFlatDepth<TYPE> == 1 && supers >= (uint64_t)cus * W * 8u;
     auto kern = dyn ? gemv_flat_kernel<TYPE, X_BF16, W, 1, true> : gemv_flat_kernel<TYPE, X_BF16, W, kFlatDepth<TYPE>, false>;

@@ -11,24 +11,40 @@ namespace {
 
 constexpr uint32_t M4 = 0x000f000fu, M2 = 0x00300030u, M1 = 0x10101010u, MAGIC = 0x43004300u;
 constexpr uint32_t N4 = 0x0f0f0f0fu, N2 = 0x30303030u;  // the Q6_K kernels work on four bytes at a time
-// A pseudo type of the flat walk (gemv_walk.h), not a GGML id: two consecutive Q8_0 blocks of a row as one lane's piece,
-// 68 bytes and 64 weights, so that a wave has twice the bytes of a window in flight (one 34-byte block per lane is
-// 2.2 KB per wave, less than the memory system needs from sixteen waves per CU).
-constexpr int HQ_Q8_0_X2 = 1008;
+// Pseudo types of the flat walk (gemv_walk.h), not GGML ids: kX2 + t is a lane's piece of type t twice over -- two
+// consecutive blocks (Q8_0, Q4_0), or the lane's quarter of two consecutive super-blocks (K-quants) -- fetched together,
+// so that a wave has twice the bytes of a window in flight: one piece per lane is 1.2 .. 3.4 KB per wave, less than the
+// memory system needs from sixteen waves per CU to run at its rate.
+constexpr int kX2 = 1000;
+template <int TYPE>
+constexpr bool kIsX2 = TYPE >= kX2;
+template <int TYPE>
+constexpr int kBaseType = TYPE >= kX2 ? TYPE - kX2 : TYPE;
+constexpr int HQ_Q8_0_X2 = kX2 + HQ_Q8_0;
 // Types whose block is one lane's piece of 32 weights (the K-quants give a lane 64 of a super-block's 256).
 template <int TYPE>
 constexpr bool kBlock32 = TYPE == HQ_Q8_0 || TYPE == HQ_Q4_0;
 template <int TYPE>
-constexpr uint32_t kBlockBytes = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q5_K ? Q5K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES
-                                 : TYPE == HQ_Q4_0 ? Q4_0_BYTES : TYPE == HQ_Q8_0_X2 ? 2 * Q8_0_BYTES : Q8_0_BYTES;
+constexpr uint32_t kBlockBytes1 = TYPE == HQ_Q4_K ? Q4K_BYTES : TYPE == HQ_Q5_K ? Q5K_BYTES : TYPE == HQ_Q6_K ? Q6K_BYTES
+                                  : TYPE == HQ_Q4_0 ? Q4_0_BYTES : Q8_0_BYTES;
+template <int TYPE>
+constexpr uint32_t kBlockBytes = kIsX2<TYPE> ? 2u * kBlockBytes1<kBaseType<TYPE>> : kBlockBytes1<TYPE>;
 template <int TYPE>
 struct Lane {  // weights per lane and step
     static constexpr int kElems = kBlock32<TYPE> ? 32 : 64;
 };
 
-// Per-lane fetch of one piece of row data.
+// Per-lane fetch of one piece of row data.  The primary template is the doubled piece of a base type (its
+// specialisations below): the same quarter of the next super-block, or the next block.
 template <int TYPE>
-struct Piece;
+struct Piece {
+    static_assert(kIsX2<TYPE>, "base types have their own pieces");
+    Piece<kBaseType<TYPE>> a, b;
+    __device__ __forceinline__ void load(const uint8_t* blk, int c) {
+        a.load(blk, c);
+        b.load(blk + kBlockBytes1<kBaseType<TYPE>>, c);
+    }
+};
 
 template <>
 struct Piece<HQ_Q4_K> {
@@ -381,6 +397,20 @@ __device__ __forceinline__ float dot_f32(const Piece<HQ_Q8_0_X2>& p, int, const 
 }
 __device__ __forceinline__ float dot_pair(const Piece<HQ_Q8_0_X2>&, int, const uint32_t*, const float*, uint32_t, uint32_t, uint32_t) {
     return 0.f;
+}
+
+// Doubled pieces: the base type's dot product of either half, each over its own activations (the second half's follow
+// the first's in xp / xf and sx), added.
+template <int TYPE>
+__device__ __forceinline__ float dot_pair(const Piece<TYPE>& p, int c, const uint32_t* xp, const float* sx, uint32_t m4, uint32_t m2,
+                                          uint32_t magic) {
+    constexpr int B = kBaseType<TYPE>;
+    return dot_pair(p.a, c, xp, sx, m4, m2, magic) + dot_pair(p.b, c, xp + (kBlock32<B> ? 16 : 32), sx + (kBlock32<B> ? 2 : 4), m4, m2, magic);
+}
+template <int TYPE>
+__device__ __forceinline__ float dot_f32(const Piece<TYPE>& p, int c, const float* xf, const float* sx) {
+    constexpr int B = kBaseType<TYPE>;
+    return dot_f32(p.a, c, xf, sx) + dot_f32(p.b, c, xf + (kBlock32<B> ? 32 : 64), sx + (kBlock32<B> ? 2 : 4));
 }
 
 // Staging of one activation row in LDS, 16 activations per thread and pass:

@@ -20,17 +20,25 @@ namespace hq {
 namespace {
 
 template <int TYPE>
-constexpr bool kLaneUnit = kBlock32<TYPE> || TYPE == HQ_Q8_0_X2;  // a unit is one lane's piece
+constexpr bool kLaneUnit = kBlock32<kBaseType<TYPE>>;  // a unit is one lane's piece
 template <int TYPE>
 constexpr uint32_t kLanesPerUnit = kLaneUnit<TYPE> ? 1u : 4u;
 template <int TYPE>
 constexpr uint32_t kUnitsPerWindow = 64u / kLanesPerUnit<TYPE>;
 template <int TYPE>
-constexpr uint32_t kUnitElems = kBlock32<TYPE> ? 32u : TYPE == HQ_Q8_0_X2 ? 64u : 256u;
+constexpr uint32_t kUnitElems = (kLaneUnit<TYPE> ? 32u : 256u) * (kIsX2<TYPE> ? 2u : 1u);
 
-// Q8_0 rows of whole block pairs are walked as pairs (HQ_Q8_0_X2) from about a window per wave of the device on; the same
-// rule wherever the walk is used, so that every caller gets the same sums.
-inline bool q80_walk_in_pairs(uint64_t n_total, uint32_t k) { return k % 64u == 0 && n_total * (k / 64u) >= 64ull * 4096ull; }
+// Whether rows of type t are walked with doubled pieces (kX2 + t): the 32-weight block types (Q8_0 12288 x 4096: 15.9 ->
+// 12.4 us; the K-quants, whose pieces are larger and whose arithmetic is heavier, lose 7 .. 50 % to the registers a
+// doubled piece takes), rows of whole doubled units, about a window per wave of the device or more.  The same rule
+// wherever the walk is used, so that every caller gets the same sums.
+template <int TYPE, bool X_BF16>
+inline bool walk_doubled(uint64_t n_total, uint32_t k) {
+    static_assert(!kIsX2<TYPE>, "asked of the base type");
+    if (!kBlock32<TYPE>) return false;
+    constexpr uint32_t UE2 = 2u * kUnitElems<TYPE>;
+    return k % UE2 == 0 && n_total * (k / UE2) >= (uint64_t)kUnitsPerWindow<TYPE> * 4096ull;
+}
 
 struct FlatGeom {
     uint32_t bu;     // units per row
@@ -85,7 +93,7 @@ inline FlatGeom flat_geom(uint32_t k, uint32_t unit_elems, uint32_t uw, uint32_t
 // halves 17 / 40 apart) so that those sixteen lanes hit sixteen different 16-byte bank groups and every chunk of a
 // piece is an immediate offset from the lane's one base address.
 template <int TYPE, bool X_BF16>
-struct FlatX {
+struct FlatX1 {
     static constexpr bool PAIR = X_BF16 && TYPE != HQ_Q8_0 && TYPE != HQ_Q8_0_X2;
     static constexpr int XW = PAIR ? (kBlock32<TYPE> ? 16 : 32) : (kBlock32<TYPE> ? 32 : 64);  // registers of one lane's activations
     static constexpr uint32_t CA = PAIR ? 8u : 4u;                                              // activations per chunk
@@ -217,6 +225,29 @@ struct FlatX {
     }
 };
 
+// Base types (and the Q8_0 block pair, which has a piece and a layout of its own): as above.  The other doubled types:
+// the base type's layout, a lane's activations are those of unit 2 ur and of unit 2 ur + 1.
+template <int TYPE, bool X_BF16, bool = (kIsX2<TYPE> && TYPE != HQ_Q8_0_X2)>
+struct FlatX : FlatX1<TYPE, X_BF16> {};
+template <int TYPE, bool X_BF16>
+struct FlatX<TYPE, X_BF16, true> {
+    using B = FlatX1<kBaseType<TYPE>, X_BF16>;
+    static constexpr bool PAIR = B::PAIR;
+    static constexpr int XW = 2 * B::XW;
+    static constexpr int RUNS1 = kBlock32<kBaseType<TYPE>> ? 2 : 4;
+    static constexpr uint32_t CA = B::CA, G = B::G;
+    static __host__ __device__ __forceinline__ uint32_t slot(uint32_t ch) { return B::slot(ch); }
+    static __host__ __device__ __forceinline__ size_t value_bytes(uint32_t k) { return B::value_bytes(k); }
+    static __host__ __device__ __forceinline__ size_t lds_bytes(uint32_t k) { return B::lds_bytes(k); }
+    static __device__ __forceinline__ void stage(const void* x, uint32_t k, uint4* lds_x, float* lds_s, uint32_t tid, uint32_t nthreads) {
+        B::stage(x, k, lds_x, lds_s, tid, nthreads);
+    }
+    static __device__ __forceinline__ void load(const uint4* lds_x, const float* lds_s, uint32_t ur, int c, uint32_t* xr, float* sx) {
+        B::load(lds_x, lds_s, 2u * ur, c, xr, sx);
+        B::load(lds_x, lds_s, 2u * ur + 1u, c, xr + B::XW, sx + RUNS1);
+    }
+};
+
 // XHALF: f32 activations of a K-quant are read from LDS 32 at a time (half the registers; the same sums).
 // DYN (D == 1): the waves of a workgroup take the workgroup's super-tasks from a counter in LDS instead of a fixed split.
 // The SIMD's issue arbitration favours its oldest wave, so with equal shares the youngest wave of every SIMD finishes long
@@ -328,9 +359,9 @@ struct FlatWalk {
         uint32_t c_m = 0, c_w = 0, done = 0;
         float keep0 = 0.f, keep1 = 0.f;
         uint32_t keep_row = 0;
-        constexpr bool HALVES = XHALF && !X::PAIR && !kLaneUnit<TYPE>;
+        constexpr bool HALVES = XHALF && !X::PAIR && !kLaneUnit<TYPE> && !kIsX2<TYPE>;
         uint32_t xr[HALVES ? 32 : X::XW];
-        float sx[4] = {0.f, 0.f, 0.f, 0.f};
+        float sx[kIsX2<TYPE> ? 8 : 4] = {};
         // every window is one whole row (and not a ragged one): the lane's activations never change
         const bool xinv = !HALVES && g.st == 1u && g.log_r == 0u && g.uwe == g.bu;
         if constexpr (!HALVES)
