@@ -422,6 +422,36 @@ __device__ __forceinline__ void stream_load_x(const uint4* lds_x, const float* l
     }
 }
 
+// ROWS bf16 activation rows of k values into LDS as paired words (16 per thread and pass) with their per-16 sums.
+template <int TYPE, int ROWS>
+__device__ __forceinline__ void stream_stage_x(const void* x, uint32_t k, uint4* lds_x, float* lds_s, uint32_t tid, uint32_t nt) {
+    for (uint32_t ii = tid; ii < ROWS * (k / 16u); ii += nt) {
+        const uint32_t xr = ROWS == 1 ? 0u : ii / (k / 16u), i = ROWS == 1 ? ii : ii % (k / 16u);
+        XRaw<true> raw;
+        raw.fetch(static_cast<const uint8_t*>(x) + (size_t)xr * k * 2u, i);
+        const uint4 p = raw.r[0], q = raw.r[1];
+        const uint32_t w[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
+        uint4 o0, o1;
+        o0.x = (w[0] & 0xffffu) | (w[1] << 16);
+        o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
+        o0.z = (w[2] & 0xffffu) | (w[3] << 16);
+        o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
+        o1.x = (w[4] & 0xffffu) | (w[5] << 16);
+        o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
+        o1.z = (w[6] & 0xffffu) | (w[7] << 16);
+        o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
+        lds_x[xr * (k / 8u) + stream_swz<TYPE>(2 * i)] = o0;
+        lds_x[xr * (k / 8u) + stream_swz<TYPE>(2 * i + 1)] = o1;
+        float sum = 0.f;  // the same order of additions as stage_store
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            sum += bf16_bits_to_f32(w[j] & 0xffffu);
+            sum += bf16_bits_to_f32(w[j] >> 16);
+        }
+        lds_s[xr * (k / 16u) + i] = sum;
+    }
+}
+
 // ROWS = 2 .. 4: that many activation rows (x[r] -> y[r] of one matrix) share every weight fetch and the
 // nibble-to-bf16 work; the dot products and sums are per row, in the order of the one-row form.  Three and four rows
 // read their activations from LDS per piece (in registers they would be 32 each per row).
@@ -441,31 +471,7 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     const uint32_t ntask = rows_mine * S;
 
     // the activations first, nothing else of this workgroup in front of them
-    for (uint32_t ii = tid; ii < ROWS * (a.k / 16u); ii += NT) {
-        const uint32_t xr = ROWS == 1 ? 0u : ii / (a.k / 16u), i = ROWS == 1 ? ii : ii % (a.k / 16u);
-        XRaw<true> raw;
-        raw.fetch(static_cast<const uint8_t*>(a.x) + (size_t)xr * a.k * 2u, i);
-        const uint4 p = raw.r[0], q = raw.r[1];
-        const uint32_t w[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
-        uint4 o0, o1;
-        o0.x = (w[0] & 0xffffu) | (w[1] << 16);
-        o0.y = (w[0] >> 16) | (w[1] & 0xffff0000u);
-        o0.z = (w[2] & 0xffffu) | (w[3] << 16);
-        o0.w = (w[2] >> 16) | (w[3] & 0xffff0000u);
-        o1.x = (w[4] & 0xffffu) | (w[5] << 16);
-        o1.y = (w[4] >> 16) | (w[5] & 0xffff0000u);
-        o1.z = (w[6] & 0xffffu) | (w[7] << 16);
-        o1.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
-        lds_x[xr * (a.k / 8u) + stream_swz<TYPE>(2 * i)] = o0;
-        lds_x[xr * (a.k / 8u) + stream_swz<TYPE>(2 * i + 1)] = o1;
-        float s = 0.f;  // the same order of additions as stage_store
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            s += bf16_bits_to_f32(w[j] & 0xffffu);
-            s += bf16_bits_to_f32(w[j] >> 16);
-        }
-        lds_s[xr * (a.k / 16u) + i] = s;
-    }
+    stream_stage_x<TYPE, ROWS>(a.x, a.k, lds_x, lds_s, tid, NT);
 
     // One piece per lane in flight, refilled after every use (past the wave's last task: the last task again, not
     // used).  Results are not stored row by row from lane 0 but kept, lane i the wave's row i, and stored 64 rows at a
@@ -537,6 +543,103 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
 }
 
 
+// Q6_K rows of k = 4096 (3360 bytes, a multiple of 16), bf16 activations: the streaming kernel above with the weights
+// fetched differently.  A lane fetching its own piece touches a row's 128-byte lines with five instructions; here a wave
+// copies a row as 210 consecutive 16-byte pieces (four non-temporal loads per lane: each line is asked for once and
+// not kept in the caches) into 4 KB of LDS it owns, and its lanes read their pieces back from there.  A wave takes
+// groups of FOUR consecutive rows, 13440 bytes = 105 whole lines, so that no line is shared with another wave (a
+// non-temporal line fetched by two waves crosses the memory system twice).  Read alone this way the 510 MB matrix takes
+// 75 us, with the lanes fetching their own pieces 82-84.  The blocks lie in LDS as in memory, 210 bytes apart, so a
+// lane's fields start at even addresses: each is read as aligned words and shifted into place by v_alignbyte.  The
+// pieces, the dot products and the order of the sums are those of gemv_stream_kernel: the same bits.
+constexpr int Q6K_LDS_WAVES = 16;
+__global__ __launch_bounds__(64 * Q6K_LDS_WAVES) void gemv_q6k_rowcopy_kernel(SArgs a) {
+    constexpr uint32_t W = Q6K_LDS_WAVES, NT = 64 * W, ROWB = 16u * Q6K_BYTES, PIECES = ROWB / 16u;  // 3360 bytes, 210 pieces
+    extern __shared__ uint4 smem[];
+    uint4* lds_x = smem;                                           // [k / 8]
+    float* lds_s = reinterpret_cast<float*>(lds_x + 4096u / 8u);   // [k / 16]
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    uint4* wbuf = reinterpret_cast<uint4*>(lds_s + 4096u / 16u) + wv * 256u;  // this wave's row: 256 slots of 16 bytes
+    const int c = (int)(lane & 3u);
+    const uint32_t groups = (a.n + 3u) / 4u, stride = W * gridDim.x;
+    const uint32_t g_first = wv * gridDim.x + blockIdx.x;
+    const uint32_t groups_mine = g_first < groups ? (groups - g_first + stride - 1u) / stride : 0u;
+    const uint32_t ntask = groups_mine * 4u;
+
+    stream_stage_x<HQ_Q6_K, 1>(a.x, 4096u, lds_x, lds_s, tid, NT);
+
+    // task t of this wave: row 4 (g_first + (t / 4) stride) + t % 4, clamped to the matrix (a clamped row is not stored)
+    auto row_of = [&](uint32_t t) { return 4u * (g_first + (t >> 2) * stride) + (t & 3u); };
+    uint4 pv[4];
+    auto fetch = [&](uint32_t t) {
+        uint32_t row = row_of(t);
+        row = row < a.n ? row : a.n - 1u;
+        const uint8_t* base = (row < a.n0 ? a.w0 + (size_t)row * ROWB : a.w1 + (size_t)(row - a.n0) * ROWB);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t pc = lane + 64u * (uint32_t)i;
+            pv[i] = ldnt16(base + 16u * (pc < PIECES ? pc : PIECES - 1u));
+        }
+    };
+    if (ntask) fetch(0);
+    __syncthreads();
+
+    uint32_t m4, m2, magic;
+    asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5" : "=v"(m4), "=v"(m2), "=v"(magic) : "s"(a.m4), "s"(a.m2), "s"(a.magic));
+    uint32_t xp[32];
+    float sx[4];
+    stream_load_x<HQ_Q6_K>(lds_x, lds_s, 0, lane, c, xp, sx);
+
+    // this lane's piece in the row buffer: block lane / 4 at byte 210 (lane / 4), fields at even offsets; sh = the bytes by
+    // which a field's first aligned word starts early (0 or 2)
+    const uint32_t blk = (lane >> 2) * Q6K_BYTES, h = (uint32_t)c >> 1, lr = (uint32_t)c & 1u;
+    const uint32_t* wb32 = reinterpret_cast<const uint32_t*>(wbuf);
+    const uint32_t o_qa = blk + 64u * h + 16u * lr, o_qb = o_qa + 32u, o_qh = blk + 128u + 32u * h + 16u * lr, o_sc = blk + 192u + 8u * h,
+                   o_d = blk + 206u;
+    auto field16 = [&](uint32_t o) -> uint4 {
+        const uint32_t* p = wb32 + (o >> 2);
+        const uint32_t sh = o & 3u, w0 = p[0], w1 = p[1], w2 = p[2], w3 = p[3], w4 = p[4];
+        return make_uint4(__builtin_amdgcn_alignbyte(w1, w0, sh), __builtin_amdgcn_alignbyte(w2, w1, sh), __builtin_amdgcn_alignbyte(w3, w2, sh),
+                          __builtin_amdgcn_alignbyte(w4, w3, sh));
+    };
+
+    uint32_t done = 0;
+    float keep = 0.f;
+    auto flush = [&](uint32_t first, uint32_t count) {
+        if (lane < count) {
+            const uint32_t row = row_of(first + lane);
+            if (row < a.n) {
+                if (row < a.n0) a.y0[row] = keep;
+                else a.y1[row - a.n0] = keep;
+            }
+        }
+    };
+    for (uint32_t t = 0; t < ntask; ++t) {
+        // the row fetched a task ago goes to LDS (the wave's earlier reads of the buffer precede these writes: one wave's
+        // LDS operations are served in order), the next row's fetch is issued, then this row's pieces are read back
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wbuf[lane + 64u * (uint32_t)i] = pv[i];
+        asm volatile("" ::: "memory");  // (for the compiler: the reads below are of what was just written)
+        if (t + 1u < ntask) fetch(t + 1u);
+        Piece<HQ_Q6_K> pc;
+        pc.qa = field16(o_qa);
+        pc.qb = field16(o_qb);
+        pc.qh = field16(o_qh);
+        {
+            const uint32_t* p = wb32 + (o_sc >> 2);
+            const uint32_t sh = o_sc & 3u, w0 = p[0], w1 = p[1], w2 = p[2];
+            pc.sc = make_uint2(__builtin_amdgcn_alignbyte(w1, w0, sh), __builtin_amdgcn_alignbyte(w2, w1, sh));
+            const uint32_t* q = wb32 + (o_d >> 2);
+            pc.d = __builtin_amdgcn_alignbyte(q[1], q[0], o_d & 3u);
+        }
+        const float v = group_sum(dot_pair(pc, c, xp, sx, m4, m2, magic), 6);
+        keep = lane == (done & 63u) ? v : keep;
+        if ((++done & 63u) == 0u) flush(done - 64u, 64u);
+    }
+    if (done & 63u) flush(done & ~63u, done & 63u);
+}
+
 // Whether the streaming form takes (type, k, rows): K-quants, whole 4096-element steps, enough rows to occupy the waves.
 template <int TYPE>
 constexpr bool kStreamType = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K;
@@ -549,6 +652,16 @@ int launch_stream(hipStream_t s, const SArgs& sa, uint32_t cus) {
     // (three and four rows in registers would spill, so would the two-row Q5_K form: not instantiated)
     constexpr bool XREG_FITS = ROWS <= 2 && !(TYPE == HQ_Q5_K && ROWS == 2);
     bool launched = false;
+    if constexpr (TYPE == HQ_Q6_K && ROWS == 1) {
+        // rows of 3360 bytes from a 16-byte aligned matrix, many rows per wave: the row-copy form
+        if (sa.k == 4096 && sa.n0 == sa.n && (reinterpret_cast<uintptr_t>(sa.w0) & 15u) == 0 && sa.n >= 64u * Q6K_LDS_WAVES * cus / 4u) {
+            const size_t lds_rc = lds + (size_t)Q6K_LDS_WAVES * 4096u;
+            if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(gemv_q6k_rowcopy_kernel), lds_rc, "hipFuncSetAttribute(gemv row-copy LDS)"))
+                return rc;
+            hipLaunchKernelGGL(gemv_q6k_rowcopy_kernel, dim3(cus), dim3(64 * Q6K_LDS_WAVES), lds_rc, s, sa);
+            return check_launch("gemv row-copy kernel launch");
+        }
+    }
     if constexpr (XREG_FITS) {
         if (sa.k == 4096) {
             auto kern = gemv_stream_kernel<TYPE, W, true, ROWS>;

@@ -245,6 +245,31 @@ __device__ __forceinline__ uint32_t ld4_unaligned(const uint8_t* p) {
 __device__ __forceinline__ uint32_t ld2(const uint8_t* p) {
     return *reinterpret_cast<const uint16_t*>(p);
 }
+// The same loads marked non-temporal, for data a kernel reads exactly once (the weights of a single-row product): the
+// lines are not kept in the caches on their way in, and a streaming read of 510 MB runs at 6.9 instead of 6.0 TB/s.
+typedef uint32_t hq_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t hq_u32x2 __attribute__((ext_vector_type(2)));
+typedef hq_u32x4 hq_u32x4_a2 __attribute__((aligned(2)));
+typedef hq_u32x2 hq_u32x2_a2 __attribute__((aligned(2)));
+typedef uint32_t hq_u32_a2 __attribute__((aligned(2)));
+__device__ __forceinline__ uint4 ldnt16(const uint8_t* p) {  // 16-byte aligned
+    const hq_u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const hq_u32x4*>(p));
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ uint4 ldnt16_unaligned(const uint8_t* p) {  // 2-byte aligned, like the ones below
+    const hq_u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const hq_u32x4_a2*>(p));
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ uint2 ldnt8_unaligned(const uint8_t* p) {
+    const hq_u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const hq_u32x2_a2*>(p));
+    return make_uint2(t.x, t.y);
+}
+__device__ __forceinline__ uint32_t ldnt4_unaligned(const uint8_t* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const hq_u32_a2*>(p));
+}
+__device__ __forceinline__ uint32_t ldnt2(const uint8_t* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(p));
+}
 
 // a.x*b.x + a.y*b.y + c on two packed bf16 pairs, f32 accumulate (v_dot2c_f32_bf16).
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
