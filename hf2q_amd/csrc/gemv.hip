@@ -455,9 +455,15 @@ __device__ __forceinline__ void stream_stage_x(const void* x, uint32_t k, uint4*
 // ROWS = 2 .. 4: that many activation rows (x[r] -> y[r] of one matrix) share every weight fetch and the
 // nibble-to-bf16 work; the dot products and sums are per row, in the order of the one-row form.  Three and four rows
 // read their activations from LDS per piece (in registers they would be 32 each per row).
-template <int TYPE, int W, bool XREG, int ROWS = 1>
+// COPY (Q4_K / Q5_K, whose blocks are whole 16-byte pieces and whose steps of sixteen blocks are whole 128-byte lines:
+// 2304 / 2816 bytes): a step is not fetched by the lanes that use it, three to five instructions touching each line,
+// but copied -- consecutive lanes consecutive 16-byte pieces, non-temporal loads, every line asked for once -- into 3 KB
+// of LDS the wave owns and read back from there as the same pieces; the next step's copy is in flight meanwhile.
+template <int TYPE, int W, bool XREG, int ROWS = 1, bool COPY = false>
 __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
+    static_assert(!COPY || TYPE == HQ_Q4_K || TYPE == HQ_Q5_K, "blocks of whole 16-byte pieces");
     constexpr uint32_t NT = 64 * W, BB = kBlockBytes<TYPE>;
+    constexpr uint32_t PIECES = 16u * BB / 16u, NPV = (PIECES + 63u) / 64u;  // 16-byte pieces of a step; per lane
     extern __shared__ uint4 smem[];
     uint4* lds_x = smem;                                                // [ROWS][k / 8]
     float* lds_s = reinterpret_cast<float*>(lds_x + ROWS * (a.k / 8));  // [ROWS][k / 16]
@@ -478,10 +484,21 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     // time: no store among the fetches, and the loop has one path.  (Two and three pieces in flight were measured,
     // with every wait of the loop allowing for the younger fetches: 103 against 94 us on the 151936 x 4096 Q6_K matrix.)
     Piece<TYPE> pc;
+    [[maybe_unused]] uint4 pv[COPY ? NPV : 1];
+    // (COPY: the wave's step buffer, 64 * NPV slots of 16 bytes, behind the activations and their sums)
+    [[maybe_unused]] uint4* wbuf = reinterpret_cast<uint4*>(lds_s + ROWS * (a.k / 16)) + wv * (64u * NPV);
     uint32_t f_row = row_first, f_st = 0, f_left = ntask;  // the next task to fetch; tasks not yet fetched
     auto fetch_next = [&](Piece<TYPE>& p) {
         const uint8_t* base = f_row < a.n0 ? a.w0 + (size_t)f_row * rowb : a.w1 + (size_t)(f_row - a.n0) * rowb;
-        p.load(base + (f_st * 16u + (lane >> 2)) * BB, c);
+        if constexpr (COPY) {
+#pragma unroll
+            for (uint32_t i = 0; i < NPV; ++i) {
+                const uint32_t pi = lane + 64u * i;
+                pv[i] = ldnt16(base + (size_t)f_st * (16u * BB) + 16u * (pi < PIECES ? pi : PIECES - 1u));
+            }
+        } else {
+            p.load(base + (f_st * 16u + (lane >> 2)) * BB, c);
+        }
         if (f_left > 1u) {  // (scalar: no memory operation inside)
             --f_left;
             if (++f_st == S) {
@@ -519,6 +536,25 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
         }
     };
     auto task = [&](Piece<TYPE>& p) {
+        if constexpr (COPY) {
+            // the copied step goes to LDS (behind the wave's reads of the previous one: a wave's LDS operations are served
+            // in order), the next step's copy is issued, this step's pieces are read back
+#pragma unroll
+            for (uint32_t i = 0; i < NPV; ++i) wbuf[lane + 64u * i] = pv[i];
+            asm volatile("" ::: "memory");
+            fetch_next(p);
+            const uint4* blk = wbuf + (lane >> 2) * (BB / 16u);
+            p.hdr = blk[0];
+            if constexpr (TYPE == HQ_Q5_K) {
+                p.h0 = blk[1];
+                p.h1 = blk[2];
+                p.q0 = blk[3 + 2 * c];
+                p.q1 = blk[4 + 2 * c];
+            } else {
+                p.q0 = blk[1 + 2 * c];
+                p.q1 = blk[2 + 2 * c];
+            }
+        }
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
             if constexpr (!XREG) stream_load_x<TYPE>(lds_x + r * (a.k / 8u), lds_s + r * (a.k / 16u), st, lane, c, xp[r], sx[r]);
@@ -526,7 +562,7 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
         }
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) asm volatile("" : "+v"(acc[r]));  // the refill follows the arithmetic that frees its registers
-        fetch_next(p);
+        if constexpr (!COPY) fetch_next(p);
         if (++st == S) {
 #pragma unroll
             for (int r = 0; r < ROWS; ++r) {
@@ -660,6 +696,16 @@ int launch_stream(hipStream_t s, const SArgs& sa, uint32_t cus) {
                 return rc;
             hipLaunchKernelGGL(gemv_q6k_rowcopy_kernel, dim3(cus), dim3(64 * Q6K_LDS_WAVES), lds_rc, s, sa);
             return check_launch("gemv row-copy kernel launch");
+        }
+    }
+    if constexpr ((TYPE == HQ_Q4_K || TYPE == HQ_Q5_K) && ROWS == 1) {
+        // (Q4_K 12288 x 4096: 7.75 -> 7.4 us, 151936 x 4096: 63 -> 59 us; Q5_K 12288 x 4096: 9.07 -> 8.46 us; the same bits)
+        if (((reinterpret_cast<uintptr_t>(sa.w0) | reinterpret_cast<uintptr_t>(sa.w1)) & 15u) == 0) {
+            constexpr size_t wbytes = (size_t)W * 64u * ((kBlockBytes<TYPE> + 63u) / 64u) * 16u;
+            auto kern = sa.k == 4096 ? gemv_stream_kernel<TYPE, W, true, 1, true> : gemv_stream_kernel<TYPE, W, false, 1, true>;
+            if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds + wbytes, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
+            hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds + wbytes, s, sa);
+            return check_launch("gemv stream kernel launch");
         }
     }
     if constexpr (XREG_FITS) {

@@ -610,7 +610,7 @@ HQ_API int hq_dense_matmul(void* stream, const void* x, hq_act_dtype xdt, const 
 
 /* ---- measurement aid ---- */
 
-/* Reads `bytes` (a multiple of 16) of device memory at `buf` (16-byte aligned) once with plain 16-byte loads, eight
+/* Reads `bytes` (a multiple of 16) of device memory at `buf` (16-byte aligned) once with non-temporal 16-byte loads, eight
  * workgroups of four waves per CU walking the buffer front to back in runs of 8 KiB, and nothing else: the time of this launch over a buffer the caches do not hold is
  * what streaming that many bytes costs on the device, the rate the bandwidth-bound kernels of this library can be read
  * against beside the published peak.  `sink`: 4 writable bytes (written only if the data xor to a value they do not).
