@@ -64,12 +64,12 @@ def test_decode_gemv_full_size(oracle, dev, n, k, t, m):
     assert torch.equal(run(xa * 4.0), ya * 4.0)
 
 
-@pytest.mark.parametrize("n", [65536, 65539, 70001, 70002])
+@pytest.mark.parametrize("n", [8192, 65539, 70001, 70002])
 def test_q6k_head_rows_copied_through_lds(oracle, dev, n):
-    """Q6_K matrices of 4096 columns with 65536 rows or more and one bf16 activation row: a wave copies groups of four
+    """Q6_K matrices of 4096 columns with 8192 rows or more and one bf16 activation row: a wave copies groups of four
     whole rows through LDS.  Row counts that leave the last group with 4, 3, 1 and 2 rows; every output row against the
-    same rows as a matrix of their own below the size that takes this form (the other kernel, which gives the same bits),
-    sampled rows against the f64 oracle."""
+    two-row pass over the same activations twice (the kernel whose lanes fetch their own pieces, which gives the same
+    bits), sampled rows against the f64 oracle."""
     k, t = 4096, HQ_Q6_K
     w = _quantized(dev, n, k, t, 3 + n)
     rng = np.random.default_rng(n)
@@ -78,13 +78,9 @@ def test_q6k_head_rows_copied_through_lds(oracle, dev, n):
     y = torch.full((1, n), float("nan"), device=dev)
     ops.quantized_matmul_ggml(xd, w, y, GgmlQuantizedMatmulParams(1, n, k, t))
     assert torch.isfinite(y).all()
-    rb = k // 256 * 210
-    half = 32768  # rows per slice: below the form's threshold
-    for r0 in range(0, n, half):
-        r1 = min(n, r0 + half)
-        part = torch.full((1, r1 - r0), float("nan"), device=dev)
-        ops.quantized_matmul_ggml(xd, w[r0 * rb:r1 * rb], part, GgmlQuantizedMatmulParams(1, r1 - r0, k, t))
-        assert torch.equal(part, y[:, r0:r1]), f"rows {r0}..{r1}"
+    y2 = torch.full((2, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(torch.cat([xd, xd]), w, y2, GgmlQuantizedMatmulParams(2, n, k, t))
+    assert torch.equal(y2[0:1], y) and torch.equal(y2[1:2], y)
     rows = np.unique(np.concatenate([[0, 1, 2, 3, n - 4, n - 3, n - 2, n - 1], rng.integers(0, n, 40)]))
     ref = oracle.qmatmul_f64(oracle.f32_to_bf16_bits(x), _rows_of(w, rows, k, t, oracle), 1, rows.size, k, t)
     assert_matmul_close(y[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, f"q6_k {n}x{k}, sampled rows")
