@@ -32,6 +32,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
+SETTLE_STEPS = 2400  # untimed decode steps before the steady-state measurements of the decode workload (about 0.25 s)
 
 # HBM bytes per launch of the dominant kernel of each workload, from rocprofv3 --pmc runs of this
 # file (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
@@ -840,6 +841,18 @@ def bench_decode_gemv(a):
         fused_step(i)
     torch.cuda.synchronize()
 
+    # The same K steps as the region behind `value` below, timed here, a few milliseconds of work after set-up: the
+    # device is not at its steady rate yet (the same steps get faster over the first 100-200 ms of continuous work
+    # after an idle period: 108 -> 98 us per step in one process), so this figure is reported beside `value`, which
+    # is measured after the per-kernel measurements that follow, as a decode loop of more than a second sees the device.
+    first_region_us = None
+    if not a.no_graph:
+        el_first, _ = _timed_steps(a, fused_step, n_sets * n_heads)
+        first_region_us = el_first / a.steps * 1e6
+    for i in range(SETTLE_STEPS):  # untimed: about a quarter of a second of decode steps
+        fused_step(i)
+    torch.cuda.synchronize()
+
     # K steps launched one kernel at a time from the host (Python + ctypes per launch).
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -849,14 +862,6 @@ def bench_decode_gemv(a):
     el_host = time.perf_counter() - t0
     host = {"ms_per_step": round(el_host / a.steps * 1e3, 4), "GBps": round(step_bytes * a.steps / el_host / 1e9, 1),
             "frac_hbm_peak": round(step_bytes * a.steps / el_host / 1e9 / HBM_PEAK_GBS, 4)}
-
-    # The timed region behind `value`: exactly K steps replayed from HIP graphs of their three launches
-    # (runs of consecutive steps over the rotated weight sets and heads), as a decode loop that records
-    # its token step does; the host's per-launch cost (Python, ctypes) is then out of the way, like in
-    # the other workloads.
-    elapsed, step_us_events = el_host, None
-    if not a.no_graph:
-        elapsed, step_us_events = _timed_steps(a, fused_step, n_sets * n_heads)
 
     # Per-kernel durations behind `roofline` and `kernels`: HIP events around back-to-back launches of ONE kernel
     # over distinct matrices (every set's gate and up for the 12288 x 4096 shape: 2 * n_sets * 28 MB, the sets'
@@ -957,6 +962,14 @@ def bench_decode_gemv(a):
     probe["what"] = ("one plain read of the same buffers, 16 bytes per lane, no arithmetic (hq_stream_read_probe), timed like `kernels`: the "
                      "streaming rate this device reaches; kernels[...].us / this us = how far a kernel is from it")
 
+    # The timed region behind `value`: exactly K steps replayed from HIP graphs of their three launches
+    # (runs of consecutive steps over the rotated weight sets and heads), as a decode loop that records
+    # its token step does; the host's per-launch cost (Python, ctypes) is then out of the way, like in
+    # the other workloads.
+    elapsed, step_us_events = el_host, None
+    if not a.no_graph:
+        elapsed, step_us_events = _timed_steps(a, fused_step, n_sets * n_heads)
+
     value = step_bytes * a.steps / elapsed / 1e9
     head_us = kern_us["head_151936x4096"]
     head_gbs = nbytes["head"] / head_us / 1e3
@@ -979,7 +992,10 @@ def bench_decode_gemv(a):
                                   "gate + up in one batched launch, down, head = 3 launches replayed as a HIP graph"),
                    "bytes_per_step": step_bytes, "weight_sets": n_sets, "head_copies": n_heads,
                    "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-                   "step_us_by_hip_events": None if step_us_events is None else round(step_us_events, 2)},
+                   "step_us_by_hip_events": None if step_us_events is None else round(step_us_events, 2),
+                   "timed_after": f"{a.warmup} warm-up steps, {SETTLE_STEPS} more untimed steps and the per-kernel measurements of this line "
+                                  "(the device at its steady rate)",
+                   "us_per_step_first_region": None if first_region_us is None else round(first_region_us, 2)},
         "roofline": {"bound": "hbm", "kernel": "gemv Q6_K head 151936x4096", "achieved": round(head_gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head_gbs / HBM_PEAK_GBS, 4),
                      "traffic": PMC_TRAFFIC_BYTES["gemv_head_q6_k_151936x4096"],
