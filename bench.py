@@ -864,21 +864,37 @@ def bench_decode_gemv(a):
             "frac_hbm_peak": round(step_bytes * a.steps / el_host / 1e9 / HBM_PEAK_GBS, 4)}
 
     # Per-kernel durations behind `roofline` and `kernels`: HIP events around back-to-back launches of ONE kernel
-    # over distinct matrices (every set's gate and up for the 12288 x 4096 shape: 2 * n_sets * 28 MB, the sets'
-    # down matrices, the two heads twice), see _launch_us.
+    # over distinct matrices, see _launch_us.  The 28 MB shapes rotate over all 3 * n_sets FFN buffers (a buffer of
+    # Q4_K blocks reads as 12288 x 4096 or as 4096 x 12288 alike): 510 MB between two uses of a buffer, twice the
+    # 256 MB Infinity Cache -- over the six down matrices alone (170 MB) a kernel that fetches with ordinary loads
+    # finds them there (4096 x 12288 with f32 activations: 7.7 instead of 8.6 us).
+    ffn_bufs = [ws[nm] for ws in sets for nm in ("gate", "up", "down")]
     kern_us = {
-        "gate_up_12288x4096": _launch_us([one(nm, ws[nm]) for ws in sets for nm in ("gate", "up")] * 4),
-        "down_4096x12288": _launch_us([one("down", ws["down"]) for ws in sets] * 8),
+        "gate_up_12288x4096": _launch_us([one("gate", b) for b in ffn_bufs] * 3),
+        "down_4096x12288": _launch_us([one("down", b) for b in ffn_bufs] * 3),
         "head_151936x4096": _launch_us([one("head", h) for h in heads] * 8),
         "gate_and_up_one_launch": _launch_us([
-            (lambda ws=ws: ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x_h, ws["gate"], y["gate"], 1, F, H),
-                                                            ops.QmatmulJob(x_h, ws["up"], y["up"], 1, F, H)], HQ_Q4_K))
-            for ws in sets] * 8),
+            (lambda b0=b0, b1=b1: ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x_h, b0, y["gate"], 1, F, H),
+                                                                  ops.QmatmulJob(x_h, b1, y["up"], 1, F, H)], HQ_Q4_K))
+            for b0, b1 in zip(ffn_bufs[0::2], ffn_bufs[1::2])] * 5),
     }
     kbytes = {"gate_up_12288x4096": nbytes["gate"], "down_4096x12288": nbytes["down"], "head_151936x4096": nbytes["head"],
               "gate_and_up_one_launch": nbytes["gate"] + nbytes["up"]}
     kernels = {nm: {"us": round(kern_us[nm], 3), "bytes": kbytes[nm], "GBps": round(kbytes[nm] / kern_us[nm] / 1e3, 1),
                     "frac_hbm_peak": round(kbytes[nm] / kern_us[nm] / 1e3 / HBM_PEAK_GBS, 4)} for nm in kern_us}
+    # The same three matrices under f32 activations, the dtype the reference's call sites pass (gpu_full_attn.rs:835).
+    x_h32, x_f32 = x_h.float(), x_f.float()
+
+    def one32(nm, w):
+        return lambda: ops.quantized_matmul_ggml(x_f32 if nm == "down" else x_h32, w, y[nm], params[nm])
+
+    kern32_us = {
+        "gate_up_12288x4096": _launch_us([one32("gate", b) for b in ffn_bufs] * 3),
+        "down_4096x12288": _launch_us([one32("down", b) for b in ffn_bufs] * 3),
+        "head_151936x4096": _launch_us([one32("head", h) for h in heads] * 8),
+    }
+    kernels_f32 = {nm: {"us": round(us, 3), "bytes": kbytes[nm], "GBps": round(kbytes[nm] / us / 1e3, 1),
+                        "frac_hbm_peak": round(kbytes[nm] / us / 1e3 / HBM_PEAK_GBS, 4)} for nm, us in kern32_us.items()}
     q4_bytes = 2 * nbytes["gate"] + nbytes["down"]
     q4_us = 2 * kern_us["gate_up_12288x4096"] + kern_us["down_4096x12288"]
     q4_us_fewer = kern_us["gate_and_up_one_launch"] + kern_us["down_4096x12288"]
@@ -938,7 +954,7 @@ def bench_decode_gemv(a):
     small_batch = {}
     big = [make_weight(65536, H, HQ_Q4_K) for _ in range(4)]
     for nm, mats, (n_, k_, t_) in (("head_q6_k_151936x4096", heads, shapes["head"]), ("q4_k_65536x4096", big, (65536, H, HQ_Q4_K)),
-                                   ("gate_q4_k_12288x4096", [ws["gate"] for ws in sets] + [ws["up"] for ws in sets], shapes["gate"])):
+                                   ("gate_q4_k_12288x4096", ffn_bufs, shapes["gate"])):
         entry = {"bytes": mats[0].numel()}
         for m_ in (2, 4, 8):
             xm = torch.randn(m_, k_, generator=gx, device=dev, dtype=torch.float32).to(torch.bfloat16)
@@ -955,7 +971,7 @@ def bench_decode_gemv(a):
     # the published peak.
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     probe = {}
-    for nm, bufs, reps in (("head_510MB", heads, 8), ("gate_28MB", [ws["gate"] for ws in sets] + [ws["up"] for ws in sets], 4)):
+    for nm, bufs, reps in (("head_510MB", heads, 8), ("gate_28MB", ffn_bufs, 3)):
         us = _launch_us([(lambda b=b: ops.stream_read_probe(b, sink)) for b in bufs] * reps)
         nb_ = bufs[0].numel()
         probe[nm] = {"us": round(us, 3), "bytes": nb_, "GBps": round(nb_ / us / 1e3, 1), "frac_hbm_peak": round(nb_ / us / 1e3 / HBM_PEAK_GBS, 4)}
@@ -1002,6 +1018,7 @@ def bench_decode_gemv(a):
                      "traffic_source": "recorded: rocprofv3 --pmc runs of this file, profiles/gemv_decode_config2_pmc_traffic.md",
                      "us_per_launch": round(head_us, 3), "bytes_per_launch": nbytes["head"]},
         "kernels": kernels,
+        "kernels_f32_activations": kernels_f32,
         "host_launched": host,
         "q4_k_gemv": {"GBps": round(q4_bytes / q4_us / 1e3, 1), "frac_hbm_peak": round(q4_bytes / q4_us / 1e3 / HBM_PEAK_GBS, 4),
                       "what": "gate, up, down as three launches of their own (bf16 activations each)",

@@ -459,14 +459,19 @@ __device__ __forceinline__ void stream_stage_x(const void* x, uint32_t k, uint4*
 // 2304 / 2816 bytes): a step is not fetched by the lanes that use it, three to five instructions touching each line,
 // but copied -- consecutive lanes consecutive 16-byte pieces, non-temporal loads, every line asked for once -- into 3 KB
 // of LDS the wave owns and read back from there as the same pieces; the next step's copy is in flight meanwhile.
-template <int TYPE, int W, bool XREG, int ROWS = 1, bool COPY = false>
+// X_BF16 = false (one row, COPY): f32 activations, the dtype of the reference's call sites, staged and multiplied as in
+// the flat walk (a lane's 64 activations as f32, exact products; the same bits as that walk gives for these rows).
+template <int TYPE, int W, bool XREG, int ROWS = 1, bool COPY = false, bool X_BF16 = true>
 __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     static_assert(!COPY || TYPE == HQ_Q4_K || TYPE == HQ_Q5_K, "blocks of whole 16-byte pieces");
+    static_assert(X_BF16 || (ROWS == 1 && COPY), "f32 activations: the one-row copy form");
     constexpr uint32_t NT = 64 * W, BB = kBlockBytes<TYPE>;
     constexpr uint32_t PIECES = 16u * BB / 16u, NPV = (PIECES + 63u) / 64u;  // 16-byte pieces of a step; per lane
+    using XF = FlatX1<TYPE, false>;
     extern __shared__ uint4 smem[];
-    uint4* lds_x = smem;                                                // [ROWS][k / 8]
-    float* lds_s = reinterpret_cast<float*>(lds_x + ROWS * (a.k / 8));  // [ROWS][k / 16]
+    uint4* lds_x = smem;  // bf16: [ROWS][k / 8] paired words; f32: XF's layout
+    float* lds_s = X_BF16 ? reinterpret_cast<float*>(lds_x + ROWS * (a.k / 8))  // [ROWS][k / 16]
+                          : reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(smem) + XF::value_bytes(a.k));
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));  // the same in a wave: scalar loop control
     const int c = (int)(lane & 3u);
@@ -477,7 +482,8 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     const uint32_t ntask = rows_mine * S;
 
     // the activations first, nothing else of this workgroup in front of them
-    stream_stage_x<TYPE, ROWS>(a.x, a.k, lds_x, lds_s, tid, NT);
+    if constexpr (X_BF16) stream_stage_x<TYPE, ROWS>(a.x, a.k, lds_x, lds_s, tid, NT);
+    else XF::stage(a.x, a.k, lds_x, lds_s, tid, NT);
 
     // One piece per lane in flight, refilled after every use (past the wave's last task: the last task again, not
     // used).  Results are not stored row by row from lane 0 but kept, lane i the wave's row i, and stored 64 rows at a
@@ -510,15 +516,20 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
     if (ntask) fetch_next(pc);
     __syncthreads();
 
-    uint32_t m4, m2, magic;
-    asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
-                 : "=v"(m4), "=v"(m2), "=v"(magic)
-                 : "s"(a.m4), "s"(a.m2), "s"(a.magic));
-    uint32_t xp[ROWS][32];
+    [[maybe_unused]] uint32_t m4, m2, magic;
+    if constexpr (X_BF16)
+        asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5"
+                     : "=v"(m4), "=v"(m2), "=v"(magic)
+                     : "s"(a.m4), "s"(a.m2), "s"(a.magic));
+    uint32_t xp[ROWS][X_BF16 ? 32 : 64];
     float sx[ROWS][4];
+    auto load_x = [&](int r, uint32_t step) {
+        if constexpr (X_BF16) stream_load_x<TYPE>(lds_x + r * (a.k / 8u), lds_s + r * (a.k / 16u), step, lane, c, xp[r], sx[r]);
+        else XF::load(lds_x, lds_s, step * 16u + (lane >> 2), c, xp[r], sx[r]);
+    };
     if constexpr (XREG) {  // k == 4096: one piece per lane for every row
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) stream_load_x<TYPE>(lds_x + r * (a.k / 8u), lds_s + r * (a.k / 16u), 0, lane, c, xp[r], sx[r]);
+        for (int r = 0; r < ROWS; ++r) load_x(r, 0);
     }
 
     uint32_t st = 0, done = 0;  // step inside the row; rows finished
@@ -557,8 +568,9 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
         }
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
-            if constexpr (!XREG) stream_load_x<TYPE>(lds_x + r * (a.k / 8u), lds_s + r * (a.k / 16u), st, lane, c, xp[r], sx[r]);
-            acc[r] += dot_pair(p, c, xp[r], sx[r], m4, m2, magic);
+            if constexpr (!XREG) load_x(r, st);
+            if constexpr (X_BF16) acc[r] += dot_pair(p, c, xp[r], sx[r], m4, m2, magic);
+            else acc[r] += dot_f32(p, c, reinterpret_cast<const float*>(xp[r]), sx[r]);
         }
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) asm volatile("" : "+v"(acc[r]));  // the refill follows the arithmetic that frees its registers
@@ -579,55 +591,68 @@ __global__ __launch_bounds__(64 * W) void gemv_stream_kernel(SArgs a) {
 }
 
 
-// Q6_K rows of k = 4096 (3360 bytes, a multiple of 16), bf16 activations: the streaming kernel above with the weights
+// Q6_K rows of k = 4096 or 2048 elements (3360 / 1680 bytes, multiples of 16): the streaming kernel above with the weights
 // fetched differently.  A lane fetching its own piece touches a row's 128-byte lines with five instructions; here a wave
-// copies a row as 210 consecutive 16-byte pieces (four non-temporal loads per lane: each line is asked for once and
-// not kept in the caches) into 4 KB of LDS it owns, and its lanes read their pieces back from there.  A wave takes
-// groups of FOUR consecutive rows, 13440 bytes = 105 whole lines, so that no line is shared with another wave (a
-// non-temporal line fetched by two waves crosses the memory system twice).  Read alone this way the 510 MB matrix takes
-// 75 us, with the lanes fetching their own pieces 82-84.  The blocks lie in LDS as in memory, 210 bytes apart, so a
-// lane's fields start at even addresses: each is read as aligned words and shifted into place by v_alignbyte.  The
-// pieces, the dot products and the order of the sums are those of gemv_stream_kernel: the same bits.
-constexpr int Q6K_LDS_WAVES = 16;
-__global__ __launch_bounds__(64 * Q6K_LDS_WAVES) void gemv_q6k_rowcopy_kernel(SArgs a) {
-    constexpr uint32_t W = Q6K_LDS_WAVES, NT = 64 * W, ROWB = 16u * Q6K_BYTES, PIECES = ROWB / 16u;  // 3360 bytes, 210 pieces
+// copies a chunk of sixteen blocks (one row of 4096, two of 2048) as 210 consecutive 16-byte pieces (four non-temporal
+// loads per lane: each line is asked for once and not kept in the caches) into 4 KB of LDS it owns, and its lanes read
+// their pieces back from there.  A wave takes groups of FOUR consecutive chunks, 13440 bytes = 105 whole lines, so that
+// no line is shared with another wave (a non-temporal line fetched by two waves crosses the memory system twice).  Read
+// alone this way the 510 MB matrix takes 75 us, with the lanes fetching their own pieces 82-84.  The blocks lie in LDS
+// as in memory, 210 bytes apart, so a lane's fields start at even addresses: each is read as aligned words and shifted
+// into place by v_alignbyte.  With bf16 activations the pieces, the dot products and the order of the sums are those of
+// gemv_stream_kernel; with f32 activations (the dtype of the reference's call sites) those of the flat walk, a lane's 64
+// activations in registers: the same bits as those kernels give for rows of 4096.
+template <bool X_BF16>
+constexpr int kQ6kCopyWaves = X_BF16 ? 16 : 12;  // (f32: 64 activation registers per lane)
+template <bool X_BF16, int LOG_RPC>
+__global__ __launch_bounds__(64 * kQ6kCopyWaves<X_BF16>) void gemv_q6k_rowcopy_kernel(SArgs a) {
+    constexpr uint32_t W = kQ6kCopyWaves<X_BF16>, NT = 64 * W, CHUNKB = 16u * Q6K_BYTES, PIECES = CHUNKB / 16u;  // 3360 bytes, 210 pieces
+    constexpr uint32_t RPC = 1u << LOG_RPC;  // rows per chunk: k = 4096 >> LOG_RPC
+    using XF = FlatX1<HQ_Q6_K, false>;
     extern __shared__ uint4 smem[];
-    uint4* lds_x = smem;                                           // [k / 8]
-    float* lds_s = reinterpret_cast<float*>(lds_x + 4096u / 8u);   // [k / 16]
+    uint4* lds_x = smem;
+    float* lds_s = X_BF16 ? reinterpret_cast<float*>(lds_x + a.k / 8u) : reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(smem) + XF::value_bytes(a.k));
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    uint4* wbuf = reinterpret_cast<uint4*>(lds_s + 4096u / 16u) + wv * 256u;  // this wave's row: 256 slots of 16 bytes
+    uint4* wbuf = reinterpret_cast<uint4*>(lds_s + a.k / 16u) + wv * 256u;  // this wave's chunk: 256 slots of 16 bytes
     const int c = (int)(lane & 3u);
-    const uint32_t groups = (a.n + 3u) / 4u, stride = W * gridDim.x;
+    const uint32_t chunks = (a.n + RPC - 1u) >> LOG_RPC, groups = (chunks + 3u) / 4u, stride = W * gridDim.x;
+    const uint32_t tail_pieces = (a.n - ((chunks - 1u) << LOG_RPC)) * (PIECES >> LOG_RPC);  // pieces of the last chunk that exist
     const uint32_t g_first = wv * gridDim.x + blockIdx.x;
     const uint32_t groups_mine = g_first < groups ? (groups - g_first + stride - 1u) / stride : 0u;
     const uint32_t ntask = groups_mine * 4u;
 
-    stream_stage_x<HQ_Q6_K, 1>(a.x, 4096u, lds_x, lds_s, tid, NT);
+    if constexpr (X_BF16) stream_stage_x<HQ_Q6_K, 1>(a.x, a.k, lds_x, lds_s, tid, NT);
+    else XF::stage(a.x, a.k, lds_x, lds_s, tid, NT);
 
-    // task t of this wave: row 4 (g_first + (t / 4) stride) + t % 4, clamped to the matrix (a clamped row is not stored)
-    auto row_of = [&](uint32_t t) { return 4u * (g_first + (t >> 2) * stride) + (t & 3u); };
+    // task t of this wave: chunk 4 (g_first + (t / 4) stride) + t % 4, clamped to the matrix (a clamped chunk is not stored)
+    auto chunk_of = [&](uint32_t t) { return 4u * (g_first + (t >> 2) * stride) + (t & 3u); };
     uint4 pv[4];
     auto fetch = [&](uint32_t t) {
-        uint32_t row = row_of(t);
-        row = row < a.n ? row : a.n - 1u;
-        const uint8_t* base = (row < a.n0 ? a.w0 + (size_t)row * ROWB : a.w1 + (size_t)(row - a.n0) * ROWB);
+        uint32_t ch = chunk_of(t);
+        ch = ch < chunks ? ch : chunks - 1u;
+        const uint8_t* base = a.w0 + (size_t)ch * CHUNKB;
+        const uint32_t last = (ch == chunks - 1u ? tail_pieces : PIECES) - 1u;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t pc = lane + 64u * (uint32_t)i;
-            pv[i] = ldnt16(base + 16u * (pc < PIECES ? pc : PIECES - 1u));
+            pv[i] = ldnt16(base + 16u * (pc < last ? pc : last));
         }
     };
     if (ntask) fetch(0);
     __syncthreads();
 
-    uint32_t m4, m2, magic;
-    asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5" : "=v"(m4), "=v"(m2), "=v"(magic) : "s"(a.m4), "s"(a.m2), "s"(a.magic));
-    uint32_t xp[32];
+    [[maybe_unused]] uint32_t m4, m2, magic;
+    if constexpr (X_BF16)
+        asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5" : "=v"(m4), "=v"(m2), "=v"(magic) : "s"(a.m4), "s"(a.m2), "s"(a.magic));
+    // the lane's activations: block (lane / 4) of its row, quarter c
+    const uint32_t lane_in_row = lane & (63u >> LOG_RPC);
+    uint32_t xp[X_BF16 ? 32 : 64];
     float sx[4];
-    stream_load_x<HQ_Q6_K>(lds_x, lds_s, 0, lane, c, xp, sx);
+    if constexpr (X_BF16) stream_load_x<HQ_Q6_K>(lds_x, lds_s, 0, lane_in_row, c, xp, sx);
+    else XF::load(lds_x, lds_s, lane_in_row >> 2, c, xp, sx);
 
-    // this lane's piece in the row buffer: block lane / 4 at byte 210 (lane / 4), fields at even offsets; sh = the bytes by
+    // this lane's piece in the chunk buffer: block lane / 4 at byte 210 (lane / 4), fields at even offsets; sh = the bytes by
     // which a field's first aligned word starts early (0 or 2)
     const uint32_t blk = (lane >> 2) * Q6K_BYTES, h = (uint32_t)c >> 1, lr = (uint32_t)c & 1u;
     const uint32_t* wb32 = reinterpret_cast<const uint32_t*>(wbuf);
@@ -640,20 +665,18 @@ __global__ __launch_bounds__(64 * Q6K_LDS_WAVES) void gemv_q6k_rowcopy_kernel(SA
                           __builtin_amdgcn_alignbyte(w4, w3, sh));
     };
 
+    // results: lane i keeps the wave's i-th row (RPC per task), stored 64 at a time
     uint32_t done = 0;
     float keep = 0.f;
     auto flush = [&](uint32_t first, uint32_t count) {
         if (lane < count) {
-            const uint32_t row = row_of(first + lane);
-            if (row < a.n) {
-                if (row < a.n0) a.y0[row] = keep;
-                else a.y1[row - a.n0] = keep;
-            }
+            const uint32_t r = first + lane, row = (chunk_of(r >> LOG_RPC) << LOG_RPC) + (r & (RPC - 1u));
+            if (row < a.n) a.y0[row] = keep;
         }
     };
     for (uint32_t t = 0; t < ntask; ++t) {
-        // the row fetched a task ago goes to LDS (the wave's earlier reads of the buffer precede these writes: one wave's
-        // LDS operations are served in order), the next row's fetch is issued, then this row's pieces are read back
+        // the chunk fetched a task ago goes to LDS (the wave's earlier reads of the buffer precede these writes: one wave's
+        // LDS operations are served in order), the next chunk's fetch is issued, then this chunk's pieces are read back
 #pragma unroll
         for (int i = 0; i < 4; ++i) wbuf[lane + 64u * (uint32_t)i] = pv[i];
         asm volatile("" ::: "memory");  // (for the compiler: the reads below are of what was just written)
@@ -669,11 +692,36 @@ __global__ __launch_bounds__(64 * Q6K_LDS_WAVES) void gemv_q6k_rowcopy_kernel(SA
             const uint32_t* q = wb32 + (o_d >> 2);
             pc.d = __builtin_amdgcn_alignbyte(q[1], q[0], o_d & 3u);
         }
-        const float v = group_sum(dot_pair(pc, c, xp, sx, m4, m2, magic), 6);
-        keep = lane == (done & 63u) ? v : keep;
-        if ((++done & 63u) == 0u) flush(done - 64u, 64u);
+        float part;
+        if constexpr (X_BF16) part = dot_pair(pc, c, xp, sx, m4, m2, magic);
+        else part = dot_f32(pc, c, reinterpret_cast<const float*>(xp), sx);
+        const float v = group_sum(part, 6 - LOG_RPC);
+        if constexpr (RPC == 1) {
+            keep = lane == (done & 63u) ? v : keep;
+        } else {
+            // (every lane of a half holds its row's sum: lanes 0 and 32 speak for the two rows)
+            const float v0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+            const float v1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+            keep = lane == (done & 63u) ? v0 : lane == (done & 63u) + 1u ? v1 : keep;
+        }
+        done += RPC;
+        if ((done & 63u) == 0u) flush(done - 64u, 64u);
     }
     if (done & 63u) flush(done & ~63u, done & 63u);
+}
+template <bool X_BF16>
+int launch_q6k_rowcopy(hipStream_t s, const SArgs& sa, uint32_t cus) {
+    constexpr int W = kQ6kCopyWaves<X_BF16>;
+    const size_t lds_x = X_BF16 ? (size_t)sa.k * 2 + (size_t)(sa.k / 16) * 4 : FlatX1<HQ_Q6_K, false>::lds_bytes(sa.k);
+    const size_t lds = lds_x + (size_t)W * 4096u;
+    auto kern = sa.k == 4096 ? gemv_q6k_rowcopy_kernel<X_BF16, 0> : gemv_q6k_rowcopy_kernel<X_BF16, 1>;
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv row-copy LDS)")) return rc;
+    hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
+    return check_launch("gemv row-copy kernel launch");
+}
+// One Q6_K matrix, 16-byte aligned, rows of 4096 or 2048 elements, two groups of four chunks per wave or more.
+inline bool q6k_rowcopy_takes(const void* w, uint32_t n, uint32_t k, uint32_t cus) {
+    return (k == 4096 || k == 2048) && (reinterpret_cast<uintptr_t>(w) & 15u) == 0 && (uint64_t)n * (k / 256u) >= (uint64_t)512u * cus;
 }
 
 // Whether the streaming form takes (type, k, rows): K-quants, whole 4096-element steps, enough rows to occupy the waves.
@@ -689,15 +737,8 @@ int launch_stream(hipStream_t s, const SArgs& sa, uint32_t cus) {
     constexpr bool XREG_FITS = ROWS <= 2 && !(TYPE == HQ_Q5_K && ROWS == 2);
     bool launched = false;
     if constexpr (TYPE == HQ_Q6_K && ROWS == 1) {
-        // rows of 3360 bytes from a 16-byte aligned matrix, two groups of four rows per wave or more: the row-copy form
-        // (12288 rows: 9.4 against 10.7 us; 4096 rows: the same)
-        if (sa.k == 4096 && sa.n0 == sa.n && (reinterpret_cast<uintptr_t>(sa.w0) & 15u) == 0 && sa.n >= 32u * cus) {
-            const size_t lds_rc = lds + (size_t)Q6K_LDS_WAVES * 4096u;
-            if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(gemv_q6k_rowcopy_kernel), lds_rc, "hipFuncSetAttribute(gemv row-copy LDS)"))
-                return rc;
-            hipLaunchKernelGGL(gemv_q6k_rowcopy_kernel, dim3(cus), dim3(64 * Q6K_LDS_WAVES), lds_rc, s, sa);
-            return check_launch("gemv row-copy kernel launch");
-        }
+        // (12288 rows of 4096: 9.4 against 10.7 us; 4096 rows: the same)
+        if (sa.n0 == sa.n && q6k_rowcopy_takes(sa.w0, sa.n, sa.k, cus)) return launch_q6k_rowcopy<true>(s, sa, cus);
     }
     if constexpr ((TYPE == HQ_Q4_K || TYPE == HQ_Q5_K) && ROWS == 1) {
         // (Q4_K 12288 x 4096: 7.75 -> 7.4 us, 151936 x 4096: 63 -> 59 us; Q5_K 12288 x 4096: 9.07 -> 8.46 us; the same bits)
@@ -722,6 +763,21 @@ int launch_stream(hipStream_t s, const SArgs& sa, uint32_t cus) {
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
         hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
     }
+    return check_launch("gemv stream kernel launch");
+}
+
+// One f32 activation row over a 16-byte aligned Q4_K / Q5_K matrix with rows of 4096: the copy form of the streaming
+// kernel, a lane's 64 activations in registers, 12 waves (16 would spill).  Longer rows, whose activations a lane reads
+// from LDS step by step, stay with the flat walk: measured there the copy form gains nothing (4096 x 12288 Q4_K: 9.0
+// against 8.6 us, and 4 us more behind the gate / up launch of a decode FFN).
+template <int TYPE>
+int launch_stream_f32(hipStream_t s, const SArgs& sa, uint32_t cus) {
+    constexpr uint32_t W = 12;
+    constexpr size_t wbytes = (size_t)W * 64u * ((kBlockBytes<TYPE> + 63u) / 64u) * 16u;
+    const size_t lds = FlatX1<TYPE, false>::lds_bytes(sa.k) + wbytes;
+    auto kern = gemv_stream_kernel<TYPE, W, true, 1, true, false>;
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv stream LDS)")) return rc;
+    hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, sa);
     return check_launch("gemv stream kernel launch");
 }
 
@@ -900,6 +956,30 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
                                          : launch_stream<TYPE, 1>(s, sa, cus))
                     return rc;
                 r += take;
+            }
+            return HQ_OK;
+        }
+    }
+    // f32 activations over Q4_K / Q5_K rows of 4096: the copy form of the streaming kernel, a pass per row
+    // (12288 x 4096: Q4_K 8.2 -> 7.7 us, Q5_K 9.1 -> 8.2 on one device, no difference on another)
+    if constexpr (!X_BF16 && (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K)) {
+        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && a.k == 4096 && stream_takes<TYPE>(a.n, a.k, cus) &&
+            (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0) {
+            for (uint32_t r = 0; r < a.pairs; ++r) {
+                const SArgs sa{static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * 4, a.w, a.w, a.y + (size_t)r * a.n, a.y + (size_t)r * a.n,
+                               a.n, a.n, a.k, 0, 0, 0};
+                if (int rc = launch_stream_f32<TYPE>(s, sa, cus)) return rc;
+            }
+            return HQ_OK;
+        }
+    }
+    // Q6_K rows of 4096 / 2048 elements not taken above (f32 activations, k = 2048): chunks copied through LDS, a pass per row.
+    if constexpr (TYPE == HQ_Q6_K) {
+        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && q6k_rowcopy_takes(a.w, a.n, a.k, cus)) {
+            for (uint32_t r = 0; r < a.pairs; ++r) {
+                const SArgs sa{static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * (X_BF16 ? 2 : 4), a.w, a.w, a.y + (size_t)r * a.n,
+                               a.y + (size_t)r * a.n, a.n, a.n, a.k, N4, N2, MAGIC};
+                if (int rc = launch_q6k_rowcopy<X_BF16>(s, sa, cus)) return rc;
             }
             return HQ_OK;
         }

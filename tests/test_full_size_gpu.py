@@ -86,6 +86,38 @@ def test_q6k_head_rows_copied_through_lds(oracle, dev, n):
     assert_matmul_close(y[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, f"q6_k {n}x{k}, sampled rows")
 
 
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("n,k", [(8192, 4096), (65539, 4096), (16384, 2048), (40001, 2048), (40006, 2048)])
+def test_q6k_chunks_copied_through_lds_f32_and_short_rows(oracle, dev, xdt, n, k):
+    """The chunk-copy form of the Q6_K GEMV beyond the bf16 head: f32 activations (the dtype of the reference's call sites,
+    gpu_full_attn.rs:835) and rows of 2048 elements (two rows per chunk of sixteen blocks; row counts that leave the
+    last chunk with one row and the last group with 1 .. 4 chunks).  Every output row against the product over a slice
+    of the matrix small enough for the kernels whose lanes fetch their own pieces, sampled rows against the f64 oracle,
+    and the same bits on a second call."""
+    t = HQ_Q6_K
+    w = _quantized(dev, n, k, t, 5 + n)
+    rng = np.random.default_rng(n + k)
+    x = (rng.integers(-12, 13, (1, k)) / 8.0).astype(np.float32)
+    xd = torch.from_numpy(x).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    y = torch.full((1, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd, w, y, GgmlQuantizedMatmulParams(1, n, k, t))
+    assert torch.isfinite(y).all()
+    rows = np.unique(np.concatenate([[0, 1, 2, 3, n - 4, n - 3, n - 2, n - 1], rng.integers(0, n, 40)]))
+    xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
+    ref = oracle.qmatmul_f64(xv, _rows_of(w, rows, k, t, oracle), 1, rows.size, k, t)
+    assert_matmul_close(y[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, f"q6_k {xdt} {n}x{k}, sampled rows")
+    row_bytes = k // 256 * 210
+    part = 2048  # rows per slice: below what the chunk-copy form takes
+    for r0 in (0, (n - part) // 2, n - part):
+        ys = torch.full((1, part), float("nan"), device=dev)
+        ops.quantized_matmul_ggml(xd, w[r0 * row_bytes:(r0 + part) * row_bytes].clone(), ys, GgmlQuantizedMatmulParams(1, part, k, t))
+        assert (ys - y[:, r0:r0 + part]).abs().max().item() <= 2e-6 * np.abs(ref).max(), (xdt, n, k, r0)
+    y2 = torch.full((1, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd, w, y2, GgmlQuantizedMatmulParams(1, n, k, t))
+    assert torch.equal(y, y2)
+
+
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048)])
