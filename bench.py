@@ -40,7 +40,7 @@ SETTLE_STEPS = 2400  # untimed decode steps before the steady-state measurements
 # 2.0), WRITE_SIZE all of them (1.0).  The runs and their figures are in profiles/*_pmc_traffic.md.
 PMC_TRAFFIC_BYTES = {
     # (FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0) x 1024 per dispatch
-    "gemv_head_q6_k_151936x4096": int(254251.7 * 2.0 * 1024 + 1187.0 * 1.0 * 1024),
+    "gemv_head_q6_k_151936x4096": int(254241.0 * 2.0 * 1024 + 1187.0 * 1.0 * 1024),
     # activation pre-pass + tile GEMM, Q4_K, 2048 x 12288 x 4096 (the GEMM re-fetches the weights once per 256-token tile)
     "prefill_gemm_q4_k_2048x12288x4096": int((23301.6 + 132573.1) * 2.0 * 1024 + (16496.5 + 98311.8) * 1.0 * 1024),
     # split (with the q rotation) + merge (with the output rotation), 32K context, 2 kv heads, head_dim 256
@@ -978,6 +978,25 @@ def bench_decode_gemv(a):
     probe["what"] = ("one plain read of the same buffers, 16 bytes per lane, no arithmetic (hq_stream_read_probe), timed like `kernels`: the "
                      "streaming rate this device reaches; kernels[...].us / this us = how far a kernel is from it")
 
+    # The head inside the step, behind `roofline`: host-launched steps with a HIP event pair around every head launch
+    # (the pair reads the kernel's time plus the 2-4 us its two markers add).  A head launch that follows the step's
+    # FFN kernels is faster than one that follows another head launch, which is what `kernels` times (kernel trace:
+    # 80.1 us inside steps, 87.4 us back to back, under the profiler on one device), and the step is the workload.
+    n_in = max(a.steps, 64)
+    pairs_in = _events(n_in)
+    torch.cuda.synchronize()
+    for i in range(n_in):
+        ws = sets[i % n_sets]
+        ops.quantized_matmul_batch_ggml([ops.QmatmulJob(x_h, ws["gate"], y["gate"], 1, F, H),
+                                         ops.QmatmulJob(x_h, ws["up"], y["up"], 1, F, H)], HQ_Q4_K)
+        ops.quantized_matmul_ggml(x_f, ws["down"], y["down"], params["down"])
+        pairs_in[i][0].record()
+        ops.quantized_matmul_ggml(x_h, heads[i % n_heads], y["head"], params["head"])
+        pairs_in[i][1].record()
+    torch.cuda.synchronize()
+    head_in_step = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in pairs_in)
+    head_in_step_us = sum(head_in_step) / len(head_in_step)
+
     # The timed region behind `value`: exactly K steps replayed from HIP graphs of their three launches
     # (runs of consecutive steps over the rotated weight sets and heads), as a decode loop that records
     # its token step does; the host's per-launch cost (Python, ctypes) is then out of the way, like in
@@ -987,7 +1006,7 @@ def bench_decode_gemv(a):
         elapsed, step_us_events = _timed_steps(a, fused_step, n_sets * n_heads)
 
     value = step_bytes * a.steps / elapsed / 1e9
-    head_us = kern_us["head_151936x4096"]
+    head_us = head_in_step_us
     head_gbs = nbytes["head"] / head_us / 1e3
     return {
         "metric": "Q4_K/Q6_K GEMV eff. GB/s (% HBM peak)",
@@ -1018,6 +1037,9 @@ def bench_decode_gemv(a):
                      "traffic_source": "recorded: rocprofv3 --pmc runs of this file, profiles/gemv_decode_config2_pmc_traffic.md",
                      "us_per_launch": round(head_us, 3), "bytes_per_launch": nbytes["head"]},
         "kernels": kernels,
+        "head_in_step": {"us_avg": round(head_in_step_us, 3), "us_median": round(head_in_step[len(head_in_step) // 2], 3), "launches": n_in,
+                         "what": "HIP event pair around each head launch of host-launched steps (roofline.us_per_launch); "
+                                 "kernels.head_151936x4096 is head launches back to back"},
         "kernels_f32_activations": kernels_f32,
         "host_launched": host,
         "q4_k_gemv": {"GBps": round(q4_bytes / q4_us / 1e3, 1), "frac_hbm_peak": round(q4_bytes / q4_us / 1e3 / HBM_PEAK_GBS, 4),
