@@ -87,14 +87,16 @@ def test_q6k_head_rows_copied_through_lds(oracle, dev, n):
 
 
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
-@pytest.mark.parametrize("n,k", [(8192, 4096), (65539, 4096), (16384, 2048), (40001, 2048), (40006, 2048)])
-def test_q6k_chunks_copied_through_lds_f32_and_short_rows(oracle, dev, xdt, n, k):
-    """The chunk-copy form of the Q6_K GEMV beyond the bf16 head: f32 activations (the dtype of the reference's call sites,
-    gpu_full_attn.rs:835) and rows of 2048 elements (two rows per chunk of sixteen blocks; row counts that leave the
-    last chunk with one row and the last group with 1 .. 4 chunks).  Every output row against the product over a slice
-    of the matrix small enough for the kernels whose lanes fetch their own pieces, sampled rows against the f64 oracle,
-    and the same bits on a second call."""
-    t = HQ_Q6_K
+@pytest.mark.parametrize("t,n,k", [(HQ_Q6_K, 8192, 4096), (HQ_Q6_K, 65539, 4096), (HQ_Q6_K, 16384, 2048), (HQ_Q6_K, 40001, 2048),
+                                   (HQ_Q6_K, 40006, 2048), (HQ_Q4_K, 8192, 4096), (HQ_Q4_K, 12289, 4096), (HQ_Q5_K, 8192, 4096),
+                                   (HQ_Q5_K, 20001, 4096)])
+def test_weights_copied_through_lds_f32_and_short_rows(oracle, dev, xdt, t, n, k):
+    """The forms of the one-row GEMV that copy the weights through LDS, beyond the bf16 head: f32 activations (the dtype of
+    the reference's call sites, gpu_full_attn.rs:835) over Q6_K chunks and over Q4_K / Q5_K rows of 4096, and Q6_K rows
+    of 2048 elements (two rows per chunk of sixteen blocks; row counts that leave the last chunk with one row and the
+    last group with 1 .. 4 chunks).  Every output row against the product over a slice of the matrix small enough for
+    the kernels whose lanes fetch their own pieces, sampled rows against the f64 oracle, and the same bits on a second
+    call."""
     w = _quantized(dev, n, k, t, 5 + n)
     rng = np.random.default_rng(n + k)
     x = (rng.integers(-12, 13, (1, k)) / 8.0).astype(np.float32)
@@ -106,8 +108,8 @@ def test_q6k_chunks_copied_through_lds_f32_and_short_rows(oracle, dev, xdt, n, k
     rows = np.unique(np.concatenate([[0, 1, 2, 3, n - 4, n - 3, n - 2, n - 1], rng.integers(0, n, 40)]))
     xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
     ref = oracle.qmatmul_f64(xv, _rows_of(w, rows, k, t, oracle), 1, rows.size, k, t)
-    assert_matmul_close(y[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, f"q6_k {xdt} {n}x{k}, sampled rows")
-    row_bytes = k // 256 * 210
+    assert_matmul_close(y[:, torch.as_tensor(rows, device=dev)].cpu().numpy(), ref, f"type {t} {xdt} {n}x{k}, sampled rows")
+    row_bytes = k // oracle.BLOCK_ELEMS[t] * oracle.BLOCK_BYTES[t]
     part = 2048  # rows per slice: below what the chunk-copy form takes
     for r0 in (0, (n - part) // 2, n - part):
         ys = torch.full((1, part), float("nan"), device=dev)
