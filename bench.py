@@ -260,11 +260,12 @@ def _timed_steps(a, step, n_variants):
     return elapsed, e0.elapsed_time(e1) * 1e3 / a.steps
 
 
-def _launch_us(launches, reps=3):
-    """Average device time of one launch: the callables (each enqueues ONE kernel, over weights no other of them
-    touches) are recorded into a HIP graph back to back and the graph is replayed `reps` times between one HIP
-    event pair on the replay stream; elapsed / (reps * len(launches)).  A kernel of a few microseconds cannot be
-    timed by an event pair of its own: the pair adds ~2.5 us."""
+def _launch_us(launches, reps=5):
+    """Device time of one launch: the callables (each enqueues ONE kernel, over weights no other of them touches)
+    are recorded into a HIP graph back to back and the graph is replayed `reps` times, each replay between a HIP
+    event pair of its own on the replay stream; the median replay / len(launches) (a replay of a millisecond or
+    two now and then takes three times as long as its neighbours; the median leaves such a one out).  A kernel of
+    a few microseconds cannot be timed by an event pair of its own: the pair adds ~2.5 us."""
     import torch
 
     side = torch.cuda.Stream()
@@ -275,14 +276,15 @@ def _launch_us(launches, reps=3):
                 f()
     torch.cuda.synchronize()
     g.replay()
-    e0, e1 = _events(1)[0]
+    pairs = _events(reps)
     torch.cuda.synchronize()
-    e0.record()
-    for _ in range(reps):
+    for e0, e1 in pairs:
+        e0.record()
         g.replay()
-    e1.record()
+        e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / (reps * len(launches))
+    times = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+    return times[len(times) // 2] * 1e3 / len(launches)
 
 
 def _finish(a, out):
