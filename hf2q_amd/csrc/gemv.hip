@@ -828,7 +828,7 @@ struct FArgs {
 
 // DYN: the waves of a workgroup take its super-tasks from a counter (see gemv_walk.h): worth it where a wave has many
 // (the 151936-row head in f32: 101 against 108 us); with a handful per wave the three claimed ahead are all there is.
-template <int TYPE, bool X_BF16, int W, int D, bool DYN>
+template <int TYPE, bool X_BF16, int W, int D, bool DYN, bool COPY = false>
 __global__ __launch_bounds__(64 * W) void gemv_flat_kernel(FArgs a) {
     using X = FlatX<TYPE, X_BF16>;
     extern __shared__ uint4 smem[];
@@ -840,11 +840,13 @@ __global__ __launch_bounds__(64 * W) void gemv_flat_kernel(FArgs a) {
     if (tid == 0) lds_queue = W;
     // the activations first, nothing else of this workgroup in front of them
     X::stage(a.x, a.k, lds_x, lds_s, tid, 64u * W);
-    FlatWalk<TYPE, X_BF16, D, false, DYN> wk;
+    FlatWalk<TYPE, X_BF16, D, false, DYN, COPY> wk;
+    // (COPY: a window buffer of 256 slots of 16 bytes per wave behind the activations' sums)
+    uint4* wbuf = COPY ? reinterpret_cast<uint4*>(lds_s + a.k / 16u) + wv * 256u : nullptr;
     if constexpr (DYN)
-        wk.init(a.w0, a.w1, a.n, a.nm, a.g, blockIdx.x, gridDim.x, &lds_queue, wv);
+        wk.init(a.w0, a.w1, a.n, a.nm, a.g, blockIdx.x, gridDim.x, &lds_queue, wv, wbuf);
     else
-        wk.init(a.w0, a.w1, a.n, a.nm, a.g, wv * gridDim.x + blockIdx.x, W * gridDim.x);
+        wk.init(a.w0, a.w1, a.n, a.nm, a.g, wv * gridDim.x + blockIdx.x, W * gridDim.x, nullptr, 0, wbuf);
     if constexpr (!DYN) wk.prime();
     __syncthreads();
     if constexpr (DYN) wk.prime();
@@ -899,6 +901,17 @@ int launch_flat(hipStream_t s, const void* x, const uint8_t* w0, const uint8_t* 
     const bool dyn = kFlatDepth<TYPE> == 1 && supers >= (uint64_t)cus * W * 8u;
     auto kern = dyn ? gemv_flat_kernel<TYPE, X_BF16, W, 1, true> : gemv_flat_kernel<TYPE, X_BF16, W, kFlatDepth<TYPE>, false>;
     size_t lds = X::lds_bytes(k);
+    if constexpr (TYPE == HQ_Q6_K && X_BF16) {
+        // Windows copied through LDS (see FlatWalk) where every window starts on a 16-byte boundary, no copy reads past the
+        // matrix and a row is a window or more: 8192 x 28672 37.0 -> 33.5 us, 17408 x 5120 17.5 -> 16.7, 4096 x 14336 11.75 ->
+        // 11.4; rows shorter than a window gain nothing (262144 x 2816: 108.5 against 110), and with f32 activations, whose
+        // products keep the VALU busier, the form is slower (262144 x 2816: 124 against 112 us)
+        if (fa.g.bu >= kUnitsPerWindow<TYPE> && flat_copy_fits(fa.g, kUnitsPerWindow<TYPE>, n, reinterpret_cast<uintptr_t>(w0), reinterpret_cast<uintptr_t>(w1)) &&
+            lds + (size_t)W * 4096u <= 160 * 1024 - 512) {
+            kern = dyn ? gemv_flat_kernel<TYPE, X_BF16, W, 1, true, true> : gemv_flat_kernel<TYPE, X_BF16, W, 1, false, true>;
+            lds += (size_t)W * 4096u;
+        }
+    }
     if (lds < 81 * 1024) lds = 81 * 1024;  // more than half a CU's LDS: one workgroup per CU
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv flat LDS)")) return rc;
     hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, fa);

@@ -253,9 +253,18 @@ struct FlatX<TYPE, X_BF16, true> {
 // The SIMD's issue arbitration favours its oldest wave, so with equal shares the youngest wave of every SIMD finishes long
 // after the others; with the counter all waves of a CU end together.  A wave claims its next super-task one ahead, so its
 // fetch runs on across the boundary.
-template <int TYPE, bool X_BF16, int D = 1, bool XHALF = false, bool DYN = false>
+// COPY (Q6_K, D == 1): a window is not fetched by the lanes that use it, five instructions touching each 128-byte line,
+// but copied -- consecutive lanes consecutive 16-byte pieces, non-temporal loads, every line asked for once -- into 4 KB
+// of LDS the wave owns, and the lanes read their fields back from there (blocks 210 bytes apart: aligned words shifted
+// into place by v_alignbyte); the next window's copy is in flight meanwhile.  The same pieces, the same sums.  The host
+// checks flat_copy_fits: every window starts at a multiple of 16 bytes and no copy reads past the matrix.
+inline bool flat_copy_fits(const FlatGeom& g, uint32_t uw, uint32_t n, uintptr_t base0, uintptr_t base1) {
+    return g.uwe == uw && ((g.bu << g.log_r) % 8u) == 0 && ((uint64_t)n * g.bu) % 8u == 0 && ((base0 | base1) & 15u) == 0;
+}
+template <int TYPE, bool X_BF16, int D = 1, bool XHALF = false, bool DYN = false, bool COPY = false>
 struct FlatWalk {
     static_assert(!DYN || D == 1, "the dynamic split keeps one fetch in flight");
+    static_assert(!COPY || (TYPE == HQ_Q6_K && D == 1 && !XHALF), "windows of sixteen Q6_K super-blocks, one in flight");
     using X = FlatX<TYPE, X_BF16>;
     static constexpr uint32_t LPU = kLanesPerUnit<TYPE>, UW = kUnitsPerWindow<TYPE>, BB = kBlockBytes<TYPE>;
 
@@ -275,10 +284,13 @@ struct FlatWalk {
     uint32_t m4, m2, magic;
     uint32_t f_q, f_m, f_w;  // the next task to fetch
     Piece<TYPE> buf[D];
+    [[maybe_unused]] uint4 pv[COPY ? 4 : 1];  // COPY: the window in flight, 16-byte piece lane + 64 i of it
+    [[maybe_unused]] uint4* wbuf;             // COPY: the wave's 4 KB window buffer in LDS
 
     __device__ __forceinline__ void init(const uint8_t* wa, const uint8_t* wb, uint32_t n, uint32_t n_matrices, const FlatGeom& geom,
                                          uint32_t first_super, uint32_t super_stride, uint32_t* lds_queue = nullptr,
-                                         uint32_t first_claim = 0) {
+                                         uint32_t first_claim = 0, uint4* copy_buf = nullptr) {
+        wbuf = copy_buf;
         w0 = wa;
         w1 = wb;
         nrows = n;
@@ -315,7 +327,26 @@ struct FlatWalk {
         const uint32_t last = nrows * g.bu - 1u;
         u = u < last ? u : last;
         const uint8_t* base = f_m ? w1 : w0;
-        p.load(base + (size_t)u * BB, c);
+        if constexpr (COPY) {
+            // the window's units [ub, ub + cnt): a multiple of eight units from the matrix's start (whole 16-byte pieces),
+            // clamped to the matrix (n * bu is a multiple of eight); past a window that ends inside the matrix the last
+            // piece reads up to 14 bytes of the next unit
+            const uint32_t total = last + 1u;
+            uint32_t ub = (sid << g.log_r) * g.bu + g.uwe * f_w;
+            ub = ub < total ? ub : total - 8u;
+            uint32_t cnt = su - g.uwe * f_w;
+            cnt = cnt < g.uwe ? cnt : g.uwe;
+            cnt = cnt < total - ub ? cnt : total - ub;
+            const uint32_t last_piece = (cnt * BB + 15u) / 16u - 1u;
+            const uint8_t* wb = base + (size_t)ub * BB;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t pi = lane + 64u * (uint32_t)i;
+                pv[i] = ldnt16(wb + 16u * (pi < last_piece ? pi : last_piece));
+            }
+        } else {
+            p.load(base + (size_t)u * BB, c);
+        }
         // (scalar: no memory operation inside)  Past the sequence's end the last task is fetched again, not used.
         if (f_w + 1u < g.st) {
             ++f_w;
@@ -372,10 +403,37 @@ struct FlatWalk {
         [[maybe_unused]] uint32_t pending = 0;
         if constexpr (DYN)
             if (q_cur < count) pending = claim();  // the third super-task from here
+        // COPY: the lane's fields in the window buffer, block lv at byte 210 lv, at even offsets
+        [[maybe_unused]] const uint32_t* wb32 = reinterpret_cast<const uint32_t*>(wbuf);
+        [[maybe_unused]] const uint32_t cblk = lv * BB, ch = (uint32_t)c >> 1, clr = (uint32_t)c & 1u;
+        [[maybe_unused]] const uint32_t o_qa = cblk + 64u * ch + 16u * clr, o_qh = cblk + 128u + 32u * ch + 16u * clr,
+                                        o_sc = cblk + 192u + 8u * ch, o_d = cblk + 206u;
+        [[maybe_unused]] auto field16 = [&](uint32_t o) -> uint4 {
+            const uint32_t* q = wb32 + (o >> 2);
+            const uint32_t sh = o & 3u, a0 = q[0], a1 = q[1], a2 = q[2], a3 = q[3], a4 = q[4];
+            return make_uint4(__builtin_amdgcn_alignbyte(a1, a0, sh), __builtin_amdgcn_alignbyte(a2, a1, sh),
+                              __builtin_amdgcn_alignbyte(a3, a2, sh), __builtin_amdgcn_alignbyte(a4, a3, sh));
+        };
         while (q_cur < count) {
 #pragma unroll
             for (int d = 0; d < D; ++d) {
                 Piece<TYPE>& p = buf[d];
+                if constexpr (COPY) {
+                    // the window copied a task ago goes to LDS (behind the wave's reads of the previous one: a wave's LDS
+                    // operations are served in order), the next window's copy is issued, this window's fields are read back
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) wbuf[lane + 64u * (uint32_t)i] = pv[i];
+                    asm volatile("" ::: "memory");
+                    fetch_next(p);
+                    p.qa = field16(o_qa);
+                    p.qb = field16(o_qa + 32u);
+                    p.qh = field16(o_qh);
+                    const uint32_t* q = wb32 + (o_sc >> 2);
+                    const uint32_t sh = o_sc & 3u, a0 = q[0], a1 = q[1], a2 = q[2];
+                    p.sc = make_uint2(__builtin_amdgcn_alignbyte(a1, a0, sh), __builtin_amdgcn_alignbyte(a2, a1, sh));
+                    const uint32_t* qd = wb32 + (o_d >> 2);
+                    p.d = __builtin_amdgcn_alignbyte(qd[1], qd[0], o_d & 3u);
+                }
                 const uint32_t lu_raw = g.uwe * c_w + lv, su = g.bu << g.log_r;
                 const bool in_task = lu_raw < su;  // false only in the idle part of a ragged last window
                 const uint32_t lu = in_task ? lu_raw : su - 1u;
@@ -398,7 +456,7 @@ struct FlatWalk {
                         part = dot_f32(p, c, reinterpret_cast<const float*>(xr), sx);
                 }
                 asm volatile("" : "+v"(part));  // the refill follows the arithmetic that frees its registers
-                fetch_next(p);
+                if constexpr (!COPY) fetch_next(p);
                 const bool live = D == 1 || q_cur < count;  // (a ring's last round may run past the end)
                 const uint32_t row0 = (seq_first + q_cur * seq_stride) << g.log_r;
                 if (one_row) {

@@ -155,7 +155,10 @@ def test_small_batch_rows_staged_once(oracle, dev, t, xdt, n, k):
 # The reference's own decode shapes and dtype: f32 activations (gpu_full_attn.rs:835), k = 2816 (Gemma-4 projections, 11
 # super-blocks per row: windows of the streaming walk straddle rows) and k = 2048 (Qwen3.6 hidden: two rows per window), and
 # the 32-weight-block types; plus k = 4096 with f32 activations.  All of them take the flat streaming GEMV.
-FLAT_SHAPES = [(12288, 2816), (16384, 2048), (12288, 4096), (4099, 11264), (4096, 2816), (2816, 4096), (1500, 8960)]
+# (4096, 5120), (2048, 14336) and (2048, 17408): rows of a window of sixteen super-blocks or more, whole and ragged, which the
+# Q6_K walk copies through LDS under bf16 activations.
+FLAT_SHAPES = [(12288, 2816), (16384, 2048), (12288, 4096), (4099, 11264), (4096, 2816), (2816, 4096), (1500, 8960), (4096, 5120),
+               (2048, 14336), (2048, 17408)]
 
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0])
@@ -191,9 +194,9 @@ def test_decode_gemv_any_k_and_dtype(oracle, dev, t, xdt, n, k):
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q6_K, HQ_Q8_0])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
-def test_gate_and_up_in_one_launch_any_k(oracle, dev, t, xdt):
+@pytest.mark.parametrize("n,k", [(12288, 2816), (6144, 5120)])
+def test_gate_and_up_in_one_launch_any_k(oracle, dev, t, xdt, n, k):
     """Two matrices of one shape over the same activations as one batched launch: the bits of the two separate calls."""
-    n, k = 12288, 2816
     wg, wu = _quantized(dev, n, k, t, 5), _quantized(dev, n, k, t, 6)
     g = torch.Generator(device=dev)
     g.manual_seed(9)
