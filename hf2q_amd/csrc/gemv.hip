@@ -976,7 +976,16 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
     if constexpr (X_BF16 && kStreamType<TYPE>) {
-        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && stream_takes<TYPE>(a.n, a.k, cus)) {
+        // (one row over Q6_K rows longer than 4096: the flat walk with its windows copied through LDS is the faster where
+        // that form fits -- 4096 x 12288 11.2 -> 9.9 us, 128256 x 8192 145.5 -> 135.7, 8192 x 24576 32.2 -> 29.4; the same bits)
+        bool flat_copy_instead = false;
+        if constexpr (TYPE == HQ_Q6_K) {
+            if (a.pairs == 1 && a.k > 4096 && flat_takes<TYPE>(a.n, a.k, cus, FlatX<TYPE, true>::lds_bytes(a.k) + 12u * 4096u)) {
+                const FlatGeom g = flat_geom(a.k, kUnitElems<TYPE>, kUnitsPerWindow<TYPE>, a.n, 1, cus * 12u);
+                flat_copy_instead = flat_copy_fits(g, kUnitsPerWindow<TYPE>, a.n, reinterpret_cast<uintptr_t>(a.w), reinterpret_cast<uintptr_t>(a.w));
+            }
+        }
+        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && stream_takes<TYPE>(a.n, a.k, cus) && !flat_copy_instead) {
             // activation rows of a dense product up to four at a time (one pass over the weights for them)
             for (uint32_t r = 0; r < a.pairs;) {
                 const SArgs sa{static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * 2, a.w, a.w, a.y + (size_t)r * a.n, a.y + (size_t)r * a.n,
