@@ -841,8 +841,8 @@ __global__ __launch_bounds__(64 * W) void gemv_flat_kernel(FArgs a) {
     // the activations first, nothing else of this workgroup in front of them
     X::stage(a.x, a.k, lds_x, lds_s, tid, 64u * W);
     FlatWalk<TYPE, X_BF16, D, false, DYN, COPY> wk;
-    // (COPY: a window buffer of 256 slots of 16 bytes per wave behind the activations' sums)
-    uint4* wbuf = COPY ? reinterpret_cast<uint4*>(lds_s + a.k / 16u) + wv * 256u : nullptr;
+    // (COPY: a window buffer of 64 kCopyNPV slots of 16 bytes per wave behind the activations' sums)
+    uint4* wbuf = COPY ? reinterpret_cast<uint4*>(lds_s + a.k / 16u) + wv * (64u * kCopyNPV<TYPE>) : nullptr;
     if constexpr (DYN)
         wk.init(a.w0, a.w1, a.n, a.nm, a.g, blockIdx.x, gridDim.x, &lds_queue, wv, wbuf);
     else
@@ -906,10 +906,20 @@ int launch_flat(hipStream_t s, const void* x, const uint8_t* w0, const uint8_t* 
         // matrix and a row is a window or more: 8192 x 28672 37.0 -> 33.5 us, 17408 x 5120 17.5 -> 16.7, 4096 x 14336 11.75 ->
         // 11.4; rows shorter than a window gain nothing (262144 x 2816: 108.5 against 110), and with f32 activations, whose
         // products keep the VALU busier, the form is slower (262144 x 2816: 124 against 112 us)
-        if (fa.g.bu >= kUnitsPerWindow<TYPE> && flat_copy_fits(fa.g, kUnitsPerWindow<TYPE>, n, reinterpret_cast<uintptr_t>(w0), reinterpret_cast<uintptr_t>(w1)) &&
+        if (fa.g.bu >= kUnitsPerWindow<TYPE> && flat_copy_fits(fa.g, kUnitsPerWindow<TYPE>, n, kCopyAlignUnits<TYPE>, reinterpret_cast<uintptr_t>(w0), reinterpret_cast<uintptr_t>(w1)) &&
             lds + (size_t)W * 4096u <= 160 * 1024 - 512) {
             kern = dyn ? gemv_flat_kernel<TYPE, X_BF16, W, 1, true, true> : gemv_flat_kernel<TYPE, X_BF16, W, 1, false, true>;
             lds += (size_t)W * 4096u;
+        }
+    }
+    if constexpr (TYPE == HQ_Q8_0_X2) {
+        // Q8_0 block pairs (windows of 4352 bytes, read back as seventeen aligned words per lane), either activation type:
+        // lm_head 262144 x 2816 140.7 -> 127.2 us (f32 135.0 -> 122.8), 5120 x 17408 21.3 -> 20.2, 12288 x 4096 12.3 -> 12.0
+        constexpr size_t wb = (size_t)W * 64u * kCopyNPV<TYPE> * 16u;
+        if (flat_copy_fits(fa.g, kUnitsPerWindow<TYPE>, n, kCopyAlignUnits<TYPE>, reinterpret_cast<uintptr_t>(w0), reinterpret_cast<uintptr_t>(w1)) &&
+            lds + wb <= 160 * 1024 - 512) {
+            kern = dyn ? gemv_flat_kernel<TYPE, X_BF16, W, 1, true, true> : gemv_flat_kernel<TYPE, X_BF16, W, 1, false, true>;
+            lds += wb;
         }
     }
     if (lds < 81 * 1024) lds = 81 * 1024;  // more than half a CU's LDS: one workgroup per CU
@@ -982,7 +992,7 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
         if constexpr (TYPE == HQ_Q6_K) {
             if (a.pairs == 1 && a.k > 4096 && flat_takes<TYPE>(a.n, a.k, cus, FlatX<TYPE, true>::lds_bytes(a.k) + 12u * 4096u)) {
                 const FlatGeom g = flat_geom(a.k, kUnitElems<TYPE>, kUnitsPerWindow<TYPE>, a.n, 1, cus * 12u);
-                flat_copy_instead = flat_copy_fits(g, kUnitsPerWindow<TYPE>, a.n, reinterpret_cast<uintptr_t>(a.w), reinterpret_cast<uintptr_t>(a.w));
+                flat_copy_instead = flat_copy_fits(g, kUnitsPerWindow<TYPE>, a.n, kCopyAlignUnits<TYPE>, reinterpret_cast<uintptr_t>(a.w), reinterpret_cast<uintptr_t>(a.w));
             }
         }
         if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && stream_takes<TYPE>(a.n, a.k, cus) && !flat_copy_instead) {

@@ -253,18 +253,25 @@ struct FlatX<TYPE, X_BF16, true> {
 // The SIMD's issue arbitration favours its oldest wave, so with equal shares the youngest wave of every SIMD finishes long
 // after the others; with the counter all waves of a CU end together.  A wave claims its next super-task one ahead, so its
 // fetch runs on across the boundary.
-// COPY (Q6_K, D == 1): a window is not fetched by the lanes that use it, five instructions touching each 128-byte line,
-// but copied -- consecutive lanes consecutive 16-byte pieces, non-temporal loads, every line asked for once -- into 4 KB
-// of LDS the wave owns, and the lanes read their fields back from there (blocks 210 bytes apart: aligned words shifted
-// into place by v_alignbyte); the next window's copy is in flight meanwhile.  The same pieces, the same sums.  The host
-// checks flat_copy_fits: every window starts at a multiple of 16 bytes and no copy reads past the matrix.
-inline bool flat_copy_fits(const FlatGeom& g, uint32_t uw, uint32_t n, uintptr_t base0, uintptr_t base1) {
-    return g.uwe == uw && ((g.bu << g.log_r) % 8u) == 0 && ((uint64_t)n * g.bu) % 8u == 0 && ((base0 | base1) & 15u) == 0;
+// COPY (Q6_K and Q8_0 block pairs, D == 1): a window is not fetched by the lanes that use it, five instructions touching
+// each 128-byte line, but copied -- consecutive lanes consecutive 16-byte pieces, non-temporal loads, every line asked
+// for once -- into 4-5 KB of LDS the wave owns, and the lanes read their pieces back from there (Q6_K blocks lie 210
+// bytes apart: aligned words shifted into place by v_alignbyte; a Q8_0 block pair is seventeen aligned words); the next
+// window's copy is in flight meanwhile.  The same pieces, the same sums.  The host checks flat_copy_fits: every window
+// starts at a multiple of 16 bytes and no copy reads past the matrix.
+// (au: the units after which a window start is a multiple of 16 bytes again: 8 for Q6_K's 210 bytes, 4 for a Q8_0 block pair's 68)
+inline bool flat_copy_fits(const FlatGeom& g, uint32_t uw, uint32_t n, uint32_t au, uintptr_t base0, uintptr_t base1) {
+    return g.uwe == uw && ((g.bu << g.log_r) % au) == 0 && ((uint64_t)n * g.bu) % au == 0 && ((base0 | base1) & 15u) == 0;
 }
+template <int TYPE>
+constexpr uint32_t kCopyAlignUnits = TYPE == HQ_Q6_K ? 8u : 4u;
+template <int TYPE>
+constexpr uint32_t kCopyNPV = (kUnitsPerWindow<TYPE> * kBlockBytes<TYPE> / 16u + 63u) / 64u;  // 16-byte pieces of a window per lane
 template <int TYPE, bool X_BF16, int D = 1, bool XHALF = false, bool DYN = false, bool COPY = false>
 struct FlatWalk {
     static_assert(!DYN || D == 1, "the dynamic split keeps one fetch in flight");
-    static_assert(!COPY || (TYPE == HQ_Q6_K && D == 1 && !XHALF), "windows of sixteen Q6_K super-blocks, one in flight");
+    static_assert(!COPY || ((TYPE == HQ_Q6_K || TYPE == HQ_Q8_0_X2) && D == 1 && !XHALF), "Q6_K super-blocks or Q8_0 block pairs, one window in flight");
+    static constexpr uint32_t NPV = COPY ? kCopyNPV<TYPE> : 1u, CAU = kCopyAlignUnits<TYPE>;
     using X = FlatX<TYPE, X_BF16>;
     static constexpr uint32_t LPU = kLanesPerUnit<TYPE>, UW = kUnitsPerWindow<TYPE>, BB = kBlockBytes<TYPE>;
 
@@ -284,8 +291,8 @@ struct FlatWalk {
     uint32_t m4, m2, magic;
     uint32_t f_q, f_m, f_w;  // the next task to fetch
     Piece<TYPE> buf[D];
-    [[maybe_unused]] uint4 pv[COPY ? 4 : 1];  // COPY: the window in flight, 16-byte piece lane + 64 i of it
-    [[maybe_unused]] uint4* wbuf;             // COPY: the wave's 4 KB window buffer in LDS
+    [[maybe_unused]] uint4 pv[NPV];  // COPY: the window in flight, 16-byte piece lane + 64 i of it
+    [[maybe_unused]] uint4* wbuf;    // COPY: the wave's window buffer in LDS, 64 NPV slots of 16 bytes
 
     __device__ __forceinline__ void init(const uint8_t* wa, const uint8_t* wb, uint32_t n, uint32_t n_matrices, const FlatGeom& geom,
                                          uint32_t first_super, uint32_t super_stride, uint32_t* lds_queue = nullptr,
@@ -328,20 +335,20 @@ struct FlatWalk {
         u = u < last ? u : last;
         const uint8_t* base = f_m ? w1 : w0;
         if constexpr (COPY) {
-            // the window's units [ub, ub + cnt): a multiple of eight units from the matrix's start (whole 16-byte pieces),
-            // clamped to the matrix (n * bu is a multiple of eight); past a window that ends inside the matrix the last
+            // the window's units [ub, ub + cnt): a multiple of CAU units from the matrix's start (whole 16-byte pieces),
+            // clamped to the matrix (n * bu is a multiple of CAU); past a window that ends inside the matrix the last
             // piece reads up to 14 bytes of the next unit
             const uint32_t total = last + 1u;
             uint32_t ub = (sid << g.log_r) * g.bu + g.uwe * f_w;
-            ub = ub < total ? ub : total - 8u;
+            ub = ub < total ? ub : total - CAU;
             uint32_t cnt = su - g.uwe * f_w;
             cnt = cnt < g.uwe ? cnt : g.uwe;
             cnt = cnt < total - ub ? cnt : total - ub;
             const uint32_t last_piece = (cnt * BB + 15u) / 16u - 1u;
             const uint8_t* wb = base + (size_t)ub * BB;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t pi = lane + 64u * (uint32_t)i;
+            for (uint32_t i = 0; i < NPV; ++i) {
+                const uint32_t pi = lane + 64u * i;
                 pv[i] = ldnt16(wb + 16u * (pi < last_piece ? pi : last_piece));
             }
         } else {
@@ -422,17 +429,26 @@ struct FlatWalk {
                     // the window copied a task ago goes to LDS (behind the wave's reads of the previous one: a wave's LDS
                     // operations are served in order), the next window's copy is issued, this window's fields are read back
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) wbuf[lane + 64u * (uint32_t)i] = pv[i];
+                    for (uint32_t i = 0; i < NPV; ++i) wbuf[lane + 64u * i] = pv[i];
                     asm volatile("" ::: "memory");
                     fetch_next(p);
-                    p.qa = field16(o_qa);
-                    p.qb = field16(o_qa + 32u);
-                    p.qh = field16(o_qh);
-                    const uint32_t* q = wb32 + (o_sc >> 2);
-                    const uint32_t sh = o_sc & 3u, a0 = q[0], a1 = q[1], a2 = q[2];
-                    p.sc = make_uint2(__builtin_amdgcn_alignbyte(a1, a0, sh), __builtin_amdgcn_alignbyte(a2, a1, sh));
-                    const uint32_t* qd = wb32 + (o_d >> 2);
-                    p.d = __builtin_amdgcn_alignbyte(qd[1], qd[0], o_d & 3u);
+                    if constexpr (TYPE == HQ_Q6_K) {
+                        p.qa = field16(o_qa);
+                        p.qb = field16(o_qa + 32u);
+                        p.qh = field16(o_qh);
+                        const uint32_t* q = wb32 + (o_sc >> 2);
+                        const uint32_t sh = o_sc & 3u, a0 = q[0], a1 = q[1], a2 = q[2];
+                        p.sc = make_uint2(__builtin_amdgcn_alignbyte(a1, a0, sh), __builtin_amdgcn_alignbyte(a2, a1, sh));
+                        const uint32_t* qd = wb32 + (o_d >> 2);
+                        p.d = __builtin_amdgcn_alignbyte(qd[1], qd[0], o_d & 3u);
+                    } else {  // a block pair: seventeen words at a multiple of four bytes
+                        const uint32_t* q = wb32 + lv * (BB / 4u);
+                        p.a = make_uint4(q[0], q[1], q[2], q[3]);
+                        p.b = make_uint4(q[4], q[5], q[6], q[7]);
+                        p.c = make_uint4(q[8], q[9], q[10], q[11]);
+                        p.e = make_uint4(q[12], q[13], q[14], q[15]);
+                        p.t = q[16];
+                    }
                 }
                 const uint32_t lu_raw = g.uwe * c_w + lv, su = g.bu << g.log_r;
                 const bool in_task = lu_raw < su;  // false only in the idle part of a ragged last window
