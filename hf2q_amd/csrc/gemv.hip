@@ -890,10 +890,11 @@ int launch_flat(hipStream_t s, const void* x, const uint8_t* w0, const uint8_t* 
                 uint32_t nm, uint32_t cus, bool swiglu = false) {
     if constexpr (kBlock32<TYPE>)
         if (walk_doubled<TYPE, X_BF16>((uint64_t)n * nm, k)) return launch_flat<kX2 + TYPE, X_BF16>(s, x, w0, w1, y0, y1, n, k, nm, cus, swiglu);
-    // waves per CU: 16, for Q6_K 12 (measured with both activation types: f32 262144 x 2816 123 -> 117 us, 8192 x 28672
-    // 43.8 -> 38.9, 4096 x 14336 14.9 -> 13.0; bf16 112 against 121 with 16; the other types are faster or equal with 16,
-    // Q8_0 block pairs mixed: 12288 x 4096 12.3 -> 11.2 with 12, 3584 x 18944 16.4 -> 17.8)
-    constexpr int W = kBaseType<TYPE> == HQ_Q6_K ? 12 : 16;
+    // waves per CU: 16; 12 for Q6_K (measured with both activation types: f32 262144 x 2816 123 -> 117 us, 8192 x 28672
+    // 43.8 -> 38.9, 4096 x 14336 14.9 -> 13.0; bf16 112 against 121 with 16) and for Q8_0 block pairs, whose windows are
+    // copied through LDS (12288 x 4096 12.0 -> 11.1 us, 4096 x 14336 14.2 -> 13.1, 262144 x 2816 127.3 -> 123.1; 5120 x 17408
+    // 19.6 -> 20.3); Q4_K, Q5_K and Q4_0 are faster or equal with 16
+    constexpr int W = kBaseType<TYPE> == HQ_Q6_K || TYPE == HQ_Q8_0_X2 ? 12 : 16;
     using X = FlatX<TYPE, X_BF16>;
     const FArgs fa{x, w0, w1, y0, y1, n, k, nm, swiglu ? 1u : 0u, flat_geom(k, kUnitElems<TYPE>, kUnitsPerWindow<TYPE>, n, nm, cus * W),
                    kBaseType<TYPE> == HQ_Q6_K ? N4 : M4, kBaseType<TYPE> == HQ_Q5_K ? M1 : kBaseType<TYPE> == HQ_Q6_K ? N2 : M2, MAGIC};
