@@ -40,7 +40,7 @@ SETTLE_STEPS = 2400  # untimed decode steps before the steady-state measurements
 # 2.0), WRITE_SIZE all of them (1.0).  The runs and their figures are in profiles/*_pmc_traffic.md.
 PMC_TRAFFIC_BYTES = {
     # (FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0) x 1024 per dispatch
-    "gemv_head_q6_k_151936x4096": int(254241.0 * 2.0 * 1024 + 1187.0 * 1.0 * 1024),
+    "gemv_head_q6_k_151936x4096": int(254476.8 * 2.0 * 1024 + 1187.0 * 1.0 * 1024),
     # activation pre-pass + tile GEMM, Q4_K, 2048 x 12288 x 4096 (the GEMM re-fetches the weights once per 256-token tile)
     "prefill_gemm_q4_k_2048x12288x4096": int((23301.6 + 132573.1) * 2.0 * 1024 + (16496.5 + 98311.8) * 1.0 * 1024),
     # split (with the q rotation) + merge (with the output rotation), 32K context, 2 kv heads, head_dim 256
