@@ -913,6 +913,17 @@ int launch_flat(hipStream_t s, const void* x, const uint8_t* w0, const uint8_t* 
             lds += (size_t)W * 4096u;
         }
     }
+    if constexpr (TYPE == kX2 + HQ_Q4_0) {
+        // Q4_0 block pairs (windows of 2304 bytes, nine words per lane): 12288 x 4096 8.3 -> 7.4 us, 17408 x 5120 14.5 -> 12.7,
+        // 8192 x 28672 28.6 -> 26.0, f32 activations 8.5 -> 7.5 / 15.3 -> 14.0 / the same; with f32 activations and rows shorter
+        // than a window (262144 x 2816) 89.8 -> 93.9, so not there
+        constexpr size_t wb = (size_t)W * 64u * kCopyNPV<TYPE> * 16u;
+        if ((X_BF16 || fa.g.bu >= kUnitsPerWindow<TYPE>) && flat_copy_fits(fa.g, kUnitsPerWindow<TYPE>, n, kCopyAlignUnits<TYPE>, reinterpret_cast<uintptr_t>(w0), reinterpret_cast<uintptr_t>(w1)) &&
+            lds + wb <= 160 * 1024 - 512) {
+            kern = dyn ? gemv_flat_kernel<TYPE, X_BF16, W, 1, true, true> : gemv_flat_kernel<TYPE, X_BF16, W, 1, false, true>;
+            lds += wb;
+        }
+    }
     if constexpr (TYPE == HQ_Q8_0_X2) {
         // Q8_0 block pairs (windows of 4352 bytes, read back as seventeen aligned words per lane), either activation type:
         // lm_head 262144 x 2816 140.7 -> 127.2 us (f32 135.0 -> 122.8), 5120 x 17408 21.3 -> 20.2, 12288 x 4096 12.3 -> 12.0

@@ -253,10 +253,11 @@ struct FlatX<TYPE, X_BF16, true> {
 // The SIMD's issue arbitration favours its oldest wave, so with equal shares the youngest wave of every SIMD finishes long
 // after the others; with the counter all waves of a CU end together.  A wave claims its next super-task one ahead, so its
 // fetch runs on across the boundary.
-// COPY (Q6_K and Q8_0 block pairs, D == 1): a window is not fetched by the lanes that use it, five instructions touching
+// COPY (Q6_K, Q8_0 and Q4_0 block pairs, D == 1): a window is not fetched by the lanes that use it, five instructions touching
 // each 128-byte line, but copied -- consecutive lanes consecutive 16-byte pieces, non-temporal loads, every line asked
 // for once -- into 4-5 KB of LDS the wave owns, and the lanes read their pieces back from there (Q6_K blocks lie 210
-// bytes apart: aligned words shifted into place by v_alignbyte; a Q8_0 block pair is seventeen aligned words); the next
+// bytes apart: aligned words shifted into place by v_alignbyte; a Q8_0 block pair is seventeen aligned words, a Q4_0
+// pair nine); the next
 // window's copy is in flight meanwhile.  The same pieces, the same sums.  The host checks flat_copy_fits: every window
 // starts at a multiple of 16 bytes and no copy reads past the matrix.
 // (au: the units after which a window start is a multiple of 16 bytes again: 8 for Q6_K's 210 bytes, 4 for a Q8_0 block pair's 68)
@@ -270,7 +271,7 @@ constexpr uint32_t kCopyNPV = (kUnitsPerWindow<TYPE> * kBlockBytes<TYPE> / 16u +
 template <int TYPE, bool X_BF16, int D = 1, bool XHALF = false, bool DYN = false, bool COPY = false>
 struct FlatWalk {
     static_assert(!DYN || D == 1, "the dynamic split keeps one fetch in flight");
-    static_assert(!COPY || ((TYPE == HQ_Q6_K || TYPE == HQ_Q8_0_X2) && D == 1 && !XHALF), "Q6_K super-blocks or Q8_0 block pairs, one window in flight");
+    static_assert(!COPY || ((TYPE == HQ_Q6_K || TYPE == HQ_Q8_0_X2 || TYPE == kX2 + HQ_Q4_0) && D == 1 && !XHALF), "Q6_K super-blocks or block pairs, one window in flight");
     static constexpr uint32_t NPV = COPY ? kCopyNPV<TYPE> : 1u, CAU = kCopyAlignUnits<TYPE>;
     using X = FlatX<TYPE, X_BF16>;
     static constexpr uint32_t LPU = kLanesPerUnit<TYPE>, UW = kUnitsPerWindow<TYPE>, BB = kBlockBytes<TYPE>;
@@ -441,6 +442,14 @@ struct FlatWalk {
                         p.sc = make_uint2(__builtin_amdgcn_alignbyte(a1, a0, sh), __builtin_amdgcn_alignbyte(a2, a1, sh));
                         const uint32_t* qd = wb32 + (o_d >> 2);
                         p.d = __builtin_amdgcn_alignbyte(qd[1], qd[0], o_d & 3u);
+                    } else if constexpr (TYPE == kX2 + HQ_Q4_0) {  // [d0][16 bytes][d1][16 bytes] as nine words at a multiple of four bytes
+                        const uint32_t* q = wb32 + lv * (BB / 4u);
+                        const uint32_t w0 = q[0], w1 = q[1], w2 = q[2], w3 = q[3], w4 = q[4];
+                        p.a.d = w0 & 0xffffu;
+                        p.a.q = make_uint4(__builtin_amdgcn_alignbyte(w1, w0, 2), __builtin_amdgcn_alignbyte(w2, w1, 2),
+                                           __builtin_amdgcn_alignbyte(w3, w2, 2), __builtin_amdgcn_alignbyte(w4, w3, 2));
+                        p.b.d = w4 >> 16;
+                        p.b.q = make_uint4(q[5], q[6], q[7], q[8]);
                     } else {  // a block pair: seventeen words at a multiple of four bytes
                         const uint32_t* q = wb32 + lv * (BB / 4u);
                         p.a = make_uint4(q[0], q[1], q[2], q[3]);
