@@ -10,9 +10,15 @@ library's own quantizer (byte-identical to hf2q's CPU quantizers).  One "step"
 is one pass over those four GEMVs.  Several distinct weight sets are rotated so
 that no step finds its weights in the 256 MB Infinity Cache.
 
+The K timed steps behind `value` are replayed from HIP graphs after the W warm-up
+steps, a run of further untimed steps and the per-kernel measurements: the device
+takes 100-200 ms of continuous work to reach its steady rate (the same K steps
+timed right after set-up are reported as `config.us_per_step_first_region`).
+
 Prints ONE JSON line: metric = effective GB/s of packed weight bytes, with a
-`roofline` object for the dominant kernel (the Q6_K head GEMV) from HIP-event
-timings taken inside the timed region, a `kernels` table for the others, a
+`roofline` object for the dominant kernel (the Q6_K head GEMV) from HIP event
+pairs around every head launch of host-launched steps, a `kernels` table for the others
+(back-to-back launches of one kind, medians over graph replays), a
 `workloads` object with the other BASELINE configurations (MoE decode at 1 and 8
 tokens, its prefill-sized grouped mul_mat_id, the Q4_K and Q8_0 prefill GEMM, the
 TQ attention), each with its own
