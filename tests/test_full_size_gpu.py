@@ -120,6 +120,32 @@ def test_weights_copied_through_lds_f32_and_short_rows(oracle, dev, xdt, t, n, k
     assert torch.equal(y, y2)
 
 
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("t,n,k", [(HQ_Q6_K, 8192, 4096), (HQ_Q6_K, 4096, 5120), (HQ_Q6_K, 2048, 8192), (HQ_Q8_0, 8192, 4096),
+                                   (HQ_Q8_0, 12288, 2816), (HQ_Q4_0, 8192, 4096)])
+def test_copy_forms_and_their_fallbacks_give_the_same_bits(dev, xdt, t, n, k):
+    """The forms that copy weights through LDS need every copy to start on a 16-byte boundary; a matrix whose base is
+    not a multiple of 16 takes the kernels whose lanes fetch their own pieces.  Both compute the same pieces, products and
+    sums: the outputs are equal bit for bit (Q6_K chunk copy, the flat walk's copied windows for Q6_K, Q8_0 and Q4_0)."""
+    w = _quantized(dev, n, k, t, 21 + n + k)
+    g = torch.Generator(device=dev)
+    g.manual_seed(n + k)
+    x = torch.randn(1, k, generator=g, device=dev)
+    x = x.to(torch.bfloat16) if xdt == "bf16" else x
+    p = GgmlQuantizedMatmulParams(1, n, k, t)
+    y = torch.full((1, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(x, w, y, p)
+    assert torch.isfinite(y).all()
+    for off in (2, 8):
+        holder = torch.zeros(w.numel() + 32, dtype=torch.uint8, device=dev)
+        shifted = holder[off:off + w.numel()]
+        shifted.copy_(w)
+        assert shifted.data_ptr() % 16 == off
+        y2 = torch.full((1, n), float("nan"), device=dev)
+        ops.quantized_matmul_ggml(x, shifted, y2, p)
+        assert torch.equal(y, y2), (t, n, k, xdt, off)
+
+
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048)])
