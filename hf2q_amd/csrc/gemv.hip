@@ -740,9 +740,159 @@ inline bool q6k_rowcopy_takes(const void* w, uint32_t n, uint32_t k, uint32_t cu
     return (k == 4096 || k == 2048) && (reinterpret_cast<uintptr_t>(w) & 15u) == 0 && (uint64_t)n * (k / 256u) >= (uint64_t)512u * cus;
 }
 
+// Q6_K rows of 9 .. 15 super-blocks (k = 2304 .. 3840: rows shorter than a window of sixteen).  The matrix is cut into
+// the flat walk's windows of sixteen blocks; the pattern of row boundaries inside a window repeats every P = bu / gcd(bu, 16)
+// windows = R = 16 / gcd(bu, 16) rows (k = 2816: 11 windows, 16 rows).  Wave j of a workgroup takes window j of every
+// period the workgroup owns: which super-block of a row a lane's quarter belongs to never changes, so its activations sit
+// in registers (the flat walk reads them from LDS for every window), the rows a window touches are the same lane ranges
+// every time, and the window is copied through LDS as in the row-copy kernel above (windows are 26.25 lines long: a line
+// at a window's edge is asked for by two waves of the workgroup).  A window's per-row sums (one masked wave reduction per row it touches) go to slots in LDS, first-window and second-window
+// part of every row; after a barrier the workgroup adds the two in the flat walk's order and stores the rows: the same
+// bits as the flat walk gives with full windows.
+struct PArgs {
+    const void* x;
+    const uint8_t* w;
+    float* y;
+    uint32_t n, k, bu;
+    uint32_t period_windows, log_period_rows;  // P, log2 R
+    uint32_t seqs;                             // the workgroup's waves are seqs * P: sequence s takes every seqs-th period of the workgroup
+    uint32_t periods_per_round;                // slots in LDS: periods_per_round * R * 2 floats
+    uint32_t m4, m2, magic;
+};
+template <bool X_BF16>
+__global__ __launch_bounds__(1024) void gemv_q6k_period_kernel(PArgs a) {
+    constexpr uint32_t CHUNKB = 16u * Q6K_BYTES, PIECES = CHUNKB / 16u;  // 3360 bytes, 210 pieces
+    using X = FlatX<HQ_Q6_K, X_BF16>;
+    extern __shared__ uint4 smem[];
+    uint4* lds_x = smem;
+    float* lds_s = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(smem) + X::value_bytes(a.k));
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, nthreads = blockDim.x;
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    uint4* wbuf = reinterpret_cast<uint4*>(lds_s + a.k / 16u) + wv * 256u;
+    float* slots = reinterpret_cast<float*>(reinterpret_cast<uint4*>(lds_s + a.k / 16u) + (nthreads >> 6) * 256u);
+    const int c = (int)(lane & 3u);
+    const uint32_t P = a.period_windows, LR = a.log_period_rows, R = 1u << LR;
+    const uint32_t j = wv % P, sq = wv / P;  // window of the period, sequence
+    const uint32_t periods = a.n >> LR;
+    const uint32_t cnt_wg = blockIdx.x < periods ? (periods - blockIdx.x + gridDim.x - 1u) / gridDim.x : 0u;
+
+    X::stage(a.x, a.k, lds_x, lds_s, tid, nthreads);
+
+    // period i of the workgroup's, window j (non-temporal loads throughout: fetching the pieces on the two lines a window
+    // shares with its neighbours with ordinary loads measured the same, ordinary loads for all of it 4 % slower)
+    uint4 pv[4];
+    auto fetch = [&](uint32_t i) {
+        const uint8_t* base = a.w + ((size_t)(blockIdx.x + i * gridDim.x) * P + j) * CHUNKB;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t pc = lane + 64u * (uint32_t)q;
+            pv[q] = ldnt16(base + 16u * (pc < PIECES - 1u ? pc : PIECES - 1u));
+        }
+    };
+    uint32_t i_cur = sq;
+    if (i_cur < cnt_wg) fetch(i_cur);
+    __syncthreads();
+
+    [[maybe_unused]] uint32_t m4, m2, magic;
+    if constexpr (X_BF16)
+        asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5" : "=v"(m4), "=v"(m2), "=v"(magic) : "s"(a.m4), "s"(a.m2), "s"(a.magic));
+    // the lane's block of the period, its row there and its super-block of that row
+    const uint32_t bi = 16u * j + (lane >> 2), rl = bi / a.bu, ur = bi - rl * a.bu;
+    const uint32_t r_lo = (16u * j) / a.bu, nseg = (16u * j + 15u) / a.bu - r_lo + 1u;  // rows the window touches: r_lo .. r_lo + nseg - 1
+    const uint32_t seg = rl - r_lo;
+    uint32_t xr[X::XW];
+    float sx[4];
+    X::load(lds_x, lds_s, ur, c, xr, sx);
+    // lane s < nseg stores the sum of row r_lo + s: slot 0 if this is the row's first window, 1 if its second
+    const uint32_t my_row = r_lo + (lane < nseg ? lane : 0u);
+    const uint32_t my_slot = 2u * my_row + ((my_row * a.bu) / 16u == j ? 0u : 1u);
+
+    const uint32_t blk = (lane >> 2) * Q6K_BYTES, h = (uint32_t)c >> 1, lr = (uint32_t)c & 1u;
+    const uint32_t* wb32 = reinterpret_cast<const uint32_t*>(wbuf);
+    const uint32_t o_qa = blk + 64u * h + 16u * lr, o_qb = o_qa + 32u, o_qh = blk + 128u + 32u * h + 16u * lr, o_sc = blk + 192u + 8u * h,
+                   o_d = blk + 206u;
+    auto field16 = [&](uint32_t o) -> uint4 {
+        const uint32_t* p = wb32 + (o >> 2);
+        const uint32_t sh = o & 3u, w0 = p[0], w1 = p[1], w2 = p[2], w3 = p[3], w4 = p[4];
+        return make_uint4(__builtin_amdgcn_alignbyte(w1, w0, sh), __builtin_amdgcn_alignbyte(w2, w1, sh), __builtin_amdgcn_alignbyte(w3, w2, sh),
+                          __builtin_amdgcn_alignbyte(w4, w3, sh));
+    };
+
+    for (uint32_t i0 = 0; i0 < cnt_wg; i0 += a.periods_per_round) {
+        const uint32_t i1 = i0 + a.periods_per_round < cnt_wg ? i0 + a.periods_per_round : cnt_wg;
+        while (i_cur < i1) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) wbuf[lane + 64u * (uint32_t)q] = pv[q];
+            asm volatile("" ::: "memory");
+            if (i_cur + a.seqs < cnt_wg) fetch(i_cur + a.seqs);
+            Piece<HQ_Q6_K> pc;
+            pc.qa = field16(o_qa);
+            pc.qb = field16(o_qb);
+            pc.qh = field16(o_qh);
+            {
+                const uint32_t* p = wb32 + (o_sc >> 2);
+                const uint32_t sh = o_sc & 3u, w0 = p[0], w1 = p[1], w2 = p[2];
+                pc.sc = make_uint2(__builtin_amdgcn_alignbyte(w1, w0, sh), __builtin_amdgcn_alignbyte(w2, w1, sh));
+                const uint32_t* q = wb32 + (o_d >> 2);
+                pc.d = __builtin_amdgcn_alignbyte(q[1], q[0], o_d & 3u);
+            }
+            float part;
+            if constexpr (X_BF16) part = dot_pair(pc, c, xr, sx, m4, m2, magic);
+            else part = dot_f32(pc, c, reinterpret_cast<const float*>(xr), sx);
+            float mine = group_sum(seg == 0u ? part : 0.f, 6);
+            if (nseg > 1u) {
+                const float v = group_sum(seg == 1u ? part : 0.f, 6);
+                mine = lane == 1u ? v : mine;
+            }
+            if (nseg > 2u) {
+                const float v = group_sum(seg == 2u ? part : 0.f, 6);
+                mine = lane == 2u ? v : mine;
+            }
+            if (lane < nseg) slots[(((i_cur - i0) << LR) << 1) + my_slot] = mine;
+            i_cur += a.seqs;
+        }
+        __syncthreads();
+        // row r of a period lies in one window or in two: 0 + first (+ second), the flat walk's order
+        const uint32_t rows = (i1 - i0) << LR;
+        for (uint32_t idx = tid; idx < rows; idx += nthreads) {
+            const uint32_t r = idx & (R - 1u), fb = r * a.bu;
+            float y = 0.f + slots[2u * idx];
+            if (fb / 16u != (fb + a.bu - 1u) / 16u) y += slots[2u * idx + 1u];
+            a.y[((size_t)(blockIdx.x + (i0 + (idx >> LR)) * gridDim.x) << LR) + r] = y;
+        }
+        if (i1 < cnt_wg) __syncthreads();
+    }
+}
+// One 16-byte aligned Q6_K matrix with rows of 9 .. 15 super-blocks, whole periods of rows, sixteen periods per workgroup or
+// more, and the shape for which the flat walk would use full windows over whole periods (so that both give the same bits).
+inline bool q6k_period_takes(const void* w, uint32_t n, uint32_t k, uint32_t cus, bool x_bf16) {
+    if (k % 256u) return false;
+    const uint32_t bu = k / 256u;
+    if (bu <= 8u || bu >= 16u || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
+    const uint32_t g = bu % 2u ? 1u : bu % 4u ? 2u : bu % 8u ? 4u : 8u, P = bu / g, R = 16u / g;
+    if (n % R || (uint64_t)(n / R) < (uint64_t)16u * cus || (uint64_t)n * bu >= 0x7fff0000ull) return false;
+    const FlatGeom fg = flat_geom(k, 256u, 16u, n, 1u, cus * 12u);
+    return fg.uwe == 16u && (1u << fg.log_r) == R;
+}
+template <bool X_BF16>
+int launch_q6k_period(hipStream_t s, const void* x, const uint8_t* w, float* y, uint32_t n, uint32_t k, uint32_t cus) {
+    const uint32_t bu = k / 256u, g = bu % 2u ? 1u : bu % 4u ? 2u : bu % 8u ? 4u : 8u, P = bu / g, R = 16u / g;
+    const uint32_t seqs = 16u / P, W = seqs * P;
+    uint32_t log_r = 0;
+    while ((1u << log_r) < R) ++log_r;
+    const uint32_t periods = n / R, per_wg = (periods + cus - 1u) / cus;
+    const uint32_t ppr = per_wg < 128u ? per_wg : 128u;
+    const PArgs pa{x, w, y, n, k, bu, P, log_r, seqs, ppr, N4, N2, MAGIC};
+    const size_t lds = FlatX<HQ_Q6_K, X_BF16>::lds_bytes(k) + (size_t)W * 4096u + (size_t)ppr * R * 8u;
+    auto kern = gemv_q6k_period_kernel<X_BF16>;
+    if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv period LDS)")) return rc;
+    hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, pa);
+    return check_launch("gemv period kernel launch");
+}
+
 // Whether the streaming form takes (type, k, rows): K-quants, whole 4096-element steps, enough rows to occupy the waves.
 template <int TYPE>
-constexpr bool kStreamType = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K;
+constexpr bool kStreamType =TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K;
 constexpr uint32_t STREAM_MIN_ROWS_PER_WAVE = 2;
 
 template <int TYPE, int ROWS = 1>
@@ -1044,6 +1194,16 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
                                a.y + (size_t)r * a.n, a.n, a.n, a.k, N4, N2, MAGIC};
                 if (int rc = launch_q6k_rowcopy<X_BF16>(s, sa, cus)) return rc;
             }
+            return HQ_OK;
+        }
+    }
+    // Q6_K rows of 9 .. 15 super-blocks (lm_heads of hidden size 2560 .. 3840): a fixed window of the period per wave, a pass per row.
+    if constexpr (TYPE == HQ_Q6_K) {
+        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && q6k_period_takes(a.w, a.n, a.k, cus, X_BF16)) {
+            for (uint32_t r = 0; r < a.pairs; ++r)
+                if (int rc = launch_q6k_period<X_BF16>(s, static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * (X_BF16 ? 2 : 4), a.w,
+                                                       a.y + (size_t)r * a.n, a.n, a.k, cus))
+                    return rc;
             return HQ_OK;
         }
     }

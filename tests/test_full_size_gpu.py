@@ -146,6 +146,45 @@ def test_copy_forms_and_their_fallbacks_give_the_same_bits(dev, xdt, t, n, k):
         assert torch.equal(y, y2), (t, n, k, xdt, off)
 
 
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+@pytest.mark.parametrize("n,k", [(262144, 2816), (151936, 2560), (151936, 3072), (152064, 3584), (131072, 3840)])
+def test_q6k_rows_shorter_than_a_window(oracle, dev, xdt, n, k):
+    """Q6_K lm_heads whose rows are 9 .. 15 super-blocks (hidden sizes 2560 .. 3840): every wave of a workgroup takes one
+    fixed window of the period after which the row boundaries repeat (11 windows = 16 rows for k = 2816, 5 = 8 for 2560,
+    3 = 4 for 3072, 7 = 8 for 3584, 15 = 16 for 3840), the rows' parts meet in LDS.  151936 x 3072 leaves a workgroup more
+    periods than its slots hold (two rounds) and a ragged share.  Sampled rows against the f64 oracle; the same bits as
+    the flat walk, which a matrix off the 16-byte grid takes; two activation rows = two passes; the same on a second call."""
+    t = HQ_Q6_K
+    w = _quantized(dev, n, k, t, 31 + n + k)
+    rng = np.random.default_rng(n + k)
+    x = (rng.integers(-12, 13, (2, k)) / 8.0).astype(np.float32)
+    xd = torch.from_numpy(x).to(dev)
+    xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
+    p = GgmlQuantizedMatmulParams(1, n, k, t)
+    y = torch.full((1, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd[0:1], w, y, p)
+    assert torch.isfinite(y).all()
+    rows = np.unique(np.concatenate([np.arange(0, 34), np.arange(n - 34, n), rng.integers(0, n, 60)]))
+    xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
+    ref = oracle.qmatmul_f64(xv, _rows_of(w, rows, k, t, oracle), 2, rows.size, k, t)
+    sel = torch.as_tensor(rows, device=dev)
+    assert_matmul_close(y[:, sel].cpu().numpy(), ref[0:1], f"q6_k {xdt} {n}x{k}, sampled rows")
+    holder = torch.zeros(w.numel() + 32, dtype=torch.uint8, device=dev)
+    shifted = holder[2:2 + w.numel()]
+    shifted.copy_(w)
+    ys = torch.full((1, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd[0:1], shifted, ys, p)
+    assert torch.equal(y, ys), (n, k, xdt)
+    del holder, shifted, ys
+    y2 = torch.full((2, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd, w, y2, GgmlQuantizedMatmulParams(2, n, k, t))
+    assert torch.equal(y2[0:1], y)
+    assert_matmul_close(y2[:, sel].cpu().numpy(), ref, f"q6_k {xdt} {n}x{k}, two rows")
+    y3 = torch.full((1, n), float("nan"), device=dev)
+    ops.quantized_matmul_ggml(xd[0:1], w, y3, p)
+    assert torch.equal(y, y3)
+
+
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
 @pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048)])
