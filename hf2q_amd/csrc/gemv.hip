@@ -740,15 +740,19 @@ inline bool q6k_rowcopy_takes(const void* w, uint32_t n, uint32_t k, uint32_t cu
     return (k == 4096 || k == 2048) && (reinterpret_cast<uintptr_t>(w) & 15u) == 0 && (uint64_t)n * (k / 256u) >= (uint64_t)512u * cus;
 }
 
-// Q6_K rows of 9 .. 15 super-blocks (k = 2304 .. 3840: rows shorter than a window of sixteen).  The matrix is cut into
-// the flat walk's windows of sixteen blocks; the pattern of row boundaries inside a window repeats every P = bu / gcd(bu, 16)
-// windows = R = 16 / gcd(bu, 16) rows (k = 2816: 11 windows, 16 rows).  Wave j of a workgroup takes window j of every
-// period the workgroup owns: which super-block of a row a lane's quarter belongs to never changes, so its activations sit
-// in registers (the flat walk reads them from LDS for every window), the rows a window touches are the same lane ranges
-// every time, and the window is copied through LDS as in the row-copy kernel above (windows are 26.25 lines long: a line
-// at a window's edge is asked for by two waves of the workgroup).  A window's per-row sums (one masked wave reduction per row it touches) go to slots in LDS, first-window and second-window
-// part of every row; after a barrier the workgroup adds the two in the flat walk's order and stores the rows: the same
-// bits as the flat walk gives with full windows.
+// Q6_K rows of nine super-blocks or more that are not whole windows of sixteen (k = 2560, 2816, 3072, 3584, 3840, 5120, 7168,
+// 14336 ...).  The matrix is cut into the flat walk's windows of sixteen blocks; the pattern of row boundaries inside a
+// window repeats every P = bu / gcd(bu, 16) windows = R = 16 / gcd(bu, 16) rows (k = 2816: 11 windows, 16 rows; k = 5120: 5
+// windows, 4 rows).  Wave j of a sequence of P waves takes window j of every period the sequence owns: which super-block
+// of a row a lane's quarter belongs to never changes, so its activations sit in registers (the flat walk reads them from
+// LDS for every window), the rows a window touches are the same lane ranges every time, and the window is copied through
+// LDS as in the row-copy kernel above (windows are 26.25 lines long: a line at a window's edge is asked for by two waves of
+// the workgroup).  A window's per-row sums (one masked wave reduction per row it touches, three at most) go to slots in LDS,
+// one per window a row lies in; after a barrier the workgroup adds a row's slots in the flat walk's order and stores the
+// rows: the same bits as the flat walk gives with full windows.  Measured against the flat walk (bf16 / f32 activations):
+// 262144 x 2816 113 -> 100 / 118 -> 110 us, 152064 x 5120 112.6 -> 100.6 / 118.8 -> 108.9, 152064 x 3584 82.7 -> 75.3 /
+// 85.7 -> 79.9, 32768 x 14336 71.4 -> 62.6 / 74.1 -> 67.4; with fewer than a dozen windows per wave the fixed shares leave
+// waves idle at the end and the flat walk is as fast or faster.
 struct PArgs {
     const void* x;
     const uint8_t* w;
@@ -756,7 +760,8 @@ struct PArgs {
     uint32_t n, k, bu;
     uint32_t period_windows, log_period_rows;  // P, log2 R
     uint32_t seqs;                             // the workgroup's waves are seqs * P: sequence s takes every seqs-th period of the workgroup
-    uint32_t periods_per_round;                // slots in LDS: periods_per_round * R * 2 floats
+    uint32_t row_slots;                        // windows a row can lie in
+    uint32_t periods_per_round;                // slots in LDS: periods_per_round * R * row_slots floats
     uint32_t m4, m2, magic;
 };
 template <bool X_BF16>
@@ -803,9 +808,9 @@ __global__ __launch_bounds__(1024) void gemv_q6k_period_kernel(PArgs a) {
     uint32_t xr[X::XW];
     float sx[4];
     X::load(lds_x, lds_s, ur, c, xr, sx);
-    // lane s < nseg stores the sum of row r_lo + s: slot 0 if this is the row's first window, 1 if its second
-    const uint32_t my_row = r_lo + (lane < nseg ? lane : 0u);
-    const uint32_t my_slot = 2u * my_row + ((my_row * a.bu) / 16u == j ? 0u : 1u);
+    // lane s < nseg stores the sum of row r_lo + s: slot 0 if this is the row's first window, 1 if its second ...
+    const uint32_t my_row = r_lo + (lane < nseg ? lane : 0u), MW = a.row_slots;
+    const uint32_t my_slot = MW * my_row + (j - (my_row * a.bu) / 16u);
 
     const uint32_t blk = (lane >> 2) * Q6K_BYTES, h = (uint32_t)c >> 1, lr = (uint32_t)c & 1u;
     const uint32_t* wb32 = reinterpret_cast<const uint32_t*>(wbuf);
@@ -848,29 +853,35 @@ __global__ __launch_bounds__(1024) void gemv_q6k_period_kernel(PArgs a) {
                 const float v = group_sum(seg == 2u ? part : 0.f, 6);
                 mine = lane == 2u ? v : mine;
             }
-            if (lane < nseg) slots[(((i_cur - i0) << LR) << 1) + my_slot] = mine;
+            if (lane < nseg) slots[((i_cur - i0) << LR) * MW + my_slot] = mine;
             i_cur += a.seqs;
         }
         __syncthreads();
-        // row r of a period lies in one window or in two: 0 + first (+ second), the flat walk's order
+        // the windows of row r of a period, added in the flat walk's order: 0 + first + second ...
         const uint32_t rows = (i1 - i0) << LR;
         for (uint32_t idx = tid; idx < rows; idx += nthreads) {
-            const uint32_t r = idx & (R - 1u), fb = r * a.bu;
-            float y = 0.f + slots[2u * idx];
-            if (fb / 16u != (fb + a.bu - 1u) / 16u) y += slots[2u * idx + 1u];
+            const uint32_t r = idx & (R - 1u), fb = r * a.bu, nwin = (fb + a.bu - 1u) / 16u - fb / 16u + 1u;
+            float y = 0.f;
+            for (uint32_t sl = 0; sl < nwin; ++sl) y += slots[MW * idx + sl];
             a.y[((size_t)(blockIdx.x + (i0 + (idx >> LR)) * gridDim.x) << LR) + r] = y;
         }
         if (i1 < cnt_wg) __syncthreads();
     }
 }
-// One 16-byte aligned Q6_K matrix with rows of 9 .. 15 super-blocks, whole periods of rows, sixteen periods per workgroup or
-// more, and the shape for which the flat walk would use full windows over whole periods (so that both give the same bits).
+inline size_t q6k_period_lds(uint32_t k, bool x_bf16, uint32_t waves, uint32_t slots) {
+    return (x_bf16 ? FlatX<HQ_Q6_K, true>::lds_bytes(k) : FlatX<HQ_Q6_K, false>::lds_bytes(k)) + (size_t)waves * 4096u + (size_t)slots * 4u;
+}
+// One 16-byte aligned Q6_K matrix, rows of nine super-blocks or more and not whole windows, a period of sixteen windows at
+// most, whole periods of rows, 176 windows per workgroup or more, ten waves or more with f32 activations (nine: 65536 x 4608
+// 48.3 -> 49.3 us), and a shape for which the flat walk would use full windows over whole periods (so that both give the
+// same bits).
 inline bool q6k_period_takes(const void* w, uint32_t n, uint32_t k, uint32_t cus, bool x_bf16) {
     if (k % 256u) return false;
     const uint32_t bu = k / 256u;
-    if (bu <= 8u || bu >= 16u || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
+    if (bu <= 8u || bu % 16u == 0u || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
     const uint32_t g = bu % 2u ? 1u : bu % 4u ? 2u : bu % 8u ? 4u : 8u, P = bu / g, R = 16u / g;
-    if (n % R || (uint64_t)(n / R) < (uint64_t)16u * cus || (uint64_t)n * bu >= 0x7fff0000ull) return false;
+    if (P > 16u || n % R || (uint64_t)(n / R) * P < (uint64_t)176u * cus || (uint64_t)n * bu >= 0x7fff0000ull) return false;
+    if ((!x_bf16 && 16u / P * P < 10u) || q6k_period_lds(k, x_bf16, 16u / P * P, 4096u) > 160u * 1024u - 512u) return false;
     const FlatGeom fg = flat_geom(k, 256u, 16u, n, 1u, cus * 12u);
     return fg.uwe == 16u && (1u << fg.log_r) == R;
 }
@@ -881,9 +892,10 @@ int launch_q6k_period(hipStream_t s, const void* x, const uint8_t* w, float* y, 
     uint32_t log_r = 0;
     while ((1u << log_r) < R) ++log_r;
     const uint32_t periods = n / R, per_wg = (periods + cus - 1u) / cus;
-    const uint32_t ppr = per_wg < 128u ? per_wg : 128u;
-    const PArgs pa{x, w, y, n, k, bu, P, log_r, seqs, ppr, N4, N2, MAGIC};
-    const size_t lds = FlatX<HQ_Q6_K, X_BF16>::lds_bytes(k) + (size_t)W * 4096u + (size_t)ppr * R * 8u;
+    const uint32_t mw = (bu + 14u) / 16u + 1u, cap = 4096u / (R * mw);  // 16 KB of slots
+    const uint32_t ppr = per_wg < cap ? per_wg : cap;
+    const PArgs pa{x, w, y, n, k, bu, P, log_r, seqs, mw, ppr, N4, N2, MAGIC};
+    const size_t lds = q6k_period_lds(k, X_BF16, W, ppr * R * mw);
     auto kern = gemv_q6k_period_kernel<X_BF16>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv period LDS)")) return rc;
     hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, pa);
@@ -1197,7 +1209,8 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
             return HQ_OK;
         }
     }
-    // Q6_K rows of 9 .. 15 super-blocks (lm_heads of hidden size 2560 .. 3840): a fixed window of the period per wave, a pass per row.
+    // Q6_K rows that are not whole windows (lm_heads of hidden size 2560 .. 3840, 5120, 7168; k = 14336): a fixed window of the
+    // row period per wave, a pass per row.
     if constexpr (TYPE == HQ_Q6_K) {
         if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && q6k_period_takes(a.w, a.n, a.k, cus, X_BF16)) {
             for (uint32_t r = 0; r < a.pairs; ++r)

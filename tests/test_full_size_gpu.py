@@ -147,12 +147,14 @@ def test_copy_forms_and_their_fallbacks_give_the_same_bits(dev, xdt, t, n, k):
 
 
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
-@pytest.mark.parametrize("n,k", [(262144, 2816), (151936, 2560), (151936, 3072), (152064, 3584), (131072, 3840)])
-def test_q6k_rows_shorter_than_a_window(oracle, dev, xdt, n, k):
-    """Q6_K lm_heads whose rows are 9 .. 15 super-blocks (hidden sizes 2560 .. 3840): every wave of a workgroup takes one
-    fixed window of the period after which the row boundaries repeat (11 windows = 16 rows for k = 2816, 5 = 8 for 2560,
-    3 = 4 for 3072, 7 = 8 for 3584, 15 = 16 for 3840), the rows' parts meet in LDS.  151936 x 3072 leaves a workgroup more
-    periods than its slots hold (two rounds) and a ragged share.  Sampled rows against the f64 oracle; the same bits as
+@pytest.mark.parametrize("n,k", [(262144, 2816), (151936, 2560), (151936, 3072), (152064, 3584), (131072, 3840), (152064, 5120),
+                                 (65536, 7168), (32768, 14336)])
+def test_q6k_rows_that_are_not_whole_windows(oracle, dev, xdt, n, k):
+    """Q6_K matrices whose rows are not whole windows of sixteen super-blocks (hidden sizes 2560 .. 3840, 5120, 7168; k =
+    14336): every wave takes one fixed window of the period after which the row boundaries repeat (11 windows = 16 rows
+    for k = 2816, 5 = 8 for 2560, 3 = 4 for 3072, 7 = 8 for 3584, 15 = 16 for 3840, 5 = 4 for 5120, 7 = 4 for 7168, 7 = 2 for
+    14336), the rows' parts meet in LDS.  151936 x 3072 leaves a workgroup more periods than its slots hold (two rounds)
+    and a ragged share.  Sampled rows against the f64 oracle; the same bits as
     the flat walk, which a matrix off the 16-byte grid takes; two activation rows = two passes; the same on a second call."""
     t = HQ_Q6_K
     w = _quantized(dev, n, k, t, 31 + n + k)
