@@ -740,19 +740,21 @@ inline bool q6k_rowcopy_takes(const void* w, uint32_t n, uint32_t k, uint32_t cu
     return (k == 4096 || k == 2048) && (reinterpret_cast<uintptr_t>(w) & 15u) == 0 && (uint64_t)n * (k / 256u) >= (uint64_t)512u * cus;
 }
 
-// Q6_K rows of nine super-blocks or more that are not whole windows of sixteen (k = 2560, 2816, 3072, 3584, 3840, 5120, 7168,
-// 14336 ...).  The matrix is cut into the flat walk's windows of sixteen blocks; the pattern of row boundaries inside a
-// window repeats every P = bu / gcd(bu, 16) windows = R = 16 / gcd(bu, 16) rows (k = 2816: 11 windows, 16 rows; k = 5120: 5
+// K-quant rows of nine super-blocks or more that are not whole windows of sixteen (k = 2560, 2816, 3072, 3584, 3840, 5120,
+// 7168, 14336 ...).  The matrix is cut into the flat walk's windows of sixteen blocks; the pattern of row boundaries inside
+// a window repeats every P = bu / gcd(bu, 16) windows = R = 16 / gcd(bu, 16) rows (k = 2816: 11 windows, 16 rows; k = 5120: 5
 // windows, 4 rows).  Wave j of a sequence of P waves takes window j of every period the sequence owns: which super-block
 // of a row a lane's quarter belongs to never changes, so its activations sit in registers (the flat walk reads them from
 // LDS for every window), the rows a window touches are the same lane ranges every time, and the window is copied through
-// LDS as in the row-copy kernel above (windows are 26.25 lines long: a line at a window's edge is asked for by two waves of
-// the workgroup).  A window's per-row sums (one masked wave reduction per row it touches, three at most) go to slots in LDS,
-// one per window a row lies in; after a barrier the workgroup adds a row's slots in the flat walk's order and stores the
-// rows: the same bits as the flat walk gives with full windows.  Measured against the flat walk (bf16 / f32 activations):
-// 262144 x 2816 113 -> 100 / 118 -> 110 us, 152064 x 5120 112.6 -> 100.6 / 118.8 -> 108.9, 152064 x 3584 82.7 -> 75.3 /
-// 85.7 -> 79.9, 32768 x 14336 71.4 -> 62.6 / 74.1 -> 67.4; with fewer than a dozen windows per wave the fixed shares leave
-// waves idle at the end and the flat walk is as fast or faster.
+// LDS as in the kernels above (Q4_K / Q5_K: 18 / 22 whole lines; Q6_K: 26.25 lines, a line at a window's edge is asked for
+// by two waves of the workgroup).  A window's per-row sums (one masked wave reduction per row it touches, three at most)
+// go to slots in LDS, one per window a row lies in; after a barrier the workgroup adds a row's slots in the flat walk's
+// order and stores the rows: the same bits as the flat walk gives with full windows.  Measured against the flat walk
+// (bf16 / f32 activations): Q6_K 262144 x 2816 113 -> 100 / 118 -> 110 us, 152064 x 5120 112.6 -> 100.6 / 118.8 -> 108.9,
+// 152064 x 3584 82.7 -> 75.3 / 85.7 -> 79.9, 32768 x 14336 71.4 -> 62.6 / 74.1 -> 67.4; Q4_K 262144 x 2816 85.5 -> 77.8 /
+// 92.4 -> 82.2, 152064 x 5120 82.1 -> 74.0 / 89.0 -> 79.1; Q5_K 262144 x 2816 101.1 -> 90.8 / 107.5 -> 95.0, 262144 x 3840
+// 129.2 -> 114.6 / 142.3 -> 121.9; with fewer than a dozen windows per wave the fixed shares leave waves idle at the end
+// and the flat walk is as fast or faster.
 struct PArgs {
     const void* x;
     const uint8_t* w;
@@ -764,10 +766,15 @@ struct PArgs {
     uint32_t periods_per_round;                // slots in LDS: periods_per_round * R * row_slots floats
     uint32_t m4, m2, magic;
 };
-template <bool X_BF16>
-__global__ __launch_bounds__(1024) void gemv_q6k_period_kernel(PArgs a) {
-    constexpr uint32_t CHUNKB = 16u * Q6K_BYTES, PIECES = CHUNKB / 16u;  // 3360 bytes, 210 pieces
-    using X = FlatX<HQ_Q6_K, X_BF16>;
+// Waves per workgroup at most (with f32 activations, 64 registers of them per lane, the kernels take 110 .. 128 registers).
+template <int TYPE, bool X_BF16>
+constexpr uint32_t kPeriodMaxWaves = 16u;
+template <int TYPE, bool X_BF16>
+__global__ __launch_bounds__((64 * kPeriodMaxWaves<TYPE, X_BF16>)) void gemv_period_kernel(PArgs a) {
+    static_assert(TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K, "super-blocks of 256 weights");
+    constexpr uint32_t BB = kBlockBytes<TYPE>, CHUNKB = 16u * BB, PIECES = CHUNKB / 16u;  // 2304 / 2816 / 3360 bytes, 144 / 176 / 210 pieces
+    constexpr int NPV = (int)((PIECES + 63u) / 64u);
+    using X = FlatX<TYPE, X_BF16>;
     extern __shared__ uint4 smem[];
     uint4* lds_x = smem;
     float* lds_s = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(smem) + X::value_bytes(a.k));
@@ -785,11 +792,11 @@ __global__ __launch_bounds__(1024) void gemv_q6k_period_kernel(PArgs a) {
 
     // period i of the workgroup's, window j (non-temporal loads throughout: fetching the pieces on the two lines a window
     // shares with its neighbours with ordinary loads measured the same, ordinary loads for all of it 4 % slower)
-    uint4 pv[4];
+    uint4 pv[NPV];
     auto fetch = [&](uint32_t i) {
         const uint8_t* base = a.w + ((size_t)(blockIdx.x + i * gridDim.x) * P + j) * CHUNKB;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < NPV; ++q) {
             const uint32_t pc = lane + 64u * (uint32_t)q;
             pv[q] = ldnt16(base + 16u * (pc < PIECES - 1u ? pc : PIECES - 1u));
         }
@@ -812,11 +819,12 @@ __global__ __launch_bounds__(1024) void gemv_q6k_period_kernel(PArgs a) {
     const uint32_t my_row = r_lo + (lane < nseg ? lane : 0u), MW = a.row_slots;
     const uint32_t my_slot = MW * my_row + (j - (my_row * a.bu) / 16u);
 
-    const uint32_t blk = (lane >> 2) * Q6K_BYTES, h = (uint32_t)c >> 1, lr = (uint32_t)c & 1u;
-    const uint32_t* wb32 = reinterpret_cast<const uint32_t*>(wbuf);
-    const uint32_t o_qa = blk + 64u * h + 16u * lr, o_qb = o_qa + 32u, o_qh = blk + 128u + 32u * h + 16u * lr, o_sc = blk + 192u + 8u * h,
-                   o_d = blk + 206u;
-    auto field16 = [&](uint32_t o) -> uint4 {
+    // Q6_K: block lane / 4 at byte 210 (lane / 4), fields at even offsets, read as aligned words and shifted into place
+    [[maybe_unused]] const uint32_t blk = (lane >> 2) * BB, h = (uint32_t)c >> 1, lr = (uint32_t)c & 1u;
+    [[maybe_unused]] const uint32_t* wb32 = reinterpret_cast<const uint32_t*>(wbuf);
+    [[maybe_unused]] const uint32_t o_qa = blk + 64u * h + 16u * lr, o_qb = o_qa + 32u, o_qh = blk + 128u + 32u * h + 16u * lr,
+                                    o_sc = blk + 192u + 8u * h, o_d = blk + 206u;
+    [[maybe_unused]] auto field16 = [&](uint32_t o) -> uint4 {
         const uint32_t* p = wb32 + (o >> 2);
         const uint32_t sh = o & 3u, w0 = p[0], w1 = p[1], w2 = p[2], w3 = p[3], w4 = p[4];
         return make_uint4(__builtin_amdgcn_alignbyte(w1, w0, sh), __builtin_amdgcn_alignbyte(w2, w1, sh), __builtin_amdgcn_alignbyte(w3, w2, sh),
@@ -827,14 +835,26 @@ __global__ __launch_bounds__(1024) void gemv_q6k_period_kernel(PArgs a) {
         const uint32_t i1 = i0 + a.periods_per_round < cnt_wg ? i0 + a.periods_per_round : cnt_wg;
         while (i_cur < i1) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) wbuf[lane + 64u * (uint32_t)q] = pv[q];
+            for (int q = 0; q < NPV; ++q) wbuf[lane + 64u * (uint32_t)q] = pv[q];
             asm volatile("" ::: "memory");
             if (i_cur + a.seqs < cnt_wg) fetch(i_cur + a.seqs);
-            Piece<HQ_Q6_K> pc;
-            pc.qa = field16(o_qa);
-            pc.qb = field16(o_qb);
-            pc.qh = field16(o_qh);
-            {
+            Piece<TYPE> pc;
+            if constexpr (TYPE != HQ_Q6_K) {  // blocks of whole 16-byte pieces
+                const uint4* b16 = wbuf + (lane >> 2) * (BB / 16u);
+                pc.hdr = b16[0];
+                if constexpr (TYPE == HQ_Q5_K) {
+                    pc.h0 = b16[1];
+                    pc.h1 = b16[2];
+                    pc.q0 = b16[3 + 2 * c];
+                    pc.q1 = b16[4 + 2 * c];
+                } else {
+                    pc.q0 = b16[1 + 2 * c];
+                    pc.q1 = b16[2 + 2 * c];
+                }
+            } else {
+                pc.qa = field16(o_qa);
+                pc.qb = field16(o_qb);
+                pc.qh = field16(o_qh);
                 const uint32_t* p = wb32 + (o_sc >> 2);
                 const uint32_t sh = o_sc & 3u, w0 = p[0], w1 = p[1], w2 = p[2];
                 pc.sc = make_uint2(__builtin_amdgcn_alignbyte(w1, w0, sh), __builtin_amdgcn_alignbyte(w2, w1, sh));
@@ -868,35 +888,38 @@ __global__ __launch_bounds__(1024) void gemv_q6k_period_kernel(PArgs a) {
         if (i1 < cnt_wg) __syncthreads();
     }
 }
-inline size_t q6k_period_lds(uint32_t k, bool x_bf16, uint32_t waves, uint32_t slots) {
-    return (x_bf16 ? FlatX<HQ_Q6_K, true>::lds_bytes(k) : FlatX<HQ_Q6_K, false>::lds_bytes(k)) + (size_t)waves * 4096u + (size_t)slots * 4u;
+template <int TYPE, bool X_BF16>
+inline size_t period_lds(uint32_t k, uint32_t waves, uint32_t slots) {
+    return FlatX<TYPE, X_BF16>::lds_bytes(k) + (size_t)waves * 4096u + (size_t)slots * 4u;
 }
-// One 16-byte aligned Q6_K matrix, rows of nine super-blocks or more and not whole windows, a period of sixteen windows at
-// most, whole periods of rows, 176 windows per workgroup or more, ten waves or more with f32 activations (nine: 65536 x 4608
-// 48.3 -> 49.3 us), and a shape for which the flat walk would use full windows over whole periods (so that both give the
+// One 16-byte aligned K-quant matrix, rows of nine super-blocks or more and not whole windows, a period of sixteen windows at
+// most, whole periods of rows, 176 windows per workgroup or more, ten waves or more with f32 activations (nine: Q6_K 65536 x
+// 4608 48.3 -> 49.3 us), and a shape for which the flat walk would use full windows over whole periods (so that both give the
 // same bits).
-inline bool q6k_period_takes(const void* w, uint32_t n, uint32_t k, uint32_t cus, bool x_bf16) {
+template <int TYPE, bool X_BF16>
+inline bool period_takes(const void* w, uint32_t n, uint32_t k, uint32_t cus) {
+    constexpr uint32_t MAXW = kPeriodMaxWaves<TYPE, X_BF16>;
     if (k % 256u) return false;
     const uint32_t bu = k / 256u;
     if (bu <= 8u || bu % 16u == 0u || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
     const uint32_t g = bu % 2u ? 1u : bu % 4u ? 2u : bu % 8u ? 4u : 8u, P = bu / g, R = 16u / g;
-    if (P > 16u || n % R || (uint64_t)(n / R) * P < (uint64_t)176u * cus || (uint64_t)n * bu >= 0x7fff0000ull) return false;
-    if ((!x_bf16 && 16u / P * P < 10u) || q6k_period_lds(k, x_bf16, 16u / P * P, 4096u) > 160u * 1024u - 512u) return false;
-    const FlatGeom fg = flat_geom(k, 256u, 16u, n, 1u, cus * 12u);
+    if (P > MAXW || n % R || (uint64_t)(n / R) * P < (uint64_t)176u * cus || (uint64_t)n * bu >= 0x7fff0000ull) return false;
+    if ((!X_BF16 && MAXW / P * P < 10u) || period_lds<TYPE, X_BF16>(k, MAXW / P * P, 4096u) > 160u * 1024u - 512u) return false;
+    const FlatGeom fg = flat_geom(k, 256u, 16u, n, 1u, cus * (TYPE == HQ_Q6_K ? 12u : 16u));  // (as launch_flat asks)
     return fg.uwe == 16u && (1u << fg.log_r) == R;
 }
-template <bool X_BF16>
-int launch_q6k_period(hipStream_t s, const void* x, const uint8_t* w, float* y, uint32_t n, uint32_t k, uint32_t cus) {
+template <int TYPE, bool X_BF16>
+int launch_period(hipStream_t s, const void* x, const uint8_t* w, float* y, uint32_t n, uint32_t k, uint32_t cus) {
     const uint32_t bu = k / 256u, g = bu % 2u ? 1u : bu % 4u ? 2u : bu % 8u ? 4u : 8u, P = bu / g, R = 16u / g;
-    const uint32_t seqs = 16u / P, W = seqs * P;
+    const uint32_t seqs = kPeriodMaxWaves<TYPE, X_BF16> / P, W = seqs * P;
     uint32_t log_r = 0;
     while ((1u << log_r) < R) ++log_r;
     const uint32_t periods = n / R, per_wg = (periods + cus - 1u) / cus;
     const uint32_t mw = (bu + 14u) / 16u + 1u, cap = 4096u / (R * mw);  // 16 KB of slots
     const uint32_t ppr = per_wg < cap ? per_wg : cap;
-    const PArgs pa{x, w, y, n, k, bu, P, log_r, seqs, mw, ppr, N4, N2, MAGIC};
-    const size_t lds = q6k_period_lds(k, X_BF16, W, ppr * R * mw);
-    auto kern = gemv_q6k_period_kernel<X_BF16>;
+    const PArgs pa{x, w, y, n, k, bu, P, log_r, seqs, mw, ppr, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
+    const size_t lds = period_lds<TYPE, X_BF16>(k, W, ppr * R * mw);
+    auto kern = gemv_period_kernel<TYPE, X_BF16>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv period LDS)")) return rc;
     hipLaunchKernelGGL(kern, dim3(cus), dim3(64 * W), lds, s, pa);
     return check_launch("gemv period kernel launch");
@@ -904,7 +927,7 @@ int launch_q6k_period(hipStream_t s, const void* x, const uint8_t* w, float* y, 
 
 // Whether the streaming form takes (type, k, rows): K-quants, whole 4096-element steps, enough rows to occupy the waves.
 template <int TYPE>
-constexpr bool kStreamType =TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K;
+constexpr bool kStreamType = TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K;
 constexpr uint32_t STREAM_MIN_ROWS_PER_WAVE = 2;
 
 template <int TYPE, int ROWS = 1>
@@ -1209,12 +1232,12 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
             return HQ_OK;
         }
     }
-    // Q6_K rows that are not whole windows (lm_heads of hidden size 2560 .. 3840, 5120, 7168; k = 14336): a fixed window of the
-    // row period per wave, a pass per row.
-    if constexpr (TYPE == HQ_Q6_K) {
-        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && q6k_period_takes(a.w, a.n, a.k, cus, X_BF16)) {
+    // K-quant rows that are not whole windows (lm_heads of hidden size 2560 .. 3840, 5120, 7168; k = 14336): a fixed window of
+    // the row period per wave, a pass per row.
+    if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K) {
+        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && period_takes<TYPE, X_BF16>(a.w, a.n, a.k, cus)) {
             for (uint32_t r = 0; r < a.pairs; ++r)
-                if (int rc = launch_q6k_period<X_BF16>(s, static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * (X_BF16 ? 2 : 4), a.w,
+                if (int rc = launch_period<TYPE, X_BF16>(s, static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * (X_BF16 ? 2 : 4), a.w,
                                                        a.y + (size_t)r * a.n, a.n, a.k, cus))
                     return rc;
             return HQ_OK;

@@ -147,16 +147,18 @@ def test_copy_forms_and_their_fallbacks_give_the_same_bits(dev, xdt, t, n, k):
 
 
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
-@pytest.mark.parametrize("n,k", [(262144, 2816), (151936, 2560), (151936, 3072), (152064, 3584), (131072, 3840), (152064, 5120),
-                                 (65536, 7168), (32768, 14336)])
-def test_q6k_rows_that_are_not_whole_windows(oracle, dev, xdt, n, k):
-    """Q6_K matrices whose rows are not whole windows of sixteen super-blocks (hidden sizes 2560 .. 3840, 5120, 7168; k =
+@pytest.mark.parametrize("t,n,k", [(HQ_Q6_K, 262144, 2816), (HQ_Q6_K, 151936, 2560), (HQ_Q6_K, 151936, 3072), (HQ_Q6_K, 152064, 3584),
+                                   (HQ_Q6_K, 131072, 3840), (HQ_Q6_K, 152064, 5120), (HQ_Q6_K, 65536, 7168), (HQ_Q6_K, 32768, 14336),
+                                   (HQ_Q4_K, 262144, 2816), (HQ_Q4_K, 152064, 5120), (HQ_Q4_K, 151936, 3072), (HQ_Q5_K, 262144, 2816),
+                                   (HQ_Q5_K, 152064, 3584), (HQ_Q5_K, 65536, 7168)])
+def test_k_quant_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
+    """K-quant matrices whose rows are not whole windows of sixteen super-blocks (hidden sizes 2560 .. 3840, 5120, 7168; k =
     14336): every wave takes one fixed window of the period after which the row boundaries repeat (11 windows = 16 rows
     for k = 2816, 5 = 8 for 2560, 3 = 4 for 3072, 7 = 8 for 3584, 15 = 16 for 3840, 5 = 4 for 5120, 7 = 4 for 7168, 7 = 2 for
     14336), the rows' parts meet in LDS.  151936 x 3072 leaves a workgroup more periods than its slots hold (two rounds)
-    and a ragged share.  Sampled rows against the f64 oracle; the same bits as
-    the flat walk, which a matrix off the 16-byte grid takes; two activation rows = two passes; the same on a second call."""
-    t = HQ_Q6_K
+    and a ragged share.  Sampled rows against the f64 oracle; Q6_K: the same bits as the flat walk, which a matrix off the
+    16-byte grid takes; slices of 2048 rows against the kernels whose lanes fetch their own pieces; two activation rows =
+    two passes; the same on a second call."""
     w = _quantized(dev, n, k, t, 31 + n + k)
     rng = np.random.default_rng(n + k)
     x = (rng.integers(-12, 13, (2, k)) / 8.0).astype(np.float32)
@@ -170,18 +172,26 @@ def test_q6k_rows_that_are_not_whole_windows(oracle, dev, xdt, n, k):
     xv = oracle.f32_to_bf16_bits(x) if xdt == "bf16" else x
     ref = oracle.qmatmul_f64(xv, _rows_of(w, rows, k, t, oracle), 2, rows.size, k, t)
     sel = torch.as_tensor(rows, device=dev)
-    assert_matmul_close(y[:, sel].cpu().numpy(), ref[0:1], f"q6_k {xdt} {n}x{k}, sampled rows")
-    holder = torch.zeros(w.numel() + 32, dtype=torch.uint8, device=dev)
-    shifted = holder[2:2 + w.numel()]
-    shifted.copy_(w)
-    ys = torch.full((1, n), float("nan"), device=dev)
-    ops.quantized_matmul_ggml(xd[0:1], shifted, ys, p)
-    assert torch.equal(y, ys), (n, k, xdt)
-    del holder, shifted, ys
+    assert_matmul_close(y[:, sel].cpu().numpy(), ref[0:1], f"type {t} {xdt} {n}x{k}, sampled rows")
+    if t == HQ_Q6_K:  # (Q4_K / Q5_K matrices must lie on the 16-byte grid)
+        holder = torch.zeros(w.numel() + 32, dtype=torch.uint8, device=dev)
+        shifted = holder[2:2 + w.numel()]
+        shifted.copy_(w)
+        ys = torch.full((1, n), float("nan"), device=dev)
+        ops.quantized_matmul_ggml(xd[0:1], shifted, ys, p)
+        assert torch.equal(y, ys), (t, n, k, xdt)
+        del holder, shifted, ys
+    # every row against the product over slices of the matrix small enough for the kernels whose lanes fetch their own pieces
+    row_bytes = k // oracle.BLOCK_ELEMS[t] * oracle.BLOCK_BYTES[t]
+    part = 2048
+    for r0 in (0, (n - part) // 2 + 3, n - part):
+        ysl = torch.full((1, part), float("nan"), device=dev)
+        ops.quantized_matmul_ggml(xd[0:1], w[r0 * row_bytes:(r0 + part) * row_bytes].clone(), ysl, GgmlQuantizedMatmulParams(1, part, k, t))
+        assert (ysl - y[:, r0:r0 + part]).abs().max().item() <= 2e-6 * np.abs(ref).max(), (t, xdt, n, k, r0)
     y2 = torch.full((2, n), float("nan"), device=dev)
     ops.quantized_matmul_ggml(xd, w, y2, GgmlQuantizedMatmulParams(2, n, k, t))
     assert torch.equal(y2[0:1], y)
-    assert_matmul_close(y2[:, sel].cpu().numpy(), ref, f"q6_k {xdt} {n}x{k}, two rows")
+    assert_matmul_close(y2[:, sel].cpu().numpy(), ref, f"type {t} {xdt} {n}x{k}, two rows")
     y3 = torch.full((1, n), float("nan"), device=dev)
     ops.quantized_matmul_ggml(xd[0:1], w, y3, p)
     assert torch.equal(y, y3)
