@@ -240,7 +240,8 @@ int qmatmul_routes(hipStream_t stream, const void* x, hq_act_dtype xdt, const vo
     const size_t xrow_bytes = (size_t)k * (xdt == HQ_BF16 ? 2 : 4);
     for (uint32_t r0 = 0; r0 < m; r0 += kGemvMaxRows) {
         const uint32_t rows = m - r0 < kGemvMaxRows ? m - r0 : kGemvMaxRows;
-        if ((gemv_rows_supported(t, rows, k) || gemv_rows_stream_fast(t, xdt, rows, n, k)) && !gemv_stream_passes_preferred(t, xdt, rows, n, k)) {
+        if ((gemv_rows_supported(t, rows, k) || gemv_rows_stream_fast(t, xdt, rows, n, k) || gemv_rows_stream_takes(t, xdt, rows, n, k)) &&
+            !gemv_stream_passes_preferred(t, xdt, rows, n, k)) {
             if (int rc = launch_gemv_rows(stream, static_cast<const uint8_t*>(x) + (size_t)r0 * xrow_bytes, xdt, w_blocks,
                                           y + (size_t)r0 * n, rows, n, k, t))
                 return rc;

@@ -1,6 +1,7 @@
 // Dequant-fused product for 3..8 activation rows (small-batch decode) on the matrix cores:
 // y[m, n] = sum_k x[m, k] * W[n, k] with every weight fetched once for all rows, where the GEMV
-// kernel would fetch it once per row.  Q4_K, Q5_K and Q6_K weights, k a multiple of 1024.
+// kernel would fetch it once per row.  Q4_K, Q5_K and Q6_K weights, k a multiple of 1024 (the stage-once form at
+// the end of the file: any k of whole super-blocks).
 //
 // Bandwidth-bound like the GEMV (0.5625 bytes per weight); the arithmetic that depends on the row
 // count moves to v_mfma_f32_16x16x32_bf16, what is left on the VALU (nibbles -> bf16, scales) does
@@ -78,8 +79,9 @@ struct Staged {
         const uint32_t row = tid >> 5, sb = tid & 31u;
         constexpr int N = X_BF16 ? 4 : 8;
         const uint32_t src_row = row < a.m ? row : a.m - 1u;
-        const uint4* src = reinterpret_cast<const uint4*>(static_cast<const uint8_t*>(a.x) +
-                                                          ((size_t)src_row * a.k + (size_t)chunk * KC + 32u * sb) * (X_BF16 ? 2 : 4));
+        // (a last chunk of fewer than 1024 elements: the sub-blocks past the row's end read its last one; nothing uses them)
+        const uint32_t col = chunk * KC + 32u * sb < a.k ? chunk * KC + 32u * sb : a.k - 32u;
+        const uint4* src = reinterpret_cast<const uint4*>(static_cast<const uint8_t*>(a.x) + ((size_t)src_row * a.k + col) * (X_BF16 ? 2 : 4));
 #pragma unroll
         for (int i = 0; i < N; ++i) r[i] = src[i];
     }
@@ -588,7 +590,7 @@ __global__ __launch_bounds__(64 * W) void rows_stream_kernel(RowsArgs a) {
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t j = lane & 15u, g = lane >> 4;
-    const uint32_t nsb = a.k / 256u, nch = a.k / KC;
+    const uint32_t nsb = a.k / 256u, nch = (a.k + KC - 1u) / KC;  // (the last chunk may hold one to three super-blocks)
 
     // all of k, a 1024-element chunk per 256 threads and turn, each chunk a staging buffer of its own
     {
@@ -718,8 +720,8 @@ constexpr size_t kLdsPerCu = 160 * 1024 - 512;
 // Whether the stage-once form takes the product (all of k in LDS, two groups of 16 rows or more per CU), its LDS bytes,
 // and whether the wave-owned piece buffers of the transposed fetch fit beside the activations.
 bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t cus, size_t* lds, bool* xpose) {
-    const size_t lds_all = (size_t)(k / KC) * (bf ? kStage<true> : kStage<false>);
-    if (lds_all > kLdsPerCu || (n + 15u) / 16u < 2u * cus) return false;
+    const size_t lds_all = (size_t)((k + KC - 1u) / KC) * (bf ? kStage<true> : kStage<false>);
+    if (k % 256u || lds_all > kLdsPerCu || (n + 15u) / 16u < 2u * cus) return false;
     const size_t pitch16 = 16u * (t == HQ_Q4_K ? Q4kRows<false>::PITCH : t == HQ_Q5_K ? Q4kRows<true>::PITCH : Q6kRows::PITCH);
     *xpose = lds_all + kStreamWaves * pitch16 <= kLdsPerCu;
     *lds = lds_all + (*xpose ? kStreamWaves * pitch16 : 0);
@@ -730,12 +732,24 @@ bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t 
 // bf16 rows over a matrix the stage-once form takes with its transposed fetch: one pass for any 3 .. 8 rows at about the
 // cost of one and a half one-row products (Q6_K 151936 x 4096: 134 us; Q4_K 65536 x 4096: 41 us).
 bool gemv_rows_stream_fast(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
-    if (xdt != HQ_BF16 || m < 3 || m > 8 || k % KC || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K)) return false;
+    if (xdt != HQ_BF16 || m < 3 || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K)) return false;
     uint32_t cus = 0;
     if (cu_count(&cus)) return false;
     size_t lds = 0;
     bool xpose = false;
     return rows_stream_plan(t, true, n, k, cus, &lds, &xpose) && xpose;
+}
+
+// k that is whole super-blocks but not whole 1024-element chunks (2816, 3584, 5120 ...): only the stage-once form walks it,
+// with either activation type.
+bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
+    const uint32_t from = t == HQ_Q6_K ? 4u : 3u;
+    if (m < from || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K)) return false;
+    uint32_t cus = 0;
+    if (cu_count(&cus)) return false;
+    size_t lds = 0;
+    bool xpose = false;
+    return rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose);
 }
 
 int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
@@ -761,6 +775,7 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
         hipLaunchKernelGGL(sk, dim3(cus), dim3(64 * W), lds_k, s, a);
         return check_launch("rows stream kernel launch");
     }
+    if (k % KC) return fail(HQ_ERR_INVALID_ARGUMENT, "small-batch kernel: k must be a multiple of 1024 for this matrix");
     const int lds = 2 * (bf ? kStage<true> : kStage<false>);
     // more rows per workgroup once that still gives every CU three workgroups of the first round; Q6_K stops at
     // two super-blocks per wave (at four, the fetches in flight leave one wave per SIMD) except with f32

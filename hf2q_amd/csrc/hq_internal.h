@@ -83,6 +83,8 @@ int launch_gemv_swiglu(hipStream_t s, const void* x, hq_act_dtype xdt, const voi
 bool gemv_rows_supported(hq_ggml_type t, uint32_t m, uint32_t k);
 // bf16 rows the small-batch kernel takes in its stage-once form with the transposed weight fetch (gemvm.hip).
 bool gemv_rows_stream_fast(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k);
+// ... and whether the stage-once form takes the product at all (any k of whole super-blocks that fits a CU's LDS).
+bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k);
 int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,
                      uint32_t k, hq_ggml_type t);
 // The same for the 32-weight-block types (Q8_0, Q4_0), 2 <= m <= 8: exact products on the VALU, every weight fetched

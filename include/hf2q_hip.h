@@ -108,7 +108,8 @@ HQ_API int hq_quantize_ggml_imatrix(void* stream, const float* src, uint64_t n_e
  * weight once for all rows), and Q4_K / Q5_K run up to 16 rows as two such passes; larger m takes the MFMA GEMM,
  * whose tiles are 64 (Q4_K / Q5_K), 128 or 256 token rows by m; up to 256 rows k is cut into slices where the
  * weight-row tiles alone would leave CUs idle.
- * Where a K-quant's k has no small-batch kernel (k % 1024 != 0), up to 16 rows run as per-row GEMVs first.
+ * A K-quant's k that is not a multiple of 1024 (2816, 3584, 5120 ...) has the small-batch kernel where all of k fits a
+ * CU's LDS and the matrix has 8192 rows or more; otherwise up to 16 rows run as per-row GEMVs first.
  * MFMA GEMM.  The K-quant (k % 256 == 0) and Q8_0 / Q4_0 (k % 128 == 0) GEMMs multiply f16-rounded
  * weights and activations like the reference's mul_mm, the other kernels keep
  * every product exact.

@@ -199,11 +199,13 @@ def test_k_quant_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
-@pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048)])
+@pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048), (8203, 2816), (9001, 3584), (8192, 5120)])
 def test_small_batch_rows_staged_once(oracle, dev, t, xdt, n, k):
     """3 .. 8 activation rows over matrices of two groups of 16 rows per CU or more, all of k in LDS: the small-batch form
     that stages the activations once per CU (bf16: weights fetched as 16-byte pieces through LDS; f32: fetched by the
-    lanes that use them).  Ragged last group (n % 16 = 8 / 3 / 0).  Sampled rows against the f64 oracle, every row
+    lanes that use them).  Ragged last group (n % 16 = 8 / 3 / 0 / 11 / 9).  k = 2816, 3584 and 5120 are not whole chunks
+    of 1024 activations (the last chunk holds 3, 2 and 1 super-blocks): only this form takes them; 5120 as f32 does not fit
+    the LDS and runs a pass per row.  Sampled rows against the f64 oracle, every row
     against the one-row product of the same activations, and the same result on a second call."""
     w = _quantized(dev, n, k, t, 11 + n + t)
     rng = np.random.default_rng(n + k + t)
