@@ -741,15 +741,18 @@ bool gemv_rows_stream_fast(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_
 }
 
 // k that is whole super-blocks but not whole 1024-element chunks (2816, 3584, 5120 ...): only the stage-once form walks it,
-// with either activation type.
+// with either activation type.  Such k has no multi-row streaming passes either, so the form starts at three rows for
+// every type (Q6_K 262144 x 2816 f32: 228 against 318 us), and at two where the weights go through the transposed fetch
+// (bf16 rows: Q6_K 262144 x 2816 146 against 191 us for two passes, Q4_K 90 against 153, Q5_K 152064 x 3584 86 against 130).
 bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
-    const uint32_t from = t == HQ_Q6_K ? 4u : 3u;
-    if (m < from || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K)) return false;
+    if (m < 2 || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K)) return false;
     uint32_t cus = 0;
     if (cu_count(&cus)) return false;
     size_t lds = 0;
     bool xpose = false;
-    return rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose);
+    if (!rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose)) return false;
+    const uint32_t from = k % KC == 0 ? (t == HQ_Q6_K ? 4u : 3u) : xdt == HQ_BF16 && xpose ? 2u : 3u;
+    return m >= from;
 }
 
 int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void* w, float* y, uint32_t m, uint32_t n,

@@ -157,8 +157,8 @@ def test_k_quant_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
     for k = 2816, 5 = 8 for 2560, 3 = 4 for 3072, 7 = 8 for 3584, 15 = 16 for 3840, 5 = 4 for 5120, 7 = 4 for 7168, 7 = 2 for
     14336), the rows' parts meet in LDS.  151936 x 3072 leaves a workgroup more periods than its slots hold (two rounds)
     and a ragged share.  Sampled rows against the f64 oracle; Q6_K: the same bits as the flat walk, which a matrix off the
-    16-byte grid takes; slices of 2048 rows against the kernels whose lanes fetch their own pieces; two activation rows =
-    two passes; the same on a second call."""
+    16-byte grid takes; slices of 2048 rows against the kernels whose lanes fetch their own pieces; two activation rows; the
+    same on a second call."""
     w = _quantized(dev, n, k, t, 31 + n + k)
     rng = np.random.default_rng(n + k)
     x = (rng.integers(-12, 13, (2, k)) / 8.0).astype(np.float32)
@@ -190,7 +190,8 @@ def test_k_quant_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
         assert (ysl - y[:, r0:r0 + part]).abs().max().item() <= 2e-6 * np.abs(ref).max(), (t, xdt, n, k, r0)
     y2 = torch.full((2, n), float("nan"), device=dev)
     ops.quantized_matmul_ggml(xd, w, y2, GgmlQuantizedMatmulParams(2, n, k, t))
-    assert torch.equal(y2[0:1], y)
+    # (two f32 rows: two passes of this kernel; two bf16 rows: the small-batch kernel where the matrix fits its stage-once form)
+    assert (y2[0:1] - y).abs().max().item() <= 1e-4 * np.abs(ref).max()
     assert_matmul_close(y2[:, sel].cpu().numpy(), ref, f"type {t} {xdt} {n}x{k}, two rows")
     y3 = torch.full((1, n), float("nan"), device=dev)
     ops.quantized_matmul_ggml(xd[0:1], w, y3, p)
@@ -211,7 +212,7 @@ def test_small_batch_rows_staged_once(oracle, dev, t, xdt, n, k):
     rng = np.random.default_rng(n + k + t)
     rows = np.unique(np.concatenate([[0, 1, 15, 16, n - 17, n - 16, n - 2, n - 1], rng.integers(0, n, 50)]))
     wr = _rows_of(w, rows, k, t, oracle)
-    for m in (3, 5, 8):
+    for m in ((3, 5, 8) if k % 1024 == 0 else (2, 3, 5, 8)):  # (two bf16 rows of the other k take this form too)
         x = acts(m + n, m, k)
         xd = torch.from_numpy(x).to(dev)
         xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
