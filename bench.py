@@ -954,6 +954,14 @@ def bench_decode_gemv(a):
             us = _launch_us([(lambda w=w: ops.quantized_matmul_ggml(xr, w, yr, pr)) for w in wsr] * (4 if copies == 2 else 4))
             entry[dn] = {"us": round(us, 3), "GBps": round(wsr[0].numel() / us / 1e3, 1),
                          "frac_hbm_peak": round(wsr[0].numel() / us / 1e3 / HBM_PEAK_GBS, 4)}
+        if n > 100000:  # the lm_heads at a few bf16 rows (batched decode): one pass over the weights for all of them
+            for m_ in (2, 8):
+                xm = torch.randn(m_, k, generator=gx, device=dev, dtype=torch.float32).to(torch.bfloat16)
+                ym = torch.empty(m_, n, device=dev)
+                pm = GgmlQuantizedMatmulParams(m_, n, k, t)
+                us = _launch_us([(lambda w=w: ops.quantized_matmul_ggml(xm, w, ym, pm)) for w in wsr] * 4)
+                entry[f"bf16_rows_{m_}"] = {"us": round(us, 2), "GBps": round(wsr[0].numel() / us / 1e3, 1),
+                                            "frac_hbm_peak": round(wsr[0].numel() / us / 1e3 / HBM_PEAK_GBS, 4)}
         ref_shapes[nm] = entry
         del wsr
 

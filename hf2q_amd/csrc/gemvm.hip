@@ -1,7 +1,7 @@
 // Dequant-fused product for 3..8 activation rows (small-batch decode) on the matrix cores:
 // y[m, n] = sum_k x[m, k] * W[n, k] with every weight fetched once for all rows, where the GEMV
 // kernel would fetch it once per row.  Q4_K, Q5_K and Q6_K weights, k a multiple of 1024 (the stage-once form at
-// the end of the file: any k of whole super-blocks).
+// the end of the file: any k of whole super-blocks, and Q8_0 under bf16 rows).
 //
 // Bandwidth-bound like the GEMV (0.5625 bytes per weight); the arithmetic that depends on the row
 // count moves to v_mfma_f32_16x16x32_bf16, what is left on the VALU (nibbles -> bf16, scales) does
@@ -576,6 +576,66 @@ struct Q6kRows {
     }
 };
 
+// Q8_0 through the same walk: eight 34-byte blocks = 272 bytes = seventeen pieces stand for a super-block.  An int8 weight is
+// exact in bf16, so a block is one MFMA over the converted bytes and one scaling of its four results by d; no offsets, no
+// activation sums.  A block starts at an even address: in LDS (super-blocks at multiples of 16) the eight weights of lane
+// group g lie at byte 34 c + 2 + 8 g, a multiple of four for odd c and two past one for even c, where three aligned words
+// are shifted into place.
+struct Q80Rows {
+    static constexpr uint32_t BYTES = 8u * Q8_0_BYTES;
+    static constexpr bool SUM16 = false;
+    struct WBlock {
+        uint2 q[8];
+        uint32_t d[8];
+    };
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ void load(WBlock& b, const uint8_t* p, uint32_t g) const {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            b.q[c] = ld8_unaligned(p + 34 * c + 2 + 8u * g);
+            b.d[c] = ld2(p + 34 * c);
+        }
+    }
+    // (x0, x2), (x1, x3), (x4, x6), (x5, x7): the order of the staged activations
+    static __device__ __forceinline__ uint32_t pair(uint32_t w, int lo, int hi) {
+        const float a = (float)(int)(int8_t)(w >> (8 * lo)), b = (float)(int)(int8_t)(w >> (8 * hi));
+        return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);  // the upper halves: small integers are exact
+    }
+    __device__ __forceinline__ void super_block(const WBlock& wb, const uint8_t* xb, const float*, uint32_t, f32x4_t& acc) const {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float d = f16_bits_to_f32(wb.d[c] & 0xffffu);
+            const uint32_t w0 = wb.q[c].x, w1 = wb.q[c].y;
+            const uint4 b = make_uint4(pair(w0, 0, 2), pair(w0, 1, 3), pair(w1, 0, 2), pair(w1, 1, 3));
+            const uint4 av = *reinterpret_cast<const uint4*>(xb + 64 * c);
+            const f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+            const f32x4_t r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, b), z, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[v] = fmaf(d, r[v], acc[v]);
+        }
+    }
+    static constexpr uint32_t kXLane = 16u;  // eight activations per lane group
+    static constexpr uint32_t kSumsPerSb = 128u;
+    // rows 272 bytes = 68 words apart in LDS: the sixteen rows' words fall into sixteen different groups of four banks
+    static constexpr uint32_t PB = 17u, PITCH = 272u;
+    static constexpr bool kTailD = false;
+    __device__ __forceinline__ void read_lds(WBlock& b, const uint8_t* p, uint32_t g) const {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            if (c & 1) {
+                const uint32_t* q = reinterpret_cast<const uint32_t*>(p + 34 * c + 2 + 8u * g);
+                b.q[c] = make_uint2(q[0], q[1]);
+                b.d[c] = *reinterpret_cast<const uint32_t*>(p + 34 * c - 2) >> 16;
+            } else {
+                const uint32_t* q = reinterpret_cast<const uint32_t*>(p + 34 * c + 8u * g);
+                const uint32_t a0 = q[0], a1 = q[1], a2 = q[2];
+                b.q[c] = make_uint2(__builtin_amdgcn_alignbyte(a1, a0, 2), __builtin_amdgcn_alignbyte(a2, a1, 2));
+                b.d[c] = *reinterpret_cast<const uint32_t*>(p + 34 * c);
+            }
+        }
+    }
+};
+
 // XPOSE: the weights of a task (one super-block of each of the group's 16 rows) are fetched as 16-byte pieces, consecutive
 // lanes consecutive pieces of a row's block (three to five load instructions per lane where every lane fetching its own
 // operands takes five for Q4_K and fourteen for Q6_K, most of them four bytes wide), written to a region of LDS the wave
@@ -722,7 +782,7 @@ constexpr size_t kLdsPerCu = 160 * 1024 - 512;
 bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t cus, size_t* lds, bool* xpose) {
     const size_t lds_all = (size_t)((k + KC - 1u) / KC) * (bf ? kStage<true> : kStage<false>);
     if (k % 256u || lds_all > kLdsPerCu || (n + 15u) / 16u < 2u * cus) return false;
-    const size_t pitch16 = 16u * (t == HQ_Q4_K ? Q4kRows<false>::PITCH : t == HQ_Q5_K ? Q4kRows<true>::PITCH : Q6kRows::PITCH);
+    const size_t pitch16 = 16u * (t == HQ_Q4_K ? Q4kRows<false>::PITCH : t == HQ_Q5_K ? Q4kRows<true>::PITCH : t == HQ_Q6_K ? Q6kRows::PITCH : Q80Rows::PITCH);
     *xpose = lds_all + kStreamWaves * pitch16 <= kLdsPerCu;
     *lds = lds_all + (*xpose ? kStreamWaves * pitch16 : 0);
     return true;
@@ -745,12 +805,16 @@ bool gemv_rows_stream_fast(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_
 // every type (Q6_K 262144 x 2816 f32: 228 against 318 us), and at two where the weights go through the transposed fetch
 // (bf16 rows: Q6_K 262144 x 2816 146 against 191 us for two passes, Q4_K 90 against 153, Q5_K 152064 x 3584 86 against 130).
 bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
-    if (m < 2 || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K)) return false;
+    if (m < 2 || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K && t != HQ_Q8_0)) return false;
     uint32_t cus = 0;
     if (cu_count(&cus)) return false;
     size_t lds = 0;
     bool xpose = false;
     if (!rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose)) return false;
+    // Q8_0: bf16 rows where the transposed fetch fits, from two rows on (262144 x 2816: 140 .. 150 us for 2 .. 8 rows where the
+    // kernel of exact f32 products takes 237 .. 426 and one row 126; 12288 x 4096: 15.4 against 17.5 .. 30.0); without the
+    // transposed fetch, and with f32 rows (hi + lo parts: twice the LDS), that kernel stays ahead
+    if (t == HQ_Q8_0) return xdt == HQ_BF16 && xpose;
     const uint32_t from = k % KC == 0 ? (t == HQ_Q6_K ? 4u : 3u) : xdt == HQ_BF16 && xpose ? 2u : 3u;
     return m >= from;
 }
@@ -769,16 +833,18 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
         if (xpose)
             sk = t == HQ_Q4_K   ? (bf ? rows_stream_kernel<Q4kRows<false>, true, W, true> : rows_stream_kernel<Q4kRows<false>, false, W, true>)
                  : t == HQ_Q5_K ? (bf ? rows_stream_kernel<Q4kRows<true>, true, W, true> : rows_stream_kernel<Q4kRows<true>, false, W, true>)
-                                : (bf ? rows_stream_kernel<Q6kRows, true, W, true> : rows_stream_kernel<Q6kRows, false, W, true>);
+                 : t == HQ_Q6_K ? (bf ? rows_stream_kernel<Q6kRows, true, W, true> : rows_stream_kernel<Q6kRows, false, W, true>)
+                                : (bf ? rows_stream_kernel<Q80Rows, true, W, true> : rows_stream_kernel<Q80Rows, false, W, true>);
         else
             sk = t == HQ_Q4_K   ? (bf ? rows_stream_kernel<Q4kRows<false>, true, W, false> : rows_stream_kernel<Q4kRows<false>, false, W, false>)
                  : t == HQ_Q5_K ? (bf ? rows_stream_kernel<Q4kRows<true>, true, W, false> : rows_stream_kernel<Q4kRows<true>, false, W, false>)
-                                : (bf ? rows_stream_kernel<Q6kRows, true, W, false> : rows_stream_kernel<Q6kRows, false, W, false>);
+                 : t == HQ_Q6_K ? (bf ? rows_stream_kernel<Q6kRows, true, W, false> : rows_stream_kernel<Q6kRows, false, W, false>)
+                                : (bf ? rows_stream_kernel<Q80Rows, true, W, false> : rows_stream_kernel<Q80Rows, false, W, false>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(sk), lds_k, "hipFuncSetAttribute(rows stream kernel LDS)")) return rc;
         hipLaunchKernelGGL(sk, dim3(cus), dim3(64 * W), lds_k, s, a);
         return check_launch("rows stream kernel launch");
     }
-    if (k % KC) return fail(HQ_ERR_INVALID_ARGUMENT, "small-batch kernel: k must be a multiple of 1024 for this matrix");
+    if (k % KC || t == HQ_Q8_0) return fail(HQ_ERR_INVALID_ARGUMENT, "small-batch kernel: k must be a multiple of 1024 for this matrix");
     const int lds = 2 * (bf ? kStage<true> : kStage<false>);
     // more rows per workgroup once that still gives every CU three workgroups of the first round; Q6_K stops at
     // two super-blocks per wave (at four, the fetches in flight leave one wave per SIMD) except with f32
