@@ -1,7 +1,7 @@
 // Dequant-fused product for 3..8 activation rows (small-batch decode) on the matrix cores:
 // y[m, n] = sum_k x[m, k] * W[n, k] with every weight fetched once for all rows, where the GEMV
 // kernel would fetch it once per row.  Q4_K, Q5_K and Q6_K weights, k a multiple of 1024 (the stage-once form at
-// the end of the file: any k of whole super-blocks, and Q8_0 under bf16 rows).
+// the end of the file: any k of whole super-blocks, and Q8_0 / Q4_0 under bf16 rows).
 //
 // Bandwidth-bound like the GEMV (0.5625 bytes per weight); the arithmetic that depends on the row
 // count moves to v_mfma_f32_16x16x32_bf16, what is left on the VALU (nibbles -> bf16, scales) does
@@ -636,6 +636,69 @@ struct Q80Rows {
     }
 };
 
+// Q4_0 likewise: eight 18-byte blocks = 144 bytes = nine pieces.  Lane group g takes weights 8 g .. 8 g + 7 of a block: the
+// low (g < 2) or high nibbles of bytes 8 (g & 1) .. + 7, as bf16 128 + q like the Q4_K nibbles; the 128 and the format's
+// own offset of 8 leave through the activation sums, (128 + 8) d per block, in the small f32 MFMA.
+struct Q40Rows {
+    static constexpr uint32_t BYTES = 8u * Q4_0_BYTES;
+    static constexpr bool SUM16 = false;
+    struct WBlock {
+        uint2 q[8];
+        uint32_t d[8];
+    };
+    uint32_t m4, magic;
+    __device__ __forceinline__ void init() {
+        asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "=v"(m4), "=v"(magic) : "s"(M4), "s"(MAGIC));
+    }
+    __device__ __forceinline__ void load(WBlock& b, const uint8_t* p, uint32_t g) const {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            b.q[c] = ld8_unaligned(p + 18 * c + 2 + 8u * (g & 1u));
+            b.d[c] = ld2(p + 18 * c);
+        }
+    }
+    __device__ __forceinline__ void super_block(const WBlock& wb, const uint8_t* xb, const float* sums, uint32_t g, f32x4_t& acc) const {
+        float d[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) d[c] = f16_bits_to_f32(wb.d[c] & 0xffffu);
+        const float mine0 = g == 0u ? d[0] : g == 1u ? d[1] : g == 2u ? d[2] : d[3];
+        const float mine1 = g == 0u ? d[4] : g == 1u ? d[5] : g == 2u ? d[6] : d[7];
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[0], -136.f * mine0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[64], -136.f * mine1, acc, 0, 0, 0);
+        const uint32_t sh = 4u * (g >> 1);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t w0 = wb.q[c].x >> sh, w1 = wb.q[c].y >> sh;
+            const uint4 b = make_uint4(and_or(w0, m4, magic), and_or(w0 >> 8, m4, magic), and_or(w1, m4, magic), and_or(w1 >> 8, m4, magic));
+            const uint4 av = *reinterpret_cast<const uint4*>(xb + 64 * c);
+            const f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+            const f32x4_t r = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, b), z, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[v] = fmaf(d[c], r[v], acc[v]);
+        }
+    }
+    static constexpr uint32_t kXLane = 16u;
+    static constexpr uint32_t kSumsPerSb = 128u;
+    // rows 144 bytes = 36 words apart in LDS: sixteen different groups of four banks
+    static constexpr uint32_t PB = 9u, PITCH = 144u;
+    static constexpr bool kTailD = false;
+    __device__ __forceinline__ void read_lds(WBlock& b, const uint8_t* p, uint32_t g) const {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            if (c & 1) {  // 18 c + 2 is a multiple of four
+                const uint32_t* q = reinterpret_cast<const uint32_t*>(p + 18 * c + 2 + 8u * (g & 1u));
+                b.q[c] = make_uint2(q[0], q[1]);
+                b.d[c] = *reinterpret_cast<const uint32_t*>(p + 18 * c - 2) >> 16;
+            } else {
+                const uint32_t* q = reinterpret_cast<const uint32_t*>(p + 18 * c + 8u * (g & 1u));
+                const uint32_t a0 = q[0], a1 = q[1], a2 = q[2];
+                b.q[c] = make_uint2(__builtin_amdgcn_alignbyte(a1, a0, 2), __builtin_amdgcn_alignbyte(a2, a1, 2));
+                b.d[c] = *reinterpret_cast<const uint32_t*>(p + 18 * c);
+            }
+        }
+    }
+};
+
 // XPOSE: the weights of a task (one super-block of each of the group's 16 rows) are fetched as 16-byte pieces, consecutive
 // lanes consecutive pieces of a row's block (three to five load instructions per lane where every lane fetching its own
 // operands takes five for Q4_K and fourteen for Q6_K, most of them four bytes wide), written to a region of LDS the wave
@@ -782,7 +845,7 @@ constexpr size_t kLdsPerCu = 160 * 1024 - 512;
 bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t cus, size_t* lds, bool* xpose) {
     const size_t lds_all = (size_t)((k + KC - 1u) / KC) * (bf ? kStage<true> : kStage<false>);
     if (k % 256u || lds_all > kLdsPerCu || (n + 15u) / 16u < 2u * cus) return false;
-    const size_t pitch16 = 16u * (t == HQ_Q4_K ? Q4kRows<false>::PITCH : t == HQ_Q5_K ? Q4kRows<true>::PITCH : t == HQ_Q6_K ? Q6kRows::PITCH : Q80Rows::PITCH);
+    const size_t pitch16 = 16u * (t == HQ_Q4_K ? Q4kRows<false>::PITCH : t == HQ_Q5_K ? Q4kRows<true>::PITCH : t == HQ_Q6_K ? Q6kRows::PITCH : t == HQ_Q8_0 ? Q80Rows::PITCH : Q40Rows::PITCH);
     *xpose = lds_all + kStreamWaves * pitch16 <= kLdsPerCu;
     *lds = lds_all + (*xpose ? kStreamWaves * pitch16 : 0);
     return true;
@@ -805,7 +868,7 @@ bool gemv_rows_stream_fast(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_
 // every type (Q6_K 262144 x 2816 f32: 228 against 318 us), and at two where the weights go through the transposed fetch
 // (bf16 rows: Q6_K 262144 x 2816 146 against 191 us for two passes, Q4_K 90 against 153, Q5_K 152064 x 3584 86 against 130).
 bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
-    if (m < 2 || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K && t != HQ_Q8_0)) return false;
+    if (m < 2 || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K && t != HQ_Q8_0 && t != HQ_Q4_0)) return false;
     uint32_t cus = 0;
     if (cu_count(&cus)) return false;
     size_t lds = 0;
@@ -815,6 +878,9 @@ bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32
     // kernel of exact f32 products takes 237 .. 426 and one row 126; 12288 x 4096: 15.4 against 17.5 .. 30.0); without the
     // transposed fetch, and with f32 rows (hi + lo parts: twice the LDS), that kernel stays ahead
     if (t == HQ_Q8_0) return xdt == HQ_BF16 && xpose;
+    // Q4_0 likewise (262144 x 2816: 93 .. 96 us for 2 .. 8 rows, one row 91; 151936 x 4096: 78 .. 81, one row 58; that kernel: 112 ..
+    // 259); two rows of a small matrix stay with it (12288 x 4096: 13.2 against 14.9 us; from three rows 16.6 .. 25.7 against 14.9)
+    if (t == HQ_Q4_0) return xdt == HQ_BF16 && xpose && (m >= 3 || n >= 32768);
     const uint32_t from = k % KC == 0 ? (t == HQ_Q6_K ? 4u : 3u) : xdt == HQ_BF16 && xpose ? 2u : 3u;
     return m >= from;
 }
@@ -834,17 +900,19 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
             sk = t == HQ_Q4_K   ? (bf ? rows_stream_kernel<Q4kRows<false>, true, W, true> : rows_stream_kernel<Q4kRows<false>, false, W, true>)
                  : t == HQ_Q5_K ? (bf ? rows_stream_kernel<Q4kRows<true>, true, W, true> : rows_stream_kernel<Q4kRows<true>, false, W, true>)
                  : t == HQ_Q6_K ? (bf ? rows_stream_kernel<Q6kRows, true, W, true> : rows_stream_kernel<Q6kRows, false, W, true>)
-                                : (bf ? rows_stream_kernel<Q80Rows, true, W, true> : rows_stream_kernel<Q80Rows, false, W, true>);
+                 : t == HQ_Q8_0 ? (bf ? rows_stream_kernel<Q80Rows, true, W, true> : rows_stream_kernel<Q80Rows, false, W, true>)
+                                : (bf ? rows_stream_kernel<Q40Rows, true, W, true> : rows_stream_kernel<Q40Rows, false, W, true>);
         else
             sk = t == HQ_Q4_K   ? (bf ? rows_stream_kernel<Q4kRows<false>, true, W, false> : rows_stream_kernel<Q4kRows<false>, false, W, false>)
                  : t == HQ_Q5_K ? (bf ? rows_stream_kernel<Q4kRows<true>, true, W, false> : rows_stream_kernel<Q4kRows<true>, false, W, false>)
                  : t == HQ_Q6_K ? (bf ? rows_stream_kernel<Q6kRows, true, W, false> : rows_stream_kernel<Q6kRows, false, W, false>)
-                                : (bf ? rows_stream_kernel<Q80Rows, true, W, false> : rows_stream_kernel<Q80Rows, false, W, false>);
+                 : t == HQ_Q8_0 ? (bf ? rows_stream_kernel<Q80Rows, true, W, false> : rows_stream_kernel<Q80Rows, false, W, false>)
+                                : (bf ? rows_stream_kernel<Q40Rows, true, W, false> : rows_stream_kernel<Q40Rows, false, W, false>);
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(sk), lds_k, "hipFuncSetAttribute(rows stream kernel LDS)")) return rc;
         hipLaunchKernelGGL(sk, dim3(cus), dim3(64 * W), lds_k, s, a);
         return check_launch("rows stream kernel launch");
     }
-    if (k % KC || t == HQ_Q8_0) return fail(HQ_ERR_INVALID_ARGUMENT, "small-batch kernel: k must be a multiple of 1024 for this matrix");
+    if (k % KC || t == HQ_Q8_0 || t == HQ_Q4_0) return fail(HQ_ERR_INVALID_ARGUMENT, "small-batch kernel: k must be a multiple of 1024 for this matrix");
     const int lds = 2 * (bf ? kStage<true> : kStage<false>);
     // more rows per workgroup once that still gives every CU three workgroups of the first round; Q6_K stops at
     // two super-blocks per wave (at four, the fetches in flight leave one wave per SIMD) except with f32
