@@ -69,8 +69,12 @@ constexpr uint32_t ONES = 0x3f803f80u;  // (1.0, 1.0) in bf16: a dot2 with it ad
 
 // A thread's share of a chunk: input row tid / 32 (of at most 8), sub-block tid % 32 = 32 activations.
 // SUM16: the sums are kept per 16 activations (Q6_K's scale groups), two per thread, else per 32.
-template <bool X_BF16, bool SUM16>
+// HALF (f32 rows, four at most): the hi parts in rows 0 .. 3 and the lo parts in rows 4 .. 7 of a buffer of eight rows, the
+// size of the bf16 staging, where the full form puts them in rows 0 .. 7 and 8 .. 15 of sixteen.
+template <bool X_BF16, bool SUM16, bool HALF = false>
 struct Staged {
+    static_assert(!HALF || !X_BF16, "f32 rows");
+    static constexpr uint32_t LO = HALF ? 4u : 8u;  // the lo parts' row offset
     uint4 r[X_BF16 ? 4 : 8];
     __device__ __forceinline__ void fetch(const RowsArgs& a, uint32_t chunk, uint32_t tid) {
         // No branch around the loads: with conditional loads in flight the compiler can no longer count how
@@ -92,7 +96,7 @@ struct Staged {
     __device__ __forceinline__ void store(uint8_t* buf, uint32_t tid, uint32_t m) const {
         const uint32_t row = tid >> 5, sb = tid & 31u;
         const uint32_t present = row < m ? 0xffffffffu : 0u;
-        float* sums = reinterpret_cast<float*>(buf + kXBuf<X_BF16>);
+        float* sums = reinterpret_cast<float*>(buf + kXBuf<X_BF16 || HALF>);
         if constexpr (X_BF16) {
             float s[2] = {0.f, 0.f};
             uint4 o[4];
@@ -143,8 +147,9 @@ struct Staged {
                 oh[i] = make_uint4(hw[0], hw[1], hw[2], hw[3]);
                 ol[i] = make_uint4(lw[0], lw[1], lw[2], lw[3]);
             }
+            if (HALF && row >= 4u) return;  // (rows 4 .. 7 of the buffer hold the lo parts of rows 0 .. 3)
             uint4* dh = reinterpret_cast<uint4*>(buf + row * XROW + sb * 64u);
-            uint4* dl = reinterpret_cast<uint4*>(buf + (row + 8u) * XROW + sb * 64u);
+            uint4* dl = reinterpret_cast<uint4*>(buf + (row + LO) * XROW + sb * 64u);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 dh[i] = oh[i];
@@ -152,12 +157,12 @@ struct Staged {
             }
             if constexpr (SUM16) {
                 sums[(2u * sb) * 16u + row] = sh2[0];
-                sums[(2u * sb) * 16u + row + 8u] = sl2[0];
+                sums[(2u * sb) * 16u + row + LO] = sl2[0];
                 sums[(2u * sb + 1u) * 16u + row] = sh2[1];
-                sums[(2u * sb + 1u) * 16u + row + 8u] = sl2[1];
+                sums[(2u * sb + 1u) * 16u + row + LO] = sl2[1];
             } else {
                 sums[sb * 16u + row] = sh2[0];
-                sums[sb * 16u + row + 8u] = sl2[0];
+                sums[sb * 16u + row + LO] = sl2[0];
             }
         }
     }
@@ -704,12 +709,15 @@ struct Q40Rows {
 // operands takes five for Q4_K and fourteen for Q6_K, most of them four bytes wide), written to a region of LDS the wave
 // owns and read back from there as the operands each lane needs.  The pieces of the next task are in flight, in registers,
 // while the current one is worked on.
-template <typename T, bool X_BF16, int W, bool XPOSE>
+// HALF: up to four f32 rows staged in the space of eight bf16 rows (hi parts in rows 0 .. 3, lo parts in rows 4 .. 7), so that
+// the piece buffers of the transposed fetch fit beside them where sixteen rows would not leave the room.
+template <typename T, bool X_BF16, int W, bool XPOSE, bool HALF = false>
 __global__ __launch_bounds__(64 * W) void rows_stream_kernel(RowsArgs a) {
     static_assert(W % 4 == 0, "the staging works in groups of 256 threads");
     extern __shared__ uint4 smem4[];
     uint8_t* smem = reinterpret_cast<uint8_t*>(smem4);
-    constexpr uint32_t XBUF = kXBuf<X_BF16>, STAGE = kStage<X_BF16>;
+    constexpr bool ROWS8 = X_BF16 || HALF;  // eight staged rows
+    constexpr uint32_t XBUF = kXBuf<ROWS8>, STAGE = kStage<ROWS8>;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t j = lane & 15u, g = lane >> 4;
@@ -717,7 +725,7 @@ __global__ __launch_bounds__(64 * W) void rows_stream_kernel(RowsArgs a) {
 
     // all of k, a 1024-element chunk per 256 threads and turn, each chunk a staging buffer of its own
     {
-        Staged<X_BF16, T::SUM16> st;
+        Staged<X_BF16, T::SUM16, HALF> st;
         for (uint32_t ch = tid >> 8; ch < nch; ch += W / 4) {
             st.fetch(a, ch, tid & 255u);
             st.store(smem + (size_t)ch * STAGE, tid & 255u, a.m);
@@ -787,7 +795,7 @@ __global__ __launch_bounds__(64 * W) void rows_stream_kernel(RowsArgs a) {
     }
     __syncthreads();
 
-    const uint32_t arow = (X_BF16 ? (j & 7u) : j) * XROW + T::kXLane * g;
+    const uint32_t arow = (ROWS8 ? (j & 7u) : j) * XROW + T::kXLane * g;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     uint32_t sb = 0, grp = first;
     auto task = [&](typename T::WBlock& cur, typename T::WBlock& nxt) {
@@ -804,14 +812,15 @@ __global__ __launch_bounds__(64 * W) void rows_stream_kernel(RowsArgs a) {
         t.super_block(cur, bufc + arow + (sb & 3u) * 512u, reinterpret_cast<const float*>(bufc + XBUF) + (sb & 3u) * T::kSumsPerSb + 16u * g + j,
                       g, acc);
         if (++sb == nsb) {
-            // lane (j, g): activation rows 4g .. 4g + 3 of weight row 16 grp + j; f32 activations: rows 8 .. 15 are the lo parts
+            // lane (j, g): activation rows 4g .. 4g + 3 of weight row 16 grp + j; f32 activations: rows 8 .. 15 (HALF: 4 .. 7) are
+            // the lo parts
             float o[4] = {acc[0], acc[1], acc[2], acc[3]};
             if constexpr (!X_BF16) {
 #pragma unroll
-                for (int v = 0; v < 4; ++v) o[v] = xor32_add(o[v]);
+                for (int v = 0; v < 4; ++v) o[v] = HALF ? xor16_add(o[v]) : xor32_add(o[v]);
             }
             const uint32_t row = grp * 16u + j;
-            if (g < 2u && row < a.n) {
+            if (g < (HALF ? 1u : 2u) && row < a.n) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
                     if (4u * g + v < a.m) a.y[(size_t)(4u * g + v) * a.n + row] = o[v];
@@ -842,6 +851,7 @@ constexpr int kStreamWaves = 16;
 constexpr size_t kLdsPerCu = 160 * 1024 - 512;
 // Whether the stage-once form takes the product (all of k in LDS, two groups of 16 rows or more per CU), its LDS bytes,
 // and whether the wave-owned piece buffers of the transposed fetch fit beside the activations.
+// (bf: eight staged rows -- bf16 rows, or up to four f32 rows as hi and lo parts)
 bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t cus, size_t* lds, bool* xpose) {
     const size_t lds_all = (size_t)((k + KC - 1u) / KC) * (bf ? kStage<true> : kStage<false>);
     if (k % 256u || lds_all > kLdsPerCu || (n + 15u) / 16u < 2u * cus) return false;
@@ -872,16 +882,23 @@ bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32
     uint32_t cus = 0;
     if (cu_count(&cus)) return false;
     size_t lds = 0;
-    bool xpose = false;
-    if (!rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose)) return false;
-    // Q8_0: bf16 rows where the transposed fetch fits, from two rows on (262144 x 2816: 140 .. 150 us for 2 .. 8 rows where the
+    bool xpose = false, xpose_h = false;
+    // up to four f32 rows as hi and lo parts in the space of eight bf16 rows, with the transposed fetch
+    const bool half = xdt != HQ_BF16 && m <= 4 && rows_stream_plan(t, true, n, k, cus, &lds, &xpose_h) && xpose_h;
+    if (!rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose) && !half) return false;
+    const bool fast = (xdt == HQ_BF16 && xpose) || half;
+    // Q8_0: where the transposed fetch fits, from two rows on (bf16, 262144 x 2816: 140 .. 150 us for 2 .. 8 rows where the
     // kernel of exact f32 products takes 237 .. 426 and one row 126; 12288 x 4096: 15.4 against 17.5 .. 30.0); without the
-    // transposed fetch, and with f32 rows (hi + lo parts: twice the LDS), that kernel stays ahead
-    if (t == HQ_Q8_0) return xdt == HQ_BF16 && xpose;
+    // transposed fetch, and with five f32 rows or more (hi + lo parts: twice the LDS), that kernel stays ahead
+    if (t == HQ_Q8_0) return fast && (xdt == HQ_BF16 || m >= 3 || n >= 32768);  // (two f32 rows, 12288 x 4096: 18.6 against 17.5 us)
     // Q4_0 likewise (262144 x 2816: 93 .. 96 us for 2 .. 8 rows, one row 91; 151936 x 4096: 78 .. 81, one row 58; that kernel: 112 ..
     // 259); two rows of a small matrix stay with it (12288 x 4096: 13.2 against 14.9 us; from three rows 16.6 .. 25.7 against 14.9)
-    if (t == HQ_Q4_0) return xdt == HQ_BF16 && xpose && (m >= 3 || n >= 32768);
-    const uint32_t from = k % KC == 0 ? (t == HQ_Q6_K ? 4u : 3u) : xdt == HQ_BF16 && xpose ? 2u : 3u;
+    if (t == HQ_Q4_0) return fast && (m >= 3 || n >= 32768);
+    // K-quants.  Whole chunks: from three rows (Q6_K with bf16 rows: four; below, one-row or multi-row streaming passes are as
+    // fast), and from two f32 rows on large matrices (head 151936 x 4096: 128 us for 2 .. 4 rows against 158 for two passes, 240
+    // for the sixteen-row staging; Q4_K 65536 x 4096: 35 against 57).  Other k: no streaming passes, from two rows on with the
+    // transposed fetch, else three.
+    const uint32_t from = k % KC == 0 ? (half ? (n >= 32768 ? 2u : 3u) : t == HQ_Q6_K ? 4u : 3u) : fast ? 2u : 3u;
     return m >= from;
 }
 
@@ -893,6 +910,17 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
     if (int rc = cu_count(&cus)) return rc;
     size_t lds_k = 0;
     bool xpose = false;
+    if (!bf && m <= 4 && rows_stream_plan(t, true, n, k, cus, &lds_k, &xpose) && xpose) {
+        constexpr int W = kStreamWaves;
+        void (*sk)(RowsArgs) = t == HQ_Q4_K   ? rows_stream_kernel<Q4kRows<false>, false, W, true, true>
+                               : t == HQ_Q5_K ? rows_stream_kernel<Q4kRows<true>, false, W, true, true>
+                               : t == HQ_Q6_K ? rows_stream_kernel<Q6kRows, false, W, true, true>
+                               : t == HQ_Q8_0 ? rows_stream_kernel<Q80Rows, false, W, true, true>
+                                              : rows_stream_kernel<Q40Rows, false, W, true, true>;
+        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(sk), lds_k, "hipFuncSetAttribute(rows stream kernel LDS)")) return rc;
+        hipLaunchKernelGGL(sk, dim3(cus), dim3(64 * W), lds_k, s, a);
+        return check_launch("rows stream kernel launch");
+    }
     if (rows_stream_plan(t, bf, n, k, cus, &lds_k, &xpose)) {
         constexpr int W = kStreamWaves;
         void (*sk)(RowsArgs);

@@ -200,21 +200,21 @@ def test_k_quant_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
-@pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048), (8203, 2816), (9001, 3584), (8192, 5120)])
+@pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048), (8203, 2816), (9001, 3584), (8192, 5120), (33000, 2816)])
 def test_small_batch_rows_staged_once(oracle, dev, t, xdt, n, k):
     """3 .. 8 activation rows over matrices of two groups of 16 rows per CU or more, all of k in LDS: the small-batch form
     that stages the activations once per CU (bf16: weights fetched as 16-byte pieces through LDS; f32: fetched by the
     lanes that use them).  Ragged last group (n % 16 = 8 / 3 / 0 / 11 / 9).  k = 2816, 3584 and 5120 are not whole chunks
     of 1024 activations (the last chunk holds 3, 2 and 1 super-blocks): only this form takes them; 5120 as f32 does not fit
     the LDS and runs a pass per row.  Q8_0 and Q4_0 (eight blocks = a super-block of seventeen / nine pieces, one MFMA per block
-    over the bytes / nibbles as bf16) take the form with bf16 rows from two rows on; their f32 rows keep the kernel of exact
-    f32 products.  Sampled rows against the f64 oracle, every row
+    over the bytes / nibbles as bf16) take the form with bf16 rows from two rows on; f32 rows up to four likewise, five to eight as two
+    passes on matrices of 32768 rows or more (33000 x 2816), else through the kernel of exact f32 products.  Sampled rows against the f64 oracle, every row
     against the one-row product of the same activations, and the same result on a second call."""
     w = _quantized(dev, n, k, t, 11 + n + t)
     rng = np.random.default_rng(n + k + t)
     rows = np.unique(np.concatenate([[0, 1, 15, 16, n - 17, n - 16, n - 2, n - 1], rng.integers(0, n, 50)]))
     wr = _rows_of(w, rows, k, t, oracle)
-    for m in ((3, 5, 8) if k % 1024 == 0 and t not in (HQ_Q8_0, HQ_Q4_0) else (2, 3, 5, 8)):  # (two bf16 rows of the other k, of Q8_0 and of Q4_0 take this form too)
+    for m in (2, 3, 4, 5, 8):  # (up to four f32 rows are staged as hi and lo parts in the space of eight bf16 rows)
         x = acts(m + n, m, k)
         xd = torch.from_numpy(x).to(dev)
         xd = xd.to(torch.bfloat16) if xdt == "bf16" else xd
