@@ -979,6 +979,13 @@ def bench_decode_gemv(a):
             us = _launch_us([(lambda w=w: ops.quantized_matmul_ggml(xm, w, ym, pm)) for w in mats] * max(1, 12 // len(mats)))
             entry[f"rows_{m_}"] = {"us": round(us, 2), "GBps": round(mats[0].numel() / us / 1e3, 1),
                                    "frac_hbm_peak": round(mats[0].numel() / us / 1e3 / HBM_PEAK_GBS, 4)}
+        # four f32 rows (the dtype of the reference's call sites): hi and lo parts staged in the space of eight bf16 rows
+        xm = torch.randn(4, k_, generator=gx, device=dev, dtype=torch.float32)
+        ym = torch.empty(4, n_, device=dev)
+        pm = GgmlQuantizedMatmulParams(4, n_, k_, t_)
+        us = _launch_us([(lambda w=w: ops.quantized_matmul_ggml(xm, w, ym, pm)) for w in mats] * max(1, 12 // len(mats)))
+        entry["rows_4_f32"] = {"us": round(us, 2), "GBps": round(mats[0].numel() / us / 1e3, 1),
+                               "frac_hbm_peak": round(mats[0].numel() / us / 1e3 / HBM_PEAK_GBS, 4)}
         small_batch[nm] = entry
     del big
 
