@@ -741,7 +741,7 @@ inline bool q6k_rowcopy_takes(const void* w, uint32_t n, uint32_t k, uint32_t cu
 }
 
 // K-quant rows of nine super-blocks or more that are not whole windows of sixteen (k = 2560, 2816, 3072, 3584, 3840, 5120,
-// 7168, 14336 ...).  The matrix is cut into the flat walk's windows of sixteen blocks; the pattern of row boundaries inside
+// 7168, 14336 ...), and rows of Q8_0 / Q4_0 block pairs (a lane each, 64 to a window) likewise.  The matrix is cut into the flat walk's windows of sixteen blocks; the pattern of row boundaries inside
 // a window repeats every P = bu / gcd(bu, 16) windows = R = 16 / gcd(bu, 16) rows (k = 2816: 11 windows, 16 rows; k = 5120: 5
 // windows, 4 rows).  Wave j of a sequence of P waves takes window j of every period the sequence owns: which super-block
 // of a row a lane's quarter belongs to never changes, so its activations sit in registers (the flat walk reads them from
@@ -753,7 +753,8 @@ inline bool q6k_rowcopy_takes(const void* w, uint32_t n, uint32_t k, uint32_t cu
 // (bf16 / f32 activations): Q6_K 262144 x 2816 113 -> 100 / 118 -> 110 us, 152064 x 5120 112.6 -> 100.6 / 118.8 -> 108.9,
 // 152064 x 3584 82.7 -> 75.3 / 85.7 -> 79.9, 32768 x 14336 71.4 -> 62.6 / 74.1 -> 67.4; Q4_K 262144 x 2816 85.5 -> 77.8 /
 // 92.4 -> 82.2, 152064 x 5120 82.1 -> 74.0 / 89.0 -> 79.1; Q5_K 262144 x 2816 101.1 -> 90.8 / 107.5 -> 95.0, 262144 x 3840
-// 129.2 -> 114.6 / 142.3 -> 121.9; with fewer than a dozen windows per wave the fixed shares leave waves idle at the end
+// 129.2 -> 114.6 / 142.3 -> 121.9; Q4_0 262144 x 2816 81.2 -> 70.9 / 88.4 -> 78.6, Q8_0 120.2 -> 115.5 / 119.9 -> 115.6; with fewer
+// than a dozen windows per wave the fixed shares leave waves idle at the end
 // and the flat walk is as fast or faster.
 struct PArgs {
     const void* x;
@@ -771,8 +772,10 @@ template <int TYPE, bool X_BF16>
 constexpr uint32_t kPeriodMaxWaves = 16u;
 template <int TYPE, bool X_BF16>
 __global__ __launch_bounds__((64 * kPeriodMaxWaves<TYPE, X_BF16>)) void gemv_period_kernel(PArgs a) {
-    static_assert(TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K, "super-blocks of 256 weights");
-    constexpr uint32_t BB = kBlockBytes<TYPE>, CHUNKB = 16u * BB, PIECES = CHUNKB / 16u;  // 2304 / 2816 / 3360 bytes, 144 / 176 / 210 pieces
+    static_assert(TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K || TYPE == HQ_Q8_0_X2 || TYPE == kX2 + HQ_Q4_0,
+                  "super-blocks of 256 weights, four lanes each, or pairs of 32-weight blocks, one lane each");
+    // a window: 64 lanes = UW units of BB bytes; 2304 / 2816 / 3360 bytes (144 / 176 / 210 pieces), block pairs 4352 / 2304 (272 / 144)
+    constexpr uint32_t LPU = kLanesPerUnit<TYPE>, UW = kUnitsPerWindow<TYPE>, BB = kBlockBytes<TYPE>, CHUNKB = UW * BB, PIECES = CHUNKB / 16u;
     constexpr int NPV = (int)((PIECES + 63u) / 64u);
     using X = FlatX<TYPE, X_BF16>;
     extern __shared__ uint4 smem[];
@@ -780,8 +783,8 @@ __global__ __launch_bounds__((64 * kPeriodMaxWaves<TYPE, X_BF16>)) void gemv_per
     float* lds_s = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(smem) + X::value_bytes(a.k));
     const uint32_t tid = threadIdx.x, lane = tid & 63u, nthreads = blockDim.x;
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    uint4* wbuf = reinterpret_cast<uint4*>(lds_s + a.k / 16u) + wv * 256u;
-    float* slots = reinterpret_cast<float*>(reinterpret_cast<uint4*>(lds_s + a.k / 16u) + (nthreads >> 6) * 256u);
+    uint4* wbuf = reinterpret_cast<uint4*>(lds_s + a.k / 16u) + wv * (64u * NPV);
+    float* slots = reinterpret_cast<float*>(reinterpret_cast<uint4*>(lds_s + a.k / 16u) + (nthreads >> 6) * (64u * NPV));
     const int c = (int)(lane & 3u);
     const uint32_t P = a.period_windows, LR = a.log_period_rows, R = 1u << LR;
     const uint32_t j = wv % P, sq = wv / P;  // window of the period, sequence
@@ -806,18 +809,18 @@ __global__ __launch_bounds__((64 * kPeriodMaxWaves<TYPE, X_BF16>)) void gemv_per
     __syncthreads();
 
     [[maybe_unused]] uint32_t m4, m2, magic;
-    if constexpr (X_BF16)
+    if constexpr (X::PAIR)
         asm volatile("v_mov_b32 %0, %3\n\tv_mov_b32 %1, %4\n\tv_mov_b32 %2, %5" : "=v"(m4), "=v"(m2), "=v"(magic) : "s"(a.m4), "s"(a.m2), "s"(a.magic));
-    // the lane's block of the period, its row there and its super-block of that row
-    const uint32_t bi = 16u * j + (lane >> 2), rl = bi / a.bu, ur = bi - rl * a.bu;
-    const uint32_t r_lo = (16u * j) / a.bu, nseg = (16u * j + 15u) / a.bu - r_lo + 1u;  // rows the window touches: r_lo .. r_lo + nseg - 1
+    // the lane's unit of the period, its row there and its unit of that row
+    const uint32_t bi = UW * j + lane / LPU, rl = bi / a.bu, ur = bi - rl * a.bu;
+    const uint32_t r_lo = (UW * j) / a.bu, nseg = (UW * j + UW - 1u) / a.bu - r_lo + 1u;  // rows the window touches: r_lo .. r_lo + nseg - 1
     const uint32_t seg = rl - r_lo;
     uint32_t xr[X::XW];
-    float sx[4];
+    float sx[kIsX2<TYPE> ? 8 : 4] = {};
     X::load(lds_x, lds_s, ur, c, xr, sx);
     // lane s < nseg stores the sum of row r_lo + s: slot 0 if this is the row's first window, 1 if its second ...
     const uint32_t my_row = r_lo + (lane < nseg ? lane : 0u), MW = a.row_slots;
-    const uint32_t my_slot = MW * my_row + (j - (my_row * a.bu) / 16u);
+    const uint32_t my_slot = MW * my_row + (j - (my_row * a.bu) / UW);
 
     // Q6_K: block lane / 4 at byte 210 (lane / 4), fields at even offsets, read as aligned words and shifted into place
     [[maybe_unused]] const uint32_t blk = (lane >> 2) * BB, h = (uint32_t)c >> 1, lr = (uint32_t)c & 1u;
@@ -839,7 +842,22 @@ __global__ __launch_bounds__((64 * kPeriodMaxWaves<TYPE, X_BF16>)) void gemv_per
             asm volatile("" ::: "memory");
             if (i_cur + a.seqs < cnt_wg) fetch(i_cur + a.seqs);
             Piece<TYPE> pc;
-            if constexpr (TYPE != HQ_Q6_K) {  // blocks of whole 16-byte pieces
+            if constexpr (TYPE == kX2 + HQ_Q4_0) {  // [d0][16 bytes][d1][16 bytes] as nine words at a multiple of four bytes
+                const uint32_t* q = wb32 + lane * (BB / 4u);
+                const uint32_t w0 = q[0], w1 = q[1], w2 = q[2], w3 = q[3], w4 = q[4];
+                pc.a.d = w0 & 0xffffu;
+                pc.a.q = make_uint4(__builtin_amdgcn_alignbyte(w1, w0, 2), __builtin_amdgcn_alignbyte(w2, w1, 2), __builtin_amdgcn_alignbyte(w3, w2, 2),
+                                    __builtin_amdgcn_alignbyte(w4, w3, 2));
+                pc.b.d = w4 >> 16;
+                pc.b.q = make_uint4(q[5], q[6], q[7], q[8]);
+            } else if constexpr (TYPE == HQ_Q8_0_X2) {  // a block pair: seventeen words at a multiple of four bytes
+                const uint32_t* q = wb32 + lane * (BB / 4u);
+                pc.a = make_uint4(q[0], q[1], q[2], q[3]);
+                pc.b = make_uint4(q[4], q[5], q[6], q[7]);
+                pc.c = make_uint4(q[8], q[9], q[10], q[11]);
+                pc.e = make_uint4(q[12], q[13], q[14], q[15]);
+                pc.t = q[16];
+            } else if constexpr (TYPE != HQ_Q6_K) {  // blocks of whole 16-byte pieces
                 const uint4* b16 = wbuf + (lane >> 2) * (BB / 16u);
                 pc.hdr = b16[0];
                 if constexpr (TYPE == HQ_Q5_K) {
@@ -861,8 +879,15 @@ __global__ __launch_bounds__((64 * kPeriodMaxWaves<TYPE, X_BF16>)) void gemv_per
                 const uint32_t* q = wb32 + (o_d >> 2);
                 pc.d = __builtin_amdgcn_alignbyte(q[1], q[0], o_d & 3u);
             }
+            // (the sums of the activations are the same for every window: hidden from the compiler, so that no product of theirs
+            // with a constant is moved out of the loop and rounded on its own where the flat walk, which reloads them per window,
+            // fuses it into a multiply-add)
+            if constexpr (kIsX2<TYPE>) {  // (the K-quants' sums only meet block scales, which change with the window)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) asm volatile("" : "+v"(sx[q]));
+            }
             float part;
-            if constexpr (X_BF16) part = dot_pair(pc, c, xr, sx, m4, m2, magic);
+            if constexpr (X::PAIR) part = dot_pair(pc, c, xr, sx, m4, m2, magic);
             else part = dot_f32(pc, c, reinterpret_cast<const float*>(xr), sx);
             float mine = group_sum(seg == 0u ? part : 0.f, 6);
             if (nseg > 1u) {
@@ -880,7 +905,7 @@ __global__ __launch_bounds__((64 * kPeriodMaxWaves<TYPE, X_BF16>)) void gemv_per
         // the windows of row r of a period, added in the flat walk's order: 0 + first + second ...
         const uint32_t rows = (i1 - i0) << LR;
         for (uint32_t idx = tid; idx < rows; idx += nthreads) {
-            const uint32_t r = idx & (R - 1u), fb = r * a.bu, nwin = (fb + a.bu - 1u) / 16u - fb / 16u + 1u;
+            const uint32_t r = idx & (R - 1u), fb = r * a.bu, nwin = (fb + a.bu - 1u) / UW - fb / UW + 1u;
             float y = 0.f;
             for (uint32_t sl = 0; sl < nwin; ++sl) y += slots[MW * idx + sl];
             a.y[((size_t)(blockIdx.x + (i0 + (idx >> LR)) * gridDim.x) << LR) + r] = y;
@@ -888,36 +913,54 @@ __global__ __launch_bounds__((64 * kPeriodMaxWaves<TYPE, X_BF16>)) void gemv_per
         if (i1 < cnt_wg) __syncthreads();
     }
 }
+template <int TYPE>
+constexpr uint32_t kPeriodWaveBuf = (kUnitsPerWindow<TYPE> * kBlockBytes<TYPE> / 16u + 63u) / 64u * 1024u;  // bytes of a wave's window buffer
 template <int TYPE, bool X_BF16>
 inline size_t period_lds(uint32_t k, uint32_t waves, uint32_t slots) {
-    return FlatX<TYPE, X_BF16>::lds_bytes(k) + (size_t)waves * 4096u + (size_t)slots * 4u;
+    return FlatX<TYPE, X_BF16>::lds_bytes(k) + (size_t)waves * kPeriodWaveBuf<TYPE> + (size_t)slots * 4u;
 }
-// One 16-byte aligned K-quant matrix, rows of nine super-blocks or more and not whole windows, a period of sixteen windows at
+// P windows = R rows: the period of the row boundaries for rows of bu units in windows of uw
+inline void period_of(uint32_t bu, uint32_t uw, uint32_t* P, uint32_t* R) {
+    uint32_t a = bu, b = uw;
+    while (b) {
+        const uint32_t t = a % b;
+        a = b;
+        b = t;
+    }
+    *P = bu / a;
+    *R = uw / a;
+}
+// One 16-byte aligned matrix, rows of more than half a window (nine super-blocks, 33 block pairs) and not whole windows, a period of sixteen windows at
 // most, whole periods of rows, 176 windows per workgroup or more, ten waves or more with f32 activations (nine: Q6_K 65536 x
 // 4608 48.3 -> 49.3 us), and a shape for which the flat walk would use full windows over whole periods (so that both give the
 // same bits).
 template <int TYPE, bool X_BF16>
 inline bool period_takes(const void* w, uint32_t n, uint32_t k, uint32_t cus) {
-    constexpr uint32_t MAXW = kPeriodMaxWaves<TYPE, X_BF16>;
-    if (k % 256u) return false;
-    const uint32_t bu = k / 256u;
-    if (bu <= 8u || bu % 16u == 0u || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
-    const uint32_t g = bu % 2u ? 1u : bu % 4u ? 2u : bu % 8u ? 4u : 8u, P = bu / g, R = 16u / g;
+    constexpr uint32_t MAXW = kPeriodMaxWaves<TYPE, X_BF16>, UE = kUnitElems<TYPE>, UW = kUnitsPerWindow<TYPE>;
+    if (k % UE) return false;
+    const uint32_t bu = k / UE;
+    // (more than half a window per row: a window touches three rows at most)
+    if (bu <= UW / 2u || bu % UW == 0u || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
+    uint32_t P, R;
+    period_of(bu, UW, &P, &R);
     if (P > MAXW || n % R || (uint64_t)(n / R) * P < (uint64_t)176u * cus || (uint64_t)n * bu >= 0x7fff0000ull) return false;
     if ((!X_BF16 && MAXW / P * P < 10u) || period_lds<TYPE, X_BF16>(k, MAXW / P * P, 4096u) > 160u * 1024u - 512u) return false;
-    const FlatGeom fg = flat_geom(k, 256u, 16u, n, 1u, cus * (TYPE == HQ_Q6_K ? 12u : 16u));  // (as launch_flat asks)
-    return fg.uwe == 16u && (1u << fg.log_r) == R;
+    const FlatGeom fg = flat_geom(k, UE, UW, n, 1u, cus * (kBaseType<TYPE> == HQ_Q6_K || TYPE == HQ_Q8_0_X2 ? 12u : 16u));  // (as launch_flat asks)
+    return fg.uwe == UW && (1u << fg.log_r) == R;
 }
 template <int TYPE, bool X_BF16>
 int launch_period(hipStream_t s, const void* x, const uint8_t* w, float* y, uint32_t n, uint32_t k, uint32_t cus) {
-    const uint32_t bu = k / 256u, g = bu % 2u ? 1u : bu % 4u ? 2u : bu % 8u ? 4u : 8u, P = bu / g, R = 16u / g;
+    constexpr uint32_t UW = kUnitsPerWindow<TYPE>;
+    const uint32_t bu = k / kUnitElems<TYPE>;
+    uint32_t P, R;
+    period_of(bu, UW, &P, &R);
     const uint32_t seqs = kPeriodMaxWaves<TYPE, X_BF16> / P, W = seqs * P;
     uint32_t log_r = 0;
     while ((1u << log_r) < R) ++log_r;
     const uint32_t periods = n / R, per_wg = (periods + cus - 1u) / cus;
-    const uint32_t mw = (bu + 14u) / 16u + 1u, cap = 4096u / (R * mw);  // 16 KB of slots
+    const uint32_t mw = (bu + UW - 2u) / UW + 1u, cap = 4096u / (R * mw);  // 16 KB of slots
     const uint32_t ppr = per_wg < cap ? per_wg : cap;
-    const PArgs pa{x, w, y, n, k, bu, P, log_r, seqs, mw, ppr, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
+    const PArgs pa{x, w, y, n, k, bu, P, log_r, seqs, mw, ppr, kBaseType<TYPE> == HQ_Q6_K ? N4 : M4, kBaseType<TYPE> == HQ_Q5_K ? M1 : kBaseType<TYPE> == HQ_Q6_K ? N2 : M2, MAGIC};
     const size_t lds = period_lds<TYPE, X_BF16>(k, W, ppr * R * mw);
     auto kern = gemv_period_kernel<TYPE, X_BF16>;
     if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, "hipFuncSetAttribute(gemv period LDS)")) return rc;
@@ -1234,6 +1277,16 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     }
     // K-quant rows that are not whole windows (lm_heads of hidden size 2560 .. 3840, 5120, 7168; k = 14336): a fixed window of
     // the row period per wave, a pass per row.
+    if constexpr (kBlock32<TYPE>) {  // (as block pairs, where the flat walk would pair them)
+        if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && walk_doubled<TYPE, X_BF16>(a.n, a.k) &&
+            period_takes<kX2 + TYPE, X_BF16>(a.w, a.n, a.k, cus)) {
+            for (uint32_t r = 0; r < a.pairs; ++r)
+                if (int rc = launch_period<kX2 + TYPE, X_BF16>(s, static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * (X_BF16 ? 2 : 4), a.w,
+                                                               a.y + (size_t)r * a.n, a.n, a.k, cus))
+                    return rc;
+            return HQ_OK;
+        }
+    }
     if constexpr (TYPE == HQ_Q4_K || TYPE == HQ_Q5_K || TYPE == HQ_Q6_K) {
         if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && period_takes<TYPE, X_BF16>(a.w, a.n, a.k, cus)) {
             for (uint32_t r = 0; r < a.pairs; ++r)

@@ -393,7 +393,11 @@ __device__ __forceinline__ float dot_f32(const Piece<HQ_Q8_0_X2>& p, int, const 
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc1 = fmaf(sbyte(w[9 + j], i), xf[32 + 4 * j + i], acc1);
     }
-    return f16_bits_to_f32(w[0] & 0xffffu) * acc0 + f16_bits_to_f32(w[8] >> 16) * acc1;
+    // (the first product rounded on its own, the second fused into the sum: said here, so that every kernel that inlines this
+    // gets the same bits whichever of the two the compiler would have fused)
+    float first = f16_bits_to_f32(w[0] & 0xffffu) * acc0;
+    asm volatile("" : "+v"(first));
+    return fmaf(f16_bits_to_f32(w[8] >> 16), acc1, first);
 }
 __device__ __forceinline__ float dot_pair(const Piece<HQ_Q8_0_X2>&, int, const uint32_t*, const float*, uint32_t, uint32_t, uint32_t) {
     return 0.f;
@@ -405,12 +409,17 @@ template <int TYPE>
 __device__ __forceinline__ float dot_pair(const Piece<TYPE>& p, int c, const uint32_t* xp, const float* sx, uint32_t m4, uint32_t m2,
                                           uint32_t magic) {
     constexpr int B = kBaseType<TYPE>;
-    return dot_pair(p.a, c, xp, sx, m4, m2, magic) + dot_pair(p.b, c, xp + (kBlock32<B> ? 16 : 32), sx + (kBlock32<B> ? 2 : 4), m4, m2, magic);
+    // (the first half's value is final before the second is added: one way of fusing the last multiply, in every kernel)
+    float first = dot_pair(p.a, c, xp, sx, m4, m2, magic);
+    asm volatile("" : "+v"(first));
+    return first + dot_pair(p.b, c, xp + (kBlock32<B> ? 16 : 32), sx + (kBlock32<B> ? 2 : 4), m4, m2, magic);
 }
 template <int TYPE>
 __device__ __forceinline__ float dot_f32(const Piece<TYPE>& p, int c, const float* xf, const float* sx) {
     constexpr int B = kBaseType<TYPE>;
-    return dot_f32(p.a, c, xf, sx) + dot_f32(p.b, c, xf + (kBlock32<B> ? 32 : 64), sx + (kBlock32<B> ? 2 : 4));
+    float first = dot_f32(p.a, c, xf, sx);
+    asm volatile("" : "+v"(first));
+    return first + dot_f32(p.b, c, xf + (kBlock32<B> ? 32 : 64), sx + (kBlock32<B> ? 2 : 4));
 }
 
 // Staging of one activation row in LDS, 16 activations per thread and pass:

@@ -150,13 +150,14 @@ def test_copy_forms_and_their_fallbacks_give_the_same_bits(dev, xdt, t, n, k):
 @pytest.mark.parametrize("t,n,k", [(HQ_Q6_K, 262144, 2816), (HQ_Q6_K, 151936, 2560), (HQ_Q6_K, 151936, 3072), (HQ_Q6_K, 152064, 3584),
                                    (HQ_Q6_K, 131072, 3840), (HQ_Q6_K, 152064, 5120), (HQ_Q6_K, 65536, 7168), (HQ_Q6_K, 32768, 14336),
                                    (HQ_Q4_K, 262144, 2816), (HQ_Q4_K, 152064, 5120), (HQ_Q4_K, 151936, 3072), (HQ_Q5_K, 262144, 2816),
-                                   (HQ_Q5_K, 152064, 3584), (HQ_Q5_K, 65536, 7168)])
-def test_k_quant_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
-    """K-quant matrices whose rows are not whole windows of sixteen super-blocks (hidden sizes 2560 .. 3840, 5120, 7168; k =
+                                   (HQ_Q5_K, 152064, 3584), (HQ_Q5_K, 65536, 7168), (HQ_Q8_0, 262144, 2816), (HQ_Q4_0, 262144, 2816),
+                                   (HQ_Q4_0, 152064, 3584), (HQ_Q8_0, 65536, 7168)])
+def test_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
+    """Q8_0 / Q4_0 matrices (windows of 64 block pairs) and K-quant matrices whose rows are not whole windows of sixteen super-blocks (hidden sizes 2560 .. 3840, 5120, 7168; k =
     14336): every wave takes one fixed window of the period after which the row boundaries repeat (11 windows = 16 rows
     for k = 2816, 5 = 8 for 2560, 3 = 4 for 3072, 7 = 8 for 3584, 15 = 16 for 3840, 5 = 4 for 5120, 7 = 4 for 7168, 7 = 2 for
     14336), the rows' parts meet in LDS.  151936 x 3072 leaves a workgroup more periods than its slots hold (two rounds)
-    and a ragged share.  Sampled rows against the f64 oracle; Q6_K: the same bits as the flat walk, which a matrix off the
+    and a ragged share.  Sampled rows against the f64 oracle; Q6_K, Q8_0, Q4_0: the same bits as the flat walk, which a matrix off the
     16-byte grid takes; slices of 2048 rows against the kernels whose lanes fetch their own pieces; two activation rows; the
     same on a second call."""
     w = _quantized(dev, n, k, t, 31 + n + k)
@@ -173,7 +174,7 @@ def test_k_quant_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
     ref = oracle.qmatmul_f64(xv, _rows_of(w, rows, k, t, oracle), 2, rows.size, k, t)
     sel = torch.as_tensor(rows, device=dev)
     assert_matmul_close(y[:, sel].cpu().numpy(), ref[0:1], f"type {t} {xdt} {n}x{k}, sampled rows")
-    if t == HQ_Q6_K:  # (Q4_K / Q5_K matrices must lie on the 16-byte grid)
+    if t in (HQ_Q6_K, HQ_Q8_0, HQ_Q4_0):  # (Q4_K / Q5_K matrices must lie on the 16-byte grid)
         holder = torch.zeros(w.numel() + 32, dtype=torch.uint8, device=dev)
         shifted = holder[2:2 + w.numel()]
         shifted.copy_(w)
