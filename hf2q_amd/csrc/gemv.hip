@@ -1108,6 +1108,22 @@ bool flat_takes(uint64_t n_total, uint32_t k, uint32_t cus, size_t lds) {
     const uint64_t units = n_total * (k / UE);
     return units < 0x7fff0000ull && units / UW >= (uint64_t)cus * HQ_FLAT_MIN_WINDOWS_PER_CU;
 }
+// One small matrix (the projections of a decode step: 512 .. 4096 rows): the flat form from half a window per CU on, where
+// the kernel of 4-wave workgroups below is the slower one -- f32 activations (Q4_K 2048 x 1024: 4.35 -> 3.25 us, 128 x 4096: 4.2 ->
+// 3.1), 32-weight blocks with rows of 2048 weights or more (Q8_0 512 x 4096: 3.8 -> 3.55) -- and from sixteen windows on for
+// rows whose unit count is not a power of two, which that kernel's lane groups fit badly (k = 2816, 1024 rows: Q5_K 9.8 / 12.7 ->
+// 3.2 / 3.4 us, Q6_K 10.2 / 11.4 -> 3.2 / 3.4, Q8_0 8.0 -> 3.5; k = 5120, 1024 rows: Q4_K 5.7 / 11.8 -> 3.7 / 4.1).  K-quant rows
+// of a power-of-two length under bf16 activations stay with it (Q4_K 2048 x 512: 2.5 against 3.4 us).
+template <int TYPE, bool X_BF16>
+bool flat_takes_small(uint64_t n_total, uint32_t k, uint32_t cus, size_t lds) {
+    constexpr uint32_t UE = kUnitElems<TYPE>, UW = kUnitsPerWindow<TYPE>;
+    if (k % UE || k / UE < 2 || lds > 160 * 1024 - 512) return false;
+    const uint32_t bu = k / UE;
+    const uint64_t windows = n_total * bu / UW;
+    if (n_total * bu >= 0x7fff0000ull) return false;
+    if (bu & (bu - 1u)) return windows * 16u >= cus;
+    return ((!X_BF16 && bu >= 4u) || (kBlock32<TYPE> && k >= 2048u)) && windows * 2u >= cus;  // (rows of two super-blocks: 2048 x 512 f32 3.2 against 3.4 us)
+}
 // Fetches a wave keeps in flight: one (a ring of two or four windows of 32-weight blocks, which are only 1.1 / 2.2 KB,
 // measured slower: Q4_0 12288 x 4096 13.8 against 9.7 us).
 template <int TYPE>
@@ -1298,7 +1314,8 @@ int launch_t(hipStream_t s, const GemvArgs& a) {
     }
     // Other dense matrices with enough rows (any k of whole blocks, f32 activations, Q8_0 / Q4_0): the flat streaming form,
     // one pass per activation row.
-    if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits && flat_takes<TYPE>(a.n, a.k, cus, FlatX<TYPE, X_BF16>::lds_bytes(a.k))) {
+    if (a.top_k == 1 && !a.x2 && !a.ids && !a.route_logits &&
+        (flat_takes<TYPE>(a.n, a.k, cus, FlatX<TYPE, X_BF16>::lds_bytes(a.k)) || flat_takes_small<TYPE, X_BF16>(a.n, a.k, cus, FlatX<TYPE, X_BF16>::lds_bytes(a.k)))) {
         for (uint32_t r = 0; r < a.pairs; ++r)
             if (int rc = launch_flat<TYPE, X_BF16>(s, static_cast<const uint8_t*>(a.x) + (size_t)r * a.k * (X_BF16 ? 2 : 4), a.w, a.w,
                                                    a.y + (size_t)r * a.n, a.y + (size_t)r * a.n, a.n, a.k, 1, cus))

@@ -240,8 +240,11 @@ def test_small_batch_rows_staged_once(oracle, dev, t, xdt, n, k):
 # the 32-weight-block types; plus k = 4096 with f32 activations.  All of them take the flat streaming GEMV.
 # (4096, 5120), (2048, 14336) and (2048, 17408): rows of a window of sixteen super-blocks or more, whole and ragged, which the
 # Q6_K walk copies through LDS under bf16 activations.
+# (1024, 2816) ... (100, 5632): the projections of a decode step; rows whose super-block count is not a power of two take the flat
+# form from sixteen windows on, f32 activations and the 32-weight-block types from half a window per CU.
 FLAT_SHAPES = [(12288, 2816), (16384, 2048), (12288, 4096), (4099, 11264), (4096, 2816), (2816, 4096), (1500, 8960), (4096, 5120),
-               (2048, 14336), (2048, 17408)]
+               (2048, 14336), (2048, 17408), (1024, 2816), (256, 2816), (130, 2816), (24, 2816), (1024, 5120), (512, 1024), (100, 5632),
+               (300, 4096)]
 
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0])

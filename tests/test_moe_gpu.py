@@ -284,7 +284,9 @@ def test_dense_gemv_bf16_pair_equals_two_calls(dev):
 @pytest.mark.parametrize("m", [1, 4])
 @pytest.mark.parametrize("t,xdt", [(HQ_Q4_K, torch.bfloat16), (HQ_Q4_K, torch.float32), (HQ_Q6_K, torch.bfloat16)])
 def test_dense_ffn_batched_equals_separate_dispatches_and_cpu_spec(oracle, dev, m, t, xdt):
-    """dense_swiglu (ffn.rs:91-112) over the dequantised weights; two launches against four, bit for bit."""
+    """dense_swiglu (ffn.rs:91-112) over the dequantised weights; two launches against four: gate and up bit for bit, the
+    output to rounding (the down rows are five super-blocks long: as a call of its own the down GEMV takes the flat walk,
+    inside the batched launch the kernel of 4-wave workgroups, which add a row's parts in another order)."""
     H, I = 512, 1280
     raw = {"g": weights(31, I, H, 0.05), "u": weights(32, I, H, 0.05), "d": weights(33, H, I, 0.05)}
     q = {k_: oracle.quantize(v, v.shape[1], t, threads=8) for k_, v in raw.items()}
@@ -298,8 +300,8 @@ def test_dense_ffn_batched_equals_separate_dispatches_and_cpu_spec(oracle, dev, 
         out = torch.full((m, H), float("nan"), device=dev)
         ops.build_dense_ffn_layer_gpu_q_into(x, w, g, u, a, out, batched=batched)
         outs.append((out.cpu(), g.cpu(), u.cpu()))
-    for a_, b_ in zip(*outs):
-        assert torch.equal(a_, b_)
+    assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2])
+    assert (outs[0][0] - outs[1][0]).abs().max().item() <= 2e-6 * outs[0][0].abs().max().item()
     xr = x.float().cpu().numpy().astype(np.float64)
     gate, up = xr @ dq["g"].T, xr @ dq["u"].T
     want = (gate / (1 + np.exp(-gate)) * up) @ dq["d"].T
