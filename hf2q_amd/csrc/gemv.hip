@@ -57,6 +57,7 @@ struct KArgs {
     uint32_t log_l;   // log2 of the lanes that share one row
     uint32_t groups;  // row groups (one group = the rows a workgroup covers in one pass)
     uint32_t pairs;   // activation-row / output-row pairs (grid.y of the job)
+    uint32_t xpad;    // zeros staged behind the activations (elements): what the lanes past a row's last piece multiply with
     // Bit masks of the nibble -> bf16 conversion.  They are passed as arguments and
     // not written as literals so that the compiler keeps them in registers and
     // forms the three-operand v_and_or_b32 (gfx9 VOP3 takes no literals; with
@@ -122,7 +123,7 @@ struct Walk {
     const uint8_t* w;  // weight base + this lane's piece offset at step 0
     const uint32_t* lds_x;
     const float* lds_s;
-    uint32_t n, log_l, rpw, lane, li, steps, row_bytes, bstep, lane_row;
+    uint32_t n, log_l, rpw, lane, li, steps, row_bytes, bstep, lane_row, pieces, nblk, blk0;
     int c;
     uint32_t m4, m2, magic;
     Piece<TYPE> buf[D];
@@ -135,12 +136,17 @@ struct Walk {
         rpw = 64u >> log_l;
         li = lane & (L - 1u);
         lane_row = lane >> log_l;
-        steps = (a.k / EPL) >> log_l;  // pieces per row / L (host guarantees divisibility)
-        row_bytes = (a.k / (kBlock32<TYPE> ? 32 : 256)) * BYTES;
+        // pieces per row / L, rounded up: in the last step of a row whose pieces L does not divide, the lanes past the end fetch
+        // the row's last block again and multiply it with the zeros staged behind the activations
+        pieces = a.k / EPL;
+        steps = (pieces + L - 1u) >> log_l;
+        nblk = a.k / (kBlock32<TYPE> ? 32 : 256);
+        row_bytes = nblk * BYTES;
         // L >= 4 for the K-quants (k >= 256), so a lane keeps the same sub-piece index c on every step
         c = kBlock32<TYPE> ? 0 : (int)(li & 3u);
-        bstep = (kBlock32<TYPE> ? L : L >> 2) * BYTES;  // bytes of a row one step covers
-        w = wbase + (kBlock32<TYPE> ? li : li >> 2) * BYTES;
+        bstep = kBlock32<TYPE> ? L : L >> 2;  // blocks of a row one step covers
+        blk0 = kBlock32<TYPE> ? li : li >> 2;
+        w = wbase;
         lds_x = lx;
         lds_s = ls;
     }
@@ -158,7 +164,9 @@ struct Walk {
     __device__ __forceinline__ void fetch(Piece<TYPE>& f, uint32_t rowbase, int u, uint32_t s, float tie) {
         uint32_t r = rowbase + (uint32_t)u * rpw + lane_row;
         r = r < n ? r : n - 1u;
-        const uint8_t* ptr = w + (size_t)r * row_bytes + (size_t)s * bstep;
+        uint32_t blk = blk0 + s * bstep;
+        blk = blk < nblk ? blk : nblk - 1u;
+        const uint8_t* ptr = w + (size_t)r * row_bytes + (size_t)blk * BYTES;
         asm volatile("" : "+v"(ptr) : "v"(tie));
         f.load(ptr, c);
     }
@@ -179,7 +187,8 @@ struct Walk {
         for (uint32_t s = 0; s < steps; ++s) {
             uint32_t xr[XW];
             float sx[4];
-            load_x_piece<TYPE, PAIR, XW>(lds_x, lds_s, li + s * (1u << log_l), c, xr, sx);
+            const uint32_t pc = li + s * (1u << log_l);
+            load_x_piece<TYPE, PAIR, XW>(lds_x, lds_s, pc < pieces ? pc : pieces + (uint32_t)c, c, xr, sx);
             const bool more = s + 1 < steps;  // uniform
 #pragma unroll
             for (int u = 0; u < NR; ++u) {
@@ -216,11 +225,20 @@ struct Walk {
 // activations are requested first (vector loads return in order: behind a queue
 // of weight fetches they would hold the workgroup at its barrier), then the
 // first weight fetches go out so that their latency overlaps the staging.
+// The zeros behind the activations and behind their sums (rows whose pieces the lanes per row do not divide).
+template <bool PAIR>
+__device__ __forceinline__ void stage_zero_pad(const KArgs& a, uint32_t* lds_x, float* lds_s, uint32_t tid, uint32_t threads) {
+    if (!a.xpad) return;
+    const uint32_t xw = PAIR ? a.k / 2 : a.k, pw = PAIR ? a.xpad / 2 : a.xpad;
+    for (uint32_t i = tid; i < pw; i += threads) lds_x[xw + i] = 0u;
+    for (uint32_t i = tid; i < a.xpad / 16u; i += threads) lds_s[a.k / 16u + i] = 0.f;
+}
+
 template <int TYPE, bool X_BF16, bool PAIR, int NR, int D>
 __device__ __forceinline__ void gemv_body(const KArgs& a, uint32_t bx, uint32_t p) {
     extern __shared__ uint4 smem[];
     uint32_t* lds_x = reinterpret_cast<uint32_t*>(smem);
-    float* lds_s = reinterpret_cast<float*>(lds_x + (PAIR ? a.k / 2 : a.k));
+    float* lds_s = reinterpret_cast<float*>(lds_x + (PAIR ? (a.k + a.xpad) / 2 : a.k + a.xpad));
 
     const size_t xoff = (size_t)(p / a.top_k) * a.k * (X_BF16 ? 2 : 4);
     const uint8_t* xrow = static_cast<const uint8_t*>(a.x) + xoff;
@@ -276,6 +294,7 @@ __device__ __forceinline__ void gemv_body(const KArgs& a, uint32_t bx, uint32_t 
             stage_swiglu(sraw, i, lds_x, lds_s);
         }
     }
+    stage_zero_pad<PAIR>(a, lds_x, lds_s, threadIdx.x, 256u);
     wk.load_masks(a);
     __syncthreads();
 
@@ -315,8 +334,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_queue_kernel(KArgs a) {
     constexpr uint32_t THREADS = 64 * WAVES;
     extern __shared__ uint4 smem[];
     uint32_t* lds_x = reinterpret_cast<uint32_t*>(smem);
-    float* lds_s = reinterpret_cast<float*>(lds_x + (PAIR ? a.k / 2 : a.k));
-    uint32_t* lds_q = reinterpret_cast<uint32_t*>(lds_s + a.k / 16);
+    float* lds_s = reinterpret_cast<float*>(lds_x + (PAIR ? (a.k + a.xpad) / 2 : a.k + a.xpad));
+    uint32_t* lds_q = reinterpret_cast<uint32_t*>(lds_s + (a.k + a.xpad) / 16);
 
     const uint8_t* xrow = static_cast<const uint8_t*>(a.x);
     const uint32_t xchunks = a.k / 16;
@@ -344,6 +363,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_queue_kernel(KArgs a) {
         xraw.fetch(xrow, i);
         stage_store<X_BF16, PAIR>(xraw, i, lds_x, lds_s);
     }
+    stage_zero_pad<PAIR>(a, lds_x, lds_s, threadIdx.x, THREADS);
     wk.load_masks(a);
     __syncthreads();
 
@@ -1215,15 +1235,29 @@ int plan_job(const GemvArgs& a, KArgs* ka, size_t* lds, uint64_t* slots) {
     constexpr bool PAIR = X_BF16 && !kBlock32<TYPE>;
     constexpr int EPL = Lane<TYPE>::kElems;
     if (a.x2 && X_BF16) return fail(HQ_ERR_UNSUPPORTED, "gemv: the fused SwiGLU form takes f32 activations");
-    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.route_logits, a.route_ids, a.route_w, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
+    *ka = KArgs{a.x, a.x2, a.w, a.ids, a.route_logits, a.route_ids, a.route_w, a.y, a.top_k, a.n, a.k, a.n_experts, a.expert_stride, 0, 0, a.pairs, 0, TYPE == HQ_Q6_K ? N4 : M4, TYPE == HQ_Q5_K ? M1 : TYPE == HQ_Q6_K ? N2 : M2, MAGIC};
     const uint32_t pieces = a.k / EPL;
-    // L = largest power of two <= 64 that divides the pieces of a row
+    // L = largest power of two <= 64 that divides the pieces of a row ...
     uint32_t log_l = 0;
     while (log_l < 6 && pieces % (2u << log_l) == 0) ++log_l;
+    // ... unless that leaves fewer than sixteen lanes per row (k = 2816: 44 quarters of a super-block, four lanes walking eleven
+    // steps each; 1024 x 2816 Q5_K: 9.8 us): then the L of 16, 32, 64 that wastes the fewest lane steps, the last step of a row
+    // ragged, its idle lanes multiplying zeros staged behind the activations (q / k / v of 4096 + 1024 + 1024 rows x 2816 as one
+    // launch, Q5_K: 12.9 -> 8.8 us).  bf16 activations only: with f32 ones the four times as many workgroups, each staging 11 KB
+    // of them, cost more than the shorter walk saves (15.8 -> 20.3 us)
+    if (X_BF16 && log_l < 4 && pieces >= 12) {
+        uint32_t best = 0;
+        for (uint32_t l = 4; l <= 6; ++l) {
+            const uint32_t padded = (pieces + (1u << l) - 1u) >> l << l;
+            if (!best || padded <= best) best = padded, log_l = l;
+        }
+        ka->xpad = kBlock32<TYPE> ? 32u : 256u;
+    }
     ka->log_l = log_l;
     const uint32_t rpw = 64u >> log_l;
-    // activations, their per-16 sums, the queue counter
-    *lds = (size_t)(PAIR ? a.k * 2 : a.k * 4) + (size_t)(a.k / 16) * 4 + 16;
+    // activations (and the zeros behind them), their per-16 sums, the queue counter
+    const uint32_t kx = a.k + ka->xpad;
+    *lds = (size_t)(PAIR ? kx * 2 : kx * 4) + (size_t)(kx / 16) * 4 + 16;
     if (*lds > 160 * 1024 - 512)
         return fail(HQ_ERR_UNSUPPORTED, "gemv: k = %u needs %zu bytes of LDS (limit 160 KiB)", a.k, *lds);
     *slots = (uint64_t)((a.n + rpw - 1) / rpw) * a.pairs;
