@@ -127,8 +127,9 @@ def test_gemv_unaligned_weight_base(oracle, dev, t):
     assert_matmul_close(y.cpu().numpy(), ref, "unaligned base")
 
 
-ID_CASES = [  # (E, n, k, T, K)
+ID_CASES = [  # (E, n, k, T, K); k = 768, 2816, 1280: rows whose pieces no sixteen lanes divide (a ragged last step under bf16 rows)
     (8, 64, 512, 1, 2), (16, 512, 2048, 1, 8), (16, 2048, 512, 8, 1), (256, 128, 256, 8, 8), (4, 33, 768, 5, 3),
+    (8, 48, 2816, 3, 2), (4, 40, 1280, 2, 4),
 ]
 
 
