@@ -852,9 +852,10 @@ constexpr size_t kLdsPerCu = 160 * 1024 - 512;
 // Whether the stage-once form takes the product (all of k in LDS, two groups of 16 rows or more per CU), its LDS bytes,
 // and whether the wave-owned piece buffers of the transposed fetch fit beside the activations.
 // (bf: eight staged rows -- bf16 rows, or up to four f32 rows as hi and lo parts)
-bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t cus, size_t* lds, bool* xpose) {
+// min_groups8: groups of 16 rows per CU the matrix must have, in eighths (16 = two groups)
+bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t cus, size_t* lds, bool* xpose, uint32_t min_groups8 = 16u) {
     const size_t lds_all = (size_t)((k + KC - 1u) / KC) * (bf ? kStage<true> : kStage<false>);
-    if (k % 256u || lds_all > kLdsPerCu || (n + 15u) / 16u < 2u * cus) return false;
+    if (k % 256u || lds_all > kLdsPerCu || (uint64_t)((n + 15u) / 16u) * 8u < (uint64_t)min_groups8 * cus) return false;
     const size_t pitch16 = 16u * (t == HQ_Q4_K ? Q4kRows<false>::PITCH : t == HQ_Q5_K ? Q4kRows<true>::PITCH : t == HQ_Q6_K ? Q6kRows::PITCH : t == HQ_Q8_0 ? Q80Rows::PITCH : Q40Rows::PITCH);
     *xpose = lds_all + kStreamWaves * pitch16 <= kLdsPerCu;
     *lds = lds_all + (*xpose ? kStreamWaves * pitch16 : 0);
@@ -877,6 +878,13 @@ bool gemv_rows_stream_fast(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_
 // with either activation type.  Such k has no multi-row streaming passes either, so the form starts at three rows for
 // every type (Q6_K 262144 x 2816 f32: 228 against 318 us), and at two where the weights go through the transposed fetch
 // (bf16 rows: Q6_K 262144 x 2816 146 against 191 us for two passes, Q4_K 90 against 153, Q5_K 152064 x 3584 86 against 130).
+// Small K-quant matrices whose k is not whole chunks have no other kernel that reads the weights once for all rows: from four
+// rows on the stage-once form takes them down to an eighth of a group per CU (Q5_K 4096 x 2816: 11.5 us for 4 .. 8 rows against
+// 17 / 33 us as a pass per row; 1024 x 2816: 11.4 against 12.2 / 24).
+inline uint32_t rows_stream_min_groups8(hq_ggml_type t, uint32_t m, uint32_t k) {
+    return (t == HQ_Q4_K || t == HQ_Q5_K || t == HQ_Q6_K) && k % KC != 0 && k > KC && m >= 4 ? 1u : 16u;  // (k < 1024: a pass per row is quick)
+}
+
 bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32_t n, uint32_t k) {
     if (m < 2 || m > 8 || (t != HQ_Q4_K && t != HQ_Q5_K && t != HQ_Q6_K && t != HQ_Q8_0 && t != HQ_Q4_0)) return false;
     uint32_t cus = 0;
@@ -884,8 +892,9 @@ bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32
     size_t lds = 0;
     bool xpose = false, xpose_h = false;
     // up to four f32 rows as hi and lo parts in the space of eight bf16 rows, with the transposed fetch
-    const bool half = xdt != HQ_BF16 && m <= 4 && rows_stream_plan(t, true, n, k, cus, &lds, &xpose_h) && xpose_h;
-    if (!rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose) && !half) return false;
+    const uint32_t mg8 = rows_stream_min_groups8(t, m, k);
+    const bool half = xdt != HQ_BF16 && m <= 4 && rows_stream_plan(t, true, n, k, cus, &lds, &xpose_h, mg8) && xpose_h;
+    if (!rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose, mg8) && !half) return false;
     const bool fast = (xdt == HQ_BF16 && xpose) || half;
     // Q8_0: where the transposed fetch fits, from two rows on (bf16, 262144 x 2816: 140 .. 150 us for 2 .. 8 rows where the
     // kernel of exact f32 products takes 237 .. 426 and one row 126; 12288 x 4096: 15.4 against 17.5 .. 30.0); without the
@@ -910,7 +919,8 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
     if (int rc = cu_count(&cus)) return rc;
     size_t lds_k = 0;
     bool xpose = false;
-    if (!bf && m <= 4 && rows_stream_plan(t, true, n, k, cus, &lds_k, &xpose) && xpose) {
+    const uint32_t mg8 = rows_stream_min_groups8(t, m, k);
+    if (!bf && m <= 4 && rows_stream_plan(t, true, n, k, cus, &lds_k, &xpose, mg8) && xpose) {
         constexpr int W = kStreamWaves;
         void (*sk)(RowsArgs) = t == HQ_Q4_K   ? rows_stream_kernel<Q4kRows<false>, false, W, true, true>
                                : t == HQ_Q5_K ? rows_stream_kernel<Q4kRows<true>, false, W, true, true>
@@ -921,7 +931,7 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
         hipLaunchKernelGGL(sk, dim3(cus), dim3(64 * W), lds_k, s, a);
         return check_launch("rows stream kernel launch");
     }
-    if (rows_stream_plan(t, bf, n, k, cus, &lds_k, &xpose)) {
+    if (rows_stream_plan(t, bf, n, k, cus, &lds_k, &xpose, mg8)) {
         constexpr int W = kStreamWaves;
         void (*sk)(RowsArgs);
         if (xpose)

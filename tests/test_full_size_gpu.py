@@ -201,7 +201,8 @@ def test_rows_that_are_not_whole_windows(oracle, dev, xdt, t, n, k):
 
 @pytest.mark.parametrize("t", [HQ_Q4_K, HQ_Q5_K, HQ_Q6_K, HQ_Q8_0, HQ_Q4_0])
 @pytest.mark.parametrize("xdt", ["bf16", "f32"])
-@pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048), (8203, 2816), (9001, 3584), (8192, 5120), (33000, 2816)])
+@pytest.mark.parametrize("n,k", [(8200, 4096), (8195, 1024), (40000, 2048), (8203, 2816), (9001, 3584), (8192, 5120), (33000, 2816), (1000, 2816),
+                                 (4100, 3584)])
 def test_small_batch_rows_staged_once(oracle, dev, t, xdt, n, k):
     """3 .. 8 activation rows over matrices of two groups of 16 rows per CU or more, all of k in LDS: the small-batch form
     that stages the activations once per CU (bf16: weights fetched as 16-byte pieces through LDS; f32: fetched by the
@@ -209,7 +210,9 @@ def test_small_batch_rows_staged_once(oracle, dev, t, xdt, n, k):
     of 1024 activations (the last chunk holds 3, 2 and 1 super-blocks): only this form takes them; 5120 as f32 does not fit
     the LDS and runs a pass per row.  Q8_0 and Q4_0 (eight blocks = a super-block of seventeen / nine pieces, one MFMA per block
     over the bytes / nibbles as bf16) take the form with bf16 rows from two rows on; f32 rows up to four likewise, five to eight as two
-    passes on matrices of 32768 rows or more (33000 x 2816), else through the kernel of exact f32 products.  Sampled rows against the f64 oracle, every row
+    passes on matrices of 32768 rows or more (33000 x 2816), else through the kernel of exact f32 products.  1000 x 2816 and 4100 x 3584: K-quant
+    matrices too small for the form at two or three rows (a pass per row), which takes them from four rows on because such k has
+    no other kernel that reads the weights once.  Sampled rows against the f64 oracle, every row
     against the one-row product of the same activations, and the same result on a second call."""
     w = _quantized(dev, n, k, t, 11 + n + t)
     rng = np.random.default_rng(n + k + t)

@@ -301,7 +301,9 @@ def test_dense_ffn_batched_equals_separate_dispatches_and_cpu_spec(oracle, dev, 
         ops.build_dense_ffn_layer_gpu_q_into(x, w, g, u, a, out, batched=batched)
         outs.append((out.cpu(), g.cpu(), u.cpu()))
     assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2])
-    assert (outs[0][0] - outs[1][0]).abs().max().item() <= 2e-6 * outs[0][0].abs().max().item()
+    # (one row: another order of the same exact products; four rows: the separate down product runs on the matrix cores, its f32
+    # activations as bf16 hi + lo parts)
+    assert (outs[0][0] - outs[1][0]).abs().max().item() <= (2e-6 if m == 1 else 1e-4) * outs[0][0].abs().max().item()
     xr = x.float().cpu().numpy().astype(np.float64)
     gate, up = xr @ dq["g"].T, xr @ dq["u"].T
     want = (gate / (1 + np.exp(-gate)) * up) @ dq["d"].T
