@@ -109,7 +109,8 @@ HQ_API int hq_quantize_ggml_imatrix(void* stream, const float* src, uint64_t n_e
  * whose tiles are 64 (Q4_K / Q5_K), 128 or 256 token rows by m; up to 256 rows k is cut into slices where the
  * weight-row tiles alone would leave CUs idle.
  * A K-quant's k that is not a multiple of 1024 (2816, 3584, 5120 ...) has the small-batch kernel where all of k fits a
- * CU's LDS and the matrix has 8192 rows or more; otherwise up to 16 rows run as per-row GEMVs first.
+ * CU's LDS and the matrix has 8192 rows or more (512 or more from four activation rows on); otherwise up to 16 rows run
+ * as per-row GEMVs first.
  * MFMA GEMM.  The K-quant (k % 256 == 0) and Q8_0 / Q4_0 (k % 128 == 0) GEMMs multiply f16-rounded
  * weights and activations like the reference's mul_mm, the other kernels keep
  * every product exact.
