@@ -853,12 +853,21 @@ constexpr size_t kLdsPerCu = 160 * 1024 - 512;
 // and whether the wave-owned piece buffers of the transposed fetch fit beside the activations.
 // (bf: eight staged rows -- bf16 rows, or up to four f32 rows as hi and lo parts)
 // min_groups8: groups of 16 rows per CU the matrix must have, in eighths (16 = two groups)
-bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t cus, size_t* lds, bool* xpose, uint32_t min_groups8 = 16u) {
+// waves12: sixteen staged rows (f32 activations) whose piece buffers fit for twelve waves only (k <= 3072 as f32)
+bool rows_stream_plan(hq_ggml_type t, bool bf, uint32_t n, uint32_t k, uint32_t cus, size_t* lds, bool* xpose, uint32_t min_groups8 = 16u,
+                      bool* waves12 = nullptr) {
     const size_t lds_all = (size_t)((k + KC - 1u) / KC) * (bf ? kStage<true> : kStage<false>);
     if (k % 256u || lds_all > kLdsPerCu || (uint64_t)((n + 15u) / 16u) * 8u < (uint64_t)min_groups8 * cus) return false;
     const size_t pitch16 = 16u * (t == HQ_Q4_K ? Q4kRows<false>::PITCH : t == HQ_Q5_K ? Q4kRows<true>::PITCH : t == HQ_Q6_K ? Q6kRows::PITCH : t == HQ_Q8_0 ? Q80Rows::PITCH : Q40Rows::PITCH);
     *xpose = lds_all + kStreamWaves * pitch16 <= kLdsPerCu;
     *lds = lds_all + (*xpose ? kStreamWaves * pitch16 : 0);
+    if (waves12) {
+        *waves12 = !bf && !*xpose && lds_all + 12u * pitch16 <= kLdsPerCu;
+        if (*waves12) {
+            *xpose = true;
+            *lds = lds_all + 12u * pitch16;
+        }
+    }
     return true;
 }
 }  // namespace
@@ -894,8 +903,11 @@ bool gemv_rows_stream_takes(hq_ggml_type t, hq_act_dtype xdt, uint32_t m, uint32
     // up to four f32 rows as hi and lo parts in the space of eight bf16 rows, with the transposed fetch
     const uint32_t mg8 = rows_stream_min_groups8(t, m, k);
     const bool half = xdt != HQ_BF16 && m <= 4 && rows_stream_plan(t, true, n, k, cus, &lds, &xpose_h, mg8) && xpose_h;
-    if (!rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose, mg8) && !half) return false;
-    const bool fast = (xdt == HQ_BF16 && xpose) || half;
+    bool w12 = false;
+    if (!rows_stream_plan(t, xdt == HQ_BF16, n, k, cus, &lds, &xpose, mg8, &w12) && !half) return false;
+    // (five to eight f32 rows: the transposed fetch with twelve waves where sixteen staged rows leave room for that many piece
+    // buffers -- k <= 3072: Q6_K 262144 x 2816 228 us without it, Q8_0 two passes of four rows 280)
+    const bool fast = (xdt == HQ_BF16 && xpose) || half || w12;
     // Q8_0: where the transposed fetch fits, from two rows on (bf16, 262144 x 2816: 140 .. 150 us for 2 .. 8 rows where the
     // kernel of exact f32 products takes 237 .. 426 and one row 126; 12288 x 4096: 15.4 against 17.5 .. 30.0); without the
     // transposed fetch, and with five f32 rows or more (hi + lo parts: twice the LDS), that kernel stays ahead
@@ -929,6 +941,17 @@ int launch_gemv_rows(hipStream_t s, const void* x, hq_act_dtype xdt, const void*
                                               : rows_stream_kernel<Q40Rows, false, W, true, true>;
         if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(sk), lds_k, "hipFuncSetAttribute(rows stream kernel LDS)")) return rc;
         hipLaunchKernelGGL(sk, dim3(cus), dim3(64 * W), lds_k, s, a);
+        return check_launch("rows stream kernel launch");
+    }
+    bool w12 = false;
+    if (rows_stream_plan(t, bf, n, k, cus, &lds_k, &xpose, mg8, &w12) && w12) {
+        void (*sk)(RowsArgs) = t == HQ_Q4_K   ? rows_stream_kernel<Q4kRows<false>, false, 12, true>
+                               : t == HQ_Q5_K ? rows_stream_kernel<Q4kRows<true>, false, 12, true>
+                               : t == HQ_Q6_K ? rows_stream_kernel<Q6kRows, false, 12, true>
+                               : t == HQ_Q8_0 ? rows_stream_kernel<Q80Rows, false, 12, true>
+                                              : rows_stream_kernel<Q40Rows, false, 12, true>;
+        if (int rc = ensure_lds_limit(reinterpret_cast<const void*>(sk), lds_k, "hipFuncSetAttribute(rows stream kernel LDS)")) return rc;
+        hipLaunchKernelGGL(sk, dim3(cus), dim3(64 * 12), lds_k, s, a);
         return check_launch("rows stream kernel launch");
     }
     if (rows_stream_plan(t, bf, n, k, cus, &lds_k, &xpose, mg8)) {
